@@ -1,0 +1,250 @@
+/*
+ * shadow_hip.h -- C ABI of the MI355X (gfx950) device layer for Shadow's tensor
+ * hot path: Unary, Binary (N-d broadcast), Eltwise, Reduce, Activate, Scale and
+ * the elementwise part of Blas.
+ *
+ * Conventions
+ *   - every entry point returns int: 0 on success, a positive hipError_t value
+ *     when the HIP runtime failed, a negative SHDW_E_* value when the arguments
+ *     were rejected on the host before anything was enqueued.
+ *     shdw_hip_error_string() turns either into text.
+ *   - nothing throws, nothing synchronises unless its name says "sync" (the
+ *     one exception, shdw_hip_asum, is documented at its declaration).
+ *   - `stream` is a hipStream_t passed as void*; NULL means the null stream.
+ *   - all tensors are dense row-major fp32 in device memory; element counts
+ *     and indices are int32 like Shadow's Blob::count().
+ *   - pointers are borrowed for the duration of the enqueued work.  Every
+ *     purely elementwise entry point may be called in place (y == a).
+ *   - arithmetic follows Shadow's CPU kernels exactly: separate multiply and
+ *     add (never fused), std::max/std::min selection semantics, fp64
+ *     accumulation in reductions.
+ *
+ * Citations "ref:" name the file and lines of junluan/shadow that the entry
+ * point replaces on the GPU side.
+ */
+#ifndef SHADOW_HIP_H_
+#define SHADOW_HIP_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- error codes produced by this library itself (hipError_t are > 0) ---- */
+#define SHDW_OK 0
+#define SHDW_E_INVALID_ARGUMENT (-1) /* null pointer, negative count, bad enum */
+#define SHDW_E_UNSUPPORTED (-2)      /* shape outside what the kernels accept  */
+#define SHDW_E_WORKSPACE (-3)        /* workspace missing or too small         */
+
+/* ---- operation enums; values are Shadow's ---- */
+/* ref: shadow/operators/kernels/unary.hpp:9-25 */
+enum {
+  SHDW_UNARY_ABS = 0, SHDW_UNARY_SQUARE = 1, SHDW_UNARY_SQRT = 2, SHDW_UNARY_LOG = 3,
+  SHDW_UNARY_EXP = 4, SHDW_UNARY_SIN = 5, SHDW_UNARY_COS = 6, SHDW_UNARY_TAN = 7,
+  SHDW_UNARY_ASIN = 8, SHDW_UNARY_ACOS = 9, SHDW_UNARY_ATAN = 10, SHDW_UNARY_FLOOR = 11,
+  SHDW_UNARY_CEIL = 12, SHDW_UNARY_NEG = 13, SHDW_UNARY_RECIPROCAL = 14
+};
+/* ref: shadow/operators/kernels/binary.hpp:23 */
+enum {
+  SHDW_BINARY_ADD = 0, SHDW_BINARY_SUB = 1, SHDW_BINARY_MUL = 2, SHDW_BINARY_DIV = 3,
+  SHDW_BINARY_POW = 4, SHDW_BINARY_MAX = 5, SHDW_BINARY_MIN = 6
+};
+/* ref: shadow/operators/kernels/eltwise.hpp:9 */
+enum { SHDW_ELTWISE_PROD = 0, SHDW_ELTWISE_SUM = 1, SHDW_ELTWISE_MAX = 2, SHDW_ELTWISE_MIN = 3 };
+/* ref: shadow/operators/kernels/reduce.hpp:21-29 */
+enum {
+  SHDW_REDUCE_PROD = 0, SHDW_REDUCE_SUM = 1, SHDW_REDUCE_MAX = 2, SHDW_REDUCE_MIN = 3,
+  SHDW_REDUCE_AVG = 4, SHDW_REDUCE_L1 = 5, SHDW_REDUCE_L2 = 6
+};
+/* ref: shadow/operators/kernels/activate.hpp:24-34 */
+enum {
+  SHDW_ACT_PRELU = 0, SHDW_ACT_RELU = 1, SHDW_ACT_LEAKY = 2, SHDW_ACT_SIGMOID = 3,
+  SHDW_ACT_SOFTPLUS = 4, SHDW_ACT_TANH = 5, SHDW_ACT_RELU6 = 6, SHDW_ACT_HARDSWISH = 7,
+  SHDW_ACT_GELU = 8
+};
+
+/* ======================= device, stream, allocator ======================= */
+
+/* ref: shadow/core/context.cu:95-110 (check_device: cudaGetDeviceCount) */
+int shdw_hip_device_count(int* count);
+/* ref: shadow/core/context.cu:15,63 (cudaSetDevice in ctor and switch_device) */
+int shdw_hip_set_device(int device_id);
+/* ref: shadow/core/context.cu:99-108 (cudaGetDeviceProperties for the debug line).
+ * Writes "name|gcnArch|CUs|clock_khz" into buf (truncated to buf_size). */
+int shdw_hip_device_info(int device_id, char* buf, size_t buf_size);
+/* ref: shadow/core/context.cu:17-21 (cudaStreamCreate) */
+int shdw_hip_stream_create(void** stream);
+/* ref: shadow/core/context.cu:39-43 (cudaStreamDestroy) */
+int shdw_hip_stream_destroy(void* stream);
+/* ref: shadow/core/context.cu:65-67 (cudaStreamSynchronize) */
+int shdw_hip_stream_sync(void* stream);
+/* ref: shadow/core/external.hpp:39-43 (CUDA_CHECK -> cudaGetErrorString) */
+const char* shdw_hip_error_string(int rc);
+/* ref: shadow/core/external.hpp:39-43 together with the cudaPeekAtLastError
+ * after each launch (e.g. shadow/core/blas.cu:20): returns and clears the
+ * runtime's sticky launch error. */
+int shdw_hip_last_error(void);
+
+/* ref: shadow/core/allocator.cu:11-18 (GPUAllocator::malloc -> cudaMalloc) */
+int shdw_hip_malloc(void** ptr, size_t bytes);
+/* ref: shadow/core/allocator.cu:47 (GPUAllocator::free -> cudaFree) */
+int shdw_hip_free(void* ptr);
+/* ref: shadow/core/allocator.cu:29-36 (write: H2D; blocking when stream==NULL) */
+int shdw_hip_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream);
+/* ref: shadow/core/allocator.cu:20-27 (read: D2H; blocking when stream==NULL) */
+int shdw_hip_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream);
+/* ref: shadow/core/allocator.cu:38-45 (copy: D2D; blocking when stream==NULL) */
+int shdw_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream);
+/* Pinned host staging memory for the two calls above; Shadow reads back into a
+ * pageable std::vector (shadow/core/blob.hpp:52-63), which makes its D2H
+ * effectively blocking. */
+int shdw_hip_host_malloc(void** ptr, size_t bytes);
+int shdw_hip_host_free(void* ptr);
+
+/* Events: Shadow only times on the host (Util::Timer, shadow/util/util.hpp:529-657);
+ * the measurement harness needs device time for one stream. */
+int shdw_hip_event_create(void** event);
+int shdw_hip_event_destroy(void* event);
+int shdw_hip_event_record(void* event, void* stream);
+int shdw_hip_event_sync(void* event);
+int shdw_hip_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* ============================ Blas, elementwise ========================== */
+
+/* y[i] = val.  ref: shadow/core/blas.cpp:25-34, shadow/core/blas.cu:11-21 */
+int shdw_hip_set(int n, float val, float* y, void* stream);
+/* y[i] = f(a[i]), f chosen by SHDW_UNARY_*.
+ * ref: shadow/core/blas.cpp:143-168 (loop branch), shadow/core/blas.cu:77-108,
+ *      dispatch shadow/operators/kernels/unary.hpp:37-93 */
+int shdw_hip_unary(int operation, int n, const float* a, float* y, void* stream);
+/* y[i] = a[i] op b[i], SHDW_BINARY_*.
+ * ref: shadow/core/blas.cpp:103-121, shadow/core/blas.cu:23-48 */
+int shdw_hip_binary(int operation, int n, const float* a, const float* b, float* y,
+                    void* stream);
+/* y[i] = a[i] op alpha.
+ * ref: shadow/core/blas.cpp:123-141, shadow/core/blas.cu:50-75 */
+int shdw_hip_binary_scalar(int operation, int n, const float* a, float alpha, float* y,
+                           void* stream);
+/* x[i] *= alpha.  ref: shadow/core/blas.cpp:172-184, blas.cu:110-115 */
+int shdw_hip_scal(int n, float alpha, float* x, void* stream);
+/* y[i] = x[i].    ref: shadow/core/blas.cpp:186-200, blas.cu:117-122 */
+int shdw_hip_copy(int n, const float* x, float* y, void* stream);
+/* y[i] += alpha * x[i] (separate fp32 multiply and add).
+ * ref: shadow/core/blas.cpp:202-217, blas.cu:124-130 */
+int shdw_hip_axpy(int n, float alpha, const float* x, float* y, void* stream);
+/* *result_host = (float) sum_i |x[i]| accumulated in fp64.  Like cublasSasum
+ * with a host result pointer this call returns only after the value is on the
+ * host (it synchronises `stream`).  `workspace` must hold 16 bytes more than
+ * shdw_hip_reduce_workspace_bytes(1, {n}, 1, {0}) (the device-side result).
+ * ref: shadow/core/blas.cpp:219-235, blas.cu:132-138 */
+int shdw_hip_asum(int n, const float* x, float* result_host, void* workspace,
+                  size_t workspace_bytes, void* stream);
+
+/* ================================ Binary ================================= */
+
+/* Numpy-style broadcast: a_shape/b_shape/out_shape are HOST arrays of num_axes
+ * ints, already rank-aligned (each a/b dim equals the out dim or is 1).
+ * y[out index] = a[...] op b[...] with a as the left operand.
+ * The dims are collapsed on the host and travel as kernel arguments; there is
+ * no device-side shape table.
+ * ref: shadow/operators/kernels/binary.cpp:30-52, binary.cu:28-64,
+ *      caller shadow/operators/kernels/binary.hpp:80-98 */
+int shdw_hip_broadcast_binary(int operation, int num_axes, const int* a_shape,
+                              const int* b_shape, const int* out_shape, const float* a,
+                              const float* b, float* y, void* stream);
+
+/* =============================== Activate ================================ */
+
+/* y[i] = act(x[i]) for SHDW_ACT_RELU .. SHDW_ACT_GELU (type 0 is shdw_hip_prelu).
+ * ref: shadow/operators/kernels/activate.cpp:9-39, activate.cu:7-45 */
+int shdw_hip_activate(int type, float slope, int n, const float* x, float* y,
+                      void* stream);
+/* y[i] = x[i] > 0 ? x[i] : x[i] * slope[c], c = (i / dim) % channels, or c = 0
+ * when channel_shared.  n = outer * channels * dim.
+ * ref: shadow/operators/kernels/activate.cpp:41-53, activate.cu:47-69 */
+int shdw_hip_prelu(int n, int channels, int dim, int channel_shared, const float* x,
+                   const float* slope, float* y, void* stream);
+
+/* ================================= Scale ================================= */
+
+/* c = (i / inner_num) % scale_num;
+ *   scale && bias : y = x * scale[c] + bias[c]   (multiply, then add)
+ *   scale only    : y = x * scale[c]
+ *   bias only     : y = x + bias[c]
+ * followed by y = y > 0 ? y : 0 when relu != 0 (the Scale -> Activate(type 1)
+ * pair in one launch; Shadow has no such fused op, parity target is the pair).
+ * ref: shadow/operators/kernels/scale.cpp:7-39, scale.cu:7-67 */
+int shdw_hip_scale_bias(int n, int scale_num, int inner_num, const float* x,
+                        const float* scale, const float* bias, int relu, float* y,
+                        void* stream);
+
+/* ================================ Eltwise ================================ */
+
+/* K >= 2 same-shape inputs, one pass.  xs is a HOST array of k device pointers,
+ * coeff a HOST array of k floats (used by SUM only, may be NULL = all ones).
+ *   PROD/MAX/MIN : acc = op(x0, x1); acc = op(acc, x_j) ...
+ *   SUM          : acc = 0; acc = acc + coeff[j] * x_j ... (each step a separate
+ *                  multiply and add, starting from +0 like Set + Saxpy)
+ * When y aliases an input the result is what Shadow's pass-by-pass evaluation
+ * gives: SUM overwrites y first, so an aliased input j reads as the running sum
+ * (acc += coeff[j] * acc); for the other ops an aliased input j >= 2 reads as acc.
+ * ref: shadow/operators/kernels/eltwise.hpp:18-71 */
+int shdw_hip_eltwise(int operation, int k, const float* const* xs, const float* coeff,
+                     int n, float* y, void* stream);
+
+/* ================================= Reduce ================================ */
+
+/* Bytes of device scratch shdw_hip_reduce needs for this shape/axes (0 when the
+ * shape runs in a single stage).  in_shape and axes are HOST arrays.
+ * Shadow sizes its temp buffer the same way before the launch:
+ * ref: shadow/operators/kernels/reduce.hpp:72-76 (GrowTempBuffer) */
+size_t shdw_hip_reduce_workspace_bytes(int num_axes, const int* in_shape, int num_reduce,
+                                       const int* axes);
+/* y[o] = reduce over the listed axes; one output per combination of the kept
+ * axes, row-major.  Axes must be distinct and in [0, num_axes).  PROD, SUM,
+ * AVG, L1, L2 accumulate in fp64 and round once; MAX/MIN return the first
+ * element (in Shadow's list order) that attains the extremum and skip NaNs,
+ * starting from lowest()/max().
+ * ref: shadow/operators/kernels/reduce.cpp:9-76, reduce.cu:7-83,
+ *      host planning shadow/operators/kernels/reduce.hpp:41-88 */
+int shdw_hip_reduce(int operation, int num_axes, const int* in_shape, int num_reduce,
+                    const int* axes, const float* x, float* y, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+/* ============================ fused sequences ============================ */
+
+/* Scale(blob form) -> Eltwise SUM with a residual -> Activate(relu) ->
+ * Reduce AVG over the trailing `inner_num` elements, in one launch:
+ *   c = row % scale_num;  s = x*scale[c] + bias[c];
+ *   y = relu((0 + 1*s) + 1*residual);  mean[row] = (float)(sum_fp64(y) / inner_num)
+ * rows = n / inner_num.  y may be NULL when only the pooled output is wanted.
+ * Shadow runs these as four operators; parity target is that sequence:
+ * ref: shadow/operators/kernels/scale.cpp:7-18, eltwise.hpp:37-44,
+ *      activate.cpp:11-12, reduce.cpp:40-46 */
+int shdw_hip_scale_residual_relu_rowmean(int n, int scale_num, int inner_num,
+                                         const float* x, const float* scale,
+                                         const float* bias, const float* residual,
+                                         float* y, float* mean, void* stream);
+
+/* ============================ plan inspection ============================ */
+
+/* Host-only: the collapsed form shdw_hip_broadcast_binary would launch with.
+ * Writes up to 8 collapsed dims (outermost first) and both stride vectors;
+ * returns the collapsed rank (0 = single element), or a negative SHDW_E_*. */
+int shdw_hip_plan_broadcast(int num_axes, const int* a_shape, const int* b_shape,
+                            const int* out_shape, int* dims, int* a_strides,
+                            int* b_strides);
+/* Host-only: how shdw_hip_reduce would run.  kind: 0 = rows (contiguous axis),
+ * 1 = strided axis, 2 = generic N-d.  outer/reduce/inner are the collapsed
+ * extents (generic: outer = outputs, reduce = window size, inner = 0);
+ * splits = number of first-stage slices of the reduce extent. */
+int shdw_hip_plan_reduce(int num_axes, const int* in_shape, int num_reduce,
+                         const int* axes, int* kind, int* outer, int* reduce,
+                         int* inner, int* splits);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* SHADOW_HIP_H_ */

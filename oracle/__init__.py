@@ -1,0 +1,284 @@
+"""TEST INFRASTRUCTURE -- NOT PART OF THE PRODUCT.
+
+Python face of the CPU oracle: ctypes bindings to ``liboracle.so`` (the C
+restatement in ``shadow_cpu.c``) plus the operator-level shape rules of the
+reference's ``*_op.cpp`` files.  Only ``tests/``, ``__graft_entry__.smoke()`` and
+the ``cpu_baseline`` leg of ``bench.py`` may import this package.
+
+Errors that the reference raises through ``CHECK`` (a thrown
+``std::runtime_error``) are raised here as :class:`OracleCheckError`.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+_f32p = ctypes.POINTER(ctypes.c_float)
+_i32p = ctypes.POINTER(ctypes.c_int)
+
+
+class OracleCheckError(RuntimeError):
+    """A condition the reference guards with CHECK/LOG(FATAL) failed."""
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        path = os.path.join(_HERE, "liboracle.so")
+        if not os.path.exists(path):
+            raise RuntimeError("oracle/liboracle.so is not built; run `python -m shadow_amd.build oracle`")
+        _LIB = ctypes.CDLL(path)
+        _LIB.orc_asum.restype = ctypes.c_float
+    return _LIB
+
+
+def _f(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _p(a):
+    return a.ctypes.data_as(_f32p)
+
+
+def _ints(v):
+    arr = (ctypes.c_int * max(1, len(v)))(*[int(x) for x in v])
+    return arr
+
+
+def _check(cond, msg):
+    if not cond:
+        raise OracleCheckError("Check Failed: " + msg)
+
+
+# --------------------------------------------------------------------------
+# kernel level (flat arrays)
+# --------------------------------------------------------------------------
+def blas_set(n, val):
+    y = np.empty(n, np.float32)
+    lib().orc_set(n, ctypes.c_float(val), _p(y))
+    return y
+
+
+def unary(op, a):
+    a = _f(a)
+    y = np.empty_like(a)
+    _check(lib().orc_unary(int(op), a.size, _p(a), _p(y)) == 0, "unary operation")
+    return y
+
+
+def binary(op, a, b):
+    a, b = _f(a), _f(b)
+    assert a.size == b.size
+    y = np.empty_like(a)
+    _check(lib().orc_binary(int(op), a.size, _p(a), _p(b), _p(y)) == 0, "binary operation")
+    return y
+
+
+def binary_scalar(op, a, alpha):
+    a = _f(a)
+    y = np.empty_like(a)
+    _check(lib().orc_binary_scalar(int(op), a.size, _p(a), ctypes.c_float(alpha), _p(y)) == 0,
+           "binary operation")
+    return y
+
+
+def scal(alpha, x):
+    x = _f(x).copy()
+    lib().orc_scal(x.size, ctypes.c_float(alpha), _p(x))
+    return x
+
+
+def copy(x):
+    x = _f(x)
+    y = np.empty_like(x)
+    lib().orc_copy(x.size, _p(x), _p(y))
+    return y
+
+
+def axpy(alpha, x, y):
+    x, y = _f(x), _f(y).copy()
+    lib().orc_axpy(x.size, ctypes.c_float(alpha), _p(x), _p(y))
+    return y
+
+
+def asum(x):
+    x = _f(x)
+    return np.float32(lib().orc_asum(x.size, _p(x)))
+
+
+def broadcast_binary(op, a, a_shape, b, b_shape, out_shape):
+    """a_shape / b_shape / out_shape are rank-aligned lists."""
+    a, b = _f(a), _f(b)
+    count = int(np.prod(out_shape, dtype=np.int64))
+    out = np.empty(count, np.float32)
+    rc = lib().orc_broadcast_binary(_p(a), _ints(a_shape), _p(b), _ints(b_shape), int(op),
+                                    len(out_shape), count, _ints(out_shape), _p(out))
+    _check(rc == 0, "broadcast binary arguments")
+    return out
+
+
+def activate(x, act_type, slope=0.1):
+    x = _f(x)
+    y = np.empty_like(x)
+    lib().orc_activate(_p(x), _p(y), x.size, int(act_type), ctypes.c_float(slope))
+    return y
+
+
+def prelu(x, shape, channel_shared, slope):
+    x, slope = _f(x), _f(slope)
+    y = np.empty_like(x)
+    lib().orc_prelu(_p(x), _p(y), _ints(shape), len(shape), int(bool(channel_shared)), _p(slope))
+    return y
+
+
+def scale_bias(x, scale, bias, scale_num, inner_num):
+    x = _f(x)
+    y = np.empty_like(x)
+    if scale is not None and bias is not None:
+        scale, bias = _f(scale), _f(bias)
+        lib().orc_scale_bias(_p(x), x.size, _p(scale), _p(bias), scale_num, inner_num, _p(y))
+    elif scale is not None:
+        scale = _f(scale)
+        lib().orc_scale(_p(x), x.size, _p(scale), scale_num, inner_num, _p(y))
+    else:
+        bias = _f(bias)
+        lib().orc_bias(_p(x), x.size, _p(bias), scale_num, inner_num, _p(y))
+    return y
+
+
+def eltwise(op, inputs, coeff=None, out=None):
+    """`out` may be one of the input arrays to model aliasing."""
+    inputs = [x if x.dtype == np.float32 and x.flags.c_contiguous else _f(x) for x in inputs]
+    k = len(inputs)
+    n = inputs[0].size
+    if out is None:
+        out = np.empty(n, np.float32)
+    ptrs = (_f32p * k)(*[_p(x) for x in inputs])
+    co = _f(coeff if coeff is not None else np.ones(k))
+    _check(lib().orc_eltwise(int(op), k, ptrs, _p(co), n, _p(out)) == 0, "eltwise arguments")
+    return out
+
+
+def reduce(op, x, shape, axes):
+    x = _f(x)
+    out_shape = list(shape)
+    for ax in axes:
+        out_shape[ax] = 1
+    out = np.empty(int(np.prod(out_shape, dtype=np.int64)), np.float32)
+    rc = lib().orc_reduce(int(op), _p(x), _ints(shape), len(shape), _ints(axes), len(axes), _p(out))
+    _check(rc == 0, "reduce arguments")
+    return out, out_shape
+
+
+# --------------------------------------------------------------------------
+# operator level: argument checks and shape rules of shadow/operators/*_op.cpp
+# --------------------------------------------------------------------------
+def unary_op(x, operation):
+    """shadow/operators/unary_op.cpp:9-28"""
+    _check(0 <= operation <= 14, "operation_ in [0, 14]")
+    x = _f(x)
+    return unary(operation, x.ravel()).reshape(x.shape)
+
+
+def binary_op(a, b=None, operation=-1, scalar=None):
+    """shadow/operators/binary_op.cpp:9-65; `scalar` given selects the one-input form."""
+    _check(0 <= operation <= 6, "operation_ in [0, 6]")
+    a = _f(a)
+    if scalar is not None:
+        _check(b is None, "inputs.size() == 1")
+        return binary_scalar(operation, a.ravel(), scalar).reshape(a.shape)
+    _check(b is not None, "inputs.size() == 2")
+    b = _f(b)
+    if a.shape == b.shape:
+        return binary(operation, a.ravel(), b.ravel()).reshape(a.shape)
+    sa, sb = list(a.shape), list(b.shape)
+    diff = len(sa) - len(sb)
+    if diff > 0:
+        sb = [1] * diff + sb
+    elif diff < 0:
+        sa = [1] * (-diff) + sa
+    out_shape = []
+    for da, db in zip(sa, sb):
+        _check(da == db or da == 1 or db == 1, "in_dim == scalar_dim || in_dim == 1 || scalar_dim == 1")
+        out_shape.append(max(da, db))
+    out = broadcast_binary(operation, a.ravel(), sa, b.ravel(), sb, out_shape)
+    return out.reshape(out_shape)
+
+
+def eltwise_op(inputs, operation, coeff=()):
+    """shadow/operators/eltwise_op.cpp:9-47"""
+    _check(0 <= operation <= 3, "operation_ in [0, 3]")
+    _check(len(inputs) >= 2, "inputs.size() >= 2")
+    inputs = [_f(x) for x in inputs]
+    for x in inputs[1:]:
+        _check(x.shape == inputs[0].shape, "inputs[n]->shape() == input_0->shape()")
+    coeff = list(coeff)
+    _check(len(coeff) == 0 or len(coeff) == len(inputs), "one coefficient per input blob")
+    _check(not (operation != 1 and len(coeff)), "coefficients only for summation")
+    full = [1.0] * len(inputs)
+    full[:len(coeff)] = coeff
+    return eltwise(operation, [x.ravel() for x in inputs], full).reshape(inputs[0].shape)
+
+
+def reduce_op(x, operation=0, axes=(), keep_dims=True):
+    """shadow/operators/reduce_op.cpp:9-65 (non-negative, distinct axes only: the
+    reference indexes its stride table with the raw axis value)."""
+    _check(0 <= operation <= 6, "operation_ in [0, 6]")
+    x = _f(x)
+    axes = list(axes)
+    if not axes:
+        axes = list(range(x.ndim))
+    for ax in axes:
+        _check(0 <= ax < x.ndim, "axis in range")
+    out, out_shape = reduce(operation, x.ravel(), list(x.shape), axes)
+    if not keep_dims:
+        out_shape = [d for n, d in enumerate(out_shape) if n not in axes]
+    return out.reshape(out_shape)
+
+
+def activate_op(x, act_type=1, slope=0.1, slope_blob=None):
+    """shadow/operators/activate_op.cpp:9-34 and kernels/activate.hpp:44-74"""
+    _check(0 <= act_type <= 8, "activate_type_ in [0, 8]")
+    x = _f(x)
+    if act_type == 0:
+        _check(slope_blob is not None, "inputs.size() == 2")
+        _check(x.ndim >= 2, "input->num_axes() >= 2")
+        slope_blob = _f(slope_blob)
+        shared = slope_blob.size == 1
+        if not shared:
+            _check(slope_blob.size == x.shape[1], "slope->count() == input->shape(1)")
+        return prelu(x.ravel(), list(x.shape), shared, slope_blob.ravel()).reshape(x.shape)
+    _check(slope_blob is None, "inputs.size() == 1")
+    return activate(x.ravel(), act_type, slope).reshape(x.shape)
+
+
+def scale_op(x, axis=1, scale=None, bias=None, scale_value=(), bias_value=()):
+    """shadow/operators/scale_op.cpp:9-52 and kernels/scale.hpp:44-110.
+    Blob form when `scale`/`bias` arrays are given, value form otherwise."""
+    x = _f(x)
+    count = lambda start: int(np.prod(x.shape[start:], dtype=np.int64))
+    if scale is not None or bias is not None:
+        ref = _f(scale if scale is not None else bias)
+        if scale is not None and bias is not None:
+            _check(np.shape(scale) == np.shape(bias), "scale->shape() == bias->shape()")
+        inner = count(axis + ref.ndim)
+        out = scale_bias(x.ravel(), None if scale is None else _f(scale).ravel(),
+                         None if bias is None else _f(bias).ravel(), ref.size, inner)
+        return out.reshape(x.shape)
+    dim = x.shape[axis]
+    sv, bv = list(scale_value), list(bias_value)
+    if len(sv) > 1:
+        _check(len(sv) == dim, "scale_value_.size() == dim")
+    elif len(sv) == 1:
+        sv = sv * dim
+    if len(bv) > 1:
+        _check(len(bv) == dim, "bias_value_.size() == dim")
+    elif len(bv) == 1:
+        bv = bv * dim
+    _check(sv or bv, "!scale_value.empty() || !bias_value.empty()")
+    out = scale_bias(x.ravel(), np.float32(sv) if sv else None, np.float32(bv) if bv else None,
+                     dim, count(axis + 1))
+    return out.reshape(x.shape)

@@ -1,0 +1,302 @@
+/*
+ * TEST INFRASTRUCTURE -- NOT PART OF THE PRODUCT.
+ *
+ * CPU restatement, in plain C, of the loops that junluan/shadow runs on the host
+ * for its Unary / Binary / Eltwise / Reduce / Activate / Scale operators when
+ * built without Eigen/BLAS/DNNL (the "plain loop + libm" branch).  It is the
+ * checker for the HIP kernels and the CPU leg of the benchmark; nothing under
+ * shadow_amd/ may call it.
+ *
+ * Every function names the reference lines it follows.  Built with the
+ * reference's Release flags (-O3 -DNDEBUG, no -march, no fast-math) plus
+ * -ffp-contract=off.  Transcendentals are the host's libm, as in the reference.
+ *
+ * Pinning (see tests/test_oracle_*.py): IEEE closed forms against numpy fp32,
+ * brute-force N-d broadcast and reduce written independently in numpy, exact
+ * integer-valued sums, signed-zero / NaN special cases, libm results against
+ * fp64 evaluations within 1 ulp.  The reference holds no test vectors for this
+ * path and its own build needs a cmake-generated header, so no compiled
+ * reference backs these checks.
+ */
+#include <float.h>
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define API __attribute__((visibility("default")))
+
+/* std::max / std::min as libstdc++ defines them */
+static inline float std_max(float a, float b) { return (a < b) ? b : a; }
+static inline float std_min(float a, float b) { return (b < a) ? b : a; }
+
+/* ---- shadow/core/blas.cpp:25-34  Blas::Set ---- */
+API void orc_set(int n, float val, float* y) {
+  for (int i = 0; i < n; ++i) y[i] = val;
+}
+
+/* ---- shadow/core/blas.cpp:143-168  15 unary ops (loop branch);
+ *      enum values shadow/operators/kernels/unary.hpp:9-25 ---- */
+API int orc_unary(int op, int n, const float* a, float* y) {
+  switch (op) {
+    case 0: for (int i = 0; i < n; ++i) y[i] = fabsf(a[i]); break;
+    case 1: for (int i = 0; i < n; ++i) y[i] = a[i] * a[i]; break;
+    case 2: for (int i = 0; i < n; ++i) y[i] = sqrtf(a[i]); break;
+    case 3: for (int i = 0; i < n; ++i) y[i] = logf(a[i]); break;
+    case 4: for (int i = 0; i < n; ++i) y[i] = expf(a[i]); break;
+    case 5: for (int i = 0; i < n; ++i) y[i] = sinf(a[i]); break;
+    case 6: for (int i = 0; i < n; ++i) y[i] = cosf(a[i]); break;
+    case 7: for (int i = 0; i < n; ++i) y[i] = tanf(a[i]); break;
+    case 8: for (int i = 0; i < n; ++i) y[i] = asinf(a[i]); break;
+    case 9: for (int i = 0; i < n; ++i) y[i] = acosf(a[i]); break;
+    case 10: for (int i = 0; i < n; ++i) y[i] = atanf(a[i]); break;
+    case 11: for (int i = 0; i < n; ++i) y[i] = floorf(a[i]); break;
+    case 12: for (int i = 0; i < n; ++i) y[i] = ceilf(a[i]); break;
+    case 13: for (int i = 0; i < n; ++i) y[i] = -a[i]; break;
+    case 14: for (int i = 0; i < n; ++i) y[i] = 1 / a[i]; break;
+    default: return -1;
+  }
+  return 0;
+}
+
+/* one binary op on two values: shadow/core/blas.cpp:114-120 and
+ * shadow/operators/kernels/binary.cpp:9-28; enum binary.hpp:23 */
+static inline float binary_one(float a, float b, int op) {
+  switch (op) {
+    case 0: return a + b;
+    case 1: return a - b;
+    case 2: return a * b;
+    case 3: return a / b;
+    case 4: return powf(a, b);
+    case 5: return std_max(a, b);
+    case 6: return std_min(a, b);
+    default: return 0;
+  }
+}
+
+/* ---- shadow/core/blas.cpp:103-121  tensor (op) tensor ---- */
+API int orc_binary(int op, int n, const float* a, const float* b, float* y) {
+  if (op < 0 || op > 6) return -1;
+  for (int i = 0; i < n; ++i) y[i] = binary_one(a[i], b[i], op);
+  return 0;
+}
+
+/* ---- shadow/core/blas.cpp:123-141  tensor (op) scalar ---- */
+API int orc_binary_scalar(int op, int n, const float* a, float alpha, float* y) {
+  if (op < 0 || op > 6) return -1;
+  for (int i = 0; i < n; ++i) y[i] = binary_one(a[i], alpha, op);
+  return 0;
+}
+
+/* ---- shadow/core/blas.cpp:172-235  level 1 (loop branch) ---- */
+API void orc_scal(int n, float alpha, float* x) {
+  for (int i = 0; i < n; ++i) x[i] *= alpha;
+}
+API void orc_copy(int n, const float* x, float* y) {
+  for (int i = 0; i < n; ++i) y[i] = x[i];
+}
+API void orc_axpy(int n, float alpha, const float* x, float* y) {
+  for (int i = 0; i < n; ++i) y[i] += alpha * x[i];
+}
+API float orc_asum(int n, const float* x) {
+  double asum = 0;
+  for (int i = 0; i < n; ++i) asum += fabsf(x[i]);
+  return (float)asum;
+}
+
+/* ---- shadow/operators/kernels/binary.cpp:30-52  Vision::BroadcastBinary ----
+ * shapes are rank-aligned; broadcasting is the "% shape" on each operand. */
+API int orc_broadcast_binary(const float* in, const int* in_shape, const float* sc,
+                             const int* sc_shape, int op, int num_axes, int count,
+                             const int* out_shape, float* out) {
+  if (op < 0 || op > 6 || num_axes < 1) return -1;
+  int* in_acc = (int*)malloc(sizeof(int) * num_axes);
+  int* sc_acc = (int*)malloc(sizeof(int) * num_axes);
+  in_acc[num_axes - 1] = 1;
+  sc_acc[num_axes - 1] = 1;
+  for (int n = num_axes - 1; n > 0; --n) {
+    in_acc[n - 1] = in_shape[n] * in_acc[n];
+    sc_acc[n - 1] = sc_shape[n] * sc_acc[n];
+  }
+  for (int i = 0; i < count; ++i) {
+    int in_index = 0, sc_index = 0, cc = i;
+    for (int n = num_axes - 1; n >= 0; --n) {
+      int dim = cc % out_shape[n];
+      in_index += (dim % in_shape[n]) * in_acc[n];
+      sc_index += (dim % sc_shape[n]) * sc_acc[n];
+      cc /= out_shape[n];
+    }
+    out[i] = binary_one(in[in_index], sc[sc_index], op);
+  }
+  free(in_acc);
+  free(sc_acc);
+  return 0;
+}
+
+/* ---- shadow/operators/kernels/activate.cpp:9-39  Vision::Activate ----
+ * enum shadow/operators/kernels/activate.hpp:24-34 (0 = PRelu, see below) */
+static inline float activate_one(float x, int type, float slope) {
+  switch (type) {
+    case 1: return x > 0 ? x : 0;
+    case 2: return x > 0 ? x : slope * x;
+    case 3: return 1 / (1 + expf(-x));
+    case 4: return log1pf(expf(x));
+    case 5: return tanhf(x);
+    case 6: return x < 0 ? 0 : (x > 6 ? 6 : x);
+    case 7: return x < -3 ? 0 : (x > 3 ? x : (x * (x + 3) / 6.f));
+    case 8: return 0.5f * x * (1 + erff(0.707107f * x));
+    default: return x;
+  }
+}
+API void orc_activate(const float* in, float* out, int count, int type, float slope) {
+  for (int i = 0; i < count; ++i) out[i] = activate_one(in[i], type, slope);
+}
+
+/* ---- shadow/operators/kernels/activate.cpp:41-53  Vision::PRelu ---- */
+API void orc_prelu(const float* in, float* out, const int* in_shape, int num_axes,
+                   int channel_shared, const float* slope) {
+  int channels = in_shape[1], dim = 1;
+  for (int i = 2; i < num_axes; ++i) dim *= in_shape[i];
+  int count = in_shape[0] * channels * dim;
+  int div_factor = channel_shared ? channels : 1;
+  for (int i = 0; i < count; ++i) {
+    int c = (i / dim) % channels / div_factor;
+    out[i] = in[i] > 0 ? in[i] : in[i] * slope[c];
+  }
+}
+
+/* ---- shadow/operators/kernels/scale.cpp:7-39 ---- */
+API void orc_scale_bias(const float* in, int count, const float* scale, const float* bias,
+                        int scale_num, int inner_num, float* out) {
+  for (int i = 0; i < count; ++i) {
+    int index = (i / inner_num) % scale_num;
+    out[i] = in[i] * scale[index] + bias[index];
+  }
+}
+API void orc_scale(const float* in, int count, const float* scale, int scale_num,
+                   int inner_num, float* out) {
+  for (int i = 0; i < count; ++i) {
+    int index = (i / inner_num) % scale_num;
+    out[i] = in[i] * scale[index];
+  }
+}
+API void orc_bias(const float* in, int count, const float* bias, int scale_num, int inner_num,
+                  float* out) {
+  for (int i = 0; i < count; ++i) {
+    int index = (i / inner_num) % scale_num;
+    out[i] = in[i] + bias[index];
+  }
+}
+
+/* ---- shadow/operators/kernels/eltwise.hpp:18-71  EltwiseKernelDefault::Run ----
+ * enum eltwise.hpp:9: 0 Prod, 1 Sum, 2 Max, 3 Min.  Written as the same chain
+ * of whole-array passes, so aliasing out with an input behaves as it does there. */
+API int orc_eltwise(int op, int k, const float* const* in, const float* coeff, int count,
+                    float* out) {
+  if (k < 2) return -1;
+  switch (op) {
+    case 0:
+      orc_binary(2, count, in[0], in[1], out);
+      for (int n = 2; n < k; ++n) orc_binary(2, count, out, in[n], out);
+      break;
+    case 1:
+      orc_set(count, 0, out);
+      for (int n = 0; n < k; ++n) orc_axpy(count, coeff[n], in[n], out);
+      break;
+    case 2:
+      orc_binary(5, count, in[0], in[1], out);
+      for (int n = 2; n < k; ++n) orc_binary(5, count, out, in[n], out);
+      break;
+    case 3:
+      orc_binary(6, count, in[0], in[1], out);
+      for (int n = 2; n < k; ++n) orc_binary(6, count, out, in[n], out);
+      break;
+    default:
+      return -1;
+  }
+  return 0;
+}
+
+/* ---- shadow/operators/kernels/reduce.cpp:9-65  inline Reduce() ---- */
+static float reduce_one(const float* data, const int* list, int num_list, int offset, int op) {
+  switch (op) {
+    case 0: {
+      double val = 1;
+      for (int i = 0; i < num_list; ++i) val *= data[list[i] + offset];
+      return (float)val;
+    }
+    case 1: {
+      double val = 0;
+      for (int i = 0; i < num_list; ++i) val += data[list[i] + offset];
+      return (float)val;
+    }
+    case 2: {
+      float val = -FLT_MAX; /* numeric_limits<float>::lowest() */
+      for (int i = 0; i < num_list; ++i) val = std_max(val, data[list[i] + offset]);
+      return val;
+    }
+    case 3: {
+      float val = FLT_MAX;
+      for (int i = 0; i < num_list; ++i) val = std_min(val, data[list[i] + offset]);
+      return val;
+    }
+    case 4: {
+      double val = 0;
+      for (int i = 0; i < num_list; ++i) val += data[list[i] + offset];
+      return (float)(val / num_list);
+    }
+    case 5: {
+      double val = 0;
+      for (int i = 0; i < num_list; ++i) val += fabsf(data[list[i] + offset]);
+      return (float)val;
+    }
+    case 6: {
+      double val = 0;
+      for (int i = 0; i < num_list; ++i) {
+        float abs_data = fabsf(data[list[i] + offset]);
+        val += abs_data * abs_data; /* fp32 product, widened afterwards */
+      }
+      return sqrtf((float)val);
+    }
+    default:
+      return 0;
+  }
+}
+
+/* ---- shadow/operators/kernels/reduce.hpp:41-88  list/offset planning, then
+ *      shadow/operators/kernels/reduce.cpp:67-76  Vision::Reduce ----
+ * out_shape = in_shape with the reduced axes set to 1 (reduce_op.cpp:38-42). */
+API int orc_reduce(int op, const float* in, const int* in_shape, int num_axes, const int* axes,
+                   int num_reduce, float* out) {
+  if (op < 0 || op > 6) return -1;
+  int shape_acc[16], out_shape[16];
+  if (num_axes > 16) return -1;
+  if (num_axes > 0) shape_acc[num_axes - 1] = 1;
+  for (int n = num_axes - 1; n > 0; --n) shape_acc[n - 1] = in_shape[n] * shape_acc[n];
+  int out_count = 1;
+  for (int n = 0; n < num_axes; ++n) out_shape[n] = in_shape[n];
+  for (int k = 0; k < num_reduce; ++k) out_shape[axes[k]] = 1;
+  for (int n = 0; n < num_axes; ++n) out_count *= out_shape[n];
+
+  /* list: offsets inside one window, last listed axis fastest */
+  size_t cap = 1;
+  for (int k = 0; k < num_reduce; ++k) cap *= (size_t)in_shape[axes[k]];
+  int* list = (int*)malloc(sizeof(int) * cap);
+  int num_list = 1;
+  list[0] = 0;
+  for (int n = num_reduce - 1; n >= 0; --n) {
+    int axis = axes[n], cur = num_list;
+    for (int k = 1; k < in_shape[axis]; ++k)
+      for (int j = 0; j < cur; ++j) list[num_list++] = list[j] + k * shape_acc[axis];
+  }
+  for (int i = 0; i < out_count; ++i) {
+    int offset = 0, cc = i;
+    for (int n = num_axes - 1; n >= 0; --n) {
+      int dim = out_shape[n];
+      offset += (cc % dim) * shape_acc[n];
+      cc /= dim;
+    }
+    out[i] = reduce_one(in, list, num_list, offset, op);
+  }
+  free(list);
+  return 0;
+}

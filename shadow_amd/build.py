@@ -1,0 +1,107 @@
+"""Build every native piece of the repository in-tree.
+
+    python -m shadow_amd.build            # everything
+    python -m shadow_amd.build hip host   # selected targets
+
+Targets
+    hip     shadow_amd/lib/libshadow_hip.so   gfx950 kernels + C ABI (hipcc)
+    host    shadow_amd/lib/libshadow_host.so  C++ operator layer over the C ABI (g++)
+    oracle  oracle/liboracle.so               CPU restatement of the reference (gcc)
+    sweep   tests/native/libm_sweep.so        host build of the device libm code (g++)
+
+hipcc cross-compiles for gfx950 without a GPU.  The device code must keep
+multiply and add separate (the reference never fuses), hence -ffp-contract=off;
+packed fp32 instructions are disabled for every HIP translation unit.
+"""
+import concurrent.futures
+import os
+import shutil
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "shadow_amd", "csrc")
+HOST = os.path.join(ROOT, "shadow_amd", "host")
+LIB = os.path.join(ROOT, "shadow_amd", "lib")
+OBJ = os.path.join(LIB, "obj")
+
+HIPCC = os.environ.get("HIPCC", shutil.which("hipcc") or "/opt/rocm/bin/hipcc")
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+HIP_SOURCES = ["elementwise.hip", "broadcast.hip", "reduce.hip", "fused.hip", "runtime.hip"]
+# The reference's Release flags (CMakeLists.txt:30-37) plus contraction off so
+# that no host can fuse what baseline x86-64 does not.
+ORACLE_FLAGS = ["-O3", "-DNDEBUG", "-fPIC", "-ffp-contract=off", "-fno-fast-math"]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def build_hip():
+    os.makedirs(OBJ, exist_ok=True)
+    objs = []
+    jobs = []
+    with concurrent.futures.ThreadPoolExecutor(max_workers=6) as pool:
+        for src in HIP_SOURCES:
+            obj = os.path.join(OBJ, src.replace(".hip", ".o"))
+            objs.append(obj)
+            jobs.append(pool.submit(_run, [HIPCC] + HIP_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]))
+        plan_obj = os.path.join(OBJ, "plan.o")
+        objs.append(plan_obj)
+        jobs.append(pool.submit(_run, ["g++", "-O2", "-std=c++17", "-fPIC", "-c",
+                                       os.path.join(CSRC, "plan.cpp"), "-o", plan_obj]))
+        for j in jobs:
+            j.result()
+    out = os.path.join(LIB, "libshadow_hip.so")
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", out])
+    return out
+
+
+def build_host():
+    srcs = sorted(
+        os.path.join(dp, f) for dp, _, fs in os.walk(HOST) for f in fs if f.endswith(".cpp"))
+    if not srcs:
+        return None
+    out = os.path.join(LIB, "libshadow_host.so")
+    _run(["g++", "-O2", "-std=c++14", "-fPIC", "-shared", "-I", HOST, "-I", os.path.join(ROOT, "include")]
+         + srcs + ["-L", LIB, "-lshadow_hip", "-Wl,-rpath,$ORIGIN", "-o", out])
+    return out
+
+
+def build_oracle():
+    src = os.path.join(ROOT, "oracle", "shadow_cpu.c")
+    out = os.path.join(ROOT, "oracle", "liboracle.so")
+    _run(["gcc", "-std=c11"] + ORACLE_FLAGS + ["-shared", src, "-lm", "-o", out])
+    return out
+
+
+def build_sweep():
+    src = os.path.join(ROOT, "tests", "native", "libm_sweep.cpp")
+    out = os.path.join(ROOT, "tests", "native", "libm_sweep.so")
+    _run(["g++", "-std=c++17", "-O2", "-ffp-contract=off", "-fPIC", "-shared", "-pthread", src, "-o", out])
+    return out
+
+
+TARGETS = {"hip": build_hip, "host": build_host, "oracle": build_oracle, "sweep": build_sweep}
+
+
+def build_all(names=None):
+    built = []
+    for name in (names or ["hip", "host", "oracle", "sweep"]):
+        path = TARGETS[name]()
+        if path:
+            built.append(path)
+    return built
+
+
+if __name__ == "__main__":
+    for p in build_all(sys.argv[1:] or None):
+        print("built", os.path.relpath(p, ROOT))

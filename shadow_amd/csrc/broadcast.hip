@@ -1,0 +1,329 @@
+// Kernels whose second operand is indexed, not streamed:
+//   * per-row parameters (Scale / Bias / ScaleBias with an optional ReLU
+//     epilogue, PRelu): x is rows of `inner` contiguous elements and the
+//     parameter index is row % num;
+//   * numpy-style broadcast Binary on host-collapsed dims.
+// Index arithmetic is done once per 128-bit vector with multiply-high division
+// by launch-time constants; there is no per-element div/mod and no device-side
+// shape table.
+#include <hip/hip_runtime.h>
+
+#include "../../include/shadow_hip.h"
+#include "device_common.h"
+#include "functors.h"
+#include "launch.h"
+#include "plan.h"
+
+#pragma clang fp contract(off)
+
+namespace shdw {
+
+constexpr int kRowUnroll = 4;
+
+enum RowMode { kScaleBias = 0, kScaleOnly = 1, kBiasOnly = 2, kPRelu = 3 };
+
+template <int MODE, bool RELU>
+SHDW_DEVICE float row_apply(float x, float s, float b) {
+  float r;
+  if (MODE == kScaleBias) {
+    const float t = x * s;
+    r = t + b;
+  } else if (MODE == kScaleOnly) {
+    r = x * s;
+  } else if (MODE == kBiasOnly) {
+    r = x + b;
+  } else {
+    r = x > 0 ? x : x * s;
+  }
+  if (RELU) r = r > 0 ? r : 0;
+  return r;
+}
+
+// ROWVEC: inner % 4 == 0, so the four lanes of a vector share one row.
+template <int MODE, bool RELU, bool ROWVEC>
+__global__ __launch_bounds__(kBlock) void rowparam_vec_kernel(const float* x, const float* s,
+                                                               const float* b, float* y,
+                                                               uint32_t n4, uint32_t n,
+                                                               FastDiv inner, FastDiv num) {
+  const uint32_t span = kBlock * kRowUnroll;
+  const uint32_t stride = gridDim.x * span;
+  for (uint32_t base = blockIdx.x * span; base < n4; base += stride) {
+    v4f vx[kRowUnroll];
+#pragma unroll
+    for (int u = 0; u < kRowUnroll; ++u) {
+      const uint32_t i = base + u * kBlock + threadIdx.x;
+      if (i < n4) vx[u] = load4_stream(x + 4ull * i);
+    }
+#pragma unroll
+    for (int u = 0; u < kRowUnroll; ++u) {
+      const uint32_t i = base + u * kBlock + threadIdx.x;
+      if (i < n4) {
+        v4f r;
+        if (ROWVEC) {
+          uint32_t row, c;
+          row = fd_div(4 * i, inner);
+          c = row - fd_div(row, num) * num.d;
+          const float sv = (MODE != kBiasOnly) ? s[c] : 0.f;
+          const float bv = (MODE == kScaleBias || MODE == kBiasOnly) ? b[c] : 0.f;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) r[j] = row_apply<MODE, RELU>(vx[u][j], sv, bv);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const uint32_t row = fd_div(4 * i + j, inner);
+            const uint32_t c = row - fd_div(row, num) * num.d;
+            const float sv = (MODE != kBiasOnly) ? s[c] : 0.f;
+            const float bv = (MODE == kScaleBias || MODE == kBiasOnly) ? b[c] : 0.f;
+            r[j] = row_apply<MODE, RELU>(vx[u][j], sv, bv);
+          }
+        }
+        store4_stream(y + 4ull * i, r);
+      }
+    }
+  }
+  if (blockIdx.x == 0) {
+    const uint32_t i = 4 * n4 + threadIdx.x;
+    if (i < n) {
+      const uint32_t row = fd_div(i, inner);
+      const uint32_t c = row - fd_div(row, num) * num.d;
+      const float sv = (MODE != kBiasOnly) ? s[c] : 0.f;
+      const float bv = (MODE == kScaleBias || MODE == kBiasOnly) ? b[c] : 0.f;
+      y[i] = row_apply<MODE, RELU>(x[i], sv, bv);
+    }
+  }
+}
+
+template <int MODE, bool RELU>
+__global__ __launch_bounds__(kBlock) void rowparam_scalar_kernel(const float* x, const float* s,
+                                                                  const float* b, float* y,
+                                                                  uint32_t n, FastDiv inner,
+                                                                  FastDiv num) {
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+    const uint32_t row = fd_div(i, inner);
+    const uint32_t c = row - fd_div(row, num) * num.d;
+    const float sv = (MODE != kBiasOnly) ? s[c] : 0.f;
+    const float bv = (MODE == kScaleBias || MODE == kBiasOnly) ? b[c] : 0.f;
+    y[i] = row_apply<MODE, RELU>(x[i], sv, bv);
+  }
+}
+
+template <int MODE, bool RELU>
+static int launch_rowparam(int n, int num, int inner, const float* x, const float* s,
+                           const float* b, float* y, hipStream_t st) {
+  const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner));
+  const FastDiv fn = make_fastdiv(static_cast<uint32_t>(num));
+  if (aligned16(x) && aligned16(y)) {
+    const uint32_t n4 = static_cast<uint32_t>(n) / 4;
+    const uint32_t span = kBlock * kRowUnroll;
+    uint32_t grid = (n4 + span - 1) / span;
+    grid = grid < 1 ? 1 : (grid > kMaxStreamGrid ? kMaxStreamGrid : grid);
+    if (inner % 4 == 0)
+      rowparam_vec_kernel<MODE, RELU, true><<<grid, kBlock, 0, st>>>(x, s, b, y, n4, n, fi, fn);
+    else
+      rowparam_vec_kernel<MODE, RELU, false><<<grid, kBlock, 0, st>>>(x, s, b, y, n4, n, fi, fn);
+  } else {
+    uint32_t grid = (static_cast<uint32_t>(n) + kBlock - 1) / kBlock;
+    grid = grid > kMaxStreamGrid * 4 ? kMaxStreamGrid * 4 : grid;
+    rowparam_scalar_kernel<MODE, RELU><<<grid, kBlock, 0, st>>>(x, s, b, y, n, fi, fn);
+  }
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// Broadcast binary on collapsed dims.
+// ---------------------------------------------------------------------------
+struct BcastArgs {
+  FastDiv fd[4];  // divisors for dims 1..NDIM-1 are used (dim 0 is the quotient)
+  int sa[4];
+  int sb[4];
+  int a_full;  // a is not broadcast anywhere: stream it
+  int b_full;
+};
+
+// Each lane owns 4 consecutive outputs of the innermost collapsed dim, whose
+// extent is a multiple of 4.  AVEC/BVEC: the operand's innermost stride is 1
+// (128-bit load) rather than 0 (one scalar, replicated).
+template <class F, int NDIM, bool AVEC, bool BVEC>
+__global__ __launch_bounds__(kBlock) void bcast_vec_kernel(F f, BcastArgs p, const float* a,
+                                                            const float* b, float* y,
+                                                            uint32_t n4) {
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n4; i += stride) {
+    uint32_t e = 4 * i;
+    uint32_t oa = 0, ob = 0;
+#pragma unroll
+    for (int k = NDIM - 1; k >= 1; --k) {
+      uint32_t q, r;
+      fd_divmod(e, p.fd[k], q, r);
+      oa += r * static_cast<uint32_t>(p.sa[k]);
+      ob += r * static_cast<uint32_t>(p.sb[k]);
+      e = q;
+    }
+    oa += e * static_cast<uint32_t>(p.sa[0]);
+    ob += e * static_cast<uint32_t>(p.sb[0]);
+    v4f va, vb;
+    if (AVEC) {
+      va = p.a_full ? load4_stream(a + oa) : load4(a + oa);
+    } else {
+      const float t = a[oa];
+      va = {t, t, t, t};
+    }
+    if (BVEC) {
+      vb = p.b_full ? load4_stream(b + ob) : load4(b + ob);
+    } else {
+      const float t = b[ob];
+      vb = {t, t, t, t};
+    }
+    v4f r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = f(va[j], vb[j]);
+    store4_stream(y + 4ull * i, r);
+  }
+}
+
+struct BcastGenericArgs {
+  int ndim;
+  FastDiv fd[kMaxDims];
+  int sa[kMaxDims];
+  int sb[kMaxDims];
+};
+
+// Any rank up to 8, any extents, one output per lane.
+template <class F>
+__global__ __launch_bounds__(kBlock) void bcast_generic_kernel(F f, BcastGenericArgs p,
+                                                                const float* a, const float* b,
+                                                                float* y, uint32_t n) {
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+    uint32_t e = i, oa = 0, ob = 0;
+    for (int k = p.ndim - 1; k >= 1; --k) {
+      uint32_t q, r;
+      fd_divmod(e, p.fd[k], q, r);
+      oa += r * static_cast<uint32_t>(p.sa[k]);
+      ob += r * static_cast<uint32_t>(p.sb[k]);
+      e = q;
+    }
+    oa += e * static_cast<uint32_t>(p.sa[0]);
+    ob += e * static_cast<uint32_t>(p.sb[0]);
+    y[i] = f(a[oa], b[ob]);
+  }
+}
+
+template <class F, int NDIM>
+static void launch_bcast_vec(F f, const BcastArgs& p, bool avec, bool bvec, const float* a,
+                             const float* b, float* y, uint32_t n4, hipStream_t st) {
+  uint32_t grid = (n4 + kBlock - 1) / kBlock;
+  grid = grid > kMaxStreamGrid * 4 ? kMaxStreamGrid * 4 : grid;
+  if (avec && bvec)
+    bcast_vec_kernel<F, NDIM, true, true><<<grid, kBlock, 0, st>>>(f, p, a, b, y, n4);
+  else if (avec)
+    bcast_vec_kernel<F, NDIM, true, false><<<grid, kBlock, 0, st>>>(f, p, a, b, y, n4);
+  else if (bvec)
+    bcast_vec_kernel<F, NDIM, false, true><<<grid, kBlock, 0, st>>>(f, p, a, b, y, n4);
+  else
+    bcast_vec_kernel<F, NDIM, false, false><<<grid, kBlock, 0, st>>>(f, p, a, b, y, n4);
+}
+
+template <class F>
+static int launch_bcast(F f, const BroadcastPlan& plan, const float* a, const float* b, float* y,
+                        hipStream_t st) {
+  BroadcastPlan pl = plan;
+  if (pl.ndim == 0) {  // one output element
+    pl.ndim = 1;
+    pl.dims[0] = 1;
+    pl.sa[0] = pl.sb[0] = 0;
+  }
+  const int nd = pl.ndim;
+  const int last = nd - 1;
+  const uint32_t n = static_cast<uint32_t>(pl.count);
+  const bool vec_ok = nd <= 4 && pl.dims[last] % 4 == 0 && aligned16(y) &&
+                      (pl.sa[last] == 0 || aligned16(a)) && (pl.sb[last] == 0 || aligned16(b));
+  if (vec_ok) {
+    BcastArgs p;
+    p.a_full = p.b_full = 1;
+    for (int k = 0; k < 4; ++k) {
+      p.fd[k] = make_fastdiv(k < nd ? static_cast<uint32_t>(pl.dims[k]) : 1u);
+      p.sa[k] = k < nd ? pl.sa[k] : 0;
+      p.sb[k] = k < nd ? pl.sb[k] : 0;
+      if (k < nd && pl.sa[k] == 0) p.a_full = 0;
+      if (k < nd && pl.sb[k] == 0) p.b_full = 0;
+    }
+    const bool avec = pl.sa[last] == 1, bvec = pl.sb[last] == 1;
+    const uint32_t n4 = n / 4;
+    switch (nd) {
+      case 1: launch_bcast_vec<F, 1>(f, p, avec, bvec, a, b, y, n4, st); break;
+      case 2: launch_bcast_vec<F, 2>(f, p, avec, bvec, a, b, y, n4, st); break;
+      case 3: launch_bcast_vec<F, 3>(f, p, avec, bvec, a, b, y, n4, st); break;
+      default: launch_bcast_vec<F, 4>(f, p, avec, bvec, a, b, y, n4, st); break;
+    }
+  } else {
+    BcastGenericArgs p;
+    p.ndim = nd;
+    for (int k = 0; k < kMaxDims; ++k) {
+      p.fd[k] = make_fastdiv(k < nd ? static_cast<uint32_t>(pl.dims[k]) : 1u);
+      p.sa[k] = k < nd ? pl.sa[k] : 0;
+      p.sb[k] = k < nd ? pl.sb[k] : 0;
+    }
+    uint32_t grid = (n + kBlock - 1) / kBlock;
+    grid = grid > kMaxStreamGrid * 4 ? kMaxStreamGrid * 4 : grid;
+    bcast_generic_kernel<F><<<grid, kBlock, 0, st>>>(f, p, a, b, y, n);
+  }
+  return launch_status();
+}
+
+}  // namespace shdw
+
+using namespace shdw;
+
+extern "C" {
+
+int shdw_hip_scale_bias(int n, int scale_num, int inner_num, const float* x, const float* scale,
+                        const float* bias, int relu, float* y, void* stream) {
+  if (n < 0 || scale_num < 1 || inner_num < 1 || !x || !y || (!scale && !bias))
+    return SHDW_E_INVALID_ARGUMENT;
+  if (n == 0) return SHDW_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (scale && bias) {
+    return relu ? launch_rowparam<kScaleBias, true>(n, scale_num, inner_num, x, scale, bias, y, st)
+                : launch_rowparam<kScaleBias, false>(n, scale_num, inner_num, x, scale, bias, y, st);
+  } else if (scale) {
+    return relu ? launch_rowparam<kScaleOnly, true>(n, scale_num, inner_num, x, scale, bias, y, st)
+                : launch_rowparam<kScaleOnly, false>(n, scale_num, inner_num, x, scale, bias, y, st);
+  }
+  return relu ? launch_rowparam<kBiasOnly, true>(n, scale_num, inner_num, x, scale, bias, y, st)
+              : launch_rowparam<kBiasOnly, false>(n, scale_num, inner_num, x, scale, bias, y, st);
+}
+
+int shdw_hip_prelu(int n, int channels, int dim, int channel_shared, const float* x,
+                   const float* slope, float* y, void* stream) {
+  if (n < 0 || channels < 1 || dim < 1 || !x || !slope || !y) return SHDW_E_INVALID_ARGUMENT;
+  if (n == 0) return SHDW_OK;
+  // c = (i / dim) % channels / div_factor with div_factor = channels when the
+  // slope is shared: that is always 0, i.e. one parameter row.
+  const int num = channel_shared ? 1 : channels;
+  return launch_rowparam<kPRelu, false>(n, num, dim, x, slope, nullptr, y,
+                                        static_cast<hipStream_t>(stream));
+}
+
+int shdw_hip_broadcast_binary(int operation, int num_axes, const int* a_shape,
+                              const int* b_shape, const int* out_shape, const float* a,
+                              const float* b, float* y, void* stream) {
+  if (!a || !b || !y) return SHDW_E_INVALID_ARGUMENT;
+  BroadcastPlan plan;
+  const int rc = plan_broadcast(num_axes, a_shape, b_shape, out_shape, &plan);
+  if (rc != SHDW_OK) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  switch (operation) {
+    case SHDW_BINARY_ADD: return launch_bcast(BAdd(), plan, a, b, y, st);
+    case SHDW_BINARY_SUB: return launch_bcast(BSub(), plan, a, b, y, st);
+    case SHDW_BINARY_MUL: return launch_bcast(BMul(), plan, a, b, y, st);
+    case SHDW_BINARY_DIV: return launch_bcast(BDiv(), plan, a, b, y, st);
+    case SHDW_BINARY_POW: return launch_bcast(BPow(), plan, a, b, y, st);
+    case SHDW_BINARY_MAX: return launch_bcast(BMax(), plan, a, b, y, st);
+    case SHDW_BINARY_MIN: return launch_bcast(BMin(), plan, a, b, y, st);
+    default: return SHDW_E_INVALID_ARGUMENT;
+  }
+}
+
+}  // extern "C"

@@ -1,0 +1,370 @@
+// Contiguous elementwise kernels: Blas::Set, the 15 unary ops, the 7 binary ops
+// in tensor and scalar form, Scal/Copy/Axpy, Activate, and the K-ary Eltwise.
+//
+// One kernel family: every lane moves 128-bit vectors, a workgroup of 256 lanes
+// covers kUnroll consecutive 4 KiB slabs per trip so that a wave's accesses are
+// 1 KiB-contiguous, and the grid strides over the tensor.  All of these are HBM
+// bound (8 or 12 bytes per element against a handful of ALU operations).
+#include <hip/hip_runtime.h>
+
+#include "../../include/shadow_hip.h"
+#include "device_common.h"
+#include "functors.h"
+#include "launch.h"
+
+#pragma clang fp contract(off)
+
+namespace shdw {
+
+constexpr int kUnroll = 4;
+
+// NIN = 0: y = f(alpha, alpha)     (fill)
+// NIN = 1: y = f(a, alpha)
+// NIN = 2: y = f(a, b)
+template <int NIN, class F>
+__global__ __launch_bounds__(kBlock) void ew_vec_kernel(F f, const float* a,
+                                                         const float* b,
+                                                         float* y, uint32_t n4,
+                                                         uint32_t n, float alpha) {
+  const uint32_t span = kBlock * kUnroll;
+  const uint32_t stride = gridDim.x * span;
+  for (uint32_t base = blockIdx.x * span; base < n4; base += stride) {
+    v4f va[kUnroll], vb[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const uint32_t i = base + u * kBlock + threadIdx.x;
+      if (i < n4) {
+        if (NIN >= 1) va[u] = load4_stream(a + 4ull * i);
+        if (NIN >= 2) vb[u] = load4_stream(b + 4ull * i);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const uint32_t i = base + u * kBlock + threadIdx.x;
+      if (i < n4) {
+        v4f r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float x = NIN >= 1 ? va[u][j] : alpha;
+          const float w = NIN >= 2 ? vb[u][j] : alpha;
+          r[j] = f(x, w);
+        }
+        store4_stream(y + 4ull * i, r);
+      }
+    }
+  }
+  // The last n % 4 elements.
+  if (blockIdx.x == 0) {
+    const uint32_t i = 4 * n4 + threadIdx.x;
+    if (i < n) {
+      const float x = NIN >= 1 ? a[i] : alpha;
+      const float w = NIN >= 2 ? b[i] : alpha;
+      y[i] = f(x, w);
+    }
+  }
+}
+
+// Same arithmetic for pointers that are not 16-byte aligned (Blas offsets).
+template <int NIN, class F>
+__global__ __launch_bounds__(kBlock) void ew_scalar_kernel(F f, const float* a, const float* b,
+                                                            float* y, uint32_t n, float alpha) {
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+    const float x = NIN >= 1 ? a[i] : alpha;
+    const float w = NIN >= 2 ? b[i] : alpha;
+    y[i] = f(x, w);
+  }
+}
+
+template <int NIN, class F>
+static int launch_ew(F f, int n, const float* a, const float* b, float alpha, float* y,
+                     void* stream) {
+  if (n < 0 || !y || (NIN >= 1 && !a) || (NIN >= 2 && !b)) return SHDW_E_INVALID_ARGUMENT;
+  if (n == 0) return SHDW_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool vec = aligned16(y) && (NIN < 1 || aligned16(a)) && (NIN < 2 || aligned16(b));
+  if (vec) {
+    const uint32_t n4 = static_cast<uint32_t>(n) / 4;
+    const uint32_t span = kBlock * kUnroll;
+    uint32_t grid = (n4 + span - 1) / span;
+    grid = grid < 1 ? 1 : (grid > kMaxStreamGrid ? kMaxStreamGrid : grid);
+    ew_vec_kernel<NIN, F><<<grid, kBlock, 0, s>>>(f, a, b, y, n4, static_cast<uint32_t>(n), alpha);
+  } else {
+    uint32_t grid = (static_cast<uint32_t>(n) + kBlock - 1) / kBlock;
+    grid = grid > kMaxStreamGrid * 4 ? kMaxStreamGrid * 4 : grid;
+    ew_scalar_kernel<NIN, F><<<grid, kBlock, 0, s>>>(f, a, b, y, static_cast<uint32_t>(n), alpha);
+  }
+  return launch_status();
+}
+
+// Adapters onto the (x, w) functor shape used by the kernels.
+template <class U>
+struct Unary2 {
+  U u;
+  SHDW_DEVICE float operator()(float a, float) const { return u(a); }
+};
+struct Fill {
+  SHDW_DEVICE float operator()(float v, float) const { return v; }
+};
+struct ScalOp {  // x *= alpha
+  SHDW_DEVICE float operator()(float x, float alpha) const { return x * alpha; }
+};
+struct AxpyOp {  // y += alpha * x, multiply then add
+  float alpha;
+  SHDW_DEVICE float operator()(float x, float y) const {
+    const float t = alpha * x;
+    return y + t;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// K-ary Eltwise in one pass.
+// ---------------------------------------------------------------------------
+constexpr int kEltwiseMaxK = 8;
+
+struct EltwiseArgs {
+  const float* x[kEltwiseMaxK];
+  float coeff[kEltwiseMaxK];
+  int k;
+  // bit j set: input j aliases the output and Shadow's pass-by-pass evaluation
+  // would have read something else than its original contents (see header).
+  unsigned alias_mask;
+  int has_seed;  // continuation call: the accumulator starts from y
+};
+
+template <int OP, int KMAX>
+SHDW_DEVICE float eltwise_fold(const EltwiseArgs& p, const float (&v)[KMAX], float seed) {
+  // SUM starts from +0 (or the stored accumulator); the others start from the
+  // first input unless continuing.
+  float acc = (OP == SHDW_ELTWISE_SUM) ? (p.has_seed ? seed : 0.0f) : (p.has_seed ? seed : v[0]);
+  const int first = (OP == SHDW_ELTWISE_SUM || p.has_seed) ? 0 : 1;
+#pragma unroll
+  for (int j = 0; j < KMAX; ++j) {
+    if (j >= first && j < p.k) {
+      float x = v[j];
+      const bool aliased = (p.alias_mask >> j) & 1u;
+      if (OP == SHDW_ELTWISE_SUM) {
+        if (aliased) x = acc;  // y += c*y: the pass reads its own running sum
+        const float t = p.coeff[j] * x;
+        acc = acc + t;
+      } else {
+        if (aliased) x = acc;
+        if (OP == SHDW_ELTWISE_PROD) acc = acc * x;
+        if (OP == SHDW_ELTWISE_MAX) acc = sel_max(acc, x);
+        if (OP == SHDW_ELTWISE_MIN) acc = sel_min(acc, x);
+      }
+    }
+  }
+  return acc;
+}
+
+// KMAX is the compile-time bound on p.k (2, 3, 4 or 8) so that the per-input
+// registers are never indexed dynamically.
+template <int OP, int KMAX, bool VEC>
+__global__ __launch_bounds__(kBlock) void eltwise_kernel(EltwiseArgs p, float* y, uint32_t n) {
+  const uint32_t stride = gridDim.x * kBlock;
+  if (VEC) {
+    const uint32_t n4 = n / 4;
+    for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n4; i += stride) {
+      v4f v[KMAX];
+      v4f seed = {0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < KMAX; ++j)
+        if (j < p.k) v[j] = load4_stream(p.x[j] + 4ull * i);
+      if (p.has_seed) seed = load4_stream(y + 4ull * i);
+      v4f r;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        float col[KMAX];
+#pragma unroll
+        for (int j = 0; j < KMAX; ++j) col[j] = (j < p.k) ? v[j][c] : 0.0f;
+        r[c] = eltwise_fold<OP, KMAX>(p, col, seed[c]);
+      }
+      store4_stream(y + 4ull * i, r);
+    }
+  }
+  // Scalar path: everything when !VEC, otherwise the last n % 4 elements.
+  const uint32_t begin = VEC ? (n / 4) * 4 : 0;
+  for (uint32_t i = begin + blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+    float col[KMAX];
+#pragma unroll
+    for (int j = 0; j < KMAX; ++j) col[j] = (j < p.k) ? p.x[j][i] : 0.0f;
+    y[i] = eltwise_fold<OP, KMAX>(p, col, p.has_seed ? y[i] : 0.0f);
+  }
+}
+
+template <int OP, int KMAX>
+static int launch_eltwise_k(const EltwiseArgs& p, int n, float* y, hipStream_t s) {
+  bool vec = aligned16(y);
+  for (int j = 0; j < p.k; ++j) vec = vec && aligned16(p.x[j]);
+  const uint32_t work = vec ? static_cast<uint32_t>(n) / 4 + 1 : static_cast<uint32_t>(n);
+  uint32_t grid = (work + kBlock - 1) / kBlock;
+  grid = grid > kMaxStreamGrid * 4 ? kMaxStreamGrid * 4 : grid;
+  if (vec)
+    eltwise_kernel<OP, KMAX, true><<<grid, kBlock, 0, s>>>(p, y, static_cast<uint32_t>(n));
+  else
+    eltwise_kernel<OP, KMAX, false><<<grid, kBlock, 0, s>>>(p, y, static_cast<uint32_t>(n));
+  return launch_status();
+}
+
+template <int OP>
+static int launch_eltwise_chunk(const EltwiseArgs& p, int n, float* y, hipStream_t s) {
+  if (p.k <= 2) return launch_eltwise_k<OP, 2>(p, n, y, s);
+  if (p.k == 3) return launch_eltwise_k<OP, 3>(p, n, y, s);
+  if (p.k == 4) return launch_eltwise_k<OP, 4>(p, n, y, s);
+  return launch_eltwise_k<OP, kEltwiseMaxK>(p, n, y, s);
+}
+
+}  // namespace shdw
+
+using namespace shdw;
+
+extern "C" {
+
+int shdw_hip_set(int n, float val, float* y, void* stream) {
+  return launch_ew<0>(Fill(), n, nullptr, nullptr, val, y, stream);
+}
+
+int shdw_hip_unary(int operation, int n, const float* a, float* y, void* stream) {
+#define SHDW_CASE(code, functor) \
+  case code:                     \
+    return launch_ew<1>(Unary2<functor>(), n, a, nullptr, 0.f, y, stream)
+  switch (operation) {
+    SHDW_CASE(SHDW_UNARY_ABS, UAbs);
+    SHDW_CASE(SHDW_UNARY_SQUARE, USquare);
+    SHDW_CASE(SHDW_UNARY_SQRT, USqrt);
+    SHDW_CASE(SHDW_UNARY_LOG, ULog);
+    SHDW_CASE(SHDW_UNARY_EXP, UExp);
+    SHDW_CASE(SHDW_UNARY_SIN, USin);
+    SHDW_CASE(SHDW_UNARY_COS, UCos);
+    SHDW_CASE(SHDW_UNARY_TAN, UTan);
+    SHDW_CASE(SHDW_UNARY_ASIN, UAsin);
+    SHDW_CASE(SHDW_UNARY_ACOS, UAcos);
+    SHDW_CASE(SHDW_UNARY_ATAN, UAtan);
+    SHDW_CASE(SHDW_UNARY_FLOOR, UFloor);
+    SHDW_CASE(SHDW_UNARY_CEIL, UCeil);
+    SHDW_CASE(SHDW_UNARY_NEG, UNeg);
+    SHDW_CASE(SHDW_UNARY_RECIPROCAL, UReciprocal);
+    default:
+      return SHDW_E_INVALID_ARGUMENT;
+  }
+#undef SHDW_CASE
+}
+
+int shdw_hip_binary(int operation, int n, const float* a, const float* b, float* y,
+                    void* stream) {
+#define SHDW_CASE(code, functor) \
+  case code:                     \
+    return launch_ew<2>(functor(), n, a, b, 0.f, y, stream)
+  switch (operation) {
+    SHDW_CASE(SHDW_BINARY_ADD, BAdd);
+    SHDW_CASE(SHDW_BINARY_SUB, BSub);
+    SHDW_CASE(SHDW_BINARY_MUL, BMul);
+    SHDW_CASE(SHDW_BINARY_DIV, BDiv);
+    SHDW_CASE(SHDW_BINARY_POW, BPow);
+    SHDW_CASE(SHDW_BINARY_MAX, BMax);
+    SHDW_CASE(SHDW_BINARY_MIN, BMin);
+    default:
+      return SHDW_E_INVALID_ARGUMENT;
+  }
+#undef SHDW_CASE
+}
+
+int shdw_hip_binary_scalar(int operation, int n, const float* a, float alpha, float* y,
+                           void* stream) {
+#define SHDW_CASE(code, functor) \
+  case code:                     \
+    return launch_ew<1>(functor(), n, a, nullptr, alpha, y, stream)
+  switch (operation) {
+    SHDW_CASE(SHDW_BINARY_ADD, BAdd);
+    SHDW_CASE(SHDW_BINARY_SUB, BSub);
+    SHDW_CASE(SHDW_BINARY_MUL, BMul);
+    SHDW_CASE(SHDW_BINARY_DIV, BDiv);
+    SHDW_CASE(SHDW_BINARY_POW, BPow);
+    SHDW_CASE(SHDW_BINARY_MAX, BMax);
+    SHDW_CASE(SHDW_BINARY_MIN, BMin);
+    default:
+      return SHDW_E_INVALID_ARGUMENT;
+  }
+#undef SHDW_CASE
+}
+
+int shdw_hip_scal(int n, float alpha, float* x, void* stream) {
+  return launch_ew<1>(ScalOp(), n, x, nullptr, alpha, x, stream);
+}
+
+int shdw_hip_copy(int n, const float* x, float* y, void* stream) {
+  return launch_ew<1>(Unary2<UCopy>(), n, x, nullptr, 0.f, y, stream);
+}
+
+int shdw_hip_axpy(int n, float alpha, const float* x, float* y, void* stream) {
+  AxpyOp op;
+  op.alpha = alpha;
+  return launch_ew<2>(op, n, x, y, 0.f, y, stream);
+}
+
+int shdw_hip_activate(int type, float slope, int n, const float* x, float* y, void* stream) {
+#define SHDW_CASE(code, functor) \
+  case code:                     \
+    return launch_ew<1>(functor(), n, x, nullptr, slope, y, stream)
+  switch (type) {
+    SHDW_CASE(SHDW_ACT_RELU, ARelu);
+    SHDW_CASE(SHDW_ACT_LEAKY, ALeaky);
+    SHDW_CASE(SHDW_ACT_SIGMOID, ASigmoid);
+    SHDW_CASE(SHDW_ACT_SOFTPLUS, ASoftPlus);
+    SHDW_CASE(SHDW_ACT_TANH, ATanh);
+    SHDW_CASE(SHDW_ACT_RELU6, ARelu6);
+    SHDW_CASE(SHDW_ACT_HARDSWISH, AHardSwish);
+    SHDW_CASE(SHDW_ACT_GELU, AGelu);
+    default:
+      return SHDW_E_INVALID_ARGUMENT;
+  }
+#undef SHDW_CASE
+}
+
+int shdw_hip_eltwise(int operation, int k, const float* const* xs, const float* coeff, int n,
+                     float* y, void* stream) {
+  if (k < 2 || !xs || !y || n < 0) return SHDW_E_INVALID_ARGUMENT;
+  if (operation < SHDW_ELTWISE_PROD || operation > SHDW_ELTWISE_MIN) return SHDW_E_INVALID_ARGUMENT;
+  for (int j = 0; j < k; ++j)
+    if (!xs[j]) return SHDW_E_INVALID_ARGUMENT;
+  if (n == 0) return SHDW_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // Inputs are consumed kEltwiseMaxK at a time; later chunks continue from the
+  // accumulator already stored in y, which is exactly Shadow's chaining.
+  int done = 0;
+  while (done < k) {
+    EltwiseArgs p;
+    p.k = (k - done > kEltwiseMaxK) ? kEltwiseMaxK : (k - done);
+    p.alias_mask = 0;
+    p.has_seed = done > 0;
+    for (int j = 0; j < kEltwiseMaxK; ++j) {
+      p.x[j] = nullptr;
+      p.coeff[j] = 1.f;
+    }
+    for (int j = 0; j < p.k; ++j) {
+      const int g = done + j;
+      p.x[j] = xs[g];
+      p.coeff[j] = coeff ? coeff[g] : 1.f;
+      if (xs[g] == y) {
+        if (operation == SHDW_ELTWISE_SUM) {
+          p.alias_mask |= 1u << j;  // Set(out, 0) overwrote it; it now reads as the running sum
+        } else if (g >= 2) {
+          p.alias_mask |= 1u << j;  // it already holds the running result
+        }
+      }
+    }
+    int rc;
+    switch (operation) {
+      case SHDW_ELTWISE_PROD: rc = launch_eltwise_chunk<SHDW_ELTWISE_PROD>(p, n, y, s); break;
+      case SHDW_ELTWISE_SUM: rc = launch_eltwise_chunk<SHDW_ELTWISE_SUM>(p, n, y, s); break;
+      case SHDW_ELTWISE_MAX: rc = launch_eltwise_chunk<SHDW_ELTWISE_MAX>(p, n, y, s); break;
+      default: rc = launch_eltwise_chunk<SHDW_ELTWISE_MIN>(p, n, y, s); break;
+    }
+    if (rc != SHDW_OK) return rc;
+    done += p.k;
+  }
+  return SHDW_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,102 @@
+// The ResNet bottleneck tail in one launch: per-channel Scale, residual add
+// (Eltwise SUM), ReLU and the global average over the trailing `inner`
+// elements.  x and the residual are read once, y is written once and the
+// pooled value falls out of the same registers; run as four operators the
+// same data crosses HBM 8 times instead of 3.
+//
+// One wave64 owns one (n, c) row.  Arithmetic per element is exactly the
+// operator sequence: t = x*s; t = t + b; u = 0 + 1*t; u = u + 1*r;
+// y = u > 0 ? u : 0; the row sum is fp64 and rounded once after the divide.
+#include <hip/hip_runtime.h>
+
+#include "../../include/shadow_hip.h"
+#include "device_common.h"
+#include "launch.h"
+
+#pragma clang fp contract(off)
+
+namespace shdw {
+
+SHDW_DEVICE float tail_element(float x, float s, float b, float r) {
+  float t = x * s;
+  t = t + b;
+  float u = 1.0f * t;
+  u = 0.0f + u;
+  const float v = 1.0f * r;
+  u = u + v;
+  return u > 0 ? u : 0;
+}
+
+SHDW_DEVICE double wave_sum_f64(double v) {
+  v += dpp_f64<kDppXor1>(v);
+  v += dpp_f64<kDppXor2>(v);
+  v += dpp_f64<kDppHalfMirror>(v);
+  v += dpp_f64<kDppMirror>(v);
+  v += __shfl_xor(v, 16, kWave);
+  v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
+template <bool VEC, bool WRITE_Y>
+__global__ __launch_bounds__(kBlock) void scale_residual_relu_rowmean_kernel(
+    const float* x, const float* scale, const float* bias, const float* res, float* y,
+    float* mean, uint32_t rows, uint32_t inner, FastDiv num) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t row = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  if (row >= rows) return;  // wave-uniform
+  const uint32_t c = row - fd_div(row, num) * num.d;
+  const float s = scale[c], b = bias[c];
+  const size_t base = static_cast<size_t>(row) * inner;
+  double sum = 0.0;
+  if (VEC) {
+    const uint32_t nv = inner / 4;
+    for (uint32_t i = lane; i < nv; i += kWave) {
+      const v4f vx = load4_stream(x + base + 4ull * i);
+      const v4f vr = load4_stream(res + base + 4ull * i);
+      v4f o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        o[j] = tail_element(vx[j], s, b, vr[j]);
+        sum += static_cast<double>(o[j]);
+      }
+      if (WRITE_Y) store4_stream(y + base + 4ull * i, o);
+    }
+  } else {
+    for (uint32_t i = lane; i < inner; i += kWave) {
+      const float o = tail_element(x[base + i], s, b, res[base + i]);
+      sum += static_cast<double>(o);
+      if (WRITE_Y) y[base + i] = o;
+    }
+  }
+  sum = wave_sum_f64(sum);
+  if (lane == 0) mean[row] = static_cast<float>(sum / static_cast<double>(static_cast<int>(inner)));
+}
+
+}  // namespace shdw
+
+using namespace shdw;
+
+extern "C" int shdw_hip_scale_residual_relu_rowmean(int n, int scale_num, int inner_num,
+                                                    const float* x, const float* scale,
+                                                    const float* bias, const float* residual,
+                                                    float* y, float* mean, void* stream) {
+  if (n < 0 || scale_num < 1 || inner_num < 1 || !x || !scale || !bias || !residual || !mean)
+    return SHDW_E_INVALID_ARGUMENT;
+  if (n % inner_num != 0) return SHDW_E_INVALID_ARGUMENT;
+  if (n == 0) return SHDW_OK;
+  const uint32_t rows = static_cast<uint32_t>(n / inner_num);
+  const uint32_t inner = static_cast<uint32_t>(inner_num);
+  const FastDiv num = make_fastdiv(static_cast<uint32_t>(scale_num));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec = inner % 4 == 0 && aligned16(x) && aligned16(residual) && (!y || aligned16(y));
+  const uint32_t grid = (rows + kBlock / kWave - 1) / (kBlock / kWave);
+#define SHDW_LAUNCH(V, W)                                                                   \
+  scale_residual_relu_rowmean_kernel<V, W><<<grid, kBlock, 0, st>>>(x, scale, bias, residual, \
+                                                                    y, mean, rows, inner, num)
+  if (vec && y) SHDW_LAUNCH(true, true);
+  else if (vec) SHDW_LAUNCH(true, false);
+  else if (y) SHDW_LAUNCH(false, true);
+  else SHDW_LAUNCH(false, false);
+#undef SHDW_LAUNCH
+  return launch_status();
+}

@@ -1,0 +1,219 @@
+#include "plan.h"
+
+#include <algorithm>
+#include <climits>
+
+#include "../../include/shadow_hip.h"
+
+namespace shdw {
+
+int plan_broadcast(int num_axes, const int* a_shape, const int* b_shape,
+                   const int* out_shape, BroadcastPlan* plan) {
+  if (num_axes < 0 || (num_axes > 0 && (!a_shape || !b_shape || !out_shape)) || !plan)
+    return SHDW_E_INVALID_ARGUMENT;
+  *plan = BroadcastPlan();
+
+  // Contiguous strides of both operands, computed over the full rank first so
+  // that dropped size-1 dims cannot disturb them.
+  int64_t stride_a = 1, stride_b = 1, count = 1;
+  // Walk from the innermost axis outwards and build the collapsed dims in
+  // reverse; flip at the end.
+  int rdims[kMaxDims], rsa[kMaxDims], rsb[kMaxDims];
+  int n = 0;
+  bool prev_a_bc = false, prev_b_bc = false;
+  for (int ax = num_axes - 1; ax >= 0; --ax) {
+    const int da = a_shape[ax], db = b_shape[ax], dout = out_shape[ax];
+    if (da < 1 || db < 1 || dout < 1) return SHDW_E_INVALID_ARGUMENT;
+    if (dout != std::max(da, db)) return SHDW_E_INVALID_ARGUMENT;
+    if ((da != dout && da != 1) || (db != dout && db != 1)) return SHDW_E_INVALID_ARGUMENT;
+    if (dout > 1) {
+      const bool a_bc = (da == 1), b_bc = (db == 1);
+      if (n > 0 && a_bc == prev_a_bc && b_bc == prev_b_bc) {
+        // Same broadcast status as the dim just inside: one longer dim.
+        const int64_t merged = static_cast<int64_t>(rdims[n - 1]) * dout;
+        if (merged > INT_MAX) return SHDW_E_UNSUPPORTED;
+        rdims[n - 1] = static_cast<int>(merged);
+      } else {
+        if (n == kMaxDims) return SHDW_E_UNSUPPORTED;
+        rdims[n] = dout;
+        rsa[n] = a_bc ? 0 : static_cast<int>(stride_a);
+        rsb[n] = b_bc ? 0 : static_cast<int>(stride_b);
+        ++n;
+      }
+      prev_a_bc = a_bc;
+      prev_b_bc = b_bc;
+    }
+    stride_a *= da;
+    stride_b *= db;
+    count *= dout;
+    if (count > INT_MAX || stride_a > INT_MAX || stride_b > INT_MAX) return SHDW_E_UNSUPPORTED;
+  }
+  plan->ndim = n;
+  for (int k = 0; k < n; ++k) {
+    plan->dims[k] = rdims[n - 1 - k];
+    plan->sa[k] = rsa[n - 1 - k];
+    plan->sb[k] = rsb[n - 1 - k];
+  }
+  plan->count = count;
+  return SHDW_OK;
+}
+
+static int ceil_div64(int64_t a, int64_t b) { return static_cast<int>((a + b - 1) / b); }
+
+int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* axes,
+                ReducePlan* plan) {
+  if (num_axes < 0 || num_axes > kMaxDims) return num_axes < 0 ? SHDW_E_INVALID_ARGUMENT : SHDW_E_UNSUPPORTED;
+  if (num_reduce < 0 || num_reduce > num_axes) return SHDW_E_INVALID_ARGUMENT;
+  if ((num_axes > 0 && !in_shape) || (num_reduce > 0 && !axes) || !plan)
+    return SHDW_E_INVALID_ARGUMENT;
+  *plan = ReducePlan();
+
+  bool reduced[kMaxDims] = {false};
+  bool ascending = true;
+  for (int k = 0; k < num_reduce; ++k) {
+    const int ax = axes[k];
+    // Shadow indexes its stride table with the raw axis value
+    // (shadow/operators/kernels/reduce.hpp:54-57): negative or repeated axes
+    // read out of bounds there, so they are rejected here.
+    if (ax < 0 || ax >= num_axes || reduced[ax]) return SHDW_E_INVALID_ARGUMENT;
+    reduced[ax] = true;
+    if (k > 0 && axes[k] < axes[k - 1]) ascending = false;
+  }
+  int64_t stride[kMaxDims];
+  int64_t total = 1;
+  for (int ax = num_axes - 1; ax >= 0; --ax) {
+    if (in_shape[ax] < 1) return SHDW_E_INVALID_ARGUMENT;
+    stride[ax] = total;
+    total *= in_shape[ax];
+    if (total > INT_MAX) return SHDW_E_UNSUPPORTED;
+  }
+  int64_t outputs = 1, window = 1;
+  for (int ax = 0; ax < num_axes; ++ax) (reduced[ax] ? window : outputs) *= in_shape[ax];
+  plan->outputs = outputs;
+  plan->window = window;
+
+  // Collapse: drop size-1 dims, merge neighbours with the same reduced flag.
+  int64_t cdim[kMaxDims];
+  bool cred[kMaxDims];
+  int nc = 0;
+  for (int ax = 0; ax < num_axes; ++ax) {
+    if (in_shape[ax] == 1) continue;
+    if (nc > 0 && cred[nc - 1] == reduced[ax]) {
+      cdim[nc - 1] *= in_shape[ax];
+    } else {
+      cdim[nc] = in_shape[ax];
+      cred[nc] = reduced[ax];
+      ++nc;
+    }
+  }
+
+  bool fast = ascending;
+  if (fast) {
+    if (nc == 0) {
+      plan->kind = kStrided;  // single element, one output
+      plan->outer = 1, plan->reduce = 1, plan->inner = 1;
+    } else if (nc == 1 && !cred[0]) {
+      plan->kind = kStrided;  // nothing to fold: every output has a 1-element window
+      plan->outer = 1, plan->reduce = 1, plan->inner = cdim[0];
+    } else if (nc == 1 && cred[0]) {
+      plan->kind = kRows;
+      plan->outer = 1, plan->reduce = cdim[0], plan->inner = 1;
+    } else if (nc == 2 && !cred[0]) {
+      plan->kind = kRows;
+      plan->outer = cdim[0], plan->reduce = cdim[1], plan->inner = 1;
+    } else if (nc == 2 && cred[0]) {
+      plan->kind = kStrided;
+      plan->outer = 1, plan->reduce = cdim[0], plan->inner = cdim[1];
+    } else if (nc == 3 && !cred[0]) {
+      plan->kind = kStrided;
+      plan->outer = cdim[0], plan->reduce = cdim[1], plan->inner = cdim[2];
+    } else {
+      fast = false;
+    }
+  }
+
+  if (!fast) {
+    plan->kind = kGeneric;
+    plan->outer = outputs, plan->reduce = window, plan->inner = 0;
+    for (int ax = 0; ax < num_axes; ++ax) {
+      if (!reduced[ax] && in_shape[ax] > 1) {
+        plan->kdim[plan->nk] = in_shape[ax];
+        plan->kstride[plan->nk] = static_cast<int>(stride[ax]);
+        ++plan->nk;
+      }
+    }
+    for (int k = 0; k < num_reduce; ++k) {
+      const int ax = axes[k];
+      if (in_shape[ax] > 1) {
+        plan->rdim[plan->nr] = in_shape[ax];
+        plan->rstride[plan->nr] = static_cast<int>(stride[ax]);
+        ++plan->nr;
+      }
+    }
+    plan->splits = 1;
+    return SHDW_OK;
+  }
+
+  // Work split.  The aim is >= ~2k workgroups of 256 lanes when the input is
+  // large enough, so that all 256 CUs (8 XCDs) have several waves in flight,
+  // while every slice still streams a few KiB.
+  if (plan->kind == kRows) {
+    if (plan->reduce <= 4096 && plan->outer >= 256) {
+      plan->wave_per_row = true;
+      plan->splits = 1;
+    } else {
+      const int by_fill = ceil_div64(2048, plan->outer);
+      const int by_work = ceil_div64(plan->reduce, 8192);
+      plan->splits = std::max(1, std::min(by_fill, by_work));
+    }
+  } else {
+    const int vec = (plan->inner % 4 == 0) ? 4 : 1;
+    const int64_t tiles = (plan->inner + 64 * vec - 1) / (64 * vec);
+    const int64_t base_blocks = tiles * plan->outer;
+    const int by_fill = ceil_div64(2048, base_blocks);
+    const int by_work = ceil_div64(plan->reduce, 32);  // >= 8 rows per wave
+    plan->splits = std::max(1, std::min(by_fill, by_work));
+  }
+  return SHDW_OK;
+}
+
+}  // namespace shdw
+
+extern "C" {
+
+int shdw_hip_plan_broadcast(int num_axes, const int* a_shape, const int* b_shape,
+                            const int* out_shape, int* dims, int* a_strides,
+                            int* b_strides) {
+  shdw::BroadcastPlan p;
+  const int rc = shdw::plan_broadcast(num_axes, a_shape, b_shape, out_shape, &p);
+  if (rc != SHDW_OK) return rc;
+  for (int k = 0; k < p.ndim; ++k) {
+    if (dims) dims[k] = p.dims[k];
+    if (a_strides) a_strides[k] = p.sa[k];
+    if (b_strides) b_strides[k] = p.sb[k];
+  }
+  return p.ndim;
+}
+
+int shdw_hip_plan_reduce(int num_axes, const int* in_shape, int num_reduce,
+                         const int* axes, int* kind, int* outer, int* reduce,
+                         int* inner, int* splits) {
+  shdw::ReducePlan p;
+  const int rc = shdw::plan_reduce(num_axes, in_shape, num_reduce, axes, &p);
+  if (rc != SHDW_OK) return rc;
+  if (kind) *kind = p.kind;
+  if (outer) *outer = static_cast<int>(p.outer);
+  if (reduce) *reduce = static_cast<int>(p.reduce);
+  if (inner) *inner = static_cast<int>(p.inner);
+  if (splits) *splits = p.splits;
+  return SHDW_OK;
+}
+
+size_t shdw_hip_reduce_workspace_bytes(int num_axes, const int* in_shape, int num_reduce,
+                                       const int* axes) {
+  shdw::ReducePlan p;
+  if (shdw::plan_reduce(num_axes, in_shape, num_reduce, axes, &p) != SHDW_OK) return 0;
+  return shdw::reduce_workspace_bytes(p);
+}
+
+}  // extern "C"

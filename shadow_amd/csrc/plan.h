@@ -1,0 +1,70 @@
+// Host-side launch planning for the broadcast and reduce kernels.  Pure C++ (no
+// HIP types) so the same code is exercised by CPU-only tests through the
+// shdw_hip_plan_* entry points.
+#ifndef SHADOW_AMD_CSRC_PLAN_H_
+#define SHADOW_AMD_CSRC_PLAN_H_
+
+#include <cstddef>
+#include <cstdint>
+
+namespace shdw {
+
+constexpr int kMaxDims = 8;  // Shadow's CUDA broadcast kernel stops at 8 axes
+                             // (shadow/operators/kernels/binary.cu:34)
+
+// ---------------------------------------------------------------------------
+// Broadcast: the output is viewed as `ndim` dims (outermost first); operand
+// offset = sum_k idx[k] * stride[k], stride 0 on the dims an operand broadcasts.
+// Size-1 output dims are dropped and neighbouring dims with the same
+// (a broadcasts?, b broadcasts?) status are merged.
+// ---------------------------------------------------------------------------
+struct BroadcastPlan {
+  int ndim = 0;
+  int dims[kMaxDims] = {0};
+  int sa[kMaxDims] = {0};
+  int sb[kMaxDims] = {0};
+  int64_t count = 1;  // number of output elements
+};
+
+// Returns 0, or a negative SHDW_E_* code.
+int plan_broadcast(int num_axes, const int* a_shape, const int* b_shape,
+                   const int* out_shape, BroadcastPlan* plan);
+
+// ---------------------------------------------------------------------------
+// Reduce.
+//   kRows    : x viewed as [outer][reduce], reduced axis contiguous.
+//   kStrided : x viewed as [outer][reduce][inner], inner > 1 contiguous.
+//   kGeneric : any other axis pattern (several separated reduced groups, or
+//              axes not listed in ascending order, where Shadow's list order is
+//              not memory order).  Kept/reduced dims are passed uncollapsed.
+// `splits` > 1 means a first stage writes `splits` partial results per output
+// and a second stage combines them in slice order.
+// ---------------------------------------------------------------------------
+enum ReduceKind { kRows = 0, kStrided = 1, kGeneric = 2 };
+
+struct ReducePlan {
+  int kind = kRows;
+  int64_t outer = 1, reduce = 1, inner = 1;
+  int splits = 1;
+  bool wave_per_row = false;  // kRows: one wave64 per row instead of a block
+  int64_t outputs = 1;        // number of output elements
+  int64_t window = 1;         // elements per output (Shadow's num_list)
+  // kGeneric only: kept dims (outermost first) and reduced dims in LIST order,
+  // i.e. rdim[nr-1] is the fastest-varying one, as Shadow enumerates them.
+  int nk = 0, nr = 0;
+  int kdim[kMaxDims] = {0}, kstride[kMaxDims] = {0};
+  int rdim[kMaxDims] = {0}, rstride[kMaxDims] = {0};
+};
+
+constexpr size_t kReducePartialBytes = 16;  // {double value; uint32 key; pad}
+
+int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* axes,
+                ReducePlan* plan);
+
+inline size_t reduce_workspace_bytes(const ReducePlan& p) {
+  return p.splits > 1 ? static_cast<size_t>(p.outputs) * p.splits * kReducePartialBytes : 0;
+}
+
+}  // namespace shdw
+
+#endif  // SHADOW_AMD_CSRC_PLAN_H_

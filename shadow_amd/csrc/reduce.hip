@@ -1,0 +1,501 @@
+// Reduce kernels.  Shadow's kernel walks an index list serially per output
+// (shadow/operators/kernels/reduce.cpp:9-76); here the reduced extent is spread
+// over lanes, waves and, when there are few outputs, workgroups:
+//
+//   rows     x[outer][reduce]           reduced axis contiguous.  One wave64 per
+//                                       row for short rows; a workgroup per
+//                                       (row, slice) for long ones.
+//   strided  x[outer][reduce][inner]    lanes run along `inner` (coalesced),
+//                                       the four waves of a workgroup and
+//                                       optional grid.z slices split `reduce`.
+//   generic  any axis set               one wave per output, index lists
+//                                       replaced by division by constants.
+//   stage 2  combines the per-slice partials of a split first stage.
+//
+// PROD/SUM/AVG/L1/L2 accumulate in fp64 exactly as the reference does, so the
+// only difference is association order (~1e-16 relative before the single
+// rounding to fp32).  MAX/MIN must be bit-exact although the reference's
+// "first element attaining the extremum wins" depends on order when the
+// extremum is a zero (+0 and -0 compare equal): every accumulator therefore
+// also tracks the smallest list position of a zero together with its sign, and
+// the sign of a zero result is taken from there.
+#include <hip/hip_runtime.h>
+
+#include <cfloat>
+
+#include "../../include/shadow_hip.h"
+#include "device_common.h"
+#include "launch.h"
+#include "plan.h"
+
+#pragma clang fp contract(off)
+
+namespace shdw {
+
+struct Partial {
+  double v;
+  uint32_t key;
+  uint32_t pad;
+};
+static_assert(sizeof(Partial) == kReducePartialBytes, "partial layout");
+
+constexpr bool is_select(int op) { return op == SHDW_REDUCE_MAX || op == SHDW_REDUCE_MIN; }
+
+// ---- fp64 accumulating ops ----
+template <int OP, bool SELECT = is_select(OP)>
+struct Acc {
+  double v;
+  SHDW_DEVICE void init() { v = (OP == SHDW_REDUCE_PROD) ? 1.0 : 0.0; }
+  SHDW_DEVICE void add(float x, uint32_t) {
+    if (OP == SHDW_REDUCE_PROD) {
+      v *= static_cast<double>(x);
+    } else if (OP == SHDW_REDUCE_L1) {
+      v += static_cast<double>(__builtin_fabsf(x));
+    } else if (OP == SHDW_REDUCE_L2) {
+      const float ax = __builtin_fabsf(x);
+      const float sq = ax * ax;  // fp32 product, then widened
+      v += static_cast<double>(sq);
+    } else {
+      v += static_cast<double>(x);
+    }
+  }
+  SHDW_DEVICE void merge(const Acc& o) {
+    if (OP == SHDW_REDUCE_PROD) v *= o.v; else v += o.v;
+  }
+  template <int CTRL>
+  SHDW_DEVICE Acc dpp() const {
+    Acc r;
+    r.v = dpp_f64<CTRL>(v);
+    return r;
+  }
+  SHDW_DEVICE Acc shfl_xor(int m) const {
+    Acc r;
+    r.v = __shfl_xor(v, m, kWave);
+    return r;
+  }
+  SHDW_DEVICE float finalize(uint32_t window) const {
+    if (OP == SHDW_REDUCE_AVG) return static_cast<float>(v / static_cast<double>(static_cast<int>(window)));
+    if (OP == SHDW_REDUCE_L2) return __builtin_sqrtf(static_cast<float>(v));
+    return static_cast<float>(v);
+  }
+  SHDW_DEVICE Partial pack() const { return Partial{v, 0u, 0u}; }
+  SHDW_DEVICE void unpack(const Partial& p) { v = p.v; }
+};
+
+// ---- MAX / MIN ----
+template <int OP>
+struct Acc<OP, true> {
+  float v;
+  uint32_t key;  // min over zeros seen of (list position << 1 | sign bit)
+  SHDW_DEVICE void init() {
+    v = (OP == SHDW_REDUCE_MAX) ? -FLT_MAX : FLT_MAX;
+    key = 0xffffffffu;
+  }
+  SHDW_DEVICE void add(float x, uint32_t pos) {
+    if (OP == SHDW_REDUCE_MAX) v = (v < x) ? x : v; else v = (x < v) ? x : v;
+    if (x == 0.0f) {
+      const uint32_t k = (pos << 1) | (__float_as_uint(x) >> 31);
+      key = k < key ? k : key;
+    }
+  }
+  SHDW_DEVICE void merge(const Acc& o) {
+    if (OP == SHDW_REDUCE_MAX) v = (v < o.v) ? o.v : v; else v = (o.v < v) ? o.v : v;
+    key = o.key < key ? o.key : key;
+  }
+  template <int CTRL>
+  SHDW_DEVICE Acc dpp() const {
+    Acc r;
+    r.v = dpp_f32<CTRL>(v);
+    r.key = dpp_u32<CTRL>(key);
+    return r;
+  }
+  SHDW_DEVICE Acc shfl_xor(int m) const {
+    Acc r;
+    r.v = __shfl_xor(v, m, kWave);
+    r.key = __shfl_xor(key, m, kWave);
+    return r;
+  }
+  SHDW_DEVICE float finalize(uint32_t) const {
+    if (v == 0.0f) return (key & 1u) ? -0.0f : 0.0f;
+    return v;
+  }
+  SHDW_DEVICE Partial pack() const { return Partial{static_cast<double>(v), key, 0u}; }
+  SHDW_DEVICE void unpack(const Partial& p) {
+    v = static_cast<float>(p.v);
+    key = p.key;
+  }
+};
+
+// All 64 lanes must be active.  Every lane ends with the same combined value:
+// each exchange pairs two lanes that both compute merge(own, other), and every
+// merge used here is commutative bit-for-bit.
+template <class A>
+SHDW_DEVICE A wave_allreduce(A a) {
+  a.merge(a.template dpp<kDppXor1>());
+  a.merge(a.template dpp<kDppXor2>());
+  a.merge(a.template dpp<kDppHalfMirror>());
+  a.merge(a.template dpp<kDppMirror>());
+  a.merge(a.shfl_xor(16));
+  a.merge(a.shfl_xor(32));
+  return a;
+}
+
+// ---------------------------------------------------------------------------
+// rows, one wave per row
+// ---------------------------------------------------------------------------
+template <int OP, bool VEC>
+__global__ __launch_bounds__(kBlock) void reduce_rows_wave_kernel(const float* x, float* y,
+                                                                   uint32_t rows,
+                                                                   uint32_t reduce) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t row = blockIdx.x * (kBlock / kWave) + (threadIdx.x / kWave);
+  if (row >= rows) return;  // wave-uniform
+  const float* p = x + static_cast<size_t>(row) * reduce;
+  Acc<OP> acc;
+  acc.init();
+  if (VEC) {
+    const uint32_t nv = reduce / 4;
+    uint32_t i = lane;
+    for (; i + 3 * kWave < nv; i += 4 * kWave) {
+      v4f v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = load4_stream(p + 4ull * (i + u * kWave));
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc.add(v[u][j], 4 * (i + u * kWave) + j);
+    }
+    for (; i < nv; i += kWave) {
+      const v4f v = load4_stream(p + 4ull * i);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc.add(v[j], 4 * i + j);
+    }
+  } else {
+    for (uint32_t i = lane; i < reduce; i += kWave) acc.add(p[i], i);
+  }
+  acc = wave_allreduce(acc);
+  if (lane == 0) y[row] = acc.finalize(reduce);
+}
+
+// ---------------------------------------------------------------------------
+// rows, one workgroup per (slice, row)
+// ---------------------------------------------------------------------------
+template <int OP, bool VEC>
+__global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const float* x, float* y,
+                                                                    Partial* part,
+                                                                    uint32_t reduce,
+                                                                    uint32_t chunk,
+                                                                    uint32_t splits) {
+  __shared__ Partial lds[kBlock / kWave];
+  const uint32_t row = blockIdx.y, split = blockIdx.x;
+  const float* p = x + static_cast<size_t>(row) * reduce;
+  const uint32_t begin = split * chunk;  // chunk is a multiple of 4
+  uint32_t end = begin + chunk;
+  if (end > reduce || split == splits - 1) end = reduce;
+  Acc<OP> acc;
+  acc.init();
+  if (begin < end) {
+    if (VEC) {
+      const uint32_t vb = begin / 4, ve = end / 4;
+      uint32_t i = vb + threadIdx.x;
+      for (; i + 3 * kBlock < ve; i += 4 * kBlock) {
+        v4f v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = load4_stream(p + 4ull * (i + u * kBlock));
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc.add(v[u][j], 4 * (i + u * kBlock) + j);
+      }
+      for (; i < ve; i += kBlock) {
+        const v4f v = load4_stream(p + 4ull * i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc.add(v[j], 4 * i + j);
+      }
+      // elements past the last whole vector (only the final slice has any)
+      const uint32_t t = 4 * ve + threadIdx.x;
+      if (t < end) acc.add(p[t], t);
+    } else {
+      for (uint32_t i = begin + threadIdx.x; i < end; i += kBlock) acc.add(p[i], i);
+    }
+  }
+  acc = wave_allreduce(acc);
+  const uint32_t lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+  if (lane == 0) lds[w] = acc.pack();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < kBlock / kWave; ++k) {
+      Acc<OP> o;
+      o.unpack(lds[k]);
+      acc.merge(o);
+    }
+    if (splits == 1) y[row] = acc.finalize(reduce);
+    else part[static_cast<size_t>(row) * splits + split] = acc.pack();
+  }
+}
+
+// ---------------------------------------------------------------------------
+// strided: x[outer][reduce][inner] -> y[outer][inner]
+// ---------------------------------------------------------------------------
+template <int OP, int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_strided_kernel(const float* x, float* y,
+                                                                 Partial* part, uint32_t reduce,
+                                                                 uint32_t inner,
+                                                                 uint32_t rows_per_split,
+                                                                 uint32_t splits,
+                                                                 uint32_t outputs) {
+  constexpr int kWaves = kBlock / kWave;
+  __shared__ Partial lds[kWaves - 1][VEC][kWave];
+  const uint32_t lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+  const uint32_t col = (blockIdx.x * kWave + lane) * VEC;
+  const uint32_t o = blockIdx.y, split = blockIdx.z;
+  const bool col_ok = col < inner;
+  const uint32_t r_begin = split * rows_per_split;
+  uint32_t r_end = r_begin + rows_per_split;
+  if (r_end > reduce) r_end = reduce;
+
+  Acc<OP> acc[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) acc[j].init();
+
+  if (col_ok) {
+    const float* p = x + static_cast<size_t>(o) * reduce * inner + col;
+    uint32_t r = r_begin + w;
+    for (; r + 3 * kWaves < r_end; r += 4 * kWaves) {
+      float v[4][VEC];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float* q = p + static_cast<size_t>(r + u * kWaves) * inner;
+        if (VEC == 4) {
+          const v4f t = load4_stream(q);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) v[u][j] = t[j];
+        } else {
+          v[u][0] = __builtin_nontemporal_load(q);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j].add(v[u][j], r + u * kWaves);
+    }
+    for (; r < r_end; r += kWaves) {
+      const float* q = p + static_cast<size_t>(r) * inner;
+      if (VEC == 4) {
+        const v4f t = load4_stream(q);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j].add(t[j], r);
+      } else {
+        acc[0].add(__builtin_nontemporal_load(q), r);
+      }
+    }
+  }
+  if (w > 0) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) lds[w - 1][j][lane] = acc[j].pack();
+  }
+  __syncthreads();
+  if (w == 0 && col_ok) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      for (int k = 0; k < kWaves - 1; ++k) {
+        Acc<OP> t;
+        t.unpack(lds[k][j][lane]);
+        acc[j].merge(t);
+      }
+      const size_t out = static_cast<size_t>(o) * inner + col + j;
+      if (splits == 1) y[out] = acc[j].finalize(reduce);
+      else part[static_cast<size_t>(split) * outputs + out] = acc[j].pack();
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// generic: one wave per output, kept/reduced dims decoded by constant division
+// ---------------------------------------------------------------------------
+struct GenericArgs {
+  int nk, nr;
+  FastDiv kfd[kMaxDims], rfd[kMaxDims];
+  int kstride[kMaxDims], rstride[kMaxDims];
+};
+
+template <int OP>
+__global__ __launch_bounds__(kBlock) void reduce_generic_kernel(GenericArgs g, const float* x,
+                                                                 float* y, uint32_t outputs,
+                                                                 uint32_t window) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t o = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  if (o >= outputs) return;  // wave-uniform
+  uint32_t base = 0, e = o;
+  for (int k = g.nk - 1; k >= 0; --k) {
+    uint32_t q, r;
+    fd_divmod(e, g.kfd[k], q, r);
+    base += r * static_cast<uint32_t>(g.kstride[k]);
+    e = q;
+  }
+  Acc<OP> acc;
+  acc.init();
+  for (uint32_t pos = lane; pos < window; pos += kWave) {
+    uint32_t off = base, t = pos;
+    for (int k = g.nr - 1; k >= 0; --k) {
+      uint32_t q, r;
+      fd_divmod(t, g.rfd[k], q, r);
+      off += r * static_cast<uint32_t>(g.rstride[k]);
+      t = q;
+    }
+    acc.add(x[off], pos);
+  }
+  acc = wave_allreduce(acc);
+  if (lane == 0) y[o] = acc.finalize(window);
+}
+
+// ---------------------------------------------------------------------------
+// stage 2: y[o] = finalize(merge_s part[o*stride_o + s*stride_s])
+// ---------------------------------------------------------------------------
+template <int OP>
+__global__ __launch_bounds__(kBlock) void reduce_stage2_kernel(const Partial* part, float* y,
+                                                                uint32_t outputs,
+                                                                uint32_t splits, size_t stride_o,
+                                                                size_t stride_s,
+                                                                uint32_t window) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t o = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  if (o >= outputs) return;  // wave-uniform
+  Acc<OP> acc;
+  acc.init();
+  for (uint32_t s = lane; s < splits; s += kWave) {
+    Acc<OP> t;
+    t.unpack(part[o * stride_o + s * stride_s]);
+    acc.merge(t);
+  }
+  acc = wave_allreduce(acc);
+  if (lane == 0) y[o] = acc.finalize(window);
+}
+
+template <int OP>
+static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* workspace,
+                      size_t workspace_bytes, hipStream_t st) {
+  const size_t need = reduce_workspace_bytes(pl);
+  if (need > 0 && (!workspace || workspace_bytes < need)) return SHDW_E_WORKSPACE;
+  Partial* part = static_cast<Partial*>(workspace);
+  const uint32_t outputs = static_cast<uint32_t>(pl.outputs);
+  const uint32_t window = static_cast<uint32_t>(pl.window);
+  constexpr int kWaves = kBlock / kWave;
+
+  if (pl.kind == kGeneric) {
+    GenericArgs g;
+    g.nk = pl.nk;
+    g.nr = pl.nr;
+    for (int k = 0; k < kMaxDims; ++k) {
+      g.kfd[k] = make_fastdiv(k < pl.nk ? pl.kdim[k] : 1);
+      g.rfd[k] = make_fastdiv(k < pl.nr ? pl.rdim[k] : 1);
+      g.kstride[k] = k < pl.nk ? pl.kstride[k] : 0;
+      g.rstride[k] = k < pl.nr ? pl.rstride[k] : 0;
+    }
+    const uint32_t grid = (outputs + kWaves - 1) / kWaves;
+    reduce_generic_kernel<OP><<<grid, kBlock, 0, st>>>(g, x, y, outputs, window);
+    return launch_status();
+  }
+
+  if (pl.kind == kRows) {
+    const uint32_t rows = static_cast<uint32_t>(pl.outer);
+    const uint32_t reduce = static_cast<uint32_t>(pl.reduce);
+    // 128-bit loads need every row start 16-byte aligned.
+    const bool vec = aligned16(x) && (reduce % 4 == 0 || rows == 1);
+    if (pl.wave_per_row) {
+      const uint32_t grid = (rows + kWaves - 1) / kWaves;
+      if (vec && reduce % 4 == 0)
+        reduce_rows_wave_kernel<OP, true><<<grid, kBlock, 0, st>>>(x, y, rows, reduce);
+      else
+        reduce_rows_wave_kernel<OP, false><<<grid, kBlock, 0, st>>>(x, y, rows, reduce);
+      return launch_status();
+    }
+    const uint32_t splits = static_cast<uint32_t>(pl.splits);
+    uint32_t chunk = (reduce + splits - 1) / splits;
+    chunk = (chunk + 3) & ~3u;
+    const dim3 grid(splits, rows);
+    if (vec)
+      reduce_rows_block_kernel<OP, true><<<grid, kBlock, 0, st>>>(x, y, part, reduce, chunk, splits);
+    else
+      reduce_rows_block_kernel<OP, false><<<grid, kBlock, 0, st>>>(x, y, part, reduce, chunk, splits);
+    int rc = launch_status();
+    if (rc != SHDW_OK || splits == 1) return rc;
+    const uint32_t g2 = (rows + kWaves - 1) / kWaves;
+    reduce_stage2_kernel<OP><<<g2, kBlock, 0, st>>>(part, y, rows, splits, splits, 1, window);
+    return launch_status();
+  }
+
+  // strided
+  const uint32_t outer = static_cast<uint32_t>(pl.outer);
+  const uint32_t reduce = static_cast<uint32_t>(pl.reduce);
+  const uint32_t inner = static_cast<uint32_t>(pl.inner);
+  const uint32_t splits = static_cast<uint32_t>(pl.splits);
+  if (outer > 65535u || splits > 65535u) return SHDW_E_UNSUPPORTED;
+  const uint32_t rows_per_split = (reduce + splits - 1) / splits;
+  const bool vec = inner % 4 == 0 && aligned16(x);
+  const int v = vec ? 4 : 1;
+  const dim3 grid((inner + kWave * v - 1) / (kWave * v), outer, splits);
+  if (vec)
+    reduce_strided_kernel<OP, 4><<<grid, kBlock, 0, st>>>(x, y, part, reduce, inner,
+                                                          rows_per_split, splits, outputs);
+  else
+    reduce_strided_kernel<OP, 1><<<grid, kBlock, 0, st>>>(x, y, part, reduce, inner,
+                                                          rows_per_split, splits, outputs);
+  int rc = launch_status();
+  if (rc != SHDW_OK || splits == 1) return rc;
+  const uint32_t g2 = (outputs + kWaves - 1) / kWaves;
+  reduce_stage2_kernel<OP><<<g2, kBlock, 0, st>>>(part, y, outputs, splits, 1, outputs, window);
+  return launch_status();
+}
+
+static int dispatch_reduce(int operation, const ReducePlan& pl, const float* x, float* y,
+                           void* workspace, size_t workspace_bytes, hipStream_t st) {
+  switch (operation) {
+    case SHDW_REDUCE_PROD: return run_reduce<SHDW_REDUCE_PROD>(pl, x, y, workspace, workspace_bytes, st);
+    case SHDW_REDUCE_SUM: return run_reduce<SHDW_REDUCE_SUM>(pl, x, y, workspace, workspace_bytes, st);
+    case SHDW_REDUCE_MAX: return run_reduce<SHDW_REDUCE_MAX>(pl, x, y, workspace, workspace_bytes, st);
+    case SHDW_REDUCE_MIN: return run_reduce<SHDW_REDUCE_MIN>(pl, x, y, workspace, workspace_bytes, st);
+    case SHDW_REDUCE_AVG: return run_reduce<SHDW_REDUCE_AVG>(pl, x, y, workspace, workspace_bytes, st);
+    case SHDW_REDUCE_L1: return run_reduce<SHDW_REDUCE_L1>(pl, x, y, workspace, workspace_bytes, st);
+    case SHDW_REDUCE_L2: return run_reduce<SHDW_REDUCE_L2>(pl, x, y, workspace, workspace_bytes, st);
+    default: return SHDW_E_INVALID_ARGUMENT;
+  }
+}
+
+}  // namespace shdw
+
+using namespace shdw;
+
+extern "C" {
+
+int shdw_hip_reduce(int operation, int num_axes, const int* in_shape, int num_reduce,
+                    const int* axes, const float* x, float* y, void* workspace,
+                    size_t workspace_bytes, void* stream) {
+  if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
+  ReducePlan pl;
+  const int rc = plan_reduce(num_axes, in_shape, num_reduce, axes, &pl);
+  if (rc != SHDW_OK) return rc;
+  return dispatch_reduce(operation, pl, x, y, workspace, workspace_bytes,
+                         static_cast<hipStream_t>(stream));
+}
+
+int shdw_hip_asum(int n, const float* x, float* result_host, void* workspace,
+                  size_t workspace_bytes, void* stream) {
+  if (n < 1 || !x || !result_host) return SHDW_E_INVALID_ARGUMENT;
+  const int shape[1] = {n}, axes[1] = {0};
+  ReducePlan pl;
+  int rc = plan_reduce(1, shape, 1, axes, &pl);
+  if (rc != SHDW_OK) return rc;
+  // The device-side result lives in the 16 bytes after the partials.
+  const size_t need = reduce_workspace_bytes(pl);
+  if (!workspace || workspace_bytes < need + 16) return SHDW_E_WORKSPACE;
+  float* y = reinterpret_cast<float*>(static_cast<char*>(workspace) + need);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  rc = dispatch_reduce(SHDW_REDUCE_L1, pl, x, y, workspace, need, st);
+  if (rc != SHDW_OK) return rc;
+  hipError_t e = hipMemcpyAsync(result_host, y, sizeof(float), hipMemcpyDeviceToHost, st);
+  if (e != hipSuccess) return static_cast<int>(e);
+  return static_cast<int>(hipStreamSynchronize(st));
+}
+
+}  // extern "C"

@@ -1,0 +1,191 @@
+"""Thin numpy-in / numpy-out wrappers over the C ABI for the GPU tests.
+
+Every helper uploads its operands, calls exactly one ``shdw_hip_*`` entry point
+on the null stream, synchronises and downloads the result."""
+import ctypes
+
+import numpy as np
+
+import shadow_amd
+from shadow_amd import Buffer, check, ints
+
+
+def _lib():
+    return shadow_amd.hip()
+
+
+def _sync():
+    check(_lib().shdw_hip_stream_sync(None))
+
+
+def _f(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def set_(n, val):
+    y = Buffer(4 * n)
+    check(_lib().shdw_hip_set(n, val, y.ptr, None))
+    _sync()
+    return y.download(count=n)
+
+
+def unary(op, x, inplace=False, offset=0):
+    """offset (in floats) shifts both pointers off 16-byte alignment."""
+    x = _f(x).ravel()
+    n = x.size
+    a = Buffer(4 * (n + offset))
+    a.upload(x, 4 * offset)
+    y = a if inplace else Buffer(4 * (n + offset))
+    check(_lib().shdw_hip_unary(op, n, a.ptr + 4 * offset, y.ptr + 4 * offset, None))
+    _sync()
+    return y.download(count=n, offset_bytes=4 * offset)
+
+
+def binary(op, a, b, inplace=False):
+    a, b = _f(a).ravel(), _f(b).ravel()
+    da, db = Buffer.from_numpy(a), Buffer.from_numpy(b)
+    y = da if inplace else Buffer(a.nbytes)
+    check(_lib().shdw_hip_binary(op, a.size, da.ptr, db.ptr, y.ptr, None))
+    _sync()
+    return y.download(count=a.size)
+
+
+def binary_scalar(op, a, alpha):
+    a = _f(a).ravel()
+    da = Buffer.from_numpy(a)
+    y = Buffer(a.nbytes)
+    check(_lib().shdw_hip_binary_scalar(op, a.size, da.ptr, alpha, y.ptr, None))
+    _sync()
+    return y.download(count=a.size)
+
+
+def scal(alpha, x):
+    x = _f(x).ravel()
+    d = Buffer.from_numpy(x)
+    check(_lib().shdw_hip_scal(x.size, alpha, d.ptr, None))
+    _sync()
+    return d.download(count=x.size)
+
+
+def copy(x):
+    x = _f(x).ravel()
+    d = Buffer.from_numpy(x)
+    y = Buffer(x.nbytes)
+    check(_lib().shdw_hip_copy(x.size, d.ptr, y.ptr, None))
+    _sync()
+    return y.download(count=x.size)
+
+
+def axpy(alpha, x, y):
+    x, y = _f(x).ravel(), _f(y).ravel()
+    dx, dy = Buffer.from_numpy(x), Buffer.from_numpy(y)
+    check(_lib().shdw_hip_axpy(x.size, alpha, dx.ptr, dy.ptr, None))
+    _sync()
+    return dy.download(count=x.size)
+
+
+def reduce_workspace(shape, axes):
+    return _lib().shdw_hip_reduce_workspace_bytes(len(shape), ints(shape), len(axes), ints(axes))
+
+
+def asum(x):
+    x = _f(x).ravel()
+    d = Buffer.from_numpy(x)
+    need = reduce_workspace([x.size], [0]) + 16
+    ws = Buffer(need)
+    out = ctypes.c_float(0)
+    check(_lib().shdw_hip_asum(x.size, d.ptr, ctypes.byref(out), ws.ptr, need, None))
+    return np.float32(out.value)
+
+
+def broadcast_binary(op, a, a_shape, b, b_shape, out_shape):
+    a, b = _f(a).ravel(), _f(b).ravel()
+    da, db = Buffer.from_numpy(a), Buffer.from_numpy(b)
+    n = int(np.prod(out_shape, dtype=np.int64))
+    y = Buffer(4 * n)
+    check(_lib().shdw_hip_broadcast_binary(op, len(out_shape), ints(a_shape), ints(b_shape),
+                                           ints(out_shape), da.ptr, db.ptr, y.ptr, None))
+    _sync()
+    return y.download(count=n)
+
+
+def activate(x, act_type, slope=0.1, inplace=False):
+    x = _f(x).ravel()
+    d = Buffer.from_numpy(x)
+    y = d if inplace else Buffer(x.nbytes)
+    check(_lib().shdw_hip_activate(act_type, slope, x.size, d.ptr, y.ptr, None))
+    _sync()
+    return y.download(count=x.size)
+
+
+def prelu(x, shape, channel_shared, slope):
+    x, slope = _f(x).ravel(), _f(slope).ravel()
+    channels = shape[1]
+    dim = int(np.prod(shape[2:], dtype=np.int64))
+    d, ds = Buffer.from_numpy(x), Buffer.from_numpy(slope)
+    y = Buffer(x.nbytes)
+    check(_lib().shdw_hip_prelu(x.size, channels, dim, int(bool(channel_shared)), d.ptr, ds.ptr,
+                                y.ptr, None))
+    _sync()
+    return y.download(count=x.size)
+
+
+def scale_bias(x, scale, bias, scale_num, inner_num, relu=False, inplace=False, offset=0):
+    x = _f(x).ravel()
+    n = x.size
+    d = Buffer(4 * (n + offset))
+    d.upload(x, 4 * offset)
+    ds = Buffer.from_numpy(_f(scale)) if scale is not None else None
+    db = Buffer.from_numpy(_f(bias)) if bias is not None else None
+    y = d if inplace else Buffer(4 * (n + offset))
+    check(_lib().shdw_hip_scale_bias(n, scale_num, inner_num, d.ptr + 4 * offset,
+                                     ds.ptr if ds else None, db.ptr if db else None,
+                                     int(relu), y.ptr + 4 * offset, None))
+    _sync()
+    return y.download(count=n, offset_bytes=4 * offset)
+
+
+def eltwise(op, inputs, coeff=None, alias=None):
+    """alias = index of the input whose buffer is also the output."""
+    inputs = [_f(x).ravel() for x in inputs]
+    n = inputs[0].size
+    bufs = [Buffer.from_numpy(x) for x in inputs]
+    y = bufs[alias] if alias is not None else Buffer(4 * n)
+    ptrs = (ctypes.c_void_p * len(bufs))(*[b.ptr for b in bufs])
+    co = None
+    if coeff is not None:
+        co = (ctypes.c_float * len(coeff))(*[float(c) for c in coeff])
+    check(_lib().shdw_hip_eltwise(op, len(bufs), ptrs, co, n, y.ptr, None))
+    _sync()
+    return y.download(count=n)
+
+
+def reduce(op, x, shape, axes):
+    x = _f(x).ravel()
+    d = Buffer.from_numpy(x)
+    out_shape = list(shape)
+    for ax in axes:
+        out_shape[ax] = 1
+    n_out = int(np.prod(out_shape, dtype=np.int64))
+    y = Buffer(4 * n_out)
+    need = reduce_workspace(shape, axes)
+    ws = Buffer(need) if need else None
+    check(_lib().shdw_hip_reduce(op, len(shape), ints(shape), len(axes), ints(axes), d.ptr, y.ptr,
+                                 ws.ptr if ws else None, need, None))
+    _sync()
+    return y.download(count=n_out), out_shape
+
+
+def scale_residual_relu_rowmean(x, scale, bias, res, scale_num, inner_num, want_y=True):
+    x, res = _f(x).ravel(), _f(res).ravel()
+    n = x.size
+    dx, dr = Buffer.from_numpy(x), Buffer.from_numpy(res)
+    ds, db = Buffer.from_numpy(_f(scale)), Buffer.from_numpy(_f(bias))
+    y = Buffer(4 * n) if want_y else None
+    rows = n // inner_num
+    mean = Buffer(4 * rows)
+    check(_lib().shdw_hip_scale_residual_relu_rowmean(n, scale_num, inner_num, dx.ptr, ds.ptr,
+                                                      db.ptr, dr.ptr, y.ptr if y else None,
+                                                      mean.ptr, None))
+    _sync()
+    return (y.download(count=n) if y else None), mean.download(count=rows)

@@ -1,0 +1,305 @@
+"""Parity of every C-ABI kernel entry point with the CPU oracle on the same
+seeded inputs.  Bit-exact unless stated; fp64-accumulating reductions are held
+to |gpu - cpu| <= 1e-5 |cpu| (their association order differs)."""
+import numpy as np
+import pytest
+
+import oracle
+from tests import gpuops
+from tests.helpers import (assert_bit_exact, assert_rel_close, normal, ulp_distance, uniform,
+                           with_specials)
+
+pytestmark = pytest.mark.gpu
+
+EXACT_UNARY = {0: "abs", 1: "square", 2: "sqrt", 4: "exp", 11: "floor", 12: "ceil", 13: "neg",
+               14: "reciprocal"}
+LIBM_UNARY = {3: "log", 5: "sin", 6: "cos", 7: "tan", 8: "asin", 9: "acos", 10: "atan"}
+
+SIZES = [1, 3, 4, 5, 63, 64, 255, 1024, 1027, 4096 + 2, 100003, 1 << 20]
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_set(gpu, n):
+    assert_bit_exact(gpuops.set_(n, -1.25), oracle.blas_set(n, -1.25), "set")
+
+
+@pytest.mark.parametrize("op", sorted(EXACT_UNARY))
+@pytest.mark.parametrize("n", [5, 1027, 100003])
+def test_unary_exact(gpu, op, n):
+    x = with_specials(normal(10 + op, n, 2.0), op)
+    assert_bit_exact(gpuops.unary(op, x), oracle.unary(op, x), EXACT_UNARY[op])
+
+
+@pytest.mark.parametrize("op", [0, 2, 4, 14])
+def test_unary_inplace_and_misaligned(gpu, op):
+    x = with_specials(normal(20 + op, 70001, 2.0), op)
+    want = oracle.unary(op, x)
+    assert_bit_exact(gpuops.unary(op, x, inplace=True), want, "in place")
+    for off in (1, 2, 3):
+        assert_bit_exact(gpuops.unary(op, x, offset=off), want, "offset %d" % off)
+
+
+@pytest.mark.parametrize("op", sorted(LIBM_UNARY))
+def test_unary_libm_ulp(gpu, op):
+    """These still run the device math library, not a glibc restatement: parity
+    is within a few ulp, not bit-exact."""
+    x = with_specials(uniform(30 + op, 200003, -4.0, 4.0), op)
+    if op in (8, 9):
+        x = np.clip(x, -1.0, 1.0)
+    got, want = gpuops.unary(op, x), oracle.unary(op, x)
+    assert (np.isnan(got) == np.isnan(want)).all()
+    ok = np.isfinite(want)
+    assert ulp_distance(got[ok], want[ok]).max() <= 4, LIBM_UNARY[op]
+
+
+@pytest.mark.parametrize("op", [0, 1, 2, 3, 5, 6])
+@pytest.mark.parametrize("n", [7, 4099, 262144 + 1])
+def test_binary_and_scalar(gpu, op, n):
+    a = with_specials(normal(40 + op, n), op)
+    b = with_specials(uniform(50 + op, n, 0.5, 2.0), op + 1)
+    assert_bit_exact(gpuops.binary(op, a, b), oracle.binary(op, a, b), "binary %d" % op)
+    assert_bit_exact(gpuops.binary(op, a, b, inplace=True), oracle.binary(op, a, b), "in place")
+    for alpha in (1.5, -0.0, float("nan")):
+        assert_bit_exact(gpuops.binary_scalar(op, a, alpha), oracle.binary_scalar(op, a, alpha),
+                         "scalar %d" % op)
+
+
+def test_binary_pow_ulp(gpu):
+    a = uniform(60, 50001, 0.1, 4.0)
+    b = uniform(61, 50001, -3.0, 3.0)
+    got, want = gpuops.binary(4, a, b), oracle.binary(4, a, b)
+    assert ulp_distance(got, want).max() <= 4
+
+
+def test_max_min_select_semantics(gpu):
+    a = np.float32([0.0, -0.0, np.nan, 1.0, np.nan, -np.inf, 5.0])
+    b = np.float32([-0.0, 0.0, 1.0, np.nan, np.nan, np.inf, 5.0])
+    for op in (5, 6):
+        got = gpuops.binary(op, a, b)
+        assert_bit_exact(got, oracle.binary(op, a, b), "select")
+        # ties and NaN in either position return the left operand
+        assert np.signbit(got[0]) == False and np.signbit(got[1]) == True
+        assert np.isnan(got[2]) and got[3] == 1.0
+
+
+def test_level1(gpu):
+    x = with_specials(normal(70, 30011), 1)
+    y = normal(71, 30011)
+    assert_bit_exact(gpuops.scal(0.37, x), oracle.scal(0.37, x), "scal")
+    assert_bit_exact(gpuops.copy(x), oracle.copy(x), "copy")
+    assert_bit_exact(gpuops.axpy(-1.3, x, y), oracle.axpy(-1.3, x, y), "axpy")
+    z = normal(72, 1 << 20)
+    assert_rel_close(gpuops.asum(z), oracle.asum(z), 1e-6, "asum")
+    assert_rel_close(gpuops.asum(z[:77]), oracle.asum(z[:77]), 1e-6, "asum small")
+
+
+def test_axpy_is_not_fused(gpu):
+    """alpha*x + y with a product that needs rounding: an FMA would differ."""
+    x = np.float32([1.0 + 2.0 ** -12] * 8)
+    y = np.float32([-(1.0 + 2.0 ** -11)] * 8)
+    alpha = float(np.float32(1.0 + 2.0 ** -12))
+    want = oracle.axpy(alpha, x, y)
+    assert_bit_exact(gpuops.axpy(alpha, x, y), want, "axpy")
+    fused = np.float32(np.float64(alpha) * np.float64(x[0]) + np.float64(y[0]))
+    assert want[0] != fused  # the case does discriminate
+
+
+@pytest.mark.parametrize("act", [1, 2, 3, 5, 6, 7])
+@pytest.mark.parametrize("n", [9, 66001])
+def test_activate_exact(gpu, act, n):
+    x = with_specials(normal(80 + act, n, 2.0), act)
+    assert_bit_exact(gpuops.activate(x, act, 0.1), oracle.activate(x, act, 0.1), "act %d" % act)
+    assert_bit_exact(gpuops.activate(x, act, 0.1, inplace=True), oracle.activate(x, act, 0.1), "in place")
+
+
+@pytest.mark.parametrize("act", [4, 8])
+def test_activate_libm_ulp(gpu, act):
+    x = normal(90 + act, 100001, 2.0)
+    got, want = gpuops.activate(x, act), oracle.activate(x, act)
+    if act == 8:
+        # 1 + erf(.) cancels in the negative tail, so ulps of the result are not
+        # meaningful there; bound the absolute error instead.
+        assert np.abs(got.astype(np.float64) - want).max() <= 2e-6
+    else:
+        assert ulp_distance(got, want).max() <= 4
+
+
+@pytest.mark.parametrize("shape,shared", [((2, 3, 5, 7), False), ((2, 3, 5, 7), True),
+                                          ((4, 16, 12), False), ((3, 8), False), ((1, 64, 56, 56), False)])
+def test_prelu(gpu, shape, shared):
+    x = with_specials(normal(100, shape), 3)
+    slope = uniform(101, 1 if shared else shape[1], -0.5, 0.5)
+    assert_bit_exact(gpuops.prelu(x, list(shape), shared, slope),
+                     oracle.prelu(x, list(shape), shared, slope), "prelu")
+
+
+@pytest.mark.parametrize("outer,num,inner", [(2, 3, 8), (4, 16, 196), (3, 5, 7), (1, 1, 1000),
+                                             (8, 64, 3136), (5, 7, 1), (2, 256, 30)])
+@pytest.mark.parametrize("mode", ["sb", "s", "b"])
+def test_scale_bias(gpu, outer, num, inner, mode):
+    n = outer * num * inner
+    x = with_specials(normal(110, n), 4)
+    s = uniform(111, num, 0.5, 1.5) if "s" in mode else None
+    b = uniform(112, num, -0.1, 0.1) if "b" in mode else None
+    want = oracle.scale_bias(x, s, b, num, inner)
+    assert_bit_exact(gpuops.scale_bias(x, s, b, num, inner), want, "scale")
+    assert_bit_exact(gpuops.scale_bias(x, s, b, num, inner, inplace=True), want, "in place")
+    assert_bit_exact(gpuops.scale_bias(x, s, b, num, inner, offset=1), want, "misaligned")
+    relu = oracle.activate(want, 1)
+    assert_bit_exact(gpuops.scale_bias(x, s, b, num, inner, relu=True), relu, "scale+relu")
+
+
+def test_scale_is_not_fused(gpu):
+    x = np.float32([1.0 + 2.0 ** -12] * 16)
+    s = np.float32([1.0 + 2.0 ** -12])
+    b = np.float32([-(1.0 + 2.0 ** -11)])
+    want = oracle.scale_bias(x, s, b, 1, 16)
+    assert_bit_exact(gpuops.scale_bias(x, s, b, 1, 16), want, "no fma")
+    assert want[0] != np.float32(np.float64(x[0]) * np.float64(s[0]) + np.float64(b[0]))
+
+
+BCAST_CASES = [
+    ([8, 64, 12, 12], [1, 64, 1, 1]),
+    ([16, 1, 8, 64], [1, 5, 8, 1]),
+    ([4, 6, 1, 32], [1, 1, 6, 32]),
+    ([128, 64], [1, 1]),
+    ([2, 1], [1, 3]),
+    ([3, 1, 5, 1, 7], [1, 4, 1, 6, 1]),
+    ([2, 3, 1, 2, 1, 3, 1, 2], [1, 1, 4, 1, 5, 1, 2, 1]),
+    ([1, 1], [1, 1]),
+    ([5, 3], [5, 3]),
+    ([1, 7], [9, 1]),
+    ([6, 1, 10], [6, 4, 1]),
+    ([33, 4], [1, 4]),
+]
+
+
+@pytest.mark.parametrize("sa,sb", BCAST_CASES)
+@pytest.mark.parametrize("op", [0, 1, 2, 3, 5, 6])
+def test_broadcast_binary(gpu, sa, sb, op):
+    so = [max(x, y) for x, y in zip(sa, sb)]
+    a = with_specials(normal(120, sa), 5)
+    b = with_specials(uniform(121, sb, 0.5, 2.0), 6)
+    want = oracle.broadcast_binary(op, a, sa, b, sb, so)
+    assert_bit_exact(gpuops.broadcast_binary(op, a, sa, b, sb, so), want, "bcast")
+
+
+@pytest.mark.parametrize("op", [0, 1, 2, 3])
+@pytest.mark.parametrize("k", [2, 3, 4, 5, 8, 9, 11])
+def test_eltwise(gpu, op, k):
+    n = 40003
+    xs = [with_specials(normal(130 + j, n), j) for j in range(k)]
+    coeff = [1.0, -0.5, 2.0, 0.25, 1.0, 3.0, -1.0, 0.5, 1.5, -2.0, 0.75][:k] if op == 1 else None
+    want = oracle.eltwise(op, xs, coeff)
+    assert_bit_exact(gpuops.eltwise(op, xs, coeff), want, "eltwise")
+
+
+def test_eltwise_sum_signed_zero(gpu):
+    a = np.float32([-0.0, 0.0, -0.0, 1.0])
+    b = np.float32([-0.0, -0.0, 0.0, -1.0])
+    got = gpuops.eltwise(1, [a, b])
+    assert_bit_exact(got, oracle.eltwise(1, [a, b]), "sum zeros")
+    assert not np.signbit(got).any()  # the accumulator starts at +0
+
+
+@pytest.mark.parametrize("op", [0, 1, 2, 3])
+@pytest.mark.parametrize("alias", [0, 1, 2])
+def test_eltwise_aliased_output(gpu, op, alias):
+    xs = [normal(140 + j, 5003) for j in range(3)]
+    cpu_in = [x.copy() for x in xs]
+    want = oracle.eltwise(op, cpu_in, None, out=cpu_in[alias]).copy()
+    assert_bit_exact(gpuops.eltwise(op, xs, None, alias=alias), want, "aliased")
+
+
+REDUCE_CASES = [
+    ([4, 6, 7, 8], [2, 3]),      # rows, wave per row needs >= 256 rows: block path here
+    ([16, 32, 7, 8], [2, 3]),    # rows, wave per row
+    ([300, 9], [1]),             # rows, odd length
+    ([3, 50, 20], [1]),          # strided, inner % 4 == 0
+    ([3, 50, 21], [1]),          # strided, scalar lanes
+    ([40, 300], [0]),            # strided with outer == 1
+    ([5, 6, 7], []),             # no axes at kernel level: identity windows
+    ([2, 3, 4, 5], [0, 1, 2, 3]),
+    ([100003], [0]),             # full, split over blocks
+    ([1 << 20], [0]),
+    ([2, 3, 4, 5], [0, 2]),      # generic
+    ([2, 3, 4, 5], [3, 1]),      # generic, list order differs from memory order
+    ([6, 1, 5], [1]),            # reduced axis of extent 1
+    ([1, 1, 1], [0, 1, 2]),
+    ([2, 40000], [1]),           # rows, long, few
+]
+
+
+@pytest.mark.parametrize("shape,axes", REDUCE_CASES)
+@pytest.mark.parametrize("op", [0, 1, 2, 3, 4, 5, 6])
+def test_reduce(gpu, shape, axes, op):
+    x = normal(150, shape)
+    if op == 0:
+        x = uniform(151, shape, 0.9, 1.1)  # keep products in range
+    want, _ = oracle.reduce(op, x, shape, axes)
+    got, _ = gpuops.reduce(op, x, shape, axes)
+    if op in (2, 3):
+        assert_bit_exact(got, want, "reduce select")
+    else:
+        assert_rel_close(got, want, 1e-5, "reduce accumulate")
+
+
+@pytest.mark.parametrize("shape,axes", [([64, 48], [1]), ([3, 64, 8], [1]), ([2, 3, 4, 5], [3, 1]),
+                                        ([50000], [0]), ([300, 16], [1])])
+@pytest.mark.parametrize("op", [2, 3])
+def test_reduce_select_special_values(gpu, shape, axes, op):
+    """Zeros of both signs, NaNs and infinities: the first extremum in list
+    order wins, NaNs are skipped, an all-NaN window returns the identity."""
+    r = np.random.default_rng(160 + op)
+    x = r.choice(np.float32([0.0, -0.0, np.nan, -1.0, 1.0, np.inf, -np.inf]),
+                 size=int(np.prod(shape)), p=[0.3, 0.3, 0.2, 0.05, 0.05, 0.05, 0.05]).astype(np.float32)
+    # windows made only of zeros / only of NaNs
+    x = x.reshape(shape)
+    if len(shape) == 2 and axes == [1]:
+        x[0, :] = np.nan
+        x[1, :] = np.where(r.random(shape[1]) < 0.5, 0.0, -0.0)
+        x[2, :] = np.inf if op == 3 else -np.inf
+    want, _ = oracle.reduce(op, x, shape, axes)
+    got, _ = gpuops.reduce(op, x, shape, axes)
+    assert_bit_exact(got, want, "reduce select specials")
+
+
+def test_reduce_l2_and_avg_definition(gpu):
+    x = np.float32([[3, 4], [6, 8]])
+    got, _ = gpuops.reduce(6, x, [2, 2], [1])
+    assert_bit_exact(got, np.float32([5, 10]), "l2")
+    got, _ = gpuops.reduce(4, x, [2, 2], [1])
+    assert_bit_exact(got, np.float32([3.5, 7]), "avg")
+
+
+@pytest.mark.parametrize("outer,num,inner", [(2, 8, 196), (3, 5, 7), (1, 16, 1000), (4, 4, 4)])
+def test_fused_tail(gpu, outer, num, inner):
+    n = outer * num * inner
+    x, r = normal(170, n), normal(171, n)
+    s, b = uniform(172, num, 0.5, 1.5), uniform(173, num, -0.1, 0.1)
+    t = oracle.scale_bias(x, s, b, num, inner)
+    t = oracle.eltwise(1, [t, r], [1.0, 1.0])
+    want_y = oracle.activate(t, 1)
+    want_m, _ = oracle.reduce(4, want_y, [outer * num, inner], [1])
+    y, m = gpuops.scale_residual_relu_rowmean(x, s, b, r, num, inner)
+    assert_bit_exact(y, want_y, "fused y")
+    assert_rel_close(m, want_m, 1e-5, "fused mean")
+    _, m2 = gpuops.scale_residual_relu_rowmean(x, s, b, r, num, inner, want_y=False)
+    assert_bit_exact(m2, m, "mean without y")
+
+
+def test_argument_errors(gpu):
+    import shadow_amd
+    lib = gpu
+    buf = shadow_amd.Buffer(64)
+    assert lib.shdw_hip_unary(15, 4, buf.ptr, buf.ptr, None) == -1
+    assert lib.shdw_hip_binary(7, 4, buf.ptr, buf.ptr, buf.ptr, None) == -1
+    assert lib.shdw_hip_activate(0, 0.1, 4, buf.ptr, buf.ptr, None) == -1
+    assert lib.shdw_hip_unary(0, 4, None, buf.ptr, None) == -1
+    assert lib.shdw_hip_unary(0, 0, buf.ptr, buf.ptr, None) == 0
+    sh = shadow_amd.ints([2, 3])
+    assert lib.shdw_hip_broadcast_binary(0, 2, sh, shadow_amd.ints([2, 2]), sh, buf.ptr, buf.ptr,
+                                         buf.ptr, None) == -1
+    assert lib.shdw_hip_reduce(1, 2, sh, 1, shadow_amd.ints([-1]), buf.ptr, buf.ptr, None, 0, None) == -1
+    big = shadow_amd.ints([1 << 20])
+    assert lib.shdw_hip_reduce(1, 1, big, 1, shadow_amd.ints([0]), buf.ptr, buf.ptr, None, 0, None) == -3
