@@ -130,13 +130,13 @@ def test_activate_closed_forms():
 def test_activate_libm_against_fp64():
     x = uniform(31, 20000, -9.0, 9.0)
     xd = x.astype(np.float64)
-    assert ulp_distance(oracle.activate(x, 5), np.tanh(xd).astype(F)).max() <= 1
+    assert ulp_distance(oracle.activate(x, 5), np.tanh(xd).astype(F)).max() <= 2  # fdlibm tanhf: < 2 ulp
     assert ulp_distance(oracle.activate(x, 3), (1 / (1 + np.exp(-xd))).astype(F)).max() <= 2
     assert ulp_distance(oracle.activate(x, 4), np.log1p(np.exp(xd)).astype(F)).max() <= 2
     erf = np.vectorize(math.erf)
-    gelu = 0.5 * xd * (1 + erf(0.707107 * xd))
-    ok = np.abs(gelu) > 1e-3  # cancellation near the negative tail is the formula's own
-    assert ulp_distance(oracle.activate(x, 8)[ok], gelu.astype(F)[ok]).max() <= 64
+    gelu = 0.5 * xd * (1 + erf(np.float64(F(0.707107)) * xd))
+    # 1 + erf(.) cancels in the negative tail, so bound the absolute error
+    assert np.abs(oracle.activate(x, 8).astype(np.float64) - gelu).max() <= 1e-6
 
 
 def test_activate_reference_observations():
