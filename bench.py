@@ -1,0 +1,309 @@
+#!/usr/bin/env python3
+"""Benchmark of the Shadow tensor hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-configs]
+
+A "step" is one pass of the headline workload (BASELINE.json configs[1]): seven
+launches over an fp32 [64,256,56,56] tensor -- Activate relu, sigmoid, tanh;
+Unary exp, abs, sqrt(abs); Scale(per-channel gamma, beta)+ReLU in one launch.
+Inputs are generated from fixed seeds, uploaded once and stay resident in HBM;
+the timed region is K steps between two stream synchronisations.
+
+Prints ONE JSON line.  `value` is algorithmic GB/s of the whole step
+(compulsory reads + writes of every op / wall time).  `roofline` describes the
+kernel that takes the largest share of the step, timed with HIP events on the
+launch stream inside the timed region.  `cpu_baseline` is the CPU oracle (a C
+port of the reference's loops, one thread) timed on this host on the same
+buffers.  `configs` lists every op of the five BASELINE workloads measured the
+same way (events around batches of launches that rotate over >256 MB of
+buffers), so that each can be held against the 8 TB/s HBM roofline.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-configs", action="store_true", help="skip the per-config table")
+    ap.add_argument("--cpu-passes", type=int, default=2)
+    return ap.parse_args()
+
+
+def normal(seed, n, sigma=1.0):
+    return (np.random.default_rng(seed).standard_normal(n, dtype=np.float32) * np.float32(sigma))
+
+
+def uniform(seed, n, lo, hi):
+    u = np.random.default_rng(seed).random(n, dtype=np.float32)
+    return (np.float32(lo) + u * np.float32(hi - lo)).astype(np.float32)
+
+
+class Dev:
+    """Device-side plumbing over the C ABI: one stream, events, buffers."""
+
+    def __init__(self):
+        import shadow_amd
+        self.sa = shadow_amd
+        self.lib = shadow_amd.hip()
+        if shadow_amd.device_count() < 1:
+            raise SystemExit("bench.py: no HIP device visible")
+        self.ck(self.lib.shdw_hip_set_device(0))
+        s = ctypes.c_void_p()
+        self.ck(self.lib.shdw_hip_stream_create(ctypes.byref(s)))
+        self.stream = s
+        info = ctypes.create_string_buffer(256)
+        self.ck(self.lib.shdw_hip_device_info(0, info, 256))
+        self.info = info.value.decode()
+
+    def ck(self, rc):
+        self.sa.check(rc)
+
+    def buf(self, arr=None, nbytes=None):
+        if arr is not None:
+            return self.sa.Buffer.from_numpy(arr)
+        return self.sa.Buffer(nbytes)
+
+    def event(self):
+        e = ctypes.c_void_p()
+        self.ck(self.lib.shdw_hip_event_create(ctypes.byref(e)))
+        return e
+
+    def record(self, e):
+        self.ck(self.lib.shdw_hip_event_record(e, self.stream))
+
+    def elapsed_ms(self, a, b):
+        ms = ctypes.c_float(0)
+        self.ck(self.lib.shdw_hip_event_elapsed_ms(a, b, ctypes.byref(ms)))
+        return ms.value
+
+    def sync(self):
+        self.ck(self.lib.shdw_hip_stream_sync(self.stream))
+
+
+# ------------------------------------------------------------------ headline
+def headline(dev, steps, warmup):
+    lib, st = dev.lib, dev.stream
+    shape = (64, 256, 56, 56)
+    n = int(np.prod(shape))
+    C, inner = shape[1], shape[2] * shape[3]
+    x_h = normal(201, n, 2.0)
+    g_h, b_h = uniform(202, C, 0.5, 1.5), uniform(203, C, -0.1, 0.1)
+    x, g, b = dev.buf(x_h), dev.buf(g_h), dev.buf(b_h)
+    y = [dev.buf(nbytes=4 * n) for _ in range(2)]
+    a = dev.buf(nbytes=4 * n)  # abs output, input of sqrt
+
+    per_op = 8 * n
+    ops = [
+        ("activate_relu", per_op, lambda o: lib.shdw_hip_activate(1, 0.1, n, x.ptr, o.ptr, st)),
+        ("activate_sigmoid", per_op, lambda o: lib.shdw_hip_activate(3, 0.1, n, x.ptr, o.ptr, st)),
+        ("unary_exp", per_op, lambda o: lib.shdw_hip_unary(4, n, x.ptr, o.ptr, st)),
+        ("unary_abs", per_op, lambda o: lib.shdw_hip_unary(0, n, x.ptr, a.ptr, st)),
+        ("unary_sqrt_of_abs", per_op, lambda o: lib.shdw_hip_unary(2, n, a.ptr, o.ptr, st)),
+        ("activate_tanh", per_op, lambda o: lib.shdw_hip_activate(5, 0.1, n, x.ptr, o.ptr, st)),
+        ("scale_relu_fused", per_op + 8 * C,
+         lambda o: lib.shdw_hip_scale_bias(n, C, inner, x.ptr, g.ptr, b.ptr, 1, o.ptr, st)),
+    ]
+    step_bytes = sum(nb for _, nb, _ in ops)
+
+    def step(i, events=None):
+        for k, (_, _, fn) in enumerate(ops):
+            if events is not None:
+                dev.record(events[k][0])
+            dev.ck(fn(y[(i + k) & 1]))
+            if events is not None:
+                dev.record(events[k][1])
+
+    for i in range(warmup):
+        step(i)
+    dev.sync()
+    ev = [[(dev.event(), dev.event()) for _ in ops] for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i, ev[i])
+    dev.sync()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / steps
+
+    kernel_ms = []
+    for k in range(len(ops)):
+        kernel_ms.append(sum(dev.elapsed_ms(ev[i][k][0], ev[i][k][1]) for i in range(steps)) / steps)
+    detail = []
+    for (name, nb, _), ms in zip(ops, kernel_ms):
+        gbs = nb / (ms * 1e-3) / 1e9
+        detail.append({"op": name, "bytes": nb, "us": round(ms * 1e3, 2), "GBps": round(gbs, 1),
+                       "frac": round(gbs / HBM_PEAK_GBS, 4)})
+    dom = int(np.argmax(kernel_ms))
+    dom_gbs = ops[dom][1] / (kernel_ms[dom] * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": ops[dom][0], "achieved": round(dom_gbs, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
+                "traffic": None, "avg_us": round(kernel_ms[dom] * 1e3, 2),
+                "algorithmic_bytes": ops[dom][1]}
+    host = {"x": x_h, "gamma": g_h, "beta": b_h, "shape": shape}
+    return ms_per_step, step_bytes, n, roofline, detail, host
+
+
+def cpu_baseline(host, step_bytes, passes):
+    """The oracle on this host, one thread: the same seven results, with
+    Scale and ReLU as the two separate operators the reference runs."""
+    import oracle
+    x, g, b = host["x"], host["gamma"], host["beta"]
+    C, inner = host["shape"][1], host["shape"][2] * host["shape"][3]
+    oracle.lib()
+    best = None
+    for _ in range(passes):
+        t0 = time.perf_counter()
+        oracle.activate(x, 1)
+        oracle.activate(x, 3)
+        oracle.unary(4, x)
+        a = oracle.unary(0, x)
+        oracle.unary(2, a)
+        oracle.activate(x, 5)
+        s = oracle.scale_bias(x, g, b, C, inner)
+        oracle.activate(s, 1)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return {"value": round(step_bytes / best / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "%d full passes of the same step on the same buffers (51.4M elements, 8 "
+                      "operator runs each), best pass %.2f s; host has %d logical CPUs" % (
+                          passes, best, os.cpu_count() or 0),
+            "seconds_per_step": round(best, 3)}
+
+
+# ------------------------------------------------------------- config table
+def time_batch(dev, launch, sets, reps=40, warm=5):
+    """Average device time of one launch: events around `reps` back-to-back
+    launches that rotate over `sets` operand sets."""
+    for i in range(warm):
+        dev.ck(launch(i % sets))
+    e0, e1 = dev.event(), dev.event()
+    dev.record(e0)
+    for i in range(reps):
+        dev.ck(launch(i % sets))
+    dev.record(e1)
+    dev.sync()
+    return dev.elapsed_ms(e0, e1) / reps
+
+
+def config_table(dev):
+    lib, st = dev.lib, dev.stream
+    I = dev.sa.ints
+    rows = []
+
+    def add(cfg, name, nbytes, ms, elems):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        rows.append({"cfg": cfg, "op": name, "bytes": nbytes, "us": round(ms * 1e3, 2),
+                     "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "Gelem_s": round(elems / (ms * 1e-3) / 1e9, 2)})
+
+    SETS = 6  # 6 x (in + out) of 51 MB each: more than the 256 MB Infinity Cache
+    NBIG = 12845056  # elements of the cfg-3 and cfg-5 tensors (51.4 MB)
+    A = [dev.buf(normal(301 + 10 * k, NBIG)) for k in range(SETS)]
+    Y = [dev.buf(nbytes=4 * NBIG) for _ in range(SETS)]
+
+    # cfg 1: Binary add with channel broadcast (uses the first 6.4M elements of each set)
+    sa, sb = [8, 64, 112, 112], [1, 64, 1, 1]
+    n = int(np.prod(sa))
+    B = dev.buf(uniform(102, 64, -1, 1))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_broadcast_binary(0, 4, I(sa), I(sb), I(sa), A[k].ptr,
+                                                                 B.ptr, Y[k].ptr, st), SETS)
+    add(1, "binary_add_channel_broadcast", 8 * n + 256, ms, n)
+
+    # cfg 3: reductions over [32,512,28,28]
+    shp = [32, 512, 28, 28]
+    for name, op, axes, outs in [("reduce_sum_hw", 1, [2, 3], 16384), ("reduce_avg_hw", 4, [2, 3], 16384),
+                                 ("reduce_max_c", 2, [1], 25088), ("reduce_sum_all", 1, [0, 1, 2, 3], 1)]:
+        need = lib.shdw_hip_reduce_workspace_bytes(4, I(shp), len(axes), I(axes))
+        ws = dev.buf(nbytes=max(need, 16))
+        ms = time_batch(dev, lambda k: lib.shdw_hip_reduce(op, 4, I(shp), len(axes), I(axes), A[k].ptr,
+                                                           Y[k].ptr, ws.ptr, need, st), SETS)
+        add(3, name, 4 * NBIG + 4 * outs, ms, NBIG)
+
+    # cfg 5: ResNet bottleneck tail on [64,1024,14,14]
+    n5, C5, in5 = 12845056, 1024, 196
+    g5, b5 = dev.buf(uniform(502, C5, 0.5, 1.5)), dev.buf(uniform(503, C5, -0.1, 0.1))
+    M = [dev.buf(nbytes=4 * 65536) for _ in range(SETS)]
+    ms = time_batch(dev, lambda k: lib.shdw_hip_scale_bias(n5, C5, in5, A[k].ptr, g5.ptr, b5.ptr, 0,
+                                                           Y[k].ptr, st), SETS)
+    add(5, "scale", 8 * n5 + 8 * C5, ms, n5)
+
+    def eltwise_sum(k):
+        ptrs = (ctypes.c_void_p * 2)(A[k].ptr, A[(k + 1) % SETS].ptr)
+        return lib.shdw_hip_eltwise(1, 2, ptrs, None, n5, Y[k].ptr, st)
+    ms = time_batch(dev, eltwise_sum, SETS)
+    add(5, "eltwise_sum", 12 * n5, ms, n5)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_activate(1, 0.1, n5, A[k].ptr, Y[k].ptr, st), SETS)
+    add(5, "relu", 8 * n5, ms, n5)
+    sh5, ax5 = [64, 1024, 14, 14], [2, 3]
+    ms = time_batch(dev, lambda k: lib.shdw_hip_reduce(4, 4, I(sh5), 2, I(ax5), A[k].ptr, M[k].ptr,
+                                                       None, 0, st), SETS)
+    add(5, "reduce_avg_hw", 4 * n5 + 4 * 65536, ms, n5)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_scale_residual_relu_rowmean(
+        n5, C5, in5, A[k].ptr, g5.ptr, b5.ptr, A[(k + 1) % SETS].ptr, Y[k].ptr, M[k].ptr, st), SETS)
+    add(5, "fused_tail", 12 * n5 + 8 * C5 + 4 * 65536, ms, n5)
+    for bset in (A, Y):
+        for bb in bset:
+            bb.free()
+
+    # cfg 4: general broadcast; outputs dominate the traffic
+    for tag, sa4, sb4 in [("i", [16, 1, 128, 256], [1, 32, 128, 1]), ("ii", [4, 64, 1, 512], [1, 1, 64, 512]),
+                          ("iii", [128, 1024], [1, 1])]:
+        so4 = [max(p, q) for p, q in zip(sa4, sb4)]
+        na, nb_, no = int(np.prod(sa4)), int(np.prod(sb4)), int(np.prod(so4))
+        a4 = dev.buf(normal(401, na))
+        b4 = dev.buf(uniform(402, nb_, 0.5, 2.0))
+        y4 = [dev.buf(nbytes=4 * no) for _ in range(SETS)]
+        for name, op in [("mul", 2), ("sub", 1), ("div", 3), ("max", 5)]:
+            ms = time_batch(dev, lambda k: lib.shdw_hip_broadcast_binary(
+                op, len(so4), I(sa4), I(sb4), I(so4), a4.ptr, b4.ptr, y4[k].ptr, st), SETS)
+            add(4, "broadcast_%s_%s" % (name, tag), 4 * (na + nb_ + no), ms, no)
+        for bb in y4:
+            bb.free()
+    return rows
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build measures one GPU; the path shards by batch with no "
+                         "exchange, so run one process per GPU (got --gpus %d)" % args.gpus)
+    dev = Dev()
+    ms_per_step, step_bytes, n, roofline, detail, host = headline(dev, args.steps, args.warmup)
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    out = {
+        "metric": "achieved HBM GB/s (algorithmic bytes / time) over the unary-chain step",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1]: fp32 [64,256,56,56] ~N(0,2) seed 201; relu, "
+                               "sigmoid, exp, abs, sqrt(abs), tanh as single ops + fused per-channel "
+                               "Scale+ReLU (7 launches per step)",
+                   "elements": n, "bytes_per_step": step_bytes, "device": dev.info},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "elements_per_s": round(7 * n / (ms_per_step * 1e-3), 1),
+        "roofline": roofline, "step_ops": detail,
+    }
+    if not args.no_configs:
+        out["configs"] = config_table(dev)
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(host, step_bytes, args.cpu_passes)
+        out["speedup_vs_cpu"] = round(value / out["cpu_baseline"]["value"], 1)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -18,8 +18,6 @@
 
 namespace shdw {
 
-constexpr int kRowUnroll = 4;
-
 enum RowMode { kScaleBias = 0, kScaleOnly = 1, kBiasOnly = 2, kPRelu = 3 };
 
 template <int MODE, bool RELU>
@@ -39,57 +37,41 @@ SHDW_DEVICE float row_apply(float x, float s, float b) {
   return r;
 }
 
-// ROWVEC: inner % 4 == 0, so the four lanes of a vector share one row.
+template <int MODE, bool RELU>
+SHDW_DEVICE float row_element(uint32_t e, float x, const float* s, const float* b,
+                              const FastDiv& inner, const FastDiv& num) {
+  const uint32_t row = fd_div(e, inner);
+  const uint32_t c = row - fd_div(row, num) * num.d;
+  const float sv = (MODE != kBiasOnly) ? s[c] : 0.f;
+  const float bv = (MODE == kScaleBias || MODE == kBiasOnly) ? b[c] : 0.f;
+  return row_apply<MODE, RELU>(x, sv, bv);
+}
+
+// One 128-bit vector per lane.  ROWVEC: inner % 4 == 0, so the four elements of
+// a vector share one row and the parameters are fetched once per vector.
 template <int MODE, bool RELU, bool ROWVEC>
 __global__ __launch_bounds__(kBlock) void rowparam_vec_kernel(const float* x, const float* s,
                                                                const float* b, float* y,
                                                                uint32_t n4, uint32_t n,
                                                                FastDiv inner, FastDiv num) {
-  const uint32_t span = kBlock * kRowUnroll;
-  const uint32_t stride = gridDim.x * span;
-  for (uint32_t base = blockIdx.x * span; base < n4; base += stride) {
-    v4f vx[kRowUnroll];
-#pragma unroll
-    for (int u = 0; u < kRowUnroll; ++u) {
-      const uint32_t i = base + u * kBlock + threadIdx.x;
-      if (i < n4) vx[u] = load4_stream(x + 4ull * i);
-    }
-#pragma unroll
-    for (int u = 0; u < kRowUnroll; ++u) {
-      const uint32_t i = base + u * kBlock + threadIdx.x;
-      if (i < n4) {
-        v4f r;
-        if (ROWVEC) {
-          uint32_t row, c;
-          row = fd_div(4 * i, inner);
-          c = row - fd_div(row, num) * num.d;
-          const float sv = (MODE != kBiasOnly) ? s[c] : 0.f;
-          const float bv = (MODE == kScaleBias || MODE == kBiasOnly) ? b[c] : 0.f;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) r[j] = row_apply<MODE, RELU>(vx[u][j], sv, bv);
-        } else {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const uint32_t row = fd_div(4 * i + j, inner);
-            const uint32_t c = row - fd_div(row, num) * num.d;
-            const float sv = (MODE != kBiasOnly) ? s[c] : 0.f;
-            const float bv = (MODE == kScaleBias || MODE == kBiasOnly) ? b[c] : 0.f;
-            r[j] = row_apply<MODE, RELU>(vx[u][j], sv, bv);
-          }
-        }
-        store4_stream(y + 4ull * i, r);
-      }
-    }
-  }
-  if (blockIdx.x == 0) {
-    const uint32_t i = 4 * n4 + threadIdx.x;
-    if (i < n) {
-      const uint32_t row = fd_div(i, inner);
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < n4) {
+    const v4f vx = load4_stream(x + 4ull * i);
+    v4f r;
+    if (ROWVEC) {
+      const uint32_t row = fd_div(4 * i, inner);
       const uint32_t c = row - fd_div(row, num) * num.d;
       const float sv = (MODE != kBiasOnly) ? s[c] : 0.f;
       const float bv = (MODE == kScaleBias || MODE == kBiasOnly) ? b[c] : 0.f;
-      y[i] = row_apply<MODE, RELU>(x[i], sv, bv);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = row_apply<MODE, RELU>(vx[j], sv, bv);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = row_element<MODE, RELU>(4 * i + j, vx[j], s, b, inner, num);
     }
+    store4_stream(y + 4ull * i, r);
+  } else if (i == n4) {
+    for (uint32_t t = 4 * n4; t < n; ++t) y[t] = row_element<MODE, RELU>(t, x[t], s, b, inner, num);
   }
 }
 
@@ -98,14 +80,8 @@ __global__ __launch_bounds__(kBlock) void rowparam_scalar_kernel(const float* x,
                                                                   const float* b, float* y,
                                                                   uint32_t n, FastDiv inner,
                                                                   FastDiv num) {
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
-    const uint32_t row = fd_div(i, inner);
-    const uint32_t c = row - fd_div(row, num) * num.d;
-    const float sv = (MODE != kBiasOnly) ? s[c] : 0.f;
-    const float bv = (MODE == kScaleBias || MODE == kBiasOnly) ? b[c] : 0.f;
-    y[i] = row_apply<MODE, RELU>(x[i], sv, bv);
-  }
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) y[i] = row_element<MODE, RELU>(i, x[i], s, b, inner, num);
 }
 
 template <int MODE, bool RELU>
@@ -115,17 +91,13 @@ static int launch_rowparam(int n, int num, int inner, const float* x, const floa
   const FastDiv fn = make_fastdiv(static_cast<uint32_t>(num));
   if (aligned16(x) && aligned16(y)) {
     const uint32_t n4 = static_cast<uint32_t>(n) / 4;
-    const uint32_t span = kBlock * kRowUnroll;
-    uint32_t grid = (n4 + span - 1) / span;
-    grid = grid < 1 ? 1 : (grid > kMaxStreamGrid ? kMaxStreamGrid : grid);
+    const uint32_t grid = grid_for(n4 + 1);
     if (inner % 4 == 0)
       rowparam_vec_kernel<MODE, RELU, true><<<grid, kBlock, 0, st>>>(x, s, b, y, n4, n, fi, fn);
     else
       rowparam_vec_kernel<MODE, RELU, false><<<grid, kBlock, 0, st>>>(x, s, b, y, n4, n, fi, fn);
   } else {
-    uint32_t grid = (static_cast<uint32_t>(n) + kBlock - 1) / kBlock;
-    grid = grid > kMaxStreamGrid * 4 ? kMaxStreamGrid * 4 : grid;
-    rowparam_scalar_kernel<MODE, RELU><<<grid, kBlock, 0, st>>>(x, s, b, y, n, fi, fn);
+    rowparam_scalar_kernel<MODE, RELU><<<grid_for(n), kBlock, 0, st>>>(x, s, b, y, n, fi, fn);
   }
   return launch_status();
 }
@@ -148,8 +120,8 @@ template <class F, int NDIM, bool AVEC, bool BVEC>
 __global__ __launch_bounds__(kBlock) void bcast_vec_kernel(F f, BcastArgs p, const float* a,
                                                             const float* b, float* y,
                                                             uint32_t n4) {
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n4; i += stride) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < n4) {
     uint32_t e = 4 * i;
     uint32_t oa = 0, ob = 0;
 #pragma unroll
@@ -194,8 +166,8 @@ template <class F>
 __global__ __launch_bounds__(kBlock) void bcast_generic_kernel(F f, BcastGenericArgs p,
                                                                 const float* a, const float* b,
                                                                 float* y, uint32_t n) {
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) {
     uint32_t e = i, oa = 0, ob = 0;
     for (int k = p.ndim - 1; k >= 1; --k) {
       uint32_t q, r;
@@ -213,8 +185,7 @@ __global__ __launch_bounds__(kBlock) void bcast_generic_kernel(F f, BcastGeneric
 template <class F, int NDIM>
 static void launch_bcast_vec(F f, const BcastArgs& p, bool avec, bool bvec, const float* a,
                              const float* b, float* y, uint32_t n4, hipStream_t st) {
-  uint32_t grid = (n4 + kBlock - 1) / kBlock;
-  grid = grid > kMaxStreamGrid * 4 ? kMaxStreamGrid * 4 : grid;
+  const uint32_t grid = grid_for(n4);
   if (avec && bvec)
     bcast_vec_kernel<F, NDIM, true, true><<<grid, kBlock, 0, st>>>(f, p, a, b, y, n4);
   else if (avec)
@@ -265,9 +236,7 @@ static int launch_bcast(F f, const BroadcastPlan& plan, const float* a, const fl
       p.sa[k] = k < nd ? pl.sa[k] : 0;
       p.sb[k] = k < nd ? pl.sb[k] : 0;
     }
-    uint32_t grid = (n + kBlock - 1) / kBlock;
-    grid = grid > kMaxStreamGrid * 4 ? kMaxStreamGrid * 4 : grid;
-    bcast_generic_kernel<F><<<grid, kBlock, 0, st>>>(f, p, a, b, y, n);
+    bcast_generic_kernel<F><<<grid_for(n), kBlock, 0, st>>>(f, p, a, b, y, n);
   }
   return launch_status();
 }

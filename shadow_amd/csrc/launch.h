@@ -8,9 +8,9 @@
 
 namespace shdw {
 
-// Grid cap for the grid-stride streaming kernels: 8 workgroups of 256 lanes per
-// CU on 256 CUs keeps 32 wave64 resident per CU, the most gfx950 holds.
-constexpr uint32_t kMaxStreamGrid = 256 * 8;
+// Workgroups of kBlock (256) lanes needed for `work` lane-tasks.  Counts are
+// int32, so this never exceeds 2^23 + 1 workgroups.
+inline uint32_t grid_for(uint32_t work) { return (work + 255u) / 256u; }
 
 // Shadow checks cudaPeekAtLastError() after every launch
 // (e.g. shadow/core/blas.cu:20); here the error is also cleared so that one bad
