@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kBlock) void bcast_vec_kernel(F f, BcastArgs p, con
     }
     v4f r;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) r[j] = f(va[j], vb[j]);
+    for (int j = 0; j < 4; ++j) r[j] = f(va[j], vb[j], nullptr);
     store4_stream(y + 4ull * i, r);
   }
 }
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(kBlock) void bcast_generic_kernel(F f, BcastGeneric
     }
     oa += e * static_cast<uint32_t>(p.sa[0]);
     ob += e * static_cast<uint32_t>(p.sb[0]);
-    y[i] = f(a[oa], b[ob]);
+    y[i] = f(a[oa], b[ob], nullptr);
   }
 }
 

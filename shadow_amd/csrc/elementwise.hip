@@ -30,23 +30,32 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(F f, const float* a, con
                                                          float* y, uint32_t n4, uint32_t n,
                                                          float alpha) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-  if (i < n4) {
-    v4f va, vb;
+  v4f va, vb;
+  if (i < n4) {  // issue the streaming loads before anything else
     if (NIN >= 1) va = load4_stream(a + 4ull * i);
     if (NIN >= 2) vb = load4_stream(b + 4ull * i);
+  }
+  const uint64_t* tab = nullptr;
+  if (uses_exp_table<F>::value) {
+    __shared__ uint64_t lds_tab[32];
+    if (threadIdx.x < 32) lds_tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
+    __syncthreads();
+    tab = lds_tab;
+  }
+  if (i < n4) {
     v4f r;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const float x = NIN >= 1 ? va[j] : alpha;
       const float w = NIN >= 2 ? vb[j] : alpha;
-      r[j] = f(x, w);
+      r[j] = f(x, w, tab);
     }
     store4_stream(y + 4ull * i, r);
   } else if (i == n4) {
     for (uint32_t t = 4 * n4; t < n; ++t) {
       const float x = NIN >= 1 ? a[t] : alpha;
       const float w = NIN >= 2 ? b[t] : alpha;
-      y[t] = f(x, w);
+      y[t] = f(x, w, tab);
     }
   }
 }
@@ -56,10 +65,11 @@ template <int NIN, class F>
 __global__ __launch_bounds__(kBlock) void ew_scalar_kernel(F f, const float* a, const float* b,
                                                             float* y, uint32_t n, float alpha) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint64_t* tab = uses_exp_table<F>::value ? libm::kExp2fTab : nullptr;
   if (i < n) {
     const float x = NIN >= 1 ? a[i] : alpha;
     const float w = NIN >= 2 ? b[i] : alpha;
-    y[i] = f(x, w);
+    y[i] = f(x, w, tab);
   }
 }
 
@@ -85,17 +95,18 @@ static int launch_ew(F f, int n, const float* a, const float* b, float alpha, fl
 template <class U>
 struct Unary2 {
   U u;
-  SHDW_DEVICE float operator()(float a, float) const { return u(a); }
+  static constexpr bool kExpTable = uses_exp_table<U>::value;
+  SHDW_DEVICE float operator()(float a, float, const uint64_t* tab) const { return u(a, tab); }
 };
 struct Fill {
-  SHDW_DEVICE float operator()(float v, float) const { return v; }
+  SHDW_DEVICE float operator()(float v, float, const uint64_t*) const { return v; }
 };
 struct ScalOp {  // x *= alpha
-  SHDW_DEVICE float operator()(float x, float alpha) const { return x * alpha; }
+  SHDW_DEVICE float operator()(float x, float alpha, const uint64_t*) const { return x * alpha; }
 };
 struct AxpyOp {  // y += alpha * x, multiply then add
   float alpha;
-  SHDW_DEVICE float operator()(float x, float y) const {
+  SHDW_DEVICE float operator()(float x, float y, const uint64_t*) const {
     const float t = alpha * x;
     return y + t;
   }

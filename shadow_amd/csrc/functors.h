@@ -12,50 +12,58 @@
 
 namespace shdw {
 
+// Functors that evaluate exact_expf declare `static constexpr bool kExpTable =
+// true`; the kernels then stage the 32-entry 2^(i/32) table in LDS and pass it
+// as `tab` (nullptr otherwise).
+template <class F, class = void>
+struct uses_exp_table { static constexpr bool value = false; };
+template <class F>
+struct uses_exp_table<F, decltype((void)F::kExpTable)> { static constexpr bool value = F::kExpTable; };
+
 SHDW_DEVICE float sel_max(float a, float b) { return (a < b) ? b : a; }
 SHDW_DEVICE float sel_min(float a, float b) { return (b < a) ? b : a; }
 
 // ---- unary: shadow/core/blas.cpp:151-165 ----
-struct UAbs { SHDW_DEVICE float operator()(float a) const { return __builtin_fabsf(a); } };
-struct USquare { SHDW_DEVICE float operator()(float a) const { return a * a; } };
-struct USqrt { SHDW_DEVICE float operator()(float a) const { return __builtin_sqrtf(a); } };
-struct ULog { SHDW_DEVICE float operator()(float a) const { return logf(a); } };
-struct UExp { SHDW_DEVICE float operator()(float a) const { return libm::exact_expf(a); } };
-struct USin { SHDW_DEVICE float operator()(float a) const { return sinf(a); } };
-struct UCos { SHDW_DEVICE float operator()(float a) const { return cosf(a); } };
-struct UTan { SHDW_DEVICE float operator()(float a) const { return tanf(a); } };
-struct UAsin { SHDW_DEVICE float operator()(float a) const { return asinf(a); } };
-struct UAcos { SHDW_DEVICE float operator()(float a) const { return acosf(a); } };
-struct UAtan { SHDW_DEVICE float operator()(float a) const { return atanf(a); } };
-struct UFloor { SHDW_DEVICE float operator()(float a) const { return __builtin_floorf(a); } };
-struct UCeil { SHDW_DEVICE float operator()(float a) const { return __builtin_ceilf(a); } };
-struct UNeg { SHDW_DEVICE float operator()(float a) const { return -a; } };
-struct UReciprocal { SHDW_DEVICE float operator()(float a) const { return 1 / a; } };
-struct UCopy { SHDW_DEVICE float operator()(float a) const { return a; } };
+struct UAbs { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return __builtin_fabsf(a); } };
+struct USquare { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return a * a; } };
+struct USqrt { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return __builtin_sqrtf(a); } };
+struct ULog { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return logf(a); } };
+struct UExp { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return libm::exact_expf(a, tab); } };
+struct USin { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return sinf(a); } };
+struct UCos { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return cosf(a); } };
+struct UTan { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return tanf(a); } };
+struct UAsin { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return asinf(a); } };
+struct UAcos { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return acosf(a); } };
+struct UAtan { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return atanf(a); } };
+struct UFloor { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return __builtin_floorf(a); } };
+struct UCeil { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return __builtin_ceilf(a); } };
+struct UNeg { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return -a; } };
+struct UReciprocal { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return 1 / a; } };
+struct UCopy { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return a; } };
 
 // ---- binary: shadow/core/blas.cpp:114-120, kernels/binary.cpp:9-28 ----
-struct BAdd { SHDW_DEVICE float operator()(float a, float b) const { return a + b; } };
-struct BSub { SHDW_DEVICE float operator()(float a, float b) const { return a - b; } };
-struct BMul { SHDW_DEVICE float operator()(float a, float b) const { return a * b; } };
-struct BDiv { SHDW_DEVICE float operator()(float a, float b) const { return a / b; } };
-struct BPow { SHDW_DEVICE float operator()(float a, float b) const { return powf(a, b); } };
-struct BMax { SHDW_DEVICE float operator()(float a, float b) const { return sel_max(a, b); } };
-struct BMin { SHDW_DEVICE float operator()(float a, float b) const { return sel_min(a, b); } };
+struct BAdd { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return a + b; } };
+struct BSub { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return a - b; } };
+struct BMul { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return a * b; } };
+struct BDiv { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return a / b; } };
+struct BPow { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return powf(a, b); } };
+struct BMax { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return sel_max(a, b); } };
+struct BMin { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return sel_min(a, b); } };
 
 // ---- activations: shadow/operators/kernels/activate.cpp:9-31 ----
-struct ARelu { SHDW_DEVICE float operator()(float x, float) const { return x > 0 ? x : 0; } };
-struct ALeaky { SHDW_DEVICE float operator()(float x, float s) const { return x > 0 ? x : s * x; } };
-struct ASigmoid { SHDW_DEVICE float operator()(float x, float) const { return libm::exact_sigmoidf(x); } };
-struct ASoftPlus { SHDW_DEVICE float operator()(float x, float) const { return log1pf(libm::exact_expf(x)); } };
-struct ATanh { SHDW_DEVICE float operator()(float x, float) const { return libm::exact_tanhf(x); } };
-struct ARelu6 { SHDW_DEVICE float operator()(float x, float) const { return x < 0 ? 0 : (x > 6 ? 6 : x); } };
+struct ARelu { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return x > 0 ? x : 0; } };
+struct ALeaky { SHDW_DEVICE float operator()(float x, float s, const uint64_t* tab) const { return x > 0 ? x : s * x; } };
+struct ASigmoid { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_sigmoidf(x, tab); } };
+struct ASoftPlus { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return log1pf(libm::exact_expf(x, tab)); } };
+struct ATanh { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_tanhf(x); } };
+struct ARelu6 { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return x < 0 ? 0 : (x > 6 ? 6 : x); } };
 struct AHardSwish {
-  SHDW_DEVICE float operator()(float x, float) const {
+  SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const {
     return x < -3 ? 0 : (x > 3 ? x : (x * (x + 3) / 6.f));
   }
 };
 struct AGelu {
-  SHDW_DEVICE float operator()(float x, float) const {
+  SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const {
     return 0.5f * x * (1 + erff(0.707107f * x));
   }
 };

@@ -46,16 +46,11 @@ SHDW_LIBM_TABLE uint64_t kExp2fTab[32] = {
     0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
     0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
 
-SHDW_LIBM_FN float exact_expf(float x) {
-  const uint32_t ux = f2u(x);
-  const uint32_t abstop = (ux >> 20) & 0x7ff;
-  if (abstop >= 0x42b) {  // |x| >= 88 or x is NaN
-    if (ux == 0xff800000u) return 0.0f;
-    if (abstop >= 0x7f8) return x + x;
-    if (x > 0x1.62e42ep6f) return __builtin_inff();  // overflow
-    if (x < -0x1.9fe368p6f) return 0.0f;             // underflow to zero
-    if (x < -0x1.9d1d9ep6f) return 0x1p-149f;        // smallest subnormal
-  }
+// `tab` is kExp2fTab or a copy of it in faster memory (the kernels stage it in
+// LDS so that the lookup does not queue behind the streaming HBM traffic).
+SHDW_LIBM_FN float exact_expf(float x, const uint64_t* tab) {
+  // Main path, evaluated for every input (its result is discarded for the
+  // out-of-range inputs handled below; nothing in it can trap).
   const double InvLn2N = 0x1.71547652b82fep+5;  // 32 / ln 2
   const double Shift = 0x1.8p+52;
   const double xd = static_cast<double>(x);
@@ -64,7 +59,7 @@ SHDW_LIBM_FN float exact_expf(float x) {
   const uint64_t ki = d2u(kd);
   kd -= Shift;
   const double r = __builtin_fma(InvLn2N, xd, -kd);
-  const double s = u2d(kExp2fTab[ki & 31] + (ki << 47));
+  const double s = u2d(tab[ki & 31] + (ki << 47));
   const double c0 = 0x1.c6af84b912394p-20, c1 = 0x1.ebfce50fac4f3p-13,
                c2 = 0x1.62e42ff0c52d6p-6;
   const double p = __builtin_fma(c0, r, c1);
@@ -72,7 +67,17 @@ SHDW_LIBM_FN float exact_expf(float x) {
   double y = __builtin_fma(c2, r, 1.0);
   y = __builtin_fma(p, r2, y);
   y = y * s;
-  return static_cast<float>(y);
+  float res = static_cast<float>(y);
+
+  const uint32_t ux = f2u(x);
+  const uint32_t abstop = (ux >> 20) & 0x7ff;
+  if (abstop >= 0x42b) {  // |x| >= 88 or x is NaN: rare, one skipped block
+    if (x > 0x1.62e42ep6f) res = __builtin_inff();        // overflow
+    if (x < -0x1.9d1d9ep6f) res = 0x1p-149f;              // smallest subnormal
+    if (x < -0x1.9fe368p6f) res = 0.0f;                   // underflow to zero (also -inf)
+    if (abstop >= 0x7f8 && ux != 0xff800000u) res = x + x;  // +inf, NaN
+  }
+  return res;
 }
 
 SHDW_LIBM_FN float exact_expm1f(float x) {
@@ -154,36 +159,84 @@ SHDW_LIBM_FN float exact_expm1f(float x) {
   return y;
 }
 
+// tanhf without divergent control flow.  s_tanhf.c calls expm1f only with
+// a = 2|x| in [2, 44) or a = -2|x| in (-2, -2^-54], so only these expm1f cases
+// can occur: the 2^-25 early return, k = 0, k = -1, k <= -2 (a < 0) and
+// 3 <= k <= 63 (a > 0).  Every case is evaluated with the same operations in the
+// same order as the library and the applicable one is selected.
 SHDW_LIBM_FN float exact_tanhf(float x) {
-  const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
+  const float one = 1.0f, two = 2.0f;
+  const float ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f;
+  const float invln2 = 1.4426950216e+00f;
+  const float Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f,
+              Q4 = 4.0082177293e-06f, Q5 = -2.0109921195e-07f;
   const uint32_t jx = f2u(x);
   const uint32_t ix = jx & 0x7fffffffu;
-  const bool neg = (jx >> 31) != 0;
-  float t, z;
-  if (ix >= 0x7f800000u) {
-    if (!neg) return one / x + one;
-    return one / x - one;
-  }
-  if (ix < 0x41b00000u) {  // |x| < 22
-    if (ix == 0) return x;
-    if (ix < 0x24000000u) return x * (one + x);  // |x| < 2^-55
-    const float ax = u2f(ix);
-    if (ix >= 0x3f800000u) {
-      t = exact_expm1f(two * ax);
-      z = one - two / (t + two);
-    } else {
-      t = exact_expm1f(-two * ax);
-      z = -t / (t + two);
-    }
-  } else {
-    z = one - tiny;
-  }
-  return neg ? -z : z;
+  const bool big = ix >= 0x3f800000u;  // |x| >= 1: expm1f(+2|x|), else expm1f(-2|x|)
+  const float ax = u2f(ix);
+  const float a = big ? two * ax : -two * ax;  // argument of expm1f
+  const uint32_t ha = f2u(a) & 0x7fffffffu;
+  const bool aneg = !big;
+
+  // --- expm1f(a): argument reduction ---
+  const bool reduce = ha > 0x3eb17218u;   // |a| > 0.5 ln2
+  const bool unit_k = ha < 0x3F851592u;   // |a| < 1.5 ln2  ->  k = +-1
+  const int32_t kgen = static_cast<int32_t>(invln2 * a + (aneg ? -0.5f : 0.5f));
+  int32_t k = unit_k ? (aneg ? -1 : 1) : kgen;
+  k = reduce ? k : 0;
+  const float tk = static_cast<float>(k);
+  // k = +-1 uses hi = a -+ ln2_hi, lo = +-ln2_lo, which is what t*ln2_hi and
+  // t*ln2_lo give for t = +-1 (both products exact).
+  const float hi = a - tk * ln2_hi;
+  const float lo = tk * ln2_lo;
+  const float xr = reduce ? hi - lo : a;
+  const float c = reduce ? (hi - xr) - lo : 0.0f;
+
+  // --- primary range ---
+  const float hfx = 0.5f * xr;
+  const float hxs = xr * hfx;
+  const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+  const float t3 = 3.0f - r1 * hfx;
+  float e = hxs * ((r1 - t3) / (6.0f - xr * t3));
+  const float res_k0 = xr - (xr * e - hxs);
+  e = (xr * (e - c) - c);
+  e -= hxs;
+  const float res_km1 = 0.5f * (xr - e) - 0.5f;
+  // k <= -2 or k > 56: y = 1 - (e - x); 2 <= k < 23: y = (1 - 2^-k) - (e - x)
+  const bool mid = (k >= 2) && (k < 23);
+  const uint32_t ksh = static_cast<uint32_t>(k) & 31u;
+  const float t_lo = mid ? u2f(0x3f800000u - (0x1000000u >> ksh)) : one;
+  const float y_a = t_lo - (e - xr);
+  // 23 <= k <= 56: y = (x - (e + 2^-k)) + 1
+  const float t_hi = u2f(static_cast<uint32_t>(0x7f - k) << 23);
+  float y_b = xr - (e + t_hi);
+  y_b += one;
+  const bool hi_k = (k >= 23) && (k <= 56);
+  float yk = hi_k ? y_b : y_a;
+  yk = u2f(f2u(yk) + (static_cast<uint32_t>(k) << 23));  // scale by 2^k
+  const float res_gen = (mid || hi_k) ? yk : yk - one;
+  float t = (k == 0) ? res_k0 : ((k == -1) ? res_km1 : res_gen);
+  t = (ha < 0x33000000u) ? a : t;  // |a| < 2^-25: expm1f returns a
+
+  // --- tanhf ---
+  const float q = (big ? two : t) / (t + two);
+  float z = big ? one - q : -q;
+  z = (ix < 0x41b00000u) ? z : one;           // |x| >= 22 (and +-inf): 1 - tiny == 1
+  float res = (jx >> 31) ? -z : z;
+  res = (ix < 0x24000000u) ? x * (one + x) : res;  // |x| < 2^-55, including +-0
+  res = (ix > 0x7f800000u) ? x + x : res;          // NaN
+  return res;
 }
 
 // 1 / (1 + exp(-x)) in fp32, the way shadow/operators/kernels/activate.cpp:16
 // writes it.
-SHDW_LIBM_FN float exact_sigmoidf(float x) { return 1.0f / (1.0f + exact_expf(-x)); }
+SHDW_LIBM_FN float exact_sigmoidf(float x, const uint64_t* tab) {
+  return 1.0f / (1.0f + exact_expf(-x, tab));
+}
+#if !defined(__HIPCC__)
+SHDW_LIBM_FN float exact_expf(float x) { return exact_expf(x, kExp2fTab); }
+SHDW_LIBM_FN float exact_sigmoidf(float x) { return exact_sigmoidf(x, kExp2fTab); }
+#endif
 
 }  // namespace libm
 }  // namespace shdw
