@@ -151,3 +151,160 @@ class Buffer:
             self.free()
         except Exception:
             pass
+
+
+# --------------------------------------------------------------------------
+# libshadow_host.so: the C++ operator layer behind its C facade (host/src/capi.cpp)
+# --------------------------------------------------------------------------
+_host = None
+
+HOST_SIGNATURES = {
+    "shdw_host_last_error": (ctypes.c_char_p, []),
+    "shdw_host_kernel_keys": (_I, [ctypes.c_char_p, _Z]),
+    "shdw_host_operator_keys": (_I, [ctypes.c_char_p, _Z]),
+    "shdw_host_workspace_create": (_V, [ctypes.c_char_p, _I]),
+    "shdw_host_workspace_destroy": (None, [_V]),
+    "shdw_host_sync": (_I, [_V]),
+    "shdw_host_blob_create": (_I, [_V, ctypes.c_char_p, ctypes.c_char_p]),
+    "shdw_host_blob_set": (_I, [_V, ctypes.c_char_p, c_int_p, _I, _V]),
+    "shdw_host_blob_shape": (_I, [_V, ctypes.c_char_p, c_int_p, _I]),
+    "shdw_host_blob_get": (_I, [_V, ctypes.c_char_p, _V, _I]),
+    "shdw_host_opparam_create": (_V, [ctypes.c_char_p, ctypes.c_char_p]),
+    "shdw_host_opparam_destroy": (None, [_V]),
+    "shdw_host_opparam_add_bottom": (None, [_V, ctypes.c_char_p]),
+    "shdw_host_opparam_add_top": (None, [_V, ctypes.c_char_p]),
+    "shdw_host_opparam_arg_i": (None, [_V, ctypes.c_char_p, _I]),
+    "shdw_host_opparam_arg_f": (None, [_V, ctypes.c_char_p, _F]),
+    "shdw_host_opparam_arg_s": (None, [_V, ctypes.c_char_p, ctypes.c_char_p]),
+    "shdw_host_opparam_arg_vi": (None, [_V, ctypes.c_char_p, c_int_p, _I]),
+    "shdw_host_opparam_arg_vf": (None, [_V, ctypes.c_char_p, c_float_p, _I]),
+    "shdw_host_op_create": (_V, [_V, _V]),
+    "shdw_host_op_destroy": (None, [_V]),
+    "shdw_host_op_run": (_I, [_V, _V]),
+    "shdw_host_op_debug_log": (_I, [_V, _V, ctypes.c_char_p, _Z]),
+    "shdw_host_probe_create_kernel": (_I, [ctypes.c_char_p, _I]),
+    "shdw_host_probe_argument": (_I, [ctypes.c_char_p, ctypes.c_char_p]),
+}
+
+
+class ShadowError(RuntimeError):
+    """A CHECK / LOG(FATAL) of the C++ layer fired (std::runtime_error there)."""
+
+
+def host():
+    global _host
+    if _host is None:
+        hip()  # resolves libshadow_hip.so first
+        path = os.path.join(LIB_DIR, "libshadow_host.so")
+        if not os.path.exists(path):
+            raise RuntimeError("%s is missing: build it with `python -m shadow_amd.build host`" % path)
+        lib = ctypes.CDLL(path)
+        for name, (res, args) in HOST_SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _host = lib
+    return _host
+
+
+def host_check(ok):
+    if not ok:
+        raise ShadowError(host().shdw_host_last_error().decode())
+
+
+class Workspace:
+    """A Shadow::Workspace with a GPU context, plus blob and operator helpers."""
+
+    def __init__(self, backend_type="Native", device_id=0):
+        self.lib = host()
+        self.ptr = self.lib.shdw_host_workspace_create(backend_type.encode(), device_id)
+        host_check(self.ptr)
+        self._ops = []
+
+    def close(self):
+        for op in self._ops:
+            op.close()
+        self._ops = []
+        if self.ptr:
+            self.lib.shdw_host_workspace_destroy(self.ptr)
+            self.ptr = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def set_blob(self, name, array, dtype="float"):
+        array = np.ascontiguousarray(array, dtype=np.float32 if dtype == "float" else np.int32)
+        host_check(self.lib.shdw_host_blob_create(self.ptr, name.encode(), dtype.encode()) == 0)
+        shape = ints(array.shape) if array.ndim else ints([1])
+        rank = array.ndim if array.ndim else 1
+        host_check(self.lib.shdw_host_blob_set(self.ptr, name.encode(), shape, rank,
+                                               array.ctypes.data) == 0)
+
+    def blob_shape(self, name):
+        shape = (ctypes.c_int * 16)()
+        rank = self.lib.shdw_host_blob_shape(self.ptr, name.encode(), shape, 16)
+        host_check(rank >= 0)
+        return [shape[i] for i in range(rank)]
+
+    def get_blob(self, name, dtype=np.float32):
+        shape = self.blob_shape(name)
+        count = int(np.prod(shape, dtype=np.int64)) if shape else 1
+        out = np.empty(count, dtype)
+        host_check(self.lib.shdw_host_blob_get(self.ptr, name.encode(), out.ctypes.data, count) == 0)
+        return out.reshape(shape)
+
+    def sync(self):
+        host_check(self.lib.shdw_host_sync(self.ptr) == 0)
+
+    def create_op(self, op_type, bottoms, tops, args=None, name=None):
+        op = Op(self, op_type, bottoms, tops, args or {}, name or op_type.lower())
+        self._ops.append(op)
+        return op
+
+
+class Op:
+    """One Shadow operator.  `args` values: int/bool -> s_i, float -> s_f,
+    str -> s_s, list of int -> v_i, list of float -> v_f."""
+
+    def __init__(self, ws, op_type, bottoms, tops, args, name):
+        lib = ws.lib
+        self.ws = ws
+        param = lib.shdw_host_opparam_create(op_type.encode(), name.encode())
+        try:
+            for b in bottoms:
+                lib.shdw_host_opparam_add_bottom(param, b.encode())
+            for t in tops:
+                lib.shdw_host_opparam_add_top(param, t.encode())
+            for key, val in args.items():
+                k = key.encode()
+                if isinstance(val, (bool, int, np.integer)):
+                    lib.shdw_host_opparam_arg_i(param, k, int(val))
+                elif isinstance(val, (float, np.floating)):
+                    lib.shdw_host_opparam_arg_f(param, k, float(val))
+                elif isinstance(val, str):
+                    lib.shdw_host_opparam_arg_s(param, k, val.encode())
+                elif len(val) and isinstance(val[0], (float, np.floating)):
+                    arr = (ctypes.c_float * len(val))(*[float(v) for v in val])
+                    lib.shdw_host_opparam_arg_vf(param, k, arr, len(val))
+                else:
+                    lib.shdw_host_opparam_arg_vi(param, k, ints(val), len(val))
+            self.ptr = lib.shdw_host_op_create(ws.ptr, param)
+        finally:
+            lib.shdw_host_opparam_destroy(param)
+        host_check(self.ptr)
+
+    def run(self):
+        host_check(self.ws.lib.shdw_host_op_run(self.ws.ptr, self.ptr) == 0)
+
+    def debug_log(self):
+        buf = ctypes.create_string_buffer(4096)
+        host_check(self.ws.lib.shdw_host_op_debug_log(self.ws.ptr, self.ptr, buf, 4096) >= 0)
+        return buf.value.decode()
+
+    def close(self):
+        if self.ptr:
+            self.ws.lib.shdw_host_op_destroy(self.ptr)
+            self.ptr = None

@@ -1,0 +1,197 @@
+// C facade over the C++ operator layer, for callers without a C++ toolchain
+// (the Python tests, the smoke check).  It does what Native::Initial / Native::Run
+// do around the operators (shadow/backends/native/native.cpp:171-172, 78-94):
+// create operators from an OpParam, look their bottom/top blobs up by name, call
+// Operator::Run.  Every function catches the std::runtime_error that a failed
+// CHECK throws and reports it through shdw_host_last_error().
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "shadow/kernel.hpp"
+#include "shadow/operator.hpp"
+#include "shadow/workspace.hpp"
+
+using namespace Shadow;
+
+namespace {
+
+thread_local std::string g_error;
+
+template <typename F>
+int guarded(F&& body) {
+  try {
+    body();
+    return 0;
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return -1;
+  }
+}
+
+Workspace* WS(void* p) { return static_cast<Workspace*>(p); }
+shadow::OpParam* OP(void* p) { return static_cast<shadow::OpParam*>(p); }
+
+struct OpHandle {
+  std::shared_ptr<Operator> op;
+};
+
+int join(const std::vector<std::string>& keys, char* buf, size_t n) {
+  std::string all;
+  for (const auto& k : keys) all += (all.empty() ? "" : "\n") + k;
+  if (buf != nullptr && n > 0) {
+    std::strncpy(buf, all.c_str(), n - 1);
+    buf[n - 1] = '\0';
+  }
+  return static_cast<int>(all.size());
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* shdw_host_last_error(void) { return g_error.c_str(); }
+
+int shdw_host_kernel_keys(char* buf, size_t n) { return join(KernelRegistry()->Keys(), buf, n); }
+int shdw_host_operator_keys(char* buf, size_t n) { return join(OperatorRegistry()->Keys(), buf, n); }
+
+void* shdw_host_workspace_create(const char* backend_type, int device_id) {
+  Workspace* ws = nullptr;
+  guarded([&] {
+    ArgumentHelper args;
+    args.AddSingleArgument<std::string>("backend_type", backend_type ? backend_type : "");
+    args.AddSingleArgument<int>("device_id", device_id);
+    ws = new Workspace(args);
+  });
+  return ws;
+}
+
+void shdw_host_workspace_destroy(void* ws) { delete WS(ws); }
+
+int shdw_host_sync(void* ws) {
+  return guarded([&] { WS(ws)->Ctx()->synchronize(); });
+}
+
+int shdw_host_blob_create(void* ws, const char* name, const char* dtype) {
+  return guarded([&] { CHECK_NOTNULL(WS(ws)->CreateBlob(name, std::string(dtype))); });
+}
+
+// reshape, then (data != NULL) copy count() elements in from the host
+int shdw_host_blob_set(void* ws, const char* name, const int* shape, int rank, const void* data) {
+  return guarded([&] {
+    auto blob = WS(ws)->GetBlob(name);
+    CHECK_NOTNULL(blob) << "Unknown blob: " << name;
+    blob->reshape(VecInt(shape, shape + rank));
+    if (data != nullptr) {
+      if (blob->data_type() == DataType::kF32) blob->set_data<float>(data, blob->count());
+      else if (blob->data_type() == DataType::kI32) blob->set_data<std::int32_t>(data, blob->count());
+      else LOG(FATAL) << "shdw_host_blob_set: float and int32 blobs only";
+      WS(ws)->Ctx()->synchronize();  // the host buffer may go away after return
+    }
+  });
+}
+
+// Writes up to max_rank dims; returns the rank, or -1 on error.
+int shdw_host_blob_shape(void* ws, const char* name, int* shape, int max_rank) {
+  int rank = -1;
+  guarded([&] {
+    auto blob = WS(ws)->GetBlob(name);
+    CHECK_NOTNULL(blob) << "Unknown blob: " << name;
+    rank = blob->num_axes();
+    for (int n = 0; n < rank && n < max_rank; ++n) shape[n] = blob->shape(n);
+  });
+  return rank;
+}
+
+int shdw_host_blob_get(void* ws, const char* name, void* out, int count) {
+  return guarded([&] {
+    auto blob = WS(ws)->GetBlob(name);
+    CHECK_NOTNULL(blob) << "Unknown blob: " << name;
+    if (blob->data_type() == DataType::kF32) blob->get_data<float>(out, count);
+    else if (blob->data_type() == DataType::kI32) blob->get_data<std::int32_t>(out, count);
+    else LOG(FATAL) << "shdw_host_blob_get: float and int32 blobs only";
+    WS(ws)->Ctx()->synchronize();
+  });
+}
+
+void* shdw_host_opparam_create(const char* type, const char* name) {
+  auto* p = new shadow::OpParam();
+  p->set_type(type);
+  p->set_name(name);
+  return p;
+}
+void shdw_host_opparam_destroy(void* p) { delete OP(p); }
+void shdw_host_opparam_add_bottom(void* p, const char* name) { OP(p)->add_bottom(name); }
+void shdw_host_opparam_add_top(void* p, const char* name) { OP(p)->add_top(name); }
+void shdw_host_opparam_arg_i(void* p, const char* name, int v) { add_s_i(OP(p), name, v); }
+void shdw_host_opparam_arg_f(void* p, const char* name, float v) { add_s_f(OP(p), name, v); }
+void shdw_host_opparam_arg_s(void* p, const char* name, const char* v) { add_s_s(OP(p), name, v); }
+void shdw_host_opparam_arg_vi(void* p, const char* name, const int* v, int n) {
+  add_v_i(OP(p), name, std::vector<int>(v, v + n));
+}
+void shdw_host_opparam_arg_vf(void* p, const char* name, const float* v, int n) {
+  add_v_f(OP(p), name, std::vector<float>(v, v + n));
+}
+
+// Runs the operator's constructor (argument checks, output blob creation,
+// kernel lookup).  NULL on error.
+void* shdw_host_op_create(void* ws, void* opparam) {
+  OpHandle* h = nullptr;
+  guarded([&] {
+    auto op = CreateOperator(*OP(opparam), WS(ws));
+    h = new OpHandle{op};
+  });
+  return h;
+}
+void shdw_host_op_destroy(void* op) { delete static_cast<OpHandle*>(op); }
+
+// One iteration of the backend's op loop for this operator; asynchronous.
+int shdw_host_op_run(void* ws, void* op) {
+  return guarded([&] {
+    auto& oper = static_cast<OpHandle*>(op)->op;
+    std::vector<std::shared_ptr<Blob>> inputs, outputs;
+    for (const auto& name : oper->op_param().bottom()) {
+      auto blob = WS(ws)->GetBlob(name);
+      CHECK_NOTNULL(blob) << oper->name() << ": Failed to find input blob " << name;
+      inputs.push_back(blob);
+    }
+    for (const auto& name : oper->op_param().top()) {
+      auto blob = WS(ws)->GetBlob(name);
+      CHECK_NOTNULL(blob) << oper->name() << ": Failed to find output blob " << name;
+      outputs.push_back(blob);
+    }
+    oper->Run(inputs, outputs);
+  });
+}
+
+int shdw_host_op_debug_log(void* ws, void* op, char* buf, size_t n) {
+  int len = -1;
+  guarded([&] {
+    auto& oper = static_cast<OpHandle*>(op)->op;
+    std::vector<std::shared_ptr<Blob>> inputs, outputs;
+    for (const auto& name : oper->op_param().bottom()) inputs.push_back(WS(ws)->GetBlob(name));
+    for (const auto& name : oper->op_param().top()) outputs.push_back(WS(ws)->GetBlob(name));
+    len = join({oper->debug_log(inputs, outputs)}, buf, n);
+  });
+  return len;
+}
+
+// Host-only probes of ArgumentHelper / CreateKernel / CreateOperator error paths
+// (no device needed): each returns 0 when the call succeeded, -1 when it threw.
+int shdw_host_probe_create_kernel(const char* op_type, int gpu) {
+  return guarded([&] { CreateKernel(op_type, gpu ? DeviceType::kGPU : DeviceType::kCPU); });
+}
+int shdw_host_probe_argument(const char* kind, const char* ask_as) {
+  return guarded([&] {
+    ArgumentHelper args;
+    if (std::string(kind) == "int") args.AddSingleArgument<int>("x", 3);
+    if (std::string(kind) == "float") args.AddSingleArgument<float>("x", 3.f);
+    if (std::string(kind) == "string") args.AddSingleArgument<std::string>("x", "3");
+    if (std::string(ask_as) == "int") args.GetSingleArgument<int>("x", 0);
+    if (std::string(ask_as) == "float") args.GetSingleArgument<float>("x", 0.f);
+    if (std::string(ask_as) == "string") args.GetSingleArgument<std::string>("x", "");
+    if (std::string(ask_as) == "dup") args.AddSingleArgument<int>("x", 4);
+  });
+}
+
+}  // extern "C"

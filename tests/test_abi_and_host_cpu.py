@@ -1,0 +1,129 @@
+"""CPU-only checks: the C-ABI library loads and exports every symbol the header
+declares, the launch planners produce the expected collapsed forms, and the host
+layer's registries / argument handling behave like the reference's.  No kernel is
+launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import shadow_amd
+from shadow_amd import ints
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "shadow_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(shdw_hip_\w+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    lib = shadow_amd.hip()
+    names = declared_symbols()
+    assert len(names) >= 35
+    for name in names:
+        assert hasattr(lib, name), name + " is declared in include/shadow_hip.h but not exported"
+        assert name in shadow_amd.SIGNATURES, name + " has no ctypes signature"
+    assert sorted(shadow_amd.SIGNATURES) == names
+
+
+def test_error_strings():
+    lib = shadow_amd.hip()
+    assert lib.shdw_hip_error_string(0) == b"success"
+    assert b"invalid argument" in lib.shdw_hip_error_string(-1)
+    assert b"unsupported" in lib.shdw_hip_error_string(-2)
+    assert b"workspace" in lib.shdw_hip_error_string(-3)
+
+
+def plan_broadcast(a, b):
+    rank = max(len(a), len(b))
+    a = [1] * (rank - len(a)) + list(a)
+    b = [1] * (rank - len(b)) + list(b)
+    out = [max(x, y) for x, y in zip(a, b)]
+    dims, sa, sb = (ctypes.c_int * 8)(), (ctypes.c_int * 8)(), (ctypes.c_int * 8)()
+    n = shadow_amd.hip().shdw_hip_plan_broadcast(rank, ints(a), ints(b), ints(out), dims, sa, sb)
+    return n, list(dims[:max(n, 0)]), list(sa[:max(n, 0)]), list(sb[:max(n, 0)])
+
+
+def test_broadcast_plans_of_the_benchmark_shapes():
+    # channel broadcast: [8,64,112,112] + [1,64,1,1] -> [8, 64, 12544]
+    assert plan_broadcast([8, 64, 112, 112], [1, 64, 1, 1]) == (3, [8, 64, 12544], [802816, 12544, 1], [0, 1, 0])
+    # stays 4-d
+    assert plan_broadcast([16, 1, 128, 256], [1, 32, 128, 1]) == (
+        4, [16, 32, 128, 256], [32768, 0, 256, 1], [0, 128, 1, 0])
+    assert plan_broadcast([4, 64, 1, 512], [64, 512]) == (3, [256, 64, 512], [512, 0, 1], [0, 512, 1])
+    assert plan_broadcast([128, 1024], [1]) == (1, [131072], [1], [0])
+    assert plan_broadcast([5, 3], [5, 3]) == (1, [15], [1], [1])
+    assert plan_broadcast([1, 1], [1]) == (0, [], [], [])
+    assert plan_broadcast([2, 1], [3]) == (2, [2, 3], [1, 0], [0, 1])
+
+
+def test_broadcast_plan_rejects_bad_shapes():
+    lib = shadow_amd.hip()
+    d = (ctypes.c_int * 8)()
+    assert lib.shdw_hip_plan_broadcast(2, ints([2, 3]), ints([2, 2]), ints([2, 3]), d, d, d) == -1
+    assert lib.shdw_hip_plan_broadcast(1, ints([3]), ints([1]), ints([4]), d, d, d) == -1
+    assert lib.shdw_hip_plan_broadcast(1, ints([0]), ints([1]), ints([1]), d, d, d) == -1
+    nine_a, nine_b = [2, 1] * 4 + [2], [1, 2] * 4 + [1]
+    assert lib.shdw_hip_plan_broadcast(9, ints(nine_a), ints(nine_b), ints([2] * 9), d, d, d) == -2
+
+
+def plan_reduce(shape, axes):
+    out = [ctypes.c_int() for _ in range(5)]
+    rc = shadow_amd.hip().shdw_hip_plan_reduce(len(shape), ints(shape), len(axes), ints(axes),
+                                               *[ctypes.byref(o) for o in out])
+    return rc, [o.value for o in out]
+
+
+def test_reduce_plans_of_the_benchmark_shapes():
+    ROWS, STRIDED, GENERIC = 0, 1, 2
+    rc, (kind, outer, red, inner, splits) = plan_reduce([32, 512, 28, 28], [2, 3])
+    assert (rc, kind, outer, red, inner, splits) == (0, ROWS, 16384, 784, 1, 1)
+    rc, (kind, outer, red, inner, splits) = plan_reduce([32, 512, 28, 28], [1])
+    assert (rc, kind, outer, red, inner) == (0, STRIDED, 32, 512, 784) and splits > 1
+    rc, (kind, outer, red, inner, splits) = plan_reduce([32, 512, 28, 28], [0, 1, 2, 3])
+    assert (rc, kind, outer, red, inner) == (0, ROWS, 1, 12845056, 1) and splits > 64
+    rc, (kind, outer, red, inner, splits) = plan_reduce([64, 1024, 14, 14], [2, 3])
+    assert (rc, kind, outer, red, inner, splits) == (0, ROWS, 65536, 196, 1, 1)
+    assert plan_reduce([2, 3, 4, 5], [0, 2])[1][0] == GENERIC
+    assert plan_reduce([2, 3, 4, 5], [3, 2])[1][0] == GENERIC  # list order is not memory order
+    assert plan_reduce([6, 1, 5], [1])[1][:4] == [STRIDED, 1, 1, 30]
+    assert plan_reduce([2, 3], [-1])[0] == -1
+    assert plan_reduce([2, 3], [1, 1])[0] == -1
+    assert plan_reduce([2, 3], [2])[0] == -1
+    lib = shadow_amd.hip()
+    assert lib.shdw_hip_reduce_workspace_bytes(4, ints([32, 512, 28, 28]), 2, ints([2, 3])) == 0
+    assert lib.shdw_hip_reduce_workspace_bytes(1, ints([1 << 24]), 1, ints([0])) % 16 == 0
+
+
+def keys(fn):
+    buf = ctypes.create_string_buffer(8192)
+    fn(buf, 8192)
+    return buf.value.decode().split("\n")
+
+
+def test_registries_hold_exactly_the_gpu_default_kernels():
+    h = shadow_amd.host()
+    assert keys(h.shdw_host_operator_keys) == ["Activate", "Binary", "Eltwise", "Reduce", "Scale", "Unary"]
+    kk = keys(h.shdw_host_kernel_keys)
+    assert kk == ["%sGPU(Default)" % t for t in ["Activate", "Binary", "Eltwise", "Reduce", "Scale", "Unary"]]
+    # a CUDNN flavour would outrank Default; a CPU kernel would be a compute fallback
+    assert not any("CUDNN" in k or "CPU" in k for k in kk)
+
+
+def test_kernel_lookup_and_argument_errors_throw():
+    h = shadow_amd.host()
+    for op in ("Unary", "Binary", "Eltwise", "Reduce", "Activate", "Scale"):
+        assert h.shdw_host_probe_create_kernel(op.encode(), 1) == 0
+        assert h.shdw_host_probe_create_kernel(op.encode(), 0) == -1  # no CPU kernels in this build
+    assert h.shdw_host_probe_create_kernel(b"Conv", 1) == -1
+    assert b"ConvGPU(None) is not registered" in h.shdw_host_last_error()
+    assert h.shdw_host_probe_argument(b"int", b"int") == 0
+    assert h.shdw_host_probe_argument(b"int", b"float") == -1   # present, wrong kind
+    assert h.shdw_host_probe_argument(b"float", b"string") == -1
+    assert h.shdw_host_probe_argument(b"none", b"int") == 0     # absent -> default
+    assert h.shdw_host_probe_argument(b"int", b"dup") == -1
+    assert b"Duplicated argument name" in h.shdw_host_last_error()
