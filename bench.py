@@ -41,6 +41,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-configs", action="store_true", help="skip the per-config table")
     ap.add_argument("--cpu-passes", type=int, default=2)
+    ap.add_argument("--probe", action="store_true",
+                    help="counter probe: 3 launches of a plain copy and of every headline op on "
+                         "the 51.4M tensor, nothing timed, no JSON (run under rocprofv3 --pmc)")
     return ap.parse_args()
 
 
@@ -155,6 +158,27 @@ def headline(dev, steps, warmup):
                 "algorithmic_bytes": ops[dom][1]}
     host = {"x": x_h, "gamma": g_h, "beta": b_h, "shape": shape}
     return ms_per_step, step_bytes, n, roofline, detail, host
+
+
+def probe(dev):
+    """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: the copy kernel moves a
+    known 205,520,896 B each way and calibrates the counters; the other launches
+    are the headline ops on the same tensor."""
+    lib, st = dev.lib, dev.stream
+    n, C, inner = 64 * 256 * 56 * 56, 256, 56 * 56
+    x = dev.buf(normal(201, n, 2.0))
+    g, b = dev.buf(uniform(202, C, 0.5, 1.5)), dev.buf(uniform(203, C, -0.1, 0.1))
+    y = dev.buf(nbytes=4 * n)
+    for _ in range(3):
+        dev.ck(lib.shdw_hip_copy(n, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_activate(1, 0.1, n, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_activate(3, 0.1, n, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_unary(4, n, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_unary(0, n, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_unary(2, n, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_activate(5, 0.1, n, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_scale_bias(n, C, inner, x.ptr, g.ptr, b.ptr, 1, y.ptr, st))
+    dev.sync()
 
 
 def cpu_baseline(host, step_bytes, passes):
@@ -282,6 +306,9 @@ def main():
         raise SystemExit("bench.py: this build measures one GPU; the path shards by batch with no "
                          "exchange, so run one process per GPU (got --gpus %d)" % args.gpus)
     dev = Dev()
+    if args.probe:
+        probe(dev)
+        return
     ms_per_step, step_bytes, n, roofline, detail, host = headline(dev, args.steps, args.warmup)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     out = {
