@@ -66,11 +66,11 @@ enum {
 
 /* ======================= device, stream, allocator ======================= */
 
-/* ref: shadow/core/context.cu:95-110 (check_device: cudaGetDeviceCount) */
+/* ref: shadow/core/context.cu:87-92 (check_device: cudaGetDeviceCount) */
 int shdw_hip_device_count(int* count);
 /* ref: shadow/core/context.cu:15,63 (cudaSetDevice in ctor and switch_device) */
 int shdw_hip_set_device(int device_id);
-/* ref: shadow/core/context.cu:99-108 (cudaGetDeviceProperties for the debug line).
+/* ref: shadow/core/context.cu:93-101 (cudaGetDeviceProperties for the debug line).
  * Writes "name|gcnArch|CUs|clock_khz" into buf (truncated to buf_size). */
 int shdw_hip_device_info(int device_id, char* buf, size_t buf_size);
 /* ref: shadow/core/context.cu:17-21 (cudaStreamCreate) */

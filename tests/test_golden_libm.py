@@ -1,0 +1,41 @@
+"""Known-answer vectors recorded from glibc 2.35 (tests/golden/make_libm_kat.py).
+
+CPU part: the oracle on THIS host must reproduce them, i.e. the host libm is the
+one the vectors came from; if it is not, the GPU-vs-oracle comparisons elsewhere
+are comparisons against a different libm and this test says so.
+GPU part: the bit-exact device restatements reproduce the recorded exp, sigmoid
+and tanh values."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from tests.helpers import assert_bit_exact
+
+KAT = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "libm_glibc235.npz"))
+
+UNARY = {"log": 3, "exp": 4, "sin": 5, "cos": 6, "tan": 7, "asin": 8, "acos": 9, "atan": 10}
+ACT = {"sigmoid": 3, "softplus": 4, "tanh": 5, "gelu": 8}
+
+
+@pytest.mark.parametrize("name", sorted(UNARY))
+def test_host_libm_matches_recorded_unary(name):
+    assert_bit_exact(oracle.unary(UNARY[name], KAT["x"]), KAT["unary_" + name], name)
+
+
+@pytest.mark.parametrize("name", sorted(ACT))
+def test_host_libm_matches_recorded_activation(name):
+    assert_bit_exact(oracle.activate(KAT["x"], ACT[name]), KAT["act_" + name], name)
+
+
+def test_host_libm_matches_recorded_pow():
+    assert_bit_exact(oracle.binary(4, KAT["pow_a"], KAT["pow_b"]), KAT["pow"], "pow")
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_recorded_exact_functions(gpu):
+    from tests import gpuops
+    assert_bit_exact(gpuops.unary(4, KAT["x"]), KAT["unary_exp"], "exp")
+    assert_bit_exact(gpuops.activate(KAT["x"], 3), KAT["act_sigmoid"], "sigmoid")
+    assert_bit_exact(gpuops.activate(KAT["x"], 5), KAT["act_tanh"], "tanh")
