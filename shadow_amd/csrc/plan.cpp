@@ -162,16 +162,16 @@ int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* ax
       plan->wave_per_row = true;
       plan->splits = 1;
     } else {
-      const int by_fill = ceil_div64(2048, plan->outer);
-      const int by_work = ceil_div64(plan->reduce, 8192);
+      const int by_fill = ceil_div64(4096, plan->outer);
+      const int by_work = ceil_div64(plan->reduce, 4096);  // >= 4 vectors per lane
       plan->splits = std::max(1, std::min(by_fill, by_work));
     }
   } else {
     const int vec = (plan->inner % 4 == 0) ? 4 : 1;
     const int64_t tiles = (plan->inner + 64 * vec - 1) / (64 * vec);
     const int64_t base_blocks = tiles * plan->outer;
-    const int by_fill = ceil_div64(2048, base_blocks);
-    const int by_work = ceil_div64(plan->reduce, 32);  // >= 8 rows per wave
+    const int by_fill = ceil_div64(1024, base_blocks);
+    const int by_work = ceil_div64(plan->reduce, 64);  // >= 16 rows per wave
     plan->splits = std::max(1, std::min(by_fill, by_work));
   }
   return SHDW_OK;

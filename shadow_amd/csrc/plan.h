@@ -46,7 +46,7 @@ struct ReducePlan {
   int kind = kRows;
   int64_t outer = 1, reduce = 1, inner = 1;
   int splits = 1;
-  bool wave_per_row = false;  // kRows: one wave64 per row instead of a block
+  bool wave_per_row = false;  // kRows: 16/32/64 lanes per row instead of a workgroup
   int64_t outputs = 1;        // number of output elements
   int64_t window = 1;         // elements per output (Shadow's num_list)
   // kGeneric only: kept dims (outermost first) and reduced dims in LIST order,
@@ -56,7 +56,7 @@ struct ReducePlan {
   int rdim[kMaxDims] = {0}, rstride[kMaxDims] = {0};
 };
 
-constexpr size_t kReducePartialBytes = 16;  // {double value; uint32 key; pad}
+constexpr size_t kReducePartialBytes = 8;  // fp64 accumulator, or {fp32 extremum, zero key}
 
 int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* axes,
                 ReducePlan* plan);

@@ -32,10 +32,10 @@
 
 namespace shdw {
 
+// What a first stage hands to the second, 8 bytes per (output, slice): the fp64
+// accumulator, or {fp32 extremum, zero key} for MAX/MIN.
 struct Partial {
-  double v;
-  uint32_t key;
-  uint32_t pad;
+  uint64_t bits;
 };
 static_assert(sizeof(Partial) == kReducePartialBytes, "partial layout");
 
@@ -78,8 +78,8 @@ struct Acc {
     if (OP == SHDW_REDUCE_L2) return __builtin_sqrtf(static_cast<float>(v));
     return static_cast<float>(v);
   }
-  SHDW_DEVICE Partial pack() const { return Partial{v, 0u, 0u}; }
-  SHDW_DEVICE void unpack(const Partial& p) { v = p.v; }
+  SHDW_DEVICE Partial pack() const { return Partial{static_cast<uint64_t>(__double_as_longlong(v))}; }
+  SHDW_DEVICE void unpack(const Partial& p) { v = __longlong_as_double(static_cast<long long>(p.bits)); }
 };
 
 // ---- MAX / MIN ----
@@ -119,62 +119,73 @@ struct Acc<OP, true> {
     if (v == 0.0f) return (key & 1u) ? -0.0f : 0.0f;
     return v;
   }
-  SHDW_DEVICE Partial pack() const { return Partial{static_cast<double>(v), key, 0u}; }
+  SHDW_DEVICE Partial pack() const {
+    return Partial{(static_cast<uint64_t>(key) << 32) | __float_as_uint(v)};
+  }
   SHDW_DEVICE void unpack(const Partial& p) {
-    v = static_cast<float>(p.v);
-    key = p.key;
+    v = __uint_as_float(static_cast<uint32_t>(p.bits));
+    key = static_cast<uint32_t>(p.bits >> 32);
   }
 };
 
 // All 64 lanes must be active.  Every lane ends with the same combined value:
 // each exchange pairs two lanes that both compute merge(own, other), and every
 // merge used here is commutative bit-for-bit.
-template <class A>
-SHDW_DEVICE A wave_allreduce(A a) {
+template <class A, int G = kWave>
+SHDW_DEVICE A group_allreduce(A a) {  // G = 16, 32 or 64 consecutive lanes
   a.merge(a.template dpp<kDppXor1>());
   a.merge(a.template dpp<kDppXor2>());
   a.merge(a.template dpp<kDppHalfMirror>());
   a.merge(a.template dpp<kDppMirror>());
-  a.merge(a.shfl_xor(16));
-  a.merge(a.shfl_xor(32));
+  if (G >= 32) a.merge(a.shfl_xor(16));
+  if (G >= 64) a.merge(a.shfl_xor(32));
   return a;
+}
+template <class A>
+SHDW_DEVICE A wave_allreduce(A a) {
+  return group_allreduce<A, kWave>(a);
 }
 
 // ---------------------------------------------------------------------------
-// rows, one wave per row
+// rows, G lanes per row (G = 16, 32, 64): short rows share a wave so that no
+// lane idles and the combine stays inside DPP rows where possible.
 // ---------------------------------------------------------------------------
-template <int OP, bool VEC>
-__global__ __launch_bounds__(kBlock) void reduce_rows_wave_kernel(const float* x, float* y,
-                                                                   uint32_t rows,
-                                                                   uint32_t reduce) {
-  const uint32_t lane = threadIdx.x & (kWave - 1);
-  const uint32_t row = blockIdx.x * (kBlock / kWave) + (threadIdx.x / kWave);
-  if (row >= rows) return;  // wave-uniform
+template <int OP, bool VEC, int G>
+__global__ __launch_bounds__(kBlock) void reduce_rows_group_kernel(const float* x, float* y,
+                                                                    uint32_t rows,
+                                                                    uint32_t reduce) {
+  const uint32_t lane = threadIdx.x & (G - 1);
+  const uint32_t row_raw = blockIdx.x * (kBlock / G) + (threadIdx.x / G);
+  // Groups past the end recompute the last row (and do not store) so that all
+  // 64 lanes stay active for the cross-lane exchange.
+  const uint32_t row = row_raw < rows ? row_raw : rows - 1;
   const float* p = x + static_cast<size_t>(row) * reduce;
   Acc<OP> acc;
   acc.init();
   if (VEC) {
     const uint32_t nv = reduce / 4;
-    uint32_t i = lane;
-    for (; i + 3 * kWave < nv; i += 4 * kWave) {
+    for (uint32_t base = 0; base < nv; base += 4 * G) {
       v4f v[4];
+      // all loads of the trip are issued before the first value is consumed
 #pragma unroll
-      for (int u = 0; u < 4; ++u) v[u] = load4_stream(p + 4ull * (i + u * kWave));
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t i = base + u * G + lane;
+        if (i < nv) v[u] = load4_stream(p + 4ull * i);
+      }
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t i = base + u * G + lane;
+        if (i < nv) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc.add(v[u][j], 4 * (i + u * kWave) + j);
-    }
-    for (; i < nv; i += kWave) {
-      const v4f v = load4_stream(p + 4ull * i);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) acc.add(v[j], 4 * i + j);
+          for (int j = 0; j < 4; ++j) acc.add(v[u][j], 4 * i + j);
+        }
+      }
     }
   } else {
-    for (uint32_t i = lane; i < reduce; i += kWave) acc.add(p[i], i);
+    for (uint32_t i = lane; i < reduce; i += G) acc.add(p[i], i);
   }
-  acc = wave_allreduce(acc);
-  if (lane == 0) y[row] = acc.finalize(reduce);
+  acc = group_allreduce<Acc<OP>, G>(acc);
+  if (lane == 0 && row_raw < rows) y[row] = acc.finalize(reduce);
 }
 
 // ---------------------------------------------------------------------------
@@ -351,25 +362,69 @@ __global__ __launch_bounds__(kBlock) void reduce_generic_kernel(GenericArgs g, c
 
 // ---------------------------------------------------------------------------
 // stage 2: y[o] = finalize(merge_s part[o*stride_o + s*stride_s])
+//   _lane : one lane per output, slices walked serially (few slices, many
+//           outputs; coalesced when stride_o == 1)
+//   _block: one workgroup per output (many slices, few outputs)
 // ---------------------------------------------------------------------------
 template <int OP>
-__global__ __launch_bounds__(kBlock) void reduce_stage2_kernel(const Partial* part, float* y,
-                                                                uint32_t outputs,
-                                                                uint32_t splits, size_t stride_o,
-                                                                size_t stride_s,
-                                                                uint32_t window) {
-  const uint32_t lane = threadIdx.x & (kWave - 1);
-  const uint32_t o = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
-  if (o >= outputs) return;  // wave-uniform
+__global__ __launch_bounds__(kBlock) void reduce_stage2_lane_kernel(const Partial* part, float* y,
+                                                                     uint32_t outputs,
+                                                                     uint32_t splits,
+                                                                     size_t stride_o,
+                                                                     size_t stride_s,
+                                                                     uint32_t window) {
+  const uint32_t o = blockIdx.x * kBlock + threadIdx.x;
+  if (o >= outputs) return;
   Acc<OP> acc;
   acc.init();
-  for (uint32_t s = lane; s < splits; s += kWave) {
+  for (uint32_t s = 0; s < splits; ++s) {
+    Acc<OP> t;
+    t.unpack(part[o * stride_o + s * stride_s]);
+    acc.merge(t);
+  }
+  y[o] = acc.finalize(window);
+}
+
+template <int OP>
+__global__ __launch_bounds__(kBlock) void reduce_stage2_block_kernel(const Partial* part, float* y,
+                                                                      uint32_t splits,
+                                                                      size_t stride_o,
+                                                                      size_t stride_s,
+                                                                      uint32_t window) {
+  __shared__ Partial lds[kBlock / kWave];
+  const uint32_t o = blockIdx.x;
+  Acc<OP> acc;
+  acc.init();
+  for (uint32_t s = threadIdx.x; s < splits; s += kBlock) {
     Acc<OP> t;
     t.unpack(part[o * stride_o + s * stride_s]);
     acc.merge(t);
   }
   acc = wave_allreduce(acc);
-  if (lane == 0) y[o] = acc.finalize(window);
+  const uint32_t lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+  if (lane == 0) lds[w] = acc.pack();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < kBlock / kWave; ++k) {
+      Acc<OP> t;
+      t.unpack(lds[k]);
+      acc.merge(t);
+    }
+    y[o] = acc.finalize(window);
+  }
+}
+
+template <int OP>
+static int run_stage2(const Partial* part, float* y, uint32_t outputs, uint32_t splits,
+                      size_t stride_o, size_t stride_s, uint32_t window, hipStream_t st) {
+  if (splits <= 64) {
+    reduce_stage2_lane_kernel<OP><<<grid_for(outputs), kBlock, 0, st>>>(part, y, outputs, splits,
+                                                                        stride_o, stride_s, window);
+  } else {
+    reduce_stage2_block_kernel<OP><<<outputs, kBlock, 0, st>>>(part, y, splits, stride_o, stride_s,
+                                                               window);
+  }
+  return launch_status();
 }
 
 template <int OP>
@@ -403,11 +458,17 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
     // 128-bit loads need every row start 16-byte aligned.
     const bool vec = aligned16(x) && (reduce % 4 == 0 || rows == 1);
     if (pl.wave_per_row) {
-      const uint32_t grid = (rows + kWaves - 1) / kWaves;
-      if (vec && reduce % 4 == 0)
-        reduce_rows_wave_kernel<OP, true><<<grid, kBlock, 0, st>>>(x, y, rows, reduce);
-      else
-        reduce_rows_wave_kernel<OP, false><<<grid, kBlock, 0, st>>>(x, y, rows, reduce);
+      // lanes per row: enough that a lane has at most ~4 vectors to fetch
+      const uint32_t units = (vec && reduce % 4 == 0) ? reduce / 4 : reduce;
+      const int g = units <= 256 ? 16 : (units <= 512 ? 32 : 64);
+      const uint32_t grid = (rows + kBlock / g - 1) / (kBlock / g);
+#define SHDW_ROWS(V, G) reduce_rows_group_kernel<OP, V, G><<<grid, kBlock, 0, st>>>(x, y, rows, reduce)
+      if (vec && reduce % 4 == 0) {
+        if (g == 16) SHDW_ROWS(true, 16); else if (g == 32) SHDW_ROWS(true, 32); else SHDW_ROWS(true, 64);
+      } else {
+        if (g == 16) SHDW_ROWS(false, 16); else if (g == 32) SHDW_ROWS(false, 32); else SHDW_ROWS(false, 64);
+      }
+#undef SHDW_ROWS
       return launch_status();
     }
     const uint32_t splits = static_cast<uint32_t>(pl.splits);
@@ -420,9 +481,7 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
       reduce_rows_block_kernel<OP, false><<<grid, kBlock, 0, st>>>(x, y, part, reduce, chunk, splits);
     int rc = launch_status();
     if (rc != SHDW_OK || splits == 1) return rc;
-    const uint32_t g2 = (rows + kWaves - 1) / kWaves;
-    reduce_stage2_kernel<OP><<<g2, kBlock, 0, st>>>(part, y, rows, splits, splits, 1, window);
-    return launch_status();
+    return run_stage2<OP>(part, y, rows, splits, splits, 1, window, st);
   }
 
   // strided
@@ -443,9 +502,7 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
                                                           rows_per_split, splits, outputs);
   int rc = launch_status();
   if (rc != SHDW_OK || splits == 1) return rc;
-  const uint32_t g2 = (outputs + kWaves - 1) / kWaves;
-  reduce_stage2_kernel<OP><<<g2, kBlock, 0, st>>>(part, y, outputs, splits, 1, outputs, window);
-  return launch_status();
+  return run_stage2<OP>(part, y, outputs, splits, 1, outputs, window, st);
 }
 
 static int dispatch_reduce(int operation, const ReducePlan& pl, const float* x, float* y,
