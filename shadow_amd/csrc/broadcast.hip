@@ -121,6 +121,9 @@ __global__ __launch_bounds__(kBlock) void bcast_vec_kernel(F f, BcastArgs p, con
                                                             const float* b, float* y,
                                                             uint32_t n4) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  // Pow reads the 2^(i/32) table; broadcast Pow is not a throughput case, the
+  // table stays in global memory here.
+  const uint64_t* tab = uses_exp_table<F>::value ? libm::kExp2fTab : nullptr;
   if (i < n4) {
     uint32_t e = 4 * i;
     uint32_t oa = 0, ob = 0;
@@ -149,7 +152,7 @@ __global__ __launch_bounds__(kBlock) void bcast_vec_kernel(F f, BcastArgs p, con
     }
     v4f r;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) r[j] = f(va[j], vb[j], nullptr);
+    for (int j = 0; j < 4; ++j) r[j] = f(va[j], vb[j], tab);
     store4_stream(y + 4ull * i, r);
   }
 }
@@ -167,6 +170,7 @@ __global__ __launch_bounds__(kBlock) void bcast_generic_kernel(F f, BcastGeneric
                                                                 const float* a, const float* b,
                                                                 float* y, uint32_t n) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint64_t* tab = uses_exp_table<F>::value ? libm::kExp2fTab : nullptr;
   if (i < n) {
     uint32_t e = i, oa = 0, ob = 0;
     for (int k = p.ndim - 1; k >= 1; --k) {
@@ -178,7 +182,7 @@ __global__ __launch_bounds__(kBlock) void bcast_generic_kernel(F f, BcastGeneric
     }
     oa += e * static_cast<uint32_t>(p.sa[0]);
     ob += e * static_cast<uint32_t>(p.sb[0]);
-    y[i] = f(a[oa], b[ob], nullptr);
+    y[i] = f(a[oa], b[ob], tab);
   }
 }
 

@@ -27,14 +27,14 @@ SHDW_DEVICE float sel_min(float a, float b) { return (b < a) ? b : a; }
 struct UAbs { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return __builtin_fabsf(a); } };
 struct USquare { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return a * a; } };
 struct USqrt { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return __builtin_sqrtf(a); } };
-struct ULog { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return logf(a); } };
+struct ULog { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return libm::exact_logf(a); } };
 struct UExp { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return libm::exact_expf(a, tab); } };
-struct USin { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return sinf(a); } };
-struct UCos { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return cosf(a); } };
-struct UTan { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return tanf(a); } };
-struct UAsin { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return asinf(a); } };
-struct UAcos { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return acosf(a); } };
-struct UAtan { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return atanf(a); } };
+struct USin { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return libm::exact_sinf(a); } };
+struct UCos { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return libm::exact_cosf(a); } };
+struct UTan { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return libm::exact_tanf(a); } };
+struct UAsin { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return libm::exact_asinf(a); } };
+struct UAcos { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return libm::exact_acosf(a); } };
+struct UAtan { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return libm::exact_atanf(a); } };
 struct UFloor { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return __builtin_floorf(a); } };
 struct UCeil { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return __builtin_ceilf(a); } };
 struct UNeg { SHDW_DEVICE float operator()(float a, const uint64_t* tab) const { return -a; } };
@@ -46,7 +46,7 @@ struct BAdd { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab
 struct BSub { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return a - b; } };
 struct BMul { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return a * b; } };
 struct BDiv { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return a / b; } };
-struct BPow { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return powf(a, b); } };
+struct BPow { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return libm::exact_powf(a, b, tab); } };
 struct BMax { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return sel_max(a, b); } };
 struct BMin { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab) const { return sel_min(a, b); } };
 
@@ -54,7 +54,7 @@ struct BMin { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab
 struct ARelu { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return x > 0 ? x : 0; } };
 struct ALeaky { SHDW_DEVICE float operator()(float x, float s, const uint64_t* tab) const { return x > 0 ? x : s * x; } };
 struct ASigmoid { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_sigmoidf(x, tab); } };
-struct ASoftPlus { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return log1pf(libm::exact_expf(x, tab)); } };
+struct ASoftPlus { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_softplusf(x, tab); } };
 struct ATanh { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_tanhf(x); } };
 struct ARelu6 { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return x < 0 ? 0 : (x > 6 ? 6 : x); } };
 struct AHardSwish {
@@ -63,8 +63,9 @@ struct AHardSwish {
   }
 };
 struct AGelu {
+  static constexpr bool kExpTable = true;
   SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const {
-    return 0.5f * x * (1 + erff(0.707107f * x));
+    return libm::exact_geluf(x, tab);
   }
 };
 

@@ -11,9 +11,8 @@ from tests.helpers import (assert_bit_exact, assert_rel_close, normal, ulp_dista
 
 pytestmark = pytest.mark.gpu
 
-EXACT_UNARY = {0: "abs", 1: "square", 2: "sqrt", 4: "exp", 11: "floor", 12: "ceil", 13: "neg",
-               14: "reciprocal"}
-LIBM_UNARY = {3: "log", 5: "sin", 6: "cos", 7: "tan", 8: "asin", 9: "acos", 10: "atan"}
+EXACT_UNARY = {0: "abs", 1: "square", 2: "sqrt", 3: "log", 4: "exp", 5: "sin", 6: "cos", 7: "tan",
+               8: "asin", 9: "acos", 10: "atan", 11: "floor", 12: "ceil", 13: "neg", 14: "reciprocal"}
 
 SIZES = [1, 3, 4, 5, 63, 64, 255, 1024, 1027, 4096 + 2, 100003, 1 << 20]
 
@@ -39,20 +38,16 @@ def test_unary_inplace_and_misaligned(gpu, op):
         assert_bit_exact(gpuops.unary(op, x, offset=off), want, "offset %d" % off)
 
 
-@pytest.mark.parametrize("op", sorted(LIBM_UNARY))
-def test_unary_libm_ulp(gpu, op):
-    """These still run the device math library, not a glibc restatement: parity
-    is within a few ulp, not bit-exact."""
-    x = with_specials(uniform(30 + op, 200003, -4.0, 4.0), op)
-    if op in (8, 9):
-        x = np.clip(x, -1.0, 1.0)
-    got, want = gpuops.unary(op, x), oracle.unary(op, x)
-    assert (np.isnan(got) == np.isnan(want)).all()
-    ok = np.isfinite(want)
-    assert ulp_distance(got[ok], want[ok]).max() <= 4, LIBM_UNARY[op]
+@pytest.mark.parametrize("op", [3, 5, 6, 7, 8, 9, 10])
+@pytest.mark.parametrize("scale", [1.0, 100.0, 1e6, 1e30])
+def test_unary_libm_wide_ranges(gpu, op, scale):
+    """Argument-reduction paths of the trigonometric functions and the whole
+    exponent range of log: still bit-exact."""
+    x = with_specials(normal(30 + op, 150001, scale), op)
+    assert_bit_exact(gpuops.unary(op, x), oracle.unary(op, x), EXACT_UNARY[op])
 
 
-@pytest.mark.parametrize("op", [0, 1, 2, 3, 5, 6])
+@pytest.mark.parametrize("op", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("n", [7, 4099, 262144 + 1])
 def test_binary_and_scalar(gpu, op, n):
     a = with_specials(normal(40 + op, n), op)
@@ -64,11 +59,19 @@ def test_binary_and_scalar(gpu, op, n):
                          "scalar %d" % op)
 
 
-def test_binary_pow_ulp(gpu):
-    a = uniform(60, 50001, 0.1, 4.0)
-    b = uniform(61, 50001, -3.0, 3.0)
-    got, want = gpuops.binary(4, a, b), oracle.binary(4, a, b)
-    assert ulp_distance(got, want).max() <= 4
+def test_binary_pow_exact(gpu):
+    r = np.random.default_rng(60)
+    a = with_specials(uniform(60, 300001, -4.0, 6.0), 7)
+    b = with_specials(normal(61, 300001, 3.0), 8)
+    b[::7] = np.round(b[::7])  # integer exponents make negative bases finite
+    assert_bit_exact(gpuops.binary(4, a, b), oracle.binary(4, a, b), "pow")
+    for alpha in (2.0, 0.5, -3.0, 0.0, float("inf")):
+        assert_bit_exact(gpuops.binary_scalar(4, a, alpha), oracle.binary_scalar(4, a, alpha), "pow scalar")
+    sa, sb = [64, 1, 33], [1, 5, 1]
+    x, y = uniform(62, sa, 0.1, 4.0), normal(63, sb, 2.0)
+    so = [64, 5, 33]
+    assert_bit_exact(gpuops.broadcast_binary(4, x, sa, y, sb, so), oracle.broadcast_binary(4, x, sa, y, sb, so),
+                     "pow broadcast")
 
 
 def test_max_min_select_semantics(gpu):
@@ -104,7 +107,7 @@ def test_axpy_is_not_fused(gpu):
     assert want[0] != fused  # the case does discriminate
 
 
-@pytest.mark.parametrize("act", [1, 2, 3, 5, 6, 7])
+@pytest.mark.parametrize("act", [1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("n", [9, 66001])
 def test_activate_exact(gpu, act, n):
     x = with_specials(normal(80 + act, n, 2.0), act)
@@ -112,16 +115,10 @@ def test_activate_exact(gpu, act, n):
     assert_bit_exact(gpuops.activate(x, act, 0.1, inplace=True), oracle.activate(x, act, 0.1), "in place")
 
 
-@pytest.mark.parametrize("act", [4, 8])
-def test_activate_libm_ulp(gpu, act):
-    x = normal(90 + act, 100001, 2.0)
-    got, want = gpuops.activate(x, act), oracle.activate(x, act)
-    if act == 8:
-        # 1 + erf(.) cancels in the negative tail, so ulps of the result are not
-        # meaningful there; bound the absolute error instead.
-        assert np.abs(got.astype(np.float64) - want).max() <= 2e-6
-    else:
-        assert ulp_distance(got, want).max() <= 4
+@pytest.mark.parametrize("act", [3, 4, 5, 8])
+def test_activate_libm_wide_range(gpu, act):
+    x = with_specials(normal(90 + act, 200001, 30.0), act)
+    assert_bit_exact(gpuops.activate(x, act), oracle.activate(x, act), "act %d" % act)
 
 
 @pytest.mark.parametrize("shape,shared", [((2, 3, 5, 7), False), ((2, 3, 5, 7), True),

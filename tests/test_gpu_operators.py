@@ -37,13 +37,7 @@ def test_unary_op(ws, operation):
     got = run(ws, "Unary", [("x", x)], {"operation": operation})
     want = oracle.unary_op(x, operation)
     assert got.shape == want.shape
-    if operation in (3, 5, 6, 7, 8, 9, 10):  # device math library, not yet a glibc restatement
-        ok = np.isfinite(want)
-        assert (np.isnan(got) == np.isnan(want)).all()
-        from tests.helpers import ulp_distance
-        assert ulp_distance(got[ok], want[ok]).max() <= 4
-    else:
-        assert_bit_exact(got, want, "unary %d" % operation)
+    assert_bit_exact(got, want, "unary %d" % operation)
 
 
 def test_unary_op_argument_errors(ws):
@@ -57,7 +51,7 @@ def test_unary_op_argument_errors(ws):
         ws.create_op("NoSuchOp", ["x"], ["y"], {})
 
 
-@pytest.mark.parametrize("operation", [0, 1, 2, 3, 5, 6])
+@pytest.mark.parametrize("operation", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("sa,sb", [((2, 3, 4), (2, 3, 4)), ((2, 1), (3,)), ((8, 64, 12, 12), (1, 64, 1, 1)),
                                    ((16, 1, 8, 32), (1, 5, 8, 1)), ((4, 6, 1, 32), (6, 32)), ((12, 10), (1,)),
                                    ((3,), (2, 4, 3))])
@@ -155,7 +149,7 @@ def test_reduce_op_observed_reference_cases(ws):
     assert mx[0, 0] == 3 and mx.view(np.uint32)[1, 0] == 0xff7fffff
 
 
-@pytest.mark.parametrize("act", [1, 2, 3, 5, 6, 7])
+@pytest.mark.parametrize("act", [1, 2, 3, 4, 5, 6, 7, 8])
 def test_activate_op(ws, act):
     x = with_specials(normal(30, (2, 6, 9, 9), 2.0), 3).reshape(2, 6, 9, 9)
     got = run(ws, "Activate", [("x", x)], {"type": act, "slope": 0.2})

@@ -1,8 +1,10 @@
 """The device math restatements (shadow_amd/csrc/libm_exact.h), compiled for the
 host, against this machine's libm -- the arithmetic the oracle and the reference
 use.  The default run covers every 61st bit pattern plus dense windows around
-the algorithms' branch points (~10 s); SHADOW_LIBM_FULL=1 sweeps all 2^32
-patterns of each function (~2 min on 8 cores)."""
+the algorithms' branch points (~20 s); SHADOW_LIBM_FULL=1 sweeps all 2^32
+patterns of each one-argument function and 9 x 2^32 (x, y) pairs of powf
+(~10 min on 8 cores).  All of them have been swept in full with 0 mismatches
+against glibc 2.35."""
 import ctypes
 import os
 
@@ -10,11 +12,15 @@ import numpy as np
 import pytest
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-FUNCS = {"exp": 0, "tanh": 1, "sigmoid": 2, "expm1": 3}
+FUNCS = {"exp": 0, "tanh": 1, "sigmoid": 2, "expm1": 3, "log": 4, "sin": 5, "cos": 6, "atan": 7,
+         "asin": 8, "acos": 9, "log1p": 10, "erf": 11, "softplus": 12, "gelu": 13, "tan": 14}
 # float bit patterns where the restated algorithms switch paths
-EDGES = [0x00000000, 0x00800000, 0x24000000, 0x33000000, 0x3eb17218, 0x3f000000, 0x3f800000,
-         0x3F851592, 0x4195b844, 0x41b00000, 0x42b00000, 0x42b17218, 0x42cff1b5, 0x42ce8ed0,
-         0x7f800000]
+EDGES = [0x00000000, 0x00800000, 0x04000000, 0x24000000, 0x24800000, 0x31000000, 0x31800000,
+         0x32000000, 0x32800000, 0x33000000, 0x39000000, 0x39800000, 0x3eb17218, 0x3ed413d7,
+         0x3e95f61f, 0x3ee00000, 0x3f000000, 0x3f2ca140, 0x3f300000, 0x3f330000, 0x3f490fda,
+         0x3f580000, 0x3f79999a, 0x3f800000, 0x3F851592, 0x3f980000, 0x3fa00000, 0x3fc90fda,
+         0x401c0000, 0x4036db6e, 0x40490fda, 0x40c00000, 0x4195b844, 0x41b00000, 0x42b00000,
+         0x42b17218, 0x42cff1b5, 0x42ce8ed0, 0x42f00000, 0x4c000000, 0x5a000000, 0x7f800000]
 
 
 @pytest.fixture(scope="module")
@@ -44,3 +50,22 @@ def test_restatement_matches_host_libm(sweep, name):
         for sign in (0, 0x80000000):
             lo = max(0, (edge | sign) - 4096)
             run(lo, 8192, 1)
+
+
+def test_powf_restatement_matches_host_libm(sweep):
+    """y fixed at a few values and y random (all bit patterns / scaled into
+    [-40, 40]) while x walks an arithmetic progression of bit patterns."""
+    sweep.libm_sweep_pow.restype = ctypes.c_longlong
+    sweep.libm_sweep_pow.argtypes = [ctypes.c_uint32, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32,
+                                     ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_uint32),
+                                     ctypes.c_int]
+    rep = (ctypes.c_uint32 * 16)()
+    threads = min(8, os.cpu_count() or 1)
+    full = bool(os.environ.get("SHADOW_LIBM_FULL"))
+    count, stride = ((1 << 32, 1) if full else ((1 << 32) // 127 + 1, 127))
+    cases = [(1, 1), (2, 2), (2, 77), (0, 0x40000000), (0, 0x3f000000), (0, 0xc0400000), (0, 0),
+             (0, 0x7fa00000), (0, 0x41200000)]
+    for mode, ybits in cases:
+        bad = sweep.libm_sweep_pow(0, count, stride, ybits, mode, threads, rep, 16)
+        assert bad == 0, "powf mode %d y=%#x: %d mismatches, e.g. (x, y) bits %s" % (
+            mode, ybits, bad, [hex(v) for v in rep[:min(2 * bad, 8)]])
