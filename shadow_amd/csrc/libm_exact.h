@@ -41,6 +41,25 @@ SHDW_LIBM_FN float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
 SHDW_LIBM_FN uint64_t d2u(double d) { return __builtin_bit_cast(uint64_t, d); }
 SHDW_LIBM_FN double u2d(uint64_t u) { return __builtin_bit_cast(double, u); }
 
+// a / b, correctly rounded, for callers that know |a|, |b| and |a / b| are all
+// well inside the normal range (no scaling, no special cases).  On the device
+// this is the reciprocal-plus-Newton core of the compiler's own IEEE division
+// without its range scaling and fix-up instructions; on the host it is `/`.
+SHDW_LIBM_FN float div_normal(float a, float b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  float r = __builtin_amdgcn_rcpf(b);
+  float e = __builtin_fmaf(-b, r, 1.0f);
+  r = __builtin_fmaf(e, r, r);
+  float q = a * r;
+  e = __builtin_fmaf(-b, q, a);
+  q = __builtin_fmaf(e, r, q);
+  e = __builtin_fmaf(-b, q, a);
+  return __builtin_fmaf(e, r, q);
+#else
+  return a / b;
+#endif
+}
+
 // T[i] = bits(2^(i/32)) - (i << 47)
 SHDW_LIBM_TABLE uint64_t kExp2fTab[32] = {
     0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
@@ -203,7 +222,8 @@ SHDW_LIBM_FN float exact_tanhf(float x) {
   const float hxs = xr * hfx;
   const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
   const float t3 = 3.0f - r1 * hfx;
-  float e = hxs * ((r1 - t3) / (6.0f - xr * t3));
+  // numerator ~ -2, denominator in [4.9, 7.1]
+  float e = hxs * div_normal(r1 - t3, 6.0f - xr * t3);
   const float res_k0 = xr - (xr * e - hxs);
   e = (xr * (e - c) - c);
   e -= hxs;
@@ -225,11 +245,13 @@ SHDW_LIBM_FN float exact_tanhf(float x) {
   t = (ha < 0x33000000u) ? a : t;  // |a| < 2^-25: expm1f returns a
 
   // --- tanhf ---
-  const float q = (big ? two : t) / (t + two);
+  // |x| >= 1: 2 / (t + 2) with t in [6.3, 1.3e19]; else t / (t + 2) with
+  // |t| in [2^-54, 0.87] and t + 2 in (1.13, 2]: every value is normal
+  const float q = div_normal(big ? two : t, t + two);
   float z = big ? one - q : -q;
   z = (ix < 0x41b00000u) ? z : one;           // |x| >= 22 (and +-inf): 1 - tiny == 1
   float res = (jx >> 31) ? -z : z;
-  res = (ix < 0x24000000u) ? x * (one + x) : res;  // |x| < 2^-55, including +-0
+  res = (ix < 0x24000000u) ? x : res;  // |x| < 2^-55 (and +-0): x * (1 + x) == x exactly
   res = (ix > 0x7f800000u) ? x + x : res;          // NaN
   return res;
 }
