@@ -167,12 +167,32 @@ int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* ax
       plan->splits = std::max(1, std::min(by_fill, by_work));
     }
   } else {
-    const int vec = (plan->inner % 4 == 0) ? 4 : 1;
-    const int64_t tiles = (plan->inner + 64 * vec - 1) / (64 * vec);
-    const int64_t base_blocks = tiles * plan->outer;
-    const int by_fill = ceil_div64(1024, base_blocks);
-    const int by_work = ceil_div64(plan->reduce, 64);  // >= 16 rows per wave
-    plan->splits = std::max(1, std::min(by_fill, by_work));
+    // Pick columns per lane (128-bit or scalar loads) and waves per column tile
+    // so that one launch gives >= 256 workgroups (one per CU) and >= 2048 waves;
+    // only when no shape does, split the reduced axis over grid.z and add a
+    // second stage.
+    const int vec_max = (plan->inner % 4 == 0) ? 4 : 1;
+    const int cand[4][2] = {{4, 4}, {4, 16}, {1, 4}, {1, 16}};
+    bool single = false;
+    for (const auto& c : cand) {
+      if (c[0] > vec_max) continue;
+      const int64_t blocks = ((plan->inner + 64 * c[0] - 1) / (64 * c[0])) * plan->outer;
+      if (blocks >= 256 && blocks * c[1] >= 2048 && plan->reduce >= 8 * c[1]) {
+        plan->strided_vec = c[0], plan->strided_waves = c[1];
+        single = true;
+        break;
+      }
+    }
+    if (single) {
+      plan->splits = 1;
+    } else {
+      plan->strided_vec = vec_max, plan->strided_waves = 4;
+      const int64_t tiles = (plan->inner + 64 * vec_max - 1) / (64 * vec_max);
+      const int64_t base_blocks = tiles * plan->outer;
+      const int by_fill = ceil_div64(1024, base_blocks);
+      const int by_work = ceil_div64(plan->reduce, 64);  // >= 16 rows per wave
+      plan->splits = std::max(1, std::min(by_fill, by_work));
+    }
   }
   return SHDW_OK;
 }

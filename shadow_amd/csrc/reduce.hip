@@ -248,14 +248,14 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const float* 
 // ---------------------------------------------------------------------------
 // strided: x[outer][reduce][inner] -> y[outer][inner]
 // ---------------------------------------------------------------------------
-template <int OP, int VEC>
-__global__ __launch_bounds__(kBlock) void reduce_strided_kernel(const float* x, float* y,
-                                                                 Partial* part, uint32_t reduce,
-                                                                 uint32_t inner,
-                                                                 uint32_t rows_per_split,
-                                                                 uint32_t splits,
-                                                                 uint32_t outputs) {
-  constexpr int kWaves = kBlock / kWave;
+// WAVES wave64 per workgroup (4 or 16) share one tile of 64*VEC columns and
+// interleave over the rows of their slice; with 16 waves a few hundred tiles
+// already fill the GPU and no second stage is needed.
+template <int OP, int VEC, int WAVES>
+__global__ __launch_bounds__(kWave * WAVES) void reduce_strided_kernel(
+    const float* x, float* y, Partial* part, uint32_t reduce, uint32_t inner,
+    uint32_t rows_per_split, uint32_t splits, uint32_t outputs) {
+  constexpr int kWaves = WAVES;
   __shared__ Partial lds[kWaves - 1][VEC][kWave];
   const uint32_t lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
   const uint32_t col = (blockIdx.x * kWave + lane) * VEC;
@@ -491,15 +491,18 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
   const uint32_t splits = static_cast<uint32_t>(pl.splits);
   if (outer > 65535u || splits > 65535u) return SHDW_E_UNSUPPORTED;
   const uint32_t rows_per_split = (reduce + splits - 1) / splits;
-  const bool vec = inner % 4 == 0 && aligned16(x);
+  const bool vec = pl.strided_vec == 4 && inner % 4 == 0 && aligned16(x);
   const int v = vec ? 4 : 1;
   const dim3 grid((inner + kWave * v - 1) / (kWave * v), outer, splits);
-  if (vec)
-    reduce_strided_kernel<OP, 4><<<grid, kBlock, 0, st>>>(x, y, part, reduce, inner,
-                                                          rows_per_split, splits, outputs);
-  else
-    reduce_strided_kernel<OP, 1><<<grid, kBlock, 0, st>>>(x, y, part, reduce, inner,
-                                                          rows_per_split, splits, outputs);
+#define SHDW_STRIDED(V, W)                                                                   \
+  reduce_strided_kernel<OP, V, W><<<grid, kWave * W, 0, st>>>(x, y, part, reduce, inner,       \
+                                                             rows_per_split, splits, outputs)
+  if (pl.strided_waves == 16) {
+    if (vec) SHDW_STRIDED(4, 16); else SHDW_STRIDED(1, 16);
+  } else {
+    if (vec) SHDW_STRIDED(4, 4); else SHDW_STRIDED(1, 4);
+  }
+#undef SHDW_STRIDED
   int rc = launch_status();
   if (rc != SHDW_OK || splits == 1) return rc;
   return run_stage2<OP>(part, y, outputs, splits, 1, outputs, window, st);

@@ -83,7 +83,9 @@ def test_reduce_plans_of_the_benchmark_shapes():
     rc, (kind, outer, red, inner, splits) = plan_reduce([32, 512, 28, 28], [2, 3])
     assert (rc, kind, outer, red, inner, splits) == (0, ROWS, 16384, 784, 1, 1)
     rc, (kind, outer, red, inner, splits) = plan_reduce([32, 512, 28, 28], [1])
-    assert (rc, kind, outer, red, inner) == (0, STRIDED, 32, 512, 784) and splits > 1
+    assert (rc, kind, outer, red, inner, splits) == (0, STRIDED, 32, 512, 784, 1)  # single stage
+    rc, (kind, outer, red, inner, splits) = plan_reduce([2, 100000, 8], [1])
+    assert (rc, kind, outer, red, inner) == (0, STRIDED, 2, 100000, 8) and splits > 1
     rc, (kind, outer, red, inner, splits) = plan_reduce([32, 512, 28, 28], [0, 1, 2, 3])
     assert (rc, kind, outer, red, inner) == (0, ROWS, 1, 12845056, 1) and splits > 64
     rc, (kind, outer, red, inner, splits) = plan_reduce([64, 1024, 14, 14], [2, 3])

@@ -224,6 +224,8 @@ REDUCE_CASES = [
     ([6, 1, 5], [1]),            # reduced axis of extent 1
     ([1, 1, 1], [0, 1, 2]),
     ([2, 40000], [1]),           # rows, long, few
+    ([2, 30000, 8], [1]),        # strided, 16 waves per tile and a second stage
+    ([3, 200, 12], [1]),         # strided, 16 waves per tile, single stage
 ]
 
 
