@@ -227,6 +227,52 @@ int shdw_hip_scale_residual_relu_rowmean(int n, int scale_num, int inner_num,
                                          const float* bias, const float* residual,
                                          float* y, float* mean, void* stream);
 
+/* ==================== neighbouring operators of the path ==================== */
+
+/* Axpy: out[r*inner_num + i] = y[..] + alpha[r] * x[..] for r < outer_num
+ * (multiply, then add).  out may alias y; it must not alias x.
+ * ref: shadow/operators/kernels/axpy.cpp:9-21 (memcpy + one BlasSaxpy per row),
+ *      axpy.cu:7-26 */
+int shdw_hip_axpy_rows(int outer_num, int inner_num, const float* alpha, const float* x,
+                       const float* y, float* out, void* stream);
+
+/* BatchNorm with global statistics: c = (i / inner_num) % channel;
+ *   y = (x - mean[c]*scale_factor) / sqrt(|variance[c]*scale_factor| + eps)
+ * with IEEE divide and square root.  y may alias x.
+ * ref: shadow/operators/kernels/batch_norm.cpp:11-24, batch_norm.cu:9-34 */
+int shdw_hip_batch_norm(int n, int channel, int inner_num, const float* x, const float* mean,
+                        const float* variance, float scale_factor, float eps, float* y,
+                        void* stream);
+
+/* Softmax over the middle extent of x viewed as [outer_num][dim][inner_num]:
+ * running maximum, exp(x - max), fp32 running sum in index order, divide.  The
+ * per-column scratch blob of the reference is not needed.  y may alias x.
+ * ref: shadow/operators/kernels/softmax.cpp:10-42, softmax.hpp:29-41,
+ *      softmax.cu:9-70 */
+int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, float* y,
+                     void* stream);
+
+/* Normalize: y = x / max(norm_p(column), eps), the norm accumulated in fp64 in
+ * index order; p == 1 and p == 2 have their own forms, any other p goes through
+ * powf.  y may alias x.
+ * ref: shadow/operators/kernels/normalize.cpp:10-43, normalize.hpp:29-38,
+ *      normalize.cu:7-56 */
+int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps,
+                       const float* x, float* y, void* stream);
+
+/* Pooling over [N][C][H][W] (2d) or [N][C][D][H][W] (3d); shapes are HOST arrays
+ * of 4 / 5 ints and out_shape is what the operator computed.  pool_type 0 = max
+ * (start at lowest(), keep unless smaller), 1 = average: fp32 running sum in
+ * window order divided by the window size clipped to input + pad.
+ * ref: shadow/operators/kernels/pooling.cpp:7-42 (2d), :44-86 (3d), pooling.cu:7-126 */
+int shdw_hip_pooling2d(const int* in_shape, int pool_type, int kernel_h, int kernel_w,
+                       int stride_h, int stride_w, int pad_h, int pad_w, const int* out_shape,
+                       const float* x, float* y, void* stream);
+int shdw_hip_pooling3d(const int* in_shape, int pool_type, int kernel_d, int kernel_h,
+                       int kernel_w, int stride_d, int stride_h, int stride_w, int pad_d,
+                       int pad_h, int pad_w, const int* out_shape, const float* x, float* y,
+                       void* stream);
+
 /* ============================ plan inspection ============================ */
 
 /* Host-only: the collapsed form shdw_hip_broadcast_binary would launch with.

@@ -173,6 +173,53 @@ def reduce(op, x, shape, axes):
     return out, out_shape
 
 
+def axpy_rows(alpha, x, y, inner_num):
+    alpha, x, y = _f(alpha).ravel(), _f(x).ravel(), _f(y).ravel()
+    out = np.empty_like(x)
+    lib().orc_axpy_rows(_p(alpha), _p(x), _p(y), alpha.size, int(inner_num), _p(out))
+    return out
+
+
+def batch_norm(x, mean, variance, channel, inner_num, scale_factor, eps):
+    x, mean, variance = _f(x).ravel(), _f(mean).ravel(), _f(variance).ravel()
+    out = np.empty_like(x)
+    lib().orc_batch_norm(_p(x), x.size, _p(mean), _p(variance), int(channel), int(inner_num),
+                         ctypes.c_float(scale_factor), ctypes.c_float(eps), _p(out))
+    return out
+
+
+def softmax(x, outer, dim, inner):
+    x = _f(x).ravel()
+    out = np.empty_like(x)
+    val = np.empty(max(1, outer * inner), np.float32)
+    lib().orc_softmax(_p(x), int(outer), int(dim), int(inner), _p(val), _p(out))
+    return out
+
+
+def normalize(x, outer, dim, inner, p, eps):
+    x = _f(x).ravel()
+    out = np.empty_like(x)
+    val = np.empty(max(1, outer * inner), np.float32)
+    lib().orc_normalize(_p(x), int(outer), int(dim), int(inner), _p(val), ctypes.c_float(p),
+                        ctypes.c_float(eps), _p(out))
+    return out
+
+
+def pooling(x, in_shape, pool_type, kernel, stride, pad, out_shape):
+    """2-D or 3-D by len(kernel)."""
+    x = _f(x).ravel()
+    out = np.empty(int(np.prod(out_shape, dtype=np.int64)), np.float32)
+    fn = lib().orc_pooling2d if len(kernel) == 2 else lib().orc_pooling3d
+    fn(_p(x), _ints(in_shape), int(pool_type), *[int(v) for v in kernel], *[int(v) for v in stride],
+       *[int(v) for v in pad], _ints(out_shape), _p(out))
+    return out
+
+
+def pooling_out_size(dim, kernel_size, stride, pad, full_pooling):
+    return int(lib().orc_pooling_out_size(int(dim), int(kernel_size), int(stride), int(pad),
+                                          int(bool(full_pooling))))
+
+
 # --------------------------------------------------------------------------
 # operator level: argument checks and shape rules of shadow/operators/*_op.cpp
 # --------------------------------------------------------------------------
@@ -282,3 +329,80 @@ def scale_op(x, axis=1, scale=None, bias=None, scale_value=(), bias_value=()):
     out = scale_bias(x.ravel(), np.float32(sv) if sv else None, np.float32(bv) if bv else None,
                      dim, count(axis + 1))
     return out.reshape(x.shape)
+
+
+def axpy_op(alpha, x, y):
+    """shadow/operators/axpy_op.cpp:25-46"""
+    alpha, x, y = _f(alpha), _f(x), _f(y)
+    _check(alpha.shape[0] == x.shape[0], "alpha->shape(0) == x->shape(0)")
+    _check(alpha.shape[1] == x.shape[1], "alpha->shape(1) == x->shape(1)")
+    if alpha.ndim == 4:
+        _check(alpha.shape[2] == 1 and alpha.shape[3] == 1, "alpha->shape(2/3) == 1")
+    _check(x.shape == y.shape, "x->shape() == y->shape()")
+    inner = int(np.prod(x.shape[2:], dtype=np.int64))
+    return axpy_rows(alpha, x, y, inner).reshape(x.shape)
+
+
+def batch_norm_op(x, mean, variance, scale=None, eps=1e-5, use_global_stats=True):
+    """shadow/operators/batch_norm_op.cpp:9-40 and kernels/batch_norm.hpp:36-48"""
+    _check(use_global_stats, "use_global_stats")
+    x = _f(x)
+    scale_factor = np.float32(1)
+    if scale is not None:
+        sc = _f(scale)
+        _check(sc.size == 1, "inputs[3]->count() == 1")
+        scale_factor = np.float32(0) if sc.ravel()[0] == 0 else np.float32(1) / sc.ravel()[0]
+    channel = x.shape[1]
+    _check(channel == np.size(mean), "channel == mean->count()")
+    _check(channel == np.size(variance), "channel == variance->count()")
+    inner = int(np.prod(x.shape[2:], dtype=np.int64))
+    return batch_norm(x, mean, variance, channel, inner, scale_factor, np.float32(eps)).reshape(x.shape)
+
+
+def _canonical(axis, ndim):
+    _check(-ndim <= axis < ndim, "axis in range")
+    return axis + ndim if axis < 0 else axis
+
+
+def softmax_op(x, axis=1):
+    """shadow/operators/softmax_op.cpp:18-29 and kernels/softmax.hpp:29-41"""
+    x = _f(x)
+    axis = _canonical(axis, x.ndim)
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    return softmax(x, outer, x.shape[axis], inner).reshape(x.shape)
+
+
+def normalize_op(x, p=2.0, axis=1, eps=1e-12):
+    """shadow/operators/normalize_op.cpp:9-29 and kernels/normalize.hpp:29-38"""
+    x = _f(x)
+    axis = _canonical(axis, x.ndim)
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    return normalize(x, outer, x.shape[axis], inner, np.float32(p), np.float32(eps)).reshape(x.shape)
+
+
+def pooling_op(x, pool=0, kernel_size=(), stride=(1,), pad=(0,), global_pooling=False,
+               full_pooling=True):
+    """shadow/operators/pooling_op.cpp:28-95"""
+    x = _f(x)
+    _check(0 <= pool <= 1, "pool_type in [0, 1]")
+    nsp = x.ndim - 2
+    _check(nsp in (2, 3), "Only support 2D or 3D Pooling")
+    kernel_size, stride, pad = list(kernel_size), list(stride), list(pad)
+    if global_pooling:
+        stride, pad = [1], [0]
+        kernel_size = list(x.shape[2:])
+
+    def expand(v):
+        if len(v) == 1:
+            return v * nsp
+        _check(len(v) == nsp, "param.size() == num")
+        return v
+
+    kernel_size, stride, pad = expand(kernel_size), expand(stride), expand(pad)
+    out_shape = list(x.shape)
+    for n in range(nsp):
+        out_shape[n + 2] = pooling_out_size(x.shape[n + 2], kernel_size[n], stride[n], pad[n],
+                                            full_pooling)
+    return pooling(x, x.shape, pool, kernel_size, stride, pad, out_shape).reshape(out_shape)

@@ -300,3 +300,170 @@ API int orc_reduce(int op, const float* in, const int* in_shape, int num_axes, c
   free(list);
   return 0;
 }
+
+/* ======================================================================
+ * Operators next to the hot path (callers of the same Blas / Vision layer).
+ * ====================================================================== */
+
+/* ---- shadow/operators/kernels/axpy.cpp:9-21  Vision::Axpy: out = y, then one
+ *      BlasSaxpy (shadow/core/blas.cpp:214-216) per row of inner_num ---- */
+API void orc_axpy_rows(const float* alpha, const float* x, const float* y, int outer_num,
+                       int inner_num, float* out) {
+  memmove(out, y, (size_t)outer_num * inner_num * sizeof(float));
+  for (int n = 0; n < outer_num; ++n) {
+    int off = n * inner_num;
+    for (int i = 0; i < inner_num; ++i) out[off + i] += alpha[n] * x[off + i];
+  }
+}
+
+/* ---- shadow/operators/kernels/batch_norm.cpp:11-24  Vision::BatchNorm ---- */
+API void orc_batch_norm(const float* in, int count, const float* mean, const float* variance,
+                        int channel, int inner_num, float scale_factor, float eps, float* out) {
+  for (int i = 0; i < count; ++i) {
+    int index = (i / inner_num) % channel;
+    out[i] = (in[i] - mean[index] * scale_factor) /
+             sqrtf(fabsf(variance[index] * scale_factor) + eps);
+  }
+}
+
+/* ---- shadow/operators/kernels/softmax.cpp:10-42  Vision::Softmax: four passes,
+ *      std::max(x, running) for the maximum, fp32 running sum over dim ---- */
+API void orc_softmax(const float* in, int outer_num, int dim, int inner_num, float* val,
+                     float* out) {
+  int val_count = outer_num * inner_num, count = val_count * dim;
+  for (int i = 0; i < val_count; ++i) {
+    int n = i / inner_num, s = i % inner_num;
+    const float* p = in + n * dim * inner_num + s;
+    float max_val = -FLT_MAX;
+    for (int c = 0; c < dim; ++c, p += inner_num) max_val = std_max(*p, max_val);
+    val[i] = max_val;
+  }
+  for (int i = 0; i < count; ++i) {
+    int n = i / dim / inner_num, s = i % inner_num;
+    out[i] = expf(in[i] - val[n * inner_num + s]);
+  }
+  for (int i = 0; i < val_count; ++i) {
+    int n = i / inner_num, s = i % inner_num;
+    const float* p = out + n * dim * inner_num + s;
+    float sum = 0.f;
+    for (int c = 0; c < dim; ++c, p += inner_num) sum += *p;
+    val[i] = sum;
+  }
+  for (int i = 0; i < count; ++i) {
+    int n = i / dim / inner_num, s = i % inner_num;
+    out[i] /= val[n * inner_num + s];
+  }
+}
+
+/* ---- shadow/operators/kernels/normalize.cpp:10-43  Vision::Normalize: fp64
+ *      running sum over dim, then x / max(norm, eps) ---- */
+API void orc_normalize(const float* in, int outer_num, int dim, int inner_num, float* val,
+                       float p, float eps, float* out) {
+  int val_count = outer_num * inner_num, count = val_count * dim;
+  for (int i = 0; i < val_count; ++i) {
+    int n = i / inner_num, s = i % inner_num;
+    const float* q = in + n * dim * inner_num + s;
+    double acc = 0;
+    if (p == 1) {
+      for (int c = 0; c < dim; ++c, q += inner_num) acc += fabsf(*q);
+      val[i] = (float)acc;
+    } else if (p == 2) {
+      for (int c = 0; c < dim; ++c, q += inner_num) {
+        float abs_data = fabsf(*q);
+        acc += abs_data * abs_data; /* fp32 product, widened afterwards */
+      }
+      val[i] = sqrtf((float)acc);
+    } else {
+      /* std::pow(float, float) is the fp32 overload */
+      for (int c = 0; c < dim; ++c, q += inner_num) acc += powf(fabsf(*q), p);
+      val[i] = powf((float)acc, 1.f / p);
+    }
+  }
+  for (int i = 0; i < count; ++i) {
+    int n = i / dim / inner_num, s = i % inner_num;
+    out[i] = in[i] / std_max(val[n * inner_num + s], eps);
+  }
+}
+
+/* ---- shadow/operators/kernels/pooling.cpp:7-42  Vision::Pooling2D.
+ *      pool_type 0 = max, 1 = average over the window clipped to input + pad ---- */
+API void orc_pooling2d(const float* in, const int* in_shape, int pool_type, int kernel_h,
+                       int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+                       const int* out_shape, float* out) {
+  int batch = in_shape[0], channel = in_shape[1];
+  int in_h = in_shape[2], in_w = in_shape[3];
+  int out_h = out_shape[2], out_w = out_shape[3];
+  for (int b = 0; b < batch; ++b) {
+    for (int c = 0; c < channel; ++c, in += in_h * in_w) {
+      for (int h = 0; h < out_h; ++h) {
+        for (int w = 0; w < out_w; ++w) {
+          int hstart = h * stride_h - pad_h, wstart = w * stride_w - pad_w;
+          int hend = hstart + kernel_h < in_h + pad_h ? hstart + kernel_h : in_h + pad_h;
+          int wend = wstart + kernel_w < in_w + pad_w ? wstart + kernel_w : in_w + pad_w;
+          int pool_size = (hend - hstart) * (wend - wstart);
+          if (hstart < 0) hstart = 0;
+          if (wstart < 0) wstart = 0;
+          if (hend > in_h) hend = in_h;
+          if (wend > in_w) wend = in_w;
+          float max_val = -FLT_MAX, sum_val = 0.f;
+          for (int ph = hstart; ph < hend; ++ph) {
+            for (int pw = wstart; pw < wend; ++pw) {
+              float value = in[ph * in_w + pw];
+              max_val = std_max(max_val, value);
+              sum_val += value;
+            }
+          }
+          *out++ = (pool_type == 0) ? max_val : sum_val / pool_size;
+        }
+      }
+    }
+  }
+}
+
+/* ---- shadow/operators/kernels/pooling.cpp:44-86  Vision::Pooling3D ---- */
+API void orc_pooling3d(const float* in, const int* in_shape, int pool_type, int kernel_d,
+                       int kernel_h, int kernel_w, int stride_d, int stride_h, int stride_w,
+                       int pad_d, int pad_h, int pad_w, const int* out_shape, float* out) {
+  int batch = in_shape[0], channel = in_shape[1];
+  int in_d = in_shape[2], in_h = in_shape[3], in_w = in_shape[4];
+  int out_d = out_shape[2], out_h = out_shape[3], out_w = out_shape[4];
+  for (int b = 0; b < batch; ++b) {
+    for (int c = 0; c < channel; ++c, in += in_d * in_h * in_w) {
+      for (int d = 0; d < out_d; ++d) {
+        for (int h = 0; h < out_h; ++h) {
+          for (int w = 0; w < out_w; ++w) {
+            int dstart = d * stride_d - pad_d, hstart = h * stride_h - pad_h,
+                wstart = w * stride_w - pad_w;
+            int dend = dstart + kernel_d < in_d + pad_d ? dstart + kernel_d : in_d + pad_d;
+            int hend = hstart + kernel_h < in_h + pad_h ? hstart + kernel_h : in_h + pad_h;
+            int wend = wstart + kernel_w < in_w + pad_w ? wstart + kernel_w : in_w + pad_w;
+            int pool_size = (dend - dstart) * (hend - hstart) * (wend - wstart);
+            if (dstart < 0) dstart = 0;
+            if (hstart < 0) hstart = 0;
+            if (wstart < 0) wstart = 0;
+            if (dend > in_d) dend = in_d;
+            if (hend > in_h) hend = in_h;
+            if (wend > in_w) wend = in_w;
+            float max_val = -FLT_MAX, sum_val = 0.f;
+            for (int pd = dstart; pd < dend; ++pd) {
+              for (int ph = hstart; ph < hend; ++ph) {
+                for (int pw = wstart; pw < wend; ++pw) {
+                  float value = in[(pd * in_h + ph) * in_w + pw];
+                  max_val = std_max(max_val, value);
+                  sum_val += value;
+                }
+              }
+            }
+            *out++ = (pool_type == 0) ? max_val : sum_val / pool_size;
+          }
+        }
+      }
+    }
+  }
+}
+
+/* ---- shadow/operators/pooling_op.cpp:7-17  pooling_out_size (fp32 arithmetic) ---- */
+API int orc_pooling_out_size(int dim, int kernel_size, int stride, int pad, int full_pooling) {
+  float t = (dim + 2.f * pad - kernel_size) / stride;
+  return (int)((full_pooling ? ceilf(t) : floorf(t)) + 1);
+}

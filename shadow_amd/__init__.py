@@ -72,6 +72,12 @@ SIGNATURES = {
     "shdw_hip_reduce_workspace_bytes": (_Z, [_I, c_int_p, _I, c_int_p]),
     "shdw_hip_reduce": (_I, [_I, _I, c_int_p, _I, c_int_p, _V, _V, _V, _Z, _V]),
     "shdw_hip_scale_residual_relu_rowmean": (_I, [_I, _I, _I, _V, _V, _V, _V, _V, _V, _V]),
+    "shdw_hip_axpy_rows": (_I, [_I, _I, _V, _V, _V, _V, _V]),
+    "shdw_hip_batch_norm": (_I, [_I, _I, _I, _V, _V, _V, _F, _F, _V, _V]),
+    "shdw_hip_softmax": (_I, [_I, _I, _I, _V, _V, _V]),
+    "shdw_hip_normalize": (_I, [_I, _I, _I, _F, _F, _V, _V, _V]),
+    "shdw_hip_pooling2d": (_I, [c_int_p, _I, _I, _I, _I, _I, _I, _I, c_int_p, _V, _V, _V]),
+    "shdw_hip_pooling3d": (_I, [c_int_p, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, c_int_p, _V, _V, _V]),
     "shdw_hip_plan_broadcast": (_I, [_I, c_int_p, c_int_p, c_int_p, c_int_p, c_int_p, c_int_p]),
     "shdw_hip_plan_reduce": (_I, [_I, c_int_p, _I, c_int_p, c_int_p, c_int_p, c_int_p, c_int_p, c_int_p]),
 }

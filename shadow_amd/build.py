@@ -31,7 +31,8 @@ HIP_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-HIP_SOURCES = ["elementwise.hip", "broadcast.hip", "reduce.hip", "fused.hip", "runtime.hip"]
+HIP_SOURCES = ["elementwise.hip", "broadcast.hip", "reduce.hip", "fused.hip", "vision.hip", "softmax.hip",
+               "runtime.hip"]
 # The reference's Release flags (CMakeLists.txt:30-37) plus contraction off so
 # that no host can fuse what baseline x86-64 does not.
 ORACLE_FLAGS = ["-O3", "-DNDEBUG", "-fPIC", "-ffp-contract=off", "-fno-fast-math"]

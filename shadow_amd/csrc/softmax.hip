@@ -1,0 +1,240 @@
+// Softmax and Normalize: x viewed as [outer][dim][inner]; a statistic is folded
+// over `dim` for every (outer, inner) column and then applied to the column.
+//
+// Shadow folds each column front to back (an fp32 running sum for Softmax, an
+// fp64 one for Normalize); both are order-dependent, so a column is always
+// folded by ONE lane in that order and the results match bit for bit.  Two
+// layouts keep the global accesses coalesced around that constraint:
+//   * columns : inner >= 64 (or a slab too large for LDS).  Lane = column,
+//               neighbouring lanes read neighbouring addresses.
+//   * slab    : inner < 64.  One workgroup per outer index copies its
+//               contiguous [dim][inner] slab into LDS with all lanes, `inner`
+//               lanes fold the columns out of LDS, all lanes write back.
+// The elementwise parts (exp, divide) are done by every lane in both layouts.
+#include <hip/hip_runtime.h>
+
+#include <cfloat>
+
+#include "../../include/shadow_hip.h"
+#include "device_common.h"
+#include "launch.h"
+#include "libm_exact.h"
+
+#pragma clang fp contract(off)
+
+namespace shdw {
+
+constexpr int kSlabMaxFloats = 15 * 1024;  // slab + per-column statistics, 60 KB of LDS
+
+// std::max(a, b) of libstdc++: b only when a < b.
+SHDW_DEVICE float std_max(float a, float b) { return a < b ? b : a; }
+
+// ---------------------------------------------------------------------------
+// Softmax (shadow/operators/kernels/softmax.cpp:10-42)
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void softmax_columns_kernel(const float* x, float* y,
+                                                                  uint32_t columns, uint32_t dim,
+                                                                  FastDiv f_inner) {
+  __shared__ uint64_t tab[32];
+  if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
+  __syncthreads();
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= columns) return;
+  uint32_t n, s;
+  fd_divmod(i, f_inner, n, s);
+  const uint32_t inner = f_inner.d;
+  const uint64_t base = static_cast<uint64_t>(n) * dim * inner + s;
+  const float* xc = x + base;
+  float* yc = y + base;
+  float max_val = -FLT_MAX;
+  for (uint32_t c = 0; c < dim; ++c) max_val = std_max(xc[static_cast<uint64_t>(c) * inner], max_val);
+  float sum = 0.f;
+  for (uint32_t c = 0; c < dim; ++c) {
+    const float e = libm::exact_expf(xc[static_cast<uint64_t>(c) * inner] - max_val, tab);
+    yc[static_cast<uint64_t>(c) * inner] = e;
+    sum += e;
+  }
+  for (uint32_t c = 0; c < dim; ++c) yc[static_cast<uint64_t>(c) * inner] /= sum;
+}
+
+__global__ __launch_bounds__(kBlock) void softmax_slab_kernel(const float* x, float* y,
+                                                               uint32_t dim, FastDiv f_inner) {
+  extern __shared__ float lds[];
+  __shared__ uint64_t tab[32];
+  const uint32_t inner = f_inner.d;
+  const uint32_t slab = dim * inner;
+  float* stat = lds + slab;
+  const float* xs = x + static_cast<uint64_t>(blockIdx.x) * slab;
+  float* ys = y + static_cast<uint64_t>(blockIdx.x) * slab;
+  if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
+  for (uint32_t t = threadIdx.x; t < slab; t += kBlock) lds[t] = xs[t];
+  __syncthreads();
+  for (uint32_t s = threadIdx.x; s < inner; s += kBlock) {
+    float max_val = -FLT_MAX;
+    for (uint32_t c = 0; c < dim; ++c) max_val = std_max(lds[c * inner + s], max_val);
+    stat[s] = max_val;
+  }
+  __syncthreads();
+  for (uint32_t t = threadIdx.x; t < slab; t += kBlock) {
+    const uint32_t s = t - fd_div(t, f_inner) * inner;
+    lds[t] = libm::exact_expf(lds[t] - stat[s], tab);
+  }
+  __syncthreads();
+  for (uint32_t s = threadIdx.x; s < inner; s += kBlock) {
+    float sum = 0.f;
+    for (uint32_t c = 0; c < dim; ++c) sum += lds[c * inner + s];
+    stat[s] = sum;
+  }
+  __syncthreads();
+  for (uint32_t t = threadIdx.x; t < slab; t += kBlock) {
+    const uint32_t s = t - fd_div(t, f_inner) * inner;
+    ys[t] = lds[t] / stat[s];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Normalize (shadow/operators/kernels/normalize.cpp:10-43)
+//   PMODE 1: sum |x|          2: sqrt(sum |x|^2)      0: (sum |x|^p)^(1/p)
+// ---------------------------------------------------------------------------
+template <int PMODE>
+SHDW_DEVICE double norm_term(float v, float p) {
+  const float a = __builtin_fabsf(v);
+  if (PMODE == 1) return static_cast<double>(a);
+  if (PMODE == 2) {
+    const float sq = a * a;  // fp32 product, widened afterwards
+    return static_cast<double>(sq);
+  }
+  return static_cast<double>(libm::exact_powf(a, p, libm::kExp2fTab));
+}
+
+template <int PMODE>
+SHDW_DEVICE float norm_finish(double acc, float p, float eps) {
+  float val;
+  if (PMODE == 1) {
+    val = static_cast<float>(acc);
+  } else if (PMODE == 2) {
+    val = __builtin_sqrtf(static_cast<float>(acc));
+  } else {
+    const float inv = 1.f / p;
+    val = libm::exact_powf(static_cast<float>(acc), inv, libm::kExp2fTab);
+  }
+  return std_max(val, eps);
+}
+
+template <int PMODE>
+__global__ __launch_bounds__(kBlock) void normalize_columns_kernel(const float* x, float* y,
+                                                                    uint32_t columns, uint32_t dim,
+                                                                    FastDiv f_inner, float p,
+                                                                    float eps) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= columns) return;
+  uint32_t n, s;
+  fd_divmod(i, f_inner, n, s);
+  const uint32_t inner = f_inner.d;
+  const uint64_t base = static_cast<uint64_t>(n) * dim * inner + s;
+  const float* xc = x + base;
+  float* yc = y + base;
+  double acc = 0;
+  for (uint32_t c = 0; c < dim; ++c) acc += norm_term<PMODE>(xc[static_cast<uint64_t>(c) * inner], p);
+  const float div = norm_finish<PMODE>(acc, p, eps);
+  for (uint32_t c = 0; c < dim; ++c)
+    yc[static_cast<uint64_t>(c) * inner] = xc[static_cast<uint64_t>(c) * inner] / div;
+}
+
+template <int PMODE>
+__global__ __launch_bounds__(kBlock) void normalize_slab_kernel(const float* x, float* y,
+                                                                 uint32_t dim, FastDiv f_inner,
+                                                                 float p, float eps) {
+  extern __shared__ float lds[];
+  const uint32_t inner = f_inner.d;
+  const uint32_t slab = dim * inner;
+  float* stat = lds + slab;
+  const float* xs = x + static_cast<uint64_t>(blockIdx.x) * slab;
+  float* ys = y + static_cast<uint64_t>(blockIdx.x) * slab;
+  for (uint32_t t = threadIdx.x; t < slab; t += kBlock) lds[t] = xs[t];
+  __syncthreads();
+  for (uint32_t s = threadIdx.x; s < inner; s += kBlock) {
+    double acc = 0;
+    for (uint32_t c = 0; c < dim; ++c) acc += norm_term<PMODE>(lds[c * inner + s], p);
+    stat[s] = norm_finish<PMODE>(acc, p, eps);
+  }
+  __syncthreads();
+  for (uint32_t t = threadIdx.x; t < slab; t += kBlock) {
+    const uint32_t s = t - fd_div(t, f_inner) * inner;
+    ys[t] = lds[t] / stat[s];
+  }
+}
+
+// Shared launch geometry: slab layout when the columns are too narrow to
+// coalesce and one slab (plus its statistics) fits the LDS budget.
+struct ColumnGeometry {
+  bool use_slab;
+  uint32_t columns, slab_bytes;
+};
+
+static int column_geometry(int outer_num, int dim, int inner_num, ColumnGeometry* g) {
+  if (outer_num < 0 || dim < 0 || inner_num < 0) return SHDW_E_INVALID_ARGUMENT;
+  const int64_t columns = static_cast<int64_t>(outer_num) * inner_num;
+  const int64_t count = columns * dim;
+  if (count > INT32_MAX || columns > INT32_MAX) return SHDW_E_INVALID_ARGUMENT;
+  g->columns = static_cast<uint32_t>(columns);
+  const int64_t slab = static_cast<int64_t>(dim) * inner_num;
+  g->use_slab = inner_num < 64 && slab + inner_num <= kSlabMaxFloats;
+  g->slab_bytes = static_cast<uint32_t>((slab + inner_num) * sizeof(float));
+  return SHDW_OK;
+}
+
+}  // namespace shdw
+
+using namespace shdw;
+
+extern "C" {
+
+int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, float* y,
+                     void* stream) {
+  ColumnGeometry g;
+  const int rc = column_geometry(outer_num, dim, inner_num, &g);
+  if (rc != SHDW_OK) return rc;
+  if (g.columns == 0 || dim == 0) return SHDW_OK;
+  if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
+  if (g.use_slab)
+    softmax_slab_kernel<<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, static_cast<uint32_t>(dim), fi);
+  else
+    softmax_columns_kernel<<<grid_for(g.columns), kBlock, 0, st>>>(x, y, g.columns,
+                                                                  static_cast<uint32_t>(dim), fi);
+  return launch_status();
+}
+
+int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps, const float* x,
+                       float* y, void* stream) {
+  ColumnGeometry g;
+  const int rc = column_geometry(outer_num, dim, inner_num, &g);
+  if (rc != SHDW_OK) return rc;
+  if (g.columns == 0 || dim == 0) return SHDW_OK;
+  if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
+  const uint32_t d = static_cast<uint32_t>(dim);
+  const int mode = p == 1.f ? 1 : (p == 2.f ? 2 : 0);
+  if (g.use_slab) {
+    if (mode == 1)
+      normalize_slab_kernel<1><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
+    else if (mode == 2)
+      normalize_slab_kernel<2><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
+    else
+      normalize_slab_kernel<0><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
+  } else {
+    const uint32_t grid = grid_for(g.columns);
+    if (mode == 1)
+      normalize_columns_kernel<1><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
+    else if (mode == 2)
+      normalize_columns_kernel<2><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
+    else
+      normalize_columns_kernel<0><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
+  }
+  return launch_status();
+}
+
+}  // extern "C"

@@ -189,3 +189,52 @@ def scale_residual_relu_rowmean(x, scale, bias, res, scale_num, inner_num, want_
                                                       mean.ptr, None))
     _sync()
     return (y.download(count=n) if y else None), mean.download(count=rows)
+
+
+def axpy_rows(alpha, x, y, inner_num, inplace=False):
+    alpha, x, y = _f(alpha).ravel(), _f(x).ravel(), _f(y).ravel()
+    da, dx, dy = Buffer.from_numpy(alpha), Buffer.from_numpy(x), Buffer.from_numpy(y)
+    out = dy if inplace else Buffer(max(4, x.nbytes))
+    check(_lib().shdw_hip_axpy_rows(alpha.size, inner_num, da.ptr, dx.ptr, dy.ptr, out.ptr, None))
+    _sync()
+    return out.download(count=x.size)
+
+
+def batch_norm(x, mean, variance, channel, inner_num, scale_factor, eps, inplace=False):
+    x = _f(x).ravel()
+    dx, dm, dv = Buffer.from_numpy(x), Buffer.from_numpy(_f(mean)), Buffer.from_numpy(_f(variance))
+    y = dx if inplace else Buffer(max(4, x.nbytes))
+    check(_lib().shdw_hip_batch_norm(x.size, channel, inner_num, dx.ptr, dm.ptr, dv.ptr,
+                                     scale_factor, eps, y.ptr, None))
+    _sync()
+    return y.download(count=x.size)
+
+
+def softmax(x, outer, dim, inner, inplace=False):
+    x = _f(x).ravel()
+    dx = Buffer.from_numpy(x)
+    y = dx if inplace else Buffer(max(4, x.nbytes))
+    check(_lib().shdw_hip_softmax(outer, dim, inner, dx.ptr, y.ptr, None))
+    _sync()
+    return y.download(count=x.size)
+
+
+def normalize(x, outer, dim, inner, p, eps, inplace=False):
+    x = _f(x).ravel()
+    dx = Buffer.from_numpy(x)
+    y = dx if inplace else Buffer(max(4, x.nbytes))
+    check(_lib().shdw_hip_normalize(outer, dim, inner, p, eps, dx.ptr, y.ptr, None))
+    _sync()
+    return y.download(count=x.size)
+
+
+def pooling(x, in_shape, pool_type, kernel, stride, pad, out_shape):
+    """2-D or 3-D by len(kernel)."""
+    x = _f(x).ravel()
+    n_out = int(np.prod(out_shape, dtype=np.int64))
+    dx = Buffer.from_numpy(x)
+    y = Buffer(max(4, 4 * n_out))
+    fn = _lib().shdw_hip_pooling2d if len(kernel) == 2 else _lib().shdw_hip_pooling3d
+    check(fn(ints(in_shape), pool_type, *kernel, *stride, *pad, ints(out_shape), dx.ptr, y.ptr, None))
+    _sync()
+    return y.download(count=n_out)

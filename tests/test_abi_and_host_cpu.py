@@ -109,9 +109,11 @@ def keys(fn):
 
 def test_registries_hold_exactly_the_gpu_default_kernels():
     h = shadow_amd.host()
-    assert keys(h.shdw_host_operator_keys) == ["Activate", "Binary", "Eltwise", "Reduce", "Scale", "Unary"]
+    types = ["Activate", "Axpy", "BatchNorm", "Binary", "Eltwise", "Normalize", "Pooling", "Reduce",
+             "Scale", "Softmax", "Unary"]
+    assert keys(h.shdw_host_operator_keys) == types
     kk = keys(h.shdw_host_kernel_keys)
-    assert kk == ["%sGPU(Default)" % t for t in ["Activate", "Binary", "Eltwise", "Reduce", "Scale", "Unary"]]
+    assert kk == ["%sGPU(Default)" % t for t in types]
     # a CUDNN flavour would outrank Default; a CPU kernel would be a compute fallback
     assert not any("CUDNN" in k or "CPU" in k for k in kk)
 

@@ -1,0 +1,228 @@
+"""GPU parity for Axpy, BatchNorm, Softmax, Normalize and Pooling: the C ABI entry
+points and the operators through Operator::Run(), bit for bit against the oracle
+(these kernels fold every column / window in the reference's order, so there is
+no tolerance anywhere in this file)."""
+import numpy as np
+import pytest
+
+import oracle
+import shadow_amd
+from shadow_amd import ShadowError
+from tests import gpuops
+from tests.helpers import assert_bit_exact, normal, uniform, with_specials
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+@pytest.fixture()
+def ws(gpu):
+    w = shadow_amd.Workspace("Native", 0)
+    yield w
+    w.close()
+
+
+def run(ws, op_type, inputs, args, top="out"):
+    names = []
+    for name, arr in inputs:
+        ws.set_blob(name, arr)
+        names.append(name)
+    op = ws.create_op(op_type, names, [top], args)
+    op.run()
+    return ws.get_blob(top)
+
+
+# ------------------------------------------------------------------- axpy ---
+@pytest.mark.parametrize("outer,inner", [(1, 1), (6, 49), (48, 64), (10, 3136), (7, 5), (300, 3), (33, 1001)])
+def test_axpy_rows(gpu, outer, inner):
+    alpha = with_specials(normal(1, outer), 1)
+    x, y = normal(2, outer * inner, 3.0), normal(3, outer * inner)
+    want = oracle.axpy_rows(alpha, x, y, inner)
+    assert_bit_exact(gpuops.axpy_rows(alpha, x, y, inner), want, "axpy_rows")
+    assert_bit_exact(gpuops.axpy_rows(alpha, x, y, inner, inplace=True), want, "axpy_rows in place")
+
+
+def test_axpy_op(ws):
+    alpha, x, y = normal(4, (4, 16)), normal(5, (4, 16, 7, 7)), normal(6, (4, 16, 7, 7))
+    got = run(ws, "Axpy", [("alpha", alpha), ("x", x), ("y", y)], {})
+    assert got.shape == x.shape
+    assert_bit_exact(got, oracle.axpy_op(alpha, x, y), "axpy op")
+    got = run(ws, "Axpy", [("alpha", alpha.reshape(4, 16, 1, 1)), ("x", x), ("y", y)], {})
+    assert_bit_exact(got, oracle.axpy_op(alpha, x, y), "axpy op, 4-d alpha")
+    ws.set_blob("bad", np.zeros((4, 15), F))
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("Axpy", ["bad", "x", "y"], ["o2"], {}).run()
+    with pytest.raises(ShadowError, match="three inputs"):
+        ws.create_op("Axpy", ["x", "y"], ["o3"], {}).run()
+
+
+# ------------------------------------------------------------- batch norm ---
+@pytest.mark.parametrize("shape", [(2, 3, 4, 4), (4, 64, 7, 7), (3, 5, 9, 11), (2, 7, 1, 1), (1, 130, 28, 28)])
+@pytest.mark.parametrize("sf", [1.0, 0.0010000181])
+def test_batch_norm(gpu, shape, sf):
+    x = with_specials(normal(7, shape, 3.0), 7)
+    c, inner = shape[1], int(np.prod(shape[2:]))
+    mean, var = normal(8, c), uniform(9, c, -0.5, 900.0)
+    want = oracle.batch_norm(x, mean, var, c, inner, sf, 1e-5)
+    assert_bit_exact(gpuops.batch_norm(x, mean, var, c, inner, sf, 1e-5), want, "batch_norm")
+    assert_bit_exact(gpuops.batch_norm(x, mean, var, c, inner, sf, 1e-5, inplace=True), want, "in place")
+
+
+def test_batch_norm_op(ws):
+    x = normal(10, (3, 12, 6, 5), 2.0)
+    mean, var = normal(11, 12), uniform(12, 12, 0.1, 5.0)
+    got = run(ws, "BatchNorm", [("x", x), ("mean", mean), ("var", var)], {})
+    assert_bit_exact(got, oracle.batch_norm_op(x, mean, var), "bn op")
+    for scale in (999.982, 0.0):
+        got = run(ws, "BatchNorm", [("x", x), ("mean", mean), ("var", var), ("s", F([scale]))], {"eps": 1e-3})
+        assert_bit_exact(got, oracle.batch_norm_op(x, mean, var, F([scale]), eps=1e-3), "bn op scaled")
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("BatchNorm", ["x", "mean", "var"], ["o2"], {"use_global_stats": False})
+    ws.set_blob("short", np.zeros(11, F))
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("BatchNorm", ["x", "short", "var"], ["o3"], {}).run()
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("BatchNorm", ["x", "mean"], ["o4"], {}).run()
+
+
+# ---------------------------------------------------------------- softmax ---
+SOFTMAX_SHAPES = [  # outer, dim, inner: both layouts, LDS limits, odd sizes
+    (1, 1, 1), (64, 1000, 1), (3, 10, 1), (5, 7, 3), (2, 21, 63), (2, 21, 64), (2, 21, 65),
+    (4, 8, 1024), (1, 15000, 1), (1, 16000, 1), (2, 300, 50), (2, 310, 50), (300, 4, 2),
+    (1, 2, 5000), (3, 1, 17),
+]
+
+
+@pytest.mark.parametrize("outer,dim,inner", SOFTMAX_SHAPES)
+def test_softmax(gpu, outer, dim, inner):
+    x = normal(13, outer * dim * inner, 5.0)
+    want = oracle.softmax(x, outer, dim, inner)
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner), want, "softmax")
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner, inplace=True), want, "softmax in place")
+
+
+@pytest.mark.parametrize("outer,dim,inner", [(40, 50, 1), (2, 12, 200)])
+def test_softmax_special_values(gpu, outer, dim, inner):
+    x = with_specials(normal(14, outer * dim * inner, 30.0), 14)
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax specials")
+
+
+@pytest.mark.parametrize("shape,axis", [((8, 1000), 1), ((2, 21, 33, 35), 1), ((3, 4, 5), -1), ((6, 2, 3), 0)])
+def test_softmax_op(ws, shape, axis):
+    x = normal(15, shape, 3.0)
+    got = run(ws, "Softmax", [("x", x)], {"axis": axis})
+    assert got.shape == x.shape
+    assert_bit_exact(got, oracle.softmax_op(x, axis), "softmax op")
+
+
+def test_softmax_op_defaults_and_errors(ws):
+    x = normal(16, (2, 5, 3))
+    assert_bit_exact(run(ws, "Softmax", [("x", x)], {}), oracle.softmax_op(x, 1), "default axis")
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("Softmax", ["x"], ["o2"], {"axis": 3}).run()
+
+
+# -------------------------------------------------------------- normalize ---
+@pytest.mark.parametrize("p", [1.0, 2.0, 3.0, 0.5])
+@pytest.mark.parametrize("outer,dim,inner", [(64, 512, 1), (5, 7, 3), (2, 16, 100), (3, 9, 64), (1, 20000, 1),
+                                             (2, 1, 9), (1, 33, 4097)])
+def test_normalize(gpu, p, outer, dim, inner):
+    x = normal(17, outer * dim * inner, 2.0)
+    want = oracle.normalize(x, outer, dim, inner, p, 1e-12)
+    assert_bit_exact(gpuops.normalize(x, outer, dim, inner, p, 1e-12), want, "normalize")
+    assert_bit_exact(gpuops.normalize(x, outer, dim, inner, p, 1e-12, inplace=True), want, "in place")
+
+
+@pytest.mark.parametrize("p", [1.0, 2.0, 2.5])
+def test_normalize_special_values(gpu, p):
+    x = with_specials(normal(18, 30 * 64, 2.0), 18)
+    for eps in (1e-12, 0.0, 10.0):
+        assert_bit_exact(gpuops.normalize(x, 30, 64, 1, p, eps), oracle.normalize(x, 30, 64, 1, p, eps),
+                         "normalize specials eps=%g" % eps)
+    z = np.zeros(4 * 6 * 5, F)
+    assert_bit_exact(gpuops.normalize(z, 4, 6, 5, p, 1e-12), oracle.normalize(z, 4, 6, 5, p, 1e-12), "zeros")
+
+
+@pytest.mark.parametrize("args", [{}, {"p": 1.0}, {"p": 3.0, "axis": -1, "eps": 1e-6}, {"axis": 0}])
+def test_normalize_op(ws, args):
+    x = normal(19, (4, 32, 5, 3), 2.0)
+    got = run(ws, "Normalize", [("x", x)], args)
+    want = oracle.normalize_op(x, args.get("p", 2.0), args.get("axis", 1), args.get("eps", 1e-12))
+    assert got.shape == x.shape
+    assert_bit_exact(got, want, "normalize op")
+
+
+# ---------------------------------------------------------------- pooling ---
+POOL_2D = [
+    ((2, 3, 12, 12), [3], [2], [0], True), ((2, 3, 12, 12), [3], [2], [1], True),
+    ((2, 3, 12, 12), [3], [2], [1], False), ((1, 2, 7, 9), [2, 3], [2, 1], [1, 0], True),
+    ((2, 4, 7, 7), [7], [1], [0], True), ((1, 1, 5, 5), [5], [3], [2], True),
+    ((3, 2, 8, 8), [2], [2], [0], False), ((1, 2, 6, 6), [3], [3], [2], True),
+    ((2, 16, 56, 56), [3], [2], [0], True), ((1, 5, 33, 17), [5, 3], [1, 2], [2, 1], False),
+]
+
+
+@pytest.mark.parametrize("pool", [0, 1])
+@pytest.mark.parametrize("shape,kernel,stride,pad,full", POOL_2D)
+def test_pooling2d_op(ws, pool, shape, kernel, stride, pad, full):
+    x = with_specials(normal(20, shape, 2.0), 20).reshape(shape)
+    args = {"pool": pool, "kernel_size": kernel, "stride": stride, "pad": pad, "full_pooling": full}
+    got = run(ws, "Pooling", [("x", x)], args)
+    want = oracle.pooling_op(x, pool, kernel, stride, pad, full_pooling=full)
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "pooling2d")
+
+
+@pytest.mark.parametrize("pool", [0, 1])
+@pytest.mark.parametrize("shape,kernel,stride,pad", [((2, 2, 6, 7, 8), [3], [2], [1]),
+                                                     ((1, 3, 4, 5, 5), [2, 3, 2], [1, 2, 2], [0, 1, 1]),
+                                                     ((2, 2, 3, 4, 4), [3, 4, 4], [1], [0]),
+                                                     ((1, 4, 8, 14, 14), [2], [2], [0])])
+def test_pooling3d_op(ws, pool, shape, kernel, stride, pad):
+    x = normal(21, shape, 2.0)
+    got = run(ws, "Pooling", [("x", x)], {"pool": pool, "kernel_size": kernel, "stride": stride, "pad": pad})
+    want = oracle.pooling_op(x, pool, kernel, stride, pad)
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "pooling3d")
+
+
+# whole-plane windows: both workgroup shapes, chunked and unchunked rows, ragged last group
+@pytest.mark.parametrize("pool", [0, 1])
+@pytest.mark.parametrize("shape", [(4, 128, 7, 7), (3, 5, 14, 14), (2, 3, 56, 56), (1, 70, 3, 3), (2, 2, 4, 2),
+                                   (130, 2048, 7, 7), (2, 9, 10, 10), (1, 3, 2, 7, 7), (2, 65, 13, 15)])
+def test_global_pooling_op(ws, pool, shape):
+    x = normal(22, shape, 2.0)
+    got = run(ws, "Pooling", [("x", x)], {"pool": pool, "global_pooling": True})
+    want = oracle.pooling_op(x, pool, global_pooling=True)
+    assert got.shape == want.shape == tuple(shape[:2]) + (1,) * (len(shape) - 2)
+    assert_bit_exact(got, want, "global pooling")
+
+
+def test_pooling_op_errors(ws):
+    ws.set_blob("x", np.zeros((2, 3, 8, 8), F))
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("Pooling", ["x"], ["o"], {"pool": 2, "kernel_size": [2]})
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("Pooling", ["x"], ["x"], {"kernel_size": [2]}).run()  # in place is refused
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("Pooling", ["x"], ["o2"], {"kernel_size": [2, 2, 2]}).run()
+    ws.set_blob("flat", np.zeros((2, 3, 8), F))
+    with pytest.raises(ShadowError, match="2D or 3D"):
+        ws.create_op("Pooling", ["flat"], ["o3"], {"kernel_size": [2]}).run()
+
+
+def test_entry_point_argument_errors(gpu):
+    lib = shadow_amd.hip()
+    buf = shadow_amd.Buffer(1024)
+    E = -1
+    assert lib.shdw_hip_softmax(-1, 2, 2, buf.ptr, buf.ptr, None) == E
+    assert lib.shdw_hip_softmax(2, 2, 2, None, buf.ptr, None) == E
+    assert lib.shdw_hip_softmax(0, 5, 5, None, None, None) == 0
+    assert lib.shdw_hip_normalize(65536, 65536, 2, 2.0, 0.0, buf.ptr, buf.ptr, None) == E
+    assert lib.shdw_hip_batch_norm(8, 0, 1, buf.ptr, buf.ptr, buf.ptr, 1.0, 0.0, buf.ptr, None) == E
+    assert lib.shdw_hip_axpy_rows(65536, 65536, buf.ptr, buf.ptr, buf.ptr, buf.ptr, None) == E
+    sh = shadow_amd.ints([1, 1, 4, 4])
+    assert lib.shdw_hip_pooling2d(sh, 2, 2, 2, 1, 1, 0, 0, sh, buf.ptr, buf.ptr, None) == E
+    assert lib.shdw_hip_pooling2d(sh, 0, 0, 2, 1, 1, 0, 0, sh, buf.ptr, buf.ptr, None) == E
+    assert lib.shdw_hip_pooling2d(sh, 0, 2, 2, 0, 1, 0, 0, sh, buf.ptr, buf.ptr, None) == E
+    assert lib.shdw_hip_pooling2d(sh, 0, 2, 2, 1, 1, 0, 0, shadow_amd.ints([2, 1, 3, 3]), buf.ptr, buf.ptr, None) == E

@@ -1,0 +1,238 @@
+"""Pins for the oracle's Axpy / BatchNorm / Softmax / Normalize / Pooling
+restatements.  The reference holds no vectors for these either, so each is
+checked against an independent numpy formulation (axis operations and slicing,
+never the oracle's flat pointer walks), against exactly representable data with
+one right answer, and against hand-computed special cases.  numpy's float32
+`add.accumulate` is a front-to-back running sum, which is what pins the
+summation ORDER; expf/powf digits are taken from the already pinned unary and
+binary oracle functions, so only the composition is under test here."""
+import numpy as np
+import pytest
+
+import oracle
+from tests.helpers import assert_bit_exact, bits, normal, uniform, with_specials
+
+F = np.float32
+
+
+def running_sum(a, axis, dtype):
+    acc = np.add.accumulate(a.astype(dtype), axis=axis, dtype=dtype)
+    return np.take(acc, -1, axis=axis)
+
+
+# ------------------------------------------------------------------- axpy ---
+def test_axpy_rows_closed_form():
+    alpha, x, y = normal(1, (6, 5)), normal(2, (6, 5, 7, 3)), normal(3, (6, 5, 7, 3))
+    want = y + alpha[:, :, None, None] * x  # two rounded numpy operations
+    assert_bit_exact(oracle.axpy_op(alpha, x, y), want, "axpy")
+    assert_bit_exact(oracle.axpy_op(alpha.reshape(6, 5, 1, 1), x, y), want, "axpy 4-d alpha")
+    # a fused multiply-add would differ on some of these
+    fused = (y.astype(np.float64) + alpha[:, :, None, None].astype(np.float64) * x).astype(F)
+    assert (bits(fused) != bits(want)).any()
+
+
+def test_axpy_op_checks():
+    x = np.zeros((2, 3, 4, 4), F)
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.axpy_op(np.zeros((2, 4), F), x, x)
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.axpy_op(np.zeros((2, 3, 2, 1), F), x, x)
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.axpy_op(np.zeros((2, 3), F), x, np.zeros((2, 3, 4, 5), F))
+
+
+# ------------------------------------------------------------- batch norm ---
+@pytest.mark.parametrize("scale", [None, 0.0, 1.0, 999.982])
+def test_batch_norm_closed_form(scale):
+    x = with_specials(normal(4, (3, 8, 5, 5), 3.0), 4).reshape(3, 8, 5, 5)
+    mean, var = normal(5, 8), uniform(6, 8, -0.5, 4.0)  # negative variances exercise the abs
+    eps = F(1e-5)
+    sf = F(1) if scale is None else (F(0) if scale == 0 else F(1) / F(scale))
+    with np.errstate(all="ignore"):
+        m = (mean * sf)[None, :, None, None]
+        d = np.sqrt(np.abs(var * sf) + eps)[None, :, None, None]
+        want = (x - m) / d
+    got = oracle.batch_norm_op(x, mean, var, None if scale is None else F([scale]), eps=1e-5)
+    assert_bit_exact(got, want, "batch_norm")
+
+
+def test_batch_norm_known_values_and_checks():
+    # (x - 1) / sqrt(4 + 0) with eps = 0: exact halves
+    got = oracle.batch_norm_op(F([[[[1, 3, 5]]]]), F([1]), F([4]), eps=0.0)
+    assert got.ravel().tolist() == [0.0, 1.0, 2.0]
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.batch_norm_op(np.zeros((1, 2, 2, 2), F), F([0]), F([1, 1]))
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.batch_norm_op(np.zeros((1, 2, 2, 2), F), F([0, 0]), F([1, 1]), scale=F([1, 2]))
+
+
+# ---------------------------------------------------------------- softmax ---
+def softmax_numpy(x, axis):
+    mx = np.max(x, axis=axis, keepdims=True)
+    e = oracle.unary(4, (x - mx).ravel()).reshape(x.shape)  # host expf, pinned elsewhere
+    s = np.expand_dims(running_sum(e, axis, F), axis)
+    return e / s
+
+
+@pytest.mark.parametrize("shape,axis", [((4, 10), 1), ((3, 5, 7, 2), 1), ((2, 6, 9), 2), ((5, 3, 4), 0),
+                                        ((2, 1000), -1), ((2, 21, 17, 19), 1)])
+def test_softmax_against_axis_formulation(shape, axis):
+    x = normal(7, shape, 4.0)
+    assert_bit_exact(oracle.softmax_op(x, axis), softmax_numpy(x, axis % len(shape)), "softmax")
+
+
+def test_softmax_sum_is_front_to_back_fp32():
+    # Terms chosen so that fp32 running sums in other orders (or in fp64) differ.
+    x = np.log(np.array([[1.0, 2.0 ** -24, 2.0 ** -24, 2.0 ** -24, 2.0 ** -24]])).astype(F)
+    out = oracle.softmax_op(x, 1)
+    # front to back: 1 + 2^-24 rounds back to 1 every time, so the sum stays 1
+    assert out[0, 0] == F(1.0)
+    y = x[:, ::-1].copy()  # back to front the small terms add up first
+    out_r = oracle.softmax_op(y, 1)
+    assert out_r[0, -1] < F(1.0)
+
+
+def test_softmax_known_values():
+    assert_bit_exact(oracle.softmax_op(np.full((2, 8), 3.25, F)), np.full((2, 8), 0.125, F), "uniform")
+    assert_bit_exact(oracle.softmax_op(F([[5.0]]), 1), F([[1.0]]), "single")
+    out = oracle.softmax_op(F([[0.0, -np.inf, 0.0]]))
+    assert out.ravel().tolist() == [0.5, 0.0, 0.5]
+    # any NaN poisons its column; a column of -inf keeps the finite identity and ends 0/0
+    assert np.isnan(oracle.softmax_op(F([[np.nan, 1, 2], [1, 2, np.nan]]))).all()
+    assert np.isnan(oracle.softmax_op(F([[-np.inf, -np.inf]]))).all()
+    # shift by a power of two keeps x - max exact
+    x = normal(8, (3, 40))
+    x = np.round(x * 64) / 64
+    assert_bit_exact(oracle.softmax_op(x + F(8)), oracle.softmax_op(x), "shift invariance")
+
+
+# -------------------------------------------------------------- normalize ---
+def normalize_numpy(x, p, axis, eps):
+    a = np.abs(x)
+    if p == 1:
+        val = running_sum(a, axis, np.float64).astype(F)
+    elif p == 2:
+        val = np.sqrt(running_sum(a * a, axis, np.float64).astype(F))  # fp32 squares
+    else:
+        t = oracle.binary_scalar(4, a.ravel(), p).reshape(x.shape)  # host powf
+        s = running_sum(t, axis, np.float64).astype(F)
+        val = oracle.binary_scalar(4, s.ravel(), F(1) / F(p)).reshape(s.shape)
+    val = np.where(val < F(eps), F(eps), val)
+    return x / np.expand_dims(val, axis)
+
+
+@pytest.mark.parametrize("p", [1.0, 2.0, 3.0, 0.5])
+@pytest.mark.parametrize("shape,axis", [((6, 128), 1), ((2, 16, 5, 5), 1), ((3, 4, 50), -1), ((7, 3), 0)])
+def test_normalize_against_axis_formulation(p, shape, axis):
+    x = normal(9, shape, 2.0)
+    got = oracle.normalize_op(x, p, axis, 1e-12)
+    assert_bit_exact(got, normalize_numpy(x, p, axis % len(shape), 1e-12), "normalize p=%g" % p)
+
+
+def test_normalize_known_values():
+    q = F(3) / F(5), F(4) / F(5)
+    assert oracle.normalize_op(F([[3, 4]]), 2, 1).ravel().tolist() == [q[0], q[1]]
+    assert oracle.normalize_op(F([[3, -4, 1]]), 1, 1).ravel().tolist() == [F(3) / F(8), F(-4) / F(8), F(1) / F(8)]
+    # zero column: 0 / eps
+    assert oracle.normalize_op(np.zeros((1, 4), F), 2, 1).ravel().tolist() == [0.0] * 4
+    # eps takes over when the norm is below it
+    out = oracle.normalize_op(F([[1e-3, 0]]), 2, 1, eps=1.0)
+    assert out.ravel().tolist() == [F(1e-3), 0.0]
+    # the square is taken in fp32: 1e-30^2 underflows to 0 there, not in fp64
+    with np.errstate(all="ignore"):
+        assert np.isinf(oracle.normalize_op(F([[1e-30]]), 2, 1, eps=0.0)).all()
+    out = oracle.normalize_op(F([[1e-30, 1e-30]]), 2, 1, eps=1e-12)
+    assert out.ravel().tolist() == [F(1e-30) / F(1e-12)] * 2
+
+
+# ---------------------------------------------------------------- pooling ---
+def pooling_numpy(x, pool, kernel, stride, pad, out_shape):
+    """Window by slicing; running fp32 sum over the flattened window."""
+    nsp = len(kernel)
+    out = np.empty(out_shape, F)
+    for idx in np.ndindex(*out_shape[2:]):
+        lo = [i * s - p for i, s, p in zip(idx, stride, pad)]
+        hi = [min(l + k, d + p) for l, k, d, p in zip(lo, kernel, x.shape[2:], pad)]
+        size = int(np.prod([h - l for h, l in zip(hi, lo)]))
+        sl = tuple(slice(max(l, 0), min(h, d)) for l, h, d in zip(lo, hi, x.shape[2:]))
+        win = x[(slice(None), slice(None)) + sl].reshape(x.shape[0], x.shape[1], -1)
+        if pool == 0:
+            m = np.full(win.shape[:2], np.finfo(F).min, F)
+            for j in range(win.shape[2]):
+                m = np.where(m < win[:, :, j], win[:, :, j], m)
+            res = m
+        else:
+            s = np.zeros(win.shape[:2], F)
+            for j in range(win.shape[2]):
+                s = s + win[:, :, j]
+            with np.errstate(all="ignore"):
+                res = s / F(size)
+        out[(slice(None), slice(None)) + idx] = res
+    return out
+
+
+CASES_2D = [
+    ((2, 3, 12, 12), [3], [2], [0], True), ((2, 3, 12, 12), [3], [2], [1], True),
+    ((2, 3, 12, 12), [3], [2], [1], False), ((1, 2, 7, 9), [2, 3], [2, 1], [1, 0], True),
+    ((2, 4, 7, 7), [7], [1], [0], True), ((1, 1, 5, 5), [5], [3], [2], True),
+    ((3, 2, 8, 8), [2], [2], [0], False), ((1, 2, 6, 6), [3], [3], [2], True),
+]
+
+
+@pytest.mark.parametrize("pool", [0, 1])
+@pytest.mark.parametrize("shape,kernel,stride,pad,full", CASES_2D)
+def test_pooling2d_against_slicing(pool, shape, kernel, stride, pad, full):
+    x = normal(10, shape, 2.0)
+    got = oracle.pooling_op(x, pool, kernel, stride, pad, full_pooling=full)
+    k, s, p = [v * 2 if len(v) == 1 else v for v in (kernel, stride, pad)]
+    assert_bit_exact(got, pooling_numpy(x, pool, k, s, p, got.shape), "pool2d")
+
+
+@pytest.mark.parametrize("pool", [0, 1])
+@pytest.mark.parametrize("shape,kernel,stride,pad", [((2, 2, 6, 7, 8), [3], [2], [1]),
+                                                     ((1, 3, 4, 5, 5), [2, 3, 2], [1, 2, 2], [0, 1, 1]),
+                                                     ((2, 2, 3, 4, 4), [3, 4, 4], [1], [0])])
+def test_pooling3d_against_slicing(pool, shape, kernel, stride, pad):
+    x = normal(11, shape, 2.0)
+    got = oracle.pooling_op(x, pool, kernel, stride, pad)
+    k, s, p = [v * 3 if len(v) == 1 else v for v in (kernel, stride, pad)]
+    assert_bit_exact(got, pooling_numpy(x, pool, k, s, p, got.shape), "pool3d")
+
+
+def test_pooling_known_values():
+    x = np.arange(25, dtype=F).reshape(1, 1, 5, 5)
+    # 3x3 stride 2, no pad: maxima are the window corners, means the centres
+    assert oracle.pooling_op(x, 0, [3], [2], [0]).ravel().tolist() == [12, 14, 22, 24]
+    assert oracle.pooling_op(x, 1, [3], [2], [0]).ravel().tolist() == [6, 8, 16, 18]
+    # global pooling ignores kernel/stride/pad arguments
+    assert oracle.pooling_op(x, 1, [2], [5], [3], global_pooling=True).ravel().tolist() == [12]
+    assert oracle.pooling_op(x, 0, global_pooling=True).shape == (1, 1, 1, 1)
+    # the average divides by the window clipped to input + pad, not to the input:
+    # top-left 2x2 window with pad 1 holds one real value but counts 4 cells
+    got = oracle.pooling_op(np.full((1, 1, 2, 2), 8, F), 1, [2], [2], [1], full_pooling=False)
+    assert got.ravel().tolist() == [2.0, 2.0, 2.0, 2.0]
+    # max ignores NaN (NaN never compares greater) and starts from the finite identity
+    assert oracle.pooling_op(F([[[[np.nan, 1], [2, np.nan]]]]), 0, [2], [2], [0]).ravel().tolist() == [2.0]
+    assert bits(oracle.pooling_op(F([[[[-np.inf] * 2] * 2]]), 0, [2], [2], [0]))[0, 0, 0, 0] == 0xff7fffff
+    # first zero wins the sign
+    assert bits(oracle.pooling_op(F([[[[-0.0, 0.0], [0.0, 0.0]]]]), 0, [2], [2], [0])).ravel()[0] == 0x80000000
+
+
+def test_pooling_out_size_formula():
+    # ceil / floor of an fp32 quotient, plus one; no clipping of the last window
+    assert oracle.pooling_out_size(112, 3, 2, 0, True) == 56
+    assert oracle.pooling_out_size(112, 3, 2, 0, False) == 55
+    assert oracle.pooling_out_size(112, 3, 2, 1, True) == 57
+    assert oracle.pooling_out_size(112, 3, 2, 1, False) == 56
+    assert oracle.pooling_out_size(7, 7, 1, 0, True) == 1
+    assert oracle.pooling_out_size(5, 2, 2, 0, True) == 3
+    assert oracle.pooling_out_size(5, 2, 2, 0, False) == 2
+
+
+def test_pooling_op_checks():
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.pooling_op(np.zeros((2, 3, 4), F), 0, [2])
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.pooling_op(np.zeros((2, 3, 4, 4), F), 2, [2])
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.pooling_op(np.zeros((2, 3, 4, 4), F), 0, [2, 2, 2])
