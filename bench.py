@@ -292,6 +292,42 @@ def config_table(dev):
     ms = time_batch(dev, lambda k: lib.shdw_hip_scale_residual_relu_rowmean(
         n5, C5, in5, A[k].ptr, g5.ptr, b5.ptr, A[(k + 1) % SETS].ptr, Y[k].ptr, M[k].ptr, st), SETS)
     add(5, "fused_tail", 12 * n5 + 8 * C5 + 4 * 65536, ms, n5)
+
+    # Operators next to the path (label "next"), on ResNet-sized tensors of the
+    # same 51 MB: BatchNorm / Axpy on [64,1024,14,14], the stem max pooling on
+    # [16,64,112,112], global average pooling on [128,2048,7,7], Softmax and
+    # Normalize over channels of a dense map, and the classifier Softmax.
+    mean5, var5 = dev.buf(normal(601, C5)), dev.buf(uniform(602, C5, 0.5, 2.0))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_batch_norm(n5, C5, in5, A[k].ptr, mean5.ptr, var5.ptr,
+                                                           1.0, 1e-5, Y[k].ptr, st), SETS)
+    add("next", "batch_norm", 8 * n5 + 8 * C5, ms, n5)
+    al5 = dev.buf(uniform(603, 65536, 0.0, 1.0))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_axpy_rows(65536, in5, al5.ptr, A[k].ptr,
+                                                          A[(k + 1) % SETS].ptr, Y[k].ptr, st), SETS)
+    add("next", "axpy_rows", 12 * n5 + 4 * 65536, ms, n5)
+    pin, pout = [16, 64, 112, 112], [16, 64, 56, 56]
+    npo = int(np.prod(pout))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_pooling2d(I(pin), 0, 3, 3, 2, 2, 0, 0, I(pout), A[k].ptr,
+                                                          Y[k].ptr, st), SETS)
+    add("next", "pooling_max_3x3s2", 4 * (NBIG + npo), ms, NBIG)
+    gin, gout = [128, 2048, 7, 7], [128, 2048, 1, 1]
+    ms = time_batch(dev, lambda k: lib.shdw_hip_pooling2d(I(gin), 1, 7, 7, 1, 1, 0, 0, I(gout), A[k].ptr,
+                                                          Y[k].ptr, st), SETS)
+    add("next", "pooling_global_avg_7x7", 4 * (NBIG + 128 * 2048), ms, NBIG)
+    gin2, gout2 = [64, 1024, 14, 14], [64, 1024, 1, 1]
+    ms = time_batch(dev, lambda k: lib.shdw_hip_pooling2d(I(gin2), 1, 14, 14, 1, 1, 0, 0, I(gout2), A[k].ptr,
+                                                          Y[k].ptr, st), SETS)
+    add("next", "pooling_global_avg_14x14", 4 * (NBIG + 65536), ms, NBIG)
+    # [16, 49, 128, 128]: channel softmax / L2 normalize of a dense map (inner = 16384)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_softmax(16, 49, 16384, A[k].ptr, Y[k].ptr, st), SETS)
+    add("next", "softmax_channels_dense", 8 * NBIG, ms, NBIG)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_normalize(16, 49, 16384, 2.0, 1e-12, A[k].ptr, Y[k].ptr, st),
+                    SETS)
+    add("next", "normalize_l2_channels_dense", 8 * NBIG, ms, NBIG)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_softmax(64, 1000, 1, A[k].ptr, Y[k].ptr, st), SETS)
+    add("next", "softmax_classifier_64x1000", 8 * 64000, ms, 64000)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_normalize(64, 512, 1, 2.0, 1e-12, A[k].ptr, Y[k].ptr, st), SETS)
+    add("next", "normalize_l2_embedding_64x512", 8 * 64 * 512, ms, 64 * 512)
     for bset in (A, Y):
         for bb in bset:
             bb.free()

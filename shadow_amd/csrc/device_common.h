@@ -32,6 +32,9 @@ SHDW_DEVICE void store4_stream(float* p, v4f v) {
 SHDW_DEVICE v4f load4(const float* p) { return *reinterpret_cast<const v4f*>(p); }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+SHDW_DEVICE bool aligned16_device(const void* p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
 
 // ---------------------------------------------------------------------------
 // Division of a 31-bit unsigned value by a divisor fixed at launch time:

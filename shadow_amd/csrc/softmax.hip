@@ -57,18 +57,125 @@ __global__ __launch_bounds__(kBlock) void softmax_columns_kernel(const float* x,
   for (uint32_t c = 0; c < dim; ++c) yc[static_cast<uint64_t>(c) * inner] /= sum;
 }
 
+// Same layout for dim <= DMAX: the column lives in registers, so x is read once
+// and y written once, and all of a lane's loads are in flight together.
+template <int DMAX>
+__global__ __launch_bounds__(kBlock) void softmax_columns_reg_kernel(const float* x, float* y,
+                                                                      uint32_t columns,
+                                                                      uint32_t dim,
+                                                                      FastDiv f_inner) {
+  __shared__ uint64_t tab[32];
+  if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
+  __syncthreads();
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= columns) return;
+  uint32_t n, s;
+  fd_divmod(i, f_inner, n, s);
+  const uint32_t inner = f_inner.d;
+  const uint64_t base = static_cast<uint64_t>(n) * dim * inner + s;
+  const float* xc = x + base;
+  float* yc = y + base;
+  float v[DMAX];
+#pragma unroll
+  for (int c = 0; c < DMAX; ++c)
+    if (c < dim) v[c] = __builtin_nontemporal_load(xc + static_cast<uint64_t>(c) * inner);
+  float max_val = -FLT_MAX;
+#pragma unroll
+  for (int c = 0; c < DMAX; ++c)
+    if (c < dim) max_val = std_max(v[c], max_val);
+  float sum = 0.f;
+#pragma unroll
+  for (int c = 0; c < DMAX; ++c) {
+    if (c < dim) {
+      v[c] = libm::exact_expf(v[c] - max_val, tab);
+      sum += v[c];
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < DMAX; ++c)
+    if (c < dim) __builtin_nontemporal_store(v[c] / sum, yc + static_cast<uint64_t>(c) * inner);
+}
+
+// Copy a contiguous slab into LDS through `f`, a few loads in flight per lane.
+constexpr int kSlabBatch = 4;
+template <class F>
+SHDW_DEVICE void stage_slab(float* lds, const float* xs, uint32_t slab, F f) {
+  for (uint32_t t0 = 0; t0 < slab; t0 += kSlabBatch * kBlock) {
+    float reg[kSlabBatch];
+#pragma unroll
+    for (int k = 0; k < kSlabBatch; ++k) {
+      const uint32_t t = t0 + k * kBlock + threadIdx.x;
+      if (t < slab) reg[k] = xs[t];
+    }
+#pragma unroll
+    for (int k = 0; k < kSlabBatch; ++k) {
+      const uint32_t t = t0 + k * kBlock + threadIdx.x;
+      if (t < slab) lds[t] = f(reg[k]);
+    }
+  }
+}
+
+// Any-order maximum over the workgroup.  Only valid where the order cannot
+// show: see softmax_slab_kernel.
+SHDW_DEVICE float block_max_any_order(float m, float* scratch4) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) m = std_max(__shfl_xor(m, off), m);
+  if ((threadIdx.x & 63) == 0) scratch4[threadIdx.x >> 6] = m;
+  __syncthreads();
+  m = scratch4[0];
+#pragma unroll
+  for (int w = 1; w < kBlock / kWave; ++w) m = std_max(scratch4[w], m);
+  return m;
+}
+
+// Front-to-back sum of lds[0..n) by the calling lane, 128-bit LDS reads.
+template <class ACC>
+SHDW_DEVICE ACC sequential_sum(const float* lds, uint32_t n) {
+  ACC sum = 0;
+  const v4f* l4 = reinterpret_cast<const v4f*>(lds);
+  const uint32_t q = n / 4;
+#pragma unroll 8
+  for (uint32_t c = 0; c < q; ++c) {
+    const v4f v = l4[c];
+    sum += static_cast<ACC>(v[0]);
+    sum += static_cast<ACC>(v[1]);
+    sum += static_cast<ACC>(v[2]);
+    sum += static_cast<ACC>(v[3]);
+  }
+  for (uint32_t c = 4 * q; c < n; ++c) sum += static_cast<ACC>(lds[c]);
+  return sum;
+}
+
+// inner == 1 takes the maximum with all lanes in any order.  That is exact:
+// the value of the maximum does not depend on the order unless the column
+// holds a NaN, and then every output is NaN whatever maximum was used (the
+// NaN's own term poisons the sum); the sign of a zero maximum cannot reach the
+// output because exp(+-0) = 1 and x - (+-0) = x for x != 0.
 __global__ __launch_bounds__(kBlock) void softmax_slab_kernel(const float* x, float* y,
                                                                uint32_t dim, FastDiv f_inner) {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   __shared__ uint64_t tab[32];
+  __shared__ float wave_max[kBlock / kWave];
   const uint32_t inner = f_inner.d;
   const uint32_t slab = dim * inner;
   float* stat = lds + slab;
   const float* xs = x + static_cast<uint64_t>(blockIdx.x) * slab;
   float* ys = y + static_cast<uint64_t>(blockIdx.x) * slab;
   if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
-  for (uint32_t t = threadIdx.x; t < slab; t += kBlock) lds[t] = xs[t];
+  stage_slab(lds, xs, slab, [](float v) { return v; });
   __syncthreads();
+  if (inner == 1) {
+    float m = -FLT_MAX;
+    for (uint32_t t = threadIdx.x; t < slab; t += kBlock) m = std_max(lds[t], m);
+    m = block_max_any_order(m, wave_max);
+    for (uint32_t t = threadIdx.x; t < slab; t += kBlock) lds[t] = libm::exact_expf(lds[t] - m, tab);
+    __syncthreads();
+    if (threadIdx.x == 0) stat[0] = sequential_sum<float>(lds, slab);
+    __syncthreads();
+    const float sum = stat[0];
+    for (uint32_t t = threadIdx.x; t < slab; t += kBlock) ys[t] = lds[t] / sum;
+    return;
+  }
   for (uint32_t s = threadIdx.x; s < inner; s += kBlock) {
     float max_val = -FLT_MAX;
     for (uint32_t c = 0; c < dim; ++c) max_val = std_max(lds[c * inner + s], max_val);
@@ -141,27 +248,61 @@ __global__ __launch_bounds__(kBlock) void normalize_columns_kernel(const float* 
     yc[static_cast<uint64_t>(c) * inner] = xc[static_cast<uint64_t>(c) * inner] / div;
 }
 
+template <int PMODE, int DMAX>
+__global__ __launch_bounds__(kBlock) void normalize_columns_reg_kernel(const float* x, float* y,
+                                                                        uint32_t columns,
+                                                                        uint32_t dim,
+                                                                        FastDiv f_inner, float p,
+                                                                        float eps) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= columns) return;
+  uint32_t n, s;
+  fd_divmod(i, f_inner, n, s);
+  const uint32_t inner = f_inner.d;
+  const uint64_t base = static_cast<uint64_t>(n) * dim * inner + s;
+  const float* xc = x + base;
+  float* yc = y + base;
+  float v[DMAX];
+#pragma unroll
+  for (int c = 0; c < DMAX; ++c)
+    if (c < dim) v[c] = __builtin_nontemporal_load(xc + static_cast<uint64_t>(c) * inner);
+  double acc = 0;
+#pragma unroll
+  for (int c = 0; c < DMAX; ++c)
+    if (c < dim) acc += norm_term<PMODE>(v[c], p);
+  const float div = norm_finish<PMODE>(acc, p, eps);
+#pragma unroll
+  for (int c = 0; c < DMAX; ++c)
+    if (c < dim) __builtin_nontemporal_store(v[c] / div, yc + static_cast<uint64_t>(c) * inner);
+}
+
+// The slab in LDS holds the per-element terms (|x|, |x|^2 or |x|^p, computed by
+// all lanes); x itself is read again for the division, from L2.
 template <int PMODE>
 __global__ __launch_bounds__(kBlock) void normalize_slab_kernel(const float* x, float* y,
                                                                  uint32_t dim, FastDiv f_inner,
                                                                  float p, float eps) {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   const uint32_t inner = f_inner.d;
   const uint32_t slab = dim * inner;
   float* stat = lds + slab;
   const float* xs = x + static_cast<uint64_t>(blockIdx.x) * slab;
   float* ys = y + static_cast<uint64_t>(blockIdx.x) * slab;
-  for (uint32_t t = threadIdx.x; t < slab; t += kBlock) lds[t] = xs[t];
+  stage_slab(lds, xs, slab, [p](float v) { return static_cast<float>(norm_term<PMODE>(v, p)); });
   __syncthreads();
-  for (uint32_t s = threadIdx.x; s < inner; s += kBlock) {
-    double acc = 0;
-    for (uint32_t c = 0; c < dim; ++c) acc += norm_term<PMODE>(lds[c * inner + s], p);
-    stat[s] = norm_finish<PMODE>(acc, p, eps);
+  if (inner == 1) {
+    if (threadIdx.x == 0) stat[0] = norm_finish<PMODE>(sequential_sum<double>(lds, slab), p, eps);
+  } else {
+    for (uint32_t s = threadIdx.x; s < inner; s += kBlock) {
+      double acc = 0;
+      for (uint32_t c = 0; c < dim; ++c) acc += static_cast<double>(lds[c * inner + s]);
+      stat[s] = norm_finish<PMODE>(acc, p, eps);
+    }
   }
   __syncthreads();
   for (uint32_t t = threadIdx.x; t < slab; t += kBlock) {
     const uint32_t s = t - fd_div(t, f_inner) * inner;
-    ys[t] = lds[t] / stat[s];
+    ys[t] = xs[t] / stat[s];
   }
 }
 
@@ -201,6 +342,15 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
   const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
   if (g.use_slab)
     softmax_slab_kernel<<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, static_cast<uint32_t>(dim), fi);
+  else if (dim <= 16)
+    softmax_columns_reg_kernel<16><<<grid_for(g.columns), kBlock, 0, st>>>(
+        x, y, g.columns, static_cast<uint32_t>(dim), fi);
+  else if (dim <= 32)
+    softmax_columns_reg_kernel<32><<<grid_for(g.columns), kBlock, 0, st>>>(
+        x, y, g.columns, static_cast<uint32_t>(dim), fi);
+  else if (dim <= 64)
+    softmax_columns_reg_kernel<64><<<grid_for(g.columns), kBlock, 0, st>>>(
+        x, y, g.columns, static_cast<uint32_t>(dim), fi);
   else
     softmax_columns_kernel<<<grid_for(g.columns), kBlock, 0, st>>>(x, y, g.columns,
                                                                   static_cast<uint32_t>(dim), fi);
@@ -225,6 +375,21 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
       normalize_slab_kernel<2><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
     else
       normalize_slab_kernel<0><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
+  } else if (dim <= 64 && mode != 0) {
+    // p = 1 and p = 2 keep short columns in registers (one read, one write);
+    // the generic-p form would unroll a powf per element and stays two-pass.
+    const uint32_t grid = grid_for(g.columns);
+    if (mode == 1) {
+      if (dim <= 16)
+        normalize_columns_reg_kernel<1, 16><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
+      else
+        normalize_columns_reg_kernel<1, 64><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
+    } else {
+      if (dim <= 16)
+        normalize_columns_reg_kernel<2, 16><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
+      else
+        normalize_columns_reg_kernel<2, 64><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
+    }
   } else {
     const uint32_t grid = grid_for(g.columns);
     if (mode == 1)

@@ -171,6 +171,8 @@ constexpr int kPlaneTileFloats = 12608;  // 256 rows x 49 or 64 rows x 197
 
 inline int plane_pitch_cap(int rows_per_group) { return kPlaneTileFloats / rows_per_group; }
 
+constexpr int kPlaneBatch = 8;  // global loads a lane keeps in flight while staging
+
 template <bool MAX, int ROWS>
 __global__ __launch_bounds__(kBlock) void pool_plane_kernel(const float* x, float* y, uint32_t rows,
                                                              uint32_t len, uint32_t chunk,
@@ -187,10 +189,56 @@ __global__ __launch_bounds__(kBlock) void pool_plane_kernel(const float* x, floa
     const uint32_t cols = last ? len - c0 : chunk;
     const FastDiv fc = last ? f_last : f_chunk;
     const uint32_t cells = nrows * cols;
-    for (uint32_t t = threadIdx.x; t < cells; t += kBlock) {
-      uint32_t r, c;
-      fd_divmod(t, fc, r, c);
-      tile[r * pitch + c] = __builtin_nontemporal_load(base + static_cast<uint64_t>(r) * len + c0 + c);
+    if (cols == len && aligned16_device(base)) {
+      // The rows are one contiguous span: 128-bit loads, a batch in flight per
+      // lane, then scattered into the padded LDS rows.
+      const uint32_t nvec = cells / 4;
+      for (uint32_t v0 = 0; v0 < nvec; v0 += kPlaneBatch * kBlock) {
+        v4f reg[kPlaneBatch];
+#pragma unroll
+        for (int k = 0; k < kPlaneBatch; ++k) {
+          const uint32_t v = v0 + k * kBlock + threadIdx.x;
+          if (v < nvec) reg[k] = load4_stream(base + 4ull * v);
+        }
+#pragma unroll
+        for (int k = 0; k < kPlaneBatch; ++k) {
+          const uint32_t v = v0 + k * kBlock + threadIdx.x;
+          if (v < nvec) {
+            uint32_t r, c;
+            fd_divmod(4 * v, fc, r, c);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              tile[r * pitch + c] = reg[k][j];
+              if (++c == cols) c = 0, ++r;
+            }
+          }
+        }
+      }
+      for (uint32_t t = 4 * nvec + threadIdx.x; t < cells; t += kBlock) {
+        uint32_t r, c;
+        fd_divmod(t, fc, r, c);
+        tile[r * pitch + c] = base[t];
+      }
+    } else {
+      for (uint32_t t0 = 0; t0 < cells; t0 += kPlaneBatch * kBlock) {
+        float reg[kPlaneBatch];
+        uint32_t slot[kPlaneBatch];
+#pragma unroll
+        for (int k = 0; k < kPlaneBatch; ++k) {
+          const uint32_t t = t0 + k * kBlock + threadIdx.x;
+          if (t < cells) {
+            uint32_t r, c;
+            fd_divmod(t, fc, r, c);
+            slot[k] = r * pitch + c;
+            reg[k] = __builtin_nontemporal_load(base + static_cast<uint64_t>(r) * len + c0 + c);
+          }
+        }
+#pragma unroll
+        for (int k = 0; k < kPlaneBatch; ++k) {
+          const uint32_t t = t0 + k * kBlock + threadIdx.x;
+          if (t < cells) tile[slot[k]] = reg[k];
+        }
+      }
     }
     __syncthreads();
     if (threadIdx.x < nrows) {
