@@ -163,6 +163,136 @@ __global__ __launch_bounds__(kBlock) void pool_window_kernel(const float* x, flo
   y[i] = MAX ? max_val : sum_val / static_cast<float>(pool_size);
 }
 
+// 2-D windows through LDS.  A workgroup owns `band` consecutive output rows of
+// one plane.  The input rows they touch are one contiguous span of the plane,
+// copied with 128-bit loads; every input element is then fetched from HBM/L2
+// once per band instead of once per overlapping window, and the window walks
+// read LDS.  Order inside a window is unchanged.
+constexpr int kBandTileFloats = 8192;  // upper bound of the dynamic LDS tile (32 KB)
+constexpr int kBandBatch = 4;
+constexpr int kPoolBandOutputs = 512;  // outputs a workgroup aims for (measured best of 256..4096)
+
+struct BandArgs {
+  int in_h, in_w, out_h, out_w;
+  int kh, kw, sh, sw, ph, pw;
+  int band, bands_per_plane;
+  FastDiv f_out_w, f_bands;
+};
+
+// K > 0: square K x K window, walked fully unrolled with the out-of-range
+// cells predicated off (same cells, same order as the clipped loops) so that
+// all LDS reads of a window are in flight together.  K = 0: any window.
+template <bool MAX, int K>
+__global__ __launch_bounds__(kBlock) void pool_band_kernel(const float* x, float* y, BandArgs p) {
+  extern __shared__ __align__(16) float tile[];  // rows of one band, at most kBandTileFloats
+  uint32_t plane, b;
+  fd_divmod(blockIdx.x, p.f_bands, plane, b);
+  const int h0 = static_cast<int>(b) * p.band;
+  const int nh = min(p.band, p.out_h - h0);
+  const int r_lo = max(h0 * p.sh - p.ph, 0);
+  const int r_hi = min((h0 + nh - 1) * p.sh - p.ph + p.kh, p.in_h);
+  const uint32_t span = r_hi > r_lo ? static_cast<uint32_t>(r_hi - r_lo) * p.in_w : 0u;
+  const float* src = x + static_cast<uint64_t>(plane) * p.in_h * p.in_w + static_cast<uint64_t>(r_lo) * p.in_w;
+  if (aligned16_device(src)) {
+    const uint32_t nvec = span / 4;
+    for (uint32_t v0 = 0; v0 < nvec; v0 += kBandBatch * kBlock) {
+      v4f reg[kBandBatch];
+#pragma unroll
+      for (int k = 0; k < kBandBatch; ++k) {
+        const uint32_t v = v0 + k * kBlock + threadIdx.x;
+        if (v < nvec) reg[k] = load4_stream(src + 4ull * v);
+      }
+#pragma unroll
+      for (int k = 0; k < kBandBatch; ++k) {
+        const uint32_t v = v0 + k * kBlock + threadIdx.x;
+        if (v < nvec) *reinterpret_cast<v4f*>(tile + 4 * v) = reg[k];
+      }
+    }
+    for (uint32_t t = 4 * nvec + threadIdx.x; t < span; t += kBlock) tile[t] = src[t];
+  } else {
+    for (uint32_t t0 = 0; t0 < span; t0 += kBandBatch * kBlock) {
+      float reg[kBandBatch];
+#pragma unroll
+      for (int k = 0; k < kBandBatch; ++k) {
+        const uint32_t t = t0 + k * kBlock + threadIdx.x;
+        if (t < span) reg[k] = __builtin_nontemporal_load(src + t);
+      }
+#pragma unroll
+      for (int k = 0; k < kBandBatch; ++k) {
+        const uint32_t t = t0 + k * kBlock + threadIdx.x;
+        if (t < span) tile[t] = reg[k];
+      }
+    }
+  }
+  __syncthreads();
+  float* dst = y + (static_cast<uint64_t>(plane) * p.out_h + h0) * p.out_w;
+  const uint32_t outs = static_cast<uint32_t>(nh) * p.out_w;
+  for (uint32_t o = threadIdx.x; o < outs; o += kBlock) {
+    uint32_t hl, w;
+    fd_divmod(o, p.f_out_w, hl, w);
+    int hstart = (h0 + static_cast<int>(hl)) * p.sh - p.ph;
+    int wstart = static_cast<int>(w) * p.sw - p.pw;
+    int hend = min(hstart + p.kh, p.in_h + p.ph);
+    int wend = min(wstart + p.kw, p.in_w + p.pw);
+    const int pool_size = (hend - hstart) * (wend - wstart);
+    hstart = max(hstart, 0), wstart = max(wstart, 0);
+    hend = min(hend, p.in_h), wend = min(wend, p.in_w);
+    float max_val = -FLT_MAX, sum_val = 0.f;
+    if (K > 0) {
+      const int h_first = (h0 + static_cast<int>(hl)) * p.sh - p.ph;
+      const int w_first = static_cast<int>(w) * p.sw - p.pw;
+      float cell[K > 0 ? K * K : 1];
+#pragma unroll
+      for (int i = 0; i < K; ++i) {
+#pragma unroll
+        for (int j = 0; j < K; ++j) {
+          const int ph = h_first + i, pw = w_first + j;
+          const bool inside = ph >= hstart && ph < hend && pw >= wstart && pw < wend;
+          cell[i * K + j] = inside ? tile[(ph - r_lo) * p.in_w + pw] : 0.f;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < K; ++i) {
+#pragma unroll
+        for (int j = 0; j < K; ++j) {
+          const int ph = h_first + i, pw = w_first + j;
+          const bool inside = ph >= hstart && ph < hend && pw >= wstart && pw < wend;
+          if (inside) {
+            if (MAX)
+              max_val = pool_max(max_val, cell[i * K + j]);
+            else
+              sum_val += cell[i * K + j];
+          }
+        }
+      }
+    } else {
+      for (int ph = hstart; ph < hend; ++ph) {
+        const float* row = tile + (ph - r_lo) * p.in_w;
+        for (int pw = wstart; pw < wend; ++pw) {
+          const float v = row[pw];
+          if (MAX)
+            max_val = pool_max(max_val, v);
+          else
+            sum_val += v;
+        }
+      }
+    }
+    dst[o] = MAX ? max_val : sum_val / static_cast<float>(pool_size);
+  }
+}
+
+// Output rows per workgroup, or 0 when a single output row's input rows do not
+// fit the tile (the direct kernel handles that).
+static int plan_pool_band(const PoolArgs& p, int target_outputs) {
+  const int rows_cap = kBandTileFloats / p.in_w;
+  if (rows_cap < p.kh) return 0;
+  const int band_cap = (rows_cap - p.kh) / p.sh + 1;
+  int band = (target_outputs + p.out_w - 1) / p.out_w;
+  band = band < 1 ? 1 : band;
+  band = band > band_cap ? band_cap : band;
+  return band > p.out_h ? p.out_h : band;
+}
+
 // Whole-plane windows: x is [rows][len], one output per row.  A workgroup owns
 // ROWS consecutive rows; they pass through LDS in chunks of `chunk` columns
 // (coalesced loads by all lanes), then lane r folds row r element by element.
@@ -326,6 +456,39 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
   p.f_out_h = make_fastdiv(static_cast<uint32_t>(p.out_h));
   p.f_out_d = make_fastdiv(static_cast<uint32_t>(p.out_d));
   const uint32_t n_out = static_cast<uint32_t>(out_count);
+  const int band = three_d ? 0 : plan_pool_band(p, kPoolBandOutputs);
+  if (band > 0) {
+    BandArgs a;
+    a.in_h = p.in_h, a.in_w = p.in_w, a.out_h = p.out_h, a.out_w = p.out_w;
+    a.kh = p.kh, a.kw = p.kw, a.sh = p.sh, a.sw = p.sw, a.ph = p.ph, a.pw = p.pw;
+    a.band = band;
+    a.bands_per_plane = (p.out_h + band - 1) / band;
+    a.f_out_w = p.f_out_w;
+    a.f_bands = make_fastdiv(static_cast<uint32_t>(a.bands_per_plane));
+    const int64_t groups = static_cast<int64_t>(in_shape[0]) * in_shape[1] * a.bands_per_plane;
+    const int tile_rows = min((band - 1) * p.sh + p.kh, p.in_h);
+    const size_t lds = static_cast<size_t>(tile_rows) * p.in_w * sizeof(float);
+    if (groups <= INT32_MAX) {
+      const uint32_t g = static_cast<uint32_t>(groups);
+      const int k = p.kh == p.kw && (p.kh == 2 || p.kh == 3) ? p.kh : 0;
+      if (pool_type == 0) {
+        if (k == 3)
+          pool_band_kernel<true, 3><<<g, kBlock, lds, st>>>(x, y, a);
+        else if (k == 2)
+          pool_band_kernel<true, 2><<<g, kBlock, lds, st>>>(x, y, a);
+        else
+          pool_band_kernel<true, 0><<<g, kBlock, lds, st>>>(x, y, a);
+      } else {
+        if (k == 3)
+          pool_band_kernel<false, 3><<<g, kBlock, lds, st>>>(x, y, a);
+        else if (k == 2)
+          pool_band_kernel<false, 2><<<g, kBlock, lds, st>>>(x, y, a);
+        else
+          pool_band_kernel<false, 0><<<g, kBlock, lds, st>>>(x, y, a);
+      }
+      return launch_status();
+    }
+  }
   const uint32_t grid = grid_for(n_out);
   if (three_d) {
     if (pool_type == 0)

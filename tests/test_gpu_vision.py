@@ -159,6 +159,13 @@ POOL_2D = [
     ((2, 4, 7, 7), [7], [1], [0], True), ((1, 1, 5, 5), [5], [3], [2], True),
     ((3, 2, 8, 8), [2], [2], [0], False), ((1, 2, 6, 6), [3], [3], [2], True),
     ((2, 16, 56, 56), [3], [2], [0], True), ((1, 5, 33, 17), [5, 3], [1, 2], [2, 1], False),
+    # several row bands per plane, padded and unpadded; kernels with and without an unrolled form
+    ((1, 3, 112, 112), [3], [2], [0], True), ((1, 3, 112, 112), [3], [2], [1], True),
+    ((2, 2, 90, 70), [2], [2], [0], True), ((1, 2, 64, 64), [3], [1], [1], False),
+    ((1, 2, 75, 61), [4, 3], [3, 2], [1, 1], True), ((1, 1, 150, 50), [2], [1], [0], False),
+    # rows too wide for more than two output rows per band, then too wide for any band
+    ((1, 1, 9, 2000), [3], [1], [1], True), ((1, 1, 7, 3000), [3], [2], [0], True),
+    ((1, 2, 40, 40), [13], [5], [6], True),
 ]
 
 
