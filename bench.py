@@ -293,23 +293,14 @@ def config_table(dev):
         n5, C5, in5, A[k].ptr, g5.ptr, b5.ptr, A[(k + 1) % SETS].ptr, Y[k].ptr, M[k].ptr, st), SETS)
     add(5, "fused_tail", 12 * n5 + 8 * C5 + 4 * 65536, ms, n5)
 
-    # Operators next to the path (label "next"), on ResNet-sized tensors of the
-    # same 51 MB: BatchNorm / Axpy on [64,1024,14,14], the stem max pooling on
-    # [16,64,112,112], global average pooling on [128,2048,7,7], Softmax and
-    # Normalize over channels of a dense map, and the classifier Softmax.
-    mean5, var5 = dev.buf(normal(601, C5)), dev.buf(uniform(602, C5, 0.5, 2.0))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_batch_norm(n5, C5, in5, A[k].ptr, mean5.ptr, var5.ptr,
-                                                           1.0, 1e-5, Y[k].ptr, st), SETS)
-    add("next", "batch_norm", 8 * n5 + 8 * C5, ms, n5)
-    al5 = dev.buf(uniform(603, 65536, 0.0, 1.0))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_axpy_rows(65536, in5, al5.ptr, A[k].ptr,
-                                                          A[(k + 1) % SETS].ptr, Y[k].ptr, st), SETS)
-    add("next", "axpy_rows", 12 * n5 + 4 * 65536, ms, n5)
+    # Operators next to the path (label "next").  Global pooling, Softmax and
+    # Normalize run on the 51 MB sets; BatchNorm, Axpy and the stem max pooling
+    # run further down on 205 MB tensors like the headline step.
     pin, pout = [16, 64, 112, 112], [16, 64, 56, 56]
     npo = int(np.prod(pout))
     ms = time_batch(dev, lambda k: lib.shdw_hip_pooling2d(I(pin), 0, 3, 3, 2, 2, 0, 0, I(pout), A[k].ptr,
                                                           Y[k].ptr, st), SETS)
-    add("next", "pooling_max_3x3s2", 4 * (NBIG + npo), ms, NBIG)
+    add("next", "pooling_max_3x3s2 [16,64,112,112]", 4 * (NBIG + npo), ms, NBIG)
     gin, gout = [128, 2048, 7, 7], [128, 2048, 1, 1]
     ms = time_batch(dev, lambda k: lib.shdw_hip_pooling2d(I(gin), 1, 7, 7, 1, 1, 0, 0, I(gout), A[k].ptr,
                                                           Y[k].ptr, st), SETS)
@@ -329,6 +320,36 @@ def config_table(dev):
     ms = time_batch(dev, lambda k: lib.shdw_hip_normalize(64, 512, 1, 2.0, 1e-12, A[k].ptr, Y[k].ptr, st), SETS)
     add("next", "normalize_l2_embedding_64x512", 8 * 64 * 512, ms, 64 * 512)
     for bset in (A, Y):
+        for bb in bset:
+            bb.free()
+
+    # "next" operators at the size of the headline tensor (205 MB in, 3 rotating sets)
+    NH, SH = 51380224, 3
+    AH = [dev.buf(normal(701 + k, NH)) for k in range(SH)]
+    YH = [dev.buf(nbytes=4 * NH) for _ in range(SH)]
+    CH, INH = 256, 3136
+    meanh, varh = dev.buf(normal(611, CH)), dev.buf(uniform(612, CH, 0.5, 2.0))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_batch_norm(NH, CH, INH, AH[k].ptr, meanh.ptr, varh.ptr,
+                                                           1.0, 1e-5, YH[k].ptr, st), SH, reps=20)
+    add("next", "batch_norm [64,256,56,56]", 8 * NH + 8 * CH, ms, NH)
+    alh = dev.buf(uniform(613, 64 * CH, 0.0, 1.0))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_axpy_rows(64 * CH, INH, alh.ptr, AH[k].ptr,
+                                                          AH[(k + 1) % SH].ptr, YH[k].ptr, st), SH, reps=20)
+    add("next", "axpy_rows [64,256,56,56]", 12 * NH + 4 * 64 * CH, ms, NH)
+    pinh, pouth = [64, 64, 112, 112], [64, 64, 56, 56]
+    ms = time_batch(dev, lambda k: lib.shdw_hip_pooling2d(I(pinh), 0, 3, 3, 2, 2, 0, 0, I(pouth), AH[k].ptr,
+                                                          YH[k].ptr, st), SH, reps=20)
+    add("next", "pooling_max_3x3s2 [64,64,112,112]", 4 * (NH + NH // 4), ms, NH)
+    ginh, gouth = [512, 2048, 7, 7], [512, 2048, 1, 1]
+    ms = time_batch(dev, lambda k: lib.shdw_hip_pooling2d(I(ginh), 1, 7, 7, 1, 1, 0, 0, I(gouth), AH[k].ptr,
+                                                          YH[k].ptr, st), SH, reps=20)
+    add("next", "pooling_global_avg_7x7 [512,2048,7,7]", 4 * (NH + 512 * 2048), ms, NH)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_softmax(64, 49, 16384, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
+    add("next", "softmax_channels_dense [64,49,128,128]", 8 * NH, ms, NH)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_normalize(64, 49, 16384, 2.0, 1e-12, AH[k].ptr, YH[k].ptr, st),
+                    SH, reps=20)
+    add("next", "normalize_l2_channels_dense [64,49,128,128]", 8 * NH, ms, NH)
+    for bset in (AH, YH):
         for bb in bset:
             bb.free()
 

@@ -168,149 +168,241 @@ __global__ __launch_bounds__(kBlock) void pool_window_kernel(const float* x, flo
 // copied with 128-bit loads; every input element is then fetched from HBM/L2
 // once per band instead of once per overlapping window, and the window walks
 // read LDS.  Order inside a window is unchanged.
+//
+// LDS layout: rows of pitch = pad_l + in_w + pad_r, plus one spare row.  The pad
+// cells and the spare row hold the fold's neutral value (lowest() for max, +0
+// for the sum: the running sum starts at +0 and can never become -0, so adding
+// +0 leaves it unchanged bit for bit).  A window cell left or right of the
+// input reads a pad cell, a cell above or below reads the spare row, and the
+// unrolled K x K walk needs no predicates at all.
 constexpr int kBandTileFloats = 8192;  // upper bound of the dynamic LDS tile (32 KB)
 constexpr int kBandBatch = 4;
+constexpr int kBandMaxPad = 64;        // wider clipping goes to the direct kernel
 constexpr int kPoolBandOutputs = 512;  // outputs a workgroup aims for (measured best of 256..4096)
 
 struct BandArgs {
   int in_h, in_w, out_h, out_w;
   int kh, kw, sh, sw, ph, pw;
-  int band, bands_per_plane;
-  FastDiv f_out_w, f_bands;
+  int band, bands_per_plane, w_shift;
+  int pad_l, pitch, tile_rows;  // data rows in the tile; the spare row is row tile_rows
+  uint32_t total_bands, bands_per_group;
+  FastDiv f_bands, f_in_w;
 };
 
-// K > 0: square K x K window, walked fully unrolled with the out-of-range
-// cells predicated off (same cells, same order as the clipped loops) so that
-// all LDS reads of a window are in flight together.  K = 0: any window.
+// Where band g of the launch lies: plane, first output row, row count, and the
+// contiguous span of input rows it reads.
+struct BandSpan {
+  uint32_t plane;
+  int h0, nh, r_lo, r_hi;
+  uint32_t span;
+  const float* src;
+};
+
+SHDW_DEVICE BandSpan band_span(const BandArgs& p, const float* x, uint32_t g) {
+  BandSpan s;
+  uint32_t b;
+  fd_divmod(g, p.f_bands, s.plane, b);
+  s.h0 = static_cast<int>(b) * p.band;
+  s.nh = min(p.band, p.out_h - s.h0);
+  s.r_lo = max(s.h0 * p.sh - p.ph, 0);
+  s.r_hi = max(min((s.h0 + s.nh - 1) * p.sh - p.ph + p.kh, p.in_h), s.r_lo);
+  s.span = static_cast<uint32_t>(s.r_hi - s.r_lo) * p.in_w;
+  s.src = x + static_cast<uint64_t>(s.plane) * p.in_h * p.in_w + static_cast<uint64_t>(s.r_lo) * p.in_w;
+  return s;
+}
+
+// LDS offset of element t of a band's span.
+SHDW_DEVICE uint32_t band_slot(const BandArgs& p, uint32_t t) {
+  uint32_t r, c;
+  fd_divmod(t, p.f_in_w, r, c);
+  return r * p.pitch + p.pad_l + c;
+}
+
+// K > 0: square K x K window, fully unrolled, all LDS reads in flight together.
+// K = 0: any window, clipped loops.
 template <bool MAX, int K>
-__global__ __launch_bounds__(kBlock) void pool_band_kernel(const float* x, float* y, BandArgs p) {
-  extern __shared__ __align__(16) float tile[];  // rows of one band, at most kBandTileFloats
-  uint32_t plane, b;
-  fd_divmod(blockIdx.x, p.f_bands, plane, b);
-  const int h0 = static_cast<int>(b) * p.band;
-  const int nh = min(p.band, p.out_h - h0);
-  const int r_lo = max(h0 * p.sh - p.ph, 0);
-  const int r_hi = min((h0 + nh - 1) * p.sh - p.ph + p.kh, p.in_h);
-  const uint32_t span = r_hi > r_lo ? static_cast<uint32_t>(r_hi - r_lo) * p.in_w : 0u;
-  const float* src = x + static_cast<uint64_t>(plane) * p.in_h * p.in_w + static_cast<uint64_t>(r_lo) * p.in_w;
-  if (aligned16_device(src)) {
-    const uint32_t nvec = span / 4;
-    for (uint32_t v0 = 0; v0 < nvec; v0 += kBandBatch * kBlock) {
-      v4f reg[kBandBatch];
+SHDW_DEVICE void band_windows(const float* tile, float* y, const BandArgs& p, const BandSpan& bs) {
+  // Lane -> (output row, output column) by shift and mask: w_lanes is a power
+  // of two >= min(out_w, 256).  A lane keeps its column(s), so everything that
+  // depends on the column only is computed once per lane, not once per output.
+  float* dst = y + (static_cast<uint64_t>(bs.plane) * p.out_h + bs.h0) * p.out_w;
+  const int w_lanes = 1 << p.w_shift;
+  const int h_step = kBlock >> p.w_shift;
+  const int h_lane = static_cast<int>(threadIdx.x) >> p.w_shift;
+  const int spare = p.tile_rows * p.pitch;
+  for (int w = static_cast<int>(threadIdx.x) & (w_lanes - 1); w < p.out_w; w += w_lanes) {
+    const int w_first = w * p.sw - p.pw;
+    const int w_end_pad = min(w_first + p.kw, p.in_w + p.pw);
+    const int wstart = max(w_first, 0), wend = min(w_end_pad, p.in_w);
+    for (int hl = h_lane; hl < bs.nh; hl += h_step) {
+      const int h_first = (bs.h0 + hl) * p.sh - p.ph;
+      const int h_end_pad = min(h_first + p.kh, p.in_h + p.ph);
+      float max_val = -FLT_MAX, sum_val = 0.f;
+      if (K > 0) {
+        float cell[K > 0 ? K * K : 1];
 #pragma unroll
-      for (int k = 0; k < kBandBatch; ++k) {
-        const uint32_t v = v0 + k * kBlock + threadIdx.x;
-        if (v < nvec) reg[k] = load4_stream(src + 4ull * v);
-      }
+        for (int i = 0; i < K; ++i) {
+          const int ri = h_first + i;
+          const int row = ri >= bs.r_lo && ri < bs.r_hi ? (ri - bs.r_lo) * p.pitch : spare;
+          const float* cells = tile + row + p.pad_l + w_first;
 #pragma unroll
-      for (int k = 0; k < kBandBatch; ++k) {
-        const uint32_t v = v0 + k * kBlock + threadIdx.x;
-        if (v < nvec) *reinterpret_cast<v4f*>(tile + 4 * v) = reg[k];
-      }
-    }
-    for (uint32_t t = 4 * nvec + threadIdx.x; t < span; t += kBlock) tile[t] = src[t];
-  } else {
-    for (uint32_t t0 = 0; t0 < span; t0 += kBandBatch * kBlock) {
-      float reg[kBandBatch];
-#pragma unroll
-      for (int k = 0; k < kBandBatch; ++k) {
-        const uint32_t t = t0 + k * kBlock + threadIdx.x;
-        if (t < span) reg[k] = __builtin_nontemporal_load(src + t);
-      }
-#pragma unroll
-      for (int k = 0; k < kBandBatch; ++k) {
-        const uint32_t t = t0 + k * kBlock + threadIdx.x;
-        if (t < span) tile[t] = reg[k];
-      }
-    }
-  }
-  __syncthreads();
-  float* dst = y + (static_cast<uint64_t>(plane) * p.out_h + h0) * p.out_w;
-  const uint32_t outs = static_cast<uint32_t>(nh) * p.out_w;
-  for (uint32_t o = threadIdx.x; o < outs; o += kBlock) {
-    uint32_t hl, w;
-    fd_divmod(o, p.f_out_w, hl, w);
-    int hstart = (h0 + static_cast<int>(hl)) * p.sh - p.ph;
-    int wstart = static_cast<int>(w) * p.sw - p.pw;
-    int hend = min(hstart + p.kh, p.in_h + p.ph);
-    int wend = min(wstart + p.kw, p.in_w + p.pw);
-    const int pool_size = (hend - hstart) * (wend - wstart);
-    hstart = max(hstart, 0), wstart = max(wstart, 0);
-    hend = min(hend, p.in_h), wend = min(wend, p.in_w);
-    float max_val = -FLT_MAX, sum_val = 0.f;
-    if (K > 0) {
-      const int h_first = (h0 + static_cast<int>(hl)) * p.sh - p.ph;
-      const int w_first = static_cast<int>(w) * p.sw - p.pw;
-      float cell[K > 0 ? K * K : 1];
-#pragma unroll
-      for (int i = 0; i < K; ++i) {
-#pragma unroll
-        for (int j = 0; j < K; ++j) {
-          const int ph = h_first + i, pw = w_first + j;
-          const bool inside = ph >= hstart && ph < hend && pw >= wstart && pw < wend;
-          cell[i * K + j] = inside ? tile[(ph - r_lo) * p.in_w + pw] : 0.f;
+          for (int j = 0; j < K; ++j) cell[i * K + j] = cells[j];
         }
-      }
 #pragma unroll
-      for (int i = 0; i < K; ++i) {
-#pragma unroll
-        for (int j = 0; j < K; ++j) {
-          const int ph = h_first + i, pw = w_first + j;
-          const bool inside = ph >= hstart && ph < hend && pw >= wstart && pw < wend;
-          if (inside) {
+        for (int c = 0; c < K * K; ++c) {
+          if (MAX)
+            max_val = pool_max(max_val, cell[c]);
+          else
+            sum_val += cell[c];
+        }
+      } else {
+        const int hstart = max(h_first, 0), hend = min(h_end_pad, p.in_h);
+        for (int ph = hstart; ph < hend; ++ph) {
+          const float* row = tile + (ph - bs.r_lo) * p.pitch + p.pad_l;
+          for (int pw = wstart; pw < wend; ++pw) {
+            const float v = row[pw];
             if (MAX)
-              max_val = pool_max(max_val, cell[i * K + j]);
+              max_val = pool_max(max_val, v);
             else
-              sum_val += cell[i * K + j];
+              sum_val += v;
           }
         }
       }
-    } else {
-      for (int ph = hstart; ph < hend; ++ph) {
-        const float* row = tile + (ph - r_lo) * p.in_w;
-        for (int pw = wstart; pw < wend; ++pw) {
-          const float v = row[pw];
-          if (MAX)
-            max_val = pool_max(max_val, v);
-          else
-            sum_val += v;
-        }
-      }
+      const int pool_size = (h_end_pad - h_first) * (w_end_pad - w_first);
+      dst[hl * p.out_w + w] = MAX ? max_val : sum_val / static_cast<float>(pool_size);
     }
-    dst[o] = MAX ? max_val : sum_val / static_cast<float>(pool_size);
   }
 }
 
-// Output rows per workgroup, or 0 when a single output row's input rows do not
-// fit the tile (the direct kernel handles that).
-static int plan_pool_band(const PoolArgs& p, int target_outputs) {
-  const int rows_cap = kBandTileFloats / p.in_w;
-  if (rows_cap < p.kh) return 0;
+// A workgroup walks `bands_per_group` consecutive bands.  PIPE (every span
+// starts 16-byte aligned and in_w % 4 == 0): the next band's 128-bit loads are
+// issued into registers before the current band's windows are walked, so HBM
+// requests stay in flight during the LDS phase.  Otherwise each band is staged
+// on its own with scalar loads.
+constexpr int kBandMaxRegs = kBandTileFloats / 4 / kBlock;  // vectors per lane for a full tile
+static_assert(kBandMaxRegs == 8, "the launch switch covers up to 8 staged vectors per lane");
+constexpr uint32_t kBandGroupsWanted = 4096;
+constexpr uint32_t kBandMaxWalk = 16;
+
+// REGS: 128-bit vectors a lane stages per band (PIPE only; 0 otherwise).
+template <bool MAX, int K, int REGS>
+__global__ __launch_bounds__(kBlock) void pool_band_kernel(const float* x, float* y, BandArgs p) {
+  constexpr bool PIPE = REGS > 0;
+  constexpr int kBandRegs = PIPE ? REGS : 1;
+  extern __shared__ __align__(16) float tile[];  // (tile_rows + 1) x pitch
+  const uint32_t g0 = blockIdx.x * p.bands_per_group;
+  const uint32_t g1 = min(g0 + p.bands_per_group, p.total_bands);
+  {
+    const float neutral = MAX ? -FLT_MAX : 0.f;
+    const uint32_t cells = static_cast<uint32_t>(p.tile_rows + 1) * p.pitch;  // multiple of 4
+    for (uint32_t t = 4 * threadIdx.x; t < cells; t += 4 * kBlock)
+      *reinterpret_cast<v4f*>(tile + t) = v4f{neutral, neutral, neutral, neutral};
+  }
+  __syncthreads();
+  if (PIPE) {
+    v4f reg[kBandRegs];
+    BandSpan cur = band_span(p, x, g0);
+#pragma unroll
+    for (int k = 0; k < kBandRegs; ++k) {
+      const uint32_t v = k * kBlock + threadIdx.x;
+      if (4 * v < cur.span) reg[k] = load4_stream(cur.src + 4ull * v);
+    }
+    for (uint32_t g = g0; g < g1; ++g) {
+#pragma unroll
+      for (int k = 0; k < kBandRegs; ++k) {
+        const uint32_t v = k * kBlock + threadIdx.x;
+        if (4 * v < cur.span) *reinterpret_cast<v4f*>(tile + band_slot(p, 4 * v)) = reg[k];
+      }
+      __syncthreads();
+      const BandSpan walk = cur;
+      if (g + 1 < g1) {
+        cur = band_span(p, x, g + 1);
+#pragma unroll
+        for (int k = 0; k < kBandRegs; ++k) {
+          const uint32_t v = k * kBlock + threadIdx.x;
+          if (4 * v < cur.span) reg[k] = load4_stream(cur.src + 4ull * v);
+        }
+      }
+      band_windows<MAX, K>(tile, y, p, walk);
+      __syncthreads();  // the tile is rewritten next
+    }
+  } else {
+    for (uint32_t g = g0; g < g1; ++g) {
+      const BandSpan bs = band_span(p, x, g);
+      for (uint32_t t0 = 0; t0 < bs.span; t0 += kBandBatch * kBlock) {
+        float reg[kBandBatch];
+#pragma unroll
+        for (int k = 0; k < kBandBatch; ++k) {
+          const uint32_t t = t0 + k * kBlock + threadIdx.x;
+          if (t < bs.span) reg[k] = __builtin_nontemporal_load(bs.src + t);
+        }
+#pragma unroll
+        for (int k = 0; k < kBandBatch; ++k) {
+          const uint32_t t = t0 + k * kBlock + threadIdx.x;
+          if (t < bs.span) tile[band_slot(p, t)] = reg[k];
+        }
+      }
+      __syncthreads();
+      band_windows<MAX, K>(tile, y, p, bs);
+      __syncthreads();
+    }
+  }
+}
+
+// Fills the band geometry; returns false when the direct kernel must be used
+// (rows too wide for the tile, or windows that overhang the input by more than
+// kBandMaxPad columns, which only an inconsistent out_shape can ask for).
+static bool plan_pool_band(const PoolArgs& p, int target_outputs, BandArgs* a) {
+  const int over_r = (p.out_w - 1) * p.sw - p.pw + p.kw - p.in_w;
+  const int pad_l = (p.pw + 3) & ~3, pad_r = over_r > 0 ? (over_r + 3) & ~3 : 0;
+  if (pad_l > kBandMaxPad || pad_r > kBandMaxPad) return false;
+  const int pitch = pad_l + ((p.in_w + 3) & ~3) + pad_r;
+  const int rows_cap = kBandTileFloats / pitch - 1;  // one row is the spare
+  if (rows_cap < p.kh) return false;
   const int band_cap = (rows_cap - p.kh) / p.sh + 1;
   int band = (target_outputs + p.out_w - 1) / p.out_w;
   band = band < 1 ? 1 : band;
   band = band > band_cap ? band_cap : band;
-  return band > p.out_h ? p.out_h : band;
+  band = band > p.out_h ? p.out_h : band;
+  int w_shift = 0;
+  while ((1 << w_shift) < p.out_w && w_shift < 8) ++w_shift;
+  const int h_step = kBlock >> w_shift;  // output rows a workgroup walks at a time
+  if (band > h_step && band < p.out_h) band -= band % h_step;
+  a->in_h = p.in_h, a->in_w = p.in_w, a->out_h = p.out_h, a->out_w = p.out_w;
+  a->kh = p.kh, a->kw = p.kw, a->sh = p.sh, a->sw = p.sw, a->ph = p.ph, a->pw = p.pw;
+  a->band = band;
+  a->bands_per_plane = (p.out_h + band - 1) / band;
+  a->w_shift = w_shift;
+  a->pad_l = pad_l, a->pitch = pitch;
+  a->tile_rows = min((band - 1) * p.sh + p.kh, p.in_h);
+  a->f_bands = make_fastdiv(static_cast<uint32_t>(a->bands_per_plane));
+  a->f_in_w = make_fastdiv(static_cast<uint32_t>(p.in_w));
+  return true;
 }
 
 // Whole-plane windows: x is [rows][len], one output per row.  A workgroup owns
-// ROWS consecutive rows; they pass through LDS in chunks of `chunk` columns
-// (coalesced loads by all lanes), then lane r folds row r element by element.
-// The row pitch in LDS is odd, so the per-lane walks hit distinct banks.
+// `group` consecutive rows (as many as fit the tile, at most one per lane); they
+// pass through LDS (coalesced 128-bit loads by all lanes), then lane r folds
+// row r element by element.  The row pitch in LDS is odd, so the per-lane walks
+// hit distinct banks.  Rows longer than the tile are staged in column chunks.
+// Measured on 51 MB inputs: 49 KB tiles (256 rows of 7x7, 64 rows of 14x14) beat
+// 13 KB tiles by 8 % and 25 %: what the large tile loses in resident workgroups
+// it gains by having every lane of the workgroup fold a row.
 constexpr int kPlaneTileFloats = 12608;  // 256 rows x 49 or 64 rows x 197
-
-inline int plane_pitch_cap(int rows_per_group) { return kPlaneTileFloats / rows_per_group; }
+constexpr int kPlaneMaxGroup = 256;      // rows per workgroup (one lane folds one row)
+constexpr int kPlaneChunkRows = 64;      // rows per workgroup when rows are chunked
 
 constexpr int kPlaneBatch = 8;  // global loads a lane keeps in flight while staging
+constexpr int kPlaneFold = 8;   // LDS reads a lane keeps in flight while folding
 
-template <bool MAX, int ROWS>
+template <bool MAX>
 __global__ __launch_bounds__(kBlock) void pool_plane_kernel(const float* x, float* y, uint32_t rows,
-                                                             uint32_t len, uint32_t chunk,
-                                                             FastDiv f_chunk, FastDiv f_last,
-                                                             float pool_size) {
+                                                             uint32_t len, uint32_t group,
+                                                             uint32_t chunk, FastDiv f_chunk,
+                                                             FastDiv f_last, float pool_size) {
   __shared__ float tile[kPlaneTileFloats];
-  const uint32_t row0 = blockIdx.x * ROWS;
-  const uint32_t nrows = min(static_cast<uint32_t>(ROWS), rows - row0);
+  const uint32_t row0 = blockIdx.x * group;
+  const uint32_t nrows = min(group, rows - row0);
   const uint32_t pitch = chunk | 1u;
   const float* base = x + static_cast<uint64_t>(row0) * len;
   float max_val = -FLT_MAX, sum_val = 0.f;
@@ -372,8 +464,22 @@ __global__ __launch_bounds__(kBlock) void pool_plane_kernel(const float* x, floa
     }
     __syncthreads();
     if (threadIdx.x < nrows) {
+      // Eight LDS reads in flight per step of the (inherently serial) fold.
       const float* mine = tile + threadIdx.x * pitch;
-      for (uint32_t c = 0; c < cols; ++c) {
+      uint32_t c = 0;
+      for (; c + kPlaneFold <= cols; c += kPlaneFold) {
+        float v[kPlaneFold];
+#pragma unroll
+        for (int k = 0; k < kPlaneFold; ++k) v[k] = mine[c + k];
+#pragma unroll
+        for (int k = 0; k < kPlaneFold; ++k) {
+          if (MAX)
+            max_val = pool_max(max_val, v[k]);
+          else
+            sum_val += v[k];
+        }
+      }
+      for (; c < cols; ++c) {
         const float v = mine[c];
         if (MAX)
           max_val = pool_max(max_val, v);
@@ -389,18 +495,22 @@ __global__ __launch_bounds__(kBlock) void pool_plane_kernel(const float* x, floa
 template <bool MAX>
 static void launch_pool_plane(const float* x, float* y, uint32_t rows, uint32_t len,
                               hipStream_t st) {
-  // 256 rows per workgroup only when that still leaves a few workgroups per CU.
-  const int group = rows >= 256u * 1024u ? 256 : 64;
-  const uint32_t cap = static_cast<uint32_t>(plane_pitch_cap(group));  // odd
-  const uint32_t chunk = (len | 1u) <= cap ? len : cap - 1;
+  uint32_t group, chunk;
+  const uint32_t pitch = len | 1u;
+  if (pitch <= kPlaneTileFloats) {  // whole rows: as many as fit the tile
+    group = kPlaneTileFloats / pitch;
+    group = group > kPlaneMaxGroup ? kPlaneMaxGroup : group;
+    if (group >= 4) group &= ~3u;  // keeps every workgroup's first row 16-byte aligned
+    chunk = len;
+  } else {
+    group = kPlaneChunkRows;
+    chunk = (kPlaneTileFloats / kPlaneChunkRows - 1) | 1u;  // odd: it is the LDS pitch too
+  }
   const uint32_t tail = len % chunk;
   const FastDiv fc = make_fastdiv(chunk), fl = make_fastdiv(tail ? tail : chunk);
   const float size = static_cast<float>(static_cast<int>(len));
   const uint32_t grid = (rows + group - 1) / group;
-  if (group == 256)
-    pool_plane_kernel<MAX, 256><<<grid, kBlock, 0, st>>>(x, y, rows, len, chunk, fc, fl, size);
-  else
-    pool_plane_kernel<MAX, 64><<<grid, kBlock, 0, st>>>(x, y, rows, len, chunk, fc, fl, size);
+  pool_plane_kernel<MAX><<<grid, kBlock, 0, st>>>(x, y, rows, len, group, chunk, fc, fl, size);
 }
 
 static int check_pool_dims(int n, const int* in_shape, const int* out_shape) {
@@ -456,36 +566,48 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
   p.f_out_h = make_fastdiv(static_cast<uint32_t>(p.out_h));
   p.f_out_d = make_fastdiv(static_cast<uint32_t>(p.out_d));
   const uint32_t n_out = static_cast<uint32_t>(out_count);
-  const int band = three_d ? 0 : plan_pool_band(p, kPoolBandOutputs);
-  if (band > 0) {
-    BandArgs a;
-    a.in_h = p.in_h, a.in_w = p.in_w, a.out_h = p.out_h, a.out_w = p.out_w;
-    a.kh = p.kh, a.kw = p.kw, a.sh = p.sh, a.sw = p.sw, a.ph = p.ph, a.pw = p.pw;
-    a.band = band;
-    a.bands_per_plane = (p.out_h + band - 1) / band;
-    a.f_out_w = p.f_out_w;
-    a.f_bands = make_fastdiv(static_cast<uint32_t>(a.bands_per_plane));
+  BandArgs a;
+  if (!three_d && plan_pool_band(p, kPoolBandOutputs, &a)) {
     const int64_t groups = static_cast<int64_t>(in_shape[0]) * in_shape[1] * a.bands_per_plane;
-    const int tile_rows = min((band - 1) * p.sh + p.kh, p.in_h);
-    const size_t lds = static_cast<size_t>(tile_rows) * p.in_w * sizeof(float);
+    const size_t lds = static_cast<size_t>(a.tile_rows + 1) * a.pitch * sizeof(float);
     if (groups <= INT32_MAX) {
-      const uint32_t g = static_cast<uint32_t>(groups);
+      a.total_bands = static_cast<uint32_t>(groups);
+      // Enough workgroups to fill the chip a few times over, then longer walks.
+      uint32_t per = a.total_bands / kBandGroupsWanted;
+      per = per < 1 ? 1 : (per > kBandMaxWalk ? kBandMaxWalk : per);
+      a.bands_per_group = per;
+      const uint32_t g = (a.total_bands + per - 1) / per;
+      const bool pipe = p.in_w % 4 == 0 && aligned16(x);
       const int k = p.kh == p.kw && (p.kh == 2 || p.kh == 3) ? p.kh : 0;
+      const int vecs = (a.tile_rows * p.in_w / 4 + kBlock - 1) / kBlock;  // per lane and band
+      const int regs = !pipe ? 0 : (vecs <= 2 ? 2 : (vecs <= 3 ? 3 : (vecs <= 4 ? 4 : (vecs <= 6 ? 6 : 8))));
+#define SHDW_LAUNCH_BAND(MAXV, KV)                                                              \
+  do {                                                                                           \
+    switch (regs) {                                                                              \
+      case 0: pool_band_kernel<MAXV, KV, 0><<<g, kBlock, lds, st>>>(x, y, a); break;             \
+      case 2: pool_band_kernel<MAXV, KV, 2><<<g, kBlock, lds, st>>>(x, y, a); break;             \
+      case 3: pool_band_kernel<MAXV, KV, 3><<<g, kBlock, lds, st>>>(x, y, a); break;             \
+      case 4: pool_band_kernel<MAXV, KV, 4><<<g, kBlock, lds, st>>>(x, y, a); break;             \
+      case 6: pool_band_kernel<MAXV, KV, 6><<<g, kBlock, lds, st>>>(x, y, a); break;             \
+      default: pool_band_kernel<MAXV, KV, 8><<<g, kBlock, lds, st>>>(x, y, a); break;            \
+    }                                                                                            \
+  } while (0)
       if (pool_type == 0) {
         if (k == 3)
-          pool_band_kernel<true, 3><<<g, kBlock, lds, st>>>(x, y, a);
+          SHDW_LAUNCH_BAND(true, 3);
         else if (k == 2)
-          pool_band_kernel<true, 2><<<g, kBlock, lds, st>>>(x, y, a);
+          SHDW_LAUNCH_BAND(true, 2);
         else
-          pool_band_kernel<true, 0><<<g, kBlock, lds, st>>>(x, y, a);
+          SHDW_LAUNCH_BAND(true, 0);
       } else {
         if (k == 3)
-          pool_band_kernel<false, 3><<<g, kBlock, lds, st>>>(x, y, a);
+          SHDW_LAUNCH_BAND(false, 3);
         else if (k == 2)
-          pool_band_kernel<false, 2><<<g, kBlock, lds, st>>>(x, y, a);
+          SHDW_LAUNCH_BAND(false, 2);
         else
-          pool_band_kernel<false, 0><<<g, kBlock, lds, st>>>(x, y, a);
+          SHDW_LAUNCH_BAND(false, 0);
       }
+#undef SHDW_LAUNCH_BAND
       return launch_status();
     }
   }
