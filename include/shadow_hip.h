@@ -273,6 +273,23 @@ int shdw_hip_pooling3d(const int* in_shape, int pool_type, int kernel_d, int ker
                        int pad_h, int pad_w, const int* out_shape, const float* x, float* y,
                        void* stream);
 
+/* GroupNorm / InstanceNorm / LayerNorm core: x viewed as [outer_num][inner_num];
+ *   alpha = 1.f / inner_num
+ *   mean = (float) sum_fp64(alpha * x)            var = (float) sum_fp64(alpha * (x-mean)^2)
+ *   y = (x - mean) / sqrt(var + eps)              (products and differences in fp32)
+ * then, when scale and bias are given (both or neither), with i the element
+ * index in the whole tensor and c = (i / scale_inner) % scale_num:
+ *   y = y * scale[c] + bias[c]                    (multiply, then add)
+ * GroupNorm: outer = N*group, scale_num = C, scale_inner = H*W; InstanceNorm is
+ * group = C; LayerNorm: inner = prod(normalized_shape) = scale_num, scale_inner = 1.
+ * The fp64 sums are associated differently from the reference's serial loop
+ * (contract 1e-5 relative, in practice identical).  y may alias x.
+ * ref: shadow/operators/kernels/group_norm.hpp:41-86, layer_norm.hpp:22-69,
+ *      group_norm.cpp:7-27, group_norm.cu:7-48, shadow/core/blas.cpp:238-247 */
+int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
+                        const float* scale, const float* bias, int scale_num, int scale_inner,
+                        float* y, void* stream);
+
 /* ============================ plan inspection ============================ */
 
 /* Host-only: the collapsed form shdw_hip_broadcast_binary would launch with.

@@ -220,6 +220,18 @@ def pooling_out_size(dim, kernel_size, stride, pad, full_pooling):
                                           int(bool(full_pooling))))
 
 
+def normalize_rows(x, outer, inner, eps):
+    """Mean / variance normalisation of rows, as the GroupNorm and LayerNorm kernel
+    classes run it (before their ScaleBias)."""
+    x = _f(x).ravel()
+    out = np.empty_like(x)
+    mean, var = np.zeros(max(1, outer), np.float32), np.zeros(max(1, outer), np.float32)
+    temp = np.zeros(max(1, x.size), np.float32)
+    lib().orc_normalize_rows(_p(x), int(outer), int(inner), ctypes.c_float(eps), _p(mean), _p(var),
+                             _p(temp), _p(out))
+    return out
+
+
 # --------------------------------------------------------------------------
 # operator level: argument checks and shape rules of shadow/operators/*_op.cpp
 # --------------------------------------------------------------------------
@@ -406,3 +418,40 @@ def pooling_op(x, pool=0, kernel_size=(), stride=(1,), pad=(0,), global_pooling=
         out_shape[n + 2] = pooling_out_size(x.shape[n + 2], kernel_size[n], stride[n], pad[n],
                                             full_pooling)
     return pooling(x, x.shape, pool, kernel_size, stride, pad, out_shape).reshape(out_shape)
+
+
+def group_norm_op(x, group=1, eps=1e-5, scale=None, bias=None):
+    """shadow/operators/group_norm_op.cpp:9-43 and kernels/group_norm.hpp:41-86"""
+    x = _f(x)
+    _check(x.shape[1] % group == 0, "input->shape(1) % group == 0")
+    _check((scale is None) == (bias is None), "inputs.size() == 3")
+    outer = x.shape[0] * group
+    out = normalize_rows(x, outer, x.size // outer, np.float32(eps))
+    if scale is not None:
+        channel, spatial = x.shape[1], int(np.prod(x.shape[2:], dtype=np.int64))
+        _check(np.size(scale) == channel, "scale->count() == channel")
+        _check(np.size(bias) == channel, "bias->count() == channel")
+        out = scale_bias(out, _f(scale).ravel(), _f(bias).ravel(), channel, spatial)
+    return out.reshape(x.shape)
+
+
+def instance_norm_op(x, eps=1e-5, scale=None, bias=None):
+    """shadow/operators/instance_norm_op.cpp:9-36: GroupNorm with one group per channel"""
+    return group_norm_op(x, _f(x).shape[1], eps, scale, bias)
+
+
+def layer_norm_op(x, normalized_shape, eps=1e-5, scale=None, bias=None):
+    """shadow/operators/layer_norm_op.cpp:9-45 and kernels/layer_norm.hpp:22-69"""
+    x = _f(x)
+    ns = list(normalized_shape)
+    _check(len(ns) > 0, "!normalized_shape.empty()")
+    _check(len(ns) <= x.ndim and list(x.shape[x.ndim - len(ns):]) == ns,
+           "input->shape(n - size) == normalized_shape[n]")
+    _check((scale is None) == (bias is None), "inputs.size() == 3")
+    inner = int(np.prod(ns, dtype=np.int64))
+    out = normalize_rows(x, x.size // inner, inner, np.float32(eps))
+    if scale is not None:
+        _check(list(np.shape(scale)) == ns, "scale->shape() == normalized_shape")
+        _check(list(np.shape(bias)) == ns, "bias->shape() == normalized_shape")
+        out = scale_bias(out, _f(scale).ravel(), _f(bias).ravel(), inner, 1)
+    return out.reshape(x.shape)

@@ -467,3 +467,50 @@ API int orc_pooling_out_size(int dim, int kernel_size, int stride, int pad, int 
   float t = (dim + 2.f * pad - kernel_size) / stride;
   return (int)((full_pooling ? ceilf(t) : floorf(t)) + 1);
 }
+
+/* ---- shadow/core/blas.cpp:238-247, 281-285  BlasSgemv, no-transpose plain-loop
+ *      branch: y *= beta, then y[i] += (float) sum_fp64_j(alpha * A[i][j] * x[j])
+ *      with the products formed in fp32.  Used here only as the row mean of the
+ *      normalisation kernels (x = ones, beta = 0). ---- */
+API void orc_sgemv_n(int M, int N, float alpha, const float* A, const float* x, float beta,
+                     float* y) {
+  for (int i = 0; i < M; ++i) y[i] *= beta;
+  for (int i = 0; i < M; ++i) {
+    double sum = 0;
+    for (int j = 0; j < N; ++j) sum += alpha * A[i * N + j] * x[j];
+    y[i] += (float)sum;
+  }
+}
+
+/* ---- shadow/operators/kernels/group_norm.cpp:7-16  SubtractMeanAndSquare ---- */
+API void orc_subtract_mean_and_square(const float* in, const float* mean, int count,
+                                      int inner_num, float* out, float* square) {
+  for (int i = 0; i < count; ++i) {
+    float val = in[i] - mean[i / inner_num];
+    out[i] = val;
+    square[i] = val * val;
+  }
+}
+
+/* ---- shadow/operators/kernels/group_norm.cpp:18-27  DivideVariance ---- */
+API void orc_divide_variance(const float* in, const float* variance, int count, int inner_num,
+                             float eps, float* out) {
+  for (int i = 0; i < count; ++i) out[i] = in[i] / sqrtf(variance[i / inner_num] + eps);
+}
+
+/* ---- shadow/operators/kernels/group_norm.hpp:41-74 (GroupNorm, InstanceNorm) and
+ *      layer_norm.hpp:22-57 (LayerNorm): the kernel classes' sequence of calls on
+ *      x viewed as [outer_num][inner_num], without the trailing ScaleBias.
+ *      mean / variance / temp are caller scratch of outer, outer, count floats,
+ *      zero-filled like a fresh temp buffer. ---- */
+API void orc_normalize_rows(const float* in, int outer_num, int inner_num, float eps, float* mean,
+                            float* variance, float* temp, float* out) {
+  int count = outer_num * inner_num;
+  float* ones = (float*)malloc(sizeof(float) * (size_t)(inner_num > 0 ? inner_num : 1));
+  orc_set(inner_num, 1, ones);
+  orc_sgemv_n(outer_num, inner_num, 1.f / inner_num, in, ones, 0, mean);
+  orc_subtract_mean_and_square(in, mean, count, inner_num, out, temp);
+  orc_sgemv_n(outer_num, inner_num, 1.f / inner_num, temp, ones, 0, variance);
+  orc_divide_variance(out, variance, count, inner_num, eps, out);
+  free(ones);
+}

@@ -74,6 +74,7 @@ SIGNATURES = {
     "shdw_hip_scale_residual_relu_rowmean": (_I, [_I, _I, _I, _V, _V, _V, _V, _V, _V, _V]),
     "shdw_hip_axpy_rows": (_I, [_I, _I, _V, _V, _V, _V, _V]),
     "shdw_hip_batch_norm": (_I, [_I, _I, _I, _V, _V, _V, _F, _F, _V, _V]),
+    "shdw_hip_group_norm": (_I, [_I, _I, _F, _V, _V, _V, _I, _I, _V, _V]),
     "shdw_hip_softmax": (_I, [_I, _I, _I, _V, _V, _V]),
     "shdw_hip_normalize": (_I, [_I, _I, _I, _F, _F, _V, _V, _V]),
     "shdw_hip_pooling2d": (_I, [c_int_p, _I, _I, _I, _I, _I, _I, _I, c_int_p, _V, _V, _V]),

@@ -109,11 +109,12 @@ def keys(fn):
 
 def test_registries_hold_exactly_the_gpu_default_kernels():
     h = shadow_amd.host()
-    types = ["Activate", "Axpy", "BatchNorm", "Binary", "Eltwise", "Normalize", "Pooling", "Reduce",
-             "Scale", "Softmax", "Unary"]
-    assert keys(h.shdw_host_operator_keys) == types
+    kernels = ["Activate", "Axpy", "BatchNorm", "Binary", "Eltwise", "GroupNorm", "LayerNorm", "Normalize",
+               "Pooling", "Reduce", "Scale", "Softmax", "Unary"]
+    # InstanceNorm runs on the GroupNorm kernel (shadow/operators/instance_norm_op.cpp:14)
+    assert keys(h.shdw_host_operator_keys) == sorted(kernels + ["InstanceNorm"])
     kk = keys(h.shdw_host_kernel_keys)
-    assert kk == ["%sGPU(Default)" % t for t in types]
+    assert kk == ["%sGPU(Default)" % t for t in kernels]
     # a CUDNN flavour would outrank Default; a CPU kernel would be a compute fallback
     assert not any("CUDNN" in k or "CPU" in k for k in kk)
 

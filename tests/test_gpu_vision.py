@@ -9,7 +9,7 @@ import oracle
 import shadow_amd
 from shadow_amd import ShadowError
 from tests import gpuops
-from tests.helpers import assert_bit_exact, normal, uniform, with_specials
+from tests.helpers import assert_bit_exact, assert_rel_close, normal, uniform, with_specials
 
 pytestmark = pytest.mark.gpu
 F = np.float32
@@ -233,3 +233,75 @@ def test_entry_point_argument_errors(gpu):
     assert lib.shdw_hip_pooling2d(sh, 0, 0, 2, 1, 1, 0, 0, sh, buf.ptr, buf.ptr, None) == E
     assert lib.shdw_hip_pooling2d(sh, 0, 2, 2, 0, 1, 0, 0, sh, buf.ptr, buf.ptr, None) == E
     assert lib.shdw_hip_pooling2d(sh, 0, 2, 2, 1, 1, 0, 0, shadow_amd.ints([2, 1, 3, 3]), buf.ptr, buf.ptr, None) == E
+
+
+# ------------------------------------------- group / instance / layer norm ---
+# The fp64 row sums are associated differently on the GPU (per-lane partials
+# combined through LDS) than in the oracle's serial loop.  Contract: 1e-5
+# relative on every output; the tests also count differing bits, and every case
+# here comes out identical.
+NORM_ROWS = [(6, 49), (4, 784), (8, 1024), (3, 2048), (5, 3136), (2, 4096), (2, 4100), (2, 25088), (7, 5),
+             (300, 12), (1, 1), (3, 1000), (2, 8192), (2, 6002)]
+
+
+@pytest.mark.parametrize("outer,inner", NORM_ROWS)
+def test_group_norm_rows(gpu, outer, inner):
+    x = normal(40, outer * inner, 3.0) + F(0.75)
+    want = oracle.normalize_rows(x, outer, inner, 1e-5)
+    for kw in ({}, {"inplace": True}, {"offset": 1}):
+        got = gpuops.group_norm(x, outer, inner, 1e-5, **kw)
+        assert assert_rel_close(got, want, 1e-5, "norm rows %s" % kw) == 0
+
+
+@pytest.mark.parametrize("shape,group", [((2, 8, 5, 5), 1), ((2, 8, 5, 5), 4), ((4, 32, 14, 14), 8), ((2, 6, 7, 3), 6),
+                                         ((1, 64, 56, 56), 32)])
+def test_group_and_instance_norm_op(ws, shape, group):
+    x = normal(41, shape, 2.0) + F(0.5)
+    scale, bias = uniform(42, shape[1], 0.5, 2.0), normal(43, shape[1])
+    got = run(ws, "GroupNorm", [("x", x)], {"group": group})
+    assert got.shape == x.shape
+    assert assert_rel_close(got, oracle.group_norm_op(x, group), 1e-5, "group norm") == 0
+    got = run(ws, "GroupNorm", [("x", x), ("s", scale), ("b", bias)], {"group": group, "eps": 1e-3})
+    assert assert_rel_close(got, oracle.group_norm_op(x, group, 1e-3, scale, bias), 1e-5, "group norm affine") == 0
+    got = run(ws, "InstanceNorm", [("x", x), ("s", scale), ("b", bias)], {})
+    assert assert_rel_close(got, oracle.instance_norm_op(x, 1e-5, scale, bias), 1e-5, "instance norm") == 0
+    got = run(ws, "InstanceNorm", [("x", x)], {"eps": 1e-2})
+    assert assert_rel_close(got, oracle.instance_norm_op(x, 1e-2), 1e-5, "instance norm plain") == 0
+
+
+@pytest.mark.parametrize("shape,ns", [((4, 10, 32), [32]), ((2, 3, 6, 5), [6, 5]), ((64, 768), [768]), ((2, 3, 4), [3, 4]),
+                                      ((3, 5000), [5000])])
+def test_layer_norm_op(ws, shape, ns):
+    x = normal(44, shape, 2.0)
+    scale, bias = uniform(45, ns, 0.5, 2.0), normal(46, ns)
+    got = run(ws, "LayerNorm", [("x", x)], {"normalized_shape": ns})
+    assert got.shape == x.shape
+    assert assert_rel_close(got, oracle.layer_norm_op(x, ns), 1e-5, "layer norm") == 0
+    got = run(ws, "LayerNorm", [("x", x), ("s", scale), ("b", bias)], {"normalized_shape": ns, "eps": 1e-6})
+    assert assert_rel_close(got, oracle.layer_norm_op(x, ns, 1e-6, scale, bias), 1e-5, "layer norm affine") == 0
+
+
+def test_norm_special_values_and_errors(ws):
+    # a NaN or inf poisons its own row only; constant rows give 0 / sqrt(eps)
+    x = normal(47, (6, 64), 1.0)
+    x[1, 3], x[2, 5], x[4, :] = np.nan, np.inf, 2.5
+    got = run(ws, "LayerNorm", [("x", x)], {"normalized_shape": [64]})
+    assert_bit_exact(got, oracle.layer_norm_op(x, [64]), "norm specials")
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("LayerNorm", ["x"], ["o1"], {})
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("LayerNorm", ["x"], ["o2"], {"normalized_shape": [32]}).run()
+    ws.set_blob("img", np.zeros((2, 6, 4, 4), F))
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("GroupNorm", ["img"], ["o3"], {"group": 4}).run()
+    ws.set_blob("s5", np.ones(5, F))
+    ws.set_blob("b6", np.ones(6, F))
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("GroupNorm", ["img", "s5", "b6"], ["o4"], {"group": 2}).run()
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("InstanceNorm", ["img", "b6"], ["o5"], {}).run()
+    lib = shadow_amd.hip()
+    buf = shadow_amd.Buffer(1024)
+    assert lib.shdw_hip_group_norm(2, 8, 1e-5, buf.ptr, buf.ptr, None, 1, 1, buf.ptr, None) == -1
+    assert lib.shdw_hip_group_norm(-1, 8, 1e-5, buf.ptr, None, None, 1, 1, buf.ptr, None) == -1
+    assert lib.shdw_hip_group_norm(0, 8, 1e-5, None, None, None, 1, 1, None, None) == 0

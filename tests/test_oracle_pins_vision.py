@@ -236,3 +236,59 @@ def test_pooling_op_checks():
         oracle.pooling_op(np.zeros((2, 3, 4, 4), F), 2, [2])
     with pytest.raises(oracle.OracleCheckError):
         oracle.pooling_op(np.zeros((2, 3, 4, 4), F), 0, [2, 2, 2])
+
+
+# --------------------------------------------------- group / instance / layer norm ---
+def normalize_rows_numpy(x2, eps):
+    """x2: [outer, inner].  fp32 products, fp64 front-to-back sums, one rounding each."""
+    alpha = F(1) / F(x2.shape[1])
+    mean = running_sum(alpha * x2, 1, np.float64).astype(F)
+    val = x2 - mean[:, None]
+    var = running_sum(alpha * (val * val), 1, np.float64).astype(F)
+    return val / np.sqrt(var + F(eps))[:, None]
+
+
+@pytest.mark.parametrize("shape,group", [((2, 8, 5, 5), 1), ((2, 8, 5, 5), 4), ((3, 6, 7, 3), 6), ((1, 4, 1, 1), 2)])
+def test_group_norm_against_axis_formulation(shape, group):
+    x = normal(30, shape, 3.0) + F(1.5)
+    want = normalize_rows_numpy(x.reshape(shape[0] * group, -1), 1e-5).reshape(shape)
+    assert_bit_exact(oracle.group_norm_op(x, group), want, "group norm")
+    scale, bias = uniform(31, shape[1], 0.5, 2.0), normal(32, shape[1])
+    want_affine = want * scale[None, :, None, None] + bias[None, :, None, None]
+    assert_bit_exact(oracle.group_norm_op(x, group, scale=scale, bias=bias), want_affine, "group norm affine")
+    if group == shape[1]:
+        assert_bit_exact(oracle.instance_norm_op(x, scale=scale, bias=bias), want_affine, "instance norm")
+
+
+@pytest.mark.parametrize("shape,ns", [((4, 10, 32), [32]), ((2, 3, 6, 5), [6, 5]), ((5, 7), [7]), ((2, 3, 4), [3, 4])])
+def test_layer_norm_against_axis_formulation(shape, ns):
+    x = normal(33, shape, 2.0)
+    inner = int(np.prod(ns))
+    want = normalize_rows_numpy(x.reshape(-1, inner), 1e-5).reshape(shape)
+    assert_bit_exact(oracle.layer_norm_op(x, ns), want, "layer norm")
+    scale, bias = uniform(34, ns, 0.5, 2.0), normal(35, ns)
+    assert_bit_exact(oracle.layer_norm_op(x, ns, scale=scale, bias=bias), want * scale + bias, "layer norm affine")
+
+
+def test_norm_known_values_and_checks():
+    # mean 2, deviations -1/+1, variance 1, eps 0
+    assert oracle.layer_norm_op(F([[1, 3]]), [2], eps=0.0).ravel().tolist() == [-1.0, 1.0]
+    # constant row: 0 / sqrt(eps)
+    assert oracle.group_norm_op(np.full((1, 2, 2, 2), 7, F), 1).ravel().tolist() == [0.0] * 8
+    # the 1/inner factor is applied per element in fp32, before the fp64 sum:
+    # 3 * fl(fl(1/3) * 1) = 1.0000000298 in fp64, which rounds to 1 in fp32
+    assert oracle.layer_norm_op(F([[1, 1, 1]]), [3], eps=1.0).ravel().tolist() == [0.0] * 3
+    big = F([[16777216.0, 1.0, 1.0, 1.0]])  # an fp32 running sum would drop the ones
+    m = running_sum(F(0.25) * big, 1, np.float64).astype(F)
+    assert m[0] == F(4194304.75)
+    assert_bit_exact(oracle.layer_norm_op(big, [4]), normalize_rows_numpy(big, 1e-5), "fp64 accumulate")
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.group_norm_op(np.zeros((1, 6, 2, 2), F), 4)
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.group_norm_op(np.zeros((1, 6, 2, 2), F), 3, scale=np.ones(5, F), bias=np.ones(6, F))
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.layer_norm_op(np.zeros((2, 3, 4), F), [4, 3])
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.layer_norm_op(np.zeros((2, 3, 4), F), [])
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.layer_norm_op(np.zeros((2, 3, 4), F), [4], scale=np.ones(4, F))
