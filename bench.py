@@ -349,6 +349,17 @@ def config_table(dev):
     ms = time_batch(dev, lambda k: lib.shdw_hip_normalize(64, 49, 16384, 2.0, 1e-12, AH[k].ptr, YH[k].ptr, st),
                     SH, reps=20)
     add("next", "normalize_l2_channels_dense [64,49,128,128]", 8 * NH, ms, NH)
+    sch, bih = dev.buf(uniform(614, CH, 0.5, 1.5)), dev.buf(uniform(615, CH, -0.1, 0.1))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_group_norm(64 * CH, INH, 1e-5, AH[k].ptr, sch.ptr, bih.ptr,
+                                                           CH, INH, YH[k].ptr, st), SH, reps=20)
+    add("next", "instance_norm affine [64,256,56,56]", 8 * NH + 8 * CH, ms, NH)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_group_norm(64 * 32, 8 * INH, 1e-5, AH[k].ptr, sch.ptr, bih.ptr,
+                                                           CH, INH, YH[k].ptr, st), SH, reps=20)
+    add("next", "group_norm 32 groups affine [64,256,56,56]", 8 * NH + 8 * CH, ms, NH)
+    lns, lnb = dev.buf(uniform(616, 784, 0.5, 1.5)), dev.buf(uniform(617, 784, -0.1, 0.1))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_group_norm(65536, 784, 1e-5, AH[k].ptr, lns.ptr, lnb.ptr,
+                                                           784, 1, YH[k].ptr, st), SH, reps=20)
+    add("next", "layer_norm affine [65536,784]", 8 * NH + 8 * 784, ms, NH)
     for bset in (AH, YH):
         for bb in bset:
             bb.free()

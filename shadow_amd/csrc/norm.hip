@@ -6,13 +6,19 @@
 // ones: (float) of an fp64 running sum of the fp32 products alpha * v with
 // alpha = 1 / inner (shadow/core/blas.cpp:238-247), five launches and three
 // scratch blobs per call (shadow/operators/kernels/group_norm.hpp:41-86).  Here
-// one workgroup owns a row and does everything in one launch: fp64 partial sums
-// per lane, combined through LDS.  The fp64 additions are associated
+// a row is owned by one wave64 (rows up to 2048 elements) or one workgroup and
+// everything happens in one launch: fp64 partial sums per lane, combined by
+// shuffles (and LDS across waves).  The fp64 additions are associated
 // differently from the reference's front-to-back loop; the sums are then
 // rounded to fp32 once, so the statistics (and with them every output) come out
 // identical unless an fp64 sum lands within ~1e-16 relative of an fp32 rounding
-// boundary.  Rows of up to 4096 elements stay in registers between the three
+// boundary.  Rows of up to 32768 elements stay in registers between the three
 // passes (one HBM read, one write); longer rows are re-read, from L2.
+//
+// The kernels are close to VALU-bound (two fp64 accumulations and an IEEE
+// division per element), so the affine step avoids per-element index
+// arithmetic: LayerNorm's parameters are loaded as vectors by row position,
+// GroupNorm's channel is computed once per 128-bit vector.
 #include <hip/hip_runtime.h>
 
 #include "../../include/shadow_hip.h"
@@ -23,110 +29,172 @@
 
 namespace shdw {
 
+enum AffineMode {
+  kAffineNone = 0,
+  kAffineRowPos = 1,   // parameter index = position in the row (LayerNorm)
+  kAffineVector = 2,   // scale_inner % 4 == 0: one channel per aligned vector
+  kAffineElement = 3,  // anything else: channel per element
+};
+
 struct NormArgs {
-  uint32_t inner;
+  uint32_t outer, inner;
   float alpha, eps;
-  const float* scale;  // nullptr: no affine step
+  int affine;
+  const float* scale;
   const float* bias;
   FastDiv f_scale_inner, f_scale_num;  // channel = (i / scale_inner) % scale_num
 };
 
-// Sum over the workgroup, result in every lane.  `slots` holds one double per wave.
-SHDW_DEVICE double block_sum(double v, double* slots) {
+SHDW_DEVICE uint32_t norm_channel(const NormArgs& p, uint32_t i) {
+  const uint32_t q = fd_div(i, p.f_scale_inner);
+  return q - fd_div(q, p.f_scale_num) * p.f_scale_num.d;
+}
+
+SHDW_DEVICE float affine1(float v, float s, float b) {
+  const float t = v * s;
+  return t + b;
+}
+
+// Affine step for the aligned vector at row position `pos` (global index i).
+SHDW_DEVICE v4f norm_affine4(const NormArgs& p, uint32_t i, uint32_t pos, v4f v) {
+  if (p.affine == kAffineNone) return v;
+  v4f r;
+  if (p.affine == kAffineRowPos) {
+    const v4f s = load4(p.scale + pos), b = load4(p.bias + pos);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = affine1(v[j], s[j], b[j]);
+  } else if (p.affine == kAffineVector) {
+    const uint32_t c = norm_channel(p, i);
+    const float s = p.scale[c], b = p.bias[c];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = affine1(v[j], s, b);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t c = norm_channel(p, i + j);
+      r[j] = affine1(v[j], p.scale[c], p.bias[c]);
+    }
+  }
+  return r;
+}
+
+SHDW_DEVICE float norm_affine1(const NormArgs& p, uint32_t i, float v) {
+  if (p.affine == kAffineNone) return v;
+  const uint32_t c = norm_channel(p, i);
+  return affine1(v, p.scale[c], p.bias[c]);
+}
+
+SHDW_DEVICE double wave_sum(double v) {
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
+  return v;
+}
+
+// Sum over the LANES lanes that own a row, result in each of them.
+template <int LANES>
+SHDW_DEVICE double row_sum(double v, double* slots) {
+  v = wave_sum(v);
+  if (LANES == kWave) return v;
   __syncthreads();  // slots may still be read from the previous sum
   if ((threadIdx.x & 63) == 0) slots[threadIdx.x >> 6] = v;
   __syncthreads();
   double total = slots[0];
 #pragma unroll
-  for (int w = 1; w < kBlock / kWave; ++w) total += slots[w];
+  for (int w = 1; w < LANES / kWave; ++w) total += slots[w];
   return total;
 }
 
-SHDW_DEVICE float norm_affine(const NormArgs& p, uint32_t i, float v) {
-  if (p.scale == nullptr) return v;
-  const uint32_t q = fd_div(i, p.f_scale_inner);
-  const uint32_t c = q - fd_div(q, p.f_scale_num) * p.f_scale_num.d;
-  const float t = v * p.scale[c];
-  return t + p.bias[c];
+// The row (inner % 4 == 0, <= REGS * 4 * LANES elements, 16-byte aligned) is
+// held in REGS vectors per lane.  LANES = 64: four rows per 256-lane workgroup,
+// no barriers.  LANES = 256 or 1024: one row per workgroup of that size.
+constexpr int kBigBlock = 1024;
+
+template <int REGS, int LANES>
+__global__ __launch_bounds__(LANES == kWave ? kBlock : LANES) void norm_rows_reg_kernel(
+    const float* x, float* y, NormArgs p) {
+  __shared__ double slots[kBigBlock / kWave];
+  const uint32_t lane = LANES == kWave ? (threadIdx.x & 63u) : threadIdx.x;
+  const uint32_t row = LANES == kWave ? blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6) : blockIdx.x;
+  if (LANES == kWave && row >= p.outer) return;  // whole waves leave; no barrier in this form
+  const uint64_t base = static_cast<uint64_t>(row) * p.inner;
+  const float* xr = x + base;
+  float* yr = y + base;
+  const uint32_t nvec = p.inner / 4;
+  v4f reg[REGS];
+#pragma unroll
+  for (int k = 0; k < REGS; ++k) {
+    const uint32_t v = k * LANES + lane;
+    if (v < nvec) reg[k] = load4_stream(xr + 4ull * v);
+  }
+  double acc = 0;
+#pragma unroll
+  for (int k = 0; k < REGS; ++k) {
+    if (k * LANES + lane < nvec) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float t = p.alpha * reg[k][j];
+        acc += static_cast<double>(t);
+      }
+    }
+  }
+  const float mean = static_cast<float>(row_sum<LANES>(acc, slots));
+  acc = 0;
+#pragma unroll
+  for (int k = 0; k < REGS; ++k) {
+    if (k * LANES + lane < nvec) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float val = reg[k][j] - mean;
+        reg[k][j] = val;
+        const float sq = val * val;
+        const float t = p.alpha * sq;
+        acc += static_cast<double>(t);
+      }
+    }
+  }
+  const float variance = static_cast<float>(row_sum<LANES>(acc, slots));
+  const float ve = variance + p.eps;
+  const float denom = __builtin_sqrtf(ve);
+#pragma unroll
+  for (int k = 0; k < REGS; ++k) {
+    const uint32_t v = k * LANES + lane;
+    if (v < nvec) {
+      v4f r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = reg[k][j] / denom;
+      store4_stream(yr + 4ull * v, norm_affine4(p, static_cast<uint32_t>(base) + 4 * v, 4 * v, r));
+    }
+  }
 }
 
-// REGS > 0: the row (<= REGS * 4 * kBlock elements, inner % 4 == 0, 16-byte
-// aligned) is held in REGS vectors per lane.  REGS < 0: longer rows of that
-// kind, three passes with 128-bit accesses.  REGS == 0: any row, three passes
-// with scalar accesses.
-template <int REGS>
-__global__ __launch_bounds__(kBlock) void norm_rows_kernel(const float* x, float* y, NormArgs p) {
+// Any row, one workgroup per row, three passes over memory (the second and
+// third find the row in L2).  VEC: inner % 4 == 0 and 16-byte aligned.
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void norm_rows_stream_kernel(const float* x, float* y, NormArgs p) {
   __shared__ double slots[kBlock / kWave];
   const uint64_t base = static_cast<uint64_t>(blockIdx.x) * p.inner;
   const float* xr = x + base;
   float* yr = y + base;
-  if (REGS > 0) {
-    constexpr int R = REGS > 0 ? REGS : 1;
-    const uint32_t nvec = p.inner / 4;
-    v4f reg[R];
-#pragma unroll
-    for (int k = 0; k < R; ++k) {
-      const uint32_t v = k * kBlock + threadIdx.x;
-      if (v < nvec) reg[k] = load4_stream(xr + 4ull * v);
-    }
-    double acc = 0;
-#pragma unroll
-    for (int k = 0; k < R; ++k) {
-      if (k * kBlock + threadIdx.x < nvec) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float t = p.alpha * reg[k][j];
-          acc += static_cast<double>(t);
-        }
-      }
-    }
-    const float mean = static_cast<float>(block_sum(acc, slots));
-    acc = 0;
-#pragma unroll
-    for (int k = 0; k < R; ++k) {
-      if (k * kBlock + threadIdx.x < nvec) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float val = reg[k][j] - mean;
-          reg[k][j] = val;
-          const float sq = val * val;
-          const float t = p.alpha * sq;
-          acc += static_cast<double>(t);
-        }
-      }
-    }
-    const float variance = static_cast<float>(block_sum(acc, slots));
-    const float ve = variance + p.eps;
-    const float denom = __builtin_sqrtf(ve);
-#pragma unroll
-    for (int k = 0; k < R; ++k) {
-      const uint32_t v = k * kBlock + threadIdx.x;
-      if (v < nvec) {
-        v4f r;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          r[j] = norm_affine(p, static_cast<uint32_t>(base) + 4 * v + j, reg[k][j] / denom);
-        store4_stream(yr + 4ull * v, r);
-      }
-    }
-  } else if (REGS < 0) {
-    // Long rows, 128-bit accesses; passes two and three find the row in L2.
-    const uint32_t nvec = p.inner / 4;
-    double acc = 0;
-    for (uint32_t v = threadIdx.x; v < nvec; v += kBlock) {
-      const v4f q = load4(xr + 4ull * v);
+  const uint32_t steps = VEC ? p.inner / 4 : p.inner;
+  double acc = 0;
+  for (uint32_t t = threadIdx.x; t < steps; t += kBlock) {
+    if (VEC) {
+      const v4f q = load4(xr + 4ull * t);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float a = p.alpha * q[j];
         acc += static_cast<double>(a);
       }
+    } else {
+      const float a = p.alpha * xr[t];
+      acc += static_cast<double>(a);
     }
-    const float mean = static_cast<float>(block_sum(acc, slots));
-    acc = 0;
-    for (uint32_t v = threadIdx.x; v < nvec; v += kBlock) {
-      const v4f q = load4(xr + 4ull * v);
+  }
+  const float mean = static_cast<float>(row_sum<kBlock>(acc, slots));
+  acc = 0;
+  for (uint32_t t = threadIdx.x; t < steps; t += kBlock) {
+    if (VEC) {
+      const v4f q = load4(xr + 4ull * t);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float val = q[j] - mean;
@@ -134,40 +202,29 @@ __global__ __launch_bounds__(kBlock) void norm_rows_kernel(const float* x, float
         const float a = p.alpha * sq;
         acc += static_cast<double>(a);
       }
-    }
-    const float variance = static_cast<float>(block_sum(acc, slots));
-    const float ve = variance + p.eps;
-    const float denom = __builtin_sqrtf(ve);
-    for (uint32_t v = threadIdx.x; v < nvec; v += kBlock) {
-      const v4f q = load4(xr + 4ull * v);
-      v4f r;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float val = q[j] - mean;
-        r[j] = norm_affine(p, static_cast<uint32_t>(base) + 4 * v + j, val / denom);
-      }
-      store4_stream(yr + 4ull * v, r);
-    }
-  } else {
-    double acc = 0;
-    for (uint32_t t = threadIdx.x; t < p.inner; t += kBlock) {
-      const float a = p.alpha * xr[t];
-      acc += static_cast<double>(a);
-    }
-    const float mean = static_cast<float>(block_sum(acc, slots));
-    acc = 0;
-    for (uint32_t t = threadIdx.x; t < p.inner; t += kBlock) {
+    } else {
       const float val = xr[t] - mean;
       const float sq = val * val;
       const float a = p.alpha * sq;
       acc += static_cast<double>(a);
     }
-    const float variance = static_cast<float>(block_sum(acc, slots));
-    const float ve = variance + p.eps;
-    const float denom = __builtin_sqrtf(ve);
-    for (uint32_t t = threadIdx.x; t < p.inner; t += kBlock) {
+  }
+  const float variance = static_cast<float>(row_sum<kBlock>(acc, slots));
+  const float ve = variance + p.eps;
+  const float denom = __builtin_sqrtf(ve);
+  for (uint32_t t = threadIdx.x; t < steps; t += kBlock) {
+    if (VEC) {
+      const v4f q = load4(xr + 4ull * t);
+      v4f r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float val = q[j] - mean;
+        r[j] = val / denom;
+      }
+      store4_stream(yr + 4ull * t, norm_affine4(p, static_cast<uint32_t>(base) + 4 * t, 4 * t, r));
+    } else {
       const float val = xr[t] - mean;
-      yr[t] = norm_affine(p, static_cast<uint32_t>(base) + t, val / denom);
+      yr[t] = norm_affine1(p, static_cast<uint32_t>(base) + t, val / denom);
     }
   }
 }
@@ -188,6 +245,7 @@ int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
   if (!x || !y || (scale == nullptr) != (bias == nullptr)) return SHDW_E_INVALID_ARGUMENT;
   if (scale && (scale_num < 1 || scale_inner < 1)) return SHDW_E_INVALID_ARGUMENT;
   NormArgs p;
+  p.outer = static_cast<uint32_t>(outer_num);
   p.inner = static_cast<uint32_t>(inner_num);
   p.alpha = 1.f / inner_num;
   p.eps = eps;
@@ -195,20 +253,43 @@ int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
   p.bias = bias;
   p.f_scale_inner = make_fastdiv(static_cast<uint32_t>(scale ? scale_inner : 1));
   p.f_scale_num = make_fastdiv(static_cast<uint32_t>(scale ? scale_num : 1));
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  const uint32_t grid = static_cast<uint32_t>(outer_num);
   const bool vec = inner_num % 4 == 0 && aligned16(x) && aligned16(y);
-  const int vecs = (inner_num / 4 + kBlock - 1) / kBlock;
-  if (vec && vecs <= 1)
-    norm_rows_kernel<1><<<grid, kBlock, 0, st>>>(x, y, p);
-  else if (vec && vecs <= 2)
-    norm_rows_kernel<2><<<grid, kBlock, 0, st>>>(x, y, p);
-  else if (vec && vecs <= 4)
-    norm_rows_kernel<4><<<grid, kBlock, 0, st>>>(x, y, p);
-  else if (vec)
-    norm_rows_kernel<-1><<<grid, kBlock, 0, st>>>(x, y, p);
+  if (!scale)
+    p.affine = kAffineNone;
+  else if (vec && scale_inner == 1 && scale_num == inner_num && aligned16(scale) && aligned16(bias))
+    p.affine = kAffineRowPos;
+  else if (vec && scale_inner % 4 == 0)
+    p.affine = kAffineVector;
   else
-    norm_rows_kernel<0><<<grid, kBlock, 0, st>>>(x, y, p);
+    p.affine = kAffineElement;
+
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint32_t rows = p.outer;
+  const uint32_t nvec = p.inner / 4;
+  const uint32_t wave_grid = (rows + kBlock / kWave - 1) / (kBlock / kWave);
+  if (!vec) {
+    norm_rows_stream_kernel<false><<<rows, kBlock, 0, st>>>(x, y, p);
+  } else if (nvec <= 1 * kWave) {
+    norm_rows_reg_kernel<1, kWave><<<wave_grid, kBlock, 0, st>>>(x, y, p);
+  } else if (nvec <= 2 * kWave) {
+    norm_rows_reg_kernel<2, kWave><<<wave_grid, kBlock, 0, st>>>(x, y, p);
+  } else if (nvec <= 4 * kWave) {
+    norm_rows_reg_kernel<4, kWave><<<wave_grid, kBlock, 0, st>>>(x, y, p);
+  } else if (nvec <= 8 * kWave && rows >= 2048) {
+    norm_rows_reg_kernel<8, kWave><<<wave_grid, kBlock, 0, st>>>(x, y, p);
+  } else if (nvec <= 2 * kBlock) {
+    norm_rows_reg_kernel<2, kBlock><<<rows, kBlock, 0, st>>>(x, y, p);
+  } else if (nvec <= 4 * kBlock) {
+    norm_rows_reg_kernel<4, kBlock><<<rows, kBlock, 0, st>>>(x, y, p);
+  } else if (nvec <= 8 * kBlock) {
+    norm_rows_reg_kernel<8, kBlock><<<rows, kBlock, 0, st>>>(x, y, p);
+  } else if (nvec <= 4 * kBigBlock) {
+    norm_rows_reg_kernel<4, kBigBlock><<<rows, kBigBlock, 0, st>>>(x, y, p);
+  } else if (nvec <= 8 * kBigBlock) {
+    norm_rows_reg_kernel<8, kBigBlock><<<rows, kBigBlock, 0, st>>>(x, y, p);
+  } else {
+    norm_rows_stream_kernel<true><<<rows, kBlock, 0, st>>>(x, y, p);
+  }
   return launch_status();
 }
 

@@ -241,7 +241,7 @@ def test_entry_point_argument_errors(gpu):
 # relative on every output; the tests also count differing bits, and every case
 # here comes out identical.
 NORM_ROWS = [(6, 49), (4, 784), (8, 1024), (3, 2048), (5, 3136), (2, 4096), (2, 4100), (2, 25088), (7, 5),
-             (300, 12), (1, 1), (3, 1000), (2, 8192), (2, 6002)]
+             (300, 12), (1, 1), (3, 1000), (2, 8192), (2, 6002), (7, 400), (2100, 1200), (2051, 2048), (9, 256), (3, 16384), (2, 32768), (2, 32772), (1, 70000)]
 
 
 @pytest.mark.parametrize("outer,inner", NORM_ROWS)
