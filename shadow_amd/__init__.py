@@ -189,6 +189,14 @@ HOST_SIGNATURES = {
     "shdw_host_op_destroy": (None, [_V]),
     "shdw_host_op_run": (_I, [_V, _V]),
     "shdw_host_op_debug_log": (_I, [_V, _V, ctypes.c_char_p, _Z]),
+    "shdw_host_parse_net": (_I, [ctypes.c_char_p, ctypes.c_char_p, _Z]),
+    "shdw_host_backend_keys": (_I, [ctypes.c_char_p, _Z]),
+    "shdw_host_network_create": (_V, [ctypes.c_char_p, _I, _I, ctypes.c_char_p, _V]),
+    "shdw_host_network_destroy": (None, [_V]),
+    "shdw_host_network_io": (_I, [_V, _I, ctypes.c_char_p, _Z]),
+    "shdw_host_network_forward": (_I, [_V, _I, ctypes.POINTER(ctypes.c_char_p), c_void_pp, c_int_p, c_int_p]),
+    "shdw_host_network_blob_shape": (_I, [_V, ctypes.c_char_p, c_int_p, _I]),
+    "shdw_host_network_blob_get": (_I, [_V, ctypes.c_char_p, c_float_p, _I]),
     "shdw_host_probe_create_kernel": (_I, [ctypes.c_char_p, _I]),
     "shdw_host_probe_argument": (_I, [ctypes.c_char_p, ctypes.c_char_p]),
 }
@@ -315,3 +323,76 @@ class Op:
         if self.ptr:
             self.ws.lib.shdw_host_op_destroy(self.ptr)
             self.ptr = None
+
+
+def parse_net(proto_text):
+    """Canonical spelling of a text model as the C++ parser understood it (host only)."""
+    lib = host()
+    buf = ctypes.create_string_buffer(max(4096, 4 * len(proto_text) + 1024))
+    n = lib.shdw_host_parse_net(proto_text.encode(), buf, len(buf))
+    host_check(n >= 0)
+    return buf.value.decode()
+
+
+class Network:
+    """Shadow::Network over the Native backend: a text model plus packed float32
+    weights (declared-blob order), run with host inputs."""
+
+    def __init__(self, proto_text, weights=None, backend_type="Native", device_id=0, debug=False):
+        self.lib = host()
+        packed = None
+        if weights is not None and len(weights):
+            packed = np.concatenate([np.ascontiguousarray(w, np.float32).ravel() for w in weights])
+        self.ptr = self.lib.shdw_host_network_create(
+            backend_type.encode(), device_id, int(debug), proto_text.encode(),
+            packed.ctypes.data if packed is not None else None)
+        host_check(self.ptr)
+
+    def _names(self, which):
+        buf = ctypes.create_string_buffer(8192)
+        host_check(self.lib.shdw_host_network_io(self.ptr, which, buf, len(buf)) >= 0)
+        text = buf.value.decode()
+        return text.split("\n") if text else []
+
+    @property
+    def in_blob(self):
+        return self._names(0)
+
+    @property
+    def out_blob(self):
+        return self._names(1)
+
+    def forward(self, inputs, reshape=False):
+        """inputs: {blob name: float32 array}.  reshape=True passes each array's
+        shape along, so the input blob is reshaped before the copy."""
+        names = list(inputs)
+        arrays = [np.ascontiguousarray(inputs[k], np.float32) for k in names]
+        c_names = (ctypes.c_char_p * len(names))(*[k.encode() for k in names])
+        c_data = (ctypes.c_void_p * len(names))(*[a.ctypes.data for a in arrays])
+        ranks = ints([a.ndim if reshape else 0 for a in arrays])
+        dims = ints([d for a in arrays for d in (a.shape if reshape else ())])
+        host_check(self.lib.shdw_host_network_forward(self.ptr, len(names), c_names, c_data, ranks, dims) == 0)
+
+    def blob_shape(self, name):
+        shape = (ctypes.c_int * 16)()
+        rank = self.lib.shdw_host_network_blob_shape(self.ptr, name.encode(), shape, 16)
+        host_check(rank >= 0)
+        return [shape[i] for i in range(rank)]
+
+    def blob(self, name):
+        shape = self.blob_shape(name)
+        out = np.empty(int(np.prod(shape, dtype=np.int64)) if shape else 1, np.float32)
+        host_check(self.lib.shdw_host_network_blob_get(
+            self.ptr, name.encode(), out.ctypes.data_as(c_float_p), out.size) == 0)
+        return out.reshape(shape)
+
+    def close(self):
+        if self.ptr:
+            self.lib.shdw_host_network_destroy(self.ptr)
+            self.ptr = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()

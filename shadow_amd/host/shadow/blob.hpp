@@ -91,6 +91,14 @@ class Blob {
     allocator_->read(get_count * elem_size(), data<T>() + offset, cpu_data);
   }
 
+  // set_data for callers that do not know the element type statically: copies
+  // raw_size() bytes from the host.
+  void set_raw_data(const void* cpu_data) {
+    CHECK_NOTNULL(cpu_data);
+    CHECK_NOTNULL(data_);
+    allocator_->write(raw_size(), cpu_data, data_);
+  }
+
   // Alias memory owned by someone else; this blob will never free it.
   void share_data(const void* data, const VecInt& shape) {
     CHECK_NOTNULL(data);

@@ -1,0 +1,45 @@
+// The Native backend: blobs and operators of a NetParam on one Workspace, run
+// in file order.  Behaviour of shadow/backends/native/native.{hpp,cpp}; model
+// sources are a NetParam or the converter's text form plus a weight buffer
+// (protobuf files are not read by this build).
+#ifndef SHADOW_AMD_HOST_NATIVE_HPP_
+#define SHADOW_AMD_HOST_NATIVE_HPP_
+
+#include "backend.hpp"
+#include "operator.hpp"
+
+namespace Shadow {
+
+class Native : public Backend {
+ public:
+  // Arguments: backend_type, device_id, default_cuda_stream (Workspace);
+  // device_input (Run takes device pointers), debug (log every operator).
+  explicit Native(const ArgumentHelper& arguments);
+
+  void LoadModel(const shadow::NetParam& net_param) override;
+  // proto_text: the text form.  Weights follow the order of the declared blobs:
+  // one pointer per blob, or one packed buffer (each blob's raw_size() bytes).
+  void LoadModel(const std::string& proto_text, const std::vector<const void*>& weights);
+  void LoadModel(const std::string& proto_text, const void* weights_data);
+
+  void Run(const std::map<std::string, void*>& data_map,
+           const std::map<std::string, std::vector<int>>& shape_map) override;
+
+ private:
+  void Initial(const shadow::NetParam& net_param);
+  void SetInputData(const std::string& blob_name, const std::vector<int>& blob_shape,
+                    const void* blob_data);
+  // Returns the blob's size in bytes.  share_data aliases the caller's (device)
+  // memory instead of copying.
+  size_t SetWeightData(const std::string& blob_name, const std::vector<int>& blob_shape,
+                       const void* blob_data, bool share_data);
+  void CopyWeights(const shadow::NetParam& net_param, const std::vector<const void*>& weights);
+  void CopyWeights(const shadow::NetParam& net_param, const void* weights_data);
+
+  bool device_input_ = false, debug_ = false;
+  std::vector<std::shared_ptr<Operator>> ops_;
+};
+
+}  // namespace Shadow
+
+#endif  // SHADOW_AMD_HOST_NATIVE_HPP_

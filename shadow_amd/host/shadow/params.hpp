@@ -84,10 +84,47 @@ class OpParam {
   std::vector<Argument> arg_;
 };
 
+// A blob declared by a model: name, element type ("float" when absent), shape
+// and optionally its contents (shadow/core/params.hpp:54-98).
+class Blob {
+ public:
+  const std::string& name() const { return name_; }
+  void set_name(const std::string& v) { name_ = v; }
+  bool has_type() const { return has_type_; }
+  const std::string& type() const { return type_; }
+  void set_type(const std::string& v) { type_ = v, has_type_ = true; }
+
+  const std::vector<int>& shape() const { return shape_; }
+  void add_shape(int v) { shape_.push_back(v); }
+  int shape_size() const { return static_cast<int>(shape_.size()); }
+
+  const std::vector<float>& data_f() const { return data_f_; }
+  void add_data_f(float v) { data_f_.push_back(v); }
+  int data_f_size() const { return static_cast<int>(data_f_.size()); }
+  const std::vector<std::vector<char>>& data_b() const { return data_b_; }
+  const std::vector<char>& data_b(int i) const { return data_b_[i]; }
+  void add_data_b(const std::vector<char>& v) { data_b_.push_back(v); }
+  int data_b_size() const { return static_cast<int>(data_b_.size()); }
+
+ private:
+  std::string name_{"None"}, type_{"None"};
+  bool has_type_ = false;
+  std::vector<int> shape_;
+  std::vector<float> data_f_;
+  std::vector<std::vector<char>> data_b_;
+};
+
 class NetParam {
  public:
   const std::string& name() const { return name_; }
   void set_name(const std::string& v) { name_ = v; }
+  const std::vector<Blob>& blob() const { return blob_; }
+  const Blob& blob(int i) const { return blob_[i]; }
+  Blob* add_blob() {
+    blob_.emplace_back();
+    return &blob_.back();
+  }
+  int blob_size() const { return static_cast<int>(blob_.size()); }
   const std::vector<OpParam>& op() const { return op_; }
   const OpParam& op(int i) const { return op_[i]; }
   OpParam* add_op() {
@@ -103,6 +140,7 @@ class NetParam {
 
  private:
   std::string name_;
+  std::vector<Blob> blob_;
   std::vector<OpParam> op_;
   std::vector<Argument> arg_;
 };

@@ -5,11 +5,15 @@
 // Operator::Run.  Every function catches the std::runtime_error that a failed
 // CHECK throws and reports it through shdw_host_last_error().
 #include <cstring>
+#include <map>
+#include <memory>
 #include <string>
 #include <vector>
 
 #include "shadow/kernel.hpp"
+#include "shadow/network.hpp"
 #include "shadow/operator.hpp"
+#include "shadow/parser.hpp"
 #include "shadow/workspace.hpp"
 
 using namespace Shadow;
@@ -174,6 +178,97 @@ int shdw_host_op_debug_log(void* ws, void* op, char* buf, size_t n) {
     len = join({oper->debug_log(inputs, outputs)}, buf, n);
   });
   return len;
+}
+
+// ---- models: the text form, and a Network over the Native backend ----
+
+// Host-only.  Parses the text and writes its canonical spelling; returns the
+// length, or -1 when the text is malformed.
+int shdw_host_parse_net(const char* proto_text, char* buf, size_t n) {
+  int len = -1;
+  guarded([&] {
+    shadow::NetParam net;
+    Parser::ParseNet(proto_text, &net);
+    len = join({Parser::DumpNet(net)}, buf, n);
+  });
+  return len;
+}
+
+int shdw_host_backend_keys(char* buf, size_t n) { return join(BackendRegistry()->Keys(), buf, n); }
+
+// weights: one packed host buffer in declared-blob order, or NULL when the
+// model declares no blobs.  NULL on error.
+void* shdw_host_network_create(const char* backend_type, int device_id, int debug,
+                               const char* proto_text, const void* weights) {
+  Network* net = nullptr;
+  guarded([&] {
+    ArgumentHelper args;
+    args.AddSingleArgument<std::string>("backend_type", backend_type ? backend_type : "");
+    args.AddSingleArgument<int>("device_id", device_id);
+    args.AddSingleArgument<bool>("debug", debug != 0);
+    std::unique_ptr<Network> made(new Network());
+    made->LoadXModel(std::string(proto_text ? proto_text : ""), weights, args);
+    made->backend()->ws()->Ctx()->synchronize();  // the weight buffer may go away after return
+    net = made.release();
+  });
+  return net;
+}
+
+void shdw_host_network_destroy(void* net) { delete static_cast<Network*>(net); }
+
+// which: 0 = input blob names, 1 = output blob names (newline separated)
+int shdw_host_network_io(void* net, int which, char* buf, size_t n) {
+  int len = -1;
+  guarded([&] {
+    auto* nw = static_cast<Network*>(net);
+    len = join(which == 0 ? nw->in_blob() : nw->out_blob(), buf, n);
+  });
+  return len;
+}
+
+// count inputs: names[i] -> host data[i]; ranks[i] > 0 reshapes that input
+// first with the next ranks[i] entries of `shapes`.
+int shdw_host_network_forward(void* net, int count, const char* const* names, void* const* data,
+                              const int* ranks, const int* shapes) {
+  return guarded([&] {
+    std::map<std::string, void*> data_map;
+    std::map<std::string, std::vector<int>> shape_map;
+    const int* cursor = shapes;
+    for (int i = 0; i < count; ++i) {
+      data_map[names[i]] = data[i];
+      const int rank = ranks != nullptr ? ranks[i] : 0;
+      if (rank > 0) {
+        shape_map[names[i]] = std::vector<int>(cursor, cursor + rank);
+        cursor += rank;
+      }
+    }
+    static_cast<Network*>(net)->Forward(data_map, shape_map);
+  });
+}
+
+int shdw_host_network_blob_shape(void* net, const char* name, int* shape, int max_rank) {
+  int rank = -1;
+  guarded([&] {
+    auto* nw = static_cast<Network*>(net);
+    CHECK(nw->backend()->ws()->HasBlob(name)) << "Unknown blob: " << name;
+    const auto dims = nw->GetBlobShapeByName(name);
+    rank = static_cast<int>(dims.size());
+    for (int n = 0; n < rank && n < max_rank; ++n) shape[n] = dims[n];
+  });
+  return rank;
+}
+
+// float blobs only
+int shdw_host_network_blob_get(void* net, const char* name, float* out, int count) {
+  return guarded([&] {
+    auto* nw = static_cast<Network*>(net);
+    auto blob = nw->backend()->ws()->GetBlob(name);
+    CHECK_NOTNULL(blob) << "Unknown blob: " << name;
+    CHECK_LE(count, blob->count());
+    const float* host = nw->GetBlobDataByName<float>(name, "host");
+    nw->backend()->ws()->Ctx()->synchronize();
+    std::memcpy(out, host, sizeof(float) * static_cast<size_t>(count));
+  });
 }
 
 // Host-only probes of ArgumentHelper / CreateKernel / CreateOperator error paths

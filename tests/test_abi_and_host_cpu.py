@@ -112,7 +112,9 @@ def test_registries_hold_exactly_the_gpu_default_kernels():
     kernels = ["Activate", "Axpy", "BatchNorm", "Binary", "Eltwise", "GroupNorm", "LayerNorm", "Normalize",
                "Pooling", "Reduce", "Scale", "Softmax", "Unary"]
     # InstanceNorm runs on the GroupNorm kernel (shadow/operators/instance_norm_op.cpp:14)
-    assert keys(h.shdw_host_operator_keys) == sorted(kernels + ["InstanceNorm"])
+    # and the view-only operators need no kernel
+    assert keys(h.shdw_host_operator_keys) == sorted(
+        kernels + ["InstanceNorm", "Input", "Reshape", "Flatten", "Squeeze", "Unsqueeze"])
     kk = keys(h.shdw_host_kernel_keys)
     assert kk == ["%sGPU(Default)" % t for t in kernels]
     # a CUDNN flavour would outrank Default; a CPU kernel would be a compute fallback
