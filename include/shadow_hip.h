@@ -290,6 +290,60 @@ int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
                         const float* scale, const float* bias, int scale_num, int scale_inner,
                         float* y, void* stream);
 
+/* =============================== data movers =============================== */
+
+/* dst[n*dst_pitch + dst_offset + p] = src[n*src_pitch + src_offset + p] for
+ * n < outer, p < chunk (a chunk must lie inside its row on both sides).  One
+ * call per input of Concat / per output of Slice / per input of Stack:
+ *   Concat: outer = num_concats, chunk = src_pitch = in_axis*concat_size,
+ *           dst_pitch = out_axis*concat_size, dst_offset = offset_axis*concat_size
+ *   Slice : chunk = dst_pitch = out_axis*slice_size, src_pitch = in_axis*slice_size,
+ *           src_offset = offset_axis*slice_size
+ *   Stack : chunk = src_pitch = stack_size, dst_pitch = out_axis*stack_size,
+ *           dst_offset = n*stack_size
+ * ref: shadow/operators/kernels/concat.cpp:5-16, slice.cpp:5-16, stack.cpp:5-14,
+ *      concat.cu:7-33, slice.cu:7-32, stack.cu:7-30 */
+int shdw_hip_copy_chunks(int outer, int chunk, const float* src, int src_pitch, int src_offset,
+                         float* dst, int dst_pitch, int dst_offset, void* stream);
+
+/* x viewed as [outer_num][gather_dim][inner_num] -> y [outer_num][num_indexes][inner_num],
+ * y[o][k][:] = x[o][indexes[k]][:].  indexes is a DEVICE array of int32; an entry
+ * outside [0, gather_dim) gives zeros (the reference reads out of bounds).
+ * ref: shadow/operators/kernels/gather.cpp:5-17, gather.cu:7-30 */
+int shdw_hip_gather(int outer_num, int gather_dim, int inner_num, int num_indexes,
+                    const int* indexes, const float* x, float* y, void* stream);
+
+/* Channel c moves to (c % (channel/group)) * group + c / (channel/group).
+ * ref: shadow/operators/kernels/shuffle_channel.cpp:5-21, shuffle_channel.cu:7-33 */
+int shdw_hip_shuffle_channel(int batch, int channel, int spatial_dim, int group, const float* x,
+                             float* y, void* stream);
+
+/* Pads (positive) or crops (negative) the two trailing axes of [N][C][H][W];
+ * paddings = top, bottom, left, right (HOST array of 4), new cells take `value`.
+ * One pass; the reference fills the output with Blas::Set first.
+ * ref: shadow/operators/kernels/pad.cpp:5-32, pad.hpp:24-40, pad.cu:7-43 */
+int shdw_hip_pad(const int* in_shape, const int* paddings, float value, const float* x, float* y,
+                 void* stream);
+
+/* y = x with axes permuted: out axis j is in axis order[j] (HOST arrays, up to 8
+ * axes).  The step tables the reference uploads per call are kernel arguments.
+ * ref: shadow/operators/kernels/permute.cpp:5-20, permute.hpp:26-52, permute.cu:7-31 */
+int shdw_hip_permute(int num_axes, const int* in_shape, const int* order, const float* x, float* y,
+                     void* stream);
+
+/* [N][C][H][W] -> [N][C*s*s][H/s][W/s]; type 0 = Darknet's index order, 1 = natural.
+ * ref: shadow/operators/kernels/reorg.cpp:5-72, reorg.cu:7-75 */
+int shdw_hip_reorg(const int* in_shape, int type, int stride, const float* x, float* y,
+                   void* stream);
+
+/* Resize of the two trailing axes; type 0 = nearest, 1 = bilinear (align_corners
+ * as in the reference; half-pixel centres otherwise).  Coordinates and weights
+ * are computed in fp32 in the reference's operation order, no fused operations.
+ * SHDW_E_UNSUPPORTED for align_corners with a single output row or column.
+ * ref: shadow/operators/kernels/resize.cpp:5-78, resize.cu:7-92 */
+int shdw_hip_resize(const int* in_shape, const int* out_shape, int type, int align_corners,
+                    const float* x, float* y, void* stream);
+
 /* ============================ plan inspection ============================ */
 
 /* Host-only: the collapsed form shdw_hip_broadcast_binary would launch with.

@@ -455,3 +455,173 @@ def layer_norm_op(x, normalized_shape, eps=1e-5, scale=None, bias=None):
         _check(list(np.shape(bias)) == ns, "bias->shape() == normalized_shape")
         out = scale_bias(out, _f(scale).ravel(), _f(bias).ravel(), inner, 1)
     return out.reshape(x.shape)
+
+
+# --------------------------------------------------------------------------
+# data movers (operator level; the kernel classes' loops over inputs / outputs
+# are folded in)
+# --------------------------------------------------------------------------
+def _count(shape, start=0, end=None):
+    return int(np.prod(list(shape)[start:end], dtype=np.int64))
+
+
+def concat_op(inputs, axis=1):
+    """shadow/operators/concat_op.cpp:18-40 and kernels/concat.hpp:24-40"""
+    inputs = [_f(x) for x in inputs]
+    _check(len(inputs) >= 2, "inputs.size() >= 2")
+    first = inputs[0]
+    axis = _canonical(axis, first.ndim)
+    out_shape = list(first.shape)
+    for x in inputs[1:]:
+        _check(x.ndim == first.ndim, "Inputs must have the same axes!")
+        for d in range(first.ndim):
+            if d != axis:
+                _check(x.shape[d] == first.shape[d], "Inputs must have the same shape, except at concat_axis!")
+        out_shape[axis] += x.shape[axis]
+    out = np.empty(_count(out_shape), np.float32)
+    num_concats, concat_size, offset = _count(out_shape, 0, axis), _count(out_shape, axis + 1), 0
+    for x in inputs:
+        lib().orc_concat(_p(x), num_concats, concat_size, out_shape[axis], x.shape[axis], offset, _p(out))
+        offset += x.shape[axis]
+    return out.reshape(out_shape)
+
+
+def slice_op(x, num_outputs, axis=1, slice_point=()):
+    """shadow/operators/slice_op.cpp:20-55 and kernels/slice.hpp:24-40"""
+    x = _f(x)
+    _check(num_outputs >= 2, "outputs.size() >= 2")
+    axis = _canonical(axis, x.ndim)
+    extent = x.shape[axis]
+    if not slice_point:
+        _check(extent % num_outputs == 0, "in_slice_axis % num_outputs == 0")
+        slices = [extent // num_outputs] * num_outputs
+    else:
+        _check(len(slice_point) == num_outputs - 1, "slice_point_.size() == num_outputs - 1")
+        slices, prev = [], 0
+        for point in slice_point:
+            _check(point > prev, "point > prev")
+            slices.append(point - prev)
+            prev = point
+        _check(extent > prev, "in_slice_axis > prev")
+        slices.append(extent - prev)
+    outs, offset = [], 0
+    num_slices, slice_size = _count(x.shape, 0, axis), _count(x.shape, axis + 1)
+    for width in slices:
+        shape = list(x.shape)
+        shape[axis] = width
+        out = np.empty(_count(shape), np.float32)
+        lib().orc_slice(_p(x), num_slices, slice_size, extent, width, offset, _p(out))
+        outs.append(out.reshape(shape))
+        offset += width
+    return outs
+
+
+def stack_op(inputs, axis=0):
+    """shadow/operators/stack_op.cpp:18-37 and kernels/stack.hpp:23-36"""
+    inputs = [_f(x) for x in inputs]
+    _check(len(inputs) >= 2, "inputs.size() >= 2")
+    rank = inputs[0].ndim
+    _check(-(rank + 1) <= axis < rank + 1, "axis out of bound.")
+    if axis < 0:
+        axis += rank + 1
+    out_shape = list(inputs[0].shape)
+    out_shape.insert(axis, len(inputs))
+    out = np.empty(_count(out_shape), np.float32)
+    num_stacks, stack_size = _count(out_shape, 0, axis), _count(out_shape, axis + 1)
+    for n, x in enumerate(inputs):
+        lib().orc_stack(_p(x), num_stacks, stack_size, len(inputs), n, _p(out))
+    return out.reshape(out_shape)
+
+
+def gather_op(x, axis=0, indexes=()):
+    """shadow/operators/gather_op.cpp:20-48 and kernels/gather.hpp:25-34"""
+    x = _f(x)
+    axis = _canonical(axis, x.ndim)
+    idx = np.ascontiguousarray(indexes, np.int32).ravel()
+    _check(idx.size > 0, "num_indexes > 0")
+    out_shape = list(x.shape)
+    out_shape[axis] = idx.size
+    out = np.empty(_count(out_shape), np.float32)
+    lib().orc_gather(_p(x), idx.ctypes.data_as(_i32p), idx.size, x.shape[axis], _count(x.shape, axis + 1),
+                     out.size, _p(out))
+    return out.reshape(out_shape)
+
+
+def pad_op(x, paddings, value=0.0):
+    """shadow/operators/pad_op.cpp:11-37 and kernels/pad.hpp:24-40"""
+    x = _f(x)
+    paddings = [int(p) for p in paddings]
+    _check(len(paddings) == 4, "paddings_.size() == 4")
+    out_shape = list(x.shape)
+    out_shape[2] += paddings[0] + paddings[1]
+    out_shape[3] += paddings[2] + paddings[3]
+    _check(min(out_shape) > 0, "output extents > 0")
+    if not any(paddings):
+        return copy(x.ravel()).reshape(x.shape)
+    out = np.empty(_count(out_shape), np.float32)
+    lib().orc_pad(_p(x), _ints(x.shape), _ints(paddings), _ints(out_shape), ctypes.c_float(value), _p(out))
+    return out.reshape(out_shape)
+
+
+def permute_op(x, order):
+    """shadow/operators/permute_op.cpp:17-33 and kernels/permute.hpp:26-52"""
+    x = _f(x)
+    order = [int(o) for o in order]
+    _check(len(order) == x.ndim, "input->num_axes() == order_value_.size()")
+    out_shape = [x.shape[a] for a in order]
+    old_steps = [_count(x.shape, d + 1) for d in range(x.ndim)]
+    new_steps = [_count(out_shape, d + 1) for d in range(x.ndim)]
+    out = np.empty(x.size, np.float32)
+    lib().orc_permute(_p(x), x.size, x.ndim, _ints(order), _ints(old_steps), _ints(new_steps), _p(out))
+    return out.reshape(out_shape)
+
+
+def reorg_op(x, type=0, stride=2):
+    """shadow/operators/reorg_op.cpp:19-41"""
+    x = _f(x)
+    c, h, w = x.shape[1:4]
+    if type == 0:
+        _check(c % (stride * stride) == 0, "in_c % (stride * stride) == 0")
+    _check(h % stride == 0 and w % stride == 0, "in_h, in_w % stride == 0")
+    out_shape = [x.shape[0], c * stride * stride, h // stride, w // stride]
+    out = np.empty(x.size, np.float32)
+    _check(lib().orc_reorg(_p(x), _ints(x.shape), int(type), int(stride), _p(out)) == 0, "Unsupported reorg type")
+    return out.reshape(out_shape)
+
+
+def shuffle_channel_op(x, group):
+    """shadow/operators/shuffle_channel_op.cpp:9-32"""
+    x = _f(x)
+    _check(group > 0, "group must be larger than 0")
+    _check(x.shape[1] % group == 0, "input->shape(1) % group == 0")
+    out = np.empty(x.size, np.float32)
+    lib().orc_shuffle_channel(_p(x), x.shape[0], x.shape[1], _count(x.shape, 2), int(group), _p(out))
+    return out.reshape(x.shape)
+
+
+def resize_op(x, size=(0,), scale=(1.0,), type=1, align_corners=False):
+    """shadow/operators/resize_op.cpp:21-62 and kernels/resize.hpp:28-50"""
+    x = _f(x)
+    _check(0 <= type <= 1, "type in [0, 1]")
+    _check(x.ndim == 4, "Only support 2D Resize")
+
+    def expand(v):
+        v = list(v)
+        if len(v) == 1:
+            return v * 2
+        _check(len(v) == 2, "param.size() == num")
+        return v
+
+    size, scale = expand(size), expand(scale)
+    out_shape = list(x.shape)
+    for n in range(2):
+        out_shape[n + 2] = size[n] if size[n] > 0 else int(np.float32(x.shape[n + 2]) * np.float32(scale[n]))
+        _check(out_shape[n + 2] > 0, "out_shape > 0")
+    if out_shape[2:] == list(x.shape[2:]):
+        return copy(x.ravel()).reshape(x.shape)
+    out = np.empty(_count(out_shape), np.float32)
+    if type == 0:
+        lib().orc_resize_nearest(_p(x), _ints(x.shape), _ints(out_shape), _p(out))
+    else:
+        lib().orc_resize_bilinear(_p(x), _ints(x.shape), int(bool(align_corners)), _ints(out_shape), _p(out))
+    return out.reshape(out_shape)

@@ -247,6 +247,29 @@ def _run_op(op, blobs):
         oracle._check(len(x) in (1, 3), "inputs.size() == 3")
         sc, bi = (x[1], x[2]) if len(x) == 3 else (None, None)
         return oracle.layer_norm_op(x[0], _repeated(a, "normalized_shape"), _single(a, "eps", F(1e-5)), sc, bi)
+    if t == "Concat":
+        return oracle.concat_op(x, _single(a, "axis", 1))
+    if t == "Slice":
+        return oracle.slice_op(x[0], len(op["top"]), _single(a, "axis", 1), _repeated(a, "slice_point"))
+    if t == "Stack":
+        return oracle.stack_op(x, _single(a, "axis", 0))
+    if t == "Gather":
+        idx = _repeated(a, "indexes")
+        if not idx:
+            oracle._check(len(op["bottom"]) == 2, "inputs.size() == 2")
+            idx = np.asarray(blobs[op["bottom"][1]]).astype(np.int32).ravel()
+        return oracle.gather_op(x[0], _single(a, "axis", 0), idx)
+    if t == "Pad":
+        return oracle.pad_op(x[0], _repeated(a, "paddings"), _single(a, "value", F(0)))
+    if t == "Permute":
+        return oracle.permute_op(x[0], _repeated(a, "order"))
+    if t == "Reorg":
+        return oracle.reorg_op(x[0], _single(a, "type", 0), _single(a, "stride", 2))
+    if t == "ShuffleChannel":
+        return oracle.shuffle_channel_op(x[0], _single(a, "group", 0))
+    if t == "Resize":
+        return oracle.resize_op(x[0], _repeated(a, "size", [0]), _repeated(a, "scale", [F(1)]),
+                                _single(a, "type", 1), bool(_single(a, "align_corners", False)))
     if t == "Reshape":
         return x[0].reshape(reshape_shape(x[0].shape, _repeated(a, "shape"), _single(a, "axis", 0),
                                           _single(a, "num_axes", -1)))
@@ -266,8 +289,8 @@ def run(net, weights, inputs):
     oracle._check(len(weights) == len(net.get("blob", [])), "net_param.blob_size() == weights.size()")
     blobs = {}
     for (name, typ, shape), w in zip(net.get("blob", []), weights):
-        oracle._check(typ == "float", "float weights only in this oracle")
-        blobs[name] = np.asarray(w, F).reshape(shape)
+        oracle._check(typ in ("float", "int32"), "float and int32 blobs only in this oracle")
+        blobs[name] = np.asarray(w, F if typ == "float" else np.int32).reshape(shape)
     net_args = {name: value for name, _, value in net.get("arg", [])}
     oracle._check("out_blob" in net_args, "Network must have out_blob argument")
     seen_input = False
@@ -284,7 +307,10 @@ def run(net, weights, inputs):
         for b in op["bottom"]:
             oracle._check(b in blobs, op["name"] + ": Can not find input blob " + b)
         out = _run_op(op, blobs)
-        if out is not None:
+        if isinstance(out, list):  # Slice: one array per top
+            for top, part in zip(op["top"], out):
+                blobs[top] = np.asarray(part, F)
+        elif out is not None:
             oracle._check(len(op["top"]) >= 1, "an output blob")
             blobs[op["top"][0]] = np.asarray(out, F)
     return blobs

@@ -514,3 +514,178 @@ API void orc_normalize_rows(const float* in, int outer_num, int inner_num, float
   orc_divide_variance(out, variance, count, inner_num, eps, out);
   free(ones);
 }
+
+/* ======================================================================
+ * Data movers.
+ * ====================================================================== */
+
+/* ---- shadow/operators/kernels/concat.cpp:5-16  Vision::Concat (one input) ---- */
+API void orc_concat(const float* in, int num_concats, int concat_size, int out_concat_axis,
+                    int in_concat_axis, int offset_concat_axis, float* out) {
+  for (int n = 0; n < num_concats; ++n)
+    memcpy(out + (n * out_concat_axis + offset_concat_axis) * concat_size,
+           in + n * in_concat_axis * concat_size, (size_t)in_concat_axis * concat_size * sizeof(float));
+}
+
+/* ---- shadow/operators/kernels/slice.cpp:5-16  Vision::Slice (one output) ---- */
+API void orc_slice(const float* in, int num_slices, int slice_size, int in_slice_axis,
+                   int out_slice_axis, int offset_slice_axis, float* out) {
+  for (int n = 0; n < num_slices; ++n)
+    memcpy(out + n * out_slice_axis * slice_size,
+           in + (n * in_slice_axis + offset_slice_axis) * slice_size,
+           (size_t)out_slice_axis * slice_size * sizeof(float));
+}
+
+/* ---- shadow/operators/kernels/stack.cpp:5-14  Vision::Stack (one input) ---- */
+API void orc_stack(const float* in, int num_stacks, int stack_size, int out_stack_axis,
+                   int offset_stack_axis, float* out) {
+  for (int n = 0; n < num_stacks; ++n)
+    memcpy(out + (n * out_stack_axis + offset_stack_axis) * stack_size, in + n * stack_size,
+           (size_t)stack_size * sizeof(float));
+}
+
+/* ---- shadow/operators/kernels/gather.cpp:5-17  Vision::Gather ---- */
+API void orc_gather(const float* in, const int* indexes, int num_indexes, int gather_dim,
+                    int inner_num, int count, float* out) {
+  int gather_num = num_indexes * inner_num;
+  for (int i = 0; i < count; ++i) {
+    int gather_index = indexes[(i / inner_num) % num_indexes];
+    int in_index = (gather_index + i / gather_num * gather_dim) * inner_num + i % inner_num;
+    out[i] = in[in_index];
+  }
+}
+
+/* ---- shadow/operators/kernels/pad.cpp:5-32  Vision::Pad, after the Blas::Set fill of
+ *      shadow/operators/kernels/pad.hpp:33-36; paddings = top, bottom, left, right,
+ *      negative values crop ---- */
+API void orc_pad(const float* in, const int* in_shape, const int* paddings, const int* out_shape,
+                 float value, float* out) {
+  int batch = in_shape[0], channel = in_shape[1], in_h = in_shape[2], in_w = in_shape[3];
+  int out_h = out_shape[2], out_w = out_shape[3];
+  orc_set(batch * channel * out_h * out_w, value, out);
+  for (int b = 0; b < batch; ++b) {
+    for (int c = 0; c < channel; ++c) {
+      for (int h = 0; h < in_h; ++h) {
+        if (h + paddings[0] < 0 || h >= in_h + paddings[1]) continue;
+        int copy_w = in_w + (paddings[2] < 0 ? paddings[2] : 0) + (paddings[3] < 0 ? paddings[3] : 0);
+        int in_offset = ((b * channel + c) * in_h + h) * in_w;
+        int out_offset = ((b * channel + c) * out_h + h + paddings[0]) * out_w;
+        if (paddings[2] < 0) in_offset -= paddings[2];
+        else out_offset += paddings[2];
+        memcpy(out + out_offset, in + in_offset, (size_t)copy_w * sizeof(float));
+      }
+    }
+  }
+}
+
+/* ---- shadow/operators/kernels/permute.cpp:5-20  Vision::Permute with the step tables of
+ *      shadow/operators/kernels/permute.hpp:33-43 ---- */
+API void orc_permute(const float* in, int count, int num_axes, const int* order,
+                     const int* old_steps, const int* new_steps, float* out) {
+  for (int i = 0; i < count; ++i) {
+    int old_idx = 0, idx = i;
+    for (int j = 0; j < num_axes; ++j) {
+      old_idx += (idx / new_steps[j]) * old_steps[order[j]];
+      idx %= new_steps[j];
+    }
+    out[i] = in[old_idx];
+  }
+}
+
+/* ---- shadow/operators/kernels/reorg.cpp:5-72  type 0 darknet, 1 natural ---- */
+API int orc_reorg(const float* in, const int* in_shape, int type, int stride, float* out) {
+  int batch = in_shape[0], in_c = in_shape[1], in_h = in_shape[2], in_w = in_shape[3];
+  if (type == 0) {
+    int out_c = in_c / (stride * stride);
+    for (int b = 0; b < batch; ++b)
+      for (int c = 0; c < in_c; ++c)
+        for (int h = 0; h < in_h; ++h)
+          for (int w = 0; w < in_w; ++w) {
+            int c2 = c % out_c, offset = c / out_c;
+            int h2 = h * stride + offset / stride, w2 = w * stride + offset % stride;
+            int in_index = ((b * in_c + c) * in_h + h) * in_w + w;
+            int out_index = ((b * out_c + c2) * in_h * stride + h2) * in_w * stride + w2;
+            out[in_index] = in[out_index];
+          }
+  } else if (type == 1) {
+    int out_c = in_c * stride * stride, out_h = in_h / stride, out_w = in_w / stride;
+    for (int b = 0; b < batch; ++b)
+      for (int c = 0; c < out_c; ++c)
+        for (int h = 0; h < out_h; ++h)
+          for (int w = 0; w < out_w; ++w) {
+            int offset = c / stride, c2 = offset / stride;
+            int h2 = h * stride + offset % stride, w2 = w * stride + c % stride;
+            int in_index = ((b * in_c + c2) * in_h + h2) * in_w + w2;
+            int out_index = ((b * out_c + c) * out_h + h) * out_w + w;
+            out[out_index] = in[in_index];
+          }
+  } else {
+    return -1;
+  }
+  return 0;
+}
+
+/* ---- shadow/operators/kernels/shuffle_channel.cpp:5-21 ---- */
+API void orc_shuffle_channel(const float* in, int batch, int channel, int spatial_dim, int group,
+                             float* out) {
+  int num = channel * spatial_dim, group_column = channel / group;
+  for (int b = 0; b < batch; ++b, in += num, out += num)
+    for (int c = 0; c < channel; ++c) {
+      int c_out = (c % group_column) * group + c / group_column;
+      memcpy(out + c_out * spatial_dim, in + c * spatial_dim, (size_t)spatial_dim * sizeof(float));
+    }
+}
+
+/* ---- shadow/operators/kernels/resize.cpp:5-27  ResizeNearest2D ---- */
+API void orc_resize_nearest(const float* in, const int* in_shape, const int* out_shape, float* out) {
+  int outer_num = in_shape[0] * in_shape[1], in_h = in_shape[2], in_w = in_shape[3];
+  int out_h = out_shape[2], out_w = out_shape[3];
+  float fh = (float)in_h / out_h, fw = (float)in_w / out_w;
+  for (int n = 0; n < outer_num; ++n, in += in_h * in_w)
+    for (int h = 0; h < out_h; ++h) {
+      int src_h = (int)(h * fh);
+      for (int w = 0; w < out_w; ++w) {
+        int src_w = (int)(w * fw);
+        *out++ = in[src_h * in_w + src_w];
+      }
+    }
+}
+
+/* ---- shadow/operators/kernels/resize.cpp:29-78  ResizeBilinear2D ---- */
+API void orc_resize_bilinear(const float* in, const int* in_shape, int align_corners,
+                             const int* out_shape, float* out) {
+  int outer_num = in_shape[0] * in_shape[1], in_h = in_shape[2], in_w = in_shape[3];
+  int out_h = out_shape[2], out_w = out_shape[3];
+  float fh = align_corners ? (float)(in_h - 1) / (out_h - 1) : (float)in_h / out_h;
+  float fw = align_corners ? (float)(in_w - 1) / (out_w - 1) : (float)in_w / out_w;
+  for (int n = 0; n < outer_num; ++n, in += in_h * in_w) {
+    for (int h = 0; h < out_h; ++h) {
+      float src_h_f;
+      if (align_corners) {
+        src_h_f = h * fh;
+      } else {
+        src_h_f = (h + 0.5f) * fh - 0.5f;
+        src_h_f = src_h_f < 0 ? 0 : src_h_f;
+      }
+      int src_h_l = (int)src_h_f, src_h_h = src_h_l + 1;
+      if (src_h_l >= in_h - 1) src_h_h = src_h_l = in_h - 1;
+      float sh = src_h_f - src_h_l;
+      for (int w = 0; w < out_w; ++w) {
+        float src_w_f;
+        if (align_corners) {
+          src_w_f = w * fw;
+        } else {
+          src_w_f = (w + 0.5f) * fw - 0.5f;
+          src_w_f = src_w_f < 0 ? 0 : src_w_f;
+        }
+        int src_w_l = (int)src_w_f, src_w_h = src_w_l + 1;
+        if (src_w_l >= in_w - 1) src_w_h = src_w_l = in_w - 1;
+        float sw = src_w_f - src_w_l;
+        int i0 = src_h_l * in_w + src_w_l, i1 = src_h_h * in_w + src_w_l;
+        int i2 = src_h_l * in_w + src_w_h, i3 = src_h_h * in_w + src_w_h;
+        *out++ = (1 - sh) * (1 - sw) * in[i0] + sh * (1 - sw) * in[i1] + (1 - sh) * sw * in[i2] +
+                 sh * sw * in[i3];
+      }
+    }
+  }
+}

@@ -79,6 +79,13 @@ SIGNATURES = {
     "shdw_hip_normalize": (_I, [_I, _I, _I, _F, _F, _V, _V, _V]),
     "shdw_hip_pooling2d": (_I, [c_int_p, _I, _I, _I, _I, _I, _I, _I, c_int_p, _V, _V, _V]),
     "shdw_hip_pooling3d": (_I, [c_int_p, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, c_int_p, _V, _V, _V]),
+    "shdw_hip_copy_chunks": (_I, [_I, _I, _V, _I, _I, _V, _I, _I, _V]),
+    "shdw_hip_gather": (_I, [_I, _I, _I, _I, _V, _V, _V, _V]),
+    "shdw_hip_shuffle_channel": (_I, [_I, _I, _I, _I, _V, _V, _V]),
+    "shdw_hip_pad": (_I, [c_int_p, c_int_p, _F, _V, _V, _V]),
+    "shdw_hip_permute": (_I, [_I, c_int_p, c_int_p, _V, _V, _V]),
+    "shdw_hip_reorg": (_I, [c_int_p, _I, _I, _V, _V, _V]),
+    "shdw_hip_resize": (_I, [c_int_p, c_int_p, _I, _I, _V, _V, _V]),
     "shdw_hip_plan_broadcast": (_I, [_I, c_int_p, c_int_p, c_int_p, c_int_p, c_int_p, c_int_p]),
     "shdw_hip_plan_reduce": (_I, [_I, c_int_p, _I, c_int_p, c_int_p, c_int_p, c_int_p, c_int_p, c_int_p]),
 }

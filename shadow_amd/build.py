@@ -31,7 +31,7 @@ HIP_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-HIP_SOURCES = ["elementwise.hip", "broadcast.hip", "reduce.hip", "fused.hip", "vision.hip", "softmax.hip", "norm.hip",
+HIP_SOURCES = ["elementwise.hip", "broadcast.hip", "reduce.hip", "fused.hip", "vision.hip", "softmax.hip", "norm.hip", "movers.hip",
                "runtime.hip"]
 # The reference's Release flags (CMakeLists.txt:30-37) plus contraction off so
 # that no host can fuse what baseline x86-64 does not.

@@ -1,0 +1,479 @@
+// Data movers: Concat / Slice / Stack (pitched chunk copies), Gather,
+// ShuffleChannel, Pad, Permute, Reorg, Resize.  No arithmetic except Resize's
+// interpolation weights; everything is bound by HBM traffic (4 bytes read and 4
+// written per output element).  Lanes are laid along the OUTPUT so stores are
+// always coalesced; where the input is contiguous in the same direction both
+// sides move as 128-bit vectors, and a transposing Permute goes through an LDS
+// tile so that both sides stay coalesced.
+#include <hip/hip_runtime.h>
+
+#include "../../include/shadow_hip.h"
+#include "device_common.h"
+#include "launch.h"
+#include "plan.h"
+
+#pragma clang fp contract(off)
+
+namespace shdw {
+
+// ---------------------------------------------------------------------------
+// dst[n * dst_pitch + dst_off + p] = src[n * src_pitch + src_off + p], p < chunk
+// ---------------------------------------------------------------------------
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void copy_chunks_kernel(const float* src, float* dst,
+                                                              uint32_t work, FastDiv f_chunk,
+                                                              uint32_t src_pitch, uint32_t src_off,
+                                                              uint32_t dst_pitch, uint32_t dst_off) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;  // element, or vector when VEC
+  if (i >= work) return;
+  uint32_t n, p;
+  fd_divmod(i, f_chunk, n, p);  // VEC: chunk, pitches and offsets are counted in vectors
+  const uint64_t s = static_cast<uint64_t>(n) * src_pitch + src_off + p;
+  const uint64_t d = static_cast<uint64_t>(n) * dst_pitch + dst_off + p;
+  if (VEC)
+    store4_stream(dst + 4 * d, load4_stream(src + 4 * s));
+  else
+    dst[d] = src[s];
+}
+
+// ---------------------------------------------------------------------------
+// Rows of `inner` elements picked by a table: Gather (device index table) and
+// ShuffleChannel (closed-form source row).
+// ---------------------------------------------------------------------------
+struct GatherRows {
+  const int* indexes;
+  FastDiv f_num;  // rows per outer slice on the output side
+  uint32_t gather_dim;
+  // source row of output row r, or -1 when the index is outside the input
+  SHDW_DEVICE int64_t source(uint32_t r) const {
+    uint32_t o, k;
+    fd_divmod(r, f_num, o, k);
+    const int g = indexes[k];
+    if (g < 0 || static_cast<uint32_t>(g) >= gather_dim) return -1;
+    return static_cast<int64_t>(o) * gather_dim + g;
+  }
+};
+
+struct ShuffleRows {
+  FastDiv f_channel, f_group;
+  uint32_t group_column;
+  SHDW_DEVICE int64_t source(uint32_t r) const {
+    uint32_t b, c_out;
+    fd_divmod(r, f_channel, b, c_out);
+    uint32_t q, m;
+    fd_divmod(c_out, f_group, q, m);  // c_out = q * group + m  <=>  c = m * group_column + q
+    return static_cast<int64_t>(b) * f_channel.d + m * group_column + q;
+  }
+};
+
+template <class MAP, bool VEC>
+__global__ __launch_bounds__(kBlock) void rows_pick_kernel(MAP map, const float* x, float* y,
+                                                            uint32_t work, FastDiv f_inner) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= work) return;
+  uint32_t r, p;
+  fd_divmod(i, f_inner, r, p);  // VEC: inner counted in vectors
+  const int64_t s = map.source(r);
+  if (VEC) {
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    store4_stream(y + 4ull * i, s < 0 ? zero : load4(x + 4 * (s * f_inner.d + p)));
+  } else {
+    y[i] = s < 0 ? 0.f : x[s * f_inner.d + p];
+  }
+}
+
+template <class MAP>
+static int launch_rows_pick(const MAP& map, int64_t rows, int inner, const float* x, float* y,
+                            hipStream_t st) {
+  if (inner % 4 == 0 && aligned16(x) && aligned16(y)) {
+    const uint32_t work = static_cast<uint32_t>(rows * (inner / 4));
+    rows_pick_kernel<MAP, true><<<grid_for(work), kBlock, 0, st>>>(map, x, y, work, make_fastdiv(inner / 4));
+  } else {
+    const uint32_t work = static_cast<uint32_t>(rows * inner);
+    rows_pick_kernel<MAP, false><<<grid_for(work), kBlock, 0, st>>>(map, x, y, work, make_fastdiv(inner));
+  }
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// Pad / crop of the two trailing axes; cells outside the input take `value`.
+// ---------------------------------------------------------------------------
+struct PadArgs {
+  int in_h, in_w, top, left;
+  FastDiv f_out_w, f_out_h;
+};
+
+__global__ __launch_bounds__(kBlock) void pad_kernel(const float* x, float* y, uint32_t n_out,
+                                                      PadArgs p, float value) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n_out) return;
+  uint32_t rest, wo, plane, ho;
+  fd_divmod(i, p.f_out_w, rest, wo);
+  fd_divmod(rest, p.f_out_h, plane, ho);
+  const int hi = static_cast<int>(ho) - p.top, wi = static_cast<int>(wo) - p.left;
+  const bool inside = hi >= 0 && hi < p.in_h && wi >= 0 && wi < p.in_w;
+  y[i] = inside ? x[(static_cast<uint64_t>(plane) * p.in_h + hi) * p.in_w + wi] : value;
+}
+
+// ---------------------------------------------------------------------------
+// Permute.  Generic: one output element per lane, source offset from the
+// collapsed dims.  Transposing form: dims collapsed to [batch][rows][cols] ->
+// [batch][cols][rows], 64 x 64 tiles through LDS.
+// ---------------------------------------------------------------------------
+struct PermuteArgs {
+  int ndim;
+  FastDiv f_out[kMaxDims];        // output extents, outermost first
+  uint32_t src_stride[kMaxDims];  // input stride of the axis each output dim walks
+};
+
+__global__ __launch_bounds__(kBlock) void permute_generic_kernel(const float* x, float* y, uint32_t n,
+                                                                  PermuteArgs p) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  uint32_t e = i, src = 0;
+  for (int k = p.ndim - 1; k >= 1; --k) {
+    uint32_t q, r;
+    fd_divmod(e, p.f_out[k], q, r);
+    src += r * p.src_stride[k];
+    e = q;
+  }
+  src += e * p.src_stride[0];
+  y[i] = x[src];
+}
+
+constexpr int kTile = 64;
+
+__global__ __launch_bounds__(kBlock) void transpose_kernel(const float* x, float* y, uint32_t rows,
+                                                            uint32_t cols, uint32_t tiles_c,
+                                                            FastDiv f_tiles) {
+  __shared__ float tile[kTile][kTile + 1];
+  uint32_t batch, t, tr, tc;
+  fd_divmod(blockIdx.x, f_tiles, batch, t);
+  tr = t / tiles_c, tc = t - tr * tiles_c;
+  const uint64_t plane = static_cast<uint64_t>(batch) * rows * cols;
+  const uint32_t lx = threadIdx.x & 63u, ly = threadIdx.x >> 6;  // 64 x 4 lanes
+  const uint32_t r0 = tr * kTile, c0 = tc * kTile;
+#pragma unroll 4
+  for (uint32_t k = ly; k < kTile; k += kBlock / kTile) {
+    const uint32_t r = r0 + k, c = c0 + lx;
+    if (r < rows && c < cols) tile[k][lx] = __builtin_nontemporal_load(x + plane + static_cast<uint64_t>(r) * cols + c);
+  }
+  __syncthreads();
+#pragma unroll 4
+  for (uint32_t k = ly; k < kTile; k += kBlock / kTile) {
+    const uint32_t c = c0 + k, r = r0 + lx;
+    if (r < rows && c < cols) y[plane + static_cast<uint64_t>(c) * rows + r] = tile[lx][k];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Reorg: a fixed index permutation between [B][C][H][W] and
+// [B][C*s*s][H/s][W/s] (natural) or Darknet's variant of it.
+// ---------------------------------------------------------------------------
+struct ReorgArgs {
+  int in_c, in_h, in_w, stride;
+  FastDiv f_w, f_h, f_c;  // extents of the index space the lanes walk
+  FastDiv f_stride, f_out_c;
+};
+
+template <bool DARKNET>
+__global__ __launch_bounds__(kBlock) void reorg_kernel(const float* x, float* y, uint32_t n, ReorgArgs p) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  uint32_t rest, w, h, b, c;
+  fd_divmod(i, p.f_w, rest, w);
+  fd_divmod(rest, p.f_h, rest, h);
+  fd_divmod(rest, p.f_c, b, c);
+  const uint32_t s = p.stride;
+  uint32_t src;
+  if (DARKNET) {
+    // lanes walk the input index space; the value comes from the "output" index
+    uint32_t offset, c2, oh, ow;
+    fd_divmod(c, p.f_out_c, offset, c2);
+    fd_divmod(offset, p.f_stride, oh, ow);
+    const uint32_t h2 = h * s + oh, w2 = w * s + ow;
+    src = ((b * p.f_out_c.d + c2) * p.in_h * s + h2) * p.in_w * s + w2;
+  } else {
+    uint32_t offset, cw, c2, oh;
+    fd_divmod(c, p.f_stride, offset, cw);
+    fd_divmod(offset, p.f_stride, c2, oh);
+    const uint32_t h2 = h * s + oh, w2 = w * s + cw;
+    src = ((b * p.in_c + c2) * p.in_h + h2) * p.in_w + w2;
+  }
+  y[i] = x[src];
+}
+
+// ---------------------------------------------------------------------------
+// Resize of the two trailing axes.
+// ---------------------------------------------------------------------------
+struct ResizeArgs {
+  int in_h, in_w;
+  float fh, fw;
+  FastDiv f_out_w, f_out_h;
+};
+
+__global__ __launch_bounds__(kBlock) void resize_nearest_kernel(const float* x, float* y, uint32_t n,
+                                                                 ResizeArgs p) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  uint32_t rest, w, plane, h;
+  fd_divmod(i, p.f_out_w, rest, w);
+  fd_divmod(rest, p.f_out_h, plane, h);
+  const float hf = static_cast<float>(static_cast<int>(h)) * p.fh;
+  const float wf = static_cast<float>(static_cast<int>(w)) * p.fw;
+  // h * (in / out) < in for every extent below 2^24; the clamp only guards larger ones
+  const int src_h = min(static_cast<int>(hf), p.in_h - 1), src_w = min(static_cast<int>(wf), p.in_w - 1);
+  y[i] = x[(static_cast<uint64_t>(plane) * p.in_h + src_h) * p.in_w + src_w];
+}
+
+// Source coordinate, its two neighbours and the weight of the upper one.
+template <bool ALIGN>
+SHDW_DEVICE void bilinear_axis(uint32_t o, float f, int extent, int& lo, int& hi, float& frac) {
+  float src;
+  if (ALIGN) {
+    src = static_cast<float>(static_cast<int>(o)) * f;
+  } else {
+    const float centre = static_cast<float>(static_cast<int>(o)) + 0.5f;
+    const float scaled = centre * f;
+    src = scaled - 0.5f;
+    src = src < 0 ? 0 : src;
+  }
+  lo = static_cast<int>(src);
+  hi = lo + 1;
+  if (lo >= extent - 1) hi = lo = extent - 1;
+  frac = src - static_cast<float>(lo);
+}
+
+template <bool ALIGN>
+__global__ __launch_bounds__(kBlock) void resize_bilinear_kernel(const float* x, float* y, uint32_t n,
+                                                                  ResizeArgs p) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  uint32_t rest, w, plane, h;
+  fd_divmod(i, p.f_out_w, rest, w);
+  fd_divmod(rest, p.f_out_h, plane, h);
+  int h_l, h_h, w_l, w_h;
+  float sh, sw;
+  bilinear_axis<ALIGN>(h, p.fh, p.in_h, h_l, h_h, sh);
+  bilinear_axis<ALIGN>(w, p.fw, p.in_w, w_l, w_h, sw);
+  const float* img = x + static_cast<uint64_t>(plane) * p.in_h * p.in_w;
+  const float v0 = img[h_l * p.in_w + w_l], v1 = img[h_h * p.in_w + w_l];
+  const float v2 = img[h_l * p.in_w + w_h], v3 = img[h_h * p.in_w + w_h];
+  // ((1-sh)(1-sw) v0 + sh(1-sw) v1) + (1-sh) sw v2) + sh sw v3, each product
+  // formed left to right and rounded, no fused operations
+  const float ih = 1 - sh, iw = 1 - sw;
+  const float a0 = ih * iw, a1 = sh * iw, a2 = ih * sw, a3 = sh * sw;
+  const float t0 = a0 * v0, t1 = a1 * v1, t2 = a2 * v2, t3 = a3 * v3;
+  const float s01 = t0 + t1;
+  const float s012 = s01 + t2;
+  y[i] = s012 + t3;
+}
+
+static bool count_fits(const int* shape, int n, int64_t* count) {
+  int64_t c = 1;
+  for (int k = 0; k < n; ++k) {
+    if (shape[k] < 0) return false;
+    c *= shape[k];
+    if (c > INT32_MAX) return false;
+  }
+  *count = c;
+  return true;
+}
+
+}  // namespace shdw
+
+using namespace shdw;
+
+extern "C" {
+
+int shdw_hip_copy_chunks(int outer, int chunk, const float* src, int src_pitch, int src_offset,
+                         float* dst, int dst_pitch, int dst_offset, void* stream) {
+  if (outer < 0 || chunk < 0 || src_offset < 0 || dst_offset < 0) return SHDW_E_INVALID_ARGUMENT;
+  if (static_cast<int64_t>(src_offset) + chunk > src_pitch ||
+      static_cast<int64_t>(dst_offset) + chunk > dst_pitch)
+    return SHDW_E_INVALID_ARGUMENT;  // a chunk must stay inside its row
+  if (static_cast<int64_t>(outer) * src_pitch > INT32_MAX ||
+      static_cast<int64_t>(outer) * dst_pitch > INT32_MAX)
+    return SHDW_E_INVALID_ARGUMENT;
+  if (outer == 0 || chunk == 0) return SHDW_OK;
+  if (!src || !dst) return SHDW_E_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec = ((chunk | src_pitch | src_offset | dst_pitch | dst_offset) & 3) == 0 &&
+                   aligned16(src) && aligned16(dst);
+  if (vec) {
+    const uint32_t work = static_cast<uint32_t>(outer) * (chunk / 4);
+    copy_chunks_kernel<true><<<grid_for(work), kBlock, 0, st>>>(
+        src, dst, work, make_fastdiv(chunk / 4), src_pitch / 4, src_offset / 4, dst_pitch / 4,
+        dst_offset / 4);
+  } else {
+    const uint32_t work = static_cast<uint32_t>(outer) * chunk;
+    copy_chunks_kernel<false><<<grid_for(work), kBlock, 0, st>>>(
+        src, dst, work, make_fastdiv(chunk), src_pitch, src_offset, dst_pitch, dst_offset);
+  }
+  return launch_status();
+}
+
+int shdw_hip_gather(int outer_num, int gather_dim, int inner_num, int num_indexes,
+                    const int* indexes, const float* x, float* y, void* stream) {
+  if (outer_num < 0 || gather_dim < 1 || inner_num < 0 || num_indexes < 1)
+    return SHDW_E_INVALID_ARGUMENT;
+  const int64_t rows = static_cast<int64_t>(outer_num) * num_indexes;
+  if (rows * inner_num > INT32_MAX || static_cast<int64_t>(outer_num) * gather_dim * inner_num > INT32_MAX)
+    return SHDW_E_INVALID_ARGUMENT;
+  if (rows * inner_num == 0) return SHDW_OK;
+  if (!indexes || !x || !y) return SHDW_E_INVALID_ARGUMENT;
+  GatherRows map{indexes, make_fastdiv(num_indexes), static_cast<uint32_t>(gather_dim)};
+  return launch_rows_pick(map, rows, inner_num, x, y, static_cast<hipStream_t>(stream));
+}
+
+int shdw_hip_shuffle_channel(int batch, int channel, int spatial_dim, int group, const float* x,
+                             float* y, void* stream) {
+  if (batch < 0 || channel < 1 || spatial_dim < 0 || group < 1 || channel % group != 0)
+    return SHDW_E_INVALID_ARGUMENT;
+  const int64_t rows = static_cast<int64_t>(batch) * channel;
+  if (rows * spatial_dim > INT32_MAX) return SHDW_E_INVALID_ARGUMENT;
+  if (rows * spatial_dim == 0) return SHDW_OK;
+  if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
+  ShuffleRows map{make_fastdiv(channel), make_fastdiv(group), static_cast<uint32_t>(channel / group)};
+  return launch_rows_pick(map, rows, spatial_dim, x, y, static_cast<hipStream_t>(stream));
+}
+
+int shdw_hip_pad(const int* in_shape, const int* paddings, float value, const float* x, float* y,
+                 void* stream) {
+  if (!in_shape || !paddings) return SHDW_E_INVALID_ARGUMENT;
+  int out_shape[4] = {in_shape[0], in_shape[1], in_shape[2] + paddings[0] + paddings[1],
+                      in_shape[3] + paddings[2] + paddings[3]};
+  int64_t in_count, out_count;
+  if (!count_fits(in_shape, 4, &in_count) || !count_fits(out_shape, 4, &out_count))
+    return SHDW_E_INVALID_ARGUMENT;
+  if (out_count == 0) return SHDW_OK;
+  if (!y || (in_count > 0 && !x)) return SHDW_E_INVALID_ARGUMENT;
+  PadArgs p{in_shape[2], in_shape[3], paddings[0], paddings[2], make_fastdiv(out_shape[3]),
+            make_fastdiv(out_shape[2])};
+  const uint32_t n = static_cast<uint32_t>(out_count);
+  pad_kernel<<<grid_for(n), kBlock, 0, static_cast<hipStream_t>(stream)>>>(x, y, n, p, value);
+  return launch_status();
+}
+
+int shdw_hip_permute(int num_axes, const int* in_shape, const int* order, const float* x, float* y,
+                     void* stream) {
+  if (num_axes < 1 || num_axes > kMaxDims || !in_shape || !order) return SHDW_E_INVALID_ARGUMENT;
+  int64_t count;
+  if (!count_fits(in_shape, num_axes, &count)) return SHDW_E_INVALID_ARGUMENT;
+  bool seen[kMaxDims] = {false};
+  for (int k = 0; k < num_axes; ++k) {
+    if (order[k] < 0 || order[k] >= num_axes || seen[order[k]]) return SHDW_E_INVALID_ARGUMENT;
+    seen[order[k]] = true;
+  }
+  if (count == 0) return SHDW_OK;
+  if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+
+  // Input strides; then output dims (extent, input stride), dropping extent-1
+  // dims and merging neighbours that are also neighbours in the input.
+  int64_t in_stride[kMaxDims];
+  in_stride[num_axes - 1] = 1;
+  for (int d = num_axes - 2; d >= 0; --d) in_stride[d] = in_stride[d + 1] * in_shape[d + 1];
+  int nd = 0;
+  int64_t ext[kMaxDims], str[kMaxDims];
+  for (int k = 0; k < num_axes; ++k) {
+    const int64_t e = in_shape[order[k]], s = in_stride[order[k]];
+    if (e == 1) continue;
+    if (nd > 0 && str[nd - 1] == s * e) {
+      ext[nd - 1] *= e;
+      str[nd - 1] = s;
+    } else {
+      ext[nd] = e, str[nd] = s, ++nd;
+    }
+  }
+  const uint32_t n = static_cast<uint32_t>(count);
+  if (nd <= 1) {  // the order keeps memory as it is
+    return shdw_hip_copy(static_cast<int>(count), x, y, stream);
+  }
+  // [batch][rows][cols] -> [batch][cols][rows]
+  const bool plain2 = nd == 2 && str[0] == 1 && str[1] == ext[0];
+  const bool batch3 = nd == 3 && str[1] == 1 && str[2] == ext[1] && str[0] == ext[1] * ext[2];
+  if (plain2 || batch3) {
+    const uint32_t batch = plain2 ? 1u : static_cast<uint32_t>(ext[0]);
+    const uint32_t cols = static_cast<uint32_t>(plain2 ? ext[0] : ext[1]);  // input's fast axis
+    const uint32_t rows = static_cast<uint32_t>(plain2 ? ext[1] : ext[2]);
+    const uint32_t tiles_r = (rows + kTile - 1) / kTile, tiles_c = (cols + kTile - 1) / kTile;
+    const int64_t groups = static_cast<int64_t>(batch) * tiles_r * tiles_c;
+    if (groups <= INT32_MAX) {
+      transpose_kernel<<<static_cast<uint32_t>(groups), kBlock, 0, st>>>(
+          x, y, rows, cols, tiles_c, make_fastdiv(tiles_r * tiles_c));
+      return launch_status();
+    }
+  }
+  PermuteArgs p;
+  p.ndim = nd;
+  for (int k = 0; k < nd; ++k) {
+    p.f_out[k] = make_fastdiv(static_cast<uint32_t>(ext[k]));
+    p.src_stride[k] = static_cast<uint32_t>(str[k]);
+  }
+  permute_generic_kernel<<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
+  return launch_status();
+}
+
+int shdw_hip_reorg(const int* in_shape, int type, int stride, const float* x, float* y,
+                   void* stream) {
+  if (!in_shape || stride < 1 || type < 0 || type > 1) return SHDW_E_INVALID_ARGUMENT;
+  int64_t count;
+  if (!count_fits(in_shape, 4, &count)) return SHDW_E_INVALID_ARGUMENT;
+  const int in_c = in_shape[1], in_h = in_shape[2], in_w = in_shape[3];
+  if (in_h % stride != 0 || in_w % stride != 0) return SHDW_E_INVALID_ARGUMENT;
+  if (type == 0 && in_c % (stride * stride) != 0) return SHDW_E_INVALID_ARGUMENT;
+  if (count == 0) return SHDW_OK;
+  if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint32_t n = static_cast<uint32_t>(count);
+  ReorgArgs p;
+  p.in_c = in_c, p.in_h = in_h, p.in_w = in_w, p.stride = stride;
+  p.f_stride = make_fastdiv(stride);
+  if (type == 0) {
+    p.f_w = make_fastdiv(in_w), p.f_h = make_fastdiv(in_h), p.f_c = make_fastdiv(in_c);
+    p.f_out_c = make_fastdiv(in_c / (stride * stride));
+    reorg_kernel<true><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
+  } else {
+    p.f_w = make_fastdiv(in_w / stride), p.f_h = make_fastdiv(in_h / stride);
+    p.f_c = make_fastdiv(in_c * stride * stride);
+    p.f_out_c = make_fastdiv(1);
+    reorg_kernel<false><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
+  }
+  return launch_status();
+}
+
+int shdw_hip_resize(const int* in_shape, const int* out_shape, int type, int align_corners,
+                    const float* x, float* y, void* stream) {
+  if (!in_shape || !out_shape || type < 0 || type > 1) return SHDW_E_INVALID_ARGUMENT;
+  int64_t in_count, out_count;
+  if (!count_fits(in_shape, 4, &in_count) || !count_fits(out_shape, 4, &out_count))
+    return SHDW_E_INVALID_ARGUMENT;
+  if (in_shape[0] != out_shape[0] || in_shape[1] != out_shape[1]) return SHDW_E_INVALID_ARGUMENT;
+  if (out_count == 0) return SHDW_OK;
+  if (in_count == 0 || !x || !y) return SHDW_E_INVALID_ARGUMENT;
+  const int in_h = in_shape[2], in_w = in_shape[3], out_h = out_shape[2], out_w = out_shape[3];
+  // align_corners divides by (out - 1): a single output row or column has no
+  // defined source coordinate (the reference computes 0 * inf there).
+  if (type == 1 && align_corners && (out_h < 2 || out_w < 2)) return SHDW_E_UNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint32_t n = static_cast<uint32_t>(out_count);
+  ResizeArgs p;
+  p.in_h = in_h, p.in_w = in_w;
+  p.f_out_w = make_fastdiv(out_w), p.f_out_h = make_fastdiv(out_h);
+  if (type == 1 && align_corners) {
+    p.fh = static_cast<float>(in_h - 1) / (out_h - 1);
+    p.fw = static_cast<float>(in_w - 1) / (out_w - 1);
+    resize_bilinear_kernel<true><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
+  } else {
+    p.fh = static_cast<float>(in_h) / out_h;
+    p.fw = static_cast<float>(in_w) / out_w;
+    if (type == 0)
+      resize_nearest_kernel<<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
+    else
+      resize_bilinear_kernel<false><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
+  }
+  return launch_status();
+}
+
+}  // extern "C"

@@ -109,8 +109,9 @@ def keys(fn):
 
 def test_registries_hold_exactly_the_gpu_default_kernels():
     h = shadow_amd.host()
-    kernels = ["Activate", "Axpy", "BatchNorm", "Binary", "Eltwise", "GroupNorm", "LayerNorm", "Normalize",
-               "Pooling", "Reduce", "Scale", "Softmax", "Unary"]
+    kernels = ["Activate", "Axpy", "BatchNorm", "Binary", "Concat", "Eltwise", "Gather", "GroupNorm", "LayerNorm",
+               "Normalize", "Pad", "Permute", "Pooling", "Reduce", "Reorg", "Resize", "Scale", "ShuffleChannel",
+               "Slice", "Softmax", "Stack", "Unary"]
     # InstanceNorm runs on the GroupNorm kernel (shadow/operators/instance_norm_op.cpp:14)
     # and the view-only operators need no kernel
     assert keys(h.shdw_host_operator_keys) == sorted(

@@ -1,0 +1,169 @@
+"""GPU parity of the data movers through Operator::Run: bit for bit against the
+oracle (pure index maps, and Resize whose fp32 weights are computed in the
+reference's operation order)."""
+import numpy as np
+import pytest
+
+import oracle
+import shadow_amd
+from shadow_amd import ShadowError
+from tests.helpers import assert_bit_exact, normal, with_specials
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+@pytest.fixture()
+def ws(gpu):
+    w = shadow_amd.Workspace("Native", 0)
+    yield w
+    w.close()
+
+
+def run(ws, op_type, inputs, args, tops=("out",)):
+    names = []
+    for name, arr in inputs:
+        ws.set_blob(name, arr, dtype="int32" if np.asarray(arr).dtype.kind == "i" else "float")
+        names.append(name)
+    op = ws.create_op(op_type, names, list(tops), args)
+    op.run()
+    got = [ws.get_blob(t) for t in tops]
+    return got[0] if len(got) == 1 else got
+
+
+@pytest.mark.parametrize("shapes,axis", [
+    ([(2, 3, 4, 5), (2, 7, 4, 5)], 1), ([(2, 3, 4, 8), (2, 3, 4, 4), (2, 3, 4, 12)], 3),
+    ([(3, 5), (2, 5), (4, 5)], 0), ([(2, 3, 7), (2, 3, 1)], -1), ([(4, 16, 14, 14), (4, 32, 14, 14)], 1),
+    ([(2, 3, 5, 5), (2, 3, 5, 5)], 2)])
+def test_concat_op(ws, shapes, axis):
+    xs = [normal(10 + k, s) for k, s in enumerate(shapes)]
+    got = run(ws, "Concat", [("x%d" % k, x) for k, x in enumerate(xs)], {"axis": axis})
+    want = oracle.concat_op(xs, axis)
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "concat")
+
+
+@pytest.mark.parametrize("shape,axis,points,n", [((2, 12, 4, 4), 1, [], 3), ((2, 12, 4, 4), 1, [4, 5], 3),
+                                                 ((6, 5), 0, [], 2), ((2, 3, 10), -1, [3], 2),
+                                                 ((4, 48, 7, 7), 1, [16, 32], 3)])
+def test_slice_op(ws, shape, axis, points, n):
+    x = normal(20, shape)
+    args = {"axis": axis}
+    if points:
+        args["slice_point"] = points
+    got = run(ws, "Slice", [("x", x)], args, tops=["o%d" % k for k in range(n)])
+    want = oracle.slice_op(x, n, axis, points)
+    for g, w in zip(got, want):
+        assert g.shape == w.shape
+        assert_bit_exact(g, w, "slice")
+
+
+@pytest.mark.parametrize("shape,axis,k", [((2, 3, 4), 0, 2), ((2, 3, 4), 1, 3), ((2, 3, 4), 3, 2), ((2, 3, 4), -1, 2),
+                                          ((5, 8), -2, 4), ((16, 64), 1, 3)])
+def test_stack_op(ws, shape, axis, k):
+    xs = [normal(30 + j, shape) for j in range(k)]
+    got = run(ws, "Stack", [("x%d" % j, x) for j, x in enumerate(xs)], {"axis": axis})
+    want = oracle.stack_op(xs, axis)
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "stack")
+
+
+@pytest.mark.parametrize("shape,axis,idx", [((5, 8), 0, [4, 0, 0, 2]), ((3, 6, 4), 1, [5, 1]), ((2, 3, 7), -1, [6, 0, 3]),
+                                            ((4, 10, 16), 1, [9, 8, 7, 0, 1, 2, 2])])
+def test_gather_op(ws, shape, axis, idx):
+    x = normal(40, shape)
+    want = oracle.gather_op(x, axis, idx)
+    got = run(ws, "Gather", [("x", x)], {"axis": axis, "indexes": idx})
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "gather by argument")
+    got = run(ws, "Gather", [("x", x), ("idx", np.asarray(idx, np.int32))], {"axis": axis}, tops=["out2"])
+    assert_bit_exact(got, want, "gather by blob")
+
+
+def test_gather_index_checks(ws):
+    x = normal(41, (4, 6))
+    ws.set_blob("x", x)
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("Gather", ["x"], ["o"], {"axis": 0, "indexes": [4]}).run()
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("Gather", ["x"], ["o1"], {"axis": 0}).run()
+    # a bad index in a device blob cannot be checked on the host: that row comes out as zeros
+    got = run(ws, "Gather", [("x", x), ("idx", np.asarray([1, 9, -1, 3], np.int32))], {"axis": 0}, tops=["o2"])
+    assert_bit_exact(got, np.stack([x[1], np.zeros(6, F), np.zeros(6, F), x[3]]), "out-of-range rows")
+
+
+@pytest.mark.parametrize("pads", [[1, 2, 3, 4], [0, 0, 0, 1], [-1, 2, 0, -2], [-1, -1, -1, -1], [2, -1, -2, 3],
+                                  [0, 0, 0, 0]])
+@pytest.mark.parametrize("shape", [(2, 3, 6, 7), (1, 2, 16, 16)])
+def test_pad_op(ws, pads, shape):
+    x = normal(50, shape)
+    got = run(ws, "Pad", [("x", x)], {"paddings": pads, "value": -2.5})
+    want = oracle.pad_op(x, pads, -2.5)
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "pad")
+
+
+@pytest.mark.parametrize("shape,order", [
+    ((2, 3, 4, 5), [0, 2, 3, 1]), ((2, 3, 4, 5), [0, 3, 1, 2]), ((2, 3, 4, 5), [3, 2, 1, 0]), ((4, 6), [1, 0]),
+    ((2, 3, 4), [0, 1, 2]), ((2, 3, 4, 5, 6), [4, 0, 3, 1, 2]), ((7,), [0]), ((2, 1, 3), [2, 1, 0]),
+    ((3, 130, 70), [0, 2, 1]), ((200, 131), [1, 0]), ((2, 64, 28, 28), [0, 2, 3, 1]), ((2, 5, 6, 7), [1, 0, 2, 3]),
+    ((2, 3, 4, 5), [0, 1, 3, 2]), ((1, 1, 9), [2, 0, 1])])
+def test_permute_op(ws, shape, order):
+    x = normal(60, shape)
+    got = run(ws, "Permute", [("x", x)], {"order": order})
+    want = oracle.permute_op(x, order)
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "permute")
+
+
+@pytest.mark.parametrize("type_", [0, 1])
+@pytest.mark.parametrize("shape,stride", [((2, 8, 6, 4), 2), ((1, 9, 6, 9), 3), ((2, 64, 26, 26), 2), ((1, 4, 2, 2), 1)])
+def test_reorg_op(ws, type_, shape, stride):
+    x = normal(70, shape)
+    got = run(ws, "Reorg", [("x", x)], {"type": type_, "stride": stride})
+    want = oracle.reorg_op(x, type_, stride)
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "reorg")
+
+
+@pytest.mark.parametrize("shape,group", [((2, 6, 3, 5), 2), ((2, 6, 3, 5), 3), ((1, 12, 4, 4), 4), ((3, 8, 1, 1), 8),
+                                         ((2, 116, 28, 28), 2), ((2, 6, 3, 5), 1)])
+def test_shuffle_channel_op(ws, shape, group):
+    x = normal(80, shape)
+    got = run(ws, "ShuffleChannel", [("x", x)], {"group": group})
+    assert_bit_exact(got, oracle.shuffle_channel_op(x, group), "shuffle")
+
+
+@pytest.mark.parametrize("args", [
+    {"scale": [2.0]}, {"scale": [2.0], "align_corners": True}, {"size": [9, 7]}, {"size": [9, 7], "align_corners": True},
+    {"size": [3, 5], "type": 0}, {"scale": [2.0], "type": 0}, {"scale": [0.5, 1.5]}, {"size": [4, 6]},
+    {"size": [2, 2], "align_corners": True}, {"size": [1, 5]}, {"scale": [3.0]}, {"size": [13], "type": 0}])
+@pytest.mark.parametrize("shape", [(2, 3, 4, 6), (1, 2, 17, 9)])
+def test_resize_op(ws, args, shape):
+    x = with_specials(normal(90, shape, 2.0), 90).reshape(shape)
+    got = run(ws, "Resize", [("x", x)], args)
+    want = oracle.resize_op(x, args.get("size", [0]), args.get("scale", [1.0]), args.get("type", 1),
+                            args.get("align_corners", False))
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "resize %s" % args)
+
+
+def test_mover_argument_errors(ws):
+    ws.set_blob("x", np.zeros((2, 6, 4, 4), F))
+    ws.set_blob("y", np.zeros((2, 6, 4, 5), F))
+    bad = [("Concat", ["x"], ["o0"], {}), ("Concat", ["x", "y"], ["o1"], {"axis": 1}),
+           ("Slice", ["x"], ["a", "b", "c", "d"], {"axis": 1}), ("Slice", ["x"], ["a2"], {"axis": 1}),
+           ("Slice", ["x"], ["a3", "b3"], {"axis": 1, "slice_point": [6]}),
+           ("Stack", ["x", "x"], ["o2"], {"axis": 5}), ("Stack", ["x", "y"], ["o3"], {"axis": 0}),
+           ("Pad", ["x"], ["o4"], {"paddings": [-2, -2, 0, 0]}), ("Permute", ["x"], ["o5"], {"order": [0, 1, 2]}),
+           ("Permute", ["x"], ["o6"], {"order": [0, 1, 1, 2]}), ("Reorg", ["x"], ["o7"], {"type": 0, "stride": 2}),
+           ("Reorg", ["x"], ["o8"], {"type": 2, "stride": 2}), ("Reorg", ["y"], ["o9"], {"type": 1, "stride": 2}),
+           ("ShuffleChannel", ["x"], ["o10"], {"group": 4}), ("Resize", ["x"], ["o11"], {"size": [1, 2, 3]}),
+           ("Resize", ["x"], ["o12"], {"scale": [0.1]}), ("Resize", ["x"], ["o13"], {"size": [1, 8], "align_corners": True}),
+           ("Permute", ["x"], ["x"], {"order": [0, 1, 2, 3]})]
+    for op_type, bottoms, tops, args in bad:
+        with pytest.raises(ShadowError):
+            ws.create_op(op_type, bottoms, tops, args).run()
+    for op_type, args in (("Pad", {"paddings": [1, 1]}), ("ShuffleChannel", {}), ("Resize", {"type": 2})):
+        with pytest.raises(ShadowError, match="Check Failed"):
+            ws.create_op(op_type, ["x"], ["oo"], args)
