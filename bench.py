@@ -360,6 +360,40 @@ def config_table(dev):
     ms = time_batch(dev, lambda k: lib.shdw_hip_group_norm(65536, 784, 1e-5, AH[k].ptr, lns.ptr, lnb.ptr,
                                                            784, 1, YH[k].ptr, st), SH, reps=20)
     add("next", "layer_norm affine [65536,784]", 8 * NH + 8 * 784, ms, NH)
+    # data movers ("movers") on the same 205 MB tensors
+    half = NH // 2
+    def concat2(k):
+        # two [64,128,56,56] halves -> [64,256,56,56] along axis 1
+        rc = lib.shdw_hip_copy_chunks(64, 128 * INH, AH[k].ptr, 128 * INH, 0, YH[k].ptr, 256 * INH, 0, st)
+        return rc or lib.shdw_hip_copy_chunks(64, 128 * INH, AH[(k + 1) % SH].ptr, 128 * INH, 0, YH[k].ptr,
+                                              256 * INH, 128 * INH, st)
+    ms = time_batch(dev, concat2, SH, reps=20)
+    add("movers", "concat 2x[64,128,56,56] axis 1 (2 launches)", 8 * NH, ms, NH)
+    shp4 = [64, 256, 56, 56]
+    ms = time_batch(dev, lambda k: lib.shdw_hip_permute(4, I(shp4), I([0, 2, 3, 1]), AH[k].ptr, YH[k].ptr, st),
+                    SH, reps=20)
+    add("movers", "permute NCHW->NHWC [64,256,56,56]", 8 * NH, ms, NH)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_permute(4, I(shp4), I([0, 3, 1, 2]), AH[k].ptr, YH[k].ptr, st),
+                    SH, reps=20)
+    add("movers", "permute [0,3,1,2] [64,256,56,56]", 8 * NH, ms, NH)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_shuffle_channel(64, 256, INH, 2, AH[k].ptr, YH[k].ptr, st), SH,
+                    reps=20)
+    add("movers", "shuffle_channel g=2 [64,256,56,56]", 8 * NH, ms, NH)
+    pshape = [64, 64, 110, 110]
+    npi = int(np.prod(pshape))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_pad(I(pshape), I([1, 1, 1, 1]), 0.0, AH[k].ptr, YH[k].ptr, st), SH,
+                    reps=20)
+    add("movers", "pad 1 [64,64,110,110] -> 112x112", 4 * (npi + NH), ms, NH)
+    rin, rout = [64, 64, 56, 56], [64, 64, 112, 112]
+    nri = int(np.prod(rin))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_resize(I(rin), I(rout), 1, 0, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
+    add("movers", "resize bilinear x2 [64,64,56,56]", 4 * (nri + NH), ms, NH)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_resize(I(rin), I(rout), 0, 0, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
+    add("movers", "resize nearest x2 [64,64,56,56]", 4 * (nri + NH), ms, NH)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_reorg(I(rout), 1, 2, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
+    add("movers", "reorg natural s2 [64,64,112,112]", 8 * NH, ms, NH)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_reorg(I(rout), 0, 2, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
+    add("movers", "reorg darknet s2 [64,64,112,112]", 8 * NH, ms, NH)
     for bset in (AH, YH):
         for bb in bset:
             bb.free()

@@ -103,16 +103,28 @@ struct PadArgs {
   FastDiv f_out_w, f_out_h;
 };
 
-__global__ __launch_bounds__(kBlock) void pad_kernel(const float* x, float* y, uint32_t n_out,
+// Q outputs per lane (4 when out_w % 4 == 0: one 128-bit store per lane).
+template <int Q>
+__global__ __launch_bounds__(kBlock) void pad_kernel(const float* x, float* y, uint32_t work,
                                                       PadArgs p, float value) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-  if (i >= n_out) return;
+  if (i >= work) return;
   uint32_t rest, wo, plane, ho;
-  fd_divmod(i, p.f_out_w, rest, wo);
+  fd_divmod(Q * i, p.f_out_w, rest, wo);
   fd_divmod(rest, p.f_out_h, plane, ho);
   const int hi = static_cast<int>(ho) - p.top, wi = static_cast<int>(wo) - p.left;
-  const bool inside = hi >= 0 && hi < p.in_h && wi >= 0 && wi < p.in_w;
-  y[i] = inside ? x[(static_cast<uint64_t>(plane) * p.in_h + hi) * p.in_w + wi] : value;
+  const bool row_inside = hi >= 0 && hi < p.in_h;
+  const float* row = x + (static_cast<uint64_t>(plane) * p.in_h + (row_inside ? hi : 0)) * p.in_w;
+  float r[Q];
+#pragma unroll
+  for (int j = 0; j < Q; ++j) {
+    const bool inside = row_inside && wi + j >= 0 && wi + j < p.in_w;
+    r[j] = inside ? row[wi + j] : value;
+  }
+  if (Q == 4)
+    store4_stream(y + 4ull * i, v4f{r[0], r[Q > 1 ? 1 : 0], r[Q > 2 ? 2 : 0], r[Q > 3 ? 3 : 0]});
+  else
+    y[i] = r[0];
 }
 
 // ---------------------------------------------------------------------------
@@ -126,11 +138,12 @@ struct PermuteArgs {
   uint32_t src_stride[kMaxDims];  // input stride of the axis each output dim walks
 };
 
-__global__ __launch_bounds__(kBlock) void permute_generic_kernel(const float* x, float* y, uint32_t n,
+template <int Q>
+__global__ __launch_bounds__(kBlock) void permute_generic_kernel(const float* x, float* y, uint32_t work,
                                                                   PermuteArgs p) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-  if (i >= n) return;
-  uint32_t e = i, src = 0;
+  if (i >= work) return;
+  uint32_t e = Q * i, src = 0;
   for (int k = p.ndim - 1; k >= 1; --k) {
     uint32_t q, r;
     fd_divmod(e, p.f_out[k], q, r);
@@ -138,11 +151,20 @@ __global__ __launch_bounds__(kBlock) void permute_generic_kernel(const float* x,
     e = q;
   }
   src += e * p.src_stride[0];
-  y[i] = x[src];
+  if (Q == 4) {
+    // the innermost output extent is a multiple of 4: four steps along it
+    const uint32_t step = p.src_stride[p.ndim - 1];
+    store4_stream(y + 4ull * i, v4f{x[src], x[src + step], x[src + 2 * step], x[src + 3 * step]});
+  } else {
+    y[i] = x[src];
+  }
 }
 
 constexpr int kTile = 64;
 
+// VEC: rows % 4 == 0, cols % 4 == 0 and both pointers 16-byte aligned: 128-bit
+// loads along the input's fast axis and 128-bit stores along the output's.
+template <bool VEC>
 __global__ __launch_bounds__(kBlock) void transpose_kernel(const float* x, float* y, uint32_t rows,
                                                             uint32_t cols, uint32_t tiles_c,
                                                             FastDiv f_tiles) {
@@ -151,18 +173,43 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(const float* x, float
   fd_divmod(blockIdx.x, f_tiles, batch, t);
   tr = t / tiles_c, tc = t - tr * tiles_c;
   const uint64_t plane = static_cast<uint64_t>(batch) * rows * cols;
-  const uint32_t lx = threadIdx.x & 63u, ly = threadIdx.x >> 6;  // 64 x 4 lanes
   const uint32_t r0 = tr * kTile, c0 = tc * kTile;
+  if (VEC) {
+    const uint32_t q = threadIdx.x & 15u, line = threadIdx.x >> 4;  // 16 vectors x 16 lines
+#pragma unroll
+    for (uint32_t k = line; k < kTile; k += kBlock / 16) {
+      const uint32_t r = r0 + k, c = c0 + 4 * q;
+      if (r < rows && c < cols) {
+        const v4f v = load4_stream(x + plane + static_cast<uint64_t>(r) * cols + c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) tile[k][4 * q + j] = v[j];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t k = line; k < kTile; k += kBlock / 16) {
+      const uint32_t c = c0 + k, r = r0 + 4 * q;
+      if (r < rows && c < cols) {
+        v4f v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = tile[4 * q + j][k];
+        store4_stream(y + plane + static_cast<uint64_t>(c) * rows + r, v);
+      }
+    }
+  } else {
+    const uint32_t lx = threadIdx.x & 63u, ly = threadIdx.x >> 6;  // 64 x 4 lanes
 #pragma unroll 4
-  for (uint32_t k = ly; k < kTile; k += kBlock / kTile) {
-    const uint32_t r = r0 + k, c = c0 + lx;
-    if (r < rows && c < cols) tile[k][lx] = __builtin_nontemporal_load(x + plane + static_cast<uint64_t>(r) * cols + c);
-  }
-  __syncthreads();
+    for (uint32_t k = ly; k < kTile; k += kBlock / kTile) {
+      const uint32_t r = r0 + k, c = c0 + lx;
+      if (r < rows && c < cols)
+        tile[k][lx] = __builtin_nontemporal_load(x + plane + static_cast<uint64_t>(r) * cols + c);
+    }
+    __syncthreads();
 #pragma unroll 4
-  for (uint32_t k = ly; k < kTile; k += kBlock / kTile) {
-    const uint32_t c = c0 + k, r = r0 + lx;
-    if (r < rows && c < cols) y[plane + static_cast<uint64_t>(c) * rows + r] = tile[lx][k];
+    for (uint32_t k = ly; k < kTile; k += kBlock / kTile) {
+      const uint32_t c = c0 + k, r = r0 + lx;
+      if (r < rows && c < cols) y[plane + static_cast<uint64_t>(c) * rows + r] = tile[lx][k];
+    }
   }
 }
 
@@ -176,16 +223,16 @@ struct ReorgArgs {
   FastDiv f_stride, f_out_c;
 };
 
-template <bool DARKNET>
-__global__ __launch_bounds__(kBlock) void reorg_kernel(const float* x, float* y, uint32_t n, ReorgArgs p) {
+template <bool DARKNET, int Q>
+__global__ __launch_bounds__(kBlock) void reorg_kernel(const float* x, float* y, uint32_t work, ReorgArgs p) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-  if (i >= n) return;
+  if (i >= work) return;
   uint32_t rest, w, h, b, c;
-  fd_divmod(i, p.f_w, rest, w);
+  fd_divmod(Q * i, p.f_w, rest, w);
   fd_divmod(rest, p.f_h, rest, h);
   fd_divmod(rest, p.f_c, b, c);
   const uint32_t s = p.stride;
-  uint32_t src;
+  uint32_t src;  // source of the lane's first element; the next ones are `s` further
   if (DARKNET) {
     // lanes walk the input index space; the value comes from the "output" index
     uint32_t offset, c2, oh, ow;
@@ -200,7 +247,10 @@ __global__ __launch_bounds__(kBlock) void reorg_kernel(const float* x, float* y,
     const uint32_t h2 = h * s + oh, w2 = w * s + cw;
     src = ((b * p.in_c + c2) * p.in_h + h2) * p.in_w + w2;
   }
-  y[i] = x[src];
+  if (Q == 4)
+    store4_stream(y + 4ull * i, v4f{x[src], x[src + s], x[src + 2 * s], x[src + 3 * s]});
+  else
+    y[i] = x[src];
 }
 
 // ---------------------------------------------------------------------------
@@ -212,18 +262,28 @@ struct ResizeArgs {
   FastDiv f_out_w, f_out_h;
 };
 
-__global__ __launch_bounds__(kBlock) void resize_nearest_kernel(const float* x, float* y, uint32_t n,
+template <int Q>
+__global__ __launch_bounds__(kBlock) void resize_nearest_kernel(const float* x, float* y, uint32_t work,
                                                                  ResizeArgs p) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-  if (i >= n) return;
+  if (i >= work) return;
   uint32_t rest, w, plane, h;
-  fd_divmod(i, p.f_out_w, rest, w);
+  fd_divmod(Q * i, p.f_out_w, rest, w);
   fd_divmod(rest, p.f_out_h, plane, h);
   const float hf = static_cast<float>(static_cast<int>(h)) * p.fh;
-  const float wf = static_cast<float>(static_cast<int>(w)) * p.fw;
-  // h * (in / out) < in for every extent below 2^24; the clamp only guards larger ones
-  const int src_h = min(static_cast<int>(hf), p.in_h - 1), src_w = min(static_cast<int>(wf), p.in_w - 1);
-  y[i] = x[(static_cast<uint64_t>(plane) * p.in_h + src_h) * p.in_w + src_w];
+  // h * (in / out) < in for every extent below 2^24; the clamps only guard larger ones
+  const int src_h = min(static_cast<int>(hf), p.in_h - 1);
+  const float* row = x + (static_cast<uint64_t>(plane) * p.in_h + src_h) * p.in_w;
+  float r[Q];
+#pragma unroll
+  for (int j = 0; j < Q; ++j) {
+    const float wf = static_cast<float>(static_cast<int>(w) + j) * p.fw;
+    r[j] = row[min(static_cast<int>(wf), p.in_w - 1)];
+  }
+  if (Q == 4)
+    store4_stream(y + 4ull * i, v4f{r[0], r[Q > 1 ? 1 : 0], r[Q > 2 ? 2 : 0], r[Q > 3 ? 3 : 0]});
+  else
+    y[i] = r[0];
 }
 
 // Source coordinate, its two neighbours and the weight of the upper one.
@@ -244,29 +304,41 @@ SHDW_DEVICE void bilinear_axis(uint32_t o, float f, int extent, int& lo, int& hi
   frac = src - static_cast<float>(lo);
 }
 
-template <bool ALIGN>
-__global__ __launch_bounds__(kBlock) void resize_bilinear_kernel(const float* x, float* y, uint32_t n,
+template <bool ALIGN, int Q>
+__global__ __launch_bounds__(kBlock) void resize_bilinear_kernel(const float* x, float* y, uint32_t work,
                                                                   ResizeArgs p) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-  if (i >= n) return;
+  if (i >= work) return;
   uint32_t rest, w, plane, h;
-  fd_divmod(i, p.f_out_w, rest, w);
+  fd_divmod(Q * i, p.f_out_w, rest, w);
   fd_divmod(rest, p.f_out_h, plane, h);
-  int h_l, h_h, w_l, w_h;
-  float sh, sw;
+  int h_l, h_h;
+  float sh;
   bilinear_axis<ALIGN>(h, p.fh, p.in_h, h_l, h_h, sh);
-  bilinear_axis<ALIGN>(w, p.fw, p.in_w, w_l, w_h, sw);
   const float* img = x + static_cast<uint64_t>(plane) * p.in_h * p.in_w;
-  const float v0 = img[h_l * p.in_w + w_l], v1 = img[h_h * p.in_w + w_l];
-  const float v2 = img[h_l * p.in_w + w_h], v3 = img[h_h * p.in_w + w_h];
-  // ((1-sh)(1-sw) v0 + sh(1-sw) v1) + (1-sh) sw v2) + sh sw v3, each product
-  // formed left to right and rounded, no fused operations
-  const float ih = 1 - sh, iw = 1 - sw;
-  const float a0 = ih * iw, a1 = sh * iw, a2 = ih * sw, a3 = sh * sw;
-  const float t0 = a0 * v0, t1 = a1 * v1, t2 = a2 * v2, t3 = a3 * v3;
-  const float s01 = t0 + t1;
-  const float s012 = s01 + t2;
-  y[i] = s012 + t3;
+  const float* row_l = img + h_l * p.in_w;
+  const float* row_h = img + h_h * p.in_w;
+  const float ih = 1 - sh;
+  float r[Q];
+#pragma unroll
+  for (int j = 0; j < Q; ++j) {
+    int w_l, w_h;
+    float sw;
+    bilinear_axis<ALIGN>(w + j, p.fw, p.in_w, w_l, w_h, sw);
+    const float v0 = row_l[w_l], v1 = row_h[w_l], v2 = row_l[w_h], v3 = row_h[w_h];
+    // ((1-sh)(1-sw) v0 + sh(1-sw) v1) + (1-sh) sw v2) + sh sw v3, each product
+    // formed left to right and rounded, no fused operations
+    const float iw = 1 - sw;
+    const float a0 = ih * iw, a1 = sh * iw, a2 = ih * sw, a3 = sh * sw;
+    const float t0 = a0 * v0, t1 = a1 * v1, t2 = a2 * v2, t3 = a3 * v3;
+    const float s01 = t0 + t1;
+    const float s012 = s01 + t2;
+    r[j] = s012 + t3;
+  }
+  if (Q == 4)
+    store4_stream(y + 4ull * i, v4f{r[0], r[Q > 1 ? 1 : 0], r[Q > 2 ? 2 : 0], r[Q > 3 ? 3 : 0]});
+  else
+    y[i] = r[0];
 }
 
 static bool count_fits(const int* shape, int n, int64_t* count) {
@@ -351,7 +423,11 @@ int shdw_hip_pad(const int* in_shape, const int* paddings, float value, const fl
   PadArgs p{in_shape[2], in_shape[3], paddings[0], paddings[2], make_fastdiv(out_shape[3]),
             make_fastdiv(out_shape[2])};
   const uint32_t n = static_cast<uint32_t>(out_count);
-  pad_kernel<<<grid_for(n), kBlock, 0, static_cast<hipStream_t>(stream)>>>(x, y, n, p, value);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (out_shape[3] % 4 == 0 && aligned16(y))
+    pad_kernel<4><<<grid_for(n / 4), kBlock, 0, st>>>(x, y, n / 4, p, value);
+  else
+    pad_kernel<1><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p, value);
   return launch_status();
 }
 
@@ -400,8 +476,12 @@ int shdw_hip_permute(int num_axes, const int* in_shape, const int* order, const 
     const uint32_t tiles_r = (rows + kTile - 1) / kTile, tiles_c = (cols + kTile - 1) / kTile;
     const int64_t groups = static_cast<int64_t>(batch) * tiles_r * tiles_c;
     if (groups <= INT32_MAX) {
-      transpose_kernel<<<static_cast<uint32_t>(groups), kBlock, 0, st>>>(
-          x, y, rows, cols, tiles_c, make_fastdiv(tiles_r * tiles_c));
+      const FastDiv ft = make_fastdiv(tiles_r * tiles_c);
+      const uint32_t g = static_cast<uint32_t>(groups);
+      if (rows % 4 == 0 && cols % 4 == 0 && aligned16(x) && aligned16(y))
+        transpose_kernel<true><<<g, kBlock, 0, st>>>(x, y, rows, cols, tiles_c, ft);
+      else
+        transpose_kernel<false><<<g, kBlock, 0, st>>>(x, y, rows, cols, tiles_c, ft);
       return launch_status();
     }
   }
@@ -411,7 +491,10 @@ int shdw_hip_permute(int num_axes, const int* in_shape, const int* order, const 
     p.f_out[k] = make_fastdiv(static_cast<uint32_t>(ext[k]));
     p.src_stride[k] = static_cast<uint32_t>(str[k]);
   }
-  permute_generic_kernel<<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
+  if (ext[nd - 1] % 4 == 0 && aligned16(y))
+    permute_generic_kernel<4><<<grid_for(n / 4), kBlock, 0, st>>>(x, y, n / 4, p);
+  else
+    permute_generic_kernel<1><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
   return launch_status();
 }
 
@@ -433,12 +516,18 @@ int shdw_hip_reorg(const int* in_shape, int type, int stride, const float* x, fl
   if (type == 0) {
     p.f_w = make_fastdiv(in_w), p.f_h = make_fastdiv(in_h), p.f_c = make_fastdiv(in_c);
     p.f_out_c = make_fastdiv(in_c / (stride * stride));
-    reorg_kernel<true><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
+    if (in_w % 4 == 0 && aligned16(y))
+      reorg_kernel<true, 4><<<grid_for(n / 4), kBlock, 0, st>>>(x, y, n / 4, p);
+    else
+      reorg_kernel<true, 1><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
   } else {
     p.f_w = make_fastdiv(in_w / stride), p.f_h = make_fastdiv(in_h / stride);
     p.f_c = make_fastdiv(in_c * stride * stride);
     p.f_out_c = make_fastdiv(1);
-    reorg_kernel<false><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
+    if ((in_w / stride) % 4 == 0 && aligned16(y))
+      reorg_kernel<false, 4><<<grid_for(n / 4), kBlock, 0, st>>>(x, y, n / 4, p);
+    else
+      reorg_kernel<false, 1><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
   }
   return launch_status();
 }
@@ -461,17 +550,29 @@ int shdw_hip_resize(const int* in_shape, const int* out_shape, int type, int ali
   ResizeArgs p;
   p.in_h = in_h, p.in_w = in_w;
   p.f_out_w = make_fastdiv(out_w), p.f_out_h = make_fastdiv(out_h);
+  const bool quad = out_w % 4 == 0 && aligned16(y);
+  const uint32_t work = quad ? n / 4 : n;
+  const uint32_t grid = grid_for(work);
   if (type == 1 && align_corners) {
     p.fh = static_cast<float>(in_h - 1) / (out_h - 1);
     p.fw = static_cast<float>(in_w - 1) / (out_w - 1);
-    resize_bilinear_kernel<true><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
+    if (quad)
+      resize_bilinear_kernel<true, 4><<<grid, kBlock, 0, st>>>(x, y, work, p);
+    else
+      resize_bilinear_kernel<true, 1><<<grid, kBlock, 0, st>>>(x, y, work, p);
   } else {
     p.fh = static_cast<float>(in_h) / out_h;
     p.fw = static_cast<float>(in_w) / out_w;
-    if (type == 0)
-      resize_nearest_kernel<<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
-    else
-      resize_bilinear_kernel<false><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p);
+    if (type == 0) {
+      if (quad)
+        resize_nearest_kernel<4><<<grid, kBlock, 0, st>>>(x, y, work, p);
+      else
+        resize_nearest_kernel<1><<<grid, kBlock, 0, st>>>(x, y, work, p);
+    } else if (quad) {
+      resize_bilinear_kernel<false, 4><<<grid, kBlock, 0, st>>>(x, y, work, p);
+    } else {
+      resize_bilinear_kernel<false, 1><<<grid, kBlock, 0, st>>>(x, y, work, p);
+    }
   }
   return launch_status();
 }
