@@ -55,6 +55,8 @@ def parse():
     ap.add_argument("--probe", action="store_true",
                     help="counter probe: 3 launches of a plain copy and of every headline op on "
                          "the 51.4M tensor, nothing timed, no JSON (run under rocprofv3 --pmc)")
+    ap.add_argument("--probe-next", action="store_true",
+                    help="the same for the neighbouring operators and the data movers")
     return ap.parse_args()
 
 
@@ -191,6 +193,40 @@ def probe(dev):
         dev.ck(lib.shdw_hip_unary(2, n, x.ptr, y.ptr, st))
         dev.ck(lib.shdw_hip_activate(5, 0.1, n, x.ptr, y.ptr, st))
         dev.ck(lib.shdw_hip_scale_bias(n, C, inner, x.ptr, g.ptr, b.ptr, 1, y.ptr, st))
+    dev.sync()
+
+
+def probe_next(dev):
+    """Counter probe for the operators next to the path, 3 launches each on the
+    headline tensor (or the ResNet shape that feeds them); the copy calibrates."""
+    lib, st = dev.lib, dev.stream
+    I = dev.sa.ints
+    n, C, inner = 64 * 256 * 56 * 56, 256, 56 * 56
+    x, x2 = dev.buf(normal(201, n, 2.0)), dev.buf(normal(204, n))
+    g, b = dev.buf(uniform(202, C, 0.5, 1.5)), dev.buf(uniform(203, C, -0.1, 0.1))
+    alpha = dev.buf(uniform(205, 64 * C, 0.0, 1.0))
+    ls, lb = dev.buf(uniform(206, 784, 0.5, 1.5)), dev.buf(uniform(207, 784, -0.1, 0.1))
+    y = dev.buf(nbytes=4 * n)
+    stem_in, stem_out = [64, 64, 112, 112], [64, 64, 56, 56]
+    for _ in range(3):
+        dev.ck(lib.shdw_hip_copy(n, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_batch_norm(n, C, inner, x.ptr, b.ptr, g.ptr, 1.0, 1e-5, y.ptr, st))
+        dev.ck(lib.shdw_hip_axpy_rows(64 * C, inner, alpha.ptr, x.ptr, x2.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_pooling2d(I(stem_in), 0, 3, 3, 2, 2, 0, 0, I(stem_out), x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_pooling2d(I([512, 2048, 7, 7]), 1, 7, 7, 1, 1, 0, 0, I([512, 2048, 1, 1]), x.ptr,
+                                      y.ptr, st))
+        dev.ck(lib.shdw_hip_softmax(64, 49, 16384, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_normalize(64, 49, 16384, 2.0, 1e-12, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_group_norm(64 * C, inner, 1e-5, x.ptr, g.ptr, b.ptr, C, inner, y.ptr, st))
+        dev.ck(lib.shdw_hip_group_norm(64 * 32, 8 * inner, 1e-5, x.ptr, g.ptr, b.ptr, C, inner, y.ptr, st))
+        dev.ck(lib.shdw_hip_group_norm(65536, 784, 1e-5, x.ptr, ls.ptr, lb.ptr, 784, 1, y.ptr, st))
+        dev.ck(lib.shdw_hip_permute(4, I([64, 256, 56, 56]), I([0, 2, 3, 1]), x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_shuffle_channel(64, 256, inner, 2, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_pad(I([64, 64, 110, 110]), I([1, 1, 1, 1]), 0.0, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_resize(I(stem_out), I(stem_in), 1, 0, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_resize(I(stem_out), I(stem_in), 0, 0, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_reorg(I(stem_in), 1, 2, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_reorg(I(stem_in), 0, 2, x.ptr, y.ptr, st))
     dev.sync()
 
 
@@ -423,6 +459,9 @@ def main():
     dev = Dev()
     if args.probe:
         probe(dev)
+        return
+    if args.probe_next:
+        probe_next(dev)
         return
     ms_per_step, step_bytes, n, roofline, detail, host = headline(dev, args.steps, args.warmup)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
