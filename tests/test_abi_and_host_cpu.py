@@ -135,3 +135,51 @@ def test_kernel_lookup_and_argument_errors_throw():
     assert h.shdw_host_probe_argument(b"none", b"int") == 0     # absent -> default
     assert h.shdw_host_probe_argument(b"int", b"dup") == -1
     assert b"Duplicated argument name" in h.shdw_host_last_error()
+
+
+def test_entry_points_validate_before_touching_the_device():
+    """Bad arguments are refused on the host: these calls return without a GPU."""
+    lib = shadow_amd.hip()
+    ints = shadow_amd.ints
+    p = ctypes.c_void_p(4096)  # never dereferenced: validation fails first
+    E, U = -1, -2
+    assert lib.shdw_hip_softmax(-1, 2, 2, p, p, None) == E
+    assert lib.shdw_hip_softmax(2, 2, 2, None, p, None) == E
+    assert lib.shdw_hip_softmax(0, 5, 5, None, None, None) == 0
+    assert lib.shdw_hip_normalize(65536, 65536, 2, 2.0, 0.0, p, p, None) == E
+    assert lib.shdw_hip_batch_norm(8, 0, 1, p, p, p, 1.0, 0.0, p, None) == E
+    assert lib.shdw_hip_batch_norm(0, 4, 1, None, None, None, 1.0, 0.0, None, None) == 0
+    assert lib.shdw_hip_axpy_rows(65536, 65536, p, p, p, p, None) == E
+    assert lib.shdw_hip_axpy_rows(4, 4, None, p, p, p, None) == E
+    assert lib.shdw_hip_group_norm(2, 8, 1e-5, p, p, None, 1, 1, p, None) == E
+    assert lib.shdw_hip_group_norm(2, 8, 1e-5, p, p, p, 0, 1, p, None) == E
+    assert lib.shdw_hip_group_norm(0, 8, 1e-5, None, None, None, 1, 1, None, None) == 0
+    sh = ints([1, 1, 4, 4])
+    assert lib.shdw_hip_pooling2d(sh, 2, 2, 2, 1, 1, 0, 0, sh, p, p, None) == E
+    assert lib.shdw_hip_pooling2d(sh, 0, 0, 2, 1, 1, 0, 0, sh, p, p, None) == E
+    assert lib.shdw_hip_pooling2d(sh, 0, 2, 2, 0, 1, 0, 0, sh, p, p, None) == E
+    assert lib.shdw_hip_pooling2d(sh, 0, 2, 2, 1, 1, -1, 0, sh, p, p, None) == E
+    assert lib.shdw_hip_pooling2d(sh, 0, 2, 2, 1, 1, 0, 0, ints([2, 1, 3, 3]), p, p, None) == E
+    assert lib.shdw_hip_pooling2d(None, 0, 2, 2, 1, 1, 0, 0, sh, p, p, None) == E
+    assert lib.shdw_hip_pooling3d(ints([1, 1, 2, 2, 2]), 0, 2, 2, 2, 1, 1, 1, 0, 0, 0, ints([1, 1, 0, 1, 1]), p, p, None) == 0
+    assert lib.shdw_hip_copy_chunks(2, 8, p, 4, 0, p, 8, 0, None) == E       # chunk wider than its source row
+    assert lib.shdw_hip_copy_chunks(2, 4, p, 8, 0, p, 8, 6, None) == E       # chunk leaves its destination row
+    assert lib.shdw_hip_copy_chunks(-1, 4, p, 8, 0, p, 8, 0, None) == E
+    assert lib.shdw_hip_copy_chunks(0, 4, None, 8, 0, None, 8, 0, None) == 0
+    assert lib.shdw_hip_gather(2, 0, 4, 3, p, p, p, None) == E
+    assert lib.shdw_hip_gather(2, 5, 4, 0, p, p, p, None) == E
+    assert lib.shdw_hip_shuffle_channel(2, 6, 4, 4, p, p, None) == E          # 6 channels, 4 groups
+    assert lib.shdw_hip_pad(ints([1, 1, 4, 4]), ints([-3, -3, 0, 0]), 0.0, p, p, None) == E
+    assert lib.shdw_hip_pad(None, ints([0, 0, 0, 0]), 0.0, p, p, None) == E
+    assert lib.shdw_hip_permute(3, ints([2, 3, 4]), ints([0, 1, 1]), p, p, None) == E
+    assert lib.shdw_hip_permute(3, ints([2, 3, 4]), ints([0, 1, 3]), p, p, None) == E
+    assert lib.shdw_hip_permute(9, ints([1] * 9), ints(list(range(9))), p, p, None) == E
+    assert lib.shdw_hip_permute(0, ints([1]), ints([0]), p, p, None) == E
+    assert lib.shdw_hip_reorg(ints([1, 6, 4, 4]), 0, 2, p, p, None) == E       # 6 % 4 != 0
+    assert lib.shdw_hip_reorg(ints([1, 4, 5, 4]), 1, 2, p, p, None) == E
+    assert lib.shdw_hip_reorg(ints([1, 4, 4, 4]), 2, 2, p, p, None) == E
+    assert lib.shdw_hip_reorg(ints([1, 4, 4, 4]), 1, 0, p, p, None) == E
+    assert lib.shdw_hip_resize(ints([1, 1, 4, 4]), ints([1, 2, 8, 8]), 1, 0, p, p, None) == E
+    assert lib.shdw_hip_resize(ints([1, 1, 4, 4]), ints([1, 1, 8, 8]), 3, 0, p, p, None) == E
+    assert lib.shdw_hip_resize(ints([1, 1, 4, 4]), ints([1, 1, 1, 8]), 1, 1, p, p, None) == U
+    assert lib.shdw_hip_resize(ints([1, 1, 4, 4]), ints([1, 1, 0, 8]), 1, 0, p, p, None) == 0
