@@ -461,6 +461,41 @@ def config_table(dev):
     return rows
 
 
+NETWORK_TEXT = """[bottleneck_tail]
+[{out_blob, v_s, [prob]}]
+[{gamma, float, [1024]}; {beta, float, [1024]}]
+[Input] | [in] | [0 2 2] | [] | [x; r] | [{x, v_i, [64 # 1024 # 14 # 14]}; {r, v_i, [64 # 1024 # 14 # 14]}]
+[Scale] | [bn] | [3 1 3] | [x; gamma; beta] | [s] | [{axis, s_i, [1]}; {has_scale, s_i, [1]}; {has_bias, s_i, [1]}]
+[Eltwise] | [add] | [2 1 1] | [s; r] | [e] | [{operation, s_i, [1]}]
+[Activate] | [relu] | [1 1 1] | [e] | [e] | [{type, s_i, [1]}]
+[Pooling] | [gap] | [1 1 2] | [e] | [p] | [{pool, s_i, [1]}; {global_pooling, s_i, [1]}]
+[Flatten] | [flat] | [1 1 0] | [p] | [f] | []
+[Softmax] | [prob] | [1 1 1] | [f] | [prob] | [{axis, s_i, [1]}]
+"""
+
+
+def network_forward(dev, reps=50):
+    """Wall time of Network::Forward for a six-operator text model on
+    [64,1024,14,14] with device inputs: two 51 MB device-to-device input copies,
+    five launches, one stream synchronisation per call."""
+    sa = dev.sa
+    n = 64 * 1024 * 14 * 14
+    x, r = dev.buf(normal(801, n)), dev.buf(normal(802, n))
+    weights = [uniform(803, 1024, 0.5, 1.5), uniform(804, 1024, -0.1, 0.1)]
+    with sa.Network(NETWORK_TEXT, weights, device_input=True) as net:
+        for _ in range(5):
+            net.forward({"x": x, "r": r})
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            net.forward({"x": x, "r": r})
+        t1 = time.perf_counter()
+    us = (t1 - t0) * 1e6 / reps
+    moved = 4 * n * (2 * 2 + 3 + 3 + 2 + 1)  # input copies, scale, eltwise, relu, pooling read
+    return {"model": "Scale -> Eltwise -> ReLU -> global avg Pooling -> Flatten -> Softmax, [64,1024,14,14]",
+            "us_per_forward": round(us, 1), "operators": 6, "launches": 5, "input_copies": 2,
+            "bytes_moved": moved, "GBps": round(moved / us / 1e3, 1)}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -492,6 +527,7 @@ def main():
     }
     if not args.no_configs:
         out["configs"] = config_table(dev)
+        out["network"] = network_forward(dev)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(host, step_bytes, args.cpu_passes)
         out["speedup_vs_cpu"] = round(value / out["cpu_baseline"]["value"], 1)

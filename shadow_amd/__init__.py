@@ -198,7 +198,7 @@ HOST_SIGNATURES = {
     "shdw_host_op_debug_log": (_I, [_V, _V, ctypes.c_char_p, _Z]),
     "shdw_host_parse_net": (_I, [ctypes.c_char_p, ctypes.c_char_p, _Z]),
     "shdw_host_backend_keys": (_I, [ctypes.c_char_p, _Z]),
-    "shdw_host_network_create": (_V, [ctypes.c_char_p, _I, _I, ctypes.c_char_p, _V]),
+    "shdw_host_network_create": (_V, [ctypes.c_char_p, _I, _I, _I, ctypes.c_char_p, _V]),
     "shdw_host_network_destroy": (None, [_V]),
     "shdw_host_network_io": (_I, [_V, _I, ctypes.c_char_p, _Z]),
     "shdw_host_network_forward": (_I, [_V, _I, ctypes.POINTER(ctypes.c_char_p), c_void_pp, c_int_p, c_int_p]),
@@ -345,13 +345,15 @@ class Network:
     """Shadow::Network over the Native backend: a text model plus packed float32
     weights (declared-blob order), run with host inputs."""
 
-    def __init__(self, proto_text, weights=None, backend_type="Native", device_id=0, debug=False):
+    def __init__(self, proto_text, weights=None, backend_type="Native", device_id=0, debug=False,
+                 device_input=False):
         self.lib = host()
+        self.device_input = device_input
         packed = None
         if weights is not None and len(weights):
             packed = np.concatenate([np.ascontiguousarray(w, np.float32).ravel() for w in weights])
         self.ptr = self.lib.shdw_host_network_create(
-            backend_type.encode(), device_id, int(debug), proto_text.encode(),
+            backend_type.encode(), device_id, int(debug), int(device_input), proto_text.encode(),
             packed.ctypes.data if packed is not None else None)
         host_check(self.ptr)
 
@@ -373,8 +375,12 @@ class Network:
         """inputs: {blob name: float32 array}.  reshape=True passes each array's
         shape along, so the input blob is reshaped before the copy."""
         names = list(inputs)
-        arrays = [np.ascontiguousarray(inputs[k], np.float32) for k in names]
         c_names = (ctypes.c_char_p * len(names))(*[k.encode() for k in names])
+        if self.device_input:  # {name: Buffer}; shapes stay as declared
+            c_data = (ctypes.c_void_p * len(names))(*[inputs[k].ptr for k in names])
+            host_check(self.lib.shdw_host_network_forward(self.ptr, len(names), c_names, c_data, None, None) == 0)
+            return
+        arrays = [np.ascontiguousarray(inputs[k], np.float32) for k in names]
         c_data = (ctypes.c_void_p * len(names))(*[a.ctypes.data for a in arrays])
         ranks = ints([a.ndim if reshape else 0 for a in arrays])
         dims = ints([d for a in arrays for d in (a.shape if reshape else ())])

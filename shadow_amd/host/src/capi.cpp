@@ -197,15 +197,17 @@ int shdw_host_parse_net(const char* proto_text, char* buf, size_t n) {
 int shdw_host_backend_keys(char* buf, size_t n) { return join(BackendRegistry()->Keys(), buf, n); }
 
 // weights: one packed host buffer in declared-blob order, or NULL when the
-// model declares no blobs.  NULL on error.
+// model declares no blobs.  device_input: Forward takes device pointers and
+// copies device to device.  NULL on error.
 void* shdw_host_network_create(const char* backend_type, int device_id, int debug,
-                               const char* proto_text, const void* weights) {
+                               int device_input, const char* proto_text, const void* weights) {
   Network* net = nullptr;
   guarded([&] {
     ArgumentHelper args;
     args.AddSingleArgument<std::string>("backend_type", backend_type ? backend_type : "");
     args.AddSingleArgument<int>("device_id", device_id);
     args.AddSingleArgument<bool>("debug", debug != 0);
+    args.AddSingleArgument<bool>("device_input", device_input != 0);
     std::unique_ptr<Network> made(new Network());
     made->LoadXModel(std::string(proto_text ? proto_text : ""), weights, args);
     made->backend()->ws()->Ctx()->synchronize();  // the weight buffer may go away after return
@@ -226,7 +228,8 @@ int shdw_host_network_io(void* net, int which, char* buf, size_t n) {
   return len;
 }
 
-// count inputs: names[i] -> host data[i]; ranks[i] > 0 reshapes that input
+// count inputs: names[i] -> data[i] (host pointers, or device pointers for a
+// network created with device_input); ranks[i] > 0 reshapes that input
 // first with the next ranks[i] entries of `shapes`.
 int shdw_host_network_forward(void* net, int count, const char* const* names, void* const* data,
                               const int* ranks, const int* shapes) {
