@@ -51,7 +51,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-configs", action="store_true", help="skip the per-config table")
-    ap.add_argument("--cpu-passes", type=int, default=2)
+    ap.add_argument("--cpu-passes", type=int, default=10)
     ap.add_argument("--probe", action="store_true",
                     help="counter probe: 3 launches of a plain copy and of every headline op on "
                          "the 51.4M tensor, nothing timed, no JSON (run under rocprofv3 --pmc)")

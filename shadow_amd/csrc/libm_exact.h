@@ -41,19 +41,18 @@ SHDW_LIBM_FN float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
 SHDW_LIBM_FN uint64_t d2u(double d) { return __builtin_bit_cast(uint64_t, d); }
 SHDW_LIBM_FN double u2d(uint64_t u) { return __builtin_bit_cast(double, u); }
 
-// a / b, correctly rounded, for callers that know |a|, |b| and |a / b| are all
-// well inside the normal range (no scaling, no special cases).  On the device
-// this is the reciprocal-plus-Newton core of the compiler's own IEEE division
-// without its range scaling and fix-up instructions; on the host it is `/`.
+// a / b for the two quotients of exact_tanhf, whose operands and result are
+// well inside the normal range.  On the device: the hardware reciprocal (1 ulp),
+// a * r, and one correction from the exact remainder a - b * q.  That is shorter
+// than a division that is correctly rounded for every operand pair (no second
+// correction, no refinement of r); it is used only here because exact_tanhf on
+// the device returns the library's result for every one of the 2^32 inputs with
+// it, which the exhaustive device test checks.  On the host it is `/`.
 SHDW_LIBM_FN float div_normal(float a, float b) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  float r = __builtin_amdgcn_rcpf(b);
-  float e = __builtin_fmaf(-b, r, 1.0f);
-  r = __builtin_fmaf(e, r, r);
-  float q = a * r;
-  e = __builtin_fmaf(-b, q, a);
-  q = __builtin_fmaf(e, r, q);
-  e = __builtin_fmaf(-b, q, a);
+  const float r = __builtin_amdgcn_rcpf(b);
+  const float q = a * r;
+  const float e = __builtin_fmaf(-b, q, a);
   return __builtin_fmaf(e, r, q);
 #else
   return a / b;
@@ -198,24 +197,18 @@ SHDW_LIBM_FN float exact_tanhf(float x) {
   const uint32_t jx = f2u(x);
   const uint32_t ix = jx & 0x7fffffffu;
   const bool big = ix >= 0x3f800000u;  // |x| >= 1: expm1f(+2|x|), else expm1f(-2|x|)
-  const float ax = u2f(ix);
-  const float a = big ? two * ax : -two * ax;  // argument of expm1f
-  const uint32_t ha = f2u(a) & 0x7fffffffu;
-  const bool aneg = !big;
+  // from |x| = 10 on 2 / (t + 2) < 2^-25 and 1 - q rounds to 1: evaluate at 10
+  const uint32_t ic = ix < 0x41200000u ? ix : 0x41200000u;
+  const float a2 = two * u2f(ic);
+  const float a = big ? a2 : -a2;  // argument of expm1f
 
   // --- expm1f(a): argument reduction ---
-  const bool reduce = ha > 0x3eb17218u;   // |a| > 0.5 ln2
-  const bool unit_k = ha < 0x3F851592u;   // |a| < 1.5 ln2  ->  k = +-1
-  const int32_t kgen = static_cast<int32_t>(invln2 * a + (aneg ? -0.5f : 0.5f));
-  int32_t k = unit_k ? (aneg ? -1 : 1) : kgen;
-  k = reduce ? k : 0;
-  const float tk = static_cast<float>(k);
-  // k = +-1 uses hi = a -+ ln2_hi, lo = +-ln2_lo, which is what t*ln2_hi and
-  // t*ln2_lo give for t = +-1 (both products exact).
+  const float tk = __builtin_rintf(invln2 * a);
+  const int32_t k = static_cast<int32_t>(tk);
   const float hi = a - tk * ln2_hi;
   const float lo = tk * ln2_lo;
-  const float xr = reduce ? hi - lo : a;
-  const float c = reduce ? (hi - xr) - lo : 0.0f;
+  const float xr = hi - lo;
+  const float c = (hi - xr) - lo;
 
   // --- primary range ---
   const float hfx = 0.5f * xr;
@@ -228,31 +221,17 @@ SHDW_LIBM_FN float exact_tanhf(float x) {
   e = (xr * (e - c) - c);
   e -= hxs;
   const float res_km1 = 0.5f * (xr - e) - 0.5f;
-  // k <= -2 or k > 56: y = 1 - (e - x); 2 <= k < 23: y = (1 - 2^-k) - (e - x)
-  const bool mid = (k >= 2) && (k < 23);
-  const uint32_t ksh = static_cast<uint32_t>(k) & 31u;
-  const float t_lo = mid ? u2f(0x3f800000u - (0x1000000u >> ksh)) : one;
-  const float y_a = t_lo - (e - xr);
-  // 23 <= k <= 56: y = (x - (e + 2^-k)) + 1
-  const float t_hi = u2f(static_cast<uint32_t>(0x7f - k) << 23);
-  float y_b = xr - (e + t_hi);
-  y_b += one;
-  const bool hi_k = (k >= 23) && (k <= 56);
-  float yk = hi_k ? y_b : y_a;
+  const float t_lo = u2f(0x3f800000u - (0x1000000u >> (static_cast<uint32_t>(k) & 31u)));
+  float yk = t_lo - (e - xr);
   yk = u2f(f2u(yk) + (static_cast<uint32_t>(k) << 23));  // scale by 2^k
-  const float res_gen = (mid || hi_k) ? yk : yk - one;
-  float t = (k == 0) ? res_k0 : ((k == -1) ? res_km1 : res_gen);
-  t = (ha < 0x33000000u) ? a : t;  // |a| < 2^-25: expm1f returns a
+  const float res_gen = big ? yk : yk - one;
+  const float t = (k == 0) ? res_k0 : ((k == -1) ? res_km1 : res_gen);
 
   // --- tanhf ---
-  // |x| >= 1: 2 / (t + 2) with t in [6.3, 1.3e19]; else t / (t + 2) with
-  // |t| in [2^-54, 0.87] and t + 2 in (1.13, 2]: every value is normal
   const float q = div_normal(big ? two : t, t + two);
-  float z = big ? one - q : -q;
-  z = (ix < 0x41b00000u) ? z : one;           // |x| >= 22 (and +-inf): 1 - tiny == 1
-  float res = (jx >> 31) ? -z : z;
-  res = (ix < 0x24000000u) ? x : res;  // |x| < 2^-55 (and +-0): x * (1 + x) == x exactly
-  res = (ix > 0x7f800000u) ? x + x : res;          // NaN
+  const float z = big ? one - q : q;
+  float res = u2f((f2u(z) & 0x7fffffffu) | (jx & 0x80000000u));
+  res = (ix > 0x7f800000u) ? x + x : res;  // NaN
   return res;
 }
 
