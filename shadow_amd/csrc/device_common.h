@@ -14,6 +14,7 @@
 namespace shdw {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
 constexpr int kBlock = 256;  // 4 wave64 per workgroup

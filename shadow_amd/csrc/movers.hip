@@ -7,6 +7,8 @@
 // tile so that both sides stay coalesced.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include "../../include/shadow_hip.h"
 #include "device_common.h"
 #include "launch.h"
@@ -333,7 +335,8 @@ __global__ __launch_bounds__(kBlock) void resize_nearest_kernel(const float* x, 
 
 // Source coordinate, its two neighbours and the weight of the upper one.
 template <bool ALIGN>
-SHDW_DEVICE void bilinear_axis(uint32_t o, float f, int extent, int& lo, int& hi, float& frac) {
+__host__ __device__ __forceinline__ void bilinear_axis(uint32_t o, float f, int extent, int& lo, int& hi,
+                                                       float& frac) {
   float src;
   if (ALIGN) {
     src = static_cast<float>(static_cast<int>(o)) * f;
@@ -384,6 +387,166 @@ __global__ __launch_bounds__(kBlock) void resize_bilinear_kernel(const float* x,
     store4_stream(y + 4ull * i, v4f{r[0], r[Q > 1 ? 1 : 0], r[Q > 2 ? 2 : 0], r[Q > 3 ? 3 : 0]});
   else
     y[i] = r[0];
+}
+
+// Bilinear resize staged through LDS.  The kernel above issues sixteen 4-byte
+// gathers per lane, and a gather occupies the address unit for a full wave
+// whatever its width, so it runs at the gather rate and not at the HBM rate.
+// Here one workgroup owns a band of `rows` output rows of one plane: it
+//   1. evaluates the column axis once (neighbour offsets and weight per output
+//      column) into LDS,
+//   2. copies the input rows the band touches, one contiguous span of the plane,
+//      into LDS with 128-bit loads,
+//   3. forms each output from four LDS reads with the same operations, in the
+//      same order, as the gather kernel.
+// The arithmetic is unchanged, so the results are bit-identical.
+struct ResizeBandArgs {
+  int in_h, in_w, out_h, out_w;
+  float fh, fw;
+  int rows;       // output rows per band
+  int tile_rows;  // input rows the LDS tile holds (the widest band's span)
+  FastDiv f_bands;  // bands per plane
+  FastDiv f_cols;   // lane-tasks per output row: out_w / Q
+};
+
+constexpr int kResizeBandOutputs = 4096;    // outputs per workgroup aimed at
+constexpr int kResizeBandLdsBytes = 20480;  // 8 workgroups per CU keep their tiles resident
+constexpr int kResizeBandMaxLdsBytes = 65536;
+constexpr int kResizeBandGroups = 2048;     // keep at least this many workgroups when shrinking bands
+
+template <bool ALIGN, int Q>
+__global__ __launch_bounds__(kBlock) void resize_bilinear_band_kernel(const float* x, float* y,
+                                                                       ResizeBandArgs p) {
+  extern __shared__ __align__(16) float band_lds[];
+  const uint32_t cols_pad = (static_cast<uint32_t>(p.out_w) + 3u) & ~3u;
+  float* frac = band_lds;
+  uint32_t* lo_b = reinterpret_cast<uint32_t*>(band_lds + cols_pad);
+  uint32_t* hi_b = lo_b + cols_pad;
+  float* tile = band_lds + 3 * cols_pad;
+
+  uint32_t plane, band;
+  fd_divmod(blockIdx.x, p.f_bands, plane, band);
+  const int h0 = static_cast<int>(band) * p.rows;
+  const int nrows = min(p.rows, p.out_h - h0);
+
+  for (uint32_t c = threadIdx.x; c < static_cast<uint32_t>(p.out_w); c += kBlock) {
+    int w_l, w_h;
+    float sw;
+    bilinear_axis<ALIGN>(c, p.fw, p.in_w, w_l, w_h, sw);
+    frac[c] = sw;
+    lo_b[c] = static_cast<uint32_t>(w_l) * 4u;  // byte offsets inside a tile row
+    hi_b[c] = static_cast<uint32_t>(w_h) * 4u;
+  }
+
+  int first, last, unused;
+  float unused_f;
+  bilinear_axis<ALIGN>(static_cast<uint32_t>(h0), p.fh, p.in_h, first, unused, unused_f);
+  bilinear_axis<ALIGN>(static_cast<uint32_t>(h0 + nrows - 1), p.fh, p.in_h, unused, last, unused_f);
+  // The host sized the tile from these same expressions; the clamp only keeps a
+  // disagreement from writing past the tile.
+  const uint32_t span_rows = static_cast<uint32_t>(min(last - first + 1, p.tile_rows));
+  const uint32_t count = span_rows * static_cast<uint32_t>(p.in_w);
+  const float* src = x + (static_cast<uint64_t>(plane) * p.in_h + first) * p.in_w;
+  if ((p.in_w & 3) == 0 && aligned16_device(x)) {
+    for (uint32_t i = threadIdx.x; i < count / 4; i += kBlock)
+      *reinterpret_cast<v4f*>(tile + 4 * i) = load4(src + 4 * i);
+  } else {
+    for (uint32_t i = threadIdx.x; i < count; i += kBlock) tile[i] = src[i];
+  }
+  __syncthreads();
+
+  const char* tile_b = reinterpret_cast<const char*>(tile);
+  const uint32_t row_bytes = static_cast<uint32_t>(p.in_w) * 4u;
+  const uint32_t tasks = static_cast<uint32_t>(nrows) * p.f_cols.d;
+  float* out = y + (static_cast<uint64_t>(plane) * p.out_h + h0) * p.out_w;
+  for (uint32_t t = threadIdx.x; t < tasks; t += kBlock) {
+    uint32_t r, cq;
+    fd_divmod(t, p.f_cols, r, cq);
+    int h_l, h_h;
+    float sh;
+    bilinear_axis<ALIGN>(static_cast<uint32_t>(h0) + r, p.fh, p.in_h, h_l, h_h, sh);
+    const char* row_l = tile_b + static_cast<uint32_t>(h_l - first) * row_bytes;
+    const char* row_h = tile_b + static_cast<uint32_t>(h_h - first) * row_bytes;
+    const float ih = 1 - sh;
+    float sw[Q];
+    uint32_t lo[Q], hi[Q];
+    if (Q == 4) {
+      const v4f s4 = *reinterpret_cast<const v4f*>(frac + 4 * cq);
+      const v4u l4 = *reinterpret_cast<const v4u*>(lo_b + 4 * cq);
+      const v4u h4 = *reinterpret_cast<const v4u*>(hi_b + 4 * cq);
+#pragma unroll
+      for (int j = 0; j < Q; ++j) sw[j] = s4[j], lo[j] = l4[j], hi[j] = h4[j];
+    } else {
+      sw[0] = frac[cq], lo[0] = lo_b[cq], hi[0] = hi_b[cq];
+    }
+    float res[Q];
+#pragma unroll
+    for (int j = 0; j < Q; ++j) {
+      const float v0 = *reinterpret_cast<const float*>(row_l + lo[j]);
+      const float v1 = *reinterpret_cast<const float*>(row_h + lo[j]);
+      const float v2 = *reinterpret_cast<const float*>(row_l + hi[j]);
+      const float v3 = *reinterpret_cast<const float*>(row_h + hi[j]);
+      const float iw = 1 - sw[j];
+      const float a0 = ih * iw, a1 = sh * iw, a2 = ih * sw[j], a3 = sh * sw[j];
+      const float t0 = a0 * v0, t1 = a1 * v1, t2 = a2 * v2, t3 = a3 * v3;
+      const float s01 = t0 + t1;
+      const float s012 = s01 + t2;
+      res[j] = s012 + t3;
+    }
+    float* dst = out + static_cast<uint64_t>(r) * p.out_w + Q * cq;
+    if (Q == 4)
+      store4_stream(dst, v4f{res[0], res[Q > 1 ? 1 : 0], res[Q > 2 ? 2 : 0], res[Q > 3 ? 3 : 0]});
+    else
+      dst[0] = res[0];
+  }
+}
+
+// Band height and tile size for the kernel above; false when even a one-row
+// band does not fit (very wide rows or a strong vertical reduction).
+template <bool ALIGN>
+static bool plan_resize_band(int planes, int in_h, int in_w, int out_h, int out_w, float fh,
+                             ResizeBandArgs* p, size_t* lds_bytes) {
+  const size_t table_bytes = 3 * static_cast<size_t>((out_w + 3) & ~3) * 4;
+  int rows = std::max(1, std::min(out_h, kResizeBandOutputs / out_w));
+  while (rows > 1 && static_cast<int64_t>(planes) * ((out_h + rows - 1) / rows) < kResizeBandGroups)
+    rows = (rows + 1) / 2;
+  for (;; rows = (rows + 1) / 2) {
+    int tile_rows = 1;
+    for (int h0 = 0; h0 < out_h; h0 += rows) {
+      int first, last, unused;
+      float unused_f;
+      bilinear_axis<ALIGN>(static_cast<uint32_t>(h0), fh, in_h, first, unused, unused_f);
+      bilinear_axis<ALIGN>(static_cast<uint32_t>(std::min(h0 + rows, out_h) - 1), fh, in_h, unused, last,
+                           unused_f);
+      tile_rows = std::max(tile_rows, last - first + 1);
+    }
+    const size_t bytes = table_bytes + static_cast<size_t>(tile_rows) * in_w * 4;
+    if (bytes <= static_cast<size_t>(kResizeBandLdsBytes) || (rows == 1 && bytes <= kResizeBandMaxLdsBytes)) {
+      p->rows = rows, p->tile_rows = tile_rows;
+      p->f_bands = make_fastdiv((out_h + rows - 1) / rows);
+      *lds_bytes = bytes;
+      return true;
+    }
+    if (rows == 1) return false;
+  }
+}
+
+template <bool ALIGN>
+static bool launch_resize_band(int planes, int in_h, int in_w, int out_h, int out_w, float fh, float fw,
+                               bool quad, const float* x, float* y, hipStream_t st) {
+  ResizeBandArgs p;
+  size_t lds_bytes;
+  if (!plan_resize_band<ALIGN>(planes, in_h, in_w, out_h, out_w, fh, &p, &lds_bytes)) return false;
+  p.in_h = in_h, p.in_w = in_w, p.out_h = out_h, p.out_w = out_w, p.fh = fh, p.fw = fw;
+  const uint32_t grid = static_cast<uint32_t>(planes) * p.f_bands.d;
+  if (quad) {
+    p.f_cols = make_fastdiv(out_w / 4);
+    resize_bilinear_band_kernel<ALIGN, 4><<<grid, kBlock, lds_bytes, st>>>(x, y, p);
+  } else {
+    p.f_cols = make_fastdiv(out_w);
+    resize_bilinear_band_kernel<ALIGN, 1><<<grid, kBlock, lds_bytes, st>>>(x, y, p);
+  }
+  return true;
 }
 
 static bool count_fits(const int* shape, int n, int64_t* count) {
@@ -629,9 +792,12 @@ int shdw_hip_resize(const int* in_shape, const int* out_shape, int type, int ali
   const bool quad = out_w % 4 == 0 && aligned16(y);
   const uint32_t work = quad ? n / 4 : n;
   const uint32_t grid = grid_for(work);
+  const int planes = in_shape[0] * in_shape[1];
   if (type == 1 && align_corners) {
     p.fh = static_cast<float>(in_h - 1) / (out_h - 1);
     p.fw = static_cast<float>(in_w - 1) / (out_w - 1);
+    if (launch_resize_band<true>(planes, in_h, in_w, out_h, out_w, p.fh, p.fw, quad, x, y, st))
+      return launch_status();
     if (quad)
       resize_bilinear_kernel<true, 4><<<grid, kBlock, 0, st>>>(x, y, work, p);
     else
@@ -644,6 +810,8 @@ int shdw_hip_resize(const int* in_shape, const int* out_shape, int type, int ali
         resize_nearest_kernel<4><<<grid, kBlock, 0, st>>>(x, y, work, p);
       else
         resize_nearest_kernel<1><<<grid, kBlock, 0, st>>>(x, y, work, p);
+    } else if (launch_resize_band<false>(planes, in_h, in_w, out_h, out_w, p.fh, p.fw, quad, x, y, st)) {
+      return launch_status();
     } else if (quad) {
       resize_bilinear_kernel<false, 4><<<grid, kBlock, 0, st>>>(x, y, work, p);
     } else {

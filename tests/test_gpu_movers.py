@@ -126,6 +126,23 @@ def test_reorg_op(ws, type_, shape, stride):
     assert_bit_exact(got, want, "reorg")
 
 
+@pytest.mark.parametrize("align", [False, True])
+@pytest.mark.parametrize("shape,size", [
+    ((3, 5, 56, 56), [112, 112]),    # several bands per plane, 128-bit both sides
+    ((2, 3, 57, 33), [114, 66]),     # rows that are not a multiple of four floats
+    ((1, 2, 120, 64), [17, 40]),     # reduction by 7: a band spans many input rows
+    ((1, 1, 300, 5), [2, 10]),       # two output rows 150 input rows apart
+    ((1, 1, 4, 6000), [8, 9000]),    # rows too wide for the staged kernel: gather kernel
+    ((2, 2, 9, 2100), [5, 4100]),    # one-row bands with a large tile
+    ((1, 3, 200, 31), [333, 77])])   # odd output width: one output per lane
+def test_resize_bilinear_bands(ws, shape, size, align):
+    x = normal(91, shape, 2.0)
+    got = run(ws, "Resize", [("x", x)], {"size": size, "align_corners": align})
+    want = oracle.resize_op(x, size, [1.0], 1, align)
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "resize %s -> %s" % (shape, size))
+
+
 @pytest.mark.parametrize("shape,group", [((2, 6, 3, 5), 2), ((2, 6, 3, 5), 3), ((1, 12, 4, 4), 4), ((3, 8, 1, 1), 8),
                                          ((2, 116, 28, 28), 2), ((2, 6, 3, 5), 1)])
 def test_shuffle_channel_op(ws, shape, group):
