@@ -406,6 +406,20 @@ def config_table(dev):
     ms = time_batch(dev, lambda k: lib.shdw_hip_group_norm(65536, 784, 1e-5, AH[k].ptr, lns.ptr, lnb.ptr,
                                                            784, 1, YH[k].ptr, st), SH, reps=20)
     add("next", "layer_norm affine [65536,784]", 8 * NH + 8 * 784, ms, NH)
+    # SSDNormalize on the SSD conv4_3 map, batch 64: 8 bytes per element are compulsory
+    # (the per-item form reads x a second time on top of that)
+    NS = 64 * 512 * 1444
+    ssc = dev.buf(uniform(618, 512, 10.0, 30.0))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_ssd_normalize(64, 512, 1444, 0, 1e-5, AH[k].ptr, ssc.ptr, 0,
+                                                              YH[k].ptr, None, st), SH, reps=20)
+    add("next", "ssd_normalize per position, channel scale [64,512,38,38]", 8 * NS + 4 * 512, ms, NS)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_ssd_normalize(64, 256, 3136, 0, 1e-5, AH[k].ptr, ssc.ptr, 0,
+                                                              YH[k].ptr, None, st), SH, reps=20)
+    add("next", "ssd_normalize per position, channel scale [64,256,56,56]", 8 * NH + 4 * 256, ms, NH)
+    swb = dev.buf(nbytes=max(8, lib.shdw_hip_ssd_normalize_workspace_bytes(64, 512, 1444, 1)))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_ssd_normalize(64, 512, 1444, 1, 1e-5, AH[k].ptr, ssc.ptr, 0,
+                                                              YH[k].ptr, swb.ptr, st), SH, reps=20)
+    add("next", "ssd_normalize per item, channel scale [64,512,38,38] (2 launches)", 8 * NS + 4 * 512, ms, NS)
     # data movers ("movers") on the same 205 MB tensors
     half = NH // 2
     def concat2(k):

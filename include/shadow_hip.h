@@ -260,6 +260,29 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
 int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps,
                        const float* x, float* y, void* stream);
 
+/* SSDNormalize with its optional scale, one call for SSDNormalizeKernel::Run.
+ *   across_spatial == 0: every position (b, s) is divided by
+ *     (float) sqrt((double) sum_c x^2 + eps), the squares formed in fp32 and
+ *     summed in fp64 in channel order (bit-exact);
+ *   across_spatial != 0: every item b is multiplied by
+ *     1 / sqrt((float) sum x^2 + eps), all fp32 after the fp64 sum; the sum is
+ *     associated differently from the reference's loop (same contract as
+ *     shdw_hip_asum).  Needs `workspace` of
+ *     shdw_hip_ssd_normalize_workspace_bytes(...) bytes, 8-byte aligned; it is
+ *     written and read on `stream`, nothing returns to the host.
+ * scale: NULL, one value (channel_shared != 0: out *= scale[0]) or `channels`
+ * values (out * scale[c]), applied to the normalised value as a second fp32
+ * product.  It is read on the device: no synchronisation (the reference copies a
+ * shared scale to the host first).  y may alias x.
+ * ref: shadow/operators/kernels/ssd_normalize.hpp:36-83 (Square, Sasum, Mul,
+ *      Sscal, Scale), ssd_normalize.cpp:7-29 (the oracle; ssd_normalize.cu:7-43 takes the
+ *      square root in fp32 instead, sqrtf((float) sum + eps)) */
+size_t shdw_hip_ssd_normalize_workspace_bytes(int batch, int channels, int spatial_dim,
+                                              int across_spatial);
+int shdw_hip_ssd_normalize(int batch, int channels, int spatial_dim, int across_spatial, float eps,
+                           const float* x, const float* scale, int channel_shared, float* y,
+                           void* workspace, void* stream);
+
 /* Pooling over [N][C][H][W] (2d) or [N][C][D][H][W] (3d); shapes are HOST arrays
  * of 4 / 5 ints and out_shape is what the operator computed.  pool_type 0 = max
  * (start at lowest(), keep unless smaller), 1 = average: fp32 running sum in

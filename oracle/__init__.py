@@ -205,6 +205,18 @@ def normalize(x, outer, dim, inner, p, eps):
     return out
 
 
+def ssd_normalize(x, batch, channel, spatial_dim, across_spatial, channel_shared, eps, scale=None):
+    """SSDNormalizeKernelDefault::Run on flat data."""
+    x = _f(x).ravel()
+    out = np.empty_like(x)
+    val = np.empty(max(1, batch * spatial_dim), np.float32)
+    sc = None if scale is None else _f(scale).ravel()
+    lib().orc_ssd_normalize_run(_p(x), int(batch), int(channel), int(spatial_dim), int(bool(across_spatial)),
+                                int(bool(channel_shared)), ctypes.c_float(eps),
+                                _p(sc) if sc is not None else None, _p(val), _p(out))
+    return out
+
+
 def pooling(x, in_shape, pool_type, kernel, stride, pad, out_shape):
     """2-D or 3-D by len(kernel)."""
     x = _f(x).ravel()
@@ -392,6 +404,21 @@ def normalize_op(x, p=2.0, axis=1, eps=1e-12):
     outer = int(np.prod(x.shape[:axis], dtype=np.int64))
     inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
     return normalize(x, outer, x.shape[axis], inner, np.float32(p), np.float32(eps)).reshape(x.shape)
+
+
+def ssd_normalize_op(x, scale=None, across_spatial=True, channel_shared=True, eps=1e-5):
+    """shadow/operators/ssd_normalize_op.cpp:9-38 and kernels/ssd_normalize.hpp:36-83"""
+    x = _f(x)
+    _check(x.ndim >= 2, "SSDNormalize needs [batch, channel, ...]")
+    spatial = int(np.prod(x.shape[2:], dtype=np.int64))
+    if scale is not None:
+        scale = _f(scale).ravel()
+        if channel_shared:
+            _check(scale.size == 1, "scale->count() == 1")
+        else:
+            _check(scale.size >= x.shape[1], "one scale value per channel")
+    return ssd_normalize(x, x.shape[0], x.shape[1], spatial, across_spatial, channel_shared, np.float32(eps),
+                         scale).reshape(x.shape)
 
 
 def pooling_op(x, pool=0, kernel_size=(), stride=(1,), pad=(0,), global_pooling=False,

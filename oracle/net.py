@@ -233,6 +233,11 @@ def _run_op(op, blobs):
         return oracle.softmax_op(x[0], _single(a, "axis", 1))
     if t == "Normalize":
         return oracle.normalize_op(x[0], _single(a, "p", F(2)), _single(a, "axis", 1), _single(a, "eps", F(1e-12)))
+    if t == "SSDNormalize":
+        oracle._check(len(x) in (1, 2), "inputs.size() == 2")
+        return oracle.ssd_normalize_op(x[0], x[1] if len(x) == 2 else None,
+                                       bool(_single(a, "across_spatial", True)),
+                                       bool(_single(a, "channel_shared", True)), _single(a, "eps", F(1e-5)))
     if t == "Pooling":
         return oracle.pooling_op(x[0], _single(a, "pool", 0), _repeated(a, "kernel_size", [0]),
                                  _repeated(a, "stride", [1]), _repeated(a, "pad", [0]),

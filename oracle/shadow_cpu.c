@@ -385,6 +385,52 @@ API void orc_normalize(const float* in, int outer_num, int dim, int inner_num, f
   }
 }
 
+/* ---- shadow/operators/kernels/ssd_normalize.cpp:7-29  Vision::SSDNormalize: `out`
+ *      holds the squares on entry; fp64 running sum over the channels, fp64
+ *      square root, then in / val ---- */
+API void orc_ssd_normalize(const float* in, int outer_num, int channels, int inner_num, float eps,
+                           float* val, float* out) {
+  int val_count = outer_num * inner_num, count = val_count * channels;
+  for (int i = 0; i < val_count; ++i) {
+    int n = i / inner_num, s = i % inner_num;
+    const float* q = out + n * channels * inner_num + s;
+    double sum = 0;
+    for (int c = 0; c < channels; ++c, q += inner_num) sum += *q;
+    val[i] = (float)sqrt(sum + eps);
+  }
+  for (int i = 0; i < count; ++i) {
+    int n = i / channels / inner_num, s = i % inner_num;
+    out[i] = in[i] / val[n * inner_num + s];
+  }
+}
+
+/* ---- shadow/operators/kernels/ssd_normalize.hpp:36-83
+ *      SSDNormalizeKernelDefault::Run: Square into the output, then per item
+ *      Sasum and Mul by 1 / sqrt(sum + eps) (all fp32 after the sum) or the
+ *      per-position form above; then Sscal by the shared scale or Scale by the
+ *      per-channel one.  scale may be NULL.  val: batch * spatial_dim floats. ---- */
+API void orc_ssd_normalize_run(const float* in, int batch, int channel, int spatial_dim,
+                               int across_spatial, int channel_shared, float eps,
+                               const float* scale, float* val, float* out) {
+  int num = channel * spatial_dim, count = batch * num;
+  orc_unary(1, count, in, out); /* Square */
+  if (across_spatial) {
+    for (int b = 0; b < batch; ++b) {
+      int offset = b * num;
+      float sum = orc_asum(num, out + offset);
+      orc_binary_scalar(2, num, in + offset, 1.f / sqrtf(sum + eps), out + offset); /* Mul */
+    }
+  } else {
+    orc_ssd_normalize(in, batch, channel, spatial_dim, eps, val, out);
+  }
+  if (scale) {
+    if (channel_shared)
+      orc_scal(count, scale[0], out);
+    else
+      orc_scale(out, count, scale, channel, spatial_dim, out);
+  }
+}
+
 /* ---- shadow/operators/kernels/pooling.cpp:7-42  Vision::Pooling2D.
  *      pool_type 0 = max, 1 = average over the window clipped to input + pad ---- */
 API void orc_pooling2d(const float* in, const int* in_shape, int pool_type, int kernel_h,

@@ -77,6 +77,8 @@ SIGNATURES = {
     "shdw_hip_group_norm": (_I, [_I, _I, _F, _V, _V, _V, _I, _I, _V, _V]),
     "shdw_hip_softmax": (_I, [_I, _I, _I, _V, _V, _V]),
     "shdw_hip_normalize": (_I, [_I, _I, _I, _F, _F, _V, _V, _V]),
+    "shdw_hip_ssd_normalize_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "shdw_hip_ssd_normalize": (_I, [_I, _I, _I, _I, _F, _V, _V, _I, _V, _V, _V]),
     "shdw_hip_pooling2d": (_I, [c_int_p, _I, _I, _I, _I, _I, _I, _I, c_int_p, _V, _V, _V]),
     "shdw_hip_pooling3d": (_I, [c_int_p, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, c_int_p, _V, _V, _V]),
     "shdw_hip_copy_chunks": (_I, [_I, _I, _V, _I, _I, _V, _I, _I, _V]),

@@ -37,6 +37,19 @@ SHDW_DEVICE bool aligned16_device(const void* p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }
 
+// Workgroups are handed to the 8 XCDs (accelerator dies, each with its own L2)
+// round-robin by blockIdx.x, so workgroups b and b + 1 never share an L2.  A
+// kernel whose neighbouring work items touch the same cache lines (halo rows,
+// rows that straddle a line) renumbers its workgroups with this map: XCD x then
+// owns one contiguous range of work items and the shared lines are fetched from
+// HBM once.  A bijection of [0, grid) for every grid size.
+constexpr uint32_t kXcds = 8;
+SHDW_DEVICE uint32_t xcd_contiguous(uint32_t block, uint32_t grid) {
+  const uint32_t x = block % kXcds, slot = block / kXcds;
+  const uint32_t q = grid / kXcds, r = grid % kXcds;
+  return x * q + (x < r ? x : r) + slot;
+}
+
 // ---------------------------------------------------------------------------
 // Division of a 31-bit unsigned value by a divisor fixed at launch time:
 //   q = (mulhi(n, m) + n) >> s

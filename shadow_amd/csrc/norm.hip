@@ -21,6 +21,8 @@
 // GroupNorm's channel is computed once per 128-bit vector.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include "../../include/shadow_hip.h"
 #include "device_common.h"
 #include "launch.h"
@@ -229,6 +231,118 @@ __global__ __launch_bounds__(kBlock) void norm_rows_stream_kernel(const float* x
   }
 }
 
+// ---------------------------------------------------------------------------
+// SSDNormalize across the whole item (shadow/operators/kernels/
+// ssd_normalize.hpp:47-57): the reference squares x into the output, takes
+// Sasum of each item on the host (fp64 running sum, blas.cpp:229-233) and
+// multiplies the item by 1 / sqrt(sum + eps), all in fp32 after the sum.  An
+// item is usually megabytes long, so its sum is split over `parts` workgroups
+// that each fold a fixed segment (fp64 per lane, shuffles, LDS) into a slot of
+// the workspace; the second kernel adds the slots in index order, forms the
+// factor and applies it, with the optional scale of ssd_normalize.hpp:68-80 in
+// the same pass.  Nothing returns to the host in between.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kSsdSegmentQuantum = 4 * kBlock;  // keeps every segment 16-byte aligned
+constexpr uint32_t kSsdMinSegment = 4 * kSsdSegmentQuantum;
+constexpr uint32_t kSsdMaxParts = 64;
+constexpr uint32_t kSsdGroupsWanted = 2048;
+
+struct SsdRowPlan {
+  uint32_t parts, segment;
+};
+
+static SsdRowPlan plan_ssd_rows(uint32_t batch, uint32_t num) {
+  uint32_t parts = std::min(kSsdMaxParts, (kSsdGroupsWanted + batch - 1) / std::max(batch, 1u));
+  parts = std::max(1u, std::min(parts, num / kSsdMinSegment));
+  uint32_t segment = (num + parts - 1) / parts;
+  segment = (segment + kSsdSegmentQuantum - 1) / kSsdSegmentQuantum * kSsdSegmentQuantum;
+  SsdRowPlan plan;
+  plan.segment = segment;
+  plan.parts = std::max(1u, (num + segment - 1) / segment);
+  return plan;
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void ssd_row_partials_kernel(const float* x, double* partials,
+                                                                   uint32_t num, uint32_t segment) {
+  __shared__ double slots[kBlock / kWave];
+  const uint32_t begin = blockIdx.x * segment;
+  const uint32_t end = min(num, begin + segment);
+  const float* xr = x + static_cast<uint64_t>(blockIdx.y) * num;
+  double acc = 0;
+  if (VEC) {
+    for (uint32_t t = begin / 4 + threadIdx.x; t < end / 4; t += kBlock) {
+      const v4f q = load4(xr + 4ull * t);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float sq = q[j] * q[j];
+        acc += static_cast<double>(sq);
+      }
+    }
+  } else {
+    for (uint32_t t = begin + threadIdx.x; t < end; t += kBlock) {
+      const float sq = xr[t] * xr[t];
+      acc += static_cast<double>(sq);
+    }
+  }
+  const double total = row_sum<kBlock>(acc, slots);
+  if (threadIdx.x == 0) partials[blockIdx.y * gridDim.x + blockIdx.x] = total;
+}
+
+// SM: 0 no scale, 1 one shared factor (Sscal), 2 one factor per channel.
+template <bool VEC, int SM>
+__global__ __launch_bounds__(kBlock) void ssd_row_scale_kernel(const float* x, float* y,
+                                                                const double* partials, uint32_t parts,
+                                                                uint32_t num, float eps,
+                                                                const float* scale, FastDiv f_spatial) {
+  const double* mine = partials + blockIdx.y * parts;  // uniform: scalar loads
+  double sum = 0;
+  for (uint32_t k = 0; k < parts; ++k) sum += mine[k];
+  const float sum_f = static_cast<float>(sum);
+  const float se = sum_f + eps;
+  const float factor = 1.f / __builtin_sqrtf(se);
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint64_t base = static_cast<uint64_t>(blockIdx.y) * num;
+  if (VEC) {
+    if (i >= num / 4) return;
+    const v4f q = load4_stream(x + base + 4ull * i);
+    v4f r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      r[j] = q[j] * factor;
+      if (SM == 1) r[j] = r[j] * scale[0];
+      if (SM == 2) r[j] = r[j] * scale[fd_div(4 * i + j, f_spatial)];
+    }
+    store4_stream(y + base + 4ull * i, r);
+  } else {
+    if (i >= num) return;
+    float r = x[base + i] * factor;
+    if (SM == 1) r = r * scale[0];
+    if (SM == 2) r = r * scale[fd_div(i, f_spatial)];
+    y[base + i] = r;
+  }
+}
+
+template <bool VEC>
+static void launch_ssd_rows(uint32_t batch, uint32_t num, uint32_t spatial, float eps, const float* x,
+                            const float* scale, int channel_shared, float* y, double* partials,
+                            hipStream_t st) {
+  const SsdRowPlan plan = plan_ssd_rows(batch, num);
+  ssd_row_partials_kernel<VEC><<<dim3(plan.parts, batch), kBlock, 0, st>>>(x, partials, num, plan.segment);
+  const dim3 grid(grid_for(VEC ? num / 4 : num), batch);
+  const FastDiv fs = make_fastdiv(std::max(spatial, 1u));
+  if (!scale)
+    ssd_row_scale_kernel<VEC, 0><<<grid, kBlock, 0, st>>>(x, y, partials, plan.parts, num, eps, scale, fs);
+  else if (channel_shared)
+    ssd_row_scale_kernel<VEC, 1><<<grid, kBlock, 0, st>>>(x, y, partials, plan.parts, num, eps, scale, fs);
+  else
+    ssd_row_scale_kernel<VEC, 2><<<grid, kBlock, 0, st>>>(x, y, partials, plan.parts, num, eps, scale, fs);
+}
+
+// softmax.hip: the per-position form shares the Normalize column kernels.
+int ssd_normalize_columns(int outer_num, int dim, int inner_num, float eps, const float* x,
+                          const float* scale, int channel_shared, float* y, hipStream_t st);
+
 }  // namespace shdw
 
 using namespace shdw;
@@ -290,6 +404,38 @@ int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
   } else {
     norm_rows_stream_kernel<true><<<rows, kBlock, 0, st>>>(x, y, p);
   }
+  return launch_status();
+}
+
+size_t shdw_hip_ssd_normalize_workspace_bytes(int batch, int channels, int spatial_dim,
+                                              int across_spatial) {
+  if (!across_spatial || batch <= 0 || channels <= 0 || spatial_dim <= 0) return 0;
+  const int64_t num = static_cast<int64_t>(channels) * spatial_dim;
+  if (num * batch > INT32_MAX) return 0;
+  const SsdRowPlan plan = plan_ssd_rows(static_cast<uint32_t>(batch), static_cast<uint32_t>(num));
+  return static_cast<size_t>(batch) * plan.parts * sizeof(double);
+}
+
+int shdw_hip_ssd_normalize(int batch, int channels, int spatial_dim, int across_spatial, float eps,
+                           const float* x, const float* scale, int channel_shared, float* y,
+                           void* workspace, void* stream) {
+  if (batch < 0 || channels < 0 || spatial_dim < 0) return SHDW_E_INVALID_ARGUMENT;
+  const int64_t num = static_cast<int64_t>(channels) * spatial_dim;
+  if (num > INT32_MAX || num * batch > INT32_MAX) return SHDW_E_INVALID_ARGUMENT;
+  if (num * batch == 0) return SHDW_OK;
+  if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!across_spatial)
+    return ssd_normalize_columns(batch, channels, spatial_dim, eps, x, scale, channel_shared, y, st);
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 7u)) return SHDW_E_INVALID_ARGUMENT;
+  double* partials = static_cast<double*>(workspace);
+  const bool vec = num % 4 == 0 && aligned16(x) && aligned16(y);
+  if (vec)
+    launch_ssd_rows<true>(batch, static_cast<uint32_t>(num), spatial_dim, eps, x, scale, channel_shared, y,
+                          partials, st);
+  else
+    launch_ssd_rows<false>(batch, static_cast<uint32_t>(num), spatial_dim, eps, x, scale, channel_shared, y,
+                           partials, st);
   return launch_status();
 }
 

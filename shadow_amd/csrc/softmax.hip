@@ -202,7 +202,21 @@ __global__ __launch_bounds__(kBlock) void softmax_slab_kernel(const float* x, fl
 // ---------------------------------------------------------------------------
 // Normalize (shadow/operators/kernels/normalize.cpp:10-43)
 //   PMODE 1: sum |x|          2: sqrt(sum |x|^2)      0: (sum |x|^p)^(1/p)
+// SSDNormalize over channels (shadow/operators/kernels/ssd_normalize.cpp:14-28,
+// squares from Blas::Square, ssd_normalize.hpp:47) shares the kernels:
+//   PMODE 3: (float) sqrt((double) sum x^2 + eps) in fp64, no lower bound, and
+//            the optional scale of ssd_normalize.hpp:68-80 applied to the quotient.
 // ---------------------------------------------------------------------------
+enum SsdScale { kSsdNoScale = 0, kSsdSharedScale = 1, kSsdChannelScale = 2 };
+
+// SM is kSsdNoScale for Normalize; c is the channel (the position in the column).
+template <int SM>
+SHDW_DEVICE float ssd_scaled(float v, const float* scale, uint32_t c) {
+  if (SM == kSsdSharedScale) return v * scale[0];
+  if (SM == kSsdChannelScale) return v * scale[c];
+  return v;
+}
+
 template <int PMODE>
 SHDW_DEVICE double norm_term(float v, float p) {
   const float a = __builtin_fabsf(v);
@@ -211,12 +225,17 @@ SHDW_DEVICE double norm_term(float v, float p) {
     const float sq = a * a;  // fp32 product, widened afterwards
     return static_cast<double>(sq);
   }
+  if (PMODE == 3) {
+    const float sq = v * v;
+    return static_cast<double>(sq);
+  }
   return static_cast<double>(libm::exact_powf(a, p, libm::kExp2fTab));
 }
 
 template <int PMODE>
 SHDW_DEVICE float norm_finish(double acc, float p, float eps) {
   float val;
+  if (PMODE == 3) return static_cast<float>(__builtin_sqrt(acc + static_cast<double>(eps)));
   if (PMODE == 1) {
     val = static_cast<float>(acc);
   } else if (PMODE == 2) {
@@ -228,12 +247,21 @@ SHDW_DEVICE float norm_finish(double acc, float p, float eps) {
   return std_max(val, eps);
 }
 
-template <int PMODE>
-__global__ __launch_bounds__(kBlock) void normalize_columns_kernel(const float* x, float* y,
-                                                                    uint32_t columns, uint32_t dim,
-                                                                    FastDiv f_inner, float p,
-                                                                    float eps) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+// Any column length: a lane walks its column twice (the second time from cache
+// where the column still is there).  kColumnBatch loads are issued before the
+// first is consumed so that a lane keeps that many requests in flight, and a
+// workgroup is a single wave: long columns mean few of them, and 64 columns per
+// workgroup spread them over four times as many CUs.  Neighbouring waves share
+// the cache lines their 256-byte rows straddle, hence the XCD-contiguous order.
+constexpr int kColumnBatch = 16;
+
+template <int PMODE, int SM = kSsdNoScale>
+__global__ __launch_bounds__(kWave) void normalize_columns_kernel(const float* x, float* y,
+                                                                   uint32_t columns, uint32_t dim,
+                                                                   FastDiv f_inner, float p,
+                                                                   float eps,
+                                                                   const float* scale = nullptr) {
+  const uint32_t i = xcd_contiguous(blockIdx.x, gridDim.x) * kWave + threadIdx.x;
   if (i >= columns) return;
   uint32_t n, s;
   fd_divmod(i, f_inner, n, s);
@@ -242,18 +270,35 @@ __global__ __launch_bounds__(kBlock) void normalize_columns_kernel(const float* 
   const float* xc = x + base;
   float* yc = y + base;
   double acc = 0;
-  for (uint32_t c = 0; c < dim; ++c) acc += norm_term<PMODE>(xc[static_cast<uint64_t>(c) * inner], p);
+  for (uint32_t c0 = 0; c0 < dim; c0 += kColumnBatch) {
+    float v[kColumnBatch];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u)
+      if (c0 + u < dim) v[u] = xc[static_cast<uint64_t>(c0 + u) * inner];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u)
+      if (c0 + u < dim) acc += norm_term<PMODE>(v[u], p);
+  }
   const float div = norm_finish<PMODE>(acc, p, eps);
-  for (uint32_t c = 0; c < dim; ++c)
-    yc[static_cast<uint64_t>(c) * inner] = xc[static_cast<uint64_t>(c) * inner] / div;
+  for (uint32_t c0 = 0; c0 < dim; c0 += kColumnBatch) {
+    float v[kColumnBatch];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u)
+      if (c0 + u < dim) v[u] = xc[static_cast<uint64_t>(c0 + u) * inner];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u)
+      if (c0 + u < dim)
+        __builtin_nontemporal_store(ssd_scaled<SM>(v[u] / div, scale, c0 + u), yc + static_cast<uint64_t>(c0 + u) * inner);
+  }
 }
 
-template <int PMODE, int DMAX>
+template <int PMODE, int DMAX, int SM = kSsdNoScale>
 __global__ __launch_bounds__(kBlock) void normalize_columns_reg_kernel(const float* x, float* y,
                                                                         uint32_t columns,
                                                                         uint32_t dim,
                                                                         FastDiv f_inner, float p,
-                                                                        float eps) {
+                                                                        float eps,
+                                                                        const float* scale = nullptr) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
   if (i >= columns) return;
   uint32_t n, s;
@@ -273,15 +318,17 @@ __global__ __launch_bounds__(kBlock) void normalize_columns_reg_kernel(const flo
   const float div = norm_finish<PMODE>(acc, p, eps);
 #pragma unroll
   for (int c = 0; c < DMAX; ++c)
-    if (c < dim) __builtin_nontemporal_store(v[c] / div, yc + static_cast<uint64_t>(c) * inner);
+    if (c < dim)
+      __builtin_nontemporal_store(ssd_scaled<SM>(v[c] / div, scale, c), yc + static_cast<uint64_t>(c) * inner);
 }
 
 // The slab in LDS holds the per-element terms (|x|, |x|^2 or |x|^p, computed by
 // all lanes); x itself is read again for the division, from L2.
-template <int PMODE>
+template <int PMODE, int SM = kSsdNoScale>
 __global__ __launch_bounds__(kBlock) void normalize_slab_kernel(const float* x, float* y,
                                                                  uint32_t dim, FastDiv f_inner,
-                                                                 float p, float eps) {
+                                                                 float p, float eps,
+                                                                 const float* scale = nullptr) {
   extern __shared__ __align__(16) float lds[];
   const uint32_t inner = f_inner.d;
   const uint32_t slab = dim * inner;
@@ -301,9 +348,133 @@ __global__ __launch_bounds__(kBlock) void normalize_slab_kernel(const float* x, 
   }
   __syncthreads();
   for (uint32_t t = threadIdx.x; t < slab; t += kBlock) {
-    const uint32_t s = t - fd_div(t, f_inner) * inner;
-    ys[t] = xs[t] / stat[s];
+    const uint32_t c = fd_div(t, f_inner);
+    const uint32_t s = t - c * inner;
+    ys[t] = ssd_scaled<SM>(xs[t] / stat[s], scale, c);
   }
+}
+
+// Columns of 65 to 512 elements over a wide inner extent: a workgroup owns a
+// tile of TS = 64 or 32 neighbouring positions with all their `dim`
+// elements, 64 KB at most, so x is read from HBM once.  Each lane keeps its
+// share of the tile (16 vectors at most) in registers and also parks it in LDS;
+// wave 0 folds the TS columns from LDS in index order, one column per lane, and
+// then overwrites the first tile row with the TS divisors (nobody else reads
+// the tile, and the fold is done with it); after the barrier every lane divides
+// its registers.  Only one SIMD pays for the serial fold, the other waves of
+// the CU keep their SIMDs free for the second resident workgroup.
+// p other than 1 and 2 is not taken here: powf per element inside the serial
+// fold would dominate.
+constexpr int kTilePerLane = 16;  // 64 KB / (256 lanes x 16 bytes)
+
+template <int PMODE, int SM, bool VEC, int TS_SHIFT>
+__global__ __launch_bounds__(kBlock) void normalize_tile_kernel(const float* x, float* y, uint32_t dim,
+                                                                 uint32_t inner, FastDiv f_tiles, float p,
+                                                                 float eps, const float* scale) {
+  extern __shared__ __align__(16) float lds[];
+  constexpr uint32_t TS = 1u << TS_SHIFT;
+  uint32_t n, tile;
+  // neighbouring tiles share the cache lines their 64..256-byte rows straddle
+  fd_divmod(xcd_contiguous(blockIdx.x, gridDim.x), f_tiles, n, tile);
+  const uint32_t p0 = tile << TS_SHIFT;
+  const uint32_t width = min(TS, inner - p0);
+  const uint64_t base = static_cast<uint64_t>(n) * dim * inner + p0;
+  const float* xs = x + base;
+  float* ys = y + base;
+  // VEC: a lane owns the 4 positions j..j+3 of rows c0, c0 + step, ...;
+  // otherwise position j of four times as many rows.
+  constexpr uint32_t LANES_PER_ROW = VEC ? TS / 4 : TS;
+  constexpr uint32_t STEP = kBlock / LANES_PER_ROW;
+  constexpr int UNITS = VEC ? kTilePerLane : 4 * kTilePerLane;
+  const uint32_t j = (threadIdx.x & (LANES_PER_ROW - 1)) * (VEC ? 4 : 1);
+  const uint32_t c0 = threadIdx.x / LANES_PER_ROW;
+  const bool mine = j < width;
+  v4f rv[VEC ? kTilePerLane : 1];
+  float rs[VEC ? 1 : 4 * kTilePerLane];
+  if (mine) {
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+      const uint32_t c = c0 + u * STEP;
+      if (c < dim) {
+        if (VEC)
+          rv[u] = load4_stream(xs + static_cast<uint64_t>(c) * inner + j);
+        else
+          rs[u] = __builtin_nontemporal_load(xs + static_cast<uint64_t>(c) * inner + j);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+      const uint32_t c = c0 + u * STEP;
+      if (c < dim) {
+        if (VEC)
+          *reinterpret_cast<v4f*>(lds + (c << TS_SHIFT) + j) = rv[u];
+        else
+          lds[(c << TS_SHIFT) + j] = rs[u];
+      }
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < width) {  // width <= TS <= 64: lanes of wave 0, one column each
+    const float* column = lds + threadIdx.x;
+    double acc = 0;
+#pragma unroll 16
+    for (uint32_t c = 0; c < dim; ++c) acc += norm_term<PMODE>(column[c << TS_SHIFT], p);
+    lds[threadIdx.x] = norm_finish<PMODE>(acc, p, eps);
+  }
+  __syncthreads();
+  if (!mine) return;
+  if (VEC) {
+    const v4f d = *reinterpret_cast<const v4f*>(lds + j);
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+      const uint32_t c = c0 + u * STEP;
+      if (c < dim) {
+        v4f r;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) r[k] = ssd_scaled<SM>(rv[u][k] / d[k], scale, c);
+        store4_stream(ys + static_cast<uint64_t>(c) * inner + j, r);
+      }
+    }
+  } else {
+    const float d = lds[j];
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+      const uint32_t c = c0 + u * STEP;
+      if (c < dim)
+        __builtin_nontemporal_store(ssd_scaled<SM>(rs[u] / d, scale, c), ys + static_cast<uint64_t>(c) * inner + j);
+    }
+  }
+}
+
+constexpr int kTileMinDim = 65, kTileMaxDim = 512, kTileMinInner = 16;  // beyond 512 a tile row is 64 bytes
+constexpr int kTileLdsBytes = 65536;
+
+static bool tile_fits(int dim, int inner_num) {
+  return dim >= kTileMinDim && dim <= kTileMaxDim && inner_num >= kTileMinInner;
+}
+
+template <int PMODE, int SM, int TS_SHIFT>
+static void launch_normalize_tile_ts(int outer_num, int dim, int inner_num, float p, float eps, const float* x,
+                                     const float* scale, float* y, hipStream_t st) {
+  const uint32_t tiles = (static_cast<uint32_t>(inner_num) + (1u << TS_SHIFT) - 1) >> TS_SHIFT;
+  const uint32_t grid = static_cast<uint32_t>(outer_num) * tiles;
+  const size_t bytes = (static_cast<size_t>(dim) << TS_SHIFT) * sizeof(float);
+  const FastDiv ft = make_fastdiv(tiles);
+  const uint32_t d = static_cast<uint32_t>(dim), in = static_cast<uint32_t>(inner_num);
+  if (inner_num % 4 == 0 && aligned16(x) && aligned16(y))
+    normalize_tile_kernel<PMODE, SM, true, TS_SHIFT><<<grid, kBlock, bytes, st>>>(x, y, d, in, ft, p, eps, scale);
+  else
+    normalize_tile_kernel<PMODE, SM, false, TS_SHIFT><<<grid, kBlock, bytes, st>>>(x, y, d, in, ft, p, eps, scale);
+}
+
+template <int PMODE, int SM>
+static void launch_normalize_tile(int outer_num, int dim, int inner_num, float p, float eps, const float* x,
+                                  const float* scale, float* y, hipStream_t st) {
+  // the widest tile whose dim rows fit 64 KB
+  if (dim * 64 * sizeof(float) <= kTileLdsBytes)
+    launch_normalize_tile_ts<PMODE, SM, 6>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
+  else
+    launch_normalize_tile_ts<PMODE, SM, 5>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
 }
 
 // Shared launch geometry: slab layout when the columns are too narrow to
@@ -375,6 +546,11 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
       normalize_slab_kernel<2><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
     else
       normalize_slab_kernel<0><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
+  } else if (mode != 0 && tile_fits(dim, inner_num)) {
+    if (mode == 1)
+      launch_normalize_tile<1, kSsdNoScale>(outer_num, dim, inner_num, p, eps, x, nullptr, y, st);
+    else
+      launch_normalize_tile<2, kSsdNoScale>(outer_num, dim, inner_num, p, eps, x, nullptr, y, st);
   } else if (dim <= 64 && mode != 0) {
     // p = 1 and p = 2 keep short columns in registers (one read, one write);
     // the generic-p form would unroll a powf per element and stays two-pass.
@@ -391,15 +567,56 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
         normalize_columns_reg_kernel<2, 64><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
     }
   } else {
-    const uint32_t grid = grid_for(g.columns);
+    const uint32_t grid = (g.columns + kWave - 1) / kWave;
     if (mode == 1)
-      normalize_columns_kernel<1><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
+      normalize_columns_kernel<1><<<grid, kWave, 0, st>>>(x, y, g.columns, d, fi, p, eps);
     else if (mode == 2)
-      normalize_columns_kernel<2><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
+      normalize_columns_kernel<2><<<grid, kWave, 0, st>>>(x, y, g.columns, d, fi, p, eps);
     else
-      normalize_columns_kernel<0><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
+      normalize_columns_kernel<0><<<grid, kWave, 0, st>>>(x, y, g.columns, d, fi, p, eps);
   }
   return launch_status();
 }
 
 }  // extern "C"
+
+namespace shdw {
+
+// SSDNormalize over the channels of every position; called from
+// shdw_hip_ssd_normalize (norm.hip owns the across-spatial form).
+template <int SM>
+static void launch_ssd_columns(const ColumnGeometry& g, int outer_num, int dim, int inner_num, float eps,
+                               const float* x, const float* scale, float* y, hipStream_t st) {
+  const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
+  const uint32_t d = static_cast<uint32_t>(dim);
+  const uint32_t grid = grid_for(g.columns);
+  if (g.use_slab)
+    normalize_slab_kernel<3, SM><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, 2.f, eps, scale);
+  else if (tile_fits(dim, inner_num))
+    launch_normalize_tile<3, SM>(outer_num, dim, inner_num, 2.f, eps, x, scale, y, st);
+  else if (dim <= 16)
+    normalize_columns_reg_kernel<3, 16, SM><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, 2.f, eps, scale);
+  else if (dim <= 64)
+    normalize_columns_reg_kernel<3, 64, SM><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, 2.f, eps, scale);
+  else
+    normalize_columns_kernel<3, SM><<<(g.columns + kWave - 1) / kWave, kWave, 0, st>>>(x, y, g.columns, d, fi, 2.f,
+                                                                                  eps, scale);
+}
+
+int ssd_normalize_columns(int outer_num, int dim, int inner_num, float eps, const float* x,
+                          const float* scale, int channel_shared, float* y, hipStream_t st) {
+  ColumnGeometry g;
+  const int rc = column_geometry(outer_num, dim, inner_num, &g);
+  if (rc != SHDW_OK) return rc;
+  if (g.columns == 0 || dim == 0) return SHDW_OK;
+  if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
+  if (!scale)
+    launch_ssd_columns<kSsdNoScale>(g, outer_num, dim, inner_num, eps, x, scale, y, st);
+  else if (channel_shared)
+    launch_ssd_columns<kSsdSharedScale>(g, outer_num, dim, inner_num, eps, x, scale, y, st);
+  else
+    launch_ssd_columns<kSsdChannelScale>(g, outer_num, dim, inner_num, eps, x, scale, y, st);
+  return launch_status();
+}
+
+}  // namespace shdw

@@ -228,6 +228,20 @@ def normalize(x, outer, dim, inner, p, eps, inplace=False):
     return y.download(count=x.size)
 
 
+def ssd_normalize(x, batch, channel, spatial, across_spatial, channel_shared, eps, scale=None, inplace=False):
+    x = _f(x).ravel()
+    dx = Buffer.from_numpy(x)
+    y = dx if inplace else Buffer(max(4, x.nbytes))
+    ds = None if scale is None else Buffer.from_numpy(_f(scale).ravel())
+    nbytes = _lib().shdw_hip_ssd_normalize_workspace_bytes(batch, channel, spatial, int(across_spatial))
+    ws = Buffer(nbytes) if nbytes else None
+    check(_lib().shdw_hip_ssd_normalize(batch, channel, spatial, int(across_spatial), eps, dx.ptr,
+                                        ds.ptr if ds else None, int(channel_shared), y.ptr,
+                                        ws.ptr if ws else None, None))
+    _sync()
+    return y.download(count=x.size)
+
+
 def pooling(x, in_shape, pool_type, kernel, stride, pad, out_shape):
     """2-D or 3-D by len(kernel)."""
     x = _f(x).ravel()

@@ -110,8 +110,8 @@ def keys(fn):
 def test_registries_hold_exactly_the_gpu_default_kernels():
     h = shadow_amd.host()
     kernels = ["Activate", "Axpy", "BatchNorm", "Binary", "Concat", "Eltwise", "Gather", "GroupNorm", "LayerNorm",
-               "Normalize", "Pad", "Permute", "Pooling", "Reduce", "Reorg", "Resize", "Scale", "ShuffleChannel",
-               "Slice", "Softmax", "Stack", "Unary"]
+               "Normalize", "Pad", "Permute", "Pooling", "Reduce", "Reorg", "Resize", "SSDNormalize", "Scale",
+               "ShuffleChannel", "Slice", "Softmax", "Stack", "Unary"]
     # InstanceNorm runs on the GroupNorm kernel (shadow/operators/instance_norm_op.cpp:14)
     # and the view-only operators need no kernel
     assert keys(h.shdw_host_operator_keys) == sorted(
@@ -148,6 +148,15 @@ def test_entry_points_validate_before_touching_the_device():
     assert lib.shdw_hip_softmax(0, 5, 5, None, None, None) == 0
     assert lib.shdw_hip_normalize(65536, 65536, 2, 2.0, 0.0, p, p, None) == E
     assert lib.shdw_hip_batch_norm(8, 0, 1, p, p, p, 1.0, 0.0, p, None) == E
+    assert lib.shdw_hip_ssd_normalize(2, -1, 4, 0, 1e-5, p, None, 1, p, None, None) == E
+    assert lib.shdw_hip_ssd_normalize(2, 65536, 65536, 0, 1e-5, p, None, 1, p, None, None) == E
+    assert lib.shdw_hip_ssd_normalize(2, 8, 4, 1, 1e-5, p, None, 1, p, None, None) == E   # no workspace
+    assert lib.shdw_hip_ssd_normalize(2, 8, 4, 1, 1e-5, p, None, 1, p, ctypes.c_void_p(4100), None) == E
+    assert lib.shdw_hip_ssd_normalize(2, 8, 4, 0, 1e-5, None, None, 1, p, None, None) == E
+    assert lib.shdw_hip_ssd_normalize(0, 8, 4, 1, 1e-5, None, None, 1, None, None, None) == 0
+    assert lib.shdw_hip_ssd_normalize_workspace_bytes(8, 512, 1444, 0) == 0
+    assert 8 * 8 < lib.shdw_hip_ssd_normalize_workspace_bytes(8, 512, 1444, 1) <= 8 * 64 * 8  # several parts per item
+    assert lib.shdw_hip_ssd_normalize_workspace_bytes(4096, 2, 8, 1) == 4096 * 8
     assert lib.shdw_hip_batch_norm(0, 4, 1, None, None, None, 1.0, 0.0, None, None) == 0
     assert lib.shdw_hip_axpy_rows(65536, 65536, p, p, p, p, None) == E
     assert lib.shdw_hip_axpy_rows(4, 4, None, p, p, p, None) == E

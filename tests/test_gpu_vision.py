@@ -125,7 +125,10 @@ def test_softmax_op_defaults_and_errors(ws):
 # -------------------------------------------------------------- normalize ---
 @pytest.mark.parametrize("p", [1.0, 2.0, 3.0, 0.5])
 @pytest.mark.parametrize("outer,dim,inner", [(64, 512, 1), (5, 7, 3), (2, 16, 100), (3, 9, 64), (1, 20000, 1),
-                                             (2, 1, 9), (1, 33, 4097)])
+                                             (2, 1, 9), (1, 33, 4097),
+                                             # 65..1024 deep over a wide inner extent: tiles of 64, 32, 16 positions
+                                             (2, 100, 100), (1, 512, 72), (3, 300, 37), (2, 1024, 20), (1, 65, 4097),
+                                             (2, 256, 64), (1, 1025, 40)])
 def test_normalize(gpu, p, outer, dim, inner):
     x = normal(17, outer * dim * inner, 2.0)
     want = oracle.normalize(x, outer, dim, inner, p, 1e-12)
@@ -150,6 +153,70 @@ def test_normalize_op(ws, args):
     want = oracle.normalize_op(x, args.get("p", 2.0), args.get("axis", 1), args.get("eps", 1e-12))
     assert got.shape == x.shape
     assert_bit_exact(got, want, "normalize op")
+
+
+# ----------------------------------------------------------- SSDNormalize ---
+SSD_SHAPES = [(2, 5, 12), (3, 512, 1), (2, 16, 100), (3, 9, 64), (1, 600, 3), (2, 1, 9), (1, 33, 4097),
+              (2, 64, 1444), (5, 3, 7), (1, 128, 4096), (3, 20, 1025), (2, 512, 361), (1, 1000, 50), (2, 70, 33),
+              (1, 512, 1444), (2, 1030, 24)]
+
+
+@pytest.mark.parametrize("scale_kind", ["none", "shared", "channel"])
+@pytest.mark.parametrize("batch,channel,spatial", SSD_SHAPES)
+def test_ssd_normalize_per_position(gpu, batch, channel, spatial, scale_kind):
+    """Channel sums fold in index order on one lane: no tolerance."""
+    x = normal(60, batch * channel * spatial, 2.0)
+    scale = {"none": None, "shared": F([20.0]), "channel": normal(61, channel) + F(20)}[scale_kind]
+    shared = scale_kind != "channel"
+    want = oracle.ssd_normalize(x, batch, channel, spatial, False, shared, 1e-5, scale)
+    assert_bit_exact(gpuops.ssd_normalize(x, batch, channel, spatial, False, shared, 1e-5, scale), want, "ssd")
+    assert_bit_exact(gpuops.ssd_normalize(x, batch, channel, spatial, False, shared, 1e-5, scale, inplace=True), want,
+                     "ssd in place")
+
+
+@pytest.mark.parametrize("scale_kind", ["none", "shared", "channel"])
+@pytest.mark.parametrize("batch,channel,spatial", SSD_SHAPES + [(2, 512, 1444), (70, 8, 2048), (3, 7, 11111)])
+def test_ssd_normalize_per_item(gpu, batch, channel, spatial, scale_kind):
+    """The item's fp64 sum is split over workgroups and lanes: 1e-5 relative, and
+    the count of differing outputs (none in these cases) is checked as well."""
+    x = normal(62, batch * channel * spatial, 2.0) + F(0.25)
+    scale = {"none": None, "shared": F([20.0]), "channel": normal(63, channel) + F(20)}[scale_kind]
+    shared = scale_kind != "channel"
+    want = oracle.ssd_normalize(x, batch, channel, spatial, True, shared, 1e-5, scale)
+    got = gpuops.ssd_normalize(x, batch, channel, spatial, True, shared, 1e-5, scale)
+    assert assert_rel_close(got, want, 1e-5, "ssd per item") == 0
+    got = gpuops.ssd_normalize(x, batch, channel, spatial, True, shared, 1e-5, scale, inplace=True)
+    assert assert_rel_close(got, want, 1e-5, "ssd per item in place") == 0
+
+
+def test_ssd_normalize_special_values(gpu):
+    x = with_specials(normal(64, 6 * 32 * 10, 2.0), 64)
+    for across in (False, True):
+        for eps in (1e-5, 0.0):
+            want = oracle.ssd_normalize(x, 6, 32, 10, across, True, eps)
+            assert_bit_exact(gpuops.ssd_normalize(x, 6, 32, 10, across, True, eps), want,
+                             "ssd specials across=%s eps=%g" % (across, eps))
+    z = np.zeros(4 * 6 * 5, F)
+    for across in (False, True):
+        for eps in (1e-5, 0.0):
+            assert_bit_exact(gpuops.ssd_normalize(z, 4, 6, 5, across, True, eps),
+                             oracle.ssd_normalize(z, 4, 6, 5, across, True, eps), "ssd zeros")
+
+
+@pytest.mark.parametrize("args", [{}, {"across_spatial": False}, {"across_spatial": False, "channel_shared": False},
+                                  {"channel_shared": False, "eps": 1e-3}])
+def test_ssd_normalize_op(ws, args):
+    x = normal(65, (3, 24, 9, 7), 2.0)
+    across, shared, eps = args.get("across_spatial", True), args.get("channel_shared", True), args.get("eps", 1e-5)
+    scale = F([20.0]) if shared else uniform(66, 24, 10.0, 30.0)
+    got = run(ws, "SSDNormalize", [("x", x)], args)
+    assert got.shape == x.shape
+    assert assert_rel_close(got, oracle.ssd_normalize_op(x, None, across, shared, eps), 1e-5, "ssd op") == 0
+    got = run(ws, "SSDNormalize", [("x", x), ("s", scale)], args)
+    assert assert_rel_close(got, oracle.ssd_normalize_op(x, scale, across, shared, eps), 1e-5, "ssd op scale") == 0
+    if shared:
+        with pytest.raises(ShadowError, match="Check Failed"):
+            run(ws, "SSDNormalize", [("x", x), ("s2", F([1.0, 2.0]))], args)
 
 
 # ---------------------------------------------------------------- pooling ---

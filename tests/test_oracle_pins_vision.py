@@ -145,6 +145,73 @@ def test_normalize_known_values():
     assert out.ravel().tolist() == [F(1e-30) / F(1e-12)] * 2
 
 
+# ----------------------------------------------------------- SSDNormalize ---
+def ssd_numpy(x, scale, across_spatial, channel_shared, eps):
+    """Array formulation with numpy's own rounded operations."""
+    eps = F(eps)
+    sq = x * x  # fp32 squares
+    if across_spatial:
+        flat = sq.reshape(x.shape[0], -1)
+        total = running_sum(flat, 1, np.float64).astype(F)        # Sasum: fp64 fold, fp32 result
+        factor = F(1) / np.sqrt(total + eps, dtype=F)             # fp32 add, sqrt, divide
+        out = x * factor.reshape((-1,) + (1,) * (x.ndim - 1))
+    else:
+        total = running_sum(sq, 1, np.float64)                    # stays fp64
+        val = np.sqrt(total + np.float64(eps)).astype(F)          # fp64 add and sqrt
+        out = x / np.expand_dims(val, 1)
+    if scale is not None:
+        sc = scale.ravel()
+        out = out * sc[0] if channel_shared else out * sc[:x.shape[1]].reshape((1, -1) + (1,) * (x.ndim - 2))
+    return out.astype(F)
+
+
+@pytest.mark.parametrize("across", [False, True])
+@pytest.mark.parametrize("scale_kind", ["none", "shared", "channel"])
+@pytest.mark.parametrize("shape", [(2, 5, 3, 4), (3, 7, 1, 1), (1, 33, 6, 2), (2, 3, 9)])
+def test_ssd_normalize_against_array_formulation(across, scale_kind, shape):
+    x = normal(40, shape, 3.0)
+    scale = {"none": None, "shared": F([20.0]), "channel": normal(41, (shape[1],)) + F(20)}[scale_kind]
+    got = oracle.ssd_normalize_op(x, scale, across, scale_kind != "channel", 1e-5)
+    assert_bit_exact(got, ssd_numpy(x, scale, across, scale_kind != "channel", 1e-5), "ssd %s" % scale_kind)
+
+
+def test_ssd_normalize_known_values():
+    # per position: four equal channels, 1.5 / sqrt(4 * 2.25) = 0.5 exactly
+    x = np.full((1, 4, 2, 2), 1.5, F)
+    assert (oracle.ssd_normalize_op(x, None, False, True, 0.0) == F(0.5)).all()
+    # per item: 16 values of 1.5, 1 / sqrt(36) rounded, times 1.5, times the shared scale
+    want = F(1.5) * (F(1) / np.sqrt(F(36), dtype=F)) * F(20)
+    assert (oracle.ssd_normalize_op(x, F([20]), True, True, 0.0) == want).all()
+    # eps sits inside the square root, not under a max: a zero item gives 0 * (1 / sqrt(eps))
+    z = np.zeros((1, 2, 2, 2), F)
+    assert (oracle.ssd_normalize_op(z, None, True, True, 1e-5) == 0).all()
+    assert (oracle.ssd_normalize_op(z, None, False, True, 1e-5) == 0).all()
+    with np.errstate(all="ignore"):
+        assert np.isnan(oracle.ssd_normalize_op(z, None, False, True, 0.0)).all()  # 0 / 0
+    # the per-position root is taken in fp64 and rounded once: an fp32 root of the fp32
+    # sum is a different number for some columns
+    x = normal(42, (1, 16, 64, 64), 2.0)
+    got = oracle.ssd_normalize_op(x, None, False, True, 1e-5)
+    sq = x * x
+    total32 = running_sum(sq, 1, np.float64).astype(F)
+    other = x / np.expand_dims(np.sqrt(total32 + F(1e-5), dtype=F), 1)
+    assert (got.view(np.uint32) != other.view(np.uint32)).any()
+    # both arguments default to true in the operator (ssd_normalize_op.cpp:11-12)
+    assert_bit_exact(oracle.ssd_normalize_op(x, F([3])), oracle.ssd_normalize_op(x, F([3]), True, True, 1e-5), "defaults")
+
+
+def test_ssd_normalize_unit_norm_and_scale_checks():
+    x = normal(43, (3, 8, 5, 5), 4.0)
+    per_item = oracle.ssd_normalize_op(x, None, True, True, 0.0).astype(np.float64)
+    np.testing.assert_allclose((per_item ** 2).reshape(3, -1).sum(1), 1.0, rtol=1e-5)
+    per_pos = oracle.ssd_normalize_op(x, None, False, True, 0.0).astype(np.float64)
+    np.testing.assert_allclose((per_pos ** 2).sum(1), 1.0, rtol=1e-5)
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.ssd_normalize_op(x, F([1, 2]), True, True)   # shared scale holds one value
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.ssd_normalize_op(x, F([1, 2]), True, False)  # fewer values than channels
+
+
 # ---------------------------------------------------------------- pooling ---
 def pooling_numpy(x, pool, kernel, stride, pad, out_shape):
     """Window by slicing; running fp32 sum over the flattened window."""
