@@ -392,6 +392,12 @@ def config_table(dev):
     add("next", "pooling_global_avg_7x7 [512,2048,7,7]", 4 * (NH + 512 * 2048), ms, NH)
     ms = time_batch(dev, lambda k: lib.shdw_hip_softmax(64, 49, 16384, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
     add("next", "softmax_channels_dense [64,49,128,128]", 8 * NH, ms, NH)
+    NSEG = 64 * 150 * 5329  # a 150-class segmentation head, 73 x 73
+    ms = time_batch(dev, lambda k: lib.shdw_hip_softmax(64, 150, 5329, AH[k].ptr, YH[k].ptr, st), SH, reps=10)
+    add("next", "softmax_150_classes [64,150,73,73]", 8 * NSEG, ms, NSEG)
+    NSEG = 64 * 150 * 5184  # the same head on 72 x 72: rows of whole 128-bit vectors
+    ms = time_batch(dev, lambda k: lib.shdw_hip_softmax(64, 150, 5184, AH[k].ptr, YH[k].ptr, st), SH, reps=10)
+    add("next", "softmax_150_classes [64,150,72,72]", 8 * NSEG, ms, NSEG)
     ms = time_batch(dev, lambda k: lib.shdw_hip_normalize(64, 49, 16384, 2.0, 1e-12, AH[k].ptr, YH[k].ptr, st),
                     SH, reps=20)
     add("next", "normalize_l2_channels_dense [64,49,128,128]", 8 * NH, ms, NH)

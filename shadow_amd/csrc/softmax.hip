@@ -32,13 +32,22 @@ SHDW_DEVICE float std_max(float a, float b) { return a < b ? b : a; }
 // ---------------------------------------------------------------------------
 // Softmax (shadow/operators/kernels/softmax.cpp:10-42)
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void softmax_columns_kernel(const float* x, float* y,
-                                                                  uint32_t columns, uint32_t dim,
-                                                                  FastDiv f_inner) {
+// Any column length: a lane walks its column three times (max, exp and running
+// sum, divide).  kColumnBatch loads are issued before the first is consumed so
+// that a lane keeps that many requests in flight, and a workgroup is a single
+// wave: long columns mean few of them, and 64 columns per workgroup spread them
+// over four times as many CUs.  Neighbouring waves share the cache lines their
+// 256-byte rows straddle, hence the XCD-contiguous order.  Every fold keeps the
+// reference's index order.
+constexpr int kColumnBatch = 16;
+
+__global__ __launch_bounds__(kWave) void softmax_columns_kernel(const float* x, float* y,
+                                                                 uint32_t columns, uint32_t dim,
+                                                                 FastDiv f_inner) {
   __shared__ uint64_t tab[32];
   if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
   __syncthreads();
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t i = xcd_contiguous(blockIdx.x, gridDim.x) * kWave + threadIdx.x;
   if (i >= columns) return;
   uint32_t n, s;
   fd_divmod(i, f_inner, n, s);
@@ -47,14 +56,39 @@ __global__ __launch_bounds__(kBlock) void softmax_columns_kernel(const float* x,
   const float* xc = x + base;
   float* yc = y + base;
   float max_val = -FLT_MAX;
-  for (uint32_t c = 0; c < dim; ++c) max_val = std_max(xc[static_cast<uint64_t>(c) * inner], max_val);
-  float sum = 0.f;
-  for (uint32_t c = 0; c < dim; ++c) {
-    const float e = libm::exact_expf(xc[static_cast<uint64_t>(c) * inner] - max_val, tab);
-    yc[static_cast<uint64_t>(c) * inner] = e;
-    sum += e;
+  for (uint32_t c0 = 0; c0 < dim; c0 += kColumnBatch) {
+    float v[kColumnBatch];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u)
+      if (c0 + u < dim) v[u] = xc[static_cast<uint64_t>(c0 + u) * inner];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u)
+      if (c0 + u < dim) max_val = std_max(v[u], max_val);
   }
-  for (uint32_t c = 0; c < dim; ++c) yc[static_cast<uint64_t>(c) * inner] /= sum;
+  float sum = 0.f;
+  for (uint32_t c0 = 0; c0 < dim; c0 += kColumnBatch) {
+    float v[kColumnBatch];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u)
+      if (c0 + u < dim) v[u] = xc[static_cast<uint64_t>(c0 + u) * inner];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u) {
+      if (c0 + u < dim) {
+        const float e = libm::exact_expf(v[u] - max_val, tab);
+        yc[static_cast<uint64_t>(c0 + u) * inner] = e;
+        sum += e;
+      }
+    }
+  }
+  for (uint32_t c0 = 0; c0 < dim; c0 += kColumnBatch) {
+    float v[kColumnBatch];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u)
+      if (c0 + u < dim) v[u] = yc[static_cast<uint64_t>(c0 + u) * inner];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u)
+      if (c0 + u < dim) __builtin_nontemporal_store(v[u] / sum, yc + static_cast<uint64_t>(c0 + u) * inner);
+  }
 }
 
 // Same layout for dim <= DMAX: the column lives in registers, so x is read once
@@ -248,12 +282,7 @@ SHDW_DEVICE float norm_finish(double acc, float p, float eps) {
 }
 
 // Any column length: a lane walks its column twice (the second time from cache
-// where the column still is there).  kColumnBatch loads are issued before the
-// first is consumed so that a lane keeps that many requests in flight, and a
-// workgroup is a single wave: long columns mean few of them, and 64 columns per
-// workgroup spread them over four times as many CUs.  Neighbouring waves share
-// the cache lines their 256-byte rows straddle, hence the XCD-contiguous order.
-constexpr int kColumnBatch = 16;
+// where the column still is there), launched like softmax_columns_kernel.
 
 template <int PMODE, int SM = kSsdNoScale>
 __global__ __launch_bounds__(kWave) void normalize_columns_kernel(const float* x, float* y,
@@ -355,64 +384,93 @@ __global__ __launch_bounds__(kBlock) void normalize_slab_kernel(const float* x, 
 }
 
 // Columns of 65 to 512 elements over a wide inner extent: a workgroup owns a
-// tile of TS = 64 or 32 neighbouring positions with all their `dim`
-// elements, 64 KB at most, so x is read from HBM once.  Each lane keeps its
-// share of the tile (16 vectors at most) in registers and also parks it in LDS;
-// wave 0 folds the TS columns from LDS in index order, one column per lane, and
-// then overwrites the first tile row with the TS divisors (nobody else reads
-// the tile, and the fold is done with it); after the barrier every lane divides
+// tile of TS = 64 or 32 neighbouring positions with all their `dim` elements,
+// 64 KB at most, so x is read from HBM once.  Each lane keeps its share of the
+// tile (16 vectors of 4 positions at most) in registers and also parks it in
+// LDS; wave 0 folds the TS columns from LDS in index order, one column per lane,
+// and hands the TS results over in the first tile row (nobody else reads the
+// tile, and the fold is done with it); after the barrier every lane finishes
 // its registers.  Only one SIMD pays for the serial fold, the other waves of
-// the CU keep their SIMDs free for the second resident workgroup.
+// the CU keep their SIMDs free for the other resident workgroups.
+//
+// Rows of the tile start wherever inner and the tile offset put them, so the
+// 128-bit global accesses are only 4-byte aligned (the hardware splits the ones
+// that straddle a line; that is still far cheaper than four 4-byte accesses per
+// lane, which run at the address-unit rate: 185 us against 84 us on
+// [64,150,73,73] / [64,150,72,72]).  Neighbouring tiles share the straddled
+// lines, hence the XCD-contiguous workgroup order.
+constexpr int kTilePerLane = 16;  // 64 KB / (256 lanes x 16 bytes)
+typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+
+// TAIL: inner % 4 != 0, so a tile row may end inside a lane's four positions.
+template <int TS_SHIFT, bool TAIL>
+struct TileLane {
+  static constexpr uint32_t TS = 1u << TS_SHIFT;
+  static constexpr uint32_t LANES_PER_ROW = TS / 4;
+  static constexpr uint32_t STEP = kBlock / LANES_PER_ROW;  // rows between a lane's vectors
+  uint32_t j, c0, valid;  // first position, first row, positions of j..j+3 inside the tile
+  uint32_t dim, inner;
+
+  SHDW_DEVICE TileLane(uint32_t width, uint32_t dim_, uint32_t inner_) : dim(dim_), inner(inner_) {
+    j = (threadIdx.x & (LANES_PER_ROW - 1)) * 4;
+    c0 = threadIdx.x / LANES_PER_ROW;
+    valid = j < width ? min(4u, width - j) : 0u;
+  }
+  SHDW_DEVICE void load(const float* xs, v4f (&r)[kTilePerLane]) const {
+    if (valid == 0) return;
+#pragma unroll
+    for (int u = 0; u < kTilePerLane; ++u) {
+      const uint32_t c = c0 + u * STEP;
+      if (c >= dim) continue;
+      const float* src = xs + static_cast<uint64_t>(c) * inner + j;
+      if (!TAIL || valid == 4) {
+        r[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f_unaligned*>(src));
+      } else {
+        r[u] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+          if (k < valid) r[u][k] = src[k];
+      }
+    }
+  }
+  SHDW_DEVICE void park(float* lds, const v4f (&r)[kTilePerLane]) const {
+    if (valid == 0) return;
+#pragma unroll
+    for (int u = 0; u < kTilePerLane; ++u) {
+      const uint32_t c = c0 + u * STEP;
+      if (c < dim) *reinterpret_cast<v4f*>(lds + (c << TS_SHIFT) + j) = r[u];
+    }
+  }
+  SHDW_DEVICE void store(float* ys, uint32_t u, v4f v) const {
+    const uint32_t c = c0 + u * STEP;
+    float* dst = ys + static_cast<uint64_t>(c) * inner + j;
+    if (!TAIL || valid == 4) {
+      __builtin_nontemporal_store(v, reinterpret_cast<v4f_unaligned*>(dst));
+    } else {
+#pragma unroll
+      for (int k = 0; k < 3; ++k)
+        if (k < valid) dst[k] = v[k];
+    }
+  }
+};
+
 // p other than 1 and 2 is not taken here: powf per element inside the serial
 // fold would dominate.
-constexpr int kTilePerLane = 16;  // 64 KB / (256 lanes x 16 bytes)
-
-template <int PMODE, int SM, bool VEC, int TS_SHIFT>
+template <int PMODE, int SM, int TS_SHIFT, bool TAIL>
 __global__ __launch_bounds__(kBlock) void normalize_tile_kernel(const float* x, float* y, uint32_t dim,
                                                                  uint32_t inner, FastDiv f_tiles, float p,
                                                                  float eps, const float* scale) {
   extern __shared__ __align__(16) float lds[];
   constexpr uint32_t TS = 1u << TS_SHIFT;
   uint32_t n, tile;
-  // neighbouring tiles share the cache lines their 64..256-byte rows straddle
   fd_divmod(xcd_contiguous(blockIdx.x, gridDim.x), f_tiles, n, tile);
   const uint32_t p0 = tile << TS_SHIFT;
   const uint32_t width = min(TS, inner - p0);
   const uint64_t base = static_cast<uint64_t>(n) * dim * inner + p0;
-  const float* xs = x + base;
-  float* ys = y + base;
-  // VEC: a lane owns the 4 positions j..j+3 of rows c0, c0 + step, ...;
-  // otherwise position j of four times as many rows.
-  constexpr uint32_t LANES_PER_ROW = VEC ? TS / 4 : TS;
-  constexpr uint32_t STEP = kBlock / LANES_PER_ROW;
-  constexpr int UNITS = VEC ? kTilePerLane : 4 * kTilePerLane;
-  const uint32_t j = (threadIdx.x & (LANES_PER_ROW - 1)) * (VEC ? 4 : 1);
-  const uint32_t c0 = threadIdx.x / LANES_PER_ROW;
-  const bool mine = j < width;
-  v4f rv[VEC ? kTilePerLane : 1];
-  float rs[VEC ? 1 : 4 * kTilePerLane];
-  if (mine) {
-#pragma unroll
-    for (int u = 0; u < UNITS; ++u) {
-      const uint32_t c = c0 + u * STEP;
-      if (c < dim) {
-        if (VEC)
-          rv[u] = load4_stream(xs + static_cast<uint64_t>(c) * inner + j);
-        else
-          rs[u] = __builtin_nontemporal_load(xs + static_cast<uint64_t>(c) * inner + j);
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < UNITS; ++u) {
-      const uint32_t c = c0 + u * STEP;
-      if (c < dim) {
-        if (VEC)
-          *reinterpret_cast<v4f*>(lds + (c << TS_SHIFT) + j) = rv[u];
-        else
-          lds[(c << TS_SHIFT) + j] = rs[u];
-      }
-    }
-  }
+  const TileLane<TS_SHIFT, TAIL> lane(width, dim, inner);
+  v4f r[kTilePerLane];
+  lane.load(x + base, r);
+  lane.park(lds, r);
   __syncthreads();
   if (threadIdx.x < width) {  // width <= TS <= 64: lanes of wave 0, one column each
     const float* column = lds + threadIdx.x;
@@ -422,27 +480,16 @@ __global__ __launch_bounds__(kBlock) void normalize_tile_kernel(const float* x, 
     lds[threadIdx.x] = norm_finish<PMODE>(acc, p, eps);
   }
   __syncthreads();
-  if (!mine) return;
-  if (VEC) {
-    const v4f d = *reinterpret_cast<const v4f*>(lds + j);
+  if (lane.valid == 0) return;
+  const v4f d = *reinterpret_cast<const v4f*>(lds + lane.j);
 #pragma unroll
-    for (int u = 0; u < UNITS; ++u) {
-      const uint32_t c = c0 + u * STEP;
-      if (c < dim) {
-        v4f r;
+  for (int u = 0; u < kTilePerLane; ++u) {
+    const uint32_t c = lane.c0 + u * lane.STEP;
+    if (c >= dim) continue;
+    v4f q;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) r[k] = ssd_scaled<SM>(rv[u][k] / d[k], scale, c);
-        store4_stream(ys + static_cast<uint64_t>(c) * inner + j, r);
-      }
-    }
-  } else {
-    const float d = lds[j];
-#pragma unroll
-    for (int u = 0; u < UNITS; ++u) {
-      const uint32_t c = c0 + u * STEP;
-      if (c < dim)
-        __builtin_nontemporal_store(ssd_scaled<SM>(rs[u] / d, scale, c), ys + static_cast<uint64_t>(c) * inner + j);
-    }
+    for (int k = 0; k < 4; ++k) q[k] = ssd_scaled<SM>(r[u][k] / d[k], scale, c);
+    lane.store(y + base, u, q);
   }
 }
 
@@ -459,12 +506,13 @@ static void launch_normalize_tile_ts(int outer_num, int dim, int inner_num, floa
   const uint32_t tiles = (static_cast<uint32_t>(inner_num) + (1u << TS_SHIFT) - 1) >> TS_SHIFT;
   const uint32_t grid = static_cast<uint32_t>(outer_num) * tiles;
   const size_t bytes = (static_cast<size_t>(dim) << TS_SHIFT) * sizeof(float);
-  const FastDiv ft = make_fastdiv(tiles);
   const uint32_t d = static_cast<uint32_t>(dim), in = static_cast<uint32_t>(inner_num);
-  if (inner_num % 4 == 0 && aligned16(x) && aligned16(y))
-    normalize_tile_kernel<PMODE, SM, true, TS_SHIFT><<<grid, kBlock, bytes, st>>>(x, y, d, in, ft, p, eps, scale);
+  if (inner_num % 4 == 0)
+    normalize_tile_kernel<PMODE, SM, TS_SHIFT, false><<<grid, kBlock, bytes, st>>>(x, y, d, in, make_fastdiv(tiles),
+                                                                                 p, eps, scale);
   else
-    normalize_tile_kernel<PMODE, SM, false, TS_SHIFT><<<grid, kBlock, bytes, st>>>(x, y, d, in, ft, p, eps, scale);
+    normalize_tile_kernel<PMODE, SM, TS_SHIFT, true><<<grid, kBlock, bytes, st>>>(x, y, d, in, make_fastdiv(tiles),
+                                                                                p, eps, scale);
 }
 
 template <int PMODE, int SM>
@@ -475,6 +523,83 @@ static void launch_normalize_tile(int outer_num, int dim, int inner_num, float p
     launch_normalize_tile_ts<PMODE, SM, 6>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
   else
     launch_normalize_tile_ts<PMODE, SM, 5>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
+}
+
+// Softmax on the same tile layout (65 <= dim <= 511 so that the exp table fits
+// beside the tile).  The lanes hold x, later exp(x - max), in registers; the tile
+// in LDS serves wave 0's two serial folds: the running maximum of x, then the
+// fp32 running sum of the exponentials, both in index order.  The maxima and
+// then the sums are handed over in the first tile row.
+template <int TS_SHIFT, bool TAIL>
+__global__ __launch_bounds__(kBlock) void softmax_tile_kernel(const float* x, float* y, uint32_t dim,
+                                                               uint32_t inner, FastDiv f_tiles) {
+  extern __shared__ __align__(16) float lds[];
+  constexpr uint32_t TS = 1u << TS_SHIFT;
+  uint64_t* tab = reinterpret_cast<uint64_t*>(lds + (dim << TS_SHIFT));  // after the tile, 16-byte aligned
+  if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
+  uint32_t n, tile;
+  fd_divmod(xcd_contiguous(blockIdx.x, gridDim.x), f_tiles, n, tile);
+  const uint32_t p0 = tile << TS_SHIFT;
+  const uint32_t width = min(TS, inner - p0);
+  const uint64_t base = static_cast<uint64_t>(n) * dim * inner + p0;
+  const TileLane<TS_SHIFT, TAIL> lane(width, dim, inner);
+  v4f r[kTilePerLane];
+  lane.load(x + base, r);
+  lane.park(lds, r);
+  __syncthreads();
+  if (threadIdx.x < width) {
+    const float* column = lds + threadIdx.x;
+    float max_val = -FLT_MAX;
+#pragma unroll 16
+    for (uint32_t c = 0; c < dim; ++c) max_val = std_max(column[c << TS_SHIFT], max_val);
+    lds[threadIdx.x] = max_val;
+  }
+  __syncthreads();
+  const v4f m = *reinterpret_cast<const v4f*>(lds + lane.j);
+  __syncthreads();  // the maxima are read before the exponentials overwrite their row
+  if (lane.valid != 0) {
+#pragma unroll
+    for (int u = 0; u < kTilePerLane; ++u) {
+      if (lane.c0 + u * lane.STEP >= dim) continue;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) r[u][k] = libm::exact_expf(r[u][k] - m[k], tab);
+    }
+  }
+  lane.park(lds, r);
+  __syncthreads();
+  if (threadIdx.x < width) {
+    const float* column = lds + threadIdx.x;
+    float sum = 0.f;
+#pragma unroll 16
+    for (uint32_t c = 0; c < dim; ++c) sum += column[c << TS_SHIFT];
+    lds[threadIdx.x] = sum;
+  }
+  __syncthreads();
+  if (lane.valid == 0) return;
+  const v4f d = *reinterpret_cast<const v4f*>(lds + lane.j);
+#pragma unroll
+  for (int u = 0; u < kTilePerLane; ++u) {
+    if (lane.c0 + u * lane.STEP >= dim) continue;
+    v4f q;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) q[k] = r[u][k] / d[k];
+    lane.store(y + base, u, q);
+  }
+}
+
+constexpr int kSoftmaxTileMaxDim = 511;  // 511 x 32 positions + the exp table <= 64 KB
+
+template <int TS_SHIFT>
+static void launch_softmax_tile_ts(int outer_num, int dim, int inner_num, const float* x, float* y,
+                                   hipStream_t st) {
+  const uint32_t tiles = (static_cast<uint32_t>(inner_num) + (1u << TS_SHIFT) - 1) >> TS_SHIFT;
+  const uint32_t grid = static_cast<uint32_t>(outer_num) * tiles;
+  const size_t bytes = (static_cast<size_t>(dim) << TS_SHIFT) * sizeof(float) + 32 * sizeof(uint64_t);
+  const uint32_t d = static_cast<uint32_t>(dim), in = static_cast<uint32_t>(inner_num);
+  if (inner_num % 4 == 0)
+    softmax_tile_kernel<TS_SHIFT, false><<<grid, kBlock, bytes, st>>>(x, y, d, in, make_fastdiv(tiles));
+  else
+    softmax_tile_kernel<TS_SHIFT, true><<<grid, kBlock, bytes, st>>>(x, y, d, in, make_fastdiv(tiles));
 }
 
 // Shared launch geometry: slab layout when the columns are too narrow to
@@ -522,9 +647,13 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
   else if (dim <= 64)
     softmax_columns_reg_kernel<64><<<grid_for(g.columns), kBlock, 0, st>>>(
         x, y, g.columns, static_cast<uint32_t>(dim), fi);
+  else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner && dim * 64 * sizeof(float) + 256 <= kTileLdsBytes)
+    launch_softmax_tile_ts<6>(outer_num, dim, inner_num, x, y, st);
+  else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner)
+    launch_softmax_tile_ts<5>(outer_num, dim, inner_num, x, y, st);
   else
-    softmax_columns_kernel<<<grid_for(g.columns), kBlock, 0, st>>>(x, y, g.columns,
-                                                                  static_cast<uint32_t>(dim), fi);
+    softmax_columns_kernel<<<(g.columns + kWave - 1) / kWave, kWave, 0, st>>>(x, y, g.columns,
+                                                                             static_cast<uint32_t>(dim), fi);
   return launch_status();
 }
 

@@ -90,6 +90,8 @@ SOFTMAX_SHAPES = [  # outer, dim, inner: both layouts, LDS limits, odd sizes
     (1, 1, 1), (64, 1000, 1), (3, 10, 1), (5, 7, 3), (2, 21, 63), (2, 21, 64), (2, 21, 65),
     (4, 8, 1024), (1, 15000, 1), (1, 16000, 1), (2, 300, 50), (2, 310, 50), (300, 4, 2),
     (1, 2, 5000), (3, 1, 17),
+    # columns too long for registers over a wide inner extent: the three-walk kernel
+    (2, 150, 300), (1, 65, 4097), (3, 100, 64), (1, 1000, 70),
 ]
 
 
@@ -101,7 +103,7 @@ def test_softmax(gpu, outer, dim, inner):
     assert_bit_exact(gpuops.softmax(x, outer, dim, inner, inplace=True), want, "softmax in place")
 
 
-@pytest.mark.parametrize("outer,dim,inner", [(40, 50, 1), (2, 12, 200)])
+@pytest.mark.parametrize("outer,dim,inner", [(40, 50, 1), (2, 12, 200), (2, 80, 100)])
 def test_softmax_special_values(gpu, outer, dim, inner):
     x = with_specials(normal(14, outer * dim * inner, 30.0), 14)
     assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax specials")
