@@ -201,6 +201,10 @@ HOST_SIGNATURES = {
     "shdw_host_parse_net": (_I, [ctypes.c_char_p, ctypes.c_char_p, _Z]),
     "shdw_host_backend_keys": (_I, [ctypes.c_char_p, _Z]),
     "shdw_host_network_create": (_V, [ctypes.c_char_p, _I, _I, _I, ctypes.c_char_p, _V]),
+    "shdw_host_network_create_from_binary": (_V, [ctypes.c_char_p, _I, _I, _I, _V, _I, _I]),
+    "shdw_host_parse_net_binary": (_I, [_V, _I, _I, ctypes.c_char_p, _Z]),
+    "shdw_host_proto_reencode": (_I, [_V, _I, _I, _V, _Z]),
+    "shdw_host_serialize_net": (_I, [ctypes.c_char_p, _V, _Z]),
     "shdw_host_network_destroy": (None, [_V]),
     "shdw_host_network_io": (_I, [_V, _I, ctypes.c_char_p, _Z]),
     "shdw_host_network_forward": (_I, [_V, _I, ctypes.POINTER(ctypes.c_char_p), c_void_pp, c_int_p, c_int_p]),
@@ -343,9 +347,52 @@ def parse_net(proto_text):
     return buf.value.decode()
 
 
+def parse_net_binary(data, network_index=-1):
+    """Canonical text form of a binary model: a serialized NetParam, or network
+    `network_index` of a serialized MetaNetParam (host only)."""
+    lib = host()
+    data = bytes(data)
+    buf = ctypes.create_string_buffer(max(4096, 8 * len(data) + 1024))
+    n = lib.shdw_host_parse_net_binary(data, len(data), network_index, buf, len(buf))
+    host_check(n >= 0)
+    return buf.value.decode()
+
+
+def reencode_proto(data, meta=False):
+    """Decode and re-encode a serialized NetParam / MetaNetParam (host only)."""
+    lib = host()
+    data = bytes(data)
+    buf = ctypes.create_string_buffer(2 * len(data) + 1024)
+    n = lib.shdw_host_proto_reencode(data, len(data), int(meta), buf, len(buf))
+    host_check(0 <= n <= len(buf))
+    return buf.raw[:n]
+
+
+def serialize_net(proto_text):
+    """A text model as a serialized NetParam (host only)."""
+    lib = host()
+    buf = ctypes.create_string_buffer(4 * len(proto_text) + 1024)
+    n = lib.shdw_host_serialize_net(proto_text.encode(), buf, len(buf))
+    host_check(0 <= n <= len(buf))
+    return buf.raw[:n]
+
+
 class Network:
     """Shadow::Network over the Native backend: a text model plus packed float32
-    weights (declared-blob order), run with host inputs."""
+    weights (declared-blob order), run with host inputs.  from_binary() takes a
+    serialized model whose blobs carry their contents instead."""
+
+    @classmethod
+    def from_binary(cls, data, network_index=-1, backend_type="Native", device_id=0, debug=False,
+                    device_input=False):
+        self = cls.__new__(cls)
+        self.lib = host()
+        self.device_input = device_input
+        data = bytes(data)
+        self.ptr = self.lib.shdw_host_network_create_from_binary(
+            backend_type.encode(), device_id, int(debug), int(device_input), data, len(data), network_index)
+        host_check(self.ptr)
+        return self
 
     def __init__(self, proto_text, weights=None, backend_type="Native", device_id=0, debug=False,
                  device_input=False):

@@ -21,6 +21,10 @@ class Native : public Backend {
   // one pointer per blob, or one packed buffer (each blob's raw_size() bytes).
   void LoadModel(const std::string& proto_text, const std::vector<const void*>& weights);
   void LoadModel(const std::string& proto_text, const void* weights_data);
+  // A serialized NetParam in memory, or in the file `proto_bin`
+  // (shadow/backends/native/native.cpp:11-21).
+  void LoadModel(const void* proto_data, int proto_size);
+  void LoadModel(const std::string& proto_bin);
 
   void Run(const std::map<std::string, void*>& data_map,
            const std::map<std::string, std::vector<int>>& shape_map) override;

@@ -101,6 +101,9 @@ class Blob {
   const std::vector<float>& data_f() const { return data_f_; }
   void add_data_f(float v) { data_f_.push_back(v); }
   int data_f_size() const { return static_cast<int>(data_f_.size()); }
+  const std::vector<int>& data_i() const { return data_i_; }
+  void add_data_i(int v) { data_i_.push_back(v); }
+  int data_i_size() const { return static_cast<int>(data_i_.size()); }
   const std::vector<std::vector<char>>& data_b() const { return data_b_; }
   const std::vector<char>& data_b(int i) const { return data_b_[i]; }
   void add_data_b(const std::vector<char>& v) { data_b_.push_back(v); }
@@ -111,6 +114,7 @@ class Blob {
   bool has_type_ = false;
   std::vector<int> shape_;
   std::vector<float> data_f_;
+  std::vector<int> data_i_;
   std::vector<std::vector<char>> data_b_;
 };
 
@@ -142,6 +146,30 @@ class NetParam {
   std::string name_;
   std::vector<Blob> blob_;
   std::vector<OpParam> op_;
+  std::vector<Argument> arg_;
+};
+
+// A model file: several networks under one name (shadow/proto/shadow.proto:42-47).
+class MetaNetParam {
+ public:
+  const std::string& name() const { return name_; }
+  void set_name(const std::string& v) { name_ = v; }
+  const std::vector<NetParam>& network() const { return network_; }
+  const NetParam& network(int i) const { return network_[i]; }
+  NetParam* add_network() {
+    network_.emplace_back();
+    return &network_.back();
+  }
+  int network_size() const { return static_cast<int>(network_.size()); }
+  const std::vector<Argument>& arg() const { return arg_; }
+  Argument* add_arg() {
+    arg_.emplace_back();
+    return &arg_.back();
+  }
+
+ private:
+  std::string name_;
+  std::vector<NetParam> network_;
   std::vector<Argument> arg_;
 };
 

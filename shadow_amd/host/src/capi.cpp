@@ -10,6 +10,7 @@
 #include <string>
 #include <vector>
 
+#include "shadow/io.hpp"
 #include "shadow/kernel.hpp"
 #include "shadow/network.hpp"
 #include "shadow/operator.hpp"
@@ -194,6 +195,75 @@ int shdw_host_parse_net(const char* proto_text, char* buf, size_t n) {
   return len;
 }
 
+namespace {
+
+// network_index < 0: `data` is a serialized NetParam; otherwise a MetaNetParam
+// whose network(network_index) is taken.
+void read_binary_net(const void* data, int size, int network_index, shadow::NetParam* net) {
+  if (network_index < 0) {
+    CHECK(IO::ReadProtoFromArray(data, size, net)) << "Error when loading proto array data";
+  } else {
+    shadow::MetaNetParam meta;
+    CHECK(IO::ReadProtoFromArray(data, size, &meta)) << "Error when loading proto array data";
+    CHECK_LT(network_index, meta.network_size());
+    *net = meta.network(network_index);
+  }
+}
+
+int copy_out(const std::string& bytes, void* buf, size_t n) {
+  if (buf != nullptr && n >= bytes.size()) std::memcpy(buf, bytes.data(), bytes.size());
+  return static_cast<int>(bytes.size());
+}
+
+}  // namespace
+
+// Host-only.  Decodes a binary model and writes the canonical text form of the
+// chosen network (the text form carries no blob contents); returns the length,
+// or -1 when the bytes are malformed.
+int shdw_host_parse_net_binary(const void* data, int size, int network_index, char* buf, size_t n) {
+  int len = -1;
+  guarded([&] {
+    shadow::NetParam net;
+    read_binary_net(data, size, network_index, &net);
+    len = join({Parser::DumpNet(net)}, buf, n);
+  });
+  return len;
+}
+
+// Host-only.  Decodes and re-encodes a binary NetParam (is_meta == 0) or
+// MetaNetParam; returns the encoded length (the bytes are copied when they fit
+// `n`), or -1 when the input is malformed.
+int shdw_host_proto_reencode(const void* data, int size, int is_meta, void* buf, size_t n) {
+  int len = -1;
+  guarded([&] {
+    std::string bytes;
+    if (is_meta) {
+      shadow::MetaNetParam meta;
+      CHECK(IO::ReadProtoFromArray(data, size, &meta)) << "Error when loading proto array data";
+      IO::WriteProtoToString(meta, &bytes);
+    } else {
+      shadow::NetParam net;
+      CHECK(IO::ReadProtoFromArray(data, size, &net)) << "Error when loading proto array data";
+      IO::WriteProtoToString(net, &bytes);
+    }
+    len = copy_out(bytes, buf, n);
+  });
+  return len;
+}
+
+// Host-only.  The text form encoded as a binary NetParam.
+int shdw_host_serialize_net(const char* proto_text, void* buf, size_t n) {
+  int len = -1;
+  guarded([&] {
+    shadow::NetParam net;
+    Parser::ParseNet(proto_text, &net);
+    std::string bytes;
+    IO::WriteProtoToString(net, &bytes);
+    len = copy_out(bytes, buf, n);
+  });
+  return len;
+}
+
 int shdw_host_backend_keys(char* buf, size_t n) { return join(BackendRegistry()->Keys(), buf, n); }
 
 // weights: one packed host buffer in declared-blob order, or NULL when the
@@ -211,6 +281,28 @@ void* shdw_host_network_create(const char* backend_type, int device_id, int debu
     std::unique_ptr<Network> made(new Network());
     made->LoadXModel(std::string(proto_text ? proto_text : ""), weights, args);
     made->backend()->ws()->Ctx()->synchronize();  // the weight buffer may go away after return
+    net = made.release();
+  });
+  return net;
+}
+
+// The same from a binary model whose blobs carry their contents
+// (network_index as in shdw_host_parse_net_binary).
+void* shdw_host_network_create_from_binary(const char* backend_type, int device_id, int debug,
+                                           int device_input, const void* data, int size,
+                                           int network_index) {
+  Network* net = nullptr;
+  guarded([&] {
+    ArgumentHelper args;
+    args.AddSingleArgument<std::string>("backend_type", backend_type ? backend_type : "");
+    args.AddSingleArgument<int>("device_id", device_id);
+    args.AddSingleArgument<bool>("debug", debug != 0);
+    args.AddSingleArgument<bool>("device_input", device_input != 0);
+    shadow::NetParam net_param;
+    read_binary_net(data, size, network_index, &net_param);
+    std::unique_ptr<Network> made(new Network());
+    made->LoadXModel(net_param, args);
+    made->backend()->ws()->Ctx()->synchronize();
     net = made.release();
   });
   return net;

@@ -1,5 +1,6 @@
 #include "shadow/native.hpp"
 
+#include "shadow/io.hpp"
 #include "shadow/parser.hpp"
 
 namespace Shadow {
@@ -26,6 +27,18 @@ void Native::LoadModel(const std::string& proto_text, const void* weights_data) 
   Parser::ParseNet(proto_text, &net_param);
   Initial(net_param);
   CopyWeights(net_param, weights_data);
+}
+
+void Native::LoadModel(const void* proto_data, int proto_size) {
+  shadow::NetParam net_param;
+  CHECK(IO::ReadProtoFromArray(proto_data, proto_size, &net_param)) << "Error when loading proto array data";
+  Initial(net_param);
+}
+
+void Native::LoadModel(const std::string& proto_bin) {
+  shadow::NetParam net_param;
+  CHECK(IO::ReadProtoFromBinaryFile(proto_bin, &net_param)) << "Error when loading proto binary file: " << proto_bin;
+  Initial(net_param);
 }
 
 // Declared blobs first (with their contents when the NetParam carries them),

@@ -114,6 +114,36 @@ def test_mixed_graph(gpu):
         assert nw.blob_shape("r") == [3, 40, 6] and nw.blob_shape("u") == [3, 1, 40, 6]
 
 
+def test_binary_models_with_embedded_weights(gpu):
+    """The same graphs from serialized NetParam / MetaNetParam bytes whose blobs
+    carry their contents (python-protobuf writes them, the C++ reader decodes
+    them): every blob as from the text form with separate weights."""
+    from tests import shadow_proto as sp
+    net, weights, inputs = resnet_tail()
+    want = onet.run(net, weights, inputs)
+    wire = sp.from_oracle_net(net, weights).SerializeToString()
+    with shadow_amd.Network.from_binary(wire) as nw:
+        assert nw.in_blob == ["data", "skip"] and nw.out_blob == ["prob", "feat"]
+        nw.forward(inputs)
+        compare(nw, want, ["bn_out", "sum", "feat", "pooled", "flat", "prob"])
+    net2, weights2, inputs2 = mixed_graph()
+    meta = sp.MetaNetParam()
+    meta.name = "two networks"
+    meta.network.add().CopyFrom(sp.from_oracle_net(net, weights))
+    meta.network.add().CopyFrom(sp.from_oracle_net(net2, weights2))
+    want2 = onet.run(net2, weights2, inputs2)
+    with shadow_amd.Network.from_binary(meta.SerializeToString(), network_index=1) as nw:
+        nw.forward(inputs2)
+        compare(nw, want2, ["bn", "p", "nz", "rmax", "ln", "ax", "inn", "ravg", "fms", "out"])
+    # a blob whose contents do not match its shape is refused (native.cpp:155)
+    bad = sp.from_oracle_net(net, weights)
+    bad.blob[0].data_f.append(1.0)
+    with pytest.raises(ShadowError, match="Check Failed"):
+        shadow_amd.Network.from_binary(bad.SerializeToString())
+    with pytest.raises(ShadowError, match="Error when loading proto"):
+        shadow_amd.Network.from_binary(wire[:-3])
+
+
 def test_inputs_can_be_reshaped_per_call(gpu):
     net, weights, _ = resnet_tail()
     with shadow_amd.Network(onet.write_text(net), weights) as nw:
