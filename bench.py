@@ -217,6 +217,8 @@ def probe_next(dev):
     alpha = dev.buf(uniform(205, 64 * C, 0.0, 1.0))
     ls, lb = dev.buf(uniform(206, 784, 0.5, 1.5)), dev.buf(uniform(207, 784, -0.1, 0.1))
     y = dev.buf(nbytes=4 * n)
+    ssd_ws = dev.buf(nbytes=max(8, lib.shdw_hip_ssd_normalize_workspace_bytes(64, 512, 1444, 1)))
+    ssd_sc = dev.buf(uniform(208, 512, 10.0, 30.0))
     stem_in, stem_out = [64, 64, 112, 112], [64, 64, 56, 56]
     for _ in range(3):
         dev.ck(lib.shdw_hip_copy(n, x.ptr, y.ptr, st))
@@ -237,6 +239,11 @@ def probe_next(dev):
         dev.ck(lib.shdw_hip_resize(I(stem_out), I(stem_in), 0, 0, x.ptr, y.ptr, st))
         dev.ck(lib.shdw_hip_reorg(I(stem_in), 1, 2, x.ptr, y.ptr, st))
         dev.ck(lib.shdw_hip_reorg(I(stem_in), 0, 2, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_softmax(64, 150, 5184, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_softmax(64, 150, 5329, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_ssd_normalize(64, 512, 1444, 0, 1e-5, x.ptr, ssd_sc.ptr, 0, y.ptr, None, st))
+        dev.ck(lib.shdw_hip_ssd_normalize(64, 256, 3136, 0, 1e-5, x.ptr, ssd_sc.ptr, 0, y.ptr, None, st))
+        dev.ck(lib.shdw_hip_ssd_normalize(64, 512, 1444, 1, 1e-5, x.ptr, ssd_sc.ptr, 0, y.ptr, ssd_ws.ptr, st))
     dev.sync()
 
 

@@ -402,9 +402,15 @@ __global__ __launch_bounds__(kBlock) void normalize_slab_kernel(const float* x, 
 constexpr int kTilePerLane = 16;  // 64 KB / (256 lanes x 16 bytes)
 typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
 
-// TAIL: inner % 4 != 0, so a tile row may end inside a lane's four positions.
-template <int TS_SHIFT, bool TAIL>
+// ROWS says how the tile rows lie in memory:
+//   kRowsSector: inner % 16 == 0, every row starts on a 64-byte boundary;
+//   kRowsQuad:   inner % 4 == 0, rows start on a multiple of four positions;
+//   kRowsAny:    a row may end inside a lane's four positions.
+enum TileRows { kRowsSector = 0, kRowsQuad = 1, kRowsAny = 2 };
+
+template <int TS_SHIFT, int ROWS>
 struct TileLane {
+  static constexpr bool TAIL = ROWS == kRowsAny;
   static constexpr uint32_t TS = 1u << TS_SHIFT;
   static constexpr uint32_t LANES_PER_ROW = TS / 4;
   static constexpr uint32_t STEP = kBlock / LANES_PER_ROW;  // rows between a lane's vectors
@@ -444,8 +450,15 @@ struct TileLane {
   SHDW_DEVICE void store(float* ys, uint32_t u, v4f v) const {
     const uint32_t c = c0 + u * STEP;
     float* dst = ys + static_cast<uint64_t>(c) * inner + j;
+    // Rows that do not start on a 64-byte boundary end inside a sector whose
+    // other part the neighbouring tile writes: with a plain store the two parts
+    // merge in L2 before they go to HBM, a streaming store sends each on its own
+    // (+37 % write traffic on [64,512,38,38]).  Aligned rows stream.
     if (!TAIL || valid == 4) {
-      __builtin_nontemporal_store(v, reinterpret_cast<v4f_unaligned*>(dst));
+      if (ROWS == kRowsSector)
+        __builtin_nontemporal_store(v, reinterpret_cast<v4f_unaligned*>(dst));
+      else
+        *reinterpret_cast<v4f_unaligned*>(dst) = v;
     } else {
 #pragma unroll
       for (int k = 0; k < 3; ++k)
@@ -456,7 +469,7 @@ struct TileLane {
 
 // p other than 1 and 2 is not taken here: powf per element inside the serial
 // fold would dominate.
-template <int PMODE, int SM, int TS_SHIFT, bool TAIL>
+template <int PMODE, int SM, int TS_SHIFT, int ROWS>
 __global__ __launch_bounds__(kBlock) void normalize_tile_kernel(const float* x, float* y, uint32_t dim,
                                                                  uint32_t inner, FastDiv f_tiles, float p,
                                                                  float eps, const float* scale) {
@@ -467,7 +480,7 @@ __global__ __launch_bounds__(kBlock) void normalize_tile_kernel(const float* x, 
   const uint32_t p0 = tile << TS_SHIFT;
   const uint32_t width = min(TS, inner - p0);
   const uint64_t base = static_cast<uint64_t>(n) * dim * inner + p0;
-  const TileLane<TS_SHIFT, TAIL> lane(width, dim, inner);
+  const TileLane<TS_SHIFT, ROWS> lane(width, dim, inner);
   v4f r[kTilePerLane];
   lane.load(x + base, r);
   lane.park(lds, r);
@@ -496,6 +509,11 @@ __global__ __launch_bounds__(kBlock) void normalize_tile_kernel(const float* x, 
 constexpr int kTileMinDim = 65, kTileMaxDim = 512, kTileMinInner = 16;  // beyond 512 a tile row is 64 bytes
 constexpr int kTileLdsBytes = 65536;
 
+static int tile_rows(int inner_num, const float* y) {
+  if (inner_num % 16 == 0 && (reinterpret_cast<uintptr_t>(y) & 63u) == 0) return kRowsSector;
+  return inner_num % 4 == 0 ? kRowsQuad : kRowsAny;
+}
+
 static bool tile_fits(int dim, int inner_num) {
   return dim >= kTileMinDim && dim <= kTileMaxDim && inner_num >= kTileMinInner;
 }
@@ -507,12 +525,17 @@ static void launch_normalize_tile_ts(int outer_num, int dim, int inner_num, floa
   const uint32_t grid = static_cast<uint32_t>(outer_num) * tiles;
   const size_t bytes = (static_cast<size_t>(dim) << TS_SHIFT) * sizeof(float);
   const uint32_t d = static_cast<uint32_t>(dim), in = static_cast<uint32_t>(inner_num);
-  if (inner_num % 4 == 0)
-    normalize_tile_kernel<PMODE, SM, TS_SHIFT, false><<<grid, kBlock, bytes, st>>>(x, y, d, in, make_fastdiv(tiles),
-                                                                                 p, eps, scale);
-  else
-    normalize_tile_kernel<PMODE, SM, TS_SHIFT, true><<<grid, kBlock, bytes, st>>>(x, y, d, in, make_fastdiv(tiles),
-                                                                                p, eps, scale);
+  const FastDiv ft = make_fastdiv(tiles);
+  switch (tile_rows(inner_num, y)) {
+    case kRowsSector:
+      normalize_tile_kernel<PMODE, SM, TS_SHIFT, kRowsSector><<<grid, kBlock, bytes, st>>>(x, y, d, in, ft, p, eps, scale);
+      break;
+    case kRowsQuad:
+      normalize_tile_kernel<PMODE, SM, TS_SHIFT, kRowsQuad><<<grid, kBlock, bytes, st>>>(x, y, d, in, ft, p, eps, scale);
+      break;
+    default:
+      normalize_tile_kernel<PMODE, SM, TS_SHIFT, kRowsAny><<<grid, kBlock, bytes, st>>>(x, y, d, in, ft, p, eps, scale);
+  }
 }
 
 template <int PMODE, int SM>
@@ -530,7 +553,7 @@ static void launch_normalize_tile(int outer_num, int dim, int inner_num, float p
 // in LDS serves wave 0's two serial folds: the running maximum of x, then the
 // fp32 running sum of the exponentials, both in index order.  The maxima and
 // then the sums are handed over in the first tile row.
-template <int TS_SHIFT, bool TAIL>
+template <int TS_SHIFT, int ROWS>
 __global__ __launch_bounds__(kBlock) void softmax_tile_kernel(const float* x, float* y, uint32_t dim,
                                                                uint32_t inner, FastDiv f_tiles) {
   extern __shared__ __align__(16) float lds[];
@@ -542,7 +565,7 @@ __global__ __launch_bounds__(kBlock) void softmax_tile_kernel(const float* x, fl
   const uint32_t p0 = tile << TS_SHIFT;
   const uint32_t width = min(TS, inner - p0);
   const uint64_t base = static_cast<uint64_t>(n) * dim * inner + p0;
-  const TileLane<TS_SHIFT, TAIL> lane(width, dim, inner);
+  const TileLane<TS_SHIFT, ROWS> lane(width, dim, inner);
   v4f r[kTilePerLane];
   lane.load(x + base, r);
   lane.park(lds, r);
@@ -596,10 +619,12 @@ static void launch_softmax_tile_ts(int outer_num, int dim, int inner_num, const 
   const uint32_t grid = static_cast<uint32_t>(outer_num) * tiles;
   const size_t bytes = (static_cast<size_t>(dim) << TS_SHIFT) * sizeof(float) + 32 * sizeof(uint64_t);
   const uint32_t d = static_cast<uint32_t>(dim), in = static_cast<uint32_t>(inner_num);
-  if (inner_num % 4 == 0)
-    softmax_tile_kernel<TS_SHIFT, false><<<grid, kBlock, bytes, st>>>(x, y, d, in, make_fastdiv(tiles));
-  else
-    softmax_tile_kernel<TS_SHIFT, true><<<grid, kBlock, bytes, st>>>(x, y, d, in, make_fastdiv(tiles));
+  const FastDiv ft = make_fastdiv(tiles);
+  switch (tile_rows(inner_num, y)) {
+    case kRowsSector: softmax_tile_kernel<TS_SHIFT, kRowsSector><<<grid, kBlock, bytes, st>>>(x, y, d, in, ft); break;
+    case kRowsQuad: softmax_tile_kernel<TS_SHIFT, kRowsQuad><<<grid, kBlock, bytes, st>>>(x, y, d, in, ft); break;
+    default: softmax_tile_kernel<TS_SHIFT, kRowsAny><<<grid, kBlock, bytes, st>>>(x, y, d, in, ft);
+  }
 }
 
 // Shared launch geometry: slab layout when the columns are too narrow to
