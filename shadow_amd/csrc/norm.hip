@@ -262,13 +262,17 @@ static SsdRowPlan plan_ssd_rows(uint32_t batch, uint32_t num) {
   return plan;
 }
 
+// Workgroup b * parts + k folds segment k of item b.
 template <bool VEC>
 __global__ __launch_bounds__(kBlock) void ssd_row_partials_kernel(const float* x, double* partials,
-                                                                   uint32_t num, uint32_t segment) {
+                                                                   uint32_t num, uint32_t segment,
+                                                                   FastDiv f_parts) {
   __shared__ double slots[kBlock / kWave];
-  const uint32_t begin = blockIdx.x * segment;
+  uint32_t item, part;
+  fd_divmod(blockIdx.x, f_parts, item, part);
+  const uint32_t begin = part * segment;
   const uint32_t end = min(num, begin + segment);
-  const float* xr = x + static_cast<uint64_t>(blockIdx.y) * num;
+  const float* xr = x + static_cast<uint64_t>(item) * num;
   double acc = 0;
   if (VEC) {
     for (uint32_t t = begin / 4 + threadIdx.x; t < end / 4; t += kBlock) {
@@ -286,7 +290,7 @@ __global__ __launch_bounds__(kBlock) void ssd_row_partials_kernel(const float* x
     }
   }
   const double total = row_sum<kBlock>(acc, slots);
-  if (threadIdx.x == 0) partials[blockIdx.y * gridDim.x + blockIdx.x] = total;
+  if (threadIdx.x == 0) partials[blockIdx.x] = total;
 }
 
 // SM: 0 no scale, 1 one shared factor (Sscal), 2 one factor per channel.
@@ -294,15 +298,18 @@ template <bool VEC, int SM>
 __global__ __launch_bounds__(kBlock) void ssd_row_scale_kernel(const float* x, float* y,
                                                                 const double* partials, uint32_t parts,
                                                                 uint32_t num, float eps,
-                                                                const float* scale, FastDiv f_spatial) {
-  const double* mine = partials + blockIdx.y * parts;  // uniform: scalar loads
+                                                                const float* scale, FastDiv f_spatial,
+                                                                FastDiv f_groups) {
+  uint32_t item, group;  // workgroup `group` of the item's grid_for(steps) workgroups
+  fd_divmod(blockIdx.x, f_groups, item, group);
+  const double* mine = partials + item * parts;  // uniform: scalar loads
   double sum = 0;
   for (uint32_t k = 0; k < parts; ++k) sum += mine[k];
   const float sum_f = static_cast<float>(sum);
   const float se = sum_f + eps;
   const float factor = 1.f / __builtin_sqrtf(se);
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-  const uint64_t base = static_cast<uint64_t>(blockIdx.y) * num;
+  const uint32_t i = group * kBlock + threadIdx.x;
+  const uint64_t base = static_cast<uint64_t>(item) * num;
   if (VEC) {
     if (i >= num / 4) return;
     const v4f q = load4_stream(x + base + 4ull * i);
@@ -328,15 +335,17 @@ static void launch_ssd_rows(uint32_t batch, uint32_t num, uint32_t spatial, floa
                             const float* scale, int channel_shared, float* y, double* partials,
                             hipStream_t st) {
   const SsdRowPlan plan = plan_ssd_rows(batch, num);
-  ssd_row_partials_kernel<VEC><<<dim3(plan.parts, batch), kBlock, 0, st>>>(x, partials, num, plan.segment);
-  const dim3 grid(grid_for(VEC ? num / 4 : num), batch);
-  const FastDiv fs = make_fastdiv(std::max(spatial, 1u));
+  ssd_row_partials_kernel<VEC><<<batch * plan.parts, kBlock, 0, st>>>(x, partials, num, plan.segment,
+                                                                    make_fastdiv(plan.parts));
+  const uint32_t groups = grid_for(VEC ? num / 4 : num);  // batch * groups <= count / 256 + batch
+  const uint32_t grid = batch * groups;
+  const FastDiv fs = make_fastdiv(std::max(spatial, 1u)), fg = make_fastdiv(groups);
   if (!scale)
-    ssd_row_scale_kernel<VEC, 0><<<grid, kBlock, 0, st>>>(x, y, partials, plan.parts, num, eps, scale, fs);
+    ssd_row_scale_kernel<VEC, 0><<<grid, kBlock, 0, st>>>(x, y, partials, plan.parts, num, eps, scale, fs, fg);
   else if (channel_shared)
-    ssd_row_scale_kernel<VEC, 1><<<grid, kBlock, 0, st>>>(x, y, partials, plan.parts, num, eps, scale, fs);
+    ssd_row_scale_kernel<VEC, 1><<<grid, kBlock, 0, st>>>(x, y, partials, plan.parts, num, eps, scale, fs, fg);
   else
-    ssd_row_scale_kernel<VEC, 2><<<grid, kBlock, 0, st>>>(x, y, partials, plan.parts, num, eps, scale, fs);
+    ssd_row_scale_kernel<VEC, 2><<<grid, kBlock, 0, st>>>(x, y, partials, plan.parts, num, eps, scale, fs, fg);
 }
 
 // softmax.hip: the per-position form shares the Normalize column kernels.

@@ -177,7 +177,8 @@ def test_ssd_normalize_per_position(gpu, batch, channel, spatial, scale_kind):
 
 
 @pytest.mark.parametrize("scale_kind", ["none", "shared", "channel"])
-@pytest.mark.parametrize("batch,channel,spatial", SSD_SHAPES + [(2, 512, 1444), (70, 8, 2048), (3, 7, 11111)])
+@pytest.mark.parametrize("batch,channel,spatial", SSD_SHAPES + [(2, 512, 1444), (70, 8, 2048), (3, 7, 11111),
+                                                                  (70000, 2, 3), (66000, 1, 8)])
 def test_ssd_normalize_per_item(gpu, batch, channel, spatial, scale_kind):
     """The item's fp64 sum is split over workgroups and lanes: 1e-5 relative, and
     the count of differing outputs (none in these cases) is checked as well."""
