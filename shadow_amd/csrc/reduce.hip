@@ -198,7 +198,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const float* 
                                                                     uint32_t chunk,
                                                                     uint32_t splits) {
   __shared__ Partial lds[kBlock / kWave];
-  const uint32_t row = blockIdx.y, split = blockIdx.x;
+  const uint32_t row = blockIdx.x, split = blockIdx.y;  // rows can exceed the 65535 limit of grid.y
   const float* p = x + static_cast<size_t>(row) * reduce;
   const uint32_t begin = split * chunk;  // chunk is a multiple of 4
   uint32_t end = begin + chunk;
@@ -254,12 +254,15 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const float* 
 template <int OP, int VEC, int WAVES>
 __global__ __launch_bounds__(kWave * WAVES) void reduce_strided_kernel(
     const float* x, float* y, Partial* part, uint32_t reduce, uint32_t inner,
-    uint32_t rows_per_split, uint32_t splits, uint32_t outputs) {
+    uint32_t rows_per_split, uint32_t splits, uint32_t outputs, FastDiv f_tiles) {
   constexpr int kWaves = WAVES;
   __shared__ Partial lds[kWaves - 1][VEC][kWave];
   const uint32_t lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
-  const uint32_t col = (blockIdx.x * kWave + lane) * VEC;
-  const uint32_t o = blockIdx.y, split = blockIdx.z;
+  // grid.x = outer * tiles (either can exceed the 65535 limit of grid.y), grid.y = slices
+  uint32_t o, tile;
+  fd_divmod(blockIdx.x, f_tiles, o, tile);
+  const uint32_t col = (tile * kWave + lane) * VEC;
+  const uint32_t split = blockIdx.y;
   const bool col_ok = col < inner;
   const uint32_t r_begin = split * rows_per_split;
   uint32_t r_end = r_begin + rows_per_split;
@@ -474,7 +477,7 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
     const uint32_t splits = static_cast<uint32_t>(pl.splits);
     uint32_t chunk = (reduce + splits - 1) / splits;
     chunk = (chunk + 3) & ~3u;
-    const dim3 grid(splits, rows);
+    const dim3 grid(rows, splits);
     if (vec)
       reduce_rows_block_kernel<OP, true><<<grid, kBlock, 0, st>>>(x, y, part, reduce, chunk, splits);
     else
@@ -489,14 +492,15 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
   const uint32_t reduce = static_cast<uint32_t>(pl.reduce);
   const uint32_t inner = static_cast<uint32_t>(pl.inner);
   const uint32_t splits = static_cast<uint32_t>(pl.splits);
-  if (outer > 65535u || splits > 65535u) return SHDW_E_UNSUPPORTED;
   const uint32_t rows_per_split = (reduce + splits - 1) / splits;
   const bool vec = pl.strided_vec == 4 && inner % 4 == 0 && aligned16(x);
   const int v = vec ? 4 : 1;
-  const dim3 grid((inner + kWave * v - 1) / (kWave * v), outer, splits);
+  const uint32_t tiles = (inner + kWave * v - 1) / (kWave * v);
+  const dim3 grid(tiles * outer, splits);  // tiles * outer <= outputs; splits <= 1024
+  const FastDiv f_tiles = make_fastdiv(tiles);
 #define SHDW_STRIDED(V, W)                                                                   \
   reduce_strided_kernel<OP, V, W><<<grid, kWave * W, 0, st>>>(x, y, part, reduce, inner,       \
-                                                             rows_per_split, splits, outputs)
+                                                             rows_per_split, splits, outputs, f_tiles)
   if (pl.strided_waves == 16) {
     if (vec) SHDW_STRIDED(4, 16); else SHDW_STRIDED(1, 16);
   } else {

@@ -243,6 +243,20 @@ def test_reduce(gpu, shape, axes, op):
         assert_rel_close(got, want, 1e-5, "reduce accumulate")
 
 
+@pytest.mark.parametrize("shape,axes", [([70000, 8, 100], [1]),   # strided with more than 65535 outer slices
+                                        ([66000, 4100], [1]),     # long rows, more than 65535 of them
+                                        ([2, 9, 4200000], [1])])  # strided with more than 65535 column tiles
+@pytest.mark.parametrize("op", [1, 2])
+def test_reduce_beyond_the_second_grid_dimension(gpu, shape, axes, op):
+    x = normal(152, shape)
+    want, _ = oracle.reduce(op, x, shape, axes)
+    got, _ = gpuops.reduce(op, x, shape, axes)
+    if op == 2:
+        assert_bit_exact(got, want, "reduce max")
+    else:
+        assert_rel_close(got, want, 1e-5, "reduce sum")
+
+
 @pytest.mark.parametrize("shape,axes", [([64, 48], [1]), ([3, 64, 8], [1]), ([2, 3, 4, 5], [3, 1]),
                                         ([50000], [0]), ([300, 16], [1])])
 @pytest.mark.parametrize("op", [2, 3])
