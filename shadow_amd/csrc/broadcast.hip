@@ -50,11 +50,11 @@ SHDW_DEVICE float row_element(uint32_t e, float x, const float* s, const float* 
 // One 128-bit vector per lane.  ROWVEC: inner % 4 == 0, so the four elements of
 // a vector share one row and the parameters are fetched once per vector.
 template <int MODE, bool RELU, bool ROWVEC>
-__global__ __launch_bounds__(kBlock) void rowparam_vec_kernel(const float* x, const float* s,
+__global__ __launch_bounds__(kStream) void rowparam_vec_kernel(const float* x, const float* s,
                                                                const float* b, float* y,
                                                                uint32_t n4, uint32_t n,
                                                                FastDiv inner, FastDiv num) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
   if (i < n4) {
     const v4f vx = load4_stream(x + 4ull * i);
     v4f r;
@@ -76,11 +76,11 @@ __global__ __launch_bounds__(kBlock) void rowparam_vec_kernel(const float* x, co
 }
 
 template <int MODE, bool RELU>
-__global__ __launch_bounds__(kBlock) void rowparam_scalar_kernel(const float* x, const float* s,
+__global__ __launch_bounds__(kStream) void rowparam_scalar_kernel(const float* x, const float* s,
                                                                   const float* b, float* y,
                                                                   uint32_t n, FastDiv inner,
                                                                   FastDiv num) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
   if (i < n) y[i] = row_element<MODE, RELU>(i, x[i], s, b, inner, num);
 }
 
@@ -91,13 +91,13 @@ static int launch_rowparam(int n, int num, int inner, const float* x, const floa
   const FastDiv fn = make_fastdiv(static_cast<uint32_t>(num));
   if (aligned16(x) && aligned16(y)) {
     const uint32_t n4 = static_cast<uint32_t>(n) / 4;
-    const uint32_t grid = grid_for(n4 + 1);
+    const uint32_t grid = stream_grid(n4 + 1);
     if (inner % 4 == 0)
-      rowparam_vec_kernel<MODE, RELU, true><<<grid, kBlock, 0, st>>>(x, s, b, y, n4, n, fi, fn);
+      rowparam_vec_kernel<MODE, RELU, true><<<grid, kStream, 0, st>>>(x, s, b, y, n4, n, fi, fn);
     else
-      rowparam_vec_kernel<MODE, RELU, false><<<grid, kBlock, 0, st>>>(x, s, b, y, n4, n, fi, fn);
+      rowparam_vec_kernel<MODE, RELU, false><<<grid, kStream, 0, st>>>(x, s, b, y, n4, n, fi, fn);
   } else {
-    rowparam_scalar_kernel<MODE, RELU><<<grid_for(n), kBlock, 0, st>>>(x, s, b, y, n, fi, fn);
+    rowparam_scalar_kernel<MODE, RELU><<<stream_grid(n), kStream, 0, st>>>(x, s, b, y, n, fi, fn);
   }
   return launch_status();
 }
@@ -120,7 +120,7 @@ template <class F, int NDIM, bool AVEC, bool BVEC>
 __global__ __launch_bounds__(kBlock) void bcast_vec_kernel(F f, BcastArgs p, const float* a,
                                                             const float* b, float* y,
                                                             uint32_t n4) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;  // 64 or 256 lanes, see the launch
   // Pow reads the 2^(i/32) table; broadcast Pow is not a throughput case, the
   // table stays in global memory here.
   const uint64_t* tab = uses_exp_table<F>::value ? libm::kExp2fTab : nullptr;
@@ -189,15 +189,20 @@ __global__ __launch_bounds__(kBlock) void bcast_generic_kernel(F f, BcastGeneric
 template <class F, int NDIM>
 static void launch_bcast_vec(F f, const BcastArgs& p, bool avec, bool bvec, const float* a,
                              const float* b, float* y, uint32_t n4, hipStream_t st) {
-  const uint32_t grid = grid_for(n4);
+  // An operand as large as the output makes this a read-and-write stream, which
+  // runs best as single-wave workgroups; when both operands are broadcast the
+  // kernel mostly writes, and 256-lane workgroups are 1.5x faster than single
+  // waves there (11.3 us against 16.5 us for [16,1,128,256] x [1,32,128,1]).
+  const uint32_t lanes = (p.a_full || p.b_full) ? kStream : kBlock;
+  const uint32_t grid = (n4 + lanes - 1) / lanes;
   if (avec && bvec)
-    bcast_vec_kernel<F, NDIM, true, true><<<grid, kBlock, 0, st>>>(f, p, a, b, y, n4);
+    bcast_vec_kernel<F, NDIM, true, true><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4);
   else if (avec)
-    bcast_vec_kernel<F, NDIM, true, false><<<grid, kBlock, 0, st>>>(f, p, a, b, y, n4);
+    bcast_vec_kernel<F, NDIM, true, false><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4);
   else if (bvec)
-    bcast_vec_kernel<F, NDIM, false, true><<<grid, kBlock, 0, st>>>(f, p, a, b, y, n4);
+    bcast_vec_kernel<F, NDIM, false, true><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4);
   else
-    bcast_vec_kernel<F, NDIM, false, false><<<grid, kBlock, 0, st>>>(f, p, a, b, y, n4);
+    bcast_vec_kernel<F, NDIM, false, false><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4);
 }
 
 template <class F>

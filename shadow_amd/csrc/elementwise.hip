@@ -26,10 +26,10 @@ namespace shdw {
 // Lane i owns vector i; lane n4 (one past the last whole vector) owns the
 // n % 4 trailing elements.
 template <int NIN, class F>
-__global__ __launch_bounds__(kBlock) void ew_vec_kernel(F f, const float* a, const float* b,
+__global__ __launch_bounds__(kStream) void ew_vec_kernel(F f, const float* a, const float* b,
                                                          float* y, uint32_t n4, uint32_t n,
                                                          float alpha) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
   v4f va, vb;
   if (i < n4) {  // issue the streaming loads before anything else
     if (NIN >= 1) va = load4_stream(a + 4ull * i);
@@ -62,9 +62,9 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(F f, const float* a, con
 
 // Same arithmetic for pointers that are not 16-byte aligned (Blas offsets).
 template <int NIN, class F>
-__global__ __launch_bounds__(kBlock) void ew_scalar_kernel(F f, const float* a, const float* b,
+__global__ __launch_bounds__(kStream) void ew_scalar_kernel(F f, const float* a, const float* b,
                                                             float* y, uint32_t n, float alpha) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
   const uint64_t* tab = uses_exp_table<F>::value ? libm::kExp2fTab : nullptr;
   if (i < n) {
     const float x = NIN >= 1 ? a[i] : alpha;
@@ -82,11 +82,11 @@ static int launch_ew(F f, int n, const float* a, const float* b, float alpha, fl
   const bool vec = aligned16(y) && (NIN < 1 || aligned16(a)) && (NIN < 2 || aligned16(b));
   if (vec) {
     const uint32_t n4 = static_cast<uint32_t>(n) / 4;
-    const uint32_t grid = grid_for(n4 + 1);
-    ew_vec_kernel<NIN, F><<<grid, kBlock, 0, s>>>(f, a, b, y, n4, static_cast<uint32_t>(n), alpha);
+    const uint32_t grid = stream_grid(n4 + 1);
+    ew_vec_kernel<NIN, F><<<grid, kStream, 0, s>>>(f, a, b, y, n4, static_cast<uint32_t>(n), alpha);
   } else {
-    const uint32_t grid = grid_for(static_cast<uint32_t>(n));
-    ew_scalar_kernel<NIN, F><<<grid, kBlock, 0, s>>>(f, a, b, y, static_cast<uint32_t>(n), alpha);
+    const uint32_t grid = stream_grid(static_cast<uint32_t>(n));
+    ew_scalar_kernel<NIN, F><<<grid, kStream, 0, s>>>(f, a, b, y, static_cast<uint32_t>(n), alpha);
   }
   return launch_status();
 }
@@ -156,8 +156,8 @@ SHDW_DEVICE float eltwise_fold(const EltwiseArgs& p, const float (&v)[KMAX], flo
 // KMAX is the compile-time bound on p.k (2, 3, 4 or 8) so that the per-input
 // registers are never indexed dynamically.
 template <int OP, int KMAX, bool VEC>
-__global__ __launch_bounds__(kBlock) void eltwise_kernel(EltwiseArgs p, float* y, uint32_t n) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+__global__ __launch_bounds__(kStream) void eltwise_kernel(EltwiseArgs p, float* y, uint32_t n) {
+  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
   if (VEC) {
     const uint32_t n4 = n / 4;
     if (i < n4) {
@@ -196,11 +196,11 @@ template <int OP, int KMAX>
 static int launch_eltwise_k(const EltwiseArgs& p, int n, float* y, hipStream_t s) {
   bool vec = aligned16(y);
   for (int j = 0; j < p.k; ++j) vec = vec && aligned16(p.x[j]);
-  const uint32_t grid = grid_for(vec ? static_cast<uint32_t>(n) / 4 + 1 : static_cast<uint32_t>(n));
+  const uint32_t grid = stream_grid(vec ? static_cast<uint32_t>(n) / 4 + 1 : static_cast<uint32_t>(n));
   if (vec)
-    eltwise_kernel<OP, KMAX, true><<<grid, kBlock, 0, s>>>(p, y, static_cast<uint32_t>(n));
+    eltwise_kernel<OP, KMAX, true><<<grid, kStream, 0, s>>>(p, y, static_cast<uint32_t>(n));
   else
-    eltwise_kernel<OP, KMAX, false><<<grid, kBlock, 0, s>>>(p, y, static_cast<uint32_t>(n));
+    eltwise_kernel<OP, KMAX, false><<<grid, kStream, 0, s>>>(p, y, static_cast<uint32_t>(n));
   return launch_status();
 }
 

@@ -11,6 +11,8 @@ namespace shdw {
 // Workgroups of kBlock (256) lanes needed for `work` lane-tasks.  Counts are
 // int32, so this never exceeds 2^23 + 1 workgroups.
 inline uint32_t grid_for(uint32_t work) { return (work + 255u) / 256u; }
+// The same for kStream (64) lanes: at most 2^25 + 1 workgroups.
+inline uint32_t stream_grid(uint32_t work) { return (work + 63u) / 64u; }
 
 // Shadow checks cudaPeekAtLastError() after every launch
 // (e.g. shadow/core/blas.cu:20); here the error is also cleared so that one bad

@@ -1,7 +1,10 @@
 // Data movers: Concat / Slice / Stack (pitched chunk copies), Gather,
 // ShuffleChannel, Pad, Permute, Reorg, Resize.  No arithmetic except Resize's
 // interpolation weights; everything is bound by HBM traffic (4 bytes read and 4
-// written per output element).  Lanes are laid along the OUTPUT so stores are
+// written per output element).  The contiguous copies (chunks, picked rows) run
+// as single-wave workgroups like the elementwise kernels (+3 %); the kernels
+// that scatter or gather (Reorg, Permute, Resize) were measured slower that way
+// (Reorg 72 -> 91 us) and keep 256 lanes.  Lanes are laid along the OUTPUT so stores are
 // always coalesced; where the input is contiguous in the same direction both
 // sides move as 128-bit vectors, and a transposing Permute goes through an LDS
 // tile so that both sides stay coalesced.
@@ -22,11 +25,11 @@ namespace shdw {
 // dst[n * dst_pitch + dst_off + p] = src[n * src_pitch + src_off + p], p < chunk
 // ---------------------------------------------------------------------------
 template <bool VEC>
-__global__ __launch_bounds__(kBlock) void copy_chunks_kernel(const float* src, float* dst,
+__global__ __launch_bounds__(kStream) void copy_chunks_kernel(const float* src, float* dst,
                                                               uint32_t work, FastDiv f_chunk,
                                                               uint32_t src_pitch, uint32_t src_off,
                                                               uint32_t dst_pitch, uint32_t dst_off) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;  // element, or vector when VEC
+  const uint32_t i = blockIdx.x * kStream + threadIdx.x;  // element, or vector when VEC
   if (i >= work) return;
   uint32_t n, p;
   fd_divmod(i, f_chunk, n, p);  // VEC: chunk, pitches and offsets are counted in vectors
@@ -69,9 +72,9 @@ struct ShuffleRows {
 };
 
 template <class MAP, bool VEC>
-__global__ __launch_bounds__(kBlock) void rows_pick_kernel(MAP map, const float* x, float* y,
+__global__ __launch_bounds__(kStream) void rows_pick_kernel(MAP map, const float* x, float* y,
                                                             uint32_t work, FastDiv f_inner) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
   if (i >= work) return;
   uint32_t r, p;
   fd_divmod(i, f_inner, r, p);  // VEC: inner counted in vectors
@@ -89,10 +92,10 @@ static int launch_rows_pick(const MAP& map, int64_t rows, int inner, const float
                             hipStream_t st) {
   if (inner % 4 == 0 && aligned16(x) && aligned16(y)) {
     const uint32_t work = static_cast<uint32_t>(rows * (inner / 4));
-    rows_pick_kernel<MAP, true><<<grid_for(work), kBlock, 0, st>>>(map, x, y, work, make_fastdiv(inner / 4));
+    rows_pick_kernel<MAP, true><<<stream_grid(work), kStream, 0, st>>>(map, x, y, work, make_fastdiv(inner / 4));
   } else {
     const uint32_t work = static_cast<uint32_t>(rows * inner);
-    rows_pick_kernel<MAP, false><<<grid_for(work), kBlock, 0, st>>>(map, x, y, work, make_fastdiv(inner));
+    rows_pick_kernel<MAP, false><<<stream_grid(work), kStream, 0, st>>>(map, x, y, work, make_fastdiv(inner));
   }
   return launch_status();
 }
@@ -582,12 +585,12 @@ int shdw_hip_copy_chunks(int outer, int chunk, const float* src, int src_pitch, 
                    aligned16(src) && aligned16(dst);
   if (vec) {
     const uint32_t work = static_cast<uint32_t>(outer) * (chunk / 4);
-    copy_chunks_kernel<true><<<grid_for(work), kBlock, 0, st>>>(
+    copy_chunks_kernel<true><<<stream_grid(work), kStream, 0, st>>>(
         src, dst, work, make_fastdiv(chunk / 4), src_pitch / 4, src_offset / 4, dst_pitch / 4,
         dst_offset / 4);
   } else {
     const uint32_t work = static_cast<uint32_t>(outer) * chunk;
-    copy_chunks_kernel<false><<<grid_for(work), kBlock, 0, st>>>(
+    copy_chunks_kernel<false><<<stream_grid(work), kStream, 0, st>>>(
         src, dst, work, make_fastdiv(chunk), src_pitch, src_offset, dst_pitch, dst_offset);
   }
   return launch_status();

@@ -60,9 +60,9 @@ struct BatchNormRows {
 
 // ROWVEC: inner % 4 == 0, the four elements of a vector share a row.
 template <class P, bool ROWVEC>
-__global__ __launch_bounds__(kBlock) void rows_vec_kernel(P p, const float* x, float* out,
+__global__ __launch_bounds__(kStream) void rows_vec_kernel(P p, const float* x, float* out,
                                                            uint32_t n4, uint32_t n, FastDiv inner) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
   if (i < n4) {
     const v4f vx = load4_stream(x + 4ull * i);
     const v4f vo = p.load_other(4ull * i);
@@ -89,9 +89,9 @@ __global__ __launch_bounds__(kBlock) void rows_vec_kernel(P p, const float* x, f
 }
 
 template <class P>
-__global__ __launch_bounds__(kBlock) void rows_scalar_kernel(P p, const float* x, float* out,
+__global__ __launch_bounds__(kStream) void rows_scalar_kernel(P p, const float* x, float* out,
                                                               uint32_t n, FastDiv inner) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
   if (i < n) out[i] = p.apply(x[i], p.other(i), p.row(fd_div(i, inner)));
 }
 
@@ -101,13 +101,13 @@ static int launch_rows(const P& p, uint32_t n, uint32_t inner, const float* x, c
   const FastDiv fi = make_fastdiv(inner);
   if (aligned16(x) && aligned16(out) && (!P::kTwoInputs || aligned16(other))) {
     const uint32_t n4 = n / 4;
-    const uint32_t grid = grid_for(n4 + 1);
+    const uint32_t grid = stream_grid(n4 + 1);
     if (inner % 4 == 0)
-      rows_vec_kernel<P, true><<<grid, kBlock, 0, st>>>(p, x, out, n4, n, fi);
+      rows_vec_kernel<P, true><<<grid, kStream, 0, st>>>(p, x, out, n4, n, fi);
     else
-      rows_vec_kernel<P, false><<<grid, kBlock, 0, st>>>(p, x, out, n4, n, fi);
+      rows_vec_kernel<P, false><<<grid, kStream, 0, st>>>(p, x, out, n4, n, fi);
   } else {
-    rows_scalar_kernel<P><<<grid_for(n), kBlock, 0, st>>>(p, x, out, n, fi);
+    rows_scalar_kernel<P><<<stream_grid(n), kStream, 0, st>>>(p, x, out, n, fi);
   }
   return launch_status();
 }
