@@ -384,7 +384,7 @@ __global__ __launch_bounds__(kBlock) void normalize_slab_kernel(const float* x, 
 }
 
 // Columns of 65 to 512 elements over a wide inner extent: a workgroup owns a
-// tile of TS = 64 or 32 neighbouring positions with all their `dim` elements,
+// tile of TS = 64, 32 or 16 neighbouring positions with all their `dim` elements,
 // 64 KB at most, so x is read from HBM once.  Each lane keeps its share of the
 // tile (16 vectors of 4 positions at most) in registers and also parks it in
 // LDS; wave 0 folds the TS columns from LDS in index order, one column per lane,
@@ -506,7 +506,7 @@ __global__ __launch_bounds__(kBlock) void normalize_tile_kernel(const float* x, 
   }
 }
 
-constexpr int kTileMinDim = 65, kTileMaxDim = 512, kTileMinInner = 16;  // beyond 512 a tile row is 64 bytes
+constexpr int kTileMinDim = 65, kTileMaxDim = 512, kTileMinInner = 16;
 constexpr int kTileLdsBytes = 65536;
 
 static int tile_rows(int inner_num, const float* y) {
@@ -541,11 +541,16 @@ static void launch_normalize_tile_ts(int outer_num, int dim, int inner_num, floa
 template <int PMODE, int SM>
 static void launch_normalize_tile(int outer_num, int dim, int inner_num, float p, float eps, const float* x,
                                   const float* scale, float* y, hipStream_t st) {
-  // the widest tile whose dim rows fit 64 KB
-  if (dim * 64 * sizeof(float) <= kTileLdsBytes)
+  // The tile width that keeps a tile within 32 KB (four and more workgroups per
+  // CU): [64,256,56,56] 92 us with 64-position tiles (64 KB), 87 us with 32;
+  // [64,512,38,38] 131 us with 32 (64 KB), 123 us with 16.  Softmax, with its
+  // five barriers per tile, is the other way round and takes the widest tile.
+  if (dim * 64 * sizeof(float) <= kTileLdsBytes / 2)
     launch_normalize_tile_ts<PMODE, SM, 6>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
-  else
+  else if (dim * 32 * sizeof(float) <= kTileLdsBytes / 2)
     launch_normalize_tile_ts<PMODE, SM, 5>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
+  else
+    launch_normalize_tile_ts<PMODE, SM, 4>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
 }
 
 // Softmax on the same tile layout (65 <= dim <= 511 so that the exp table fits
