@@ -23,17 +23,23 @@ namespace shdw {
 // NIN = 0: y = f(alpha, alpha)     (fill)
 // NIN = 1: y = f(a, alpha)
 // NIN = 2: y = f(a, b)
-// Lane i owns vector i; lane n4 (one past the last whole vector) owns the
+// A lane owns V vectors (V = 1 except where the functor asks for more), kStream
+// vectors apart so that every load instruction of the wave is contiguous; the
+// lane whose vector index is n4 (one past the last whole vector) owns the
 // n % 4 trailing elements.
-template <int NIN, class F>
+template <int NIN, class F, int V>
 __global__ __launch_bounds__(kStream) void ew_vec_kernel(F f, const float* a, const float* b,
-                                                         float* y, uint32_t n4, uint32_t n,
-                                                         float alpha) {
-  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
-  v4f va, vb;
-  if (i < n4) {  // issue the streaming loads before anything else
-    if (NIN >= 1) va = load4_stream(a + 4ull * i);
-    if (NIN >= 2) vb = load4_stream(b + 4ull * i);
+                                                          float* y, uint32_t n4, uint32_t n,
+                                                          float alpha) {
+  const uint32_t first = blockIdx.x * (kStream * V) + threadIdx.x;
+  v4f va[V], vb[V];
+#pragma unroll
+  for (int u = 0; u < V; ++u) {  // issue the streaming loads before anything else
+    const uint32_t i = first + u * kStream;
+    if (i < n4) {
+      if (NIN >= 1) va[u] = load4_stream(a + 4ull * i);
+      if (NIN >= 2) vb[u] = load4_stream(b + 4ull * i);
+    }
   }
   const uint64_t* tab = nullptr;
   if (uses_exp_table<F>::value) {
@@ -42,20 +48,24 @@ __global__ __launch_bounds__(kStream) void ew_vec_kernel(F f, const float* a, co
     __syncthreads();
     tab = lds_tab;
   }
-  if (i < n4) {
-    v4f r;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float x = NIN >= 1 ? va[j] : alpha;
-      const float w = NIN >= 2 ? vb[j] : alpha;
-      r[j] = f(x, w, tab);
-    }
-    store4_stream(y + 4ull * i, r);
-  } else if (i == n4) {
-    for (uint32_t t = 4 * n4; t < n; ++t) {
-      const float x = NIN >= 1 ? a[t] : alpha;
-      const float w = NIN >= 2 ? b[t] : alpha;
-      y[t] = f(x, w, tab);
+  for (int u = 0; u < V; ++u) {
+    const uint32_t i = first + u * kStream;
+    if (i < n4) {
+      v4f r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float x = NIN >= 1 ? va[u][j] : alpha;
+        const float w = NIN >= 2 ? vb[u][j] : alpha;
+        r[j] = f(x, w, tab);
+      }
+      store4_stream(y + 4ull * i, r);
+    } else if (i == n4) {
+      for (uint32_t t = 4 * n4; t < n; ++t) {
+        const float x = NIN >= 1 ? a[t] : alpha;
+        const float w = NIN >= 2 ? b[t] : alpha;
+        y[t] = f(x, w, tab);
+      }
     }
   }
 }
@@ -82,8 +92,9 @@ static int launch_ew(F f, int n, const float* a, const float* b, float alpha, fl
   const bool vec = aligned16(y) && (NIN < 1 || aligned16(a)) && (NIN < 2 || aligned16(b));
   if (vec) {
     const uint32_t n4 = static_cast<uint32_t>(n) / 4;
-    const uint32_t grid = stream_grid(n4 + 1);
-    ew_vec_kernel<NIN, F><<<grid, kStream, 0, s>>>(f, a, b, y, n4, static_cast<uint32_t>(n), alpha);
+    constexpr int V = vectors_per_lane<F>::value;
+    const uint32_t grid = stream_grid((n4 + V) / V);  // n4 + 1 vector slots, V per lane
+    ew_vec_kernel<NIN, F, V><<<grid, kStream, 0, s>>>(f, a, b, y, n4, static_cast<uint32_t>(n), alpha);
   } else {
     const uint32_t grid = stream_grid(static_cast<uint32_t>(n));
     ew_scalar_kernel<NIN, F><<<grid, kStream, 0, s>>>(f, a, b, y, static_cast<uint32_t>(n), alpha);

@@ -20,6 +20,14 @@ struct uses_exp_table { static constexpr bool value = false; };
 template <class F>
 struct uses_exp_table<F, decltype((void)F::kExpTable)> { static constexpr bool value = F::kExpTable; };
 
+// Functors with a long dependent chain per element declare
+// `static constexpr int kVectorsPerLane = 2`: a lane then owns two vectors and
+// has the second one's load in flight while it works on the first.
+template <class F, class = void>
+struct vectors_per_lane { static constexpr int value = 1; };
+template <class F>
+struct vectors_per_lane<F, decltype((void)F::kVectorsPerLane)> { static constexpr int value = F::kVectorsPerLane; };
+
 SHDW_DEVICE float sel_max(float a, float b) { return (a < b) ? b : a; }
 SHDW_DEVICE float sel_min(float a, float b) { return (b < a) ? b : a; }
 
@@ -53,7 +61,7 @@ struct BMin { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab
 // ---- activations: shadow/operators/kernels/activate.cpp:9-31 ----
 struct ARelu { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return x > 0 ? x : 0; } };
 struct ALeaky { SHDW_DEVICE float operator()(float x, float s, const uint64_t* tab) const { return x > 0 ? x : s * x; } };
-struct ASigmoid { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_sigmoidf(x, tab); } };
+struct ASigmoid { static constexpr bool kExpTable = true; static constexpr int kVectorsPerLane = 2; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_sigmoidf(x, tab); } };
 struct ASoftPlus { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_softplusf(x, tab); } };
 struct ATanh { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_tanhf(x); } };
 struct ARelu6 { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return x < 0 ? 0 : (x > 6 ? 6 : x); } };

@@ -253,7 +253,21 @@ SHDW_LIBM_FN float exact_tanhf(float x) {
 // 1 / (1 + exp(-x)) in fp32, the way shadow/operators/kernels/activate.cpp:16
 // writes it.
 SHDW_LIBM_FN float exact_sigmoidf(float x, const uint64_t* tab) {
-  return 1.0f / (1.0f + exact_expf(-x, tab));
+  const float d = 1.0f + exact_expf(-x, tab);
+#if defined(__HIP_DEVICE_COMPILE__)
+  // d >= 1.  While d < 2^126 the quotient is a normal number and the hardware
+  // reciprocal plus one correction from the exact remainder 1 - d * r is the
+  // correctly rounded 1 / d for every d this function can produce (all 2^32
+  // inputs compared with the full division on the device); from 2^126 on
+  // (x < -87.3) the quotient is subnormal and only the full division is right.
+  // The wave takes the short form when none of its lanes is in that range.
+  if (__builtin_amdgcn_ballot_w64(!(d < 0x1p126f)) == 0) {
+    const float r = __builtin_amdgcn_rcpf(d);
+    const float e = __builtin_fmaf(-d, r, 1.0f);
+    return __builtin_fmaf(e, r, r);
+  }
+#endif
+  return 1.0f / d;
 }
 #if !defined(__HIPCC__)
 SHDW_LIBM_FN float exact_expf(float x) { return exact_expf(x, kExp2fTab); }
