@@ -187,8 +187,11 @@ SHDW_LIBM_FN float exact_expm1f(float x) {
 // with the library's operations in the library's order and the applicable one is
 // selected.  Where a cheaper form gives the same bits on every input it replaces
 // the library's:
-//   * k = rint(a / ln2) instead of the truncation of a / ln2 -+ 0.5 and of the
-//     separate |a| < 0.5 ln2 and |a| < 1.5 ln2 cases (k = 0, k = +-1 there too);
+//   * k = rint(a / ln2), taken from one fused multiply-add with 1.5 * 2^23,
+//     instead of the truncation of a / ln2 -+ 0.5 and of the separate
+//     |a| < 0.5 ln2 and |a| < 1.5 ln2 cases (k = 0, k = +-1 there too);
+//   * fused operations where the product is exact and the fusion therefore
+//     changes nothing (a - k * ln2_hi, 0.5 * v - 0.5);
 //   * hi - lo and the correction term c are taken for k = 0 as well (lo = 0
 //     makes them x and 0);
 //   * y = (1 - 2^-k) - (e - x) also for 23 <= k, where the library switches to
@@ -214,9 +217,15 @@ SHDW_LIBM_FN float exact_tanhf(float x) {
   const float a = big ? a2 : -a2;  // argument of expm1f
 
   // --- expm1f(a): argument reduction ---
-  const float tk = __builtin_rintf(invln2 * a);
-  const int32_t k = static_cast<int32_t>(tk);
-  const float hi = a - tk * ln2_hi;
+  // k = rint(a / ln2) by the 1.5 * 2^23 trick: the sum's low mantissa bits are k
+  // in two's complement, which is all the shifts below need of it.
+  const float magic = 12582912.0f;
+  const float tsum = __builtin_fmaf(invln2, a, magic);
+  const float tk = tsum - magic;
+  const uint32_t kbits = f2u(tsum);  // k modulo 2^22 in the low bits
+  // tk * ln2_hi is exact (|tk| <= 29, ln2_hi has 17 significant bits), so the
+  // fused form is the library's a - tk * ln2_hi bit for bit
+  const float hi = __builtin_fmaf(-tk, ln2_hi, a);
   const float lo = tk * ln2_lo;
   const float xr = hi - lo;
   const float c = (hi - xr) - lo;
@@ -231,14 +240,14 @@ SHDW_LIBM_FN float exact_tanhf(float x) {
   const float res_k0 = xr - (xr * e - hxs);
   e = (xr * (e - c) - c);
   e -= hxs;
-  const float res_km1 = 0.5f * (xr - e) - 0.5f;
+  const float res_km1 = __builtin_fmaf(0.5f, xr - e, -0.5f);  // the halving is exact: same as 0.5f * (xr - e) - 0.5f
   // k >= 3: y = (1 - 2^-k) - (e - x), result y * 2^k.  k <= -2: y = 1 - (e - x),
   // result y * 2^k - 1; the shift count k & 31 is then 29 or more and leaves 1.
-  const float t_lo = u2f(0x3f800000u - (0x1000000u >> (static_cast<uint32_t>(k) & 31u)));
+  const float t_lo = u2f(0x3f800000u - (0x1000000u >> (kbits & 31u)));
   float yk = t_lo - (e - xr);
-  yk = u2f(f2u(yk) + (static_cast<uint32_t>(k) << 23));  // scale by 2^k
+  yk = u2f(f2u(yk) + (kbits << 23));  // scale by 2^k
   const float res_gen = big ? yk : yk - one;
-  const float t = (k == 0) ? res_k0 : ((k == -1) ? res_km1 : res_gen);
+  const float t = (tk == 0.0f) ? res_k0 : ((tk == -1.0f) ? res_km1 : res_gen);
 
   // --- tanhf ---
   const float q = div_normal(big ? two : t, t + two);
