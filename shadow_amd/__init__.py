@@ -205,6 +205,7 @@ HOST_SIGNATURES = {
     "shdw_host_parse_net_binary": (_I, [_V, _I, _I, ctypes.c_char_p, _Z]),
     "shdw_host_proto_reencode": (_I, [_V, _I, _I, _V, _Z]),
     "shdw_host_serialize_net": (_I, [ctypes.c_char_p, _V, _Z]),
+    "shdw_host_proto_file_reencode": (_I, [ctypes.c_char_p, ctypes.c_char_p, _I]),
     "shdw_host_network_destroy": (None, [_V]),
     "shdw_host_network_io": (_I, [_V, _I, ctypes.c_char_p, _Z]),
     "shdw_host_network_forward": (_I, [_V, _I, ctypes.POINTER(ctypes.c_char_p), c_void_pp, c_int_p, c_int_p]),

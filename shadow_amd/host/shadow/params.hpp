@@ -19,7 +19,8 @@ namespace shadow {
 class Argument {
  public:
   const std::string& name() const { return name_; }
-  void set_name(const std::string& v) { name_ = v; }
+  void set_name(const std::string& v) { name_ = v, has_name_ = true; }
+  bool has_name() const { return has_name_; }
 
   bool has_s_f() const { return has_f_; }
   float s_f() const { return s_f_; }
@@ -48,7 +49,7 @@ class Argument {
   float s_f_ = 0.f;
   int s_i_ = 0;
   std::string s_s_;
-  bool has_f_ = false, has_i_ = false, has_s_ = false;
+  bool has_f_ = false, has_i_ = false, has_s_ = false, has_name_ = false;
   std::vector<float> v_f_;
   std::vector<int> v_i_;
   std::vector<std::string> v_s_;
@@ -57,9 +58,11 @@ class Argument {
 class OpParam {
  public:
   const std::string& name() const { return name_; }
-  void set_name(const std::string& v) { name_ = v; }
+  void set_name(const std::string& v) { name_ = v, has_name_ = true; }
+  bool has_name() const { return has_name_; }
   const std::string& type() const { return type_; }
-  void set_type(const std::string& v) { type_ = v; }
+  void set_type(const std::string& v) { type_ = v, op_has_type_ = true; }
+  bool has_type() const { return op_has_type_; }
 
   const std::vector<std::string>& bottom() const { return bottom_; }
   const std::string& bottom(int i) const { return bottom_[i]; }
@@ -80,6 +83,7 @@ class OpParam {
 
  private:
   std::string name_, type_;
+  bool has_name_ = false, op_has_type_ = false;
   std::vector<std::string> bottom_, top_;
   std::vector<Argument> arg_;
 };
@@ -89,7 +93,8 @@ class OpParam {
 class Blob {
  public:
   const std::string& name() const { return name_; }
-  void set_name(const std::string& v) { name_ = v; }
+  void set_name(const std::string& v) { name_ = v, has_name_ = true; }
+  bool has_name() const { return has_name_; }
   bool has_type() const { return has_type_; }
   const std::string& type() const { return type_; }
   void set_type(const std::string& v) { type_ = v, has_type_ = true; }
@@ -111,7 +116,7 @@ class Blob {
 
  private:
   std::string name_{"None"}, type_{"None"};
-  bool has_type_ = false;
+  bool has_type_ = false, has_name_ = false;
   std::vector<int> shape_;
   std::vector<float> data_f_;
   std::vector<int> data_i_;
@@ -121,7 +126,8 @@ class Blob {
 class NetParam {
  public:
   const std::string& name() const { return name_; }
-  void set_name(const std::string& v) { name_ = v; }
+  void set_name(const std::string& v) { name_ = v, has_name_ = true; }
+  bool has_name() const { return has_name_; }
   const std::vector<Blob>& blob() const { return blob_; }
   const Blob& blob(int i) const { return blob_[i]; }
   Blob* add_blob() {
@@ -144,6 +150,7 @@ class NetParam {
 
  private:
   std::string name_;
+  bool has_name_ = false;
   std::vector<Blob> blob_;
   std::vector<OpParam> op_;
   std::vector<Argument> arg_;
@@ -153,7 +160,8 @@ class NetParam {
 class MetaNetParam {
  public:
   const std::string& name() const { return name_; }
-  void set_name(const std::string& v) { name_ = v; }
+  void set_name(const std::string& v) { name_ = v, has_name_ = true; }
+  bool has_name() const { return has_name_; }
   const std::vector<NetParam>& network() const { return network_; }
   const NetParam& network(int i) const { return network_[i]; }
   NetParam* add_network() {
@@ -169,6 +177,7 @@ class MetaNetParam {
 
  private:
   std::string name_;
+  bool has_name_ = false;
   std::vector<NetParam> network_;
   std::vector<Argument> arg_;
 };

@@ -251,6 +251,22 @@ int shdw_host_proto_reencode(const void* data, int size, int is_meta, void* buf,
   return len;
 }
 
+// Host-only.  The same through files: reads `path_in`, writes `path_out`.
+// 0 on success, -1 when the file is missing or malformed.
+int shdw_host_proto_file_reencode(const char* path_in, const char* path_out, int is_meta) {
+  return guarded([&] {
+    if (is_meta) {
+      shadow::MetaNetParam meta;
+      CHECK(IO::ReadProtoFromBinaryFile(path_in, &meta)) << "Error when loading proto binary file: " << path_in;
+      CHECK(IO::WriteProtoToBinaryFile(meta, path_out));
+    } else {
+      shadow::NetParam net;
+      CHECK(IO::ReadProtoFromBinaryFile(path_in, &net)) << "Error when loading proto binary file: " << path_in;
+      CHECK(IO::WriteProtoToBinaryFile(net, path_out));
+    }
+  });
+}
+
 // Host-only.  The text form encoded as a binary NetParam.
 int shdw_host_serialize_net(const char* proto_text, void* buf, size_t n) {
   int len = -1;

@@ -241,11 +241,10 @@ void put_bytes(std::string* out, uint32_t field, const char* data, size_t size) 
 }
 void put_string(std::string* out, uint32_t field, const std::string& v) { put_bytes(out, field, v.data(), v.size()); }
 
-// proto2 writes an optional field only when it was set; the records here keep a
-// presence bit for the three scalars and for Blob.type, and treat a name as set
-// when it differs from the record's initial value.
+// proto2 writes an optional field only when it was set (an empty string that was
+// set is written); the records keep a presence bit per optional field.
 void write(const shadow::Argument& arg, std::string* out) {
-  if (!arg.name().empty()) put_string(out, 1, arg.name());
+  if (arg.has_name()) put_string(out, 1, arg.name());
   if (arg.has_s_f()) put_tag(out, 2, kFixed32), put_fixed32(out, arg.s_f());
   if (arg.has_s_i()) put_tag(out, 3, kVarint), put_int32(out, arg.s_i());
   if (arg.has_s_s()) put_string(out, 4, arg.s_s());
@@ -255,7 +254,7 @@ void write(const shadow::Argument& arg, std::string* out) {
 }
 
 void write(const shadow::Blob& blob, std::string* out) {
-  if (blob.name() != "None") put_string(out, 1, blob.name());
+  if (blob.has_name()) put_string(out, 1, blob.name());
   if (blob.has_type()) put_string(out, 2, blob.type());
   for (int v : blob.shape()) put_tag(out, 3, kVarint), put_int32(out, v);
   if (blob.data_f_size() > 0) {
@@ -280,22 +279,22 @@ void put_message(std::string* out, uint32_t field, const Sub& sub) {
 }
 
 void write(const shadow::OpParam& op, std::string* out) {
-  if (!op.name().empty()) put_string(out, 1, op.name());
-  if (!op.type().empty()) put_string(out, 2, op.type());
+  if (op.has_name()) put_string(out, 1, op.name());
+  if (op.has_type()) put_string(out, 2, op.type());
   for (const auto& v : op.bottom()) put_string(out, 3, v);
   for (const auto& v : op.top()) put_string(out, 4, v);
   for (const auto& a : op.arg()) put_message(out, 11, a);
 }
 
 void write(const shadow::NetParam& net, std::string* out) {
-  if (!net.name().empty()) put_string(out, 1, net.name());
+  if (net.has_name()) put_string(out, 1, net.name());
   for (const auto& b : net.blob()) put_message(out, 5, b);
   for (const auto& o : net.op()) put_message(out, 11, o);
   for (const auto& a : net.arg()) put_message(out, 12, a);
 }
 
 void write(const shadow::MetaNetParam& meta, std::string* out) {
-  if (!meta.name().empty()) put_string(out, 1, meta.name());
+  if (meta.has_name()) put_string(out, 1, meta.name());
   for (const auto& n : meta.network()) put_message(out, 11, n);
   for (const auto& a : meta.arg()) put_message(out, 12, a);
 }

@@ -165,3 +165,74 @@ def test_text_form_and_binary_form_describe_the_same_net():
     got = sp.NetParam()
     got.ParseFromString(shadow_amd.serialize_net(onet.write_text(text_net)))
     assert got == sp.from_oracle_net(text_net)
+
+
+def test_model_files(tmp_path):
+    lib = shadow_amd.host()
+    meta = sp.MetaNetParam()
+    meta.name = "file model"
+    meta.network.add().CopyFrom(rich_net())
+    src, dst = tmp_path / "in.shadowmodel", tmp_path / "out.shadowmodel"
+    src.write_bytes(meta.SerializeToString())
+    assert lib.shdw_host_proto_file_reencode(str(src).encode(), str(dst).encode(), 1) == 0
+    again = sp.MetaNetParam()
+    again.ParseFromString(dst.read_bytes())
+    assert again == meta
+    # an absent file is a CHECK failure like the reference's "File not found"
+    assert lib.shdw_host_proto_file_reencode(str(tmp_path / "absent").encode(), str(dst).encode(), 1) != 0
+    assert "File not found" in lib.shdw_host_last_error().decode()
+    src.write_bytes(meta.SerializeToString()[:-2])
+    assert lib.shdw_host_proto_file_reencode(str(src).encode(), str(dst).encode(), 1) != 0
+
+
+def test_random_nets_round_trip():
+    """Seeded random messages of every shape the schema allows, both directions."""
+    rng = np.random.default_rng(7)
+    words = ["", "a", "conv1/out", "x y", "\u00e9\u4e2d", "blob_%d"]
+
+    def word():
+        w = words[rng.integers(len(words))]
+        return w % rng.integers(100) if "%d" in w else w
+
+    def fill_arg(a):
+        a.name = word()
+        kind = rng.integers(7)
+        if kind == 0:
+            a.s_f = float(np.float32(rng.normal() * 10.0 ** int(rng.integers(-30, 30))))
+        elif kind == 1:
+            a.s_i = int(rng.integers(-2 ** 31, 2 ** 31))
+        elif kind == 2:
+            a.s_s = word()
+        elif kind == 3:
+            a.v_f.extend(float(np.float32(v)) for v in rng.normal(size=rng.integers(0, 6)))
+        elif kind == 4:
+            a.v_i.extend(int(v) for v in rng.integers(-2 ** 31, 2 ** 31, size=rng.integers(0, 6)))
+        elif kind == 5:
+            a.v_s.extend(word() for _ in range(rng.integers(0, 4)))
+
+    for _ in range(60):
+        n = sp.NetParam()
+        if rng.integers(2):
+            n.name = word()
+        for _ in range(rng.integers(0, 4)):
+            b = n.blob.add()
+            if rng.integers(4):
+                b.name = word() or "w"
+            if rng.integers(2):
+                b.type = ["float", "int32", "uint8"][rng.integers(3)]
+            b.shape.extend(int(v) for v in rng.integers(0, 300, size=rng.integers(0, 5)))
+            b.data_f.extend(float(np.float32(v)) for v in rng.normal(size=rng.integers(0, 9)))
+            b.data_i.extend(int(v) for v in rng.integers(-2 ** 31, 2 ** 31, size=rng.integers(0, 9)))
+            for _ in range(rng.integers(0, 3)):
+                b.data_b.append(rng.integers(0, 256, size=rng.integers(0, 40), dtype=np.uint8).tobytes())
+        for _ in range(rng.integers(0, 5)):
+            o = n.op.add()
+            o.type, o.name = word() or "T", word() or "n"
+            o.bottom.extend(word() for _ in range(rng.integers(0, 3)))
+            o.top.extend(word() for _ in range(rng.integers(0, 3)))
+            for _ in range(rng.integers(0, 4)):
+                fill_arg(o.arg.add())
+        for _ in range(rng.integers(0, 3)):
+            fill_arg(n.arg.add())
+        wire = n.SerializeToString()
+        assert shadow_amd.reencode_proto(wire) == wire
