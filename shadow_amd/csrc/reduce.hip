@@ -262,7 +262,7 @@ __global__ __launch_bounds__(kWave * WAVES) void reduce_strided_kernel(
   const uint32_t lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
   // grid.x = outer * tiles (either can exceed the 65535 limit of grid.y), grid.y = slices
   uint32_t o, tile;
-  fd_divmod(blockIdx.x, f_tiles, o, tile);
+  fd_divmod(xcd_contiguous(blockIdx.x, gridDim.x), f_tiles, o, tile);
   const uint32_t col = (tile * kWave + lane) * VEC;
   const uint32_t split = blockIdx.y;
   const bool col_ok = col < inner;

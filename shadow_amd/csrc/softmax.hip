@@ -101,7 +101,7 @@ __global__ __launch_bounds__(kBlock) void softmax_columns_reg_kernel(const float
   __shared__ uint64_t tab[32];
   if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
   __syncthreads();
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t i = xcd_contiguous(blockIdx.x, gridDim.x) * kBlock + threadIdx.x;  // neighbours share straddled lines
   if (i >= columns) return;
   uint32_t n, s;
   fd_divmod(i, f_inner, n, s);
@@ -328,7 +328,7 @@ __global__ __launch_bounds__(kBlock) void normalize_columns_reg_kernel(const flo
                                                                         FastDiv f_inner, float p,
                                                                         float eps,
                                                                         const float* scale = nullptr) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t i = xcd_contiguous(blockIdx.x, gridDim.x) * kBlock + threadIdx.x;  // neighbours share straddled lines
   if (i >= columns) return;
   uint32_t n, s;
   fd_divmod(i, f_inner, n, s);
