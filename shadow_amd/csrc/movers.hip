@@ -276,7 +276,11 @@ typedef float v2f __attribute__((ext_vector_type(2)));
 template <bool DARKNET, bool S2>
 __global__ __launch_bounds__(kBlock) void reorg_scatter_kernel(const float* x, float* y, uint32_t n4,
                                                                 ReorgScatterArgs p) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  // The natural order writes neighbouring source rows into the same destination
+  // lines: XCD-contiguous workgroups let those halves meet in one L2 (72 -> 69 us);
+  // the Darknet order does not share lines and is 3 us slower that way.
+  const uint32_t block = DARKNET ? blockIdx.x : xcd_contiguous(blockIdx.x, gridDim.x);
+  const uint32_t i = block * kBlock + threadIdx.x;
   if (i >= n4) return;
   const v4f v = load4_stream(x + 4ull * i);
   uint32_t rest, ws, hs, b, cs, h, oh;
