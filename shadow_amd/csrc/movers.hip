@@ -319,7 +319,8 @@ struct ResizeArgs {
 template <int Q>
 __global__ __launch_bounds__(kBlock) void resize_nearest_kernel(const float* x, float* y, uint32_t work,
                                                                  ResizeArgs p) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  // neighbouring workgroups read the same input rows
+  const uint32_t i = xcd_contiguous(blockIdx.x, gridDim.x) * kBlock + threadIdx.x;
   if (i >= work) return;
   uint32_t rest, w, plane, h;
   fd_divmod(Q * i, p.f_out_w, rest, w);
