@@ -56,7 +56,7 @@ __global__ __launch_bounds__(kStream) void rowparam_vec_kernel(const float* x, c
                                                                FastDiv inner, FastDiv num) {
   const uint32_t i = blockIdx.x * kStream + threadIdx.x;
   if (i < n4) {
-    const v4f vx = load4_stream(x + 4ull * i);
+    const v4f vx = load4_stream_any(x + 4ull * i);  // any float pointer
     v4f r;
     if (ROWVEC) {
       const uint32_t row = fd_div(4 * i, inner);
@@ -69,19 +69,10 @@ __global__ __launch_bounds__(kStream) void rowparam_vec_kernel(const float* x, c
 #pragma unroll
       for (int j = 0; j < 4; ++j) r[j] = row_element<MODE, RELU>(4 * i + j, vx[j], s, b, inner, num);
     }
-    store4_stream(y + 4ull * i, r);
+    store4_stream_any(y + 4ull * i, r);
   } else if (i == n4) {
     for (uint32_t t = 4 * n4; t < n; ++t) y[t] = row_element<MODE, RELU>(t, x[t], s, b, inner, num);
   }
-}
-
-template <int MODE, bool RELU>
-__global__ __launch_bounds__(kStream) void rowparam_scalar_kernel(const float* x, const float* s,
-                                                                  const float* b, float* y,
-                                                                  uint32_t n, FastDiv inner,
-                                                                  FastDiv num) {
-  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
-  if (i < n) y[i] = row_element<MODE, RELU>(i, x[i], s, b, inner, num);
 }
 
 template <int MODE, bool RELU>
@@ -89,16 +80,12 @@ static int launch_rowparam(int n, int num, int inner, const float* x, const floa
                            const float* b, float* y, hipStream_t st) {
   const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner));
   const FastDiv fn = make_fastdiv(static_cast<uint32_t>(num));
-  if (aligned16(x) && aligned16(y)) {
-    const uint32_t n4 = static_cast<uint32_t>(n) / 4;
-    const uint32_t grid = stream_grid(n4 + 1);
-    if (inner % 4 == 0)
-      rowparam_vec_kernel<MODE, RELU, true><<<grid, kStream, 0, st>>>(x, s, b, y, n4, n, fi, fn);
-    else
-      rowparam_vec_kernel<MODE, RELU, false><<<grid, kStream, 0, st>>>(x, s, b, y, n4, n, fi, fn);
-  } else {
-    rowparam_scalar_kernel<MODE, RELU><<<stream_grid(n), kStream, 0, st>>>(x, s, b, y, n, fi, fn);
-  }
+  const uint32_t n4 = static_cast<uint32_t>(n) / 4;
+  const uint32_t grid = stream_grid(n4 + 1);
+  if (inner % 4 == 0)
+    rowparam_vec_kernel<MODE, RELU, true><<<grid, kStream, 0, st>>>(x, s, b, y, n4, n, fi, fn);
+  else
+    rowparam_vec_kernel<MODE, RELU, false><<<grid, kStream, 0, st>>>(x, s, b, y, n4, n, fi, fn);
   return launch_status();
 }
 

@@ -37,8 +37,8 @@ __global__ __launch_bounds__(kStream) void ew_vec_kernel(F f, const float* a, co
   for (int u = 0; u < V; ++u) {  // issue the streaming loads before anything else
     const uint32_t i = first + u * kStream;
     if (i < n4) {
-      if (NIN >= 1) va[u] = load4_stream(a + 4ull * i);
-      if (NIN >= 2) vb[u] = load4_stream(b + 4ull * i);
+      if (NIN >= 1) va[u] = load4_stream_any(a + 4ull * i);
+      if (NIN >= 2) vb[u] = load4_stream_any(b + 4ull * i);
     }
   }
   const uint64_t* tab = nullptr;
@@ -59,7 +59,7 @@ __global__ __launch_bounds__(kStream) void ew_vec_kernel(F f, const float* a, co
         const float w = NIN >= 2 ? vb[u][j] : alpha;
         r[j] = f(x, w, tab);
       }
-      store4_stream(y + 4ull * i, r);
+      store4_stream_any(y + 4ull * i, r);
     } else if (i == n4) {
       for (uint32_t t = 4 * n4; t < n; ++t) {
         const float x = NIN >= 1 ? a[t] : alpha;
@@ -70,35 +70,17 @@ __global__ __launch_bounds__(kStream) void ew_vec_kernel(F f, const float* a, co
   }
 }
 
-// Same arithmetic for pointers that are not 16-byte aligned (Blas offsets).
-template <int NIN, class F>
-__global__ __launch_bounds__(kStream) void ew_scalar_kernel(F f, const float* a, const float* b,
-                                                            float* y, uint32_t n, float alpha) {
-  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
-  const uint64_t* tab = uses_exp_table<F>::value ? libm::kExp2fTab : nullptr;
-  if (i < n) {
-    const float x = NIN >= 1 ? a[i] : alpha;
-    const float w = NIN >= 2 ? b[i] : alpha;
-    y[i] = f(x, w, tab);
-  }
-}
-
 template <int NIN, class F>
 static int launch_ew(F f, int n, const float* a, const float* b, float alpha, float* y,
                      void* stream) {
   if (n < 0 || !y || (NIN >= 1 && !a) || (NIN >= 2 && !b)) return SHDW_E_INVALID_ARGUMENT;
   if (n == 0) return SHDW_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool vec = aligned16(y) && (NIN < 1 || aligned16(a)) && (NIN < 2 || aligned16(b));
-  if (vec) {
-    const uint32_t n4 = static_cast<uint32_t>(n) / 4;
-    constexpr int V = vectors_per_lane<F>::value;
-    const uint32_t grid = stream_grid((n4 + V) / V);  // n4 + 1 vector slots, V per lane
-    ew_vec_kernel<NIN, F, V><<<grid, kStream, 0, s>>>(f, a, b, y, n4, static_cast<uint32_t>(n), alpha);
-  } else {
-    const uint32_t grid = stream_grid(static_cast<uint32_t>(n));
-    ew_scalar_kernel<NIN, F><<<grid, kStream, 0, s>>>(f, a, b, y, static_cast<uint32_t>(n), alpha);
-  }
+  // Any float pointers: the 128-bit accesses need dword alignment only.
+  const uint32_t n4 = static_cast<uint32_t>(n) / 4;
+  constexpr int V = vectors_per_lane<F>::value;
+  const uint32_t grid = stream_grid((n4 + V) / V);  // n4 + 1 vector slots, V per lane
+  ew_vec_kernel<NIN, F, V><<<grid, kStream, 0, s>>>(f, a, b, y, n4, static_cast<uint32_t>(n), alpha);
   return launch_status();
 }
 
@@ -166,52 +148,40 @@ SHDW_DEVICE float eltwise_fold(const EltwiseArgs& p, const float (&v)[KMAX], flo
 
 // KMAX is the compile-time bound on p.k (2, 3, 4 or 8) so that the per-input
 // registers are never indexed dynamically.
-template <int OP, int KMAX, bool VEC>
+template <int OP, int KMAX>
 __global__ __launch_bounds__(kStream) void eltwise_kernel(EltwiseArgs p, float* y, uint32_t n) {
   const uint32_t i = blockIdx.x * kStream + threadIdx.x;
-  if (VEC) {
-    const uint32_t n4 = n / 4;
-    if (i < n4) {
-      v4f v[KMAX];
-      v4f seed = {0, 0, 0, 0};
+  const uint32_t n4 = n / 4;
+  if (i < n4) {
+    v4f v[KMAX];
+    v4f seed = {0, 0, 0, 0};
 #pragma unroll
-      for (int j = 0; j < KMAX; ++j)
-        if (j < p.k) v[j] = load4_stream(p.x[j] + 4ull * i);
-      if (p.has_seed) seed = load4_stream(y + 4ull * i);
-      v4f r;
+    for (int j = 0; j < KMAX; ++j)
+      if (j < p.k) v[j] = load4_stream_any(p.x[j] + 4ull * i);
+    if (p.has_seed) seed = load4_stream_any(y + 4ull * i);
+    v4f r;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        float col[KMAX];
+    for (int c = 0; c < 4; ++c) {
+      float col[KMAX];
 #pragma unroll
-        for (int j = 0; j < KMAX; ++j) col[j] = (j < p.k) ? v[j][c] : 0.0f;
-        r[c] = eltwise_fold<OP, KMAX>(p, col, seed[c]);
-      }
-      store4_stream(y + 4ull * i, r);
-    } else if (i == n4) {
-      for (uint32_t t = 4 * n4; t < n; ++t) {
-        float col[KMAX];
-#pragma unroll
-        for (int j = 0; j < KMAX; ++j) col[j] = (j < p.k) ? p.x[j][t] : 0.0f;
-        y[t] = eltwise_fold<OP, KMAX>(p, col, p.has_seed ? y[t] : 0.0f);
-      }
+      for (int j = 0; j < KMAX; ++j) col[j] = (j < p.k) ? v[j][c] : 0.0f;
+      r[c] = eltwise_fold<OP, KMAX>(p, col, seed[c]);
     }
-  } else if (i < n) {
-    float col[KMAX];
+    store4_stream_any(y + 4ull * i, r);
+  } else if (i == n4) {
+    for (uint32_t t = 4 * n4; t < n; ++t) {
+      float col[KMAX];
 #pragma unroll
-    for (int j = 0; j < KMAX; ++j) col[j] = (j < p.k) ? p.x[j][i] : 0.0f;
-    y[i] = eltwise_fold<OP, KMAX>(p, col, p.has_seed ? y[i] : 0.0f);
+      for (int j = 0; j < KMAX; ++j) col[j] = (j < p.k) ? p.x[j][t] : 0.0f;
+      y[t] = eltwise_fold<OP, KMAX>(p, col, p.has_seed ? y[t] : 0.0f);
+    }
   }
 }
 
 template <int OP, int KMAX>
 static int launch_eltwise_k(const EltwiseArgs& p, int n, float* y, hipStream_t s) {
-  bool vec = aligned16(y);
-  for (int j = 0; j < p.k; ++j) vec = vec && aligned16(p.x[j]);
-  const uint32_t grid = stream_grid(vec ? static_cast<uint32_t>(n) / 4 + 1 : static_cast<uint32_t>(n));
-  if (vec)
-    eltwise_kernel<OP, KMAX, true><<<grid, kStream, 0, s>>>(p, y, static_cast<uint32_t>(n));
-  else
-    eltwise_kernel<OP, KMAX, false><<<grid, kStream, 0, s>>>(p, y, static_cast<uint32_t>(n));
+  const uint32_t grid = stream_grid(static_cast<uint32_t>(n) / 4 + 1);
+  eltwise_kernel<OP, KMAX><<<grid, kStream, 0, s>>>(p, y, static_cast<uint32_t>(n));
   return launch_status();
 }
 

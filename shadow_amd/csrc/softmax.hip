@@ -400,7 +400,6 @@ __global__ __launch_bounds__(kBlock) void normalize_slab_kernel(const float* x, 
 // [64,150,73,73] / [64,150,72,72]).  Neighbouring tiles share the straddled
 // lines, hence the XCD-contiguous workgroup order.
 constexpr int kTilePerLane = 16;  // 64 KB / (256 lanes x 16 bytes)
-typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
 
 // ROWS says how the tile rows lie in memory:
 //   kRowsSector: inner % 16 == 0, every row starts on a 64-byte boundary;

@@ -25,7 +25,7 @@ namespace shdw {
 struct AxpyRows {
   const float* alpha;
   const float* y;
-  SHDW_DEVICE v4f load_other(uint64_t off) const { return load4_stream(y + off); }
+  SHDW_DEVICE v4f load_other(uint64_t off) const { return load4_stream_any(y + off); }
   SHDW_DEVICE float other(uint64_t off) const { return y[off]; }
   struct Row {
     float a;
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(kStream) void rows_vec_kernel(P p, const float* x, 
                                                            uint32_t n4, uint32_t n, FastDiv inner) {
   const uint32_t i = blockIdx.x * kStream + threadIdx.x;
   if (i < n4) {
-    const v4f vx = load4_stream(x + 4ull * i);
+    const v4f vx = load4_stream_any(x + 4ull * i);
     const v4f vo = p.load_other(4ull * i);
     v4f r;
     if (ROWVEC) {
@@ -82,33 +82,22 @@ __global__ __launch_bounds__(kStream) void rows_vec_kernel(P p, const float* x, 
         r[j] = p.apply(vx[j], vo[j], rj == r0 ? rp0 : p.row(rj));
       }
     }
-    store4_stream(out + 4ull * i, r);
+    store4_stream_any(out + 4ull * i, r);
   } else if (i == n4) {
     for (uint32_t t = 4 * n4; t < n; ++t) out[t] = p.apply(x[t], p.other(t), p.row(fd_div(t, inner)));
   }
 }
 
 template <class P>
-__global__ __launch_bounds__(kStream) void rows_scalar_kernel(P p, const float* x, float* out,
-                                                              uint32_t n, FastDiv inner) {
-  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
-  if (i < n) out[i] = p.apply(x[i], p.other(i), p.row(fd_div(i, inner)));
-}
-
-template <class P>
 static int launch_rows(const P& p, uint32_t n, uint32_t inner, const float* x, const float* other,
                        float* out, hipStream_t st) {
   const FastDiv fi = make_fastdiv(inner);
-  if (aligned16(x) && aligned16(out) && (!P::kTwoInputs || aligned16(other))) {
-    const uint32_t n4 = n / 4;
-    const uint32_t grid = stream_grid(n4 + 1);
-    if (inner % 4 == 0)
-      rows_vec_kernel<P, true><<<grid, kStream, 0, st>>>(p, x, out, n4, n, fi);
-    else
-      rows_vec_kernel<P, false><<<grid, kStream, 0, st>>>(p, x, out, n4, n, fi);
-  } else {
-    rows_scalar_kernel<P><<<stream_grid(n), kStream, 0, st>>>(p, x, out, n, fi);
-  }
+  const uint32_t n4 = n / 4;  // any float pointers: the 128-bit accesses need dword alignment only
+  const uint32_t grid = stream_grid(n4 + 1);
+  if (inner % 4 == 0)
+    rows_vec_kernel<P, true><<<grid, kStream, 0, st>>>(p, x, out, n4, n, fi);
+  else
+    rows_vec_kernel<P, false><<<grid, kStream, 0, st>>>(p, x, out, n4, n, fi);
   return launch_status();
 }
 

@@ -1,15 +1,20 @@
 """Parity of every C-ABI kernel entry point with the CPU oracle on the same
 seeded inputs.  Bit-exact unless stated; fp64-accumulating reductions are held
 to |gpu - cpu| <= 1e-5 |cpu| (their association order differs)."""
+import ctypes
+
 import numpy as np
 import pytest
 
 import oracle
+import shadow_amd
+from shadow_amd import Buffer
 from tests import gpuops
 from tests.helpers import (assert_bit_exact, assert_rel_close, normal, ulp_distance, uniform,
                            with_specials)
 
 pytestmark = pytest.mark.gpu
+F = np.float32
 
 EXACT_UNARY = {0: "abs", 1: "square", 2: "sqrt", 3: "log", 4: "exp", 5: "sin", 6: "cos", 7: "tan",
                8: "asin", 9: "acos", 10: "atan", 11: "floor", 12: "ceil", 13: "neg", 14: "reciprocal"}
@@ -36,6 +41,46 @@ def test_unary_inplace_and_misaligned(gpu, op):
     assert_bit_exact(gpuops.unary(op, x, inplace=True), want, "in place")
     for off in (1, 2, 3):
         assert_bit_exact(gpuops.unary(op, x, offset=off), want, "offset %d" % off)
+
+
+def _shifted(x, off):
+    """x on the device, `off` floats past a 16-byte boundary."""
+    buf = Buffer(4 * (x.size + off) + 16)
+    buf.upload(x, 4 * off)
+    return buf, buf.ptr + 4 * off
+
+
+@pytest.mark.parametrize("offs", [(1, 2, 3), (0, 1, 0), (3, 3, 1), (2, 0, 2)])
+def test_operands_on_different_dword_offsets(gpu, offs):
+    """The 128-bit accesses of the streaming kernels take any float pointer: every
+    operand shifted by its own number of floats off 16-byte alignment."""
+    lib = shadow_amd.hip()
+    n = 70003
+    a, b = normal(30, n, 2.0), uniform(31, n, 0.5, 2.0)
+    (ba, pa), (bb, pb), (by, py) = _shifted(a, offs[0]), _shifted(b, offs[1]), _shifted(np.zeros(n, F), offs[2])
+    for op in (0, 3, 5):  # add, div, max
+        gpuops.check(lib.shdw_hip_binary(op, n, pa, pb, py, None))
+        assert_bit_exact(by.download(count=n, offset_bytes=4 * offs[2]), oracle.binary(op, a, b), "binary %d" % op)
+    # Eltwise sum with coefficients, three inputs
+    c = normal(32, n)
+    (bc, pc) = _shifted(c, offs[0])
+    ptrs = (ctypes.c_void_p * 3)(pa, pb, pc)
+    co = (ctypes.c_float * 3)(0.5, -1.25, 2.0)
+    gpuops.check(lib.shdw_hip_eltwise(1, 3, ptrs, co, n, py, None))
+    assert_bit_exact(by.download(count=n, offset_bytes=4 * offs[2]), oracle.eltwise(1, [a, b, c], [0.5, -1.25, 2.0]),
+                     "eltwise")
+    # BatchNorm and Axpy rows: row parameters per 7 x 11 = 77 elements (rows never vector-aligned)
+    rows, inner = 909, 77
+    m = rows * inner
+    mean, var = normal(33, rows), uniform(34, rows, 0.2, 3.0)
+    dm, dv = Buffer.from_numpy(mean), Buffer.from_numpy(var)
+    gpuops.check(lib.shdw_hip_batch_norm(m, rows, inner, pa, dm.ptr, dv.ptr, 0.999, 1e-5, py, None))
+    assert_bit_exact(by.download(count=m, offset_bytes=4 * offs[2]),
+                     oracle.batch_norm(a[:m], mean, var, rows, inner, F(0.999), F(1e-5)), "batch norm")
+    alpha = Buffer.from_numpy(normal(35, rows))
+    gpuops.check(lib.shdw_hip_axpy_rows(rows, inner, alpha.ptr, pa, pb, py, None))
+    assert_bit_exact(by.download(count=m, offset_bytes=4 * offs[2]),
+                     oracle.axpy_rows(normal(35, rows), a[:m], b[:m], inner), "axpy rows")
 
 
 @pytest.mark.parametrize("op", [3, 5, 6, 7, 8, 9, 10])
