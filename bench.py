@@ -342,6 +342,11 @@ def config_table(dev):
     ms = time_batch(dev, lambda k: lib.shdw_hip_reduce(4, 4, I(sh5), 2, I(ax5), A[k].ptr, M[k].ptr,
                                                        None, 0, st), SETS)
     add(5, "reduce_avg_hw", 4 * n5 + 4 * 65536, ms, n5)
+    sh7 = [128, 2048, 7, 7]  # the same reduction over 7 x 7 planes: rows of 49 floats start on odd dwords
+    M7 = [dev.buf(nbytes=4 * 128 * 2048) for _ in range(SETS)]
+    ms = time_batch(dev, lambda k: lib.shdw_hip_reduce(4, 4, I(sh7), 2, I(ax5), A[k].ptr, M7[k].ptr,
+                                                       None, 0, st), SETS)
+    add("next", "reduce_avg_hw 7x7 planes [128,2048,7,7]", 4 * n5 + 4 * 128 * 2048, ms, n5)
     ms = time_batch(dev, lambda k: lib.shdw_hip_scale_residual_relu_rowmean(
         n5, C5, in5, A[k].ptr, g5.ptr, b5.ptr, A[(k + 1) % SETS].ptr, Y[k].ptr, M[k].ptr, st), SETS)
     add(5, "fused_tail", 12 * n5 + 8 * C5 + 4 * 65536, ms, n5)

@@ -172,7 +172,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_group_kernel(const float* 
 #pragma unroll
       for (int u = 0; u < kRowBatch; ++u) {
         const uint32_t i = base + u * G + lane;
-        if (i < nv) v[u] = load4_stream(p + 4ull * i);
+        if (i < nv) v[u] = load4_stream_any(p + 4ull * i);  // rows start on any dword
       }
 #pragma unroll
       for (int u = 0; u < kRowBatch; ++u) {
@@ -183,6 +183,8 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_group_kernel(const float* 
         }
       }
     }
+    const uint32_t t = 4 * nv + lane;  // the reduce % 4 elements past the last whole vector
+    if (t < reduce) acc.add(p[t], t);
   } else {
     for (uint32_t i = lane; i < reduce; i += G) acc.add(p[i], i);
   }
@@ -214,14 +216,14 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const float* 
       for (; i + 3 * kBlock < ve; i += 4 * kBlock) {
         v4f v[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = load4_stream(p + 4ull * (i + u * kBlock));
+        for (int u = 0; u < 4; ++u) v[u] = load4_stream_any(p + 4ull * (i + u * kBlock));
 #pragma unroll
         for (int u = 0; u < 4; ++u)
 #pragma unroll
           for (int j = 0; j < 4; ++j) acc.add(v[u][j], 4 * (i + u * kBlock) + j);
       }
       for (; i < ve; i += kBlock) {
-        const v4f v = load4_stream(p + 4ull * i);
+        const v4f v = load4_stream_any(p + 4ull * i);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc.add(v[j], 4 * i + j);
       }
@@ -460,17 +462,17 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
   if (pl.kind == kRows) {
     const uint32_t rows = static_cast<uint32_t>(pl.outer);
     const uint32_t reduce = static_cast<uint32_t>(pl.reduce);
-    // 128-bit loads need every row start 16-byte aligned.
-    const bool vec = aligned16(x) && (reduce % 4 == 0 || rows == 1);
+    // 128-bit loads on any dword address: rows need not start 16-byte aligned.
+    const bool vec = reduce >= 4;
     if (pl.wave_per_row) {
       // lanes per row: a lane fetches up to 8 vectors, all requested before the
       // first is consumed (measured on 784-float rows: 16 lanes 9.4 us, 32 lanes
       // 9.0 us, 64 lanes 10.4 us; with 4 requests in flight 9.9 us)
-      const uint32_t units = (vec && reduce % 4 == 0) ? reduce / 4 : reduce;
+      const uint32_t units = vec ? (reduce + 3) / 4 : reduce;
       const int g = units <= 128 ? 16 : (units <= 256 ? 32 : 64);
       const uint32_t grid = (rows + kBlock / g - 1) / (kBlock / g);
 #define SHDW_ROWS(V, G) reduce_rows_group_kernel<OP, V, G><<<grid, kBlock, 0, st>>>(x, y, rows, reduce)
-      if (vec && reduce % 4 == 0) {
+      if (vec) {
         if (g == 16) SHDW_ROWS(true, 16); else if (g == 32) SHDW_ROWS(true, 32); else SHDW_ROWS(true, 64);
       } else {
         if (g == 16) SHDW_ROWS(false, 16); else if (g == 32) SHDW_ROWS(false, 32); else SHDW_ROWS(false, 64);

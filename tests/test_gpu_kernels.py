@@ -271,6 +271,10 @@ REDUCE_CASES = [
     ([2, 40000], [1]),           # rows, long, few
     ([2, 30000, 8], [1]),        # strided, 16 waves per tile and a second stage
     ([3, 200, 12], [1]),         # strided, 16 waves per tile, single stage
+    ([1000, 49], [1]),           # rows of 49: unaligned 128-bit loads plus one tail element
+    ([300, 6, 7, 7], [2, 3]),
+    ([3, 40001], [1]),           # long rows that start on odd dwords
+    ([500, 3], [1]),             # rows shorter than one vector
 ]
 
 
