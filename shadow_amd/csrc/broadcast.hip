@@ -144,6 +144,74 @@ __global__ __launch_bounds__(kBlock) void bcast_vec_kernel(F f, BcastArgs p, con
   }
 }
 
+// The same for an innermost extent that is not a multiple of 4 (7 x 7, 13 x 13
+// maps) or operands on odd dwords: a lane still owns 4 consecutive outputs and
+// one 128-bit store, but they may lie in two or more innermost rows.  Lanes whose
+// four outputs share a row take one vector (or one replicated scalar) per
+// operand; the others decode each output on its own.  One output per lane ran
+// at 2.0-2.8 TB/s on such shapes against 5.7 TB/s for their aligned cousins.
+template <class F, int NDIM>
+SHDW_DEVICE void bcast_offsets(const BcastArgs& p, uint32_t e, uint32_t& oa, uint32_t& ob, uint32_t& col) {
+  oa = 0, ob = 0, col = e;
+#pragma unroll
+  for (int k = NDIM - 1; k >= 1; --k) {
+    uint32_t q, r;
+    fd_divmod(e, p.fd[k], q, r);
+    if (k == NDIM - 1) col = r;
+    oa += r * static_cast<uint32_t>(p.sa[k]);
+    ob += r * static_cast<uint32_t>(p.sb[k]);
+    e = q;
+  }
+  oa += e * static_cast<uint32_t>(p.sa[0]);
+  ob += e * static_cast<uint32_t>(p.sb[0]);
+}
+
+template <class F, int NDIM>
+__global__ __launch_bounds__(kBlock) void bcast_flat_kernel(F f, BcastArgs p, const float* a,
+                                                             const float* b, float* y, uint32_t n4,
+                                                             uint32_t n) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;  // 64 or 256 lanes, see the launch
+  const uint64_t* tab = uses_exp_table<F>::value ? libm::kExp2fTab : nullptr;
+  const uint32_t last = p.fd[NDIM - 1].d;
+  const int sa = p.sa[NDIM - 1], sb = p.sb[NDIM - 1];  // 0 or 1
+  if (i < n4) {
+    uint32_t oa, ob, col;
+    bcast_offsets<F, NDIM>(p, 4 * i, oa, ob, col);
+    v4f va, vb;
+    if (col + 4 <= last) {
+      if (sa) {  // a re-used (broadcast) operand stays cacheable
+        va = p.a_full ? load4_stream_any(a + oa) : load4_any(a + oa);
+      } else {
+        const float t = a[oa];
+        va = {t, t, t, t};
+      }
+      if (sb) {
+        vb = p.b_full ? load4_stream_any(b + ob) : load4_any(b + ob);
+      } else {
+        const float t = b[ob];
+        vb = {t, t, t, t};
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t pa, pb, unused;
+        bcast_offsets<F, NDIM>(p, 4 * i + j, pa, pb, unused);
+        va[j] = a[pa], vb[j] = b[pb];
+      }
+    }
+    v4f r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = f(va[j], vb[j], tab);
+    store4_stream_any(y + 4ull * i, r);
+  } else if (i == n4) {
+    for (uint32_t t = 4 * n4; t < n; ++t) {
+      uint32_t pa, pb, unused;
+      bcast_offsets<F, NDIM>(p, t, pa, pb, unused);
+      y[t] = f(a[pa], b[pb], tab);
+    }
+  }
+}
+
 struct BcastGenericArgs {
   int ndim;
   FastDiv fd[kMaxDims];
@@ -223,6 +291,25 @@ static int launch_bcast(F f, const BroadcastPlan& plan, const float* a, const fl
       case 2: launch_bcast_vec<F, 2>(f, p, avec, bvec, a, b, y, n4, st); break;
       case 3: launch_bcast_vec<F, 3>(f, p, avec, bvec, a, b, y, n4, st); break;
       default: launch_bcast_vec<F, 4>(f, p, avec, bvec, a, b, y, n4, st); break;
+    }
+  } else if (nd <= 4) {
+    BcastArgs p;
+    p.a_full = p.b_full = 1;
+    for (int k = 0; k < 4; ++k) {
+      p.fd[k] = make_fastdiv(k < nd ? static_cast<uint32_t>(pl.dims[k]) : 1u);
+      p.sa[k] = k < nd ? pl.sa[k] : 0;
+      p.sb[k] = k < nd ? pl.sb[k] : 0;
+      if (k < nd && pl.sa[k] == 0) p.a_full = 0;
+      if (k < nd && pl.sb[k] == 0) p.b_full = 0;
+    }
+    const uint32_t n4 = n / 4;
+    const uint32_t lanes = (p.a_full || p.b_full) ? kStream : kBlock;  // as in launch_bcast_vec
+    const uint32_t grid = (n4 + 1 + lanes - 1) / lanes;
+    switch (nd) {
+      case 1: bcast_flat_kernel<F, 1><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
+      case 2: bcast_flat_kernel<F, 2><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
+      case 3: bcast_flat_kernel<F, 3><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
+      default: bcast_flat_kernel<F, 4><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
     }
   } else {
     BcastGenericArgs p;

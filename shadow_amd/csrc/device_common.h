@@ -48,6 +48,7 @@ typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
 SHDW_DEVICE v4f load4_stream_any(const float* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const v4f_unaligned*>(p));
 }
+SHDW_DEVICE v4f load4_any(const float* p) { return *reinterpret_cast<const v4f_unaligned*>(p); }
 SHDW_DEVICE void store4_stream_any(float* p, v4f v) {
   __builtin_nontemporal_store(v, reinterpret_cast<v4f_unaligned*>(p));
 }

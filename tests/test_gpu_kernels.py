@@ -213,6 +213,14 @@ BCAST_CASES = [
     ([1, 7], [9, 1]),
     ([6, 1, 10], [6, 4, 1]),
     ([33, 4], [1, 4]),
+    # innermost extent not a multiple of 4: four outputs per lane across row ends
+    ([6, 20, 7, 7], [1, 20, 1, 1]),
+    ([5, 1, 13, 13], [1, 9, 13, 1]),
+    ([3, 7, 1, 9], [1, 1, 5, 9]),
+    ([1001, 3], [1, 3]),
+    ([2, 3], [2, 3]),
+    ([17, 1, 3], [1, 11, 1]),
+    ([3, 1, 2, 1, 7], [1, 4, 1, 6, 1]),   # five dims after collapsing: one output per lane
 ]
 
 
