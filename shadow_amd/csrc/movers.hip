@@ -71,19 +71,39 @@ struct ShuffleRows {
   }
 };
 
-template <class MAP, bool VEC>
+// inner % 4 == 0 and 16-byte aligned pointers: lane i moves vector i.
+template <class MAP>
 __global__ __launch_bounds__(kStream) void rows_pick_kernel(MAP map, const float* x, float* y,
                                                             uint32_t work, FastDiv f_inner) {
   const uint32_t i = blockIdx.x * kStream + threadIdx.x;
   if (i >= work) return;
   uint32_t r, p;
-  fd_divmod(i, f_inner, r, p);  // VEC: inner counted in vectors
+  fd_divmod(i, f_inner, r, p);  // inner counted in vectors
   const int64_t s = map.source(r);
-  if (VEC) {
+  const v4f zero = {0.f, 0.f, 0.f, 0.f};
+  store4_stream(y + 4ull * i, s < 0 ? zero : load4(x + 4 * (s * f_inner.d + p)));
+}
+
+// Rows of any length on any dword address: a lane moves the vector at floats
+// 4p .. 4p + 3 of its row with 128-bit accesses, the last lane of a row the
+// inner % 4 floats that remain (rows of 49 ran 2.2x slower with one float per lane).
+template <class MAP>
+__global__ __launch_bounds__(kStream) void rows_pick_any_kernel(MAP map, const float* x, float* y,
+                                                                uint32_t work, uint32_t inner,
+                                                                FastDiv f_units) {
+  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
+  if (i >= work) return;
+  uint32_t r, p;
+  fd_divmod(i, f_units, r, p);
+  const int64_t s = map.source(r);
+  const uint32_t first = 4 * p;
+  float* dst = y + static_cast<uint64_t>(r) * inner + first;
+  const float* src = x + s * inner + first;
+  if (first + 4 <= inner) {
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
-    store4_stream(y + 4ull * i, s < 0 ? zero : load4(x + 4 * (s * f_inner.d + p)));
+    store4_stream_any(dst, s < 0 ? zero : load4_stream_any(src));
   } else {
-    y[i] = s < 0 ? 0.f : x[s * f_inner.d + p];
+    for (uint32_t j = 0; first + j < inner; ++j) dst[j] = s < 0 ? 0.f : src[j];
   }
 }
 
@@ -92,10 +112,12 @@ static int launch_rows_pick(const MAP& map, int64_t rows, int inner, const float
                             hipStream_t st) {
   if (inner % 4 == 0 && aligned16(x) && aligned16(y)) {
     const uint32_t work = static_cast<uint32_t>(rows * (inner / 4));
-    rows_pick_kernel<MAP, true><<<stream_grid(work), kStream, 0, st>>>(map, x, y, work, make_fastdiv(inner / 4));
+    rows_pick_kernel<MAP><<<stream_grid(work), kStream, 0, st>>>(map, x, y, work, make_fastdiv(inner / 4));
   } else {
-    const uint32_t work = static_cast<uint32_t>(rows * inner);
-    rows_pick_kernel<MAP, false><<<stream_grid(work), kStream, 0, st>>>(map, x, y, work, make_fastdiv(inner));
+    const uint32_t units = (static_cast<uint32_t>(inner) + 3) / 4;
+    const uint32_t work = static_cast<uint32_t>(rows * units);
+    rows_pick_any_kernel<MAP><<<stream_grid(work), kStream, 0, st>>>(map, x, y, work, static_cast<uint32_t>(inner),
+                                                                  make_fastdiv(units));
   }
   return launch_status();
 }
@@ -108,28 +130,46 @@ struct PadArgs {
   FastDiv f_out_w, f_out_h;
 };
 
-// Q outputs per lane (4 when out_w % 4 == 0: one 128-bit store per lane).
-template <int Q>
-__global__ __launch_bounds__(kBlock) void pad_kernel(const float* x, float* y, uint32_t work,
+// Four consecutive outputs and one 128-bit store per lane.  ROWQUAD: out_w % 4
+// == 0, so the four share an output row; otherwise the lane steps over row and
+// plane ends (rows of 230 after padding 224 by 3 ran 2.1x slower with one
+// output per lane).  Lane n4 owns the n % 4 trailing outputs.
+template <bool ROWQUAD>
+__global__ __launch_bounds__(kBlock) void pad_kernel(const float* x, float* y, uint32_t n4, uint32_t n,
                                                       PadArgs p, float value) {
   const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-  if (i >= work) return;
+  if (i > n4) return;
+  const uint32_t count = i < n4 ? 4u : n - 4 * n4;
   uint32_t rest, wo, plane, ho;
-  fd_divmod(Q * i, p.f_out_w, rest, wo);
+  fd_divmod(4 * i, p.f_out_w, rest, wo);
   fd_divmod(rest, p.f_out_h, plane, ho);
-  const int hi = static_cast<int>(ho) - p.top, wi = static_cast<int>(wo) - p.left;
-  const bool row_inside = hi >= 0 && hi < p.in_h;
-  const float* row = x + (static_cast<uint64_t>(plane) * p.in_h + (row_inside ? hi : 0)) * p.in_w;
-  float r[Q];
+  float r[4];
+  if (ROWQUAD) {  // one input row serves the four outputs
+    const int hi = static_cast<int>(ho) - p.top, wi = static_cast<int>(wo) - p.left;
+    const bool row_inside = hi >= 0 && hi < p.in_h && count == 4;
+    const float* row = x + (static_cast<uint64_t>(plane) * p.in_h + (row_inside ? hi : 0)) * p.in_w;
 #pragma unroll
-  for (int j = 0; j < Q; ++j) {
-    const bool inside = row_inside && wi + j >= 0 && wi + j < p.in_w;
-    r[j] = inside ? row[wi + j] : value;
+    for (int j = 0; j < 4; ++j) {
+      const bool inside = row_inside && wi + j >= 0 && wi + j < p.in_w;
+      r[j] = inside ? row[wi + j] : value;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int hi = static_cast<int>(ho) - p.top, wi = static_cast<int>(wo) - p.left;
+      const bool inside = hi >= 0 && hi < p.in_h && wi >= 0 && wi < p.in_w && static_cast<uint32_t>(j) < count;
+      r[j] = inside ? x[(static_cast<uint64_t>(plane) * p.in_h + hi) * p.in_w + wi] : value;
+      if (++wo == p.f_out_w.d) {
+        wo = 0;
+        if (++ho == p.f_out_h.d) ho = 0, ++plane;
+      }
+    }
   }
-  if (Q == 4)
-    store4_stream(y + 4ull * i, v4f{r[0], r[Q > 1 ? 1 : 0], r[Q > 2 ? 2 : 0], r[Q > 3 ? 3 : 0]});
-  else
-    y[i] = r[0];
+  if (count == 4) {
+    store4_stream_any(y + 4ull * i, v4f{r[0], r[1], r[2], r[3]});
+  } else {
+    for (uint32_t j = 0; j < count; ++j) y[4ull * i + j] = r[j];
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -640,10 +680,10 @@ int shdw_hip_pad(const int* in_shape, const int* paddings, float value, const fl
             make_fastdiv(out_shape[2])};
   const uint32_t n = static_cast<uint32_t>(out_count);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (out_shape[3] % 4 == 0 && aligned16(y))
-    pad_kernel<4><<<grid_for(n / 4), kBlock, 0, st>>>(x, y, n / 4, p, value);
+  if (out_shape[3] % 4 == 0)
+    pad_kernel<true><<<grid_for(n / 4 + 1), kBlock, 0, st>>>(x, y, n / 4, n, p, value);
   else
-    pad_kernel<1><<<grid_for(n), kBlock, 0, st>>>(x, y, n, p, value);
+    pad_kernel<false><<<grid_for(n / 4 + 1), kBlock, 0, st>>>(x, y, n / 4, n, p, value);
   return launch_status();
 }
 

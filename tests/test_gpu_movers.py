@@ -69,7 +69,9 @@ def test_stack_op(ws, shape, axis, k):
 
 
 @pytest.mark.parametrize("shape,axis,idx", [((5, 8), 0, [4, 0, 0, 2]), ((3, 6, 4), 1, [5, 1]), ((2, 3, 7), -1, [6, 0, 3]),
-                                            ((4, 10, 16), 1, [9, 8, 7, 0, 1, 2, 2])])
+                                            ((4, 10, 16), 1, [9, 8, 7, 0, 1, 2, 2]),
+                                            ((3, 6, 7), 1, [5, 1]), ((2, 9, 7, 7), 1, [8, 8, 0]),  # rows of 7 and 49 floats
+                                            ((5, 3), 0, [4, 1, 1])])
 def test_gather_op(ws, shape, axis, idx):
     x = normal(40, shape)
     want = oracle.gather_op(x, axis, idx)
@@ -94,7 +96,7 @@ def test_gather_index_checks(ws):
 
 @pytest.mark.parametrize("pads", [[1, 2, 3, 4], [0, 0, 0, 1], [-1, 2, 0, -2], [-1, -1, -1, -1], [2, -1, -2, 3],
                                   [0, 0, 0, 0]])
-@pytest.mark.parametrize("shape", [(2, 3, 6, 7), (1, 2, 16, 16)])
+@pytest.mark.parametrize("shape", [(2, 3, 6, 7), (1, 2, 16, 16), (1, 3, 33, 29)])
 def test_pad_op(ws, pads, shape):
     x = normal(50, shape)
     got = run(ws, "Pad", [("x", x)], {"paddings": pads, "value": -2.5})
@@ -144,7 +146,7 @@ def test_resize_bilinear_bands(ws, shape, size, align):
 
 
 @pytest.mark.parametrize("shape,group", [((2, 6, 3, 5), 2), ((2, 6, 3, 5), 3), ((1, 12, 4, 4), 4), ((3, 8, 1, 1), 8),
-                                         ((2, 116, 28, 28), 2), ((2, 6, 3, 5), 1)])
+                                         ((2, 116, 28, 28), 2), ((2, 6, 3, 5), 1), ((2, 116, 7, 7), 2), ((3, 4, 1, 3), 2)])
 def test_shuffle_channel_op(ws, shape, group):
     x = normal(80, shape)
     got = run(ws, "ShuffleChannel", [("x", x)], {"group": group})
