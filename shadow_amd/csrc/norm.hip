@@ -92,11 +92,16 @@ SHDW_DEVICE double wave_sum(double v) {
   return v;
 }
 
-// Sum over the LANES lanes that own a row, result in each of them.
+// Sum over the LANES lanes that own a row, result in each of them.  LANES <= 64:
+// the lanes are neighbours inside one wave; more: whole waves, through `slots`.
 template <int LANES>
 SHDW_DEVICE double row_sum(double v, double* slots) {
+  if (LANES <= kWave) {
+#pragma unroll
+    for (int off = LANES / 2; off >= 1; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+  }
   v = wave_sum(v);
-  if (LANES == kWave) return v;
   __syncthreads();  // slots may still be read from the previous sum
   if ((threadIdx.x & 63) == 0) slots[threadIdx.x >> 6] = v;
   __syncthreads();
@@ -106,34 +111,51 @@ SHDW_DEVICE double row_sum(double v, double* slots) {
   return total;
 }
 
-// The row (inner % 4 == 0, <= REGS * 4 * LANES elements, 16-byte aligned) is
-// held in REGS vectors per lane.  LANES = 64: four rows per 256-lane workgroup,
-// no barriers.  LANES = 256 or 1024: one row per workgroup of that size.
+// The row (<= REGS * 4 * LANES elements) is held in REGS vectors per lane.
+// LANES = 16, 32 or 64: 16, 8 or 4 rows per 256-lane workgroup, no barriers (a
+// wave-per-row layout leaves 3/4 of the lanes idle on rows of 64 floats: 85 us
+// per 58 MB, and rows of 49 went through the one-workgroup-per-row kernel at
+// 307 us).  LANES = 256 or 1024: one row per workgroup of that size.
+// TAIL = false: inner % 4 == 0 and 16-byte aligned pointers.  TAIL = true: any
+// row length on any dword address; a lane's vector may end inside its four
+// positions, whole vectors still move as (unaligned) 128-bit accesses.
 constexpr int kBigBlock = 1024;
 
-template <int REGS, int LANES>
-__global__ __launch_bounds__(LANES == kWave ? kBlock : LANES) void norm_rows_reg_kernel(
+template <int REGS, int LANES, bool TAIL>
+__global__ __launch_bounds__(LANES <= kWave ? kBlock : LANES) void norm_rows_reg_kernel(
     const float* x, float* y, NormArgs p) {
   __shared__ double slots[kBigBlock / kWave];
-  const uint32_t lane = LANES == kWave ? (threadIdx.x & 63u) : threadIdx.x;
-  const uint32_t row = LANES == kWave ? blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6) : blockIdx.x;
-  if (LANES == kWave && row >= p.outer) return;  // whole waves leave; no barrier in this form
+  const uint32_t lane = LANES <= kWave ? (threadIdx.x & (LANES - 1)) : threadIdx.x;
+  const uint32_t row = LANES <= kWave ? blockIdx.x * (kBlock / LANES) + threadIdx.x / LANES : blockIdx.x;
+  if (LANES <= kWave && row >= p.outer) return;  // whole rows of lanes leave; no barrier in this form
   const uint64_t base = static_cast<uint64_t>(row) * p.inner;
   const float* xr = x + base;
   float* yr = y + base;
-  const uint32_t nvec = p.inner / 4;
+  // elements of vector k that exist: 4, or fewer at the end of a TAIL row
+  auto count = [&](int k) -> uint32_t {
+    const uint32_t first = 4 * (k * LANES + lane);
+    return first >= p.inner ? 0u : min(4u, p.inner - first);
+  };
   v4f reg[REGS];
 #pragma unroll
   for (int k = 0; k < REGS; ++k) {
-    const uint32_t v = k * LANES + lane;
-    if (v < nvec) reg[k] = load4_stream(xr + 4ull * v);
+    const uint32_t first = 4 * (k * LANES + lane), c = count(k);
+    if (c == 4) {
+      reg[k] = TAIL ? load4_stream_any(xr + first) : load4_stream(xr + first);
+    } else if (TAIL && c > 0) {
+      reg[k] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 3; ++j)
+        if (j < c) reg[k][j] = xr[first + j];
+    }
   }
   double acc = 0;
 #pragma unroll
   for (int k = 0; k < REGS; ++k) {
-    if (k * LANES + lane < nvec) {
+    const uint32_t c = count(k);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < 4; ++j) {
+      if (j < c) {
         const float t = p.alpha * reg[k][j];
         acc += static_cast<double>(t);
       }
@@ -143,9 +165,10 @@ __global__ __launch_bounds__(LANES == kWave ? kBlock : LANES) void norm_rows_reg
   acc = 0;
 #pragma unroll
   for (int k = 0; k < REGS; ++k) {
-    if (k * LANES + lane < nvec) {
+    const uint32_t c = count(k);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < 4; ++j) {
+      if (j < c) {
         const float val = reg[k][j] - mean;
         reg[k][j] = val;
         const float sq = val * val;
@@ -159,12 +182,24 @@ __global__ __launch_bounds__(LANES == kWave ? kBlock : LANES) void norm_rows_reg
   const float denom = __builtin_sqrtf(ve);
 #pragma unroll
   for (int k = 0; k < REGS; ++k) {
-    const uint32_t v = k * LANES + lane;
-    if (v < nvec) {
-      v4f r;
+    const uint32_t first = 4 * (k * LANES + lane), c = count(k);
+    if (c == 0) continue;
+    v4f r;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) r[j] = reg[k][j] / denom;
-      store4_stream(yr + 4ull * v, norm_affine4(p, static_cast<uint32_t>(base) + 4 * v, 4 * v, r));
+    for (int j = 0; j < 4; ++j) r[j] = reg[k][j] / denom;
+    if (!TAIL) {
+      store4_stream(yr + first, norm_affine4(p, static_cast<uint32_t>(base) + first, first, r));
+    } else {
+      // any alignment: the affine parameters are looked up per element
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = norm_affine1(p, static_cast<uint32_t>(base) + first + j, r[j]);
+      if (c == 4) {
+        store4_stream_any(yr + first, r);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+          if (j < c) yr[first + j] = r[j];
+      }
     }
   }
 }
@@ -389,27 +424,50 @@ int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint32_t rows = p.outer;
   const uint32_t nvec = p.inner / 4;
-  const uint32_t wave_grid = (rows + kBlock / kWave - 1) / (kBlock / kWave);
+  // workgroups of 256 lanes holding 256 / lanes rows each
+  auto groups = [rows](uint32_t lanes) { return (rows + kBlock / lanes - 1) / (kBlock / lanes); };
   if (!vec) {
-    norm_rows_stream_kernel<false><<<rows, kBlock, 0, st>>>(x, y, p);
+    // any row length, any dword address: whole vectors plus a partial one per row
+    const uint32_t units = (p.inner + 3) / 4;
+    if (units <= 16) {
+      norm_rows_reg_kernel<1, 16, true><<<groups(16), kBlock, 0, st>>>(x, y, p);
+    } else if (units <= 32) {
+      norm_rows_reg_kernel<1, 32, true><<<groups(32), kBlock, 0, st>>>(x, y, p);
+    } else if (units <= 1 * kWave) {
+      norm_rows_reg_kernel<1, kWave, true><<<groups(kWave), kBlock, 0, st>>>(x, y, p);
+    } else if (units <= 2 * kWave) {
+      norm_rows_reg_kernel<2, kWave, true><<<groups(kWave), kBlock, 0, st>>>(x, y, p);
+    } else if (units <= 4 * kWave) {
+      norm_rows_reg_kernel<4, kWave, true><<<groups(kWave), kBlock, 0, st>>>(x, y, p);
+    } else if (units <= 8 * kWave) {
+      norm_rows_reg_kernel<8, kWave, true><<<groups(kWave), kBlock, 0, st>>>(x, y, p);
+    } else if (units <= 8 * kBlock) {
+      norm_rows_reg_kernel<8, kBlock, true><<<rows, kBlock, 0, st>>>(x, y, p);
+    } else {
+      norm_rows_stream_kernel<false><<<rows, kBlock, 0, st>>>(x, y, p);
+    }
+  } else if (nvec <= 16) {
+    norm_rows_reg_kernel<1, 16, false><<<groups(16), kBlock, 0, st>>>(x, y, p);
+  } else if (nvec <= 32) {
+    norm_rows_reg_kernel<1, 32, false><<<groups(32), kBlock, 0, st>>>(x, y, p);
   } else if (nvec <= 1 * kWave) {
-    norm_rows_reg_kernel<1, kWave><<<wave_grid, kBlock, 0, st>>>(x, y, p);
+    norm_rows_reg_kernel<1, kWave, false><<<groups(kWave), kBlock, 0, st>>>(x, y, p);
   } else if (nvec <= 2 * kWave) {
-    norm_rows_reg_kernel<2, kWave><<<wave_grid, kBlock, 0, st>>>(x, y, p);
+    norm_rows_reg_kernel<2, kWave, false><<<groups(kWave), kBlock, 0, st>>>(x, y, p);
   } else if (nvec <= 4 * kWave) {
-    norm_rows_reg_kernel<4, kWave><<<wave_grid, kBlock, 0, st>>>(x, y, p);
+    norm_rows_reg_kernel<4, kWave, false><<<groups(kWave), kBlock, 0, st>>>(x, y, p);
   } else if (nvec <= 8 * kWave && rows >= 2048) {
-    norm_rows_reg_kernel<8, kWave><<<wave_grid, kBlock, 0, st>>>(x, y, p);
+    norm_rows_reg_kernel<8, kWave, false><<<groups(kWave), kBlock, 0, st>>>(x, y, p);
   } else if (nvec <= 2 * kBlock) {
-    norm_rows_reg_kernel<2, kBlock><<<rows, kBlock, 0, st>>>(x, y, p);
+    norm_rows_reg_kernel<2, kBlock, false><<<rows, kBlock, 0, st>>>(x, y, p);
   } else if (nvec <= 4 * kBlock) {
-    norm_rows_reg_kernel<4, kBlock><<<rows, kBlock, 0, st>>>(x, y, p);
+    norm_rows_reg_kernel<4, kBlock, false><<<rows, kBlock, 0, st>>>(x, y, p);
   } else if (nvec <= 8 * kBlock) {
-    norm_rows_reg_kernel<8, kBlock><<<rows, kBlock, 0, st>>>(x, y, p);
+    norm_rows_reg_kernel<8, kBlock, false><<<rows, kBlock, 0, st>>>(x, y, p);
   } else if (nvec <= 4 * kBigBlock) {
-    norm_rows_reg_kernel<4, kBigBlock><<<rows, kBigBlock, 0, st>>>(x, y, p);
+    norm_rows_reg_kernel<4, kBigBlock, false><<<rows, kBigBlock, 0, st>>>(x, y, p);
   } else if (nvec <= 8 * kBigBlock) {
-    norm_rows_reg_kernel<8, kBigBlock><<<rows, kBigBlock, 0, st>>>(x, y, p);
+    norm_rows_reg_kernel<8, kBigBlock, false><<<rows, kBigBlock, 0, st>>>(x, y, p);
   } else {
     norm_rows_stream_kernel<true><<<rows, kBlock, 0, st>>>(x, y, p);
   }
