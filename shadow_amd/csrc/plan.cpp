@@ -171,7 +171,10 @@ int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* ax
     // so that one launch gives >= 256 workgroups (one per CU) and >= 2048 waves;
     // only when no shape does, split the reduced axis over grid.z and add a
     // second stage.
-    const int vec_max = (plan->inner % 4 == 0) ? 4 : 1;
+    // A tile of 128-bit loads spans 256 columns; fewer than 128 columns leave
+    // most of its lanes idle (56 columns: 14 of 64), and one column per lane
+    // does better (reduce 2048 over [128, 2048, 56]: 26.5 us -> 18 us).
+    const int vec_max = (plan->inner % 4 == 0 && plan->inner >= 128) ? 4 : 1;
     const int cand[4][2] = {{4, 4}, {4, 16}, {1, 4}, {1, 16}};
     bool single = false;
     for (const auto& c : cand) {

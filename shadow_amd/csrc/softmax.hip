@@ -571,16 +571,16 @@ static void launch_normalize_tile_ts(int outer_num, int dim, int inner_num, floa
 template <int PMODE, int SM>
 static void launch_normalize_tile(int outer_num, int dim, int inner_num, float p, float eps, const float* x,
                                   const float* scale, float* y, hipStream_t st) {
-  // The tile width that keeps a tile within 32 KB (four and more workgroups per
-  // CU): [64,256,56,56] 92 us with 64-position tiles (64 KB), 87 us with 32;
-  // [64,512,38,38] 131 us with 32 (64 KB), 123 us with 16.  Softmax, with its
-  // five barriers per tile, is the other way round and takes the widest tile.
+  // 64 positions per tile row while the tile stays within 32 KB (four and more
+  // workgroups per CU), else 32, up to 64 KB: rows of 16 positions (64 bytes)
+  // cost more than the lower occupancy does.  [64,256,56,56]: 85 us with 64
+  // positions (64 KB), 80 us with 32; [64,512,38,38]: 105 us with 32 (64 KB),
+  // 115 us with 16.  Softmax, with its five barriers per tile, takes the widest
+  // tile that fits.
   if (dim * 64 * sizeof(float) <= kTileLdsBytes / 2)
     launch_normalize_tile_ts<PMODE, SM, 6>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
-  else if (dim * 32 * sizeof(float) <= kTileLdsBytes / 2)
-    launch_normalize_tile_ts<PMODE, SM, 5>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
   else
-    launch_normalize_tile_ts<PMODE, SM, 4>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
+    launch_normalize_tile_ts<PMODE, SM, 5>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
 }
 
 // Softmax on the same tile layout (65 <= dim <= 511 so that the exp table fits
@@ -699,7 +699,7 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
   else if (dim <= 32)
     softmax_columns_reg_kernel<32><<<grid_for(g.columns), kBlock, 0, st>>>(
         x, y, g.columns, static_cast<uint32_t>(dim), fi);
-  else if (dim <= 64)
+  else if (dim <= 64)  // the tile kernel is slower here: [64,49,128,128] 115 us against 88
     softmax_columns_reg_kernel<64><<<grid_for(g.columns), kBlock, 0, st>>>(
         x, y, g.columns, static_cast<uint32_t>(dim), fi);
   else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner && dim * 64 * sizeof(float) + 256 <= kTileLdsBytes)

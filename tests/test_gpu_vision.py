@@ -109,6 +109,18 @@ def test_softmax_special_values(gpu, outer, dim, inner):
     assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax specials")
 
 
+# Spreads wide enough for exp to reach tiny, denormal and zero results, next to
+# ordinary columns, in each kernel layout.
+@pytest.mark.parametrize("outer,dim,inner", [(3, 40, 1), (2, 12, 200), (2, 48, 130), (2, 150, 300), (1, 100, 70),
+                                             (1, 1000, 70), (2, 300, 50), (2, 21, 63)])
+def test_softmax_with_underflowing_exponentials(gpu, outer, dim, inner):
+    x = normal(19, (outer, dim, inner), 3.0)
+    x[:, :, ::3] *= F(12.0)      # gaps up to ~100: exp down to 1e-44 and 0
+    x[:, 1::2, 1::5] -= F(95.0)  # every other class far below the rest
+    x = x.reshape(-1)
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax tails")
+
+
 @pytest.mark.parametrize("shape,axis", [((8, 1000), 1), ((2, 21, 33, 35), 1), ((3, 4, 5), -1), ((6, 2, 3), 0)])
 def test_softmax_op(ws, shape, axis):
     x = normal(15, shape, 3.0)
@@ -128,7 +140,7 @@ def test_softmax_op_defaults_and_errors(ws):
 @pytest.mark.parametrize("p", [1.0, 2.0, 3.0, 0.5])
 @pytest.mark.parametrize("outer,dim,inner", [(64, 512, 1), (5, 7, 3), (2, 16, 100), (3, 9, 64), (1, 20000, 1),
                                              (2, 1, 9), (1, 33, 4097),
-                                             # 65..1024 deep over a wide inner extent: tiles of 64, 32, 16 positions
+                                             # 65..1024 deep over a wide inner extent: tiles of 64 and 32 positions
                                              (2, 100, 100), (1, 512, 72), (3, 300, 37), (2, 1024, 20), (1, 65, 4097),
                                              (2, 256, 64), (1, 1025, 40)])
 def test_normalize(gpu, p, outer, dim, inner):
@@ -310,6 +322,38 @@ def test_entry_point_argument_errors(gpu):
 # combined through LDS) than in the oracle's serial loop.  Contract: 1e-5
 # relative on every output; the tests also count differing bits, and every case
 # here comes out identical.
+@pytest.mark.parametrize("p", [1.0, 2.0])
+@pytest.mark.parametrize("outer,dim,inner", [(2, 16, 100), (2, 100, 100), (1, 300, 37), (4, 30, 1), (1, 1000, 70)])
+def test_normalize_extreme_magnitudes(gpu, p, outer, dim, inner):
+    """Columns of tiny (1e-33, with denormal members), huge (1e30) and mixed
+    magnitude, signed zeros, beside ordinary ones."""
+    x = normal(20, (outer, dim, inner), 1.0)
+    x[:, :, 0::7] *= F(1e-33)
+    x[:, :, 1::7] *= F(1e30)
+    x[:, ::3, 2::7] *= F(1e-36)
+    x[:, 1::4, 3::7] = 0
+    x[:, 0, 3::7] = -0.0
+    x = x.reshape(-1)
+    for eps in (1e-12, 0.0):
+        assert_bit_exact(gpuops.normalize(x, outer, dim, inner, p, eps), oracle.normalize(x, outer, dim, inner, p, eps),
+                         "normalize ranges eps=%g" % eps)
+    got = gpuops.ssd_normalize(x, outer, dim, inner, False, True, 1e-10)
+    assert_bit_exact(got, oracle.ssd_normalize(x, outer, dim, inner, False, True, 1e-10), "ssd ranges")
+
+
+@pytest.mark.parametrize("outer,inner", [(16, 49), (9, 256), (5, 3136), (4, 25088), (4, 70000)])
+def test_group_norm_rows_extreme_magnitudes(gpu, outer, inner):
+    x = normal(41, (outer, inner), 1.0)
+    x[0] *= F(1e-33)
+    x[1] *= F(1e28)
+    x[2, ::2] = x[2, 0]          # half of the row equal: zero or rounding-size deviations
+    x[3, 5:] = F(1.5)            # one outlier, the rest a hair from the mean
+    x = x.reshape(-1)
+    for eps in (1e-5, 0.0):
+        want = oracle.normalize_rows(x, outer, inner, eps)
+        assert assert_rel_close(gpuops.group_norm(x, outer, inner, eps), want, 1e-5, "norm rows ranges") == 0
+
+
 NORM_ROWS = [(6, 49), (4, 784), (8, 1024), (3, 2048), (5, 3136), (2, 4096), (2, 4100), (2, 25088), (7, 5),
              (300, 12), (1, 1), (3, 1000), (2, 8192), (2, 6002), (7, 400), (2100, 1200), (2051, 2048), (9, 256), (3, 16384), (2, 32768), (2, 32772), (1, 70000)]
 
