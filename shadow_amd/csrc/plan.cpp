@@ -7,6 +7,10 @@
 
 namespace shdw {
 
+// kStrided with kFlatMinInner <= inner < kFlatMaxInner goes through the flat
+// kernel (4 * inner <= 1024 must hold for odd inner: 127 * 4 = 508).
+constexpr int64_t kFlatMinInner = 8, kFlatMaxInner = 128;
+
 int plan_broadcast(int num_axes, const int* a_shape, const int* b_shape,
                    const int* out_shape, BroadcastPlan* plan) {
   if (num_axes < 0 || (num_axes > 0 && (!a_shape || !b_shape || !out_shape)) || !plan)
@@ -166,6 +170,17 @@ int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* ax
       const int by_work = ceil_div64(plan->reduce, 4096);  // >= 4 vectors per lane
       plan->splits = std::max(1, std::min(by_fill, by_work));
     }
+  } else if (plan->inner < kFlatMaxInner && plan->inner >= kFlatMinInner) {
+    // Few columns: a column tile would leave most lanes idle (56 columns use 14
+    // of a wave's 64 lanes with 128-bit loads).  The [reduce][inner] slab of one
+    // outer index is contiguous, so the 256 lanes of a workgroup walk it flat,
+    // four consecutive elements per lane, in steps of `flat_period` elements: a
+    // multiple of inner, so each lane keeps meeting the same four columns.
+    const int64_t unit = (plan->inner % 4 == 0) ? plan->inner : (plan->inner % 2 == 0 ? 2 : 4) * plan->inner;
+    plan->flat_period = static_cast<int>(1024 / unit * unit);
+    const int by_fill = ceil_div64(1024, plan->outer);
+    const int by_work = ceil_div64(plan->reduce * plan->inner, 8 * 1024);  // >= 8 steps per workgroup
+    plan->splits = std::max(1, std::min(std::min(by_fill, by_work), 1024));
   } else {
     // Pick columns per lane (128-bit or scalar loads) and waves per column tile
     // so that one launch gives >= 256 workgroups (one per CU) and >= 2048 waves;

@@ -49,6 +49,8 @@ struct ReducePlan {
   bool wave_per_row = false;  // kRows: 16/32/64 lanes per row instead of a workgroup
   int strided_waves = 4;      // kStrided: wave64 per workgroup sharing a column tile (4 or 16)
   int strided_vec = 4;        // kStrided: columns per lane (4 = 128-bit loads, 1 = scalar)
+  int flat_period = 0;        // kStrided with fewer than 128 columns: > 0 selects the flat kernel; elements
+                              // the 256 lanes cover per step (a multiple of inner and of 4, <= 1024)
   int64_t outputs = 1;        // number of output elements
   int64_t window = 1;         // elements per output (Shadow's num_list)
   // kGeneric only: kept dims (outermost first) and reduced dims in LIST order,

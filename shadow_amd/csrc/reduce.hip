@@ -250,6 +250,77 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const float* 
 }
 
 // ---------------------------------------------------------------------------
+// strided with few columns (8 <= inner < 128): the slab [reduce][inner] of one
+// outer index is contiguous, and a workgroup walks its share of it flat.  Lane
+// t takes elements 4t .. 4t+3 of every step of `period` elements; period is a
+// multiple of inner (and of 4), so the lane meets the same four columns at every
+// step and keeps one accumulator for each, and its rows advance by period /
+// inner per step.  The loads are 128-bit on whatever dword address the slab has.
+// At the end the accumulators go to LDS by position inside the period and lane
+// c < inner combines positions c, c + inner, c + 2 inner, ...
+// ---------------------------------------------------------------------------
+template <int OP>
+__global__ __launch_bounds__(kBlock) void reduce_strided_flat_kernel(
+    const float* x, float* y, Partial* part, uint32_t reduce, uint32_t inner, uint32_t rows_per_split,
+    uint32_t splits, uint32_t outputs, uint32_t period, FastDiv f_inner) {
+  __shared__ Partial lds[4 * kBlock];
+  const uint32_t o = blockIdx.x, split = blockIdx.y;
+  const uint32_t r_begin = min(split * rows_per_split, reduce);
+  const uint32_t r_end = min(r_begin + rows_per_split, reduce);
+  const uint32_t t4 = 4 * threadIdx.x;
+  const bool active = t4 < period;  // period % 4 == 0: a lane has four positions or none
+  const uint32_t rows_per_step = period / inner;
+
+  Acc<OP> acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc[j].init();
+
+  if (active) {
+    uint32_t drow[4];  // row of position t4 + j inside a step
+#pragma unroll
+    for (int j = 0; j < 4; ++j) drow[j] = fd_div(t4 + j, f_inner);
+    const float* slab = x + static_cast<size_t>(o) * reduce * inner;
+    const uint32_t end = r_end * inner;  // < 2^31: the tensor has at most INT32_MAX elements
+    uint32_t f = r_begin * inner + t4, row = r_begin;
+    for (; f + 3 * period + 3 < end; f += 4 * period, row += 4 * rows_per_step) {
+      v4f v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = load4_stream_any(slab + f + u * period);
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j].add(v[u][j], row + u * rows_per_step + drow[j]);
+    }
+    for (; f < end; f += period, row += rows_per_step) {
+      if (f + 3 < end) {
+        const v4f v = load4_stream_any(slab + f);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j].add(v[j], row + drow[j]);
+      } else {  // the share ends inside this lane's four elements
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+          if (f + j < end) acc[j].add(slab[f + j], row + drow[j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) lds[t4 + j] = acc[j].pack();
+  }
+  __syncthreads();
+  if (threadIdx.x < inner) {  // inner < 128
+    Acc<OP> total;
+    total.init();
+    for (uint32_t s = threadIdx.x; s < period; s += inner) {
+      Acc<OP> t;
+      t.unpack(lds[s]);
+      total.merge(t);
+    }
+    const size_t out = static_cast<size_t>(o) * inner + threadIdx.x;
+    if (splits == 1) y[out] = total.finalize(reduce);
+    else part[static_cast<size_t>(split) * outputs + out] = total.pack();
+  }
+}
+
+// ---------------------------------------------------------------------------
 // strided: x[outer][reduce][inner] -> y[outer][inner]
 // ---------------------------------------------------------------------------
 // WAVES wave64 per workgroup (4 or 16) share one tile of 64*VEC columns and
@@ -499,6 +570,15 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
   const uint32_t inner = static_cast<uint32_t>(pl.inner);
   const uint32_t splits = static_cast<uint32_t>(pl.splits);
   const uint32_t rows_per_split = (reduce + splits - 1) / splits;
+  if (pl.flat_period > 0) {
+    // grid.x carries outer (at most INT32_MAX, as the element count), grid.y the slices (<= 1024)
+    reduce_strided_flat_kernel<OP><<<dim3(outer, splits), kBlock, 0, st>>>(
+        x, y, part, reduce, inner, rows_per_split, splits, outputs, static_cast<uint32_t>(pl.flat_period),
+        make_fastdiv(inner));
+    int rc = launch_status();
+    if (rc != SHDW_OK || splits == 1) return rc;
+    return run_stage2<OP>(part, y, outputs, splits, 1, outputs, window, st);
+  }
   const bool vec = pl.strided_vec == 4 && inner % 4 == 0 && aligned16(x);
   const int v = vec ? 4 : 1;
   const uint32_t tiles = (inner + kWave * v - 1) / (kWave * v);

@@ -283,6 +283,14 @@ REDUCE_CASES = [
     ([300, 6, 7, 7], [2, 3]),
     ([3, 40001], [1]),           # long rows that start on odd dwords
     ([500, 3], [1]),             # rows shorter than one vector
+    # strided with 8..127 columns: the flat walk over [reduce][inner]
+    ([5, 333, 49], [1]),         # odd columns: steps of 980 elements
+    ([2, 4097, 127], [1]),       # steps of 508, second stage
+    ([4, 1000, 126], [1]),       # steps of 1008
+    ([3, 7, 100], [1]),          # less than one step
+    ([2, 512, 7, 8], [1]),       # channels over a 7x8 map
+    ([130, 64, 7, 7], [1]),
+    ([3, 2, 9], [1]),
 ]
 
 
@@ -315,7 +323,7 @@ def test_reduce_beyond_the_second_grid_dimension(gpu, shape, axes, op):
 
 
 @pytest.mark.parametrize("shape,axes", [([64, 48], [1]), ([3, 64, 8], [1]), ([2, 3, 4, 5], [3, 1]),
-                                        ([50000], [0]), ([300, 16], [1])])
+                                        ([50000], [0]), ([300, 16], [1]), ([3, 500, 49], [1]), ([2, 6000, 12], [1])])
 @pytest.mark.parametrize("op", [2, 3])
 def test_reduce_select_special_values(gpu, shape, axes, op):
     """Zeros of both signs, NaNs and infinities: the first extremum in list
