@@ -52,6 +52,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-configs", action="store_true", help="skip the per-config table")
     ap.add_argument("--cpu-passes", type=int, default=10)
+    ap.add_argument("--operand-sets", type=int, default=1,
+                    help="multiplier on the number of rotating operand sets of the config table")
     ap.add_argument("--probe", action="store_true",
                     help="counter probe: 3 launches of a plain copy and of every headline op on "
                          "the 51.4M tensor, nothing timed, no JSON (run under rocprofv3 --pmc)")
@@ -289,7 +291,7 @@ def time_batch(dev, launch, sets, reps=40, warm=5):
     return dev.elapsed_ms(e0, e1) / reps
 
 
-def config_table(dev):
+def config_table(dev, sets_scale=1):
     lib, st = dev.lib, dev.stream
     I = dev.sa.ints
     rows = []
@@ -300,17 +302,20 @@ def config_table(dev):
                      "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "Gelem_s": round(elems / (ms * 1e-3) / 1e9, 2)})
 
-    SETS = 6  # 6 x (in + out) of 51 MB each: more than the 256 MB Infinity Cache
+    SETS = 6 * sets_scale  # 6 x (in + out) of 51 MB each: more than the 256 MB Infinity Cache
     NBIG = 12845056  # elements of the cfg-3 and cfg-5 tensors (51.4 MB)
     A = [dev.buf(normal(301 + 10 * k, NBIG)) for k in range(SETS)]
     Y = [dev.buf(nbytes=4 * NBIG) for _ in range(SETS)]
 
-    # cfg 1: Binary add with channel broadcast (uses the first 6.4M elements of each set)
+    # cfg 1: Binary add with channel broadcast.  Its tensor is half of a set (25.7 MB):
+    # both halves of every set take turns, 12 x 25.7 MB of inputs, so that no launch
+    # finds its input still in the 256 MB Infinity Cache (with six inputs, 154 MB,
+    # it did, and measured 8.7 us instead of 10.7).
     sa, sb = [8, 64, 112, 112], [1, 64, 1, 1]
     n = int(np.prod(sa))
     B = dev.buf(uniform(102, 64, -1, 1))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_broadcast_binary(0, 4, I(sa), I(sb), I(sa), A[k].ptr,
-                                                                 B.ptr, Y[k].ptr, st), SETS)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_broadcast_binary(
+        0, 4, I(sa), I(sb), I(sa), A[k % SETS].ptr + (k // SETS) * 4 * n, B.ptr, Y[k % SETS].ptr, st), 2 * SETS)
     add(1, "binary_add_channel_broadcast", 8 * n + 256, ms, n)
 
     # cfg 3: reductions over [32,512,28,28]
@@ -382,7 +387,7 @@ def config_table(dev):
             bb.free()
 
     # "next" operators at the size of the headline tensor (205 MB in, 3 rotating sets)
-    NH, SH = 51380224, 3
+    NH, SH = 51380224, 3 * sets_scale
     AH = [dev.buf(normal(701 + k, NH)) for k in range(SH)]
     YH = [dev.buf(nbytes=4 * NH) for _ in range(SH)]
     CH, INH = 256, 3136
@@ -464,9 +469,17 @@ def config_table(dev):
     add("movers", "pad 1 [64,64,110,110] -> 112x112", 4 * (npi + NH), ms, NH)
     rin, rout = [64, 64, 56, 56], [64, 64, 112, 112]
     nri = int(np.prod(rin))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_resize(I(rin), I(rout), 1, 0, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
+    # The resize input is a quarter of a set (51 MB): all four quarters of every set
+    # take turns (12 inputs, 617 MB).  With three inputs the gathers found them in the
+    # Infinity Cache and the kernels looked faster than they are from HBM (nearest:
+    # 38 us against 64).
+    def resize_in(k):
+        return AH[k % SH].ptr + (k // SH) * 4 * nri
+    ms = time_batch(dev, lambda k: lib.shdw_hip_resize(I(rin), I(rout), 1, 0, resize_in(k), YH[k % SH].ptr, st),
+                    4 * SH, reps=24)
     add("movers", "resize bilinear x2 [64,64,56,56]", 4 * (nri + NH), ms, NH)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_resize(I(rin), I(rout), 0, 0, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_resize(I(rin), I(rout), 0, 0, resize_in(k), YH[k % SH].ptr, st),
+                    4 * SH, reps=24)
     add("movers", "resize nearest x2 [64,64,56,56]", 4 * (nri + NH), ms, NH)
     ms = time_batch(dev, lambda k: lib.shdw_hip_reorg(I(rout), 1, 2, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
     add("movers", "reorg natural s2 [64,64,112,112]", 8 * NH, ms, NH)
@@ -558,7 +571,7 @@ def main():
                          "launch; roofline.avg_us from events around the dominant kernel inside the timed region",
     }
     if not args.no_configs:
-        out["configs"] = config_table(dev)
+        out["configs"] = config_table(dev, args.operand_sets)
         out["network"] = network_forward(dev)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(host, step_bytes, args.cpu_passes)

@@ -136,13 +136,37 @@ def test_reorg_op(ws, type_, shape, stride):
     ((1, 1, 300, 5), [2, 10]),       # two output rows 150 input rows apart
     ((1, 1, 4, 6000), [8, 9000]),    # rows too wide for the staged kernel: gather kernel
     ((2, 2, 9, 2100), [5, 4100]),    # one-row bands with a large tile
-    ((1, 3, 200, 31), [333, 77])])   # odd output width: one output per lane
+    ((1, 3, 200, 31), [333, 77]),    # odd output width: a lane's four outputs span two rows
+    ((2, 3, 75, 75), [150, 150]),    # x2 of odd maps: bands start on any dword
+    ((2, 2, 13, 13), [26, 26]),
+    ((2, 3, 19, 19), [38, 38]),
+    ((1, 5, 7, 3), [9, 2]),          # rows shorter than a lane's four outputs
+    ((1, 4, 10, 10), [23, 2]),
+    ((64, 64, 13, 13), [26, 26]),    # small maps, many planes: two whole planes per workgroup
+    ((96, 128, 5, 3), [10, 6]),      # five planes per workgroup, three in the last
+    ((65, 64, 7, 5), [10, 9])])      # odd rows across the planes of a group
 def test_resize_bilinear_bands(ws, shape, size, align):
     x = normal(91, shape, 2.0)
     got = run(ws, "Resize", [("x", x)], {"size": size, "align_corners": align})
     want = oracle.resize_op(x, size, [1.0], 1, align)
     assert got.shape == want.shape
     assert_bit_exact(got, want, "resize %s -> %s" % (shape, size))
+
+
+@pytest.mark.parametrize("shape,size", [((3, 5, 56, 56), [112, 112]), ((2, 3, 75, 75), [150, 150]),
+                                        ((2, 2, 13, 13), [26, 26]), ((2, 3, 19, 19), [38, 38]), ((1, 5, 7, 3), [9, 2]),
+                                        ((1, 4, 10, 10), [23, 1]), ((3, 2, 33, 21), [50, 47]), ((1, 1, 50, 47), [33, 21]),
+                                        ((1, 1, 1, 1), [3, 3]), ((64, 64, 13, 13), [26, 26]),
+                                        ((96, 128, 5, 3), [10, 6]), ((65, 64, 7, 5), [10, 9]),
+                                        ((1, 1, 4, 6000), [8, 9000])])  # rows too wide to stage: gathers
+def test_resize_nearest_any_width(ws, shape, size):
+    """Output rows of any length: four consecutive outputs per lane, across row
+    ends where the width is not a multiple of four."""
+    x = normal(92, shape, 2.0)
+    got = run(ws, "Resize", [("x", x)], {"size": size, "type": 0})
+    want = oracle.resize_op(x, size, [1.0], 0, False)
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "nearest %s -> %s" % (shape, size))
 
 
 @pytest.mark.parametrize("shape,group", [((2, 6, 3, 5), 2), ((2, 6, 3, 5), 3), ((1, 12, 4, 4), 4), ((3, 8, 1, 1), 8),
