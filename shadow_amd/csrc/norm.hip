@@ -122,7 +122,10 @@ SHDW_DEVICE double row_sum(double v, double* slots) {
 constexpr int kBigBlock = 1024;
 
 template <int REGS, int LANES, bool TAIL>
-__global__ __launch_bounds__(LANES <= kWave ? kBlock : LANES) void norm_rows_reg_kernel(
+// Two 1024-lane workgroups per CU are 8 waves per SIMD, at most 64 registers
+// per lane (the second launch bound asks for that; unasked the compiler took
+// 67 and left room for one workgroup).
+__global__ __launch_bounds__(LANES <= kWave ? kBlock : LANES, LANES == kBigBlock ? 8 : 1) void norm_rows_reg_kernel(
     const float* x, float* y, NormArgs p) {
   __shared__ double slots[kBigBlock / kWave];
   const uint32_t lane = LANES <= kWave ? (threadIdx.x & (LANES - 1)) : threadIdx.x;
