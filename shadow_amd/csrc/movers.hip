@@ -638,20 +638,13 @@ __global__ __launch_bounds__(kBlock) void resize_band_kernel(const float* x, flo
     const char* row_l = tile_b + (row0 + static_cast<uint32_t>(h_l)) * row_bytes;
     const char* row_h = tile_b + (row0 + static_cast<uint32_t>(h_h)) * row_bytes;
     const float ih = 1 - sh;
-    float sw[Q];
-    uint32_t lo[Q], hi[Q];
-    if (Q == 4) {
-      const v4f s4 = *reinterpret_cast<const v4f*>(frac + 4 * cq);
-      const v4u l4 = *reinterpret_cast<const v4u*>(lo_b + 4 * cq);
-      const v4u h4 = *reinterpret_cast<const v4u*>(hi_b + 4 * cq);
+    // Q == 4 from here on: rows of a multiple of four positions on an aligned y
+    const v4f sw = *reinterpret_cast<const v4f*>(frac + 4 * cq);
+    const v4u lo = *reinterpret_cast<const v4u*>(lo_b + 4 * cq);
+    const v4u hi = *reinterpret_cast<const v4u*>(hi_b + 4 * cq);
+    v4f res;
 #pragma unroll
-      for (int j = 0; j < Q; ++j) sw[j] = s4[j], lo[j] = l4[j], hi[j] = h4[j];
-    } else {
-      sw[0] = frac[cq], lo[0] = lo_b[cq], hi[0] = hi_b[cq];
-    }
-    float res[Q];
-#pragma unroll
-    for (int j = 0; j < Q; ++j) {
+    for (int j = 0; j < 4; ++j) {
       const float v0 = *reinterpret_cast<const float*>(row_l + lo[j]);
       if (MODE == kResizeNearest) {
         res[j] = v0;
@@ -667,11 +660,7 @@ __global__ __launch_bounds__(kBlock) void resize_band_kernel(const float* x, flo
       const float s012 = s01 + t2;
       res[j] = s012 + t3;
     }
-    float* dst = out + static_cast<uint64_t>(r) * p.out_w + Q * cq;
-    if (Q == 4)
-      store4_stream(dst, v4f{res[0], res[Q > 1 ? 1 : 0], res[Q > 2 ? 2 : 0], res[Q > 3 ? 3 : 0]});
-    else
-      dst[0] = res[0];
+    store4_stream(out + static_cast<uint64_t>(r) * p.out_w + 4 * cq, res);
   }
 }
 
