@@ -583,7 +583,7 @@ static void launch_normalize_tile(int outer_num, int dim, int inner_num, float p
     launch_normalize_tile_ts<PMODE, SM, 5>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
 }
 
-// Softmax on the same tile layout (65 <= dim <= 511 so that the exp table fits
+// Softmax on the same tile layout (65 <= dim <= 510 so that the exp table fits
 // beside the tile).  The lanes hold x, later exp(x - max), in registers; the tile
 // in LDS serves wave 0's two serial folds: the running maximum of x, then the
 // fp32 running sum of the exponentials, both in index order.  The maxima and
@@ -640,14 +640,15 @@ __global__ __launch_bounds__(kBlock) void softmax_tile_kernel(const float* x, fl
   }
 }
 
-constexpr int kSoftmaxTileMaxDim = 511;  // 511 x 32 positions + the exp table <= 64 KB
+constexpr size_t kExpTabBytes = 32 * sizeof(uint64_t);
+constexpr int kSoftmaxTileMaxDim = (kTileLdsBytes - kExpTabBytes) / (32 * sizeof(float));  // 32 positions + the exp table <= 64 KB: 510
 
 template <int TS_SHIFT>
 static void launch_softmax_tile_ts(int outer_num, int dim, int inner_num, const float* x, float* y,
                                    hipStream_t st) {
   const uint32_t tiles = (static_cast<uint32_t>(inner_num) + (1u << TS_SHIFT) - 1) >> TS_SHIFT;
   const uint32_t grid = static_cast<uint32_t>(outer_num) * tiles;
-  const size_t bytes = (static_cast<size_t>(dim) << TS_SHIFT) * sizeof(float) + 32 * sizeof(uint64_t);
+  const size_t bytes = (static_cast<size_t>(dim) << TS_SHIFT) * sizeof(float) + kExpTabBytes;
   const uint32_t d = static_cast<uint32_t>(dim), in = static_cast<uint32_t>(inner_num);
   const FastDiv ft = make_fastdiv(tiles);
   switch (tile_rows(inner_num, y)) {
@@ -702,7 +703,7 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
   else if (dim <= 64)  // the tile kernel is slower here: [64,49,128,128] 115 us against 88
     softmax_columns_reg_kernel<64><<<grid_for(g.columns), kBlock, 0, st>>>(
         x, y, g.columns, static_cast<uint32_t>(dim), fi);
-  else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner && dim * 64 * sizeof(float) + 256 <= kTileLdsBytes)
+  else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner && dim * 64 * sizeof(float) + kExpTabBytes <= kTileLdsBytes)
     launch_softmax_tile_ts<6>(outer_num, dim, inner_num, x, y, st);
   else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner)
     launch_softmax_tile_ts<5>(outer_num, dim, inner_num, x, y, st);

@@ -92,6 +92,8 @@ SOFTMAX_SHAPES = [  # outer, dim, inner: both layouts, LDS limits, odd sizes
     (1, 2, 5000), (3, 1, 17),
     # columns too long for registers over a wide inner extent: the three-walk kernel
     (2, 150, 300), (1, 65, 4097), (3, 100, 64), (1, 1000, 70),
+    # around the longest column whose tile fits LDS beside the exp table
+    (1, 509, 40), (1, 510, 40), (1, 511, 20), (1, 512, 33),
 ]
 
 
