@@ -291,6 +291,8 @@ REDUCE_CASES = [
     ([2, 512, 7, 8], [1]),       # channels over a 7x8 map
     ([130, 64, 7, 7], [1]),
     ([3, 2, 9], [1]),
+    # short rows of odd length through LDS, one lane per row
+    ([700, 9], [1]), ([513, 127], [1]), ([260, 5], [1]), ([257, 5, 5], [1, 2]), ([1027, 66], [1]),
 ]
 
 
@@ -323,7 +325,8 @@ def test_reduce_beyond_the_second_grid_dimension(gpu, shape, axes, op):
 
 
 @pytest.mark.parametrize("shape,axes", [([64, 48], [1]), ([3, 64, 8], [1]), ([2, 3, 4, 5], [3, 1]),
-                                        ([50000], [0]), ([300, 16], [1]), ([3, 500, 49], [1]), ([2, 6000, 12], [1])])
+                                        ([50000], [0]), ([300, 16], [1]), ([3, 500, 49], [1]), ([2, 6000, 12], [1]), ([300, 49], [1]),
+                                        ([1000, 9], [1])])
 @pytest.mark.parametrize("op", [2, 3])
 def test_reduce_select_special_values(gpu, shape, axes, op):
     """Zeros of both signs, NaNs and infinities: the first extremum in list
