@@ -38,8 +38,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # raw readings and the factors is profiles/headline_unary_chain_hbm_counters.txt).
 # They cannot be collected from inside this process, so they are recorded here.
 MEASURED_TRAFFIC_BYTES = {
-    "activate_relu": 411.01e6, "activate_sigmoid": 411.06e6, "unary_exp": 411.01e6,
-    "unary_abs": 411.02e6, "unary_sqrt_of_abs": 411.00e6, "activate_tanh": 411.02e6,
+    "activate_relu": 411.04e6, "activate_sigmoid": 411.06e6, "unary_exp": 411.01e6,
+    "unary_abs": 411.04e6, "unary_sqrt_of_abs": 411.00e6, "activate_tanh": 411.02e6,
     "scale_relu_fused": 411.02e6,
 }
 
