@@ -352,6 +352,20 @@ def config_table(dev, sets_scale=1):
     ms = time_batch(dev, lambda k: lib.shdw_hip_reduce(4, 4, I(sh7), 2, I(ax5), A[k].ptr, M7[k].ptr,
                                                        None, 0, st), SETS)
     add("next", "reduce_avg_hw 7x7 planes [128,2048,7,7]", 4 * n5 + 4 * 128 * 2048, ms, n5)
+    # more of the same late-stage tensor, whose rows and planes are not multiples of four floats
+    ws7 = dev.buf(nbytes=1 << 20)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_reduce(2, 4, I(sh7), 1, I([1]), A[k].ptr, M7[k].ptr,
+                                                       ws7.ptr, 1 << 20, st), SETS)
+    add("next", "reduce_max_c 7x7 maps [128,2048,7,7]", 4 * n5 + 4 * 128 * 49, ms, n5)
+    g7, b7 = dev.buf(uniform(507, 2048, 0.5, 1.5)), dev.buf(uniform(508, 2048, -0.1, 0.1))
+    ms = time_batch(dev, lambda k: lib.shdw_hip_group_norm(128 * 2048, 49, 1e-5, A[k].ptr, g7.ptr, b7.ptr,
+                                                           2048, 49, Y[k].ptr, st), SETS)
+    add("next", "instance_norm affine 7x7 planes [128,2048,7,7]", 8 * n5 + 8 * 2048, ms, n5)
+    ms = time_batch(dev, lambda k: lib.shdw_hip_broadcast_binary(
+        0, 4, I(sh7), I([1, 2048, 1, 1]), I(sh7), A[k].ptr, b7.ptr, Y[k].ptr, st), SETS)
+    add("next", "binary_add_channel_broadcast 7x7 maps [128,2048,7,7]", 8 * n5 + 4 * 2048, ms, n5)
+    for bb in M7 + [ws7, g7, b7]:
+        bb.free()
     ms = time_batch(dev, lambda k: lib.shdw_hip_scale_residual_relu_rowmean(
         n5, C5, in5, A[k].ptr, g5.ptr, b5.ptr, A[(k + 1) % SETS].ptr, Y[k].ptr, M[k].ptr, st), SETS)
     add(5, "fused_tail", 12 * n5 + 8 * C5 + 4 * 65536, ms, n5)

@@ -36,6 +36,7 @@ enum AffineMode {
   kAffineRowPos = 1,   // parameter index = position in the row (LayerNorm)
   kAffineVector = 2,   // scale_inner % 4 == 0: one channel per aligned vector
   kAffineElement = 3,  // anything else: channel per element
+  kAffineRow = 4,      // scale_inner % inner == 0: one channel per row (InstanceNorm), looked up once
 };
 
 struct NormArgs {
@@ -77,6 +78,25 @@ SHDW_DEVICE v4f norm_affine4(const NormArgs& p, uint32_t i, uint32_t pos, v4f v)
       r[j] = affine1(v[j], p.scale[c], p.bias[c]);
     }
   }
+  return r;
+}
+
+// Scale and bias of the row that starts at global index `base` (kAffineRow).
+struct RowAffine {
+  float s, b;
+};
+SHDW_DEVICE RowAffine norm_row_affine(const NormArgs& p, uint32_t base) {
+  RowAffine ra = {1.f, 0.f};
+  if (p.affine == kAffineRow) {
+    const uint32_t c = norm_channel(p, base);
+    ra.s = p.scale[c], ra.b = p.bias[c];
+  }
+  return ra;
+}
+SHDW_DEVICE v4f norm_row_affine4(const RowAffine& ra, v4f v) {
+  v4f r;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) r[j] = affine1(v[j], ra.s, ra.b);
   return r;
 }
 
@@ -183,6 +203,13 @@ __global__ __launch_bounds__(LANES <= kWave ? kBlock : LANES, LANES == kBigBlock
   const float variance = static_cast<float>(row_sum<LANES>(acc, slots));
   const float ve = variance + p.eps;
   const float denom = __builtin_sqrtf(ve);
+  // One lookup per row where the row shares its scale and bias; only in the
+  // forms of up to 64 lanes per row (the host asks for it only there): the
+  // 1024-lane form has no register to spare for it.
+  constexpr bool kRowForm = LANES <= kWave;
+  const bool row_affine = kRowForm && p.affine == kAffineRow;
+  RowAffine ra = {1.f, 0.f};
+  if (kRowForm) ra = norm_row_affine(p, static_cast<uint32_t>(base));
 #pragma unroll
   for (int k = 0; k < REGS; ++k) {
     const uint32_t first = 4 * (k * LANES + lane), c = count(k);
@@ -190,12 +217,16 @@ __global__ __launch_bounds__(LANES <= kWave ? kBlock : LANES, LANES == kBigBlock
     v4f r;
 #pragma unroll
     for (int j = 0; j < 4; ++j) r[j] = reg[k][j] / denom;
+    if (row_affine) r = norm_row_affine4(ra, r);
     if (!TAIL) {
-      store4_stream(yr + first, norm_affine4(p, static_cast<uint32_t>(base) + first, first, r));
+      if (!row_affine) r = norm_affine4(p, static_cast<uint32_t>(base) + first, first, r);
+      store4_stream(yr + first, r);
     } else {
-      // any alignment: the affine parameters are looked up per element
+      // any alignment: the affine parameters are looked up per element unless the row shares them
+      if (!row_affine) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) r[j] = norm_affine1(p, static_cast<uint32_t>(base) + first + j, r[j]);
+        for (int j = 0; j < 4; ++j) r[j] = norm_affine1(p, static_cast<uint32_t>(base) + first + j, r[j]);
+      }
       if (c == 4) {
         store4_stream_any(yr + first, r);
       } else {
@@ -252,6 +283,7 @@ __global__ __launch_bounds__(kBlock) void norm_rows_stream_kernel(const float* x
   const float variance = static_cast<float>(row_sum<kBlock>(acc, slots));
   const float ve = variance + p.eps;
   const float denom = __builtin_sqrtf(ve);
+  const RowAffine ra = norm_row_affine(p, static_cast<uint32_t>(base));
   for (uint32_t t = threadIdx.x; t < steps; t += kBlock) {
     if (VEC) {
       const v4f q = load4(xr + 4ull * t);
@@ -261,10 +293,13 @@ __global__ __launch_bounds__(kBlock) void norm_rows_stream_kernel(const float* x
         const float val = q[j] - mean;
         r[j] = val / denom;
       }
-      store4_stream(yr + 4ull * t, norm_affine4(p, static_cast<uint32_t>(base) + 4 * t, 4 * t, r));
+      r = p.affine == kAffineRow ? norm_row_affine4(ra, r)
+                                 : norm_affine4(p, static_cast<uint32_t>(base) + 4 * t, 4 * t, r);
+      store4_stream(yr + 4ull * t, r);
     } else {
       const float val = xr[t] - mean;
-      yr[t] = norm_affine1(p, static_cast<uint32_t>(base) + t, val / denom);
+      const float q = val / denom;
+      yr[t] = p.affine == kAffineRow ? affine1(q, ra.s, ra.b) : norm_affine1(p, static_cast<uint32_t>(base) + t, q);
     }
   }
 }
@@ -417,6 +452,8 @@ int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
   const bool vec = inner_num % 4 == 0 && aligned16(x) && aligned16(y);
   if (!scale)
     p.affine = kAffineNone;
+  else if (scale_inner % inner_num == 0 && inner_num <= 1024)  // rows that up to 64 lanes hold
+    p.affine = kAffineRow;
   else if (vec && scale_inner == 1 && scale_num == inner_num && aligned16(scale) && aligned16(bias))
     p.affine = kAffineRowPos;
   else if (vec && scale_inner % 4 == 0)
