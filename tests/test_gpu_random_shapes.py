@@ -1,0 +1,119 @@
+"""Randomly drawn shapes (fixed seeds) through the kernels whose launch shape
+depends on row length, alignment or extent, against the oracle: the hand-picked
+cases of the other files name the paths, these look for what falls between."""
+import numpy as np
+import pytest
+
+import oracle
+import shadow_amd
+from shadow_amd import Buffer, check, ints
+from tests import gpuops
+from tests.helpers import assert_bit_exact, assert_rel_close
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_reduce_random_shapes(gpu, seed):
+    rng = np.random.default_rng(seed)
+    for _ in range(40):
+        kind = rng.integers(0, 3)
+        if kind == 0:    # strided, few to many columns
+            shape = [int(rng.integers(1, 40)), int(rng.integers(1, 600)), int(rng.integers(2, 140))]
+        elif kind == 1:  # rows, short and long
+            shape = [int(rng.integers(200, 3000)), int(rng.integers(1, 140))]
+        else:            # channels over small maps
+            shape = [int(rng.integers(1, 6)), int(rng.integers(1, 300)), int(rng.integers(1, 12)),
+                     int(rng.integers(1, 12))]
+        op = int(rng.integers(0, 7))
+        x = rng.normal(0, 1, shape).astype(F) if op else rng.uniform(0.9, 1.1, shape).astype(F)
+        if rng.random() < 0.3:
+            x[rng.random(shape) < 0.3] = 0.0
+        if rng.random() < 0.3:
+            x[rng.random(shape) < 0.2] = -0.0
+        want, _ = oracle.reduce(op, x, shape, [1])
+        got, _ = gpuops.reduce(op, x, shape, [1])
+        if op in (2, 3):
+            assert_bit_exact(got, want, "reduce %d over axis 1 of %s" % (op, shape))
+        else:
+            assert_rel_close(got, want, 1e-5, "reduce %d over axis 1 of %s" % (op, shape))
+
+
+@pytest.mark.parametrize("seed", [4, 5])
+def test_norm_rows_random_shapes(gpu, seed):
+    rng = np.random.default_rng(seed)
+    for _ in range(40):
+        outer, inner = int(rng.integers(1, 600)), int(rng.integers(1, 2300))
+        x = (rng.normal(0, 3, outer * inner) + 0.75).astype(F)
+        want = oracle.normalize_rows(x, outer, inner, 1e-5)
+        got = gpuops.group_norm(x, outer, inner, 1e-5, offset=int(rng.integers(0, 4)))
+        assert_rel_close(got, want, 1e-5, "norm rows %d x %d" % (outer, inner))
+
+
+@pytest.mark.parametrize("seed", [6, 7])
+def test_column_ops_random_shapes(gpu, seed):
+    rng = np.random.default_rng(seed)
+    for _ in range(40):
+        outer, dim, inner = int(rng.integers(1, 5)), int(rng.integers(1, 600)), int(rng.integers(1, 200))
+        if rng.random() < 0.3:
+            inner = 1
+        x = rng.normal(0, 4, outer * dim * inner).astype(F)
+        what = "[%d, %d, %d]" % (outer, dim, inner)
+        assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax " + what)
+        p = float(rng.choice([1.0, 2.0]))
+        assert_bit_exact(gpuops.normalize(x, outer, dim, inner, p, 1e-12),
+                         oracle.normalize(x, outer, dim, inner, p, 1e-12), "normalize " + what)
+        assert_bit_exact(gpuops.ssd_normalize(x, outer, dim, inner, False, True, 1e-10),
+                         oracle.ssd_normalize(x, outer, dim, inner, False, True, 1e-10), "ssd normalize " + what)
+
+
+@pytest.mark.parametrize("seed", [8, 9])
+def test_broadcast_random_shapes(gpu, seed):
+    rng = np.random.default_rng(seed)
+    for _ in range(60):
+        nd = int(rng.integers(1, 5))
+        out = [int(rng.integers(1, 20)) for _ in range(nd)]
+        a = [d if rng.random() < 0.7 else 1 for d in out]
+        b = [d if rng.random() < 0.5 else 1 for d in out]
+        out = [max(p, q) for p, q in zip(a, b)]
+        op = int(rng.choice([0, 1, 2, 3, 5, 6]))
+        xa, xb = rng.normal(0, 1, a).astype(F), rng.uniform(0.5, 2, b).astype(F)
+        assert_bit_exact(gpuops.broadcast_binary(op, xa, a, xb, b, out), oracle.broadcast_binary(op, xa, a, xb, b, out),
+                         "broadcast %d %s x %s" % (op, a, b))
+
+
+@pytest.mark.parametrize("seed", [10, 11])
+def test_mover_random_shapes(gpu, seed):
+    rng = np.random.default_rng(seed)
+    lib = shadow_amd.hip()
+    for _ in range(50):
+        n, c = int(rng.integers(1, 4)), int(rng.integers(1, 70))
+        ih, iw, oh, ow = [int(v) for v in rng.integers(1, 60, 4)]
+        typ = int(rng.integers(0, 2))
+        align = int(rng.integers(0, 2)) if typ == 1 else 0
+        if align and (oh < 2 or ow < 2):
+            continue
+        x = rng.normal(0, 2, (n, c, ih, iw)).astype(F)
+        want = oracle.resize_op(x, [oh, ow], [1.0], typ, bool(align))
+        dx, dy = Buffer.from_numpy(x.ravel()), Buffer(4 * want.size)
+        check(lib.shdw_hip_resize(ints([n, c, ih, iw]), ints([n, c, oh, ow]), typ, align, dx.ptr, dy.ptr, None))
+        gpuops._sync()
+        assert_bit_exact(dy.download(count=want.size), want.ravel(),
+                         "resize type %d align %d %s -> %s" % (typ, align, x.shape, [oh, ow]))
+        dy.free()
+        pads = [int(v) for v in rng.integers(0, 4, 4)]
+        want = oracle.pad_op(x, pads, 0.5)
+        dy = Buffer(4 * want.size)
+        check(lib.shdw_hip_pad(ints([n, c, ih, iw]), ints(pads), 0.5, dx.ptr, dy.ptr, None))
+        gpuops._sync()
+        assert_bit_exact(dy.download(count=want.size), want.ravel(), "pad %s of %s" % (pads, x.shape))
+        dy.free()
+        group = int(rng.choice([d for d in range(1, c + 1) if c % d == 0]))
+        dy = Buffer(4 * x.size)
+        check(lib.shdw_hip_shuffle_channel(n, c, ih * iw, group, dx.ptr, dy.ptr, None))
+        gpuops._sync()
+        assert_bit_exact(dy.download(count=x.size), oracle.shuffle_channel_op(x, group).ravel(),
+                         "shuffle %d groups of %s" % (group, x.shape))
+        dx.free()
+        dy.free()
