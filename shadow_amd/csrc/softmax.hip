@@ -93,7 +93,11 @@ __global__ __launch_bounds__(kWave) void softmax_columns_kernel(const float* x, 
 
 // Same layout for dim <= DMAX: the column lives in registers, so x is read once
 // and y written once, and all of a lane's loads are in flight together.
-template <int DMAX>
+// The first DFULL rows exist for every column this instance is launched for
+// (DFULL < dim <= DMAX) and run as straight-line code, which lets the compiler
+// interleave the exp chains of neighbouring rows; only the last DMAX - DFULL
+// rows carry the `c < dim` test (each guarded row is a basic block of its own).
+template <int DMAX, int DFULL>
 __global__ __launch_bounds__(kBlock) void softmax_columns_reg_kernel(const float* x, float* y,
                                                                       uint32_t columns,
                                                                       uint32_t dim,
@@ -112,22 +116,22 @@ __global__ __launch_bounds__(kBlock) void softmax_columns_reg_kernel(const float
   float v[DMAX];
 #pragma unroll
   for (int c = 0; c < DMAX; ++c)
-    if (c < dim) v[c] = __builtin_nontemporal_load(xc + static_cast<uint64_t>(c) * inner);
+    if (c < DFULL || c < dim) v[c] = __builtin_nontemporal_load(xc + static_cast<uint64_t>(c) * inner);
   float max_val = -FLT_MAX;
 #pragma unroll
   for (int c = 0; c < DMAX; ++c)
-    if (c < dim) max_val = std_max(v[c], max_val);
+    if (c < DFULL || c < dim) max_val = std_max(v[c], max_val);
   float sum = 0.f;
 #pragma unroll
   for (int c = 0; c < DMAX; ++c) {
-    if (c < dim) {
+    if (c < DFULL || c < dim) {
       v[c] = libm::exact_expf(v[c] - max_val, tab);
       sum += v[c];
     }
   }
 #pragma unroll
   for (int c = 0; c < DMAX; ++c)
-    if (c < dim) __builtin_nontemporal_store(v[c] / sum, yc + static_cast<uint64_t>(c) * inner);
+    if (c < DFULL || c < dim) __builtin_nontemporal_store(v[c] / sum, yc + static_cast<uint64_t>(c) * inner);
 }
 
 // Copy a contiguous slab into LDS through `f`, a few loads in flight per lane.
@@ -694,15 +698,18 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
   const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
   if (g.use_slab)
     softmax_slab_kernel<<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, static_cast<uint32_t>(dim), fi);
-  else if (dim <= 16)
-    softmax_columns_reg_kernel<16><<<grid_for(g.columns), kBlock, 0, st>>>(
-        x, y, g.columns, static_cast<uint32_t>(dim), fi);
-  else if (dim <= 32)
-    softmax_columns_reg_kernel<32><<<grid_for(g.columns), kBlock, 0, st>>>(
-        x, y, g.columns, static_cast<uint32_t>(dim), fi);
-  else if (dim <= 64)  // the tile kernel is slower here: [64,49,128,128] 115 us against 88
-    softmax_columns_reg_kernel<64><<<grid_for(g.columns), kBlock, 0, st>>>(
-        x, y, g.columns, static_cast<uint32_t>(dim), fi);
+  else if (dim <= 64) {
+    // the tile kernel is slower here: [64,49,128,128] 115 us against 88
+    const uint32_t grid = grid_for(g.columns), d = static_cast<uint32_t>(dim);
+    if (dim <= 16)
+      softmax_columns_reg_kernel<16, 0><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi);
+    else if (dim <= 32)
+      softmax_columns_reg_kernel<32, 16><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi);
+    else if (dim <= 48)
+      softmax_columns_reg_kernel<48, 32><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi);
+    else
+      softmax_columns_reg_kernel<64, 48><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi);
+  }
   else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner && dim * 64 * sizeof(float) + kExpTabBytes <= kTileLdsBytes)
     launch_softmax_tile_ts<6>(outer_num, dim, inner_num, x, y, st);
   else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner)
