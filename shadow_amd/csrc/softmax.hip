@@ -66,7 +66,22 @@ __global__ __launch_bounds__(kWave) void softmax_columns_kernel(const float* x, 
       if (c0 + u < dim) max_val = std_max(v[u], max_val);
   }
   float sum = 0.f;
-  for (uint32_t c0 = 0; c0 < dim; c0 += kColumnBatch) {
+  // Whole batches run without the `c < dim` test: a tested row is a basic block
+  // of its own and the exp chains of different blocks are not interleaved.
+  uint32_t c0 = 0;
+  for (; c0 + kColumnBatch <= dim; c0 += kColumnBatch) {
+    float v[kColumnBatch];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u) v[u] = xc[static_cast<uint64_t>(c0 + u) * inner];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u) v[u] = libm::exact_expf(v[u] - max_val, tab);
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u) {
+      yc[static_cast<uint64_t>(c0 + u) * inner] = v[u];
+      sum += v[u];
+    }
+  }
+  if (c0 < dim) {
     float v[kColumnBatch];
 #pragma unroll
     for (int u = 0; u < kColumnBatch; ++u)
