@@ -95,7 +95,17 @@ __global__ __launch_bounds__(kWave) void softmax_columns_kernel(const float* x, 
       }
     }
   }
-  for (uint32_t c0 = 0; c0 < dim; c0 += kColumnBatch) {
+  for (c0 = 0; c0 + kColumnBatch <= dim; c0 += kColumnBatch) {
+    float v[kColumnBatch];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u) v[u] = yc[static_cast<uint64_t>(c0 + u) * inner];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u) v[u] = v[u] / sum;
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u)
+      __builtin_nontemporal_store(v[u], yc + static_cast<uint64_t>(c0 + u) * inner);
+  }
+  if (c0 < dim) {
     float v[kColumnBatch];
 #pragma unroll
     for (int u = 0; u < kColumnBatch; ++u)
@@ -328,7 +338,18 @@ __global__ __launch_bounds__(kWave) void normalize_columns_kernel(const float* x
       if (c0 + u < dim) acc += norm_term<PMODE>(v[u], p);
   }
   const float div = norm_finish<PMODE>(acc, p, eps);
-  for (uint32_t c0 = 0; c0 < dim; c0 += kColumnBatch) {
+  uint32_t c0 = 0;
+  for (; c0 + kColumnBatch <= dim; c0 += kColumnBatch) {  // whole batches: no per-row test between the divisions
+    float v[kColumnBatch];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u) v[u] = xc[static_cast<uint64_t>(c0 + u) * inner];
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u) v[u] = ssd_scaled<SM>(v[u] / div, scale, c0 + u);
+#pragma unroll
+    for (int u = 0; u < kColumnBatch; ++u)
+      __builtin_nontemporal_store(v[u], yc + static_cast<uint64_t>(c0 + u) * inner);
+  }
+  if (c0 < dim) {
     float v[kColumnBatch];
 #pragma unroll
     for (int u = 0; u < kColumnBatch; ++u)
