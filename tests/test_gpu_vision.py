@@ -357,7 +357,9 @@ def test_group_norm_rows_extreme_magnitudes(gpu, outer, inner):
 
 
 NORM_ROWS = [(6, 49), (4, 784), (8, 1024), (3, 2048), (5, 3136), (2, 4096), (2, 4100), (2, 25088), (7, 5),
-             (300, 12), (1, 1), (3, 1000), (2, 8192), (2, 6002), (7, 400), (2100, 1200), (2051, 2048), (9, 256), (3, 16384), (2, 32768), (2, 32772), (1, 70000)]
+             (300, 12), (1, 1), (3, 1000), (2, 8192), (2, 6002), (7, 400), (2100, 1200), (2051, 2048), (9, 256), (3, 16384), (2, 32768), (2, 32772), (1, 70000),
+             # a thousand and more short rows: through LDS, one lane per row
+             (2000, 49), (1025, 127), (1500, 5), (4099, 56), (1024, 9), (3000, 66)]
 
 
 @pytest.mark.parametrize("outer,inner", NORM_ROWS)
@@ -370,6 +372,7 @@ def test_group_norm_rows(gpu, outer, inner):
 
 
 @pytest.mark.parametrize("shape,group", [((2, 8, 5, 5), 1), ((2, 8, 5, 5), 4), ((4, 32, 14, 14), 8), ((2, 6, 7, 3), 6),
+                                         ((4, 512, 7, 7), 512), ((8, 256, 3, 3), 128), ((2, 1024, 5, 5), 1024),
                                          ((1, 64, 56, 56), 32)])
 def test_group_and_instance_norm_op(ws, shape, group):
     x = normal(41, shape, 2.0) + F(0.5)
