@@ -119,3 +119,61 @@ def test_mover_random_shapes(gpu, seed):
                          "shuffle %d groups of %s" % (group, x.shape))
         dx.free()
         dy.free()
+
+
+@pytest.fixture()
+def ws(gpu):
+    w = shadow_amd.Workspace("Native", 0)
+    yield w
+    w.close()
+
+
+def _run(ws, op_type, x, args, top):
+    ws.set_blob("x", x)
+    op = ws.create_op(op_type, ["x"], [top], args)
+    op.run()
+    return ws.get_blob(top)
+
+
+@pytest.mark.parametrize("seed", [12, 13])
+def test_pooling_random_shapes(ws, seed):
+    rng = np.random.default_rng(seed)
+    for t in range(60):
+        n, c = int(rng.integers(1, 4)), int(rng.integers(1, 40))
+        h, w = int(rng.integers(1, 70)), int(rng.integers(1, 70))
+        kh, kw = int(rng.integers(1, min(h, 7) + 1)), int(rng.integers(1, min(w, 7) + 1))
+        sh, sw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        ph, pw = int(rng.integers(0, kh)), int(rng.integers(0, kw))
+        pool, full = int(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        x = rng.normal(0, 2, (n, c, h, w)).astype(F)
+        args = {"pool": pool, "kernel_size": [kh, kw], "stride": [sh, sw], "pad": [ph, pw], "full_pooling": full}
+        try:
+            want = oracle.pooling_op(x, pool, [kh, kw], [sh, sw], [ph, pw], full_pooling=full)
+        except oracle.OracleCheckError:
+            continue
+        got = _run(ws, "Pooling", x, args, "pool%d" % t)
+        assert got.shape == want.shape
+        assert_bit_exact(got, want, "pooling %s %s" % (x.shape, args))
+
+
+@pytest.mark.parametrize("seed", [14, 15])
+def test_permute_reorg_gather_random_shapes(ws, seed):
+    rng = np.random.default_rng(seed)
+    for t in range(50):
+        nd = int(rng.integers(2, 6))
+        shape = [int(rng.integers(1, 12)) for _ in range(nd)]
+        order = [int(v) for v in rng.permutation(nd)]
+        x = rng.normal(0, 1, shape).astype(F)
+        assert_bit_exact(_run(ws, "Permute", x, {"order": order}, "perm%d" % t), oracle.permute_op(x, order),
+                         "permute %s by %s" % (shape, order))
+        s = int(rng.integers(1, 4))
+        shape = (int(rng.integers(1, 3)), s * s * int(rng.integers(1, 6)), s * int(rng.integers(1, 12)),
+                 s * int(rng.integers(1, 12)))
+        typ = int(rng.integers(0, 2))
+        x = rng.normal(0, 1, shape).astype(F)
+        assert_bit_exact(_run(ws, "Reorg", x, {"type": typ, "stride": s}, "reorg%d" % t), oracle.reorg_op(x, typ, s),
+                         "reorg type %d stride %d of %s" % (typ, s, shape))
+        axis = int(rng.integers(0, 4))
+        idx = [int(v) for v in rng.integers(0, shape[axis], int(rng.integers(1, 6)))]
+        assert_bit_exact(_run(ws, "Gather", x, {"axis": axis, "indexes": idx}, "gather%d" % t),
+                         oracle.gather_op(x, axis, idx), "gather %s on axis %d of %s" % (idx, axis, shape))
