@@ -181,22 +181,36 @@ int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* ax
     const int by_fill = ceil_div64(1024, plan->outer);
     const int by_work = ceil_div64(plan->reduce * plan->inner, 8 * 1024);  // >= 8 steps per workgroup
     plan->splits = std::max(1, std::min(std::min(by_fill, by_work), 1024));
+  } else if (plan->inner % 4 == 0) {
+    // Whole 128-bit vectors per row.  A workgroup of 512 lanes owns a tile of 4 L
+    // columns (L lanes per row piece, 512 / L rows per step); wider pieces are
+    // longer contiguous reads, narrower ones give more workgroups.  Take the
+    // widest piece up to 512 bytes that still gives 192 workgroups (6 waves per
+    // CU, each with eight 128-bit loads in flight); when even 128-byte pieces do
+    // not, slice the reduced axis.
+    const int64_t inner4 = plan->inner / 4;
+    int lanes = 8;
+    for (int l : {32, 16, 8}) {
+      if (((inner4 + l - 1) / l) * plan->outer >= 192) {
+        lanes = l;
+        break;
+      }
+    }
+    plan->strided_lanes = lanes;
+    const int64_t blocks = ((inner4 + lanes - 1) / lanes) * plan->outer;
+    const int by_fill = ceil_div64(192, blocks);
+    const int by_work = ceil_div64(plan->reduce, 8 * (512 / lanes));  // a full batch of loads per lane
+    plan->splits = std::max(1, std::min(std::min(by_fill, by_work), 1024));
   } else {
-    // Pick columns per lane (128-bit or scalar loads) and waves per column tile
-    // so that one launch gives >= 256 workgroups (one per CU) and >= 2048 waves;
-    // only when no shape does, split the reduced axis over grid.z and add a
-    // second stage.
-    // A tile of 128-bit loads spans 256 columns; fewer than 128 columns leave
-    // most of its lanes idle (56 columns: 14 of 64), and one column per lane
-    // does better (reduce 2048 over [128, 2048, 56]: 26.5 us -> 18 us).
-    const int vec_max = (plan->inner % 4 == 0 && plan->inner >= 128) ? 4 : 1;
-    const int cand[4][2] = {{4, 4}, {4, 16}, {1, 4}, {1, 16}};
+    // One column per lane: 4 or 16 waves per 64-column tile, so that one launch
+    // gives >= 256 workgroups (one per CU) and >= 2048 waves; only when neither
+    // does, slice the reduced axis and fold the slices afterwards.
+    const int64_t tiles = (plan->inner + 63) / 64;
+    const int64_t base_blocks = tiles * plan->outer;
     bool single = false;
-    for (const auto& c : cand) {
-      if (c[0] > vec_max) continue;
-      const int64_t blocks = ((plan->inner + 64 * c[0] - 1) / (64 * c[0])) * plan->outer;
-      if (blocks >= 256 && blocks * c[1] >= 2048 && plan->reduce >= 8 * c[1]) {
-        plan->strided_vec = c[0], plan->strided_waves = c[1];
+    for (int waves : {4, 16}) {
+      if (base_blocks >= 256 && base_blocks * waves >= 2048 && plan->reduce >= 8 * waves) {
+        plan->strided_waves = waves;
         single = true;
         break;
       }
@@ -204,9 +218,7 @@ int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* ax
     if (single) {
       plan->splits = 1;
     } else {
-      plan->strided_vec = vec_max, plan->strided_waves = 4;
-      const int64_t tiles = (plan->inner + 64 * vec_max - 1) / (64 * vec_max);
-      const int64_t base_blocks = tiles * plan->outer;
+      plan->strided_waves = 4;
       const int by_fill = ceil_div64(1024, base_blocks);
       const int by_work = ceil_div64(plan->reduce, 64);  // >= 16 rows per wave
       plan->splits = std::max(1, std::min(by_fill, by_work));

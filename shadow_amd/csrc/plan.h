@@ -47,8 +47,10 @@ struct ReducePlan {
   int64_t outer = 1, reduce = 1, inner = 1;
   int splits = 1;
   bool wave_per_row = false;  // kRows: 16/32/64 lanes per row instead of a workgroup
-  int strided_waves = 4;      // kStrided: wave64 per workgroup sharing a column tile (4 or 16)
-  int strided_vec = 4;        // kStrided: columns per lane (4 = 128-bit loads, 1 = scalar)
+  int strided_lanes = 0;      // kStrided with whole 128-bit vectors per row (inner % 4 == 0, inner >= 128):
+                              // lanes per row piece (8, 16, 32 or 64), a column tile is 4 * lanes wide;
+                              // 0 selects one column per lane
+  int strided_waves = 4;      // kStrided, one column per lane: wave64 per workgroup sharing a column tile (4 or 16)
   int flat_period = 0;        // kStrided with fewer than 128 columns: > 0 selects the flat kernel; elements
                               // the 256 lanes cover per step (a multiple of inner and of 4, <= 1024)
   int64_t outputs = 1;        // number of output elements

@@ -2,23 +2,18 @@
 // (shadow/operators/kernels/reduce.cpp:9-76); here the reduced extent is spread
 // over lanes, waves and, when there are few outputs, workgroups:
 //
-//   rows     x[outer][reduce]           reduced axis contiguous.  One wave64 per
-//                                       row for short rows; a workgroup per
-//                                       (row, slice) for long ones.
-//   strided  x[outer][reduce][inner]    lanes run along `inner` (coalesced),
-//                                       the four waves of a workgroup and
-//                                       optional grid.z slices split `reduce`.
+//   rows     x[outer][reduce]           reduced axis contiguous.  A group of 16,
+//                                       32 or 64 lanes per row for short rows; a
+//                                       workgroup per (row, slice) for long ones.
+//   strided  x[outer][reduce][inner]    lanes run along `inner` (coalesced); the
+//                                       lane groups or waves of a workgroup and
+//                                       optional grid.y slices split `reduce`.
 //   generic  any axis set               one wave per output, index lists
 //                                       replaced by division by constants.
 //   stage 2  combines the per-slice partials of a split first stage.
 //
-// PROD/SUM/AVG/L1/L2 accumulate in fp64 exactly as the reference does, so the
-// only difference is association order (~1e-16 relative before the single
-// rounding to fp32).  MAX/MIN must be bit-exact although the reference's
-// "first element attaining the extremum wins" depends on order when the
-// extremum is a zero (+0 and -0 compare equal): every accumulator therefore
-// also tracks the smallest list position of a zero together with its sign, and
-// the sign of a zero result is taken from there.
+// The accumulators (fp64 sums, or an fp32 extremum with the position of its
+// first zero) are in reduce_acc.h.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -28,131 +23,18 @@
 #include "device_common.h"
 #include "launch.h"
 #include "plan.h"
+#include "reduce_acc.h"
 
 #pragma clang fp contract(off)
 
 namespace shdw {
 
-// What a first stage hands to the second, 8 bytes per (output, slice): the fp64
-// accumulator, or {fp32 extremum, zero key} for MAX/MIN.
-struct Partial {
-  uint64_t bits;
-};
-static_assert(sizeof(Partial) == kReducePartialBytes, "partial layout");
-
-constexpr bool is_select(int op) { return op == SHDW_REDUCE_MAX || op == SHDW_REDUCE_MIN; }
-
-// ---- fp64 accumulating ops ----
-template <int OP, bool SELECT = is_select(OP)>
-struct Acc {
-  double v;
-  SHDW_DEVICE void init() { v = (OP == SHDW_REDUCE_PROD) ? 1.0 : 0.0; }
-  SHDW_DEVICE void add(float x, uint32_t) {
-    if (OP == SHDW_REDUCE_PROD) {
-      v *= static_cast<double>(x);
-    } else if (OP == SHDW_REDUCE_L1) {
-      v += static_cast<double>(__builtin_fabsf(x));
-    } else if (OP == SHDW_REDUCE_L2) {
-      const float ax = __builtin_fabsf(x);
-      const float sq = ax * ax;  // fp32 product, then widened
-      v += static_cast<double>(sq);
-    } else {
-      v += static_cast<double>(x);
-    }
-  }
-  SHDW_DEVICE void merge(const Acc& o) {
-    if (OP == SHDW_REDUCE_PROD) v *= o.v; else v += o.v;
-  }
-  template <int CTRL>
-  SHDW_DEVICE Acc dpp() const {
-    Acc r;
-    r.v = dpp_f64<CTRL>(v);
-    return r;
-  }
-  SHDW_DEVICE Acc shfl_xor(int m) const {
-    Acc r;
-    r.v = __shfl_xor(v, m, kWave);
-    return r;
-  }
-  SHDW_DEVICE float finalize(uint32_t window) const {
-    if (OP == SHDW_REDUCE_AVG) return static_cast<float>(v / static_cast<double>(static_cast<int>(window)));
-    if (OP == SHDW_REDUCE_L2) return __builtin_sqrtf(static_cast<float>(v));
-    return static_cast<float>(v);
-  }
-  SHDW_DEVICE Partial pack() const { return Partial{static_cast<uint64_t>(__double_as_longlong(v))}; }
-  SHDW_DEVICE void unpack(const Partial& p) { v = __longlong_as_double(static_cast<long long>(p.bits)); }
-};
-
-// ---- MAX / MIN ----
-template <int OP>
-struct Acc<OP, true> {
-  float v;
-  uint32_t key;  // min over zeros seen of (list position << 1 | sign bit)
-  SHDW_DEVICE void init() {
-    v = (OP == SHDW_REDUCE_MAX) ? -FLT_MAX : FLT_MAX;
-    key = 0xffffffffu;
-  }
-  SHDW_DEVICE void add(float x, uint32_t pos) {
-    if (OP == SHDW_REDUCE_MAX) v = (v < x) ? x : v; else v = (x < v) ? x : v;
-    if (x == 0.0f) {
-      const uint32_t k = (pos << 1) | (__float_as_uint(x) >> 31);
-      key = k < key ? k : key;
-    }
-  }
-  SHDW_DEVICE void merge(const Acc& o) {
-    if (OP == SHDW_REDUCE_MAX) v = (v < o.v) ? o.v : v; else v = (o.v < v) ? o.v : v;
-    key = o.key < key ? o.key : key;
-  }
-  template <int CTRL>
-  SHDW_DEVICE Acc dpp() const {
-    Acc r;
-    r.v = dpp_f32<CTRL>(v);
-    r.key = dpp_u32<CTRL>(key);
-    return r;
-  }
-  SHDW_DEVICE Acc shfl_xor(int m) const {
-    Acc r;
-    r.v = __shfl_xor(v, m, kWave);
-    r.key = __shfl_xor(key, m, kWave);
-    return r;
-  }
-  SHDW_DEVICE float finalize(uint32_t) const {
-    if (v == 0.0f) return (key & 1u) ? -0.0f : 0.0f;
-    return v;
-  }
-  SHDW_DEVICE Partial pack() const {
-    return Partial{(static_cast<uint64_t>(key) << 32) | __float_as_uint(v)};
-  }
-  SHDW_DEVICE void unpack(const Partial& p) {
-    v = __uint_as_float(static_cast<uint32_t>(p.bits));
-    key = static_cast<uint32_t>(p.bits >> 32);
-  }
-};
-
-// All 64 lanes must be active.  Every lane ends with the same combined value:
-// each exchange pairs two lanes that both compute merge(own, other), and every
-// merge used here is commutative bit-for-bit.
-template <class A, int G = kWave>
-SHDW_DEVICE A group_allreduce(A a) {  // G = 16, 32 or 64 consecutive lanes
-  a.merge(a.template dpp<kDppXor1>());
-  a.merge(a.template dpp<kDppXor2>());
-  a.merge(a.template dpp<kDppHalfMirror>());
-  a.merge(a.template dpp<kDppMirror>());
-  if (G >= 32) a.merge(a.shfl_xor(16));
-  if (G >= 64) a.merge(a.shfl_xor(32));
-  return a;
-}
-template <class A>
-SHDW_DEVICE A wave_allreduce(A a) {
-  return group_allreduce<A, kWave>(a);
-}
+constexpr int kBatch = 8;  // vectors a lane requests before it consumes the first
 
 // ---------------------------------------------------------------------------
 // rows, G lanes per row (G = 16, 32, 64): short rows share a wave so that no
 // lane idles and the combine stays inside DPP rows where possible.
 // ---------------------------------------------------------------------------
-constexpr int kRowBatch = 8;  // vectors a lane requests before it consumes the first
-
 template <int OP, bool VEC, int G>
 __global__ __launch_bounds__(kBlock) void reduce_rows_group_kernel(const float* x, float* y,
                                                                     uint32_t rows,
@@ -167,22 +49,17 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_group_kernel(const float* 
   acc.init();
   if (VEC) {
     const uint32_t nv = reduce / 4;
-    for (uint32_t base = 0; base < nv; base += kRowBatch * G) {
-      v4f v[kRowBatch];
+    for (uint32_t base = 0; base < nv; base += kBatch * G) {
+      v4f v[kBatch];
+      bool valid[kBatch];
       // all loads of the trip are issued before the first value is consumed
 #pragma unroll
-      for (int u = 0; u < kRowBatch; ++u) {
+      for (int u = 0; u < kBatch; ++u) {
         const uint32_t i = base + u * G + lane;
-        if (i < nv) v[u] = load4_stream_any(p + 4ull * i);  // rows start on any dword
+        valid[u] = i < nv;
+        if (valid[u]) v[u] = load4_stream_any(p + 4ull * i);  // rows start on any dword
       }
-#pragma unroll
-      for (int u = 0; u < kRowBatch; ++u) {
-        const uint32_t i = base + u * G + lane;
-        if (i < nv) {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) acc.add(v[u][j], 4 * i + j);
-        }
-      }
+      fold_batch<kBatch, true>(&acc, v, valid, [&](int u, int j) { return 4 * (base + u * G + lane) + j; });
     }
     const uint32_t t = 4 * nv + lane;  // the reduce % 4 elements past the last whole vector
     if (t < reduce) acc.add(p[t], t);
@@ -213,20 +90,25 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const float* 
   if (begin < end) {
     if (VEC) {
       const uint32_t vb = begin / 4, ve = end / 4;
-      uint32_t i = vb + threadIdx.x;
-      for (; i + 3 * kBlock < ve; i += 4 * kBlock) {
+      // a slice is 1024 vectors unless the row is shorter: one batch of four per lane
+      uint32_t base = vb;
+      for (; base + 4 * kBlock <= ve; base += 4 * kBlock) {  // whole batches: no per-load tests
         v4f v[4];
+        const bool valid[4] = {true, true, true, true};
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = load4_stream_any(p + 4ull * (i + u * kBlock));
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) acc.add(v[u][j], 4 * (i + u * kBlock) + j);
+        for (int u = 0; u < 4; ++u) v[u] = load4_stream_any(p + 4ull * (base + u * kBlock + threadIdx.x));
+        fold_batch<4, true>(&acc, v, valid, [&](int u, int j) { return 4 * (base + u * kBlock + threadIdx.x) + j; });
       }
-      for (; i < ve; i += kBlock) {
-        const v4f v = load4_stream_any(p + 4ull * i);
+      if (base < ve) {
+        v4f v[4];
+        bool valid[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc.add(v[j], 4 * i + j);
+        for (int u = 0; u < 4; ++u) {
+          const uint32_t i = base + u * kBlock + threadIdx.x;
+          valid[u] = i < ve;
+          if (valid[u]) v[u] = load4_stream_any(p + 4ull * i);
+        }
+        fold_batch<4, true>(&acc, v, valid, [&](int u, int j) { return 4 * (base + u * kBlock + threadIdx.x) + j; });
       }
       // elements past the last whole vector (only the final slice has any)
       const uint32_t t = 4 * ve + threadIdx.x;
@@ -352,12 +234,10 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_flat_kernel(
     uint32_t f = r_begin * inner + t4, row = r_begin;
     for (; f + 3 * period + 3 < end; f += 4 * period, row += 4 * rows_per_step) {
       v4f v[4];
+      const bool valid[4] = {true, true, true, true};
 #pragma unroll
       for (int u = 0; u < 4; ++u) v[u] = load4_stream_any(slab + f + u * period);
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j].add(v[u][j], row + u * rows_per_step + drow[j]);
+      fold_batch<4, false>(acc, v, valid, [&](int u, int j) { return row + u * rows_per_step + drow[j]; });
     }
     for (; f < end; f += period, row += rows_per_step) {
       if (f + 3 < end) {
@@ -389,80 +269,128 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_flat_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// strided: x[outer][reduce][inner] -> y[outer][inner]
+// strided, one column per lane (inner % 4 != 0): x[outer][reduce][inner] ->
+// y[outer][inner].  WAVES wave64 per workgroup (4 or 16) share one tile of 64
+// columns and interleave over the rows of their slice; with 16 waves a few
+// hundred tiles already fill the GPU and no second stage is needed.
 // ---------------------------------------------------------------------------
-// WAVES wave64 per workgroup (4 or 16) share one tile of 64*VEC columns and
-// interleave over the rows of their slice; with 16 waves a few hundred tiles
-// already fill the GPU and no second stage is needed.
-template <int OP, int VEC, int WAVES>
+template <int OP, int WAVES>
 __global__ __launch_bounds__(kWave * WAVES) void reduce_strided_kernel(
     const float* x, float* y, Partial* part, uint32_t reduce, uint32_t inner,
     uint32_t rows_per_split, uint32_t splits, uint32_t outputs, FastDiv f_tiles) {
   constexpr int kWaves = WAVES;
-  __shared__ Partial lds[kWaves - 1][VEC][kWave];
+  __shared__ Partial lds[kWaves - 1][kWave];
   const uint32_t lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
   // grid.x = outer * tiles (either can exceed the 65535 limit of grid.y), grid.y = slices
   uint32_t o, tile;
   fd_divmod(xcd_contiguous(blockIdx.x, gridDim.x), f_tiles, o, tile);
-  const uint32_t col = (tile * kWave + lane) * VEC;
+  const uint32_t col = tile * kWave + lane;
   const uint32_t split = blockIdx.y;
   const bool col_ok = col < inner;
   const uint32_t r_begin = split * rows_per_split;
   uint32_t r_end = r_begin + rows_per_split;
   if (r_end > reduce) r_end = reduce;
 
-  Acc<OP> acc[VEC];
-#pragma unroll
-  for (int j = 0; j < VEC; ++j) acc[j].init();
-
+  Acc<OP> acc;
+  acc.init();
   if (col_ok) {
     const float* p = x + static_cast<size_t>(o) * reduce * inner + col;
     uint32_t r = r_begin + w;
     for (; r + 3 * kWaves < r_end; r += 4 * kWaves) {
-      float v[4][VEC];
+      float v[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float* q = p + static_cast<size_t>(r + u * kWaves) * inner;
-        if (VEC == 4) {
-          const v4f t = load4_stream(q);
+      for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(p + static_cast<size_t>(r + u * kWaves) * inner);
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) v[u][j] = t[j];
-        } else {
-          v[u][0] = __builtin_nontemporal_load(q);
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j].add(v[u][j], r + u * kWaves);
+      for (int u = 0; u < 4; ++u) acc.add(v[u], r + u * kWaves);
     }
-    for (; r < r_end; r += kWaves) {
-      const float* q = p + static_cast<size_t>(r) * inner;
-      if (VEC == 4) {
-        const v4f t = load4_stream(q);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j].add(t[j], r);
-      } else {
-        acc[0].add(__builtin_nontemporal_load(q), r);
-      }
-    }
+    for (; r < r_end; r += kWaves) acc.add(__builtin_nontemporal_load(p + static_cast<size_t>(r) * inner), r);
   }
-  if (w > 0) {
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) lds[w - 1][j][lane] = acc[j].pack();
-  }
+  if (w > 0) lds[w - 1][lane] = acc.pack();
   __syncthreads();
   if (w == 0 && col_ok) {
+    for (int k = 0; k < kWaves - 1; ++k) {
+      Acc<OP> t;
+      t.unpack(lds[k][lane]);
+      acc.merge(t);
+    }
+    const size_t out = static_cast<size_t>(o) * inner + col;
+    if (splits == 1) y[out] = acc.finalize(reduce);
+    else part[static_cast<size_t>(split) * outputs + out] = acc.pack();
+  }
+}
+
+// ---------------------------------------------------------------------------
+// strided with whole 128-bit vectors per row (inner % 4 == 0, inner >= 128): a
+// workgroup of 512 lanes owns a tile of 4 L columns; L lanes cover one row piece
+// of the tile with one 128-bit load each and the 512 / L lane groups take rows
+// r, r + 512/L, ...  All loads of a batch of eight rows per lane are requested
+// before the first is used.  The accumulators meet in LDS and lane c < 4 L
+// folds column c over the lane groups in group order.  Measured on max over the
+// 512 channels of [32,512,28,28] (rows of 3136 bytes): 512-byte pieces (L = 32)
+// 9.9 us, 256-byte pieces 10.6 us, 128-byte pieces 11.2 us, one column per lane
+// with 8 / 16 waves per tile 10.1 / 11.2 us; workgroups of 256 or 1024 lanes and
+// batches of 16 were level or slower.
+// ---------------------------------------------------------------------------
+constexpr int kTileThreads = 512;
+
+template <int OP, int L>
+__global__ __launch_bounds__(kTileThreads) void reduce_strided_tile_kernel(
+    const float* x, float* y, Partial* part, uint32_t reduce, uint32_t inner, uint32_t rows_per_split,
+    uint32_t splits, uint32_t outputs, FastDiv f_tiles) {
+  constexpr uint32_t kGroups = kTileThreads / L;
+  __shared__ Partial lds[kTileThreads * 4];
+  uint32_t o, tile;
+  fd_divmod(xcd_contiguous(blockIdx.x, gridDim.x), f_tiles, o, tile);
+  const uint32_t pl = threadIdx.x % L, rg = threadIdx.x / L;
+  const uint32_t col = (tile * L + pl) * 4;
+  const uint32_t split = blockIdx.y;
+  const uint32_t r_begin = min(split * rows_per_split, reduce);
+  const uint32_t r_end = min(r_begin + rows_per_split, reduce);
+
+  Acc<OP> acc[4];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      for (int k = 0; k < kWaves - 1; ++k) {
-        Acc<OP> t;
-        t.unpack(lds[k][j][lane]);
-        acc[j].merge(t);
+  for (int j = 0; j < 4; ++j) acc[j].init();
+
+  if (col < inner) {
+    const float* p = x + static_cast<size_t>(o) * reduce * inner + col;
+    uint32_t base = r_begin + rg;
+    // whole batches run without per-load tests: a tested load is a branch of its
+    // own and the loads of a batch then no longer issue back to back
+    for (; base + (kBatch - 1) * kGroups < r_end; base += kBatch * kGroups) {
+      v4f v[kBatch];
+      const bool valid[kBatch] = {true, true, true, true, true, true, true, true};
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) v[u] = load4_stream_any(p + static_cast<size_t>(base + u * kGroups) * inner);
+      fold_batch<kBatch, false>(acc, v, valid, [&](int u, int) { return base + u * kGroups; });
+    }
+    if (base < r_end) {
+      v4f v[kBatch];
+      bool valid[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const uint32_t r = base + u * kGroups;
+        valid[u] = r < r_end;
+        if (valid[u]) v[u] = load4_stream_any(p + static_cast<size_t>(r) * inner);
       }
-      const size_t out = static_cast<size_t>(o) * inner + col + j;
-      if (splits == 1) y[out] = acc[j].finalize(reduce);
-      else part[static_cast<size_t>(split) * outputs + out] = acc[j].pack();
+      fold_batch<kBatch, false>(acc, v, valid, [&](int u, int) { return base + u * kGroups; });
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) lds[threadIdx.x * 4 + j] = acc[j].pack();  // [group][column of the tile]
+  __syncthreads();
+  if (threadIdx.x < 4 * L) {
+    const uint32_t c = tile * 4 * L + threadIdx.x;
+    Acc<OP> total;
+    total.init();
+    for (uint32_t g = 0; g < kGroups; ++g) {
+      Acc<OP> t;
+      t.unpack(lds[g * 4 * L + threadIdx.x]);
+      total.merge(t);
+    }
+    if (c < inner) {
+      const size_t out = static_cast<size_t>(o) * inner + c;
+      if (splits == 1) y[out] = total.finalize(reduce);
+      else part[static_cast<size_t>(split) * outputs + out] = total.pack();
     }
   }
 }
@@ -510,7 +438,9 @@ __global__ __launch_bounds__(kBlock) void reduce_generic_kernel(GenericArgs g, c
 // stage 2: y[o] = finalize(merge_s part[o*stride_o + s*stride_s])
 //   _lane : one lane per output, slices walked serially (few slices, many
 //           outputs; coalesced when stride_o == 1)
-//   _block: one workgroup per output (many slices, few outputs)
+//   _block: one workgroup per output (many slices, few outputs).  The full sum
+//           of 12.8 M elements leaves 3136 partials for one output: 1024 lanes
+//           fold them in 2.3 us including the launch, 256 lanes in 4 us.
 // ---------------------------------------------------------------------------
 template <int OP>
 __global__ __launch_bounds__(kBlock) void reduce_stage2_lane_kernel(const Partial* part, float* y,
@@ -531,17 +461,17 @@ __global__ __launch_bounds__(kBlock) void reduce_stage2_lane_kernel(const Partia
   y[o] = acc.finalize(window);
 }
 
-template <int OP>
-__global__ __launch_bounds__(kBlock) void reduce_stage2_block_kernel(const Partial* part, float* y,
-                                                                      uint32_t splits,
-                                                                      size_t stride_o,
-                                                                      size_t stride_s,
-                                                                      uint32_t window) {
-  __shared__ Partial lds[kBlock / kWave];
+template <int OP, int THREADS>
+__global__ __launch_bounds__(THREADS) void reduce_stage2_block_kernel(const Partial* part, float* y,
+                                                                       uint32_t splits,
+                                                                       size_t stride_o,
+                                                                       size_t stride_s,
+                                                                       uint32_t window) {
+  __shared__ Partial lds[THREADS / kWave];
   const uint32_t o = blockIdx.x;
   Acc<OP> acc;
   acc.init();
-  for (uint32_t s = threadIdx.x; s < splits; s += kBlock) {
+  for (uint32_t s = threadIdx.x; s < splits; s += THREADS) {
     Acc<OP> t;
     t.unpack(part[o * stride_o + s * stride_s]);
     acc.merge(t);
@@ -551,7 +481,7 @@ __global__ __launch_bounds__(kBlock) void reduce_stage2_block_kernel(const Parti
   if (lane == 0) lds[w] = acc.pack();
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int k = 1; k < kBlock / kWave; ++k) {
+    for (int k = 1; k < THREADS / kWave; ++k) {
       Acc<OP> t;
       t.unpack(lds[k]);
       acc.merge(t);
@@ -566,9 +496,12 @@ static int run_stage2(const Partial* part, float* y, uint32_t outputs, uint32_t 
   if (splits <= 64) {
     reduce_stage2_lane_kernel<OP><<<grid_for(outputs), kBlock, 0, st>>>(part, y, outputs, splits,
                                                                         stride_o, stride_s, window);
+  } else if (splits <= 256) {
+    reduce_stage2_block_kernel<OP, kBlock><<<outputs, kBlock, 0, st>>>(part, y, splits, stride_o, stride_s,
+                                                                       window);
   } else {
-    reduce_stage2_block_kernel<OP><<<outputs, kBlock, 0, st>>>(part, y, splits, stride_o, stride_s,
-                                                               window);
+    reduce_stage2_block_kernel<OP, 1024><<<outputs, 1024, 0, st>>>(part, y, splits, stride_o, stride_s,
+                                                                   window);
   }
   return launch_status();
 }
@@ -650,24 +583,27 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
     reduce_strided_flat_kernel<OP><<<dim3(outer, splits), kBlock, 0, st>>>(
         x, y, part, reduce, inner, rows_per_split, splits, outputs, static_cast<uint32_t>(pl.flat_period),
         make_fastdiv(inner));
-    int rc = launch_status();
-    if (rc != SHDW_OK || splits == 1) return rc;
-    return run_stage2<OP>(part, y, outputs, splits, 1, outputs, window, st);
-  }
-  const bool vec = pl.strided_vec == 4 && inner % 4 == 0 && aligned16(x);
-  const int v = vec ? 4 : 1;
-  const uint32_t tiles = (inner + kWave * v - 1) / (kWave * v);
-  const dim3 grid(tiles * outer, splits);  // tiles * outer <= outputs; splits <= 1024
-  const FastDiv f_tiles = make_fastdiv(tiles);
-#define SHDW_STRIDED(V, W)                                                                   \
-  reduce_strided_kernel<OP, V, W><<<grid, kWave * W, 0, st>>>(x, y, part, reduce, inner,       \
-                                                             rows_per_split, splits, outputs, f_tiles)
-  if (pl.strided_waves == 16) {
-    if (vec) SHDW_STRIDED(4, 16); else SHDW_STRIDED(1, 16);
+  } else if (pl.strided_lanes > 0) {  // inner % 4 == 0: tiles of 4 * lanes columns, 128-bit loads
+    const uint32_t l = static_cast<uint32_t>(pl.strided_lanes);
+    const uint32_t tiles = (inner / 4 + l - 1) / l;
+    const dim3 grid(tiles * outer, splits);  // tiles * outer <= outputs; splits <= 1024
+    const FastDiv f_tiles = make_fastdiv(tiles);
+#define SHDW_TILE(LANES)                                                                                   \
+  reduce_strided_tile_kernel<OP, LANES><<<grid, kTileThreads, 0, st>>>(x, y, part, reduce, inner, rows_per_split, \
+                                                                       splits, outputs, f_tiles)
+    if (l == 8) SHDW_TILE(8); else if (l == 16) SHDW_TILE(16); else if (l == 32) SHDW_TILE(32); else SHDW_TILE(64);
+#undef SHDW_TILE
   } else {
-    if (vec) SHDW_STRIDED(4, 4); else SHDW_STRIDED(1, 4);
+    const uint32_t tiles = (inner + kWave - 1) / kWave;  // one column per lane
+    const dim3 grid(tiles * outer, splits);
+    const FastDiv f_tiles = make_fastdiv(tiles);
+    if (pl.strided_waves == 16)
+      reduce_strided_kernel<OP, 16><<<grid, kWave * 16, 0, st>>>(x, y, part, reduce, inner, rows_per_split, splits,
+                                                                 outputs, f_tiles);
+    else
+      reduce_strided_kernel<OP, 4><<<grid, kWave * 4, 0, st>>>(x, y, part, reduce, inner, rows_per_split, splits,
+                                                               outputs, f_tiles);
   }
-#undef SHDW_STRIDED
   int rc = launch_status();
   if (rc != SHDW_OK || splits == 1) return rc;
   return run_stage2<OP>(part, y, outputs, splits, 1, outputs, window, st);
