@@ -36,6 +36,7 @@ extern "C" {
 #define SHDW_E_INVALID_ARGUMENT (-1) /* null pointer, negative count, bad enum */
 #define SHDW_E_UNSUPPORTED (-2)      /* shape outside what the kernels accept  */
 #define SHDW_E_WORKSPACE (-3)        /* workspace missing or too small         */
+#define SHDW_E_STATIC_SCRATCH (-4)   /* needs more than the library's static scratch */
 
 /* ---- operation enums; values are Shadow's ---- */
 /* ref: shadow/operators/kernels/unary.hpp:9-25 */
@@ -211,6 +212,21 @@ size_t shdw_hip_reduce_workspace_bytes(int num_axes, const int* in_shape, int nu
 int shdw_hip_reduce(int operation, int num_axes, const int* in_shape, int num_reduce,
                     const int* axes, const float* x, float* y, void* workspace,
                     size_t workspace_bytes, void* stream);
+
+/* shdw_hip_reduce for callers that cannot allocate device memory or pass a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It has no counterpart in the reference.  Same arguments,
+ * results and kernels as shdw_hip_reduce; the partial results of sliced shapes
+ * go to a buffer inside the library's own device memory (1 MiB on every GPU the
+ * library runs on, held until the process ends) instead of a workspace, and the
+ * call allocates nothing.  A shape whose partials need more than
+ * shdw_hip_reduce_static_max_workspace_bytes() is rejected with
+ * SHDW_E_STATIC_SCRATCH and nothing is launched.  All calls on one GPU share the
+ * buffer: calls that overlap in time on one GPU (different streams, different
+ * threads) race; calls on one stream are ordered and safe. */
+int shdw_hip_reduce_static(int operation, int num_axes, const int* in_shape, int num_reduce,
+                           const int* axes, const float* x, float* y, void* stream);
+size_t shdw_hip_reduce_static_max_workspace_bytes(void);
 
 /* ============================ fused sequences ============================ */
 

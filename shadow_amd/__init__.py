@@ -71,6 +71,8 @@ SIGNATURES = {
     "shdw_hip_eltwise": (_I, [_I, _I, c_void_pp, c_float_p, _I, _V, _V]),
     "shdw_hip_reduce_workspace_bytes": (_Z, [_I, c_int_p, _I, c_int_p]),
     "shdw_hip_reduce": (_I, [_I, _I, c_int_p, _I, c_int_p, _V, _V, _V, _Z, _V]),
+    "shdw_hip_reduce_static": (_I, [_I, _I, c_int_p, _I, c_int_p, _V, _V, _V]),
+    "shdw_hip_reduce_static_max_workspace_bytes": (_Z, []),
     "shdw_hip_scale_residual_relu_rowmean": (_I, [_I, _I, _I, _V, _V, _V, _V, _V, _V, _V]),
     "shdw_hip_axpy_rows": (_I, [_I, _I, _V, _V, _V, _V, _V]),
     "shdw_hip_batch_norm": (_I, [_I, _I, _I, _V, _V, _V, _F, _F, _V, _V]),

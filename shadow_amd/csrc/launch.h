@@ -19,6 +19,11 @@ inline uint32_t stream_grid(uint32_t work) { return (work + 63u) / 64u; }
 // launch does not fail every later call.
 inline int launch_status() { return static_cast<int>(hipGetLastError()); }
 
+// Device memory owned by the library (reduce.hip): the partial results of
+// shdw_hip_reduce_static.  Resolves its address on the current device, once per
+// device; returns 0 or an error code.
+int library_scratch_prepare();
+
 }  // namespace shdw
 
 #endif  // SHADOW_AMD_CSRC_LAUNCH_H_

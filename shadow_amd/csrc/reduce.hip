@@ -18,6 +18,7 @@
 
 #include <algorithm>
 #include <cfloat>
+#include <mutex>
 
 #include "../../include/shadow_hip.h"
 #include "device_common.h"
@@ -506,6 +507,40 @@ static int run_stage2(const Partial* part, float* y, uint32_t outputs, uint32_t 
   return launch_status();
 }
 
+// ---------------------------------------------------------------------------
+// Partial results of shdw_hip_reduce_static: device memory of the library
+// itself, one copy on every GPU the library runs on.  Host code uses the address
+// that hipGetSymbolAddress returns for the current device (static_scratch), never
+// this name.
+// ---------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = static_cast<size_t>(1) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices];  // device address of `scratch`, per device
+
+static int static_scratch(void** ptr) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (dev < 0 || dev >= kMaxDevices) return SHDW_E_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return static_cast<int>(e);
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return SHDW_OK;
+}
+
+int library_scratch_prepare() {
+  void* p = nullptr;
+  return static_scratch(&p);
+}
+
 template <int OP>
 static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* workspace,
                       size_t workspace_bytes, hipStream_t st) {
@@ -639,6 +674,21 @@ int shdw_hip_reduce(int operation, int num_axes, const int* in_shape, int num_re
   return dispatch_reduce(operation, pl, x, y, workspace, workspace_bytes,
                          static_cast<hipStream_t>(stream));
 }
+
+int shdw_hip_reduce_static(int operation, int num_axes, const int* in_shape, int num_reduce,
+                           const int* axes, const float* x, float* y, void* stream) {
+  if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
+  ReducePlan pl;
+  int rc = plan_reduce(num_axes, in_shape, num_reduce, axes, &pl);
+  if (rc != SHDW_OK) return rc;
+  if (reduce_workspace_bytes(pl) > kStaticScratchBytes) return SHDW_E_STATIC_SCRATCH;
+  void* ptr = nullptr;
+  rc = static_scratch(&ptr);
+  if (rc != SHDW_OK) return rc;
+  return dispatch_reduce(operation, pl, x, y, ptr, kStaticScratchBytes, static_cast<hipStream_t>(stream));
+}
+
+size_t shdw_hip_reduce_static_max_workspace_bytes(void) { return kStaticScratchBytes; }
 
 int shdw_hip_asum(int n, const float* x, float* result_host, void* workspace,
                   size_t workspace_bytes, void* stream) {

@@ -6,6 +6,7 @@
 #include <cstring>
 
 #include "../../include/shadow_hip.h"
+#include "launch.h"
 
 namespace {
 inline int rc(hipError_t e) { return static_cast<int>(e); }
@@ -28,7 +29,13 @@ int shdw_hip_device_count(int* count) {
   return rc(hipGetDeviceCount(count));
 }
 
-int shdw_hip_set_device(int device_id) { return rc(hipSetDevice(device_id)); }
+int shdw_hip_set_device(int device_id) {
+  const hipError_t e = hipSetDevice(device_id);
+  if (e != hipSuccess) return rc(e);
+  // the library's own device memory is looked up here, once per device, so that
+  // no later call has to do it at a time when it cannot (a stream being captured)
+  return shdw::library_scratch_prepare();
+}
 
 int shdw_hip_device_info(int device_id, char* buf, size_t buf_size) {
   if (!buf || buf_size == 0) return SHDW_E_INVALID_ARGUMENT;
@@ -61,6 +68,9 @@ const char* shdw_hip_error_string(int code) {
     case SHDW_E_INVALID_ARGUMENT: return "shadow_hip: invalid argument";
     case SHDW_E_UNSUPPORTED: return "shadow_hip: unsupported shape";
     case SHDW_E_WORKSPACE: return "shadow_hip: workspace missing or too small";
+    case SHDW_E_STATIC_SCRATCH:
+      return "shadow_hip: this shape needs more scratch than the library's static buffer holds "
+             "(shdw_hip_reduce_static_max_workspace_bytes); use shdw_hip_reduce with a workspace";
     default: break;
   }
   if (code < 0) return "shadow_hip: unknown error";
