@@ -29,7 +29,7 @@ def lib():
     if _LIB is None:
         path = os.path.join(_HERE, "liboracle.so")
         if not os.path.exists(path):
-            raise RuntimeError("oracle/liboracle.so is not built; run `python -m shadow_amd.build oracle`")
+            raise RuntimeError("oracle/liboracle.so is not built; run `python -m oracle.build`")
         _LIB = ctypes.CDLL(path)
         _LIB.orc_asum.restype = ctypes.c_float
     return _LIB

@@ -1,13 +1,15 @@
-"""Build every native piece of the repository in-tree.
+"""Build the two product libraries in-tree.
 
-    python -m shadow_amd.build            # everything
-    python -m shadow_amd.build hip host   # selected targets
+    python -m shadow_amd.build            # both
+    python -m shadow_amd.build hip        # selected targets
 
 Targets
     hip     shadow_amd/lib/libshadow_hip.so   gfx950 kernels + C ABI (hipcc)
     host    shadow_amd/lib/libshadow_host.so  C++ operator layer over the C ABI (g++)
-    oracle  oracle/liboracle.so               CPU restatement of the reference (gcc)
-    sweep   tests/native/libm_sweep.so        host build of the device libm code (g++)
+
+The test-side libraries have their own recipes: `python -m oracle.build` (the
+CPU restatement of the reference) and `python -m tests.native.build` (the host
+build of the device math code).
 
 hipcc cross-compiles for gfx950 without a GPU.  The device code must keep
 multiply and add separate (the reference never fuses), hence -ffp-contract=off;
@@ -33,10 +35,6 @@ HIP_FLAGS = [
 ]
 HIP_SOURCES = ["elementwise.hip", "broadcast.hip", "reduce.hip", "fused.hip", "vision.hip", "softmax.hip", "norm.hip", "movers.hip",
                "runtime.hip"]
-# The reference's Release flags (CMakeLists.txt:30-37) plus contraction off so
-# that no host can fuse what baseline x86-64 does not.
-ORACLE_FLAGS = ["-O3", "-DNDEBUG", "-fPIC", "-ffp-contract=off", "-fno-fast-math"]
-
 
 def _run(cmd):
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -77,26 +75,12 @@ def build_host():
     return out
 
 
-def build_oracle():
-    src = os.path.join(ROOT, "oracle", "shadow_cpu.c")
-    out = os.path.join(ROOT, "oracle", "liboracle.so")
-    _run(["gcc", "-std=c11"] + ORACLE_FLAGS + ["-shared", src, "-lm", "-o", out])
-    return out
-
-
-def build_sweep():
-    src = os.path.join(ROOT, "tests", "native", "libm_sweep.cpp")
-    out = os.path.join(ROOT, "tests", "native", "libm_sweep.so")
-    _run(["g++", "-std=c++17", "-O2", "-ffp-contract=off", "-fPIC", "-shared", "-pthread", src, "-o", out])
-    return out
-
-
-TARGETS = {"hip": build_hip, "host": build_host, "oracle": build_oracle, "sweep": build_sweep}
+TARGETS = {"hip": build_hip, "host": build_host}
 
 
 def build_all(names=None):
     built = []
-    for name in (names or ["hip", "host", "oracle", "sweep"]):
+    for name in (names or ["hip", "host"]):
         path = TARGETS[name]()
         if path:
             built.append(path)
