@@ -61,7 +61,7 @@ struct BMin { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab
 // ---- activations: shadow/operators/kernels/activate.cpp:9-31 ----
 struct ARelu { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return x > 0 ? x : 0; } };
 struct ALeaky { SHDW_DEVICE float operator()(float x, float s, const uint64_t* tab) const { return x > 0 ? x : s * x; } };
-struct ASigmoid { static constexpr bool kExpTable = true; static constexpr int kVectorsPerLane = 2; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_sigmoidf(x, tab); } };
+struct ASigmoid { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_sigmoidf(x, tab); } };
 struct ASoftPlus { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_softplusf(x, tab); } };
 struct ATanh { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_tanhf(x); } };
 struct ARelu6 { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return x < 0 ? 0 : (x > 6 ? 6 : x); } };

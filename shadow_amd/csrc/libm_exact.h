@@ -72,10 +72,13 @@ SHDW_LIBM_TABLE uint64_t kExp2fTab[32] = {
 
 // `tab` is kExp2fTab or a copy of it in faster memory (the kernels stage it in
 // LDS so that the lookup does not queue behind the streaming HBM traffic).
-SHDW_LIBM_FN float exact_expf(float x, const uint64_t* tab) {
-  // Main path, evaluated for every input (its result is discarded for the
-  // out-of-range inputs handled below; nothing in it can trap, and the table
-  // index is masked).
+//
+// The library's main path.  By itself it is the whole function for
+// -0x1.9fe368p6 <= x <= 0x1.62e42ep6 (where the conversion at the end rounds to
+// a subnormal or to 2^-149 exactly as the library's own cases do) and for NaN;
+// outside, the table scale may wrap, so the result must be replaced.  Nothing in
+// it can trap and the table index is masked.
+SHDW_LIBM_FN float expf_main(float x, const uint64_t* tab) {
   const double InvLn2N = 0x1.71547652b82fep+5;  // 32 / ln 2
   const double Shift = 0x1.8p+52;
   const double xd = static_cast<double>(x);
@@ -92,11 +95,13 @@ SHDW_LIBM_FN float exact_expf(float x, const uint64_t* tab) {
   double y = __builtin_fma(c2, r, 1.0);
   y = __builtin_fma(p, r2, y);
   y = y * s;
-  float res = static_cast<float>(y);
+  return static_cast<float>(y);
+}
 
+SHDW_LIBM_FN float exact_expf(float x, const uint64_t* tab) {
+  float res = expf_main(x, tab);
   // Out of range: both comparisons are false for NaN, which the main path has
-  // already propagated.  Between the two bounds the conversion above rounds to
-  // +inf, to a subnormal or to 2^-149 exactly as the library's own cases do.
+  // already propagated.
   res = (x > 0x1.62e42ep6f) ? __builtin_inff() : res;  // overflow (and +inf)
   res = (x < -0x1.9fe368p6f) ? 0.0f : res;             // underflow to zero (and -inf)
   return res;
@@ -186,24 +191,33 @@ SHDW_LIBM_FN float exact_expm1f(float x) {
 // k = 0, k = -1, k <= -2 (a < 0) and k >= 3 (a > 0) can occur; each is evaluated
 // with the library's operations in the library's order and the applicable one is
 // selected.  Where a cheaper form gives the same bits on every input it replaces
-// the library's:
+// the library's.  Exact rewrites (they change no rounding):
+//   * hxs = x * (0.5 x) is half of s = x * x, and a halving commutes with every
+//     rounding here, so 0.5 * round(s * p) stands for the library's round(hxs * p)
+//     and "v - hxs" is one fused -0.5 * s + v; hfx and hxs are never formed;
+//   * fused operations where the product is exact (a - k * ln2_hi, 0.5 * v - 0.5);
+//   * k = 0 has lo = 0 and therefore c = 0, which makes the library's special
+//     form x - (x * e - hxs) equal to x - e with the general e = x * (e - c) - c
+//     - hxs; k = -1 is 0.5 * (x - e) - 0.5 on the same difference d = x - e, and
+//     the general y = (1 - 2^-k) - (e - x) is (1 - 2^-k) + d.
+// Rewrites that do change intermediate roundings, kept because the function
+// still returns the library's bits for all 2^32 inputs with them (compared on
+// the host and on the device; none of it is argued from error bounds):
 //   * k = rint(a / ln2), taken from one fused multiply-add with 1.5 * 2^23,
 //     instead of the truncation of a / ln2 -+ 0.5 and of the separate
 //     |a| < 0.5 ln2 and |a| < 1.5 ln2 cases (k = 0, k = +-1 there too);
-//   * fused operations where the product is exact and the fusion therefore
-//     changes nothing (a - k * ln2_hi, 0.5 * v - 0.5);
-//   * hi - lo and the correction term c are taken for k = 0 as well (lo = 0
-//     makes them x and 0);
-//   * y = (1 - 2^-k) - (e - x) also for 23 <= k, where the library switches to
+//   * the four innermost steps of the degree-5 polynomial are fused
+//     multiply-adds (their rounding differences are attenuated by the steps that
+//     follow; fusing the outermost one as well differs on 70 inputs, fusing the
+//     products of t3, of the divisor or of e on thousands);
+//   * y = (1 - 2^-k) + d also for 23 <= k, where the library switches to
 //     (x - (e + 2^-k)) + 1: the two differ far below what 1 - 2 / (t + 2) keeps;
 //   * |x| >= 10 is evaluated at 10 (the result is already exactly 1 there;
 //     the library's own cut is at 22), which also bounds k by 29;
 //   * the |x| < 2^-55 and |a| < 2^-25 early returns are left to the general
 //     path, which returns x there as well.
-// None of this is argued from error bounds: the function is compared with the
-// library on all 2^32 inputs, on the host and on the device.
 SHDW_LIBM_FN float exact_tanhf(float x) {
-  const float one = 1.0f, two = 2.0f;
+  const float one = 1.0f, two = 2.0f, half = 0.5f;
   const float ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f;
   const float invln2 = 1.4426950216e+00f;
   const float Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f,
@@ -231,52 +245,60 @@ SHDW_LIBM_FN float exact_tanhf(float x) {
   const float c = (hi - xr) - lo;
 
   // --- primary range ---
-  const float hfx = 0.5f * xr;
-  const float hxs = xr * hfx;
-  const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
-  const float t3 = 3.0f - r1 * hfx;
-  // numerator ~ -2, denominator in [4.9, 7.1]
-  float e = hxs * div_normal(r1 - t3, 6.0f - xr * t3);
-  const float res_k0 = xr - (xr * e - hxs);
-  e = (xr * (e - c) - c);
-  e -= hxs;
-  const float res_km1 = __builtin_fmaf(0.5f, xr - e, -0.5f);  // the halving is exact: same as 0.5f * (xr - e) - 0.5f
-  // k >= 3: y = (1 - 2^-k) - (e - x), result y * 2^k.  k <= -2: y = 1 - (e - x),
-  // result y * 2^k - 1; the shift count k & 31 is then 29 or more and leaves 1.
+  const float s = xr * xr;  // 2 hxs
+  // r1 = 1 + hxs (Q1 + hxs (Q2 + hxs (Q3 + hxs (Q4 + hxs Q5)))); the first fused
+  // step produces half of its value so that the next one needs no 0.5
+  float p = __builtin_fmaf(s, Q5 * 0.25f, Q4 * half);  // (Q4 + hxs Q5) / 2
+  p = __builtin_fmaf(s, p, Q3);
+  p = __builtin_fmaf(s, half * p, Q2);
+  p = __builtin_fmaf(s, half * p, Q1);
+  const float r1 = __builtin_fmaf(half, s * p, one);
+  const float t3 = __builtin_fmaf(-half, r1 * xr, 3.0f);  // 3 - r1 * hfx
+  // numerator ~ -2, denominator in [4.9, 7.1]; twice the library's e = hxs * (...)
+  const float e2x = s * div_normal(r1 - t3, 6.0f - xr * t3);
+  float e = xr * __builtin_fmaf(half, e2x, -c) - c;  // x * (e - c) - c
+  e = __builtin_fmaf(-half, s, e);                   // - hxs
+  const float d = xr - e;                            // the k = 0 result
+  const float res_km1 = __builtin_fmaf(half, d, -half);
+  // k >= 3: y = (1 - 2^-k) + d, result y * 2^k.  k <= -2: y = 1 + d, result
+  // y * 2^k - 1; the shift count k & 31 is then 29 or more and leaves 1.
   const float t_lo = u2f(0x3f800000u - (0x1000000u >> (kbits & 31u)));
-  float yk = t_lo - (e - xr);
+  float yk = t_lo + d;
   yk = u2f(f2u(yk) + (kbits << 23));  // scale by 2^k
   const float res_gen = big ? yk : yk - one;
-  const float t = (tk == 0.0f) ? res_k0 : ((tk == -1.0f) ? res_km1 : res_gen);
+  const float t = (tk == 0.0f) ? d : ((tk == -1.0f) ? res_km1 : res_gen);
 
   // --- tanhf ---
   const float q = div_normal(big ? two : t, t + two);
   // |x| >= 1: 1 - 2 / (t + 2); else -t / (t + 2), whose magnitude is |q|.
-  // The result takes x's sign.
   const float z = big ? one - q : q;
-  float res = u2f((f2u(z) & 0x7fffffffu) | (jx & 0x80000000u));
-  res = (ix > 0x7f800000u) ? x + x : res;  // NaN
-  return res;
+  // The result takes x's sign; a NaN keeps all of its bits.
+  const uint32_t keep = (ix > 0x7f800000u) ? 0u : 0x7fffffffu;
+  return u2f((f2u(z) & keep) | (jx & ~keep));
 }
 
 // 1 / (1 + exp(-x)) in fp32, the way shadow/operators/kernels/activate.cpp:16
 // writes it.
 SHDW_LIBM_FN float exact_sigmoidf(float x, const uint64_t* tab) {
-  const float d = 1.0f + exact_expf(-x, tab);
 #if defined(__HIP_DEVICE_COMPILE__)
-  // d >= 1.  While d < 2^126 the quotient is a normal number and the hardware
-  // reciprocal plus one correction from the exact remainder 1 - d * r is the
-  // correctly rounded 1 / d for every d this function can produce (all 2^32
-  // inputs compared with the full division on the device); from 2^126 on
-  // (x < -87.3) the quotient is subnormal and only the full division is right.
-  // The wave takes the short form when none of its lanes is in that range.
-  if (__builtin_amdgcn_ballot_w64(!(d < 0x1p126f)) == 0) {
+  // |x| < 87: exp(-x) lies in (2^-126, 2^126), so expf's main path is the whole
+  // function, d = 1 + exp(-x) is in [1, 2^126) and the quotient is a normal
+  // number; the hardware reciprocal plus one correction from the exact remainder
+  // 1 - d * r is then the correctly rounded 1 / d for every d this function can
+  // produce (all 2^32 inputs compared with the full form on the device).  The
+  // wave takes this short form when all of its lanes are in that range; a NaN,
+  // an infinity or a large |x| anywhere in the wave sends it through the full
+  // form below (from 2^126 on, x < -87.3, the quotient is subnormal and only the
+  // full division is right).
+  const bool plain = __builtin_fabsf(x) < 87.0f;
+  if (__builtin_amdgcn_ballot_w64(!plain) == 0) {
+    const float d = 1.0f + expf_main(-x, tab);
     const float r = __builtin_amdgcn_rcpf(d);
     const float e = __builtin_fmaf(-d, r, 1.0f);
     return __builtin_fmaf(e, r, r);
   }
 #endif
-  return 1.0f / d;
+  return 1.0f / (1.0f + exact_expf(-x, tab));
 }
 #if !defined(__HIPCC__)
 SHDW_LIBM_FN float exact_expf(float x) { return exact_expf(x, kExp2fTab); }
