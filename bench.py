@@ -6,22 +6,29 @@
 A "step" is one pass of the headline workload (BASELINE.json configs[1]): seven
 launches over an fp32 [64,256,56,56] tensor -- Activate relu, sigmoid, tanh;
 Unary exp, abs, sqrt(abs); Scale(per-channel gamma, beta)+ReLU in one launch.
-Inputs are generated from fixed seeds, uploaded once and stay resident in HBM;
-the timed region is K steps between two stream synchronisations.
+Inputs are generated from fixed seeds, uploaded once and stay resident in HBM
+(two copies of the input take turns, 411 MB, more than the 256 MB Infinity
+Cache); the timed region is K steps between two stream synchronisations.
 
 Prints ONE JSON line.  `value` is algorithmic GB/s of the whole step
 (compulsory reads + writes of every op / wall time).  `roofline` describes the
 kernel that takes the largest share of the step, timed with HIP events on the
-launch stream inside the timed region.  `cpu_baseline` is the CPU oracle (a C
-port of the reference's loops, one thread) timed on this host on the same
-buffers.  `configs` lists every op of the five BASELINE workloads measured the
-same way (events around batches of launches that rotate over >256 MB of
-buffers), so that each can be held against the 8 TB/s HBM roofline.
+launch stream inside the timed region; its `bound` is "hbm" unless the kernel
+takes over 10 % longer than a plain copy of the same tensor measured in the same
+run, in which case it is "valu" and carries the instruction counters of the
+profile summary.  `cpu_baseline` is the CPU oracle (a C port of the reference's
+loops, one thread) timed on this host on the same buffers, outputs allocated
+beforehand.  `configs` lists every op of the five BASELINE workloads measured
+the same way (events around batches of launches that rotate over >256 MB of
+buffers), each with the time of a plain copy / read / write of the same number
+of bytes (`ceiling_us`, whichever matches the op's traffic) and, for the
+BASELINE rows, the oracle's time on this host.
 """
 import argparse
 import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -32,16 +39,43 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
-# HBM bytes per launch of the headline kernels, from the FETCH_SIZE / WRITE_SIZE
-# counters of `rocprofv3 --pmc` runs of `bench.py --probe`, each scaled by what
-# the same counter reads for a plain copy of known size (the summary with the
-# raw readings and the factors is profiles/headline_unary_chain_hbm_counters.txt).
-# They cannot be collected from inside this process, so they are recorded here.
-MEASURED_TRAFFIC_BYTES = {
-    "activate_relu": 411.04e6, "activate_sigmoid": 411.06e6, "unary_exp": 411.01e6,
-    "unary_abs": 411.04e6, "unary_sqrt_of_abs": 411.00e6, "activate_tanh": 411.02e6,
-    "scale_relu_fused": 411.02e6,
-}
+# rocprofv3 summaries that `roofline` quotes (counters cannot be collected from
+# inside this process): HBM bytes per launch of the headline kernels from
+# FETCH_SIZE / WRITE_SIZE, and their VALU instruction counters.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "headline_unary_chain_hbm_counters.txt")
+VALU_PROFILE = os.path.join(ROOT, "profiles", "headline_unary_chain_valu_counters.txt")
+PROFILE_LABEL = {"activate_relu": "Activate relu", "activate_sigmoid": "Activate sigmoid",
+                 "unary_exp": "Unary exp", "unary_abs": "Unary abs", "unary_sqrt_of_abs": "Unary sqrt",
+                 "activate_tanh": "Activate tanh", "scale_relu_fused": "Scale+ReLU fused"}
+
+
+def profile_rows(path):
+    """{workload label: [columns...]} of a profiles/ table (columns two or more blanks apart)."""
+    rows = {}
+    if os.path.exists(path):
+        for line in open(path):
+            cols = re.split(r"\s{2,}", line.strip())
+            if len(cols) >= 4:
+                rows[cols[0]] = cols[1:]
+    return rows
+
+
+def measured_traffic(op):
+    """HBM bytes per launch (reads + writes) from the counter summary, or None."""
+    cols = profile_rows(TRAFFIC_PROFILE).get(PROFILE_LABEL.get(op, ""))
+    try:
+        return round((float(cols[3]) + float(cols[5])) * 1e6)  # read MB, write MB
+    except (TypeError, IndexError, ValueError):
+        return None
+
+
+def measured_valu(op):
+    """{"insts_per_element", "valu_busy"} from the VALU counter summary, or None."""
+    cols = profile_rows(VALU_PROFILE).get(PROFILE_LABEL.get(op, ""))
+    try:
+        return {"insts_per_element": float(cols[-2]), "valu_busy": float(cols[-1])}
+    except (TypeError, IndexError, ValueError):
+        return None
 
 
 def parse():
@@ -49,11 +83,13 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-configs", action="store_true", help="skip the per-config table")
-    ap.add_argument("--cpu-passes", type=int, default=10)
+    ap.add_argument("--cpu-passes", type=int, default=5)
     ap.add_argument("--operand-sets", type=int, default=1,
                     help="multiplier on the number of rotating operand sets of the config table")
+    ap.add_argument("--single-input", action="store_true",
+                    help="headline step on one input instead of two taking turns (A/B of the cache effect)")
     ap.add_argument("--probe", action="store_true",
                     help="counter probe: 3 launches of a plain copy and of every headline op on "
                          "the 51.4M tensor, nothing timed, no JSON (run under rocprofv3 --pmc)")
@@ -116,37 +152,40 @@ class Dev:
 
 
 # ------------------------------------------------------------------ headline
-def headline(dev, steps, warmup):
+def headline(dev, steps, warmup, single_input=False):
     lib, st = dev.lib, dev.stream
     shape = (64, 256, 56, 56)
     n = int(np.prod(shape))
     C, inner = shape[1], shape[2] * shape[3]
     x_h = normal(201, n, 2.0)
     g_h, b_h = uniform(202, C, 0.5, 1.5), uniform(203, C, -0.1, 0.1)
-    x, g, b = dev.buf(x_h), dev.buf(g_h), dev.buf(b_h)
+    g, b = dev.buf(g_h), dev.buf(b_h)
+    # two resident copies of the input take turns step by step
+    xs = [dev.buf(x_h)] if single_input else [dev.buf(x_h), dev.buf(x_h)]
     y = [dev.buf(nbytes=4 * n) for _ in range(2)]
     a = dev.buf(nbytes=4 * n)  # abs output, input of sqrt
 
     per_op = 8 * n
     ops = [
-        ("activate_relu", per_op, lambda o: lib.shdw_hip_activate(1, 0.1, n, x.ptr, o.ptr, st)),
-        ("activate_sigmoid", per_op, lambda o: lib.shdw_hip_activate(3, 0.1, n, x.ptr, o.ptr, st)),
-        ("unary_exp", per_op, lambda o: lib.shdw_hip_unary(4, n, x.ptr, o.ptr, st)),
-        ("unary_abs", per_op, lambda o: lib.shdw_hip_unary(0, n, x.ptr, a.ptr, st)),
-        ("unary_sqrt_of_abs", per_op, lambda o: lib.shdw_hip_unary(2, n, a.ptr, o.ptr, st)),
-        ("activate_tanh", per_op, lambda o: lib.shdw_hip_activate(5, 0.1, n, x.ptr, o.ptr, st)),
+        ("activate_relu", per_op, lambda x, o: lib.shdw_hip_activate(1, 0.1, n, x.ptr, o.ptr, st)),
+        ("activate_sigmoid", per_op, lambda x, o: lib.shdw_hip_activate(3, 0.1, n, x.ptr, o.ptr, st)),
+        ("unary_exp", per_op, lambda x, o: lib.shdw_hip_unary(4, n, x.ptr, o.ptr, st)),
+        ("unary_abs", per_op, lambda x, o: lib.shdw_hip_unary(0, n, x.ptr, a.ptr, st)),
+        ("unary_sqrt_of_abs", per_op, lambda x, o: lib.shdw_hip_unary(2, n, a.ptr, o.ptr, st)),
+        ("activate_tanh", per_op, lambda x, o: lib.shdw_hip_activate(5, 0.1, n, x.ptr, o.ptr, st)),
         ("scale_relu_fused", per_op + 8 * C,
-         lambda o: lib.shdw_hip_scale_bias(n, C, inner, x.ptr, g.ptr, b.ptr, 1, o.ptr, st)),
+         lambda x, o: lib.shdw_hip_scale_bias(n, C, inner, x.ptr, g.ptr, b.ptr, 1, o.ptr, st)),
     ]
     step_bytes = sum(nb for _, nb, _ in ops)
 
     def step(i, events=None, only=None):
         """events: one (start, stop) pair per op; only: record just around that op."""
+        x = xs[i % len(xs)]
         for k, (_, _, fn) in enumerate(ops):
             marked = events is not None and (only is None or only == k)
             if marked:
                 dev.record(events[k][0])
-            dev.ck(fn(y[(i + k) & 1]))
+            dev.ck(fn(x, y[(i + k) & 1]))
             if marked:
                 dev.record(events[k][1])
 
@@ -156,19 +195,28 @@ def headline(dev, steps, warmup):
 
     # Untimed pass with events around every launch: the per-op table, and which
     # kernel dominates.  Event records between launches cost ~2.5 us each, so the
-    # timed region below carries them around the dominant kernel only.
+    # timed region below carries them around the dominant kernel only.  A plain
+    # copy of the same tensor, bracketed the same way, rides along as the yardstick.
     ev = [[(dev.event(), dev.event()) for _ in ops] for _ in range(steps)]
+    cev = [(dev.event(), dev.event()) for _ in range(steps)]
     for i in range(steps):
         step(i, ev[i])
+        dev.record(cev[i][0])
+        dev.ck(lib.shdw_hip_copy(n, xs[i % len(xs)].ptr, y[i & 1].ptr, st))
+        dev.record(cev[i][1])
     dev.sync()
     kernel_ms = []
     for k in range(len(ops)):
         kernel_ms.append(sum(dev.elapsed_ms(ev[i][k][0], ev[i][k][1]) for i in range(steps)) / steps)
+    copy_ms = sum(dev.elapsed_ms(c0, c1) for c0, c1 in cev) / steps
     detail = []
     for (name, nb, _), ms in zip(ops, kernel_ms):
         gbs = nb / (ms * 1e-3) / 1e9
         detail.append({"op": name, "bytes": nb, "us": round(ms * 1e3, 2), "GBps": round(gbs, 1),
-                       "frac": round(gbs / HBM_PEAK_GBS, 4)})
+                       "frac": round(gbs / HBM_PEAK_GBS, 4), "vs_copy": round(ms / copy_ms, 3)})
+    detail.append({"op": "plain_copy (yardstick, not part of the step)", "bytes": per_op,
+                   "us": round(copy_ms * 1e3, 2), "GBps": round(per_op / (copy_ms * 1e-3) / 1e9, 1),
+                   "frac": round(per_op / (copy_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "vs_copy": 1.0})
     dom = int(np.argmax(kernel_ms))
 
     t0 = time.perf_counter()
@@ -177,13 +225,23 @@ def headline(dev, steps, warmup):
     dev.sync()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / steps
+    vs_copy = kernel_ms[dom] / copy_ms  # both from the pass that brackets every launch
     kernel_ms[dom] = sum(dev.elapsed_ms(ev[i][dom][0], ev[i][dom][1]) for i in range(steps)) / steps
     dom_gbs = ops[dom][1] / (kernel_ms[dom] * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": ops[dom][0], "achieved": round(dom_gbs, 1),
+    name = ops[dom][0]
+    roofline = {"bound": "valu" if vs_copy > 1.10 else "hbm", "kernel": name, "achieved": round(dom_gbs, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get(ops[dom][0]), "avg_us": round(kernel_ms[dom] * 1e3, 2),
-                "algorithmic_bytes": ops[dom][1]}
+                "traffic": measured_traffic(name), "traffic_source": os.path.relpath(TRAFFIC_PROFILE, ROOT),
+                "avg_us": round(kernel_ms[dom] * 1e3, 2), "algorithmic_bytes": ops[dom][1],
+                "same_size_copy_us": round(copy_ms * 1e3, 2), "time_vs_same_size_copy": round(vs_copy, 3)}
+    if roofline["bound"] == "valu":
+        roofline["valu"] = measured_valu(name)
+        roofline["valu_source"] = os.path.relpath(VALU_PROFILE, ROOT)
+        roofline["note"] = ("achieved/peak/frac stay in HBM terms (algorithmic bytes / kernel time against 8 TB/s); "
+                            "the kernel is held back by vector-ALU issue, not by memory")
     host = {"x": x_h, "gamma": g_h, "beta": b_h, "shape": shape}
+    for bb in xs + y + [a, g, b]:
+        bb.free()
     return ms_per_step, step_bytes, n, roofline, detail, host
 
 
@@ -249,31 +307,114 @@ def probe_next(dev):
     dev.sync()
 
 
-def cpu_baseline(host, step_bytes, passes):
-    """The oracle on this host, one thread: the same seven results, with
-    Scale and ReLU as the two separate operators the reference runs."""
-    import oracle
+# ------------------------------------------------------------- CPU baseline
+class Cpu:
+    """The oracle's C functions called directly on arrays allocated beforehand, so
+    that only the operator's work is timed (the reference's blobs are grow-only
+    and resident), one thread.  best / median of `runs` calls."""
+
+    def __init__(self, runs):
+        import oracle
+        self.o = oracle
+        self.lib = oracle.lib()
+        self.runs = runs
+        self.f32p = ctypes.POINTER(ctypes.c_float)
+
+    def p(self, a):
+        return a.ctypes.data_as(self.f32p)
+
+    def ints(self, v):
+        return (ctypes.c_int * max(1, len(v)))(*[int(x) for x in v])
+
+    def time(self, fn):
+        fn()  # pages of the outputs are touched before anything is timed
+        ts = []
+        for _ in range(self.runs):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        ts.sort()
+        return ts[0], ts[len(ts) // 2]
+
+    # --- the operator bodies (reference lines in oracle/shadow_cpu.c) ---
+    def activate(self, x, y, kind):
+        return lambda: self.lib.orc_activate(self.p(x), self.p(y), x.size, kind, ctypes.c_float(0.1))
+
+    def unary(self, x, y, op):
+        return lambda: self.lib.orc_unary(op, x.size, self.p(x), self.p(y))
+
+    def scale_bias(self, x, g, b, num, inner, y):
+        return lambda: self.lib.orc_scale_bias(self.p(x), x.size, self.p(g), self.p(b), num, inner, self.p(y))
+
+    def broadcast(self, op, a, sa, b, sb, so, y):
+        return lambda: self.lib.orc_broadcast_binary(self.p(a), self.ints(sa), self.p(b), self.ints(sb), op,
+                                                     len(so), y.size, self.ints(so), self.p(y))
+
+    def binary_scalar(self, op, a, alpha, y):
+        return lambda: self.lib.orc_binary_scalar(op, a.size, self.p(a), ctypes.c_float(alpha), self.p(y))
+
+    def eltwise_sum(self, xs, y):
+        ptrs = (self.f32p * len(xs))(*[self.p(x) for x in xs])
+        co = np.ones(len(xs), np.float32)
+        return lambda: self.lib.orc_eltwise(1, len(xs), ptrs, self.p(co), y.size, self.p(y))
+
+    def reduce(self, op, x, shape, axes, y):
+        """Vision::Reduce on index lists built beforehand: the reference keeps them
+        while the input shape is unchanged (kernels/reduce.hpp:45)."""
+        window = int(np.prod([shape[a] for a in axes])) if axes else 1
+        lst, off = np.empty(window, np.int32), np.empty(y.size, np.int32)
+        i32p = ctypes.POINTER(ctypes.c_int)
+        num_list = self.lib.orc_reduce_lists(self.ints(shape), len(shape), self.ints(axes), len(axes),
+                                             lst.ctypes.data_as(i32p), off.ctypes.data_as(i32p))
+        assert num_list == window
+        keep = (lst, off)
+        return lambda: self.lib.orc_vision_reduce(self.p(x), keep[0].ctypes.data_as(i32p),
+                                                  keep[1].ctypes.data_as(i32p), num_list, op, y.size, self.p(y))
+
+
+def cpu_headline(cpu, host, step_bytes):
+    """The same seven results as the step, with Scale and ReLU as the two separate
+    operators the reference runs; per-op and whole-step times."""
     x, g, b = host["x"], host["gamma"], host["beta"]
     C, inner = host["shape"][1], host["shape"][2] * host["shape"][3]
-    oracle.lib()
-    best = None
-    for _ in range(passes):
-        t0 = time.perf_counter()
-        oracle.activate(x, 1)
-        oracle.activate(x, 3)
-        oracle.unary(4, x)
-        a = oracle.unary(0, x)
-        oracle.unary(2, a)
-        oracle.activate(x, 5)
-        s = oracle.scale_bias(x, g, b, C, inner)
-        oracle.activate(s, 1)
-        dt = time.perf_counter() - t0
-        best = dt if best is None else min(best, dt)
+    y, a = np.empty_like(x), np.empty_like(x)
+    legs = [("activate_relu", [cpu.activate(x, y, 1)]), ("activate_sigmoid", [cpu.activate(x, y, 3)]),
+            ("unary_exp", [cpu.unary(x, y, 4)]), ("unary_abs", [cpu.unary(x, a, 0)]),
+            ("unary_sqrt_of_abs", [cpu.unary(a, y, 2)]), ("activate_tanh", [cpu.activate(x, y, 5)]),
+            ("scale_relu_fused", [cpu.scale_bias(x, g, b, C, inner, y), cpu.activate(y, y, 1)])]
+    for _, fns in legs:
+        for fn in fns:
+            fn()
+    per_op = {name: [] for name, _ in legs}
+    totals = []
+    for _ in range(cpu.runs):
+        total = 0.0
+        for name, fns in legs:
+            t0 = time.perf_counter()
+            for fn in fns:
+                fn()
+            dt = time.perf_counter() - t0
+            per_op[name].append(dt)
+            total += dt
+        totals.append(total)
+    best = min(totals)
+    ops = {name: {"best_us": round(min(v) * 1e6, 1), "median_us": round(sorted(v)[len(v) // 2] * 1e6, 1)}
+           for name, v in per_op.items()}
     return {"value": round(step_bytes / best / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "%d full passes of the same step on the same buffers (51.4M elements, 8 "
-                      "operator runs each), best pass %.2f s; host has %d logical CPUs" % (
-                          passes, best, os.cpu_count() or 0),
-            "seconds_per_step": round(best, 3)}
+            "sample": "%d full passes of the same step on the same buffers (51.4M elements, 8 operator runs "
+                      "each, outputs allocated beforehand), best pass %.2f s; host: %s, %d logical CPUs" % (
+                          cpu.runs, best, cpu_model(), os.cpu_count() or 0),
+            "seconds_per_step": round(best, 3), "ops": ops}
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown CPU"
 
 
 # ------------------------------------------------------------- config table
@@ -291,32 +432,98 @@ def time_batch(dev, launch, sets, reps=40, warm=5):
     return dev.elapsed_ms(e0, e1) / reps
 
 
-def config_table(dev, sets_scale=1):
+def time_median(dev, launch, sets, reps=40):
+    """Median of three batches."""
+    return sorted(time_batch(dev, launch, sets, reps) for _ in range(3))[1]
+
+
+class Ceilings:
+    """Plain copy / read-only / write-only passes over a given number of bytes, in the
+    launch shape of the elementwise kernels, rotating through 1.2 GB pools."""
+    POOL = 6 * 205520896
+
+    def __init__(self, dev):
+        self.dev = dev
+        self.rp, self.wp = dev.buf(nbytes=self.POOL), dev.buf(nbytes=self.POOL)
+        seed = dev.buf(normal(999, 12845056))
+        piece = 4 * 12845056
+        for k in range(self.POOL // piece):
+            dev.ck(dev.lib.shdw_hip_memcpy_d2d(self.rp.ptr + k * piece, seed.ptr, piece, dev.stream))
+        dev.sync()
+        seed.free()
+        self.sink = dev.buf(nbytes=256)
+        self.cache = {}
+
+    def us(self, kind, nbytes):
+        key = (kind, nbytes)
+        if key in self.cache:
+            return self.cache[key]
+        dev, lib, st = self.dev, self.dev.lib, self.dev.stream
+        per_side = nbytes // 2 if kind == "copy" else nbytes
+        n = max(4, per_side // 4)
+        m = max(1, min(64, self.POOL // (4 * n)))
+        rp, wp, sink = self.rp.ptr, self.wp.ptr, self.sink.ptr
+        if kind == "copy":
+            fn = lambda k: lib.shdw_hip_copy(n, rp + k * 4 * n, wp + k * 4 * n, st)
+        elif kind == "read":
+            fn = lambda k: lib.shdw_hip_probe_read(n, rp + k * 4 * n, 1e30, sink, st)
+        else:
+            fn = lambda k: lib.shdw_hip_set(n, 1.0, wp + k * 4 * n, st)
+        self.cache[key] = time_median(dev, fn, m) * 1e3
+        return self.cache[key]
+
+    def free(self):
+        for b in (self.rp, self.wp, self.sink):
+            b.free()
+
+
+def traffic_kind(read_bytes, write_bytes):
+    if read_bytes >= 4 * write_bytes:
+        return "read"
+    if write_bytes >= 4 * read_bytes:
+        return "write"
+    return "copy"
+
+
+def config_table(dev, sets_scale=1, cpu=None):
     lib, st = dev.lib, dev.stream
     I = dev.sa.ints
     rows = []
+    ceil = Ceilings(dev)
 
-    def add(cfg, name, nbytes, ms, elems):
+    def add(cfg, name, rd, wr, ms, elems, cpu_fn=None):
+        nbytes = rd + wr
         gbs = nbytes / (ms * 1e-3) / 1e9
-        rows.append({"cfg": cfg, "op": name, "bytes": nbytes, "us": round(ms * 1e3, 2),
-                     "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "Gelem_s": round(elems / (ms * 1e-3) / 1e9, 2)})
+        kind = traffic_kind(rd, wr)
+        cus = ceil.us(kind, nbytes)
+        row = {"cfg": cfg, "op": name, "bytes": nbytes, "us": round(ms * 1e3, 2),
+               "GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+               "Gelem_s": round(elems / (ms * 1e-3) / 1e9, 2),
+               "ceiling": kind, "ceiling_us": round(cus, 2), "frac_of_ceiling": round(cus / (ms * 1e3), 3)}
+        if cpu is not None and cpu_fn is not None:
+            best, med = cpu.time(cpu_fn)
+            row.update({"cpu_us": round(best * 1e6, 1), "cpu_median_us": round(med * 1e6, 1),
+                        "cpu_GBps": round(nbytes / best / 1e9, 3), "speedup_vs_cpu": round(best * 1e3 / ms, 1)})
+        rows.append(row)
 
     SETS = 6 * sets_scale  # 6 x (in + out) of 51 MB each: more than the 256 MB Infinity Cache
     NBIG = 12845056  # elements of the cfg-3 and cfg-5 tensors (51.4 MB)
     A = [dev.buf(normal(301 + 10 * k, NBIG)) for k in range(SETS)]
     Y = [dev.buf(nbytes=4 * NBIG) for _ in range(SETS)]
+    hx = normal(301, NBIG) if cpu else None   # host copy of the 51 MB tensor for the oracle
+    hy = np.empty(NBIG, np.float32) if cpu else None
 
     # cfg 1: Binary add with channel broadcast.  Its tensor is half of a set (25.7 MB):
     # both halves of every set take turns, 12 x 25.7 MB of inputs, so that no launch
-    # finds its input still in the 256 MB Infinity Cache (with six inputs, 154 MB,
-    # it did, and measured 8.7 us instead of 10.7).
+    # finds its input still in the 256 MB Infinity Cache.
     sa, sb = [8, 64, 112, 112], [1, 64, 1, 1]
     n = int(np.prod(sa))
-    B = dev.buf(uniform(102, 64, -1, 1))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_broadcast_binary(
+    hb = uniform(102, 64, -1, 1)
+    B = dev.buf(hb)
+    ms = time_median(dev, lambda k: lib.shdw_hip_broadcast_binary(
         0, 4, I(sa), I(sb), I(sa), A[k % SETS].ptr + (k // SETS) * 4 * n, B.ptr, Y[k % SETS].ptr, st), 2 * SETS)
-    add(1, "binary_add_channel_broadcast", 8 * n + 256, ms, n)
+    add(1, "binary_add_channel_broadcast", 4 * n + 256, 4 * n, ms, n,
+        cpu and cpu.broadcast(0, uniform(101, n, -1, 1), sa, hb, sb, sa, hy[:n]))
 
     # cfg 3: reductions over [32,512,28,28]
     shp = [32, 512, 28, 28]
@@ -324,79 +531,88 @@ def config_table(dev, sets_scale=1):
                                  ("reduce_max_c", 2, [1], 25088), ("reduce_sum_all", 1, [0, 1, 2, 3], 1)]:
         need = lib.shdw_hip_reduce_workspace_bytes(4, I(shp), len(axes), I(axes))
         ws = dev.buf(nbytes=max(need, 16))
-        ms = time_batch(dev, lambda k: lib.shdw_hip_reduce(op, 4, I(shp), len(axes), I(axes), A[k].ptr,
-                                                           Y[k].ptr, ws.ptr, need, st), SETS)
-        add(3, name, 4 * NBIG + 4 * outs, ms, NBIG)
+        ms = time_median(dev, lambda k: lib.shdw_hip_reduce(op, 4, I(shp), len(axes), I(axes), A[k].ptr,
+                                                            Y[k].ptr, ws.ptr, need, st), SETS)
+        add(3, name, 4 * NBIG, 4 * outs, ms, NBIG, cpu and cpu.reduce(op, hx, shp, axes, hy[:outs]))
+        ws.free()
 
     # cfg 5: ResNet bottleneck tail on [64,1024,14,14]
     n5, C5, in5 = 12845056, 1024, 196
-    g5, b5 = dev.buf(uniform(502, C5, 0.5, 1.5)), dev.buf(uniform(503, C5, -0.1, 0.1))
+    hg5, hb5 = uniform(502, C5, 0.5, 1.5), uniform(503, C5, -0.1, 0.1)
+    g5, b5 = dev.buf(hg5), dev.buf(hb5)
+    hr = normal(504, n5) if cpu else None
     M = [dev.buf(nbytes=4 * 65536) for _ in range(SETS)]
-    ms = time_batch(dev, lambda k: lib.shdw_hip_scale_bias(n5, C5, in5, A[k].ptr, g5.ptr, b5.ptr, 0,
-                                                           Y[k].ptr, st), SETS)
-    add(5, "scale", 8 * n5 + 8 * C5, ms, n5)
+    ms = time_median(dev, lambda k: lib.shdw_hip_scale_bias(n5, C5, in5, A[k].ptr, g5.ptr, b5.ptr, 0,
+                                                            Y[k].ptr, st), SETS)
+    add(5, "scale", 4 * n5 + 8 * C5, 4 * n5, ms, n5, cpu and cpu.scale_bias(hx, hg5, hb5, C5, in5, hy))
 
     def eltwise_sum(k):
         ptrs = (ctypes.c_void_p * 2)(A[k].ptr, A[(k + 1) % SETS].ptr)
         return lib.shdw_hip_eltwise(1, 2, ptrs, None, n5, Y[k].ptr, st)
-    ms = time_batch(dev, eltwise_sum, SETS)
-    add(5, "eltwise_sum", 12 * n5, ms, n5)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_activate(1, 0.1, n5, A[k].ptr, Y[k].ptr, st), SETS)
-    add(5, "relu", 8 * n5, ms, n5)
+    ms = time_median(dev, eltwise_sum, SETS)
+    add(5, "eltwise_sum", 8 * n5, 4 * n5, ms, n5, cpu and cpu.eltwise_sum([hx, hr], hy))
+    ms = time_median(dev, lambda k: lib.shdw_hip_activate(1, 0.1, n5, A[k].ptr, Y[k].ptr, st), SETS)
+    add(5, "relu", 4 * n5, 4 * n5, ms, n5, cpu and cpu.activate(hx, hy, 1))
     sh5, ax5 = [64, 1024, 14, 14], [2, 3]
-    ms = time_batch(dev, lambda k: lib.shdw_hip_reduce(4, 4, I(sh5), 2, I(ax5), A[k].ptr, M[k].ptr,
-                                                       None, 0, st), SETS)
-    add(5, "reduce_avg_hw", 4 * n5 + 4 * 65536, ms, n5)
+    ms = time_median(dev, lambda k: lib.shdw_hip_reduce(4, 4, I(sh5), 2, I(ax5), A[k].ptr, M[k].ptr,
+                                                        None, 0, st), SETS)
+    add(5, "reduce_avg_hw", 4 * n5, 4 * 65536, ms, n5, cpu and cpu.reduce(4, hx, sh5, ax5, hy[:65536]))
+    ms = time_median(dev, lambda k: lib.shdw_hip_scale_residual_relu_rowmean(
+        n5, C5, in5, A[k].ptr, g5.ptr, b5.ptr, A[(k + 1) % SETS].ptr, Y[k].ptr, M[k].ptr, st), SETS)
+    if cpu:
+        hs, hm = np.empty(n5, np.float32), np.empty(65536, np.float32)
+        chain = [cpu.scale_bias(hx, hg5, hb5, C5, in5, hs), cpu.eltwise_sum([hs, hr], hy), cpu.activate(hy, hy, 1),
+                 cpu.reduce(4, hy, sh5, ax5, hm)]
+        tail_cpu = lambda: [f() for f in chain]
+    add(5, "fused_tail (CPU: the four operators)", 8 * n5 + 8 * C5, 4 * n5 + 4 * 65536, ms, n5, cpu and tail_cpu)
+
     sh7 = [128, 2048, 7, 7]  # the same reduction over 7 x 7 planes: rows of 49 floats start on odd dwords
     M7 = [dev.buf(nbytes=4 * 128 * 2048) for _ in range(SETS)]
-    ms = time_batch(dev, lambda k: lib.shdw_hip_reduce(4, 4, I(sh7), 2, I(ax5), A[k].ptr, M7[k].ptr,
-                                                       None, 0, st), SETS)
-    add("next", "reduce_avg_hw 7x7 planes [128,2048,7,7]", 4 * n5 + 4 * 128 * 2048, ms, n5)
+    ms = time_median(dev, lambda k: lib.shdw_hip_reduce(4, 4, I(sh7), 2, I(ax5), A[k].ptr, M7[k].ptr,
+                                                        None, 0, st), SETS)
+    add("next", "reduce_avg_hw 7x7 planes [128,2048,7,7]", 4 * n5, 4 * 128 * 2048, ms, n5)
     # more of the same late-stage tensor, whose rows and planes are not multiples of four floats
     ws7 = dev.buf(nbytes=1 << 20)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_reduce(2, 4, I(sh7), 1, I([1]), A[k].ptr, M7[k].ptr,
-                                                       ws7.ptr, 1 << 20, st), SETS)
-    add("next", "reduce_max_c 7x7 maps [128,2048,7,7]", 4 * n5 + 4 * 128 * 49, ms, n5)
+    ms = time_median(dev, lambda k: lib.shdw_hip_reduce(2, 4, I(sh7), 1, I([1]), A[k].ptr, M7[k].ptr,
+                                                        ws7.ptr, 1 << 20, st), SETS)
+    add("next", "reduce_max_c 7x7 maps [128,2048,7,7]", 4 * n5, 4 * 128 * 49, ms, n5)
     g7, b7 = dev.buf(uniform(507, 2048, 0.5, 1.5)), dev.buf(uniform(508, 2048, -0.1, 0.1))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_group_norm(128 * 2048, 49, 1e-5, A[k].ptr, g7.ptr, b7.ptr,
-                                                           2048, 49, Y[k].ptr, st), SETS)
-    add("next", "instance_norm affine 7x7 planes [128,2048,7,7]", 8 * n5 + 8 * 2048, ms, n5)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_broadcast_binary(
+    ms = time_median(dev, lambda k: lib.shdw_hip_group_norm(128 * 2048, 49, 1e-5, A[k].ptr, g7.ptr, b7.ptr,
+                                                            2048, 49, Y[k].ptr, st), SETS)
+    add("next", "instance_norm affine 7x7 planes [128,2048,7,7]", 4 * n5 + 8 * 2048, 4 * n5, ms, n5)
+    ms = time_median(dev, lambda k: lib.shdw_hip_broadcast_binary(
         0, 4, I(sh7), I([1, 2048, 1, 1]), I(sh7), A[k].ptr, b7.ptr, Y[k].ptr, st), SETS)
-    add("next", "binary_add_channel_broadcast 7x7 maps [128,2048,7,7]", 8 * n5 + 4 * 2048, ms, n5)
+    add("next", "binary_add_channel_broadcast 7x7 maps [128,2048,7,7]", 4 * n5 + 4 * 2048, 4 * n5, ms, n5)
     for bb in M7 + [ws7, g7, b7]:
         bb.free()
-    ms = time_batch(dev, lambda k: lib.shdw_hip_scale_residual_relu_rowmean(
-        n5, C5, in5, A[k].ptr, g5.ptr, b5.ptr, A[(k + 1) % SETS].ptr, Y[k].ptr, M[k].ptr, st), SETS)
-    add(5, "fused_tail", 12 * n5 + 8 * C5 + 4 * 65536, ms, n5)
 
     # Operators next to the path (label "next").  Global pooling, Softmax and
     # Normalize run on the 51 MB sets; BatchNorm, Axpy and the stem max pooling
     # run further down on 205 MB tensors like the headline step.
     pin, pout = [16, 64, 112, 112], [16, 64, 56, 56]
     npo = int(np.prod(pout))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_pooling2d(I(pin), 0, 3, 3, 2, 2, 0, 0, I(pout), A[k].ptr,
-                                                          Y[k].ptr, st), SETS)
-    add("next", "pooling_max_3x3s2 [16,64,112,112]", 4 * (NBIG + npo), ms, NBIG)
+    ms = time_median(dev, lambda k: lib.shdw_hip_pooling2d(I(pin), 0, 3, 3, 2, 2, 0, 0, I(pout), A[k].ptr,
+                                                           Y[k].ptr, st), SETS)
+    add("next", "pooling_max_3x3s2 [16,64,112,112]", 4 * NBIG, 4 * npo, ms, NBIG)
     gin, gout = [128, 2048, 7, 7], [128, 2048, 1, 1]
-    ms = time_batch(dev, lambda k: lib.shdw_hip_pooling2d(I(gin), 1, 7, 7, 1, 1, 0, 0, I(gout), A[k].ptr,
-                                                          Y[k].ptr, st), SETS)
-    add("next", "pooling_global_avg_7x7", 4 * (NBIG + 128 * 2048), ms, NBIG)
+    ms = time_median(dev, lambda k: lib.shdw_hip_pooling2d(I(gin), 1, 7, 7, 1, 1, 0, 0, I(gout), A[k].ptr,
+                                                           Y[k].ptr, st), SETS)
+    add("next", "pooling_global_avg_7x7", 4 * NBIG, 4 * 128 * 2048, ms, NBIG)
     gin2, gout2 = [64, 1024, 14, 14], [64, 1024, 1, 1]
-    ms = time_batch(dev, lambda k: lib.shdw_hip_pooling2d(I(gin2), 1, 14, 14, 1, 1, 0, 0, I(gout2), A[k].ptr,
-                                                          Y[k].ptr, st), SETS)
-    add("next", "pooling_global_avg_14x14", 4 * (NBIG + 65536), ms, NBIG)
+    ms = time_median(dev, lambda k: lib.shdw_hip_pooling2d(I(gin2), 1, 14, 14, 1, 1, 0, 0, I(gout2), A[k].ptr,
+                                                           Y[k].ptr, st), SETS)
+    add("next", "pooling_global_avg_14x14", 4 * NBIG, 4 * 65536, ms, NBIG)
     # [16, 49, 128, 128]: channel softmax / L2 normalize of a dense map (inner = 16384)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_softmax(16, 49, 16384, A[k].ptr, Y[k].ptr, st), SETS)
-    add("next", "softmax_channels_dense", 8 * NBIG, ms, NBIG)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_normalize(16, 49, 16384, 2.0, 1e-12, A[k].ptr, Y[k].ptr, st),
-                    SETS)
-    add("next", "normalize_l2_channels_dense", 8 * NBIG, ms, NBIG)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_softmax(64, 1000, 1, A[k].ptr, Y[k].ptr, st), SETS)
-    add("next", "softmax_classifier_64x1000", 8 * 64000, ms, 64000)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_normalize(64, 512, 1, 2.0, 1e-12, A[k].ptr, Y[k].ptr, st), SETS)
-    add("next", "normalize_l2_embedding_64x512", 8 * 64 * 512, ms, 64 * 512)
-    for bset in (A, Y):
+    ms = time_median(dev, lambda k: lib.shdw_hip_softmax(16, 49, 16384, A[k].ptr, Y[k].ptr, st), SETS)
+    add("next", "softmax_channels_dense", 4 * NBIG, 4 * NBIG, ms, NBIG)
+    ms = time_median(dev, lambda k: lib.shdw_hip_normalize(16, 49, 16384, 2.0, 1e-12, A[k].ptr, Y[k].ptr, st),
+                     SETS)
+    add("next", "normalize_l2_channels_dense", 4 * NBIG, 4 * NBIG, ms, NBIG)
+    ms = time_median(dev, lambda k: lib.shdw_hip_softmax(64, 1000, 1, A[k].ptr, Y[k].ptr, st), SETS)
+    add("next", "softmax_classifier_64x1000", 4 * 64000, 4 * 64000, ms, 64000)
+    ms = time_median(dev, lambda k: lib.shdw_hip_normalize(64, 512, 1, 2.0, 1e-12, A[k].ptr, Y[k].ptr, st), SETS)
+    add("next", "normalize_l2_embedding_64x512", 4 * 64 * 512, 4 * 64 * 512, ms, 64 * 512)
+    for bset in (A, Y, M, [B, g5, b5]):
         for bb in bset:
             bb.free()
 
@@ -406,100 +622,98 @@ def config_table(dev, sets_scale=1):
     YH = [dev.buf(nbytes=4 * NH) for _ in range(SH)]
     CH, INH = 256, 3136
     meanh, varh = dev.buf(normal(611, CH)), dev.buf(uniform(612, CH, 0.5, 2.0))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_batch_norm(NH, CH, INH, AH[k].ptr, meanh.ptr, varh.ptr,
-                                                           1.0, 1e-5, YH[k].ptr, st), SH, reps=20)
-    add("next", "batch_norm [64,256,56,56]", 8 * NH + 8 * CH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_batch_norm(NH, CH, INH, AH[k].ptr, meanh.ptr, varh.ptr,
+                                                            1.0, 1e-5, YH[k].ptr, st), SH, reps=20)
+    add("next", "batch_norm [64,256,56,56]", 4 * NH + 8 * CH, 4 * NH, ms, NH)
     alh = dev.buf(uniform(613, 64 * CH, 0.0, 1.0))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_axpy_rows(64 * CH, INH, alh.ptr, AH[k].ptr,
-                                                          AH[(k + 1) % SH].ptr, YH[k].ptr, st), SH, reps=20)
-    add("next", "axpy_rows [64,256,56,56]", 12 * NH + 4 * 64 * CH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_axpy_rows(64 * CH, INH, alh.ptr, AH[k].ptr,
+                                                           AH[(k + 1) % SH].ptr, YH[k].ptr, st), SH, reps=20)
+    add("next", "axpy_rows [64,256,56,56]", 8 * NH + 4 * 64 * CH, 4 * NH, ms, NH)
     pinh, pouth = [64, 64, 112, 112], [64, 64, 56, 56]
-    ms = time_batch(dev, lambda k: lib.shdw_hip_pooling2d(I(pinh), 0, 3, 3, 2, 2, 0, 0, I(pouth), AH[k].ptr,
-                                                          YH[k].ptr, st), SH, reps=20)
-    add("next", "pooling_max_3x3s2 [64,64,112,112]", 4 * (NH + NH // 4), ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_pooling2d(I(pinh), 0, 3, 3, 2, 2, 0, 0, I(pouth), AH[k].ptr,
+                                                           YH[k].ptr, st), SH, reps=20)
+    add("next", "pooling_max_3x3s2 [64,64,112,112]", 4 * NH, NH, ms, NH)
     ginh, gouth = [512, 2048, 7, 7], [512, 2048, 1, 1]
-    ms = time_batch(dev, lambda k: lib.shdw_hip_pooling2d(I(ginh), 1, 7, 7, 1, 1, 0, 0, I(gouth), AH[k].ptr,
-                                                          YH[k].ptr, st), SH, reps=20)
-    add("next", "pooling_global_avg_7x7 [512,2048,7,7]", 4 * (NH + 512 * 2048), ms, NH)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_softmax(64, 49, 16384, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
-    add("next", "softmax_channels_dense [64,49,128,128]", 8 * NH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_pooling2d(I(ginh), 1, 7, 7, 1, 1, 0, 0, I(gouth), AH[k].ptr,
+                                                           YH[k].ptr, st), SH, reps=20)
+    add("next", "pooling_global_avg_7x7 [512,2048,7,7]", 4 * NH, 4 * 512 * 2048, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_softmax(64, 49, 16384, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
+    add("next", "softmax_channels_dense [64,49,128,128]", 4 * NH, 4 * NH, ms, NH)
     NSEG = 64 * 150 * 5329  # a 150-class segmentation head, 73 x 73
-    ms = time_batch(dev, lambda k: lib.shdw_hip_softmax(64, 150, 5329, AH[k].ptr, YH[k].ptr, st), SH, reps=10)
-    add("next", "softmax_150_classes [64,150,73,73]", 8 * NSEG, ms, NSEG)
+    ms = time_median(dev, lambda k: lib.shdw_hip_softmax(64, 150, 5329, AH[k].ptr, YH[k].ptr, st), SH, reps=10)
+    add("next", "softmax_150_classes [64,150,73,73]", 4 * NSEG, 4 * NSEG, ms, NSEG)
     NSEG = 64 * 150 * 5184  # the same head on 72 x 72: rows of whole 128-bit vectors
-    ms = time_batch(dev, lambda k: lib.shdw_hip_softmax(64, 150, 5184, AH[k].ptr, YH[k].ptr, st), SH, reps=10)
-    add("next", "softmax_150_classes [64,150,72,72]", 8 * NSEG, ms, NSEG)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_normalize(64, 49, 16384, 2.0, 1e-12, AH[k].ptr, YH[k].ptr, st),
-                    SH, reps=20)
-    add("next", "normalize_l2_channels_dense [64,49,128,128]", 8 * NH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_softmax(64, 150, 5184, AH[k].ptr, YH[k].ptr, st), SH, reps=10)
+    add("next", "softmax_150_classes [64,150,72,72]", 4 * NSEG, 4 * NSEG, ms, NSEG)
+    ms = time_median(dev, lambda k: lib.shdw_hip_normalize(64, 49, 16384, 2.0, 1e-12, AH[k].ptr, YH[k].ptr, st),
+                     SH, reps=20)
+    add("next", "normalize_l2_channels_dense [64,49,128,128]", 4 * NH, 4 * NH, ms, NH)
     sch, bih = dev.buf(uniform(614, CH, 0.5, 1.5)), dev.buf(uniform(615, CH, -0.1, 0.1))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_group_norm(64 * CH, INH, 1e-5, AH[k].ptr, sch.ptr, bih.ptr,
-                                                           CH, INH, YH[k].ptr, st), SH, reps=20)
-    add("next", "instance_norm affine [64,256,56,56]", 8 * NH + 8 * CH, ms, NH)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_group_norm(64 * 32, 8 * INH, 1e-5, AH[k].ptr, sch.ptr, bih.ptr,
-                                                           CH, INH, YH[k].ptr, st), SH, reps=20)
-    add("next", "group_norm 32 groups affine [64,256,56,56]", 8 * NH + 8 * CH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_group_norm(64 * CH, INH, 1e-5, AH[k].ptr, sch.ptr, bih.ptr,
+                                                            CH, INH, YH[k].ptr, st), SH, reps=20)
+    add("next", "instance_norm affine [64,256,56,56]", 4 * NH + 8 * CH, 4 * NH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_group_norm(64 * 32, 8 * INH, 1e-5, AH[k].ptr, sch.ptr, bih.ptr,
+                                                            CH, INH, YH[k].ptr, st), SH, reps=20)
+    add("next", "group_norm 32 groups affine [64,256,56,56]", 4 * NH + 8 * CH, 4 * NH, ms, NH)
     lns, lnb = dev.buf(uniform(616, 784, 0.5, 1.5)), dev.buf(uniform(617, 784, -0.1, 0.1))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_group_norm(65536, 784, 1e-5, AH[k].ptr, lns.ptr, lnb.ptr,
-                                                           784, 1, YH[k].ptr, st), SH, reps=20)
-    add("next", "layer_norm affine [65536,784]", 8 * NH + 8 * 784, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_group_norm(65536, 784, 1e-5, AH[k].ptr, lns.ptr, lnb.ptr,
+                                                            784, 1, YH[k].ptr, st), SH, reps=20)
+    add("next", "layer_norm affine [65536,784]", 4 * NH + 8 * 784, 4 * NH, ms, NH)
     # SSDNormalize on the SSD conv4_3 map, batch 64: 8 bytes per element are compulsory
     # (the per-item form reads x a second time on top of that)
     NS = 64 * 512 * 1444
     ssc = dev.buf(uniform(618, 512, 10.0, 30.0))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_ssd_normalize(64, 512, 1444, 0, 1e-5, AH[k].ptr, ssc.ptr, 0,
-                                                              YH[k].ptr, None, st), SH, reps=20)
-    add("next", "ssd_normalize per position, channel scale [64,512,38,38]", 8 * NS + 4 * 512, ms, NS)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_ssd_normalize(64, 256, 3136, 0, 1e-5, AH[k].ptr, ssc.ptr, 0,
-                                                              YH[k].ptr, None, st), SH, reps=20)
-    add("next", "ssd_normalize per position, channel scale [64,256,56,56]", 8 * NH + 4 * 256, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_ssd_normalize(64, 512, 1444, 0, 1e-5, AH[k].ptr, ssc.ptr, 0,
+                                                               YH[k].ptr, None, st), SH, reps=20)
+    add("next", "ssd_normalize per position, channel scale [64,512,38,38]", 4 * NS + 4 * 512, 4 * NS, ms, NS)
+    ms = time_median(dev, lambda k: lib.shdw_hip_ssd_normalize(64, 256, 3136, 0, 1e-5, AH[k].ptr, ssc.ptr, 0,
+                                                               YH[k].ptr, None, st), SH, reps=20)
+    add("next", "ssd_normalize per position, channel scale [64,256,56,56]", 4 * NH + 4 * 256, 4 * NH, ms, NH)
     swb = dev.buf(nbytes=max(8, lib.shdw_hip_ssd_normalize_workspace_bytes(64, 512, 1444, 1)))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_ssd_normalize(64, 512, 1444, 1, 1e-5, AH[k].ptr, ssc.ptr, 0,
-                                                              YH[k].ptr, swb.ptr, st), SH, reps=20)
-    add("next", "ssd_normalize per item, channel scale [64,512,38,38] (2 launches)", 8 * NS + 4 * 512, ms, NS)
+    ms = time_median(dev, lambda k: lib.shdw_hip_ssd_normalize(64, 512, 1444, 1, 1e-5, AH[k].ptr, ssc.ptr, 0,
+                                                               YH[k].ptr, swb.ptr, st), SH, reps=20)
+    add("next", "ssd_normalize per item, channel scale [64,512,38,38] (2 launches)", 4 * NS + 4 * 512, 4 * NS, ms, NS)
     # data movers ("movers") on the same 205 MB tensors
-    half = NH // 2
     def concat2(k):
         # two [64,128,56,56] halves -> [64,256,56,56] along axis 1
         rc = lib.shdw_hip_copy_chunks(64, 128 * INH, AH[k].ptr, 128 * INH, 0, YH[k].ptr, 256 * INH, 0, st)
         return rc or lib.shdw_hip_copy_chunks(64, 128 * INH, AH[(k + 1) % SH].ptr, 128 * INH, 0, YH[k].ptr,
                                               256 * INH, 128 * INH, st)
-    ms = time_batch(dev, concat2, SH, reps=20)
-    add("movers", "concat 2x[64,128,56,56] axis 1 (2 launches)", 8 * NH, ms, NH)
+    ms = time_median(dev, concat2, SH, reps=20)
+    add("movers", "concat 2x[64,128,56,56] axis 1 (2 launches)", 4 * NH, 4 * NH, ms, NH)
     shp4 = [64, 256, 56, 56]
-    ms = time_batch(dev, lambda k: lib.shdw_hip_permute(4, I(shp4), I([0, 2, 3, 1]), AH[k].ptr, YH[k].ptr, st),
-                    SH, reps=20)
-    add("movers", "permute NCHW->NHWC [64,256,56,56]", 8 * NH, ms, NH)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_permute(4, I(shp4), I([0, 3, 1, 2]), AH[k].ptr, YH[k].ptr, st),
-                    SH, reps=20)
-    add("movers", "permute [0,3,1,2] [64,256,56,56]", 8 * NH, ms, NH)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_shuffle_channel(64, 256, INH, 2, AH[k].ptr, YH[k].ptr, st), SH,
-                    reps=20)
-    add("movers", "shuffle_channel g=2 [64,256,56,56]", 8 * NH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_permute(4, I(shp4), I([0, 2, 3, 1]), AH[k].ptr, YH[k].ptr, st),
+                     SH, reps=20)
+    add("movers", "permute NCHW->NHWC [64,256,56,56]", 4 * NH, 4 * NH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_permute(4, I(shp4), I([0, 3, 1, 2]), AH[k].ptr, YH[k].ptr, st),
+                     SH, reps=20)
+    add("movers", "permute [0,3,1,2] [64,256,56,56]", 4 * NH, 4 * NH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_shuffle_channel(64, 256, INH, 2, AH[k].ptr, YH[k].ptr, st), SH,
+                     reps=20)
+    add("movers", "shuffle_channel g=2 [64,256,56,56]", 4 * NH, 4 * NH, ms, NH)
     pshape = [64, 64, 110, 110]
     npi = int(np.prod(pshape))
-    ms = time_batch(dev, lambda k: lib.shdw_hip_pad(I(pshape), I([1, 1, 1, 1]), 0.0, AH[k].ptr, YH[k].ptr, st), SH,
-                    reps=20)
-    add("movers", "pad 1 [64,64,110,110] -> 112x112", 4 * (npi + NH), ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_pad(I(pshape), I([1, 1, 1, 1]), 0.0, AH[k].ptr, YH[k].ptr, st), SH,
+                     reps=20)
+    add("movers", "pad 1 [64,64,110,110] -> 112x112", 4 * npi, 4 * NH, ms, NH)
     rin, rout = [64, 64, 56, 56], [64, 64, 112, 112]
     nri = int(np.prod(rin))
     # The resize input is a quarter of a set (51 MB): all four quarters of every set
-    # take turns (12 inputs, 617 MB).  With three inputs the gathers found them in the
-    # Infinity Cache and the kernels looked faster than they are from HBM (nearest:
-    # 38 us against 64).
+    # take turns (12 inputs, 617 MB), so that the gathers do not find them in the
+    # Infinity Cache.
     def resize_in(k):
         return AH[k % SH].ptr + (k // SH) * 4 * nri
-    ms = time_batch(dev, lambda k: lib.shdw_hip_resize(I(rin), I(rout), 1, 0, resize_in(k), YH[k % SH].ptr, st),
-                    4 * SH, reps=24)
-    add("movers", "resize bilinear x2 [64,64,56,56]", 4 * (nri + NH), ms, NH)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_resize(I(rin), I(rout), 0, 0, resize_in(k), YH[k % SH].ptr, st),
-                    4 * SH, reps=24)
-    add("movers", "resize nearest x2 [64,64,56,56]", 4 * (nri + NH), ms, NH)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_reorg(I(rout), 1, 2, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
-    add("movers", "reorg natural s2 [64,64,112,112]", 8 * NH, ms, NH)
-    ms = time_batch(dev, lambda k: lib.shdw_hip_reorg(I(rout), 0, 2, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
-    add("movers", "reorg darknet s2 [64,64,112,112]", 8 * NH, ms, NH)
-    for bset in (AH, YH):
+    ms = time_median(dev, lambda k: lib.shdw_hip_resize(I(rin), I(rout), 1, 0, resize_in(k), YH[k % SH].ptr, st),
+                     4 * SH, reps=24)
+    add("movers", "resize bilinear x2 [64,64,56,56]", 4 * nri, 4 * NH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_resize(I(rin), I(rout), 0, 0, resize_in(k), YH[k % SH].ptr, st),
+                     4 * SH, reps=24)
+    add("movers", "resize nearest x2 [64,64,56,56]", 4 * nri, 4 * NH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_reorg(I(rout), 1, 2, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
+    add("movers", "reorg natural s2 [64,64,112,112]", 4 * NH, 4 * NH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_reorg(I(rout), 0, 2, AH[k].ptr, YH[k].ptr, st), SH, reps=20)
+    add("movers", "reorg darknet s2 [64,64,112,112]", 4 * NH, 4 * NH, ms, NH)
+    for bset in (AH, YH, [meanh, varh, alh, sch, bih, lns, lnb, ssc, swb]):
         for bb in bset:
             bb.free()
 
@@ -508,15 +722,31 @@ def config_table(dev, sets_scale=1):
                           ("iii", [128, 1024], [1, 1])]:
         so4 = [max(p, q) for p, q in zip(sa4, sb4)]
         na, nb_, no = int(np.prod(sa4)), int(np.prod(sb4)), int(np.prod(so4))
-        a4 = dev.buf(normal(401, na))
-        b4 = dev.buf(uniform(402, nb_, 0.5, 2.0))
+        ha, hb4 = normal(401, na), uniform(402, nb_, 0.5, 2.0)
+        a4, b4 = dev.buf(ha), dev.buf(hb4)
         y4 = [dev.buf(nbytes=4 * no) for _ in range(SETS)]
+        hy4 = np.empty(no, np.float32) if cpu else None
         for name, op in [("mul", 2), ("sub", 1), ("div", 3), ("max", 5)]:
-            ms = time_batch(dev, lambda k: lib.shdw_hip_broadcast_binary(
+            ms = time_median(dev, lambda k: lib.shdw_hip_broadcast_binary(
                 op, len(so4), I(sa4), I(sb4), I(so4), a4.ptr, b4.ptr, y4[k].ptr, st), SETS)
-            add(4, "broadcast_%s_%s" % (name, tag), 4 * (na + nb_ + no), ms, no)
-        for bb in y4:
+            add(4, "broadcast_%s_%s" % (name, tag), 4 * (na + nb_), 4 * no, ms, no,
+                cpu and cpu.broadcast(op, ha, sa4, hb4, sb4, so4, hy4))
+        if tag == "iii":  # the same pair through the scalar-argument form
+            alpha = float(hb4[0])
+            for name, op in [("mul", 2), ("sub", 1), ("div", 3), ("max", 5)]:
+                ms = time_median(dev, lambda k: lib.shdw_hip_binary_scalar(op, na, a4.ptr, alpha, y4[k].ptr, st), SETS)
+                add(4, "scalar_%s_iii" % name, 4 * na, 4 * no, ms, no, cpu and cpu.binary_scalar(op, ha, alpha, hy4))
+        for bb in y4 + [a4, b4]:
             bb.free()
+
+    # The yardsticks themselves, at the byte counts of the BASELINE rows.
+    for mb, nbytes in [(25.7, 25690112), (34, 34209792), (51, 51380224), (69, 69222400), (103, 102760448),
+                       (154, 154140672), (411, 411041792)]:
+        for kind in ("copy", "read", "write"):
+            us = ceil.us(kind, nbytes)
+            rows.append({"cfg": "ceiling", "op": "%s of %s MB" % (kind, mb), "bytes": nbytes, "us": round(us, 2),
+                         "GBps": round(nbytes / us / 1e3, 1), "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+    ceil.free()
     return rows
 
 
@@ -567,7 +797,7 @@ def main():
     if args.probe_next:
         probe_next(dev)
         return
-    ms_per_step, step_bytes, n, roofline, detail, host = headline(dev, args.steps, args.warmup)
+    ms_per_step, step_bytes, n, roofline, detail, host = headline(dev, args.steps, args.warmup, args.single_input)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     out = {
         "metric": "achieved HBM GB/s (% of MI355X peak) per op; speedup vs host-CPU Shadow",
@@ -576,7 +806,9 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "BASELINE configs[1]: fp32 [64,256,56,56] ~N(0,2) seed 201; relu, "
                                "sigmoid, exp, abs, sqrt(abs), tanh as single ops + fused per-channel "
-                               "Scale+ReLU (7 launches per step)",
+                               "Scale+ReLU (7 launches per step); %s" % (
+                                   "one resident input" if args.single_input else
+                                   "two resident copies of the input take turns step by step"),
                    "elements": n, "bytes_per_step": step_bytes, "device": dev.info},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "elements_per_s": round(7 * n / (ms_per_step * 1e-3), 1),
@@ -584,12 +816,23 @@ def main():
         "step_ops_note": "per-op times from an untimed pass of the same K steps with events around every "
                          "launch; roofline.avg_us from events around the dominant kernel inside the timed region",
     }
-    if not args.no_configs:
-        out["configs"] = config_table(dev, args.operand_sets)
-        out["network"] = network_forward(dev)
-    if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(host, step_bytes, args.cpu_passes)
+    cpu = None if args.no_cpu else Cpu(args.cpu_passes)
+    if cpu is not None:
+        out["cpu_baseline"] = cpu_headline(cpu, host, step_bytes)
         out["speedup_vs_cpu"] = round(value / out["cpu_baseline"]["value"], 1)
+        for d in detail:
+            c = out["cpu_baseline"]["ops"].get(d["op"])
+            if c:
+                d["cpu_us"] = c["best_us"]
+                d["speedup_vs_cpu"] = round(c["best_us"] / d["us"], 1)
+    host = None
+    if not args.no_configs:
+        out["configs"] = config_table(dev, args.operand_sets, cpu)
+        out["configs_note"] = ("us: median of three batches of back-to-back launches rotating over operand sets; "
+                               "ceiling_us: a plain copy / read / write of the same number of bytes timed the same "
+                               "way (rows at the end); cpu_us: the oracle's C loop for the same operator on this "
+                               "host, one thread, outputs allocated beforehand, best of %d" % args.cpu_passes)
+        out["network"] = network_forward(dev)
     print(json.dumps(out))
 
 

@@ -111,6 +111,12 @@ int shdw_hip_event_record(void* event, void* stream);
 int shdw_hip_event_sync(void* event);
 int shdw_hip_event_elapsed_ms(void* start, void* stop, float* ms);
 
+/* Reads the n / 4 whole vectors of x, one per lane, and writes nothing, except `sentinel` to *sink (device memory) from a
+ * lane whose four values add up to it.  With shdw_hip_copy and shdw_hip_set it
+ * gives the harness the read, copy and write ceilings of a tensor size; the
+ * reference has no counterpart. */
+int shdw_hip_probe_read(int n, const float* x, float sentinel, float* sink, void* stream);
+
 /* ============================ Blas, elementwise ========================== */
 
 /* y[i] = val.  ref: shadow/core/blas.cpp:25-34, shadow/core/blas.cu:11-21 */

@@ -262,12 +262,13 @@ static float reduce_one(const float* data, const int* list, int num_list, int of
   }
 }
 
-/* ---- shadow/operators/kernels/reduce.hpp:41-88  list/offset planning, then
- *      shadow/operators/kernels/reduce.cpp:67-76  Vision::Reduce ----
- * out_shape = in_shape with the reduced axes set to 1 (reduce_op.cpp:38-42). */
-API int orc_reduce(int op, const float* in, const int* in_shape, int num_axes, const int* axes,
-                   int num_reduce, float* out) {
-  if (op < 0 || op > 6) return -1;
+/* ---- shadow/operators/kernels/reduce.hpp:41-71  the index lists of ReduceKernelDefault::Run:
+ *      list[num_list] = offsets inside one window, last listed axis fastest;
+ *      offset[out_count] = origin of every output.  The reference rebuilds them only
+ *      when the input shape changes (reduce.hpp:45).  Returns num_list, or -1.
+ *      out_shape = in_shape with the reduced axes set to 1 (reduce_op.cpp:38-42). */
+API int orc_reduce_lists(const int* in_shape, int num_axes, const int* axes, int num_reduce, int* list,
+                         int* offset) {
   int shape_acc[16], out_shape[16];
   if (num_axes > 16) return -1;
   if (num_axes > 0) shape_acc[num_axes - 1] = 1;
@@ -276,11 +277,6 @@ API int orc_reduce(int op, const float* in, const int* in_shape, int num_axes, c
   for (int n = 0; n < num_axes; ++n) out_shape[n] = in_shape[n];
   for (int k = 0; k < num_reduce; ++k) out_shape[axes[k]] = 1;
   for (int n = 0; n < num_axes; ++n) out_count *= out_shape[n];
-
-  /* list: offsets inside one window, last listed axis fastest */
-  size_t cap = 1;
-  for (int k = 0; k < num_reduce; ++k) cap *= (size_t)in_shape[axes[k]];
-  int* list = (int*)malloc(sizeof(int) * cap);
   int num_list = 1;
   list[0] = 0;
   for (int n = num_reduce - 1; n >= 0; --n) {
@@ -289,15 +285,37 @@ API int orc_reduce(int op, const float* in, const int* in_shape, int num_axes, c
       for (int j = 0; j < cur; ++j) list[num_list++] = list[j] + k * shape_acc[axis];
   }
   for (int i = 0; i < out_count; ++i) {
-    int offset = 0, cc = i;
+    int off = 0, cc = i;
     for (int n = num_axes - 1; n >= 0; --n) {
       int dim = out_shape[n];
-      offset += (cc % dim) * shape_acc[n];
+      off += (cc % dim) * shape_acc[n];
       cc /= dim;
     }
-    out[i] = reduce_one(in, list, num_list, offset, op);
+    offset[i] = off;
   }
+  return num_list;
+}
+
+/* ---- shadow/operators/kernels/reduce.cpp:67-76  Vision::Reduce ---- */
+API void orc_vision_reduce(const float* in, const int* list, const int* offset, int num_list, int operation,
+                           int count, float* out) {
+  for (int i = 0; i < count; ++i) out[i] = reduce_one(in, list, num_list, offset[i], operation);
+}
+
+/* ---- shadow/operators/kernels/reduce.hpp:41-88  both steps for one call ---- */
+API int orc_reduce(int op, const float* in, const int* in_shape, int num_axes, const int* axes,
+                   int num_reduce, float* out) {
+  if (op < 0 || op > 6 || num_axes > 16) return -1;
+  size_t cap = 1, out_count = 1;
+  for (int k = 0; k < num_reduce; ++k) cap *= (size_t)in_shape[axes[k]];
+  for (int n = 0; n < num_axes; ++n) out_count *= (size_t)in_shape[n];
+  out_count /= cap;
+  int* list = (int*)malloc(sizeof(int) * cap);
+  int* offset = (int*)malloc(sizeof(int) * out_count);
+  int num_list = orc_reduce_lists(in_shape, num_axes, axes, num_reduce, list, offset);
+  orc_vision_reduce(in, list, offset, num_list, op, (int)out_count, out);
   free(list);
+  free(offset);
   return 0;
 }
 

@@ -27,15 +27,20 @@ namespace shdw {
 // vectors apart so that every load instruction of the wave is contiguous; the
 // lane whose vector index is n4 (one past the last whole vector) owns the
 // n % 4 trailing elements.
-template <int NIN, class F, int V>
-__global__ __launch_bounds__(kStream) void ew_vec_kernel(F f, const float* a, const float* b,
-                                                          float* y, uint32_t n4, uint32_t n,
-                                                          float alpha) {
-  const uint32_t first = blockIdx.x * (kStream * V) + threadIdx.x;
+// The workgroup is a single wave64 where something is read (T = kStream); a fill
+// (NIN = 0) takes 256 lanes: a wave that only stores 1 KB is gone so quickly that
+// single-wave workgroups are bounded by the rate at which workgroups can be
+// started (4.2 per ns: 4.3 TB/s of stores, measured 12.1 us for 51 MB against
+// 8.4 us with 256 lanes; a copy moves 2 KB per wave and is not bounded by it).
+template <int NIN, class F, int V, int T>
+__global__ __launch_bounds__(T) void ew_vec_kernel(F f, const float* a, const float* b,
+                                                    float* y, uint32_t n4, uint32_t n,
+                                                    float alpha) {
+  const uint32_t first = blockIdx.x * (T * V) + threadIdx.x;
   v4f va[V], vb[V];
 #pragma unroll
   for (int u = 0; u < V; ++u) {  // issue the streaming loads before anything else
-    const uint32_t i = first + u * kStream;
+    const uint32_t i = first + u * T;
     if (i < n4) {
       if (NIN >= 1) va[u] = load4_stream_any(a + 4ull * i);
       if (NIN >= 2) vb[u] = load4_stream_any(b + 4ull * i);
@@ -50,7 +55,7 @@ __global__ __launch_bounds__(kStream) void ew_vec_kernel(F f, const float* a, co
   }
 #pragma unroll
   for (int u = 0; u < V; ++u) {
-    const uint32_t i = first + u * kStream;
+    const uint32_t i = first + u * T;
     if (i < n4) {
       v4f r;
 #pragma unroll
@@ -79,8 +84,9 @@ static int launch_ew(F f, int n, const float* a, const float* b, float alpha, fl
   // Any float pointers: the 128-bit accesses need dword alignment only.
   const uint32_t n4 = static_cast<uint32_t>(n) / 4;
   constexpr int V = vectors_per_lane<F>::value;
-  const uint32_t grid = stream_grid((n4 + V) / V);  // n4 + 1 vector slots, V per lane
-  ew_vec_kernel<NIN, F, V><<<grid, kStream, 0, s>>>(f, a, b, y, n4, static_cast<uint32_t>(n), alpha);
+  constexpr int T = NIN == 0 ? kBlock : kStream;
+  const uint32_t slots = (n4 + V) / V;  // n4 + 1 vector slots, V per lane
+  ew_vec_kernel<NIN, F, V, T><<<(slots + T - 1) / T, T, 0, s>>>(f, a, b, y, n4, static_cast<uint32_t>(n), alpha);
   return launch_status();
 }
 
@@ -104,6 +110,22 @@ struct AxpyOp {  // y += alpha * x, multiply then add
     return y + t;
   }
 };
+
+// Read-only pass: every lane requests one vector and stores nothing unless its
+// four values add up to `sentinel`.  It exists for the measurement harness (the
+// read ceiling of a tensor size).  1024-lane workgroups: of the shapes measured
+// (64, 256, 1024 lanes x 1, 2, 4, 8 vectors per lane) the fastest or level with
+// it at every size from 25 to 411 MB (411 MB: 55.8 us, 256 lanes 59.5 us, single
+// waves 86.5 us).
+constexpr int kReadProbeThreads = 1024;
+__global__ __launch_bounds__(kReadProbeThreads) void read_probe_kernel(const float* a, float* sink, uint32_t n4,
+                                                                        float sentinel) {
+  const uint32_t i = blockIdx.x * kReadProbeThreads + threadIdx.x;
+  if (i < n4) {
+    const v4f v = load4_stream_any(a + 4ull * i);
+    if ((v[0] + v[1]) + (v[2] + v[3]) == sentinel) *sink = sentinel;
+  }
+}
 
 // ---------------------------------------------------------------------------
 // K-ary Eltwise in one pass.
@@ -273,6 +295,15 @@ int shdw_hip_scal(int n, float alpha, float* x, void* stream) {
 
 int shdw_hip_copy(int n, const float* x, float* y, void* stream) {
   return launch_ew<1>(Unary2<UCopy>(), n, x, nullptr, 0.f, y, stream);
+}
+
+int shdw_hip_probe_read(int n, const float* x, float sentinel, float* sink, void* stream) {
+  if (n < 0 || !x || !sink) return SHDW_E_INVALID_ARGUMENT;
+  const uint32_t n4 = static_cast<uint32_t>(n) / 4;
+  if (n4 == 0) return SHDW_OK;
+  const uint32_t grid = (n4 + kReadProbeThreads - 1) / kReadProbeThreads;
+  read_probe_kernel<<<grid, kReadProbeThreads, 0, static_cast<hipStream_t>(stream)>>>(x, sink, n4, sentinel);
+  return launch_status();
 }
 
 int shdw_hip_axpy(int n, float alpha, const float* x, float* y, void* stream) {
