@@ -214,6 +214,10 @@ HOST_SIGNATURES = {
     "shdw_host_network_forward": (_I, [_V, _I, ctypes.POINTER(ctypes.c_char_p), c_void_pp, c_int_p, c_int_p]),
     "shdw_host_network_blob_shape": (_I, [_V, ctypes.c_char_p, c_int_p, _I]),
     "shdw_host_network_blob_get": (_I, [_V, ctypes.c_char_p, c_float_p, _I]),
+    "shdw_host_face_blas": (_I, [_V, ctypes.c_char_p, _I, c_float_p, _I, _I, c_float_p, _I, _I, _F, c_float_p, _I, _I]),
+    "shdw_host_face_conv_epilogue": (_I, [_V, c_float_p, _I, c_float_p, _I, _I, _I, _I]),
+    "shdw_host_face_eltwise_sum": (_I, [_V, _I, ctypes.POINTER(c_float_p), c_float_p, _I, c_float_p]),
+    "shdw_host_face_ssd_normalize": (_I, [_V, c_float_p, _I, _I, _I, _I, _I, _F, c_float_p, c_float_p]),
     "shdw_host_probe_create_kernel": (_I, [ctypes.c_char_p, _I]),
     "shdw_host_probe_argument": (_I, [ctypes.c_char_p, ctypes.c_char_p]),
 }

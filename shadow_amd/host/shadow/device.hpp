@@ -43,6 +43,12 @@ class Context {
   virtual void synchronize() = 0;
   virtual void* stream() const { return nullptr; }
 
+  // Device scratch that lives as long as the context, grow-only, for the level-1
+  // routines whose signature carries no Workspace (BlasSasum): what the cuBLAS
+  // handle's own workspace was in the reference.  Valid until the next call with
+  // a larger size; one stream, so one user at a time.
+  virtual void* level1_scratch(size_t bytes) { return nullptr; }
+
   // Vendor-library handles of the reference; nothing on this path uses them.
   virtual void* cublas_handle() const { return nullptr; }
   virtual void* cudnn_handle() const { return nullptr; }

@@ -79,15 +79,16 @@ void BlasSaxpy<G, float>(int n, float alpha, const float* x, int offx, float* y,
 template <>
 void BlasSasum<G, float>(int n, const float* x, int offx, float* y, Context* ctx) {
   // The signature has no Workspace to borrow scratch from (it did not need one
-  // on top of cuBLAS), so the partial sums live in a small allocation made for
-  // the call: at most 2048 partials of 16 bytes plus the result.
+  // on top of cuBLAS): the partial sums live in the context's own scratch, which
+  // is allocated once.  The reference calls this once per batch item
+  // (kernels/ssd_normalize.hpp:51-57); an allocation per call would stall the
+  // device every time.
+  CHECK_NOTNULL(ctx);
   const int shape[1] = {n}, axes[1] = {0};
   const size_t bytes = shdw_hip_reduce_workspace_bytes(1, shape, 1, axes) + 16;
-  void* scratch = nullptr;
-  SHADOW_HIP_CHECK(shdw_hip_malloc(&scratch, bytes));
-  const int rc = shdw_hip_asum(n, x + offx, y, scratch, bytes, stream_of(ctx));
-  SHADOW_HIP_CHECK(shdw_hip_free(scratch));
-  SHADOW_HIP_CHECK(rc);
+  void* scratch = ctx->level1_scratch(bytes);
+  CHECK_NOTNULL(scratch);
+  SHADOW_HIP_CHECK(shdw_hip_asum(n, x + offx, y, scratch, bytes, stream_of(ctx)));
 }
 
 }  // namespace Blas

@@ -56,6 +56,11 @@ int join(const std::vector<std::string>& keys, char* buf, size_t n) {
 extern "C" {
 
 const char* shdw_host_last_error(void) { return g_error.c_str(); }
+// for the other translation units of the facade
+int shdw_host_set_error(const char* text) {
+  g_error = text ? text : "";
+  return 0;
+}
 
 int shdw_host_kernel_keys(char* buf, size_t n) { return join(KernelRegistry()->Keys(), buf, n); }
 int shdw_host_operator_keys(char* buf, size_t n) { return join(OperatorRegistry()->Keys(), buf, n); }

@@ -65,7 +65,23 @@ class HipContext : public Context {
     allocator_->set_stream(stream_);
   }
   ~HipContext() override {
+    if (scratch_ != nullptr) shdw_hip_free(scratch_);
     if (own_stream_ && stream_ != nullptr) shdw_hip_stream_destroy(stream_);
+  }
+
+  void* level1_scratch(size_t bytes) override {
+    if (bytes > scratch_bytes_) {
+      // the old buffer may still be in use by work enqueued on the stream
+      if (scratch_ != nullptr) {
+        synchronize();
+        SHADOW_HIP_CHECK(shdw_hip_free(scratch_));
+        scratch_ = nullptr;
+      }
+      const size_t want = bytes < kMinScratch ? kMinScratch : bytes;
+      SHADOW_HIP_CHECK(shdw_hip_malloc(&scratch_, want));
+      scratch_bytes_ = want;
+    }
+    return scratch_;
   }
 
   Allocator* allocator() const override { return allocator_.get(); }
@@ -80,6 +96,10 @@ class HipContext : public Context {
   bool own_stream_ = true;
   void* stream_ = nullptr;
   std::shared_ptr<Allocator> allocator_;
+  // 4096 partial sums of 8 bytes and the result: what BlasSasum needs for any n
+  static constexpr size_t kMinScratch = 64 * 1024;
+  void* scratch_ = nullptr;
+  size_t scratch_bytes_ = 0;
 };
 
 }  // namespace

@@ -64,6 +64,12 @@ void Native::Initial(const shadow::NetParam& net_param) {
     }
   }
 
+  // The uploads above were enqueued on the context's stream from memory that
+  // the caller's NetParam owns (the LoadModel overloads above destroy theirs on
+  // return): wait for them here rather than rely on how the runtime treats
+  // pageable sources.
+  ws_->Ctx()->synchronize();
+
   ops_.clear(), in_blob_.clear();
   for (const auto& op_param : net_param.op()) {
     ops_.emplace_back(CreateOperator(op_param, ws_.get()));
