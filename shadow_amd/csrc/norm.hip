@@ -116,6 +116,16 @@ SHDW_DEVICE double wave_sum(double v) {
 // the lanes are neighbours inside one wave; more: whole waves, through `slots`.
 template <int LANES>
 SHDW_DEVICE double row_sum(double v, double* slots) {
+  if (LANES <= 16) {
+    // inside a row of 16 lanes the exchanges are DPP moves (no LDS traffic); after
+    // each step the lanes that have met hold the same sum, so the mirrors of the
+    // last two steps pair every lane with one from the other half
+    if (LANES >= 2) v += dpp_f64<kDppXor1>(v);
+    if (LANES >= 4) v += dpp_f64<kDppXor2>(v);
+    if (LANES >= 8) v += dpp_f64<kDppHalfMirror>(v);
+    if (LANES >= 16) v += dpp_f64<kDppMirror>(v);
+    return v;
+  }
   if (LANES <= kWave) {
 #pragma unroll
     for (int off = LANES / 2; off >= 1; off >>= 1) v += __shfl_xor(v, off);
@@ -236,6 +246,137 @@ __global__ __launch_bounds__(LANES <= kWave ? kBlock : LANES, LANES == kBigBlock
       }
     }
   }
+}
+
+// Rows of 17 to 256 elements, at least a thousand of them.  The register forms
+// above give such rows 16 to 64 lanes with one vector each, and what a lane does
+// once per row (two fp64 exchanges, four IEEE divisions' worth of setup, the
+// square root, the parameter lookup, the vector-tail logic) then outweighs what
+// it does per element: rows of 49 on 16 lanes ran at the instruction issue rate
+// (258 vector instructions per wave of four rows, 32 us per 103 MB).  Giving a
+// lane 16 neighbouring elements straight from global memory does not work
+// either: 128-bit loads whose lanes are 64 bytes apart run at the address rate
+// (53 us).  Here a workgroup's 256 / L rows, one contiguous span, pass through
+// LDS as they lie, with 128-bit copies on both sides, and L lanes share a row,
+// each walking its own piece of about 13 to 16 elements three times in LDS (mean,
+// variance, output in place).  The lane partials of the two sums meet by DPP.
+constexpr int kNormLdsMaxInner = 256;
+
+// PADDED: inner % 4 == 0.  Such rows would start on the same few LDS banks (rows
+// of 64 or 128 floats: all on one), so they get a pitch of inner + 4 floats (the
+// 128-bit copies then never cross a row end); other row lengths are copied as
+// they lie.  The pieces are an odd number of elements long for the same reason.
+template <int L, bool PADDED>
+__global__ __launch_bounds__(kBlock) void norm_rows_lds_kernel(const float* x, float* y, NormArgs p,
+                                                                uint32_t seg, FastDiv f_inner4) {
+  constexpr uint32_t kRows = kBlock / L;
+  __shared__ __align__(16) float tile[kRows * (16 * L + 4)];  // 16 to 17 KB: inner <= 16 L
+  __shared__ float sc[16 * L], bi[16 * L];                   // LayerNorm: scale and bias by row position
+  const uint32_t inner = p.inner;
+  const uint32_t pitch = PADDED ? inner + 4 : inner;
+  const uint32_t row0 = blockIdx.x * kRows;
+  const uint32_t nrows = min(kRows, p.outer - row0);
+  const uint64_t base = static_cast<uint64_t>(row0) * inner;
+  const float* xs = x + base;
+  float* ys = y + base;
+  const uint32_t cells = nrows * inner, nvec = cells / 4;
+  // LDS offset of the vector that starts at element 4 v of the span
+  auto slot = [&](uint32_t v) -> uint32_t {
+    if (!PADDED) return 4 * v;
+    const uint32_t r = fd_div(v, f_inner4);  // inner / 4 vectors per row
+    return 4 * v + 4 * r;
+  };
+  for (uint32_t v0 = 0; v0 < nvec; v0 += 4 * kBlock) {
+    v4f reg[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t v = min(v0 + k * kBlock + threadIdx.x, nvec - 1);  // past the end: the last piece again
+      reg[k] = load4_stream_any(xs + 4ull * v);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t v = v0 + k * kBlock + threadIdx.x;
+      if (v < nvec) *reinterpret_cast<v4f*>(tile + slot(v)) = reg[k];
+    }
+  }
+  if (!PADDED && threadIdx.x < (cells & 3u)) tile[4 * nvec + threadIdx.x] = xs[4 * nvec + threadIdx.x];
+  if (p.affine == kAffineRowPos) {
+    for (uint32_t t = threadIdx.x; t < inner; t += kBlock) sc[t] = p.scale[t], bi[t] = p.bias[t];
+  }
+  __syncthreads();
+
+  const uint32_t r = threadIdx.x / L, h = threadIdx.x % L;
+  // rows past the end compute on whatever the tile holds and store nothing: all
+  // lanes of a wave stay together for the exchanges
+  const uint32_t c_begin = min(h * seg, inner), c_end = min(c_begin + seg, inner);
+  const uint32_t n = c_end - c_begin;
+  float* mine = tile + (r < nrows ? r : 0) * pitch + c_begin;
+  double acc = 0;
+  uint32_t c = 0;
+  for (; c + 4 <= n; c += 4) {
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = mine[c + k];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float t = p.alpha * v[k];
+      acc += static_cast<double>(t);
+    }
+  }
+  for (; c < n; ++c) {
+    const float t = p.alpha * mine[c];
+    acc += static_cast<double>(t);
+  }
+  const float mean = static_cast<float>(row_sum<L>(acc, nullptr));
+  acc = 0;
+  for (c = 0; c + 4 <= n; c += 4) {
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = mine[c + k];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float val = v[k] - mean;
+      const float sq = val * val;
+      const float t = p.alpha * sq;
+      acc += static_cast<double>(t);
+    }
+  }
+  for (; c < n; ++c) {
+    const float val = mine[c] - mean;
+    const float sq = val * val;
+    const float t = p.alpha * sq;
+    acc += static_cast<double>(t);
+  }
+  const float variance = static_cast<float>(row_sum<L>(acc, nullptr));
+  const float ve = variance + p.eps;
+  const float denom = __builtin_sqrtf(ve);
+  if (r < nrows) {
+    const uint32_t first = static_cast<uint32_t>(base) + r * inner;  // global index of the row
+    const RowAffine ra = norm_row_affine(p, first);
+    auto finish = [&](uint32_t pos, float v) -> float {
+      const float val = v - mean;
+      float q = val / denom;
+      if (p.affine == kAffineRow) q = affine1(q, ra.s, ra.b);
+      else if (p.affine == kAffineRowPos) q = affine1(q, sc[c_begin + pos], bi[c_begin + pos]);
+      else if (p.affine != kAffineNone) q = norm_affine1(p, first + c_begin + pos, q);
+      return q;
+    };
+    for (c = 0; c + 4 <= n; c += 4) {
+      float v[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] = mine[c + k];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] = finish(c + k, v[k]);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) mine[c + k] = v[k];
+    }
+    for (; c < n; ++c) mine[c] = finish(c, mine[c]);
+  }
+  __syncthreads();
+
+  for (uint32_t v = threadIdx.x; v < nvec; v += kBlock)
+    store4_stream_any(ys + 4ull * v, *reinterpret_cast<const v4f*>(tile + slot(v)));
+  if (!PADDED && threadIdx.x < (cells & 3u)) ys[4 * nvec + threadIdx.x] = tile[4 * nvec + threadIdx.x];
 }
 
 // Any row, one workgroup per row, three passes over memory (the second and
@@ -466,6 +607,35 @@ int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
   const uint32_t nvec = p.inner / 4;
   // workgroups of 256 lanes holding 256 / lanes rows each
   auto groups = [rows](uint32_t lanes) { return (rows + kBlock / lanes - 1) / (kBlock / lanes); };
+  if (p.inner > 16 && p.inner <= kNormLdsMaxInner && rows >= 1024) {
+    // short rows through LDS, L lanes per row (any row length, any dword address)
+    if (!scale)
+      p.affine = kAffineNone;
+    else if (scale_inner % inner_num == 0)
+      p.affine = kAffineRow;
+    else if (scale_inner == 1 && scale_num == inner_num)
+      p.affine = kAffineRowPos;  // scalar lookups by row position: no alignment asked of the parameters
+    else
+      p.affine = kAffineElement;
+    const uint32_t want = (p.inner + 15) / 16;  // lanes for pieces of at most 16 elements
+    const uint32_t lanes = want <= 2 ? 2 : (want <= 4 ? 4 : (want <= 8 ? 8 : 16));
+    const uint32_t seg = ((p.inner + lanes - 1) / lanes) | 1u;  // an odd number of elements per lane
+    const uint32_t grid = (rows + kBlock / lanes - 1) / (kBlock / lanes);
+    const FastDiv f4 = make_fastdiv(std::max<uint32_t>(1, p.inner / 4));
+#define SHDW_LDS(LANES)                                                                        \
+  do {                                                                                         \
+    if (p.inner % 4 == 0) norm_rows_lds_kernel<LANES, true><<<grid, kBlock, 0, st>>>(x, y, p, seg, f4);  \
+    else norm_rows_lds_kernel<LANES, false><<<grid, kBlock, 0, st>>>(x, y, p, seg, f4);        \
+  } while (0)
+    switch (lanes) {
+      case 2: SHDW_LDS(2); break;
+      case 4: SHDW_LDS(4); break;
+      case 8: SHDW_LDS(8); break;
+      default: SHDW_LDS(16); break;
+    }
+#undef SHDW_LDS
+    return launch_status();
+  }
   if (!vec) {
     // any row length, any dword address: whole vectors plus a partial one per row
     const uint32_t units = (p.inner + 3) / 4;
