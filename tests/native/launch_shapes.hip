@@ -1,0 +1,199 @@
+// Measurement of the launch shapes the kernels were given, on the device it runs on.
+// Prints one table per question; tests/test_gpu_launch_shapes.py runs it and
+// checks that the shapes the library uses are still the fast ones.
+//
+//   stream  : a plain copy, a read-only and a write-only pass over 51 MB and
+//             411 MB (rotating through 1.2 GB so that the 256 MB Infinity Cache
+//             cannot serve repeats), as workgroups of 64, 256 or 1024 lanes with
+//             1, 2 or 4 vectors per lane that cover the tensor, and as a
+//             2048-workgroup grid-stride loop with 4 vectors in flight per lane.
+//   strided : max over the 512 channels of [32,512,28,28] with the library's
+//             column-tile kernel shape, workgroups numbered round-robin over the
+//             8 XCDs (as dispatched) or XCD-contiguously, for three tile widths.
+//
+// Usage: launch_shapes            (all tables)
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "../../shadow_amd/csrc/device_common.h"
+#include "../../shadow_amd/csrc/reduce_acc.h"
+
+using namespace shdw;
+
+#define CK(x)                                                                      \
+  do {                                                                             \
+    hipError_t err_ = (x);                                                         \
+    if (err_ != hipSuccess) {                                                      \
+      printf("error: %s at line %d\n", hipGetErrorString(err_), __LINE__);         \
+      return 1;                                                                    \
+    }                                                                              \
+  } while (0)
+
+enum { kCopy = 0, kRead = 1, kWrite = 2 };
+
+// A workgroup covers T * V consecutive vectors; vector u of lane t is first + u * T.
+// STRIDE: the grid is fixed and every workgroup walks the tensor in steps of grid * T * V.
+template <int KIND, int T, int V, bool STRIDE>
+__global__ __launch_bounds__(T) void stream_kernel(const float* a, float* y, uint32_t n4, float val) {
+  const uint32_t step = STRIDE ? gridDim.x * (T * V) : 0xffffffffu;
+  for (uint32_t first = blockIdx.x * (T * V) + threadIdx.x; first < n4; first += step) {
+    v4f v[V];
+    if (KIND != kWrite) {
+#pragma unroll
+      for (int u = 0; u < V; ++u)
+        if (first + u * T < n4) v[u] = load4_stream(a + 4ull * (first + u * T));
+    }
+    if (KIND == kRead) {
+      float s = 0;
+#pragma unroll
+      for (int u = 0; u < V; ++u)
+        if (first + u * T < n4) s += (v[u][0] + v[u][1]) + (v[u][2] + v[u][3]);
+      if (s == val) *y = s;
+    } else {
+#pragma unroll
+      for (int u = 0; u < V; ++u)
+        if (first + u * T < n4) {
+          v4f w;
+          if (KIND == kWrite) w = v4f{val, val, val, val}; else w = v[u];
+          store4_stream(y + 4ull * (first + u * T), w);
+        }
+    }
+    if (!STRIDE) break;
+  }
+}
+
+// The shape of the library's reduce_strided_tile_kernel (reduce.hip), with the
+// workgroup numbering as a template switch.
+template <int OP, int L, bool XCD>
+__global__ __launch_bounds__(512) void tile_kernel(const float* x, float* y, uint32_t reduce, uint32_t inner,
+                                                    FastDiv f_tiles) {
+  constexpr uint32_t kGroups = 512 / L;
+  constexpr int kBatch = 8;
+  __shared__ Partial lds[512 * 4];
+  uint32_t o, tile;
+  fd_divmod(XCD ? xcd_contiguous(blockIdx.x, gridDim.x) : blockIdx.x, f_tiles, o, tile);
+  const uint32_t pl = threadIdx.x % L, rg = threadIdx.x / L;
+  const uint32_t col = (tile * L + pl) * 4;
+  Acc<OP> acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc[j].init();
+  if (col < inner) {
+    const float* p = x + static_cast<size_t>(o) * reduce * inner + col;
+    uint32_t base = rg;
+    for (; base + (kBatch - 1) * kGroups < reduce; base += kBatch * kGroups) {
+      v4f v[kBatch];
+      const bool valid[kBatch] = {true, true, true, true, true, true, true, true};
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) v[u] = load4_stream_any(p + static_cast<size_t>(base + u * kGroups) * inner);
+      fold_batch<kBatch, false>(acc, v, valid, [&](int u, int) { return base + u * kGroups; });
+    }
+    for (; base < reduce; base += kGroups) {
+      const v4f v = load4_stream_any(p + static_cast<size_t>(base) * inner);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j].add(v[j], base);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) lds[threadIdx.x * 4 + j] = acc[j].pack();
+  __syncthreads();
+  if (threadIdx.x < 4 * L) {
+    const uint32_t c = tile * 4 * L + threadIdx.x;
+    Acc<OP> total;
+    total.init();
+    for (uint32_t g = 0; g < kGroups; ++g) {
+      Acc<OP> t;
+      t.unpack(lds[g * 4 * L + threadIdx.x]);
+      total.merge(t);
+    }
+    if (c < inner) y[static_cast<size_t>(o) * inner + c] = total.finalize(reduce);
+  }
+}
+
+static hipEvent_t e0, e1;
+
+// Average time of one launch in us: best of three batches of `reps` back-to-back launches.
+template <class F>
+static int time_us(F launch, int reps, float* us) {
+  for (int i = 0; i < 5; ++i) launch(i);
+  float best = 1e30f;
+  for (int rep = 0; rep < 3; ++rep) {
+    CK(hipEventRecord(e0));
+    for (int i = 0; i < reps; ++i) launch(i);
+    CK(hipEventRecord(e1));
+    CK(hipEventSynchronize(e1));
+    float ms;
+    CK(hipEventElapsedTime(&ms, e0, e1));
+    best = std::min(best, ms);
+  }
+  CK(hipGetLastError());
+  *us = best / reps * 1e3f;
+  return 0;
+}
+
+int main() {
+  const size_t kPool = 6ull * 205520896;
+  float *rp, *wp;
+  CK(hipMalloc(&rp, kPool));
+  CK(hipMalloc(&wp, kPool));
+  CK(hipMemset(rp, 0x3c, kPool));
+  CK(hipEventCreate(&e0));
+  CK(hipEventCreate(&e1));
+
+  printf("# stream: us per launch; total bytes moved = the size given (copy: half read, half written)\n");
+  const size_t sizes[] = {51380224, 411041792};
+  const char* kinds[] = {"copy", "read", "write"};
+  for (size_t total : sizes) {
+    for (int kind = 0; kind < 3; ++kind) {
+      const size_t side = kind == kCopy ? total / 2 : total;
+      const uint32_t n4 = static_cast<uint32_t>(side / 16);
+      const int m = static_cast<int>(std::max<size_t>(1, std::min<size_t>(64, kPool / side)));
+      printf("stream %-5s %3zu MB:", kinds[kind], total / 1000000);
+#define RUN(KIND, T, V, STRIDE)                                                                        \
+  if (kind == KIND) {                                                                                  \
+    const uint32_t grid = STRIDE ? 2048u : (n4 + T * V - 1) / (T * V);                                 \
+    float us;                                                                                          \
+    if (time_us([&](int i) {                                                                           \
+          const size_t off = (i % m) * (side / 4);                                                     \
+          stream_kernel<KIND, T, V, STRIDE><<<grid, T>>>(rp + off, wp + off, n4, 1e30f);               \
+        }, 40, &us)) return 1;                                                                         \
+    printf("  %s%dx%d %.2f", STRIDE ? "stride" : "T", T, V, us);                                       \
+    fflush(stdout);                                                                                    \
+  }
+#define ALLV(KIND, T) RUN(KIND, T, 1, false) RUN(KIND, T, 2, false) RUN(KIND, T, 4, false)
+#define ALL(KIND) ALLV(KIND, 64) ALLV(KIND, 256) ALLV(KIND, 1024) RUN(KIND, 256, 4, true)
+      ALL(kCopy) ALL(kRead) ALL(kWrite)
+      printf("\n");
+    }
+  }
+
+  // strided reduce: [32][512][784], max over the middle extent
+  {
+    const uint32_t outer = 32, reduce = 512, inner = 784;
+    const size_t n = static_cast<size_t>(outer) * reduce * inner;
+    const int sets = 6;
+    std::vector<float> h(n);
+    for (size_t i = 0; i < n; ++i) h[i] = static_cast<float>((i * 2654435761u) >> 8 & 0xffff) / 65536.f - 0.5f;
+    for (int k = 0; k < sets; ++k) CK(hipMemcpy(rp + k * n, h.data(), 4 * n, hipMemcpyHostToDevice));
+    printf("# strided: max over 512 channels of [32,512,28,28], us per launch; L = lanes per row piece (4 L columns per tile)\n");
+    std::vector<float> ref, got(outer * inner);
+#define TILE(L, XCD)                                                                                   \
+  {                                                                                                    \
+    const uint32_t tiles = (inner / 4 + L - 1) / L;                                                    \
+    const FastDiv f = make_fastdiv(tiles);                                                             \
+    float us;                                                                                          \
+    if (time_us([&](int i) {                                                                           \
+          tile_kernel<SHDW_REDUCE_MAX, L, XCD><<<tiles * outer, 512>>>(rp + (i % sets) * n, wp + (i % sets) * n, reduce, inner, f); \
+        }, 40, &us)) return 1;                                                                         \
+    CK(hipMemcpy(got.data(), wp, 4 * outer * inner, hipMemcpyDeviceToHost));                           \
+    if (ref.empty()) ref = got;                                                                        \
+    printf("strided L%-2d %-14s %.2f %s\n", L, XCD ? "xcd-contiguous" : "round-robin", us,             \
+           memcmp(ref.data(), got.data(), 4 * outer * inner) == 0 ? "same" : "DIFFERENT");             \
+  }
+    TILE(32, true) TILE(32, false) TILE(16, true) TILE(16, false) TILE(8, true) TILE(8, false)
+  }
+  return 0;
+}
