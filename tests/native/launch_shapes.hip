@@ -10,6 +10,18 @@
 //   strided : max over the 512 channels of [32,512,28,28] with the library's
 //             column-tile kernel shape, workgroups numbered round-robin over the
 //             8 XCDs (as dispatched) or XCD-contiguously, for three tile widths.
+//   tile    : a plain copy of [64,256,56,56] and [64,512,38,38] in the access
+//             pattern of the channel-tile kernels (Normalize, SSDNormalize, Softmax
+//             over 65..512 channels): a workgroup owns 32 neighbouring positions
+//             with all their channels, i.e. one 128-byte piece of every row of
+//             an image, holds them in registers and writes them back, as 256
+//             lanes with room for 16 vectors each (the library's shape) or 1024
+//             lanes with 4, with streaming or plain stores, and with the tile also
+//             parked in LDS between two barriers as the kernels do; for the
+//             256-channel shape also with room for 8 vectors, which lets eight
+//             instead of five workgroups share a CU.  The same
+//             bytes as a flat copy give the yardstick: what the pattern costs
+//             before any arithmetic.
 //
 // Usage: launch_shapes            (all tables)
 #include <hip/hip_runtime.h>
@@ -113,6 +125,62 @@ __global__ __launch_bounds__(512) void tile_kernel(const float* x, float* y, uin
   }
 }
 
+// The tile of the channel-tile kernels (softmax.hip), as a copy.  PARK: the tile
+// also passes through LDS between two barriers, and the stores depend on it.
+typedef float v4f_any __attribute__((ext_vector_type(4), aligned(4)));
+template <int T, int PER, bool NT, bool PARK>
+__global__ __launch_bounds__(T) void tile_copy_kernel(const float* x, float* y, uint32_t dim, uint32_t inner,
+                                                       FastDiv f_tiles) {
+  extern __shared__ __align__(16) float tile_lds[];
+  constexpr uint32_t TS = 32, LPR = TS / 4, STEP = T / LPR;
+  uint32_t n, tile;
+  fd_divmod(xcd_contiguous(blockIdx.x, gridDim.x), f_tiles, n, tile);
+  const uint32_t p0 = tile * TS;
+  const uint32_t width = min(TS, inner - p0);
+  const uint64_t base = static_cast<uint64_t>(n) * dim * inner + p0;
+  const uint32_t j = (threadIdx.x & (LPR - 1)) * 4, c0 = threadIdx.x / LPR;
+  const bool valid = j + 4 <= width;  // inner is a multiple of 4 here
+  v4f r[PER];
+  if (valid) {
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const uint32_t c = c0 + u * STEP;
+      if (c < dim)
+        r[u] = __builtin_nontemporal_load(reinterpret_cast<const v4f_any*>(x + base + static_cast<uint64_t>(c) * inner + j));
+    }
+  }
+  float m = 1.f;
+  if (PARK) {
+    if (valid) {
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        const uint32_t c = c0 + u * STEP;
+        if (c < dim) *reinterpret_cast<v4f*>(tile_lds + c * TS + j) = r[u];
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < width) {
+      float a = 0.f;
+      for (int c = 0; c < 16; ++c) a += tile_lds[c * TS + threadIdx.x];
+      tile_lds[threadIdx.x] = a;
+    }
+    __syncthreads();
+    m = tile_lds[j] == 12345.f ? 2.f : 1.f;
+  }
+  if (!valid) return;
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const uint32_t c = c0 + u * STEP;
+    if (c >= dim) continue;
+    const v4f q = r[u] * m;
+    float* dst = y + base + static_cast<uint64_t>(c) * inner + j;
+    if (NT)
+      __builtin_nontemporal_store(q, reinterpret_cast<v4f_any*>(dst));
+    else
+      *reinterpret_cast<v4f_any*>(dst) = q;
+  }
+}
+
 static hipEvent_t e0, e1;
 
 // Average time of one launch in us: best of three batches of `reps` back-to-back launches.
@@ -194,6 +262,41 @@ int main() {
            memcmp(ref.data(), got.data(), 4 * outer * inner) == 0 ? "same" : "DIFFERENT");             \
   }
     TILE(32, true) TILE(32, false) TILE(16, true) TILE(16, false) TILE(8, true) TILE(8, false)
+  }
+
+  // channel tiles as a copy: [64][256][3136] (rows start on 64-byte boundaries) and [64][512][1444] (they do not)
+  {
+    printf("# tile: copy of [outer,dim,inner] in the channel-tile pattern, us per launch; flat = the same bytes as a flat copy\n");
+    const uint32_t shapes[2][3] = {{64, 256, 3136}, {64, 512, 1444}};
+    for (const auto& sh : shapes) {
+      const uint32_t outer = sh[0], dim = sh[1], inner = sh[2];
+      const size_t n = static_cast<size_t>(outer) * dim * inner;
+      const int sets = static_cast<int>(kPool / (4 * n));
+      std::vector<float> h(n), got(n);
+      for (size_t i = 0; i < n; ++i) h[i] = static_cast<float>((i * 2654435761u) >> 8 & 0xffff) / 65536.f - 0.5f;
+      for (int k = 0; k < sets; ++k) CK(hipMemcpy(rp + k * n, h.data(), 4 * n, hipMemcpyHostToDevice));
+      const uint32_t n4 = static_cast<uint32_t>(n / 4);
+      float us;
+      if (time_us([&](int i) { stream_kernel<kCopy, 64, 1, false><<<(n4 + 63) / 64, 64>>>(rp + (i % sets) * n, wp + (i % sets) * n, n4, 0.f); }, 20, &us)) return 1;
+      printf("tile [%u,%u,%u] flat %.2f\n", outer, dim, inner, us);
+      const uint32_t tiles = (inner + 31) / 32;
+      const FastDiv f = make_fastdiv(tiles);
+      const size_t lds = static_cast<size_t>(dim) * 32 * sizeof(float);
+#define TILECOPY(T, PER, NT, PARK)                                                                     \
+  {                                                                                                    \
+    CK(hipMemset(wp, 0, 4 * n));                                                                       \
+    if (time_us([&](int i) {                                                                           \
+          tile_copy_kernel<T, PER, NT, PARK><<<tiles * outer, T, PARK ? lds : 0>>>(rp + (i % sets) * n, wp + (i % sets) * n, dim, inner, f); \
+        }, 20, &us)) return 1;                                                                         \
+    CK(hipMemcpy(got.data(), wp, 4 * n, hipMemcpyDeviceToHost));                                       \
+    printf("tile [%u,%u,%u] T%dx%d %-9s %-6s %.2f %s\n", outer, dim, inner, T, PER, NT ? "streaming" : "plain", \
+           PARK ? "parked" : "direct", us, memcmp(h.data(), got.data(), 4 * n) == 0 ? "same" : "DIFFERENT"); \
+  }
+      TILECOPY(256, 16, true, false) TILECOPY(256, 16, false, false) TILECOPY(256, 16, true, true) TILECOPY(256, 16, false, true)
+      TILECOPY(1024, 4, true, false) TILECOPY(1024, 4, false, true)
+      // half the registers per lane: eight instead of five workgroups fit a CU, and the copy gets slower
+      if (dim <= 256) TILECOPY(256, 8, true, false)
+    }
   }
   return 0;
 }

@@ -59,3 +59,30 @@ def test_xcd_contiguous_numbering_of_the_strided_reduce(table):
     t = {(int(l), kind): float(us) for l, kind, us, _ in rows}
     assert t[(32, "xcd-contiguous")] <= SLACK * min(t.values())
     assert t[(32, "xcd-contiguous")] <= 1.02 * t[(32, "round-robin")]
+
+
+def tile_rows(table):
+    flat, rows = {}, {}
+    for line in table.splitlines():
+        m = re.match(r"tile \[(\d+),(\d+),(\d+)\] flat (\d+\.\d+)", line)
+        if m:
+            flat[int(m.group(3))] = float(m.group(4))
+        m = re.match(r"tile \[(\d+),(\d+),(\d+)\] (T\d+x\d+) (\w+)\s+(\w+)\s+(\d+\.\d+) (\w+)", line)
+        if m:
+            assert m.group(8) == "same", line
+            rows[(int(m.group(3)), m.group(4), m.group(5), m.group(6))] = float(m.group(7))
+    return flat, rows
+
+
+def test_channel_tile_shape_in_use_and_what_the_pattern_costs(table):
+    """The channel-tile kernels use 256 lanes, streaming stores where the rows start on
+    64-byte boundaries and plain ones elsewhere, and park the tile in LDS.  As a pure
+    copy that shape is within the slack of the alternatives, LDS and barriers included,
+    and the pattern itself stays well behind a flat copy of the same bytes: that, not
+    the folds, bounds those kernels."""
+    flat, rows = tile_rows(table)
+    assert len(rows) == 13
+    for inner, used in ((3136, ("T256x16", "streaming", "parked")), (1444, ("T256x16", "plain", "parked"))):
+        mine = {k[1:]: v for k, v in rows.items() if k[0] == inner}
+        assert mine[used] <= SLACK * min(mine.values()), (inner, mine)
+        assert min(mine.values()) > 1.10 * flat[inner], (inner, flat[inner], mine)
