@@ -623,8 +623,8 @@ static void launch_normalize_tile(int outer_num, int dim, int inner_num, float p
     launch_normalize_tile_ts<PMODE, SM, 5>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
 }
 
-// Softmax on the same tile layout (65 <= dim <= 510 so that the exp table fits
-// beside the tile).  The lanes hold x, later exp(x - max), in registers; the tile
+// Softmax on the same tile layout (65 <= dim <= 512; the exp table lies behind
+// the tile).  The lanes hold x, later exp(x - max), in registers; the tile
 // in LDS serves wave 0's two serial folds: the running maximum of x, then the
 // fp32 running sum of the exponentials, both in index order.  The maxima and
 // then the sums are handed over in the first tile row.
@@ -681,7 +681,7 @@ __global__ __launch_bounds__(kBlock) void softmax_tile_kernel(const float* x, fl
 }
 
 constexpr size_t kExpTabBytes = 32 * sizeof(uint64_t);
-constexpr int kSoftmaxTileMaxDim = (kTileLdsBytes - kExpTabBytes) / (32 * sizeof(float));  // 32 positions + the exp table <= 64 KB: 510
+constexpr int kSoftmaxTileMaxDim = kTileMaxDim;  // 32 positions of 512 channels plus the exp table: 64 KB + 256 bytes, two workgroups per CU all the same
 
 template <int TS_SHIFT>
 static void launch_softmax_tile_ts(int outer_num, int dim, int inner_num, const float* x, float* y,
