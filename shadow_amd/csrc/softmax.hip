@@ -615,7 +615,7 @@ static void launch_normalize_tile(int outer_num, int dim, int inner_num, float p
   // workgroups per CU), else 32, up to 64 KB: rows of 16 positions (64 bytes)
   // cost more than the lower occupancy does.  [64,256,56,56]: 85 us with 64
   // positions (64 KB), 80 us with 32; [64,512,38,38]: 105 us with 32 (64 KB),
-  // 115 us with 16.  Softmax, with its five barriers per tile, takes the widest
+  // 115 us with 16.  Softmax, with its four barriers per tile, takes the widest
   // tile that fits.
   if (dim * 64 * sizeof(float) <= kTileLdsBytes / 2)
     launch_normalize_tile_ts<PMODE, SM, 6>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
@@ -623,37 +623,83 @@ static void launch_normalize_tile(int outer_num, int dim, int inner_num, float p
     launch_normalize_tile_ts<PMODE, SM, 5>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
 }
 
-// Softmax on the same tile layout (65 <= dim <= 512; the exp table lies behind
-// the tile).  The lanes hold x, later exp(x - max), in registers; the tile
-// in LDS serves wave 0's two serial folds: the running maximum of x, then the
-// fp32 running sum of the exponentials, both in index order.  The maxima and
-// then the sums are handed over in the first tile row.
+// Softmax on the same tile layout (65 <= dim <= 512).  The lanes hold x, later
+// exp(x - max), in registers.  Behind the tile lie the exp table, a row that
+// hands the maxima and later the sums over, and a flag.
+//
+// The running maximum max = std_max(x[c], max), started at -FLT_MAX, is the
+// largest element whatever the order as long as no element is NaN (a NaN takes
+// the maximum over and the next element takes it back, so then the order
+// counts; which of two zeros wins does not change exp(x - max)).  Every lane
+// therefore takes the maximum of its own rows, the STEP partial maxima per
+// position meet in the first tile rows and one lane per position folds them; a
+// lane that met a NaN hands a NaN over instead, and a tile with one anywhere
+// parks x and walks the columns in index order like the sums.  The sum of the
+// exponentials is an fp32 running sum and always walks.
 template <int TS_SHIFT, int ROWS>
 __global__ __launch_bounds__(kBlock) void softmax_tile_kernel(const float* x, float* y, uint32_t dim,
                                                                uint32_t inner, FastDiv f_tiles) {
   extern __shared__ __align__(16) float lds[];
   constexpr uint32_t TS = 1u << TS_SHIFT;
+  using Lane = TileLane<TS_SHIFT, ROWS>;
   uint64_t* tab = reinterpret_cast<uint64_t*>(lds + (dim << TS_SHIFT));  // after the tile, 16-byte aligned
+  float* handed = reinterpret_cast<float*>(tab + 32);
+  uint32_t* any_nan = reinterpret_cast<uint32_t*>(handed + TS);
   if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
   uint32_t n, tile;
   fd_divmod(xcd_contiguous(blockIdx.x, gridDim.x), f_tiles, n, tile);
   const uint32_t p0 = tile << TS_SHIFT;
   const uint32_t width = min(TS, inner - p0);
   const uint64_t base = static_cast<uint64_t>(n) * dim * inner + p0;
-  const TileLane<TS_SHIFT, ROWS> lane(width, dim, inner);
+  const Lane lane(width, dim, inner);
   v4f r[kTilePerLane];
   lane.load(x + base, r);
-  lane.park(lds, r);
-  __syncthreads();
-  if (threadIdx.x < width) {
-    const float* column = lds + threadIdx.x;
-    lds[threadIdx.x] = fold_tile_column<TS_SHIFT>(column, dim, -FLT_MAX,
-                                                  [](float m, float v) { return std_max(v, m); });
+  if (lane.valid != 0) {
+    v4f m = {-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+    bool nan[4] = {false, false, false, false};
+#pragma unroll
+    for (int u = 0; u < kTilePerLane; ++u) {
+      if (lane.c0 + u * Lane::STEP >= dim) continue;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float v = r[u][k];
+        nan[k] |= v != v;
+        m[k] = m[k] < v ? v : m[k];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) m[k] = nan[k] ? __builtin_nanf("") : m[k];
+    *reinterpret_cast<v4f*>(lds + (lane.c0 << TS_SHIFT) + lane.j) = m;  // row c0 < STEP <= 64 < dim
   }
   __syncthreads();
-  const v4f m = *reinterpret_cast<const v4f*>(lds + lane.j);
-  __syncthreads();  // the maxima are read before the exponentials overwrite their row
+  if (threadIdx.x < kWave) {  // all of wave 0, so that its lanes agree on the flag
+    float m = -FLT_MAX;
+    bool nan = false;
+    if (threadIdx.x < width) {
+      const uint32_t groups = min(Lane::STEP, dim);
+      for (uint32_t g = 0; g < groups; ++g) {
+        const float v = lds[(g << TS_SHIFT) + threadIdx.x];
+        nan |= v != v;
+        m = m < v ? v : m;
+      }
+      handed[threadIdx.x] = m;
+    }
+    const uint64_t seen = __builtin_amdgcn_ballot_w64(nan);
+    if (threadIdx.x == 0) *any_nan = seen != 0;
+  }
+  __syncthreads();
+  if (*any_nan != 0) {  // the whole workgroup: the maxima in index order
+    lane.park(lds, r);
+    __syncthreads();
+    if (threadIdx.x < width) {
+      const float* column = lds + threadIdx.x;
+      handed[threadIdx.x] = fold_tile_column<TS_SHIFT>(column, dim, -FLT_MAX,
+                                                      [](float m, float v) { return std_max(v, m); });
+    }
+    __syncthreads();
+  }
   if (lane.valid != 0) {
+    const v4f m = *reinterpret_cast<const v4f*>(handed + lane.j);
 #pragma unroll
     for (int u = 0; u < kTilePerLane; ++u) {
       if (lane.c0 + u * lane.STEP >= dim) continue;
@@ -662,14 +708,14 @@ __global__ __launch_bounds__(kBlock) void softmax_tile_kernel(const float* x, fl
     }
   }
   lane.park(lds, r);
-  __syncthreads();
+  __syncthreads();  // also: every lane has its maxima before the sums replace them
   if (threadIdx.x < width) {
     const float* column = lds + threadIdx.x;
-    lds[threadIdx.x] = fold_tile_column<TS_SHIFT>(column, dim, 0.f, [](float a, float v) { return a + v; });
+    handed[threadIdx.x] = fold_tile_column<TS_SHIFT>(column, dim, 0.f, [](float a, float v) { return a + v; });
   }
   __syncthreads();
   if (lane.valid == 0) return;
-  const v4f d = *reinterpret_cast<const v4f*>(lds + lane.j);
+  const v4f d = *reinterpret_cast<const v4f*>(handed + lane.j);
 #pragma unroll
   for (int u = 0; u < kTilePerLane; ++u) {
     if (lane.c0 + u * lane.STEP >= dim) continue;
@@ -681,6 +727,7 @@ __global__ __launch_bounds__(kBlock) void softmax_tile_kernel(const float* x, fl
 }
 
 constexpr size_t kExpTabBytes = 32 * sizeof(uint64_t);
+constexpr size_t kSoftmaxTileExtraBytes = kExpTabBytes + 64 * sizeof(float) + 16;  // table, hand-over row, flag
 constexpr int kSoftmaxTileMaxDim = kTileMaxDim;  // 32 positions of 512 channels plus the exp table: 64 KB + 256 bytes, two workgroups per CU all the same
 
 template <int TS_SHIFT>
@@ -688,7 +735,7 @@ static void launch_softmax_tile_ts(int outer_num, int dim, int inner_num, const 
                                    hipStream_t st) {
   const uint32_t tiles = (static_cast<uint32_t>(inner_num) + (1u << TS_SHIFT) - 1) >> TS_SHIFT;
   const uint32_t grid = static_cast<uint32_t>(outer_num) * tiles;
-  const size_t bytes = (static_cast<size_t>(dim) << TS_SHIFT) * sizeof(float) + kExpTabBytes;
+  const size_t bytes = (static_cast<size_t>(dim) << TS_SHIFT) * sizeof(float) + kSoftmaxTileExtraBytes;
   const uint32_t d = static_cast<uint32_t>(dim), in = static_cast<uint32_t>(inner_num);
   const FastDiv ft = make_fastdiv(tiles);
   switch (tile_rows(inner_num, y)) {
@@ -746,7 +793,7 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
     else
       softmax_columns_reg_kernel<64, 48><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi);
   }
-  else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner && dim * 64 * sizeof(float) + kExpTabBytes <= kTileLdsBytes)
+  else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner && dim * 64 * sizeof(float) <= kTileLdsBytes - 1024)
     launch_softmax_tile_ts<6>(outer_num, dim, inner_num, x, y, st);
   else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner)
     launch_softmax_tile_ts<5>(outer_num, dim, inner_num, x, y, st);

@@ -111,6 +111,23 @@ def test_softmax_special_values(gpu, outer, dim, inner):
     assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax specials")
 
 
+# A NaN takes the running maximum over and the next element takes it back, so with
+# NaNs in a column the order of the walk shows in the result (first, middle and last
+# row, several in one column); the tile kernel takes the maxima in parallel only where
+# the tile holds none.  Both tile widths, ragged rows, tiles with and without NaNs.
+@pytest.mark.parametrize("outer,dim,inner", [(2, 80, 100), (1, 150, 333), (2, 300, 70), (1, 512, 41), (3, 66, 16)])
+def test_softmax_with_nans_in_the_columns(gpu, outer, dim, inner):
+    x = normal(23, (outer, dim, inner), 4.0)
+    x[0, 0, 1] = np.nan
+    x[0, dim - 1, 5] = np.nan
+    x[0, dim // 2, 9] = np.nan
+    x[0, 3, 13] = x[0, dim - 2, 13] = x[0, 40, 13] = np.nan
+    x[outer - 1, 17, inner - 1] = np.nan
+    x[0, :, 15] = np.nan
+    x = x.reshape(-1)
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax with NaNs")
+
+
 # Spreads wide enough for exp to reach tiny, denormal and zero results, next to
 # ordinary columns, in each kernel layout.
 @pytest.mark.parametrize("outer,dim,inner", [(3, 40, 1), (2, 12, 200), (2, 48, 130), (2, 150, 300), (1, 100, 70),
