@@ -24,6 +24,11 @@ inline int launch_status() { return static_cast<int>(hipGetLastError()); }
 // device; returns 0 or an error code.
 int library_scratch_prepare();
 
+// Max over every row of x [rows][len] with Reduce's kernels (reduce.hip), if that
+// takes a single stage and so no workspace: then *rc holds the launch result and
+// the return value is true.
+bool reduce_rows_max(uint32_t rows, uint32_t len, const float* x, float* y, hipStream_t st, int* rc);
+
 }  // namespace shdw
 
 #endif  // SHADOW_AMD_CSRC_LAUNCH_H_

@@ -662,6 +662,16 @@ static int dispatch_reduce(int operation, const ReducePlan& pl, const float* x, 
 
 using namespace shdw;
 
+// Max over every row of x [rows][len] when that needs no workspace (enough rows
+// for a single stage): for the whole-plane max pooling, whose walk is the same.
+bool shdw::reduce_rows_max(uint32_t rows, uint32_t len, const float* x, float* y, hipStream_t st, int* rc) {
+  const int shape[2] = {static_cast<int>(rows), static_cast<int>(len)}, axes[1] = {1};
+  ReducePlan pl;
+  if (plan_reduce(2, shape, 1, axes, &pl) != SHDW_OK || reduce_workspace_bytes(pl) != 0) return false;
+  *rc = dispatch_reduce(SHDW_REDUCE_MAX, pl, x, y, nullptr, 0, st);
+  return true;
+}
+
 extern "C" {
 
 int shdw_hip_reduce(int operation, int num_axes, const int* in_shape, int num_reduce,

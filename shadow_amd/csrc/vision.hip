@@ -502,6 +502,132 @@ static void launch_pool_plane(const float* x, float* y, uint32_t rows, uint32_t 
   pool_plane_kernel<MAX><<<grid, kBlock, 0, st>>>(x, y, rows, len, group, chunk, fc, fl, size);
 }
 
+// Whole-plane average over rows of any length, without a barrier: every wave of a
+// workgroup works by itself on G consecutive rows, which it walks in chunks of
+// W = 4096 / G columns.  All lanes fetch a chunk (16 vectors each, 16 KB per wave)
+// and lay it down in the wave's LDS rows; lane g < G then adds row g's columns in
+// index order (an fp32 running sum has no other order; a dependent addition takes
+// six clocks, so a row of 3136 takes 8 us whatever else happens) while the next
+// chunk is already on its way.  A wave never waits for another wave, so a CU's
+// eight resident waves overlap each other's fetches and folds.  G shrinks as the
+// rows get longer and fewer: what matters is enough waves in flight (16 KB each)
+// to cover HBM's latency, not how many lanes of a wave fold.  The four waves of a
+// workgroup exist for their placement only: one per SIMD.  Single-wave
+// workgroups were measured to pile up on one SIMD of a CU when only four of
+// them fit the launch, and waves that share a SIMD take turns at every addition.
+// The LDS pitch of W + 4 floats keeps 128-bit accesses aligned and puts the
+// folding lanes on distinct banks.
+constexpr int kStreamVectors = 16;  // per lane and chunk
+constexpr int kStreamWaves = kBlock / kWave;
+
+template <int G>
+__global__ __launch_bounds__(kBlock) void pool_rows_stream_kernel(const float* x, float* y, uint32_t rows,
+                                                                   uint32_t len, float pool_size) {
+  constexpr uint32_t W = 256u * kStreamVectors / G, VW = W / 4, PITCH = W + 4;
+  __shared__ __align__(16) float tiles[kStreamWaves * G * PITCH];
+  const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  float* tile = tiles + wave * (G * PITCH);
+  const uint32_t row0 = (blockIdx.x * kStreamWaves + wave) * G;
+  if (row0 >= rows) return;  // the whole wave
+  v4f reg[kStreamVectors];
+  auto request = [&](uint32_t c0) {
+#pragma unroll
+    for (int i = 0; i < kStreamVectors; ++i) {
+      const uint32_t v = lane + kWave * i;
+      const uint32_t g = v / VW, c = c0 + 4 * (v % VW);
+      if (row0 + g >= rows || c >= len) continue;
+      const float* src = x + static_cast<uint64_t>(row0 + g) * len + c;
+      if (c + 4 <= len) {
+        reg[i] = __builtin_nontemporal_load(reinterpret_cast<const v4f_unaligned*>(src));
+      } else {
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+          if (c + k < len) reg[i][k] = __builtin_nontemporal_load(src + k);
+      }
+    }
+  };
+  float sum = 0.f;
+  request(0);
+  for (uint32_t c0 = 0; c0 < len; c0 += W) {
+#pragma unroll
+    for (int i = 0; i < kStreamVectors; ++i) {
+      const uint32_t v = lane + kWave * i;
+      *reinterpret_cast<v4f*>(tile + (v / VW) * PITCH + 4 * (v % VW)) = reg[i];
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (c0 + W < len) request(c0 + W);
+    if (lane < G) {
+      const uint32_t cols = min(W, len - c0);
+      const float* mine = tile + lane * PITCH;
+      // 32 values per step and two steps per turn, each step's values requested
+      // one step ahead: the additions, not the LDS latency, set the pace.
+      constexpr int kAhead = 8, kStep = 4 * kAhead;
+      uint32_t c = 0;
+      if (cols >= kStep) {
+        v4f q[kAhead], w[kAhead];
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) q[k] = *reinterpret_cast<const v4f*>(mine + 4 * k);
+        for (c = kStep; c + 2 * kStep <= cols; c += 2 * kStep) {
+#pragma unroll
+          for (int k = 0; k < kAhead; ++k) w[k] = *reinterpret_cast<const v4f*>(mine + c + 4 * k);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int k = 0; k < kStep; ++k) sum += q[k / 4][k % 4];
+#pragma unroll
+          for (int k = 0; k < kAhead; ++k) q[k] = *reinterpret_cast<const v4f*>(mine + c + kStep + 4 * k);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int k = 0; k < kStep; ++k) sum += w[k / 4][k % 4];
+        }
+#pragma unroll
+        for (int k = 0; k < kStep; ++k) sum += q[k / 4][k % 4];
+      }
+      for (; c < cols; ++c) sum += mine[c];
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (lane < G && row0 + lane < rows) y[row0 + lane] = sum / pool_size;
+}
+
+// From this row length on the whole-plane average takes the streaming kernel
+// (per 51 MB, against pool_plane_kernel: 28x28 planes 15.1 / 23.5 us, 56x56 planes
+// 24.6 / 59 us; 14x14 planes 13.2 / 14.2 us but 45.8 / 42.0 us per 205 MB, 7x7 planes
+// 12.6 / 12.7 and 44.1 / 39.6 us).
+constexpr int kPlaneStreamMinLen = 256;
+// ... and from this many rows on: a wave per row needs rows to fill the chip
+// (256 planes of 112x112: 168 us against 99 us).
+constexpr uint32_t kPlaneStreamMinRows = 512;
+
+// From this row length on the whole-plane maximum goes to Reduce's row kernels
+// (rows of 49: 14.4 us there against 13.1 us here per 51 MB; rows of 196: 11.2 against 16.5).
+constexpr int kPlaneMaxByReduce = 128;
+
+// Rows per wave: about 2048 waves in all (eight per CU, what their LDS lets reside
+// at once, two per SIMD), so long and few rows get a wave each.  Measured per
+// 51 MB: 28x28 planes 15.1 us with 8 rows per wave (20.0 with 4, 16.1 with 16),
+// 56x56 planes 24.6 us with 2 (39 with 1 or 4).
+static int stream_rows_per_wave(uint32_t rows) {
+  int g = 1;
+  while (g < 64 && rows / static_cast<uint32_t>(2 * g) >= 2048u) g <<= 1;
+  return g;
+}
+
+static void launch_pool_rows_stream(const float* x, float* y, uint32_t rows, uint32_t len, hipStream_t st) {
+  const float size = static_cast<float>(static_cast<int>(len));
+  const int g = stream_rows_per_wave(rows);
+  const uint32_t per_wg = static_cast<uint32_t>(g) * kStreamWaves;
+  const uint32_t grid = (rows + per_wg - 1) / per_wg;
+  switch (g) {
+    case 64: pool_rows_stream_kernel<64><<<grid, kBlock, 0, st>>>(x, y, rows, len, size); break;
+    case 32: pool_rows_stream_kernel<32><<<grid, kBlock, 0, st>>>(x, y, rows, len, size); break;
+    case 16: pool_rows_stream_kernel<16><<<grid, kBlock, 0, st>>>(x, y, rows, len, size); break;
+    case 8: pool_rows_stream_kernel<8><<<grid, kBlock, 0, st>>>(x, y, rows, len, size); break;
+    case 4: pool_rows_stream_kernel<4><<<grid, kBlock, 0, st>>>(x, y, rows, len, size); break;
+    case 2: pool_rows_stream_kernel<2><<<grid, kBlock, 0, st>>>(x, y, rows, len, size); break;
+    default: pool_rows_stream_kernel<1><<<grid, kBlock, 0, st>>>(x, y, rows, len, size);
+  }
+}
+
 static int check_pool_dims(int n, const int* in_shape, const int* out_shape) {
   int64_t in_count = 1, out_count = 1;
   for (int k = 0; k < n; ++k) {
@@ -537,10 +663,17 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
   }
   if (whole_plane && plane >= 8) {
     const uint32_t rows = static_cast<uint32_t>(out_count);
-    if (pool_type == 0)
+    if (pool_type == 0) {
+      // The running maximum of a plane is Reduce's Max over a row: the same
+      // std::max(v, x) walk from -FLT_MAX, which that kernel takes in parallel.
+      int rc = SHDW_OK;
+      if (plane >= kPlaneMaxByReduce && reduce_rows_max(rows, static_cast<uint32_t>(plane), x, y, st, &rc)) return rc;
       launch_pool_plane<true>(x, y, rows, static_cast<uint32_t>(plane), st);
-    else
+    } else if (plane >= kPlaneStreamMinLen && rows >= kPlaneStreamMinRows) {
+      launch_pool_rows_stream(x, y, rows, static_cast<uint32_t>(plane), st);
+    } else {
       launch_pool_plane<false>(x, y, rows, static_cast<uint32_t>(plane), st);
+    }
     return launch_status();
   }
 

@@ -297,7 +297,13 @@ def test_pooling3d_op(ws, pool, shape, kernel, stride, pad):
 # whole-plane windows: both workgroup shapes, chunked and unchunked rows, ragged last group
 @pytest.mark.parametrize("pool", [0, 1])
 @pytest.mark.parametrize("shape", [(4, 128, 7, 7), (3, 5, 14, 14), (2, 3, 56, 56), (1, 70, 3, 3), (2, 2, 4, 2),
-                                   (130, 2048, 7, 7), (2, 9, 10, 10), (1, 3, 2, 7, 7), (2, 65, 13, 15)])
+                                   (130, 2048, 7, 7), (2, 9, 10, 10), (1, 3, 2, 7, 7), (2, 65, 13, 15),
+                                   # planes of 256 elements and more: the streaming average with 1, 2, 8, 32
+                                   # and 64 rows per wave, one chunk and several, odd lengths, ragged last
+                                   # wave and workgroup; the maximum by Reduce's row kernels or, with few rows,
+                                   # by the plane kernel
+                                   (20, 30, 17, 17), (8, 64, 70, 70), (13, 41, 129, 65), (40, 128, 16, 16),
+                                   (64, 300, 18, 18), (71, 1023, 16, 17), (300, 1024, 16, 16), (1, 1, 16, 16)])
 def test_global_pooling_op(ws, pool, shape):
     x = normal(22, shape, 2.0)
     got = run(ws, "Pooling", [("x", x)], {"pool": pool, "global_pooling": True})
