@@ -602,6 +602,14 @@ def config_table(dev, sets_scale=1, cpu=None):
     ms = time_median(dev, lambda k: lib.shdw_hip_pooling2d(I(gin2), 1, 14, 14, 1, 1, 0, 0, I(gout2), A[k].ptr,
                                                            Y[k].ptr, st), SETS)
     add("next", "pooling_global_avg_14x14", 4 * NBIG, 4 * 65536, ms, NBIG)
+    ms = time_median(dev, lambda k: lib.shdw_hip_pooling2d(I(gin2), 0, 14, 14, 1, 1, 0, 0, I(gout2), A[k].ptr,
+                                                           Y[k].ptr, st), SETS)
+    add("next", "pooling_global_max_14x14 (Reduce's row kernel)", 4 * NBIG, 4 * 65536, ms, NBIG)
+    for gshape in ([32, 512, 28, 28], [16, 256, 56, 56]):  # squeeze-and-excitation stages: long planes
+        gside, grows = gshape[2], gshape[0] * gshape[1]
+        ms = time_median(dev, lambda k: lib.shdw_hip_pooling2d(I(gshape), 1, gside, gside, 1, 1, 0, 0,
+                                                               I(gshape[:2] + [1, 1]), A[k].ptr, Y[k].ptr, st), SETS)
+        add("next", "pooling_global_avg_%dx%d (streamed rows)" % (gside, gside), 4 * NBIG, 4 * grows, ms, NBIG)
     # [16, 49, 128, 128]: channel softmax / L2 normalize of a dense map (inner = 16384)
     ms = time_median(dev, lambda k: lib.shdw_hip_softmax(16, 49, 16384, A[k].ptr, Y[k].ptr, st), SETS)
     add("next", "softmax_channels_dense", 4 * NBIG, 4 * NBIG, ms, NBIG)

@@ -263,9 +263,10 @@ __global__ __launch_bounds__(LANES <= kWave ? kBlock : LANES, LANES == kBigBlock
 constexpr int kNormLdsMaxInner = 256;
 
 // PADDED: inner % 4 == 0.  Such rows would start on the same few LDS banks (rows
-// of 64 or 128 floats: all on one), so they get a pitch of inner + 4 floats (the
-// 128-bit copies then never cross a row end); other row lengths are copied as
-// they lie.  The pieces are an odd number of elements long for the same reason.
+// of 64 or 128 floats: all on one), so their pitch is the next odd number of
+// 128-bit pieces, inner + 4 or inner + 8 floats (the 128-bit copies then never
+// cross a row end, and 16 neighbouring rows start on 16 different banks); other
+// row lengths are copied as they lie.  The pieces are an odd number of elements long for the same reason.
 template <int L, bool PADDED>
 __global__ __launch_bounds__(kBlock) void norm_rows_lds_kernel(const float* x, float* y, NormArgs p,
                                                                 uint32_t seg, FastDiv f_inner4) {
@@ -273,7 +274,7 @@ __global__ __launch_bounds__(kBlock) void norm_rows_lds_kernel(const float* x, f
   __shared__ __align__(16) float tile[kRows * (16 * L + 4)];  // 16 to 17 KB: inner <= 16 L
   __shared__ float sc[16 * L], bi[16 * L];                   // LayerNorm: scale and bias by row position
   const uint32_t inner = p.inner;
-  const uint32_t pitch = PADDED ? inner + 4 : inner;
+  const uint32_t pitch = PADDED ? 4 * ((inner / 4 + 1) | 1u) : inner;  // an odd number of 128-bit pieces
   const uint32_t row0 = blockIdx.x * kRows;
   const uint32_t nrows = min(kRows, p.outer - row0);
   const uint64_t base = static_cast<uint64_t>(row0) * inner;
@@ -284,7 +285,7 @@ __global__ __launch_bounds__(kBlock) void norm_rows_lds_kernel(const float* x, f
   auto slot = [&](uint32_t v) -> uint32_t {
     if (!PADDED) return 4 * v;
     const uint32_t r = fd_div(v, f_inner4);  // inner / 4 vectors per row
-    return 4 * v + 4 * r;
+    return 4 * v + (pitch - inner) * r;
   };
   for (uint32_t v0 = 0; v0 < nvec; v0 += 4 * kBlock) {
     v4f reg[4];

@@ -134,70 +134,131 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const float* 
 }
 
 // ---------------------------------------------------------------------------
-// rows shorter than 128 floats whose length is not a multiple of four (7x7 and
-// 5x5 planes, 3x3 windows): a group of lanes per row leaves lanes idle (a row of
-// 49 uses 13 of 16, a row of 9 three) and needs a second, 4-byte load for the
-// row ends.  Here a workgroup's rows, one contiguous span of x, pass through LDS:
-// every lane copies 128-bit pieces of the span (on whatever dword address it
-// starts) into rows of odd pitch, then lane r folds row r from LDS, eight reads
-// in flight, on distinct banks.  Mean over the 7x7 planes of [128,2048,7,7]:
-// 18.4 us with 16 lanes per row.
+// rows of up to 255 floats (7x7 and 5x5 planes, 3x3 and 4x4 windows): a group of
+// 16 lanes per row leaves lanes idle (a row of 49 uses 13 of 16, a row of 16
+// four) and, where the length is no multiple of four, needs a second, 4-byte
+// load for the row ends.  Here a workgroup's 256 / L rows, one contiguous span
+// of x, pass through LDS (128-bit copies on whatever dword address the span
+// starts), and L = 1, 2, 4, 8 or 16 lanes share a row, each folding its own piece of
+// at most 17 elements (an odd number, so that the lanes of a row start on
+// different banks); the L partial results meet by DPP.  PADDED (length a
+// multiple of four): such rows would start on the same few banks, so their pitch
+// is the next odd number of 128-bit pieces (rows of 12 at a pitch of 16 floats:
+// 15.4 us per 51 MB, at 20 floats: see below), which the 128-bit copies never
+// straddle; other lengths are copied as they lie.  Per 51 MB: mean over 7x7 planes 18.4 us with
+// 16 lanes per row from global memory, 12.8 us with one lane per row from 49 KB
+// tiles, 9.4 us here; max over 4x4 windows 56 us with 16 lanes per row.
 // ---------------------------------------------------------------------------
-constexpr int kShortRowTileFloats = 12608;  // 256 rows x 49
-constexpr int kShortRowBatch = 8;
+constexpr int kShortRowMaxFloats = 5120;  // 256 / L rows of at most 16 L (+ 4) floats
+constexpr uint32_t kShortRowMaxLen = 256;  // rows up to 255 floats: 16 lanes each
 
-template <int OP>
+template <int OP, int L, bool PADDED>
 __global__ __launch_bounds__(kBlock) void reduce_rows_lds_kernel(const float* x, float* y, uint32_t rows,
-                                                                  uint32_t reduce, uint32_t group,
-                                                                  FastDiv f_reduce) {
-  __shared__ float tile[kShortRowTileFloats];
-  const uint32_t row0 = blockIdx.x * group;
-  const uint32_t nrows = min(group, rows - row0);
-  const uint32_t pitch = reduce | 1u;
+                                                                  uint32_t reduce, uint32_t seg,
+                                                                  FastDiv f_reduce4) {
+  constexpr uint32_t kRows = kBlock / L;
+  __shared__ __align__(16) float tile[kShortRowMaxFloats];
+  const uint32_t pitch = PADDED ? 4 * ((reduce / 4 + 1) | 1u) : reduce;  // an odd number of 128-bit pieces
+  const uint32_t row0 = blockIdx.x * kRows;
+  const uint32_t nrows = min(kRows, rows - row0);
   const float* base = x + static_cast<uint64_t>(row0) * reduce;
   const uint32_t cells = nrows * reduce, nvec = cells / 4;
-  for (uint32_t v0 = 0; v0 < nvec; v0 += kShortRowBatch * kBlock) {
-    v4f reg[kShortRowBatch];
+  for (uint32_t v0 = 0; v0 < nvec; v0 += 4 * kBlock) {  // nvec may be 0: a last workgroup with under four elements
+    v4f reg[4];
 #pragma unroll
-    for (int k = 0; k < kShortRowBatch; ++k) {
+    for (int k = 0; k < 4; ++k) {
       const uint32_t v = min(v0 + k * kBlock + threadIdx.x, nvec - 1);  // past the end: the last piece again
       reg[k] = load4_stream_any(base + 4ull * v);
     }
 #pragma unroll
-    for (int k = 0; k < kShortRowBatch; ++k) {
+    for (int k = 0; k < 4; ++k) {
       const uint32_t v = v0 + k * kBlock + threadIdx.x;
       if (v < nvec) {
-        uint32_t r, c;
-        fd_divmod(4 * v, f_reduce, r, c);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          tile[r * pitch + c] = reg[k][j];
-          if (++c == reduce) c = 0, ++r;
-        }
+        const uint32_t slot = PADDED ? 4 * v + (pitch - reduce) * fd_div(v, f_reduce4) : 4 * v;  // reduce / 4 vectors per row
+        *reinterpret_cast<v4f*>(tile + slot) = reg[k];
       }
     }
   }
-  if (threadIdx.x < (cells & 3u)) {
-    const uint32_t t = 4 * nvec + threadIdx.x;
-    uint32_t r, c;
-    fd_divmod(t, f_reduce, r, c);
-    tile[r * pitch + c] = base[t];
-  }
+  if (!PADDED && threadIdx.x < (cells & 3u)) tile[4 * nvec + threadIdx.x] = base[4 * nvec + threadIdx.x];
   __syncthreads();
-  if (threadIdx.x >= nrows) return;
-  const float* mine = tile + threadIdx.x * pitch;
+  // rows past the end fold whatever the tile holds and store nothing: the lanes
+  // of a wave stay together for the exchanges
+  const uint32_t r = threadIdx.x / L, h = threadIdx.x % L;
+  const uint32_t c_begin = min(h * seg, reduce), c_end = min(c_begin + seg, reduce);
+  const float* mine = tile + (r < nrows ? r : 0) * pitch;
   Acc<OP> acc;
   acc.init();
-  uint32_t c = 0;
-  for (; c + kShortRowBatch <= reduce; c += kShortRowBatch) {
-    float v[kShortRowBatch];
+  uint32_t c = c_begin;
+  for (; c + 4 <= c_end; c += 4) {
+    float v[4];
 #pragma unroll
-    for (int k = 0; k < kShortRowBatch; ++k) v[k] = mine[c + k];
+    for (int k = 0; k < 4; ++k) v[k] = mine[c + k];
 #pragma unroll
-    for (int k = 0; k < kShortRowBatch; ++k) acc.add(v[k], c + k);
+    for (int k = 0; k < 4; ++k) acc.add(v[k], c + k);
   }
-  for (; c < reduce; ++c) acc.add(mine[c], c);
-  y[row0 + threadIdx.x] = acc.finalize(reduce);
+  for (; c < c_end; ++c) acc.add(mine[c], c);
+  if (L > 1) acc = group_allreduce<Acc<OP>, (L > 1 ? L : 2)>(acc);
+  if (h == 0 && r < nrows) y[row0 + r] = acc.finalize(reduce);
+}
+
+// ---------------------------------------------------------------------------
+// strided over a short reduced extent (a sum over a batch of 8, a max over 4
+// maps): the column-tile kernels below give a tile 16 or more row groups and an
+// LDS fold, which rows this few leave idle ([4][3.2M]: sum 32 us, max 71 us per
+// 51 MB).  Here a lane owns four neighbouring columns (one, where the column
+// count is no multiple of four) and walks the rows itself, eight loads in
+// flight; nothing is exchanged.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kShortStridedMaxReduce = 32;
+
+template <int OP, bool VEC>
+__global__ __launch_bounds__(kBlock) void reduce_strided_short_kernel(const float* x, float* y, uint32_t reduce,
+                                                                       uint32_t inner, uint32_t units,
+                                                                       FastDiv f_units_per_outer) {
+  constexpr int W = VEC ? 4 : 1;
+  const uint32_t u = blockIdx.x * kBlock + threadIdx.x;
+  if (u >= units) return;
+  uint32_t o, c;
+  fd_divmod(u, f_units_per_outer, o, c);
+  const float* p = x + static_cast<uint64_t>(o) * reduce * inner + static_cast<uint64_t>(c) * W;
+  Acc<OP> acc[W];
+#pragma unroll
+  for (int j = 0; j < W; ++j) acc[j].init();
+  auto fetch = [&](uint32_t r) -> v4f {
+    const float* src = p + static_cast<uint64_t>(r) * inner;
+    if (VEC) return load4_stream_any(src);
+    return v4f{__builtin_nontemporal_load(src), 0.f, 0.f, 0.f};
+  };
+  uint32_t r = 0;
+  for (; r + 8 <= reduce; r += 8) {
+    v4f v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = fetch(r + k);
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+#pragma unroll
+      for (int j = 0; j < W; ++j) acc[j].add(v[k][j], r + k);
+  }
+  if (r < reduce) {
+    v4f v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (r + k < reduce) v[k] = fetch(r + k);
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (r + k < reduce)
+#pragma unroll
+        for (int j = 0; j < W; ++j) acc[j].add(v[k][j], r + k);
+  }
+  float* dst = y + static_cast<uint64_t>(o) * inner + static_cast<uint64_t>(c) * W;
+  if (VEC) {
+    v4f out;
+#pragma unroll
+    for (int j = 0; j < W; ++j) out[j] = acc[j].finalize(reduce);
+    *reinterpret_cast<v4f_unaligned*>(dst) = out;
+  } else {
+    dst[0] = acc[0].finalize(reduce);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -454,9 +515,25 @@ __global__ __launch_bounds__(kBlock) void reduce_stage2_lane_kernel(const Partia
   if (o >= outputs) return;
   Acc<OP> acc;
   acc.init();
-  for (uint32_t s = 0; s < splits; ++s) {
+  // eight partials requested together, merged in slice order: one lane walks up
+  // to 64 of them, and a request per turn of the loop would cost a memory
+  // latency each (64 rows of 200 000: 9 us of the 20 us the two launches took)
+  const Partial* mine = part + o * stride_o;
+  uint32_t s = 0;
+  for (; s + 8 <= splits; s += 8) {
+    Partial p[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) p[k] = mine[(s + k) * stride_s];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      Acc<OP> t;
+      t.unpack(p[k]);
+      acc.merge(t);
+    }
+  }
+  for (; s < splits; ++s) {
     Acc<OP> t;
-    t.unpack(part[o * stride_o + s * stride_s]);
+    t.unpack(mine[s * stride_s]);
     acc.merge(t);
   }
   y[o] = acc.finalize(window);
@@ -571,11 +648,23 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
     const uint32_t reduce = static_cast<uint32_t>(pl.reduce);
     // 128-bit loads on any dword address: rows need not start 16-byte aligned.
     const bool vec = reduce >= 4;
-    if (pl.wave_per_row && reduce < 128 && reduce % 4 != 0 && reduce >= 4) {
-      uint32_t group = std::min<uint32_t>(kBlock, kShortRowTileFloats / (reduce | 1u));
-      group &= ~3u;  // a multiple of four rows is a whole number of 128-bit pieces
-      reduce_rows_lds_kernel<OP><<<(rows + group - 1) / group, kBlock, 0, st>>>(x, y, rows, reduce, group,
-                                                                                 make_fastdiv(reduce));
+    if (pl.wave_per_row && reduce < kShortRowMaxLen) {
+      const uint32_t want = (reduce + 15) / 16;  // lanes for pieces of at most 16 elements (17 where that is even)
+      const uint32_t lanes = want <= 1 ? 1 : (want <= 2 ? 2 : (want <= 4 ? 4 : (want <= 8 ? 8 : 16)));
+      const uint32_t seg = ((reduce + lanes - 1) / lanes) | 1u;
+      const uint32_t grid = (rows + kBlock / lanes - 1) / (kBlock / lanes);
+      const FastDiv f4 = make_fastdiv(std::max<uint32_t>(1, reduce / 4));
+#define SHDW_SHORT(LANES)                                                                                  \
+  do {                                                                                                     \
+    if (reduce % 4 == 0) reduce_rows_lds_kernel<OP, LANES, true><<<grid, kBlock, 0, st>>>(x, y, rows, reduce, seg, f4);  \
+    else reduce_rows_lds_kernel<OP, LANES, false><<<grid, kBlock, 0, st>>>(x, y, rows, reduce, seg, f4);   \
+  } while (0)
+      if (lanes == 1) SHDW_SHORT(1);
+      else if (lanes == 2) SHDW_SHORT(2);
+      else if (lanes == 4) SHDW_SHORT(4);
+      else if (lanes == 8) SHDW_SHORT(8);
+      else SHDW_SHORT(16);
+#undef SHDW_SHORT
       return launch_status();
     }
     if (pl.wave_per_row) {
@@ -613,6 +702,15 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
   const uint32_t inner = static_cast<uint32_t>(pl.inner);
   const uint32_t splits = static_cast<uint32_t>(pl.splits);
   const uint32_t rows_per_split = (reduce + splits - 1) / splits;
+  if (pl.flat_period == 0 && splits == 1 && reduce <= kShortStridedMaxReduce) {
+    const bool vec = inner % 4 == 0;
+    const uint32_t per_outer = vec ? inner / 4 : inner;
+    const uint32_t units = outer * per_outer;  // <= outputs
+    const FastDiv f = make_fastdiv(per_outer);
+    if (vec) reduce_strided_short_kernel<OP, true><<<grid_for(units), kBlock, 0, st>>>(x, y, reduce, inner, units, f);
+    else reduce_strided_short_kernel<OP, false><<<grid_for(units), kBlock, 0, st>>>(x, y, reduce, inner, units, f);
+    return launch_status();
+  }
   if (pl.flat_period > 0) {
     // grid.x carries outer (at most INT32_MAX, as the element count), grid.y the slices (<= 1024)
     reduce_strided_flat_kernel<OP><<<dim3(outer, splits), kBlock, 0, st>>>(

@@ -165,11 +165,11 @@ SHDW_DEVICE void fold_batch(A* acc, const v4f (&v)[N], const bool (&valid)[N], P
 // each exchange pairs two lanes that both compute merge(own, other), and every
 // merge used here is commutative bit-for-bit.
 template <class A, int G = kWave>
-SHDW_DEVICE A group_allreduce(A a) {  // G = 16, 32 or 64 consecutive lanes
+SHDW_DEVICE A group_allreduce(A a) {  // G = 2, 4, 8, 16, 32 or 64 consecutive lanes
   a.merge(a.template dpp<kDppXor1>());
-  a.merge(a.template dpp<kDppXor2>());
-  a.merge(a.template dpp<kDppHalfMirror>());
-  a.merge(a.template dpp<kDppMirror>());
+  if (G >= 4) a.merge(a.template dpp<kDppXor2>());
+  if (G >= 8) a.merge(a.template dpp<kDppHalfMirror>());
+  if (G >= 16) a.merge(a.template dpp<kDppMirror>());
   if (G >= 32) a.merge(a.shfl_xor(16));
   if (G >= 64) a.merge(a.shfl_xor(32));
   return a;

@@ -598,10 +598,6 @@ constexpr int kPlaneStreamMinLen = 256;
 // (256 planes of 112x112: 168 us against 99 us).
 constexpr uint32_t kPlaneStreamMinRows = 512;
 
-// From this row length on the whole-plane maximum goes to Reduce's row kernels
-// (rows of 49: 14.4 us there against 13.1 us here per 51 MB; rows of 196: 11.2 against 16.5).
-constexpr int kPlaneMaxByReduce = 128;
-
 // Rows per wave: about 2048 waves in all (eight per CU, what their LDS lets reside
 // at once, two per SIMD), so long and few rows get a wave each.  Measured per
 // 51 MB: 28x28 planes 15.1 us with 8 rows per wave (20.0 with 4, 16.1 with 16),
@@ -665,9 +661,11 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
     const uint32_t rows = static_cast<uint32_t>(out_count);
     if (pool_type == 0) {
       // The running maximum of a plane is Reduce's Max over a row: the same
-      // std::max(v, x) walk from -FLT_MAX, which that kernel takes in parallel.
+      // std::max(v, x) walk from -FLT_MAX, which those kernels take in parallel
+      // (per 51 MB: 3x3 planes 10.9 us against 19.1 us here, 7x7 10.3 / 12.9,
+      // 14x14 10.1 / 16.5, 56x56 10.7 / 99).
       int rc = SHDW_OK;
-      if (plane >= kPlaneMaxByReduce && reduce_rows_max(rows, static_cast<uint32_t>(plane), x, y, st, &rc)) return rc;
+      if (reduce_rows_max(rows, static_cast<uint32_t>(plane), x, y, st, &rc)) return rc;
       launch_pool_plane<true>(x, y, rows, static_cast<uint32_t>(plane), st);
     } else if (plane >= kPlaneStreamMinLen && rows >= kPlaneStreamMinRows) {
       launch_pool_rows_stream(x, y, rows, static_cast<uint32_t>(plane), st);
