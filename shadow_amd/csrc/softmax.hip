@@ -13,6 +13,7 @@
 // The elementwise parts (exp, divide) are done by every lane in both layouts.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cfloat>
 
 #include "../../include/shadow_hip.h"
@@ -423,6 +424,194 @@ __global__ __launch_bounds__(kBlock) void normalize_slab_kernel(const float* x, 
   }
 }
 
+// ---------------------------------------------------------------------------
+// Small slabs (inner < 64, dim * inner up to 3 K floats): class scores per box
+// ([batch * boxes, 21], inner = 1), per-position embeddings, 2-class maps.  One
+// workgroup per slab, as the slab kernels above do it, leaves a workgroup with a
+// few dozen elements (softmax over [6.4M, 2]: 5 ms per 51 MB).  Here a
+// workgroup takes `group` consecutive slabs, one contiguous span: 128-bit loads
+// and stores on the global side, and in LDS every slab at a pitch of
+// inner * (dim | 1) floats, so that lane q = slab * inner + s, which walks the
+// column (slab, s) in index order with a stride of inner floats, meets the other
+// lanes of its wave on different banks (all of them where inner is a power of
+// two).  The per-element work between the walks (exp, the division) is done by
+// all lanes over the span as it lies.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kPackedTileFloats = 12288;  // 48 KB: three workgroups per CU
+
+struct PackedSpan {
+  uint32_t slab, pitch, inner, ncols, cells;
+  FastDiv f_slab, f_inner;
+  // element t of the span -> LDS offset, column, row
+  SHDW_DEVICE void place(uint32_t t, uint32_t& at, uint32_t& q, uint32_t& c) const {
+    uint32_t g, rem, s;
+    fd_divmod(t, f_slab, g, rem);
+    fd_divmod(rem, f_inner, c, s);
+    at = g * pitch + rem;
+    q = g * inner + s;
+  }
+};
+
+SHDW_DEVICE PackedSpan packed_span(uint32_t slabs, uint32_t dim, FastDiv f_inner, FastDiv f_slab, uint32_t group,
+                                   uint32_t* first_slab) {
+  PackedSpan sp;
+  sp.inner = f_inner.d;
+  sp.slab = dim * sp.inner;
+  sp.pitch = sp.inner * (dim | 1u);
+  sp.f_slab = f_slab, sp.f_inner = f_inner;
+  *first_slab = blockIdx.x * group;
+  const uint32_t n = min(group, slabs - *first_slab);
+  sp.ncols = n * sp.inner;
+  sp.cells = n * sp.slab;
+  return sp;
+}
+
+// The span into LDS: four vectors in flight per lane, scattered by element
+// because a vector may straddle two slabs.
+SHDW_DEVICE void packed_stage_in(float* lds, const float* xs, const PackedSpan& sp) {
+  const uint32_t nvec = sp.cells / 4;
+  for (uint32_t v0 = 0; v0 < nvec; v0 += 4 * kBlock) {
+    v4f reg[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t v = v0 + k * kBlock + threadIdx.x;
+      if (v < nvec) reg[k] = load4_stream_any(xs + 4ull * v);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t v = v0 + k * kBlock + threadIdx.x;
+      if (v < nvec) {
+        uint32_t g, rem;
+        fd_divmod(4 * v, sp.f_slab, g, rem);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          lds[g * sp.pitch + rem] = reg[k][j];
+          if (++rem == sp.slab) rem = 0, ++g;
+        }
+      }
+    }
+  }
+  const uint32_t t = 4 * nvec + threadIdx.x;
+  if (t < sp.cells) {
+    uint32_t at, q, c;
+    sp.place(t, at, q, c);
+    lds[at] = xs[t];
+  }
+}
+
+// Walks the four elements that start at element t of the span: one division by
+// the slab and one by inner for the first, then steps.
+struct PackedWalk {
+  uint32_t at, q, c, s, rem;
+  SHDW_DEVICE PackedWalk(const PackedSpan& sp, uint32_t t) {
+    uint32_t g;
+    fd_divmod(t, sp.f_slab, g, rem);
+    fd_divmod(rem, sp.f_inner, c, s);
+    at = g * sp.pitch + rem;
+    q = g * sp.inner + s;
+  }
+  SHDW_DEVICE void step(const PackedSpan& sp) {
+    ++at, ++q, ++s, ++rem;
+    if (s == sp.inner) s = 0, q -= sp.inner, ++c;          // next row of the same slab: its columns again
+    if (rem == sp.slab) rem = 0, c = 0, q += sp.inner, at += sp.pitch - sp.slab;  // next slab
+  }
+};
+
+// f(value in LDS, column, row) -> new value in LDS, for the whole span.
+template <class F>
+SHDW_DEVICE void packed_update(float* lds, const PackedSpan& sp, F f) {
+  const uint32_t nvec = (sp.cells + 3) / 4;
+  for (uint32_t v = threadIdx.x; v < nvec; v += kBlock) {
+    PackedWalk w(sp, 4 * v);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (4 * v + j < sp.cells) lds[w.at] = f(lds[w.at], w.q, w.c);
+      w.step(sp);
+    }
+  }
+}
+
+// f(value in LDS, column, row) -> output element, for the whole span, 128-bit stores.
+template <class F>
+SHDW_DEVICE void packed_stage_out(const float* lds, float* ys, const PackedSpan& sp, F f) {
+  const uint32_t nvec = sp.cells / 4;
+  for (uint32_t v = threadIdx.x; v < nvec; v += kBlock) {
+    PackedWalk w(sp, 4 * v);
+    v4f r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      r[j] = f(lds[w.at], w.q, w.c);
+      w.step(sp);
+    }
+    store4_stream_any(ys + 4ull * v, r);
+  }
+  const uint32_t t = 4 * nvec + threadIdx.x;
+  if (t < sp.cells) {
+    uint32_t at, q, c;
+    sp.place(t, at, q, c);
+    ys[t] = f(lds[at], q, c);
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void softmax_packed_kernel(const float* x, float* y, uint32_t slabs,
+                                                                 uint32_t dim, FastDiv f_inner, FastDiv f_slab,
+                                                                 uint32_t group) {
+  extern __shared__ __align__(16) float lds[];  // group * pitch floats
+  __shared__ uint64_t tab[32];
+  __shared__ float stat[kBlock];
+  if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
+  uint32_t first;
+  const PackedSpan sp = packed_span(slabs, dim, f_inner, f_slab, group, &first);
+  const uint64_t base = static_cast<uint64_t>(first) * sp.slab;
+  packed_stage_in(lds, x + base, sp);
+  __syncthreads();
+  const uint32_t q = threadIdx.x;
+  float* col = lds + fd_div(q, f_inner) * sp.pitch + (q - fd_div(q, f_inner) * sp.inner);
+  if (q < sp.ncols) {
+    float m = -FLT_MAX;
+#pragma unroll 4
+    for (uint32_t c = 0; c < dim; ++c) m = std_max(col[c * sp.inner], m);
+    stat[q] = m;
+  }
+  __syncthreads();
+  packed_update(lds, sp, [&](float v, uint32_t cq, uint32_t) { return libm::exact_expf(v - stat[cq], tab); });
+  __syncthreads();
+  if (q < sp.ncols) {
+    float sum = 0.f;
+#pragma unroll 4
+    for (uint32_t c = 0; c < dim; ++c) sum += col[c * sp.inner];
+    stat[q] = sum;
+  }
+  __syncthreads();
+  packed_stage_out(lds, y + base, sp, [&](float e, uint32_t cq, uint32_t) { return e / stat[cq]; });
+}
+
+template <int PMODE, int SM>
+__global__ __launch_bounds__(kBlock) void normalize_packed_kernel(const float* x, float* y, uint32_t slabs,
+                                                                   uint32_t dim, FastDiv f_inner, FastDiv f_slab,
+                                                                   uint32_t group, float p, float eps,
+                                                                   const float* scale) {
+  extern __shared__ __align__(16) float lds[];
+  __shared__ float stat[kBlock];
+  uint32_t first;
+  const PackedSpan sp = packed_span(slabs, dim, f_inner, f_slab, group, &first);
+  const uint64_t base = static_cast<uint64_t>(first) * sp.slab;
+  packed_stage_in(lds, x + base, sp);
+  __syncthreads();
+  const uint32_t q = threadIdx.x;
+  if (q < sp.ncols) {
+    const uint32_t g = fd_div(q, f_inner);
+    const float* col = lds + g * sp.pitch + (q - g * sp.inner);
+    double acc = 0;
+#pragma unroll 4
+    for (uint32_t c = 0; c < dim; ++c) acc += norm_term<PMODE>(col[c * sp.inner], p);
+    stat[q] = norm_finish<PMODE>(acc, p, eps);
+  }
+  __syncthreads();
+  packed_stage_out(lds, y + base, sp,
+                   [&](float v, uint32_t cq, uint32_t c) { return ssd_scaled<SM>(v / stat[cq], scale, c); });
+}
+
 // Columns of 65 to 512 elements over a wide inner extent: a workgroup owns a
 // tile of TS = 64, 32 or 16 neighbouring positions with all their `dim` elements,
 // 64 KB at most, so x is read from HBM once.  Each lane keeps its share of the
@@ -752,6 +941,23 @@ struct ColumnGeometry {
   uint32_t columns, slab_bytes;
 };
 
+// Slabs per workgroup of the packed kernels, 0 where they do not apply (a slab
+// of more than a quarter of the tile stays with one workgroup per slab).
+static uint32_t packed_group(int dim, int inner_num) {
+  if (inner_num >= 64) return 0;
+  const uint64_t pitch = static_cast<uint64_t>(inner_num) * (static_cast<uint32_t>(dim) | 1u);
+  if (pitch * 4 > kPackedTileFloats) return 0;
+  uint32_t group = std::min<uint32_t>(kBlock / inner_num, kPackedTileFloats / static_cast<uint32_t>(pitch));
+  group &= ~3u;  // whole 128-bit pieces per workgroup
+  // the walks are done by group * inner lanes: under 32 of them (rows of 512 and
+  // more with inner = 1) the slab kernels' all-lane forms do better
+  return group * inner_num >= 32 ? group : 0;
+}
+
+static size_t packed_bytes(int dim, int inner_num, uint32_t group) {
+  return static_cast<size_t>(group) * inner_num * (static_cast<uint32_t>(dim) | 1u) * sizeof(float);
+}
+
 static int column_geometry(int outer_num, int dim, int inner_num, ColumnGeometry* g) {
   if (outer_num < 0 || dim < 0 || inner_num < 0) return SHDW_E_INVALID_ARGUMENT;
   const int64_t columns = static_cast<int64_t>(outer_num) * inner_num;
@@ -779,7 +985,11 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
   if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
-  if (g.use_slab)
+  if (const uint32_t group = packed_group(dim, inner_num)) {
+    const uint32_t slabs = static_cast<uint32_t>(outer_num);
+    softmax_packed_kernel<<<(slabs + group - 1) / group, kBlock, packed_bytes(dim, inner_num, group), st>>>(
+        x, y, slabs, static_cast<uint32_t>(dim), fi, make_fastdiv(static_cast<uint32_t>(dim) * inner_num), group);
+  } else if (g.use_slab)
     softmax_slab_kernel<<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, static_cast<uint32_t>(dim), fi);
   else if (dim <= 64) {
     // the tile kernel is slower here: [64,49,128,128] 115 us against 88
@@ -814,7 +1024,18 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
   const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
   const uint32_t d = static_cast<uint32_t>(dim);
   const int mode = p == 1.f ? 1 : (p == 2.f ? 2 : 0);
-  if (g.use_slab) {
+  if (const uint32_t group = packed_group(dim, inner_num)) {
+    const uint32_t slabs = static_cast<uint32_t>(outer_num);
+    const uint32_t grid = (slabs + group - 1) / group;
+    const size_t bytes = packed_bytes(dim, inner_num, group);
+    const FastDiv fs = make_fastdiv(d * inner_num);
+    if (mode == 1)
+      normalize_packed_kernel<1, kSsdNoScale><<<grid, kBlock, bytes, st>>>(x, y, slabs, d, fi, fs, group, p, eps, nullptr);
+    else if (mode == 2)
+      normalize_packed_kernel<2, kSsdNoScale><<<grid, kBlock, bytes, st>>>(x, y, slabs, d, fi, fs, group, p, eps, nullptr);
+    else
+      normalize_packed_kernel<0, kSsdNoScale><<<grid, kBlock, bytes, st>>>(x, y, slabs, d, fi, fs, group, p, eps, nullptr);
+  } else if (g.use_slab) {
     if (mode == 1)
       normalize_slab_kernel<1><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
     else if (mode == 2)
@@ -865,7 +1086,11 @@ static void launch_ssd_columns(const ColumnGeometry& g, int outer_num, int dim, 
   const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
   const uint32_t d = static_cast<uint32_t>(dim);
   const uint32_t grid = grid_for(g.columns);
-  if (g.use_slab)
+  if (const uint32_t group = packed_group(dim, inner_num)) {
+    const uint32_t slabs = static_cast<uint32_t>(outer_num);
+    normalize_packed_kernel<3, SM><<<(slabs + group - 1) / group, kBlock, packed_bytes(dim, inner_num, group), st>>>(
+        x, y, slabs, d, fi, make_fastdiv(d * inner_num), group, 2.f, eps, scale);
+  } else if (g.use_slab)
     normalize_slab_kernel<3, SM><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, 2.f, eps, scale);
   else if (tile_fits(dim, inner_num))
     launch_normalize_tile<3, SM>(outer_num, dim, inner_num, 2.f, eps, x, scale, y, st);
