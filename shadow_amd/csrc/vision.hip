@@ -9,6 +9,7 @@
 // plane (global pooling) go through LDS so that global loads stay coalesced.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cfloat>
 
 #include "../../include/shadow_hip.h"
@@ -369,6 +370,134 @@ static bool plan_pool_band(const PoolArgs& p, int target_outputs, BandArgs* a) {
   return true;
 }
 
+// Planes too small to keep a workgroup busy (14x14 and 7x7 maps with 3x3 / 2x2 /
+// 5x5 .. 13x13 windows): with a workgroup per band of one plane, a 7x7 plane
+// gives 49 outputs to 256 lanes (3x3 stride 1 on [128,2048,7,7]: 179 us per
+// 51 MB).  Here a workgroup takes `planes` consecutive planes, one contiguous
+// span of x, into LDS, each with its padding in place: ph rows above, pw
+// columns left, and as many below and to the right as the last window reaches
+// over, all holding the fold's neutral value (lowest() for max, +0 for the sum:
+// the running sum starts at +0 and can never become -0, so adding +0 leaves it
+// unchanged bit for bit).  A lane then walks the window of one output after the
+// other, rows and columns in ascending order, without a test.
+constexpr int kSmallPlanesTileFloats = 12288;  // 48 KB: three workgroups per CU
+constexpr int kSmallPlanesMaxOutputs = 512;    // larger planes go to the band kernel
+
+struct SmallPlanesArgs {
+  int in_h, in_w, out_h, out_w, kh, kw, sh, sw, ph, pw;
+  int pitch, plane_lds;  // padded row and plane in LDS, in floats
+  uint32_t planes, total_planes;
+  FastDiv f_plane_in, f_in_w, f_plane_out, f_out_w;
+};
+
+template <bool MAX, int K>
+__global__ __launch_bounds__(kBlock) void pool_small_planes_kernel(const float* x, float* y, SmallPlanesArgs a) {
+  extern __shared__ __align__(16) float tile[];  // planes * plane_lds floats, a multiple of 4
+  const uint32_t first = blockIdx.x * a.planes;
+  const uint32_t np = min(a.planes, a.total_planes - first);
+  const uint32_t plane_in = a.f_plane_in.d, plane_out = a.f_plane_out.d;
+  {
+    const float neutral = MAX ? -FLT_MAX : 0.f;
+    const uint32_t cells = a.planes * static_cast<uint32_t>(a.plane_lds);
+    for (uint32_t t = 4 * threadIdx.x; t < cells; t += 4 * kBlock)
+      *reinterpret_cast<v4f*>(tile + t) = v4f{neutral, neutral, neutral, neutral};
+  }
+  __syncthreads();
+  const float* xs = x + static_cast<uint64_t>(first) * plane_in;
+  const uint32_t span = np * plane_in, nvec = span / 4;
+  auto slot = [&](uint32_t t) -> uint32_t {
+    uint32_t pl, rem, r, c;
+    fd_divmod(t, a.f_plane_in, pl, rem);
+    fd_divmod(rem, a.f_in_w, r, c);
+    return pl * a.plane_lds + (r + a.ph) * a.pitch + a.pw + c;
+  };
+  for (uint32_t v0 = 0; v0 < nvec; v0 += 4 * kBlock) {
+    v4f reg[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t v = v0 + k * kBlock + threadIdx.x;
+      if (v < nvec) reg[k] = load4_stream_any(xs + 4ull * v);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t v = v0 + k * kBlock + threadIdx.x;
+      if (v < nvec) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) tile[slot(4 * v + j)] = reg[k][j];
+      }
+    }
+  }
+  if (4 * nvec + threadIdx.x < span) tile[slot(4 * nvec + threadIdx.x)] = xs[4 * nvec + threadIdx.x];
+  __syncthreads();
+  float* ys = y + static_cast<uint64_t>(first) * plane_out;
+  const uint32_t outputs = np * plane_out;
+  for (uint32_t o = threadIdx.x; o < outputs; o += kBlock) {
+    uint32_t pl, rem, oh, ow;
+    fd_divmod(o, a.f_plane_out, pl, rem);
+    fd_divmod(rem, a.f_out_w, oh, ow);
+    const float* win = tile + pl * a.plane_lds + (oh * a.sh) * a.pitch + ow * a.sw;
+    float max_val = -FLT_MAX, sum_val = 0.f;
+    if (K > 0) {
+      float cell[K > 0 ? K * K : 1];
+#pragma unroll
+      for (int i = 0; i < K; ++i)
+#pragma unroll
+        for (int j = 0; j < K; ++j) cell[i * K + j] = win[i * a.pitch + j];
+#pragma unroll
+      for (int c = 0; c < K * K; ++c) {
+        if (MAX)
+          max_val = pool_max(max_val, cell[c]);
+        else
+          sum_val += cell[c];
+      }
+    } else {
+      for (int i = 0; i < a.kh; ++i) {
+        const float* row = win + i * a.pitch;
+        for (int j = 0; j < a.kw; ++j) {
+          const float v = row[j];
+          if (MAX)
+            max_val = pool_max(max_val, v);
+          else
+            sum_val += v;
+        }
+      }
+    }
+    if (MAX) {
+      ys[o] = max_val;
+    } else {
+      const int h_first = static_cast<int>(oh) * a.sh - a.ph, w_first = static_cast<int>(ow) * a.sw - a.pw;
+      const int pool_size = (min(h_first + a.kh, a.in_h + a.ph) - h_first) * (min(w_first + a.kw, a.in_w + a.pw) - w_first);
+      ys[o] = sum_val / static_cast<float>(pool_size);
+    }
+  }
+}
+
+// Fills `a` and returns true where the kernel above applies: several padded
+// planes fit the tile and one plane alone would leave lanes idle.
+static bool plan_small_planes(const PoolArgs& p, int64_t total_planes, SmallPlanesArgs* a) {
+  const int64_t plane_out = static_cast<int64_t>(p.out_h) * p.out_w, plane_in = static_cast<int64_t>(p.in_h) * p.in_w;
+  if (plane_out > kSmallPlanesMaxOutputs || plane_out < 1 || total_planes > INT32_MAX) return false;
+  const int over_b = std::max(0, (p.out_h - 1) * p.sh - p.ph + p.kh - p.in_h);
+  const int over_r = std::max(0, (p.out_w - 1) * p.sw - p.pw + p.kw - p.in_w);
+  const int64_t pitch = static_cast<int64_t>(p.pw) + p.in_w + over_r;
+  int64_t plane_lds = (static_cast<int64_t>(p.ph) + p.in_h + over_b) * pitch;
+  plane_lds = (plane_lds + 3) & ~int64_t{3};
+  if (plane_lds * 2 > kSmallPlanesTileFloats) return false;
+  int64_t planes = kSmallPlanesTileFloats / plane_lds;
+  const int64_t want = (4 * kBlock + plane_out - 1) / plane_out;  // about four outputs per lane
+  planes = std::min(planes, std::max<int64_t>(2, want));
+  if (planes >= 4) planes &= ~int64_t{3};  // whole 128-bit pieces wherever the plane count allows
+  a->in_h = p.in_h, a->in_w = p.in_w, a->out_h = p.out_h, a->out_w = p.out_w;
+  a->kh = p.kh, a->kw = p.kw, a->sh = p.sh, a->sw = p.sw, a->ph = p.ph, a->pw = p.pw;
+  a->pitch = static_cast<int>(pitch), a->plane_lds = static_cast<int>(plane_lds);
+  a->planes = static_cast<uint32_t>(planes), a->total_planes = static_cast<uint32_t>(total_planes);
+  a->f_plane_in = make_fastdiv(static_cast<uint32_t>(plane_in));
+  a->f_in_w = make_fastdiv(static_cast<uint32_t>(p.in_w));
+  a->f_plane_out = make_fastdiv(static_cast<uint32_t>(plane_out));
+  a->f_out_w = make_fastdiv(static_cast<uint32_t>(p.out_w));
+  return true;
+}
+
 // Whole-plane windows: x is [rows][len], one output per row.  A workgroup owns
 // `group` consecutive rows (as many as fit the tile, at most one per lane); they
 // pass through LDS (coalesced 128-bit loads by all lanes), then lane r folds
@@ -686,6 +815,21 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
   p.f_out_h = make_fastdiv(static_cast<uint32_t>(p.out_h));
   p.f_out_d = make_fastdiv(static_cast<uint32_t>(p.out_d));
   const uint32_t n_out = static_cast<uint32_t>(out_count);
+  SmallPlanesArgs sp;
+  if (!three_d && plan_small_planes(p, static_cast<int64_t>(in_shape[0]) * in_shape[1], &sp)) {
+    const uint32_t grid = (sp.total_planes + sp.planes - 1) / sp.planes;
+    const size_t lds = static_cast<size_t>(sp.planes) * sp.plane_lds * sizeof(float);
+    const int k = p.kh == p.kw && (p.kh == 2 || p.kh == 3) ? p.kh : 0;
+#define SHDW_SMALL(MAXV)                                                                      \
+  do {                                                                                        \
+    if (k == 3) pool_small_planes_kernel<MAXV, 3><<<grid, kBlock, lds, st>>>(x, y, sp);       \
+    else if (k == 2) pool_small_planes_kernel<MAXV, 2><<<grid, kBlock, lds, st>>>(x, y, sp);  \
+    else pool_small_planes_kernel<MAXV, 0><<<grid, kBlock, lds, st>>>(x, y, sp);              \
+  } while (0)
+    if (pool_type == 0) SHDW_SMALL(true); else SHDW_SMALL(false);
+#undef SHDW_SMALL
+    return launch_status();
+  }
   BandArgs a;
   if (!three_d && plan_pool_band(p, kPoolBandOutputs, &a)) {
     const int64_t groups = static_cast<int64_t>(in_shape[0]) * in_shape[1] * a.bands_per_plane;
