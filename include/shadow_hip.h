@@ -335,6 +335,20 @@ int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
                         const float* scale, const float* bias, int scale_num, int scale_inner,
                         float* y, void* stream);
 
+/* The same with scratch memory of the caller, for rows too long and too few to
+ * give a workgroup each (GroupNorm with few groups at batch 1, LayerNorm over
+ * C*H*W): with it such rows are cut into slices that three launches work on side
+ * by side, fp64 partial sums going through the scratch.  `workspace` holds at
+ * least shdw_hip_group_norm_workspace_bytes(outer_num, inner_num) bytes, 8-byte
+ * aligned (0 bytes: the rows need none); NULL / fewer bytes: as
+ * shdw_hip_group_norm, a workgroup per row.  The reference keeps mean, variance
+ * and a squared copy of the input in temp blobs of the Workspace.
+ * ref: shadow/operators/kernels/group_norm.hpp:49-72, layer_norm.hpp:30-55 */
+size_t shdw_hip_group_norm_workspace_bytes(int outer_num, int inner_num);
+int shdw_hip_group_norm_ws(int outer_num, int inner_num, float eps, const float* x,
+                           const float* scale, const float* bias, int scale_num, int scale_inner,
+                           float* y, void* workspace, size_t workspace_bytes, void* stream);
+
 /* =============================== data movers =============================== */
 
 /* dst[n*dst_pitch + dst_offset + p] = src[n*src_pitch + src_offset + p] for

@@ -248,7 +248,7 @@ __global__ __launch_bounds__(LANES <= kWave ? kBlock : LANES, LANES == kBigBlock
   }
 }
 
-// Rows of 17 to 256 elements, at least a thousand of them.  The register forms
+// Rows of up to 256 elements, at least a thousand of them.  The register forms
 // above give such rows 16 to 64 lanes with one vector each, and what a lane does
 // once per row (two fp64 exchanges, four IEEE divisions' worth of setup, the
 // square root, the parameter lookup, the vector-tail logic) then outweighs what
@@ -446,6 +446,107 @@ __global__ __launch_bounds__(kBlock) void norm_rows_stream_kernel(const float* x
   }
 }
 
+// Rows too long and too few for a workgroup each (GroupNorm of a detector's
+// feature map at batch 1: 32 rows of 320 000; one row of 12.8 M elements took
+// 17 ms): every row is cut into `splits` slices, a workgroup per slice, in three
+// launches that hand fp64 partial sums on through scratch memory of the caller:
+//   pass 1: partial sums of alpha * x
+//   pass 2: the mean from pass 1's partials, partial sums of alpha * (x - mean)^2
+//   pass 3: mean and variance from the partials, then the row's slice of y.
+// Every workgroup of a row folds the row's partials in the same fixed order, so
+// all of them hold the same mean and variance.
+template <bool VEC>
+SHDW_DEVICE double slice_sum(const float* xr, uint32_t begin, uint32_t end, float alpha, bool centred, float mean) {
+  double acc = 0;
+  auto term = [&](float v) {
+    float t;
+    if (centred) {
+      const float val = v - mean;
+      const float sq = val * val;
+      t = alpha * sq;
+    } else {
+      t = alpha * v;
+    }
+    acc += static_cast<double>(t);
+  };
+  if (VEC) {
+    for (uint32_t t = begin / 4 + threadIdx.x; t < end / 4; t += kBlock) {
+      const v4f q = load4(xr + 4ull * t);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) term(q[j]);
+    }
+  } else {
+    for (uint32_t t = begin + threadIdx.x; t < end; t += kBlock) term(xr[t]);
+  }
+  return acc;
+}
+
+// Sum of a row's `splits` partials (<= 1024), the same tree in every workgroup.
+SHDW_DEVICE double fold_partials(const double* part, uint32_t splits, double* slots) {
+  double acc = 0;
+  for (uint32_t s = threadIdx.x; s < splits; s += kBlock) acc += part[s];
+  return row_sum<kBlock>(acc, slots);
+}
+
+template <int PASS, bool VEC>
+__global__ __launch_bounds__(kBlock) void norm_rows_split_kernel(const float* x, float* y, NormArgs p,
+                                                                  uint32_t splits, uint32_t chunk,
+                                                                  double* sums, double* squares) {
+  __shared__ double slots[kBlock / kWave];
+  const uint32_t row = blockIdx.x, slice = blockIdx.y;
+  const uint64_t base = static_cast<uint64_t>(row) * p.inner;
+  const float* xr = x + base;
+  const uint32_t begin = min(slice * chunk, p.inner), end = min(begin + chunk, p.inner);
+  const double* row_sums = sums + static_cast<size_t>(row) * splits;
+  double* row_squares = squares + static_cast<size_t>(row) * splits;
+  if (PASS == 1) {
+    const double acc = row_sum<kBlock>(slice_sum<VEC>(xr, begin, end, p.alpha, false, 0.f), slots);
+    if (threadIdx.x == 0) sums[static_cast<size_t>(row) * splits + slice] = acc;
+    return;
+  }
+  const float mean = static_cast<float>(fold_partials(row_sums, splits, slots));
+  if (PASS == 2) {
+    const double acc = row_sum<kBlock>(slice_sum<VEC>(xr, begin, end, p.alpha, true, mean), slots);
+    if (threadIdx.x == 0) row_squares[slice] = acc;
+    return;
+  }
+  const float variance = static_cast<float>(fold_partials(row_squares, splits, slots));
+  const float ve = variance + p.eps;
+  const float denom = __builtin_sqrtf(ve);
+  float* yr = y + base;
+  const RowAffine ra = norm_row_affine(p, static_cast<uint32_t>(base));
+  if (VEC) {
+    for (uint32_t t = begin / 4 + threadIdx.x; t < end / 4; t += kBlock) {
+      const v4f q = load4(xr + 4ull * t);
+      v4f r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float val = q[j] - mean;
+        r[j] = val / denom;
+      }
+      r = p.affine == kAffineRow ? norm_row_affine4(ra, r)
+                                 : norm_affine4(p, static_cast<uint32_t>(base) + 4 * t, 4 * t, r);
+      store4_stream(yr + 4ull * t, r);
+    }
+  } else {
+    for (uint32_t t = begin + threadIdx.x; t < end; t += kBlock) {
+      const float val = xr[t] - mean;
+      const float q = val / denom;
+      yr[t] = p.affine == kAffineRow ? affine1(q, ra.s, ra.b) : norm_affine1(p, static_cast<uint32_t>(base) + t, q);
+    }
+  }
+}
+
+constexpr uint32_t kNormSplitMaxRows = 512, kNormSplitMinInner = 32768, kNormSplitMinChunk = 8192;
+
+// Slices per row: enough for about a thousand workgroups, each with at least
+// 8192 elements; 1 where rows are many or short.
+static uint32_t norm_row_splits(int64_t rows, int64_t inner) {
+  if (rows >= kNormSplitMaxRows || inner < kNormSplitMinInner || rows < 1) return 1;
+  const int64_t by_fill = (1024 + rows - 1) / rows, by_work = inner / kNormSplitMinChunk;
+  return static_cast<uint32_t>(std::max<int64_t>(1, std::min<int64_t>(std::min(by_fill, by_work), 1024)));
+}
+
 // ---------------------------------------------------------------------------
 // SSDNormalize across the whole item (shadow/operators/kernels/
 // ssd_normalize.hpp:47-57): the reference squares x into the output, takes
@@ -573,9 +674,22 @@ using namespace shdw;
 
 extern "C" {
 
+size_t shdw_hip_group_norm_workspace_bytes(int outer_num, int inner_num) {
+  if (outer_num <= 0 || inner_num <= 0) return 0;
+  const uint32_t splits = norm_row_splits(outer_num, inner_num);
+  return splits > 1 ? static_cast<size_t>(2) * outer_num * splits * sizeof(double) : 0;
+}
+
 int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
                         const float* scale, const float* bias, int scale_num, int scale_inner,
                         float* y, void* stream) {
+  return shdw_hip_group_norm_ws(outer_num, inner_num, eps, x, scale, bias, scale_num, scale_inner, y, nullptr, 0,
+                                stream);
+}
+
+int shdw_hip_group_norm_ws(int outer_num, int inner_num, float eps, const float* x,
+                           const float* scale, const float* bias, int scale_num, int scale_inner,
+                           float* y, void* workspace, size_t workspace_bytes, void* stream) {
   if (outer_num < 0 || inner_num < 0) return SHDW_E_INVALID_ARGUMENT;
   const int64_t count = static_cast<int64_t>(outer_num) * inner_num;
   if (count > INT32_MAX) return SHDW_E_INVALID_ARGUMENT;
@@ -606,9 +720,28 @@ int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint32_t rows = p.outer;
   const uint32_t nvec = p.inner / 4;
+  const uint32_t splits = norm_row_splits(outer_num, inner_num);
+  if (splits > 1 && workspace && workspace_bytes >= shdw_hip_group_norm_workspace_bytes(outer_num, inner_num)) {
+    if (reinterpret_cast<uintptr_t>(workspace) & 7u) return SHDW_E_INVALID_ARGUMENT;
+    double* sums = static_cast<double*>(workspace);
+    double* squares = sums + static_cast<size_t>(rows) * splits;
+    uint32_t chunk = (p.inner + splits - 1) / splits;
+    chunk = (chunk + 3) & ~3u;  // slices start on whole vectors
+    const dim3 grid(rows, splits);
+#define SHDW_SPLIT(PASS)                                                                                       \
+  do {                                                                                                         \
+    if (vec) norm_rows_split_kernel<PASS, true><<<grid, kBlock, 0, st>>>(x, y, p, splits, chunk, sums, squares);  \
+    else norm_rows_split_kernel<PASS, false><<<grid, kBlock, 0, st>>>(x, y, p, splits, chunk, sums, squares);  \
+  } while (0)
+    SHDW_SPLIT(1);
+    SHDW_SPLIT(2);
+    SHDW_SPLIT(3);
+#undef SHDW_SPLIT
+    return launch_status();
+  }
   // workgroups of 256 lanes holding 256 / lanes rows each
   auto groups = [rows](uint32_t lanes) { return (rows + kBlock / lanes - 1) / (kBlock / lanes); };
-  if (p.inner > 16 && p.inner <= kNormLdsMaxInner && rows >= 1024) {
+  if (p.inner <= kNormLdsMaxInner && rows >= 1024) {
     // short rows through LDS, L lanes per row (any row length, any dword address)
     if (!scale)
       p.affine = kAffineNone;
@@ -619,7 +752,7 @@ int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
     else
       p.affine = kAffineElement;
     const uint32_t want = (p.inner + 15) / 16;  // lanes for pieces of at most 16 elements
-    const uint32_t lanes = want <= 2 ? 2 : (want <= 4 ? 4 : (want <= 8 ? 8 : 16));
+    const uint32_t lanes = want <= 1 ? 1 : (want <= 2 ? 2 : (want <= 4 ? 4 : (want <= 8 ? 8 : 16)));
     const uint32_t seg = ((p.inner + lanes - 1) / lanes) | 1u;  // an odd number of elements per lane
     const uint32_t grid = (rows + kBlock / lanes - 1) / (kBlock / lanes);
     const FastDiv f4 = make_fastdiv(std::max<uint32_t>(1, p.inner / 4));
@@ -629,6 +762,7 @@ int shdw_hip_group_norm(int outer_num, int inner_num, float eps, const float* x,
     else norm_rows_lds_kernel<LANES, false><<<grid, kBlock, 0, st>>>(x, y, p, seg, f4);        \
   } while (0)
     switch (lanes) {
+      case 1: SHDW_LDS(1); break;
       case 2: SHDW_LDS(2); break;
       case 4: SHDW_LDS(4); break;
       case 8: SHDW_LDS(8); break;

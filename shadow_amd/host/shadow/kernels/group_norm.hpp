@@ -5,6 +5,8 @@
 #ifndef SHADOW_AMD_HOST_KERNELS_GROUP_NORM_HPP_
 #define SHADOW_AMD_HOST_KERNELS_GROUP_NORM_HPP_
 
+#include <cstddef>
+
 #include "shadow/kernel.hpp"
 
 namespace Shadow {
@@ -13,10 +15,14 @@ namespace Vision {
 // x viewed as [outer_num][inner_num]: (x - mean) / sqrt(var + eps) per row, then
 // y * scale[c] + bias[c] with c = (i / scale_inner) % scale_num when scale_data
 // and bias_data are not null.
+// scratch: NormalizeRowsScratchBytes(outer_num, inner_num) bytes of device memory
+// (8-byte aligned; nullptr where that is 0), where rows too long and too few for
+// a workgroup each leave their partial sums.
+size_t NormalizeRowsScratchBytes(int outer_num, int inner_num);
 template <DeviceType D, typename T>
 void NormalizeRows(const T* in_data, int outer_num, int inner_num, float eps, const T* scale_data,
-                   const T* bias_data, int scale_num, int scale_inner, T* out_data,
-                   Context* context);
+                   const T* bias_data, int scale_num, int scale_inner, T* out_data, void* scratch,
+                   size_t scratch_bytes, Context* context);
 }  // namespace Vision
 
 class GroupNormKernel : public Kernel {

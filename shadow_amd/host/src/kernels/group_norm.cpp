@@ -7,13 +7,30 @@ namespace Shadow {
 
 namespace Vision {
 
+size_t NormalizeRowsScratchBytes(int outer_num, int inner_num) {
+  return shdw_hip_group_norm_workspace_bytes(outer_num, inner_num);
+}
+
 template <>
 void NormalizeRows<DeviceType::kGPU, float>(const float* in_data, int outer_num, int inner_num,
                                             float eps, const float* scale_data,
                                             const float* bias_data, int scale_num,
-                                            int scale_inner, float* out_data, Context* context) {
-  SHADOW_HIP_CHECK(shdw_hip_group_norm(outer_num, inner_num, eps, in_data, scale_data, bias_data,
-                                       scale_num, scale_inner, out_data, context->stream()));
+                                            int scale_inner, float* out_data, void* scratch,
+                                            size_t scratch_bytes, Context* context) {
+  SHADOW_HIP_CHECK(shdw_hip_group_norm_ws(outer_num, inner_num, eps, in_data, scale_data, bias_data,
+                                          scale_num, scale_inner, out_data, scratch, scratch_bytes,
+                                          context->stream()));
+}
+
+// Scratch from the workspace's temp buffer, as the reference takes its mean /
+// variance / temp blobs (group_norm.hpp:49-54); nullptr when the rows need none.
+static void* NormalizeRowsScratch(Workspace* ws, int outer_num, int inner_num, size_t* bytes,
+                                  std::shared_ptr<Blob>* hold) {
+  *bytes = NormalizeRowsScratchBytes(outer_num, inner_num);
+  if (*bytes == 0) return nullptr;
+  ws->GrowTempBuffer(*bytes + 8);
+  *hold = ws->CreateTempBlob({static_cast<int>((*bytes + 3) / 4)}, DataType::kI32);
+  return (*hold)->mutable_data<int>();
 }
 
 }  // namespace Vision
@@ -34,9 +51,12 @@ class GroupNormKernelHip : public GroupNormKernel {
       CHECK_EQ(bias->count(), channel);
       scale_data = scale->data<float>(), bias_data = bias->data<float>();
     }
+    size_t scratch_bytes = 0;
+    std::shared_ptr<Blob> hold;
+    void* scratch = Vision::NormalizeRowsScratch(ws, outer_num, inner_num, &scratch_bytes, &hold);
     Vision::NormalizeRows<DeviceType::kGPU, float>(
         input->data<float>(), outer_num, inner_num, eps, scale_data, bias_data, channel,
-        spatial_dim, output->mutable_data<float>(), ws->Ctx().get());
+        spatial_dim, output->mutable_data<float>(), scratch, scratch_bytes, ws->Ctx().get());
   }
 
   DeviceType device_type() const override { return DeviceType::kGPU; }
@@ -60,9 +80,12 @@ class LayerNormKernelHip : public LayerNormKernel {
       CHECK(bias->shape() == normalized_shape);
       scale_data = scale->data<float>(), bias_data = bias->data<float>();
     }
+    size_t scratch_bytes = 0;
+    std::shared_ptr<Blob> hold;
+    void* scratch = Vision::NormalizeRowsScratch(ws, outer_num, inner_num, &scratch_bytes, &hold);
     Vision::NormalizeRows<DeviceType::kGPU, float>(
         input->data<float>(), outer_num, inner_num, eps, scale_data, bias_data, inner_num, 1,
-        output->mutable_data<float>(), ws->Ctx().get());
+        output->mutable_data<float>(), scratch, scratch_bytes, ws->Ctx().get());
   }
 
   DeviceType device_type() const override { return DeviceType::kGPU; }

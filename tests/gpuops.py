@@ -255,16 +255,24 @@ def pooling(x, in_shape, pool_type, kernel, stride, pad, out_shape):
 
 
 def group_norm(x, outer, inner, eps, scale=None, bias=None, scale_num=1, scale_inner=1, inplace=False,
-               offset=0):
-    """offset (in floats) shifts x and y off 16-byte alignment."""
+               offset=0, scratch=False):
+    """offset (in floats) shifts x and y off 16-byte alignment; scratch: through the entry
+    point that takes the caller's scratch memory (sliced rows where they are long and few)."""
     x = _f(x).ravel()
     dx = Buffer(4 * (x.size + offset) + 16)
     dx.upload(x, 4 * offset)
     y = dx if inplace else Buffer(4 * (x.size + offset) + 16)
     ds = Buffer.from_numpy(_f(scale)) if scale is not None else None
     db = Buffer.from_numpy(_f(bias)) if bias is not None else None
-    check(_lib().shdw_hip_group_norm(outer, inner, eps, dx.ptr + 4 * offset, ds.ptr if ds else None,
-                                     db.ptr if db else None, scale_num, scale_inner,
-                                     y.ptr + 4 * offset, None))
+    if scratch:
+        need = _lib().shdw_hip_group_norm_workspace_bytes(outer, inner)
+        ws = Buffer(need) if need else None
+        check(_lib().shdw_hip_group_norm_ws(outer, inner, eps, dx.ptr + 4 * offset, ds.ptr if ds else None,
+                                            db.ptr if db else None, scale_num, scale_inner,
+                                            y.ptr + 4 * offset, ws.ptr if ws else None, need, None))
+    else:
+        check(_lib().shdw_hip_group_norm(outer, inner, eps, dx.ptr + 4 * offset, ds.ptr if ds else None,
+                                         db.ptr if db else None, scale_num, scale_inner,
+                                         y.ptr + 4 * offset, None))
     _sync()
     return y.download(count=x.size, offset_bytes=4 * offset)

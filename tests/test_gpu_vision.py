@@ -381,8 +381,9 @@ def test_group_norm_rows_extreme_magnitudes(gpu, outer, inner):
 
 NORM_ROWS = [(6, 49), (4, 784), (8, 1024), (3, 2048), (5, 3136), (2, 4096), (2, 4100), (2, 25088), (7, 5),
              (300, 12), (1, 1), (3, 1000), (2, 8192), (2, 6002), (7, 400), (2100, 1200), (2051, 2048), (9, 256), (3, 16384), (2, 32768), (2, 32772), (1, 70000),
-             # a thousand and more short rows: through LDS, one lane per row
-             (2000, 49), (1025, 127), (1500, 5), (4099, 56), (1024, 9), (3000, 66)]
+             # a thousand and more short rows: through LDS, 1 to 16 lanes per row
+             (2000, 49), (1025, 127), (1500, 5), (4099, 56), (1024, 9), (3000, 66), (5000, 1), (3001, 2), (2048, 4),
+             (1031, 12), (1024, 16), (1500, 28), (1111, 60), (1024, 124), (1030, 252), (1024, 255)]
 
 
 @pytest.mark.parametrize("outer,inner", NORM_ROWS)
@@ -394,9 +395,32 @@ def test_group_norm_rows(gpu, outer, inner):
         assert assert_rel_close(got, want, 1e-5, "norm rows %s" % kw) == 0
 
 
+# Long rows, few of them: with the caller's scratch memory every row is cut into slices
+# (three launches); without it a workgroup walks a whole row.  Same results either way.
+@pytest.mark.parametrize("outer,inner", [(1, 70000), (3, 32768), (2, 32770), (5, 100003), (40, 40000), (511, 32768),
+                                         (1, 1000000), (512, 32768), (7, 4000)])
+def test_group_norm_long_rows_with_scratch(gpu, outer, inner):
+    x = normal(44, outer * inner, 3.0) + F(0.75)
+    want = oracle.normalize_rows(x, outer, inner, 1e-5)
+    need = shadow_amd.hip().shdw_hip_group_norm_workspace_bytes(outer, inner)
+    assert (need > 0) == (outer < 512 and inner >= 32768)
+    for kw in ({}, {"inplace": True}, {"offset": 1}):
+        got = gpuops.group_norm(x, outer, inner, 1e-5, scratch=True, **kw)
+        assert assert_rel_close(got, want, 1e-5, "sliced norm rows %s" % kw) == 0
+    s, b = uniform(45, inner, 0.5, 2.0), normal(46, inner)   # LayerNorm's affine pair per position
+    want2 = oracle.scale_bias(want, s, b, inner, 1)
+    got = gpuops.group_norm(x, outer, inner, 1e-5, s, b, inner, 1, scratch=True)
+    assert assert_rel_close(got, want2, 1e-5, "sliced norm rows, per-position affine") == 0
+    if inner % 8 == 0:  # GroupNorm's: 8 channels per row
+        s, b = uniform(47, 8 * outer, 0.5, 2.0), normal(48, 8 * outer)
+        want3 = oracle.scale_bias(want, s, b, 8 * outer, inner // 8)
+        got = gpuops.group_norm(x, outer, inner, 1e-5, s, b, 8 * outer, inner // 8, scratch=True)
+        assert assert_rel_close(got, want3, 1e-5, "sliced norm rows, per-channel affine") == 0
+
+
 @pytest.mark.parametrize("shape,group", [((2, 8, 5, 5), 1), ((2, 8, 5, 5), 4), ((4, 32, 14, 14), 8), ((2, 6, 7, 3), 6),
                                          ((4, 512, 7, 7), 512), ((8, 256, 3, 3), 128), ((2, 1024, 5, 5), 1024),
-                                         ((1, 64, 56, 56), 32)])
+                                         ((1, 64, 56, 56), 32), ((2, 16, 64, 64), 1)])
 def test_group_and_instance_norm_op(ws, shape, group):
     x = normal(41, shape, 2.0) + F(0.5)
     scale, bias = uniform(42, shape[1], 0.5, 2.0), normal(43, shape[1])
