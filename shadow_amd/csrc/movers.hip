@@ -205,6 +205,67 @@ __global__ __launch_bounds__(kBlock) void permute_generic_kernel(const float* x,
   }
 }
 
+// Transposition with one thin side (interleaved <-> planar images: [H*W][3] <->
+// [3][H*W]): the 64 x 64 tiles below would be 3 wide, nine tenths of every
+// workgroup idle ([4.3M][3] -> [3][4.3M]: 229 us per 51 MB).  Here a tile takes the
+// whole thin side and `span` elements of the long one; the side that is
+// contiguous in memory moves with 128-bit accesses as it lies, the element
+// shuffle happens in LDS.
+constexpr uint32_t kThinMax = 16;          // thin side up to this many elements
+constexpr uint32_t kThinTileFloats = 8192;  // 32 KB
+
+// COLS_THIN: x[batch][big][thin] -> y[batch][thin][big]; else x[batch][thin][big] -> y[batch][big][thin].
+template <bool COLS_THIN>
+__global__ __launch_bounds__(kBlock) void transpose_thin_kernel(const float* x, float* y, uint32_t big,
+                                                                 uint32_t thin, uint32_t span,
+                                                                 FastDiv f_tiles) {
+  __shared__ __align__(16) float tile[kThinTileFloats];  // [span][thin], the interleaved side's order
+  uint32_t b, t;
+  fd_divmod(blockIdx.x, f_tiles, b, t);
+  const uint32_t first = t * span, n = min(span, big - first);  // elements of the long side in this tile
+  const uint64_t image = static_cast<uint64_t>(b) * big * thin;
+  const uint32_t cells = n * thin;
+  const float* inter = (COLS_THIN ? x : y) + image + static_cast<uint64_t>(first) * thin;  // contiguous, cells long
+  const float* planar_src = x + image + first;  // row i at + i * big (not COLS_THIN)
+  float* planar_dst = y + image + first;        // row j at + j * big (COLS_THIN)
+  const uint32_t quads = n / 4;                 // whole vectors per planar row
+  if (COLS_THIN) {
+    for (uint32_t v = threadIdx.x; v < cells / 4; v += kBlock)
+      *reinterpret_cast<v4f*>(tile + 4 * v) = load4_stream_any(inter + 4ull * v);
+    for (uint32_t e = (cells & ~3u) + threadIdx.x; e < cells; e += kBlock) tile[e] = inter[e];
+    __syncthreads();
+    for (uint32_t u = threadIdx.x; u < thin * quads; u += kBlock) {
+      const uint32_t j = u / quads, q = u - j * quads;
+      v4f r;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) r[k] = tile[(4 * q + k) * thin + j];
+      store4_stream_any(planar_dst + static_cast<uint64_t>(j) * big + 4 * q, r);
+    }
+    const uint32_t rest = n - 4 * quads;
+    for (uint32_t u = threadIdx.x; u < thin * rest; u += kBlock) {
+      const uint32_t j = u / rest, r = 4 * quads + (u - j * rest);
+      planar_dst[static_cast<uint64_t>(j) * big + r] = tile[r * thin + j];
+    }
+  } else {
+    for (uint32_t u = threadIdx.x; u < thin * quads; u += kBlock) {
+      const uint32_t i = u / quads, q = u - i * quads;
+      const v4f r = load4_stream_any(planar_src + static_cast<uint64_t>(i) * big + 4 * q);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) tile[(4 * q + k) * thin + i] = r[k];
+    }
+    const uint32_t rest = n - 4 * quads;
+    for (uint32_t u = threadIdx.x; u < thin * rest; u += kBlock) {
+      const uint32_t i = u / rest, c = 4 * quads + (u - i * rest);
+      tile[c * thin + i] = planar_src[static_cast<uint64_t>(i) * big + c];
+    }
+    __syncthreads();
+    float* out = const_cast<float*>(inter);
+    for (uint32_t v = threadIdx.x; v < cells / 4; v += kBlock)
+      store4_stream_any(out + 4ull * v, *reinterpret_cast<const v4f*>(tile + 4 * v));
+    for (uint32_t e = (cells & ~3u) + threadIdx.x; e < cells; e += kBlock) out[e] = tile[e];
+  }
+}
+
 constexpr int kTile = 64;
 
 // VEC: rows % 4 == 0, cols % 4 == 0 and both pointers 16-byte aligned: 128-bit
@@ -862,6 +923,21 @@ int shdw_hip_permute(int num_axes, const int* in_shape, const int* order, const 
     const uint32_t batch = plain2 ? 1u : static_cast<uint32_t>(ext[0]);
     const uint32_t cols = static_cast<uint32_t>(plain2 ? ext[0] : ext[1]);  // input's fast axis
     const uint32_t rows = static_cast<uint32_t>(plain2 ? ext[1] : ext[2]);
+    if (std::min(rows, cols) <= kThinMax && std::max(rows, cols) >= 256) {
+      const bool cols_thin = cols <= rows;
+      const uint32_t thin = cols_thin ? cols : rows, big = cols_thin ? rows : cols;
+      const uint32_t span = (kThinTileFloats / thin) & ~63u;
+      const uint32_t tiles = (big + span - 1) / span;
+      const int64_t groups = static_cast<int64_t>(batch) * tiles;
+      if (groups <= INT32_MAX) {
+        const FastDiv ft = make_fastdiv(tiles);
+        if (cols_thin)
+          transpose_thin_kernel<true><<<static_cast<uint32_t>(groups), kBlock, 0, st>>>(x, y, big, thin, span, ft);
+        else
+          transpose_thin_kernel<false><<<static_cast<uint32_t>(groups), kBlock, 0, st>>>(x, y, big, thin, span, ft);
+        return launch_status();
+      }
+    }
     const uint32_t tiles_r = (rows + kTile - 1) / kTile, tiles_c = (cols + kTile - 1) / kTile;
     const int64_t groups = static_cast<int64_t>(batch) * tiles_r * tiles_c;
     if (groups <= INT32_MAX) {

@@ -109,7 +109,11 @@ def test_pad_op(ws, pads, shape):
     ((2, 3, 4, 5), [0, 2, 3, 1]), ((2, 3, 4, 5), [0, 3, 1, 2]), ((2, 3, 4, 5), [3, 2, 1, 0]), ((4, 6), [1, 0]),
     ((2, 3, 4), [0, 1, 2]), ((2, 3, 4, 5, 6), [4, 0, 3, 1, 2]), ((7,), [0]), ((2, 1, 3), [2, 1, 0]),
     ((3, 130, 70), [0, 2, 1]), ((200, 131), [1, 0]), ((2, 64, 28, 28), [0, 2, 3, 1]), ((2, 5, 6, 7), [1, 0, 2, 3]),
-    ((2, 3, 4, 5), [0, 1, 3, 2]), ((1, 1, 9), [2, 0, 1])])
+    ((2, 3, 4, 5), [0, 1, 3, 2]), ((1, 1, 9), [2, 0, 1]),
+    # one thin side (interleaved <-> planar images): whole and ragged tiles, odd lengths, batches
+    ((1000, 3), [1, 0]), ((3, 1000), [1, 0]), ((2, 37, 41, 3), [0, 3, 1, 2]), ((2, 3, 37, 41), [0, 2, 3, 1]),
+    ((3, 777, 5), [0, 2, 1]), ((2, 16, 9001), [0, 2, 1]), ((9001, 16), [1, 0]), ((1, 6000, 1), [1, 0, 2]),
+    ((4, 260, 1, 2), [0, 3, 2, 1]), ((5462, 3), [1, 0]), ((2, 257, 13), [0, 2, 1]), ((17, 300), [1, 0])])
 def test_permute_op(ws, shape, order):
     x = normal(60, shape)
     got = run(ws, "Permute", [("x", x)], {"order": order})
