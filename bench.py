@@ -93,6 +93,9 @@ def parse():
     ap.add_argument("--probe", action="store_true",
                     help="counter probe: 3 launches of a plain copy and of every headline op on "
                          "the 51.4M tensor, nothing timed, no JSON (run under rocprofv3 --pmc)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="time the operators over shapes off the benchmark's (short and long rows, thin and "
+                         "small extents) against a plain copy of the same bytes, print a table, exit")
     ap.add_argument("--probe-next", action="store_true",
                     help="the same for the neighbouring operators and the data movers")
     return ap.parse_args()
@@ -305,6 +308,89 @@ def probe_next(dev):
         dev.ck(lib.shdw_hip_ssd_normalize(64, 256, 3136, 0, 1e-5, x.ptr, ssd_sc.ptr, 0, y.ptr, None, st))
         dev.ck(lib.shdw_hip_ssd_normalize(64, 512, 1444, 1, 1e-5, x.ptr, ssd_sc.ptr, 0, y.ptr, ssd_ws.ptr, st))
     dev.sync()
+
+
+def sweep(dev):
+    """Shapes off the benchmark's: every line is one operator on about 51 MB with the
+    time of a plain copy (51 MB read + 51 MB written) scaled to the bytes the operator
+    has to move, so 1.0 means the speed of a copy.  Prints the worst ratio of each
+    family (operators that share a set of kernels) at the end."""
+    lib, st = dev.lib, dev.stream
+    I = dev.sa.ints
+    SETS, N = 4, 12845056
+    X = [dev.buf(normal(11 + k, N, 2.0)) for k in range(SETS)]
+    Y = [dev.buf(nbytes=4 * N) for _ in range(SETS)]
+    P, Q = dev.buf(uniform(5, N, 0.5, 1.5)), dev.buf(uniform(6, N, -0.5, 0.5))
+    scratch = dev.buf(nbytes=64 << 20)
+    tm = lambda fn: time_median(dev, fn, SETS, reps=20) * 1e3
+    t_copy = tm(lambda k: lib.shdw_hip_copy(N, X[k].ptr, Y[k].ptr, st))
+    print("plain copy of 12,845,056 floats (51 MB read, 51 MB written): %.2f us" % t_copy)
+    worst = {}
+
+    def show(family, name, us, nbytes):
+        ratio = us / (t_copy * nbytes / (8.0 * N))
+        worst[family] = max(worst.get(family, (0.0, "")), (ratio, name))
+        print("%-14s %-58s %9.2f us  %6.2f x copy" % (family, name, us, ratio), flush=True)
+
+    for L in (1, 2, 3, 4, 5, 8, 9, 12, 16, 17, 49, 64, 65, 127, 128, 129, 196, 255, 256, 257, 512, 784, 1024, 3136,
+              4097, 12544, 50176, 200000, 12845056):
+        rows = N // L
+        for kind, shape, axes in (("reduce rows", [rows, L], [1]), ("reduce strided", [L, rows], [0])):
+            need = lib.shdw_hip_reduce_workspace_bytes(2, I(shape), 1, I(axes))
+            assert need <= (64 << 20)
+            for op, nm in ((1, "sum"), (2, "max")):
+                us = tm(lambda k: lib.shdw_hip_reduce(op, 2, I(shape), 1, I(axes), X[k].ptr, Y[k].ptr,
+                                                      scratch.ptr if need else None, need, st))
+                show(kind, "%s over %d of [%s]" % (nm, L, "x".join(map(str, shape))), us, 4 * (rows * L + rows))
+    for which in ("softmax", "normalize"):
+        for dim in (2, 8, 21, 49, 64, 65, 150, 256, 512, 513, 1000, 4096):
+            for inner in (1, 2, 7, 16, 49, 196, 3136):
+                if dim * inner > N:
+                    continue
+                outer = N // (dim * inner)
+                n = outer * dim * inner
+                if which == "softmax":
+                    us = tm(lambda k: lib.shdw_hip_softmax(outer, dim, inner, X[k].ptr, Y[k].ptr, st))
+                else:
+                    us = tm(lambda k: lib.shdw_hip_normalize(outer, dim, inner, 2.0, 1e-12, X[k].ptr, Y[k].ptr, st))
+                show(which, "[%d,%d,%d]" % (outer, dim, inner), us, 8 * n)
+    for inner in (1, 2, 4, 8, 16, 17, 49, 196, 256, 257, 784, 3136, 12544, 50176, 400000, 12845056):
+        outer = N // inner
+        need = lib.shdw_hip_group_norm_workspace_bytes(outer, inner)
+        assert need <= (64 << 20)
+        us = tm(lambda k: lib.shdw_hip_group_norm_ws(outer, inner, 1e-5, X[k].ptr, None, None, 1, 1, Y[k].ptr,
+                                                     scratch.ptr if need else None, need, st))
+        show("row norm", "[%d,%d]%s" % (outer, inner, " (sliced rows)" if need else ""), us, 8 * outer * inner)
+    for shape, k, s, p in (([16, 64, 112, 112], 3, 2, 1), ([16, 64, 112, 112], 2, 2, 0), ([16, 64, 112, 112], 3, 1, 1),
+                           ([64, 1024, 14, 14], 2, 2, 0), ([64, 1024, 14, 14], 3, 1, 1), ([128, 2048, 7, 7], 3, 1, 1),
+                           ([512, 512, 7, 7], 7, 1, 3), ([64, 1024, 14, 14], 13, 1, 6), ([16, 64, 112, 112], 5, 1, 2)):
+        n_, c_, h_, w_ = shape
+        oh, ow = (h_ + 2 * p - k) // s + 1, (w_ + 2 * p - k) // s + 1
+        for pt, nm in ((0, "max"), (1, "avg")):
+            us = tm(lambda kk: lib.shdw_hip_pooling2d(I(shape), pt, k, k, s, s, p, p, I([n_, c_, oh, ow]), X[kk].ptr,
+                                                      Y[kk].ptr, st))
+            show("pooling", "%s %dx%d s%d p%d on %s" % (nm, k, k, s, p, shape), us, 4 * (n_ * c_ * (h_ * w_ + oh * ow)))
+    for side in (3, 7, 14, 28, 56):
+        rows = N // (side * side)
+        shape = [rows // 64, 64, side, side]
+        for pt, nm in ((0, "max"), (1, "avg")):
+            us = tm(lambda kk: lib.shdw_hip_pooling2d(I(shape), pt, side, side, 1, 1, 0, 0, I(shape[:2] + [1, 1]),
+                                                      X[kk].ptr, Y[kk].ptr, st))
+            show("global pool", "%s over %dx%d planes of %s" % (nm, side, side, shape), us,
+                 4 * shape[0] * 64 * (side * side + 1))
+    for inner in (1, 2, 4):
+        for num in (3, 64, 1000):
+            n = (N // (num * inner)) * num * inner
+            us = tm(lambda k: lib.shdw_hip_scale_bias(n, num, inner, X[k].ptr, P.ptr, Q.ptr, 0, Y[k].ptr, st))
+            show("scale", "%d parameters, inner %d" % (num, inner), us, 8 * n)
+    for shape, order in (([N // 3, 3], [1, 0]), ([3, N // 3], [1, 0]), ([16, 224, 224, 16], [0, 3, 1, 2]),
+                         ([64, 256, 28, 28], [0, 2, 3, 1]), ([8, 3, 85, 76, 76], [0, 1, 3, 4, 2])):
+        n = int(np.prod(shape))
+        us = tm(lambda k: lib.shdw_hip_permute(len(shape), I(shape), I(order), X[k].ptr, Y[k].ptr, st))
+        show("permute", "%s order %s" % (shape, order), us, 8 * n)
+    print("worst of each family:")
+    for family, (ratio, name) in worst.items():
+        print("  %-14s %6.2f x copy  (%s)" % (family, ratio, name))
 
 
 # ------------------------------------------------------------- CPU baseline
@@ -799,6 +885,9 @@ def main():
         raise SystemExit("bench.py: this build measures one GPU; the path shards by batch with no "
                          "exchange, so run one process per GPU (got --gpus %d)" % args.gpus)
     dev = Dev()
+    if args.sweep:
+        sweep(dev)
+        return
     if args.probe:
         probe(dev)
         return

@@ -25,7 +25,7 @@
 
 namespace shdw {
 
-constexpr int kSlabMaxFloats = 15 * 1024;  // slab + per-column statistics, 60 KB of LDS
+constexpr int kSlabMaxFloats = 39 * 1024;  // slab + per-column statistics: up to 156 of the CU's 160 KB of LDS
 
 // std::max(a, b) of libstdc++: b only when a < b.
 SHDW_DEVICE float std_max(float a, float b) { return a < b ? b : a; }
@@ -160,11 +160,32 @@ __global__ __launch_bounds__(kBlock) void softmax_columns_reg_kernel(const float
     if (c < DFULL || c < dim) __builtin_nontemporal_store(v[c] / sum, yc + static_cast<uint64_t>(c) * inner);
 }
 
-// Copy a contiguous slab into LDS through `f`, a few loads in flight per lane.
-constexpr int kSlabBatch = 4;
+// Copy a contiguous slab into LDS through `f`: 128-bit loads, eight in flight per
+// lane, where the slab starts on a 16-byte boundary, single floats elsewhere.
+constexpr int kSlabBatch = 8;
 template <class F>
 SHDW_DEVICE void stage_slab(float* lds, const float* xs, uint32_t slab, F f) {
-  for (uint32_t t0 = 0; t0 < slab; t0 += kSlabBatch * kBlock) {
+  uint32_t done = 0;
+  if ((reinterpret_cast<uintptr_t>(xs) & 15) == 0) {
+    const v4f* x4 = reinterpret_cast<const v4f*>(xs);
+    v4f* l4 = reinterpret_cast<v4f*>(lds);
+    const uint32_t quads = slab / 4;
+    for (uint32_t t0 = 0; t0 < quads; t0 += kSlabBatch * kBlock) {
+      v4f reg[kSlabBatch];
+#pragma unroll
+      for (int k = 0; k < kSlabBatch; ++k) {
+        const uint32_t t = t0 + k * kBlock + threadIdx.x;
+        if (t < quads) reg[k] = x4[t];
+      }
+#pragma unroll
+      for (int k = 0; k < kSlabBatch; ++k) {
+        const uint32_t t = t0 + k * kBlock + threadIdx.x;
+        if (t < quads) l4[t] = v4f{f(reg[k][0]), f(reg[k][1]), f(reg[k][2]), f(reg[k][3])};
+      }
+    }
+    done = 4 * quads;
+  }
+  for (uint32_t t0 = done; t0 < slab; t0 += kSlabBatch * kBlock) {
     float reg[kSlabBatch];
 #pragma unroll
     for (int k = 0; k < kSlabBatch; ++k) {
@@ -177,6 +198,36 @@ SHDW_DEVICE void stage_slab(float* lds, const float* xs, uint32_t slab, F f) {
       if (t < slab) lds[t] = f(reg[k]);
     }
   }
+}
+
+// Rows 0 .. n-1 of a column in LDS (`stride` floats apart) handed to `fold` in
+// index order.  Two sets of registers take turns, so that the loads of one
+// batch are on their way while the other is folded: the walk then costs the
+// dependent chain of the fold and nothing else.
+template <class F>
+SHDW_DEVICE void walk_column(const float* col, uint32_t stride, uint32_t n, F&& fold) {
+  constexpr int kBatch = 8;
+  const uint32_t batches = n / kBatch;
+  float a[kBatch], b[kBatch];
+  auto request = [&](float(&v)[kBatch], uint32_t batch) {
+    const float* at = col + batch * kBatch * stride;
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) v[k] = at[k * stride];
+  };
+  auto consume = [&](const float(&v)[kBatch]) {
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) fold(v[k]);
+  };
+  if (batches) request(a, 0);
+  uint32_t i = 0;
+  for (; i + 2 <= batches; i += 2) {
+    request(b, i + 1);
+    consume(a);
+    if (i + 2 < batches) request(a, i + 2);
+    consume(b);
+  }
+  if (i < batches) consume(a);
+  for (uint32_t c = batches * kBatch; c < n; ++c) fold(col[c * stride]);
 }
 
 // Any-order maximum over the workgroup.  Only valid where the order cannot
@@ -220,6 +271,7 @@ __global__ __launch_bounds__(kBlock) void softmax_slab_kernel(const float* x, fl
   extern __shared__ __align__(16) float lds[];
   __shared__ uint64_t tab[32];
   __shared__ float wave_max[kBlock / kWave];
+  __shared__ float part[kBlock];
   const uint32_t inner = f_inner.d;
   const uint32_t slab = dim * inner;
   float* stat = lds + slab;
@@ -240,10 +292,25 @@ __global__ __launch_bounds__(kBlock) void softmax_slab_kernel(const float* x, fl
     for (uint32_t t = threadIdx.x; t < slab; t += kBlock) ys[t] = lds[t] / sum;
     return;
   }
-  for (uint32_t s = threadIdx.x; s < inner; s += kBlock) {
+  // inner < 64 here.  The maxima in any order as well (a NaN in a column makes all
+  // of that column NaN whatever maximum was used): 256 / inner lanes per column
+  // take every lanes-th row, lane s folds their partials.
+  const uint32_t lanes = kBlock / inner;
+  {
+    uint32_t g, s;
+    fd_divmod(threadIdx.x, f_inner, g, s);
+    if (g < lanes) {
+      float max_val = -FLT_MAX;
+      const uint32_t n = g < dim ? (dim - g + lanes - 1) / lanes : 0;
+      walk_column(lds + g * inner + s, lanes * inner, n, [&](float v) { max_val = std_max(v, max_val); });
+      part[threadIdx.x] = max_val;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < inner) {
     float max_val = -FLT_MAX;
-    for (uint32_t c = 0; c < dim; ++c) max_val = std_max(lds[c * inner + s], max_val);
-    stat[s] = max_val;
+    for (uint32_t g = 0; g < lanes; ++g) max_val = std_max(part[g * inner + threadIdx.x], max_val);
+    stat[threadIdx.x] = max_val;
   }
   __syncthreads();
   for (uint32_t t = threadIdx.x; t < slab; t += kBlock) {
@@ -251,10 +318,10 @@ __global__ __launch_bounds__(kBlock) void softmax_slab_kernel(const float* x, fl
     lds[t] = libm::exact_expf(lds[t] - stat[s], tab);
   }
   __syncthreads();
-  for (uint32_t s = threadIdx.x; s < inner; s += kBlock) {
+  if (threadIdx.x < inner) {
     float sum = 0.f;
-    for (uint32_t c = 0; c < dim; ++c) sum += lds[c * inner + s];
-    stat[s] = sum;
+    walk_column(lds + threadIdx.x, inner, dim, [&](float v) { sum += v; });
+    stat[threadIdx.x] = sum;
   }
   __syncthreads();
   for (uint32_t t = threadIdx.x; t < slab; t += kBlock) {
@@ -410,17 +477,28 @@ __global__ __launch_bounds__(kBlock) void normalize_slab_kernel(const float* x, 
   if (inner == 1) {
     if (threadIdx.x == 0) stat[0] = norm_finish<PMODE>(sequential_sum<double>(lds, slab), p, eps);
   } else {
-    for (uint32_t s = threadIdx.x; s < inner; s += kBlock) {
+    if (threadIdx.x < inner) {  // inner < 64 here
       double acc = 0;
-      for (uint32_t c = 0; c < dim; ++c) acc += static_cast<double>(lds[c * inner + s]);
-      stat[s] = norm_finish<PMODE>(acc, p, eps);
+      walk_column(lds + threadIdx.x, inner, dim, [&](float v) { acc += static_cast<double>(v); });
+      stat[threadIdx.x] = norm_finish<PMODE>(acc, p, eps);
     }
   }
   __syncthreads();
-  for (uint32_t t = threadIdx.x; t < slab; t += kBlock) {
-    const uint32_t c = fd_div(t, f_inner);
-    const uint32_t s = t - c * inner;
-    ys[t] = ssd_scaled<SM>(xs[t] / stat[s], scale, c);
+  for (uint32_t t0 = 0; t0 < slab; t0 += kSlabBatch * kBlock) {
+    float reg[kSlabBatch];
+#pragma unroll
+    for (int k = 0; k < kSlabBatch; ++k) {
+      const uint32_t t = t0 + k * kBlock + threadIdx.x;
+      if (t < slab) reg[k] = xs[t];
+    }
+#pragma unroll
+    for (int k = 0; k < kSlabBatch; ++k) {
+      const uint32_t t = t0 + k * kBlock + threadIdx.x;
+      if (t < slab) {
+        const uint32_t c = fd_div(t, f_inner);
+        ys[t] = ssd_scaled<SM>(reg[k] / stat[t - c * inner], scale, c);
+      }
+    }
   }
 }
 
@@ -934,6 +1012,249 @@ static void launch_softmax_tile_ts(int outer_num, int dim, int inner_num, const 
   }
 }
 
+// ---------------------------------------------------------------------------
+// Tall columns: more rows than the tile kernels hold in LDS and, with that, few
+// columns (a softmax over 1000 or 4096 channels of a 56x56 map has 3136 per
+// image), which a lane per column leaves to a handful of waves.  Here a
+// workgroup owns 16, 32 or 64 neighbouring positions of one outer index and
+// moves down their rows in chunks of 4096 floats with all 256 lanes.  The
+// maxima are folded in any order (see softmax_slab_kernel); the ordered sums are
+// walked by one lane per column out of LDS, chunk after chunk, while the loads
+// of the next chunk are in flight.  x is read once per pass (Softmax: maxima,
+// sums, quotients; Normalize: sums, quotients), y written once.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kTallChunkFloats = 4096;
+constexpr uint32_t kTallMinInner = 16;
+constexpr int kTallAhead = 4;  // chunks requested at a time by the passes that only stream
+
+template <int VEC>
+struct TallVec { using type = float; };
+template <>
+struct TallVec<4> { using type = v4f; };
+
+SHDW_DEVICE float& tall_elem(float& v, int) { return v; }
+SHDW_DEVICE float tall_elem(const v4f& v, int e) { return v[e]; }
+SHDW_DEVICE void tall_set(float& v, int, float a) { v = a; }
+SHDW_DEVICE void tall_set(v4f& v, int e, float a) { v[e] = a; }
+
+template <int VEC>
+struct TallTile {
+  using V = typename TallVec<VEC>::type;
+  static constexpr int kLoads = 16 / VEC;  // per lane and chunk
+  uint32_t dim, inner, width, rows_per_sweep, chunk_rows, row0, col;
+  bool live;      // the lane's positions exist (the last tile of a row may be cut)
+  uint64_t base;  // of (outer index, row 0, the lane's first position)
+
+  SHDW_DEVICE TallTile(uint32_t dim_, uint32_t inner_, uint32_t width_log2, FastDiv f_tiles) {
+    dim = dim_, inner = inner_, width = 1u << width_log2;
+    const uint32_t lanes_log2 = width_log2 - (VEC == 4 ? 2 : 0);  // lanes per row of the tile
+    rows_per_sweep = kBlock >> lanes_log2;
+    chunk_rows = rows_per_sweep * kLoads;
+    row0 = threadIdx.x >> lanes_log2;
+    col = (threadIdx.x & ((1u << lanes_log2) - 1)) * VEC;
+    uint32_t n, tile;
+    fd_divmod(xcd_contiguous(blockIdx.x, gridDim.x), f_tiles, n, tile);  // neighbours share cache lines
+    const uint32_t p = tile * width + col;
+    live = p < inner;  // VEC == 4 only where inner is a multiple of four: whole vectors exist or not
+    base = static_cast<uint64_t>(n) * dim * inner + p;
+  }
+  SHDW_DEVICE uint32_t chunks() const { return (dim + chunk_rows - 1) / chunk_rows; }
+  SHDW_DEVICE uint32_t rows_in(uint32_t k) const { return min(chunk_rows, dim - k * chunk_rows); }
+  SHDW_DEVICE uint32_t row(uint32_t k, int i) const { return k * chunk_rows + i * rows_per_sweep + row0; }
+  SHDW_DEVICE bool has(uint32_t k, int i) const { return live && row(k, i) < dim; }
+  SHDW_DEVICE uint32_t slot(int i) const { return (i * rows_per_sweep + row0) * width + col; }
+  SHDW_DEVICE void load(const float* x, uint32_t k, V (&v)[kLoads]) const {
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i)
+      if (has(k, i)) v[i] = *reinterpret_cast<const V*>(x + base + static_cast<uint64_t>(row(k, i)) * inner);
+  }
+};
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void softmax_tall_kernel(const float* x, float* y, uint32_t dim,
+                                                               uint32_t inner, uint32_t width_log2,
+                                                               FastDiv f_tiles) {
+  using T = TallTile<VEC>;
+  using V = typename T::V;
+  __shared__ __align__(16) float chunk[2][kTallChunkFloats];
+  __shared__ float stat[64];
+  __shared__ uint64_t tab[32];
+  if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
+  const T t(dim, inner, width_log2, f_tiles);
+  const uint32_t chunks = t.chunks();
+  V v[T::kLoads];
+
+  float part[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) part[e] = -FLT_MAX;
+  for (uint32_t k = 0; k < chunks; k += kTallAhead) {  // chunks past the end hold no rows
+    V w[kTallAhead][T::kLoads];
+#pragma unroll
+    for (int j = 0; j < kTallAhead; ++j) t.load(x, k + j, w[j]);
+#pragma unroll
+    for (int j = 0; j < kTallAhead; ++j)
+#pragma unroll
+      for (int i = 0; i < T::kLoads; ++i)
+        if (t.has(k + j, i))
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) part[e] = std_max(tall_elem(w[j][i], e), part[e]);
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) chunk[0][t.row0 * t.width + t.col + e] = part[e];
+  __syncthreads();
+  if (threadIdx.x < t.width) {
+    float m = -FLT_MAX;
+    for (uint32_t r = 0; r < t.rows_per_sweep; ++r) m = std_max(chunk[0][r * t.width + threadIdx.x], m);
+    stat[threadIdx.x] = m;
+  }
+  __syncthreads();
+  float max_val[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) max_val[e] = stat[t.col + e];
+
+  float sum = 0.f;
+  // chunk k: its exponentials into LDS by all lanes, then the walk by one lane per
+  // column while the loads of chunk k + 2 fly.  Two buffers: the slowest walker is
+  // at most one chunk behind.
+  auto pass = [&](uint32_t k, V(&reg)[T::kLoads]) {
+    float* buf = chunk[k & 1];
+#pragma unroll
+    for (int i = 0; i < T::kLoads; ++i)
+      if (t.has(k, i)) {
+        V ex;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) tall_set(ex, e, libm::exact_expf(tall_elem(reg[i], e) - max_val[e], tab));
+        *reinterpret_cast<V*>(buf + t.slot(i)) = ex;
+      }
+    __syncthreads();
+    t.load(x, k + 2, reg);
+    if (threadIdx.x < t.width) walk_column(buf + threadIdx.x, t.width, t.rows_in(k), [&](float a) { sum += a; });
+  };
+  V v2[T::kLoads];
+  t.load(x, 0, v);
+  t.load(x, 1, v2);
+  for (uint32_t k = 0; k < chunks; k += 2) {
+    pass(k, v);
+    if (k + 1 < chunks) pass(k + 1, v2);
+  }
+  __syncthreads();
+  if (threadIdx.x < t.width) stat[threadIdx.x] = sum;
+  __syncthreads();
+  float total[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) total[e] = stat[t.col + e];
+
+  for (uint32_t k = 0; k < chunks; k += kTallAhead) {
+    V w[kTallAhead][T::kLoads];
+#pragma unroll
+    for (int j = 0; j < kTallAhead; ++j) t.load(x, k + j, w[j]);
+#pragma unroll
+    for (int j = 0; j < kTallAhead; ++j)
+#pragma unroll
+      for (int i = 0; i < T::kLoads; ++i)
+        if (t.has(k + j, i)) {
+          V q;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e)
+            tall_set(q, e, libm::exact_expf(tall_elem(w[j][i], e) - max_val[e], tab) / total[e]);
+          __builtin_nontemporal_store(
+              q, reinterpret_cast<V*>(y + t.base + static_cast<uint64_t>(t.row(k + j, i)) * inner));
+        }
+  }
+}
+
+template <int PMODE, int SM, int VEC>
+__global__ __launch_bounds__(kBlock) void normalize_tall_kernel(const float* x, float* y, uint32_t dim,
+                                                                 uint32_t inner, uint32_t width_log2,
+                                                                 FastDiv f_tiles, float p, float eps,
+                                                                 const float* scale) {
+  using T = TallTile<VEC>;
+  using V = typename T::V;
+  __shared__ __align__(16) float chunk[2][kTallChunkFloats];
+  __shared__ float stat[64];
+  const T t(dim, inner, width_log2, f_tiles);
+  const uint32_t chunks = t.chunks();
+  V v[T::kLoads];
+
+  double acc = 0;
+  auto pass = [&](uint32_t k, V(&reg)[T::kLoads]) {  // as in softmax_tall_kernel
+    float* buf = chunk[k & 1];
+#pragma unroll
+    for (int i = 0; i < T::kLoads; ++i)
+      if (t.has(k, i)) {
+        V term;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) tall_set(term, e, static_cast<float>(norm_term<PMODE>(tall_elem(reg[i], e), p)));
+        *reinterpret_cast<V*>(buf + t.slot(i)) = term;
+      }
+    __syncthreads();
+    t.load(x, k + 2, reg);
+    if (threadIdx.x < t.width)
+      walk_column(buf + threadIdx.x, t.width, t.rows_in(k), [&](float a) { acc += static_cast<double>(a); });
+  };
+  V v2[T::kLoads];
+  t.load(x, 0, v);
+  t.load(x, 1, v2);
+  for (uint32_t k = 0; k < chunks; k += 2) {
+    pass(k, v);
+    if (k + 1 < chunks) pass(k + 1, v2);
+  }
+  __syncthreads();
+  if (threadIdx.x < t.width) stat[threadIdx.x] = norm_finish<PMODE>(acc, p, eps);
+  __syncthreads();
+  float div[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) div[e] = stat[t.col + e];
+
+  for (uint32_t k = 0; k < chunks; k += kTallAhead) {
+    V w[kTallAhead][T::kLoads];
+#pragma unroll
+    for (int j = 0; j < kTallAhead; ++j) t.load(x, k + j, w[j]);
+#pragma unroll
+    for (int j = 0; j < kTallAhead; ++j)
+#pragma unroll
+      for (int i = 0; i < T::kLoads; ++i)
+        if (t.has(k + j, i)) {
+          const uint32_t r = t.row(k + j, i);
+          V q;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) tall_set(q, e, ssd_scaled<SM>(tall_elem(w[j][i], e) / div[e], scale, r));
+          __builtin_nontemporal_store(q, reinterpret_cast<V*>(y + t.base + static_cast<uint64_t>(r) * inner));
+        }
+  }
+}
+
+// Where the tall kernels apply, and their launch: positions per workgroup as wide
+// as still leaves a thousand workgroups, 128-bit accesses where every row piece
+// starts on a 16-byte boundary.
+struct TallLaunch {
+  uint32_t grid, width_log2;
+  FastDiv f_tiles;
+  bool vec4;
+};
+
+static bool tall_launch(int outer_num, int dim, int inner_num, const float* x, const float* y, TallLaunch* t) {
+  if (static_cast<uint32_t>(inner_num) < kTallMinInner || dim < 128) return false;
+  uint32_t w = 6;
+  while (w > 4 && static_cast<uint64_t>(outer_num) * ((inner_num + (1u << w) - 1) >> w) < 1024) --w;
+  const uint32_t tiles = (static_cast<uint32_t>(inner_num) + (1u << w) - 1) >> w;
+  t->grid = static_cast<uint32_t>(outer_num) * tiles;
+  t->width_log2 = w;
+  t->f_tiles = make_fastdiv(tiles);
+  t->vec4 = inner_num % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+  return true;
+}
+
+template <int PMODE, int SM>
+static void launch_normalize_tall(const TallLaunch& t, int dim, int inner_num, float p, float eps, const float* x,
+                                  const float* scale, float* y, hipStream_t st) {
+  const uint32_t d = static_cast<uint32_t>(dim), in = static_cast<uint32_t>(inner_num);
+  if (t.vec4)
+    normalize_tall_kernel<PMODE, SM, 4><<<t.grid, kBlock, 0, st>>>(x, y, d, in, t.width_log2, t.f_tiles, p, eps, scale);
+  else
+    normalize_tall_kernel<PMODE, SM, 1><<<t.grid, kBlock, 0, st>>>(x, y, d, in, t.width_log2, t.f_tiles, p, eps, scale);
+}
+
 // Shared launch geometry: slab layout when the columns are too narrow to
 // coalesce and one slab (plus its statistics) fits the LDS budget.
 struct ColumnGeometry {
@@ -1007,7 +1328,13 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
     launch_softmax_tile_ts<6>(outer_num, dim, inner_num, x, y, st);
   else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner)
     launch_softmax_tile_ts<5>(outer_num, dim, inner_num, x, y, st);
-  else
+  else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, x, y, &t)) {
+    const uint32_t d = static_cast<uint32_t>(dim), in = static_cast<uint32_t>(inner_num);
+    if (t.vec4)
+      softmax_tall_kernel<4><<<t.grid, kBlock, 0, st>>>(x, y, d, in, t.width_log2, t.f_tiles);
+    else
+      softmax_tall_kernel<1><<<t.grid, kBlock, 0, st>>>(x, y, d, in, t.width_log2, t.f_tiles);
+  } else
     softmax_columns_kernel<<<(g.columns + kWave - 1) / kWave, kWave, 0, st>>>(x, y, g.columns,
                                                                              static_cast<uint32_t>(dim), fi);
   return launch_status();
@@ -1062,6 +1389,13 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
       else
         normalize_columns_reg_kernel<2, 64><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
     }
+  } else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, x, y, &t)) {
+    if (mode == 1)
+      launch_normalize_tall<1, kSsdNoScale>(t, dim, inner_num, p, eps, x, nullptr, y, st);
+    else if (mode == 2)
+      launch_normalize_tall<2, kSsdNoScale>(t, dim, inner_num, p, eps, x, nullptr, y, st);
+    else
+      launch_normalize_tall<0, kSsdNoScale>(t, dim, inner_num, p, eps, x, nullptr, y, st);
   } else {
     const uint32_t grid = (g.columns + kWave - 1) / kWave;
     if (mode == 1)
@@ -1098,6 +1432,8 @@ static void launch_ssd_columns(const ColumnGeometry& g, int outer_num, int dim, 
     normalize_columns_reg_kernel<3, 16, SM><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, 2.f, eps, scale);
   else if (dim <= 64)
     normalize_columns_reg_kernel<3, 64, SM><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, 2.f, eps, scale);
+  else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, x, y, &t))
+    launch_normalize_tall<3, SM>(t, dim, inner_num, 2.f, eps, x, scale, y, st);
   else
     normalize_columns_kernel<3, SM><<<(g.columns + kWave - 1) / kWave, kWave, 0, st>>>(x, y, g.columns, d, fi, 2.f,
                                                                                   eps, scale);

@@ -380,17 +380,27 @@ static bool plan_pool_band(const PoolArgs& p, int target_outputs, BandArgs* a) {
 // the running sum starts at +0 and can never become -0, so adding +0 leaves it
 // unchanged bit for bit).  A lane then walks the window of one output after the
 // other, rows and columns in ascending order, without a test.
+//
+// Max windows of 16 and more cells (5x5 .. 13x13 at stride 1: the pyramid
+// pooling of detection heads) are folded in two steps, SEP: first the maximum of
+// every window-wide piece of every row into a second LDS array, then down the
+// window's rows of that array, kh + kw comparisons for an output instead of
+// kh * kw.  pool_max never takes a NaN and keeps the earlier of equal values
+// (+0 and -0), so the result of the row-major walk is the earliest largest cell,
+// and that is what the two steps return as well: the earliest of a row, then the
+// earliest row.
 constexpr int kSmallPlanesTileFloats = 12288;  // 48 KB: three workgroups per CU
 constexpr int kSmallPlanesMaxOutputs = 512;    // larger planes go to the band kernel
 
 struct SmallPlanesArgs {
   int in_h, in_w, out_h, out_w, kh, kw, sh, sw, ph, pw;
   int pitch, plane_lds;  // padded row and plane in LDS, in floats
+  int rows_lds;          // padded rows of a plane
   uint32_t planes, total_planes;
-  FastDiv f_plane_in, f_in_w, f_plane_out, f_out_w;
+  FastDiv f_plane_in, f_in_w, f_plane_out, f_out_w, f_row_maxima;  // the last: rows_lds * out_w
 };
 
-template <bool MAX, int K>
+template <bool MAX, int K, bool SEP = false>
 __global__ __launch_bounds__(kBlock) void pool_small_planes_kernel(const float* x, float* y, SmallPlanesArgs a) {
   extern __shared__ __align__(16) float tile[];  // planes * plane_lds floats, a multiple of 4
   const uint32_t first = blockIdx.x * a.planes;
@@ -431,6 +441,30 @@ __global__ __launch_bounds__(kBlock) void pool_small_planes_kernel(const float* 
   __syncthreads();
   float* ys = y + static_cast<uint64_t>(first) * plane_out;
   const uint32_t outputs = np * plane_out;
+  if (SEP) {
+    float* row_maxima = tile + a.planes * static_cast<uint32_t>(a.plane_lds);  // [plane][padded row][out_w]
+    const uint32_t per_plane = a.f_row_maxima.d, pieces = np * per_plane;
+    for (uint32_t t = threadIdx.x; t < pieces; t += kBlock) {
+      uint32_t pl, rem, r, ow;
+      fd_divmod(t, a.f_row_maxima, pl, rem);
+      fd_divmod(rem, a.f_out_w, r, ow);
+      const float* piece = tile + pl * a.plane_lds + r * a.pitch + ow * a.sw;
+      float max_val = -FLT_MAX;
+      for (int j = 0; j < a.kw; ++j) max_val = pool_max(max_val, piece[j]);
+      row_maxima[t] = max_val;
+    }
+    __syncthreads();
+    for (uint32_t o = threadIdx.x; o < outputs; o += kBlock) {
+      uint32_t pl, rem, oh, ow;
+      fd_divmod(o, a.f_plane_out, pl, rem);
+      fd_divmod(rem, a.f_out_w, oh, ow);
+      const float* win = row_maxima + pl * per_plane + (oh * a.sh) * a.out_w + ow;
+      float max_val = -FLT_MAX;
+      for (int i = 0; i < a.kh; ++i) max_val = pool_max(max_val, win[i * a.out_w]);
+      ys[o] = max_val;
+    }
+    return;
+  }
   for (uint32_t o = threadIdx.x; o < outputs; o += kBlock) {
     uint32_t pl, rem, oh, ow;
     fd_divmod(o, a.f_plane_out, pl, rem);
@@ -474,7 +508,10 @@ __global__ __launch_bounds__(kBlock) void pool_small_planes_kernel(const float* 
 
 // Fills `a` and returns true where the kernel above applies: several padded
 // planes fit the tile and one plane alone would leave lanes idle.
-static bool plan_small_planes(const PoolArgs& p, int64_t total_planes, SmallPlanesArgs* a) {
+constexpr int kSeparableMinCells = 16;
+
+static bool plan_small_planes(const PoolArgs& p, int64_t total_planes, bool max_pool, SmallPlanesArgs* a,
+                              bool* separable) {
   const int64_t plane_out = static_cast<int64_t>(p.out_h) * p.out_w, plane_in = static_cast<int64_t>(p.in_h) * p.in_w;
   if (plane_out > kSmallPlanesMaxOutputs || plane_out < 1 || total_planes > INT32_MAX) return false;
   const int over_b = std::max(0, (p.out_h - 1) * p.sh - p.ph + p.kh - p.in_h);
@@ -483,13 +520,18 @@ static bool plan_small_planes(const PoolArgs& p, int64_t total_planes, SmallPlan
   int64_t plane_lds = (static_cast<int64_t>(p.ph) + p.in_h + over_b) * pitch;
   plane_lds = (plane_lds + 3) & ~int64_t{3};
   if (plane_lds * 2 > kSmallPlanesTileFloats) return false;
-  int64_t planes = kSmallPlanesTileFloats / plane_lds;
+  const int64_t rows_lds = static_cast<int64_t>(p.ph) + p.in_h + over_b;
+  const int64_t row_maxima = rows_lds * p.out_w;
+  *separable = max_pool && p.kh * p.kw >= kSeparableMinCells && (plane_lds + row_maxima) * 2 <= kSmallPlanesTileFloats;
+  int64_t planes = kSmallPlanesTileFloats / (plane_lds + (*separable ? row_maxima : 0));
   const int64_t want = (4 * kBlock + plane_out - 1) / plane_out;  // about four outputs per lane
   planes = std::min(planes, std::max<int64_t>(2, want));
   if (planes >= 4) planes &= ~int64_t{3};  // whole 128-bit pieces wherever the plane count allows
   a->in_h = p.in_h, a->in_w = p.in_w, a->out_h = p.out_h, a->out_w = p.out_w;
   a->kh = p.kh, a->kw = p.kw, a->sh = p.sh, a->sw = p.sw, a->ph = p.ph, a->pw = p.pw;
   a->pitch = static_cast<int>(pitch), a->plane_lds = static_cast<int>(plane_lds);
+  a->rows_lds = static_cast<int>(rows_lds);
+  a->f_row_maxima = make_fastdiv(static_cast<uint32_t>(row_maxima));
   a->planes = static_cast<uint32_t>(planes), a->total_planes = static_cast<uint32_t>(total_planes);
   a->f_plane_in = make_fastdiv(static_cast<uint32_t>(plane_in));
   a->f_in_w = make_fastdiv(static_cast<uint32_t>(p.in_w));
@@ -816,10 +858,16 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
   p.f_out_d = make_fastdiv(static_cast<uint32_t>(p.out_d));
   const uint32_t n_out = static_cast<uint32_t>(out_count);
   SmallPlanesArgs sp;
-  if (!three_d && plan_small_planes(p, static_cast<int64_t>(in_shape[0]) * in_shape[1], &sp)) {
+  bool separable = false;
+  if (!three_d && plan_small_planes(p, static_cast<int64_t>(in_shape[0]) * in_shape[1], pool_type == 0, &sp, &separable)) {
     const uint32_t grid = (sp.total_planes + sp.planes - 1) / sp.planes;
-    const size_t lds = static_cast<size_t>(sp.planes) * sp.plane_lds * sizeof(float);
     const int k = p.kh == p.kw && (p.kh == 2 || p.kh == 3) ? p.kh : 0;
+    if (separable) {
+      const size_t both = static_cast<size_t>(sp.planes) * (sp.plane_lds + sp.f_row_maxima.d) * sizeof(float);
+      pool_small_planes_kernel<true, 0, true><<<grid, kBlock, both, st>>>(x, y, sp);
+      return launch_status();
+    }
+    const size_t lds = static_cast<size_t>(sp.planes) * sp.plane_lds * sizeof(float);
 #define SHDW_SMALL(MAXV)                                                                      \
   do {                                                                                        \
     if (k == 3) pool_small_planes_kernel<MAXV, 3><<<grid, kBlock, lds, st>>>(x, y, sp);       \

@@ -94,6 +94,12 @@ SOFTMAX_SHAPES = [  # outer, dim, inner: both layouts, LDS limits, odd sizes
     (2, 150, 300), (1, 65, 4097), (3, 100, 64), (1, 1000, 70),
     # around the longest column whose tile fits LDS beside the exp table
     (1, 509, 40), (1, 510, 40), (1, 511, 20), (1, 512, 33),
+    # slabs of 60 to 156 KB: one workgroup per slab with most of a CU's LDS
+    (3, 4096, 7), (2, 20000, 1), (2, 1300, 15), (1, 39000, 1), (1, 39936, 1), (1, 40000, 1),
+    # tall columns: chunks of rows through LDS, tiles of 16 / 32 / 64 positions, vectors or not,
+    # a cut last tile, a last chunk of one row, many workgroups
+    (2, 1300, 30), (2, 600, 64), (1, 1000, 100), (3, 513, 17), (1, 2048, 196), (2, 700, 68), (1, 4097, 16),
+    (1, 1025, 3136), (40, 520, 128), (1100, 513, 16), (2, 769, 49), (1, 20000, 20),
 ]
 
 
@@ -115,7 +121,8 @@ def test_softmax_special_values(gpu, outer, dim, inner):
 # NaNs in a column the order of the walk shows in the result (first, middle and last
 # row, several in one column); the tile kernel takes the maxima in parallel only where
 # the tile holds none.  Both tile widths, ragged rows, tiles with and without NaNs.
-@pytest.mark.parametrize("outer,dim,inner", [(2, 80, 100), (1, 150, 333), (2, 300, 70), (1, 512, 41), (3, 66, 16)])
+@pytest.mark.parametrize("outer,dim,inner", [(2, 80, 100), (1, 150, 333), (2, 300, 70), (1, 512, 41), (3, 66, 16),
+                                             (2, 600, 41), (1, 1030, 64)])
 def test_softmax_with_nans_in_the_columns(gpu, outer, dim, inner):
     x = normal(23, (outer, dim, inner), 4.0)
     x[0, 0, 1] = np.nan
@@ -161,7 +168,10 @@ def test_softmax_op_defaults_and_errors(ws):
                                              (2, 1, 9), (1, 33, 4097),
                                              # 65..1024 deep over a wide inner extent: tiles of 64 and 32 positions
                                              (2, 100, 100), (1, 512, 72), (3, 300, 37), (2, 1024, 20), (1, 65, 4097),
-                                             (2, 256, 64), (1, 1025, 40)])
+                                             (2, 256, 64), (1, 1025, 40),
+                                             # tall columns in chunks through LDS; slabs of more than 60 KB
+                                             (2, 1300, 30), (1, 2048, 196), (2, 1100, 68), (1, 4097, 16),
+                                             (30, 1026, 128), (3, 4096, 7), (1, 39000, 1)])
 def test_normalize(gpu, p, outer, dim, inner):
     x = normal(17, outer * dim * inner, 2.0)
     want = oracle.normalize(x, outer, dim, inner, p, 1e-12)
@@ -191,7 +201,7 @@ def test_normalize_op(ws, args):
 # ----------------------------------------------------------- SSDNormalize ---
 SSD_SHAPES = [(2, 5, 12), (3, 512, 1), (2, 16, 100), (3, 9, 64), (1, 600, 3), (2, 1, 9), (1, 33, 4097),
               (2, 64, 1444), (5, 3, 7), (1, 128, 4096), (3, 20, 1025), (2, 512, 361), (1, 1000, 50), (2, 70, 33),
-              (1, 512, 1444), (2, 1030, 24)]
+              (1, 512, 1444), (2, 1030, 24), (2, 1100, 68), (1, 2049, 31), (3, 4096, 7)]
 
 
 @pytest.mark.parametrize("scale_kind", ["none", "shared", "channel"])
@@ -267,6 +277,10 @@ POOL_2D = [
     # rows too wide for more than two output rows per band, then too wide for any band
     ((1, 1, 9, 2000), [3], [1], [1], True), ((1, 1, 7, 3000), [3], [2], [0], True),
     ((1, 2, 40, 40), [13], [5], [6], True),
+    # windows of 16 cells and more on small planes: the two-step maximum (pyramid pooling: 5, 9, 13 at stride 1)
+    ((2, 8, 13, 13), [5], [1], [2], False), ((2, 8, 13, 13), [9], [1], [4], False), ((2, 8, 13, 13), [13], [1], [6], False),
+    ((1, 5, 19, 19), [13], [1], [6], True), ((3, 3, 14, 14), [7], [1], [3], True), ((1, 7, 20, 20), [4, 5], [2, 1], [1, 2], True),
+    ((2, 2, 16, 11), [6, 4], [3, 2], [0, 1], False),
 ]
 
 
@@ -279,6 +293,22 @@ def test_pooling2d_op(ws, pool, shape, kernel, stride, pad, full):
     want = oracle.pooling_op(x, pool, kernel, stride, pad, full_pooling=full)
     assert got.shape == want.shape
     assert_bit_exact(got, want, "pooling2d")
+
+
+# The maximum keeps the earlier of equal cells and never takes a NaN: planes of signed
+# zeros, -inf, lowest() and NaNs show whether an implementation that folds rows first
+# returns the cell the row-major walk returns.
+@pytest.mark.parametrize("shape,kernel,pad", [((3, 4, 13, 13), [5], [2]), ((2, 3, 14, 14), [13], [6]),
+                                               ((2, 2, 19, 19), [9], [4]), ((1, 3, 56, 56), [5], [2])])
+def test_max_pooling_ties_and_nans_in_wide_windows(ws, shape, kernel, pad):
+    rng = np.random.default_rng(31)
+    pick = rng.integers(0, 6, size=shape)
+    x = np.choose(pick, [F(0.0), F(-0.0), F(-np.inf), F(np.finfo(F).min), F(np.nan), F(-1.0)]).astype(F)
+    x[0, 0] = np.where(rng.random(shape[2:]) < 0.5, F(0.0), F(-0.0))
+    x[-1, -1] = np.nan
+    args = {"pool": 0, "kernel_size": kernel, "stride": [1], "pad": pad, "full_pooling": False}
+    got = run(ws, "Pooling", [("x", x)], args)
+    assert_bit_exact(got, oracle.pooling_op(x, 0, kernel, [1], pad, full_pooling=False), "max pooling ties")
 
 
 @pytest.mark.parametrize("pool", [0, 1])
