@@ -210,48 +210,56 @@ def batch_norm(x, mean, variance, channel, inner_num, scale_factor, eps, inplace
     return y.download(count=x.size)
 
 
-def softmax(x, outer, dim, inner, inplace=False):
+def _shifted(x, offset, inplace, n_out=None):
+    """x on the device `offset` floats into its buffer, and the output buffer likewise."""
+    dx = Buffer(max(4, x.nbytes) + 4 * offset)
+    dx.upload(x, 4 * offset)
+    n_out = x.size if n_out is None else n_out
+    y = dx if inplace else Buffer(max(4, 4 * n_out) + 4 * offset)
+    return dx, y
+
+
+def softmax(x, outer, dim, inner, inplace=False, offset=0):
+    """offset (in floats) shifts both pointers off 16-byte alignment."""
     x = _f(x).ravel()
-    dx = Buffer.from_numpy(x)
-    y = dx if inplace else Buffer(max(4, x.nbytes))
-    check(_lib().shdw_hip_softmax(outer, dim, inner, dx.ptr, y.ptr, None))
+    dx, y = _shifted(x, offset, inplace)
+    check(_lib().shdw_hip_softmax(outer, dim, inner, dx.ptr + 4 * offset, y.ptr + 4 * offset, None))
     _sync()
-    return y.download(count=x.size)
+    return y.download(count=x.size, offset_bytes=4 * offset)
 
 
-def normalize(x, outer, dim, inner, p, eps, inplace=False):
+def normalize(x, outer, dim, inner, p, eps, inplace=False, offset=0):
     x = _f(x).ravel()
-    dx = Buffer.from_numpy(x)
-    y = dx if inplace else Buffer(max(4, x.nbytes))
-    check(_lib().shdw_hip_normalize(outer, dim, inner, p, eps, dx.ptr, y.ptr, None))
+    dx, y = _shifted(x, offset, inplace)
+    check(_lib().shdw_hip_normalize(outer, dim, inner, p, eps, dx.ptr + 4 * offset, y.ptr + 4 * offset, None))
     _sync()
-    return y.download(count=x.size)
+    return y.download(count=x.size, offset_bytes=4 * offset)
 
 
-def ssd_normalize(x, batch, channel, spatial, across_spatial, channel_shared, eps, scale=None, inplace=False):
+def ssd_normalize(x, batch, channel, spatial, across_spatial, channel_shared, eps, scale=None, inplace=False,
+                  offset=0):
     x = _f(x).ravel()
-    dx = Buffer.from_numpy(x)
-    y = dx if inplace else Buffer(max(4, x.nbytes))
+    dx, y = _shifted(x, offset, inplace)
     ds = None if scale is None else Buffer.from_numpy(_f(scale).ravel())
     nbytes = _lib().shdw_hip_ssd_normalize_workspace_bytes(batch, channel, spatial, int(across_spatial))
     ws = Buffer(nbytes) if nbytes else None
-    check(_lib().shdw_hip_ssd_normalize(batch, channel, spatial, int(across_spatial), eps, dx.ptr,
-                                        ds.ptr if ds else None, int(channel_shared), y.ptr,
+    check(_lib().shdw_hip_ssd_normalize(batch, channel, spatial, int(across_spatial), eps, dx.ptr + 4 * offset,
+                                        ds.ptr if ds else None, int(channel_shared), y.ptr + 4 * offset,
                                         ws.ptr if ws else None, None))
     _sync()
-    return y.download(count=x.size)
+    return y.download(count=x.size, offset_bytes=4 * offset)
 
 
-def pooling(x, in_shape, pool_type, kernel, stride, pad, out_shape):
+def pooling(x, in_shape, pool_type, kernel, stride, pad, out_shape, offset=0):
     """2-D or 3-D by len(kernel)."""
     x = _f(x).ravel()
     n_out = int(np.prod(out_shape, dtype=np.int64))
-    dx = Buffer.from_numpy(x)
-    y = Buffer(max(4, 4 * n_out))
+    dx, y = _shifted(x, offset, False, n_out)
     fn = _lib().shdw_hip_pooling2d if len(kernel) == 2 else _lib().shdw_hip_pooling3d
-    check(fn(ints(in_shape), pool_type, *kernel, *stride, *pad, ints(out_shape), dx.ptr, y.ptr, None))
+    check(fn(ints(in_shape), pool_type, *kernel, *stride, *pad, ints(out_shape), dx.ptr + 4 * offset,
+             y.ptr + 4 * offset, None))
     _sync()
-    return y.download(count=n_out)
+    return y.download(count=n_out, offset_bytes=4 * offset)
 
 
 def group_norm(x, outer, inner, eps, scale=None, bias=None, scale_num=1, scale_inner=1, inplace=False,

@@ -342,6 +342,41 @@ def test_global_pooling_op(ws, pool, shape):
     assert_bit_exact(got, want, "global pooling")
 
 
+# Blobs start on allocator boundaries; pointers made of a blob and an offset, as the
+# Blas face passes them, may start on any float.  One shape per kernel layout.
+ODD_POINTER_COLUMNS = [(64, 1000, 1), (300, 4, 2), (5000, 21, 1), (2, 21, 63), (4, 8, 1024), (2, 150, 300),
+                       (1, 512, 33), (2, 100, 100), (3, 4096, 7), (2, 1300, 30), (2, 600, 64), (1, 2048, 196)]
+
+
+@pytest.mark.parametrize("offset", [1, 2, 3])
+@pytest.mark.parametrize("outer,dim,inner", ODD_POINTER_COLUMNS)
+def test_column_ops_on_pointers_off_the_vector_boundary(gpu, outer, dim, inner, offset):
+    x = normal(29, outer * dim * inner, 3.0)
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner, offset=offset), oracle.softmax(x, outer, dim, inner), "softmax")
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner, inplace=True, offset=offset),
+                     oracle.softmax(x, outer, dim, inner), "softmax in place")
+    assert_bit_exact(gpuops.normalize(x, outer, dim, inner, 2.0, 1e-12, offset=offset),
+                     oracle.normalize(x, outer, dim, inner, 2.0, 1e-12), "normalize")
+    scale = uniform(30, dim, 0.5, 2.0)
+    assert_bit_exact(gpuops.ssd_normalize(x, outer, dim, inner, False, False, 1e-5, scale, offset=offset),
+                     oracle.ssd_normalize(x, outer, dim, inner, False, False, 1e-5, scale), "ssd normalize")
+
+
+@pytest.mark.parametrize("offset", [1, 3])
+@pytest.mark.parametrize("pool", [0, 1])
+@pytest.mark.parametrize("shape,kernel,stride,pad", [
+    ((2, 3, 12, 12), [3], [2], [1]), ((2, 16, 56, 56), [3], [2], [0]), ((1, 3, 112, 112), [3], [2], [1]),
+    ((130, 64, 7, 7), [3], [1], [1]), ((2, 8, 13, 13), [5], [1], [2]), ((1, 1, 9, 2000), [3], [1], [1]),
+    ((4, 128, 7, 7), [7], [1], [0]), ((3, 5, 14, 14), [14], [1], [0]), ((20, 30, 17, 17), [17], [1], [0]),
+    ((40, 128, 16, 16), [16], [1], [0]), ((2, 3, 56, 56), [56], [1], [0]), ((2, 2, 6, 7, 8), [3], [2], [1])])
+def test_pooling_on_pointers_off_the_vector_boundary(gpu, pool, shape, kernel, stride, pad, offset):
+    x = normal(32, shape, 2.0)
+    want = oracle.pooling_op(x, pool, kernel, stride, pad)
+    nsp = len(shape) - 2
+    got = gpuops.pooling(x, shape, pool, kernel * nsp, stride * nsp, pad * nsp, want.shape, offset=offset)
+    assert_bit_exact(got, want.ravel(), "pooling")
+
+
 def test_pooling_op_errors(ws):
     ws.set_blob("x", np.zeros((2, 3, 8, 8), F))
     with pytest.raises(ShadowError, match="Check Failed"):
