@@ -378,7 +378,21 @@ def sweep(dev):
                                                       X[kk].ptr, Y[kk].ptr, st))
             show("global pool", "%s over %dx%d planes of %s" % (nm, side, side, shape), us,
                  4 * shape[0] * 64 * (side * side + 1))
-    for inner in (1, 2, 4):
+    for a, b in (([64, 256, 28, 28], [1, 256, 1, 1]), ([64, 256, 28, 28], [64, 256, 1, 1]),
+                 ([64, 256, 28, 28], [1, 1, 28, 28]), ([64, 256, 28, 28], [1, 1, 1, 28]),
+                 ([64, 256, 28, 28], [64, 1, 28, 28]), ([64, 256, 28, 28], [1, 256, 28, 1]),
+                 ([64, 256, 28, 28], [1, 1, 1, 1]), ([1792, 7168], [1792, 1]), ([1792, 7168], [1, 7168]),
+                 ([4096, 49, 64], [4096, 1, 64]), ([4096, 49, 64], [1, 49, 1]), ([200704, 8, 8], [200704, 1, 8]),
+                 ([200704, 8, 8], [200704, 8, 1]), ([262144, 7, 7], [262144, 1, 1]), ([4281685, 3], [1, 3]),
+                 ([64, 256, 1, 28], [64, 1, 28, 28]), ([4, 4, 7, 8, 14, 8, 16, 7], [1, 4, 1, 8, 1, 8, 1, 7])):
+        out = [max(p_, q_) for p_, q_ in zip(a, b)]
+        n, na, nb = int(np.prod(out)), int(np.prod(a)), int(np.prod(b))
+        assert n <= N and na <= N and nb <= N
+        for op, nm in ((0, "add"), (3, "div")):
+            us = tm(lambda k: lib.shdw_hip_broadcast_binary(op, len(out), I(a), I(b), I(out), X[k].ptr, P.ptr,
+                                                            Y[k].ptr, st))
+            show("broadcast", "%s %s with %s" % (nm, a, b), us, 4 * (na + nb + n))
+    for inner in (1, 2, 3, 4):
         for num in (3, 64, 1000):
             n = (N // (num * inner)) * num * inner
             us = tm(lambda k: lib.shdw_hip_scale_bias(n, num, inner, X[k].ptr, P.ptr, Q.ptr, 0, Y[k].ptr, st))

@@ -56,8 +56,22 @@ SHDW_DEVICE float row_element(uint32_t e, float x, const float* s, const float* 
 //               128-bit fetch each (eight 4-byte fetches per lane ran at the
 //               address rate: 28 us against 17 us per 51 MB with 64 and more
 //               parameters);
-//   kRowAny:    a lookup per element.
-enum RowVectors { kRowAny = 0, kRowShared = 1, kRowEach = 2 };
+//   kRowPair:   any other inner >= 2: a vector starts in one row and may end in
+//               the next, never further, so it needs the parameters of two rows
+//               (a lookup per element: 24 us against 17 us with inner = 2 or 3);
+//   kRowAny:    a lookup per element (inner == 1, any num).
+enum RowVectors { kRowAny = 0, kRowShared = 1, kRowEach = 2, kRowPair = 3 };
+
+// Where the vector that starts at element e0 sits: the parameter index of its
+// first row and of the row after it, and how many of its elements the first row
+// still holds (4 and more: the vector does not reach the second row).
+SHDW_DEVICE void row_pair(uint32_t e0, const FastDiv& inner, const FastDiv& num, uint32_t& c0, uint32_t& c1,
+                          uint32_t& left) {
+  const uint32_t row = fd_div(e0, inner);
+  left = inner.d - (e0 - row * inner.d);
+  c0 = row - fd_div(row, num) * num.d;
+  c1 = c0 + 1 == num.d ? 0 : c0 + 1;
+}
 
 template <int MODE, bool RELU, int ROWS>
 __global__ __launch_bounds__(kStream) void rowparam_vec_kernel(const float* x, const float* s,
@@ -83,6 +97,16 @@ __global__ __launch_bounds__(kStream) void rowparam_vec_kernel(const float* x, c
       const float bv = (MODE == kScaleBias || MODE == kBiasOnly) ? b[c] : 0.f;
 #pragma unroll
       for (int j = 0; j < 4; ++j) r[j] = row_apply<MODE, RELU>(vx[j], sv, bv);
+    } else if (ROWS == kRowPair) {
+      uint32_t c0, c1, left;
+      row_pair(4 * i, inner, num, c0, c1, left);
+      const float s0 = (MODE != kBiasOnly) ? s[c0] : 0.f, s1 = (MODE != kBiasOnly) ? s[c1] : 0.f;
+      const bool biased = MODE == kScaleBias || MODE == kBiasOnly;
+      const float b0 = biased ? b[c0] : 0.f, b1 = biased ? b[c1] : 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        r[j] = row_apply<MODE, RELU>(vx[j], static_cast<uint32_t>(j) < left ? s0 : s1,
+                                     static_cast<uint32_t>(j) < left ? b0 : b1);
     } else {
 #pragma unroll
       for (int j = 0; j < 4; ++j) r[j] = row_element<MODE, RELU>(4 * i + j, vx[j], s, b, inner, num);
@@ -104,6 +128,8 @@ static int launch_rowparam(int n, int num, int inner, const float* x, const floa
     rowparam_vec_kernel<MODE, RELU, kRowShared><<<grid, kStream, 0, st>>>(x, s, b, y, n4, n, fi, fn);
   else if (inner == 1 && num % 4 == 0)
     rowparam_vec_kernel<MODE, RELU, kRowEach><<<grid, kStream, 0, st>>>(x, s, b, y, n4, n, fi, fn);
+  else if (inner >= 2)
+    rowparam_vec_kernel<MODE, RELU, kRowPair><<<grid, kStream, 0, st>>>(x, s, b, y, n4, n, fi, fn);
   else
     rowparam_vec_kernel<MODE, RELU, kRowAny><<<grid, kStream, 0, st>>>(x, s, b, y, n4, n, fi, fn);
   return launch_status();
@@ -131,6 +157,12 @@ __global__ __launch_bounds__(kStream) void rowbinary_vec_kernel(F f, const float
       const float bv = param(4 * i);
 #pragma unroll
       for (int j = 0; j < 4; ++j) r[j] = f(va[j], bv, tab);
+    } else if (inner.d >= 2) {  // two rows at the most: see kRowPair
+      uint32_t c0, c1, left;
+      row_pair(4 * i, inner, num, c0, c1, left);
+      const float b0 = b[c0], b1 = b[c1];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = f(va[j], static_cast<uint32_t>(j) < left ? b0 : b1, tab);
     } else {
 #pragma unroll
       for (int j = 0; j < 4; ++j) r[j] = f(va[j], param(4 * i + j), tab);

@@ -167,7 +167,8 @@ def test_activate_libm_wide_range(gpu, act):
 
 
 @pytest.mark.parametrize("shape,shared", [((2, 3, 5, 7), False), ((2, 3, 5, 7), True),
-                                          ((4, 16, 12), False), ((3, 8), False), ((1, 64, 56, 56), False)])
+                                          ((4, 16, 12), False), ((3, 8), False), ((1, 64, 56, 56), False),
+                                          ((5, 64, 2), False), ((3, 7, 3), False), ((2, 5, 7, 7), False)])
 def test_prelu(gpu, shape, shared):
     x = with_specials(normal(100, shape), 3)
     slope = uniform(101, 1 if shared else shape[1], -0.5, 0.5)
@@ -176,7 +177,11 @@ def test_prelu(gpu, shape, shared):
 
 
 @pytest.mark.parametrize("outer,num,inner", [(2, 3, 8), (4, 16, 196), (3, 5, 7), (1, 1, 1000),
-                                             (8, 64, 3136), (5, 7, 1), (2, 256, 30)])
+                                             (8, 64, 3136), (5, 7, 1), (2, 256, 30),
+                                             # vectors that end in the next row, the next row being parameter 0
+                                             # again, rows shorter than a vector, a ragged end
+                                             (3, 64, 2), (5, 3, 2), (7, 1000, 3), (9, 1, 3), (4, 3, 5), (2, 7, 49),
+                                             (11, 2, 6), (1, 13, 2), (3, 4, 1), (5, 64, 1)])
 @pytest.mark.parametrize("mode", ["sb", "s", "b"])
 def test_scale_bias(gpu, outer, num, inner, mode):
     n = outer * num * inner
@@ -221,6 +226,8 @@ BCAST_CASES = [
     ([2, 3], [2, 3]),
     ([17, 1, 3], [1, 11, 1]),
     ([3, 1, 2, 1, 7], [1, 4, 1, 6, 1]),   # five dims after collapsing: one output per lane
+    # a parameter per channel over rows of 2, 3, 5 and 6 elements: vectors that end in the next channel
+    ([9, 64, 2], [1, 64, 1]), ([4, 5, 3], [1, 5, 1]), ([7, 3, 5], [1, 3, 1]), ([2, 11, 2, 3], [1, 11, 1, 1]),
 ]
 
 
