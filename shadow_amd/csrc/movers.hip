@@ -211,15 +211,21 @@ __global__ __launch_bounds__(kBlock) void permute_generic_kernel(const float* x,
 // whole thin side and `span` elements of the long one; the side that is
 // contiguous in memory moves with 128-bit accesses as it lies, the element
 // shuffle happens in LDS.
-constexpr uint32_t kThinMax = 16;          // thin side up to this many elements
+constexpr uint32_t kThinMax = 128;         // thin side up to this many elements: the tile keeps 64 and more of the long side
 constexpr uint32_t kThinTileFloats = 8192;  // 32 KB
 
 // COLS_THIN: x[batch][big][thin] -> y[batch][thin][big]; else x[batch][thin][big] -> y[batch][big][thin].
-template <bool COLS_THIN>
+// PAD: thin is a multiple of 8.  The planar side walks the tile with a stride of
+// 4 * thin floats, one bank for all lanes then (thin = 64: 31 us per 51 MB against
+// 22 us for thin = 63 or 65); the tile rows get a pitch of thin + 1 instead, and
+// the contiguous side, whose vectors no longer sit on 16 bytes in LDS, moves its
+// four floats one by one there.
+template <bool COLS_THIN, bool PAD>
 __global__ __launch_bounds__(kBlock) void transpose_thin_kernel(const float* x, float* y, uint32_t big,
-                                                                 uint32_t thin, uint32_t span,
+                                                                 FastDiv f_thin, uint32_t span,
                                                                  FastDiv f_tiles) {
-  __shared__ __align__(16) float tile[kThinTileFloats];  // [span][thin], the interleaved side's order
+  __shared__ __align__(16) float tile[kThinTileFloats];  // [span][pitch], the interleaved side's order
+  const uint32_t thin = f_thin.d, pitch = PAD ? thin + 1 : thin;
   uint32_t b, t;
   fd_divmod(blockIdx.x, f_tiles, b, t);
   const uint32_t first = t * span, n = min(span, big - first);  // elements of the long side in this tile
@@ -229,48 +235,71 @@ __global__ __launch_bounds__(kBlock) void transpose_thin_kernel(const float* x, 
   const float* planar_src = x + image + first;  // row i at + i * big (not COLS_THIN)
   float* planar_dst = y + image + first;        // row j at + j * big (COLS_THIN)
   const uint32_t quads = n / 4;                 // whole vectors per planar row
+  // where vector v of the contiguous side starts in the padded tile (its four floats share a row: thin % 4 == 0)
+  auto padded = [&](uint32_t v) {
+    const uint32_t c = fd_div(4 * v, f_thin);
+    return c * pitch + (4 * v - c * thin);
+  };
   if (COLS_THIN) {
-    for (uint32_t v = threadIdx.x; v < cells / 4; v += kBlock)
-      *reinterpret_cast<v4f*>(tile + 4 * v) = load4_stream_any(inter + 4ull * v);
-    for (uint32_t e = (cells & ~3u) + threadIdx.x; e < cells; e += kBlock) tile[e] = inter[e];
+    if (PAD) {
+      for (uint32_t v = threadIdx.x; v < cells / 4; v += kBlock) {
+        const v4f r = load4_stream_any(inter + 4ull * v);
+        float* at = tile + padded(v);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) at[k] = r[k];
+      }
+    } else {
+      for (uint32_t v = threadIdx.x; v < cells / 4; v += kBlock)
+        *reinterpret_cast<v4f*>(tile + 4 * v) = load4_stream_any(inter + 4ull * v);
+      for (uint32_t e = (cells & ~3u) + threadIdx.x; e < cells; e += kBlock) tile[e] = inter[e];
+    }
     __syncthreads();
     for (uint32_t u = threadIdx.x; u < thin * quads; u += kBlock) {
       const uint32_t j = u / quads, q = u - j * quads;
       v4f r;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) r[k] = tile[(4 * q + k) * thin + j];
+      for (int k = 0; k < 4; ++k) r[k] = tile[(4 * q + k) * pitch + j];
       store4_stream_any(planar_dst + static_cast<uint64_t>(j) * big + 4 * q, r);
     }
     const uint32_t rest = n - 4 * quads;
     for (uint32_t u = threadIdx.x; u < thin * rest; u += kBlock) {
       const uint32_t j = u / rest, r = 4 * quads + (u - j * rest);
-      planar_dst[static_cast<uint64_t>(j) * big + r] = tile[r * thin + j];
+      planar_dst[static_cast<uint64_t>(j) * big + r] = tile[r * pitch + j];
     }
   } else {
     for (uint32_t u = threadIdx.x; u < thin * quads; u += kBlock) {
       const uint32_t i = u / quads, q = u - i * quads;
       const v4f r = load4_stream_any(planar_src + static_cast<uint64_t>(i) * big + 4 * q);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) tile[(4 * q + k) * thin + i] = r[k];
+      for (int k = 0; k < 4; ++k) tile[(4 * q + k) * pitch + i] = r[k];
     }
     const uint32_t rest = n - 4 * quads;
     for (uint32_t u = threadIdx.x; u < thin * rest; u += kBlock) {
       const uint32_t i = u / rest, c = 4 * quads + (u - i * rest);
-      tile[c * thin + i] = planar_src[static_cast<uint64_t>(i) * big + c];
+      tile[c * pitch + i] = planar_src[static_cast<uint64_t>(i) * big + c];
     }
     __syncthreads();
     float* out = const_cast<float*>(inter);
-    for (uint32_t v = threadIdx.x; v < cells / 4; v += kBlock)
-      store4_stream_any(out + 4ull * v, *reinterpret_cast<const v4f*>(tile + 4 * v));
-    for (uint32_t e = (cells & ~3u) + threadIdx.x; e < cells; e += kBlock) out[e] = tile[e];
+    if (PAD) {
+      for (uint32_t v = threadIdx.x; v < cells / 4; v += kBlock) {
+        const float* at = tile + padded(v);
+        store4_stream_any(out + 4ull * v, v4f{at[0], at[1], at[2], at[3]});
+      }
+    } else {
+      for (uint32_t v = threadIdx.x; v < cells / 4; v += kBlock)
+        store4_stream_any(out + 4ull * v, *reinterpret_cast<const v4f*>(tile + 4 * v));
+      for (uint32_t e = (cells & ~3u) + threadIdx.x; e < cells; e += kBlock) out[e] = tile[e];
+    }
   }
 }
 
 constexpr int kTile = 64;
 
-// VEC: rows % 4 == 0, cols % 4 == 0 and both pointers 16-byte aligned: 128-bit
-// loads along the input's fast axis and 128-bit stores along the output's.
-template <bool VEC>
+// 128-bit loads along the input's fast axis and 128-bit stores along the
+// output's, on whatever dword address a row starts (extents that are not
+// multiples of four, odd pointers); the last vector of a row that is not whole
+// moves float by float.  One float per lane instead ran at 2.2 to 2.7 times a
+// copy ([24][129][4148] -> [24][4148][129]: 38 us per 51 MB).
 __global__ __launch_bounds__(kBlock) void transpose_kernel(const float* x, float* y, uint32_t rows,
                                                             uint32_t cols, uint32_t tiles_c,
                                                             FastDiv f_tiles) {
@@ -280,41 +309,35 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(const float* x, float
   tr = t / tiles_c, tc = t - tr * tiles_c;
   const uint64_t plane = static_cast<uint64_t>(batch) * rows * cols;
   const uint32_t r0 = tr * kTile, c0 = tc * kTile;
-  if (VEC) {
-    const uint32_t q = threadIdx.x & 15u, line = threadIdx.x >> 4;  // 16 vectors x 16 lines
+  const uint32_t q = threadIdx.x & 15u, line = threadIdx.x >> 4;  // 16 vectors x 16 lines
 #pragma unroll
-    for (uint32_t k = line; k < kTile; k += kBlock / 16) {
-      const uint32_t r = r0 + k, c = c0 + 4 * q;
-      if (r < rows && c < cols) {
-        const v4f v = load4_stream(x + plane + static_cast<uint64_t>(r) * cols + c);
+  for (uint32_t k = line; k < kTile; k += kBlock / 16) {
+    const uint32_t r = r0 + k, c = c0 + 4 * q;
+    if (r < rows && c < cols) {
+      const float* src = x + plane + static_cast<uint64_t>(r) * cols + c;
+      if (c + 4 <= cols) {
+        const v4f v = load4_stream_any(src);
 #pragma unroll
         for (int j = 0; j < 4; ++j) tile[k][4 * q + j] = v[j];
+      } else {
+        for (uint32_t j = 0; c + j < cols; ++j) tile[k][4 * q + j] = __builtin_nontemporal_load(src + j);
       }
     }
-    __syncthreads();
+  }
+  __syncthreads();
 #pragma unroll
-    for (uint32_t k = line; k < kTile; k += kBlock / 16) {
-      const uint32_t c = c0 + k, r = r0 + 4 * q;
-      if (r < rows && c < cols) {
+  for (uint32_t k = line; k < kTile; k += kBlock / 16) {
+    const uint32_t c = c0 + k, r = r0 + 4 * q;
+    if (r < rows && c < cols) {
+      float* dst = y + plane + static_cast<uint64_t>(c) * rows + r;
+      if (r + 4 <= rows) {
         v4f v;
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = tile[4 * q + j][k];
-        store4_stream(y + plane + static_cast<uint64_t>(c) * rows + r, v);
+        store4_stream_any(dst, v);
+      } else {
+        for (uint32_t j = 0; r + j < rows; ++j) dst[j] = tile[4 * q + j][k];
       }
-    }
-  } else {
-    const uint32_t lx = threadIdx.x & 63u, ly = threadIdx.x >> 6;  // 64 x 4 lanes
-#pragma unroll 4
-    for (uint32_t k = ly; k < kTile; k += kBlock / kTile) {
-      const uint32_t r = r0 + k, c = c0 + lx;
-      if (r < rows && c < cols)
-        tile[k][lx] = __builtin_nontemporal_load(x + plane + static_cast<uint64_t>(r) * cols + c);
-    }
-    __syncthreads();
-#pragma unroll 4
-    for (uint32_t k = ly; k < kTile; k += kBlock / kTile) {
-      const uint32_t c = c0 + k, r = r0 + lx;
-      if (r < rows && c < cols) y[plane + static_cast<uint64_t>(c) * rows + r] = tile[lx][k];
     }
   }
 }
@@ -926,15 +949,21 @@ int shdw_hip_permute(int num_axes, const int* in_shape, const int* order, const 
     if (std::min(rows, cols) <= kThinMax && std::max(rows, cols) >= 256) {
       const bool cols_thin = cols <= rows;
       const uint32_t thin = cols_thin ? cols : rows, big = cols_thin ? rows : cols;
-      const uint32_t span = (kThinTileFloats / thin) & ~63u;
-      const uint32_t tiles = (big + span - 1) / span;
+      const bool pad = thin % 8 == 0;
+      const uint32_t span = (kThinTileFloats / (thin + (pad ? 1 : 0))) & ~63u;
+      const uint32_t tiles = span ? (big + span - 1) / span : 0;  // span 0: a padded side of 128 does not fit
       const int64_t groups = static_cast<int64_t>(batch) * tiles;
-      if (groups <= INT32_MAX) {
-        const FastDiv ft = make_fastdiv(tiles);
-        if (cols_thin)
-          transpose_thin_kernel<true><<<static_cast<uint32_t>(groups), kBlock, 0, st>>>(x, y, big, thin, span, ft);
+      if (span && groups <= INT32_MAX) {
+        const FastDiv ft = make_fastdiv(tiles), fthin = make_fastdiv(thin);
+        const uint32_t g = static_cast<uint32_t>(groups);
+        if (cols_thin && pad)
+          transpose_thin_kernel<true, true><<<g, kBlock, 0, st>>>(x, y, big, fthin, span, ft);
+        else if (cols_thin)
+          transpose_thin_kernel<true, false><<<g, kBlock, 0, st>>>(x, y, big, fthin, span, ft);
+        else if (pad)
+          transpose_thin_kernel<false, true><<<g, kBlock, 0, st>>>(x, y, big, fthin, span, ft);
         else
-          transpose_thin_kernel<false><<<static_cast<uint32_t>(groups), kBlock, 0, st>>>(x, y, big, thin, span, ft);
+          transpose_thin_kernel<false, false><<<g, kBlock, 0, st>>>(x, y, big, fthin, span, ft);
         return launch_status();
       }
     }
@@ -943,10 +972,7 @@ int shdw_hip_permute(int num_axes, const int* in_shape, const int* order, const 
     if (groups <= INT32_MAX) {
       const FastDiv ft = make_fastdiv(tiles_r * tiles_c);
       const uint32_t g = static_cast<uint32_t>(groups);
-      if (rows % 4 == 0 && cols % 4 == 0 && aligned16(x) && aligned16(y))
-        transpose_kernel<true><<<g, kBlock, 0, st>>>(x, y, rows, cols, tiles_c, ft);
-      else
-        transpose_kernel<false><<<g, kBlock, 0, st>>>(x, y, rows, cols, tiles_c, ft);
+      transpose_kernel<<<g, kBlock, 0, st>>>(x, y, rows, cols, tiles_c, ft);
       return launch_status();
     }
   }

@@ -113,7 +113,13 @@ def test_pad_op(ws, pads, shape):
     # one thin side (interleaved <-> planar images): whole and ragged tiles, odd lengths, batches
     ((1000, 3), [1, 0]), ((3, 1000), [1, 0]), ((2, 37, 41, 3), [0, 3, 1, 2]), ((2, 3, 37, 41), [0, 2, 3, 1]),
     ((3, 777, 5), [0, 2, 1]), ((2, 16, 9001), [0, 2, 1]), ((9001, 16), [1, 0]), ((1, 6000, 1), [1, 0, 2]),
-    ((4, 260, 1, 2), [0, 3, 2, 1]), ((5462, 3), [1, 0]), ((2, 257, 13), [0, 2, 1]), ((17, 300), [1, 0])])
+    ((4, 260, 1, 2), [0, 3, 2, 1]), ((5462, 3), [1, 0]), ((2, 257, 13), [0, 2, 1]), ((17, 300), [1, 0]),
+    # thin sides up to 128 (a detection head's [anchors][85][cells] -> [anchors][cells][85]); multiples of
+    # eight take the padded tile
+    ((3, 85, 1444), [0, 2, 1]), ((3, 1444, 85), [0, 2, 1]), ((2, 8, 1000), [0, 2, 1]), ((2, 1001, 8), [0, 2, 1]),
+    ((64, 300), [1, 0]), ((300, 64), [1, 0]), ((2, 24, 5000), [0, 2, 1]), ((5000, 120), [1, 0]),
+    ((120, 4999), [1, 0]), ((127, 257), [1, 0]), ((256, 128), [1, 0]), ((128, 256), [1, 0]), ((100, 333), [1, 0]),
+    ((1, 3, 85, 19, 19), [0, 1, 3, 4, 2])])
 def test_permute_op(ws, shape, order):
     x = normal(60, shape)
     got = run(ws, "Permute", [("x", x)], {"order": order})
