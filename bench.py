@@ -363,7 +363,8 @@ def sweep(dev):
         show("row norm", "[%d,%d]%s" % (outer, inner, " (sliced rows)" if need else ""), us, 8 * outer * inner)
     for shape, k, s, p in (([16, 64, 112, 112], 3, 2, 1), ([16, 64, 112, 112], 2, 2, 0), ([16, 64, 112, 112], 3, 1, 1),
                            ([64, 1024, 14, 14], 2, 2, 0), ([64, 1024, 14, 14], 3, 1, 1), ([128, 2048, 7, 7], 3, 1, 1),
-                           ([512, 512, 7, 7], 7, 1, 3), ([64, 1024, 14, 14], 13, 1, 6), ([16, 64, 112, 112], 5, 1, 2)):
+                           ([512, 512, 7, 7], 7, 1, 3), ([64, 1024, 14, 14], 13, 1, 6), ([16, 64, 112, 112], 5, 1, 2),
+                           ([64, 512, 19, 19], 9, 1, 4), ([19, 1000, 26, 26], 5, 1, 2), ([19, 1000, 26, 26], 13, 1, 6)):
         n_, c_, h_, w_ = shape
         oh, ow = (h_ + 2 * p - k) // s + 1, (w_ + 2 * p - k) // s + 1
         for pt, nm in ((0, "max"), (1, "avg")):

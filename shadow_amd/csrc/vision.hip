@@ -391,6 +391,7 @@ static bool plan_pool_band(const PoolArgs& p, int target_outputs, BandArgs* a) {
 // earliest row.
 constexpr int kSmallPlanesTileFloats = 12288;  // 48 KB: three workgroups per CU
 constexpr int kSmallPlanesMaxOutputs = 512;    // larger planes go to the band kernel
+constexpr int kSeparableMinCells = 16;         // max windows from this size on fold rows first
 
 struct SmallPlanesArgs {
   int in_h, in_w, out_h, out_w, kh, kw, sh, sw, ph, pw;
@@ -508,12 +509,14 @@ __global__ __launch_bounds__(kBlock) void pool_small_planes_kernel(const float* 
 
 // Fills `a` and returns true where the kernel above applies: several padded
 // planes fit the tile and one plane alone would leave lanes idle.
-constexpr int kSeparableMinCells = 16;
-
 static bool plan_small_planes(const PoolArgs& p, int64_t total_planes, bool max_pool, SmallPlanesArgs* a,
                               bool* separable) {
   const int64_t plane_out = static_cast<int64_t>(p.out_h) * p.out_w, plane_in = static_cast<int64_t>(p.in_h) * p.in_w;
-  if (plane_out > kSmallPlanesMaxOutputs || plane_out < 1 || total_planes > INT32_MAX) return false;
+  // the two-step maximum is worth whole planes of up to 32 x 32 as well (13x13 windows on
+  // 26x26 maps: 64 us per 51 MB; the band kernel, which walks every cell of every window,
+  // takes 369 us for the average over the same windows)
+  const bool wide_max = max_pool && p.kh * p.kw >= kSeparableMinCells;
+  if (plane_out > (wide_max ? 2 : 1) * kSmallPlanesMaxOutputs || plane_out < 1 || total_planes > INT32_MAX) return false;
   const int over_b = std::max(0, (p.out_h - 1) * p.sh - p.ph + p.kh - p.in_h);
   const int over_r = std::max(0, (p.out_w - 1) * p.sw - p.pw + p.kw - p.in_w);
   const int64_t pitch = static_cast<int64_t>(p.pw) + p.in_w + over_r;
@@ -522,7 +525,8 @@ static bool plan_small_planes(const PoolArgs& p, int64_t total_planes, bool max_
   if (plane_lds * 2 > kSmallPlanesTileFloats) return false;
   const int64_t rows_lds = static_cast<int64_t>(p.ph) + p.in_h + over_b;
   const int64_t row_maxima = rows_lds * p.out_w;
-  *separable = max_pool && p.kh * p.kw >= kSeparableMinCells && (plane_lds + row_maxima) * 2 <= kSmallPlanesTileFloats;
+  *separable = wide_max && (plane_lds + row_maxima) * 2 <= kSmallPlanesTileFloats;
+  if (plane_out > kSmallPlanesMaxOutputs && !*separable) return false;
   int64_t planes = kSmallPlanesTileFloats / (plane_lds + (*separable ? row_maxima : 0));
   const int64_t want = (4 * kBlock + plane_out - 1) / plane_out;  // about four outputs per lane
   planes = std::min(planes, std::max<int64_t>(2, want));

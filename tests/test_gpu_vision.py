@@ -281,6 +281,9 @@ POOL_2D = [
     ((2, 8, 13, 13), [5], [1], [2], False), ((2, 8, 13, 13), [9], [1], [4], False), ((2, 8, 13, 13), [13], [1], [6], False),
     ((1, 5, 19, 19), [13], [1], [6], True), ((3, 3, 14, 14), [7], [1], [3], True), ((1, 7, 20, 20), [4, 5], [2, 1], [1, 2], True),
     ((2, 2, 16, 11), [6, 4], [3, 2], [0, 1], False),
+    # planes of 513 to 1024 outputs: whole planes for the two-step maximum, bands for the rest
+    ((2, 5, 26, 26), [13], [1], [6], False), ((1, 3, 32, 32), [5], [1], [2], False), ((2, 3, 30, 23), [9, 4], [1, 1], [4, 2], True),
+    ((1, 2, 33, 32), [5], [1], [2], False),
 ]
 
 
