@@ -8,8 +8,10 @@
 namespace shdw {
 
 // kStrided with kFlatMinInner <= inner < kFlatMaxInner goes through the flat
-// kernel (4 * inner <= 1024 must hold for odd inner: 127 * 4 = 508).
-constexpr int64_t kFlatMinInner = 8, kFlatMaxInner = 128;
+// kernel (4 * inner <= 1024 must hold for odd inner: 127 * 4 = 508); so do 2 to
+// 7 columns when a slab fills at least one step of the workgroup (channels over
+// a row of 7: the column kernels would use 7 lanes of 64).
+constexpr int64_t kFlatMinInner = 8, kFlatMaxInner = 128, kFlatNarrowInner = 2, kFlatNarrowSlab = 1024;
 
 int plan_broadcast(int num_axes, const int* a_shape, const int* b_shape,
                    const int* out_shape, BroadcastPlan* plan) {
@@ -131,6 +133,18 @@ int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* ax
     } else if (nc == 3 && !cred[0]) {
       plan->kind = kStrided;
       plan->outer = cdim[0], plan->reduce = cdim[1], plan->inner = cdim[2];
+    } else if (nc == 3) {  // [lead][kept][reduce]: a channel's statistics over batch and plane
+      plan->kind = kRows;
+      plan->lead = cdim[0], plan->lead_inner = cdim[1];
+      plan->outer = cdim[0] * cdim[1], plan->reduce = cdim[2], plan->inner = 1;
+    } else if (nc == 4 && !cred[0]) {  // [kept][lead][kept][reduce]
+      plan->kind = kRows;
+      plan->lead = cdim[1], plan->lead_inner = cdim[2];
+      plan->outer = cdim[0] * cdim[1] * cdim[2], plan->reduce = cdim[3], plan->inner = 1;
+    } else if (nc == 4) {  // [lead][kept][reduce][kept]
+      plan->kind = kStrided;
+      plan->lead = cdim[0], plan->lead_inner = cdim[1];
+      plan->outer = cdim[0] * cdim[1], plan->reduce = cdim[2], plan->inner = cdim[3];
     } else {
       fast = false;
     }
@@ -170,7 +184,9 @@ int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* ax
       const int by_work = ceil_div64(plan->reduce, 4096);  // >= 4 vectors per lane
       plan->splits = std::max(1, std::min(by_fill, by_work));
     }
-  } else if (plan->inner < kFlatMaxInner && plan->inner >= kFlatMinInner) {
+  } else if (plan->inner < kFlatMaxInner &&
+             (plan->inner >= kFlatMinInner ||
+              (plan->inner >= kFlatNarrowInner && plan->reduce * plan->inner >= kFlatNarrowSlab))) {
     // Few columns: a column tile would leave most lanes idle (56 columns use 14
     // of a wave's 64 lanes with 128-bit loads).  The [reduce][inner] slab of one
     // outer index is contiguous, so the 256 lanes of a workgroup walk it flat,

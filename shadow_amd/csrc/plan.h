@@ -34,6 +34,8 @@ int plan_broadcast(int num_axes, const int* a_shape, const int* b_shape,
 // Reduce.
 //   kRows    : x viewed as [outer][reduce], reduced axis contiguous.
 //   kStrided : x viewed as [outer][reduce][inner], inner > 1 contiguous.
+//   Either view may have one more reduced dim in front (ReducePlan::lead): the
+//   statistics of a channel over batch and plane are [lead][outer][reduce].
 //   kGeneric : any other axis pattern (several separated reduced groups, or
 //              axes not listed in ascending order, where Shadow's list order is
 //              not memory order).  Kept/reduced dims are passed uncollapsed.
@@ -53,6 +55,11 @@ struct ReducePlan {
   int strided_waves = 4;      // kStrided, one column per lane: wave64 per workgroup sharing a column tile (4 or 16)
   int flat_period = 0;        // kStrided with fewer than 128 columns: > 0 selects the flat kernel; elements
                               // the 256 lanes cover per step (a multiple of inner and of 4, <= 1024)
+  int64_t lead = 1;           // > 1: one more reduced dim in front of the view above, [a][lead][b][reduce] for
+                              // kRows (outer = a * lead * b) and [lead][b][reduce][inner] for kStrided
+                              // (outer = lead * b); the first stage treats it as kept and leaves one partial
+                              // per leading index (and slice), the second stage folds them
+  int64_t lead_inner = 1;     // b
   int64_t outputs = 1;        // number of output elements
   int64_t window = 1;         // elements per output (Shadow's num_list)
   // kGeneric only: kept dims (outermost first) and reduced dims in LIST order,
@@ -67,8 +74,11 @@ constexpr size_t kReducePartialBytes = 8;  // fp64 accumulator, or {fp32 extremu
 int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* axes,
                 ReducePlan* plan);
 
+// Partials per output that the first stage leaves (1: it writes the results itself).
+inline int64_t reduce_slots(const ReducePlan& p) { return p.lead * p.splits; }
+
 inline size_t reduce_workspace_bytes(const ReducePlan& p) {
-  return p.splits > 1 ? static_cast<size_t>(p.outputs) * p.splits * kReducePartialBytes : 0;
+  return reduce_slots(p) > 1 ? static_cast<size_t>(p.outputs) * reduce_slots(p) * kReducePartialBytes : 0;
 }
 
 }  // namespace shdw

@@ -11,6 +11,9 @@
 //   generic  any axis set               one wave per output, index lists
 //                                       replaced by division by constants.
 //   stage 2  combines the per-slice partials of a split first stage.
+//   A reduced dim in front of the rows or strided view (the statistics of a
+//   channel over batch and plane: x[lead][kept][reduce]) is treated as kept by
+//   the first stage, which leaves one partial per leading index for stage 2.
 //
 // The accumulators (fp64 sums, or an fp32 extremum with the position of its
 // first zero) are in reduce_acc.h.
@@ -32,6 +35,55 @@ namespace shdw {
 
 constexpr int kBatch = 8;  // vectors a lane requests before it consumes the first
 
+// A reduced dim in front of a kernel's own view (ReducePlan::lead).  The kernels
+// run over lead * (kept outer) outer indices; where a result goes, and which list
+// positions its elements have, follows from the leading index of the outer index.
+struct Lead {
+  uint32_t count = 1;  // extent of the leading reduced dim; 1: there is none
+  uint32_t step = 0;   // list positions per leading index: the extent the kernel reduces itself
+  FastDiv f_inner, f_count;  // outer index = (a * count + lead) * inner + b
+  SHDW_DEVICE void place(uint32_t o, uint32_t& out_outer, uint32_t& lead) const {
+    uint32_t q, b, a;
+    fd_divmod(o, f_inner, q, b);
+    fd_divmod(q, f_count, a, lead);
+    out_outer = a * f_inner.d + b;
+  }
+};
+
+// The result of (row, slice) of a rows kernel: the output itself, or a partial
+// in the layout [output][slot] that stage 2 reads.
+template <class A>
+SHDW_DEVICE void emit_row(const Lead& ld, A acc, uint32_t row, uint32_t split, uint32_t splits, uint32_t reduce,
+                          float* y, Partial* part) {
+  if (ld.count == 1) {
+    if (splits == 1) y[row] = acc.finalize(reduce);
+    else part[static_cast<size_t>(row) * splits + split] = acc.pack();
+    return;
+  }
+  uint32_t out, lead;
+  ld.place(row, out, lead);
+  acc.shift_positions(lead * ld.step);
+  part[(static_cast<size_t>(out) * ld.count + lead) * splits + split] = acc.pack();
+}
+
+// The result of (outer index, column, slice) of a strided kernel; partials in
+// the layout [slot][output].
+template <class A>
+SHDW_DEVICE void emit_column(const Lead& ld, A acc, uint32_t o, uint32_t col, uint32_t inner, uint32_t split,
+                             uint32_t splits, uint32_t outputs, uint32_t reduce, float* y, Partial* part) {
+  if (ld.count == 1) {
+    const size_t out = static_cast<size_t>(o) * inner + col;
+    if (splits == 1) y[out] = acc.finalize(reduce);
+    else part[static_cast<size_t>(split) * outputs + out] = acc.pack();
+    return;
+  }
+  uint32_t oo, lead;
+  ld.place(o, oo, lead);
+  acc.shift_positions(lead * ld.step);
+  const size_t out = static_cast<size_t>(oo) * inner + col;
+  part[(static_cast<size_t>(lead) * splits + split) * outputs + out] = acc.pack();
+}
+
 // ---------------------------------------------------------------------------
 // rows, G lanes per row (G = 16, 32, 64): short rows share a wave so that no
 // lane idles and the combine stays inside DPP rows where possible.
@@ -39,7 +91,7 @@ constexpr int kBatch = 8;  // vectors a lane requests before it consumes the fir
 template <int OP, bool VEC, int G>
 __global__ __launch_bounds__(kBlock) void reduce_rows_group_kernel(const float* x, float* y,
                                                                     uint32_t rows,
-                                                                    uint32_t reduce) {
+                                                                    uint32_t reduce, Partial* part, Lead ld) {
   const uint32_t lane = threadIdx.x & (G - 1);
   const uint32_t row_raw = blockIdx.x * (kBlock / G) + (threadIdx.x / G);
   // Groups past the end recompute the last row (and do not store) so that all
@@ -68,7 +120,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_group_kernel(const float* 
     for (uint32_t i = lane; i < reduce; i += G) acc.add(p[i], i);
   }
   acc = group_allreduce<Acc<OP>, G>(acc);
-  if (lane == 0 && row_raw < rows) y[row] = acc.finalize(reduce);
+  if (lane == 0 && row_raw < rows) emit_row(ld, acc, row, 0, 1, reduce, y, part);
 }
 
 // ---------------------------------------------------------------------------
@@ -79,7 +131,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const float* 
                                                                     Partial* part,
                                                                     uint32_t reduce,
                                                                     uint32_t chunk,
-                                                                    uint32_t splits) {
+                                                                    uint32_t splits, Lead ld) {
   __shared__ Partial lds[kBlock / kWave];
   const uint32_t row = blockIdx.x, split = blockIdx.y;  // rows can exceed the 65535 limit of grid.y
   const float* p = x + static_cast<size_t>(row) * reduce;
@@ -128,8 +180,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_block_kernel(const float* 
       o.unpack(lds[k]);
       acc.merge(o);
     }
-    if (splits == 1) y[row] = acc.finalize(reduce);
-    else part[static_cast<size_t>(row) * splits + split] = acc.pack();
+    emit_row(ld, acc, row, split, splits, reduce, y, part);
   }
 }
 
@@ -155,7 +206,7 @@ constexpr uint32_t kShortRowMaxLen = 256;  // rows up to 255 floats: 16 lanes ea
 template <int OP, int L, bool PADDED>
 __global__ __launch_bounds__(kBlock) void reduce_rows_lds_kernel(const float* x, float* y, uint32_t rows,
                                                                   uint32_t reduce, uint32_t seg,
-                                                                  FastDiv f_reduce4) {
+                                                                  FastDiv f_reduce4, Partial* part, Lead ld) {
   constexpr uint32_t kRows = kBlock / L;
   __shared__ __align__(16) float tile[kShortRowMaxFloats];
   const uint32_t pitch = PADDED ? 4 * ((reduce / 4 + 1) | 1u) : reduce;  // an odd number of 128-bit pieces
@@ -198,7 +249,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_lds_kernel(const float* x,
   }
   for (; c < c_end; ++c) acc.add(mine[c], c);
   if (L > 1) acc = group_allreduce<Acc<OP>, (L > 1 ? L : 2)>(acc);
-  if (h == 0 && r < nrows) y[row0 + r] = acc.finalize(reduce);
+  if (h == 0 && r < nrows) emit_row(ld, acc, row0 + r, 0, 1, reduce, y, part);
 }
 
 // ---------------------------------------------------------------------------
@@ -214,7 +265,8 @@ constexpr uint32_t kShortStridedMaxReduce = 32;
 template <int OP, bool VEC>
 __global__ __launch_bounds__(kBlock) void reduce_strided_short_kernel(const float* x, float* y, uint32_t reduce,
                                                                        uint32_t inner, uint32_t units,
-                                                                       FastDiv f_units_per_outer) {
+                                                                       FastDiv f_units_per_outer, Partial* part,
+                                                                       uint32_t outputs, Lead ld) {
   constexpr int W = VEC ? 4 : 1;
   const uint32_t u = blockIdx.x * kBlock + threadIdx.x;
   if (u >= units) return;
@@ -250,6 +302,11 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_short_kernel(const floa
 #pragma unroll
         for (int j = 0; j < W; ++j) acc[j].add(v[k][j], r + k);
   }
+  if (ld.count > 1) {
+#pragma unroll
+    for (int j = 0; j < W; ++j) emit_column(ld, acc[j], o, c * W + j, inner, 0, 1, outputs, reduce, y, part);
+    return;
+  }
   float* dst = y + static_cast<uint64_t>(o) * inner + static_cast<uint64_t>(c) * W;
   if (VEC) {
     v4f out;
@@ -274,7 +331,7 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_short_kernel(const floa
 template <int OP>
 __global__ __launch_bounds__(kBlock) void reduce_strided_flat_kernel(
     const float* x, float* y, Partial* part, uint32_t reduce, uint32_t inner, uint32_t rows_per_split,
-    uint32_t splits, uint32_t outputs, uint32_t period, FastDiv f_inner) {
+    uint32_t splits, uint32_t outputs, uint32_t period, FastDiv f_inner, Lead ld) {
   __shared__ Partial lds[4 * kBlock];
   const uint32_t o = blockIdx.x, split = blockIdx.y;
   const uint32_t r_begin = min(split * rows_per_split, reduce);
@@ -324,9 +381,7 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_flat_kernel(
       t.unpack(lds[s]);
       total.merge(t);
     }
-    const size_t out = static_cast<size_t>(o) * inner + threadIdx.x;
-    if (splits == 1) y[out] = total.finalize(reduce);
-    else part[static_cast<size_t>(split) * outputs + out] = total.pack();
+    emit_column(ld, total, o, threadIdx.x, inner, split, splits, outputs, reduce, y, part);
   }
 }
 
@@ -339,7 +394,7 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_flat_kernel(
 template <int OP, int WAVES>
 __global__ __launch_bounds__(kWave * WAVES) void reduce_strided_kernel(
     const float* x, float* y, Partial* part, uint32_t reduce, uint32_t inner,
-    uint32_t rows_per_split, uint32_t splits, uint32_t outputs, FastDiv f_tiles) {
+    uint32_t rows_per_split, uint32_t splits, uint32_t outputs, FastDiv f_tiles, Lead ld) {
   constexpr int kWaves = WAVES;
   __shared__ Partial lds[kWaves - 1][kWave];
   const uint32_t lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
@@ -375,9 +430,7 @@ __global__ __launch_bounds__(kWave * WAVES) void reduce_strided_kernel(
       t.unpack(lds[k][lane]);
       acc.merge(t);
     }
-    const size_t out = static_cast<size_t>(o) * inner + col;
-    if (splits == 1) y[out] = acc.finalize(reduce);
-    else part[static_cast<size_t>(split) * outputs + out] = acc.pack();
+    emit_column(ld, acc, o, col, inner, split, splits, outputs, reduce, y, part);
   }
 }
 
@@ -398,7 +451,7 @@ constexpr int kTileThreads = 512;
 template <int OP, int L>
 __global__ __launch_bounds__(kTileThreads) void reduce_strided_tile_kernel(
     const float* x, float* y, Partial* part, uint32_t reduce, uint32_t inner, uint32_t rows_per_split,
-    uint32_t splits, uint32_t outputs, FastDiv f_tiles) {
+    uint32_t splits, uint32_t outputs, FastDiv f_tiles, Lead ld) {
   constexpr uint32_t kGroups = kTileThreads / L;
   __shared__ Partial lds[kTileThreads * 4];
   uint32_t o, tile;
@@ -449,11 +502,7 @@ __global__ __launch_bounds__(kTileThreads) void reduce_strided_tile_kernel(
       t.unpack(lds[g * 4 * L + threadIdx.x]);
       total.merge(t);
     }
-    if (c < inner) {
-      const size_t out = static_cast<size_t>(o) * inner + c;
-      if (splits == 1) y[out] = total.finalize(reduce);
-      else part[static_cast<size_t>(split) * outputs + out] = total.pack();
-    }
+    if (c < inner) emit_column(ld, total, o, c, inner, split, splits, outputs, reduce, y, part);
   }
 }
 
@@ -643,6 +692,13 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
     return launch_status();
   }
 
+  Lead ld;
+  ld.count = static_cast<uint32_t>(pl.lead);
+  ld.step = static_cast<uint32_t>(pl.reduce);
+  ld.f_inner = make_fastdiv(static_cast<uint32_t>(pl.lead_inner));
+  ld.f_count = make_fastdiv(ld.count);
+  const uint32_t slots = static_cast<uint32_t>(reduce_slots(pl));  // partials per output; 1: the first stage finishes
+
   if (pl.kind == kRows) {
     const uint32_t rows = static_cast<uint32_t>(pl.outer);
     const uint32_t reduce = static_cast<uint32_t>(pl.reduce);
@@ -656,8 +712,8 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
       const FastDiv f4 = make_fastdiv(std::max<uint32_t>(1, reduce / 4));
 #define SHDW_SHORT(LANES)                                                                                  \
   do {                                                                                                     \
-    if (reduce % 4 == 0) reduce_rows_lds_kernel<OP, LANES, true><<<grid, kBlock, 0, st>>>(x, y, rows, reduce, seg, f4);  \
-    else reduce_rows_lds_kernel<OP, LANES, false><<<grid, kBlock, 0, st>>>(x, y, rows, reduce, seg, f4);   \
+    if (reduce % 4 == 0) reduce_rows_lds_kernel<OP, LANES, true><<<grid, kBlock, 0, st>>>(x, y, rows, reduce, seg, f4, part, ld);  \
+    else reduce_rows_lds_kernel<OP, LANES, false><<<grid, kBlock, 0, st>>>(x, y, rows, reduce, seg, f4, part, ld);   \
   } while (0)
       if (lanes == 1) SHDW_SHORT(1);
       else if (lanes == 2) SHDW_SHORT(2);
@@ -665,7 +721,9 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
       else if (lanes == 8) SHDW_SHORT(8);
       else SHDW_SHORT(16);
 #undef SHDW_SHORT
-      return launch_status();
+      const int rc = launch_status();
+      if (rc != SHDW_OK || slots == 1) return rc;
+      return run_stage2<OP>(part, y, outputs, slots, slots, 1, window, st);
     }
     if (pl.wave_per_row) {
       // lanes per row: a lane fetches up to 8 vectors, all requested before the
@@ -674,26 +732,28 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
       const uint32_t units = vec ? (reduce + 3) / 4 : reduce;
       const int g = units <= 128 ? 16 : (units <= 256 ? 32 : 64);
       const uint32_t grid = (rows + kBlock / g - 1) / (kBlock / g);
-#define SHDW_ROWS(V, G) reduce_rows_group_kernel<OP, V, G><<<grid, kBlock, 0, st>>>(x, y, rows, reduce)
+#define SHDW_ROWS(V, G) reduce_rows_group_kernel<OP, V, G><<<grid, kBlock, 0, st>>>(x, y, rows, reduce, part, ld)
       if (vec) {
         if (g == 16) SHDW_ROWS(true, 16); else if (g == 32) SHDW_ROWS(true, 32); else SHDW_ROWS(true, 64);
       } else {
         if (g == 16) SHDW_ROWS(false, 16); else if (g == 32) SHDW_ROWS(false, 32); else SHDW_ROWS(false, 64);
       }
 #undef SHDW_ROWS
-      return launch_status();
+      const int rc = launch_status();
+      if (rc != SHDW_OK || slots == 1) return rc;
+      return run_stage2<OP>(part, y, outputs, slots, slots, 1, window, st);
     }
     const uint32_t splits = static_cast<uint32_t>(pl.splits);
     uint32_t chunk = (reduce + splits - 1) / splits;
     chunk = (chunk + 3) & ~3u;
     const dim3 grid(rows, splits);
     if (vec)
-      reduce_rows_block_kernel<OP, true><<<grid, kBlock, 0, st>>>(x, y, part, reduce, chunk, splits);
+      reduce_rows_block_kernel<OP, true><<<grid, kBlock, 0, st>>>(x, y, part, reduce, chunk, splits, ld);
     else
-      reduce_rows_block_kernel<OP, false><<<grid, kBlock, 0, st>>>(x, y, part, reduce, chunk, splits);
+      reduce_rows_block_kernel<OP, false><<<grid, kBlock, 0, st>>>(x, y, part, reduce, chunk, splits, ld);
     int rc = launch_status();
-    if (rc != SHDW_OK || splits == 1) return rc;
-    return run_stage2<OP>(part, y, rows, splits, splits, 1, window, st);
+    if (rc != SHDW_OK || slots == 1) return rc;
+    return run_stage2<OP>(part, y, outputs, slots, slots, 1, window, st);
   }
 
   // strided
@@ -707,15 +767,17 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
     const uint32_t per_outer = vec ? inner / 4 : inner;
     const uint32_t units = outer * per_outer;  // <= outputs
     const FastDiv f = make_fastdiv(per_outer);
-    if (vec) reduce_strided_short_kernel<OP, true><<<grid_for(units), kBlock, 0, st>>>(x, y, reduce, inner, units, f);
-    else reduce_strided_short_kernel<OP, false><<<grid_for(units), kBlock, 0, st>>>(x, y, reduce, inner, units, f);
-    return launch_status();
+    if (vec) reduce_strided_short_kernel<OP, true><<<grid_for(units), kBlock, 0, st>>>(x, y, reduce, inner, units, f, part, outputs, ld);
+    else reduce_strided_short_kernel<OP, false><<<grid_for(units), kBlock, 0, st>>>(x, y, reduce, inner, units, f, part, outputs, ld);
+    const int rc = launch_status();
+    if (rc != SHDW_OK || slots == 1) return rc;
+    return run_stage2<OP>(part, y, outputs, slots, 1, outputs, window, st);
   }
   if (pl.flat_period > 0) {
     // grid.x carries outer (at most INT32_MAX, as the element count), grid.y the slices (<= 1024)
     reduce_strided_flat_kernel<OP><<<dim3(outer, splits), kBlock, 0, st>>>(
         x, y, part, reduce, inner, rows_per_split, splits, outputs, static_cast<uint32_t>(pl.flat_period),
-        make_fastdiv(inner));
+        make_fastdiv(inner), ld);
   } else if (pl.strided_lanes > 0) {  // inner % 4 == 0: tiles of 4 * lanes columns, 128-bit loads
     const uint32_t l = static_cast<uint32_t>(pl.strided_lanes);
     const uint32_t tiles = (inner / 4 + l - 1) / l;
@@ -723,7 +785,7 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
     const FastDiv f_tiles = make_fastdiv(tiles);
 #define SHDW_TILE(LANES)                                                                                   \
   reduce_strided_tile_kernel<OP, LANES><<<grid, kTileThreads, 0, st>>>(x, y, part, reduce, inner, rows_per_split, \
-                                                                       splits, outputs, f_tiles)
+                                                                       splits, outputs, f_tiles, ld)
     if (l == 8) SHDW_TILE(8); else if (l == 16) SHDW_TILE(16); else if (l == 32) SHDW_TILE(32); else SHDW_TILE(64);
 #undef SHDW_TILE
   } else {
@@ -732,14 +794,14 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
     const FastDiv f_tiles = make_fastdiv(tiles);
     if (pl.strided_waves == 16)
       reduce_strided_kernel<OP, 16><<<grid, kWave * 16, 0, st>>>(x, y, part, reduce, inner, rows_per_split, splits,
-                                                                 outputs, f_tiles);
+                                                                 outputs, f_tiles, ld);
     else
       reduce_strided_kernel<OP, 4><<<grid, kWave * 4, 0, st>>>(x, y, part, reduce, inner, rows_per_split, splits,
-                                                               outputs, f_tiles);
+                                                               outputs, f_tiles, ld);
   }
   int rc = launch_status();
-  if (rc != SHDW_OK || splits == 1) return rc;
-  return run_stage2<OP>(part, y, outputs, splits, 1, outputs, window, st);
+  if (rc != SHDW_OK || slots == 1) return rc;
+  return run_stage2<OP>(part, y, outputs, slots, 1, outputs, window, st);
 }
 
 static int dispatch_reduce(int operation, const ReducePlan& pl, const float* x, float* y,

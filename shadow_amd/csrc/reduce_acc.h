@@ -71,6 +71,7 @@ struct Acc {
     if (OP == SHDW_REDUCE_L2) return __builtin_sqrtf(static_cast<float>(v));
     return static_cast<float>(v);
   }
+  SHDW_DEVICE void shift_positions(uint32_t) {}
   SHDW_DEVICE Partial pack() const { return Partial{static_cast<uint64_t>(__double_as_longlong(v))}; }
   SHDW_DEVICE void unpack(const Partial& p) { v = __longlong_as_double(static_cast<long long>(p.bits)); }
 };
@@ -122,6 +123,10 @@ struct Acc<OP, true> {
   SHDW_DEVICE float finalize(uint32_t) const {
     if (v == 0.0f) return (key & 1u) ? -0.0f : 0.0f;
     return v;
+  }
+  // the positions given to add() were relative to `by`
+  SHDW_DEVICE void shift_positions(uint32_t by) {
+    if (key != 0xffffffffu) key += by << 1;
   }
   SHDW_DEVICE Partial pack() const {
     return Partial{(static_cast<uint64_t>(key) << 32) | __float_as_uint(v)};

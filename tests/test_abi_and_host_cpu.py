@@ -90,7 +90,12 @@ def test_reduce_plans_of_the_benchmark_shapes():
     assert (rc, kind, outer, red, inner) == (0, ROWS, 1, 12845056, 1) and splits > 64
     rc, (kind, outer, red, inner, splits) = plan_reduce([64, 1024, 14, 14], [2, 3])
     assert (rc, kind, outer, red, inner, splits) == (0, ROWS, 65536, 196, 1, 1)
-    assert plan_reduce([2, 3, 4, 5], [0, 2])[1][0] == GENERIC
+    # one reduced dim in front of a rows or strided view is folded by the second stage: the view
+    # counts it among the outer indices, and the workspace holds a partial per leading index
+    assert plan_reduce([2, 3, 4, 5], [0, 2])[1][:4] == [STRIDED, 6, 4, 5]
+    assert plan_reduce([64, 256, 28, 28], [0, 2, 3])[1] == [ROWS, 64 * 256, 784, 1, 1]
+    assert plan_reduce([8, 256, 4, 28], [1, 3])[1][:4] == [ROWS, 8 * 256 * 4, 28, 1]
+    assert plan_reduce([2, 3, 4, 5, 6], [0, 2, 4])[1][0] == GENERIC
     assert plan_reduce([2, 3, 4, 5], [3, 2])[1][0] == GENERIC  # list order is not memory order
     assert plan_reduce([6, 1, 5], [1])[1][:4] == [STRIDED, 1, 1, 30]
     assert plan_reduce([2, 3], [-1])[0] == -1
@@ -99,6 +104,7 @@ def test_reduce_plans_of_the_benchmark_shapes():
     lib = shadow_amd.hip()
     assert lib.shdw_hip_reduce_workspace_bytes(4, ints([32, 512, 28, 28]), 2, ints([2, 3])) == 0
     assert lib.shdw_hip_reduce_workspace_bytes(1, ints([1 << 24]), 1, ints([0])) % 8 == 0
+    assert lib.shdw_hip_reduce_workspace_bytes(4, ints([64, 256, 28, 28]), 3, ints([0, 2, 3])) == 8 * 256 * 64
 
 
 def keys(fn):

@@ -300,6 +300,16 @@ REDUCE_CASES = [
     ([3, 2, 9], [1]),
     # short rows of odd length through LDS, one lane per row
     ([700, 9], [1]), ([513, 127], [1]), ([260, 5], [1]), ([257, 5, 5], [1, 2]), ([1027, 66], [1]),
+    # a reduced dim in front of the rows / strided view, folded by the second stage: channel statistics
+    # over batch and plane with rows short, medium and sliced; [kept][lead][kept][reduce]; strided
+    # views with short, narrow, vector and odd column counts
+    ([6, 5, 7, 7], [0, 2, 3]), ([4, 300, 28, 28], [0, 2, 3]), ([3, 2, 300, 301], [0, 2, 3]), ([70, 3, 5], [0, 2]),
+    ([3, 4, 5, 6], [1, 3]), ([2, 300, 3, 700], [1, 3]), ([5, 2, 9, 5000], [1, 3]), ([300, 2, 2, 9], [1, 3]),
+    ([6, 5, 7, 9], [0, 2]), ([5, 3, 40, 64], [0, 2]), ([3, 2, 9, 256], [0, 2]), ([4, 3, 300, 130], [0, 2]),
+    ([2, 3, 4000, 12], [0, 2]), ([7, 2, 33, 1001], [0, 2]), ([9, 4, 3, 7, 5], [0, 1, 3]), ([2, 3, 4, 5, 6], [1, 2, 4]),
+    # two to seven columns with slabs of a step and more: the flat walk
+    ([3, 1024, 7], [1]), ([5, 700, 2], [1]), ([2, 9000, 3], [1]), ([4, 300, 5], [1]), ([2, 171, 6], [1]), ([3, 170, 6], [1]),
+    ([2, 3, 600, 7], [0, 2]),
 ]
 
 
@@ -333,7 +343,11 @@ def test_reduce_beyond_the_second_grid_dimension(gpu, shape, axes, op):
 
 @pytest.mark.parametrize("shape,axes", [([64, 48], [1]), ([3, 64, 8], [1]), ([2, 3, 4, 5], [3, 1]),
                                         ([50000], [0]), ([300, 16], [1]), ([3, 500, 49], [1]), ([2, 6000, 12], [1]), ([300, 49], [1]),
-                                        ([1000, 9], [1])])
+                                        ([1000, 9], [1]),
+                                        # the first zero of a window lies under another leading index
+                                        ([6, 5, 7, 7], [0, 2, 3]), ([3, 2, 300, 301], [0, 2, 3]), ([5, 2, 9, 500], [1, 3]),
+                                        ([6, 5, 7, 9], [0, 2]), ([4, 3, 300, 130], [0, 2]), ([7, 2, 33, 101], [0, 2]),
+                                        ([3, 1024, 7], [1]), ([2, 9000, 3], [1])])
 @pytest.mark.parametrize("op", [2, 3])
 def test_reduce_select_special_values(gpu, shape, axes, op):
     """Zeros of both signs, NaNs and infinities: the first extremum in list
