@@ -26,6 +26,7 @@ BASELINE rows, the oracle's time on this host.
 """
 import argparse
 import ctypes
+import itertools
 import json
 import os
 import re
@@ -342,6 +343,19 @@ def sweep(dev):
                 us = tm(lambda k: lib.shdw_hip_reduce(op, 2, I(shape), 1, I(axes), X[k].ptr, Y[k].ptr,
                                                       scratch.ptr if need else None, need, st))
                 show(kind, "%s over %d of [%s]" % (nm, L, "x".join(map(str, shape))), us, 4 * (rows * L + rows))
+    for shape in ([64, 256, 28, 28], [256, 1024, 7, 7], [8, 3, 732, 731]):
+        n = int(np.prod(shape))
+        assert n <= N
+        for r in (1, 2, 3):
+            for axes in itertools.combinations(range(4), r):
+                axes = list(axes)
+                need = lib.shdw_hip_reduce_workspace_bytes(4, I(shape), r, I(axes))
+                assert need <= (64 << 20)
+                outs = n // int(np.prod([shape[a] for a in axes]))
+                for op, nm in ((1, "sum"), (2, "max")):
+                    us = tm(lambda k: lib.shdw_hip_reduce(op, 4, I(shape), r, I(axes), X[k].ptr, Y[k].ptr,
+                                                          scratch.ptr if need else None, need, st))
+                    show("reduce axes", "%s of %s over axes %s" % (nm, shape, axes), us, 4 * (n + outs))
     for which in ("softmax", "normalize"):
         for dim in (2, 8, 21, 49, 64, 65, 150, 256, 512, 513, 1000, 4096):
             for inner in (1, 2, 7, 16, 49, 196, 3136):

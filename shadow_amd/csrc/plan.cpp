@@ -12,6 +12,10 @@ namespace shdw {
 // 7 columns when a slab fills at least one step of the workgroup (channels over
 // a row of 7: the column kernels would use 7 lanes of 64).
 constexpr int64_t kFlatMinInner = 8, kFlatMaxInner = 128, kFlatNarrowInner = 2, kFlatNarrowSlab = 1024;
+// Two reduced dims around a kept one: the second stage takes the inner one when
+// it is this short and the leading one at least this long (the partials then
+// stay under a sixteenth of the input).
+constexpr int64_t kNestMax = 64, kNestMinLead = 32;
 
 int plan_broadcast(int num_axes, const int* a_shape, const int* b_shape,
                    const int* out_shape, BroadcastPlan* plan) {
@@ -133,18 +137,34 @@ int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* ax
     } else if (nc == 3 && !cred[0]) {
       plan->kind = kStrided;
       plan->outer = cdim[0], plan->reduce = cdim[1], plan->inner = cdim[2];
-    } else if (nc == 3) {  // [lead][kept][reduce]: a channel's statistics over batch and plane
-      plan->kind = kRows;
-      plan->lead = cdim[0], plan->lead_inner = cdim[1];
-      plan->outer = cdim[0] * cdim[1], plan->reduce = cdim[2], plan->inner = 1;
-    } else if (nc == 4 && !cred[0]) {  // [kept][lead][kept][reduce]
-      plan->kind = kRows;
-      plan->lead = cdim[1], plan->lead_inner = cdim[2];
-      plan->outer = cdim[0] * cdim[1] * cdim[2], plan->reduce = cdim[3], plan->inner = 1;
-    } else if (nc == 4) {  // [lead][kept][reduce][kept]
-      plan->kind = kStrided;
-      plan->lead = cdim[0], plan->lead_inner = cdim[1];
-      plan->outer = cdim[0] * cdim[1], plan->reduce = cdim[2], plan->inner = cdim[3];
+    } else if (nc == 3 || nc == 4) {
+      // two reduced dims with a kept one between them: [k0][lead][k1][r1] (k0 = 1 for nc == 3), or
+      // [lead][k0][r1][k1] where the last dim is kept
+      const bool rows = cred[nc - 1];
+      const int64_t k0 = rows ? (nc == 4 ? cdim[0] : 1) : cdim[1];
+      const int64_t lead = rows ? cdim[nc - 3] : cdim[0];
+      const int64_t k1 = rows ? cdim[nc - 2] : cdim[3];
+      const int64_t r1 = rows ? cdim[nc - 1] : cdim[2];
+      if (r1 <= kNestMax && lead >= kNestMinLead && r1 < lead) {
+        // the long leading dim first, as a strided reduce with all that follows as columns
+        plan->kind = kStrided;
+        plan->nest = r1;
+        if (rows) {  // columns (k1, r1): those of output (k0, k1) are neighbours
+          plan->outer = k0, plan->reduce = lead, plan->inner = k1 * r1;
+          plan->nest_olo = 1, plan->nest_ohi_stride = r1, plan->nest_stride = 1;
+        } else {  // columns (k0, r1, k1)
+          plan->outer = 1, plan->reduce = lead, plan->inner = k0 * r1 * k1;
+          plan->nest_olo = k1, plan->nest_ohi_stride = r1 * k1, plan->nest_stride = k1;
+        }
+      } else if (rows) {
+        plan->kind = kRows;
+        plan->lead = lead, plan->lead_inner = k1;
+        plan->outer = k0 * lead * k1, plan->reduce = r1, plan->inner = 1;
+      } else {
+        plan->kind = kStrided;
+        plan->lead = lead, plan->lead_inner = k0;
+        plan->outer = lead * k0, plan->reduce = r1, plan->inner = k1;
+      }
     } else {
       fast = false;
     }

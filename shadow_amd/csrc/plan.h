@@ -60,6 +60,12 @@ struct ReducePlan {
                               // (outer = lead * b); the first stage treats it as kept and leaves one partial
                               // per leading index (and slice), the second stage folds them
   int64_t lead_inner = 1;     // b
+  // nest > 1: the other order for a short reduce extent behind a long leading one ([lead][kept][nest] or
+  // [lead][kept][nest][kept'], nest <= 64 < lead): the view is kStrided over the leading dim with everything
+  // behind it as columns (lead = 1 for the kernels), the first stage leaves partials per slice and column of the
+  // view, and the second stage folds slices and the nest columns of an output: column of (output o, j) =
+  // (o / nest_olo) * nest_ohi_stride + o % nest_olo + j * nest_stride
+  int64_t nest = 1, nest_olo = 1, nest_ohi_stride = 1, nest_stride = 1;
   int64_t outputs = 1;        // number of output elements
   int64_t window = 1;         // elements per output (Shadow's num_list)
   // kGeneric only: kept dims (outermost first) and reduced dims in LIST order,
@@ -78,6 +84,7 @@ int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* ax
 inline int64_t reduce_slots(const ReducePlan& p) { return p.lead * p.splits; }
 
 inline size_t reduce_workspace_bytes(const ReducePlan& p) {
+  if (p.nest > 1) return static_cast<size_t>(p.outer * p.inner) * p.splits * kReducePartialBytes;
   return reduce_slots(p) > 1 ? static_cast<size_t>(p.outputs) * reduce_slots(p) * kReducePartialBytes : 0;
 }
 

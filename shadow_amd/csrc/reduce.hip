@@ -39,7 +39,8 @@ constexpr int kBatch = 8;  // vectors a lane requests before it consumes the fir
 // run over lead * (kept outer) outer indices; where a result goes, and which list
 // positions its elements have, follows from the leading index of the outer index.
 struct Lead {
-  uint32_t count = 1;  // extent of the leading reduced dim; 1: there is none
+  uint32_t count = 1;  // extent of the leading reduced dim; 1: there is none; 0: there is none, and the
+                       // strided kernel leaves partials even where it does not slice (a nested second stage)
   uint32_t step = 0;   // list positions per leading index: the extent the kernel reduces itself
   FastDiv f_inner, f_count;  // outer index = (a * count + lead) * inner + b
   SHDW_DEVICE void place(uint32_t o, uint32_t& out_outer, uint32_t& lead) const {
@@ -71,9 +72,9 @@ SHDW_DEVICE void emit_row(const Lead& ld, A acc, uint32_t row, uint32_t split, u
 template <class A>
 SHDW_DEVICE void emit_column(const Lead& ld, A acc, uint32_t o, uint32_t col, uint32_t inner, uint32_t split,
                              uint32_t splits, uint32_t outputs, uint32_t reduce, float* y, Partial* part) {
-  if (ld.count == 1) {
+  if (ld.count <= 1) {
     const size_t out = static_cast<size_t>(o) * inner + col;
-    if (splits == 1) y[out] = acc.finalize(reduce);
+    if (splits == 1 && ld.count == 1) y[out] = acc.finalize(reduce);
     else part[static_cast<size_t>(split) * outputs + out] = acc.pack();
     return;
   }
@@ -302,7 +303,7 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_short_kernel(const floa
 #pragma unroll
         for (int j = 0; j < W; ++j) acc[j].add(v[k][j], r + k);
   }
-  if (ld.count > 1) {
+  if (ld.count != 1) {
 #pragma unroll
     for (int j = 0; j < W; ++j) emit_column(ld, acc[j], o, c * W + j, inner, 0, 1, outputs, reduce, y, part);
     return;
@@ -634,6 +635,97 @@ static int run_stage2(const Partial* part, float* y, uint32_t outputs, uint32_t 
 }
 
 // ---------------------------------------------------------------------------
+// stage 2 after a first stage that reduced the leading dim of [lead][..][nest]
+// (ReducePlan::nest): an output folds the partials of `slices` slices times
+// `nest` columns of the first stage's view.  The first stage counted list
+// positions in leading indices; the element (leading index p, nest index j) has
+// list position p * nest + j.
+// ---------------------------------------------------------------------------
+struct Nest {
+  uint32_t nest, stride, ohi_stride;
+  FastDiv f_nest, f_olo;
+  size_t view;  // partials per slice
+  SHDW_DEVICE size_t first_column(uint32_t o) const {
+    uint32_t hi, lo;
+    fd_divmod(o, f_olo, hi, lo);
+    return static_cast<size_t>(hi) * ohi_stride + lo;
+  }
+};
+
+template <int OP>
+SHDW_DEVICE Acc<OP> nested_partial(const Partial* part, const Nest& n, size_t column0, uint32_t s) {
+  uint32_t slice, j;
+  fd_divmod(s, n.f_nest, slice, j);
+  Acc<OP> t;
+  t.unpack(part[slice * n.view + column0 + static_cast<size_t>(j) * n.stride]);
+  t.nest_positions(n.nest, j);
+  return t;
+}
+
+template <int OP>
+__global__ __launch_bounds__(kBlock) void reduce_stage2_nested_lane_kernel(const Partial* part, float* y,
+                                                                            uint32_t outputs, uint32_t slices,
+                                                                            Nest n, uint32_t window) {
+  const uint32_t o = blockIdx.x * kBlock + threadIdx.x;
+  if (o >= outputs) return;
+  const size_t column0 = n.first_column(o);
+  Acc<OP> acc;
+  acc.init();
+  const uint32_t total = slices * n.nest;
+  uint32_t s = 0;
+  for (; s + 8 <= total; s += 8) {  // eight requests in flight, as in reduce_stage2_lane_kernel
+    Acc<OP> t[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) t[k] = nested_partial<OP>(part, n, column0, s + k);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc.merge(t[k]);
+  }
+  for (; s < total; ++s) acc.merge(nested_partial<OP>(part, n, column0, s));
+  y[o] = acc.finalize(window);
+}
+
+template <int OP>
+__global__ __launch_bounds__(kBlock) void reduce_stage2_nested_block_kernel(const Partial* part, float* y,
+                                                                             uint32_t slices, Nest n,
+                                                                             uint32_t window) {
+  __shared__ Partial lds[kBlock / kWave];
+  const uint32_t o = blockIdx.x;
+  const size_t column0 = n.first_column(o);
+  Acc<OP> acc;
+  acc.init();
+  const uint32_t total = slices * n.nest;
+  for (uint32_t s = threadIdx.x; s < total; s += kBlock) acc.merge(nested_partial<OP>(part, n, column0, s));
+  acc = wave_allreduce(acc);
+  const uint32_t lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+  if (lane == 0) lds[w] = acc.pack();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < kBlock / kWave; ++k) {
+      Acc<OP> t;
+      t.unpack(lds[k]);
+      acc.merge(t);
+    }
+    y[o] = acc.finalize(window);
+  }
+}
+
+template <int OP>
+static int run_stage2_nested(const Partial* part, float* y, const ReducePlan& pl, uint32_t window, hipStream_t st) {
+  Nest n;
+  n.nest = static_cast<uint32_t>(pl.nest), n.stride = static_cast<uint32_t>(pl.nest_stride);
+  n.ohi_stride = static_cast<uint32_t>(pl.nest_ohi_stride);
+  n.f_nest = make_fastdiv(n.nest), n.f_olo = make_fastdiv(static_cast<uint32_t>(pl.nest_olo));
+  n.view = static_cast<size_t>(pl.outer * pl.inner);
+  const uint32_t outputs = static_cast<uint32_t>(pl.outputs), slices = static_cast<uint32_t>(pl.splits);
+  // a lane per output where the outputs fill the chip or the walk is a few partials, else a workgroup per output
+  if (static_cast<uint64_t>(slices) * n.nest <= 8 || outputs >= 16384)
+    reduce_stage2_nested_lane_kernel<OP><<<grid_for(outputs), kBlock, 0, st>>>(part, y, outputs, slices, n, window);
+  else
+    reduce_stage2_nested_block_kernel<OP><<<outputs, kBlock, 0, st>>>(part, y, slices, n, window);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
 // Partial results of shdw_hip_reduce_static: device memory of the library
 // itself, one copy on every GPU the library runs on.  Host code uses the address
 // that hipGetSymbolAddress returns for the current device (static_scratch), never
@@ -761,22 +853,27 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
   const uint32_t reduce = static_cast<uint32_t>(pl.reduce);
   const uint32_t inner = static_cast<uint32_t>(pl.inner);
   const uint32_t splits = static_cast<uint32_t>(pl.splits);
+  const bool nested = pl.nest > 1;  // the kernels below then leave partials per column of their own view
+  const uint32_t view = nested ? outer * inner : outputs;
+  if (nested) ld.count = 0;
   const uint32_t rows_per_split = (reduce + splits - 1) / splits;
   if (pl.flat_period == 0 && splits == 1 && reduce <= kShortStridedMaxReduce) {
     const bool vec = inner % 4 == 0;
     const uint32_t per_outer = vec ? inner / 4 : inner;
     const uint32_t units = outer * per_outer;  // <= outputs
     const FastDiv f = make_fastdiv(per_outer);
-    if (vec) reduce_strided_short_kernel<OP, true><<<grid_for(units), kBlock, 0, st>>>(x, y, reduce, inner, units, f, part, outputs, ld);
-    else reduce_strided_short_kernel<OP, false><<<grid_for(units), kBlock, 0, st>>>(x, y, reduce, inner, units, f, part, outputs, ld);
+    if (vec) reduce_strided_short_kernel<OP, true><<<grid_for(units), kBlock, 0, st>>>(x, y, reduce, inner, units, f, part, view, ld);
+    else reduce_strided_short_kernel<OP, false><<<grid_for(units), kBlock, 0, st>>>(x, y, reduce, inner, units, f, part, view, ld);
     const int rc = launch_status();
-    if (rc != SHDW_OK || slots == 1) return rc;
+    if (rc != SHDW_OK) return rc;
+    if (nested) return run_stage2_nested<OP>(part, y, pl, window, st);
+    if (slots == 1) return rc;
     return run_stage2<OP>(part, y, outputs, slots, 1, outputs, window, st);
   }
   if (pl.flat_period > 0) {
     // grid.x carries outer (at most INT32_MAX, as the element count), grid.y the slices (<= 1024)
     reduce_strided_flat_kernel<OP><<<dim3(outer, splits), kBlock, 0, st>>>(
-        x, y, part, reduce, inner, rows_per_split, splits, outputs, static_cast<uint32_t>(pl.flat_period),
+        x, y, part, reduce, inner, rows_per_split, splits, view, static_cast<uint32_t>(pl.flat_period),
         make_fastdiv(inner), ld);
   } else if (pl.strided_lanes > 0) {  // inner % 4 == 0: tiles of 4 * lanes columns, 128-bit loads
     const uint32_t l = static_cast<uint32_t>(pl.strided_lanes);
@@ -785,7 +882,7 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
     const FastDiv f_tiles = make_fastdiv(tiles);
 #define SHDW_TILE(LANES)                                                                                   \
   reduce_strided_tile_kernel<OP, LANES><<<grid, kTileThreads, 0, st>>>(x, y, part, reduce, inner, rows_per_split, \
-                                                                       splits, outputs, f_tiles, ld)
+                                                                       splits, view, f_tiles, ld)
     if (l == 8) SHDW_TILE(8); else if (l == 16) SHDW_TILE(16); else if (l == 32) SHDW_TILE(32); else SHDW_TILE(64);
 #undef SHDW_TILE
   } else {
@@ -794,13 +891,15 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
     const FastDiv f_tiles = make_fastdiv(tiles);
     if (pl.strided_waves == 16)
       reduce_strided_kernel<OP, 16><<<grid, kWave * 16, 0, st>>>(x, y, part, reduce, inner, rows_per_split, splits,
-                                                                 outputs, f_tiles, ld);
+                                                                 view, f_tiles, ld);
     else
       reduce_strided_kernel<OP, 4><<<grid, kWave * 4, 0, st>>>(x, y, part, reduce, inner, rows_per_split, splits,
-                                                               outputs, f_tiles, ld);
+                                                               view, f_tiles, ld);
   }
   int rc = launch_status();
-  if (rc != SHDW_OK || slots == 1) return rc;
+  if (rc != SHDW_OK) return rc;
+  if (nested) return run_stage2_nested<OP>(part, y, pl, window, st);
+  if (slots == 1) return rc;
   return run_stage2<OP>(part, y, outputs, slots, 1, outputs, window, st);
 }
 

@@ -72,6 +72,7 @@ struct Acc {
     return static_cast<float>(v);
   }
   SHDW_DEVICE void shift_positions(uint32_t) {}
+  SHDW_DEVICE void nest_positions(uint32_t, uint32_t) {}
   SHDW_DEVICE Partial pack() const { return Partial{static_cast<uint64_t>(__double_as_longlong(v))}; }
   SHDW_DEVICE void unpack(const Partial& p) { v = __longlong_as_double(static_cast<long long>(p.bits)); }
 };
@@ -127,6 +128,11 @@ struct Acc<OP, true> {
   // the positions given to add() were relative to `by`
   SHDW_DEVICE void shift_positions(uint32_t by) {
     if (key != 0xffffffffu) key += by << 1;
+  }
+  // the positions given to add() were leading indices p of elements (p, j) whose
+  // list position is p * nest + j
+  SHDW_DEVICE void nest_positions(uint32_t nest, uint32_t j) {
+    if (key != 0xffffffffu) key = (((key >> 1) * nest + j) << 1) | (key & 1u);
   }
   SHDW_DEVICE Partial pack() const {
     return Partial{(static_cast<uint64_t>(key) << 32) | __float_as_uint(v)};

@@ -94,7 +94,10 @@ def test_reduce_plans_of_the_benchmark_shapes():
     # counts it among the outer indices, and the workspace holds a partial per leading index
     assert plan_reduce([2, 3, 4, 5], [0, 2])[1][:4] == [STRIDED, 6, 4, 5]
     assert plan_reduce([64, 256, 28, 28], [0, 2, 3])[1] == [ROWS, 64 * 256, 784, 1, 1]
-    assert plan_reduce([8, 256, 4, 28], [1, 3])[1][:4] == [ROWS, 8 * 256 * 4, 28, 1]
+    assert plan_reduce([8, 16, 4, 28], [1, 3])[1][:4] == [ROWS, 8 * 16 * 4, 28, 1]
+    # a short reduced dim behind a long leading one: the leading dim first, over all that follows as columns
+    assert plan_reduce([8, 256, 4, 28], [1, 3])[1][:4] == [STRIDED, 8, 256, 4 * 28]
+    assert plan_reduce([256, 1024, 7, 7], [0, 2])[1][:4] == [STRIDED, 1, 256, 1024 * 49]
     assert plan_reduce([2, 3, 4, 5, 6], [0, 2, 4])[1][0] == GENERIC
     assert plan_reduce([2, 3, 4, 5], [3, 2])[1][0] == GENERIC  # list order is not memory order
     assert plan_reduce([6, 1, 5], [1])[1][:4] == [STRIDED, 1, 1, 30]

@@ -307,6 +307,11 @@ REDUCE_CASES = [
     ([3, 4, 5, 6], [1, 3]), ([2, 300, 3, 700], [1, 3]), ([5, 2, 9, 5000], [1, 3]), ([300, 2, 2, 9], [1, 3]),
     ([6, 5, 7, 9], [0, 2]), ([5, 3, 40, 64], [0, 2]), ([3, 2, 9, 256], [0, 2]), ([4, 3, 300, 130], [0, 2]),
     ([2, 3, 4000, 12], [0, 2]), ([7, 2, 33, 1001], [0, 2]), ([9, 4, 3, 7, 5], [0, 1, 3]), ([2, 3, 4, 5, 6], [1, 2, 4]),
+    # a short reduced dim behind a long leading one: the leading dim first, the second stage folds slices and
+    # the short dim (rows-like and strided-like, lane and workgroup per output, every first-stage kernel)
+    ([40, 3, 7], [0, 2]), ([300, 5, 9], [0, 2]), ([3, 33, 4, 16], [1, 3]), ([5000, 2, 3], [0, 2]), ([64, 70, 63], [0, 2]),
+    ([40, 6, 7, 5], [0, 2]), ([33, 300, 4, 8], [0, 2]), ([2000, 2, 5, 3], [0, 2]), ([32, 3, 31, 130], [0, 2]),
+    ([100, 1030, 2], [0, 2]), ([9000, 1, 4, 1, 3], [0, 2]),
     # two to seven columns with slabs of a step and more: the flat walk
     ([3, 1024, 7], [1]), ([5, 700, 2], [1]), ([2, 9000, 3], [1]), ([4, 300, 5], [1]), ([2, 171, 6], [1]), ([3, 170, 6], [1]),
     ([2, 3, 600, 7], [0, 2]),
@@ -347,7 +352,8 @@ def test_reduce_beyond_the_second_grid_dimension(gpu, shape, axes, op):
                                         # the first zero of a window lies under another leading index
                                         ([6, 5, 7, 7], [0, 2, 3]), ([3, 2, 300, 301], [0, 2, 3]), ([5, 2, 9, 500], [1, 3]),
                                         ([6, 5, 7, 9], [0, 2]), ([4, 3, 300, 130], [0, 2]), ([7, 2, 33, 101], [0, 2]),
-                                        ([3, 1024, 7], [1]), ([2, 9000, 3], [1])])
+                                        ([3, 1024, 7], [1]), ([2, 9000, 3], [1]),
+                                        ([300, 5, 9], [0, 2]), ([5000, 2, 3], [0, 2]), ([40, 6, 7, 5], [0, 2]), ([2000, 2, 5, 3], [0, 2])])
 @pytest.mark.parametrize("op", [2, 3])
 def test_reduce_select_special_values(gpu, shape, axes, op):
     """Zeros of both signs, NaNs and infinities: the first extremum in list
