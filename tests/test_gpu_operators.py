@@ -114,7 +114,10 @@ def test_eltwise_op_errors(ws):
 
 
 @pytest.mark.parametrize("shape,axes", [((4, 8, 7, 7), [2, 3]), ((4, 8, 7, 7), [1]), ((4, 8, 7, 7), []),
-                                        ((2, 3, 4, 5), [0, 2]), ((6, 10), [0]), ((5,), [0])])
+                                        ((2, 3, 4, 5), [0, 2]), ((6, 10), [0]), ((5,), [0]),
+                                        # two stages through the Workspace's temp buffer: channel statistics,
+                                        # the leading dim first, sliced rows behind a leading dim
+                                        ((6, 8, 9, 9), [0, 2, 3]), ((40, 6, 7, 5), [0, 2]), ((3, 2, 300, 301), [0, 2, 3])])
 @pytest.mark.parametrize("operation", range(7))
 @pytest.mark.parametrize("keep_dims", [True, False])
 def test_reduce_op(ws, shape, axes, operation, keep_dims):
