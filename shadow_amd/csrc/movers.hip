@@ -211,13 +211,14 @@ __global__ __launch_bounds__(kBlock) void permute_generic_kernel(const float* x,
 // whole thin side and `span` elements of the long one; the side that is
 // contiguous in memory moves with 128-bit accesses as it lies, the element
 // shuffle happens in LDS.
-constexpr uint32_t kThinMax = 128;         // thin side up to this many elements: the tile keeps 64 and more of the long side
+constexpr uint32_t kThinMax = 127;         // thin side up to this many elements: the tile keeps 64 and more of the long side
+constexpr uint32_t kThinNarrow = 16;       // ... and sides of 17 to 64 stay with the 64 x 64 tiles
 constexpr uint32_t kThinTileFloats = 8192;  // 32 KB
 
 // COLS_THIN: x[batch][big][thin] -> y[batch][thin][big]; else x[batch][thin][big] -> y[batch][big][thin].
 // PAD: thin is a multiple of 8.  The planar side walks the tile with a stride of
-// 4 * thin floats, one bank for all lanes then (thin = 64: 31 us per 51 MB against
-// 22 us for thin = 63 or 65); the tile rows get a pitch of thin + 1 instead, and
+// 4 * thin floats, one bank for all lanes then (thin = 8: 30 us per 51 MB against
+// 22 us for thin = 17); the tile rows get a pitch of thin + 1 instead (21 us), and
 // the contiguous side, whose vectors no longer sit on 16 bytes in LDS, moves its
 // four floats one by one there.
 template <bool COLS_THIN, bool PAD>
@@ -946,7 +947,9 @@ int shdw_hip_permute(int num_axes, const int* in_shape, const int* order, const 
     const uint32_t batch = plain2 ? 1u : static_cast<uint32_t>(ext[0]);
     const uint32_t cols = static_cast<uint32_t>(plain2 ? ext[0] : ext[1]);  // input's fast axis
     const uint32_t rows = static_cast<uint32_t>(plain2 ? ext[1] : ext[2]);
-    if (std::min(rows, cols) <= kThinMax && std::max(rows, cols) >= 256) {
+    // sides of 17 to 64 fill a 64 x 64 tile well enough: measured level with the thin kernel or ahead of it
+    const uint32_t side = std::min(rows, cols);
+    if ((side <= kThinNarrow || (side > static_cast<uint32_t>(kTile) && side <= kThinMax)) && std::max(rows, cols) >= 256) {
       const bool cols_thin = cols <= rows;
       const uint32_t thin = cols_thin ? cols : rows, big = cols_thin ? rows : cols;
       const bool pad = thin % 8 == 0;
