@@ -177,9 +177,9 @@ __global__ __launch_bounds__(kStream) void rowbinary_vec_kernel(F f, const float
 // Broadcast binary on collapsed dims.
 // ---------------------------------------------------------------------------
 struct BcastArgs {
-  FastDiv fd[4];  // divisors for dims 1..NDIM-1 are used (dim 0 is the quotient)
-  int sa[4];
-  int sb[4];
+  FastDiv fd[kMaxDims];  // divisors for dims 1..NDIM-1 are used (dim 0 is the quotient)
+  int sa[kMaxDims];
+  int sb[kMaxDims];
   int a_full;  // a is not broadcast anywhere: stream it
   int b_full;
 };
@@ -296,35 +296,6 @@ __global__ __launch_bounds__(kBlock) void bcast_flat_kernel(F f, BcastArgs p, co
   }
 }
 
-struct BcastGenericArgs {
-  int ndim;
-  FastDiv fd[kMaxDims];
-  int sa[kMaxDims];
-  int sb[kMaxDims];
-};
-
-// Any rank up to 8, any extents, one output per lane.
-template <class F>
-__global__ __launch_bounds__(kBlock) void bcast_generic_kernel(F f, BcastGenericArgs p,
-                                                                const float* a, const float* b,
-                                                                float* y, uint32_t n) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-  const uint64_t* tab = uses_exp_table<F>::value ? libm::kExp2fTab : nullptr;
-  if (i < n) {
-    uint32_t e = i, oa = 0, ob = 0;
-    for (int k = p.ndim - 1; k >= 1; --k) {
-      uint32_t q, r;
-      fd_divmod(e, p.fd[k], q, r);
-      oa += r * static_cast<uint32_t>(p.sa[k]);
-      ob += r * static_cast<uint32_t>(p.sb[k]);
-      e = q;
-    }
-    oa += e * static_cast<uint32_t>(p.sa[0]);
-    ob += e * static_cast<uint32_t>(p.sb[0]);
-    y[i] = f(a[oa], b[ob], tab);
-  }
-}
-
 template <class F, int NDIM>
 static void launch_bcast_vec(F f, const BcastArgs& p, bool avec, bool bvec, const float* a,
                              const float* b, float* y, uint32_t n4, hipStream_t st) {
@@ -392,10 +363,12 @@ static int launch_bcast(F f, const BroadcastPlan& plan, const float* a, const fl
       case 3: launch_bcast_vec<F, 3>(f, p, avec, bvec, a, b, y, n4, st); break;
       default: launch_bcast_vec<F, 4>(f, p, avec, bvec, a, b, y, n4, st); break;
     }
-  } else if (nd <= 4) {
+  } else {
+    // any innermost extent, any pointers, up to kMaxDims collapsed dims (more than four: operands
+    // that alternate between broadcast and full extents dim by dim)
     BcastArgs p;
     p.a_full = p.b_full = 1;
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < kMaxDims; ++k) {
       p.fd[k] = make_fastdiv(k < nd ? static_cast<uint32_t>(pl.dims[k]) : 1u);
       p.sa[k] = k < nd ? pl.sa[k] : 0;
       p.sb[k] = k < nd ? pl.sb[k] : 0;
@@ -409,17 +382,12 @@ static int launch_bcast(F f, const BroadcastPlan& plan, const float* a, const fl
       case 1: bcast_flat_kernel<F, 1><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
       case 2: bcast_flat_kernel<F, 2><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
       case 3: bcast_flat_kernel<F, 3><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
-      default: bcast_flat_kernel<F, 4><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
+      case 4: bcast_flat_kernel<F, 4><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
+      case 5: bcast_flat_kernel<F, 5><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
+      case 6: bcast_flat_kernel<F, 6><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
+      case 7: bcast_flat_kernel<F, 7><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
+      default: bcast_flat_kernel<F, 8><<<grid, lanes, 0, st>>>(f, p, a, b, y, n4, n); break;
     }
-  } else {
-    BcastGenericArgs p;
-    p.ndim = nd;
-    for (int k = 0; k < kMaxDims; ++k) {
-      p.fd[k] = make_fastdiv(k < nd ? static_cast<uint32_t>(pl.dims[k]) : 1u);
-      p.sa[k] = k < nd ? pl.sa[k] : 0;
-      p.sb[k] = k < nd ? pl.sb[k] : 0;
-    }
-    bcast_generic_kernel<F><<<grid_for(n), kBlock, 0, st>>>(f, p, a, b, y, n);
   }
   return launch_status();
 }

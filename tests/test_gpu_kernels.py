@@ -225,7 +225,7 @@ BCAST_CASES = [
     ([1001, 3], [1, 3]),
     ([2, 3], [2, 3]),
     ([17, 1, 3], [1, 11, 1]),
-    ([3, 1, 2, 1, 7], [1, 4, 1, 6, 1]),   # five dims after collapsing: one output per lane
+    ([3, 1, 2, 1, 7], [1, 4, 1, 6, 1]),   # five dims after collapsing
     # a parameter per channel over rows of 2, 3, 5 and 6 elements: vectors that end in the next channel
     ([9, 64, 2], [1, 64, 1]), ([4, 5, 3], [1, 5, 1]), ([7, 3, 5], [1, 3, 1]), ([2, 11, 2, 3], [1, 11, 1, 1]),
 ]

@@ -72,12 +72,12 @@ def test_column_ops_random_shapes(gpu, seed):
                          oracle.ssd_normalize(x, outer, dim, inner, False, True, 1e-10), "ssd normalize " + what)
 
 
-@pytest.mark.parametrize("seed", [8, 9])
+@pytest.mark.parametrize("seed", [8, 9, 20, 21])
 def test_broadcast_random_shapes(gpu, seed):
     rng = np.random.default_rng(seed)
     for _ in range(60):
-        nd = int(rng.integers(1, 5))
-        out = [int(rng.integers(1, 20)) for _ in range(nd)]
+        nd = int(rng.integers(1, 5)) if rng.random() < 0.6 else int(rng.integers(5, 9))  # up to 8 axes
+        out = [int(rng.integers(1, 20 if nd < 5 else 7)) for _ in range(nd)]
         a = [d if rng.random() < 0.7 else 1 for d in out]
         b = [d if rng.random() < 0.5 else 1 for d in out]
         out = [max(p, q) for p, q in zip(a, b)]
