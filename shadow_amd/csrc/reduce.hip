@@ -621,7 +621,8 @@ __global__ __launch_bounds__(THREADS) void reduce_stage2_block_kernel(const Part
 template <int OP>
 static int run_stage2(const Partial* part, float* y, uint32_t outputs, uint32_t splits,
                       size_t stride_o, size_t stride_s, uint32_t window, hipStream_t st) {
-  if (splits <= 64) {
+  // a lane per output where the outputs fill the chip or the slices are a handful; else a workgroup per output
+  if (splits <= 8 || (splits <= 64 && outputs >= 4096)) {
     reduce_stage2_lane_kernel<OP><<<grid_for(outputs), kBlock, 0, st>>>(part, y, outputs, splits,
                                                                         stride_o, stride_s, window);
   } else if (splits <= 256) {
