@@ -40,6 +40,33 @@ def test_reduce_random_shapes(gpu, seed):
             assert_rel_close(got, want, 1e-5, "reduce %d over axis 1 of %s" % (op, shape))
 
 
+# Any ascending axis set of a 2- to 5-d tensor: single-stage views, a reduced dim in front of them
+# (either order of the two stages), sliced windows, and what is left to the wave-per-output kernel.
+@pytest.mark.parametrize("seed", [22, 23, 24, 25])
+def test_reduce_random_axis_sets(gpu, seed):
+    rng = np.random.default_rng(seed)
+    for _ in range(50):
+        nd = int(rng.integers(2, 6))
+        shape = [int(rng.choice([1, 2, 3, 5, 7, 8, 16, 33, 40, 64, 100])) for _ in range(nd)]
+        if rng.random() < 0.4:  # one long dim: leading-dim-first plans, sliced rows
+            shape[int(rng.integers(0, nd))] = int(rng.choice([300, 1000, 5000]))
+        while np.prod(shape) > 3_000_000:
+            shape[int(np.argmax(shape))] //= 2
+        axes = [a for a in range(nd) if rng.random() < 0.5] or [int(rng.integers(0, nd))]
+        op = int(rng.integers(0, 7))
+        x = rng.normal(0, 1, shape).astype(F) if op else rng.uniform(0.97, 1.03, shape).astype(F)
+        if rng.random() < 0.4:
+            x[rng.random(shape) < 0.4] = 0.0
+            x[rng.random(shape) < 0.3] = -0.0
+        want, _ = oracle.reduce(op, x, shape, axes)
+        got, _ = gpuops.reduce(op, x, shape, axes)
+        what = "reduce %d of %s over %s" % (op, shape, axes)
+        if op in (2, 3):
+            assert_bit_exact(got, want, what)
+        else:
+            assert_rel_close(got, want, 1e-5, what)
+
+
 @pytest.mark.parametrize("seed", [4, 5])
 def test_norm_rows_random_shapes(gpu, seed):
     rng = np.random.default_rng(seed)
