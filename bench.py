@@ -849,9 +849,10 @@ def config_table(dev, sets_scale=1, cpu=None):
         a4, b4 = dev.buf(ha), dev.buf(hb4)
         y4 = [dev.buf(nbytes=4 * no) for _ in range(SETS)]
         hy4 = np.empty(no, np.float32) if cpu else None
+        isa4, isb4, iso4 = I(sa4), I(sb4), I(so4)  # built once: on 1 MB tensors the caller's own time per launch shows
         for name, op in [("mul", 2), ("sub", 1), ("div", 3), ("max", 5)]:
             ms = time_median(dev, lambda k: lib.shdw_hip_broadcast_binary(
-                op, len(so4), I(sa4), I(sb4), I(so4), a4.ptr, b4.ptr, y4[k].ptr, st), SETS)
+                op, len(so4), isa4, isb4, iso4, a4.ptr, b4.ptr, y4[k].ptr, st), SETS)
             add(4, "broadcast_%s_%s" % (name, tag), 4 * (na + nb_), 4 * no, ms, no,
                 cpu and cpu.broadcast(op, ha, sa4, hb4, sb4, so4, hy4))
         if tag == "iii":  # the same pair through the scalar-argument form
