@@ -398,9 +398,17 @@ struct SmallPlanesArgs {
   int pitch, plane_lds;  // padded row and plane in LDS, in floats
   int rows_lds;          // padded rows of a plane
   uint32_t planes, total_planes;
-  FastDiv f_plane_in, f_in_w, f_plane_out, f_out_w, f_row_maxima;  // the last: rows_lds * out_w
+  FastDiv f_plane_in, f_in_w, f_plane_out, f_out_w, f_row_maxima;  // the last: rows_lds * out_w; for the
+                                                                   // wide average: output quads per plane
+  FastDiv f_quads_w;  // wide average: output quads per row
 };
 
+// SEP with MAX false is the wide average at a column stride of one: a lane takes four
+// neighbouring outputs of a row and reads every cell of their 4 + kw - 1 columns once per
+// window row, adding it to the sums it belongs to - each sum still receives its cells row by
+// row and left to right - in place of 4 kw reads (13x13 on 14x14 maps: 256 us per 51 MB, all
+// of it LDS reads).  The tile has four spare floats behind it for the reads of a row's last,
+// partly empty quad.
 template <bool MAX, int K, bool SEP = false>
 __global__ __launch_bounds__(kBlock) void pool_small_planes_kernel(const float* x, float* y, SmallPlanesArgs a) {
   extern __shared__ __align__(16) float tile[];  // planes * plane_lds floats, a multiple of 4
@@ -442,6 +450,48 @@ __global__ __launch_bounds__(kBlock) void pool_small_planes_kernel(const float* 
   __syncthreads();
   float* ys = y + static_cast<uint64_t>(first) * plane_out;
   const uint32_t outputs = np * plane_out;
+  if (SEP && !MAX) {
+    const uint32_t quads_w = (static_cast<uint32_t>(a.out_w) + 3) / 4, per_plane = a.out_h * quads_w;
+    const FastDiv f_quads = a.f_row_maxima, f_quads_w = a.f_quads_w;  // per plane, per row
+    for (uint32_t t = threadIdx.x; t < np * per_plane; t += kBlock) {
+      uint32_t pl, rem, oh, q;
+      fd_divmod(t, f_quads, pl, rem);
+      fd_divmod(rem, f_quads_w, oh, q);
+      const uint32_t ow = 4 * q;
+      const float* win = tile + pl * a.plane_lds + (oh * a.sh) * a.pitch + ow;  // sw == 1
+      float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+      const int kw = a.kw;
+      for (int i = 0; i < a.kh; ++i) {
+        const float* row = win + i * a.pitch;
+        // cells 0 .. kw+2 of the row piece; cell j belongs to the windows j-3 .. j of the four
+        float v0 = row[0], v1 = row[1], v2 = row[2];
+        s0 += v0;
+        s0 += v1, s1 += v1;
+        s0 += v2, s1 += v2, s2 += v2;
+        for (int j = 3; j < kw; ++j) {
+          const float v = row[j];
+          s0 += v, s1 += v, s2 += v, s3 += v;
+        }
+        v0 = row[kw], v1 = row[kw + 1], v2 = row[kw + 2];
+        s1 += v0, s2 += v0, s3 += v0;
+        s2 += v1, s3 += v1;
+        s3 += v2;
+      }
+      const float sums[4] = {s0, s1, s2, s3};
+      const int h_first = static_cast<int>(oh) * a.sh - a.ph;
+      const int rows_in = min(h_first + a.kh, a.in_h + a.ph) - h_first;
+      float* dst = ys + pl * plane_out + oh * a.out_w + ow;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (ow + k < static_cast<uint32_t>(a.out_w)) {
+          const int w_first = static_cast<int>(ow + k) - a.pw;
+          const int pool_size = rows_in * (min(w_first + kw, a.in_w + a.pw) - w_first);
+          dst[k] = sums[k] / static_cast<float>(pool_size);
+        }
+      }
+    }
+    return;
+  }
   if (SEP) {
     float* row_maxima = tile + a.planes * static_cast<uint32_t>(a.plane_lds);  // [plane][padded row][out_w]
     const uint32_t per_plane = a.f_row_maxima.d, pieces = np * per_plane;
@@ -516,7 +566,11 @@ static bool plan_small_planes(const PoolArgs& p, int64_t total_planes, bool max_
   // 26x26 maps: 64 us per 51 MB; the band kernel, which walks every cell of every window,
   // takes 369 us for the average over the same windows)
   const bool wide_max = max_pool && p.kh * p.kw >= kSeparableMinCells;
-  if (plane_out > (wide_max ? 2 : 1) * kSmallPlanesMaxOutputs || plane_out < 1 || total_planes > INT32_MAX) return false;
+  // ... and so is the average that reads every cell once for four neighbouring outputs (13x13 on
+  // 26x26 maps: 369 us through the band kernel)
+  const bool wide_avg = !max_pool && p.kh * p.kw >= kSeparableMinCells && p.sw == 1 && p.kw >= 4;
+  if (plane_out > (wide_max || wide_avg ? 2 : 1) * kSmallPlanesMaxOutputs || plane_out < 1 || total_planes > INT32_MAX)
+    return false;
   const int over_b = std::max(0, (p.out_h - 1) * p.sh - p.ph + p.kh - p.in_h);
   const int over_r = std::max(0, (p.out_w - 1) * p.sw - p.pw + p.kw - p.in_w);
   const int64_t pitch = static_cast<int64_t>(p.pw) + p.in_w + over_r;
@@ -524,8 +578,8 @@ static bool plan_small_planes(const PoolArgs& p, int64_t total_planes, bool max_
   plane_lds = (plane_lds + 3) & ~int64_t{3};
   if (plane_lds * 2 > kSmallPlanesTileFloats) return false;
   const int64_t rows_lds = static_cast<int64_t>(p.ph) + p.in_h + over_b;
-  const int64_t row_maxima = rows_lds * p.out_w;
-  *separable = wide_max && (plane_lds + row_maxima) * 2 <= kSmallPlanesTileFloats;
+  const int64_t row_maxima = wide_avg ? 0 : rows_lds * p.out_w;
+  *separable = wide_avg || (wide_max && (plane_lds + row_maxima) * 2 <= kSmallPlanesTileFloats);
   if (plane_out > kSmallPlanesMaxOutputs && !*separable) return false;
   int64_t planes = kSmallPlanesTileFloats / (plane_lds + (*separable ? row_maxima : 0));
   const int64_t want = (4 * kBlock + plane_out - 1) / plane_out;  // about four outputs per lane
@@ -535,7 +589,9 @@ static bool plan_small_planes(const PoolArgs& p, int64_t total_planes, bool max_
   a->kh = p.kh, a->kw = p.kw, a->sh = p.sh, a->sw = p.sw, a->ph = p.ph, a->pw = p.pw;
   a->pitch = static_cast<int>(pitch), a->plane_lds = static_cast<int>(plane_lds);
   a->rows_lds = static_cast<int>(rows_lds);
-  a->f_row_maxima = make_fastdiv(static_cast<uint32_t>(row_maxima));
+  const uint32_t quads_w = (static_cast<uint32_t>(p.out_w) + 3) / 4;
+  a->f_row_maxima = make_fastdiv(wide_avg ? p.out_h * quads_w : static_cast<uint32_t>(row_maxima));
+  a->f_quads_w = make_fastdiv(quads_w);
   a->planes = static_cast<uint32_t>(planes), a->total_planes = static_cast<uint32_t>(total_planes);
   a->f_plane_in = make_fastdiv(static_cast<uint32_t>(plane_in));
   a->f_in_w = make_fastdiv(static_cast<uint32_t>(p.in_w));
@@ -866,9 +922,14 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
   if (!three_d && plan_small_planes(p, static_cast<int64_t>(in_shape[0]) * in_shape[1], pool_type == 0, &sp, &separable)) {
     const uint32_t grid = (sp.total_planes + sp.planes - 1) / sp.planes;
     const int k = p.kh == p.kw && (p.kh == 2 || p.kh == 3) ? p.kh : 0;
-    if (separable) {
+    if (separable && pool_type == 0) {
       const size_t both = static_cast<size_t>(sp.planes) * (sp.plane_lds + sp.f_row_maxima.d) * sizeof(float);
       pool_small_planes_kernel<true, 0, true><<<grid, kBlock, both, st>>>(x, y, sp);
+      return launch_status();
+    }
+    if (separable) {  // the wide average: four spare floats behind the planes
+      const size_t spare = (static_cast<size_t>(sp.planes) * sp.plane_lds + 4) * sizeof(float);
+      pool_small_planes_kernel<false, 0, true><<<grid, kBlock, spare, st>>>(x, y, sp);
       return launch_status();
     }
     const size_t lds = static_cast<size_t>(sp.planes) * sp.plane_lds * sizeof(float);
