@@ -441,8 +441,21 @@ __global__ __launch_bounds__(kBlock) void pool_small_planes_kernel(const float* 
     for (int k = 0; k < 4; ++k) {
       const uint32_t v = v0 + k * kBlock + threadIdx.x;
       if (v < nvec) {
+        // one division per vector: the following elements step along the row and wrap into the
+        // next row (past the right padding) or the next plane (past the bottom padding)
+        uint32_t pl, rem, r, c;
+        fd_divmod(4 * v, a.f_plane_in, pl, rem);
+        fd_divmod(rem, a.f_in_w, r, c);
+        uint32_t at = pl * a.plane_lds + (r + a.ph) * a.pitch + a.pw + c;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) tile[slot(4 * v + j)] = reg[k][j];
+        for (int j = 0; j < 4; ++j) {
+          tile[at] = reg[k][j];
+          ++at;
+          if (++c == static_cast<uint32_t>(a.in_w)) {
+            c = 0, at += a.pitch - a.in_w;
+            if (++r == static_cast<uint32_t>(a.in_h)) r = 0, at += a.plane_lds - a.in_h * a.pitch;
+          }
+        }
       }
     }
   }
