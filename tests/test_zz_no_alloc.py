@@ -41,6 +41,8 @@ PAIRS = [
     (([2, 6000, 512], [1]), ([1, 3000, 256], [1])),         # column tiles, sliced
     (([1, 65536, 128], [1]), ([1, 20000, 132], [1])),       # more partials than one workgroup folds: second launch
     (([2, 5000, 201], [1]), ([1, 3000, 129], [1])),         # one column per lane, sliced
+    (([64, 96, 28, 28], [0, 2, 3]), ([6, 5, 7, 7], [0, 2, 3])),   # a reduced dim in front: partials per leading index
+    (([300, 64, 7, 9], [0, 2]), ([40, 6, 7, 5], [0, 2])),         # the leading dim first, nested second stage
 ]
 
 
