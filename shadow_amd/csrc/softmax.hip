@@ -1224,6 +1224,234 @@ __global__ __launch_bounds__(kBlock) void normalize_tall_kernel(const float* x, 
   }
 }
 
+// ---------------------------------------------------------------------------
+// Long slabs: columns of thousands of rows over fewer than 16 positions
+// ([448][4096][7]).  The slab of an outer index is contiguous but too large to
+// stay in LDS with more than one workgroup per CU (112 KB here), so it moves
+// through LDS in chunks of whole rows, at most 4096 floats, as the tall kernels'
+// tiles do.  A chunk is a multiple of inner floats long, so the k-th element of
+// every chunk has the same position, and a lane, which always takes the same
+// elements of a chunk, keeps the statistics of its sixteen positions in
+// registers.
+// ---------------------------------------------------------------------------
+constexpr int kLongLoads = kTallChunkFloats / 4 / kBlock;  // 128-bit loads per lane and chunk
+static_assert(kLongLoads == 4, "a chunk is four vectors per lane");
+
+struct LongSlab {
+  uint32_t dim, inner, chunk_rows, chunk_cells;
+  const float* xs;
+  float* ys;
+  SHDW_DEVICE LongSlab(const float* x, float* y, uint32_t dim_, uint32_t inner_) {
+    dim = dim_, inner = inner_;
+    chunk_rows = kTallChunkFloats / inner, chunk_cells = chunk_rows * inner;
+    const uint64_t slab = static_cast<uint64_t>(blockIdx.x) * dim * inner;
+    xs = x + slab, ys = y + slab;
+  }
+  SHDW_DEVICE uint32_t chunks() const { return (dim + chunk_rows - 1) / chunk_rows; }
+  SHDW_DEVICE uint32_t rows_in(uint32_t k) const {
+    const uint32_t r0 = k * chunk_rows;
+    return r0 < dim ? min(chunk_rows, dim - r0) : 0u;  // chunks past the end hold nothing
+  }
+  SHDW_DEVICE uint32_t cells_in(uint32_t k) const { return rows_in(k) * inner; }
+  SHDW_DEVICE static uint32_t first(int i) { return 4 * (threadIdx.x + kBlock * i); }  // of vector i, in the chunk
+  SHDW_DEVICE void load(uint32_t k, v4f (&v)[kLongLoads]) const {
+    const uint32_t cells = cells_in(k);
+    const float* src = xs + static_cast<uint64_t>(k) * chunk_cells;
+#pragma unroll
+    for (int i = 0; i < kLongLoads; ++i) {
+      const uint32_t e = first(i);
+      if (e + 4 <= cells) {
+        v[i] = load4_stream_any(src + e);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+          if (e + j < cells) v[i][j] = __builtin_nontemporal_load(src + e + j);
+      }
+    }
+  }
+  // q(value, vector i, element j, row in the slab) for the lane's elements of chunk k, then stored
+  template <class Q>
+  SHDW_DEVICE void store(uint32_t k, const v4f (&v)[kLongLoads], Q q) const {
+    const uint32_t cells = cells_in(k);
+    float* dst = ys + static_cast<uint64_t>(k) * chunk_cells;
+#pragma unroll
+    for (int i = 0; i < kLongLoads; ++i) {
+      const uint32_t e = first(i);
+      if (e >= cells) continue;
+      v4f r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = q(v[i][j], i, j);
+      if (e + 4 <= cells) {
+        store4_stream_any(dst + e, r);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+          if (e + j < cells) dst[e + j] = r[j];
+      }
+    }
+  }
+};
+
+__global__ __launch_bounds__(kBlock) void softmax_long_slab_kernel(const float* x, float* y, uint32_t dim,
+                                                                    FastDiv f_inner) {
+  __shared__ __align__(16) float chunk[2][kTallChunkFloats];
+  __shared__ float stat[kTallMinInner];
+  __shared__ uint64_t tab[32];
+  if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
+  const LongSlab t(x, y, dim, f_inner.d);
+  const uint32_t chunks = t.chunks(), inner = t.inner;
+  uint32_t pos[kLongLoads][4];
+#pragma unroll
+  for (int i = 0; i < kLongLoads; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t e = LongSlab::first(i) + j;
+      pos[i][j] = e - fd_div(e, f_inner) * inner;
+    }
+  v4f v[kLongLoads], v2[kLongLoads];
+
+  // maxima in any order (see softmax_slab_kernel): per element slot of the chunk, then per position
+  float part[kLongLoads][4];
+#pragma unroll
+  for (int i = 0; i < kLongLoads; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) part[i][j] = -FLT_MAX;
+  auto fold_max = [&](uint32_t k, const v4f(&reg)[kLongLoads]) {
+    const uint32_t cells = t.cells_in(k);
+#pragma unroll
+    for (int i = 0; i < kLongLoads; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (LongSlab::first(i) + j < cells) part[i][j] = std_max(reg[i][j], part[i][j]);
+  };
+  for (uint32_t k = 0; k < chunks; k += 2) {
+    t.load(k, v);
+    t.load(k + 1, v2);
+    fold_max(k, v);
+    fold_max(k + 1, v2);
+  }
+#pragma unroll
+  for (int i = 0; i < kLongLoads; ++i)
+    *reinterpret_cast<v4f*>(chunk[0] + LongSlab::first(i)) = v4f{part[i][0], part[i][1], part[i][2], part[i][3]};
+  __syncthreads();
+  if (threadIdx.x < inner) {
+    float m = -FLT_MAX;
+    walk_column(chunk[0] + threadIdx.x, inner, t.chunk_rows, [&](float a) { m = std_max(a, m); });
+    stat[threadIdx.x] = m;
+  }
+  __syncthreads();
+  float max_val[kLongLoads][4];
+#pragma unroll
+  for (int i = 0; i < kLongLoads; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) max_val[i][j] = stat[pos[i][j]];
+
+  // exponentials of a chunk into LDS by all lanes, ordered sums by one lane per position
+  float sum = 0.f;
+  auto pass = [&](uint32_t k, v4f(&reg)[kLongLoads]) {
+    float* buf = chunk[k & 1];
+#pragma unroll
+    for (int i = 0; i < kLongLoads; ++i) {
+      v4f ex;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ex[j] = libm::exact_expf(reg[i][j] - max_val[i][j], tab);
+      *reinterpret_cast<v4f*>(buf + LongSlab::first(i)) = ex;  // slots past the chunk's cells are never walked
+    }
+    __syncthreads();
+    t.load(k + 2, reg);
+    if (threadIdx.x < inner) walk_column(buf + threadIdx.x, inner, t.rows_in(k), [&](float a) { sum += a; });
+  };
+  t.load(0, v);
+  t.load(1, v2);
+  for (uint32_t k = 0; k < chunks; k += 2) {
+    pass(k, v);
+    if (k + 1 < chunks) pass(k + 1, v2);
+  }
+  __syncthreads();
+  if (threadIdx.x < inner) stat[threadIdx.x] = sum;
+  __syncthreads();
+  float total[kLongLoads][4];
+#pragma unroll
+  for (int i = 0; i < kLongLoads; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) total[i][j] = stat[pos[i][j]];
+
+  for (uint32_t k = 0; k < chunks; k += 2) {
+    t.load(k, v);
+    t.load(k + 1, v2);
+    auto quotient = [&](float a, int i, int j) { return libm::exact_expf(a - max_val[i][j], tab) / total[i][j]; };
+    t.store(k, v, quotient);
+    t.store(k + 1, v2, quotient);
+  }
+}
+
+template <int PMODE, int SM>
+__global__ __launch_bounds__(kBlock) void normalize_long_slab_kernel(const float* x, float* y, uint32_t dim,
+                                                                      FastDiv f_inner, float p, float eps,
+                                                                      const float* scale) {
+  __shared__ __align__(16) float chunk[2][kTallChunkFloats];
+  __shared__ float stat[kTallMinInner];
+  const LongSlab t(x, y, dim, f_inner.d);
+  const uint32_t chunks = t.chunks(), inner = t.inner;
+  uint32_t pos[kLongLoads][4], row[kLongLoads][4];  // position and row inside a chunk of the lane's elements
+#pragma unroll
+  for (int i = 0; i < kLongLoads; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t e = LongSlab::first(i) + j;
+      row[i][j] = fd_div(e, f_inner);
+      pos[i][j] = e - row[i][j] * inner;
+    }
+  v4f v[kLongLoads], v2[kLongLoads];
+
+  double acc = 0;
+  auto pass = [&](uint32_t k, v4f(&reg)[kLongLoads]) {  // as in softmax_long_slab_kernel
+    float* buf = chunk[k & 1];
+#pragma unroll
+    for (int i = 0; i < kLongLoads; ++i) {
+      v4f term;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) term[j] = static_cast<float>(norm_term<PMODE>(reg[i][j], p));
+      *reinterpret_cast<v4f*>(buf + LongSlab::first(i)) = term;
+    }
+    __syncthreads();
+    t.load(k + 2, reg);
+    if (threadIdx.x < inner)
+      walk_column(buf + threadIdx.x, inner, t.rows_in(k), [&](float a) { acc += static_cast<double>(a); });
+  };
+  t.load(0, v);
+  t.load(1, v2);
+  for (uint32_t k = 0; k < chunks; k += 2) {
+    pass(k, v);
+    if (k + 1 < chunks) pass(k + 1, v2);
+  }
+  __syncthreads();
+  if (threadIdx.x < inner) stat[threadIdx.x] = norm_finish<PMODE>(acc, p, eps);
+  __syncthreads();
+  float div[kLongLoads][4];
+#pragma unroll
+  for (int i = 0; i < kLongLoads; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) div[i][j] = stat[pos[i][j]];
+
+  for (uint32_t k = 0; k < chunks; k += 2) {
+    t.load(k, v);
+    t.load(k + 1, v2);
+    t.store(k, v, [&](float a, int i, int j) { return ssd_scaled<SM>(a / div[i][j], scale, k * t.chunk_rows + row[i][j]); });
+    t.store(k + 1, v2,
+            [&](float a, int i, int j) { return ssd_scaled<SM>(a / div[i][j], scale, (k + 1) * t.chunk_rows + row[i][j]); });
+  }
+}
+
+// Slabs from this size on take the long-slab kernels where inner < 16 (smaller ones
+// stay whole in LDS: softmax_slab_kernel, normalize_slab_kernel).
+constexpr int64_t kLongSlabMinFloats = 15 * 1024;
+
+static bool long_slab(int dim, int inner_num) {
+  return static_cast<uint32_t>(inner_num) < kTallMinInner &&
+         static_cast<int64_t>(dim) * inner_num > kLongSlabMinFloats;
+}
+
 // Where the tall kernels apply, and their launch: positions per workgroup as wide
 // as still leaves a thousand workgroups, 128-bit accesses where every row piece
 // starts on a 16-byte boundary.
@@ -1310,7 +1538,9 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
     const uint32_t slabs = static_cast<uint32_t>(outer_num);
     softmax_packed_kernel<<<(slabs + group - 1) / group, kBlock, packed_bytes(dim, inner_num, group), st>>>(
         x, y, slabs, static_cast<uint32_t>(dim), fi, make_fastdiv(static_cast<uint32_t>(dim) * inner_num), group);
-  } else if (g.use_slab)
+  } else if (long_slab(dim, inner_num))
+    softmax_long_slab_kernel<<<outer_num, kBlock, 0, st>>>(x, y, static_cast<uint32_t>(dim), fi);
+  else if (g.use_slab)
     softmax_slab_kernel<<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, static_cast<uint32_t>(dim), fi);
   else if (dim <= 64) {
     // the tile kernel is slower here: [64,49,128,128] 115 us against 88
@@ -1362,6 +1592,13 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
       normalize_packed_kernel<2, kSsdNoScale><<<grid, kBlock, bytes, st>>>(x, y, slabs, d, fi, fs, group, p, eps, nullptr);
     else
       normalize_packed_kernel<0, kSsdNoScale><<<grid, kBlock, bytes, st>>>(x, y, slabs, d, fi, fs, group, p, eps, nullptr);
+  } else if (long_slab(dim, inner_num)) {
+    if (mode == 1)
+      normalize_long_slab_kernel<1, kSsdNoScale><<<outer_num, kBlock, 0, st>>>(x, y, d, fi, p, eps, nullptr);
+    else if (mode == 2)
+      normalize_long_slab_kernel<2, kSsdNoScale><<<outer_num, kBlock, 0, st>>>(x, y, d, fi, p, eps, nullptr);
+    else
+      normalize_long_slab_kernel<0, kSsdNoScale><<<outer_num, kBlock, 0, st>>>(x, y, d, fi, p, eps, nullptr);
   } else if (g.use_slab) {
     if (mode == 1)
       normalize_slab_kernel<1><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
@@ -1424,7 +1661,9 @@ static void launch_ssd_columns(const ColumnGeometry& g, int outer_num, int dim, 
     const uint32_t slabs = static_cast<uint32_t>(outer_num);
     normalize_packed_kernel<3, SM><<<(slabs + group - 1) / group, kBlock, packed_bytes(dim, inner_num, group), st>>>(
         x, y, slabs, d, fi, make_fastdiv(d * inner_num), group, 2.f, eps, scale);
-  } else if (g.use_slab)
+  } else if (long_slab(dim, inner_num))
+    normalize_long_slab_kernel<3, SM><<<outer_num, kBlock, 0, st>>>(x, y, d, fi, 2.f, eps, scale);
+  else if (g.use_slab)
     normalize_slab_kernel<3, SM><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, 2.f, eps, scale);
   else if (tile_fits(dim, inner_num))
     launch_normalize_tile<3, SM>(outer_num, dim, inner_num, 2.f, eps, x, scale, y, st);

@@ -100,6 +100,8 @@ SOFTMAX_SHAPES = [  # outer, dim, inner: both layouts, LDS limits, odd sizes
     # a cut last tile, a last chunk of one row, many workgroups
     (2, 1300, 30), (2, 600, 64), (1, 1000, 100), (3, 513, 17), (1, 2048, 196), (2, 700, 68), (1, 4097, 16),
     (1, 1025, 3136), (40, 520, 128), (1100, 513, 16), (2, 769, 49), (1, 20000, 20),
+    # long slabs over fewer than 16 positions, in chunks of whole rows: ragged last chunks, one to fifteen positions
+    (2, 5000, 3), (1, 16000, 1), (1, 1100, 14), (3, 2731, 6), (2, 8193, 2), (1, 3000, 15), (5, 1537, 10),
 ]
 
 
@@ -111,7 +113,7 @@ def test_softmax(gpu, outer, dim, inner):
     assert_bit_exact(gpuops.softmax(x, outer, dim, inner, inplace=True), want, "softmax in place")
 
 
-@pytest.mark.parametrize("outer,dim,inner", [(40, 50, 1), (2, 12, 200), (2, 80, 100)])
+@pytest.mark.parametrize("outer,dim,inner", [(40, 50, 1), (2, 12, 200), (2, 80, 100), (2, 6000, 3), (1, 700, 64)])
 def test_softmax_special_values(gpu, outer, dim, inner):
     x = with_specials(normal(14, outer * dim * inner, 30.0), 14)
     assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax specials")
@@ -171,7 +173,8 @@ def test_softmax_op_defaults_and_errors(ws):
                                              (2, 256, 64), (1, 1025, 40),
                                              # tall columns in chunks through LDS; slabs of more than 60 KB
                                              (2, 1300, 30), (1, 2048, 196), (2, 1100, 68), (1, 4097, 16),
-                                             (30, 1026, 128), (3, 4096, 7), (1, 39000, 1)])
+                                             (30, 1026, 128), (3, 4096, 7), (1, 39000, 1),
+                                             (2, 5000, 3), (1, 1100, 14), (3, 2731, 6), (2, 8193, 2)])
 def test_normalize(gpu, p, outer, dim, inner):
     x = normal(17, outer * dim * inner, 2.0)
     want = oracle.normalize(x, outer, dim, inner, p, 1e-12)
@@ -201,7 +204,7 @@ def test_normalize_op(ws, args):
 # ----------------------------------------------------------- SSDNormalize ---
 SSD_SHAPES = [(2, 5, 12), (3, 512, 1), (2, 16, 100), (3, 9, 64), (1, 600, 3), (2, 1, 9), (1, 33, 4097),
               (2, 64, 1444), (5, 3, 7), (1, 128, 4096), (3, 20, 1025), (2, 512, 361), (1, 1000, 50), (2, 70, 33),
-              (1, 512, 1444), (2, 1030, 24), (2, 1100, 68), (1, 2049, 31), (3, 4096, 7)]
+              (1, 512, 1444), (2, 1030, 24), (2, 1100, 68), (1, 2049, 31), (3, 4096, 7), (2, 5000, 3), (1, 1100, 14)]
 
 
 @pytest.mark.parametrize("scale_kind", ["none", "shared", "channel"])
