@@ -25,7 +25,9 @@
 
 namespace shdw {
 
-constexpr int kSlabMaxFloats = 39 * 1024;  // slab + per-column statistics: up to 156 of the CU's 160 KB of LDS
+constexpr int kSlabMaxFloats = 15 * 1024;  // slab + per-column statistics, 60 KB of LDS: two workgroups per CU (whole
+                                           // slabs of up to 156 KB, one workgroup per CU, ran at half the speed of the
+                                           // chunked kernels that take the larger ones now)
 
 // std::max(a, b) of libstdc++: b only when a < b.
 SHDW_DEVICE float std_max(float a, float b) { return a < b ? b : a; }
@@ -1445,7 +1447,7 @@ __global__ __launch_bounds__(kBlock) void normalize_long_slab_kernel(const float
 
 // Slabs from this size on take the long-slab kernels where inner < 16 (smaller ones
 // stay whole in LDS: softmax_slab_kernel, normalize_slab_kernel).
-constexpr int64_t kLongSlabMinFloats = 15 * 1024;
+constexpr int64_t kLongSlabMinFloats = kSlabMaxFloats;
 
 static bool long_slab(int dim, int inner_num) {
   return static_cast<uint32_t>(inner_num) < kTallMinInner &&

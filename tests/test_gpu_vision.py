@@ -94,7 +94,7 @@ SOFTMAX_SHAPES = [  # outer, dim, inner: both layouts, LDS limits, odd sizes
     (2, 150, 300), (1, 65, 4097), (3, 100, 64), (1, 1000, 70),
     # around the longest column whose tile fits LDS beside the exp table
     (1, 509, 40), (1, 510, 40), (1, 511, 20), (1, 512, 33),
-    # slabs of 60 to 156 KB: one workgroup per slab with most of a CU's LDS
+    # slabs of more than 60 KB
     (3, 4096, 7), (2, 20000, 1), (2, 1300, 15), (1, 39000, 1), (1, 39936, 1), (1, 40000, 1),
     # tall columns: chunks of rows through LDS, tiles of 16 / 32 / 64 positions, vectors or not,
     # a cut last tile, a last chunk of one row, many workgroups
