@@ -1029,68 +1029,76 @@ constexpr uint32_t kTallChunkFloats = 4096;
 constexpr uint32_t kTallMinInner = 16;
 constexpr int kTallAhead = 4;  // chunks requested at a time by the passes that only stream
 
-template <int VEC>
-struct TallVec { using type = float; };
-template <>
-struct TallVec<4> { using type = v4f; };
-
-SHDW_DEVICE float& tall_elem(float& v, int) { return v; }
-SHDW_DEVICE float tall_elem(const v4f& v, int e) { return v[e]; }
-SHDW_DEVICE void tall_set(float& v, int, float a) { v = a; }
-SHDW_DEVICE void tall_set(v4f& v, int e, float a) { v[e] = a; }
-
-template <int VEC>
+// A lane takes four neighbouring positions of a row with one 128-bit access on
+// whatever dword address they have (rows of 49 or 1001 positions start anywhere);
+// where the row ends inside the four, the ones that exist move one by one.
 struct TallTile {
-  using V = typename TallVec<VEC>::type;
-  static constexpr int kLoads = 16 / VEC;  // per lane and chunk
+  static constexpr int kLoads = 4;  // vectors per lane and chunk
   uint32_t dim, inner, width, rows_per_sweep, chunk_rows, row0, col;
-  bool live;      // the lane's positions exist (the last tile of a row may be cut)
-  uint64_t base;  // of (outer index, row 0, the lane's first position)
+  uint32_t valid;  // how many of the lane's four positions exist (the last tile of a row may be cut)
+  uint64_t base;   // of (outer index, row 0, the lane's first position)
 
   SHDW_DEVICE TallTile(uint32_t dim_, uint32_t inner_, uint32_t width_log2, FastDiv f_tiles) {
     dim = dim_, inner = inner_, width = 1u << width_log2;
-    const uint32_t lanes_log2 = width_log2 - (VEC == 4 ? 2 : 0);  // lanes per row of the tile
+    const uint32_t lanes_log2 = width_log2 - 2;  // lanes per row of the tile
     rows_per_sweep = kBlock >> lanes_log2;
     chunk_rows = rows_per_sweep * kLoads;
     row0 = threadIdx.x >> lanes_log2;
-    col = (threadIdx.x & ((1u << lanes_log2) - 1)) * VEC;
+    col = (threadIdx.x & ((1u << lanes_log2) - 1)) * 4;
     uint32_t n, tile;
     fd_divmod(xcd_contiguous(blockIdx.x, gridDim.x), f_tiles, n, tile);  // neighbours share cache lines
     const uint32_t p = tile * width + col;
-    live = p < inner;  // VEC == 4 only where inner is a multiple of four: whole vectors exist or not
+    valid = p < inner ? min(4u, inner - p) : 0u;
     base = static_cast<uint64_t>(n) * dim * inner + p;
   }
   SHDW_DEVICE uint32_t chunks() const { return (dim + chunk_rows - 1) / chunk_rows; }
   SHDW_DEVICE uint32_t rows_in(uint32_t k) const { return min(chunk_rows, dim - k * chunk_rows); }
   SHDW_DEVICE uint32_t row(uint32_t k, int i) const { return k * chunk_rows + i * rows_per_sweep + row0; }
-  SHDW_DEVICE bool has(uint32_t k, int i) const { return live && row(k, i) < dim; }
+  SHDW_DEVICE bool has(uint32_t k, int i) const { return valid > 0 && row(k, i) < dim; }
   SHDW_DEVICE uint32_t slot(int i) const { return (i * rows_per_sweep + row0) * width + col; }
-  SHDW_DEVICE void load(const float* x, uint32_t k, V (&v)[kLoads]) const {
+  SHDW_DEVICE void load(const float* x, uint32_t k, v4f (&v)[kLoads]) const {
 #pragma unroll
     for (int i = 0; i < kLoads; ++i)
-      if (has(k, i)) v[i] = *reinterpret_cast<const V*>(x + base + static_cast<uint64_t>(row(k, i)) * inner);
+      if (has(k, i)) {
+        const float* src = x + base + static_cast<uint64_t>(row(k, i)) * inner;
+        if (valid == 4) {
+          v[i] = load4_stream_any(src);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 3; ++e)
+            if (static_cast<uint32_t>(e) < valid) v[i][e] = __builtin_nontemporal_load(src + e);
+        }
+      }
+  }
+  SHDW_DEVICE void store(float* y, uint32_t r, const v4f& q) const {
+    float* dst = y + base + static_cast<uint64_t>(r) * inner;
+    if (valid == 4) {
+      store4_stream_any(dst, q);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 3; ++e)
+        if (static_cast<uint32_t>(e) < valid) dst[e] = q[e];
+    }
   }
 };
 
-template <int VEC>
 __global__ __launch_bounds__(kBlock) void softmax_tall_kernel(const float* x, float* y, uint32_t dim,
                                                                uint32_t inner, uint32_t width_log2,
                                                                FastDiv f_tiles) {
-  using T = TallTile<VEC>;
-  using V = typename T::V;
+  using T = TallTile;
   __shared__ __align__(16) float chunk[2][kTallChunkFloats];
-  __shared__ float stat[64];
+  __shared__ __align__(16) float stat[64];
   __shared__ uint64_t tab[32];
   if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
   const T t(dim, inner, width_log2, f_tiles);
   const uint32_t chunks = t.chunks();
-  V v[T::kLoads];
+  v4f v[T::kLoads];
 
-  float part[VEC];
+  float part[4];
 #pragma unroll
-  for (int e = 0; e < VEC; ++e) part[e] = -FLT_MAX;
+  for (int e = 0; e < 4; ++e) part[e] = -FLT_MAX;
   for (uint32_t k = 0; k < chunks; k += kTallAhead) {  // chunks past the end hold no rows
-    V w[kTallAhead][T::kLoads];
+    v4f w[kTallAhead][T::kLoads];
 #pragma unroll
     for (int j = 0; j < kTallAhead; ++j) t.load(x, k + j, w[j]);
 #pragma unroll
@@ -1099,10 +1107,10 @@ __global__ __launch_bounds__(kBlock) void softmax_tall_kernel(const float* x, fl
       for (int i = 0; i < T::kLoads; ++i)
         if (t.has(k + j, i))
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) part[e] = std_max(tall_elem(w[j][i], e), part[e]);
+          for (int e = 0; e < 4; ++e)
+            if (static_cast<uint32_t>(e) < t.valid) part[e] = std_max(w[j][i][e], part[e]);
   }
-#pragma unroll
-  for (int e = 0; e < VEC; ++e) chunk[0][t.row0 * t.width + t.col + e] = part[e];
+  *reinterpret_cast<v4f*>(chunk[0] + t.row0 * t.width + t.col) = v4f{part[0], part[1], part[2], part[3]};
   __syncthreads();
   if (threadIdx.x < t.width) {
     float m = -FLT_MAX;
@@ -1110,29 +1118,28 @@ __global__ __launch_bounds__(kBlock) void softmax_tall_kernel(const float* x, fl
     stat[threadIdx.x] = m;
   }
   __syncthreads();
-  float max_val[VEC];
-#pragma unroll
-  for (int e = 0; e < VEC; ++e) max_val[e] = stat[t.col + e];
+  const v4f max_val = *reinterpret_cast<const v4f*>(stat + t.col);
 
   float sum = 0.f;
   // chunk k: its exponentials into LDS by all lanes, then the walk by one lane per
   // column while the loads of chunk k + 2 fly.  Two buffers: the slowest walker is
-  // at most one chunk behind.
-  auto pass = [&](uint32_t k, V(&reg)[T::kLoads]) {
+  // at most one chunk behind.  Positions past the end of a row hold whatever the
+  // lanes had; their sums are never used.
+  auto pass = [&](uint32_t k, v4f(&reg)[T::kLoads]) {
     float* buf = chunk[k & 1];
 #pragma unroll
     for (int i = 0; i < T::kLoads; ++i)
       if (t.has(k, i)) {
-        V ex;
+        v4f ex;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) tall_set(ex, e, libm::exact_expf(tall_elem(reg[i], e) - max_val[e], tab));
-        *reinterpret_cast<V*>(buf + t.slot(i)) = ex;
+        for (int e = 0; e < 4; ++e) ex[e] = libm::exact_expf(reg[i][e] - max_val[e], tab);
+        *reinterpret_cast<v4f*>(buf + t.slot(i)) = ex;
       }
     __syncthreads();
     t.load(x, k + 2, reg);
     if (threadIdx.x < t.width) walk_column(buf + threadIdx.x, t.width, t.rows_in(k), [&](float a) { sum += a; });
   };
-  V v2[T::kLoads];
+  v4f v2[T::kLoads];
   t.load(x, 0, v);
   t.load(x, 1, v2);
   for (uint32_t k = 0; k < chunks; k += 2) {
@@ -1142,12 +1149,10 @@ __global__ __launch_bounds__(kBlock) void softmax_tall_kernel(const float* x, fl
   __syncthreads();
   if (threadIdx.x < t.width) stat[threadIdx.x] = sum;
   __syncthreads();
-  float total[VEC];
-#pragma unroll
-  for (int e = 0; e < VEC; ++e) total[e] = stat[t.col + e];
+  const v4f total = *reinterpret_cast<const v4f*>(stat + t.col);
 
   for (uint32_t k = 0; k < chunks; k += kTallAhead) {
-    V w[kTallAhead][T::kLoads];
+    v4f w[kTallAhead][T::kLoads];
 #pragma unroll
     for (int j = 0; j < kTallAhead; ++j) t.load(x, k + j, w[j]);
 #pragma unroll
@@ -1155,46 +1160,43 @@ __global__ __launch_bounds__(kBlock) void softmax_tall_kernel(const float* x, fl
 #pragma unroll
       for (int i = 0; i < T::kLoads; ++i)
         if (t.has(k + j, i)) {
-          V q;
+          v4f q;
 #pragma unroll
-          for (int e = 0; e < VEC; ++e)
-            tall_set(q, e, libm::exact_expf(tall_elem(w[j][i], e) - max_val[e], tab) / total[e]);
-          __builtin_nontemporal_store(
-              q, reinterpret_cast<V*>(y + t.base + static_cast<uint64_t>(t.row(k + j, i)) * inner));
+          for (int e = 0; e < 4; ++e) q[e] = libm::exact_expf(w[j][i][e] - max_val[e], tab) / total[e];
+          t.store(y, t.row(k + j, i), q);
         }
   }
 }
 
-template <int PMODE, int SM, int VEC>
+template <int PMODE, int SM>
 __global__ __launch_bounds__(kBlock) void normalize_tall_kernel(const float* x, float* y, uint32_t dim,
                                                                  uint32_t inner, uint32_t width_log2,
                                                                  FastDiv f_tiles, float p, float eps,
                                                                  const float* scale) {
-  using T = TallTile<VEC>;
-  using V = typename T::V;
+  using T = TallTile;
   __shared__ __align__(16) float chunk[2][kTallChunkFloats];
-  __shared__ float stat[64];
+  __shared__ __align__(16) float stat[64];
   const T t(dim, inner, width_log2, f_tiles);
   const uint32_t chunks = t.chunks();
-  V v[T::kLoads];
+  v4f v[T::kLoads];
 
   double acc = 0;
-  auto pass = [&](uint32_t k, V(&reg)[T::kLoads]) {  // as in softmax_tall_kernel
+  auto pass = [&](uint32_t k, v4f(&reg)[T::kLoads]) {  // as in softmax_tall_kernel
     float* buf = chunk[k & 1];
 #pragma unroll
     for (int i = 0; i < T::kLoads; ++i)
       if (t.has(k, i)) {
-        V term;
+        v4f term;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) tall_set(term, e, static_cast<float>(norm_term<PMODE>(tall_elem(reg[i], e), p)));
-        *reinterpret_cast<V*>(buf + t.slot(i)) = term;
+        for (int e = 0; e < 4; ++e) term[e] = static_cast<float>(norm_term<PMODE>(reg[i][e], p));
+        *reinterpret_cast<v4f*>(buf + t.slot(i)) = term;
       }
     __syncthreads();
     t.load(x, k + 2, reg);
     if (threadIdx.x < t.width)
       walk_column(buf + threadIdx.x, t.width, t.rows_in(k), [&](float a) { acc += static_cast<double>(a); });
   };
-  V v2[T::kLoads];
+  v4f v2[T::kLoads];
   t.load(x, 0, v);
   t.load(x, 1, v2);
   for (uint32_t k = 0; k < chunks; k += 2) {
@@ -1204,12 +1206,10 @@ __global__ __launch_bounds__(kBlock) void normalize_tall_kernel(const float* x, 
   __syncthreads();
   if (threadIdx.x < t.width) stat[threadIdx.x] = norm_finish<PMODE>(acc, p, eps);
   __syncthreads();
-  float div[VEC];
-#pragma unroll
-  for (int e = 0; e < VEC; ++e) div[e] = stat[t.col + e];
+  const v4f div = *reinterpret_cast<const v4f*>(stat + t.col);
 
   for (uint32_t k = 0; k < chunks; k += kTallAhead) {
-    V w[kTallAhead][T::kLoads];
+    v4f w[kTallAhead][T::kLoads];
 #pragma unroll
     for (int j = 0; j < kTallAhead; ++j) t.load(x, k + j, w[j]);
 #pragma unroll
@@ -1218,10 +1218,10 @@ __global__ __launch_bounds__(kBlock) void normalize_tall_kernel(const float* x, 
       for (int i = 0; i < T::kLoads; ++i)
         if (t.has(k + j, i)) {
           const uint32_t r = t.row(k + j, i);
-          V q;
+          v4f q;
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) tall_set(q, e, ssd_scaled<SM>(tall_elem(w[j][i], e) / div[e], scale, r));
-          __builtin_nontemporal_store(q, reinterpret_cast<V*>(y + t.base + static_cast<uint64_t>(r) * inner));
+          for (int e = 0; e < 4; ++e) q[e] = ssd_scaled<SM>(w[j][i][e] / div[e], scale, r);
+          t.store(y, r, q);
         }
   }
 }
@@ -1455,15 +1455,13 @@ static bool long_slab(int dim, int inner_num) {
 }
 
 // Where the tall kernels apply, and their launch: positions per workgroup as wide
-// as still leaves a thousand workgroups, 128-bit accesses where every row piece
-// starts on a 16-byte boundary.
+// as still leaves a thousand workgroups.
 struct TallLaunch {
   uint32_t grid, width_log2;
   FastDiv f_tiles;
-  bool vec4;
 };
 
-static bool tall_launch(int outer_num, int dim, int inner_num, const float* x, const float* y, TallLaunch* t) {
+static bool tall_launch(int outer_num, int dim, int inner_num, TallLaunch* t) {
   if (static_cast<uint32_t>(inner_num) < kTallMinInner || dim < 128) return false;
   uint32_t w = 6;
   while (w > 4 && static_cast<uint64_t>(outer_num) * ((inner_num + (1u << w) - 1) >> w) < 1024) --w;
@@ -1471,18 +1469,15 @@ static bool tall_launch(int outer_num, int dim, int inner_num, const float* x, c
   t->grid = static_cast<uint32_t>(outer_num) * tiles;
   t->width_log2 = w;
   t->f_tiles = make_fastdiv(tiles);
-  t->vec4 = inner_num % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
   return true;
 }
 
 template <int PMODE, int SM>
 static void launch_normalize_tall(const TallLaunch& t, int dim, int inner_num, float p, float eps, const float* x,
                                   const float* scale, float* y, hipStream_t st) {
-  const uint32_t d = static_cast<uint32_t>(dim), in = static_cast<uint32_t>(inner_num);
-  if (t.vec4)
-    normalize_tall_kernel<PMODE, SM, 4><<<t.grid, kBlock, 0, st>>>(x, y, d, in, t.width_log2, t.f_tiles, p, eps, scale);
-  else
-    normalize_tall_kernel<PMODE, SM, 1><<<t.grid, kBlock, 0, st>>>(x, y, d, in, t.width_log2, t.f_tiles, p, eps, scale);
+  normalize_tall_kernel<PMODE, SM><<<t.grid, kBlock, 0, st>>>(x, y, static_cast<uint32_t>(dim),
+                                                              static_cast<uint32_t>(inner_num), t.width_log2,
+                                                              t.f_tiles, p, eps, scale);
 }
 
 // Shared launch geometry: slab layout when the columns are too narrow to
@@ -1560,13 +1555,10 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
     launch_softmax_tile_ts<6>(outer_num, dim, inner_num, x, y, st);
   else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner)
     launch_softmax_tile_ts<5>(outer_num, dim, inner_num, x, y, st);
-  else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, x, y, &t)) {
-    const uint32_t d = static_cast<uint32_t>(dim), in = static_cast<uint32_t>(inner_num);
-    if (t.vec4)
-      softmax_tall_kernel<4><<<t.grid, kBlock, 0, st>>>(x, y, d, in, t.width_log2, t.f_tiles);
-    else
-      softmax_tall_kernel<1><<<t.grid, kBlock, 0, st>>>(x, y, d, in, t.width_log2, t.f_tiles);
-  } else
+  else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, &t))
+    softmax_tall_kernel<<<t.grid, kBlock, 0, st>>>(x, y, static_cast<uint32_t>(dim), static_cast<uint32_t>(inner_num),
+                                                   t.width_log2, t.f_tiles);
+  else
     softmax_columns_kernel<<<(g.columns + kWave - 1) / kWave, kWave, 0, st>>>(x, y, g.columns,
                                                                              static_cast<uint32_t>(dim), fi);
   return launch_status();
@@ -1628,7 +1620,7 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
       else
         normalize_columns_reg_kernel<2, 64><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
     }
-  } else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, x, y, &t)) {
+  } else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, &t)) {
     if (mode == 1)
       launch_normalize_tall<1, kSsdNoScale>(t, dim, inner_num, p, eps, x, nullptr, y, st);
     else if (mode == 2)
@@ -1673,7 +1665,7 @@ static void launch_ssd_columns(const ColumnGeometry& g, int outer_num, int dim, 
     normalize_columns_reg_kernel<3, 16, SM><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, 2.f, eps, scale);
   else if (dim <= 64)
     normalize_columns_reg_kernel<3, 64, SM><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, 2.f, eps, scale);
-  else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, x, y, &t))
+  else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, &t))
     launch_normalize_tall<3, SM>(t, dim, inner_num, 2.f, eps, x, scale, y, st);
   else
     normalize_columns_kernel<3, SM><<<(g.columns + kWave - 1) / kWave, kWave, 0, st>>>(x, y, g.columns, d, fi, 2.f,
