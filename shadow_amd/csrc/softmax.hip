@@ -1015,6 +1015,329 @@ static void launch_softmax_tile_ts(int outer_num, int dim, int inner_num, const 
 }
 
 // ---------------------------------------------------------------------------
+// Rows: the statistic over the last axis (inner == 1: class scores, attention
+// rows), 17 to 4096 long.  The ordered sum of a row is one lane's walk, a few
+// microseconds for a thousand elements, and with a workgroup per row (the slab
+// kernels) a CU has eight such walks in flight and 255 of 256 lanes wait for
+// each.  Here every wave works by itself, without a barrier, on R consecutive
+// rows (R a power of two, R * pitch floats of LDS: one contiguous piece of x):
+// all 64 lanes stage them, 64 / R lanes share a row for the maximum (any order,
+// see softmax_slab_kernel), the exponentials and the division, the first lane
+// of each row adds it up front to back, and the piece goes back as it came.  A
+// wave never waits for another, so a CU has 8 or 16 of them, each with R walks,
+// at different points of their work.  The four waves of a workgroup exist for
+// their placement, one per SIMD (see pool_rows_stream_kernel).
+// ---------------------------------------------------------------------------
+constexpr uint32_t kRowsMinDim = 17;
+
+struct WaveRows {
+  uint32_t dim, pitch, rows_per_wave, group_log2;  // lanes per row = 1 << group_log2
+  FastDiv f_dim;
+};
+
+// The wave's rows into its tile: 128-bit loads of the contiguous piece, eight in flight, scattered
+// by element (a vector may end in the next row).
+SHDW_DEVICE void rows_stage_in(float* tile, const float* xs, uint32_t cells, const WaveRows& w, uint32_t lane) {
+  const uint32_t nvec = cells / 4;
+  for (uint32_t v0 = 0; v0 < nvec; v0 += 8 * kWave) {
+    v4f reg[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const uint32_t v = v0 + k * kWave + lane;
+      if (v < nvec) reg[k] = load4_stream_any(xs + 4ull * v);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const uint32_t v = v0 + k * kWave + lane;
+      if (v < nvec) {
+        uint32_t r, c;
+        fd_divmod(4 * v, w.f_dim, r, c);
+        uint32_t at = r * w.pitch + c;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          tile[at] = reg[k][j];
+          ++at;
+          if (++c == w.dim) c = 0, at += w.pitch - w.dim;
+        }
+      }
+    }
+  }
+  const uint32_t t = 4 * nvec + lane;
+  if (t < cells) {
+    uint32_t r, c;
+    fd_divmod(t, w.f_dim, r, c);
+    tile[r * w.pitch + c] = xs[t];
+  }
+}
+
+// f(value in the tile, row, column) for every element, written to the contiguous piece of y.
+template <class F>
+SHDW_DEVICE void rows_stage_out(const float* tile, float* ys, uint32_t cells, const WaveRows& w, uint32_t lane, F f) {
+  const uint32_t nvec = cells / 4;
+  for (uint32_t v = lane; v < nvec; v += kWave) {
+    uint32_t r, c;
+    fd_divmod(4 * v, w.f_dim, r, c);
+    uint32_t at = r * w.pitch + c;
+    v4f q;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      q[j] = f(tile[at], r, c);
+      ++at;
+      if (++c == w.dim) c = 0, ++r, at += w.pitch - w.dim;
+    }
+    store4_stream_any(ys + 4ull * v, q);
+  }
+  const uint32_t t = 4 * nvec + lane;
+  if (t < cells) {
+    uint32_t r, c;
+    fd_divmod(t, w.f_dim, r, c);
+    ys[t] = f(tile[r * w.pitch + c], r, c);
+  }
+}
+
+template <int TILE>
+__global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const float* x, float* y, uint32_t rows, WaveRows w) {
+  __shared__ __align__(16) float tiles[kBlock / kWave][TILE];
+  __shared__ float stats[kBlock / kWave][kWave];
+  __shared__ uint64_t tab[32];
+  if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
+  __syncthreads();  // the only one: from here on every wave is on its own
+  const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  float* tile = tiles[wave];
+  float* stat = stats[wave];
+  const uint32_t row0 = (blockIdx.x * (kBlock / kWave) + wave) * w.rows_per_wave;
+  if (row0 >= rows) return;  // the whole wave
+  const uint32_t nrows = min(w.rows_per_wave, rows - row0), cells = nrows * w.dim;
+  const uint64_t base = static_cast<uint64_t>(row0) * w.dim;
+  rows_stage_in(tile, x + base, cells, w, lane);
+  __builtin_amdgcn_wave_barrier();
+  const uint32_t group = 1u << w.group_log2;
+  const uint32_t r = lane >> w.group_log2, sub = lane & (group - 1);
+  float* mine = tile + (r < nrows ? r : 0) * w.pitch;  // rows past the end: their lanes read row 0 and write nothing
+  float m = -FLT_MAX;
+  for (uint32_t c = sub; c < w.dim; c += group) m = std_max(mine[c], m);
+  for (uint32_t off = 1; off < group; off <<= 1) m = std_max(__shfl_xor(m, off), m);  // all 64 lanes are here
+  __builtin_amdgcn_wave_barrier();
+  if (r < nrows)
+    for (uint32_t c = sub; c < w.dim; c += group) mine[c] = libm::exact_expf(mine[c] - m, tab);
+  __builtin_amdgcn_wave_barrier();
+  if (sub == 0 && r < nrows) {
+    float sum = 0.f;
+    walk_column(mine, 1, w.dim, [&](float a) { sum += a; });
+    stat[r] = sum;
+  }
+  __builtin_amdgcn_wave_barrier();
+  rows_stage_out(tile, y + base, cells, w, lane, [&](float e, uint32_t rr, uint32_t) { return e / stat[rr]; });
+}
+
+// PMODE 1, 2 (Normalize) and 3 (SSDNormalize per position); the terms of the sum are formed by the walking lane.
+template <int PMODE, int SM, int TILE>
+__global__ __launch_bounds__(kBlock) void normalize_rows_kernel(const float* x, float* y, uint32_t rows, WaveRows w,
+                                                                 float p, float eps, const float* scale) {
+  __shared__ __align__(16) float tiles[kBlock / kWave][TILE];
+  __shared__ float stats[kBlock / kWave][kWave];
+  const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  float* tile = tiles[wave];
+  float* stat = stats[wave];
+  const uint32_t row0 = (blockIdx.x * (kBlock / kWave) + wave) * w.rows_per_wave;
+  if (row0 >= rows) return;  // the whole wave
+  const uint32_t nrows = min(w.rows_per_wave, rows - row0), cells = nrows * w.dim;
+  const uint64_t base = static_cast<uint64_t>(row0) * w.dim;
+  rows_stage_in(tile, x + base, cells, w, lane);
+  __builtin_amdgcn_wave_barrier();
+  const uint32_t group = 1u << w.group_log2;
+  const uint32_t r = lane >> w.group_log2, sub = lane & (group - 1);
+  if (sub == 0 && r < nrows) {
+    double acc = 0;
+    walk_column(tile + r * w.pitch, 1, w.dim, [&](float a) { acc += norm_term<PMODE>(a, p); });
+    stat[r] = norm_finish<PMODE>(acc, p, eps);
+  }
+  __builtin_amdgcn_wave_barrier();
+  rows_stage_out(tile, y + base, cells, w, lane,
+                 [&](float v, uint32_t rr, uint32_t c) { return ssd_scaled<SM>(v / stat[rr], scale, c); });
+}
+
+// Rows per wave and lanes per row for the kernels above; false where they do not apply.
+template <int TILE>
+static bool wave_rows(int dim, WaveRows* w) {
+  const uint32_t d = static_cast<uint32_t>(dim);
+  uint32_t r = 1;
+  while (r < kWave && 2 * r * (d | 1u) <= static_cast<uint32_t>(TILE)) r *= 2;
+  w->dim = d, w->pitch = r > 1 ? (d | 1u) : d;
+  if (w->pitch * r > static_cast<uint32_t>(TILE)) return false;
+  w->rows_per_wave = r;
+  w->group_log2 = 0;
+  while ((r << w->group_log2) < kWave) ++w->group_log2;
+  w->f_dim = make_fastdiv(d);
+  return true;
+}
+
+// ---------------------------------------------------------------------------
+// Normalize over long rows (inner == 1, more than a few hundred elements).  One
+// lane walking a row costs its wave a full instruction slot per element whether
+// one lane walks or sixty-four (rows of 2048 with a row per wave: 105 us per
+// 51 MB, all of it the walks), and whole rows of this length leave room for one
+// or two per wave in LDS.  Here a wave takes G rows and moves along them in
+// equal chunks of at most W = 4096 / G columns: all lanes fetch a chunk (up to
+// 16 vectors each) into the wave's tile, lane g < G folds row g's piece in
+// index order, and the next chunk's requests are already out; a second pass
+// scales x straight from the registers, no tile.  No barriers; four waves per
+// workgroup for their placement only.  (Softmax in this form takes every
+// exponential twice and came out slower than the kernels it would replace.)
+// ---------------------------------------------------------------------------
+constexpr int kStreamVectors = 16;  // per lane and chunk
+
+template <int G>
+struct RowStream {
+  static constexpr uint32_t W = 256u * kStreamVectors / G, VW = W / 4, PITCH = W + 4;
+  uint32_t rows, len, row0, lane;
+  uint32_t step;  // columns per chunk: the row cut into equal pieces of at most W (a multiple of 4), not W + a rest
+  SHDW_DEVICE void init(uint32_t rows_, uint32_t len_, uint32_t row0_, uint32_t lane_) {
+    rows = rows_, len = len_, row0 = row0_, lane = lane_;
+    const uint32_t pieces = (len + W - 1) / W;
+    step = (((len + pieces - 1) / pieces) + 3) & ~3u;
+  }
+  // vector i of the lane's share of the chunk at column c0: its row (of the wave's G) and first column
+  SHDW_DEVICE static uint32_t row_of(uint32_t lane, int i) { return (lane + kWave * i) / VW; }
+  SHDW_DEVICE static uint32_t col_of(uint32_t lane, int i) { return 4 * ((lane + kWave * i) % VW); }
+  SHDW_DEVICE uint32_t count(int i, uint32_t c0) const {  // elements of vector i that exist
+    if (row0 + row_of(lane, i) >= rows || col_of(lane, i) >= step) return 0;
+    const uint32_t c = c0 + col_of(lane, i);
+    return c >= len ? 0u : min(4u, len - c);
+  }
+  SHDW_DEVICE uint32_t cols(uint32_t c0) const { return min(step, len - c0); }  // of the chunk at c0
+  SHDW_DEVICE void request(const float* x, uint32_t c0, v4f (&reg)[kStreamVectors]) const {
+#pragma unroll
+    for (int i = 0; i < kStreamVectors; ++i) {
+      const uint32_t n = count(i, c0);
+      if (n == 0) continue;
+      const float* src = x + static_cast<uint64_t>(row0 + row_of(lane, i)) * len + c0 + col_of(lane, i);
+      if (n == 4) {
+        reg[i] = load4_stream_any(src);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+          if (static_cast<uint32_t>(k) < n) reg[i][k] = __builtin_nontemporal_load(src + k);
+      }
+    }
+  }
+  // f(vector, i) for every vector of the chunk, into the wave's tile
+  template <class F>
+  SHDW_DEVICE void lay_down(float* tile, const v4f (&reg)[kStreamVectors], F f) const {
+#pragma unroll
+    for (int i = 0; i < kStreamVectors; ++i)
+      *reinterpret_cast<v4f*>(tile + row_of(lane, i) * PITCH + col_of(lane, i)) = f(reg[i], i);
+  }
+};
+
+template <int PMODE, int SM, int G>
+__global__ __launch_bounds__(kBlock) void normalize_rows_stream_kernel(const float* x, float* y, uint32_t rows,
+                                                                        uint32_t len, float p, float eps,
+                                                                        const float* scale) {
+  using S = RowStream<G>;
+  __shared__ __align__(16) float tiles[kBlock / kWave][G * S::PITCH];
+  __shared__ float divisors[kBlock / kWave][G];
+  S s;
+  const uint32_t wave = threadIdx.x / kWave;
+  s.init(rows, len, (blockIdx.x * (kBlock / kWave) + wave) * G, threadIdx.x % kWave);
+  if (s.row0 >= rows) return;  // the whole wave
+  float* tile = tiles[wave];
+  const float* mine = tile + s.lane * S::PITCH;
+  v4f reg[kStreamVectors];
+
+  double acc = 0;
+  s.request(x, 0, reg);
+  for (uint32_t c0 = 0; c0 < len; c0 += s.step) {
+    s.lay_down(tile, reg, [](const v4f& v, int) { return v; });
+    __builtin_amdgcn_wave_barrier();
+    if (c0 + s.step < len) s.request(x, c0 + s.step, reg);
+    if (s.lane < G) walk_column(mine, 1, s.cols(c0), [&](float a) { acc += norm_term<PMODE>(a, p); });
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (s.lane < G) divisors[wave][s.lane] = norm_finish<PMODE>(acc, p, eps);
+  __builtin_amdgcn_wave_barrier();
+
+  for (uint32_t c0 = 0; c0 < len; c0 += s.step) {
+    s.request(x, c0, reg);
+#pragma unroll
+    for (int i = 0; i < kStreamVectors; ++i) {
+      const uint32_t n = s.count(i, c0);
+      if (n == 0) continue;
+      const uint32_t g = S::row_of(s.lane, i), c = c0 + S::col_of(s.lane, i);
+      const float div = divisors[wave][g];
+      v4f q = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (static_cast<uint32_t>(k) < n) q[k] = ssd_scaled<SM>(reg[i][k] / div, scale, c + k);  // scale[] ends with the row
+      float* dst = y + static_cast<uint64_t>(s.row0 + g) * len + c;
+      if (n == 4) {
+        store4_stream_any(dst, q);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+          if (static_cast<uint32_t>(k) < n) dst[k] = q[k];
+      }
+    }
+  }
+}
+
+constexpr int kRowsSmallTile = 2048;  // floats per wave: 16 waves per CU
+constexpr int kRowsMinRows = 1024;                          // fewer rows: a workgroup per row keeps more lanes busy
+
+static bool rows_apply(int outer_num, int dim, int inner_num) {
+  return inner_num == 1 && static_cast<uint32_t>(dim) >= kRowsMinDim && outer_num >= kRowsMinRows;
+}
+
+// Normalize: from this row length on the rows move in chunks, G rows per wave (512: 34 us against 47 per 51 MB).
+// Softmax stays with the rows in LDS while two rows fit a wave's tile (1000: 49 us; in chunks 62, since the
+// exponentials then have to be taken twice) and with a workgroup per row beyond (4096: 62 us; in chunks 94).
+constexpr int kRowsStreamMinDim = 401;
+constexpr int kRowsSoftmaxMaxDim = 1023;
+
+// Rows per wave of the streaming kernels: as many as still leave a thousand waves.
+static int stream_rows(uint32_t rows, uint32_t len) {
+  int best = 4;
+  uint64_t best_cost = ~0ull;
+  for (int g = 4; g <= 64; g *= 2) {
+    if (g > 4 && rows / static_cast<uint32_t>(g) < 1024u) break;
+    const uint32_t w = 256u * kStreamVectors / static_cast<uint32_t>(g);
+    const uint64_t cost = static_cast<uint64_t>((len + w - 1) / w) * w;  // vector slots a row takes, filled or not
+    if (cost <= best_cost) best = g, best_cost = cost;
+  }
+  return best;
+}
+
+template <int PMODE, int SM>
+static void launch_normalize_rows_stream(uint32_t rows, uint32_t len, float p, float eps, const float* x,
+                                         const float* scale, float* y, hipStream_t st) {
+  const int g = stream_rows(rows, len);
+  const uint32_t per_wg = static_cast<uint32_t>(g) * (kBlock / kWave), grid = (rows + per_wg - 1) / per_wg;
+  switch (g) {
+    case 64: normalize_rows_stream_kernel<PMODE, SM, 64><<<grid, kBlock, 0, st>>>(x, y, rows, len, p, eps, scale); break;
+    case 32: normalize_rows_stream_kernel<PMODE, SM, 32><<<grid, kBlock, 0, st>>>(x, y, rows, len, p, eps, scale); break;
+    case 8: normalize_rows_stream_kernel<PMODE, SM, 8><<<grid, kBlock, 0, st>>>(x, y, rows, len, p, eps, scale); break;
+    case 16: normalize_rows_stream_kernel<PMODE, SM, 16><<<grid, kBlock, 0, st>>>(x, y, rows, len, p, eps, scale); break;
+    default: normalize_rows_stream_kernel<PMODE, SM, 4><<<grid, kBlock, 0, st>>>(x, y, rows, len, p, eps, scale);
+  }
+}
+
+static uint32_t rows_grid(uint32_t rows, const WaveRows& w) {
+  const uint32_t per_group = w.rows_per_wave * (kBlock / kWave);
+  return (rows + per_group - 1) / per_group;
+}
+
+template <int PMODE, int SM>
+static void launch_normalize_rows(int outer_num, int dim, float p, float eps, const float* x, const float* scale,
+                                  float* y, hipStream_t st) {
+  WaveRows w;
+  const uint32_t rows = static_cast<uint32_t>(outer_num);
+  if (dim < kRowsStreamMinDim && wave_rows<kRowsSmallTile>(dim, &w))
+    normalize_rows_kernel<PMODE, SM, kRowsSmallTile><<<rows_grid(rows, w), kBlock, 0, st>>>(x, y, rows, w, p, eps, scale);
+  else
+    launch_normalize_rows_stream<PMODE, SM>(rows, static_cast<uint32_t>(dim), p, eps, x, scale, y, st);
+}
+
+// ---------------------------------------------------------------------------
 // Tall columns: more rows than the tile kernels hold in LDS and, with that, few
 // columns (a softmax over 1000 or 4096 channels of a 56x56 map has 3136 per
 // image), which a lane per column leaves to a handful of waves.  Here a
@@ -1531,6 +1854,12 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
   if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
+  if (WaveRows w; rows_apply(outer_num, dim, inner_num) && dim <= kRowsSoftmaxMaxDim &&
+                  wave_rows<kRowsSmallTile>(dim, &w)) {
+    const uint32_t rows = static_cast<uint32_t>(outer_num);
+    softmax_rows_kernel<kRowsSmallTile><<<rows_grid(rows, w), kBlock, 0, st>>>(x, y, rows, w);
+    return launch_status();
+  }
   if (const uint32_t group = packed_group(dim, inner_num)) {
     const uint32_t slabs = static_cast<uint32_t>(outer_num);
     softmax_packed_kernel<<<(slabs + group - 1) / group, kBlock, packed_bytes(dim, inner_num, group), st>>>(
@@ -1575,6 +1904,11 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
   const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
   const uint32_t d = static_cast<uint32_t>(dim);
   const int mode = p == 1.f ? 1 : (p == 2.f ? 2 : 0);
+  if (mode != 0 && rows_apply(outer_num, dim, inner_num)) {
+    if (mode == 1) launch_normalize_rows<1, kSsdNoScale>(outer_num, dim, p, eps, x, nullptr, y, st);
+    else launch_normalize_rows<2, kSsdNoScale>(outer_num, dim, p, eps, x, nullptr, y, st);
+    return launch_status();
+  }
   if (const uint32_t group = packed_group(dim, inner_num)) {
     const uint32_t slabs = static_cast<uint32_t>(outer_num);
     const uint32_t grid = (slabs + group - 1) / group;
@@ -1651,6 +1985,10 @@ static void launch_ssd_columns(const ColumnGeometry& g, int outer_num, int dim, 
   const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
   const uint32_t d = static_cast<uint32_t>(dim);
   const uint32_t grid = grid_for(g.columns);
+  if (rows_apply(outer_num, dim, inner_num)) {
+    launch_normalize_rows<3, SM>(outer_num, dim, 2.f, eps, x, scale, y, st);
+    return;
+  }
   if (const uint32_t group = packed_group(dim, inner_num)) {
     const uint32_t slabs = static_cast<uint32_t>(outer_num);
     normalize_packed_kernel<3, SM><<<(slabs + group - 1) / group, kBlock, packed_bytes(dim, inner_num, group), st>>>(

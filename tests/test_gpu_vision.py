@@ -100,6 +100,10 @@ SOFTMAX_SHAPES = [  # outer, dim, inner: both layouts, LDS limits, odd sizes
     # a cut last tile, a last chunk of one row, many workgroups
     (2, 1300, 30), (2, 600, 64), (1, 1000, 100), (3, 513, 17), (1, 2048, 196), (2, 700, 68), (1, 4097, 16),
     (1, 1025, 3136), (40, 520, 128), (1100, 513, 16), (2, 769, 49), (1, 20000, 20),
+    # a thousand and more rows over the last axis: every wave on its own rows (1 to 32 rows per wave, both
+    # tile sizes, a ragged last wave and workgroup)
+    (1100, 17, 1), (2000, 49, 1), (1025, 1000, 1), (1024, 1023, 1), (1030, 1024, 1), (1100, 2049, 1), (1024, 4096, 1),
+    (1500, 64, 1), (3001, 21, 1), (1027, 333, 1), (5000, 150, 1),
     # long slabs over fewer than 16 positions, in chunks of whole rows: ragged last chunks, one to fifteen positions
     (2, 5000, 3), (1, 16000, 1), (1, 1100, 14), (3, 2731, 6), (2, 8193, 2), (1, 3000, 15), (5, 1537, 10),
 ]
@@ -113,7 +117,27 @@ def test_softmax(gpu, outer, dim, inner):
     assert_bit_exact(gpuops.softmax(x, outer, dim, inner, inplace=True), want, "softmax in place")
 
 
-@pytest.mark.parametrize("outer,dim,inner", [(40, 50, 1), (2, 12, 200), (2, 80, 100), (2, 6000, 3), (1, 700, 64)])
+# Long rows over the last axis: Normalize moves along 4, 8, 16, 32 or 64 rows per wave by the number and the
+# length of the rows (whole and cut chunks, a cut last vector, a last wave with rows missing); Softmax has
+# the rows in LDS up to 1023 elements and a workgroup per row beyond.
+@pytest.mark.parametrize("outer,dim", [(1500, 401), (1024, 4097), (1100, 8191), (40003, 402), (70001, 401),
+                                       (131077, 403), (2049, 513), (1030, 20000), (9001, 500), (17001, 405),
+                                       (1201, 1023), (1201, 1024), (8563, 1500)])
+def test_softmax_and_normalize_over_long_rows(gpu, outer, dim):
+    x = normal(33, outer * dim, 4.0)
+    assert_bit_exact(gpuops.softmax(x, outer, dim, 1), oracle.softmax(x, outer, dim, 1), "softmax")
+    assert_bit_exact(gpuops.normalize(x, outer, dim, 1, 2.0, 1e-12), oracle.normalize(x, outer, dim, 1, 2.0, 1e-12),
+                     "normalize")
+    if outer < 3000:
+        assert_bit_exact(gpuops.softmax(x, outer, dim, 1, inplace=True, offset=1), oracle.softmax(x, outer, dim, 1),
+                         "softmax in place, off the vector boundary")
+        scale = uniform(34, dim, 0.5, 2.0)
+        assert_bit_exact(gpuops.ssd_normalize(x, outer, dim, 1, False, False, 1e-5, scale),
+                         oracle.ssd_normalize(x, outer, dim, 1, False, False, 1e-5, scale), "ssd normalize")
+
+
+@pytest.mark.parametrize("outer,dim,inner", [(40, 50, 1), (2, 12, 200), (2, 80, 100), (2, 6000, 3), (1, 700, 64),
+                                             (1200, 100, 1), (1030, 1500, 1)])
 def test_softmax_special_values(gpu, outer, dim, inner):
     x = with_specials(normal(14, outer * dim * inner, 30.0), 14)
     assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax specials")
@@ -174,7 +198,8 @@ def test_softmax_op_defaults_and_errors(ws):
                                              # tall columns in chunks through LDS; slabs of more than 60 KB
                                              (2, 1300, 30), (1, 2048, 196), (2, 1100, 68), (1, 4097, 16),
                                              (30, 1026, 128), (3, 4096, 7), (1, 39000, 1),
-                                             (2, 5000, 3), (1, 1100, 14), (3, 2731, 6), (2, 8193, 2)])
+                                             (2, 5000, 3), (1, 1100, 14), (3, 2731, 6), (2, 8193, 2),
+                                             (1100, 17, 1), (1025, 1000, 1), (1030, 1024, 1), (1024, 4096, 1), (3001, 21, 1)])
 def test_normalize(gpu, p, outer, dim, inner):
     x = normal(17, outer * dim * inner, 2.0)
     want = oracle.normalize(x, outer, dim, inner, p, 1e-12)
@@ -204,7 +229,8 @@ def test_normalize_op(ws, args):
 # ----------------------------------------------------------- SSDNormalize ---
 SSD_SHAPES = [(2, 5, 12), (3, 512, 1), (2, 16, 100), (3, 9, 64), (1, 600, 3), (2, 1, 9), (1, 33, 4097),
               (2, 64, 1444), (5, 3, 7), (1, 128, 4096), (3, 20, 1025), (2, 512, 361), (1, 1000, 50), (2, 70, 33),
-              (1, 512, 1444), (2, 1030, 24), (2, 1100, 68), (1, 2049, 31), (3, 4096, 7), (2, 5000, 3), (1, 1100, 14)]
+              (1, 512, 1444), (2, 1030, 24), (2, 1100, 68), (1, 2049, 31), (3, 4096, 7), (2, 5000, 3), (1, 1100, 14),
+              (1100, 17, 1), (1025, 1000, 1), (1030, 2049, 1)]
 
 
 @pytest.mark.parametrize("scale_kind", ["none", "shared", "channel"])
@@ -350,7 +376,7 @@ def test_global_pooling_op(ws, pool, shape):
 
 # Blobs start on allocator boundaries; pointers made of a blob and an offset, as the
 # Blas face passes them, may start on any float.  One shape per kernel layout.
-ODD_POINTER_COLUMNS = [(64, 1000, 1), (300, 4, 2), (5000, 21, 1), (2, 21, 63), (4, 8, 1024), (2, 150, 300),
+ODD_POINTER_COLUMNS = [(64, 1000, 1), (300, 4, 2), (5000, 21, 1), (1100, 333, 1), (2, 21, 63), (4, 8, 1024), (2, 150, 300),
                        (1, 512, 33), (2, 100, 100), (3, 4096, 7), (2, 1300, 30), (2, 600, 64), (1, 2048, 196)]
 
 
