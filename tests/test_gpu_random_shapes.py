@@ -99,6 +99,28 @@ def test_column_ops_random_shapes(gpu, seed):
                          oracle.ssd_normalize(x, outer, dim, inner, False, True, 1e-10), "ssd normalize " + what)
 
 
+# The last axis of a thousand rows and more: whole rows per wave in LDS (2 to 64 of them), Normalize over
+# rows from 401 on in chunks along 4 to 64 rows per wave; zeros, infinities and NaNs in some rows.
+@pytest.mark.parametrize("seed", [26, 27, 28])
+def test_last_axis_random_shapes(gpu, seed):
+    rng = np.random.default_rng(seed)
+    for t in range(14):
+        dim = int(np.exp(rng.uniform(np.log(17), np.log(2500))))
+        outer = int(rng.integers(1024, max(1025, min(150000, 3_000_000 // dim))))
+        x = rng.normal(0, 4, outer * dim).astype(F)
+        if t % 3 == 0:
+            x[rng.random(x.size) < 0.2] = 0.0
+            x[rng.random(x.size) < 0.001] = rng.choice([np.inf, -np.inf, np.nan])
+        what = "[%d, %d, 1]" % (outer, dim)
+        assert_bit_exact(gpuops.softmax(x, outer, dim, 1), oracle.softmax(x, outer, dim, 1), "softmax " + what)
+        p = float(rng.choice([1.0, 2.0, 3.0]))
+        assert_bit_exact(gpuops.normalize(x, outer, dim, 1, p, 1e-12), oracle.normalize(x, outer, dim, 1, p, 1e-12),
+                         "normalize p=%g %s" % (p, what))
+        scale = rng.uniform(0.5, 2.0, dim).astype(F)
+        assert_bit_exact(gpuops.ssd_normalize(x, outer, dim, 1, False, False, 1e-10, scale),
+                         oracle.ssd_normalize(x, outer, dim, 1, False, False, 1e-10, scale), "ssd normalize " + what)
+
+
 @pytest.mark.parametrize("seed", [8, 9, 20, 21])
 def test_broadcast_random_shapes(gpu, seed):
     rng = np.random.default_rng(seed)
