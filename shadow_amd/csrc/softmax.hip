@@ -461,6 +461,130 @@ __global__ __launch_bounds__(kBlock) void normalize_columns_reg_kernel(const flo
       __builtin_nontemporal_store(ssd_scaled<SM>(v[c] / div, scale, c), yc + static_cast<uint64_t>(c) * inner);
 }
 
+// ---------------------------------------------------------------------------
+// Columns of up to DMAX elements over four and more positions: a lane takes four
+// neighbouring positions of one slab, every row of them as one 128-bit access on
+// any dword address, and keeps its four columns in registers.  One division per
+// lane in place of four, a quarter of the memory instructions of the
+// column-per-lane kernels above (softmax over [2048,2,3136]: 38 us per 51 MB with
+// a column per lane).  The last quad of a slab holds inner % 4 positions where
+// that is not zero and moves float by float.
+// ---------------------------------------------------------------------------
+struct QuadLane {
+  uint64_t base;  // first row, first position
+  uint32_t n;     // positions that exist: 1 .. 4
+};
+
+SHDW_DEVICE QuadLane quad_lane(uint32_t i, FastDiv f_quads, uint32_t dim, uint32_t inner) {
+  uint32_t slab, quad;
+  fd_divmod(i, f_quads, slab, quad);
+  QuadLane q;
+  q.base = static_cast<uint64_t>(slab) * dim * inner + 4 * quad;
+  q.n = min(4u, inner - 4 * quad);
+  return q;
+}
+
+template <int DMAX>
+SHDW_DEVICE void quad_load(const float* xc, const QuadLane& q, uint32_t dim, uint32_t inner, v4f (&v)[DMAX]) {
+  if (q.n == 4) {
+#pragma unroll
+    for (int c = 0; c < DMAX; ++c)
+      if (c < dim) v[c] = load4_stream_any(xc + static_cast<uint64_t>(c) * inner);
+  } else {
+#pragma unroll
+    for (int c = 0; c < DMAX; ++c) {
+      if (c < dim) {
+        v[c] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+          if (static_cast<uint32_t>(k) < q.n) v[c][k] = __builtin_nontemporal_load(xc + static_cast<uint64_t>(c) * inner + k);
+      }
+    }
+  }
+}
+
+SHDW_DEVICE void quad_store(float* at, const QuadLane& q, const v4f& r) {
+  if (q.n == 4) {
+    store4_stream_any(at, r);
+  } else {
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+      if (static_cast<uint32_t>(k) < q.n) __builtin_nontemporal_store(r[k], at + k);
+  }
+}
+
+template <int DMAX>
+__global__ __launch_bounds__(kBlock) void softmax_quads_reg_kernel(const float* x, float* y, uint32_t quads,
+                                                                    uint32_t dim, uint32_t inner, FastDiv f_quads) {
+  __shared__ uint64_t tab[32];
+  if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
+  __syncthreads();
+  const uint32_t i = xcd_contiguous(blockIdx.x, gridDim.x) * kBlock + threadIdx.x;  // neighbours share straddled lines
+  if (i >= quads) return;
+  const QuadLane q = quad_lane(i, f_quads, dim, inner);
+  v4f v[DMAX];
+  quad_load<DMAX>(x + q.base, q, dim, inner, v);
+  v4f max_val = {-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+#pragma unroll
+  for (int c = 0; c < DMAX; ++c) {
+    if (c < dim) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) max_val[k] = std_max(v[c][k], max_val[k]);
+    }
+  }
+  v4f sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c = 0; c < DMAX; ++c) {
+    if (c < dim) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        v[c][k] = libm::exact_expf(v[c][k] - max_val[k], tab);
+        sum[k] += v[c][k];
+      }
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < DMAX; ++c) {
+    if (c < dim) {
+      v4f r;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) r[k] = v[c][k] / sum[k];
+      quad_store(y + q.base + static_cast<uint64_t>(c) * inner, q, r);
+    }
+  }
+}
+
+template <int PMODE, int DMAX, int SM>
+__global__ __launch_bounds__(kBlock) void normalize_quads_reg_kernel(const float* x, float* y, uint32_t quads,
+                                                                      uint32_t dim, uint32_t inner, FastDiv f_quads,
+                                                                      float p, float eps, const float* scale) {
+  const uint32_t i = xcd_contiguous(blockIdx.x, gridDim.x) * kBlock + threadIdx.x;
+  if (i >= quads) return;
+  const QuadLane q = quad_lane(i, f_quads, dim, inner);
+  v4f v[DMAX];
+  quad_load<DMAX>(x + q.base, q, dim, inner, v);
+  double acc[4] = {0, 0, 0, 0};
+#pragma unroll
+  for (int c = 0; c < DMAX; ++c) {
+    if (c < dim) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) acc[k] += norm_term<PMODE>(v[c][k], p);
+    }
+  }
+  float div[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) div[k] = norm_finish<PMODE>(acc[k], p, eps);
+#pragma unroll
+  for (int c = 0; c < DMAX; ++c) {
+    if (c < dim) {
+      v4f r;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) r[k] = ssd_scaled<SM>(v[c][k] / div[k], scale, c);
+      quad_store(y + q.base + static_cast<uint64_t>(c) * inner, q, r);
+    }
+  }
+}
+
 // The slab in LDS holds the per-element terms (|x|, |x|^2 or |x|^p, computed by
 // all lanes); x itself is read again for the division, from L2.
 template <int PMODE, int SM = kSsdNoScale>
@@ -646,7 +770,7 @@ __global__ __launch_bounds__(kBlock) void softmax_packed_kernel(const float* x, 
   packed_stage_in(lds, x + base, sp);
   __syncthreads();
   const uint32_t q = threadIdx.x;
-  float* col = lds + fd_div(q, f_inner) * sp.pitch + (q - fd_div(q, f_inner) * sp.inner);
+  const float* col = lds + fd_div(q, f_inner) * sp.pitch + (q - fd_div(q, f_inner) * sp.inner);
   if (q < sp.ncols) {
     float m = -FLT_MAX;
 #pragma unroll 4
@@ -1095,6 +1219,75 @@ SHDW_DEVICE void rows_stage_out(const float* tile, float* ys, uint32_t cells, co
   }
 }
 
+// Softmax over rows of D = 2 .. 16 elements (two to a handful of class scores per box): a lane owns four
+// whole rows, 4 * D consecutive floats, in registers.  The wave's span moves between memory and the wave's
+// own tile in LDS as it lies, 128 bits per lane and access, and between the tile and the lanes' registers
+// with a lane's rows at a pitch of an odd number of 128-bit pieces; no divisions, no workgroup barrier
+// after the first.
+template <int D>
+__global__ __launch_bounds__(kBlock) void softmax_short_rows_kernel(const float* x, float* y, uint32_t rows) {
+  constexpr uint32_t kMine = 4 * D;                          // floats of a lane
+  constexpr uint32_t kPitch = kMine + (D % 2 == 0 ? 4 : 0);  // of the lanes in the tile
+  constexpr uint32_t kSpan = kWave * kMine;                  // floats of a wave
+  __shared__ __align__(16) float tiles[kBlock / kWave][kWave * kPitch];
+  __shared__ uint64_t tab[32];
+  if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
+  __syncthreads();  // the only one
+  const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const uint64_t total = static_cast<uint64_t>(rows) * D;
+  const uint64_t first = (static_cast<uint64_t>(blockIdx.x) * (kBlock / kWave) + wave) * kSpan;
+  if (first >= total) return;  // the whole wave
+  const uint32_t cells = static_cast<uint32_t>(min(static_cast<uint64_t>(kSpan), total - first));
+  const float* xs = x + first;
+  float* ys = y + first;
+  float* tile = tiles[wave];
+  auto place = [](uint32_t t) { return (t / kMine) * kPitch + t % kMine; };  // element t of the span in the tile
+  v4f reg[D];
+  // No branch around a load (vectors past the end re-read the tensor's first): with one, the compiler
+  // copied the whole register array at every join, 500 moves at D = 8 and 42 us per 51 MB in place of 25.
+#pragma unroll
+  for (int k = 0; k < D; ++k) {
+    const uint32_t t = 4 * (k * kWave + lane);
+    reg[k] = load4_stream_any(t + 4 <= cells ? xs + t : x);
+  }
+#pragma unroll
+  for (int k = 0; k < D; ++k) {
+    const uint32_t t = 4 * (k * kWave + lane);
+    if (t + 4 <= cells) *reinterpret_cast<v4f*>(tile + place(t)) = reg[k];
+  }
+  const uint32_t rest = (cells & ~3u) + lane;  // a span that ends the tensor may end inside a vector
+  if (lane < 3 && rest < cells) tile[place(rest)] = xs[rest];
+  __builtin_amdgcn_wave_barrier();
+  float* mine = tile + lane * kPitch;
+  // A row at a time, from and to the tile: the 4 * D exponentials of a lane side by side (each a chain of
+  // fp64 operations) would take over 200 registers at D = 8.
+#pragma unroll 1
+  for (uint32_t r = 0; r < 4; ++r) {  // rows past the end of the tensor hold what the tile held; nothing of them is stored
+    float* row = mine + r * D;
+    float e[D];
+#pragma unroll
+    for (int c = 0; c < D; ++c) e[c] = row[c];
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int c = 0; c < D; ++c) m = std_max(e[c], m);
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < D; ++c) {
+      e[c] = libm::exact_expf(e[c] - m, tab);
+      sum += e[c];
+    }
+#pragma unroll
+    for (int c = 0; c < D; ++c) row[c] = e[c] / sum;
+  }
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int k = 0; k < D; ++k) {
+    const uint32_t t = 4 * (k * kWave + lane);
+    if (t + 4 <= cells) store4_stream_any(ys + t, *reinterpret_cast<const v4f*>(tile + place(t)));
+  }
+  if (lane < 3 && rest < cells) ys[rest] = tile[place(rest)];
+}
+
 template <int TILE>
 __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const float* x, float* y, uint32_t rows, WaveRows w) {
   __shared__ __align__(16) float tiles[kBlock / kWave][TILE];
@@ -1319,6 +1512,28 @@ static void launch_normalize_rows_stream(uint32_t rows, uint32_t len, float p, f
     case 16: normalize_rows_stream_kernel<PMODE, SM, 16><<<grid, kBlock, 0, st>>>(x, y, rows, len, p, eps, scale); break;
     default: normalize_rows_stream_kernel<PMODE, SM, 4><<<grid, kBlock, 0, st>>>(x, y, rows, len, p, eps, scale);
   }
+}
+
+// Quads of positions with their columns in registers: how many there are, 0 where the quad kernels do not apply.
+constexpr int kQuadMaxDim = 4, kQuadMinInner = 16;
+constexpr int kShortRowsMaxDim = 16;  // rows of up to this many elements: four to a lane, in registers
+static uint32_t quad_count(int outer_num, int dim, int inner_num, bool softmax, FastDiv* f_quads) {
+  // Measured against the column-per-lane and packed kernels (per 51 MB): ahead where the per-column
+  // work is small against a lane's set-up, behind from five rows on (softmax [512,8,3136] 32 us against 21)
+  // and where a slab has fewer than four quads (the lanes of a wave then scatter over many lines).
+  const bool whole = inner_num % 4 == 0;
+  const bool apply = softmax ? (dim <= 3 || (dim == 4 && whole)) : (dim <= 2 && whole);
+  if (!apply || inner_num < kQuadMinInner) return 0;
+  const uint32_t per_slab = (static_cast<uint32_t>(inner_num) + 3) / 4;
+  *f_quads = make_fastdiv(per_slab);
+  return static_cast<uint32_t>(outer_num) * per_slab;  // at most the number of columns
+}
+
+template <int PMODE, int SM>
+static void launch_normalize_quads(uint32_t quads, FastDiv fq, int dim, int inner_num, float p, float eps, const float* x,
+                                   const float* scale, float* y, hipStream_t st) {
+  const uint32_t d = static_cast<uint32_t>(dim), inner = static_cast<uint32_t>(inner_num);
+  normalize_quads_reg_kernel<PMODE, kQuadMaxDim, SM><<<grid_for(quads), kBlock, 0, st>>>(x, y, quads, d, inner, fq, p, eps, scale);
 }
 
 static uint32_t rows_grid(uint32_t rows, const WaveRows& w) {
@@ -1816,6 +2031,8 @@ static uint32_t packed_group(int dim, int inner_num) {
   if (inner_num >= 64) return 0;
   const uint64_t pitch = static_cast<uint64_t>(inner_num) * (static_cast<uint32_t>(dim) | 1u);
   if (pitch * 4 > kPackedTileFloats) return 0;
+  // (more than 256 columns to a workgroup, a lane walking several, measured slower for every dim but 2:
+  // softmax over [1.6M,8]: 33 -> 48 us per 51 MB with 1024 columns)
   uint32_t group = std::min<uint32_t>(kBlock / inner_num, kPackedTileFloats / static_cast<uint32_t>(pitch));
   group &= ~3u;  // whole 128-bit pieces per workgroup
   // the walks are done by group * inner lanes: under 32 of them (rows of 512 and
@@ -1858,6 +2075,24 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
                   wave_rows<kRowsSmallTile>(dim, &w)) {
     const uint32_t rows = static_cast<uint32_t>(outer_num);
     softmax_rows_kernel<kRowsSmallTile><<<rows_grid(rows, w), kBlock, 0, st>>>(x, y, rows, w);
+    return launch_status();
+  }
+  if (inner_num == 1 && dim >= 2 && dim <= kShortRowsMaxDim && outer_num >= kRowsMinRows) {
+    const uint32_t rows = static_cast<uint32_t>(outer_num);
+    const uint64_t per_group = 4ull * kBlock;  // rows of a workgroup
+    const uint32_t grid = static_cast<uint32_t>((rows + per_group - 1) / per_group);
+    switch (dim) {
+#define SHDW_SHORT_ROWS(D) case D: softmax_short_rows_kernel<D><<<grid, kBlock, 0, st>>>(x, y, rows); break;
+      SHDW_SHORT_ROWS(2) SHDW_SHORT_ROWS(3) SHDW_SHORT_ROWS(4) SHDW_SHORT_ROWS(5) SHDW_SHORT_ROWS(6)
+      SHDW_SHORT_ROWS(7) SHDW_SHORT_ROWS(8) SHDW_SHORT_ROWS(9) SHDW_SHORT_ROWS(10) SHDW_SHORT_ROWS(11)
+      SHDW_SHORT_ROWS(12) SHDW_SHORT_ROWS(13) SHDW_SHORT_ROWS(14) SHDW_SHORT_ROWS(15) SHDW_SHORT_ROWS(16)
+#undef SHDW_SHORT_ROWS
+    }
+    return launch_status();
+  }
+  if (FastDiv fq; const uint32_t quads = quad_count(outer_num, dim, inner_num, true, &fq)) {
+    const uint32_t d = static_cast<uint32_t>(dim), inner = static_cast<uint32_t>(inner_num);
+    softmax_quads_reg_kernel<kQuadMaxDim><<<grid_for(quads), kBlock, 0, st>>>(x, y, quads, d, inner, fq);
     return launch_status();
   }
   if (const uint32_t group = packed_group(dim, inner_num)) {
@@ -1907,6 +2142,11 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
   if (mode != 0 && rows_apply(outer_num, dim, inner_num)) {
     if (mode == 1) launch_normalize_rows<1, kSsdNoScale>(outer_num, dim, p, eps, x, nullptr, y, st);
     else launch_normalize_rows<2, kSsdNoScale>(outer_num, dim, p, eps, x, nullptr, y, st);
+    return launch_status();
+  }
+  if (FastDiv fq; const uint32_t quads = mode != 0 ? quad_count(outer_num, dim, inner_num, false, &fq) : 0) {
+    if (mode == 1) launch_normalize_quads<1, kSsdNoScale>(quads, fq, dim, inner_num, p, eps, x, nullptr, y, st);
+    else launch_normalize_quads<2, kSsdNoScale>(quads, fq, dim, inner_num, p, eps, x, nullptr, y, st);
     return launch_status();
   }
   if (const uint32_t group = packed_group(dim, inner_num)) {
@@ -1987,6 +2227,10 @@ static void launch_ssd_columns(const ColumnGeometry& g, int outer_num, int dim, 
   const uint32_t grid = grid_for(g.columns);
   if (rows_apply(outer_num, dim, inner_num)) {
     launch_normalize_rows<3, SM>(outer_num, dim, 2.f, eps, x, scale, y, st);
+    return;
+  }
+  if (FastDiv fq; const uint32_t quads = quad_count(outer_num, dim, inner_num, false, &fq)) {
+    launch_normalize_quads<3, SM>(quads, fq, dim, inner_num, 2.f, eps, x, scale, y, st);
     return;
   }
   if (const uint32_t group = packed_group(dim, inner_num)) {

@@ -136,6 +136,20 @@ def test_softmax_and_normalize_over_long_rows(gpu, outer, dim):
                          oracle.ssd_normalize(x, outer, dim, 1, False, False, 1e-5, scale), "ssd normalize")
 
 
+# Rows of 2 to 16 elements over the last axis, four rows per lane: row counts that end inside a lane's four
+# rows, inside a vector and inside a wave's span; off the vector boundary in place; infinities and NaNs.
+@pytest.mark.parametrize("dim", list(range(2, 17)))
+def test_softmax_over_short_rows(gpu, dim):
+    for outer in (1024, 1027, 4099, 70001):
+        x = normal(40 + dim, outer * dim, 4.0)
+        want = oracle.softmax(x, outer, dim, 1)
+        assert_bit_exact(gpuops.softmax(x, outer, dim, 1), want, "softmax [%d,%d,1]" % (outer, dim))
+        assert_bit_exact(gpuops.softmax(x, outer, dim, 1, inplace=True, offset=1 + outer % 3), want,
+                         "softmax [%d,%d,1] in place, off the vector boundary" % (outer, dim))
+    x = with_specials(normal(41, 5003 * dim, 30.0), 41)
+    assert_bit_exact(gpuops.softmax(x, 5003, dim, 1), oracle.softmax(x, 5003, dim, 1), "softmax specials")
+
+
 @pytest.mark.parametrize("outer,dim,inner", [(40, 50, 1), (2, 12, 200), (2, 80, 100), (2, 6000, 3), (1, 700, 64),
                                              (1200, 100, 1), (1030, 1500, 1)])
 def test_softmax_special_values(gpu, outer, dim, inner):
