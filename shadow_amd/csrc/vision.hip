@@ -169,11 +169,13 @@ constexpr int kBandTileFloats = 8192;  // upper bound of the dynamic LDS tile (3
 constexpr int kBandBatch = 4;
 constexpr int kBandMaxPad = 64;        // wider clipping goes to the direct kernel
 constexpr int kPoolBandOutputs = 512;  // outputs a workgroup aims for (measured best of 256..4096)
+constexpr int kBandWideMinCols = 3;    // windows this wide at a column stride of 1: four outputs per lane
 
 struct BandArgs {
   int in_h, in_w, out_h, out_w;
   int kh, kw, sh, sw, ph, pw;
   int band, bands_per_plane, w_shift;
+  int wide;  // a lane walks four neighbouring outputs (w_shift then counts quads of outputs)
   int pad_l, pitch, tile_rows;  // data rows in the tile; the spare row is row tile_rows
   uint32_t total_bands, bands_per_group;
   FastDiv f_bands, f_in_w;
@@ -264,6 +266,82 @@ SHDW_DEVICE void band_windows(const float* tile, float* y, const BandArgs& p, co
   }
 }
 
+// Windows of three and more columns at a column stride of one: a lane takes four
+// neighbouring outputs of a row and reads the kw + 3 cells under them once per
+// window row, handing each to the outputs it belongs to, in place of 4 kw reads
+// (the walks are bound by their LDS reads: 5x5 on 112x112 planes 77 us per
+// 51 MB, 25 reads an output).  Every output still receives its cells row by
+// row and left to right.  The four outputs start at a column w with w = pw
+// (mod 4): their cells then start on a 16-byte boundary of the tile and come
+// as 128-bit reads, neighbouring lanes on neighbouring banks (single floats at
+// a lane stride of four met the same bank four at a time: 43 us).  The first
+// quad of a row may so begin left of column 0 and the last end right of
+// out_w - 1; those outputs read the padding, the next row or the eight floats
+// behind the tile, and are not stored.
+template <bool MAX, int K>
+SHDW_DEVICE void band_windows_wide(const float* tile, float* y, const BandArgs& p, const BandSpan& bs) {
+  float* dst = y + (static_cast<uint64_t>(bs.plane) * p.out_h + bs.h0) * p.out_w;
+  const int q_lanes = 1 << p.w_shift;
+  const int h_step = kBlock >> p.w_shift;
+  const int h_lane = static_cast<int>(threadIdx.x) >> p.w_shift;
+  const int spare = p.tile_rows * p.pitch;
+  const int kh = K > 0 ? K : p.kh, kw = K > 0 ? K : p.kw;
+  const int lead = p.pad_l - p.pw;  // outputs of the first quad left of column 0: 0 .. 3
+  const int quads = (p.out_w + lead + 3) >> 2;
+  for (int q = static_cast<int>(threadIdx.x) & (q_lanes - 1); q < quads; q += q_lanes) {
+    const int w = 4 * q - lead, w_first = w - p.pw;  // sw == 1; pad_l + w_first = 4 q
+    for (int hl = h_lane; hl < bs.nh; hl += h_step) {
+      const int h_first = (bs.h0 + hl) * p.sh - p.ph;
+      const int rows_pad = min(h_first + p.kh, p.in_h + p.ph) - h_first;
+      float acc[4];
+#pragma unroll
+      for (int o = 0; o < 4; ++o) acc[o] = MAX ? -FLT_MAX : 0.f;
+      for (int i = 0; i < kh; ++i) {
+        const int ri = h_first + i;
+        const int row = ri >= bs.r_lo && ri < bs.r_hi ? (ri - bs.r_lo) * p.pitch : spare;
+        const v4f* cells = reinterpret_cast<const v4f*>(tile + row + 4 * q);
+        if (K > 0) {
+          constexpr int kVecs = (K + 3 + 3) / 4;
+          float c[4 * kVecs];
+#pragma unroll
+          for (int t = 0; t < kVecs; ++t) {
+            const v4f v = cells[t];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) c[4 * t + e] = v[e];
+          }
+#pragma unroll
+          for (int j = 0; j < K; ++j) {
+#pragma unroll
+            for (int o = 0; o < 4; ++o) acc[o] = MAX ? pool_max(acc[o], c[o + j]) : acc[o] + c[o + j];
+          }
+        } else {
+          v4f cur = cells[0];
+          for (int j0 = 0; j0 < kw; j0 += 4) {
+            const v4f next = cells[(j0 >> 2) + 1];
+            float c[8] = {cur[0], cur[1], cur[2], cur[3], next[0], next[1], next[2], next[3]};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              if (j0 + j < kw) {
+#pragma unroll
+                for (int o = 0; o < 4; ++o) acc[o] = MAX ? pool_max(acc[o], c[o + j]) : acc[o] + c[o + j];
+              }
+            }
+            cur = next;
+          }
+        }
+      }
+      float* out = dst + hl * p.out_w + w;
+#pragma unroll
+      for (int o = 0; o < 4; ++o) {
+        if (w + o >= 0 && w + o < p.out_w) {
+          const int cols_pad = min(w_first + o + p.kw, p.in_w + p.pw) - (w_first + o);
+          out[o] = MAX ? acc[o] : acc[o] / static_cast<float>(rows_pad * cols_pad);
+        }
+      }
+    }
+  }
+}
+
 // A workgroup walks `bands_per_group` consecutive bands.  PIPE (every span
 // starts 16-byte aligned and in_w % 4 == 0): the next band's 128-bit loads are
 // issued into registers before the current band's windows are walked, so HBM
@@ -313,7 +391,8 @@ __global__ __launch_bounds__(kBlock) void pool_band_kernel(const float* x, float
           if (4 * v < cur.span) reg[k] = load4_stream(cur.src + 4ull * v);
         }
       }
-      band_windows<MAX, K>(tile, y, p, walk);
+      if (p.wide) band_windows_wide<MAX, K>(tile, y, p, walk);
+      else band_windows<MAX, K>(tile, y, p, walk);
       __syncthreads();  // the tile is rewritten next
     }
   } else {
@@ -333,7 +412,8 @@ __global__ __launch_bounds__(kBlock) void pool_band_kernel(const float* x, float
         }
       }
       __syncthreads();
-      band_windows<MAX, K>(tile, y, p, bs);
+      if (p.wide) band_windows_wide<MAX, K>(tile, y, p, bs);
+      else band_windows<MAX, K>(tile, y, p, bs);
       __syncthreads();
     }
   }
@@ -350,12 +430,15 @@ static bool plan_pool_band(const PoolArgs& p, int target_outputs, BandArgs* a) {
   const int rows_cap = kBandTileFloats / pitch - 1;  // one row is the spare
   if (rows_cap < p.kh) return false;
   const int band_cap = (rows_cap - p.kh) / p.sh + 1;
+  const bool wide = p.sw == 1 && p.kw >= kBandWideMinCols && p.out_w >= 16;
+  if (wide) target_outputs *= 4;
   int band = (target_outputs + p.out_w - 1) / p.out_w;
   band = band < 1 ? 1 : band;
   band = band > band_cap ? band_cap : band;
   band = band > p.out_h ? p.out_h : band;
+  const int w_units = wide ? (p.out_w + pad_l - p.pw + 3) / 4 : p.out_w;  // what a lane takes along a row
   int w_shift = 0;
-  while ((1 << w_shift) < p.out_w && w_shift < 8) ++w_shift;
+  while ((1 << w_shift) < w_units && w_shift < 8) ++w_shift;
   const int h_step = kBlock >> w_shift;  // output rows a workgroup walks at a time
   if (band > h_step && band < p.out_h) band -= band % h_step;
   a->in_h = p.in_h, a->in_w = p.in_w, a->out_h = p.out_h, a->out_w = p.out_w;
@@ -363,6 +446,7 @@ static bool plan_pool_band(const PoolArgs& p, int target_outputs, BandArgs* a) {
   a->band = band;
   a->bands_per_plane = (p.out_h + band - 1) / band;
   a->w_shift = w_shift;
+  a->wide = wide ? 1 : 0;
   a->pad_l = pad_l, a->pitch = pitch;
   a->tile_rows = min((band - 1) * p.sh + p.kh, p.in_h);
   a->f_bands = make_fastdiv(static_cast<uint32_t>(a->bands_per_plane));
@@ -959,7 +1043,7 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
   BandArgs a;
   if (!three_d && plan_pool_band(p, kPoolBandOutputs, &a)) {
     const int64_t groups = static_cast<int64_t>(in_shape[0]) * in_shape[1] * a.bands_per_plane;
-    const size_t lds = static_cast<size_t>(a.tile_rows + 1) * a.pitch * sizeof(float);
+    const size_t lds = (static_cast<size_t>(a.tile_rows + 1) * a.pitch + 8) * sizeof(float);  // eight spare: band_windows_wide
     if (groups <= INT32_MAX) {
       a.total_bands = static_cast<uint32_t>(groups);
       // Enough workgroups to fill the chip a few times over, then longer walks.
@@ -968,7 +1052,7 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
       a.bands_per_group = per;
       const uint32_t g = (a.total_bands + per - 1) / per;
       const bool pipe = p.in_w % 4 == 0 && aligned16(x);
-      const int k = p.kh == p.kw && (p.kh == 2 || p.kh == 3) ? p.kh : 0;
+      const int k = p.kh == p.kw && (p.kh == 2 || p.kh == 3 || (p.kh == 5 && a.wide)) ? p.kh : 0;
       const int vecs = (a.tile_rows * p.in_w / 4 + kBlock - 1) / kBlock;  // per lane and band
       const int regs = !pipe ? 0 : (vecs <= 2 ? 2 : (vecs <= 3 ? 3 : (vecs <= 4 ? 4 : (vecs <= 6 ? 6 : 8))));
 #define SHDW_LAUNCH_BAND(MAXV, KV)                                                              \
@@ -985,6 +1069,8 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
       if (pool_type == 0) {
         if (k == 3)
           SHDW_LAUNCH_BAND(true, 3);
+        else if (k == 5)
+          SHDW_LAUNCH_BAND(true, 5);
         else if (k == 2)
           SHDW_LAUNCH_BAND(true, 2);
         else
@@ -992,6 +1078,8 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
       } else {
         if (k == 3)
           SHDW_LAUNCH_BAND(false, 3);
+        else if (k == 5)
+          SHDW_LAUNCH_BAND(false, 5);
         else if (k == 2)
           SHDW_LAUNCH_BAND(false, 2);
         else

@@ -327,6 +327,14 @@ POOL_2D = [
     # planes of 513 to 1024 outputs: whole planes for the two-step maximum, bands for the rest
     ((2, 5, 26, 26), [13], [1], [6], False), ((1, 3, 32, 32), [5], [1], [2], False), ((2, 3, 30, 23), [9, 4], [1, 1], [4, 2], True),
     ((1, 2, 33, 32), [5], [1], [2], False),
+    # row bands at a column stride of 1, four outputs per lane: pads of 0 .. 3 (the first quad starts 0 .. 3
+    # outputs left of the row), rows that end inside a quad, the unrolled 3x3 and 5x5 and other windows,
+    # a row stride of 2, windows that overhang below and to the right
+    ((1, 3, 40, 45), [3], [1], [1], False), ((1, 2, 40, 47), [5], [1], [2], False), ((1, 2, 41, 46), [5], [1], [0], False),
+    ((2, 2, 36, 50), [5, 3], [1, 1], [2, 1], True), ((1, 2, 50, 37), [3, 7], [2, 1], [1, 3], True),
+    ((1, 3, 33, 65), [4, 6], [1, 1], [3, 3], False), ((1, 2, 70, 70), [7], [1], [3], False),
+    ((1, 1, 30, 130), [9, 5], [1, 1], [4, 2], True), ((1, 2, 112, 112), [5], [1], [2], False),
+    ((1, 1, 64, 300), [3], [1], [1], True), ((1, 2, 28, 61), [13], [1], [6], False),
 ]
 
 
@@ -345,7 +353,8 @@ def test_pooling2d_op(ws, pool, shape, kernel, stride, pad, full):
 # zeros, -inf, lowest() and NaNs show whether an implementation that folds rows first
 # returns the cell the row-major walk returns.
 @pytest.mark.parametrize("shape,kernel,pad", [((3, 4, 13, 13), [5], [2]), ((2, 3, 14, 14), [13], [6]),
-                                               ((2, 2, 19, 19), [9], [4]), ((1, 3, 56, 56), [5], [2])])
+                                               ((2, 2, 19, 19), [9], [4]), ((1, 3, 56, 56), [5], [2]),
+                                               ((1, 2, 40, 61), [7], [3]), ((1, 2, 45, 50), [3], [1])])
 def test_max_pooling_ties_and_nans_in_wide_windows(ws, shape, kernel, pad):
     rng = np.random.default_rng(31)
     pick = rng.integers(0, 6, size=shape)
@@ -414,7 +423,8 @@ def test_column_ops_on_pointers_off_the_vector_boundary(gpu, outer, dim, inner, 
     ((2, 3, 12, 12), [3], [2], [1]), ((2, 16, 56, 56), [3], [2], [0]), ((1, 3, 112, 112), [3], [2], [1]),
     ((130, 64, 7, 7), [3], [1], [1]), ((2, 8, 13, 13), [5], [1], [2]), ((1, 1, 9, 2000), [3], [1], [1]),
     ((4, 128, 7, 7), [7], [1], [0]), ((3, 5, 14, 14), [14], [1], [0]), ((20, 30, 17, 17), [17], [1], [0]),
-    ((40, 128, 16, 16), [16], [1], [0]), ((2, 3, 56, 56), [56], [1], [0]), ((2, 2, 6, 7, 8), [3], [2], [1])])
+    ((40, 128, 16, 16), [16], [1], [0]), ((2, 3, 56, 56), [56], [1], [0]), ((2, 2, 6, 7, 8), [3], [2], [1]),
+    ((1, 3, 64, 64), [5], [1], [2]), ((1, 2, 60, 44), [3], [1], [1])])
 def test_pooling_on_pointers_off_the_vector_boundary(gpu, pool, shape, kernel, stride, pad, offset):
     x = normal(32, shape, 2.0)
     want = oracle.pooling_op(x, pool, kernel, stride, pad)
