@@ -1224,8 +1224,12 @@ SHDW_DEVICE void rows_stage_out(const float* tile, float* ys, uint32_t cells, co
 // own tile in LDS as it lies, 128 bits per lane and access, and between the tile and the lanes' registers
 // with a lane's rows at a pitch of an odd number of 128-bit pieces; no divisions, no workgroup barrier
 // after the first.
+//
+// The same for slabs of D = dim * inner floats with inner > 1 (two classes over a few positions or anchors
+// per cell): a lane owns four slabs and walks their inner columns one after the other, at a stride of inner.
 template <int D>
-__global__ __launch_bounds__(kBlock) void softmax_short_rows_kernel(const float* x, float* y, uint32_t rows) {
+__global__ __launch_bounds__(kBlock) void softmax_short_rows_kernel(const float* x, float* y, uint32_t rows,
+                                                                     uint32_t dim, uint32_t inner) {
   constexpr uint32_t kMine = 4 * D;                          // floats of a lane
   constexpr uint32_t kPitch = kMine + (D % 2 == 0 ? 4 : 0);  // of the lanes in the tile
   constexpr uint32_t kSpan = kWave * kMine;                  // floats of a wave
@@ -1264,6 +1268,21 @@ __global__ __launch_bounds__(kBlock) void softmax_short_rows_kernel(const float*
 #pragma unroll 1
   for (uint32_t r = 0; r < 4; ++r) {  // rows past the end of the tensor hold what the tile held; nothing of them is stored
     float* row = mine + r * D;
+    if (inner != 1) {
+      for (uint32_t s = 0; s < inner; ++s) {
+        float* col = row + s;
+        float m = -FLT_MAX;
+        for (uint32_t c = 0; c < dim; ++c) m = std_max(col[c * inner], m);
+        float sum = 0.f;
+        for (uint32_t c = 0; c < dim; ++c) {
+          const float v = libm::exact_expf(col[c * inner] - m, tab);
+          col[c * inner] = v;
+          sum += v;
+        }
+        for (uint32_t c = 0; c < dim; ++c) col[c * inner] = col[c * inner] / sum;
+      }
+      continue;
+    }
     float e[D];
 #pragma unroll
     for (int c = 0; c < D; ++c) e[c] = row[c];
@@ -1516,7 +1535,8 @@ static void launch_normalize_rows_stream(uint32_t rows, uint32_t len, float p, f
 
 // Quads of positions with their columns in registers: how many there are, 0 where the quad kernels do not apply.
 constexpr int kQuadMaxDim = 4, kQuadMinInner = 16;
-constexpr int kShortRowsMaxDim = 16;  // rows of up to this many elements: four to a lane, in registers
+constexpr int kShortRowsMaxDim = 16;  // rows of up to this many elements: four to a lane
+constexpr int kShortSlabMax = 9;      // slabs of dim * inner floats, inner > 1, likewise
 static uint32_t quad_count(int outer_num, int dim, int inner_num, bool softmax, FastDiv* f_quads) {
   // Measured against the column-per-lane and packed kernels (per 51 MB): ahead where the per-column
   // work is small against a lane's set-up, behind from five rows on (softmax [512,8,3136] 32 us against 21)
@@ -2077,12 +2097,16 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
     softmax_rows_kernel<kRowsSmallTile><<<rows_grid(rows, w), kBlock, 0, st>>>(x, y, rows, w);
     return launch_status();
   }
-  if (inner_num == 1 && dim >= 2 && dim <= kShortRowsMaxDim && outer_num >= kRowsMinRows) {
+  // slabs with inner > 1 walk their columns in loops, one exponential after the other: ahead of the packed
+  // kernel up to nine floats ([3.2M,2,2] 58 -> 27 us per 51 MB, [1.4M,3,3] 40 -> 34), behind from twelve on
+  if (dim >= 2 && inner_num <= kShortSlabMax / 2 && dim * inner_num <= (inner_num == 1 ? kShortRowsMaxDim : kShortSlabMax) &&
+      outer_num >= kRowsMinRows) {
     const uint32_t rows = static_cast<uint32_t>(outer_num);
-    const uint64_t per_group = 4ull * kBlock;  // rows of a workgroup
+    const uint64_t per_group = 4ull * kBlock;  // rows (slabs) of a workgroup
     const uint32_t grid = static_cast<uint32_t>((rows + per_group - 1) / per_group);
-    switch (dim) {
-#define SHDW_SHORT_ROWS(D) case D: softmax_short_rows_kernel<D><<<grid, kBlock, 0, st>>>(x, y, rows); break;
+    const uint32_t d = static_cast<uint32_t>(dim), inner = static_cast<uint32_t>(inner_num);
+    switch (dim * inner_num) {
+#define SHDW_SHORT_ROWS(D) case D: softmax_short_rows_kernel<D><<<grid, kBlock, 0, st>>>(x, y, rows, d, inner); break;
       SHDW_SHORT_ROWS(2) SHDW_SHORT_ROWS(3) SHDW_SHORT_ROWS(4) SHDW_SHORT_ROWS(5) SHDW_SHORT_ROWS(6)
       SHDW_SHORT_ROWS(7) SHDW_SHORT_ROWS(8) SHDW_SHORT_ROWS(9) SHDW_SHORT_ROWS(10) SHDW_SHORT_ROWS(11)
       SHDW_SHORT_ROWS(12) SHDW_SHORT_ROWS(13) SHDW_SHORT_ROWS(14) SHDW_SHORT_ROWS(15) SHDW_SHORT_ROWS(16)

@@ -150,6 +150,18 @@ def test_softmax_over_short_rows(gpu, dim):
     assert_bit_exact(gpuops.softmax(x, 5003, dim, 1), oracle.softmax(x, 5003, dim, 1), "softmax specials")
 
 
+# Slabs of dim * inner <= 9 floats with inner > 1 go the same way, four slabs per lane; the next larger ones.
+@pytest.mark.parametrize("outer,dim,inner", [(5003, 2, 2), (4099, 2, 4), (1027, 3, 3), (70001, 4, 2), (1500, 3, 2),
+                                             (1029, 2, 3), (2001, 5, 2), (1025, 3, 4), (1024, 2, 7), (33333, 7, 2)])
+def test_softmax_over_short_slabs(gpu, outer, dim, inner):
+    x = normal(43, outer * dim * inner, 4.0)
+    want = oracle.softmax(x, outer, dim, inner)
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner), want, "softmax")
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner, inplace=True, offset=3), want, "softmax in place, off the vector boundary")
+    x = with_specials(normal(44, outer * dim * inner, 30.0), 44)
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax specials")
+
+
 @pytest.mark.parametrize("outer,dim,inner", [(40, 50, 1), (2, 12, 200), (2, 80, 100), (2, 6000, 3), (1, 700, 64),
                                              (1200, 100, 1), (1030, 1500, 1)])
 def test_softmax_special_values(gpu, outer, dim, inner):
