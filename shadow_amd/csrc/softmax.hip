@@ -1855,7 +1855,7 @@ struct LongSlab {
 __global__ __launch_bounds__(kBlock) void softmax_long_slab_kernel(const float* x, float* y, uint32_t dim,
                                                                     FastDiv f_inner) {
   __shared__ __align__(16) float chunk[2][kTallChunkFloats];
-  __shared__ float stat[kTallMinInner];
+  __shared__ float stat[kBlock];
   __shared__ uint64_t tab[32];
   if (threadIdx.x < 32) tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
   const LongSlab t(x, y, dim, f_inner.d);
@@ -1950,7 +1950,7 @@ __global__ __launch_bounds__(kBlock) void normalize_long_slab_kernel(const float
                                                                       FastDiv f_inner, float p, float eps,
                                                                       const float* scale) {
   __shared__ __align__(16) float chunk[2][kTallChunkFloats];
-  __shared__ float stat[kTallMinInner];
+  __shared__ float stat[kBlock];
   const LongSlab t(x, y, dim, f_inner.d);
   const uint32_t chunks = t.chunks(), inner = t.inner;
   uint32_t pos[kLongLoads][4], row[kLongLoads][4];  // position and row inside a chunk of the lane's elements
@@ -2007,9 +2007,18 @@ __global__ __launch_bounds__(kBlock) void normalize_long_slab_kernel(const float
 // stay whole in LDS: softmax_slab_kernel, normalize_slab_kernel).
 constexpr int64_t kLongSlabMinFloats = kSlabMaxFloats;
 
-static bool long_slab(int dim, int inner_num) {
-  return static_cast<uint32_t>(inner_num) < kTallMinInner &&
-         static_cast<int64_t>(dim) * inner_num > kLongSlabMinFloats;
+// ... and where inner >= 16 with a few hundred slabs to hand out, one per workgroup: rows that do not
+// start on 64-byte boundaries (inner not a multiple of 16) cost the tall and tile kernels, which cut every
+// row into pieces of 16 to 64 positions, up to half their speed, and the slab moves as it lies
+// ([513,1000,25] softmax 101 -> 68 us per 51 MB, normalize 76 -> 45; [511,513,49] 79 -> 56, 55 -> 37).
+// Normalize gains on aligned rows too ([782,513,32] 46 -> 36); Softmax does not ([782,513,32] 59 -> 71).
+constexpr int kLongSlabMinSlabs = 192, kLongSlabMinSlabsAligned = 384;
+static bool long_slab(int outer_num, int dim, int inner_num, bool softmax) {
+  if (static_cast<int64_t>(dim) * inner_num <= kLongSlabMinFloats) return false;
+  if (static_cast<uint32_t>(inner_num) < kTallMinInner) return true;
+  if (inner_num > kBlock) return false;  // a lane per position walks the sums
+  if (inner_num % 16 != 0) return outer_num >= kLongSlabMinSlabs;
+  return !softmax && outer_num >= kLongSlabMinSlabsAligned;
 }
 
 // Where the tall kernels apply, and their launch: positions per workgroup as wide
@@ -2123,7 +2132,7 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
     const uint32_t slabs = static_cast<uint32_t>(outer_num);
     softmax_packed_kernel<<<(slabs + group - 1) / group, kBlock, packed_bytes(dim, inner_num, group), st>>>(
         x, y, slabs, static_cast<uint32_t>(dim), fi, make_fastdiv(static_cast<uint32_t>(dim) * inner_num), group);
-  } else if (long_slab(dim, inner_num))
+  } else if (long_slab(outer_num, dim, inner_num, true))
     softmax_long_slab_kernel<<<outer_num, kBlock, 0, st>>>(x, y, static_cast<uint32_t>(dim), fi);
   else if (g.use_slab)
     softmax_slab_kernel<<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, static_cast<uint32_t>(dim), fi);
@@ -2184,7 +2193,7 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
       normalize_packed_kernel<2, kSsdNoScale><<<grid, kBlock, bytes, st>>>(x, y, slabs, d, fi, fs, group, p, eps, nullptr);
     else
       normalize_packed_kernel<0, kSsdNoScale><<<grid, kBlock, bytes, st>>>(x, y, slabs, d, fi, fs, group, p, eps, nullptr);
-  } else if (long_slab(dim, inner_num)) {
+  } else if (long_slab(outer_num, dim, inner_num, false)) {
     if (mode == 1)
       normalize_long_slab_kernel<1, kSsdNoScale><<<outer_num, kBlock, 0, st>>>(x, y, d, fi, p, eps, nullptr);
     else if (mode == 2)
@@ -2261,7 +2270,7 @@ static void launch_ssd_columns(const ColumnGeometry& g, int outer_num, int dim, 
     const uint32_t slabs = static_cast<uint32_t>(outer_num);
     normalize_packed_kernel<3, SM><<<(slabs + group - 1) / group, kBlock, packed_bytes(dim, inner_num, group), st>>>(
         x, y, slabs, d, fi, make_fastdiv(d * inner_num), group, 2.f, eps, scale);
-  } else if (long_slab(dim, inner_num))
+  } else if (long_slab(outer_num, dim, inner_num, false))
     normalize_long_slab_kernel<3, SM><<<outer_num, kBlock, 0, st>>>(x, y, d, fi, 2.f, eps, scale);
   else if (g.use_slab)
     normalize_slab_kernel<3, SM><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, 2.f, eps, scale);

@@ -117,6 +117,27 @@ def test_softmax(gpu, outer, dim, inner):
     assert_bit_exact(gpuops.softmax(x, outer, dim, inner, inplace=True), want, "softmax in place")
 
 
+# Slabs of more than 60 KB over 16 to 256 positions with a few hundred slabs to hand out, a workgroup per slab
+# in chunks of whole rows: positions that are and are not multiples of 16 (Softmax takes only the latter),
+# one row per chunk, the slab counts either side of where the form starts.
+@pytest.mark.parametrize("outer,dim,inner", [(192, 700, 25), (200, 350, 49), (193, 160, 100), (192, 65, 255),
+                                             (384, 61, 256), (400, 130, 128), (191, 700, 25), (383, 130, 128),
+                                             (200, 1000, 17), (385, 500, 32), (192, 61, 257)])
+def test_column_ops_over_long_slabs_of_many_positions(gpu, outer, dim, inner):
+    x = normal(45, outer * dim * inner, 4.0)
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax")
+    for p in (1.0, 2.0, 2.5):
+        assert_bit_exact(gpuops.normalize(x, outer, dim, inner, p, 1e-12), oracle.normalize(x, outer, dim, inner, p, 1e-12),
+                         "normalize p=%g" % p)
+    assert_bit_exact(gpuops.normalize(x, outer, dim, inner, 2.0, 1e-12, inplace=True, offset=1),
+                     oracle.normalize(x, outer, dim, inner, 2.0, 1e-12), "normalize in place, off the vector boundary")
+    scale = uniform(46, dim, 0.5, 2.0)
+    assert_bit_exact(gpuops.ssd_normalize(x, outer, dim, inner, False, False, 1e-5, scale),
+                     oracle.ssd_normalize(x, outer, dim, inner, False, False, 1e-5, scale), "ssd normalize")
+    z = with_specials(x.copy(), 47)
+    assert_bit_exact(gpuops.softmax(z, outer, dim, inner), oracle.softmax(z, outer, dim, inner), "softmax specials")
+
+
 # Long rows over the last axis: Normalize moves along 4, 8, 16, 32 or 64 rows per wave by the number and the
 # length of the rows (whole and cut chunks, a cut last vector, a last wave with rows missing); Softmax has
 # the rows in LDS up to 1023 elements and a workgroup per row beyond.
