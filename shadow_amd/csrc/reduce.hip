@@ -254,12 +254,74 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_lds_kernel(const float* x,
 }
 
 // ---------------------------------------------------------------------------
+// rows of D = 2 .. 7 floats (pairs, 2x2 windows): with a lane per row
+// a workgroup of the kernel above has 2 KB to work on and its barrier to pay
+// (sum over [6.4M][2]: 24 us per 51 MB, 13 us here).  Here a lane owns four whole rows, 4 D
+// consecutive floats.  The wave's span moves from memory into the wave's own
+// LDS tile as it lies, 128 bits per lane and access, and a lane reads its rows
+// back at a pitch of an odd number of 128-bit pieces; no workgroup barrier.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kTinyRowMaxLen = 7;  // rows of 8: 10.9 us here, 10.3 us with a lane per row from LDS
+
+template <int OP, int D>
+__global__ __launch_bounds__(kBlock) void reduce_rows_tiny_kernel(const float* x, float* y, uint32_t rows,
+                                                                   Partial* part, Lead ld) {
+  constexpr uint32_t kMine = 4 * D;                          // floats of a lane
+  constexpr uint32_t kPitch = kMine + (D % 2 == 0 ? 4 : 0);  // of the lanes in the tile
+  constexpr uint32_t kSpan = kWave * kMine;                  // floats of a wave
+  __shared__ __align__(16) float tiles[kBlock / kWave][kWave * kPitch];
+  const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const uint64_t total = static_cast<uint64_t>(rows) * D;
+  const uint64_t wave_index = static_cast<uint64_t>(blockIdx.x) * (kBlock / kWave) + wave;
+  const uint64_t first = wave_index * kSpan;
+  if (first >= total) return;  // the whole wave
+  const uint32_t cells = static_cast<uint32_t>(min(static_cast<uint64_t>(kSpan), total - first));
+  const float* xs = x + first;
+  float* tile = tiles[wave];
+  auto place = [](uint32_t t) { return (t / kMine) * kPitch + t % kMine; };  // element t of the span in the tile
+  v4f reg[D];
+  // no branch around a load: vectors past the end re-read the tensor's first (rows * D >= 4 here)
+#pragma unroll
+  for (int k = 0; k < D; ++k) {
+    const uint32_t t = 4 * (k * kWave + lane);
+    reg[k] = load4_stream_any(t + 4 <= cells ? xs + t : x);
+  }
+#pragma unroll
+  for (int k = 0; k < D; ++k) {
+    const uint32_t t = 4 * (k * kWave + lane);
+    if (t + 4 <= cells) *reinterpret_cast<v4f*>(tile + place(t)) = reg[k];
+  }
+  const uint32_t rest = (cells & ~3u) + lane;  // a span that ends the tensor may end inside a vector
+  if (lane < 3 && rest < cells) tile[place(rest)] = xs[rest];
+  __builtin_amdgcn_wave_barrier();
+  const float* mine = tile + lane * kPitch;
+#pragma unroll
+  for (int k = 0; k < D; ++k) reg[k] = *reinterpret_cast<const v4f*>(mine + 4 * k);
+  const uint64_t row0 = wave_index * (4 * kWave) + 4 * lane;
+  Acc<OP> acc[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    acc[r].init();
+#pragma unroll
+    for (int c = 0; c < D; ++c) acc[r].add(reg[(r * D + c) / 4][(r * D + c) % 4], c);
+  }
+  if (ld.count == 1 && row0 + 4 <= rows) {  // the lane's four results as one 128-bit store
+    store4_stream_any(y + row0, v4f{acc[0].finalize(D), acc[1].finalize(D), acc[2].finalize(D), acc[3].finalize(D)});
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (row0 + r < rows) emit_row(ld, acc[r], static_cast<uint32_t>(row0 + r), 0, 1, D, y, part);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // strided over a short reduced extent (a sum over a batch of 8, a max over 4
 // maps): the column-tile kernels below give a tile 16 or more row groups and an
 // LDS fold, which rows this few leave idle ([4][3.2M]: sum 32 us, max 71 us per
-// 51 MB).  Here a lane owns four neighbouring columns (one, where the column
-// count is no multiple of four) and walks the rows itself, eight loads in
-// flight; nothing is exchanged.
+// 51 MB).  Here a lane owns four neighbouring columns (the last lane of a row
+// the one to three that are left; one column where there are fewer than four),
+// 128-bit loads on whatever dword address the rows start, and walks the rows
+// itself, eight loads in flight; nothing is exchanged.
 // ---------------------------------------------------------------------------
 constexpr uint32_t kShortStridedMaxReduce = 32;
 
@@ -277,10 +339,17 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_short_kernel(const floa
   Acc<OP> acc[W];
 #pragma unroll
   for (int j = 0; j < W; ++j) acc[j].init();
+  // columns of the lane that exist: four, or fewer in the last unit of a row that is no multiple of four long
+  const uint32_t n = VEC ? min(4u, inner - 4 * c) : 1u;
   auto fetch = [&](uint32_t r) -> v4f {
     const float* src = p + static_cast<uint64_t>(r) * inner;
-    if (VEC) return load4_stream_any(src);
-    return v4f{__builtin_nontemporal_load(src), 0.f, 0.f, 0.f};
+    if (!VEC) return v4f{__builtin_nontemporal_load(src), 0.f, 0.f, 0.f};
+    if (n == 4) return load4_stream_any(src);  // any dword address: rows need not be whole vectors
+    v4f v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+      if (static_cast<uint32_t>(j) < n) v[j] = __builtin_nontemporal_load(src + j);
+    return v;
   };
   uint32_t r = 0;
   for (; r + 8 <= reduce; r += 8) {
@@ -305,7 +374,8 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_short_kernel(const floa
   }
   if (ld.count != 1) {
 #pragma unroll
-    for (int j = 0; j < W; ++j) emit_column(ld, acc[j], o, c * W + j, inner, 0, 1, outputs, reduce, y, part);
+    for (int j = 0; j < W; ++j)
+      if (static_cast<uint32_t>(j) < n) emit_column(ld, acc[j], o, c * W + j, inner, 0, 1, outputs, reduce, y, part);
     return;
   }
   float* dst = y + static_cast<uint64_t>(o) * inner + static_cast<uint64_t>(c) * W;
@@ -313,7 +383,13 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_short_kernel(const floa
     v4f out;
 #pragma unroll
     for (int j = 0; j < W; ++j) out[j] = acc[j].finalize(reduce);
-    *reinterpret_cast<v4f_unaligned*>(dst) = out;
+    if (n == 4) {
+      *reinterpret_cast<v4f_unaligned*>(dst) = out;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 3; ++j)
+        if (static_cast<uint32_t>(j) < n) dst[j] = out[j];
+    }
   } else {
     dst[0] = acc[0].finalize(reduce);
   }
@@ -797,6 +873,17 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
     const uint32_t reduce = static_cast<uint32_t>(pl.reduce);
     // 128-bit loads on any dword address: rows need not start 16-byte aligned.
     const bool vec = reduce >= 4;
+    if (pl.wave_per_row && reduce >= 2 && reduce <= kTinyRowMaxLen && rows >= 4096) {
+      const uint32_t grid = static_cast<uint32_t>((static_cast<uint64_t>(rows) + 4 * kBlock - 1) / (4 * kBlock));
+      switch (reduce) {
+#define SHDW_TINY(DV) case DV: reduce_rows_tiny_kernel<OP, DV><<<grid, kBlock, 0, st>>>(x, y, rows, part, ld); break;
+        SHDW_TINY(2) SHDW_TINY(3) SHDW_TINY(4) SHDW_TINY(5) SHDW_TINY(6) SHDW_TINY(7)
+#undef SHDW_TINY
+      }
+      const int rc = launch_status();
+      if (rc != SHDW_OK || slots == 1) return rc;
+      return run_stage2<OP>(part, y, outputs, slots, slots, 1, window, st);
+    }
     if (pl.wave_per_row && reduce < kShortRowMaxLen) {
       const uint32_t want = (reduce + 15) / 16;  // lanes for pieces of at most 16 elements (17 where that is even)
       const uint32_t lanes = want <= 1 ? 1 : (want <= 2 ? 2 : (want <= 4 ? 4 : (want <= 8 ? 8 : 16)));
@@ -859,8 +946,13 @@ static int run_reduce(const ReducePlan& pl, const float* x, float* y, void* work
   if (nested) ld.count = 0;
   const uint32_t rows_per_split = (reduce + splits - 1) / splits;
   if (pl.flat_period == 0 && splits == 1 && reduce <= kShortStridedMaxReduce) {
-    const bool vec = inner % 4 == 0;
-    const uint32_t per_outer = vec ? inner / 4 : inner;
+    // rows that are no whole vectors long: four columns per lane where a column per lane would have under
+    // eight loads in flight (sum over 3 of [3][4.3M]: 17.5 -> 13.2 us per 51 MB; over 12 or 17 rows the
+    // 128-bit loads off their alignment cost more than they bring, 11.5 -> 13.6 and 15.4 us) and the rows
+    // are 64 columns and more (below, the lanes of a row's cut end scatter: max over 7 of [262144][7][7]
+    // 24 us with a column per lane, 78 us with four)
+    const bool vec = inner % 4 == 0 || (inner >= 64 && reduce < 8);
+    const uint32_t per_outer = vec ? (inner + 3) / 4 : inner;
     const uint32_t units = outer * per_outer;  // <= outputs
     const FastDiv f = make_fastdiv(per_outer);
     if (vec) reduce_strided_short_kernel<OP, true><<<grid_for(units), kBlock, 0, st>>>(x, y, reduce, inner, units, f, part, view, ld);

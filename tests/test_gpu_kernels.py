@@ -315,6 +315,14 @@ REDUCE_CASES = [
     # two to seven columns with slabs of a step and more: the flat walk
     ([3, 1024, 7], [1]), ([5, 700, 2], [1]), ([2, 9000, 3], [1]), ([4, 300, 5], [1]), ([2, 171, 6], [1]), ([3, 170, 6], [1]),
     ([2, 3, 600, 7], [0, 2]),
+    # 4096 and more rows of 2 .. 7 (and 8, the first length past it): four rows per lane; row counts that end inside a lane's rows, a vector, a
+    # wave's span; the same behind a reduced leading dim (partials, second stage)
+    ([4096, 2], [1]), ([4099, 3], [1]), ([5001, 4], [1]), ([70001, 5], [1]), ([4097, 6], [1]), ([9999, 7], [1]),
+    ([4098, 8], [1]), ([1300, 5, 2, 2], [2, 3]), ([3, 5000, 4], [0, 2]), ([2, 4100, 2, 3], [0, 2, 3]),
+    # under eight rows over a strided axis whose rows are no whole vectors: four columns per lane on any
+    # dword address, the row's cut end (1 to 3 columns) float by float; 63 and 64 columns either side of it
+    ([3, 1001], [0]), ([2, 5, 66], [1]), ([7, 130003], [0]), ([4, 2, 65], [1]), ([3, 6, 63], [1]), ([2, 3, 64], [1]),
+    ([5, 3, 777], [0, 1]), ([6, 4, 3, 67], [0, 2]),
 ]
 
 
