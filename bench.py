@@ -417,6 +417,64 @@ def sweep(dev):
         n = int(np.prod(shape))
         us = tm(lambda k: lib.shdw_hip_permute(len(shape), I(shape), I(order), X[k].ptr, Y[k].ptr, st))
         show("permute", "%s order %s" % (shape, order), us, 8 * n)
+    # the channel-parameter operators at row lengths that are and are not whole vectors
+    for inner in (1, 2, 3, 7, 16, 49, 196, 3136):
+        for ch in (3, 64, 1000):
+            n = (N // (ch * inner)) * ch * inner
+            us = tm(lambda k: lib.shdw_hip_batch_norm(n, ch, inner, X[k].ptr, Q.ptr, P.ptr, 1.0, 1e-5, Y[k].ptr, st))
+            show("batch norm", "%d channels, inner %d" % (ch, inner), us, 8 * n)
+            us = tm(lambda k: lib.shdw_hip_prelu(n, ch, inner, 0, X[k].ptr, P.ptr, Y[k].ptr, st))
+            show("prelu", "%d channels, inner %d" % (ch, inner), us, 8 * n)
+    for inner in (1, 3, 16, 49, 196, 3136, 50176):
+        rows = N // inner
+        us = tm(lambda k: lib.shdw_hip_axpy_rows(rows, inner, P.ptr, X[k].ptr, X[(k + 1) % SETS].ptr, Y[k].ptr, st))
+        show("axpy rows", "[%d,%d]" % (rows, inner), us, 12 * rows * inner + 4 * rows)
+    for k_in in (2, 3, 5):
+        m = N // 2
+        ptrs = (ctypes.c_void_p * k_in)(*[X[j % SETS].ptr + (4 * m if j >= SETS else 0) for j in range(k_in)])
+        for op, nm in ((0, "prod"), (1, "sum"), (2, "max")):
+            coeff = (ctypes.c_float * k_in)(*[0.5 + 0.25 * j for j in range(k_in)]) if op == 1 else None
+            us = tm(lambda k: lib.shdw_hip_eltwise(op, k_in, ptrs, coeff, m, Y[k].ptr, st))
+            show("eltwise", "%s of %d inputs" % (nm, k_in), us, 4 * m * (k_in + 1))
+    # Concat / Slice / Stack chunks: rows of `chunk` floats copied into rows of a different pitch
+    for chunk, dst_pitch, off in ((1, 2, 1), (3, 7, 2), (49, 98, 49), (100, 300, 100), (3136, 6272, 3136), (12544, 12545, 1),
+                                  (401408, 802816, 0), (200704 * 3, 200704 * 4, 200704)):
+        outer = min(N // chunk, N // dst_pitch)
+        us = tm(lambda k: lib.shdw_hip_copy_chunks(outer, chunk, X[k].ptr, chunk, 0, Y[k].ptr, dst_pitch, off, st))
+        show("copy chunks", "%d chunks of %d into rows of %d at %d (concat)" % (outer, chunk, dst_pitch, off), us, 8 * outer * chunk)
+        us = tm(lambda k: lib.shdw_hip_copy_chunks(outer, chunk, X[k].ptr, dst_pitch, off, Y[k].ptr, chunk, 0, st))
+        show("copy chunks", "%d chunks of %d out of rows of %d at %d (slice)" % (outer, chunk, dst_pitch, off), us, 8 * outer * chunk)
+    for shape, pads in (([64, 64, 54, 54], [1, 1, 1, 1]), ([64, 64, 50, 50], [3, 3, 3, 3]), ([256, 64, 27, 27], [0, 1, 0, 1]),
+                        ([64, 64, 56, 56], [-1, -1, -1, -1]), ([2400, 64, 7, 7], [1, 1, 1, 1]), ([16, 3, 500, 501], [2, 1, 3, 0])):
+        n_in = int(np.prod(shape))
+        n_out = shape[0] * shape[1] * (shape[2] + pads[0] + pads[1]) * (shape[3] + pads[2] + pads[3])
+        assert n_in <= N and n_out <= N
+        us = tm(lambda k: lib.shdw_hip_pad(I(shape), I(pads), 0.5, X[k].ptr, Y[k].ptr, st))
+        show("pad", "%s by %s" % (shape, pads), us, 4 * (min(n_in, n_out) + n_out))
+    for shape, out_hw in (([64, 64, 28, 28], (56, 56)), ([64, 64, 28, 28], (55, 57)), ([64, 64, 56, 56], (28, 28)),
+                          ([16, 3, 300, 300], (513, 513)), ([256, 256, 7, 7], (14, 14)), ([8, 255, 19, 19], (76, 76)),
+                          ([4, 3, 720, 1280], (360, 640))):
+        out = shape[:2] + list(out_hw)
+        n_in, n_out = int(np.prod(shape)), int(np.prod(out))
+        assert n_in <= N and n_out <= N
+        for typ, nm in ((0, "nearest"), (1, "bilinear")):
+            us = tm(lambda k: lib.shdw_hip_resize(I(shape), I(out), typ, 0, X[k].ptr, Y[k].ptr, st))
+            show("resize", "%s %s -> %dx%d" % (nm, shape, out_hw[0], out_hw[1]), us, 4 * (min(n_in, 4 * n_out) + n_out))
+    for shape, stride in (([64, 64, 56, 56], 2), ([138, 64, 38, 38], 2), ([64, 16, 112, 112], 4), ([36, 512, 26, 26], 2)):
+        n = int(np.prod(shape))
+        for typ, nm in ((0, "darknet"), (1, "natural")):
+            us = tm(lambda k: lib.shdw_hip_reorg(I(shape), typ, stride, X[k].ptr, Y[k].ptr, st))
+            show("reorg", "%s %s stride %d" % (nm, shape, stride), us, 8 * n)
+    for batch, ch, sp, group in ((64, 256, 784, 2), (1120, 232, 49, 2), (15000, 116, 7, 4), (8, 480, 3136, 3), (50176, 256, 1, 8)):
+        n = batch * ch * sp
+        assert n <= N
+        us = tm(lambda k: lib.shdw_hip_shuffle_channel(batch, ch, sp, group, X[k].ptr, Y[k].ptr, st))
+        show("shuffle", "[%d,%d,%d] in %d groups" % (batch, ch, sp, group), us, 8 * n)
+    idx_host = np.arange(0, 1000, 3, dtype=np.int32)
+    idx = dev.buf(idx_host.view(np.float32))
+    for outer, inner in ((12, 1000), (1, 12845), (12845, 1), (256, 49), (3000, 4)):
+        us = tm(lambda k: lib.shdw_hip_gather(outer, 1000, inner, idx_host.size, idx.ptr, X[k].ptr, Y[k].ptr, st))
+        show("gather", "%d of 1000 rows of %d, %d times" % (idx_host.size, inner, outer), us, 8 * outer * idx_host.size * inner)
     print("worst of each family:")
     for family, (ratio, name) in worst.items():
         print("  %-14s %6.2f x copy  (%s)" % (family, ratio, name))

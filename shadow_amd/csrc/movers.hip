@@ -41,11 +41,34 @@ __global__ __launch_bounds__(kStream) void copy_chunks_kernel(const float* src, 
     dst[d] = src[s];
 }
 
+// Chunks, pitches or offsets that are no whole vectors (rows of 49, a pitch of 12545): a lane still
+// moves four floats of its chunk with 128-bit accesses, on whatever dword address they lie, and the
+// last lane of a chunk the chunk % 4 floats that remain (one float per lane: 46 us per 51 MB for chunks
+// of 12544 at a pitch of 12545, 24 us for chunks of 49).
+__global__ __launch_bounds__(kStream) void copy_chunks_any_kernel(const float* src, float* dst, uint32_t work,
+                                                                  uint32_t chunk, FastDiv f_units,
+                                                                  uint32_t src_pitch, uint32_t src_off,
+                                                                  uint32_t dst_pitch, uint32_t dst_off) {
+  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
+  if (i >= work) return;
+  uint32_t n, p;
+  fd_divmod(i, f_units, n, p);
+  const uint32_t first = 4 * p;
+  const float* s = src + static_cast<uint64_t>(n) * src_pitch + src_off + first;
+  float* d = dst + static_cast<uint64_t>(n) * dst_pitch + dst_off + first;
+  if (first + 4 <= chunk) {
+    store4_stream_any(d, load4_stream_any(s));
+  } else {
+    for (uint32_t j = 0; first + j < chunk; ++j) d[j] = s[j];
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Rows of `inner` elements picked by a table: Gather (device index table) and
 // ShuffleChannel (closed-form source row).
 // ---------------------------------------------------------------------------
 struct GatherRows {
+  static constexpr bool kFlat = false;
   const int* indexes;
   FastDiv f_num;  // rows per outer slice on the output side
   uint32_t gather_dim;
@@ -60,6 +83,7 @@ struct GatherRows {
 };
 
 struct ShuffleRows {
+  static constexpr bool kFlat = true;
   FastDiv f_channel, f_group;
   uint32_t group_column;
   SHDW_DEVICE int64_t source(uint32_t r) const {
@@ -87,6 +111,9 @@ __global__ __launch_bounds__(kStream) void rows_pick_kernel(MAP map, const float
 // Rows of any length on any dword address: a lane moves the vector at floats
 // 4p .. 4p + 3 of its row with 128-bit accesses, the last lane of a row the
 // inner % 4 floats that remain (rows of 49 ran 2.2x slower with one float per lane).
+// Gather keeps this form: its source rows come from a table in memory, and a lane
+// that looks up a row per element (below) waits for one dependent load after the
+// other (rows of 1: 17 us against 30 us per 17 MB gathered).
 template <class MAP>
 __global__ __launch_bounds__(kStream) void rows_pick_any_kernel(MAP map, const float* x, float* y,
                                                                 uint32_t work, uint32_t inner,
@@ -107,12 +134,53 @@ __global__ __launch_bounds__(kStream) void rows_pick_any_kernel(MAP map, const f
   }
 }
 
+// Rows of any length on any dword address: a lane owns four consecutive floats of the
+// OUTPUT, one 128-bit store.  Where they lie in one output row (most do, from rows of a
+// dozen floats on) they are four consecutive floats of one source row as well, one
+// 128-bit load; a vector that runs over the end of its row takes its floats one by
+// one, each from the row it belongs to.  For maps that are arithmetic only
+// (ShuffleChannel; with four floats of a row per lane, above, rows of 49 ran at 1.8 x,
+// rows of 7 at 3.1 x and rows of 1 at 2.7 x the time of a copy; here 1.4, 2.0, 1.1).
+template <class MAP>
+__global__ __launch_bounds__(kStream) void rows_pick_flat_kernel(MAP map, const float* x, float* y,
+                                                                 uint32_t n4, uint32_t n, FastDiv f_inner) {
+  const uint32_t i = blockIdx.x * kStream + threadIdx.x;
+  const uint32_t inner = f_inner.d;
+  if (i < n4) {
+    uint32_t r, p;
+    fd_divmod(4 * i, f_inner, r, p);
+    int64_t s = map.source(r);
+    v4f v;
+    if (p + 4 <= inner) {
+      v = s < 0 ? v4f{0.f, 0.f, 0.f, 0.f} : load4_stream_any(x + s * inner + p);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[j] = s < 0 ? 0.f : __builtin_nontemporal_load(x + s * inner + p);
+        if (++p == inner) p = 0, s = map.source(++r);  // never past the last row: 4 i + 3 < n
+      }
+    }
+    store4_stream_any(y + 4ull * i, v);
+  } else if (i == n4) {
+    for (uint32_t t = 4 * n4; t < n; ++t) {
+      uint32_t r, p;
+      fd_divmod(t, f_inner, r, p);
+      const int64_t s = map.source(r);
+      y[t] = s < 0 ? 0.f : x[s * inner + p];
+    }
+  }
+}
+
 template <class MAP>
 static int launch_rows_pick(const MAP& map, int64_t rows, int inner, const float* x, float* y,
                             hipStream_t st) {
   if (inner % 4 == 0 && aligned16(x) && aligned16(y)) {
     const uint32_t work = static_cast<uint32_t>(rows * (inner / 4));
     rows_pick_kernel<MAP><<<stream_grid(work), kStream, 0, st>>>(map, x, y, work, make_fastdiv(inner / 4));
+  } else if (MAP::kFlat) {
+    const uint32_t n = static_cast<uint32_t>(rows * inner), n4 = n / 4;
+    rows_pick_flat_kernel<MAP><<<stream_grid(n4 + 1), kStream, 0, st>>>(map, x, y, n4, n,
+                                                                       make_fastdiv(static_cast<uint32_t>(inner)));
   } else {
     const uint32_t units = (static_cast<uint32_t>(inner) + 3) / 4;
     const uint32_t work = static_cast<uint32_t>(rows * units);
@@ -423,12 +491,22 @@ __global__ __launch_bounds__(kBlock) void reorg_scatter_kernel(const float* x, f
     }
     return;
   }
+  // any row length: the vector may run over the end of its source row (rows of 38 or 26 floats), then the
+  // next element starts the next row, channel or image
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     uint32_t w, ow;
-    fd_divmod(ws + j, p.f_s, w, ow);
+    fd_divmod(ws, p.f_s, w, ow);
     const uint32_t c = DARKNET ? (oh * p.s + ow) * p.src_c + cs : (cs * p.s + oh) * p.s + ow;
     y[((static_cast<uint64_t>(b) * p.dst_c + c) * p.dst_h + h) * p.dst_w + w] = v[j];
+    if (++ws == p.f_src_w.d) {
+      ws = 0;
+      if (++hs == p.f_src_h.d) {
+        hs = 0;
+        if (++cs == p.f_src_c.d) cs = 0, ++b;
+      }
+      fd_divmod(hs, p.f_s, h, oh);
+    }
   }
 }
 
@@ -851,6 +929,12 @@ int shdw_hip_copy_chunks(int outer, int chunk, const float* src, int src_pitch, 
     copy_chunks_kernel<true><<<stream_grid(work), kStream, 0, st>>>(
         src, dst, work, make_fastdiv(chunk / 4), src_pitch / 4, src_offset / 4, dst_pitch / 4,
         dst_offset / 4);
+  } else if (chunk >= 4) {
+    const uint32_t units = (static_cast<uint32_t>(chunk) + 3) / 4;
+    const uint32_t work = static_cast<uint32_t>(outer) * units;  // <= outer * chunk
+    copy_chunks_any_kernel<<<stream_grid(work), kStream, 0, st>>>(src, dst, work, static_cast<uint32_t>(chunk),
+                                                                 make_fastdiv(units), src_pitch, src_offset,
+                                                                 dst_pitch, dst_offset);
   } else {
     const uint32_t work = static_cast<uint32_t>(outer) * chunk;
     copy_chunks_kernel<false><<<stream_grid(work), kStream, 0, st>>>(
@@ -1005,9 +1089,10 @@ int shdw_hip_reorg(const int* in_shape, int type, int stride, const float* x, fl
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint32_t n = static_cast<uint32_t>(count);
   const int ss = stride * stride;
-  // source-side walk whenever the source rows are whole vectors
+  // source-side walk whenever the tensor is whole vectors (one float per lane from the destination side ran
+  // the natural order on 38x38 maps at 39 us per 51 MB against 20 us)
   const int src_w = type == 0 ? in_w * stride : in_w;
-  if (src_w % 4 == 0 && aligned16(x)) {
+  if (n % 4 == 0 && aligned16(x)) {
     ReorgScatterArgs a;
     a.s = stride;
     if (type == 0) {  // source = the [B][C/ss][H*s][W*s] view, destination = [B][C][H][W]
@@ -1020,7 +1105,7 @@ int shdw_hip_reorg(const int* in_shape, int type, int stride, const float* x, fl
     a.f_src_c = make_fastdiv(a.src_c);
     a.f_s = make_fastdiv(stride);
     // 64-bit stores need an even destination row length and an 8-byte aligned base
-    const bool s2 = stride == 2 && a.dst_w % 2 == 0 && (reinterpret_cast<uintptr_t>(y) & 7u) == 0;
+    const bool s2 = stride == 2 && src_w % 4 == 0 && a.dst_w % 2 == 0 && (reinterpret_cast<uintptr_t>(y) & 7u) == 0;
     const uint32_t g = grid_for(n / 4);
     if (type == 0) {
       if (s2)

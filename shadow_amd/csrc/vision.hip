@@ -73,14 +73,25 @@ __global__ __launch_bounds__(kStream) void rows_vec_kernel(P p, const float* x, 
 #pragma unroll
       for (int j = 0; j < 4; ++j) r[j] = p.apply(vx[j], vo[j], rp);
     } else {
-      // Most vectors still lie inside one row: fetch its parameters once and
-      // only the lanes whose vector straddles a boundary look up a second row.
+      // One division per vector.  Rows of four and more: the vector ends in the
+      // next row at the furthest, so the parameters of two rows serve it (the
+      // second is the first again where the vector lies inside one row); a
+      // division and a test per element ran BatchNorm over 7x7 maps at 24 us
+      // per 51 MB against 17 us for rows of whole vectors.  Shorter rows: the
+      // row steps along with the elements.
       const uint32_t r0 = fd_div(4 * i, inner);
-      const typename P::Row rp0 = p.row(r0);
+      const uint32_t left = (r0 + 1) * inner.d - 4 * i;  // elements of the vector in row r0: 1 ..
+      if (inner.d >= 4) {
+        const typename P::Row rp0 = p.row(r0), rp1 = p.row(left < 4 ? r0 + 1 : r0);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t rj = fd_div(4 * i + j, inner);
-        r[j] = p.apply(vx[j], vo[j], rj == r0 ? rp0 : p.row(rj));
+        for (int j = 0; j < 4; ++j) r[j] = p.apply(vx[j], vo[j], static_cast<uint32_t>(j) < left ? rp0 : rp1);
+      } else {
+        uint32_t row = r0, togo = left;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          r[j] = p.apply(vx[j], vo[j], p.row(row));
+          if (--togo == 0) ++row, togo = inner.d;
+        }
       }
     }
     store4_stream_any(out + 4ull * i, r);

@@ -34,7 +34,11 @@ def run(ws, op_type, inputs, args, tops=("out",)):
 @pytest.mark.parametrize("shapes,axis", [
     ([(2, 3, 4, 5), (2, 7, 4, 5)], 1), ([(2, 3, 4, 8), (2, 3, 4, 4), (2, 3, 4, 12)], 3),
     ([(3, 5), (2, 5), (4, 5)], 0), ([(2, 3, 7), (2, 3, 1)], -1), ([(4, 16, 14, 14), (4, 32, 14, 14)], 1),
-    ([(2, 3, 5, 5), (2, 3, 5, 5)], 2)])
+    ([(2, 3, 5, 5), (2, 3, 5, 5)], 2),
+    # chunks and pitches that are no whole vectors: 128-bit accesses on any dword address with the chunk's cut
+    # end float by float (chunks of 49, 5, 75 and 1001 floats), chunks under four floats
+    ([(3, 1, 7, 7), (3, 2, 7, 7)], 1), ([(40, 5), (40, 9), (40, 2)], 1), ([(6, 3, 25), (6, 4, 25)], 1),
+    ([(5, 1001), (5, 1003)], 1), ([(4, 7, 3), (4, 7, 1)], 2)])
 def test_concat_op(ws, shapes, axis):
     xs = [normal(10 + k, s) for k, s in enumerate(shapes)]
     got = run(ws, "Concat", [("x%d" % k, x) for k, x in enumerate(xs)], {"axis": axis})
@@ -45,7 +49,9 @@ def test_concat_op(ws, shapes, axis):
 
 @pytest.mark.parametrize("shape,axis,points,n", [((2, 12, 4, 4), 1, [], 3), ((2, 12, 4, 4), 1, [4, 5], 3),
                                                  ((6, 5), 0, [], 2), ((2, 3, 10), -1, [3], 2),
-                                                 ((4, 48, 7, 7), 1, [16, 32], 3)])
+                                                 ((4, 48, 7, 7), 1, [16, 32], 3),
+                                                 ((3, 5, 7, 7), 1, [1, 3], 3), ((30, 21), 1, [5, 14], 3),
+                                                 ((4, 2004), 1, [1001], 2), ((6, 9, 5), 1, [2], 2)])
 def test_slice_op(ws, shape, axis, points, n):
     x = normal(20, shape)
     args = {"axis": axis}
@@ -59,7 +65,7 @@ def test_slice_op(ws, shape, axis, points, n):
 
 
 @pytest.mark.parametrize("shape,axis,k", [((2, 3, 4), 0, 2), ((2, 3, 4), 1, 3), ((2, 3, 4), 3, 2), ((2, 3, 4), -1, 2),
-                                          ((5, 8), -2, 4), ((16, 64), 1, 3)])
+                                          ((5, 8), -2, 4), ((16, 64), 1, 3), ((7, 49), 1, 3), ((3, 5, 13), 1, 2)])
 def test_stack_op(ws, shape, axis, k):
     xs = [normal(30 + j, shape) for j in range(k)]
     got = run(ws, "Stack", [("x%d" % j, x) for j, x in enumerate(xs)], {"axis": axis})
@@ -129,7 +135,11 @@ def test_permute_op(ws, shape, order):
 
 
 @pytest.mark.parametrize("type_", [0, 1])
-@pytest.mark.parametrize("shape,stride", [((2, 8, 6, 4), 2), ((1, 9, 6, 9), 3), ((2, 64, 26, 26), 2), ((1, 4, 2, 2), 1)])
+# rows that are whole vectors and rows that are not (26, 38, 6 and 9 floats: a lane's four source floats run
+# over the end of a row, a channel and an image), strides 1 to 4, a tensor that is no whole vectors
+@pytest.mark.parametrize("shape,stride", [((2, 8, 6, 4), 2), ((1, 9, 6, 9), 3), ((2, 64, 26, 26), 2), ((1, 4, 2, 2), 1),
+                                          ((3, 16, 38, 38), 2), ((2, 4, 6, 6), 2), ((3, 9, 3, 3), 3), ((2, 16, 8, 12), 4),
+                                          ((1, 4, 2, 6), 2), ((5, 4, 10, 2), 2)])
 def test_reorg_op(ws, type_, shape, stride):
     x = normal(70, shape)
     got = run(ws, "Reorg", [("x", x)], {"type": type_, "stride": stride})
@@ -180,7 +190,10 @@ def test_resize_nearest_any_width(ws, shape, size):
 
 
 @pytest.mark.parametrize("shape,group", [((2, 6, 3, 5), 2), ((2, 6, 3, 5), 3), ((1, 12, 4, 4), 4), ((3, 8, 1, 1), 8),
-                                         ((2, 116, 28, 28), 2), ((2, 6, 3, 5), 1), ((2, 116, 7, 7), 2), ((3, 4, 1, 3), 2)])
+                                         ((2, 116, 28, 28), 2), ((2, 6, 3, 5), 1), ((2, 116, 7, 7), 2), ((3, 4, 1, 3), 2),
+                                         # rows of 7, 1, 2, 5 and 49 floats: a lane's four outputs from up to four rows
+                                         ((9, 12, 1, 7), 4), ((33, 10, 1, 1), 5), ((7, 6, 1, 2), 3), ((5, 9, 5, 1), 3),
+                                         ((3, 232, 7, 7), 2), ((1, 3, 1, 1), 3)])
 def test_shuffle_channel_op(ws, shape, group):
     x = normal(80, shape)
     got = run(ws, "ShuffleChannel", [("x", x)], {"group": group})

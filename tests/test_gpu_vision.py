@@ -57,7 +57,11 @@ def test_axpy_op(ws):
 
 
 # ------------------------------------------------------------- batch norm ---
-@pytest.mark.parametrize("shape", [(2, 3, 4, 4), (4, 64, 7, 7), (3, 5, 9, 11), (2, 7, 1, 1), (1, 130, 28, 28)])
+# Rows (inner extents) of 1, 2 and 3: up to four rows per 128-bit vector; of 5, 6, 7, 49, 99: a vector ends
+# in the next row; a last vector that ends with the tensor.
+@pytest.mark.parametrize("shape", [(2, 3, 4, 4), (4, 64, 7, 7), (3, 5, 9, 11), (2, 7, 1, 1), (1, 130, 28, 28),
+                                   (5, 9, 1, 2), (3, 7, 1, 3), (4, 6, 5, 1), (3, 11, 2, 3), (2, 5, 1, 7), (7, 3, 1, 1),
+                                   (9, 1, 1, 1), (2, 2, 9, 11), (3, 1001, 1, 1), (2, 1000, 1, 3)])
 @pytest.mark.parametrize("sf", [1.0, 0.0010000181])
 def test_batch_norm(gpu, shape, sf):
     x = with_specials(normal(7, shape, 3.0), 7)
