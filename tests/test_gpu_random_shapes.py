@@ -172,6 +172,42 @@ def test_mover_random_shapes(gpu, seed):
         dy.free()
 
 
+# Concat / Slice / Stack all go through one strided chunk copy: chunks, pitches and offsets that are and are
+# not whole vectors, chunks of one to three floats, pointers off the vector boundary.
+@pytest.mark.parametrize("seed", [29, 30])
+def test_copy_chunks_random(gpu, seed):
+    rng = np.random.default_rng(seed)
+    lib = shadow_amd.hip()
+    for _ in range(80):
+        outer = int(rng.integers(1, 60))
+        chunk = int(np.exp(rng.uniform(0, np.log(3000))))
+        if rng.random() < 0.3:
+            chunk = 4 * max(1, chunk // 4)
+        src_off, dst_off = int(rng.integers(0, 9)), int(rng.integers(0, 9))
+        src_pitch = src_off + chunk + int(rng.integers(0, 9))
+        dst_pitch = dst_off + chunk + int(rng.integers(0, 9))
+        if rng.random() < 0.3:
+            src_off, dst_off, src_pitch, dst_pitch = [4 * (v // 4 + (k >= 2)) + (chunk if k >= 2 else 0)
+                                                      for k, v in enumerate((src_off, dst_off, src_pitch - chunk,
+                                                                             dst_pitch - chunk))]
+            src_pitch, dst_pitch = max(src_pitch, src_off + chunk), max(dst_pitch, dst_off + chunk)
+        shift = int(rng.integers(0, 4)) if rng.random() < 0.3 else 0
+        src = rng.normal(0, 1, outer * src_pitch + shift).astype(F)
+        dst = rng.normal(0, 1, outer * dst_pitch + shift).astype(F)
+        want = dst.copy()
+        for n in range(outer):
+            want[shift + n * dst_pitch + dst_off: shift + n * dst_pitch + dst_off + chunk] = \
+                src[shift + n * src_pitch + src_off: shift + n * src_pitch + src_off + chunk]
+        ds, dd = Buffer.from_numpy(src), Buffer.from_numpy(dst)
+        check(lib.shdw_hip_copy_chunks(outer, chunk, ds.ptr + 4 * shift, src_pitch, src_off, dd.ptr + 4 * shift,
+                                       dst_pitch, dst_off, None))
+        gpuops._sync()
+        assert_bit_exact(dd.download(count=dst.size), want, "chunks of %d, pitches %d -> %d, offsets %d -> %d, shift %d"
+                         % (chunk, src_pitch, dst_pitch, src_off, dst_off, shift))
+        ds.free()
+        dd.free()
+
+
 @pytest.fixture()
 def ws(gpu):
     w = shadow_amd.Workspace("Native", 0)
