@@ -1,5 +1,6 @@
 """The largest tensors the int32 element counts of the interface admit: 2^31 - 1 floats
-(8.6 GB) through the elementwise, per-channel, reduction, softmax and pooling kernels.
+(8.6 GB) through the elementwise, per-channel, reduction, softmax, pooling, broadcast,
+norm and data-moving kernels.
 The expected values come from numpy or the oracle on the same data, compared in pieces
 so that the host never holds more than the input and one output; the data is a 2^20-float random block
 repeated, which keeps every index of the tensor in play (the last vector ends
@@ -164,3 +165,89 @@ def test_pooling_at_the_largest_count(gpu, big):
     got = dy.download(count=planes)
     want = oracle.pooling(x[:planes * 256 * 255], shape, 1, [256, 255], [1, 1], [0, 0], out)
     assert np.array_equal(bits(got), bits(np.asarray(want, F).ravel())), "whole-plane average"
+
+
+def test_broadcast_and_batch_norm_at_the_largest_count(gpu, big):
+    x, dx, dy = big
+    lib = shadow_amd.hip()
+    shape, n = [8, 64, 2048, 2047], 8 * 64 * 2048 * 2047
+    plane = 2048 * 2047
+    b = np.linspace(-3.0, 3.0, 64).astype(F)
+    db = Buffer.from_numpy(b)
+    check(lib.shdw_hip_broadcast_binary(0, 4, ints(shape), ints([1, 64, 1, 1]), ints(shape), dx.ptr, db.ptr, dy.ptr, None))
+    gpuops._sync()
+    got = dy.download(count=n)
+    for lo in range(0, n, PIECE):
+        hi = min(n, lo + PIECE)
+        c = (np.arange(lo, hi, dtype=np.int64) // plane) % 64
+        assert np.array_equal(bits(got[lo:hi]), bits(x[lo:hi] + b[c])), "channel add from %d" % lo
+    # BatchNorm over rows of 2047 floats: a vector ends in the next row
+    mean, var = np.linspace(-1.0, 1.0, 64).astype(F), np.linspace(0.25, 9.0, 64).astype(F)
+    dm, dv = Buffer.from_numpy(mean), Buffer.from_numpy(var)
+    rows = n // 2047
+    check(lib.shdw_hip_batch_norm(rows * 2047, 64, 2047, dx.ptr, dm.ptr, dv.ptr, 1.0, 1e-5, dy.ptr, None))
+    gpuops._sync()
+    got = dy.download(count=rows * 2047)
+    d = np.sqrt(np.abs(var * F(1.0)) + F(1e-5)).astype(F)
+    for lo in range(0, rows * 2047, PIECE):
+        hi = min(rows * 2047, lo + PIECE)
+        c = (np.arange(lo, hi, dtype=np.int64) // 2047) % 64
+        assert np.array_equal(bits(got[lo:hi]), bits((x[lo:hi] - mean[c] * F(1.0)) / d[c])), "batch norm from %d" % lo
+    for buf in (db, dm, dv):
+        buf.free()
+
+
+def test_movers_at_the_largest_count(gpu, big):
+    x, dx, dy = big
+    lib = shadow_amd.hip()
+    # interleaved -> planar: the thin transposition
+    rows = N // 3
+    check(lib.shdw_hip_permute(2, ints([rows, 3]), ints([1, 0]), dx.ptr, dy.ptr, None))
+    gpuops._sync()
+    got = dy.download(count=3 * rows)
+    src = x[:3 * rows].reshape(rows, 3)
+    for k in range(3):
+        assert np.array_equal(bits(got[k * rows:(k + 1) * rows]), bits(src[:, k])), "planar channel %d" % k
+    # a square-ish transposition through the LDS tiles
+    r, c = 32768, 65535
+    check(lib.shdw_hip_permute(2, ints([r, c]), ints([1, 0]), dx.ptr, dy.ptr, None))
+    gpuops._sync()
+    got = dy.download(count=r * c).reshape(c, r)
+    src = x[:r * c].reshape(r, c)
+    for lo in range(0, c, 4096):
+        assert np.array_equal(bits(got[lo:lo + 4096]), bits(np.ascontiguousarray(src[:, lo:lo + 4096].T))), \
+            "transposed rows from %d" % lo
+    # Concat of two inputs along the middle axis: chunks of 1023 rows of 1025 floats into rows of twice that
+    chunk = 1023 * 1025
+    outer = N // (2 * chunk)
+    for k in range(2):
+        check(lib.shdw_hip_copy_chunks(outer, chunk, dx.ptr + 4 * k * outer * chunk, chunk, 0, dy.ptr, 2 * chunk,
+                                       k * chunk, None))
+    gpuops._sync()
+    got = dy.download(count=2 * outer * chunk).reshape(outer, 2, chunk)
+    for k in range(2):
+        src = x[k * outer * chunk:(k + 1) * outer * chunk].reshape(outer, chunk)
+        assert np.array_equal(bits(got[:, k, :]), bits(src)), "concat input %d" % k
+
+
+def test_normalize_and_row_norm_at_the_largest_count(gpu, big):
+    x, dx, dy = big
+    lib = shadow_amd.hip()
+    for dim, inner in ((512, 1), (64, 49)):
+        outer = N // (dim * inner)
+        check(lib.shdw_hip_normalize(outer, dim, inner, 2.0, 1e-12, dx.ptr, dy.ptr, None))
+        gpuops._sync()
+        slab = dim * inner
+        slabs = max(1, (1 << 22) // slab)
+        for s0 in (0, (outer - slabs) // 2, outer - slabs):
+            got = dy.download(count=slabs * slab, offset_bytes=4 * s0 * slab)
+            want = oracle.normalize(x[s0 * slab:(s0 + slabs) * slab], slabs, dim, inner, 2.0, 1e-12)
+            assert np.array_equal(bits(got), bits(np.asarray(want, F).ravel())), "normalize [%d,%d] from %d" % (dim, inner, s0)
+    rows, length = N // 784, 784
+    check(lib.shdw_hip_group_norm(rows, length, 1e-5, dx.ptr, None, None, 1, 1, dy.ptr, None))
+    gpuops._sync()
+    count = (1 << 22) // length
+    for r0 in (0, rows - count):
+        got = dy.download(count=count * length, offset_bytes=4 * r0 * length)
+        want = oracle.normalize_rows(x[r0 * length:(r0 + count) * length], count, length, 1e-5)
+        assert np.max(np.abs(got - np.asarray(want, F).ravel())) <= 2e-5, "row norm from %d" % r0
