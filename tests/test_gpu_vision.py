@@ -175,6 +175,26 @@ def test_softmax_over_short_rows(gpu, dim):
     assert_bit_exact(gpuops.softmax(x, 5003, dim, 1), oracle.softmax(x, 5003, dim, 1), "softmax specials")
 
 
+# Two to four rows over 16 and more positions: four positions per lane with their columns in registers; rows that
+# are and are not whole vectors long (the last quad of a slab cut), Normalize / SSDNormalize over two rows.
+@pytest.mark.parametrize("outer,dim,inner", [(5, 2, 16), (3, 3, 17), (2, 4, 64), (7, 2, 49), (1, 3, 1001), (300, 2, 20),
+                                             (2, 4, 18), (9, 1, 33), (4, 2, 3136)])
+def test_column_ops_over_two_to_four_rows(gpu, outer, dim, inner):
+    x = with_specials(normal(48, outer * dim * inner, 6.0), 48)
+    want = oracle.softmax(x, outer, dim, inner)
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner), want, "softmax")
+    assert_bit_exact(gpuops.softmax(x, outer, dim, inner, inplace=True, offset=1), want, "softmax in place, off the vector boundary")
+    x = normal(49, outer * dim * inner, 3.0)
+    for p in (1.0, 2.0):
+        want = oracle.normalize(x, outer, dim, inner, p, 1e-12)
+        assert_bit_exact(gpuops.normalize(x, outer, dim, inner, p, 1e-12), want, "normalize p=%g" % p)
+        assert_bit_exact(gpuops.normalize(x, outer, dim, inner, p, 1e-12, inplace=True, offset=3), want, "normalize in place")
+    for shared in (True, False):
+        scale = uniform(50, 1 if shared else dim, 0.5, 2.0)
+        assert_bit_exact(gpuops.ssd_normalize(x, outer, dim, inner, False, shared, 1e-6, scale),
+                         oracle.ssd_normalize(x, outer, dim, inner, False, shared, 1e-6, scale), "ssd normalize")
+
+
 # Slabs of dim * inner <= 9 floats with inner > 1 go the same way, four slabs per lane; the next larger ones.
 @pytest.mark.parametrize("outer,dim,inner", [(5003, 2, 2), (4099, 2, 4), (1027, 3, 3), (70001, 4, 2), (1500, 3, 2),
                                              (1029, 2, 3), (2001, 5, 2), (1025, 3, 4), (1024, 2, 7), (33333, 7, 2)])
