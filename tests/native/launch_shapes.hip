@@ -202,6 +202,33 @@ static int time_us(F launch, int reps, float* us) {
   return 0;
 }
 
+// A chain of dependent fp32 additions, as the in-order sums of Pooling, Softmax and Normalize are one per
+// row or column: CHAINS independent chains per wave, all lanes alike.  The asm statement keeps the
+// compiler from reassociating or hoisting the chain.  Workgroups of four waves: one wave to each SIMD of a CU
+// (single-wave workgroups may share a SIMD while others idle).
+template <int CHAINS>
+__global__ __launch_bounds__(256) void add_chain_kernel(const float* in, float* out, int n) {
+  float s[CHAINS];
+#pragma unroll
+  for (int c = 0; c < CHAINS; ++c) s[c] = in[threadIdx.x + c];
+  const float a = in[256 + threadIdx.x], b = in[512 + threadIdx.x];
+  for (int i = 0; i < n; i += 8) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+#pragma unroll
+      for (int c = 0; c < CHAINS; ++c) s[c] += a;
+#pragma unroll
+      for (int c = 0; c < CHAINS; ++c) s[c] += b;
+    }
+#pragma unroll
+    for (int c = 0; c < CHAINS; ++c) asm volatile("" : "+v"(s[c]));
+  }
+  float t = 0.f;
+#pragma unroll
+  for (int c = 0; c < CHAINS; ++c) t += s[c];
+  out[blockIdx.x * 256 + threadIdx.x] = t;
+}
+
 int main() {
   const size_t kPool = 6ull * 205520896;
   float *rp, *wp;
@@ -297,6 +324,20 @@ int main() {
       // half the registers per lane: eight instead of five workgroups fit a CU, and the copy gets slower
       if (dim <= 256) TILECOPY(256, 8, true, false)
     }
+  }
+  // ordered sums: what one dependent fp32 addition costs a chain, by the waves that share a SIMD
+  {
+    printf("# add chain: ns per addition of one chain / of the SIMD, 2^18 dependent fp32 additions per chain; "
+           "waves = per SIMD (workgroups of four waves, one to a SIMD, 256 workgroups per wave wanted), chains = independent "
+           "chains per wave\n");
+    const int n = 1 << 18;
+#define CHAIN(WAVES, CHAINS)                                                                           \
+  {                                                                                                    \
+    float us;                                                                                          \
+    if (time_us([&](int) { add_chain_kernel<CHAINS><<<256 * WAVES, 256>>>(rp, wp, n); }, 3, &us)) return 1; \
+    printf("add chain waves %d chains %d: %.2f %.2f\n", WAVES, CHAINS, us * 1e3f / n, us * 1e3f / n / (WAVES * CHAINS)); \
+  }
+    CHAIN(1, 1) CHAIN(1, 2) CHAIN(1, 4) CHAIN(2, 1) CHAIN(4, 1) CHAIN(8, 1) CHAIN(8, 2)
   }
   return 0;
 }

@@ -86,3 +86,16 @@ def test_channel_tile_shape_in_use_and_what_the_pattern_costs(table):
         mine = {k[1:]: v for k, v in rows.items() if k[0] == inner}
         assert mine[used] <= SLACK * min(mine.values()), (inner, mine)
         assert min(mine.values()) > 1.10 * flat[inner], (inner, flat[inner], mine)
+
+
+def test_a_lone_chain_of_ordered_additions_is_bound_by_latency(table):
+    """The in-order sums (whole-plane average, Softmax, Normalize) are one dependent chain per row or column:
+    a chain alone on its SIMD pays the latency of every addition, several waves (or chains) per SIMD share it.
+    The kernels' rows-per-wave choices rest on these figures."""
+    rows = {(int(w), int(c)): (float(a), float(b))
+            for w, c, a, b in re.findall(r"add chain waves (\d+) chains (\d+): (\d+\.\d+) (\d+\.\d+)", table)}
+    assert len(rows) == 7
+    lone_chain, _ = rows[(1, 1)]
+    _, simd_rate = rows[(8, 1)]
+    assert lone_chain > 2.0 * simd_rate, rows  # one chain leaves most of the SIMD's issue slots empty
+    assert rows[(1, 4)][1] < lone_chain, rows   # chains interleaved inside one wave share the latency too
