@@ -898,26 +898,17 @@ __global__ __launch_bounds__(kBlock) void pool_rows_stream_kernel(const float* x
     if (lane < G) {
       const uint32_t cols = min(W, len - c0);
       const float* mine = tile + lane * PITCH;
-      // 32 values per step and two steps per turn, each step's values requested
-      // one step ahead: the additions, not the LDS latency, set the pace.
-      constexpr int kAhead = 8, kStep = 4 * kAhead;
+      // 64 values per step, read with sixteen 128-bit reads and then added in order.  One set of
+      // registers: with two sets taking turns (the next step's reads behind this step's additions) the
+      // compiler copied one set into the other every turn, 32 moves per 64 additions, and a wave
+      // alone on its SIMD issues an instruction every 2.8 ns whatever it is; the LDS latency that is
+      // exposed instead is a twentieth of a step's additions.
+      constexpr int kAhead = 16, kStep = 4 * kAhead;
       uint32_t c = 0;
-      if (cols >= kStep) {
-        v4f q[kAhead], w[kAhead];
+      for (; c + kStep <= cols; c += kStep) {
+        v4f q[kAhead];
 #pragma unroll
-        for (int k = 0; k < kAhead; ++k) q[k] = *reinterpret_cast<const v4f*>(mine + 4 * k);
-        for (c = kStep; c + 2 * kStep <= cols; c += 2 * kStep) {
-#pragma unroll
-          for (int k = 0; k < kAhead; ++k) w[k] = *reinterpret_cast<const v4f*>(mine + c + 4 * k);
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int k = 0; k < kStep; ++k) sum += q[k / 4][k % 4];
-#pragma unroll
-          for (int k = 0; k < kAhead; ++k) q[k] = *reinterpret_cast<const v4f*>(mine + c + kStep + 4 * k);
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int k = 0; k < kStep; ++k) sum += w[k / 4][k % 4];
-        }
+        for (int k = 0; k < kAhead; ++k) q[k] = *reinterpret_cast<const v4f*>(mine + c + 4 * k);
 #pragma unroll
         for (int k = 0; k < kStep; ++k) sum += q[k / 4][k % 4];
       }
@@ -933,17 +924,16 @@ __global__ __launch_bounds__(kBlock) void pool_rows_stream_kernel(const float* x
 // 24.6 / 59 us; 14x14 planes 13.2 / 14.2 us but 45.8 / 42.0 us per 205 MB, 7x7 planes
 // 12.6 / 12.7 and 44.1 / 39.6 us).
 constexpr int kPlaneStreamMinLen = 256;
-// ... and from this many rows on: a wave per row needs rows to fill the chip
-// (256 planes of 112x112: 168 us against 99 us).
-constexpr uint32_t kPlaneStreamMinRows = 512;
-
-// Rows per wave: about 2048 waves in all (eight per CU, what their LDS lets reside
-// at once, two per SIMD), so long and few rows get a wave each.  Measured per
-// 51 MB: 28x28 planes 15.1 us with 8 rows per wave (20.0 with 4, 16.1 with 16),
-// 56x56 planes 24.6 us with 2 (39 with 1 or 4).
+// Few rows as well: a wave per row walks at 5 ns per element where the workgroup form above, which stages
+// a chunk, meets at a barrier and then walks it, takes 10 to 18 ([1,3,224,224]: 252 us against 630 us,
+// 64 planes of 56x56: 29 against 30).
+// Rows per wave: as many as leave 1536 waves and more (six per CU), so long and few rows get a wave
+// each.  Measured per 51 MB: 16x16 planes 10.2 us with 32 rows per wave (12.7 with 16), 20x20 11.7 with
+// 16 (14.6 with 8), 28x28 13.1 with 8 (17.2 with 4, 13.7 with 16), 40x40 16.6 with 4 (21.7 with 2),
+// 56x56 21.3 with 2 (26.3 with 4, 33.9 with 1).
 static int stream_rows_per_wave(uint32_t rows) {
   int g = 1;
-  while (g < 64 && rows / static_cast<uint32_t>(2 * g) >= 2048u) g <<= 1;
+  while (g < 64 && rows / static_cast<uint32_t>(2 * g) >= 1536u) g <<= 1;
   return g;
 }
 
@@ -1006,7 +996,7 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
       int rc = SHDW_OK;
       if (reduce_rows_max(rows, static_cast<uint32_t>(plane), x, y, st, &rc)) return rc;
       launch_pool_plane<true>(x, y, rows, static_cast<uint32_t>(plane), st);
-    } else if (plane >= kPlaneStreamMinLen && rows >= kPlaneStreamMinRows) {
+    } else if (plane >= kPlaneStreamMinLen) {
       launch_pool_rows_stream(x, y, rows, static_cast<uint32_t>(plane), st);
     } else {
       launch_pool_plane<false>(x, y, rows, static_cast<uint32_t>(plane), st);
