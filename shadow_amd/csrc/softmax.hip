@@ -224,6 +224,16 @@ SHDW_DEVICE void walk_column(const float* col, uint32_t stride, uint32_t n, F&& 
   for (; c < n; ++c) fold(col[c * stride]);
 }
 
+// The same for the strides the tall kernels have (16, 32 or 64 floats): with the stride a constant the
+// sixteen reads of a batch share one address register and differ in their immediate offsets, one
+// instruction less per element for the walking lane.
+template <class F>
+SHDW_DEVICE void walk_column_tile(const float* col, uint32_t width, uint32_t n, F&& fold) {
+  if (width == 16) walk_column(col, 16, n, fold);
+  else if (width == 32) walk_column(col, 32, n, fold);
+  else walk_column(col, 64, n, fold);
+}
+
 // Any-order maximum over the workgroup.  Only valid where the order cannot
 // show: see softmax_slab_kernel.
 SHDW_DEVICE float block_max_any_order(float m, float* scratch4) {
@@ -1687,7 +1697,7 @@ __global__ __launch_bounds__(kBlock) void softmax_tall_kernel(const float* x, fl
       }
     __syncthreads();
     t.load(x, k + 2, reg);
-    if (threadIdx.x < t.width) walk_column(buf + threadIdx.x, t.width, t.rows_in(k), [&](float a) { sum += a; });
+    if (threadIdx.x < t.width) walk_column_tile(buf + threadIdx.x, t.width, t.rows_in(k), [&](float a) { sum += a; });
   };
   v4f v2[T::kLoads];
   t.load(x, 0, v);
@@ -1744,7 +1754,7 @@ __global__ __launch_bounds__(kBlock) void normalize_tall_kernel(const float* x, 
     __syncthreads();
     t.load(x, k + 2, reg);
     if (threadIdx.x < t.width)
-      walk_column(buf + threadIdx.x, t.width, t.rows_in(k), [&](float a) { acc += static_cast<double>(a); });
+      walk_column_tile(buf + threadIdx.x, t.width, t.rows_in(k), [&](float a) { acc += static_cast<double>(a); });
   };
   v4f v2[T::kLoads];
   t.load(x, 0, v);
