@@ -234,6 +234,22 @@ SHDW_DEVICE void walk_column_tile(const float* col, uint32_t width, uint32_t n, 
   else walk_column(col, 64, n, fold);
 }
 
+// ... and for the small position counts of the slab kernels (a column per position, `inner` floats apart).
+template <class F>
+SHDW_DEVICE void walk_column_inner(const float* col, uint32_t inner, uint32_t n, F&& fold) {
+  switch (inner) {
+    case 1: walk_column(col, 1, n, fold); break;
+    case 2: walk_column(col, 2, n, fold); break;
+    case 3: walk_column(col, 3, n, fold); break;
+    case 4: walk_column(col, 4, n, fold); break;
+    case 7: walk_column(col, 7, n, fold); break;
+    case 8: walk_column(col, 8, n, fold); break;
+    case 16: walk_column(col, 16, n, fold); break;
+    case 49: walk_column(col, 49, n, fold); break;
+    default: walk_column(col, inner, n, fold);
+  }
+}
+
 // Any-order maximum over the workgroup.  Only valid where the order cannot
 // show: see softmax_slab_kernel.
 SHDW_DEVICE float block_max_any_order(float m, float* scratch4) {
@@ -324,7 +340,7 @@ __global__ __launch_bounds__(kBlock) void softmax_slab_kernel(const float* x, fl
   __syncthreads();
   if (threadIdx.x < inner) {
     float sum = 0.f;
-    walk_column(lds + threadIdx.x, inner, dim, [&](float v) { sum += v; });
+    walk_column_inner(lds + threadIdx.x, inner, dim, [&](float v) { sum += v; });
     stat[threadIdx.x] = sum;
   }
   __syncthreads();
@@ -607,7 +623,7 @@ __global__ __launch_bounds__(kBlock) void normalize_slab_kernel(const float* x, 
   } else {
     if (threadIdx.x < inner) {  // inner < 64 here
       double acc = 0;
-      walk_column(lds + threadIdx.x, inner, dim, [&](float v) { acc += static_cast<double>(v); });
+      walk_column_inner(lds + threadIdx.x, inner, dim, [&](float v) { acc += static_cast<double>(v); });
       stat[threadIdx.x] = norm_finish<PMODE>(acc, p, eps);
     }
   }
@@ -1898,7 +1914,7 @@ __global__ __launch_bounds__(kBlock) void softmax_long_slab_kernel(const float* 
   __syncthreads();
   if (threadIdx.x < inner) {
     float m = -FLT_MAX;
-    walk_column(chunk[0] + threadIdx.x, inner, t.chunk_rows, [&](float a) { m = std_max(a, m); });
+    walk_column_inner(chunk[0] + threadIdx.x, inner, t.chunk_rows, [&](float a) { m = std_max(a, m); });
     stat[threadIdx.x] = m;
   }
   __syncthreads();
@@ -1921,7 +1937,7 @@ __global__ __launch_bounds__(kBlock) void softmax_long_slab_kernel(const float* 
     }
     __syncthreads();
     t.load(k + 2, reg);
-    if (threadIdx.x < inner) walk_column(buf + threadIdx.x, inner, t.rows_in(k), [&](float a) { sum += a; });
+    if (threadIdx.x < inner) walk_column_inner(buf + threadIdx.x, inner, t.rows_in(k), [&](float a) { sum += a; });
   };
   t.load(0, v);
   t.load(1, v2);
@@ -1979,7 +1995,7 @@ __global__ __launch_bounds__(kBlock) void normalize_long_slab_kernel(const float
     __syncthreads();
     t.load(k + 2, reg);
     if (threadIdx.x < inner)
-      walk_column(buf + threadIdx.x, inner, t.rows_in(k), [&](float a) { acc += static_cast<double>(a); });
+      walk_column_inner(buf + threadIdx.x, inner, t.rows_in(k), [&](float a) { acc += static_cast<double>(a); });
   };
   t.load(0, v);
   t.load(1, v2);
