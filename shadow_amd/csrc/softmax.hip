@@ -775,6 +775,18 @@ SHDW_DEVICE void packed_stage_out(const float* lds, float* ys, const PackedSpan&
   }
 }
 
+// A lane's walk down its column: batches of sixteen reads at a constant stride from sixteen rows on, a
+// plain loop for the short columns (two classes, a handful of channels), which a batch would not fill.
+template <class F>
+SHDW_DEVICE void packed_walk(const float* col, uint32_t inner, uint32_t dim, F&& fold) {
+  if (dim >= 16) {
+    walk_column_inner(col, inner, dim, fold);
+  } else {
+#pragma unroll 4
+    for (uint32_t c = 0; c < dim; ++c) fold(col[c * inner]);
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void softmax_packed_kernel(const float* x, float* y, uint32_t slabs,
                                                                  uint32_t dim, FastDiv f_inner, FastDiv f_slab,
                                                                  uint32_t group) {
@@ -791,8 +803,7 @@ __global__ __launch_bounds__(kBlock) void softmax_packed_kernel(const float* x, 
   const float* col = lds + fd_div(q, f_inner) * sp.pitch + (q - fd_div(q, f_inner) * sp.inner);
   if (q < sp.ncols) {
     float m = -FLT_MAX;
-#pragma unroll 4
-    for (uint32_t c = 0; c < dim; ++c) m = std_max(col[c * sp.inner], m);
+    packed_walk(col, sp.inner, dim, [&](float v) { m = std_max(v, m); });
     stat[q] = m;
   }
   __syncthreads();
@@ -800,8 +811,7 @@ __global__ __launch_bounds__(kBlock) void softmax_packed_kernel(const float* x, 
   __syncthreads();
   if (q < sp.ncols) {
     float sum = 0.f;
-#pragma unroll 4
-    for (uint32_t c = 0; c < dim; ++c) sum += col[c * sp.inner];
+    packed_walk(col, sp.inner, dim, [&](float v) { sum += v; });
     stat[q] = sum;
   }
   __syncthreads();
@@ -825,8 +835,7 @@ __global__ __launch_bounds__(kBlock) void normalize_packed_kernel(const float* x
     const uint32_t g = fd_div(q, f_inner);
     const float* col = lds + g * sp.pitch + (q - g * sp.inner);
     double acc = 0;
-#pragma unroll 4
-    for (uint32_t c = 0; c < dim; ++c) acc += norm_term<PMODE>(col[c * sp.inner], p);
+    packed_walk(col, sp.inner, dim, [&](float v) { acc += norm_term<PMODE>(v, p); });
     stat[q] = norm_finish<PMODE>(acc, p, eps);
   }
   __syncthreads();
