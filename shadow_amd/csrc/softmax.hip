@@ -2044,6 +2044,7 @@ static bool long_slab(int outer_num, int dim, int inner_num, bool softmax) {
   if (static_cast<int64_t>(dim) * inner_num <= kLongSlabMinFloats) return false;
   if (static_cast<uint32_t>(inner_num) < kTallMinInner) return true;
   if (inner_num > kBlock) return false;  // a lane per position walks the sums
+  if (tile_fits(dim, inner_num)) return false;  // the tile kernels are ahead up to 512 rows ([256,256,196]: 32 us, 65 us here)
   if (inner_num % 16 != 0) return outer_num >= kLongSlabMinSlabs;
   return !softmax && outer_num >= kLongSlabMinSlabsAligned;
 }

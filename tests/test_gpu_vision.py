@@ -122,11 +122,13 @@ def test_softmax(gpu, outer, dim, inner):
 
 
 # Slabs of more than 60 KB over 16 to 256 positions with a few hundred slabs to hand out, a workgroup per slab
-# in chunks of whole rows: positions that are and are not multiples of 16 (Softmax takes only the latter),
-# one row per chunk, the slab counts either side of where the form starts.
+# in chunks of whole rows where the columns are too short or too long for the tile kernels (under 65 or over
+# 512 rows): positions that are and are not multiples of 16 (Softmax takes only the latter), one row per
+# chunk, the slab counts either side of where the form starts; the same shapes inside the tile kernels' range.
 @pytest.mark.parametrize("outer,dim,inner", [(192, 700, 25), (200, 350, 49), (193, 160, 100), (192, 65, 255),
                                              (384, 61, 256), (400, 130, 128), (191, 700, 25), (383, 130, 128),
-                                             (200, 1000, 17), (385, 500, 32), (192, 61, 257)])
+                                             (200, 1000, 17), (385, 500, 32), (192, 61, 257), (192, 600, 100),
+                                             (384, 520, 64), (193, 513, 255)])
 def test_column_ops_over_long_slabs_of_many_positions(gpu, outer, dim, inner):
     x = normal(45, outer * dim * inner, 4.0)
     assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax")
