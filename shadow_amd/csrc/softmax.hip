@@ -928,29 +928,21 @@ struct TileLane {
 
 // Serial fold of one tile column (stride 1 << TS_SHIFT floats in LDS) by one
 // lane, in index order: acc = f(acc, column[c]) for c = 0 .. dim - 1.  The
-// values come in batches of 16 and the next batch is requested before the
-// current one is folded: written as a plain loop, the compiler waits for each
-// pair of LDS reads right before it uses them, and the LDS latency, not the
-// chain of additions, sets the pace (about 130 clocks per two values; 512-long
-// columns then take 14 us per tile).
+// values come in batches of 16 reads that are all requested before the first is
+// folded: written as a plain loop, the compiler waits for each pair of LDS
+// reads right before it uses them, and the LDS latency, not the chain of
+// additions, sets the pace (about 130 clocks per two values; 512-long columns
+// then take 14 us per tile).  One set of registers: the folding waves of the
+// workgroups on a CU share one SIMD, and a second set that the next batch is
+// read into while this one is folded costs that SIMD a move per value.
 template <int TS_SHIFT, typename T, typename F>
 SHDW_DEVICE T fold_tile_column(const float* column, uint32_t dim, T acc, F f) {
   constexpr int kBatch = 16;
   uint32_t c = 0;
-  if (dim >= kBatch) {
+  for (; c + kBatch <= dim; c += kBatch) {
     float v[kBatch];
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) v[u] = column[u << TS_SHIFT];
-    for (c = kBatch; c + kBatch <= dim; c += kBatch) {
-      float w[kBatch];
-#pragma unroll
-      for (int u = 0; u < kBatch; ++u) w[u] = column[(c + u) << TS_SHIFT];
-      __builtin_amdgcn_sched_barrier(0);  // the requests above stay ahead of the fold below
-#pragma unroll
-      for (int u = 0; u < kBatch; ++u) acc = f(acc, v[u]);
-#pragma unroll
-      for (int u = 0; u < kBatch; ++u) v[u] = w[u];
-    }
+    for (int u = 0; u < kBatch; ++u) v[u] = column[(c + u) << TS_SHIFT];
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) acc = f(acc, v[u]);
   }
