@@ -1479,10 +1479,15 @@ __global__ __launch_bounds__(kBlock) void normalize_rows_stream_kernel(const flo
   double acc = 0;
   s.request(x, 0, reg);
   for (uint32_t c0 = 0; c0 < len; c0 += s.step) {
-    s.lay_down(tile, reg, [](const v4f& v, int) { return v; });
+    // the terms of the sums (exactly representable in fp32: they are widened fp32 values) are formed by all
+    // lanes on the way into the tile; the walking lanes, whose every instruction is paid in full, only widen and add
+    s.lay_down(tile, reg, [p](const v4f& v, int) {
+      return v4f{static_cast<float>(norm_term<PMODE>(v[0], p)), static_cast<float>(norm_term<PMODE>(v[1], p)),
+                 static_cast<float>(norm_term<PMODE>(v[2], p)), static_cast<float>(norm_term<PMODE>(v[3], p))};
+    });
     __builtin_amdgcn_wave_barrier();
     if (c0 + s.step < len) s.request(x, c0 + s.step, reg);
-    if (s.lane < G) walk_column(mine, 1, s.cols(c0), [&](float a) { acc += norm_term<PMODE>(a, p); });
+    if (s.lane < G) walk_column(mine, 1, s.cols(c0), [&](float a) { acc += static_cast<double>(a); });
     __builtin_amdgcn_wave_barrier();
   }
   if (s.lane < G) divisors[wave][s.lane] = norm_finish<PMODE>(acc, p, eps);
