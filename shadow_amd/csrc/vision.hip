@@ -496,13 +496,15 @@ struct SmallPlanesArgs {
   FastDiv f_plane_in, f_in_w, f_plane_out, f_out_w, f_row_maxima;  // the last: rows_lds * out_w; for the
                                                                    // wide average: output quads per plane
   FastDiv f_quads_w;  // wide average: output quads per row
+  FastDiv f_out_quads;  // maximum by quads: output quads per plane (f_row_maxima: row-maximum quads per plane)
+  bool quads_max;       // the maximum by quads applies
 };
 
 // SEP with MAX false is the wide average at a column stride of one: a lane takes four
 // neighbouring outputs of a row and reads every cell of their 4 + kw - 1 columns once per
 // window row, adding it to the sums it belongs to - each sum still receives its cells row by
 // row and left to right - in place of 4 kw reads (13x13 on 14x14 maps: 256 us per 51 MB, all
-// of it LDS reads).  The tile has four spare floats behind it for the reads of a row's last,
+// of it LDS reads).  The tile has eight spare floats behind it for the reads of a row's last,
 // partly empty quad.
 template <bool MAX, int K, bool SEP = false>
 __global__ __launch_bounds__(kBlock) void pool_small_planes_kernel(const float* x, float* y, SmallPlanesArgs a) {
@@ -572,6 +574,30 @@ __global__ __launch_bounds__(kBlock) void pool_small_planes_kernel(const float* 
       for (int i = 0; i < a.kh; ++i) {
         const float* row = win + i * a.pitch;
         // cells 0 .. kw+2 of the row piece; cell j belongs to the windows j-3 .. j of the four
+        if (K > 0) {
+          // the window width known: all reads of the row piece are asked for before the first sum
+          // waits for one (a lane otherwise waits out the LDS latency once per cell, with three
+          // waves per SIMD to cover it)
+          // (as 128-bit pieces: the launch keeps the pitch a multiple of four floats for these widths,
+          // and a lane's first column is one; single floats four columns apart from lane to lane meet
+          // in a quarter of the banks)
+          constexpr int kPieces = (K + 3 + 3) / 4;
+          float v[4 * kPieces];
+#pragma unroll
+          for (int q4 = 0; q4 < kPieces; ++q4) {
+            const v4f piece = *reinterpret_cast<const v4f*>(row + 4 * q4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[4 * q4 + e] = piece[e];
+          }
+#pragma unroll
+          for (int j = 0; j < K + 3; ++j) {
+            if (j < K) s0 += v[j];
+            if (j >= 1 && j < K + 1) s1 += v[j];
+            if (j >= 2 && j < K + 2) s2 += v[j];
+            if (j >= 3) s3 += v[j];
+          }
+          continue;
+        }
         float v0 = row[0], v1 = row[1], v2 = row[2];
         s0 += v0;
         s0 += v1, s1 += v1;
@@ -597,6 +623,61 @@ __global__ __launch_bounds__(kBlock) void pool_small_planes_kernel(const float* 
           dst[k] = sums[k] / static_cast<float>(pool_size);
         }
       }
+    }
+    return;
+  }
+  if (SEP && K > 0) {
+    // The two-step maximum for square K x K windows at a column stride of one, four neighbouring outputs
+    // per lane: a row piece of K + 3 cells is read once as 128-bit pieces (the pitch is a multiple of four
+    // floats) and gives four row maxima, which share the fold of the cells 3 .. K - 1; the leftmost of equal
+    // maxima wins in every partial fold, as in the fold cell by cell.  The row maxima lie as quads,
+    // [plane][padded row][quad], so the second step reads a column of K quads.
+    float* row_maxima = tile + a.planes * static_cast<uint32_t>(a.plane_lds);
+    const uint32_t quads_w = a.f_quads_w.d;
+    const uint32_t pieces = np * a.f_row_maxima.d;  // rows_lds * quads_w per plane
+    for (uint32_t t = threadIdx.x; t < pieces; t += kBlock) {
+      uint32_t pl, rem, r, q;
+      fd_divmod(t, a.f_row_maxima, pl, rem);
+      fd_divmod(rem, a.f_quads_w, r, q);
+      const float* row = tile + pl * a.plane_lds + r * a.pitch + 4 * q;
+      constexpr int kPieces = (K + 3 + 3) / 4;
+      float v[4 * kPieces];
+#pragma unroll
+      for (int q4 = 0; q4 < kPieces; ++q4) {
+        const v4f piece = *reinterpret_cast<const v4f*>(row + 4 * q4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[4 * q4 + e] = piece[e];
+      }
+      float core = -FLT_MAX;
+#pragma unroll
+      for (int j = 3; j < K; ++j) core = pool_max(core, v[j]);
+      const float lo = -FLT_MAX;
+      v4f m;
+      m[0] = pool_max(pool_max(pool_max(pool_max(lo, v[0]), v[1]), v[2]), core);
+      m[1] = pool_max(pool_max(pool_max(pool_max(lo, v[1]), v[2]), core), v[K]);
+      m[2] = pool_max(pool_max(pool_max(pool_max(lo, v[2]), core), v[K]), v[K + 1]);
+      m[3] = pool_max(pool_max(pool_max(pool_max(lo, core), v[K]), v[K + 1]), v[K + 2]);
+      *reinterpret_cast<v4f*>(row_maxima + 4 * t) = m;
+    }
+    __syncthreads();
+    const uint32_t out_quads = np * a.f_out_quads.d;  // out_h * quads_w per plane
+    for (uint32_t t = threadIdx.x; t < out_quads; t += kBlock) {
+      uint32_t pl, rem, oh, q;
+      fd_divmod(t, a.f_out_quads, pl, rem);
+      fd_divmod(rem, a.f_quads_w, oh, q);
+      const float* col = row_maxima + 4 * ((pl * a.rows_lds + oh * a.sh) * quads_w + q);
+      v4f v[K > 0 ? K : 1];
+#pragma unroll
+      for (int i = 0; i < K; ++i) v[i] = *reinterpret_cast<const v4f*>(col + 4 * i * quads_w);
+      v4f m = {-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+#pragma unroll
+      for (int i = 0; i < K; ++i)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) m[k] = pool_max(m[k], v[i][k]);
+      float* dst = ys + pl * plane_out + oh * a.out_w + 4 * q;
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (4 * q + k < static_cast<uint32_t>(a.out_w)) dst[k] = m[k];
     }
     return;
   }
@@ -665,6 +746,9 @@ __global__ __launch_bounds__(kBlock) void pool_small_planes_kernel(const float* 
   }
 }
 
+// Window widths whose row pieces the kernels for four outputs per lane unroll and read as 128-bit pieces.
+static bool wide_unrolled(int kw) { return kw == 5 || kw == 7 || kw == 9 || kw == 13; }
+
 // Fills `a` and returns true where the kernel above applies: several padded
 // planes fit the tile and one plane alone would leave lanes idle.
 static bool plan_small_planes(const PoolArgs& p, int64_t total_planes, bool max_pool, SmallPlanesArgs* a,
@@ -681,12 +765,19 @@ static bool plan_small_planes(const PoolArgs& p, int64_t total_planes, bool max_
     return false;
   const int over_b = std::max(0, (p.out_h - 1) * p.sh - p.ph + p.kh - p.in_h);
   const int over_r = std::max(0, (p.out_w - 1) * p.sw - p.pw + p.kw - p.in_w);
-  const int64_t pitch = static_cast<int64_t>(p.pw) + p.in_w + over_r;
-  int64_t plane_lds = (static_cast<int64_t>(p.ph) + p.in_h + over_b) * pitch;
+  const int64_t rows_lds = static_cast<int64_t>(p.ph) + p.in_h + over_b;
+  const int64_t quads_w = (static_cast<int64_t>(p.out_w) + 3) / 4;
+  int64_t pitch = static_cast<int64_t>(p.pw) + p.in_w + over_r;
+  // the maximum by quads where its wider rows leave room for two planes
+  const int64_t pitch4 = (pitch + 3) & ~int64_t{3};
+  const bool quads_max = wide_max && p.sw == 1 && p.kh == p.kw && wide_unrolled(p.kw) &&
+                         (rows_lds * pitch4 + rows_lds * 4 * quads_w) * 2 <= kSmallPlanesTileFloats;
+  if (wide_avg) pitch = wide_unrolled(p.kw) ? pitch4 : pitch | 1;
+  if (quads_max) pitch = pitch4;
+  int64_t plane_lds = rows_lds * pitch;
   plane_lds = (plane_lds + 3) & ~int64_t{3};
   if (plane_lds * 2 > kSmallPlanesTileFloats) return false;
-  const int64_t rows_lds = static_cast<int64_t>(p.ph) + p.in_h + over_b;
-  const int64_t row_maxima = wide_avg ? 0 : rows_lds * p.out_w;
+  const int64_t row_maxima = wide_avg ? 0 : rows_lds * (quads_max ? 4 * quads_w : p.out_w);
   *separable = wide_avg || (wide_max && (plane_lds + row_maxima) * 2 <= kSmallPlanesTileFloats);
   if (plane_out > kSmallPlanesMaxOutputs && !*separable) return false;
   int64_t planes = kSmallPlanesTileFloats / (plane_lds + (*separable ? row_maxima : 0));
@@ -697,9 +788,11 @@ static bool plan_small_planes(const PoolArgs& p, int64_t total_planes, bool max_
   a->kh = p.kh, a->kw = p.kw, a->sh = p.sh, a->sw = p.sw, a->ph = p.ph, a->pw = p.pw;
   a->pitch = static_cast<int>(pitch), a->plane_lds = static_cast<int>(plane_lds);
   a->rows_lds = static_cast<int>(rows_lds);
-  const uint32_t quads_w = (static_cast<uint32_t>(p.out_w) + 3) / 4;
-  a->f_row_maxima = make_fastdiv(wide_avg ? p.out_h * quads_w : static_cast<uint32_t>(row_maxima));
-  a->f_quads_w = make_fastdiv(quads_w);
+  const uint32_t qw = static_cast<uint32_t>(quads_w);
+  a->f_row_maxima = make_fastdiv(wide_avg ? p.out_h * qw : static_cast<uint32_t>(quads_max ? rows_lds * qw : row_maxima));
+  a->f_quads_w = make_fastdiv(qw);
+  a->f_out_quads = make_fastdiv(p.out_h * qw);
+  a->quads_max = quads_max;
   a->planes = static_cast<uint32_t>(planes), a->total_planes = static_cast<uint32_t>(total_planes);
   a->f_plane_in = make_fastdiv(static_cast<uint32_t>(plane_in));
   a->f_in_w = make_fastdiv(static_cast<uint32_t>(p.in_w));
@@ -1021,13 +1114,25 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
     const uint32_t grid = (sp.total_planes + sp.planes - 1) / sp.planes;
     const int k = p.kh == p.kw && (p.kh == 2 || p.kh == 3) ? p.kh : 0;
     if (separable && pool_type == 0) {
-      const size_t both = static_cast<size_t>(sp.planes) * (sp.plane_lds + sp.f_row_maxima.d) * sizeof(float);
-      pool_small_planes_kernel<true, 0, true><<<grid, kBlock, both, st>>>(x, y, sp);
+      const size_t both = static_cast<size_t>(sp.planes) * (sp.plane_lds + (sp.quads_max ? 4 : 1) * sp.f_row_maxima.d) * sizeof(float);
+      switch (sp.quads_max ? p.kw : 0) {  // the common square windows at a column stride of one: by quads
+        case 5: pool_small_planes_kernel<true, 5, true><<<grid, kBlock, both, st>>>(x, y, sp); break;
+        case 7: pool_small_planes_kernel<true, 7, true><<<grid, kBlock, both, st>>>(x, y, sp); break;
+        case 9: pool_small_planes_kernel<true, 9, true><<<grid, kBlock, both, st>>>(x, y, sp); break;
+        case 13: pool_small_planes_kernel<true, 13, true><<<grid, kBlock, both, st>>>(x, y, sp); break;
+        default: pool_small_planes_kernel<true, 0, true><<<grid, kBlock, both, st>>>(x, y, sp);
+      }
       return launch_status();
     }
-    if (separable) {  // the wide average: four spare floats behind the planes
-      const size_t spare = (static_cast<size_t>(sp.planes) * sp.plane_lds + 4) * sizeof(float);
-      pool_small_planes_kernel<false, 0, true><<<grid, kBlock, spare, st>>>(x, y, sp);
+    if (separable) {  // the wide average: eight spare floats behind the planes
+      const size_t spare = (static_cast<size_t>(sp.planes) * sp.plane_lds + 8) * sizeof(float);
+      switch (wide_unrolled(p.kw) ? p.kw : 0) {
+        case 5: pool_small_planes_kernel<false, 5, true><<<grid, kBlock, spare, st>>>(x, y, sp); break;
+        case 7: pool_small_planes_kernel<false, 7, true><<<grid, kBlock, spare, st>>>(x, y, sp); break;
+        case 9: pool_small_planes_kernel<false, 9, true><<<grid, kBlock, spare, st>>>(x, y, sp); break;
+        case 13: pool_small_planes_kernel<false, 13, true><<<grid, kBlock, spare, st>>>(x, y, sp); break;
+        default: pool_small_planes_kernel<false, 0, true><<<grid, kBlock, spare, st>>>(x, y, sp);
+      }
       return launch_status();
     }
     const size_t lds = static_cast<size_t>(sp.planes) * sp.plane_lds * sizeof(float);

@@ -394,6 +394,11 @@ POOL_2D = [
     ((1, 3, 33, 65), [4, 6], [1, 1], [3, 3], False), ((1, 2, 70, 70), [7], [1], [3], False),
     ((1, 1, 30, 130), [9, 5], [1, 1], [4, 2], True), ((1, 2, 112, 112), [5], [1], [2], False),
     ((1, 1, 64, 300), [3], [1], [1], True), ((1, 2, 28, 61), [13], [1], [6], False),
+    # small planes, square windows of 5, 7, 9, 13 at a column stride of 1, four outputs per lane from 128-bit
+    # row pieces: output rows that end 1, 2, 3 outputs into a quad, a row stride of 2 and 3, no padding,
+    # overhanging windows; 11 wide: the same lanes cell by cell
+    ((3, 5, 17, 17), [7], [2, 1], [3], True), ((2, 4, 21, 18), [9], [1], [4], False), ((2, 6, 15, 15), [5], [1], [0], False),
+    ((5, 3, 12, 22), [13], [3, 1], [6], True), ((2, 3, 11, 11), [11], [1], [5], False), ((9, 2, 13, 13), [13], [1], [6], False),
 ]
 
 
@@ -413,7 +418,8 @@ def test_pooling2d_op(ws, pool, shape, kernel, stride, pad, full):
 # returns the cell the row-major walk returns.
 @pytest.mark.parametrize("shape,kernel,pad", [((3, 4, 13, 13), [5], [2]), ((2, 3, 14, 14), [13], [6]),
                                                ((2, 2, 19, 19), [9], [4]), ((1, 3, 56, 56), [5], [2]),
-                                               ((1, 2, 40, 61), [7], [3]), ((1, 2, 45, 50), [3], [1])])
+                                               ((1, 2, 40, 61), [7], [3]), ((1, 2, 45, 50), [3], [1]),
+                                               ((2, 3, 15, 17), [7], [3])])
 def test_max_pooling_ties_and_nans_in_wide_windows(ws, shape, kernel, pad):
     rng = np.random.default_rng(31)
     pick = rng.integers(0, 6, size=shape)
