@@ -843,7 +843,7 @@ __global__ __launch_bounds__(kBlock) void normalize_packed_kernel(const float* x
                    [&](float v, uint32_t cq, uint32_t c) { return ssd_scaled<SM>(v / stat[cq], scale, c); });
 }
 
-// Columns of 65 to 512 elements over a wide inner extent: a workgroup owns a
+// Columns of 65 to 1024 elements over a wide inner extent: a workgroup owns a
 // tile of TS = 64, 32 or 16 neighbouring positions with all their `dim` elements,
 // 64 KB at most, so x is read from HBM once.  Each lane keeps its share of the
 // tile (16 vectors of 4 positions at most) in registers and also parks it in
@@ -898,13 +898,18 @@ struct TileLane {
       }
     }
   }
-  SHDW_DEVICE void park(float* lds, const v4f (&r)[kTilePerLane]) const {
+  // f(v): what the folding lanes are to find in the tile for the vector v
+  template <typename F>
+  SHDW_DEVICE void park(float* lds, const v4f (&r)[kTilePerLane], F f) const {
     if (valid == 0) return;
 #pragma unroll
     for (int u = 0; u < kTilePerLane; ++u) {
       const uint32_t c = c0 + u * STEP;
-      if (c < dim) *reinterpret_cast<v4f*>(lds + (c << TS_SHIFT) + j) = r[u];
+      if (c < dim) *reinterpret_cast<v4f*>(lds + (c << TS_SHIFT) + j) = f(r[u]);
     }
+  }
+  SHDW_DEVICE void park(float* lds, const v4f (&r)[kTilePerLane]) const {
+    park(lds, r, [](const v4f& v) { return v; });
   }
   SHDW_DEVICE void store(float* ys, uint32_t u, v4f v) const {
     const uint32_t c = c0 + u * STEP;
@@ -966,12 +971,17 @@ __global__ __launch_bounds__(kBlock) void normalize_tile_kernel(const float* x, 
   const TileLane<TS_SHIFT, ROWS> lane(width, dim, inner);
   v4f r[kTilePerLane];
   lane.load(x + base, r);
-  lane.park(lds, r);
+  // the tile holds the terms of the sums, fp32 values that widen exactly: the folding wave's chain sets the
+  // pace of a tall, narrow tile, and every instruction taken off it is time off the tile
+  lane.park(lds, r, [p](const v4f& v) {
+    return v4f{static_cast<float>(norm_term<PMODE>(v[0], p)), static_cast<float>(norm_term<PMODE>(v[1], p)),
+               static_cast<float>(norm_term<PMODE>(v[2], p)), static_cast<float>(norm_term<PMODE>(v[3], p))};
+  });
   __syncthreads();
   if (threadIdx.x < width) {  // width <= TS <= 64: lanes of wave 0, one column each
     const float* column = lds + threadIdx.x;
-    const double acc = fold_tile_column<TS_SHIFT>(
-        column, dim, 0.0, [p](double a, float v) { return a + norm_term<PMODE>(v, p); });
+    const double acc =
+        fold_tile_column<TS_SHIFT>(column, dim, 0.0, [](double a, float t) { return a + static_cast<double>(t); });
     lds[threadIdx.x] = norm_finish<PMODE>(acc, p, eps);
   }
   __syncthreads();
@@ -988,7 +998,7 @@ __global__ __launch_bounds__(kBlock) void normalize_tile_kernel(const float* x, 
   }
 }
 
-constexpr int kTileMinDim = 65, kTileMaxDim = 512, kTileMinInner = 16;
+constexpr int kTileMinDim = 65, kTileMaxDim = 1024, kTileMinInner = 16;
 constexpr int kTileLdsBytes = 65536;
 
 static int tile_rows(int inner_num, const float* y) {
@@ -996,8 +1006,15 @@ static int tile_rows(int inner_num, const float* y) {
   return inner_num % 4 == 0 ? kRowsQuad : kRowsAny;
 }
 
-static bool tile_fits(int dim, int inner_num) {
-  return dim >= kTileMinDim && dim <= kTileMaxDim && inner_num >= kTileMinInner;
+// Columns of 513 to 1024 rows take tiles of 16 positions (64-byte row pieces), which pay from 32 (Softmax)
+// or 64 (Normalize) positions on: [127,513,196] softmax 89 -> 39 us, normalize 68 -> 31; [65,1000,196]
+// 94 -> 51, 69 -> 41; below, the slab kernels stay ahead ([513,1000,25] normalize 46 against 61).
+constexpr int kTileWideDim = 512, kTileMinInnerTallSoftmax = 32, kTileMinInnerTallNormalize = 64;
+
+static bool tile_fits(int dim, int inner_num, bool softmax) {
+  if (dim < kTileMinDim || dim > kTileMaxDim) return false;
+  if (dim <= kTileWideDim) return inner_num >= kTileMinInner;
+  return inner_num >= (softmax ? kTileMinInnerTallSoftmax : kTileMinInnerTallNormalize);
 }
 
 template <int PMODE, int SM, int TS_SHIFT>
@@ -1031,11 +1048,13 @@ static void launch_normalize_tile(int outer_num, int dim, int inner_num, float p
   // tile that fits.
   if (dim * 64 * sizeof(float) <= kTileLdsBytes / 2)
     launch_normalize_tile_ts<PMODE, SM, 6>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
-  else
+  else if (dim * 32 * sizeof(float) <= kTileLdsBytes)
     launch_normalize_tile_ts<PMODE, SM, 5>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
+  else
+    launch_normalize_tile_ts<PMODE, SM, 4>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
 }
 
-// Softmax on the same tile layout (65 <= dim <= 512).  The lanes hold x, later
+// Softmax on the same tile layout (65 <= dim <= 1024).  The lanes hold x, later
 // exp(x - max), in registers.  Behind the tile lie the exp table, a row that
 // hands the maxima and later the sums over, and a flag.
 //
@@ -1140,7 +1159,7 @@ __global__ __launch_bounds__(kBlock) void softmax_tile_kernel(const float* x, fl
 
 constexpr size_t kExpTabBytes = 32 * sizeof(uint64_t);
 constexpr size_t kSoftmaxTileExtraBytes = kExpTabBytes + 64 * sizeof(float) + 16;  // table, hand-over row, flag
-constexpr int kSoftmaxTileMaxDim = kTileMaxDim;  // 32 positions of 512 channels plus the exp table: 64 KB + 256 bytes, two workgroups per CU all the same
+// (32 positions of 512 channels, or 16 of 1024, plus the exp table: 64 KB + 256 bytes, two workgroups per CU all the same)
 
 template <int TS_SHIFT>
 static void launch_softmax_tile_ts(int outer_num, int dim, int inner_num, const float* x, float* y,
@@ -2041,7 +2060,7 @@ static bool long_slab(int outer_num, int dim, int inner_num, bool softmax) {
   if (static_cast<int64_t>(dim) * inner_num <= kLongSlabMinFloats) return false;
   if (static_cast<uint32_t>(inner_num) < kTallMinInner) return true;
   if (inner_num > kBlock) return false;  // a lane per position walks the sums
-  if (tile_fits(dim, inner_num)) return false;  // the tile kernels are ahead up to 512 rows ([256,256,196]: 32 us, 65 us here)
+  if (tile_fits(dim, inner_num, softmax)) return false;  // the tile kernels are ahead where they apply ([256,256,196]: 32 us, 65 us here)
   if (inner_num % 16 != 0) return outer_num >= kLongSlabMinSlabs;
   return !softmax && outer_num >= kLongSlabMinSlabsAligned;
 }
@@ -2173,10 +2192,12 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
     else
       softmax_columns_reg_kernel<64, 48><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi);
   }
-  else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner && dim * 64 * sizeof(float) <= kTileLdsBytes - 1024)
+  else if (tile_fits(dim, inner_num, true) && dim * 64 * sizeof(float) <= kTileLdsBytes - 1024)
     launch_softmax_tile_ts<6>(outer_num, dim, inner_num, x, y, st);
-  else if (dim <= kSoftmaxTileMaxDim && inner_num >= kTileMinInner)
+  else if (tile_fits(dim, inner_num, true) && dim * 32 * sizeof(float) <= kTileLdsBytes)
     launch_softmax_tile_ts<5>(outer_num, dim, inner_num, x, y, st);
+  else if (tile_fits(dim, inner_num, true))
+    launch_softmax_tile_ts<4>(outer_num, dim, inner_num, x, y, st);
   else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, &t))
     softmax_tall_kernel<<<t.grid, kBlock, 0, st>>>(x, y, static_cast<uint32_t>(dim), static_cast<uint32_t>(inner_num),
                                                    t.width_log2, t.f_tiles);
@@ -2232,7 +2253,7 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
       normalize_slab_kernel<2><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
     else
       normalize_slab_kernel<0><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
-  } else if (mode != 0 && tile_fits(dim, inner_num)) {
+  } else if (mode != 0 && tile_fits(dim, inner_num, false)) {
     if (mode == 1)
       launch_normalize_tile<1, kSsdNoScale>(outer_num, dim, inner_num, p, eps, x, nullptr, y, st);
     else
@@ -2299,7 +2320,7 @@ static void launch_ssd_columns(const ColumnGeometry& g, int outer_num, int dim, 
     normalize_long_slab_kernel<3, SM><<<outer_num, kBlock, 0, st>>>(x, y, d, fi, 2.f, eps, scale);
   else if (g.use_slab)
     normalize_slab_kernel<3, SM><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, 2.f, eps, scale);
-  else if (tile_fits(dim, inner_num))
+  else if (tile_fits(dim, inner_num, false))
     launch_normalize_tile<3, SM>(outer_num, dim, inner_num, 2.f, eps, x, scale, y, st);
   else if (dim <= 16)
     normalize_columns_reg_kernel<3, 16, SM><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, 2.f, eps, scale);

@@ -128,7 +128,12 @@ def test_softmax(gpu, outer, dim, inner):
 @pytest.mark.parametrize("outer,dim,inner", [(192, 700, 25), (200, 350, 49), (193, 160, 100), (192, 65, 255),
                                              (384, 61, 256), (400, 130, 128), (191, 700, 25), (383, 130, 128),
                                              (200, 1000, 17), (385, 500, 32), (192, 61, 257), (192, 600, 100),
-                                             (384, 520, 64), (193, 513, 255)])
+                                             (384, 520, 64), (193, 513, 255),
+                                             # columns of 513 to 1024 rows in tiles of 16 positions: rows on 64-byte
+                                             # boundaries, on multiples of four, ending inside a lane's four; the
+                                             # position counts either side of where Softmax and Normalize take them
+                                             (2, 1024, 64), (3, 513, 196), (2, 1000, 67), (1, 700, 130), (5, 1023, 33),
+                                             (2, 600, 49), (3, 1024, 31), (2, 800, 63)])
 def test_column_ops_over_long_slabs_of_many_positions(gpu, outer, dim, inner):
     x = normal(45, outer * dim * inner, 4.0)
     assert_bit_exact(gpuops.softmax(x, outer, dim, inner), oracle.softmax(x, outer, dim, inner), "softmax")
