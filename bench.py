@@ -10,7 +10,9 @@ Inputs are generated from fixed seeds, uploaded once and stay resident in HBM
 (two copies of the input take turns, 411 MB, more than the 256 MB Infinity
 Cache); the timed region is K steps between two stream synchronisations.
 
-Prints ONE JSON line.  `value` is algorithmic GB/s of the whole step
+Prints ONE JSON line on stdout, under 4 KB (see final_record); every row of the
+measurement goes to the --table file and, one short text line per row, to stderr.
+`value` is algorithmic GB/s of the whole step
 (compulsory reads + writes of every op / wall time).  `roofline` describes the
 kernel that takes the largest share of the step, timed with HIP events on the
 launch stream inside the timed region; its `bound` is "hbm" unless the kernel
@@ -99,6 +101,8 @@ def parse():
                          "small extents) against a plain copy of the same bytes, print a table, exit")
     ap.add_argument("--probe-next", action="store_true",
                     help="the same for the neighbouring operators and the data movers")
+    ap.add_argument("--table", default=os.path.join(ROOT, "gpurun_out", "bench_table.json"),
+                    help="file that receives every row of the measurement; the final stdout line is a short record")
     return ap.parse_args()
 
 
@@ -967,6 +971,66 @@ def network_forward(dev, reps=50):
             "bytes_moved": moved, "GBps": round(moved / us / 1e3, 1)}
 
 
+SHORT_OP = {"binary_add_channel_broadcast": "add_chan_bcast", "fused_tail (CPU: the four operators)": "fused_tail"}
+FINAL_LINE_LIMIT = 4096  # the driver keeps a bounded tail of stdout: the record has to fit in it whole
+
+
+def final_record(full, table_path=None):
+    """The one line printed last: the fields the contract names, the roofline of the
+    dominant kernel, the CPU baseline and one short row per BASELINE operator
+    ([cfg, op, us, frac of 8 TB/s, frac of the same-size ceiling, cpu_us]).  Everything
+    else (per-op step table, neighbouring operators, movers, ceilings, notes) stays in
+    the table file.  Kept free of device calls so that its size can be tested anywhere."""
+    keep = ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+            "vs_baseline", "dtype", "data", "config", "frac_of_hbm_peak", "elements_per_s")
+    rec = {k: full[k] for k in keep if k in full}
+    roof = dict(full["roofline"])
+    for k in ("note", "traffic_source", "valu_source"):
+        roof.pop(k, None)
+    rec["roofline"] = roof
+    if "cpu_baseline" in full:
+        rec["cpu_baseline"] = {k: v for k, v in full["cpu_baseline"].items() if k != "ops"}
+        rec["speedup_vs_cpu"] = full.get("speedup_vs_cpu")
+    rec["step_ops"] = [[d["op"], d["us"], d["frac"]] for d in full.get("step_ops", []) if "yardstick" not in d["op"]]
+    rows = [r for r in full.get("configs", []) if r["cfg"] in (1, 3, 4, 5)]
+    if rows:
+        rec["baseline_rows_columns"] = ["cfg", "op", "us", "frac", "of_ceiling", "cpu_us"]
+        rec["baseline_rows"] = [[r["cfg"], SHORT_OP.get(r["op"], r["op"]), r["us"], round(r["frac"], 3),
+                                 round(r["frac_of_ceiling"], 2), r.get("cpu_us") and round(r["cpu_us"])] for r in rows]
+        big = [r for r in rows if r["bytes"] >= (8 << 20)]  # cfg 4(iii) is a 1 MB tensor: launch-bound by size
+        worst = min(big, key=lambda r: r["frac_of_ceiling"])
+        rec["worst_of_ceiling"] = [worst["cfg"], SHORT_OP.get(worst["op"], worst["op"]), worst["frac_of_ceiling"]]
+    if "network" in full:
+        rec["network"] = {k: v for k, v in full["network"].items() if k != "model"}
+    if table_path:
+        rec["table"] = table_path
+    return rec
+
+
+def final_line(full, table_path=None):
+    """final_record as one line of JSON below FINAL_LINE_LIMIT.  Should a host with a long
+    device or CPU name push it over, the optional tables go first (they are in the file)."""
+    rec = final_record(full, table_path)
+    for optional in (None, "step_ops", "baseline_rows", "baseline_rows_columns", "network"):
+        rec.pop(optional, None)
+        line = json.dumps(rec, separators=(",", ":"))
+        if len(line) < FINAL_LINE_LIMIT:
+            return line
+    raise RuntimeError("bench.py: the final record is %d characters, the limit is %d" % (len(line), FINAL_LINE_LIMIT))
+
+
+def write_table(full, path):
+    """The whole measurement (every row, every note) as a JSON file; None when the
+    directory cannot be written (the final line then names no table)."""
+    try:
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        with open(path, "w") as f:
+            json.dump(full, f, indent=1)
+        return os.path.relpath(path, ROOT)
+    except OSError:
+        return None
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -1018,7 +1082,12 @@ def main():
                                "way (rows at the end); cpu_us: the oracle's C loop for the same operator on this "
                                "host, one thread, outputs allocated beforehand, best of %d" % args.cpu_passes)
         out["network"] = network_forward(dev)
-    print(json.dumps(out))
+    table = write_table(out, args.table)
+    for r in out.get("configs", []):
+        print("%-8s %-62s %9.2f us  %.3f of 8 TB/s%s" % (r["cfg"], r["op"], r["us"], r["frac"],
+              "  %.3f of ceiling" % r["frac_of_ceiling"] if "frac_of_ceiling" in r else ""), file=sys.stderr)
+    sys.stderr.flush()
+    print(final_line(out, table), flush=True)
 
 
 if __name__ == "__main__":
