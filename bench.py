@@ -101,6 +101,9 @@ def parse():
                          "small extents) against a plain copy of the same bytes, print a table, exit")
     ap.add_argument("--probe-next", action="store_true",
                     help="the same for the neighbouring operators and the data movers")
+    ap.add_argument("--launch-shapes", action="store_true",
+                    help="run tests/native/launch_shapes (alternative launch shapes of the streaming, strided-reduce "
+                         "and channel-tile kernels), print its table and how the shapes in use compare, exit")
     ap.add_argument("--table", default=os.path.join(ROOT, "gpurun_out", "bench_table.json"),
                     help="file that receives every row of the measurement; the final stdout line is a short record")
     return ap.parse_args()
@@ -482,6 +485,56 @@ def sweep(dev):
     print("worst of each family:")
     for family, (ratio, name) in worst.items():
         print("  %-14s %6.2f x copy  (%s)" % (family, ratio, name))
+
+
+def launch_shapes():
+    """Timing comparison of the launch shapes the library uses against their alternatives
+    (tests/native/launch_shapes.hip).  A report, not a gate: each line ends in `ok` or `BEHIND`."""
+    import subprocess
+    exe = os.path.join(ROOT, "tests", "native", "launch_shapes")
+    if not os.path.exists(exe):
+        raise SystemExit("bench.py: tests/native/launch_shapes is not built; run `python -m tests.native.build`")
+    out = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    print(out.stdout)
+    if out.returncode != 0:
+        raise SystemExit("bench.py: launch_shapes exited with %d" % out.returncode)
+    table, slack = out.stdout, 1.12
+
+    def verdict(what, mine, best, bound):
+        print("%-72s %8.2f vs %8.2f  %s" % (what, mine, best, "ok" if mine <= bound * best else "BEHIND"))
+
+    # elementwise kernels: single waves, one vector per lane; Blas::Set: 256 lanes; the read probe: 1024 lanes
+    used = {"copy": "T64x1", "write": "T256x1", "read": "T1024x1"}
+    for m in re.finditer(r"stream (\w+)\s+(\d+) MB:(.*)", table):
+        row = {k: float(v) for k, v in re.findall(r"(\S+x\d) (\d+\.\d+)", m.group(3))}
+        if m.group(1) in used and row:
+            verdict("stream %s %s MB, %s against the best of %d shapes (us)" % (m.group(1), m.group(2), used[m.group(1)],
+                                                                              len(row)), row[used[m.group(1)]],
+                    min(row.values()), slack)
+    t = {(int(l), kind): float(us) for l, kind, us, _ in re.findall(r"strided L(\d+)\s+(\S+)\s+(\d+\.\d+) (\w+)", table)}
+    if (32, "xcd-contiguous") in t:
+        verdict("strided reduce, 32-wide tiles numbered XCD-contiguously against the best (us)",
+                t[(32, "xcd-contiguous")], min(t.values()), slack)
+    flat, rows = {}, {}
+    for line in table.splitlines():
+        m = re.match(r"tile \[(\d+),(\d+),(\d+)\] flat (\d+\.\d+)", line)
+        if m:
+            flat[int(m.group(3))] = float(m.group(4))
+        m = re.match(r"tile \[(\d+),(\d+),(\d+)\] (T\d+x\d+) (\w+)\s+(\w+)\s+(\d+\.\d+) (\w+)", line)
+        if m:
+            rows[(int(m.group(3)), m.group(4), m.group(5), m.group(6))] = float(m.group(7))
+    for inner, shape in ((3136, ("T256x16", "streaming", "parked")), (1444, ("T256x16", "plain", "parked"))):
+        mine = {k[1:]: v for k, v in rows.items() if k[0] == inner}
+        if shape in mine:
+            verdict("channel tile, rows of %d: %s against the best variant (us)" % (inner, " ".join(shape)),
+                    mine[shape], min(mine.values()), slack)
+            print("%-72s %8.2f vs %8.2f" % ("  the pattern against a flat copy of the same bytes (us)",
+                                            min(mine.values()), flat.get(inner, float("nan"))))
+    chains = {(int(w), int(c)): (float(a), float(b))
+              for w, c, a, b in re.findall(r"add chain waves (\d+) chains (\d+): (\d+\.\d+) (\d+\.\d+)", table)}
+    if (1, 1) in chains and (8, 1) in chains:
+        print("%-72s %8.2f vs %8.2f" % ("one dependent add chain alone on a SIMD against eight waves sharing it",
+                                        chains[(1, 1)][0], chains[(8, 1)][1]))
 
 
 # ------------------------------------------------------------- CPU baseline
@@ -1036,6 +1089,9 @@ def main():
     if args.gpus != 1:
         raise SystemExit("bench.py: this build measures one GPU; the path shards by batch with no "
                          "exchange, so run one process per GPU (got --gpus %d)" % args.gpus)
+    if args.launch_shapes:
+        launch_shapes()
+        return
     dev = Dev()
     if args.sweep:
         sweep(dev)

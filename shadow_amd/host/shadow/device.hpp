@@ -43,13 +43,10 @@ class Context {
   virtual void synchronize() = 0;
   virtual void* stream() const { return nullptr; }
 
-  // Device scratch that lives as long as the context, grow-only, for the level-1
-  // routines whose signature carries no Workspace (BlasSasum): what the cuBLAS
-  // handle's own workspace was in the reference.  Valid until the next call with
-  // a larger size; one stream, so one user at a time.
-  virtual void* level1_scratch(size_t bytes) { return nullptr; }
-
-  // Vendor-library handles of the reference; nothing on this path uses them.
+  // Vendor-library handles of the reference.  The GPU context of this build answers
+  // cublas_handle() with its Level1Handle (src/level1_handle.hpp): the device scratch
+  // of the level-1 routines, which is what the cuBLAS handle's own workspace was.
+  // Nothing on this path uses the other three.
   virtual void* cublas_handle() const { return nullptr; }
   virtual void* cudnn_handle() const { return nullptr; }
   virtual void* nnpack_handle() const { return nullptr; }

@@ -3,6 +3,7 @@
 // shadow/core/blas.cu:11-138.
 #include "shadow/blas.hpp"
 
+#include "level1_handle.hpp"
 #include "shadow_hip.h"
 
 namespace Shadow {
@@ -79,16 +80,17 @@ void BlasSaxpy<G, float>(int n, float alpha, const float* x, int offx, float* y,
 template <>
 void BlasSasum<G, float>(int n, const float* x, int offx, float* y, Context* ctx) {
   // The signature has no Workspace to borrow scratch from (it did not need one
-  // on top of cuBLAS): the partial sums live in the context's own scratch, which
-  // is allocated once.  The reference calls this once per batch item
+  // on top of cuBLAS): the partial sums live in the scratch behind the context's
+  // cublas_handle() slot, which is allocated with the context.  The reference calls this once per batch item
   // (kernels/ssd_normalize.hpp:51-57); an allocation per call would stall the
   // device every time.
   CHECK_NOTNULL(ctx);
   const int shape[1] = {n}, axes[1] = {0};
   const size_t bytes = shdw_hip_reduce_workspace_bytes(1, shape, 1, axes) + 16;
-  void* scratch = ctx->level1_scratch(bytes);
-  CHECK_NOTNULL(scratch);
-  SHADOW_HIP_CHECK(shdw_hip_asum(n, x + offx, y, scratch, bytes, stream_of(ctx)));
+  const Level1Handle* handle = static_cast<const Level1Handle*>(ctx->cublas_handle());
+  CHECK_NOTNULL(handle);
+  CHECK_LE(bytes, handle->bytes) << "BlasSasum: the context's level-1 scratch is too small";
+  SHADOW_HIP_CHECK(shdw_hip_asum(n, x + offx, y, handle->scratch, bytes, stream_of(ctx)));
 }
 
 }  // namespace Blas

@@ -1,5 +1,6 @@
 #include "shadow/device.hpp"
 
+#include "level1_handle.hpp"
 #include "shadow_hip.h"
 
 namespace Shadow {
@@ -63,25 +64,12 @@ class HipContext : public Context {
     }
     allocator_ = GetAllocator<DeviceType::kGPU>();
     allocator_->set_stream(stream_);
+    SHADOW_HIP_CHECK(shdw_hip_malloc(&level1_.scratch, kLevel1Scratch));
+    level1_.bytes = kLevel1Scratch;
   }
   ~HipContext() override {
-    if (scratch_ != nullptr) shdw_hip_free(scratch_);
+    if (level1_.scratch != nullptr) shdw_hip_free(level1_.scratch);
     if (own_stream_ && stream_ != nullptr) shdw_hip_stream_destroy(stream_);
-  }
-
-  void* level1_scratch(size_t bytes) override {
-    if (bytes > scratch_bytes_) {
-      // the old buffer may still be in use by work enqueued on the stream
-      if (scratch_ != nullptr) {
-        synchronize();
-        SHADOW_HIP_CHECK(shdw_hip_free(scratch_));
-        scratch_ = nullptr;
-      }
-      const size_t want = bytes < kMinScratch ? kMinScratch : bytes;
-      SHADOW_HIP_CHECK(shdw_hip_malloc(&scratch_, want));
-      scratch_bytes_ = want;
-    }
-    return scratch_;
   }
 
   Allocator* allocator() const override { return allocator_.get(); }
@@ -90,6 +78,7 @@ class HipContext : public Context {
   void switch_device() override { SHADOW_HIP_CHECK(shdw_hip_set_device(device_id_)); }
   void synchronize() override { SHADOW_HIP_CHECK(shdw_hip_stream_sync(stream_)); }
   void* stream() const override { return stream_; }
+  void* cublas_handle() const override { return const_cast<Level1Handle*>(&level1_); }
 
  private:
   int device_id_ = 0;
@@ -97,9 +86,8 @@ class HipContext : public Context {
   void* stream_ = nullptr;
   std::shared_ptr<Allocator> allocator_;
   // 4096 partial sums of 8 bytes and the result: what BlasSasum needs for any n
-  static constexpr size_t kMinScratch = 64 * 1024;
-  void* scratch_ = nullptr;
-  size_t scratch_bytes_ = 0;
+  static constexpr size_t kLevel1Scratch = 64 * 1024;
+  Level1Handle level1_;
 };
 
 }  // namespace
