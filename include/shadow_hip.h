@@ -249,6 +249,18 @@ int shdw_hip_scale_residual_relu_rowmean(int n, int scale_num, int inner_num,
                                          const float* bias, const float* residual,
                                          float* y, float* mean, void* stream);
 
+/* The same sequence in the forms a converted network holds it in (the Native
+ * backend's fusion pass calls this one): `scale` or `bias` may be NULL (the Scale
+ * operator with has_scale or has_bias only: s = x*scale[c], or s = x + bias[c]);
+ * residual_first != 0 when the residual is the Eltwise operator's first input,
+ * y = relu((0 + 1*residual) + 1*s); `mean` may be NULL when no Reduce follows
+ * (y is then required), `y` may be NULL when only the mean is wanted.
+ * ref: shadow/operators/scale_op.cpp:25-33, eltwise_op.cpp:19-34,
+ *      shadow/python/converter/shadow/optimizer.py:155-394 (where the reference fuses) */
+int shdw_hip_scale_residual_relu(int n, int scale_num, int inner_num, const float* x,
+                                 const float* scale, const float* bias, const float* residual,
+                                 int residual_first, float* y, float* mean, void* stream);
+
 /* ==================== neighbouring operators of the path ==================== */
 
 /* Axpy: out[r*inner_num + i] = y[..] + alpha[r] * x[..] for r < outer_num

@@ -205,8 +205,8 @@ HOST_SIGNATURES = {
     "shdw_host_op_debug_log": (_I, [_V, _V, ctypes.c_char_p, _Z]),
     "shdw_host_parse_net": (_I, [ctypes.c_char_p, ctypes.c_char_p, _Z]),
     "shdw_host_backend_keys": (_I, [ctypes.c_char_p, _Z]),
-    "shdw_host_network_create": (_V, [ctypes.c_char_p, _I, _I, _I, ctypes.c_char_p, _V]),
-    "shdw_host_network_create_from_binary": (_V, [ctypes.c_char_p, _I, _I, _I, _V, _I, _I]),
+    "shdw_host_network_create": (_V, [ctypes.c_char_p, _I, _I, _I, _I, ctypes.c_char_p, _V]),
+    "shdw_host_network_create_from_binary": (_V, [ctypes.c_char_p, _I, _I, _I, _I, _V, _I, _I]),
     "shdw_host_parse_net_binary": (_I, [_V, _I, _I, ctypes.c_char_p, _Z]),
     "shdw_host_proto_reencode": (_I, [_V, _I, _I, _V, _Z]),
     "shdw_host_serialize_net": (_I, [ctypes.c_char_p, _V, _Z]),
@@ -394,25 +394,26 @@ class Network:
 
     @classmethod
     def from_binary(cls, data, network_index=-1, backend_type="Native", device_id=0, debug=False,
-                    device_input=False):
+                    device_input=False, fuse=True):
         self = cls.__new__(cls)
         self.lib = host()
         self.device_input = device_input
         data = bytes(data)
         self.ptr = self.lib.shdw_host_network_create_from_binary(
-            backend_type.encode(), device_id, int(debug), int(device_input), data, len(data), network_index)
+            backend_type.encode(), device_id, int(debug), int(device_input), int(fuse), data, len(data),
+            network_index)
         host_check(self.ptr)
         return self
 
     def __init__(self, proto_text, weights=None, backend_type="Native", device_id=0, debug=False,
-                 device_input=False):
+                 device_input=False, fuse=True):
         self.lib = host()
         self.device_input = device_input
         packed = None
         if weights is not None and len(weights):
             packed = np.concatenate([np.ascontiguousarray(w, np.float32).ravel() for w in weights])
         self.ptr = self.lib.shdw_host_network_create(
-            backend_type.encode(), device_id, int(debug), int(device_input), proto_text.encode(),
+            backend_type.encode(), device_id, int(debug), int(device_input), int(fuse), proto_text.encode(),
             packed.ctypes.data if packed is not None else None)
         host_check(self.ptr)
 
@@ -429,6 +430,11 @@ class Network:
     @property
     def out_blob(self):
         return self._names(1)
+
+    @property
+    def fused(self):
+        """One line per group of operators that the backend runs as one launch."""
+        return self._names(2)
 
     def forward(self, inputs, reshape=False):
         """inputs: {blob name: float32 array}.  reshape=True passes each array's

@@ -17,13 +17,18 @@
 
 namespace shdw {
 
+// The operator sequence on one element.  HAS_SCALE / HAS_BIAS: which parameter
+// blobs the Scale operator has (Vision::ScaleBias, Scale or Bias); RES_FIRST: the
+// residual is the Eltwise operator's first input and the scaled value its second.
+template <bool HAS_SCALE, bool HAS_BIAS, bool RES_FIRST>
 SHDW_DEVICE float tail_element(float x, float s, float b, float r) {
-  float t = x * s;
-  t = t + b;
-  float u = 1.0f * t;
-  u = 0.0f + u;
-  const float v = 1.0f * r;
-  u = u + v;
+  float t = x;
+  if (HAS_SCALE) t = t * s;
+  if (HAS_BIAS) t = t + b;
+  // Eltwise SUM with unit coefficients: Set(0), then y += 1 * input, input by input
+  const float first = 1.0f * (RES_FIRST ? r : t), second = 1.0f * (RES_FIRST ? t : r);
+  float u = 0.0f + first;
+  u = u + second;
   return u > 0 ? u : 0;
 }
 
@@ -37,7 +42,7 @@ SHDW_DEVICE double wave_sum_f64(double v) {
   return v;
 }
 
-template <bool VEC, bool WRITE_Y>
+template <bool VEC, bool WRITE_Y, bool MEAN, bool HAS_SCALE, bool HAS_BIAS, bool RES_FIRST>
 __global__ __launch_bounds__(kBlock) void scale_residual_relu_rowmean_kernel(
     const float* x, const float* scale, const float* bias, const float* res, float* y,
     float* mean, uint32_t rows, uint32_t inner, FastDiv num) {
@@ -45,7 +50,7 @@ __global__ __launch_bounds__(kBlock) void scale_residual_relu_rowmean_kernel(
   const uint32_t row = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
   if (row >= rows) return;  // wave-uniform
   const uint32_t c = row - fd_div(row, num) * num.d;
-  const float s = scale[c], b = bias[c];
+  const float s = HAS_SCALE ? scale[c] : 1.0f, b = HAS_BIAS ? bias[c] : 0.0f;
   const size_t base = static_cast<size_t>(row) * inner;
   double sum = 0.0;
   if (VEC) {
@@ -56,18 +61,19 @@ __global__ __launch_bounds__(kBlock) void scale_residual_relu_rowmean_kernel(
       v4f o;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        o[j] = tail_element(vx[j], s, b, vr[j]);
-        sum += static_cast<double>(o[j]);
+        o[j] = tail_element<HAS_SCALE, HAS_BIAS, RES_FIRST>(vx[j], s, b, vr[j]);
+        if (MEAN) sum += static_cast<double>(o[j]);
       }
       if (WRITE_Y) store4_stream(y + base + 4ull * i, o);
     }
   } else {
     for (uint32_t i = lane; i < inner; i += kWave) {
-      const float o = tail_element(x[base + i], s, b, res[base + i]);
-      sum += static_cast<double>(o);
+      const float o = tail_element<HAS_SCALE, HAS_BIAS, RES_FIRST>(x[base + i], s, b, res[base + i]);
+      if (MEAN) sum += static_cast<double>(o);
       if (WRITE_Y) y[base + i] = o;
     }
   }
+  if (!MEAN) return;
   sum = wave_sum_f64(sum);
   if (lane == 0) mean[row] = static_cast<float>(sum / static_cast<double>(static_cast<int>(inner)));
 }
@@ -76,11 +82,35 @@ __global__ __launch_bounds__(kBlock) void scale_residual_relu_rowmean_kernel(
 
 using namespace shdw;
 
-extern "C" int shdw_hip_scale_residual_relu_rowmean(int n, int scale_num, int inner_num,
-                                                    const float* x, const float* scale,
-                                                    const float* bias, const float* residual,
-                                                    float* y, float* mean, void* stream) {
-  if (n < 0 || scale_num < 1 || inner_num < 1 || !x || !scale || !bias || !residual || !mean)
+namespace {
+
+template <bool HAS_SCALE, bool HAS_BIAS, bool RES_FIRST>
+int launch_tail(uint32_t rows, uint32_t inner, FastDiv num, const float* x, const float* scale, const float* bias,
+                const float* residual, float* y, float* mean, bool vec, hipStream_t st) {
+  const uint32_t grid = (rows + kBlock / kWave - 1) / (kBlock / kWave);
+#define SHDW_LAUNCH(V, W, M)                                                                              \
+  scale_residual_relu_rowmean_kernel<V, W, M, HAS_SCALE, HAS_BIAS, RES_FIRST><<<grid, kBlock, 0, st>>>(   \
+      x, scale, bias, residual, y, mean, rows, inner, num)
+  if (vec) {
+    if (y && mean) SHDW_LAUNCH(true, true, true);
+    else if (y) SHDW_LAUNCH(true, true, false);
+    else SHDW_LAUNCH(true, false, true);
+  } else {
+    if (y && mean) SHDW_LAUNCH(false, true, true);
+    else if (y) SHDW_LAUNCH(false, true, false);
+    else SHDW_LAUNCH(false, false, true);
+  }
+#undef SHDW_LAUNCH
+  return launch_status();
+}
+
+}  // namespace
+
+extern "C" int shdw_hip_scale_residual_relu(int n, int scale_num, int inner_num, const float* x,
+                                            const float* scale, const float* bias,
+                                            const float* residual, int residual_first, float* y,
+                                            float* mean, void* stream) {
+  if (n < 0 || scale_num < 1 || inner_num < 1 || !x || (!scale && !bias) || !residual || (!y && !mean))
     return SHDW_E_INVALID_ARGUMENT;
   if (n % inner_num != 0) return SHDW_E_INVALID_ARGUMENT;
   if (n == 0) return SHDW_OK;
@@ -89,14 +119,19 @@ extern "C" int shdw_hip_scale_residual_relu_rowmean(int n, int scale_num, int in
   const FastDiv num = make_fastdiv(static_cast<uint32_t>(scale_num));
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool vec = inner % 4 == 0 && aligned16(x) && aligned16(residual) && (!y || aligned16(y));
-  const uint32_t grid = (rows + kBlock / kWave - 1) / (kBlock / kWave);
-#define SHDW_LAUNCH(V, W)                                                                   \
-  scale_residual_relu_rowmean_kernel<V, W><<<grid, kBlock, 0, st>>>(x, scale, bias, residual, \
-                                                                    y, mean, rows, inner, num)
-  if (vec && y) SHDW_LAUNCH(true, true);
-  else if (vec) SHDW_LAUNCH(true, false);
-  else if (y) SHDW_LAUNCH(false, true);
-  else SHDW_LAUNCH(false, false);
-#undef SHDW_LAUNCH
-  return launch_status();
+#define SHDW_FORM(S, B)                                                                                       \
+  (residual_first ? launch_tail<S, B, true>(rows, inner, num, x, scale, bias, residual, y, mean, vec, st)     \
+                  : launch_tail<S, B, false>(rows, inner, num, x, scale, bias, residual, y, mean, vec, st))
+  if (scale && bias) return SHDW_FORM(true, true);
+  if (scale) return SHDW_FORM(true, false);
+  return SHDW_FORM(false, true);
+#undef SHDW_FORM
+}
+
+extern "C" int shdw_hip_scale_residual_relu_rowmean(int n, int scale_num, int inner_num,
+                                                    const float* x, const float* scale,
+                                                    const float* bias, const float* residual,
+                                                    float* y, float* mean, void* stream) {
+  if (!scale || !bias || !mean) return SHDW_E_INVALID_ARGUMENT;
+  return shdw_hip_scale_residual_relu(n, scale_num, inner_num, x, scale, bias, residual, 0, y, mean, stream);
 }

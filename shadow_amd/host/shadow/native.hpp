@@ -6,6 +6,7 @@
 #define SHADOW_AMD_HOST_NATIVE_HPP_
 
 #include "backend.hpp"
+#include "fusion.hpp"
 #include "operator.hpp"
 
 namespace Shadow {
@@ -13,7 +14,10 @@ namespace Shadow {
 class Native : public Backend {
  public:
   // Arguments: backend_type, device_id, default_cuda_stream (Workspace);
-  // device_input (Run takes device pointers), debug (log every operator).
+  // device_input (Run takes device pointers), debug (log every operator and every
+  // fused group), fuse (default true: runs of elementwise operators that one launch
+  // can stand for are run that way, see fusion.hpp; a blob inside such a run that
+  // nothing else reads is then not written).
   explicit Native(const ArgumentHelper& arguments);
 
   void LoadModel(const shadow::NetParam& net_param) override;
@@ -29,7 +33,11 @@ class Native : public Backend {
   void Run(const std::map<std::string, void*>& data_map,
            const std::map<std::string, std::vector<int>>& shape_map) override;
 
+  // One line per fused group (FusedGroup::describe), in running order.
+  std::vector<std::string> fused() const;
+
  private:
+  void RunOperator(Operator* op);
   void Initial(const shadow::NetParam& net_param);
   void SetInputData(const std::string& blob_name, const std::vector<int>& blob_shape,
                     const void* blob_data);
@@ -40,8 +48,10 @@ class Native : public Backend {
   void CopyWeights(const shadow::NetParam& net_param, const std::vector<const void*>& weights);
   void CopyWeights(const shadow::NetParam& net_param, const void* weights_data);
 
-  bool device_input_ = false, debug_ = false;
+  bool device_input_ = false, debug_ = false, fuse_ = true;
   std::vector<std::shared_ptr<Operator>> ops_;
+  std::vector<std::unique_ptr<FusedGroup>> groups_;
+  std::vector<int> group_of_;  // per operator: its group, or -1
 };
 
 }  // namespace Shadow

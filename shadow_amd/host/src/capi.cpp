@@ -12,6 +12,7 @@
 
 #include "shadow/io.hpp"
 #include "shadow/kernel.hpp"
+#include "shadow/native.hpp"
 #include "shadow/network.hpp"
 #include "shadow/operator.hpp"
 #include "shadow/parser.hpp"
@@ -291,7 +292,7 @@ int shdw_host_backend_keys(char* buf, size_t n) { return join(BackendRegistry()-
 // model declares no blobs.  device_input: Forward takes device pointers and
 // copies device to device.  NULL on error.
 void* shdw_host_network_create(const char* backend_type, int device_id, int debug,
-                               int device_input, const char* proto_text, const void* weights) {
+                               int device_input, int fuse, const char* proto_text, const void* weights) {
   Network* net = nullptr;
   guarded([&] {
     ArgumentHelper args;
@@ -299,6 +300,7 @@ void* shdw_host_network_create(const char* backend_type, int device_id, int debu
     args.AddSingleArgument<int>("device_id", device_id);
     args.AddSingleArgument<bool>("debug", debug != 0);
     args.AddSingleArgument<bool>("device_input", device_input != 0);
+    args.AddSingleArgument<bool>("fuse", fuse != 0);
     std::unique_ptr<Network> made(new Network());
     made->LoadXModel(std::string(proto_text ? proto_text : ""), weights, args);
     made->backend()->ws()->Ctx()->synchronize();  // the weight buffer may go away after return
@@ -310,7 +312,7 @@ void* shdw_host_network_create(const char* backend_type, int device_id, int debu
 // The same from a binary model whose blobs carry their contents
 // (network_index as in shdw_host_parse_net_binary).
 void* shdw_host_network_create_from_binary(const char* backend_type, int device_id, int debug,
-                                           int device_input, const void* data, int size,
+                                           int device_input, int fuse, const void* data, int size,
                                            int network_index) {
   Network* net = nullptr;
   guarded([&] {
@@ -319,6 +321,7 @@ void* shdw_host_network_create_from_binary(const char* backend_type, int device_
     args.AddSingleArgument<int>("device_id", device_id);
     args.AddSingleArgument<bool>("debug", debug != 0);
     args.AddSingleArgument<bool>("device_input", device_input != 0);
+    args.AddSingleArgument<bool>("fuse", fuse != 0);
     shadow::NetParam net_param;
     read_binary_net(data, size, network_index, &net_param);
     std::unique_ptr<Network> made(new Network());
@@ -331,12 +334,18 @@ void* shdw_host_network_create_from_binary(const char* backend_type, int device_
 
 void shdw_host_network_destroy(void* net) { delete static_cast<Network*>(net); }
 
-// which: 0 = input blob names, 1 = output blob names (newline separated)
+// which: 0 = input blob names, 1 = output blob names, 2 = the fused groups of the
+// Native backend, one description each (newline separated)
 int shdw_host_network_io(void* net, int which, char* buf, size_t n) {
   int len = -1;
   guarded([&] {
     auto* nw = static_cast<Network*>(net);
-    len = join(which == 0 ? nw->in_blob() : nw->out_blob(), buf, n);
+    if (which == 2) {
+      auto native = std::dynamic_pointer_cast<Native>(nw->backend());
+      len = join(native != nullptr ? native->fused() : std::vector<std::string>(), buf, n);
+    } else {
+      len = join(which == 0 ? nw->in_blob() : nw->out_blob(), buf, n);
+    }
   });
   return len;
 }

@@ -1,0 +1,290 @@
+#include "shadow/fusion.hpp"
+
+#include <algorithm>
+#include <set>
+
+#include "shadow_hip.h"
+
+namespace Shadow {
+
+namespace {
+
+constexpr int kActivateRelu = 1;  // shadow/operators/kernels/activate.hpp:12
+constexpr int kEltwiseSum = 1;    // shadow/operators/kernels/eltwise.hpp:10
+constexpr int kReduceAvg = 4;     // shadow/operators/kernels/reduce.hpp:18
+
+using OpList = std::vector<std::shared_ptr<Operator>>;
+
+bool reads(const Operator& op, const std::string& blob) {
+  const auto& b = op.op_param().bottom();
+  return std::find(b.begin(), b.end(), blob) != b.end();
+}
+bool writes(const Operator& op, const std::string& blob) {
+  const auto& t = op.op_param().top();
+  return std::find(t.begin(), t.end(), blob) != t.end();
+}
+
+// What the reference's optimizer asks of a producer (exactly one successor,
+// optimizer.py:87-94), on blob names that may be written again further down:
+// between `producer` and the next operator that overwrites `blob`, `reader` is the
+// only operator that reads it, and the network does not hand it out.
+bool sole_reader(const OpList& ops, const std::vector<std::string>& out_blob, const std::string& blob,
+                 int producer, int reader) {
+  if (std::find(out_blob.begin(), out_blob.end(), blob) != out_blob.end()) return false;
+  bool seen = false;
+  for (int j = producer + 1; j < static_cast<int>(ops.size()); ++j) {
+    if (reads(*ops[j], blob)) {
+      if (j != reader) return false;
+      seen = true;
+    }
+    if (writes(*ops[j], blob)) break;
+  }
+  return seen;
+}
+
+// The first operator after `producer` that reads `blob` before it is overwritten.
+int next_reader(const OpList& ops, const std::string& blob, int producer) {
+  for (int j = producer + 1; j < static_cast<int>(ops.size()); ++j) {
+    if (reads(*ops[j], blob)) return j;
+    if (writes(*ops[j], blob)) break;
+  }
+  return -1;
+}
+
+// The members run together where the last one stood.  That is the order of the
+// file as long as no operator between them writes a blob the members read or
+// write, or reads a blob they write.
+bool movable(const OpList& ops, const std::vector<int>& members) {
+  std::set<std::string> in, out;
+  for (int m : members) {
+    in.insert(ops[m]->op_param().bottom().begin(), ops[m]->op_param().bottom().end());
+    out.insert(ops[m]->op_param().top().begin(), ops[m]->op_param().top().end());
+  }
+  for (int j = members.front() + 1; j < members.back(); ++j) {
+    if (std::find(members.begin(), members.end(), j) != members.end()) continue;
+    for (const auto& t : ops[j]->op_param().top())
+      if (in.count(t) || out.count(t)) return false;
+    for (const auto& b : ops[j]->op_param().bottom())
+      if (out.count(b)) return false;
+  }
+  return true;
+}
+
+bool is_relu(const Operator& op) {
+  return op.type() == "Activate" && op.get_single_argument<int>("type", 1) == kActivateRelu &&
+         op.op_param().bottom_size() == 1 && op.op_param().top_size() == 1;
+}
+
+// Scale with its parameters as input blobs (not scale_value / bias_value, which
+// are staged through the temp buffer on every run).
+bool is_blob_scale(const Operator& op) {
+  if (op.type() != "Scale" || op.op_param().top_size() != 1) return false;
+  const bool has_scale = op.get_single_argument<bool>("has_scale", false);
+  const bool has_bias = op.get_single_argument<bool>("has_bias", false);
+  return (has_scale || has_bias) && op.op_param().bottom_size() == (has_scale && has_bias ? 3 : 2);
+}
+
+bool is_residual_sum(const Operator& op) {
+  if (op.type() != "Eltwise" || op.op_param().bottom_size() != 2 || op.op_param().top_size() != 1) return false;
+  if (op.get_single_argument<int>("operation", -1) != kEltwiseSum) return false;
+  for (float c : op.get_repeated_argument<float>("coeff"))
+    if (c != 1.f) return false;
+  const auto& p = op.op_param();
+  // an output that is one of the inputs is cleared before it is read
+  // (shadow/operators/kernels/eltwise.hpp:37-44): nothing to gain from that form
+  return p.bottom(0) != p.bottom(1) && p.top(0) != p.bottom(0) && p.top(0) != p.bottom(1);
+}
+
+bool is_mean(const Operator& op) {
+  return op.type() == "Reduce" && op.get_single_argument<int>("operation", 0) == kReduceAvg &&
+         op.op_param().bottom_size() == 1 && op.op_param().top_size() == 1 &&
+         op.op_param().top(0) != op.op_param().bottom(0);
+}
+
+std::shared_ptr<Blob> float_blob(Workspace* ws, const std::string& name) {
+  auto blob = ws->GetBlob(name);
+  return blob != nullptr && blob->data_type() == DataType::kF32 ? blob : nullptr;
+}
+
+// The Scale member's view of its input: the parameter blobs cover the axes from
+// `axis` on, one parameter per run of `inner` elements
+// (shadow/operators/kernels/scale.hpp:45-62).
+struct ScaleView {
+  std::shared_ptr<Blob> x, scale, bias;
+  int num = 0, inner = 0;
+};
+
+bool view_scale(const Operator& op, Workspace* ws, ScaleView* v) {
+  const auto& p = op.op_param();
+  const bool has_scale = op.get_single_argument<bool>("has_scale", false);
+  const bool has_bias = op.get_single_argument<bool>("has_bias", false);
+  v->x = float_blob(ws, p.bottom(0));
+  if (has_scale) v->scale = float_blob(ws, p.bottom(1));
+  if (has_bias) v->bias = float_blob(ws, p.bottom(has_scale ? 2 : 1));
+  if (v->x == nullptr || (has_scale && v->scale == nullptr) || (has_bias && v->bias == nullptr)) return false;
+  if (has_scale && has_bias && v->scale->shape() != v->bias->shape()) return false;
+  const auto& param = has_scale ? v->scale : v->bias;
+  const int rank = v->x->num_axes();
+  int axis = op.get_single_argument<int>("axis", 1);
+  if (axis < 0) axis += rank;
+  if (axis < 0 || axis + param->num_axes() > rank || v->x->count() == 0) return false;
+  for (int k = 0; k < param->num_axes(); ++k)
+    if (param->shape(k) != v->x->shape(axis + k)) return false;
+  v->num = param->count();
+  v->inner = v->x->count(axis + param->num_axes());
+  return v->num > 0 && v->inner > 0;
+}
+
+std::string label(const Operator& op) { return op.name() + "(" + op.type() + ")"; }
+
+// ---- Scale -> Activate(relu): shdw_hip_scale_bias with its relu epilogue ----
+class ScaleRelu : public FusedGroup {
+ public:
+  ScaleRelu(const OpList& ops, int scale, int relu) : scale_(ops[scale]), relu_(ops[relu]) {
+    members_ = {scale, relu};
+  }
+
+  bool Run(Workspace* ws) override {
+    ScaleView v;
+    if (!view_scale(*scale_, ws, &v)) return false;
+    auto y = float_blob(ws, relu_->op_param().top(0));
+    if (y == nullptr) return false;
+    y->reshape(v.x->shape());
+    SHADOW_HIP_CHECK(shdw_hip_scale_bias(v.x->count(), v.num, v.inner, v.x->data<float>(),
+                                         v.scale ? v.scale->data<float>() : nullptr,
+                                         v.bias ? v.bias->data<float>() : nullptr, 1,
+                                         y->mutable_data<float>(), ws->Ctx()->stream()));
+    return true;
+  }
+
+  std::string describe() const override {
+    return label(*scale_) + " + " + label(*relu_) + " -> " + relu_->op_param().top(0);
+  }
+
+ private:
+  std::shared_ptr<Operator> scale_, relu_;
+};
+
+// ---- Scale -> Eltwise(SUM) -> Activate(relu) [-> Reduce(AVG)]: shdw_hip_scale_residual_relu ----
+class ResidualTail : public FusedGroup {
+ public:
+  ResidualTail(const OpList& ops, int scale, int sum, int relu, int mean)
+      : scale_(ops[scale]), sum_(ops[sum]), relu_(ops[relu]) {
+    members_ = {scale, sum, relu};
+    if (mean >= 0) {
+      mean_ = ops[mean];
+      members_.push_back(mean);
+    }
+    residual_first_ = sum_->op_param().bottom(1) == scale_->op_param().top(0);
+  }
+
+  bool Run(Workspace* ws) override {
+    ScaleView v;
+    if (!view_scale(*scale_, ws, &v)) return false;
+    auto r = float_blob(ws, sum_->op_param().bottom(residual_first_ ? 0 : 1));
+    auto y = float_blob(ws, relu_->op_param().top(0));
+    if (r == nullptr || y == nullptr || r->shape() != v.x->shape()) return false;
+    std::shared_ptr<Blob> mean;
+    VecInt mean_shape, squeezed;
+    if (mean_ != nullptr) {
+      mean = float_blob(ws, mean_->op_param().top(0));
+      if (mean == nullptr || mean == y || mean == v.x || mean == r) return false;
+      // the reduced axes must be exactly the run one parameter applies to
+      const int rank = v.x->num_axes();
+      VecInt axes = mean_->get_repeated_argument<int>("axes");
+      if (axes.empty())
+        for (int n = 0; n < rank; ++n) axes.push_back(n);
+      std::vector<bool> listed(rank, false);
+      for (int a : axes) {
+        if (a < -rank || a >= rank) return false;
+        listed[a < 0 ? a + rank : a] = true;
+      }
+      int first = rank;
+      while (first > 0 && listed[first - 1]) --first;
+      for (int n = 0; n < first; ++n)
+        if (listed[n]) return false;
+      if (first == rank || v.x->count(first) != v.inner) return false;
+      mean_shape = v.x->shape();
+      for (int n = first; n < rank; ++n) mean_shape[n] = 1;
+      squeezed.assign(mean_shape.begin(), mean_shape.begin() + first);
+    }
+    y->reshape(v.x->shape());
+    if (mean != nullptr) mean->reshape(mean_shape);
+    SHADOW_HIP_CHECK(shdw_hip_scale_residual_relu(
+        v.x->count(), v.num, v.inner, v.x->data<float>(), v.scale ? v.scale->data<float>() : nullptr,
+        v.bias ? v.bias->data<float>() : nullptr, r->data<float>(), residual_first_ ? 1 : 0,
+        y->mutable_data<float>(), mean != nullptr ? mean->mutable_data<float>() : nullptr,
+        ws->Ctx()->stream()));
+    if (mean != nullptr && !mean_->get_single_argument<bool>("keep_dims", true)) mean->set_shape(squeezed);
+    return true;
+  }
+
+  std::string describe() const override {
+    std::string text = label(*scale_) + " + " + label(*sum_) + " + " + label(*relu_);
+    if (mean_ != nullptr) text += " + " + label(*mean_);
+    text += " -> " + relu_->op_param().top(0);
+    if (mean_ != nullptr) text += ", " + mean_->op_param().top(0);
+    return text;
+  }
+
+ private:
+  std::shared_ptr<Operator> scale_, sum_, relu_, mean_;
+  bool residual_first_ = false;
+};
+
+}  // namespace
+
+std::vector<std::unique_ptr<FusedGroup>> FindFusedGroups(const OpList& ops,
+                                                         const std::vector<std::string>& out_blob) {
+  std::vector<std::unique_ptr<FusedGroup>> groups;
+  std::vector<bool> taken(ops.size(), false);
+  const int count = static_cast<int>(ops.size());
+  for (int i = 0; i < count; ++i) {
+    if (taken[i] || !is_blob_scale(*ops[i])) continue;
+    const std::string& s = ops[i]->op_param().top(0);
+    const int next = next_reader(ops, s, i);
+    if (next < 0 || taken[next]) continue;
+
+    if (is_relu(*ops[next])) {
+      // in place the Scale output is the group's output and every later reader sees the
+      // activated values either way; elsewhere it is no longer written
+      if (ops[next]->op_param().top(0) != s && !sole_reader(ops, out_blob, s, i, next)) continue;
+      std::vector<int> members = {i, next};
+      if (!movable(ops, members)) continue;
+      groups.emplace_back(new ScaleRelu(ops, i, next));
+      taken[i] = taken[next] = true;
+      continue;
+    }
+
+    if (!is_residual_sum(*ops[next]) || !sole_reader(ops, out_blob, s, i, next)) continue;
+    const std::string& e = ops[next]->op_param().top(0);
+    const int relu = next_reader(ops, e, next);
+    if (relu < 0 || taken[relu] || !is_relu(*ops[relu])) continue;
+    const std::string& y = ops[relu]->op_param().top(0);
+    // not in place: the sum itself is no longer written, so nobody else may want it;
+    // in place: every reader further down sees the activated values either way
+    if (y != e && !sole_reader(ops, out_blob, e, next, relu)) continue;
+    if (y == e && next_reader(ops, e, next) != relu) continue;
+    std::vector<int> members = {i, next, relu};
+    if (!movable(ops, members)) continue;
+    int mean = -1;
+    for (int j = relu + 1; j < count; ++j) {
+      if (!taken[j] && is_mean(*ops[j]) && ops[j]->op_param().bottom(0) == y) {
+        std::vector<int> with_mean = {i, next, relu, j};
+        if (movable(ops, with_mean)) mean = j;
+        break;
+      }
+      if (writes(*ops[j], y)) break;
+    }
+    groups.emplace_back(new ResidualTail(ops, i, next, relu, mean));
+    taken[i] = taken[next] = taken[relu] = true;
+    if (mean >= 0) taken[mean] = true;
+  }
+  std::sort(groups.begin(), groups.end(),
+            [](const std::unique_ptr<FusedGroup>& a, const std::unique_ptr<FusedGroup>& b) {
+              return a->members().back() < b->members().back();
+            });
+  return groups;
+}
+
+}  // namespace Shadow

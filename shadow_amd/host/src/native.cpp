@@ -8,6 +8,7 @@ namespace Shadow {
 Native::Native(const ArgumentHelper& arguments) {
   device_input_ = arguments.GetSingleArgument<bool>("device_input", false);
   debug_ = arguments.GetSingleArgument<bool>("debug", false);
+  fuse_ = arguments.GetSingleArgument<bool>("fuse", true);
   ws_ = std::make_shared<Workspace>(arguments);
 }
 
@@ -85,7 +86,37 @@ void Native::Initial(const shadow::NetParam& net_param) {
   arg_helper_ = ArgumentHelper(net_param);
   CHECK(arg_helper_.HasArgument("out_blob")) << "Network must have out_blob argument";
   out_blob_ = arg_helper_.GetRepeatedArgument<std::string>("out_blob");
+
+  groups_.clear();
+  group_of_.assign(ops_.size(), -1);
+  if (fuse_) {
+    groups_ = FindFusedGroups(ops_, out_blob_);
+    for (size_t g = 0; g < groups_.size(); ++g) {
+      for (int member : groups_[g]->members()) group_of_[member] = static_cast<int>(g);
+      if (debug_) LOG(INFO) << "Fused: " << groups_[g]->describe();
+    }
+  }
   if (debug_) LOG(INFO) << "Initial Network!";
+}
+
+std::vector<std::string> Native::fused() const {
+  std::vector<std::string> lines;
+  for (const auto& group : groups_) lines.push_back(group->describe());
+  return lines;
+}
+
+void Native::RunOperator(Operator* op) {
+  std::vector<std::shared_ptr<Blob>> inputs, outputs;
+  for (const auto& name : op->op_param().bottom()) {
+    CHECK(ws_->HasBlob(name)) << op->name() << ": Can not find input blob " << name;
+    inputs.push_back(ws_->GetBlob(name));
+  }
+  for (const auto& name : op->op_param().top()) {
+    CHECK(ws_->HasBlob(name)) << op->name() << ":  Can not find output blob " << name;
+    outputs.push_back(ws_->GetBlob(name));
+  }
+  op->Run(inputs, outputs);
+  if (debug_) LOG(INFO) << op->debug_log(inputs, outputs);
 }
 
 void Native::Run(const std::map<std::string, void*>& data_map,
@@ -100,18 +131,21 @@ void Native::Run(const std::map<std::string, void*>& data_map,
                  in_map.second);
   }
 
-  for (auto& op : ops_) {
-    std::vector<std::shared_ptr<Blob>> inputs, outputs;
-    for (const auto& name : op->op_param().bottom()) {
-      CHECK(ws_->HasBlob(name)) << op->name() << ": Can not find input blob " << name;
-      inputs.push_back(ws_->GetBlob(name));
+  for (size_t i = 0; i < ops_.size(); ++i) {
+    const int g = group_of_[i];
+    if (g < 0) {
+      RunOperator(ops_[i].get());
+      continue;
     }
-    for (const auto& name : op->op_param().top()) {
-      CHECK(ws_->HasBlob(name)) << op->name() << ":  Can not find output blob " << name;
-      outputs.push_back(ws_->GetBlob(name));
+    // a group runs where its last member stands, as one launch; when the shapes of
+    // this run do not fit it, as its members one by one
+    auto& group = *groups_[g];
+    if (static_cast<int>(i) != group.members().back()) continue;
+    if (group.Run(ws_.get())) {
+      if (debug_) LOG(INFO) << "Fused: " << group.describe();
+    } else {
+      for (int member : group.members()) RunOperator(ops_[member].get());
     }
-    op->Run(inputs, outputs);
-    if (debug_) LOG(INFO) << op->debug_log(inputs, outputs);
   }
   if (debug_) LOG(INFO) << "Forward Network!";
 }

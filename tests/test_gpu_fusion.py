@@ -1,0 +1,232 @@
+"""The Native backend's fusion pass: Scale -> Activate(relu) and
+Scale -> Eltwise(SUM) -> Activate(relu) [-> Reduce(AVG)] run as one launch.
+Every network here runs three ways: fused (the default), with fuse=False, and
+through oracle.net.run (the operators one by one on the CPU).  The blobs a fused
+run still writes must carry the same bits as the unfused run's, and the oracle's
+too, except the mean, which the device sums in fp64 either way: fused and
+unfused agree bit for bit there and both are within 1e-5 of the oracle.  Blobs
+that have another reader, or that the network hands out, must block the fusion
+that would stop writing them."""
+import numpy as np
+import pytest
+
+import shadow_amd
+from oracle import net as onet
+from tests.helpers import assert_bit_exact, assert_rel_close, normal, uniform, with_specials
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+def arg_i(name, v):
+    return (name, "s_i", int(v))
+
+
+def op(typ, name, bottom, top, *args):
+    return {"type": typ, "name": name, "bottom": list(bottom), "top": list(top), "arg": list(args)}
+
+
+def scale_op(bottom, top, has_scale=True, has_bias=True, name="bn", axis=1):
+    params = (["gamma"] if has_scale else []) + (["beta"] if has_bias else [])
+    return op("Scale", name, [bottom] + params, [top], arg_i("axis", axis), arg_i("has_scale", has_scale),
+              arg_i("has_bias", has_bias))
+
+
+SHAPE = (3, 6, 5, 7)  # rows of 35 floats: not whole 128-bit vectors
+
+
+def make(ops, out, shape=SHAPE, inputs=("x",), params=("gamma", "beta"), param_shape=None):
+    c = shape[1]
+    pshape = list(param_shape or [c])
+    return {"name": "fusion", "arg": [("out_blob", "v_s", list(out))],
+            "blob": [(p, "float", pshape) for p in params],
+            "op": [op("Input", "in", [], list(inputs), *[(n, "v_i", list(shape)) for n in inputs])] + list(ops)}
+
+
+def data(shape=SHAPE, inputs=("x",), seed=0, specials=True, nparams=2, param_shape=None):
+    pshape = tuple(param_shape or [shape[1]])
+    weights = [uniform(seed + 1, pshape, 0.5, 1.5), normal(seed + 2, pshape, 0.3)][:nparams]
+    feed = {}
+    for k, name in enumerate(inputs):
+        a = normal(seed + 10 + k, shape, 2.0)
+        if specials:
+            a = with_specials(a, seed + k).reshape(shape)
+        feed[name] = a
+    return weights, feed
+
+
+def run_all(net, weights, feed, written, fp64=(), expect_fused=None, reshape=False):
+    """Fused and unfused runs against each other (bit for bit) and against the oracle."""
+    text = onet.write_text(net)
+    want = onet.run(net, weights, feed)
+    with shadow_amd.Network(text, weights, fuse=False) as plain:
+        assert plain.fused == []
+        plain.forward(feed, reshape=reshape)
+        ref = {name: plain.blob(name) for name in written}
+    with shadow_amd.Network(text, weights) as nw:
+        if expect_fused is not None:
+            assert nw.fused == expect_fused
+        for _ in range(2):  # a second forward finds the blobs already shaped
+            nw.forward(feed, reshape=reshape)
+            for name in written:
+                got = nw.blob(name)
+                assert list(got.shape) == list(want[name].shape) == list(ref[name].shape), name
+                assert_bit_exact(got, ref[name], name + " fused against unfused")
+                if name in fp64:
+                    assert assert_rel_close(got, want[name], 1e-5, name) == 0
+                else:
+                    assert_bit_exact(got, want[name], name + " against the oracle")
+        return nw.fused
+
+
+@pytest.mark.parametrize("in_place", [False, True])
+@pytest.mark.parametrize("has_scale,has_bias", [(True, True), (True, False), (False, True)])
+def test_scale_relu(gpu, in_place, has_scale, has_bias):
+    """has_bias alone is the Bias -> Activate pair of the convolution epilogue."""
+    top = "s" if in_place else "y"
+    params = (["gamma"] if has_scale else []) + (["beta"] if has_bias else [])
+    net = make([scale_op("x", "s", has_scale, has_bias), op("Activate", "relu", ["s"], [top], arg_i("type", 1)),
+                op("Unary", "neg", [top], ["out"], arg_i("operation", 13))], ["out"], params=params)
+    weights, feed = data()
+    weights = [w for w, keep in zip(weights, (has_scale, has_bias)) if keep]
+    run_all(net, weights, feed, [top, "out"], expect_fused=["bn(Scale) + relu(Activate) -> " + top])
+
+
+def test_scale_relu_with_parameters_over_two_axes_and_a_long_tensor(gpu):
+    shape = (2, 4, 6, 64)
+    net = make([scale_op("x", "s"), op("Activate", "relu", ["s"], ["s"])], ["s"], shape=shape, param_shape=[4, 6])
+    weights, feed = data(shape, param_shape=[4, 6])
+    assert run_all(net, weights, feed, ["s"]) == ["bn(Scale) + relu(Activate) -> s"]
+
+
+TAIL = ["bn(Scale) + add(Eltwise) + relu(Activate) + gap(Reduce) -> e, pool"]
+
+
+def tail_ops(relu_top="e", residual_first=False, keep_dims=True, axes=(2, 3), scale_in="x", scale_top="s"):
+    return [scale_op(scale_in, scale_top),
+            op("Eltwise", "add", ["r", scale_top] if residual_first else [scale_top, "r"], ["e"], arg_i("operation", 1)),
+            op("Activate", "relu", ["e"], [relu_top], arg_i("type", 1)),
+            op("Reduce", "gap", [relu_top], ["pool"], arg_i("operation", 4), ("axes", "v_i", list(axes)),
+               arg_i("keep_dims", keep_dims))]
+
+
+@pytest.mark.parametrize("shape", [SHAPE, (2, 8, 4, 8), (5, 3, 1, 1), (2, 5, 14, 14)])
+@pytest.mark.parametrize("residual_first", [False, True])
+@pytest.mark.parametrize("keep_dims", [True, False])
+def test_residual_tail_with_mean(gpu, shape, residual_first, keep_dims):
+    net = make(tail_ops(residual_first=residual_first, keep_dims=keep_dims), ["e", "pool"], shape=shape, inputs=("x", "r"))
+    weights, feed = data(shape, ("x", "r"), seed=3, specials=False)
+    run_all(net, weights, feed, ["e", "pool"], fp64=("pool",), expect_fused=TAIL)
+
+
+def test_residual_tail_with_special_values(gpu):
+    """Signed zeros, infinities and NaNs go through x*s + b, 0 + t, + r and the select
+    exactly as through the four operators; the means of rows that hold them follow."""
+    net = make(tail_ops()[:3], ["e"], inputs=("x", "r"))
+    weights, feed = data(SHAPE, ("x", "r"), seed=5, specials=True)
+    feed["r"][0, 0, 0, :4] = [0.0, -0.0, np.inf, -np.inf]
+    feed["x"][0, 0, 0, :4] = [-0.0, -0.0, -np.inf, 1.0]
+    run_all(net, weights, feed, ["e"], expect_fused=["bn(Scale) + add(Eltwise) + relu(Activate) -> e"])
+
+
+def test_residual_tail_relu_into_another_blob_and_scale_in_place(gpu):
+    net = make(tail_ops(relu_top="a", scale_in="x", scale_top="x"), ["a", "pool"], inputs=("x", "r"))
+    weights, feed = data(SHAPE, ("x", "r"), seed=7, specials=False)
+    run_all(net, weights, feed, ["a", "pool"], fp64=("pool",),
+            expect_fused=["bn(Scale) + add(Eltwise) + relu(Activate) + gap(Reduce) -> a, pool"])
+
+
+def test_tail_whose_reduce_covers_other_axes_runs_its_members_one_by_one(gpu):
+    """The group is found from the operator list; whether the reduced axes are the run
+    one parameter applies to is known when the blobs have their shapes."""
+    for axes in ([3], [1, 2, 3], [0], []):
+        net = make(tail_ops(axes=axes), ["e", "pool"], inputs=("x", "r"))
+        weights, feed = data(SHAPE, ("x", "r"), seed=9, specials=False)
+        run_all(net, weights, feed, ["e", "pool"], fp64=("pool",), expect_fused=TAIL)
+
+
+def test_a_later_reader_of_the_activated_sum_keeps_the_mean_out_of_the_group(gpu):
+    ops = tail_ops()
+    ops.insert(3, op("Unary", "abs", ["e"], ["m"], arg_i("operation", 0)))
+    net = make(ops, ["m", "pool"], inputs=("x", "r"))
+    weights, feed = data(SHAPE, ("x", "r"), seed=11, specials=False)
+    run_all(net, weights, feed, ["e", "m", "pool"], fp64=("pool",),
+            expect_fused=["bn(Scale) + add(Eltwise) + relu(Activate) -> e"])
+
+
+def test_an_operator_between_the_members_that_touches_nothing_of_theirs_is_stepped_over(gpu):
+    ops = tail_ops()
+    ops.insert(1, op("Unary", "abs", ["r"], ["m"], arg_i("operation", 0)))  # reads an input of the group: harmless
+    net = make(ops, ["m", "pool"], inputs=("x", "r"))
+    weights, feed = data(SHAPE, ("x", "r"), seed=13, specials=False)
+    run_all(net, weights, feed, ["e", "m", "pool"], fp64=("pool",), expect_fused=TAIL)
+
+
+BLOCKED = {
+    "the Scale output is an output of the network":
+        (tail_ops(), ["s", "pool"], ["s", "e", "pool"]),
+    "the Scale output has a second reader":
+        (tail_ops() + [op("Unary", "abs", ["s"], ["m"], arg_i("operation", 0))], ["m", "pool"], ["s", "e", "m", "pool"]),
+    "an operator in between rewrites the residual":
+        (tail_ops()[:1] + [op("Unary", "neg", ["r"], ["r"], arg_i("operation", 13))] + tail_ops()[1:], ["pool"],
+         ["s", "e", "pool"]),
+    "the sum has coefficients":
+        ([scale_op("x", "s"), op("Eltwise", "add", ["s", "r"], ["e"], arg_i("operation", 1), ("coeff", "v_f", [F(1), F(0.5)])),
+          op("Activate", "relu", ["e"], ["e"], arg_i("type", 1))], ["e"], ["s", "e"]),
+    "the Eltwise is a maximum":
+        ([scale_op("x", "s"), op("Eltwise", "add", ["s", "r"], ["e"], arg_i("operation", 2)),
+          op("Activate", "relu", ["e"], ["e"], arg_i("type", 1))], ["e"], ["s", "e"]),
+    "the activation is not relu":
+        ([scale_op("x", "s"), op("Activate", "act", ["s"], ["y"], arg_i("type", 6))], ["y"], ["s", "y"]),
+    "the sum is read before it is activated elsewhere":
+        ([scale_op("x", "s"), op("Eltwise", "add", ["s", "r"], ["e"], arg_i("operation", 1)),
+          op("Activate", "relu", ["e"], ["a"], arg_i("type", 1)), op("Unary", "abs", ["e"], ["m"], arg_i("operation", 0))],
+         ["a", "m"], ["s", "e", "a", "m"]),
+}
+
+
+@pytest.mark.parametrize("why", sorted(BLOCKED))
+def test_blocked(gpu, why):
+    ops, out, written = BLOCKED[why]
+    net = make(ops, out, inputs=("x", "r"))
+    weights, feed = data(SHAPE, ("x", "r"), seed=17, specials=False)
+    run_all(net, weights, feed, written, fp64=("pool",), expect_fused=[])
+
+
+def test_scale_with_host_values_stays_an_operator(gpu):
+    net = make([op("Scale", "sc", ["x"], ["s"], arg_i("axis", 1), ("scale_value", "v_f", [F(0.5)]),
+                   ("bias_value", "v_f", [F(0.25)])), op("Activate", "relu", ["s"], ["s"], arg_i("type", 1))], ["s"], params=())
+    _, feed = data(nparams=0)
+    run_all(net, [], feed, ["s"], expect_fused=[])
+
+
+def test_inputs_reshaped_between_forwards(gpu):
+    net = make(tail_ops(keep_dims=False), ["e", "pool"], inputs=("x", "r"))
+    text = onet.write_text(net)
+    weights, _ = data(SHAPE, ("x", "r"))
+    with shadow_amd.Network(text, weights) as nw:
+        assert nw.fused == TAIL
+        for shape in (SHAPE, (2, 6, 9, 4), (4, 6, 3, 3), SHAPE):
+            _, feed = data(shape, ("x", "r"), seed=sum(shape), specials=False)
+            want = onet.run(make(tail_ops(keep_dims=False), ["e", "pool"], shape=shape, inputs=("x", "r")), weights, feed)
+            nw.forward(feed, reshape=True)
+            assert_bit_exact(nw.blob("e"), want["e"], "e %s" % (shape,))
+            assert nw.blob_shape("pool") == list(shape[:2])
+            assert assert_rel_close(nw.blob("pool"), want["pool"], 1e-5, "pool") == 0
+
+
+def test_full_size_bottleneck_tail_through_the_network(gpu):
+    """BASELINE configs[4] as a converted model would hold it."""
+    shape = (64, 1024, 14, 14)
+    net = make(tail_ops(), ["e", "pool"], shape=shape, inputs=("x", "r"))
+    weights = [uniform(502, 1024, 0.5, 1.5), uniform(503, 1024, -0.1, 0.1)]
+    feed = {"x": normal(501, shape), "r": normal(504, shape)}
+    text = onet.write_text(net)
+    with shadow_amd.Network(text, weights, fuse=False) as plain:
+        plain.forward(feed)
+        e, pool = plain.blob("e"), plain.blob("pool")
+    with shadow_amd.Network(text, weights) as nw:
+        assert nw.fused == TAIL
+        nw.forward(feed)
+        assert_bit_exact(nw.blob("e"), e, "e")
+        assert_bit_exact(nw.blob("pool"), pool, "pool")

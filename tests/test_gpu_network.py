@@ -93,11 +93,17 @@ def compare(nw, want, names):
 def test_resnet_tail_graph(gpu):
     net, weights, inputs = resnet_tail()
     want = onet.run(net, weights, inputs)
+    with shadow_amd.Network(onet.write_text(net), weights, fuse=False) as nw:
+        assert nw.fused == []
+        nw.forward(inputs)
+        compare(nw, want, ["bn_out", "sum", "feat", "pooled", "flat", "prob"])
     with shadow_amd.Network(onet.write_text(net), weights) as nw:
         assert nw.in_blob == ["data", "skip"] and nw.out_blob == ["prob", "feat"]
         assert nw.blob_shape("data") == [4, 16, 7, 7]
+        # Scale, Eltwise and the in-place relu run as one launch; bn_out, which only the Eltwise reads, is not written
+        assert nw.fused == ["bn(Scale) + add(Eltwise) + relu(Activate) -> sum"]
         nw.forward(inputs)
-        compare(nw, want, ["bn_out", "sum", "feat", "pooled", "flat", "prob"])
+        compare(nw, want, ["sum", "feat", "pooled", "flat", "prob"])
         # a second pass over the same network gives the same bits
         first = nw.blob("prob").copy()
         nw.forward(inputs)
@@ -122,10 +128,14 @@ def test_binary_models_with_embedded_weights(gpu):
     net, weights, inputs = resnet_tail()
     want = onet.run(net, weights, inputs)
     wire = sp.from_oracle_net(net, weights).SerializeToString()
-    with shadow_amd.Network.from_binary(wire) as nw:
+    with shadow_amd.Network.from_binary(wire, fuse=False) as nw:
         assert nw.in_blob == ["data", "skip"] and nw.out_blob == ["prob", "feat"]
         nw.forward(inputs)
         compare(nw, want, ["bn_out", "sum", "feat", "pooled", "flat", "prob"])
+    with shadow_amd.Network.from_binary(wire) as nw:
+        assert len(nw.fused) == 1
+        nw.forward(inputs)
+        compare(nw, want, ["sum", "feat", "pooled", "flat", "prob"])
     net2, weights2, inputs2 = mixed_graph()
     meta = sp.MetaNetParam()
     meta.name = "two networks"
