@@ -1005,23 +1005,81 @@ NETWORK_TEXT = """[bottleneck_tail]
 def network_forward(dev, reps=50):
     """Wall time of Network::Forward for a six-operator text model on
     [64,1024,14,14] with device inputs: two 51 MB device-to-device input copies,
-    five launches, one stream synchronisation per call."""
+    the launches (three with the backend's fusion pass, five without), one stream
+    synchronisation per call."""
     sa = dev.sa
     n = 64 * 1024 * 14 * 14
     x, r = dev.buf(normal(801, n)), dev.buf(normal(802, n))
     weights = [uniform(803, 1024, 0.5, 1.5), uniform(804, 1024, -0.1, 0.1)]
-    with sa.Network(NETWORK_TEXT, weights, device_input=True) as net:
-        for _ in range(5):
-            net.forward({"x": x, "r": r})
-        t0 = time.perf_counter()
-        for _ in range(reps):
-            net.forward({"x": x, "r": r})
-        t1 = time.perf_counter()
-    us = (t1 - t0) * 1e6 / reps
-    moved = 4 * n * (2 * 2 + 3 + 3 + 2 + 1)  # input copies, scale, eltwise, relu, pooling read
-    return {"model": "Scale -> Eltwise -> ReLU -> global avg Pooling -> Flatten -> Softmax, [64,1024,14,14]",
-            "us_per_forward": round(us, 1), "operators": 6, "launches": 5, "input_copies": 2,
-            "bytes_moved": moved, "GBps": round(moved / us / 1e3, 1)}
+    out = {"model": "Scale -> Eltwise -> ReLU -> global avg Pooling -> Flatten -> Softmax, [64,1024,14,14]",
+           "operators": 6, "input_copies": 2}
+    for fuse, key in ((True, "us_per_forward"), (False, "us_per_forward_unfused")):
+        with sa.Network(NETWORK_TEXT, weights, device_input=True, fuse=fuse) as net:
+            for _ in range(5):
+                net.forward({"x": x, "r": r})
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                net.forward({"x": x, "r": r})
+            t1 = time.perf_counter()
+            if fuse:
+                out["fused"] = net.fused
+        out[key] = round((t1 - t0) * 1e6 / reps, 1)
+    x.free(), r.free()
+    return out
+
+
+def tail_text(copies):
+    """BASELINE configs[4] as a converted model holds it, `copies` times side by side on
+    blobs of their own, so that one run walks over more than the 256 MB Infinity Cache."""
+    shape = "64 # 1024 # 14 # 14"
+    names = ["x%d" % k for k in range(copies)] + ["r%d" % k for k in range(copies)]
+    lines = ["[bottleneck_tails]", "[{out_blob, v_s, [%s]}]" % " # ".join("pool%d" % k for k in range(copies)),
+             "[{gamma, float, [1024]}; {beta, float, [1024]}]",
+             "[Input] | [in] | [0 %d %d] | [] | [%s] | [%s]" % (
+                 len(names), len(names), "; ".join(names), "; ".join("{%s, v_i, [%s]}" % (nm, shape) for nm in names))]
+    for k in range(copies):
+        lines += ["[Scale] | [bn%d] | [3 1 3] | [x%d; gamma; beta] | [s%d] | [{axis, s_i, [1]}; {has_scale, s_i, [1]}; "
+                  "{has_bias, s_i, [1]}]" % (k, k, k),
+                  "[Eltwise] | [add%d] | [2 1 1] | [s%d; r%d] | [e%d] | [{operation, s_i, [1]}]" % (k, k, k, k),
+                  "[Activate] | [relu%d] | [1 1 1] | [e%d] | [e%d] | [{type, s_i, [1]}]" % (k, k, k),
+                  "[Reduce] | [gap%d] | [1 1 2] | [e%d] | [pool%d] | [{operation, s_i, [4]}; {axes, v_i, [2 # 3]}]" % (
+                      k, k, k)]
+    return "\n".join(lines) + "\n"
+
+
+def network_tail(dev, copies=6, reps=20):
+    """Device time of the bottleneck tail (Scale -> Eltwise SUM -> ReLU -> Reduce AVG on
+    [64,1024,14,14]) run by the Native backend from a model text, per tail: events on the
+    backend's stream around `reps` runs of a network that holds `copies` such tails on
+    separate blobs, nothing waited for in between.  Fused: one launch per tail."""
+    sa, lib = dev.sa, dev.lib
+    n = 64 * 1024 * 14 * 14
+    src = [dev.buf(normal(811 + k, n)) for k in range(2)]
+    weights = [uniform(803, 1024, 0.5, 1.5), uniform(804, 1024, -0.1, 0.1)]
+    feed = {}
+    for k in range(copies):
+        feed["x%d" % k], feed["r%d" % k] = src[k & 1], src[(k + 1) & 1]
+    out = {"model": "%d x (Scale -> Eltwise SUM -> ReLU -> Reduce AVG{2,3}) on [64,1024,14,14]" % copies}
+    for fuse, key in ((True, "us_per_tail"), (False, "us_per_tail_unfused")):
+        with sa.Network(tail_text(copies), weights, device_input=True, fuse=fuse) as net:
+            net.forward(feed)
+            st = net.stream
+            e0, e1 = dev.event(), dev.event()
+            best = None
+            for _ in range(3):
+                net.run()
+                dev.ck(lib.shdw_hip_event_record(e0, st))
+                for _ in range(reps):
+                    net.run()
+                dev.ck(lib.shdw_hip_event_record(e1, st))
+                dev.ck(lib.shdw_hip_stream_sync(st))
+                ms = dev.elapsed_ms(e0, e1) / (reps * copies)
+                best = ms if best is None else min(best, ms)
+            out[key] = round(best * 1e3, 2)
+            out["launches_per_tail" if fuse else "launches_per_tail_unfused"] = 1 if net.fused else 4
+    for b in src:
+        b.free()
+    return out
 
 
 SHORT_OP = {"binary_add_channel_broadcast": "add_chan_bcast", "fused_tail (CPU: the four operators)": "fused_tail"}
@@ -1054,7 +1112,9 @@ def final_record(full, table_path=None):
         worst = min(big, key=lambda r: r["frac_of_ceiling"])
         rec["worst_of_ceiling"] = [worst["cfg"], SHORT_OP.get(worst["op"], worst["op"]), worst["frac_of_ceiling"]]
     if "network" in full:
-        rec["network"] = {k: v for k, v in full["network"].items() if k != "model"}
+        rec["network"] = {k: v for k, v in full["network"].items() if k not in ("model", "fused")}
+    if "network_tail" in full:
+        rec["network_tail"] = {k: v for k, v in full["network_tail"].items() if k != "model"}
     if table_path:
         rec["table"] = table_path
     return rec
@@ -1064,7 +1124,7 @@ def final_line(full, table_path=None):
     """final_record as one line of JSON below FINAL_LINE_LIMIT.  Should a host with a long
     device or CPU name push it over, the optional tables go first (they are in the file)."""
     rec = final_record(full, table_path)
-    for optional in (None, "step_ops", "baseline_rows", "baseline_rows_columns", "network"):
+    for optional in (None, "step_ops", "baseline_rows", "baseline_rows_columns", "network", "network_tail"):
         rec.pop(optional, None)
         line = json.dumps(rec, separators=(",", ":"))
         if len(line) < FINAL_LINE_LIMIT:
@@ -1138,6 +1198,7 @@ def main():
                                "way (rows at the end); cpu_us: the oracle's C loop for the same operator on this "
                                "host, one thread, outputs allocated beforehand, best of %d" % args.cpu_passes)
         out["network"] = network_forward(dev)
+        out["network_tail"] = network_tail(dev)
     table = write_table(out, args.table)
     for r in out.get("configs", []):
         print("%-8s %-62s %9.2f us  %.3f of 8 TB/s%s" % (r["cfg"], r["op"], r["us"], r["frac"],

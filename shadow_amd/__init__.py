@@ -75,6 +75,7 @@ SIGNATURES = {
     "shdw_hip_reduce_static": (_I, [_I, _I, c_int_p, _I, c_int_p, _V, _V, _V]),
     "shdw_hip_reduce_static_max_workspace_bytes": (_Z, []),
     "shdw_hip_scale_residual_relu_rowmean": (_I, [_I, _I, _I, _V, _V, _V, _V, _V, _V, _V]),
+    "shdw_hip_scale_residual_relu": (_I, [_I, _I, _I, _V, _V, _V, _V, _I, _V, _V, _V]),
     "shdw_hip_axpy_rows": (_I, [_I, _I, _V, _V, _V, _V, _V]),
     "shdw_hip_batch_norm": (_I, [_I, _I, _I, _V, _V, _V, _F, _F, _V, _V]),
     "shdw_hip_group_norm": (_I, [_I, _I, _F, _V, _V, _V, _I, _I, _V, _V]),
@@ -214,6 +215,8 @@ HOST_SIGNATURES = {
     "shdw_host_network_destroy": (None, [_V]),
     "shdw_host_network_io": (_I, [_V, _I, ctypes.c_char_p, _Z]),
     "shdw_host_network_forward": (_I, [_V, _I, ctypes.POINTER(ctypes.c_char_p), c_void_pp, c_int_p, c_int_p]),
+    "shdw_host_network_run": (_I, [_V]),
+    "shdw_host_network_stream": (_V, [_V]),
     "shdw_host_network_blob_shape": (_I, [_V, ctypes.c_char_p, c_int_p, _I]),
     "shdw_host_network_blob_get": (_I, [_V, ctypes.c_char_p, c_float_p, _I]),
     "shdw_host_face_blas": (_I, [_V, ctypes.c_char_p, _I, c_float_p, _I, _I, c_float_p, _I, _I, _F, c_float_p, _I, _I]),
@@ -280,6 +283,14 @@ class Workspace:
         rank = array.ndim if array.ndim else 1
         host_check(self.lib.shdw_host_blob_set(self.ptr, name.encode(), shape, rank,
                                                array.ctypes.data) == 0)
+
+    def run(self):
+        """The operators once more on what the input blobs hold; enqueued, not waited for."""
+        host_check(self.lib.shdw_host_network_run(self.ptr) == 0)
+
+    @property
+    def stream(self):
+        return ctypes.c_void_p(self.lib.shdw_host_network_stream(self.ptr))
 
     def blob_shape(self, name):
         shape = (ctypes.c_int * 16)()
@@ -450,6 +461,14 @@ class Network:
         ranks = ints([a.ndim if reshape else 0 for a in arrays])
         dims = ints([d for a in arrays for d in (a.shape if reshape else ())])
         host_check(self.lib.shdw_host_network_forward(self.ptr, len(names), c_names, c_data, ranks, dims) == 0)
+
+    def run(self):
+        """The operators once more on what the input blobs hold; enqueued, not waited for."""
+        host_check(self.lib.shdw_host_network_run(self.ptr) == 0)
+
+    @property
+    def stream(self):
+        return ctypes.c_void_p(self.lib.shdw_host_network_stream(self.ptr))
 
     def blob_shape(self, name):
         shape = (ctypes.c_int * 16)()

@@ -371,6 +371,24 @@ int shdw_host_network_forward(void* net, int count, const char* const* names, vo
   });
 }
 
+// The operators of the network once more on whatever its input blobs hold, enqueued
+// on the context's stream and not waited for (Backend::Run without Network::Forward's
+// synchronize): for a caller that times or overlaps several runs.
+int shdw_host_network_run(void* net) {
+  return guarded([&] {
+    auto* nw = static_cast<Network*>(net);
+    nw->backend()->ws()->Ctx()->switch_device();
+    nw->backend()->Run({}, {});
+  });
+}
+
+// The context's stream (a hipStream_t), NULL on error.
+void* shdw_host_network_stream(void* net) {
+  void* stream = nullptr;
+  guarded([&] { stream = static_cast<Network*>(net)->backend()->ws()->Ctx()->stream(); });
+  return stream;
+}
+
 int shdw_host_network_blob_shape(void* net, const char* name, int* shape, int max_rank) {
   int rank = -1;
   guarded([&] {

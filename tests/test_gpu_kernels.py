@@ -404,6 +404,31 @@ def test_fused_tail(gpu, outer, num, inner):
     assert_bit_exact(m2, m, "mean without y")
 
 
+@pytest.mark.parametrize("form", ["scale", "bias", "both"])
+@pytest.mark.parametrize("residual_first", [False, True])
+@pytest.mark.parametrize("outer,num,inner", [(2, 8, 196), (3, 5, 7), (2, 3, 1030)])
+def test_fused_tail_forms(gpu, form, residual_first, outer, num, inner):
+    """The forms a network holds the sequence in: Scale with one parameter blob only, the
+    residual as the first Eltwise input, no Reduce behind it."""
+    n = outer * num * inner
+    x, r = with_specials(normal(174, n), 3), with_specials(normal(175, n), 4)
+    s = uniform(176, num, 0.5, 1.5) if form != "bias" else None
+    b = uniform(177, num, -0.1, 0.1) if form != "scale" else None
+    t = oracle.scale_bias(x, s, b, num, inner)
+    t = oracle.eltwise(1, [r, t] if residual_first else [t, r], [1.0, 1.0])
+    want_y = oracle.activate(t, 1)
+    y, none = gpuops.scale_residual_relu(x, s, b, r, num, inner, residual_first, want_mean=False)
+    assert none is None
+    assert_bit_exact(y, want_y, "y")
+    x, r = normal(174, n), normal(175, n)  # finite values for the mean
+    y2, m = gpuops.scale_residual_relu(x, s, b, r, num, inner, residual_first)
+    t = oracle.scale_bias(x, s, b, num, inner)
+    clean = oracle.activate(oracle.eltwise(1, [r, t] if residual_first else [t, r], [1.0, 1.0]), 1)
+    assert_bit_exact(y2, clean, "y with the mean")
+    want_m, _ = oracle.reduce(4, clean, [outer * num, inner], [1])
+    assert assert_rel_close(m, want_m, 1e-5, "mean") == 0
+
+
 def test_argument_errors(gpu):
     import shadow_amd
     lib = gpu
@@ -419,3 +444,9 @@ def test_argument_errors(gpu):
     assert lib.shdw_hip_reduce(1, 2, sh, 1, shadow_amd.ints([-1]), buf.ptr, buf.ptr, None, 0, None) == -1
     big = shadow_amd.ints([1 << 20])
     assert lib.shdw_hip_reduce(1, 1, big, 1, shadow_amd.ints([0]), buf.ptr, buf.ptr, None, 0, None) == -3
+    p = buf.ptr
+    assert lib.shdw_hip_scale_residual_relu(16, 2, 8, p, None, None, p, 0, p, p, None) == -1  # no parameters
+    assert lib.shdw_hip_scale_residual_relu(16, 2, 8, p, p, p, p, 0, None, None, None) == -1  # no output
+    assert lib.shdw_hip_scale_residual_relu(16, 2, 8, p, p, p, None, 0, p, p, None) == -1     # no residual
+    assert lib.shdw_hip_scale_residual_relu(15, 2, 8, p, p, p, p, 0, p, p, None) == -1        # not whole rows
+    assert lib.shdw_hip_scale_residual_relu_rowmean(16, 2, 8, p, p, None, p, p, p, None) == -1
