@@ -94,6 +94,10 @@ struct Acc<OP, true> {
   SHDW_DEVICE void add_value(float x) {
     if (OP == SHDW_REDUCE_MAX) v = (v < x) ? x : v; else v = (x < v) ? x : v;
   }
+  // the hardware's maximum / minimum; x must not be a signalling NaN (see fold_batch)
+  SHDW_DEVICE void take(float x) {
+    if (OP == SHDW_REDUCE_MAX) v = __builtin_fmaxf(v, x); else v = __builtin_fminf(v, x);
+  }
   SHDW_DEVICE void add_key(float x, uint32_t pos) {
     if (x == 0.0f) {
       const uint32_t k = (pos << 1) | (__float_as_uint(x) >> 31);
@@ -145,23 +149,33 @@ struct Acc<OP, true> {
 
 // Folds a batch of N vectors into the four column accumulators of a lane (or,
 // with ONE, into a single accumulator): element j of vector u has list position
-// pos(u, j); vectors with valid[u] false are skipped.  The vote is over the
+// pos(u, j); vectors with valid[u] false are skipped.  The votes are over the
 // lanes that are active here, which then all take the same branch.
+//
+// MAX / MIN take the batch with v_max3_f32 / v_min3_f32 (two elements per
+// instruction, where compare-and-select is two instructions and a wait per
+// element).  Those give the reference's `(v < x) ? x : v` for every pair of
+// numbers (up to the sign of a zero, which the key decides) and skip a quiet NaN
+// as the comparison does; a signalling NaN they would hand on as a NaN, so every
+// element is made quiet first (v_max_f32 x, x), which leaves numbers as they
+// are.  Zeros: the smallest magnitude of the batch is zero exactly when it
+// holds one (a NaN never is the minimum), so the keys cost one v_min3_f32 per
+// two elements and one comparison per batch unless a zero is there.
 template <int N, bool ONE, class A, class POS>
 SHDW_DEVICE void fold_batch(A* acc, const v4f (&v)[N], const bool (&valid)[N], POS pos) {
-#pragma unroll
-  for (int u = 0; u < N; ++u)
-    if (valid[u]) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) acc[ONE ? 0 : j].add_value(v[u][j]);
-    }
-  if (A::kSelect) {
-    bool zero = false;
+  if constexpr (A::kSelect) {
+    float smallest = FLT_MAX;
 #pragma unroll
     for (int u = 0; u < N; ++u)
+      if (valid[u]) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) zero |= valid[u] && (v[u][j] == 0.0f);
-    if (__builtin_amdgcn_ballot_w64(zero) != 0) {
+        for (int j = 0; j < 4; ++j) {
+          const float q = __builtin_canonicalizef(v[u][j]);
+          acc[ONE ? 0 : j].take(q);
+          smallest = __builtin_fminf(smallest, __builtin_fabsf(q));
+        }
+      }
+    if (__builtin_amdgcn_ballot_w64(smallest == 0.0f) != 0) {
 #pragma unroll
       for (int u = 0; u < N; ++u)
         if (valid[u]) {
@@ -169,6 +183,13 @@ SHDW_DEVICE void fold_batch(A* acc, const v4f (&v)[N], const bool (&valid)[N], P
           for (int j = 0; j < 4; ++j) acc[ONE ? 0 : j].add_key(v[u][j], pos(u, j));
         }
     }
+  } else {
+#pragma unroll
+    for (int u = 0; u < N; ++u)
+      if (valid[u]) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[ONE ? 0 : j].add_value(v[u][j]);
+      }
   }
 }
 

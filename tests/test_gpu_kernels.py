@@ -380,6 +380,30 @@ def test_reduce_select_special_values(gpu, shape, axes, op):
     assert_bit_exact(got, want, "reduce select specials")
 
 
+@pytest.mark.parametrize("shape,axes", [([64, 48], [1]), ([300, 49], [1]), ([50000], [0]), ([3, 500, 49], [1]), ([2, 600, 784], [1]),
+                                        ([3, 700, 256], [1]), ([2, 6000, 12], [1]), ([3, 1024, 7], [1]), ([300, 5, 9], [0, 2]),
+                                        ([4, 300, 28, 28], [0, 2, 3]), ([9, 4100], [1]), ([4099, 3], [1]), ([7, 130003], [0])])
+@pytest.mark.parametrize("op", [2, 3])
+def test_reduce_select_signalling_nans(gpu, shape, axes, op):
+    """Signalling and negative NaNs among ordinary values are skipped like quiet ones:
+    the comparison `v < x` is false for every NaN, whatever the hardware's own maximum
+    and minimum instructions make of a signalling one."""
+    n = int(np.prod(shape))
+    r = np.random.default_rng(165 + op)
+    bits = normal(166, n).view(np.uint32).copy()
+    where = r.random(n)
+    bits[where < 0.02] = 0x7FA00000   # signalling NaN
+    bits[(where >= 0.02) & (where < 0.03)] = 0xFFA00001  # negative signalling NaN
+    bits[(where >= 0.03) & (where < 0.04)] = 0xFFC00000  # negative quiet NaN
+    bits[(where >= 0.04) & (where < 0.05)] = 0x80000000  # -0
+    bits[(where >= 0.05) & (where < 0.06)] = 0x00000000  # +0
+    x = bits.view(np.float32).reshape(shape)
+    want, _ = oracle.reduce(op, x, shape, axes)
+    assert not np.isnan(want).any()
+    got, _ = gpuops.reduce(op, x, shape, axes)
+    assert_bit_exact(got, want, "reduce select with signalling NaNs")
+
+
 def test_reduce_l2_and_avg_definition(gpu):
     x = np.float32([[3, 4], [6, 8]])
     got, _ = gpuops.reduce(6, x, [2, 2], [1])
