@@ -58,11 +58,15 @@ __global__ __launch_bounds__(T) void ew_vec_kernel(F f, const float* a, const fl
     const uint32_t i = first + u * T;
     if (i < n4) {
       v4f r;
+      if constexpr (NIN == 1 && has_four<F>::value) {
+        r = f.four(va[u], tab);
+      } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float x = NIN >= 1 ? va[u][j] : alpha;
-        const float w = NIN >= 2 ? vb[u][j] : alpha;
-        r[j] = f(x, w, tab);
+        for (int j = 0; j < 4; ++j) {
+          const float x = NIN >= 1 ? va[u][j] : alpha;
+          const float w = NIN >= 2 ? vb[u][j] : alpha;
+          r[j] = f(x, w, tab);
+        }
       }
       store4_stream_any(y + 4ull * i, r);
     } else if (i == n4) {

@@ -28,6 +28,20 @@ struct vectors_per_lane { static constexpr int value = 1; };
 template <class F>
 struct vectors_per_lane<F, decltype((void)F::kVectorsPerLane)> { static constexpr int value = F::kVectorsPerLane; };
 
+// Functors whose arithmetic has a short form for ordinary arguments and a long
+// one for the rest define `four(x)`: the four elements of a lane's vector at once,
+// with one wave-wide choice for all of them, so that the four evaluations stay
+// interleaved instead of each sitting behind a branch of its own.
+template <class F, class = void>
+struct has_four { static constexpr bool value = false; };
+template <class F>
+struct has_four<F, decltype((void)&F::four)> { static constexpr bool value = true; };
+
+// Both forms are pure arithmetic, which the compiler is free to evaluate side by
+// side and select from; an empty statement it may not move keeps the rare form
+// behind its wave-wide branch.
+SHDW_DEVICE void keep_branch() { asm volatile("" ::: "memory"); }
+
 SHDW_DEVICE float sel_max(float a, float b) { return (a < b) ? b : a; }
 SHDW_DEVICE float sel_min(float a, float b) { return (b < a) ? b : a; }
 
@@ -61,9 +75,44 @@ struct BMin { SHDW_DEVICE float operator()(float a, float b, const uint64_t* tab
 // ---- activations: shadow/operators/kernels/activate.cpp:9-31 ----
 struct ARelu { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return x > 0 ? x : 0; } };
 struct ALeaky { SHDW_DEVICE float operator()(float x, float s, const uint64_t* tab) const { return x > 0 ? x : s * x; } };
-struct ASigmoid { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_sigmoidf(x, tab); } };
+struct ASigmoid {
+  static constexpr bool kExpTable = true;
+  SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_sigmoidf(x, tab); }
+  SHDW_DEVICE v4f four(v4f x, const uint64_t* tab) const {
+    bool ok = true;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ok &= libm::sigmoidf_short_ok(x[j]);
+    v4f r;
+    if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = libm::sigmoidf_short(x[j], tab);
+    } else {
+      keep_branch();
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = libm::sigmoidf_any(x[j], tab);
+    }
+    return r;
+  }
+};
 struct ASoftPlus { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_softplusf(x, tab); } };
-struct ATanh { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_tanhf(x); } };
+struct ATanh {
+  SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_tanhf(x); }
+  SHDW_DEVICE v4f four(v4f x, const uint64_t*) const {
+    bool ok = true;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ok &= libm::tanhf_short_ok(x[j]);
+    v4f r;
+    if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = libm::tanhf_short(x[j]);
+    } else {
+      keep_branch();
+#pragma unroll
+      for (int j = 0; j < 4; ++j) r[j] = libm::tanhf_any(x[j]);
+    }
+    return r;
+  }
+};
 struct ARelu6 { SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return x < 0 ? 0 : (x > 6 ? 6 : x); } };
 struct AHardSwish {
   SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const {

@@ -33,6 +33,14 @@
 #define SHDW_LIBM_TABLE static const
 #endif
 
+// The divisions that are a hardware reciprocal plus one correction (div_normal,
+// sigmoidf_short) return the library's bits on gfx950's v_rcp_f32, which is what
+// the exhaustive device tests establish; another architecture's reciprocal would
+// have to be swept again before this header is compiled for it.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "libm_exact.h: the reciprocal-based divisions are verified for gfx950 only"
+#endif
+
 namespace shdw {
 namespace libm {
 
@@ -216,18 +224,18 @@ SHDW_LIBM_FN float exact_expm1f(float x) {
 //     the library's own cut is at 22), which also bounds k by 29;
 //   * the |x| < 2^-55 and |a| < 2^-25 early returns are left to the general
 //     path, which returns x there as well.
-SHDW_LIBM_FN float exact_tanhf(float x) {
+//
+// tanhf_magnitude is |tanhf(x)| from a2 = 2|x| (at most 20) and big = |x| >= 1;
+// exact_tanhf puts the sign back.  On the device a wave whose lanes all have
+// |x| < 10 (no NaN among them) needs neither the cut at 10 nor the NaN case and
+// takes a2 and the sign with one operation each; any other wave goes the long way.
+// Both ways run the same tanhf_magnitude on the same a2.
+SHDW_LIBM_FN float tanhf_magnitude(float a2, bool big) {
   const float one = 1.0f, two = 2.0f, half = 0.5f;
   const float ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f;
   const float invln2 = 1.4426950216e+00f;
   const float Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f,
               Q4 = 4.0082177293e-06f, Q5 = -2.0109921195e-07f;
-  const uint32_t jx = f2u(x);
-  const uint32_t ix = jx & 0x7fffffffu;
-  const bool big = ix >= 0x3f800000u;  // |x| >= 1: expm1f(+2|x|), else expm1f(-2|x|)
-  // from |x| = 10 on 2 / (t + 2) < 2^-25 and 1 - q rounds to 1: evaluate at 10
-  const uint32_t ic = ix < 0x41200000u ? ix : 0x41200000u;
-  const float a2 = two * u2f(ic);
   const float a = big ? a2 : -a2;  // argument of expm1f
 
   // --- expm1f(a): argument reduction ---
@@ -246,12 +254,14 @@ SHDW_LIBM_FN float exact_tanhf(float x) {
 
   // --- primary range ---
   const float s = xr * xr;  // 2 hxs
-  // r1 = 1 + hxs (Q1 + hxs (Q2 + hxs (Q3 + hxs (Q4 + hxs Q5)))); the first fused
-  // step produces half of its value so that the next one needs no 0.5
-  float p = __builtin_fmaf(s, Q5 * 0.25f, Q4 * half);  // (Q4 + hxs Q5) / 2
-  p = __builtin_fmaf(s, p, Q3);
-  p = __builtin_fmaf(s, half * p, Q2);
-  p = __builtin_fmaf(s, half * p, Q1);
+  // r1 = 1 + hxs (Q1 + hxs (Q2 + hxs (Q3 + hxs (Q4 + hxs Q5)))).  Step i of the
+  // fused part works on its value divided by 2^(i-1): hxs * v = s * (v / 2), and a
+  // power of two passes through every rounding here, so the halvings sit in the
+  // constants and each step is one fused multiply-add on s.
+  float p = __builtin_fmaf(s, Q5 * 0.0625f, Q4 * 0.125f);
+  p = __builtin_fmaf(s, p, Q3 * 0.25f);
+  p = __builtin_fmaf(s, p, Q2 * half);
+  p = __builtin_fmaf(s, p, Q1);
   const float r1 = __builtin_fmaf(half, s * p, one);
   const float t3 = __builtin_fmaf(-half, r1 * xr, 3.0f);  // 3 - r1 * hfx
   // numerator ~ -2, denominator in [4.9, 7.1]; twice the library's e = hxs * (...)
@@ -271,34 +281,68 @@ SHDW_LIBM_FN float exact_tanhf(float x) {
   // --- tanhf ---
   const float q = div_normal(big ? two : t, t + two);
   // |x| >= 1: 1 - 2 / (t + 2); else -t / (t + 2), whose magnitude is |q|.
-  const float z = big ? one - q : q;
+  return big ? one - q : q;
+}
+
+// The long way: any x.
+SHDW_LIBM_FN float tanhf_any(float x) {
+  const uint32_t jx = f2u(x);
+  const uint32_t ix = jx & 0x7fffffffu;
+  // from |x| = 10 on 2 / (t + 2) < 2^-25 and 1 - q rounds to 1: evaluate at 10
+  const uint32_t ic = ix < 0x41200000u ? ix : 0x41200000u;
+  const float z = tanhf_magnitude(2.0f * u2f(ic), ix >= 0x3f800000u);
   // The result takes x's sign; a NaN keeps all of its bits.
   const uint32_t keep = (ix > 0x7f800000u) ? 0u : 0x7fffffffu;
   return u2f((f2u(z) & keep) | (jx & ~keep));
 }
 
+// The short way: |x| < 10 (tanhf_short_ok), and so no NaN.
+SHDW_LIBM_FN bool tanhf_short_ok(float x) { return 2.0f * __builtin_fabsf(x) < 20.0f; }
+SHDW_LIBM_FN float tanhf_short(float x) {
+  const float a2 = 2.0f * __builtin_fabsf(x);
+  return __builtin_copysignf(tanhf_magnitude(a2, a2 >= 2.0f), x);
+}
+
+SHDW_LIBM_FN float exact_tanhf(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  if (__builtin_amdgcn_ballot_w64(!tanhf_short_ok(x)) == 0) return tanhf_short(x);
+#endif
+  return tanhf_any(x);
+}
+
 // 1 / (1 + exp(-x)) in fp32, the way shadow/operators/kernels/activate.cpp:16
 // writes it.
+SHDW_LIBM_FN float sigmoidf_any(float x, const uint64_t* tab) {
+  return 1.0f / (1.0f + exact_expf(-x, tab));
+}
+#if defined(__HIPCC__)
+// |x| < 87: exp(-x) lies in (2^-126, 2^126), so expf's main path is the whole
+// function, d = 1 + exp(-x) is in [1, 2^126) and the quotient is a normal
+// number; the hardware reciprocal of gfx950 plus one correction from the exact
+// remainder 1 - d * r is then the correctly rounded 1 / d for every d this
+// function can produce (all 2^32 inputs compared with the full form on that
+// device; nothing here is argued for another architecture's reciprocal).  From
+// 2^126 on, x < -87.3, the quotient is subnormal and only the full division is
+// right.
+SHDW_LIBM_FN bool sigmoidf_short_ok(float x) { return __builtin_fabsf(x) < 87.0f; }
+SHDW_LIBM_FN float sigmoidf_short(float x, const uint64_t* tab) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const float d = 1.0f + expf_main(-x, tab);
+  const float r = __builtin_amdgcn_rcpf(d);
+  const float e = __builtin_fmaf(-d, r, 1.0f);
+  return __builtin_fmaf(e, r, r);
+#else
+  return sigmoidf_any(x, tab);  // the compiler's host pass over device code; never called
+#endif
+}
+#endif
 SHDW_LIBM_FN float exact_sigmoidf(float x, const uint64_t* tab) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  // |x| < 87: exp(-x) lies in (2^-126, 2^126), so expf's main path is the whole
-  // function, d = 1 + exp(-x) is in [1, 2^126) and the quotient is a normal
-  // number; the hardware reciprocal plus one correction from the exact remainder
-  // 1 - d * r is then the correctly rounded 1 / d for every d this function can
-  // produce (all 2^32 inputs compared with the full form on the device).  The
-  // wave takes this short form when all of its lanes are in that range; a NaN,
-  // an infinity or a large |x| anywhere in the wave sends it through the full
-  // form below (from 2^126 on, x < -87.3, the quotient is subnormal and only the
-  // full division is right).
-  const bool plain = __builtin_fabsf(x) < 87.0f;
-  if (__builtin_amdgcn_ballot_w64(!plain) == 0) {
-    const float d = 1.0f + expf_main(-x, tab);
-    const float r = __builtin_amdgcn_rcpf(d);
-    const float e = __builtin_fmaf(-d, r, 1.0f);
-    return __builtin_fmaf(e, r, r);
-  }
+  // The wave takes the short form when all of its lanes may; a NaN, an infinity
+  // or a large |x| anywhere in the wave sends it through the full form.
+  if (__builtin_amdgcn_ballot_w64(!sigmoidf_short_ok(x)) == 0) return sigmoidf_short(x, tab);
 #endif
-  return 1.0f / (1.0f + exact_expf(-x, tab));
+  return sigmoidf_any(x, tab);
 }
 #if !defined(__HIPCC__)
 SHDW_LIBM_FN float exact_expf(float x) { return exact_expf(x, kExp2fTab); }

@@ -11,6 +11,15 @@ algorithms, the same set the host sweep uses; SHADOW_GPU_FULL_SWEEP=1 (or a
 comma-separated list of names) sweeps all 2^32 for them too.
 
     SHADOW_GPU_FULL_SWEEP=1 python -m pytest tests/test_gpu_exhaustive.py -m gpu -s
+
+tanh and sigmoid choose between a short and a long form per wave (all 64 lanes,
+four consecutive elements each, inside |x| < 10 resp. |x| < 87: short).  The
+sweep above hands every wave 256 consecutive bit patterns starting at a multiple
+of 256, and both limits are multiples of 256 as bit patterns, so there every
+in-range input is computed by the short form and every other input by the long
+one.  test_in_range_inputs_through_the_long_form covers what is left: all
+in-range inputs again, 255 to a wave with a NaN as the 256th, which sends the
+wave the long way.
 """
 import concurrent.futures
 import os
@@ -78,3 +87,32 @@ def test_all_float_inputs(gpu, name):
             bad_total, first = _compare(name, bits, pool)
             covered = "%d sampled" % bits.size
     assert bad_total == 0, "%s: %d of %s inputs differ, e.g. %s" % (name, bad_total, covered, first)
+
+
+WAVE_ELEMENTS = 256  # 64 lanes, one 128-bit vector each: what one wave of the elementwise kernels covers
+SHORT_FORM_LIMIT = {"tanh": 0x41200000, "sigmoid": 0x42AE0000}  # bit patterns of 10.0f and 87.0f
+
+
+@pytest.mark.parametrize("name", sorted(SHORT_FORM_LIMIT))
+def test_in_range_inputs_through_the_long_form(gpu, name):
+    limit = SHORT_FORM_LIMIT[name]
+    assert limit % WAVE_ELEMENTS == 0 and CHUNK % WAVE_ELEMENTS == 0
+    oracle.lib()
+    per_chunk = (CHUNK // WAVE_ELEMENTS) * (WAVE_ELEMENTS - 1)
+    bad_total, first, done = 0, [], 0
+    with concurrent.futures.ThreadPoolExecutor(min(16, os.cpu_count() or 1)) as pool:
+        for sign in (0, 0x80000000):
+            for start in range(0, limit, per_chunk):
+                count = min(per_chunk, limit - start)
+                groups = -(-count // (WAVE_ELEMENTS - 1))
+                bits = np.full(groups * WAVE_ELEMENTS, 0x7FC00000, np.uint32)  # NaN wherever nothing else is put
+                tmp = np.full(groups * (WAVE_ELEMENTS - 1), 0x7FC00000, np.uint32)
+                tmp[:count] = (np.arange(start, start + count, dtype=np.uint64) | sign).astype(np.uint32)
+                bits.reshape(groups, WAVE_ELEMENTS)[:, :WAVE_ELEMENTS - 1] = tmp.reshape(groups, WAVE_ELEMENTS - 1)
+                bad, where = _compare(name, bits, pool)
+                bad_total += bad
+                first = (first + where)[:8]
+                done += count
+        print("%s: %d in-range inputs through the long form, %d mismatches" % (name, done, bad_total), flush=True)
+    assert done == 2 * limit
+    assert bad_total == 0, "%s: %d inputs differ, e.g. %s" % (name, bad_total, first)
