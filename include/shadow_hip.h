@@ -431,6 +431,43 @@ int shdw_hip_plan_reduce(int num_axes, const int* in_shape, int num_reduce,
                          const int* axes, int* kind, int* outer, int* reduce,
                          int* inner, int* splits);
 
+/* Host-only: which family of kernels shdw_hip_softmax / shdw_hip_normalize /
+ * shdw_hip_pooling2d would launch for a shape, decided by the same code that
+ * launches (nothing is launched, no device is needed).  *path is one of
+ * SHDW_PATH_* below, *variant the family's own parameter, *grid the number of
+ * workgroups of the (first) launch.  Pointer alignment, which some families look
+ * at for a choice of loads, is taken as 16 bytes.  Any of the three may be NULL.
+ * They exist so that a change of a threshold shows up in a test: the operators
+ * have no counterpart of them in the reference. */
+enum {
+  SHDW_PATH_NONE = 0,         /* nothing to do (an empty extent) */
+  SHDW_PATH_ROWS = 1,         /* inner_num == 1, whole rows in a wave's LDS tile; variant = rows per wave */
+  SHDW_PATH_ROWS_STREAM = 2,  /* inner_num == 1, rows streamed in chunks; variant = rows per wave */
+  SHDW_PATH_SHORT_ROWS = 3,   /* slabs of up to 16 floats, four to a lane; variant = floats per slab */
+  SHDW_PATH_QUADS = 4,        /* dim <= 4: four positions per lane in registers */
+  SHDW_PATH_PACKED = 5,       /* several small slabs per workgroup in LDS; variant = slabs per workgroup */
+  SHDW_PATH_LONG_SLAB = 6,    /* one slab per workgroup, streamed in chunks */
+  SHDW_PATH_SLAB = 7,         /* one slab per workgroup, whole in LDS */
+  SHDW_PATH_COLUMNS_REG = 8,  /* a column per lane in registers; variant = registers per column */
+  SHDW_PATH_TILE = 9,         /* 2^variant positions x dim channels per workgroup in LDS */
+  SHDW_PATH_TALL = 10,        /* 2^variant positions per workgroup, channels in chunks */
+  SHDW_PATH_COLUMNS = 11,     /* a column per lane, two passes over memory */
+  /* pooling */
+  SHDW_PATH_POOL_PLANE_REDUCE = 20, /* global max: Reduce's row kernels */
+  SHDW_PATH_POOL_PLANE = 21,        /* global pooling, planes in LDS */
+  SHDW_PATH_POOL_PLANE_STREAM = 22, /* global average of long planes, streamed */
+  SHDW_PATH_POOL_SMALL_PLANES = 23, /* whole planes in LDS; variant = 100 * separable + window unrolled for (0: loops) */
+  SHDW_PATH_POOL_BAND = 24,         /* bands of input rows in LDS; variant = 100 * registers per lane + window unrolled for */
+  SHDW_PATH_POOL_WINDOW = 25        /* a lane per output, windows from memory */
+};
+int shdw_hip_softmax_plan(int outer_num, int dim, int inner_num, int* path, int* variant,
+                          unsigned* grid);
+int shdw_hip_normalize_plan(int outer_num, int dim, int inner_num, float p, int* path,
+                            int* variant, unsigned* grid);
+int shdw_hip_pooling2d_plan(const int* in_shape, int pool_type, int kernel_h, int kernel_w,
+                            int stride_h, int stride_w, int pad_h, int pad_w,
+                            const int* out_shape, int* path, int* variant, unsigned* grid);
+
 #ifdef __cplusplus
 }
 #endif

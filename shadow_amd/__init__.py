@@ -75,6 +75,10 @@ SIGNATURES = {
     "shdw_hip_reduce_static": (_I, [_I, _I, c_int_p, _I, c_int_p, _V, _V, _V]),
     "shdw_hip_reduce_static_max_workspace_bytes": (_Z, []),
     "shdw_hip_scale_residual_relu_rowmean": (_I, [_I, _I, _I, _V, _V, _V, _V, _V, _V, _V]),
+    "shdw_hip_softmax_plan": (_I, [_I, _I, _I, c_int_p, c_int_p, ctypes.POINTER(ctypes.c_uint)]),
+    "shdw_hip_normalize_plan": (_I, [_I, _I, _I, _F, c_int_p, c_int_p, ctypes.POINTER(ctypes.c_uint)]),
+    "shdw_hip_pooling2d_plan": (_I, [c_int_p, _I, _I, _I, _I, _I, _I, _I, c_int_p, c_int_p, c_int_p,
+                                     ctypes.POINTER(ctypes.c_uint)]),
     "shdw_hip_scale_residual_relu": (_I, [_I, _I, _I, _V, _V, _V, _V, _I, _V, _V, _V]),
     "shdw_hip_axpy_rows": (_I, [_I, _I, _V, _V, _V, _V, _V]),
     "shdw_hip_batch_norm": (_I, [_I, _I, _I, _V, _V, _V, _F, _F, _V, _V]),

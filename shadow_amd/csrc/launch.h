@@ -28,6 +28,7 @@ int library_scratch_prepare();
 // takes a single stage and so no workspace: then *rc holds the launch result and
 // the return value is true.
 bool reduce_rows_max(uint32_t rows, uint32_t len, const float* x, float* y, hipStream_t st, int* rc);
+bool reduce_rows_max_applies(uint32_t rows, uint32_t len);  // whether it would (host only)
 
 }  // namespace shdw
 

@@ -1016,10 +1016,19 @@ using namespace shdw;
 
 // Max over every row of x [rows][len] when that needs no workspace (enough rows
 // for a single stage): for the whole-plane max pooling, whose walk is the same.
-bool shdw::reduce_rows_max(uint32_t rows, uint32_t len, const float* x, float* y, hipStream_t st, int* rc) {
+static bool rows_max_plan(uint32_t rows, uint32_t len, ReducePlan* pl) {
   const int shape[2] = {static_cast<int>(rows), static_cast<int>(len)}, axes[1] = {1};
+  return plan_reduce(2, shape, 1, axes, pl) == SHDW_OK && reduce_workspace_bytes(*pl) == 0;
+}
+
+bool shdw::reduce_rows_max_applies(uint32_t rows, uint32_t len) {
   ReducePlan pl;
-  if (plan_reduce(2, shape, 1, axes, &pl) != SHDW_OK || reduce_workspace_bytes(pl) != 0) return false;
+  return rows_max_plan(rows, len, &pl);
+}
+
+bool shdw::reduce_rows_max(uint32_t rows, uint32_t len, const float* x, float* y, hipStream_t st, int* rc) {
+  ReducePlan pl;
+  if (!rows_max_plan(rows, len, &pl)) return false;
   *rc = dispatch_reduce(SHDW_REDUCE_MAX, pl, x, y, nullptr, 0, st);
   return true;
 }

@@ -1037,6 +1037,8 @@ static void launch_normalize_tile_ts(int outer_num, int dim, int inner_num, floa
   }
 }
 
+static int normalize_tile_shift(int dim);
+
 template <int PMODE, int SM>
 static void launch_normalize_tile(int outer_num, int dim, int inner_num, float p, float eps, const float* x,
                                   const float* scale, float* y, hipStream_t st) {
@@ -1046,9 +1048,10 @@ static void launch_normalize_tile(int outer_num, int dim, int inner_num, float p
   // positions (64 KB), 80 us with 32; [64,512,38,38]: 105 us with 32 (64 KB),
   // 115 us with 16.  Softmax, with its four barriers per tile, takes the widest
   // tile that fits.
-  if (dim * 64 * sizeof(float) <= kTileLdsBytes / 2)
+  const int shift = normalize_tile_shift(dim);
+  if (shift == 6)
     launch_normalize_tile_ts<PMODE, SM, 6>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
-  else if (dim * 32 * sizeof(float) <= kTileLdsBytes)
+  else if (shift == 5)
     launch_normalize_tile_ts<PMODE, SM, 5>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
   else
     launch_normalize_tile_ts<PMODE, SM, 4>(outer_num, dim, inner_num, p, eps, x, scale, y, st);
@@ -2117,6 +2120,20 @@ static size_t packed_bytes(int dim, int inner_num, uint32_t group) {
   return static_cast<size_t>(group) * inner_num * (static_cast<uint32_t>(dim) | 1u) * sizeof(float);
 }
 
+// Which family of kernels a shape goes to, for shdw_hip_softmax_plan and its
+// siblings: the entry points below decide as they always do and, asked for a
+// report, hand the decision back instead of launching.
+struct ColumnPlan {
+  int path = SHDW_PATH_NONE, variant = 0;
+  uint32_t grid = 0;
+  bool want = false;  // report only
+  // true: the caller returns without launching
+  bool chosen(int p, int v, uint32_t g) {
+    path = p, variant = v, grid = g;
+    return want;
+  }
+};
+
 static int column_geometry(int outer_num, int dim, int inner_num, ColumnGeometry* g) {
   if (outer_num < 0 || dim < 0 || inner_num < 0) return SHDW_E_INVALID_ARGUMENT;
   const int64_t columns = static_cast<int64_t>(outer_num) * inner_num;
@@ -2129,25 +2146,44 @@ static int column_geometry(int outer_num, int dim, int inner_num, ColumnGeometry
   return SHDW_OK;
 }
 
-}  // namespace shdw
+// What launch_normalize_rows and launch_normalize_tile would launch.
+static int report_normalize_rows(int outer_num, int dim, ColumnPlan* pl) {
+  WaveRows w;
+  const uint32_t rows = static_cast<uint32_t>(outer_num);
+  if (dim < kRowsStreamMinDim && wave_rows<kRowsSmallTile>(dim, &w)) {
+    pl->chosen(SHDW_PATH_ROWS, static_cast<int>(w.rows_per_wave), rows_grid(rows, w));
+  } else {
+    const int g = stream_rows(rows, static_cast<uint32_t>(dim));
+    const uint32_t per_wg = static_cast<uint32_t>(g) * (kBlock / kWave);
+    pl->chosen(SHDW_PATH_ROWS_STREAM, g, (rows + per_wg - 1) / per_wg);
+  }
+  return SHDW_OK;
+}
 
-using namespace shdw;
+static int normalize_tile_shift(int dim) {
+  return dim * 64 * sizeof(float) <= kTileLdsBytes / 2 ? 6 : (dim * 32 * sizeof(float) <= kTileLdsBytes ? 5 : 4);
+}
 
-extern "C" {
+static int report_normalize_tile(int outer_num, int dim, int inner_num, ColumnPlan* pl) {
+  const int shift = normalize_tile_shift(dim);
+  const uint32_t tiles = (static_cast<uint32_t>(inner_num) + (1u << shift) - 1) >> shift;
+  pl->chosen(SHDW_PATH_TILE, shift, static_cast<uint32_t>(outer_num) * tiles);
+  return SHDW_OK;
+}
 
-int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, float* y,
-                     void* stream) {
+static int run_softmax(int outer_num, int dim, int inner_num, const float* x, float* y, hipStream_t st,
+                       ColumnPlan* pl) {
   ColumnGeometry g;
   const int rc = column_geometry(outer_num, dim, inner_num, &g);
   if (rc != SHDW_OK) return rc;
   if (g.columns == 0 || dim == 0) return SHDW_OK;
-  if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!pl->want && (!x || !y)) return SHDW_E_INVALID_ARGUMENT;
   const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
   if (WaveRows w; rows_apply(outer_num, dim, inner_num) && dim <= kRowsSoftmaxMaxDim &&
                   wave_rows<kRowsSmallTile>(dim, &w)) {
     const uint32_t rows = static_cast<uint32_t>(outer_num);
-    softmax_rows_kernel<kRowsSmallTile><<<rows_grid(rows, w), kBlock, 0, st>>>(x, y, rows, w);
+    if (pl->chosen(SHDW_PATH_ROWS, static_cast<int>(w.rows_per_wave), rows_grid(rows, w))) return SHDW_OK;
+    softmax_rows_kernel<kRowsSmallTile><<<pl->grid, kBlock, 0, st>>>(x, y, rows, w);
     return launch_status();
   }
   // slabs with inner > 1 walk their columns in loops, one exponential after the other: ahead of the packed
@@ -2158,6 +2194,7 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
     const uint64_t per_group = 4ull * kBlock;  // rows (slabs) of a workgroup
     const uint32_t grid = static_cast<uint32_t>((rows + per_group - 1) / per_group);
     const uint32_t d = static_cast<uint32_t>(dim), inner = static_cast<uint32_t>(inner_num);
+    if (pl->chosen(SHDW_PATH_SHORT_ROWS, dim * inner_num, grid)) return SHDW_OK;
     switch (dim * inner_num) {
 #define SHDW_SHORT_ROWS(D) case D: softmax_short_rows_kernel<D><<<grid, kBlock, 0, st>>>(x, y, rows, d, inner); break;
       SHDW_SHORT_ROWS(2) SHDW_SHORT_ROWS(3) SHDW_SHORT_ROWS(4) SHDW_SHORT_ROWS(5) SHDW_SHORT_ROWS(6)
@@ -2169,61 +2206,71 @@ int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, floa
   }
   if (FastDiv fq; const uint32_t quads = quad_count(outer_num, dim, inner_num, true, &fq)) {
     const uint32_t d = static_cast<uint32_t>(dim), inner = static_cast<uint32_t>(inner_num);
-    softmax_quads_reg_kernel<kQuadMaxDim><<<grid_for(quads), kBlock, 0, st>>>(x, y, quads, d, inner, fq);
+    if (pl->chosen(SHDW_PATH_QUADS, 0, grid_for(quads))) return SHDW_OK;
+    softmax_quads_reg_kernel<kQuadMaxDim><<<pl->grid, kBlock, 0, st>>>(x, y, quads, d, inner, fq);
     return launch_status();
   }
   if (const uint32_t group = packed_group(dim, inner_num)) {
     const uint32_t slabs = static_cast<uint32_t>(outer_num);
-    softmax_packed_kernel<<<(slabs + group - 1) / group, kBlock, packed_bytes(dim, inner_num, group), st>>>(
+    if (pl->chosen(SHDW_PATH_PACKED, static_cast<int>(group), (slabs + group - 1) / group)) return SHDW_OK;
+    softmax_packed_kernel<<<pl->grid, kBlock, packed_bytes(dim, inner_num, group), st>>>(
         x, y, slabs, static_cast<uint32_t>(dim), fi, make_fastdiv(static_cast<uint32_t>(dim) * inner_num), group);
-  } else if (long_slab(outer_num, dim, inner_num, true))
+  } else if (long_slab(outer_num, dim, inner_num, true)) {
+    if (pl->chosen(SHDW_PATH_LONG_SLAB, 0, static_cast<uint32_t>(outer_num))) return SHDW_OK;
     softmax_long_slab_kernel<<<outer_num, kBlock, 0, st>>>(x, y, static_cast<uint32_t>(dim), fi);
-  else if (g.use_slab)
+  } else if (g.use_slab) {
+    if (pl->chosen(SHDW_PATH_SLAB, 0, static_cast<uint32_t>(outer_num))) return SHDW_OK;
     softmax_slab_kernel<<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, static_cast<uint32_t>(dim), fi);
-  else if (dim <= 64) {
+  } else if (dim <= 64) {
     // the tile kernel is slower here: [64,49,128,128] 115 us against 88
     const uint32_t grid = grid_for(g.columns), d = static_cast<uint32_t>(dim);
-    if (dim <= 16)
+    const int dmax = dim <= 16 ? 16 : (dim <= 32 ? 32 : (dim <= 48 ? 48 : 64));
+    if (pl->chosen(SHDW_PATH_COLUMNS_REG, dmax, grid)) return SHDW_OK;
+    if (dmax == 16)
       softmax_columns_reg_kernel<16, 0><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi);
-    else if (dim <= 32)
+    else if (dmax == 32)
       softmax_columns_reg_kernel<32, 16><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi);
-    else if (dim <= 48)
+    else if (dmax == 48)
       softmax_columns_reg_kernel<48, 32><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi);
     else
       softmax_columns_reg_kernel<64, 48><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi);
-  }
-  else if (tile_fits(dim, inner_num, true) && dim * 64 * sizeof(float) <= kTileLdsBytes - 1024)
-    launch_softmax_tile_ts<6>(outer_num, dim, inner_num, x, y, st);
-  else if (tile_fits(dim, inner_num, true) && dim * 32 * sizeof(float) <= kTileLdsBytes)
-    launch_softmax_tile_ts<5>(outer_num, dim, inner_num, x, y, st);
-  else if (tile_fits(dim, inner_num, true))
-    launch_softmax_tile_ts<4>(outer_num, dim, inner_num, x, y, st);
-  else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, &t))
+  } else if (tile_fits(dim, inner_num, true)) {
+    // the widest tile (64, 32 or 16 positions) that fits 64 KB beside the table and the hand-over row
+    const int shift = dim * 64 * sizeof(float) <= kTileLdsBytes - 1024 ? 6 : (dim * 32 * sizeof(float) <= kTileLdsBytes ? 5 : 4);
+    const uint32_t tiles = (static_cast<uint32_t>(inner_num) + (1u << shift) - 1) >> shift;
+    if (pl->chosen(SHDW_PATH_TILE, shift, static_cast<uint32_t>(outer_num) * tiles)) return SHDW_OK;
+    if (shift == 6) launch_softmax_tile_ts<6>(outer_num, dim, inner_num, x, y, st);
+    else if (shift == 5) launch_softmax_tile_ts<5>(outer_num, dim, inner_num, x, y, st);
+    else launch_softmax_tile_ts<4>(outer_num, dim, inner_num, x, y, st);
+  } else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, &t)) {
+    if (pl->chosen(SHDW_PATH_TALL, static_cast<int>(t.width_log2), t.grid)) return SHDW_OK;
     softmax_tall_kernel<<<t.grid, kBlock, 0, st>>>(x, y, static_cast<uint32_t>(dim), static_cast<uint32_t>(inner_num),
                                                    t.width_log2, t.f_tiles);
-  else
-    softmax_columns_kernel<<<(g.columns + kWave - 1) / kWave, kWave, 0, st>>>(x, y, g.columns,
-                                                                             static_cast<uint32_t>(dim), fi);
+  } else {
+    if (pl->chosen(SHDW_PATH_COLUMNS, 0, (g.columns + kWave - 1) / kWave)) return SHDW_OK;
+    softmax_columns_kernel<<<pl->grid, kWave, 0, st>>>(x, y, g.columns, static_cast<uint32_t>(dim), fi);
+  }
   return launch_status();
 }
 
-int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps, const float* x,
-                       float* y, void* stream) {
+static int run_normalize(int outer_num, int dim, int inner_num, float p, float eps, const float* x, float* y,
+                         hipStream_t st, ColumnPlan* pl) {
   ColumnGeometry g;
   const int rc = column_geometry(outer_num, dim, inner_num, &g);
   if (rc != SHDW_OK) return rc;
   if (g.columns == 0 || dim == 0) return SHDW_OK;
-  if (!x || !y) return SHDW_E_INVALID_ARGUMENT;
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!pl->want && (!x || !y)) return SHDW_E_INVALID_ARGUMENT;
   const FastDiv fi = make_fastdiv(static_cast<uint32_t>(inner_num));
   const uint32_t d = static_cast<uint32_t>(dim);
   const int mode = p == 1.f ? 1 : (p == 2.f ? 2 : 0);
   if (mode != 0 && rows_apply(outer_num, dim, inner_num)) {
+    if (pl->want) return report_normalize_rows(outer_num, dim, pl);
     if (mode == 1) launch_normalize_rows<1, kSsdNoScale>(outer_num, dim, p, eps, x, nullptr, y, st);
     else launch_normalize_rows<2, kSsdNoScale>(outer_num, dim, p, eps, x, nullptr, y, st);
     return launch_status();
   }
   if (FastDiv fq; const uint32_t quads = mode != 0 ? quad_count(outer_num, dim, inner_num, false, &fq) : 0) {
+    if (pl->chosen(SHDW_PATH_QUADS, 0, grid_for(quads))) return SHDW_OK;
     if (mode == 1) launch_normalize_quads<1, kSsdNoScale>(quads, fq, dim, inner_num, p, eps, x, nullptr, y, st);
     else launch_normalize_quads<2, kSsdNoScale>(quads, fq, dim, inner_num, p, eps, x, nullptr, y, st);
     return launch_status();
@@ -2233,6 +2280,7 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
     const uint32_t grid = (slabs + group - 1) / group;
     const size_t bytes = packed_bytes(dim, inner_num, group);
     const FastDiv fs = make_fastdiv(d * inner_num);
+    if (pl->chosen(SHDW_PATH_PACKED, static_cast<int>(group), grid)) return SHDW_OK;
     if (mode == 1)
       normalize_packed_kernel<1, kSsdNoScale><<<grid, kBlock, bytes, st>>>(x, y, slabs, d, fi, fs, group, p, eps, nullptr);
     else if (mode == 2)
@@ -2240,6 +2288,7 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
     else
       normalize_packed_kernel<0, kSsdNoScale><<<grid, kBlock, bytes, st>>>(x, y, slabs, d, fi, fs, group, p, eps, nullptr);
   } else if (long_slab(outer_num, dim, inner_num, false)) {
+    if (pl->chosen(SHDW_PATH_LONG_SLAB, 0, static_cast<uint32_t>(outer_num))) return SHDW_OK;
     if (mode == 1)
       normalize_long_slab_kernel<1, kSsdNoScale><<<outer_num, kBlock, 0, st>>>(x, y, d, fi, p, eps, nullptr);
     else if (mode == 2)
@@ -2247,6 +2296,7 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
     else
       normalize_long_slab_kernel<0, kSsdNoScale><<<outer_num, kBlock, 0, st>>>(x, y, d, fi, p, eps, nullptr);
   } else if (g.use_slab) {
+    if (pl->chosen(SHDW_PATH_SLAB, 0, static_cast<uint32_t>(outer_num))) return SHDW_OK;
     if (mode == 1)
       normalize_slab_kernel<1><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
     else if (mode == 2)
@@ -2254,6 +2304,7 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
     else
       normalize_slab_kernel<0><<<outer_num, kBlock, g.slab_bytes, st>>>(x, y, d, fi, p, eps);
   } else if (mode != 0 && tile_fits(dim, inner_num, false)) {
+    if (pl->want) return report_normalize_tile(outer_num, dim, inner_num, pl);
     if (mode == 1)
       launch_normalize_tile<1, kSsdNoScale>(outer_num, dim, inner_num, p, eps, x, nullptr, y, st);
     else
@@ -2262,6 +2313,7 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
     // p = 1 and p = 2 keep short columns in registers (one read, one write);
     // the generic-p form would unroll a powf per element and stays two-pass.
     const uint32_t grid = grid_for(g.columns);
+    if (pl->chosen(SHDW_PATH_COLUMNS_REG, dim <= 16 ? 16 : 64, grid)) return SHDW_OK;
     if (mode == 1) {
       if (dim <= 16)
         normalize_columns_reg_kernel<1, 16><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
@@ -2274,6 +2326,7 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
         normalize_columns_reg_kernel<2, 64><<<grid, kBlock, 0, st>>>(x, y, g.columns, d, fi, p, eps);
     }
   } else if (TallLaunch t; tall_launch(outer_num, dim, inner_num, &t)) {
+    if (pl->chosen(SHDW_PATH_TALL, static_cast<int>(t.width_log2), t.grid)) return SHDW_OK;
     if (mode == 1)
       launch_normalize_tall<1, kSsdNoScale>(t, dim, inner_num, p, eps, x, nullptr, y, st);
     else if (mode == 2)
@@ -2282,6 +2335,7 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
       launch_normalize_tall<0, kSsdNoScale>(t, dim, inner_num, p, eps, x, nullptr, y, st);
   } else {
     const uint32_t grid = (g.columns + kWave - 1) / kWave;
+    if (pl->chosen(SHDW_PATH_COLUMNS, 0, grid)) return SHDW_OK;
     if (mode == 1)
       normalize_columns_kernel<1><<<grid, kWave, 0, st>>>(x, y, g.columns, d, fi, p, eps);
     else if (mode == 2)
@@ -2290,6 +2344,46 @@ int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps
       normalize_columns_kernel<0><<<grid, kWave, 0, st>>>(x, y, g.columns, d, fi, p, eps);
   }
   return launch_status();
+}
+
+}  // namespace shdw
+
+using namespace shdw;
+
+extern "C" {
+
+int shdw_hip_softmax(int outer_num, int dim, int inner_num, const float* x, float* y,
+                     void* stream) {
+  ColumnPlan pl;
+  return run_softmax(outer_num, dim, inner_num, x, y, static_cast<hipStream_t>(stream), &pl);
+}
+
+int shdw_hip_normalize(int outer_num, int dim, int inner_num, float p, float eps, const float* x,
+                       float* y, void* stream) {
+  ColumnPlan pl;
+  return run_normalize(outer_num, dim, inner_num, p, eps, x, y, static_cast<hipStream_t>(stream), &pl);
+}
+
+static int hand_back(const ColumnPlan& pl, int* path, int* variant, unsigned* grid) {
+  if (path) *path = pl.path;
+  if (variant) *variant = pl.variant;
+  if (grid) *grid = pl.grid;
+  return SHDW_OK;
+}
+
+int shdw_hip_softmax_plan(int outer_num, int dim, int inner_num, int* path, int* variant, unsigned* grid) {
+  ColumnPlan pl;
+  pl.want = true;
+  const int rc = run_softmax(outer_num, dim, inner_num, nullptr, nullptr, nullptr, &pl);
+  return rc != SHDW_OK ? rc : hand_back(pl, path, variant, grid);
+}
+
+int shdw_hip_normalize_plan(int outer_num, int dim, int inner_num, float p, int* path, int* variant,
+                            unsigned* grid) {
+  ColumnPlan pl;
+  pl.want = true;
+  const int rc = run_normalize(outer_num, dim, inner_num, p, 1e-12f, nullptr, nullptr, nullptr, &pl);
+  return rc != SHDW_OK ? rc : hand_back(pl, path, variant, grid);
 }
 
 }  // extern "C"

@@ -1058,9 +1058,21 @@ static int check_pool_dims(int n, const int* in_shape, const int* out_shape) {
   return SHDW_OK;
 }
 
+// The decision of run_pooling, handed back instead of a launch when `want` is set
+// (shdw_hip_pooling2d_plan).
+struct PoolPlan {
+  int path = SHDW_PATH_NONE, variant = 0;
+  uint32_t grid = 0;
+  bool want = false;
+  bool chosen(int p, int v, uint32_t g) {
+    path = p, variant = v, grid = g;
+    return want;
+  }
+};
+
 static int run_pooling(bool three_d, const int* in_shape, int pool_type, const int* kernel,
                        const int* stride, const int* pad, const int* out_shape, const float* x,
-                       float* y, hipStream_t st) {
+                       float* y, hipStream_t st, PoolPlan* pl) {
   const int nsp = three_d ? 3 : 2;
   if (!in_shape || !out_shape || pool_type < 0 || pool_type > 1) return SHDW_E_INVALID_ARGUMENT;
   const int rc = check_pool_dims(nsp + 2, in_shape, out_shape);
@@ -1070,7 +1082,7 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
   int64_t out_count = 1, in_count = 1;
   for (int k = 0; k < nsp + 2; ++k) out_count *= out_shape[k], in_count *= in_shape[k];
   if (out_count == 0) return SHDW_OK;
-  if (!x || !y || in_count == 0) return SHDW_E_INVALID_ARGUMENT;
+  if (in_count == 0 || (!pl->want && (!x || !y))) return SHDW_E_INVALID_ARGUMENT;
 
   // One window that is exactly the unpadded plane: rows of contiguous elements.
   bool whole_plane = true;
@@ -1087,11 +1099,18 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
       // (per 51 MB: 3x3 planes 10.9 us against 19.1 us here, 7x7 10.3 / 12.9,
       // 14x14 10.1 / 16.5, 56x56 10.7 / 99).
       int rc = SHDW_OK;
+      if (pl->want) {
+        pl->chosen(reduce_rows_max_applies(rows, static_cast<uint32_t>(plane)) ? SHDW_PATH_POOL_PLANE_REDUCE
+                                                                               : SHDW_PATH_POOL_PLANE, 0, 0);
+        return SHDW_OK;
+      }
       if (reduce_rows_max(rows, static_cast<uint32_t>(plane), x, y, st, &rc)) return rc;
       launch_pool_plane<true>(x, y, rows, static_cast<uint32_t>(plane), st);
     } else if (plane >= kPlaneStreamMinLen) {
+      if (pl->chosen(SHDW_PATH_POOL_PLANE_STREAM, 0, 0)) return SHDW_OK;
       launch_pool_rows_stream(x, y, rows, static_cast<uint32_t>(plane), st);
     } else {
+      if (pl->chosen(SHDW_PATH_POOL_PLANE, 0, 0)) return SHDW_OK;
       launch_pool_plane<false>(x, y, rows, static_cast<uint32_t>(plane), st);
     }
     return launch_status();
@@ -1113,6 +1132,8 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
   if (!three_d && plan_small_planes(p, static_cast<int64_t>(in_shape[0]) * in_shape[1], pool_type == 0, &sp, &separable)) {
     const uint32_t grid = (sp.total_planes + sp.planes - 1) / sp.planes;
     const int k = p.kh == p.kw && (p.kh == 2 || p.kh == 3) ? p.kh : 0;
+    const int unrolled = !separable ? k : (pool_type == 0 ? (sp.quads_max ? p.kw : 0) : (wide_unrolled(p.kw) ? p.kw : 0));
+    if (pl->chosen(SHDW_PATH_POOL_SMALL_PLANES, (separable ? 100 : 0) + unrolled, grid)) return SHDW_OK;
     if (separable && pool_type == 0) {
       const size_t both = static_cast<size_t>(sp.planes) * (sp.plane_lds + (sp.quads_max ? 4 : 1) * sp.f_row_maxima.d) * sizeof(float);
       switch (sp.quads_max ? p.kw : 0) {  // the common square windows at a column stride of one: by quads
@@ -1161,6 +1182,7 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
       const int k = p.kh == p.kw && (p.kh == 2 || p.kh == 3 || (p.kh == 5 && a.wide)) ? p.kh : 0;
       const int vecs = (a.tile_rows * p.in_w / 4 + kBlock - 1) / kBlock;  // per lane and band
       const int regs = !pipe ? 0 : (vecs <= 2 ? 2 : (vecs <= 3 ? 3 : (vecs <= 4 ? 4 : (vecs <= 6 ? 6 : 8))));
+      if (pl->chosen(SHDW_PATH_POOL_BAND, 100 * regs + k, g)) return SHDW_OK;
 #define SHDW_LAUNCH_BAND(MAXV, KV)                                                              \
   do {                                                                                           \
     switch (regs) {                                                                              \
@@ -1196,6 +1218,7 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
     }
   }
   const uint32_t grid = grid_for(n_out);
+  if (pl->chosen(SHDW_PATH_POOL_WINDOW, 0, grid)) return SHDW_OK;
   if (three_d) {
     if (pool_type == 0)
       pool_window_kernel<true, true><<<grid, kBlock, 0, st>>>(x, y, n_out, p);
@@ -1244,8 +1267,25 @@ int shdw_hip_pooling2d(const int* in_shape, int pool_type, int kernel_h, int ker
                        const float* x, float* y, void* stream) {
   const int kernel[2] = {kernel_h, kernel_w}, stride[2] = {stride_h, stride_w},
             pad[2] = {pad_h, pad_w};
+  PoolPlan pl;
   return run_pooling(false, in_shape, pool_type, kernel, stride, pad, out_shape, x, y,
-                     static_cast<hipStream_t>(stream));
+                     static_cast<hipStream_t>(stream), &pl);
+}
+
+int shdw_hip_pooling2d_plan(const int* in_shape, int pool_type, int kernel_h, int kernel_w,
+                            int stride_h, int stride_w, int pad_h, int pad_w, const int* out_shape,
+                            int* path, int* variant, unsigned* grid) {
+  const int kernel[2] = {kernel_h, kernel_w}, stride[2] = {stride_h, stride_w},
+            pad[2] = {pad_h, pad_w};
+  PoolPlan pl;
+  pl.want = true;
+  const int rc = run_pooling(false, in_shape, pool_type, kernel, stride, pad, out_shape, nullptr, nullptr,
+                             nullptr, &pl);
+  if (rc != SHDW_OK) return rc;
+  if (path) *path = pl.path;
+  if (variant) *variant = pl.variant;
+  if (grid) *grid = pl.grid;
+  return SHDW_OK;
 }
 
 int shdw_hip_pooling3d(const int* in_shape, int pool_type, int kernel_d, int kernel_h,
@@ -1254,8 +1294,9 @@ int shdw_hip_pooling3d(const int* in_shape, int pool_type, int kernel_d, int ker
                        void* stream) {
   const int kernel[3] = {kernel_d, kernel_h, kernel_w}, stride[3] = {stride_d, stride_h, stride_w},
             pad[3] = {pad_d, pad_h, pad_w};
+  PoolPlan pl;
   return run_pooling(true, in_shape, pool_type, kernel, stride, pad, out_shape, x, y,
-                     static_cast<hipStream_t>(stream));
+                     static_cast<hipStream_t>(stream), &pl);
 }
 
 }  // extern "C"
