@@ -91,6 +91,10 @@ int shdw_hip_last_error(void);
 int shdw_hip_malloc(void** ptr, size_t bytes);
 /* ref: shadow/core/allocator.cu:47 (GPUAllocator::free -> cudaFree) */
 int shdw_hip_free(void* ptr);
+/* Free and total memory of the current device (hipMemGetInfo).  No counterpart in
+ * the reference: it lets a caller, and the tests, see that an entry point which
+ * promises not to allocate leaves the device's free memory as it was. */
+int shdw_hip_mem_info(size_t* free_bytes, size_t* total_bytes);
 /* ref: shadow/core/allocator.cu:29-36 (write: H2D; blocking when stream==NULL) */
 int shdw_hip_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream);
 /* ref: shadow/core/allocator.cu:20-27 (read: D2H; blocking when stream==NULL) */
@@ -229,7 +233,10 @@ int shdw_hip_reduce(int operation, int num_axes, const int* in_shape, int num_re
  * shdw_hip_reduce_static_max_workspace_bytes() is rejected with
  * SHDW_E_STATIC_SCRATCH and nothing is launched.  All calls on one GPU share the
  * buffer: calls that overlap in time on one GPU (different streams, different
- * threads) race; calls on one stream are ordered and safe. */
+ * threads) race; calls on one stream are ordered and safe.  The buffer's address
+ * is looked up once per device, by shdw_hip_set_device or else by the first call
+ * of this entry point on that device: a caller that captures a stream makes
+ * either of the two before the capture begins. */
 int shdw_hip_reduce_static(int operation, int num_axes, const int* in_shape, int num_reduce,
                            const int* axes, const float* x, float* y, void* stream);
 size_t shdw_hip_reduce_static_max_workspace_bytes(void);

@@ -75,6 +75,7 @@ SIGNATURES = {
     "shdw_hip_reduce_static": (_I, [_I, _I, c_int_p, _I, c_int_p, _V, _V, _V]),
     "shdw_hip_reduce_static_max_workspace_bytes": (_Z, []),
     "shdw_hip_scale_residual_relu_rowmean": (_I, [_I, _I, _I, _V, _V, _V, _V, _V, _V, _V]),
+    "shdw_hip_mem_info": (_I, [ctypes.POINTER(_Z), ctypes.POINTER(_Z)]),
     "shdw_hip_softmax_plan": (_I, [_I, _I, _I, c_int_p, c_int_p, ctypes.POINTER(ctypes.c_uint)]),
     "shdw_hip_normalize_plan": (_I, [_I, _I, _I, _F, c_int_p, c_int_p, ctypes.POINTER(ctypes.c_uint)]),
     "shdw_hip_pooling2d_plan": (_I, [c_int_p, _I, _I, _I, _I, _I, _I, _I, c_int_p, c_int_p, c_int_p,

@@ -90,6 +90,14 @@ int shdw_hip_free(void* ptr) {
   return rc(hipFree(ptr));
 }
 
+int shdw_hip_mem_info(size_t* free_bytes, size_t* total_bytes) {
+  size_t f = 0, t = 0;
+  const int code = rc(hipMemGetInfo(&f, &t));
+  if (free_bytes) *free_bytes = f;
+  if (total_bytes) *total_bytes = t;
+  return code;
+}
+
 int shdw_hip_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream) {
   return copy(dst, src, bytes, hipMemcpyHostToDevice, stream);
 }

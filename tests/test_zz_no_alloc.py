@@ -70,3 +70,31 @@ def test_unsliced_shapes_and_errors(gpu):
     rc = lib.shdw_hip_reduce_static(1, 3, ints(shape), 1, ints(axes), d.ptr, y.ptr, None)
     assert rc == -4 and b"static" in lib.shdw_hip_error_string(rc)
     assert lib.shdw_hip_reduce_static(1, 1, ints([8]), 1, ints([0]), None, y.ptr, None) == -1
+
+
+def test_a_warmed_up_call_leaves_the_free_device_memory_as_it_was(gpu):
+    """Sliced shapes, whose partials go to the library's own buffer: nothing is allocated for them."""
+    import ctypes
+    lib = shadow_amd.hip()
+
+    def free_bytes():
+        f, t = ctypes.c_size_t(), ctypes.c_size_t()
+        check(lib.shdw_hip_mem_info(ctypes.byref(f), ctypes.byref(t)))
+        assert 0 < f.value <= t.value
+        return f.value
+
+    shape, axes = [2, 6000, 512], [1]
+    assert lib.shdw_hip_reduce_workspace_bytes(3, ints(shape), 1, ints(axes)) > 0
+    d, y = Buffer.from_numpy(normal(920, shape).ravel()), Buffer(4 * 2 * 512)
+    check(lib.shdw_hip_reduce_static(1, 3, ints(shape), 1, ints(axes), d.ptr, y.ptr, None))  # warm-up: module, symbol
+    check(lib.shdw_hip_stream_sync(None))
+    before = free_bytes()
+    for op in (1, 2, 4):
+        check(lib.shdw_hip_reduce_static(op, 3, ints(shape), 1, ints(axes), d.ptr, y.ptr, None))
+    check(lib.shdw_hip_reduce_static(1, 1, ints([1 << 22]), 1, ints([0]), d.ptr, y.ptr, None))
+    check(lib.shdw_hip_stream_sync(None))
+    assert free_bytes() == before
+    # the workspace form of the same call, by contrast, has its caller allocate: the probe sees that
+    ws = Buffer(64 << 20)
+    assert free_bytes() < before
+    ws.free()
