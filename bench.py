@@ -104,6 +104,9 @@ def parse():
     ap.add_argument("--launch-shapes", action="store_true",
                     help="run tests/native/launch_shapes (alternative launch shapes of the streaming, strided-reduce "
                          "and channel-tile kernels), print its table and how the shapes in use compare, exit")
+    ap.add_argument("--scaling", action="store_true",
+                    help="time the BASELINE reductions, broadcasts and the bottleneck tail at 1x, 2x and 4x their batch "
+                         "and fit time = fixed + bytes / rate per operator (what a launch costs before it streams), exit")
     ap.add_argument("--table", default=os.path.join(ROOT, "gpurun_out", "bench_table.json"),
                     help="file that receives every row of the measurement; the final stdout line is a short record")
     return ap.parse_args()
@@ -485,6 +488,105 @@ def sweep(dev):
     print("worst of each family:")
     for family, (ratio, name) in worst.items():
         print("  %-14s %6.2f x copy  (%s)" % (family, ratio, name))
+
+
+def scaling(dev):
+    """Each BASELINE operator whose tensor is 25-70 MB at 1x, 2x and 4x its batch (the leading
+    extent), operands rotating through 1.2 GB pools, with a plain read / write / copy of the
+    same bytes beside it.  A least-squares line time = fixed + bytes / rate through the three
+    points separates what a launch costs before and after it streams (ramp, the last
+    workgroups, a dependent second launch) from the rate it streams at."""
+    lib, st = dev.lib, dev.stream
+    I = dev.sa.ints
+    POOL = 6 * 205520896
+    rp, wp = dev.buf(nbytes=POOL), dev.buf(nbytes=POOL)
+    seed = dev.buf(normal(999, 12845056))
+    piece = 4 * 12845056
+    for k in range(POOL // piece):
+        dev.ck(lib.shdw_hip_memcpy_d2d(rp.ptr + k * piece, seed.ptr, piece, st))
+    dev.sync()
+    seed.free()
+    small = dev.buf(uniform(5, 1 << 20, 0.5, 2.0))
+    ws = dev.buf(nbytes=64 << 20)
+    sink = dev.buf(nbytes=256)
+
+    def reduce_case(op, shape, axes):
+        def make(m):
+            shp = [shape[0] * m] + shape[1:]
+            n = int(np.prod(shp))
+            outs = n // int(np.prod([shp[a] for a in axes]))
+            need = lib.shdw_hip_reduce_workspace_bytes(len(shp), I(shp), len(axes), I(axes))
+            assert need <= (64 << 20)
+            sets = POOL // (4 * n)
+            fn = lambda k: lib.shdw_hip_reduce(op, len(shp), I(shp), len(axes), I(axes), rp.ptr + k * 4 * n,
+                                               wp.ptr + k * 4 * outs, ws.ptr if need else None, need, st)
+            return fn, sets, 4 * n, 4 * outs
+        return make
+
+    def bcast_case(op, sa, sb):
+        def make(m):
+            a_shape, b_shape = [sa[0] * m] + sa[1:], list(sb)
+            out = [max(p, q) for p, q in zip(a_shape, b_shape)]
+            na, nb, no = int(np.prod(a_shape)), int(np.prod(b_shape)), int(np.prod(out))
+            sets = POOL // (4 * no)
+            ia, ib, io = I(a_shape), I(b_shape), I(out)
+            fn = lambda k: lib.shdw_hip_broadcast_binary(op, len(out), ia, ib, io, rp.ptr, small.ptr, wp.ptr + k * 4 * no, st)
+            return fn, sets, 4 * (na + nb), 4 * no
+        return make
+
+    def tail_case(m):
+        n, C, inner = 12845056 * m, 1024, 196
+        sets = POOL // (4 * n) - 1
+        fn = lambda k: lib.shdw_hip_scale_residual_relu_rowmean(n, C, inner, rp.ptr + k * 4 * n, small.ptr, small.ptr + 4096,
+                                                                 rp.ptr + (k + 1) * 4 * n, wp.ptr + k * 4 * n,
+                                                                 ws.ptr, st)
+        return fn, sets, 8 * n + 8 * C, 4 * n + 4 * (n // inner)
+
+    def plain(kind):
+        def make(m, nbytes):
+            per_side = nbytes // 2 if kind == "copy" else nbytes
+            n = per_side // 4
+            sets = max(1, POOL // (4 * n))
+            if kind == "copy":
+                return (lambda k: lib.shdw_hip_copy(n, rp.ptr + k * 4 * n, wp.ptr + k * 4 * n, st)), sets
+            if kind == "read":
+                return (lambda k: lib.shdw_hip_probe_read(n, rp.ptr + k * 4 * n, 1e30, sink.ptr, st)), sets
+            return (lambda k: lib.shdw_hip_set(n, 1.0, wp.ptr + k * 4 * n, st)), sets
+        return make
+
+    cases = [("cfg3 reduce sum {2,3} [32m,512,28,28]", reduce_case(1, [32, 512, 28, 28], [2, 3]), "read"),
+             ("cfg3 reduce max {1} [32m,512,28,28]", reduce_case(2, [32, 512, 28, 28], [1]), "read"),
+             ("cfg3 reduce sum {1} [32m,512,28,28]", reduce_case(1, [32, 512, 28, 28], [1]), "read"),
+             ("cfg3 reduce sum all [32m,512,28,28] (2 launches)", reduce_case(1, [32, 512, 28, 28], [0, 1, 2, 3]), "read"),
+             ("cfg5 reduce avg {2,3} [64m,1024,14,14]", reduce_case(4, [64, 1024, 14, 14], [2, 3]), "read"),
+             ("cfg5 fused tail [64m,1024,14,14]", tail_case, "copy"),
+             ("cfg1 add [8m,64,112,112] + [1,64,1,1]", bcast_case(0, [8, 64, 112, 112], [1, 64, 1, 1]), "copy"),
+             ("cfg4(i) mul [16m,1,128,256] x [1,32,128,1]", bcast_case(2, [16, 1, 128, 256], [1, 32, 128, 1]), "write"),
+             ("cfg4(i) div", bcast_case(3, [16, 1, 128, 256], [1, 32, 128, 1]), "write"),
+             ("cfg4(ii) mul [4m,64,1,512] x [1,1,64,512]", bcast_case(2, [4, 64, 1, 512], [1, 1, 64, 512]), "write")]
+
+    def fit(points):  # [(bytes, us)] -> fixed us, GB/s
+        b = np.array([p[0] for p in points], np.float64)
+        t = np.array([p[1] for p in points], np.float64)
+        slope, fixed = np.polyfit(b, t, 1)
+        return fixed, 1e-3 / slope
+
+    print("%-52s %27s %27s %27s   %s" % ("operator (m = 1, 2, 4)", "bytes", "us", "us of a plain pass", "fit: fixed us + bytes / GB/s"))
+    for name, make, kind in cases:
+        mine, yard, sizes = [], [], []
+        for m in (1, 2, 4):
+            fn, sets, rd, wr = make(m)
+            us = time_median(dev, fn, max(1, sets), reps=20) * 1e3
+            pfn, psets = plain(kind)(m, rd + wr)
+            pus = time_median(dev, pfn, psets, reps=20) * 1e3
+            mine.append((rd + wr, us)), yard.append((rd + wr, pus)), sizes.append(rd + wr)
+        f0, r0 = fit(mine)
+        f1, r1 = fit(yard)
+        print("%-52s %27s %27s %27s   %.2f us + bytes / %.0f GB/s   (plain %s: %.2f us + bytes / %.0f GB/s)" % (
+            name, " ".join("%d" % b for b in sizes), " ".join("%7.2f" % p[1] for p in mine),
+            " ".join("%7.2f" % p[1] for p in yard), f0, r0, kind, f1, r1), flush=True)
+    for b in (rp, wp, small, ws, sink):
+        b.free()
 
 
 def launch_shapes():
@@ -1153,6 +1255,9 @@ def main():
         launch_shapes()
         return
     dev = Dev()
+    if args.scaling:
+        scaling(dev)
+        return
     if args.sweep:
         sweep(dev)
         return
