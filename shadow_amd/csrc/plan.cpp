@@ -235,6 +235,12 @@ int plan_reduce(int num_axes, const int* in_shape, int num_reduce, const int* ax
         break;
       }
     }
+    // 1024-byte pieces stream at the rate of a plain read where 512-byte pieces reach
+    // four fifths of it (max over 512 of [128,512,784]: 35.8 -> 32.9 us), but a launch of
+    // few such tiles starts and ends slowly (2.5 us more at 128 workgroups, level at 256):
+    // taken from two workgroups per CU on, and only where they are mostly full.
+    if (inner4 >= 64 && ((inner4 + 63) / 64) * plan->outer >= 512 && inner4 * 4 >= ((inner4 + 63) / 64) * 64 * 3)
+      lanes = 64;
     plan->strided_lanes = lanes;
     const int64_t blocks = ((inner4 + lanes - 1) / lanes) * plan->outer;
     const int by_fill = ceil_div64(want, blocks);
