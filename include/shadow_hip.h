@@ -203,6 +203,14 @@ int shdw_hip_scale_bias(int n, int scale_num, int inner_num, const float* x,
  * ref: shadow/operators/kernels/eltwise.hpp:18-71 */
 int shdw_hip_eltwise(int operation, int k, const float* const* xs, const float* coeff,
                      int n, float* y, void* stream);
+/* The same followed by Activate(relu) on the result, in the same pass: the
+ * residual add and ReLU that close a block of a converted network whose
+ * normalisation was folded into the convolution (the Native backend's fusion
+ * pass calls this one).  Results are those of shdw_hip_eltwise followed by
+ * shdw_hip_activate(relu) in place.
+ * ref: shadow/operators/kernels/eltwise.hpp:18-71, activate.cpp:11-12 */
+int shdw_hip_eltwise_relu(int operation, int k, const float* const* xs, const float* coeff,
+                          int n, float* y, void* stream);
 
 /* ================================= Reduce ================================ */
 

@@ -69,6 +69,7 @@ SIGNATURES = {
     "shdw_hip_prelu": (_I, [_I, _I, _I, _I, _V, _V, _V, _V]),
     "shdw_hip_scale_bias": (_I, [_I, _I, _I, _V, _V, _V, _I, _V, _V]),
     "shdw_hip_eltwise": (_I, [_I, _I, c_void_pp, c_float_p, _I, _V, _V]),
+    "shdw_hip_eltwise_relu": (_I, [_I, _I, c_void_pp, c_float_p, _I, _V, _V]),
     "shdw_hip_probe_read": (_I, [_I, _V, _F, _V, _V]),
     "shdw_hip_reduce_workspace_bytes": (_Z, [_I, c_int_p, _I, c_int_p]),
     "shdw_hip_reduce": (_I, [_I, _I, c_int_p, _I, c_int_p, _V, _V, _V, _Z, _V]),

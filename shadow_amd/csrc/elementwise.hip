@@ -174,7 +174,8 @@ SHDW_DEVICE float eltwise_fold(const EltwiseArgs& p, const float (&v)[KMAX], flo
 
 // KMAX is the compile-time bound on p.k (2, 3, 4 or 8) so that the per-input
 // registers are never indexed dynamically.
-template <int OP, int KMAX>
+// RELU: Activate(relu) on the folded value, the Eltwise -> Activate pair in one pass.
+template <int OP, int KMAX, bool RELU = false>
 __global__ __launch_bounds__(kStream) void eltwise_kernel(EltwiseArgs p, float* y, uint32_t n) {
   const uint32_t i = blockIdx.x * kStream + threadIdx.x;
   const uint32_t n4 = n / 4;
@@ -192,6 +193,7 @@ __global__ __launch_bounds__(kStream) void eltwise_kernel(EltwiseArgs p, float* 
 #pragma unroll
       for (int j = 0; j < KMAX; ++j) col[j] = (j < p.k) ? v[j][c] : 0.0f;
       r[c] = eltwise_fold<OP, KMAX>(p, col, seed[c]);
+      if (RELU) r[c] = r[c] > 0 ? r[c] : 0;
     }
     store4_stream_any(y + 4ull * i, r);
   } else if (i == n4) {
@@ -199,24 +201,27 @@ __global__ __launch_bounds__(kStream) void eltwise_kernel(EltwiseArgs p, float* 
       float col[KMAX];
 #pragma unroll
       for (int j = 0; j < KMAX; ++j) col[j] = (j < p.k) ? p.x[j][t] : 0.0f;
-      y[t] = eltwise_fold<OP, KMAX>(p, col, p.has_seed ? y[t] : 0.0f);
+      float r = eltwise_fold<OP, KMAX>(p, col, p.has_seed ? y[t] : 0.0f);
+      if (RELU) r = r > 0 ? r : 0;
+      y[t] = r;
     }
   }
 }
 
 template <int OP, int KMAX>
-static int launch_eltwise_k(const EltwiseArgs& p, int n, float* y, hipStream_t s) {
+static int launch_eltwise_k(const EltwiseArgs& p, int n, float* y, bool relu, hipStream_t s) {
   const uint32_t grid = stream_grid(static_cast<uint32_t>(n) / 4 + 1);
-  eltwise_kernel<OP, KMAX><<<grid, kStream, 0, s>>>(p, y, static_cast<uint32_t>(n));
+  if (relu) eltwise_kernel<OP, KMAX, true><<<grid, kStream, 0, s>>>(p, y, static_cast<uint32_t>(n));
+  else eltwise_kernel<OP, KMAX><<<grid, kStream, 0, s>>>(p, y, static_cast<uint32_t>(n));
   return launch_status();
 }
 
 template <int OP>
-static int launch_eltwise_chunk(const EltwiseArgs& p, int n, float* y, hipStream_t s) {
-  if (p.k <= 2) return launch_eltwise_k<OP, 2>(p, n, y, s);
-  if (p.k == 3) return launch_eltwise_k<OP, 3>(p, n, y, s);
-  if (p.k == 4) return launch_eltwise_k<OP, 4>(p, n, y, s);
-  return launch_eltwise_k<OP, kEltwiseMaxK>(p, n, y, s);
+static int launch_eltwise_chunk(const EltwiseArgs& p, int n, float* y, bool relu, hipStream_t s) {
+  if (p.k <= 2) return launch_eltwise_k<OP, 2>(p, n, y, relu, s);
+  if (p.k == 3) return launch_eltwise_k<OP, 3>(p, n, y, relu, s);
+  if (p.k == 4) return launch_eltwise_k<OP, 4>(p, n, y, relu, s);
+  return launch_eltwise_k<OP, kEltwiseMaxK>(p, n, y, relu, s);
 }
 
 }  // namespace shdw
@@ -335,8 +340,8 @@ int shdw_hip_activate(int type, float slope, int n, const float* x, float* y, vo
 #undef SHDW_CASE
 }
 
-int shdw_hip_eltwise(int operation, int k, const float* const* xs, const float* coeff, int n,
-                     float* y, void* stream) {
+static int run_eltwise(int operation, int k, const float* const* xs, const float* coeff, int n, float* y, bool relu,
+                       void* stream) {
   if (k < 2 || !xs || !y || n < 0) return SHDW_E_INVALID_ARGUMENT;
   if (operation < SHDW_ELTWISE_PROD || operation > SHDW_ELTWISE_MIN) return SHDW_E_INVALID_ARGUMENT;
   for (int j = 0; j < k; ++j)
@@ -368,16 +373,27 @@ int shdw_hip_eltwise(int operation, int k, const float* const* xs, const float* 
       }
     }
     int rc;
+    const bool last = relu && done + p.k == k;  // the activation belongs to the last chunk
     switch (operation) {
-      case SHDW_ELTWISE_PROD: rc = launch_eltwise_chunk<SHDW_ELTWISE_PROD>(p, n, y, s); break;
-      case SHDW_ELTWISE_SUM: rc = launch_eltwise_chunk<SHDW_ELTWISE_SUM>(p, n, y, s); break;
-      case SHDW_ELTWISE_MAX: rc = launch_eltwise_chunk<SHDW_ELTWISE_MAX>(p, n, y, s); break;
-      default: rc = launch_eltwise_chunk<SHDW_ELTWISE_MIN>(p, n, y, s); break;
+      case SHDW_ELTWISE_PROD: rc = launch_eltwise_chunk<SHDW_ELTWISE_PROD>(p, n, y, last, s); break;
+      case SHDW_ELTWISE_SUM: rc = launch_eltwise_chunk<SHDW_ELTWISE_SUM>(p, n, y, last, s); break;
+      case SHDW_ELTWISE_MAX: rc = launch_eltwise_chunk<SHDW_ELTWISE_MAX>(p, n, y, last, s); break;
+      default: rc = launch_eltwise_chunk<SHDW_ELTWISE_MIN>(p, n, y, last, s); break;
     }
     if (rc != SHDW_OK) return rc;
     done += p.k;
   }
   return SHDW_OK;
+}
+
+int shdw_hip_eltwise(int operation, int k, const float* const* xs, const float* coeff, int n,
+                     float* y, void* stream) {
+  return run_eltwise(operation, k, xs, coeff, n, y, false, stream);
+}
+
+int shdw_hip_eltwise_relu(int operation, int k, const float* const* xs, const float* coeff, int n,
+                          float* y, void* stream) {
+  return run_eltwise(operation, k, xs, coeff, n, y, true, stream);
 }
 
 }  // extern "C"

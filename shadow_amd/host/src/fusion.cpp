@@ -232,6 +232,60 @@ class ResidualTail : public FusedGroup {
   bool residual_first_ = false;
 };
 
+// ---- Eltwise -> Activate(relu): shdw_hip_eltwise_relu ----
+// What closes a residual block once the converter has folded the normalisation into
+// the convolution (optimizer.py:181-252): the add and the ReLU.
+bool is_plain_eltwise(const Operator& op) {
+  if (op.type() != "Eltwise" || op.op_param().bottom_size() < 2 || op.op_param().top_size() != 1) return false;
+  const int operation = op.get_single_argument<int>("operation", -1);
+  if (operation < 0 || operation > 3) return false;
+  const auto& p = op.op_param();
+  for (const auto& b : p.bottom())
+    if (b == p.top(0)) return false;  // an output among the inputs has its own pass-by-pass meaning
+  return true;
+}
+
+class EltwiseRelu : public FusedGroup {
+ public:
+  EltwiseRelu(const OpList& ops, int eltwise, int relu) : eltwise_(ops[eltwise]), relu_(ops[relu]) {
+    members_ = {eltwise, relu};
+  }
+
+  bool Run(Workspace* ws) override {
+    const auto& p = eltwise_->op_param();
+    const int operation = eltwise_->get_single_argument<int>("operation", -1);
+    const VecFloat coeff_arg = eltwise_->get_repeated_argument<float>("coeff");
+    if (!coeff_arg.empty() && (operation != kEltwiseSum || coeff_arg.size() != p.bottom().size())) return false;
+    std::vector<const float*> ptrs;
+    std::shared_ptr<Blob> first;
+    for (const auto& name : p.bottom()) {
+      auto blob = float_blob(ws, name);
+      if (blob == nullptr || blob->count() == 0) return false;
+      if (first == nullptr) first = blob;
+      if (blob->shape() != first->shape()) return false;
+      ptrs.push_back(blob->data<float>());
+    }
+    auto y = float_blob(ws, relu_->op_param().top(0));
+    if (y == nullptr) return false;
+    for (const auto& name : p.bottom())
+      if (ws->GetBlob(name) == y) return false;
+    VecFloat coeff(ptrs.size(), 1.f);
+    std::copy(coeff_arg.begin(), coeff_arg.end(), coeff.begin());
+    y->reshape(first->shape());
+    SHADOW_HIP_CHECK(shdw_hip_eltwise_relu(operation, static_cast<int>(ptrs.size()), ptrs.data(),
+                                           operation == kEltwiseSum ? coeff.data() : nullptr, first->count(),
+                                           y->mutable_data<float>(), ws->Ctx()->stream()));
+    return true;
+  }
+
+  std::string describe() const override {
+    return label(*eltwise_) + " + " + label(*relu_) + " -> " + relu_->op_param().top(0);
+  }
+
+ private:
+  std::shared_ptr<Operator> eltwise_, relu_;
+};
+
 }  // namespace
 
 std::vector<std::unique_ptr<FusedGroup>> FindFusedGroups(const OpList& ops,
@@ -279,6 +333,17 @@ std::vector<std::unique_ptr<FusedGroup>> FindFusedGroups(const OpList& ops,
     groups.emplace_back(new ResidualTail(ops, i, next, relu, mean));
     taken[i] = taken[next] = taken[relu] = true;
     if (mean >= 0) taken[mean] = true;
+  }
+  for (int i = 0; i < count; ++i) {
+    if (taken[i] || !is_plain_eltwise(*ops[i])) continue;
+    const std::string& e = ops[i]->op_param().top(0);
+    const int relu = next_reader(ops, e, i);
+    if (relu < 0 || taken[relu] || !is_relu(*ops[relu])) continue;
+    if (ops[relu]->op_param().top(0) != e && !sole_reader(ops, out_blob, e, i, relu)) continue;
+    std::vector<int> members = {i, relu};
+    if (!movable(ops, members)) continue;
+    groups.emplace_back(new EltwiseRelu(ops, i, relu));
+    taken[i] = taken[relu] = true;
   }
   std::sort(groups.begin(), groups.end(),
             [](const std::unique_ptr<FusedGroup>& a, const std::unique_ptr<FusedGroup>& b) {

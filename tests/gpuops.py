@@ -145,8 +145,8 @@ def scale_bias(x, scale, bias, scale_num, inner_num, relu=False, inplace=False, 
     return y.download(count=n, offset_bytes=4 * offset)
 
 
-def eltwise(op, inputs, coeff=None, alias=None):
-    """alias = index of the input whose buffer is also the output."""
+def eltwise(op, inputs, coeff=None, alias=None, relu=False):
+    """alias = index of the input whose buffer is also the output; relu: the fused Eltwise + Activate entry."""
     inputs = [_f(x).ravel() for x in inputs]
     n = inputs[0].size
     bufs = [Buffer.from_numpy(x) for x in inputs]
@@ -155,7 +155,8 @@ def eltwise(op, inputs, coeff=None, alias=None):
     co = None
     if coeff is not None:
         co = (ctypes.c_float * len(coeff))(*[float(c) for c in coeff])
-    check(_lib().shdw_hip_eltwise(op, len(bufs), ptrs, co, n, y.ptr, None))
+    fn = _lib().shdw_hip_eltwise_relu if relu else _lib().shdw_hip_eltwise
+    check(fn(op, len(bufs), ptrs, co, n, y.ptr, None))
     _sync()
     return y.download(count=n)
 

@@ -55,10 +55,10 @@ def data(shape=SHAPE, inputs=("x",), seed=0, specials=True, nparams=2, param_sha
     return weights, feed
 
 
-def run_all(net, weights, feed, written, fp64=(), expect_fused=None, reshape=False):
+def run_all(net, weights, feed, written, fp64=(), expect_fused=None, reshape=False, against_oracle=True):
     """Fused and unfused runs against each other (bit for bit) and against the oracle."""
     text = onet.write_text(net)
-    want = onet.run(net, weights, feed)
+    want = onet.run(net, weights, feed) if against_oracle else None
     with shadow_amd.Network(text, weights, fuse=False) as plain:
         assert plain.fused == []
         plain.forward(feed, reshape=reshape)
@@ -70,8 +70,11 @@ def run_all(net, weights, feed, written, fp64=(), expect_fused=None, reshape=Fal
             nw.forward(feed, reshape=reshape)
             for name in written:
                 got = nw.blob(name)
-                assert list(got.shape) == list(want[name].shape) == list(ref[name].shape), name
+                assert list(got.shape) == list(ref[name].shape), name
                 assert_bit_exact(got, ref[name], name + " fused against unfused")
+                if want is None:
+                    continue
+                assert list(got.shape) == list(want[name].shape), name
                 if name in fp64:
                     assert assert_rel_close(got, want[name], 1e-5, name) == 0
                 else:
@@ -162,35 +165,63 @@ def test_an_operator_between_the_members_that_touches_nothing_of_theirs_is_stepp
     run_all(net, weights, feed, ["e", "m", "pool"], fp64=("pool",), expect_fused=TAIL)
 
 
+ADD_RELU = ["add(Eltwise) + relu(Activate) -> e"]
+# what keeps the Scale out of a group, and what is fused all the same: (operators, out_blob, blobs written, groups)
 BLOCKED = {
     "the Scale output is an output of the network":
-        (tail_ops(), ["s", "pool"], ["s", "e", "pool"]),
+        (tail_ops(), ["s", "pool"], ["s", "e", "pool"], ADD_RELU),
     "the Scale output has a second reader":
-        (tail_ops() + [op("Unary", "abs", ["s"], ["m"], arg_i("operation", 0))], ["m", "pool"], ["s", "e", "m", "pool"]),
+        (tail_ops() + [op("Unary", "abs", ["s"], ["m"], arg_i("operation", 0))], ["m", "pool"], ["s", "e", "m", "pool"],
+         ADD_RELU),
     "an operator in between rewrites the residual":
         (tail_ops()[:1] + [op("Unary", "neg", ["r"], ["r"], arg_i("operation", 13))] + tail_ops()[1:], ["pool"],
-         ["s", "e", "pool"]),
+         ["s", "e", "pool"], ADD_RELU),
     "the sum has coefficients":
         ([scale_op("x", "s"), op("Eltwise", "add", ["s", "r"], ["e"], arg_i("operation", 1), ("coeff", "v_f", [F(1), F(0.5)])),
-          op("Activate", "relu", ["e"], ["e"], arg_i("type", 1))], ["e"], ["s", "e"]),
+          op("Activate", "relu", ["e"], ["e"], arg_i("type", 1))], ["e"], ["s", "e"], ADD_RELU),
     "the Eltwise is a maximum":
         ([scale_op("x", "s"), op("Eltwise", "add", ["s", "r"], ["e"], arg_i("operation", 2)),
-          op("Activate", "relu", ["e"], ["e"], arg_i("type", 1))], ["e"], ["s", "e"]),
+          op("Activate", "relu", ["e"], ["e"], arg_i("type", 1))], ["e"], ["s", "e"], ADD_RELU),
     "the activation is not relu":
-        ([scale_op("x", "s"), op("Activate", "act", ["s"], ["y"], arg_i("type", 6))], ["y"], ["s", "y"]),
+        ([scale_op("x", "s"), op("Activate", "act", ["s"], ["y"], arg_i("type", 6))], ["y"], ["s", "y"], []),
     "the sum is read before it is activated elsewhere":
         ([scale_op("x", "s"), op("Eltwise", "add", ["s", "r"], ["e"], arg_i("operation", 1)),
           op("Activate", "relu", ["e"], ["a"], arg_i("type", 1)), op("Unary", "abs", ["e"], ["m"], arg_i("operation", 0))],
-         ["a", "m"], ["s", "e", "a", "m"]),
+         ["a", "m"], ["s", "e", "a", "m"], []),
 }
 
 
 @pytest.mark.parametrize("why", sorted(BLOCKED))
 def test_blocked(gpu, why):
-    ops, out, written = BLOCKED[why]
+    ops, out, written, groups = BLOCKED[why]
     net = make(ops, out, inputs=("x", "r"))
     weights, feed = data(SHAPE, ("x", "r"), seed=17, specials=False)
-    run_all(net, weights, feed, written, fp64=("pool",), expect_fused=[])
+    run_all(net, weights, feed, written, fp64=("pool",), expect_fused=groups)
+
+
+@pytest.mark.parametrize("operation", [0, 1, 2, 3])
+@pytest.mark.parametrize("inputs", [2, 3, 9])
+@pytest.mark.parametrize("in_place", [True, False])
+def test_eltwise_relu(gpu, operation, inputs, in_place):
+    """The add and the ReLU that close a residual block whose normalisation the converter
+    folded into the convolution; any operation, any number of inputs (nine: two passes)."""
+    names = ["x%d" % k for k in range(inputs)]
+    top = "e" if in_place else "a"
+    args = [arg_i("operation", operation)]
+    if operation == 1 and inputs == 3:
+        args.append(("coeff", "v_f", [F(1), F(-0.5), F(2)]))
+    net = make([op("Eltwise", "add", names, ["e"], *args), op("Activate", "relu", ["e"], [top], arg_i("type", 1)),
+                op("Unary", "abs", [top], ["out"], arg_i("operation", 0))], ["out"], inputs=names, params=())
+    _, feed = data(SHAPE, names, seed=19 + operation, specials=True, nparams=0)
+    run_all(net, [], feed, [top, "out"], expect_fused=["add(Eltwise) + relu(Activate) -> " + top])
+
+
+def test_eltwise_whose_output_is_an_input_stays_an_operator(gpu):
+    net = make([op("Eltwise", "add", ["x", "r"], ["x"], arg_i("operation", 1)),
+                op("Activate", "relu", ["x"], ["x"], arg_i("type", 1))], ["x"], inputs=("x", "r"), params=())
+    _, feed = data(SHAPE, ("x", "r"), seed=23, specials=False, nparams=0)
+    # (the network oracle keeps blobs apart and does not model the cleared input: the two device runs only)
+    run_all(net, [], feed, ["x"], expect_fused=[], against_oracle=False)
 
 
 def test_scale_with_host_values_stays_an_operator(gpu):

@@ -251,6 +251,19 @@ def test_eltwise(gpu, op, k):
     assert_bit_exact(gpuops.eltwise(op, xs, coeff), want, "eltwise")
 
 
+@pytest.mark.parametrize("op", [0, 1, 2, 3])
+@pytest.mark.parametrize("k", [2, 4, 9])
+def test_eltwise_relu(gpu, op, k):
+    """shdw_hip_eltwise_relu is shdw_hip_eltwise followed by relu; with nine inputs the
+    activation belongs to the second pass only."""
+    n = 70003
+    xs = [with_specials(normal(135 + j, n), j) for j in range(k)]
+    coeff = [1.0, -0.5, 2.0, 0.25, 1.0, 1.0, -1.0, 3.0, 0.5][:k] if op == 1 else None
+    want = oracle.activate(oracle.eltwise(op, xs, coeff if coeff else [1.0] * k), 1)
+    got = gpuops.eltwise(op, xs, coeff, relu=True)
+    assert_bit_exact(got, want, "eltwise + relu")
+
+
 def test_eltwise_sum_signed_zero(gpu):
     a = np.float32([-0.0, 0.0, -0.0, 1.0])
     b = np.float32([-0.0, -0.0, 0.0, -1.0])
