@@ -37,6 +37,13 @@ __global__ __launch_bounds__(T) void ew_vec_kernel(F f, const float* a, const fl
                                                     float* y, uint32_t n4, uint32_t n,
                                                     float alpha) {
   const uint32_t first = blockIdx.x * (T * V) + threadIdx.x;
+  // The tanh table's piece is requested first: it comes from the caches and is in
+  // LDS long before the streamed vector arrives.
+  constexpr int kPieces = libm::kTanhSteps * sizeof(libm::TanhStep) / sizeof(v4f);
+  static_assert(!uses_tanh_table<F>::value || kPieces <= T, "one piece per lane");
+  v4f piece;
+  if (uses_tanh_table<F>::value && (kPieces == T || threadIdx.x < kPieces))
+    piece = reinterpret_cast<const v4f*>(libm::kTanhStepTab)[threadIdx.x];
   v4f va[V], vb[V];
 #pragma unroll
   for (int u = 0; u < V; ++u) {  // issue the streaming loads before anything else
@@ -52,6 +59,12 @@ __global__ __launch_bounds__(T) void ew_vec_kernel(F f, const float* a, const fl
     if (threadIdx.x < 32) lds_tab[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
     __syncthreads();
     tab = lds_tab;
+  }
+  if (uses_tanh_table<F>::value) {
+    __shared__ __align__(32) v4f lds_steps[kPieces];
+    if (kPieces == T || threadIdx.x < kPieces) lds_steps[threadIdx.x] = piece;
+    __syncthreads();
+    tab = reinterpret_cast<const uint64_t*>(lds_steps);
   }
 #pragma unroll
   for (int u = 0; u < V; ++u) {

@@ -14,11 +14,17 @@ namespace shdw {
 
 // Functors that evaluate exact_expf declare `static constexpr bool kExpTable =
 // true`; the kernels then stage the 32-entry 2^(i/32) table in LDS and pass it
-// as `tab` (nullptr otherwise).
+// as `tab` (nullptr otherwise).  ATanh declares `kTanhTable` instead and gets the
+// 32 TanhStep entries the same way, behind the same pointer.
 template <class F, class = void>
 struct uses_exp_table { static constexpr bool value = false; };
 template <class F>
 struct uses_exp_table<F, decltype((void)F::kExpTable)> { static constexpr bool value = F::kExpTable; };
+
+template <class F, class = void>
+struct uses_tanh_table { static constexpr bool value = false; };
+template <class F>
+struct uses_tanh_table<F, decltype((void)F::kTanhTable)> { static constexpr bool value = F::kTanhTable; };
 
 // Functors with a long dependent chain per element declare
 // `static constexpr int kVectorsPerLane = 2`: a lane then owns two vectors and
@@ -96,19 +102,31 @@ struct ASigmoid {
 };
 struct ASoftPlus { static constexpr bool kExpTable = true; SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_softplusf(x, tab); } };
 struct ATanh {
-  SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_tanhf(x); }
-  SHDW_DEVICE v4f four(v4f x, const uint64_t*) const {
+  static constexpr bool kTanhTable = true;
+  static constexpr int kVectorsPerLane = 2;
+  static SHDW_DEVICE const libm::TanhStep* steps(const uint64_t* tab) {
+    return reinterpret_cast<const libm::TanhStep*>(tab);
+  }
+  SHDW_DEVICE float operator()(float x, float, const uint64_t* tab) const { return libm::exact_tanhf(x, steps(tab)); }
+  SHDW_DEVICE v4f four(v4f x, const uint64_t* tab) const {
     bool ok = true;
 #pragma unroll
     for (int j = 0; j < 4; ++j) ok &= libm::tanhf_short_ok(x[j]);
     v4f r;
     if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) r[j] = libm::tanhf_short(x[j]);
+      for (int j = 0; j < 4; ++j) r[j] = libm::tanhf_short(x[j], steps(tab));
     } else {
       keep_branch();
 #pragma unroll
-      for (int j = 0; j < 4; ++j) r[j] = libm::tanhf_any(x[j]);
+      for (int j = 0; j < 4; ++j) {
+        // A copy the compiler cannot relate to x[j]: the integer |x| that this form
+        // needs is then computed here and not ahead of the branch, where the short
+        // form (which takes |x| as an operand modifier) would pay for it too.
+        float xj = x[j];
+        asm("" : "+v"(xj));
+        r[j] = libm::tanhf_any(xj, steps(tab));
+      }
     }
     return r;
   }

@@ -196,18 +196,26 @@ SHDW_LIBM_FN float exact_expm1f(float x) {
 
 // tanhf without divergent control flow.  s_tanhf.c calls expm1f only with
 // a = 2|x| in [2, 44) or a = -2|x| in (-2, -2^-54], so of expm1f's cases only
-// k = 0, k = -1, k <= -2 (a < 0) and k >= 3 (a > 0) can occur; each is evaluated
-// with the library's operations in the library's order and the applicable one is
-// selected.  Where a cheaper form gives the same bits on every input it replaces
-// the library's.  Exact rewrites (they change no rounding):
+// k = 0, k = -1, k <= -2 (a < 0) and k >= 3 (a > 0) can occur.  They differ in
+// constants only, which a table indexed by k holds (TanhStep), so every lane runs
+// the same operations whatever its k, in the library's order.  Where a cheaper
+// form gives the same bits on every input it replaces the library's.  Exact
+// rewrites (they change no rounding):
 //   * hxs = x * (0.5 x) is half of s = x * x, and a halving commutes with every
 //     rounding here, so 0.5 * round(s * p) stands for the library's round(hxs * p)
 //     and "v - hxs" is one fused -0.5 * s + v; hfx and hxs are never formed;
-//   * fused operations where the product is exact (a - k * ln2_hi, 0.5 * v - 0.5);
+//   * a = 2 h is never formed either: invln2 * a is (2 invln2) * h, and
+//     a - k * ln2_hi is one fused 2 h - khi, the product k * ln2_hi being exact;
 //   * k = 0 has lo = 0 and therefore c = 0, which makes the library's special
 //     form x - (x * e - hxs) equal to x - e with the general e = x * (e - c) - c
-//     - hxs; k = -1 is 0.5 * (x - e) - 0.5 on the same difference d = x - e, and
-//     the general y = (1 - 2^-k) - (e - x) is (1 - 2^-k) + d.
+//     - hxs.  With d = x - e, the library's results are
+//         k = 0:   d                     k = -1:  0.5 d - 0.5
+//         k <= -2: 2^k (1 + d) - 1       k >= 3:  2^k ((1 - 2^-k) + d)
+//     which are all fma(2^k, T + d, off) with T = 0, 0, 1, 1 - 2^-k and
+//     off = 0, -0.5, -1, 0: T + d is exact where T = 0, the scaling by 2^k is exact
+//     everywhere, so each is rounded where the library rounds it;
+//   * |x| >= 1 returns 1 - q and |x| < 1 the magnitude of q: base - q with base = 1
+//     or 0, which the table holds as well since k >= 3 exactly when |x| >= 1.
 // Rewrites that do change intermediate roundings, kept because the function
 // still returns the library's bits for all 2^32 inputs with them (compared on
 // the host and on the device; none of it is argued from error bounds):
@@ -220,37 +228,83 @@ SHDW_LIBM_FN float exact_expm1f(float x) {
 //     products of t3, of the divisor or of e on thousands);
 //   * y = (1 - 2^-k) + d also for 23 <= k, where the library switches to
 //     (x - (e + 2^-k)) + 1: the two differ far below what 1 - 2 / (t + 2) keeps;
-//   * |x| >= 10 is evaluated at 10 (the result is already exactly 1 there;
-//     the library's own cut is at 22), which also bounds k by 29;
+//   * |x| >= 9.75 is evaluated at 9.75 (the result is already exactly 1 there;
+//     the library's own cut is at 22), which also bounds k by 28;
 //   * the |x| < 2^-55 and |a| < 2^-25 early returns are left to the general
 //     path, which returns x there as well.
-//
-// tanhf_magnitude is |tanhf(x)| from a2 = 2|x| (at most 20) and big = |x| >= 1;
-// exact_tanhf puts the sign back.  On the device a wave whose lanes all have
-// |x| < 10 (no NaN among them) needs neither the cut at 10 nor the NaN case and
-// takes a2 and the sign with one operation each; any other wave goes the long way.
-// Both ways run the same tanhf_magnitude on the same a2.
-SHDW_LIBM_FN float tanhf_magnitude(float a2, bool big) {
+struct alignas(32) TanhStep {
+  float khi, klo;  // k * ln2_hi (exact), k * ln2_lo (rounded as the library's product is)
+  float T, off;    // expm1f(a) = fma(scale, T + d, off)
+  float scale;     // 2^k
+  float base;      // 1 where k >= 1 (|x| >= 1), else 0
+  float pad[2];
+};
+constexpr int kTanhStepLog2Bytes = 5;
+constexpr int kTanhSteps = 32;            // k = -3 ... 28
+constexpr float kTanhCut = 9.75f;         // 2 * 9.75 / ln2 = 28.13
+SHDW_LIBM_TABLE TanhStep kTanhStepTab[kTanhSteps] = {
+    {-0x1.0a2a4p+1f, -0x1.c7e774p-16f, 0x1.0p+0f, -0x1.0p+0f, 0x1.0p-3f, 0.0f, 0.0f, 0.0f},  // k = -3
+    {-0x1.62e3p+0f, -0x1.2fefa2p-16f, 0x1.0p+0f, -0x1.0p+0f, 0x1.0p-2f, 0.0f, 0.0f, 0.0f},  // k = -2
+    {-0x1.62e3p-1f, -0x1.2fefa2p-17f, 0.0f, -0x1.0p-1f, 0x1.0p-1f, 0.0f, 0.0f, 0.0f},  // k = -1
+    {0.0f, 0.0f, 0.0f, 0.0f, 0x1.0p+0f, 0.0f, 0.0f, 0.0f},  // k = 0
+    {0x1.62e3p-1f, 0x1.2fefa2p-17f, 0x1.0p-1f, 0.0f, 0x1.0p+1f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 1
+    {0x1.62e3p+0f, 0x1.2fefa2p-16f, 0x1.8p-1f, 0.0f, 0x1.0p+2f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 2
+    {0x1.0a2a4p+1f, 0x1.c7e774p-16f, 0x1.cp-1f, 0.0f, 0x1.0p+3f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 3
+    {0x1.62e3p+1f, 0x1.2fefa2p-15f, 0x1.ep-1f, 0.0f, 0x1.0p+4f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 4
+    {0x1.bb9bcp+1f, 0x1.7beb8ap-15f, 0x1.fp-1f, 0.0f, 0x1.0p+5f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 5
+    {0x1.0a2a4p+2f, 0x1.c7e774p-15f, 0x1.f8p-1f, 0.0f, 0x1.0p+6f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 6
+    {0x1.3686ap+2f, 0x1.09f1aep-14f, 0x1.fcp-1f, 0.0f, 0x1.0p+7f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 7
+    {0x1.62e3p+2f, 0x1.2fefa2p-14f, 0x1.fep-1f, 0.0f, 0x1.0p+8f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 8
+    {0x1.8f3f6p+2f, 0x1.55ed96p-14f, 0x1.ffp-1f, 0.0f, 0x1.0p+9f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 9
+    {0x1.bb9bcp+2f, 0x1.7beb8ap-14f, 0x1.ff8p-1f, 0.0f, 0x1.0p+10f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 10
+    {0x1.e7f82p+2f, 0x1.a1e97ep-14f, 0x1.ffcp-1f, 0.0f, 0x1.0p+11f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 11
+    {0x1.0a2a4p+3f, 0x1.c7e774p-14f, 0x1.ffep-1f, 0.0f, 0x1.0p+12f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 12
+    {0x1.20587p+3f, 0x1.ede568p-14f, 0x1.fffp-1f, 0.0f, 0x1.0p+13f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 13
+    {0x1.3686ap+3f, 0x1.09f1aep-13f, 0x1.fff8p-1f, 0.0f, 0x1.0p+14f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 14
+    {0x1.4cb4dp+3f, 0x1.1cf0a8p-13f, 0x1.fffcp-1f, 0.0f, 0x1.0p+15f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 15
+    {0x1.62e3p+3f, 0x1.2fefa2p-13f, 0x1.fffep-1f, 0.0f, 0x1.0p+16f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 16
+    {0x1.79113p+3f, 0x1.42ee9cp-13f, 0x1.ffffp-1f, 0.0f, 0x1.0p+17f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 17
+    {0x1.8f3f6p+3f, 0x1.55ed96p-13f, 0x1.ffff8p-1f, 0.0f, 0x1.0p+18f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 18
+    {0x1.a56d9p+3f, 0x1.68ec9p-13f, 0x1.ffffcp-1f, 0.0f, 0x1.0p+19f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 19
+    {0x1.bb9bcp+3f, 0x1.7beb8ap-13f, 0x1.ffffep-1f, 0.0f, 0x1.0p+20f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 20
+    {0x1.d1c9fp+3f, 0x1.8eea84p-13f, 0x1.fffffp-1f, 0.0f, 0x1.0p+21f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 21
+    {0x1.e7f82p+3f, 0x1.a1e97ep-13f, 0x1.fffff8p-1f, 0.0f, 0x1.0p+22f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 22
+    {0x1.fe265p+3f, 0x1.b4e878p-13f, 0x1.fffffcp-1f, 0.0f, 0x1.0p+23f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 23
+    {0x1.0a2a4p+4f, 0x1.c7e774p-13f, 0x1.fffffep-1f, 0.0f, 0x1.0p+24f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 24
+    {0x1.154158p+4f, 0x1.dae66ep-13f, 0x1.0p+0f, 0.0f, 0x1.0p+25f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 25
+    {0x1.20587p+4f, 0x1.ede568p-13f, 0x1.0p+0f, 0.0f, 0x1.0p+26f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 26
+    {0x1.2b6f88p+4f, 0x1.00723p-12f, 0x1.0p+0f, 0.0f, 0x1.0p+27f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 27
+    {0x1.3686ap+4f, 0x1.09f1aep-12f, 0x1.0p+0f, 0.0f, 0x1.0p+28f, 0x1.0p+0f, 0.0f, 0.0f},  // k = 28
+};
+
+// tanhf_magnitude is |tanhf(x)| from h = |x| where |x| >= 1 (`big`) and -|x|
+// otherwise, |x| <= 9.75; exact_tanhf puts the sign back.  `steps` is
+// kTanhStepTab or a copy of it in faster memory.  On the device a wave whose
+// lanes all have |x| < 9.75 (no NaN among them) needs neither the cut nor the NaN
+// case; any other wave goes the long way.  Both ways run the same
+// tanhf_magnitude on the same h.
+SHDW_LIBM_FN float tanhf_magnitude(float h, bool big, const TanhStep* steps) {
   const float one = 1.0f, two = 2.0f, half = 0.5f;
-  const float ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f;
   const float invln2 = 1.4426950216e+00f;
   const float Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f,
               Q4 = 4.0082177293e-06f, Q5 = -2.0109921195e-07f;
-  const float a = big ? a2 : -a2;  // argument of expm1f
 
-  // --- expm1f(a): argument reduction ---
-  // k = rint(a / ln2) by the 1.5 * 2^23 trick: the sum's low mantissa bits are k
-  // in two's complement, which is all the shifts below need of it.
+  // --- expm1f(a), a = 2 h: argument reduction ---
+  // k = rint(a / ln2) by the 1.5 * 2^23 trick, three added so that the sum's low
+  // mantissa bits are the table index k + 3 (0 ... 31 for the h allowed here).
   const float magic = 12582912.0f;
-  const float tsum = __builtin_fmaf(invln2, a, magic);
-  const float tk = tsum - magic;
-  const uint32_t kbits = f2u(tsum);  // k modulo 2^22 in the low bits
-  // tk * ln2_hi is exact (|tk| <= 29, ln2_hi has 17 significant bits), so the
-  // fused form is the library's a - tk * ln2_hi bit for bit
-  const float hi = __builtin_fmaf(-tk, ln2_hi, a);
-  const float lo = tk * ln2_lo;
-  const float xr = hi - lo;
-  const float c = (hi - xr) - lo;
+  const float tsum = __builtin_fmaf(two * invln2, h, magic + 3.0f);
+  uint32_t byte_offset = (f2u(tsum) << kTanhStepLog2Bytes) - (f2u(magic) << kTanhStepLog2Bytes);
+#if defined(__HIP_DEVICE_COMPILE__)
+  // One shift-and-add.  Opaque to the compiler from here on, so that the fields
+  // of the entry are fixed offsets from one address and not a sum each.
+  asm("" : "+v"(byte_offset));
+#endif
+  const TanhStep& st = *static_cast<const TanhStep*>(
+      __builtin_assume_aligned(reinterpret_cast<const char*>(steps) + byte_offset, sizeof(TanhStep)));
+  const float hi = __builtin_fmaf(two, h, -st.khi);
+  const float xr = hi - st.klo;
+  const float c = (hi - xr) - st.klo;
 
   // --- primary range ---
   const float s = xr * xr;  // 2 hxs
@@ -268,46 +322,42 @@ SHDW_LIBM_FN float tanhf_magnitude(float a2, bool big) {
   const float e2x = s * div_normal(r1 - t3, 6.0f - xr * t3);
   float e = xr * __builtin_fmaf(half, e2x, -c) - c;  // x * (e - c) - c
   e = __builtin_fmaf(-half, s, e);                   // - hxs
-  const float d = xr - e;                            // the k = 0 result
-  const float res_km1 = __builtin_fmaf(half, d, -half);
-  // k >= 3: y = (1 - 2^-k) + d, result y * 2^k.  k <= -2: y = 1 + d, result
-  // y * 2^k - 1; the shift count k & 31 is then 29 or more and leaves 1.
-  const float t_lo = u2f(0x3f800000u - (0x1000000u >> (kbits & 31u)));
-  float yk = t_lo + d;
-  yk = u2f(f2u(yk) + (kbits << 23));  // scale by 2^k
-  const float res_gen = big ? yk : yk - one;
-  const float t = (tk == 0.0f) ? d : ((tk == -1.0f) ? res_km1 : res_gen);
+  const float d = xr - e;
+  const float t = __builtin_fmaf(st.scale, st.T + d, st.off);
 
   // --- tanhf ---
-  const float q = div_normal(big ? two : t, t + two);
   // |x| >= 1: 1 - 2 / (t + 2); else -t / (t + 2), whose magnitude is |q|.
-  return big ? one - q : q;
+  const float q = div_normal(big ? two : t, t + two);
+  return st.base - q;
 }
 
 // The long way: any x.
-SHDW_LIBM_FN float tanhf_any(float x) {
+SHDW_LIBM_FN float tanhf_any(float x, const TanhStep* steps) {
   const uint32_t jx = f2u(x);
   const uint32_t ix = jx & 0x7fffffffu;
-  // from |x| = 10 on 2 / (t + 2) < 2^-25 and 1 - q rounds to 1: evaluate at 10
-  const uint32_t ic = ix < 0x41200000u ? ix : 0x41200000u;
-  const float z = tanhf_magnitude(2.0f * u2f(ic), ix >= 0x3f800000u);
+  // from |x| = 9.75 on 2 / (t + 2) < 2^-25 and 1 - q rounds to 1: evaluate there
+  const uint32_t cut = f2u(kTanhCut);
+  const float ac = u2f(ix < cut ? ix : cut);
+  const bool big = ix >= 0x3f800000u;
+  const float z = tanhf_magnitude(big ? ac : -ac, big, steps);
   // The result takes x's sign; a NaN keeps all of its bits.
   const uint32_t keep = (ix > 0x7f800000u) ? 0u : 0x7fffffffu;
   return u2f((f2u(z) & keep) | (jx & ~keep));
 }
 
-// The short way: |x| < 10 (tanhf_short_ok), and so no NaN.
-SHDW_LIBM_FN bool tanhf_short_ok(float x) { return 2.0f * __builtin_fabsf(x) < 20.0f; }
-SHDW_LIBM_FN float tanhf_short(float x) {
-  const float a2 = 2.0f * __builtin_fabsf(x);
-  return __builtin_copysignf(tanhf_magnitude(a2, a2 >= 2.0f), x);
+// The short way: |x| < 9.75 (tanhf_short_ok), and so no NaN.
+SHDW_LIBM_FN bool tanhf_short_ok(float x) { return __builtin_fabsf(x) < kTanhCut; }
+SHDW_LIBM_FN float tanhf_short(float x, const TanhStep* steps) {
+  const float ax = __builtin_fabsf(x);
+  const bool big = ax >= 1.0f;
+  return __builtin_copysignf(tanhf_magnitude(big ? ax : -ax, big, steps), x);
 }
 
-SHDW_LIBM_FN float exact_tanhf(float x) {
+SHDW_LIBM_FN float exact_tanhf(float x, const TanhStep* steps) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  if (__builtin_amdgcn_ballot_w64(!tanhf_short_ok(x)) == 0) return tanhf_short(x);
+  if (__builtin_amdgcn_ballot_w64(!tanhf_short_ok(x)) == 0) return tanhf_short(x, steps);
 #endif
-  return tanhf_any(x);
+  return tanhf_any(x, steps);
 }
 
 // 1 / (1 + exp(-x)) in fp32, the way shadow/operators/kernels/activate.cpp:16
@@ -347,6 +397,7 @@ SHDW_LIBM_FN float exact_sigmoidf(float x, const uint64_t* tab) {
 #if !defined(__HIPCC__)
 SHDW_LIBM_FN float exact_expf(float x) { return exact_expf(x, kExp2fTab); }
 SHDW_LIBM_FN float exact_sigmoidf(float x) { return exact_sigmoidf(x, kExp2fTab); }
+SHDW_LIBM_FN float exact_tanhf(float x) { return exact_tanhf(x, kTanhStepTab); }
 #endif
 
 

@@ -78,6 +78,15 @@ float libm_host_eval(int func, float x) {
   return p.ref ? p.ref(x) : NAN;
 }
 
+// Entry `index` of the tanh step table as eight floats; returns the bytes of an
+// entry, or the number of entries for a negative index.
+int libm_tanh_step(int index, float* out) {
+  using namespace shdw::libm;
+  if (index < 0 || index >= kTanhSteps) return kTanhSteps;
+  std::memcpy(out, &kTanhStepTab[index], sizeof(TanhStep));
+  return static_cast<int>(sizeof(TanhStep));
+}
+
 // Compare on patterns start, start+stride, ... (count of them), split over
 // `threads` threads.  Returns the number of mismatches and stores up to
 // max_report offending input patterns.

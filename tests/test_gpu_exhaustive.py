@@ -90,7 +90,7 @@ def test_all_float_inputs(gpu, name):
 
 
 WAVE_ELEMENTS = 256  # 64 lanes, one 128-bit vector each: what one wave of the elementwise kernels covers
-SHORT_FORM_LIMIT = {"tanh": 0x41200000, "sigmoid": 0x42AE0000}  # bit patterns of 10.0f and 87.0f
+SHORT_FORM_LIMIT = {"tanh": 0x411C0000, "sigmoid": 0x42AE0000}  # bit patterns of 9.75f and 87.0f
 
 
 @pytest.mark.parametrize("name", sorted(SHORT_FORM_LIMIT))

@@ -19,7 +19,7 @@ EDGES = [0x00000000, 0x00800000, 0x04000000, 0x24000000, 0x24800000, 0x31000000,
          0x32000000, 0x32800000, 0x33000000, 0x39000000, 0x39800000, 0x3eb17218, 0x3ed413d7,
          0x3e95f61f, 0x3ee00000, 0x3f000000, 0x3f2ca140, 0x3f300000, 0x3f330000, 0x3f490fda,
          0x3f580000, 0x3f79999a, 0x3f800000, 0x3F851592, 0x3f980000, 0x3fa00000, 0x3fc90fda,
-         0x401c0000, 0x4036db6e, 0x40490fda, 0x40c00000, 0x4195b844, 0x41b00000, 0x42b00000,
+         0x401c0000, 0x4036db6e, 0x40490fda, 0x40c00000, 0x411c0000, 0x41200000, 0x4195b844, 0x41b00000, 0x42b00000,
          0x42b17218, 0x42cff1b5, 0x42ce8ed0, 0x42f00000, 0x4c000000, 0x5a000000, 0x7f800000]
 
 
@@ -50,6 +50,28 @@ def test_restatement_matches_host_libm(sweep, name):
         for sign in (0, 0x80000000):
             lo = max(0, (edge | sign) - 4096)
             run(lo, 8192, 1)
+
+
+def test_tanh_step_table_holds_its_definitions(sweep):
+    """kTanhStepTab[k + 3] = {k ln2_hi (exact), fl(k ln2_lo), T, off, 2^k, k >= 1} for k = -3 ... 28, with
+    T = 0 (k = 0, -1), 1 (k <= -2), fl(1 - 2^-k) otherwise and off = -0.5 (k = -1), -1 (k <= -2), 0 otherwise --
+    recomputed here in numpy fp32."""
+    sweep.libm_tanh_step.restype = ctypes.c_int
+    sweep.libm_tanh_step.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
+    f = np.float32
+    ln2_hi, ln2_lo = f(6.9313812256e-01), f(9.0580006145e-06)
+    entry = (ctypes.c_float * 8)()
+    n = sweep.libm_tanh_step(-1, entry)
+    assert n == 32
+    for i in range(n):
+        k = i - 3
+        assert sweep.libm_tanh_step(i, entry) == 32  # bytes per entry
+        assert float(f(k) * ln2_hi) == k * float(ln2_hi)  # the product is exact
+        T = f(0) if k in (0, -1) else (f(1) if k <= -2 else f(1) - f(2.0 ** -k))
+        off = f(-0.5) if k == -1 else (f(-1) if k <= -2 else f(0))
+        want = [f(k) * ln2_hi, f(k) * ln2_lo, T, off, f(2.0 ** k), f(1 if k >= 1 else 0), f(0), f(0)]
+        got = np.array(list(entry), np.float32)
+        assert np.array_equal(got.view(np.uint32), np.array(want, np.float32).view(np.uint32)), (k, got, want)
 
 
 def test_powf_restatement_matches_host_libm(sweep):
