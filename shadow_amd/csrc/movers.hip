@@ -893,6 +893,150 @@ static bool launch_resize_band(int planes, int in_h, int in_w, int out_h, int ou
   return true;
 }
 
+// ---------------------------------------------------------------------------
+// Resize by exactly two along both axes (decoder and pyramid upsampling), rows
+// of an even number (>= 4) of positions: no staging.  fh = fw = 0.5 exactly, so
+// every output vector of four columns 4o ... 4o+3 reads the input columns
+// 2o-1 ... 2o+2 (bilinear) or 2o, 2o+1 (nearest) of one or two rows: one or two
+// 128-bit loads per lane on whatever dword address, neighbours overlapping in the
+// caches, and one 128-bit store per output row.  Source indices and weights
+// still come from resize_axis / bilinear_axis and the sums are formed in the
+// same order as everywhere else, so the results are the same bits.
+// ---------------------------------------------------------------------------
+struct ResizeDoubleArgs {
+  int in_h, in_w;
+  uint32_t out_w;
+  FastDiv f_vecs;   // output vectors per row: out_w / 4 = in_w / 2
+  FastDiv f_pairs;  // bilinear: row pairs per plane, in_h + 1
+};
+
+// Nearest: lane t owns the input pair x[2t], x[2t + 1] (the input is one flat
+// array of such pairs) and writes it, doubled, to two output rows: 43 us for
+// [64,64,56,56] where the staged kernel takes 48.  Two pairs per lane (a
+// 128-bit load, two stores side by side per row) took 93 us: a store instruction
+// then covers every other 16 bytes.  Workgroups of 256 lanes and plain instead of
+// streaming stores: 44 to 46 us.
+__global__ __launch_bounds__(kStream) void resize_double_nearest_kernel(const float* x, float* y, uint32_t tasks,
+                                                                        ResizeDoubleArgs p) {
+  const uint32_t t = blockIdx.x * kStream + threadIdx.x;
+  if (t >= tasks) return;
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  const v2f v = __builtin_nontemporal_load(reinterpret_cast<const v2f*>(x) + t);
+  uint32_t row, o;  // row counts input rows over all planes; o the lane's place in the row
+  fd_divmod(t, p.f_vecs, row, o);
+  float* dst = y + 2 * row * p.out_w + 4 * o;
+  const v4f r = {v[0], v[0], v[1], v[1]};
+  store4_stream(dst, r);
+  store4_stream(dst + p.out_w, r);
+}
+
+// Bilinear: output rows 2q - 1 and 2q (q = 0 ... in_h; the first pair has only
+// its second row, the last only its first) have the same two source rows.
+// With f = 0.5 the axis rule (bilinear_axis) gives, for output index i:
+//   i = 0: neighbours 0, 1, weight 0 (the coordinate -0.25 is clamped to 0);
+//   i = 2m - 1: neighbours m-1, m, weight 0.25;   i = 2m: m-1, m, weight 0.75;
+// an upper neighbour beyond the extent is the lower one again.  All of these
+// weights and their products are exact, so forming them here from constants
+// gives the bits of the general kernels, which take them from bilinear_axis; the
+// host checks the rule against bilinear_axis before it launches this kernel.
+__global__ __launch_bounds__(kBlock) void resize_double_bilinear_kernel(const float* x, float* y, uint32_t tasks,
+                                                                        ResizeDoubleArgs p) {
+  const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+  if (t >= tasks) return;
+  uint32_t rest, o, plane, q;
+  fd_divmod(t, p.f_vecs, rest, o);
+  fd_divmod(rest, p.f_pairs, plane, q);
+  const uint32_t in_h = static_cast<uint32_t>(p.in_h), in_w = static_cast<uint32_t>(p.in_w);
+  const bool top = q == 0, has_b = q < in_h;
+  const uint32_t h_l = top ? 0u : q - 1;
+  const uint32_t h_h = min(top ? 1u : q, in_h - 1);
+  const float sh_b = top ? 0.f : 0.75f, ih_b = top ? 1.f : 0.25f;  // row 2q; row 2q - 1: 0.25, 0.75
+
+  // columns 2o-1 ... 2o+2, of which the first lane of a row lacks the first and
+  // the last lane the last: the window moves inside the row and e[] repeats the
+  // edge column, which is what the clamped neighbours read there
+  const int want = 2 * static_cast<int>(o) - 1;
+  const int base = min(max(want, 0), p.in_w - 4);
+  const bool first = want < 0, last = want > base;
+  const uint32_t plane_at = plane * in_h * in_w + static_cast<uint32_t>(base);
+  const v4f wl = load4_any(x + (plane_at + h_l * in_w)), wh = load4_any(x + (plane_at + h_h * in_w));
+  float el[4], eh[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int down = k > 0 ? k - 1 : 0, up = k < 3 ? k + 1 : 3;
+    el[k] = first ? wl[down] : (last ? wl[up] : wl[k]);
+    eh[k] = first ? wh[down] : (last ? wh[up] : wh[k]);
+  }
+  v4f res_a, res_b;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    // neighbours e[kl], e[kl + 1] with kl = 0, 1, 1, 2; column 0 of the row has
+    // e[1], e[2] (columns 0 and 1) and weight 0
+    const int kl = j == 0 ? 0 : (j == 3 ? 2 : 1);
+    const bool col0 = j == 0 && first;
+    const float v0 = col0 ? el[1] : el[kl], v1 = col0 ? eh[1] : eh[kl];
+    const float v2 = col0 ? el[2] : el[kl + 1], v3 = col0 ? eh[2] : eh[kl + 1];
+    const float sw = (j & 1) ? 0.25f : (col0 ? 0.f : 0.75f);
+    const float iw = (j & 1) ? 0.75f : (col0 ? 1.f : 0.25f);
+    {
+      const float ih = 0.75f, sh = 0.25f;
+      const float a0 = ih * iw, a1 = sh * iw, a2 = ih * sw, a3 = sh * sw;
+      const float t0 = a0 * v0, t1 = a1 * v1, t2 = a2 * v2, t3 = a3 * v3;
+      const float s01 = t0 + t1;
+      const float s012 = s01 + t2;
+      res_a[j] = s012 + t3;
+    }
+    {
+      const float a0 = ih_b * iw, a1 = sh_b * iw, a2 = ih_b * sw, a3 = sh_b * sw;
+      const float t0 = a0 * v0, t1 = a1 * v1, t2 = a2 * v2, t3 = a3 * v3;
+      const float s01 = t0 + t1;
+      const float s012 = s01 + t2;
+      res_b[j] = s012 + t3;
+    }
+  }
+  float* dst = y + ((plane * (2 * in_h) + 2 * q) * p.out_w + 4 * o);  // row 2q
+  if (!top) store4_stream(dst - p.out_w, res_a);
+  if (has_b) store4_stream(dst, res_b);
+}
+
+// The rule the bilinear kernel above is written from, against bilinear_axis.
+static bool double_rule_holds(int extent) {
+  for (int i = 0; i < std::min(2 * extent, 64); ++i) {
+    int lo, hi;
+    float frac;
+    bilinear_axis<false>(static_cast<uint32_t>(i), 0.5f, extent, lo, hi, frac);
+    const int m = (i + 1) / 2;
+    const int want_lo = i == 0 ? 0 : m - 1, want_hi = std::min(i == 0 ? 1 : m, extent - 1);
+    const float want_frac = i == 0 ? 0.f : ((i & 1) ? 0.25f : 0.75f);
+    if (lo != want_lo || hi != want_hi || frac != want_frac) return false;
+  }
+  return true;
+}
+
+// True when the kernels above apply (and then they have been launched).
+static bool launch_resize_double(int type, int planes, int in_h, int in_w, int out_h, int out_w, const float* x,
+                                 float* y, hipStream_t st) {
+  if (out_h != 2 * in_h || out_w != 2 * in_w || in_w % 2 != 0 || in_w < 4 || !aligned16(y)) return false;
+  ResizeDoubleArgs p;
+  p.in_h = in_h, p.in_w = in_w, p.out_w = static_cast<uint32_t>(out_w);
+  // the factors as shdw_hip_resize forms them: exactly one half
+  if (static_cast<float>(in_h) / out_h != 0.5f || static_cast<float>(in_w) / out_w != 0.5f) return false;
+  p.f_vecs = make_fastdiv(in_w / 2), p.f_pairs = make_fastdiv(in_h + 1);
+  if (type == 0) {
+    const uintptr_t at = reinterpret_cast<uintptr_t>(x);
+    const uint32_t pairs = static_cast<uint32_t>(planes) * in_h * (in_w / 2);
+    if ((at & 7u) != 0) return false;
+    resize_double_nearest_kernel<<<stream_grid(pairs), kStream, 0, st>>>(x, y, pairs, p);
+    return true;
+  }
+  const int64_t tasks = static_cast<int64_t>(planes) * (in_h + 1) * (in_w / 2);
+  if (tasks > INT32_MAX || !double_rule_holds(in_h) || !double_rule_holds(in_w)) return false;
+  // 256 lanes per workgroup: 47 to 48 us for [64,64,56,56] against 50 for single waves (staged kernel: 56)
+  resize_double_bilinear_kernel<<<grid_for(static_cast<uint32_t>(tasks)), kBlock, 0, st>>>(
+      x, y, static_cast<uint32_t>(tasks), p);
+  return true;
+}
+
 static bool count_fits(const int* shape, int n, int64_t* count) {
   int64_t c = 1;
   for (int k = 0; k < n; ++k) {
@@ -1176,6 +1320,7 @@ int shdw_hip_resize(const int* in_shape, const int* out_shape, int type, int ali
   } else {
     p.fh = static_cast<float>(in_h) / out_h;
     p.fw = static_cast<float>(in_w) / out_w;
+    if (launch_resize_double(type, planes, in_h, in_w, out_h, out_w, x, y, st)) return launch_status();
     if (type == 0) {
       // Maps of a few hundred positions keep the gathers: their tensors are small
       // enough to come from cache (x2 of [64,256,13,13]: 12 us, staged 17 us).

@@ -189,6 +189,23 @@ def test_resize_nearest_any_width(ws, shape, size):
     assert_bit_exact(got, want, "nearest %s -> %s" % (shape, size))
 
 
+@pytest.mark.parametrize("typ", [0, 1])
+@pytest.mark.parametrize("shape", [(1, 1, 1, 4), (2, 3, 1, 6), (1, 2, 2, 4), (3, 1, 3, 8), (2, 2, 57, 6), (1, 3, 5, 130),
+                                   (3, 5, 56, 56), (2, 2, 38, 38), (1, 1, 9, 4096)])
+def test_resize_by_two_of_even_rows(ws, typ, shape):
+    """Exactly x2 on rows of an even number (>= 4) of positions: the kernels without staging.  Infinities and NaNs
+    are planted (a weight of zero times an infinity is a NaN, as in the reference's sum), also in the edge
+    columns and rows."""
+    x = with_specials(normal(93, shape, 2.0), 93).reshape(shape)
+    x[..., 0, 1] = np.inf
+    x[..., -1, -1] = -np.inf
+    x[0, 0, 0, 0] = np.nan
+    got = run(ws, "Resize", [("x", x)], {"scale": [2.0], "type": typ})
+    want = oracle.resize_op(x, [0], [2.0], typ, False)
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "x2 type %d %s" % (typ, shape))
+
+
 @pytest.mark.parametrize("shape,group", [((2, 6, 3, 5), 2), ((2, 6, 3, 5), 3), ((1, 12, 4, 4), 4), ((3, 8, 1, 1), 8),
                                          ((2, 116, 28, 28), 2), ((2, 6, 3, 5), 1), ((2, 116, 7, 7), 2), ((3, 4, 1, 3), 2),
                                          # rows of 7, 1, 2, 5 and 49 floats: a lane's four outputs from up to four rows
