@@ -1012,7 +1012,7 @@ def config_table(dev, sets_scale=1, cpu=None):
     swb = dev.buf(nbytes=max(8, lib.shdw_hip_ssd_normalize_workspace_bytes(64, 512, 1444, 1)))
     ms = time_median(dev, lambda k: lib.shdw_hip_ssd_normalize(64, 512, 1444, 1, 1e-5, AH[k].ptr, ssc.ptr, 0,
                                                                YH[k].ptr, swb.ptr, st), SH, reps=20)
-    add("next", "ssd_normalize per item, channel scale [64,512,38,38] (2 launches)", 4 * NS + 4 * 512, 4 * NS, ms, NS)
+    add("next", "ssd_normalize per item, channel scale [64,512,38,38] (3 launches)", 4 * NS + 4 * 512, 4 * NS, ms, NS)
     # data movers ("movers") on the same 205 MB tensors
     def concat2(k):
         # two [64,128,56,56] halves -> [64,256,56,56] along axis 1

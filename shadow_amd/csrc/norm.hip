@@ -561,7 +561,7 @@ static uint32_t norm_row_splits(int64_t rows, int64_t inner) {
 constexpr uint32_t kSsdSegmentQuantum = 4 * kBlock;  // keeps every segment 16-byte aligned
 constexpr uint32_t kSsdMinSegment = 4 * kSsdSegmentQuantum;
 constexpr uint32_t kSsdMaxParts = 64;
-constexpr uint32_t kSsdGroupsWanted = 2048;
+constexpr uint32_t kSsdGroupsWanted = 1024;
 
 struct SsdRowPlan {
   uint32_t parts, segment;
@@ -591,8 +591,25 @@ __global__ __launch_bounds__(kBlock) void ssd_row_partials_kernel(const float* x
   const float* xr = x + static_cast<uint64_t>(item) * num;
   double acc = 0;
   if (VEC) {
-    for (uint32_t t = begin / 4 + threadIdx.x; t < end / 4; t += kBlock) {
-      const v4f q = load4(xr + 4ull * t);
+    // eight loads under way per lane; the squares are added in the order of t
+    constexpr int kAhead = 8;
+    uint32_t t = begin / 4 + threadIdx.x;
+    const uint32_t stop = end / 4;
+    for (; t + (kAhead - 1) * kBlock < stop; t += kAhead * kBlock) {
+      v4f q[kAhead];
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) q[u] = load4_stream(xr + 4ull * (t + u * kBlock));
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float sq = q[u][j] * q[u][j];
+          acc += static_cast<double>(sq);
+        }
+      }
+    }
+    for (; t < stop; t += kBlock) {
+      const v4f q = load4_stream(xr + 4ull * t);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float sq = q[j] * q[j];
@@ -609,37 +626,68 @@ __global__ __launch_bounds__(kBlock) void ssd_row_partials_kernel(const float* x
   if (threadIdx.x == 0) partials[blockIdx.x] = total;
 }
 
-// SM: 0 no scale, 1 one shared factor (Sscal), 2 one factor per channel.
-template <bool VEC, int SM>
-__global__ __launch_bounds__(kBlock) void ssd_row_scale_kernel(const float* x, float* y,
-                                                                const double* partials, uint32_t parts,
-                                                                uint32_t num, float eps,
-                                                                const float* scale, FastDiv f_spatial,
-                                                                FastDiv f_groups) {
-  uint32_t item, group;  // workgroup `group` of the item's grid_for(steps) workgroups
-  fd_divmod(blockIdx.x, f_groups, item, group);
-  const double* mine = partials + item * parts;  // uniform: scalar loads
+// One lane per item: adds the item's partial sums in index order and leaves
+// 1 / sqrt((float)sum + eps) in the item's first slot (a float, widened exactly).
+// In the scaling kernel itself this chain of dependent loads and additions ran
+// once per wave and set its pace: 75 us for [64,512,38,38] where the same pass
+// with the factor ready takes 57.
+__global__ __launch_bounds__(kBlock) void ssd_row_finish_kernel(double* partials, uint32_t parts, uint32_t batch,
+                                                                float eps) {
+  const uint32_t item = blockIdx.x * kBlock + threadIdx.x;
+  if (item >= batch) return;
+  double* mine = partials + item * parts;
   double sum = 0;
   for (uint32_t k = 0; k < parts; ++k) sum += mine[k];
   const float sum_f = static_cast<float>(sum);
   const float se = sum_f + eps;
   const float factor = 1.f / __builtin_sqrtf(se);
-  const uint32_t i = group * kBlock + threadIdx.x;
+  mine[0] = static_cast<double>(factor);
+}
+
+// SM: 0 no scale, 1 one shared factor (Sscal), 2 one factor per channel.
+template <bool VEC, int SM>
+__global__ __launch_bounds__(kStream) void ssd_row_scale_kernel(const float* x, float* y,
+                                                                const double* partials, uint32_t parts,
+                                                                uint32_t num, const float* scale,
+                                                                FastDiv f_spatial,
+                                                                FastDiv f_groups) {
+  uint32_t item, group;  // wave `group` of the item's stream_grid(steps) waves
+  fd_divmod(blockIdx.x, f_groups, item, group);
+  const uint32_t i = group * kStream + threadIdx.x;
   const uint64_t base = static_cast<uint64_t>(item) * num;
+  const bool mine_valid = i < (VEC ? num / 4 : num);
+  v4f q = {0.f, 0.f, 0.f, 0.f};
+  if (mine_valid) {
+    if (VEC) q = load4_stream(x + base + 4ull * i);
+    else q[0] = x[base + i];
+  }
+  const float factor = static_cast<float>(partials[item * parts]);  // uniform: one scalar load
+  if (!mine_valid) return;
   if (VEC) {
-    if (i >= num / 4) return;
-    const v4f q = load4_stream(x + base + 4ull * i);
     v4f r;
+    if (SM == 2 && f_spatial.d >= 4) {
+      // four neighbours lie in one channel or in two: one division and two factors
+      // per lane (a gather per element keeps the address unit busier than the
+      // streamed load and store together)
+      const uint32_t c0 = fd_div(4 * i, f_spatial);
+      const uint32_t edge = (c0 + 1) * f_spatial.d;  // first element of the next channel
+      const float s0 = scale[c0], s1 = scale[edge < num ? c0 + 1 : c0];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      r[j] = q[j] * factor;
-      if (SM == 1) r[j] = r[j] * scale[0];
-      if (SM == 2) r[j] = r[j] * scale[fd_div(4 * i + j, f_spatial)];
+      for (int j = 0; j < 4; ++j) {
+        r[j] = q[j] * factor;
+        r[j] = r[j] * (4 * i + j < edge ? s0 : s1);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        r[j] = q[j] * factor;
+        if (SM == 1) r[j] = r[j] * scale[0];
+        if (SM == 2) r[j] = r[j] * scale[fd_div(4 * i + j, f_spatial)];
+      }
     }
     store4_stream(y + base + 4ull * i, r);
   } else {
-    if (i >= num) return;
-    float r = x[base + i] * factor;
+    float r = q[0] * factor;
     if (SM == 1) r = r * scale[0];
     if (SM == 2) r = r * scale[fd_div(i, f_spatial)];
     y[base + i] = r;
@@ -653,15 +701,16 @@ static void launch_ssd_rows(uint32_t batch, uint32_t num, uint32_t spatial, floa
   const SsdRowPlan plan = plan_ssd_rows(batch, num);
   ssd_row_partials_kernel<VEC><<<batch * plan.parts, kBlock, 0, st>>>(x, partials, num, plan.segment,
                                                                     make_fastdiv(plan.parts));
-  const uint32_t groups = grid_for(VEC ? num / 4 : num);  // batch * groups <= count / 256 + batch
+  ssd_row_finish_kernel<<<grid_for(batch), kBlock, 0, st>>>(partials, plan.parts, batch, eps);
+  const uint32_t groups = stream_grid(VEC ? num / 4 : num);  // single waves: batch * groups <= count / 64 + batch
   const uint32_t grid = batch * groups;
   const FastDiv fs = make_fastdiv(std::max(spatial, 1u)), fg = make_fastdiv(groups);
   if (!scale)
-    ssd_row_scale_kernel<VEC, 0><<<grid, kBlock, 0, st>>>(x, y, partials, plan.parts, num, eps, scale, fs, fg);
+    ssd_row_scale_kernel<VEC, 0><<<grid, kStream, 0, st>>>(x, y, partials, plan.parts, num, scale, fs, fg);
   else if (channel_shared)
-    ssd_row_scale_kernel<VEC, 1><<<grid, kBlock, 0, st>>>(x, y, partials, plan.parts, num, eps, scale, fs, fg);
+    ssd_row_scale_kernel<VEC, 1><<<grid, kStream, 0, st>>>(x, y, partials, plan.parts, num, scale, fs, fg);
   else
-    ssd_row_scale_kernel<VEC, 2><<<grid, kBlock, 0, st>>>(x, y, partials, plan.parts, num, eps, scale, fs, fg);
+    ssd_row_scale_kernel<VEC, 2><<<grid, kStream, 0, st>>>(x, y, partials, plan.parts, num, scale, fs, fg);
 }
 
 // softmax.hip: the per-position form shares the Normalize column kernels.
