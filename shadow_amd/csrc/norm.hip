@@ -560,7 +560,8 @@ static uint32_t norm_row_splits(int64_t rows, int64_t inner) {
 // ---------------------------------------------------------------------------
 constexpr uint32_t kSsdSegmentQuantum = 4 * kBlock;  // keeps every segment 16-byte aligned
 constexpr uint32_t kSsdMinSegment = 4 * kSsdSegmentQuantum;
-constexpr uint32_t kSsdMaxParts = 64;
+constexpr uint32_t kSsdMaxParts = 64;  // one lane of a wave per part (ssd_row_finish_kernel)
+static_assert(kSsdMaxParts <= static_cast<uint32_t>(kWave), "one lane per part");
 constexpr uint32_t kSsdGroupsWanted = 1024;
 
 struct SsdRowPlan {
@@ -626,22 +627,25 @@ __global__ __launch_bounds__(kBlock) void ssd_row_partials_kernel(const float* x
   if (threadIdx.x == 0) partials[blockIdx.x] = total;
 }
 
-// One lane per item: adds the item's partial sums in index order and leaves
-// 1 / sqrt((float)sum + eps) in the item's first slot (a float, widened exactly).
-// In the scaling kernel itself this chain of dependent loads and additions ran
-// once per wave and set its pace: 75 us for [64,512,38,38] where the same pass
+// One wave per item: lane k fetches partial k (at most 64 of them, one round
+// trip for all), the sum walks the lanes in index order, and
+// 1 / sqrt((float)sum + eps) goes to the item's first slot (a float, widened
+// exactly).  In the scaling kernel itself this chain ran once per wave behind
+// dependent loads and set its pace: 75 us for [64,512,38,38] where the same pass
 // with the factor ready takes 57.
-__global__ __launch_bounds__(kBlock) void ssd_row_finish_kernel(double* partials, uint32_t parts, uint32_t batch,
-                                                                float eps) {
-  const uint32_t item = blockIdx.x * kBlock + threadIdx.x;
-  if (item >= batch) return;
-  double* mine = partials + item * parts;
+__global__ __launch_bounds__(kWave) void ssd_row_finish_kernel(double* partials, uint32_t parts, float eps) {
+  double* mine = partials + blockIdx.x * parts;
+  const double part = threadIdx.x < parts ? mine[threadIdx.x] : 0.0;
   double sum = 0;
-  for (uint32_t k = 0; k < parts; ++k) sum += mine[k];
+  for (uint32_t k = 0; k < parts; ++k) {  // k is uniform: two v_readlane_b32 per step
+    const int lo = __builtin_amdgcn_readlane(__double2loint(part), static_cast<int>(k));
+    const int hi = __builtin_amdgcn_readlane(__double2hiint(part), static_cast<int>(k));
+    sum += __hiloint2double(hi, lo);
+  }
   const float sum_f = static_cast<float>(sum);
   const float se = sum_f + eps;
   const float factor = 1.f / __builtin_sqrtf(se);
-  mine[0] = static_cast<double>(factor);
+  if (threadIdx.x == 0) mine[0] = static_cast<double>(factor);
 }
 
 // SM: 0 no scale, 1 one shared factor (Sscal), 2 one factor per channel.
@@ -701,7 +705,7 @@ static void launch_ssd_rows(uint32_t batch, uint32_t num, uint32_t spatial, floa
   const SsdRowPlan plan = plan_ssd_rows(batch, num);
   ssd_row_partials_kernel<VEC><<<batch * plan.parts, kBlock, 0, st>>>(x, partials, num, plan.segment,
                                                                     make_fastdiv(plan.parts));
-  ssd_row_finish_kernel<<<grid_for(batch), kBlock, 0, st>>>(partials, plan.parts, batch, eps);
+  ssd_row_finish_kernel<<<batch, kWave, 0, st>>>(partials, plan.parts, eps);
   const uint32_t groups = stream_grid(VEC ? num / 4 : num);  // single waves: batch * groups <= count / 64 + batch
   const uint32_t grid = batch * groups;
   const FastDiv fs = make_fastdiv(std::max(spatial, 1u)), fg = make_fastdiv(groups);
