@@ -465,6 +465,93 @@ static bool plan_pool_band(const PoolArgs& p, int target_outputs, BandArgs* a) {
   return true;
 }
 
+// Windows of 3x3 (pad 0 or 1) or 2x2 (no pad) at stride 2 over rows of a multiple
+// of four columns, out_w = in_w / 2 (the stem pooling of a classifier in either
+// rounding of the output size; VGG-style halving): no staging.  A lane owns two
+// neighbouring outputs of one row: their windows lie in the columns 4v ... 4v+3
+// of two or three input rows, one 128-bit load per row (a wave's loads are whole
+// rows of consecutive vectors), plus, for three columns, the one column before
+// (pad 1) or after (pad 0) them, which the neighbouring lane loads as part of
+// its own vector and this one fetches as a single float.  Cells outside the input
+// take the fold's neutral value, as the padding of the band tile does, and every
+// window is folded row by row, left to right.  (Four outputs per lane from two
+// vectors per row, so that a load instruction covers every other 16 bytes, ran
+// at 59 us on [64,64,112,112] where the band kernel takes 49 and this one 43;
+// workgroups of 64 or 1024 lanes 47 to 48 us, XCD-contiguous numbering no change.)
+struct HalveArgs {
+  int in_h, in_w, out_h, out_w, pad;
+  FastDiv f_pairs;  // out_w / 2 = in_w / 4
+  FastDiv f_out_h;
+};
+
+constexpr int kHalveLanes = kBlock;
+
+template <bool MAX, int K>
+__global__ __launch_bounds__(kHalveLanes) void pool_halve_kernel(const float* x, float* y, uint32_t tasks,
+                                                             HalveArgs p) {
+  const uint32_t t = blockIdx.x * kHalveLanes + threadIdx.x;
+  if (t >= tasks) return;
+  uint32_t rest, v, plane, r;
+  fd_divmod(t, p.f_pairs, rest, v);
+  fd_divmod(rest, p.f_out_h, plane, r);
+  constexpr int kCells = K == 3 ? 5 : 4;  // columns under the two windows
+  const float neutral = MAX ? -FLT_MAX : 0.f;
+  const int h_first = 2 * static_cast<int>(r) - p.pad;
+  const float* img = x + plane * static_cast<uint32_t>(p.in_h * p.in_w) + 4 * v;
+  const int halo_col = p.pad ? -1 : 4;  // relative to column 4v
+  const int halo_abs = 4 * static_cast<int>(v) + halo_col;
+  const bool halo_valid = K == 3 && halo_abs >= 0 && halo_abs < p.in_w;
+  float c[K][kCells];
+#pragma unroll
+  for (int i = 0; i < K; ++i) {
+    const int ri = h_first + i;
+    const bool row_valid = ri >= 0 && ri < p.in_h;
+    const float* row = img + min(max(ri, 0), p.in_h - 1) * p.in_w;
+    const v4f q = load4(row);
+    float cells[kCells];
+    const int at = (K == 3 && p.pad) ? 1 : 0;  // where column 4v sits among the cells
+#pragma unroll
+    for (int e = 0; e < 4; ++e) cells[at + e] = q[e];
+    if (K == 3) {
+      const float h = row[halo_valid ? halo_col : 0];
+      cells[p.pad ? 0 : 4] = halo_valid ? h : neutral;
+    }
+#pragma unroll
+    for (int e = 0; e < kCells; ++e) c[i][e] = row_valid ? cells[e] : neutral;
+  }
+  float res[2];
+  const int h_end_pad = min(h_first + K, p.in_h + p.pad);
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    float max_val = -FLT_MAX, sum_val = 0.f;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        if (MAX)
+          max_val = pool_max(max_val, c[i][2 * j + k]);
+        else
+          sum_val += c[i][2 * j + k];
+      }
+    }
+    const int w_first = 2 * (2 * static_cast<int>(v) + j) - p.pad;
+    const int w_end_pad = min(w_first + K, p.in_w + p.pad);
+    const int pool_size = (h_end_pad - h_first) * (w_end_pad - w_first);
+    res[j] = MAX ? max_val : sum_val / static_cast<float>(pool_size);
+  }
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  float* dst = y + ((plane * static_cast<uint32_t>(p.out_h) + r) * static_cast<uint32_t>(p.out_w) + 2 * v);
+  __builtin_nontemporal_store(v2f{res[0], res[1]}, reinterpret_cast<v2f*>(dst));
+}
+
+// True when the kernel above applies to p (2-D).
+static bool pool_halve_applies(const PoolArgs& p, const float* x, const float* y, bool planning) {
+  if (p.kh != p.kw || p.sh != 2 || p.sw != 2 || p.ph != p.pw) return false;
+  if (!((p.kh == 3 && p.pw <= 1) || (p.kh == 2 && p.pw == 0))) return false;
+  if (p.in_w % 4 != 0 || p.out_w * 2 != p.in_w || p.in_h < 1) return false;
+  return planning || (aligned16(x) && aligned16(y));
+}
+
 // Planes too small to keep a workgroup busy (14x14 and 7x7 maps with 3x3 / 2x2 /
 // 5x5 .. 13x13 windows): with a workgroup per band of one plane, a 7x7 plane
 // gives 49 outputs to 256 lanes (3x3 stride 1 on [128,2048,7,7]: 179 us per
@@ -1165,6 +1252,23 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
   } while (0)
     if (pool_type == 0) SHDW_SMALL(true); else SHDW_SMALL(false);
 #undef SHDW_SMALL
+    return launch_status();
+  }
+  if (!three_d && pool_halve_applies(p, x, y, pl->want)) {
+    const uint32_t tasks = n_out / 2;
+    const uint32_t grid = (tasks + kHalveLanes - 1) / kHalveLanes;
+    if (pl->chosen(SHDW_PATH_POOL_HALVE, p.kh, grid)) return SHDW_OK;
+    HalveArgs h;
+    h.in_h = p.in_h, h.in_w = p.in_w, h.out_h = p.out_h, h.out_w = p.out_w, h.pad = p.pw;
+    h.f_pairs = make_fastdiv(static_cast<uint32_t>(p.out_w / 2));
+    h.f_out_h = make_fastdiv(static_cast<uint32_t>(p.out_h));
+    if (p.kh == 3) {
+      if (pool_type == 0) pool_halve_kernel<true, 3><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h);
+      else pool_halve_kernel<false, 3><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h);
+    } else {
+      if (pool_type == 0) pool_halve_kernel<true, 2><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h);
+      else pool_halve_kernel<false, 2><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h);
+    }
     return launch_status();
   }
   BandArgs a;

@@ -2,6 +2,8 @@
 points and the operators through Operator::Run(), bit for bit against the oracle
 (these kernels fold every column / window in the reference's order, so there is
 no tolerance anywhere in this file)."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -416,6 +418,34 @@ def test_pooling2d_op(ws, pool, shape, kernel, stride, pad, full):
     want = oracle.pooling_op(x, pool, kernel, stride, pad, full_pooling=full)
     assert got.shape == want.shape
     assert_bit_exact(got, want, "pooling2d")
+
+
+@pytest.mark.parametrize("pool", [0, 1])
+@pytest.mark.parametrize("full", [False, True])
+@pytest.mark.parametrize("shape,kernel,pad", [
+    ((2, 3, 112, 112), 3, 0), ((2, 3, 112, 112), 3, 1), ((1, 2, 56, 64), 2, 0), ((3, 2, 33, 40), 3, 1),
+    ((1, 2, 41, 72), 3, 0), ((1, 1, 3, 8), 3, 1), ((2, 2, 1, 16), 3, 1), ((1, 3, 50, 48), 2, 0),
+    ((2, 1, 64, 256), 3, 1), ((1, 1, 30, 1024), 3, 0)])
+def test_pooling_by_two_without_staging(ws, gpu, pool, full, shape, kernel, pad):
+    """3x3 (pad 0 or 1) and 2x2 windows at stride 2 over rows of a multiple of eight columns: where the output
+    is half as wide as the input (with either rounding of the output size) the kernel without staging runs --
+    asked of the plan query -- and the results are those of the reference's walk, clipped windows, NaNs,
+    infinities and equal cells included."""
+    x = with_specials(normal(23, shape, 2.0), 23).reshape(shape)
+    x[..., 0, :] = np.where(np.arange(shape[3]) % 3 == 0, -np.inf, x[..., 0, :])
+    x[..., -1] = np.float32(-3.4028235e38)  # lowest(): equal to the fold's start value
+    args = {"pool": pool, "kernel_size": [kernel], "stride": [2], "pad": [pad], "full_pooling": full}
+    got = run(ws, "Pooling", [("x", x)], args)
+    want = oracle.pooling_op(x, pool, [kernel], [2], [pad], full_pooling=full)
+    assert got.shape == want.shape
+    assert_bit_exact(got, want, "pooling by two")
+    path, variant, grid = ctypes.c_int(), ctypes.c_int(), ctypes.c_uint()
+    assert shadow_amd.hip().shdw_hip_pooling2d_plan(shadow_amd.ints(list(shape)), pool, kernel, kernel, 2, 2, pad, pad,
+                                                    shadow_amd.ints(list(want.shape)), ctypes.byref(path),
+                                                    ctypes.byref(variant), ctypes.byref(grid)) == 0
+    halves = want.shape[3] * 2 == shape[3]
+    small = path.value == 23  # whole small planes in LDS keep their kernel
+    assert small or (path.value == 26) == halves, (path.value, want.shape)
 
 
 # The maximum keeps the earlier of equal cells and never takes a NaN: planes of signed

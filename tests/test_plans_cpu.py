@@ -16,7 +16,7 @@ import shadow_amd
 from shadow_amd import ints
 
 ROWS, ROWS_STREAM, SHORT_ROWS, QUADS, PACKED, LONG_SLAB, SLAB, COLUMNS_REG, TILE, TALL, COLUMNS = range(1, 12)
-PLANE_REDUCE, PLANE, PLANE_STREAM, SMALL_PLANES, BAND, WINDOW = range(20, 26)
+PLANE_REDUCE, PLANE, PLANE_STREAM, SMALL_PLANES, BAND, WINDOW, HALVE = range(20, 27)
 
 SOFTMAX = {  # (outer, dim, inner)
     (16, 49, 16384): (COLUMNS_REG, 64, 1024),      # softmax_channels_dense
@@ -67,8 +67,8 @@ NORMALIZE = {  # (outer, dim, inner, p)
 POOLING = {  # ((n, c, h, w), pool type, kernel, stride, pad)
     ((16, 64, 112, 112), 0, 3, 2, 0): (BAND, 203, 7168),       # the ResNet stem
     ((64, 64, 112, 112), 0, 3, 2, 0): (BAND, 203, 4096),
-    ((16, 64, 112, 112), 0, 3, 2, 1): (BAND, 203, 7168),
-    ((16, 64, 112, 112), 1, 2, 2, 0): (BAND, 202, 7168),
+    ((16, 64, 112, 112), 0, 3, 2, 1): (HALVE, 3, 6272),         # half as wide: no staging
+    ((16, 64, 112, 112), 1, 2, 2, 0): (HALVE, 2, 6272),
     ((128, 2048, 7, 7), 1, 7, 1, 0): (PLANE, 0, 0),            # global average
     ((128, 2048, 7, 7), 0, 7, 1, 0): (PLANE_REDUCE, 0, 0),
     ((64, 1024, 14, 14), 1, 14, 1, 0): (PLANE, 0, 0),
@@ -112,6 +112,15 @@ def test_pooling_plan(case):
     assert got == (0, POOLING[case])
 
 
+def test_pooling_plan_of_the_stem_with_the_output_size_rounded_up():
+    """3x3 at stride 2 without padding on 112 x 112 with Shadow's default rounding gives 56 x 56: the last window
+    of a row hangs over by one column, and the row is still half as wide as its input."""
+    lib = shadow_amd.hip()
+    for n, grid in ((16, 6272), (64, 25088)):
+        got = ask(lib.shdw_hip_pooling2d_plan, ints([n, 64, 112, 112]), 0, 3, 3, 2, 2, 0, 0, ints([n, 64, 56, 56]))
+        assert got == (0, (HALVE, 3, grid))
+
+
 def test_plans_of_empty_and_invalid_shapes():
     lib = shadow_amd.hip()
     assert ask(lib.shdw_hip_softmax_plan, 0, 5, 7) == (0, (0, 0, 0))
@@ -130,5 +139,5 @@ def test_path_values_match_the_header():
             "LONG_SLAB": LONG_SLAB, "SLAB": SLAB, "COLUMNS_REG": COLUMNS_REG, "TILE": TILE, "TALL": TALL,
             "COLUMNS": COLUMNS, "POOL_PLANE_REDUCE": PLANE_REDUCE, "POOL_PLANE": PLANE,
             "POOL_PLANE_STREAM": PLANE_STREAM, "POOL_SMALL_PLANES": SMALL_PLANES, "POOL_BAND": BAND,
-            "POOL_WINDOW": WINDOW, "NONE": 0}
+            "POOL_WINDOW": WINDOW, "POOL_HALVE": HALVE, "NONE": 0}
     assert found == mine
