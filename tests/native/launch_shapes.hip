@@ -23,10 +23,20 @@
 //             bytes as a flat copy give the yardstick: what the pattern costs
 //             before any arithmetic.
 //
+//   full sum: one value from 12.8 M floats, as two launches (slices, then a
+//             fold) and as one launch whose last workgroup to draw a ticket
+//             from a device-scope counter folds the slices: with one counter
+//             and with two levels of counters.  No workgroup waits for
+//             another; the partials and the tickets are relaxed device-scope
+//             atomics, ordered by a data dependency (the ticket's increment
+//             is computed from what the exchange that stores the partial
+//             returns).
+//
 // Usage: launch_shapes            (all tables)
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdio>
 #include <cstring>
 #include <vector>
@@ -179,6 +189,99 @@ __global__ __launch_bounds__(T) void tile_copy_kernel(const float* x, float* y, 
     else
       *reinterpret_cast<v4f_any*>(dst) = q;
   }
+}
+
+// ---- full sum ----
+template <int T>
+__device__ double block_sum(double v, double* lds) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();  // lds may still be read from an earlier call
+  if (lane == 0) lds[w] = v;
+  __syncthreads();
+  double t = 0;
+  for (int k = 0; k < T / 64; ++k) t += lds[k];
+  return t;
+}
+
+// Slice blockIdx.x of x (per = vectors per lane) summed in fp64.
+template <int T>
+__device__ double slice_sum(const float* x, uint32_t n4, uint32_t per, double* lds) {
+  double acc = 0;
+  const uint32_t first = blockIdx.x * (T * per) + threadIdx.x;
+  for (uint32_t u0 = 0; u0 < per; u0 += 4) {
+    v4f v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t i = first + (u0 + u) * T;
+      v[u] = (u0 + u < per && i < n4) ? load4_stream(x + 4ull * i) : v4f{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc += static_cast<double>(v[u][j]);
+  }
+  return block_sum<T>(acc, lds);
+}
+
+template <int T>
+__global__ __launch_bounds__(T) void sum_slices_kernel(const float* x, uint32_t n4, uint32_t per, double* part) {
+  __shared__ double lds[T / 64];
+  const double s = slice_sum<T>(x, n4, per, lds);
+  if (threadIdx.x == 0) part[blockIdx.x] = s;
+}
+
+__global__ __launch_bounds__(1024) void sum_fold_kernel(const double* part, uint32_t count, float* out) {
+  __shared__ double lds[16];
+  double acc = 0;
+  for (uint32_t i = threadIdx.x; i < count; i += 1024) acc += part[i];
+  const double s = block_sum<1024>(acc, lds);
+  if (threadIdx.x == 0) *out = static_cast<float>(s);
+}
+
+__device__ unsigned long long dbits(double d) { return __builtin_bit_cast(unsigned long long, d); }
+__device__ double bitsd(unsigned long long u) { return __builtin_bit_cast(double, u); }
+
+// One launch.  GROUP = 0: one counter; otherwise workgroups draw from the counter of their group of
+// GROUP and the last of a group from the top counter (counters 256 bytes apart).  The workgroup that
+// draws the last ticket folds all partials and puts the counters back to zero.
+template <int T, int GROUP>
+__global__ __launch_bounds__(T) void sum_ticket_kernel(const float* x, uint32_t n4, uint32_t per,
+                                                        unsigned long long* part, unsigned* counters, float* out) {
+  __shared__ double lds[T / 64];
+  __shared__ bool last;
+  const double s = slice_sum<T>(x, n4, per, lds);
+  if (threadIdx.x == 0) {
+    // the exchange has been performed when its result is here, and the ticket depends on that result
+    const unsigned long long old =
+        __hip_atomic_exchange(part + blockIdx.x, dbits(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned one = 1u + static_cast<unsigned>(old & 0);
+    bool mine;
+    if (GROUP == 0) {
+      mine = __hip_atomic_fetch_add(counters, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1;
+    } else {
+      const unsigned g = blockIdx.x / GROUP, groups = (gridDim.x + GROUP - 1) / GROUP;
+      const unsigned members = min(static_cast<unsigned>(GROUP), gridDim.x - g * GROUP);
+      const unsigned t = __hip_atomic_fetch_add(counters + 64 * (1 + g), one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      mine = false;
+      if (t == members - 1) {
+        const unsigned up = 1u + (t & 0);
+        mine = __hip_atomic_fetch_add(counters, up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1;
+      }
+    }
+    last = mine;
+  }
+  __syncthreads();
+  if (!last) return;
+  double acc = 0;
+  for (uint32_t i = threadIdx.x; i < gridDim.x; i += T)
+    acc += bitsd(__hip_atomic_load(part + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  const double total = block_sum<T>(acc, lds);
+  if (threadIdx.x == 0) *out = static_cast<float>(total);
+  const unsigned groups = GROUP ? (gridDim.x + GROUP - 1) / GROUP : 0;
+  for (unsigned c = threadIdx.x; c <= groups; c += T)
+    __hip_atomic_store(counters + 64 * c, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 static hipEvent_t e0, e1;
@@ -338,6 +441,57 @@ int main() {
     printf("add chain waves %d chains %d: %.2f %.2f\n", WAVES, CHAINS, us * 1e3f / n, us * 1e3f / n / (WAVES * CHAINS)); \
   }
     CHAIN(1, 1) CHAIN(1, 2) CHAIN(1, 4) CHAIN(2, 1) CHAIN(4, 1) CHAIN(8, 1) CHAIN(8, 2)
+  }
+  // full sum of [32,512,28,28]
+  {
+    const size_t n = 12845056;
+    const uint32_t n4 = static_cast<uint32_t>(n / 4);
+    const int sets = 6;
+    std::vector<float> h(n);
+    double exact = 0;
+    for (size_t i = 0; i < n; ++i) {
+      h[i] = static_cast<float>((i * 2654435761u) >> 8 & 0xffff) / 65536.f - 0.25f;
+      exact += h[i];
+    }
+    for (int k = 0; k < sets; ++k) CK(hipMemcpy(rp + k * n, h.data(), 4 * n, hipMemcpyHostToDevice));
+    double* part = reinterpret_cast<double*>(wp);
+    unsigned* counters = reinterpret_cast<unsigned*>(wp + (1 << 20));
+    float* out = wp + (2 << 20);
+    CK(hipMemset(counters, 0, 64 * 4 * 128));
+    printf("# full sum: one value from 12.8 M floats (51 MB), us per call; two launches = slices then a fold; ticket = one "
+           "launch, the last workgroup to draw from a device-scope counter folds\n");
+    const float want = static_cast<float>(exact);
+    float got, us;
+#define CHECK(label)                                                                                   \
+  CK(hipMemcpy(&got, out, 4, hipMemcpyDeviceToHost));                                                  \
+  printf("full sum %-44s %.2f %s\n", label, us, std::fabs(got - want) <= 1e-6f * std::fabs(want) ? "same" : "DIFFERENT");                   \
+  fflush(stdout);
+    if (time_us([&](int i) {
+          sum_slices_kernel<256><<<3136, 256>>>(rp + (i % sets) * n, n4, 4, part);
+          sum_fold_kernel<<<1, 1024>>>(part, 3136, out);
+        }, 40, &us)) return 1;
+    CHECK("two launches, 3136 x 256 lanes")
+    if (time_us([&](int i) {
+          sum_slices_kernel<1024><<<392, 1024>>>(rp + (i % sets) * n, n4, 8, part);
+          sum_fold_kernel<<<1, 1024>>>(part, 392, out);
+        }, 40, &us)) return 1;
+    CHECK("two launches, 392 x 1024 lanes")
+    if (time_us([&](int i) {
+          sum_ticket_kernel<256, 0><<<3136, 256>>>(rp + (i % sets) * n, n4, 4, reinterpret_cast<unsigned long long*>(part), counters, out);
+        }, 40, &us)) return 1;
+    CHECK("ticket, 3136 x 256 lanes, one counter")
+    if (time_us([&](int i) {
+          sum_ticket_kernel<1024, 0><<<392, 1024>>>(rp + (i % sets) * n, n4, 8, reinterpret_cast<unsigned long long*>(part), counters, out);
+        }, 40, &us)) return 1;
+    CHECK("ticket, 392 x 1024 lanes, one counter")
+    if (time_us([&](int i) {
+          sum_ticket_kernel<256, 56><<<3136, 256>>>(rp + (i % sets) * n, n4, 4, reinterpret_cast<unsigned long long*>(part), counters, out);
+        }, 40, &us)) return 1;
+    CHECK("ticket, 3136 x 256 lanes, counters of 56 + 1")
+    if (time_us([&](int i) {
+          sum_slices_kernel<256><<<3136, 256>>>(rp + (i % sets) * n, n4, 4, part);
+        }, 40, &us)) return 1;
+    printf("full sum %-44s %.2f\n", "slices alone (first of the two launches)", us);
   }
   return 0;
 }

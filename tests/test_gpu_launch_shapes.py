@@ -37,3 +37,8 @@ def test_both_numberings_of_the_strided_reduce_give_the_same_maxima(table):
 def test_every_channel_tile_variant_copies_the_tensor_unchanged(table):
     rows = re.findall(r"tile \[\d+,\d+,\d+\] T\d+x\d+ \w+\s+\w+\s+\d+\.\d+ (\w+)", table)
     assert len(rows) == 13 and all(r == "same" for r in rows), rows
+
+
+def test_the_single_launch_sums_agree_with_the_two_launches(table):
+    rows = re.findall(r"^full sum (two launches|ticket)[^\n]*? (\d+\.\d+) (\w+)$", table, re.M)
+    assert len(rows) == 5 and all(r[2] == "same" for r in rows), rows
