@@ -472,9 +472,10 @@ static bool plan_pool_band(const PoolArgs& p, int target_outputs, BandArgs* a) {
 // of two or three input rows, one 128-bit load per row (a wave's loads are whole
 // rows of consecutive vectors), plus, for three columns, the one column before
 // (pad 1) or after (pad 0) them, which the neighbouring lane loads as part of
-// its own vector and this one fetches as a single float.  Cells outside the input
-// take the fold's neutral value, as the padding of the band tile does, and every
-// window is folded row by row, left to right.  (Four outputs per lane from two
+// its own vector: it comes from that lane's register (a wave shift), and only
+// the lane at the wave's end fetches it from memory.  Cells outside the input take
+// the fold's neutral value, as the padding of the band tile does, and every window
+// is folded row by row, left to right.  (Four outputs per lane from two
 // vectors per row, so that a load instruction covers every other 16 bytes, ran
 // at 59 us on [64,64,112,112] where the band kernel takes 49 and this one 43;
 // workgroups of 64 or 1024 lanes 47 to 48 us, XCD-contiguous numbering no change.)
@@ -486,22 +487,37 @@ struct HalveArgs {
 
 constexpr int kHalveLanes = kBlock;
 
-template <bool MAX, int K>
+// Lane i receives `from` of lane i - 1 (SHIFT = -1) or i + 1 (SHIFT = +1) of its
+// wave; the lane at the wave's end keeps `own`.
+template <int SHIFT>
+SHDW_DEVICE float neighbour(float own, float from) {
+  constexpr int kWaveShr1 = 0x138, kWaveShl1 = 0x130;
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(own), __float_as_int(from),
+                                                    SHIFT < 0 ? kWaveShr1 : kWaveShl1, 0xf, 0xf, false));
+}
+
+template <bool MAX, int K, int PAD>
 __global__ __launch_bounds__(kHalveLanes) void pool_halve_kernel(const float* x, float* y, uint32_t tasks,
-                                                             HalveArgs p) {
+                                                                 HalveArgs p) {
   const uint32_t t = blockIdx.x * kHalveLanes + threadIdx.x;
   if (t >= tasks) return;
   uint32_t rest, v, plane, r;
   fd_divmod(t, p.f_pairs, rest, v);
   fd_divmod(rest, p.f_out_h, plane, r);
   constexpr int kCells = K == 3 ? 5 : 4;  // columns under the two windows
+  constexpr int kAt = (K == 3 && PAD) ? 1 : 0;  // where column 4v sits among the cells
   const float neutral = MAX ? -FLT_MAX : 0.f;
-  const int h_first = 2 * static_cast<int>(r) - p.pad;
+  const int h_first = 2 * static_cast<int>(r) - PAD;
   const float* img = x + plane * static_cast<uint32_t>(p.in_h * p.in_w) + 4 * v;
-  const int halo_col = p.pad ? -1 : 4;  // relative to column 4v
-  const int halo_abs = 4 * static_cast<int>(v) + halo_col;
+  // The one column beside the vector belongs to the neighbouring lane's vector (the
+  // lanes of a wave walk along a row); only the lane at the wave's end fetches it.
+  constexpr int kHaloCol = PAD ? -1 : 4;  // relative to column 4v
+  const int halo_abs = 4 * static_cast<int>(v) + kHaloCol;
   const bool halo_valid = K == 3 && halo_abs >= 0 && halo_abs < p.in_w;
-  float c[K][kCells];
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const bool fetch_halo = halo_valid && lane == (PAD ? 0u : static_cast<uint32_t>(kWave - 1));
+  float acc[2];
+  acc[0] = acc[1] = MAX ? -FLT_MAX : 0.f;
 #pragma unroll
   for (int i = 0; i < K; ++i) {
     const int ri = h_first + i;
@@ -509,35 +525,32 @@ __global__ __launch_bounds__(kHalveLanes) void pool_halve_kernel(const float* x,
     const float* row = img + min(max(ri, 0), p.in_h - 1) * p.in_w;
     const v4f q = load4(row);
     float cells[kCells];
-    const int at = (K == 3 && p.pad) ? 1 : 0;  // where column 4v sits among the cells
 #pragma unroll
-    for (int e = 0; e < 4; ++e) cells[at + e] = q[e];
+    for (int e = 0; e < 4; ++e) cells[kAt + e] = q[e];
     if (K == 3) {
-      const float h = row[halo_valid ? halo_col : 0];
-      cells[p.pad ? 0 : 4] = halo_valid ? h : neutral;
+      float own = neutral;
+      if (fetch_halo) own = row[kHaloCol];
+      const float h = PAD ? neighbour<-1>(own, q[3]) : neighbour<+1>(own, q[0]);
+      cells[PAD ? 0 : 4] = halo_valid ? h : neutral;
     }
+    // a row above or below the input leaves the running values as they are,
+    // which is what folding the neutral value into them does
 #pragma unroll
-    for (int e = 0; e < kCells; ++e) c[i][e] = row_valid ? cells[e] : neutral;
+    for (int j = 0; j < 2; ++j) {
+      float next = acc[j];
+#pragma unroll
+      for (int k = 0; k < K; ++k) next = MAX ? pool_max(next, cells[2 * j + k]) : next + cells[2 * j + k];
+      acc[j] = row_valid ? next : acc[j];
+    }
   }
   float res[2];
-  const int h_end_pad = min(h_first + K, p.in_h + p.pad);
+  const int h_end_pad = min(h_first + K, p.in_h + PAD);
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    float max_val = -FLT_MAX, sum_val = 0.f;
-#pragma unroll
-    for (int i = 0; i < K; ++i) {
-#pragma unroll
-      for (int k = 0; k < K; ++k) {
-        if (MAX)
-          max_val = pool_max(max_val, c[i][2 * j + k]);
-        else
-          sum_val += c[i][2 * j + k];
-      }
-    }
-    const int w_first = 2 * (2 * static_cast<int>(v) + j) - p.pad;
-    const int w_end_pad = min(w_first + K, p.in_w + p.pad);
+    const int w_first = 2 * (2 * static_cast<int>(v) + j) - PAD;
+    const int w_end_pad = min(w_first + K, p.in_w + PAD);
     const int pool_size = (h_end_pad - h_first) * (w_end_pad - w_first);
-    res[j] = MAX ? max_val : sum_val / static_cast<float>(pool_size);
+    res[j] = MAX ? acc[j] : acc[j] / static_cast<float>(pool_size);
   }
   typedef float v2f __attribute__((ext_vector_type(2)));
   float* dst = y + ((plane * static_cast<uint32_t>(p.out_h) + r) * static_cast<uint32_t>(p.out_w) + 2 * v);
@@ -1262,13 +1275,15 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
     h.in_h = p.in_h, h.in_w = p.in_w, h.out_h = p.out_h, h.out_w = p.out_w, h.pad = p.pw;
     h.f_pairs = make_fastdiv(static_cast<uint32_t>(p.out_w / 2));
     h.f_out_h = make_fastdiv(static_cast<uint32_t>(p.out_h));
-    if (p.kh == 3) {
-      if (pool_type == 0) pool_halve_kernel<true, 3><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h);
-      else pool_halve_kernel<false, 3><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h);
-    } else {
-      if (pool_type == 0) pool_halve_kernel<true, 2><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h);
-      else pool_halve_kernel<false, 2><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h);
-    }
+#define SHDW_HALVE(KV, PV)                                                                     \
+  do {                                                                                         \
+    if (pool_type == 0) pool_halve_kernel<true, KV, PV><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h); \
+    else pool_halve_kernel<false, KV, PV><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h);       \
+  } while (0)
+    if (p.kh == 2) SHDW_HALVE(2, 0);
+    else if (p.pw == 0) SHDW_HALVE(3, 0);
+    else SHDW_HALVE(3, 1);
+#undef SHDW_HALVE
     return launch_status();
   }
   BandArgs a;
