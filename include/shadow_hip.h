@@ -474,7 +474,8 @@ enum {
   SHDW_PATH_POOL_SMALL_PLANES = 23, /* whole planes in LDS; variant = 100 * separable + window unrolled for (0: loops) */
   SHDW_PATH_POOL_BAND = 24,         /* bands of input rows in LDS; variant = 100 * registers per lane + window unrolled for */
   SHDW_PATH_POOL_WINDOW = 25,       /* a lane per output, windows from memory */
-  SHDW_PATH_POOL_HALVE = 26         /* 3x3 / 2x2 at stride 2, output rows half as long as input rows of 4 m columns: no staging; variant = window side */
+  SHDW_PATH_POOL_HALVE = 26,        /* 3x3 / 2x2 at stride 2, output rows half as long as input rows of 4 m columns: no staging; variant = window side */
+  SHDW_PATH_POOL_SAME = 27          /* 3x3 at stride 1 with pad 1 on rows of 4 m columns: no staging */
 };
 int shdw_hip_softmax_plan(int outer_num, int dim, int inner_num, int* path, int* variant,
                           unsigned* grid);

@@ -557,6 +557,66 @@ __global__ __launch_bounds__(kHalveLanes) void pool_halve_kernel(const float* x,
   __builtin_nontemporal_store(v2f{res[0], res[1]}, reinterpret_cast<v2f*>(dst));
 }
 
+// 3x3 windows at stride 1 with one cell of padding (the output as large as the
+// input; rows of a multiple of four columns): a lane owns four neighbouring outputs
+// of one row, whose windows lie in its own vector of three input rows and in the
+// columns left and right of it, which are elements of the neighbouring lanes'
+// vectors (wave shifts; the lanes at the two ends of a wave fetch theirs).  One
+// 128-bit load per input row, one 128-bit store.
+template <bool MAX>
+__global__ __launch_bounds__(kHalveLanes) void pool_same_kernel(const float* x, float* y, uint32_t tasks,
+                                                                HalveArgs p) {
+  const uint32_t t = blockIdx.x * kHalveLanes + threadIdx.x;
+  if (t >= tasks) return;
+  uint32_t rest, v, plane, r;
+  fd_divmod(t, p.f_pairs, rest, v);  // f_pairs: vectors per row here
+  fd_divmod(rest, p.f_out_h, plane, r);
+  const float neutral = MAX ? -FLT_MAX : 0.f;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const bool left_valid = v > 0, right_valid = 4 * v + 4 < static_cast<uint32_t>(p.in_w);
+  const bool fetch_left = left_valid && lane == 0, fetch_right = right_valid && lane == kWave - 1;
+  const float* img = x + plane * static_cast<uint32_t>(p.in_h * p.in_w) + 4 * v;
+  const int h_first = static_cast<int>(r) - 1;
+  float acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc[j] = MAX ? -FLT_MAX : 0.f;
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    const int ri = h_first + i;
+    const bool row_valid = ri >= 0 && ri < p.in_h;
+    const float* row = img + min(max(ri, 0), p.in_h - 1) * p.in_w;
+    const v4f q = load4(row);
+    float own_l = neutral, own_r = neutral;
+    if (fetch_left) own_l = row[-1];
+    if (fetch_right) own_r = row[4];
+    const float hl = neighbour<-1>(own_l, q[3]), hr = neighbour<+1>(own_r, q[0]);
+    const float cells[6] = {left_valid ? hl : neutral, q[0], q[1], q[2], q[3], right_valid ? hr : neutral};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float next = acc[j];
+#pragma unroll
+      for (int k = 0; k < 3; ++k) next = MAX ? pool_max(next, cells[j + k]) : next + cells[j + k];
+      acc[j] = row_valid ? next : acc[j];
+    }
+  }
+  v4f res;
+  const int h_end_pad = min(h_first + 3, p.in_h + 1);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int w_first = 4 * static_cast<int>(v) + j - 1;
+    const int w_end_pad = min(w_first + 3, p.in_w + 1);
+    const int pool_size = (h_end_pad - h_first) * (w_end_pad - w_first);
+    res[j] = MAX ? acc[j] : acc[j] / static_cast<float>(pool_size);
+  }
+  store4_stream(y + ((plane * static_cast<uint32_t>(p.out_h) + r) * static_cast<uint32_t>(p.out_w) + 4 * v), res);
+}
+
+static bool pool_same_applies(const PoolArgs& p, const float* x, const float* y, bool planning) {
+  if (p.kh != 3 || p.kw != 3 || p.sh != 1 || p.sw != 1 || p.ph != 1 || p.pw != 1) return false;
+  if (p.in_w % 4 != 0 || p.out_w != p.in_w || p.out_h != p.in_h) return false;
+  return planning || (aligned16(x) && aligned16(y));
+}
+
 // True when the kernel above applies to p (2-D).
 static bool pool_halve_applies(const PoolArgs& p, const float* x, const float* y, bool planning) {
   if (p.kh != p.kw || p.sh != 2 || p.sw != 2 || p.ph != p.pw) return false;
@@ -1284,6 +1344,18 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
     else if (p.pw == 0) SHDW_HALVE(3, 0);
     else SHDW_HALVE(3, 1);
 #undef SHDW_HALVE
+    return launch_status();
+  }
+  if (!three_d && pool_same_applies(p, x, y, pl->want)) {
+    const uint32_t tasks = n_out / 4;
+    const uint32_t grid = (tasks + kHalveLanes - 1) / kHalveLanes;
+    if (pl->chosen(SHDW_PATH_POOL_SAME, 3, grid)) return SHDW_OK;
+    HalveArgs h;
+    h.in_h = p.in_h, h.in_w = p.in_w, h.out_h = p.out_h, h.out_w = p.out_w, h.pad = 1;
+    h.f_pairs = make_fastdiv(static_cast<uint32_t>(p.in_w / 4));
+    h.f_out_h = make_fastdiv(static_cast<uint32_t>(p.out_h));
+    if (pool_type == 0) pool_same_kernel<true><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h);
+    else pool_same_kernel<false><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h);
     return launch_status();
   }
   BandArgs a;

@@ -448,6 +448,29 @@ def test_pooling_by_two_without_staging(ws, gpu, pool, full, shape, kernel, pad)
     assert small or (path.value == 26) == halves, (path.value, want.shape)
 
 
+@pytest.mark.parametrize("pool", [0, 1])
+@pytest.mark.parametrize("shape", [(2, 3, 40, 64), (1, 2, 33, 128), (1, 1, 5, 4), (2, 2, 1, 8), (1, 1, 70, 260),
+                                   (3, 1, 2, 1028), (1, 4, 112, 112)])
+def test_pooling_3x3_stride_1_without_staging(ws, gpu, pool, shape):
+    """3x3 at stride 1 with one cell of padding on rows of a multiple of four columns: the output is as large
+    as the input, and planes too large for the whole-plane kernel take the kernel without staging (asked of
+    the plan query).  Edge columns and rows, NaNs, infinities, signed zeros and lowest() are planted."""
+    x = with_specials(normal(24, shape, 2.0), 24).reshape(shape)
+    x[..., 0] = np.where(np.arange(shape[2])[:, None].repeat(1, 1)[:, 0] % 2 == 0, -0.0, 0.0).astype(np.float32)
+    x[..., -1] = np.float32(-3.4028235e38)
+    x[..., 0, 1:3] = np.inf
+    args = {"pool": pool, "kernel_size": [3], "stride": [1], "pad": [1], "full_pooling": False}
+    got = run(ws, "Pooling", [("x", x)], args)
+    want = oracle.pooling_op(x, pool, [3], [1], [1], full_pooling=False)
+    assert got.shape == want.shape == x.shape
+    assert_bit_exact(got, want, "pooling 3x3 s1")
+    path, variant, grid = ctypes.c_int(), ctypes.c_int(), ctypes.c_uint()
+    assert shadow_amd.hip().shdw_hip_pooling2d_plan(shadow_amd.ints(list(shape)), pool, 3, 3, 1, 1, 1, 1,
+                                                    shadow_amd.ints(list(shape)), ctypes.byref(path),
+                                                    ctypes.byref(variant), ctypes.byref(grid)) == 0
+    assert path.value in (23, 27), path.value  # whole small planes in LDS, or no staging
+
+
 # The maximum keeps the earlier of equal cells and never takes a NaN: planes of signed
 # zeros, -inf, lowest() and NaNs show whether an implementation that folds rows first
 # returns the cell the row-major walk returns.

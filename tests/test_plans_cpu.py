@@ -16,7 +16,7 @@ import shadow_amd
 from shadow_amd import ints
 
 ROWS, ROWS_STREAM, SHORT_ROWS, QUADS, PACKED, LONG_SLAB, SLAB, COLUMNS_REG, TILE, TALL, COLUMNS = range(1, 12)
-PLANE_REDUCE, PLANE, PLANE_STREAM, SMALL_PLANES, BAND, WINDOW, HALVE = range(20, 27)
+PLANE_REDUCE, PLANE, PLANE_STREAM, SMALL_PLANES, BAND, WINDOW, HALVE, SAME = range(20, 28)
 
 SOFTMAX = {  # (outer, dim, inner)
     (16, 49, 16384): (COLUMNS_REG, 64, 1024),      # softmax_channels_dense
@@ -83,6 +83,8 @@ POOLING = {  # ((n, c, h, w), pool type, kernel, stride, pad)
     ((64, 512, 19, 19), 0, 9, 1, 4): (SMALL_PLANES, 109, 10923),
     ((19, 1000, 26, 26), 0, 5, 1, 2): (SMALL_PLANES, 105, 9500),
     ((16, 64, 112, 112), 0, 5, 1, 2): (BAND, 305, 7168),
+    ((16, 64, 112, 112), 0, 3, 1, 1): (SAME, 3, 12544),        # as large as its input: no staging
+    ((16, 64, 112, 112), 1, 3, 1, 1): (SAME, 3, 12544),
     ((4, 3, 720, 1280), 1, 5, 3, 1): (BAND, 800, 2880),
     ((2, 3, 2000, 3000), 0, 4, 4, 0): (WINDOW, 0, 8790),
 }
@@ -139,5 +141,5 @@ def test_path_values_match_the_header():
             "LONG_SLAB": LONG_SLAB, "SLAB": SLAB, "COLUMNS_REG": COLUMNS_REG, "TILE": TILE, "TALL": TALL,
             "COLUMNS": COLUMNS, "POOL_PLANE_REDUCE": PLANE_REDUCE, "POOL_PLANE": PLANE,
             "POOL_PLANE_STREAM": PLANE_STREAM, "POOL_SMALL_PLANES": SMALL_PLANES, "POOL_BAND": BAND,
-            "POOL_WINDOW": WINDOW, "POOL_HALVE": HALVE, "NONE": 0}
+            "POOL_WINDOW": WINDOW, "POOL_HALVE": HALVE, "POOL_SAME": SAME, "NONE": 0}
     assert found == mine
