@@ -206,6 +206,25 @@ def test_resize_by_two_of_even_rows(ws, typ, shape):
     assert_bit_exact(got, want, "x2 type %d %s" % (typ, shape))
 
 
+@pytest.mark.parametrize("typ", [0, 1])
+@pytest.mark.parametrize("x_off,y_off", [(1, 0), (2, 0), (3, 0), (0, 1), (2, 2), (1, 3)])
+def test_resize_by_two_on_pointers_off_the_vector_boundary(gpu, typ, x_off, y_off):
+    """x2 through the C ABI with the input and the output 1 to 3 floats off 16-byte alignment: whichever kernel
+    the alignment leaves (the one without staging needs y on 16 bytes and, for nearest, x on 8), same bits."""
+    shape = (2, 3, 19, 24)
+    x = with_specials(normal(94, shape, 2.0), 94).reshape(shape)
+    want = oracle.resize_op(x, [0], [2.0], typ, False)
+    lib = shadow_amd.hip()
+    dx = shadow_amd.Buffer(x.nbytes + 16)
+    dx.upload(x, 4 * x_off)
+    dy = shadow_amd.Buffer(want.nbytes + 16)
+    shadow_amd.check(lib.shdw_hip_resize(shadow_amd.ints(list(shape)), shadow_amd.ints(list(want.shape)), typ, 0,
+                                         dx.ptr + 4 * x_off, dy.ptr + 4 * y_off, None))
+    shadow_amd.check(lib.shdw_hip_stream_sync(None))
+    got = dy.download(count=want.size, offset_bytes=4 * y_off).reshape(want.shape)
+    assert_bit_exact(got, want, "x2 type %d, x + %d, y + %d floats" % (typ, x_off, y_off))
+
+
 @pytest.mark.parametrize("shape,group", [((2, 6, 3, 5), 2), ((2, 6, 3, 5), 3), ((1, 12, 4, 4), 4), ((3, 8, 1, 1), 8),
                                          ((2, 116, 28, 28), 2), ((2, 6, 3, 5), 1), ((2, 116, 7, 7), 2), ((3, 4, 1, 3), 2),
                                          # rows of 7, 1, 2, 5 and 49 floats: a lane's four outputs from up to four rows
