@@ -71,6 +71,19 @@ SHDW_DEVICE uint32_t xcd_contiguous(uint32_t block, uint32_t grid) {
   return x * q + (x < r ? x : r) + slot;
 }
 
+// Between the two: XCD x gets runs of 2^log2_run consecutive work items (its
+// workgroups b, b + 8, ... of one run), the runs of the eight XCDs interleaved.
+// For kernels that stream and also write a few bytes per workgroup (a row's mean,
+// a row's maximum): the workgroups whose small results share a cache line then
+// complete that line in one L2, while the stream stays spread over all XCDs.  A
+// bijection of [0, grid); the incomplete last span keeps its numbering.
+SHDW_DEVICE uint32_t xcd_runs(uint32_t block, uint32_t grid, uint32_t log2_run) {
+  const uint32_t span = kXcds << log2_run;
+  if (block >= grid - grid % span) return block;
+  const uint32_t turn = block / kXcds, xcd = block % kXcds;
+  return (turn >> log2_run) * span + (xcd << log2_run) + (turn & ((1u << log2_run) - 1u));
+}
+
 // ---------------------------------------------------------------------------
 // Division of a 31-bit unsigned value by a divisor fixed at launch time:
 //   q = (mulhi(n, m) + n) >> s

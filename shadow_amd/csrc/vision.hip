@@ -566,7 +566,8 @@ __global__ __launch_bounds__(kHalveLanes) void pool_halve_kernel(const float* x,
 template <bool MAX>
 __global__ __launch_bounds__(kHalveLanes) void pool_same_kernel(const float* x, float* y, uint32_t tasks,
                                                                 HalveArgs p) {
-  const uint32_t t = blockIdx.x * kHalveLanes + threadIdx.x;
+  // runs of eight workgroups on one XCD: every input row is read for three output rows
+  const uint32_t t = xcd_runs(blockIdx.x, gridDim.x, 3) * kHalveLanes + threadIdx.x;
   if (t >= tasks) return;
   uint32_t rest, v, plane, r;
   fd_divmod(t, p.f_pairs, rest, v);  // f_pairs: vectors per row here
