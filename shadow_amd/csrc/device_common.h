@@ -65,7 +65,7 @@ SHDW_DEVICE bool aligned16_device(const void* p) {
 // owns one contiguous range of work items and the shared lines are fetched from
 // HBM once.  A bijection of [0, grid) for every grid size.
 constexpr uint32_t kXcds = 8;
-SHDW_DEVICE uint32_t xcd_contiguous(uint32_t block, uint32_t grid) {
+__host__ SHDW_DEVICE uint32_t xcd_contiguous(uint32_t block, uint32_t grid) {
   const uint32_t x = block % kXcds, slot = block / kXcds;
   const uint32_t q = grid / kXcds, r = grid % kXcds;
   return x * q + (x < r ? x : r) + slot;
@@ -77,7 +77,7 @@ SHDW_DEVICE uint32_t xcd_contiguous(uint32_t block, uint32_t grid) {
 // a row's maximum): the workgroups whose small results share a cache line then
 // complete that line in one L2, while the stream stays spread over all XCDs.  A
 // bijection of [0, grid); the incomplete last span keeps its numbering.
-SHDW_DEVICE uint32_t xcd_runs(uint32_t block, uint32_t grid, uint32_t log2_run) {
+__host__ SHDW_DEVICE uint32_t xcd_runs(uint32_t block, uint32_t grid, uint32_t log2_run) {
   const uint32_t span = kXcds << log2_run;
   if (block >= grid - grid % span) return block;
   const uint32_t turn = block / kXcds, xcd = block % kXcds;

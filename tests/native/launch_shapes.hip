@@ -332,7 +332,23 @@ __global__ __launch_bounds__(256) void add_chain_kernel(const float* in, float* 
   out[blockIdx.x * 256 + threadIdx.x] = t;
 }
 
+// Both renumberings of the workgroups must visit every work item exactly once, whatever the grid.
+static bool numberings_are_bijections() {
+  std::vector<uint8_t> seen;
+  for (uint32_t grid = 1; grid <= 3000; grid += (grid < 300 ? 1 : 7)) {
+    for (int k = -1; k <= 5; ++k) {  // -1: xcd_contiguous
+      seen.assign(grid, 0);
+      for (uint32_t b = 0; b < grid; ++b) {
+        const uint32_t w = k < 0 ? xcd_contiguous(b, grid) : xcd_runs(b, grid, static_cast<uint32_t>(k));
+        if (w >= grid || seen[w]++) return false;
+      }
+    }
+  }
+  return true;
+}
+
 int main() {
+  printf("numberings %s\n", numberings_are_bijections() ? "same" : "DIFFERENT");
   const size_t kPool = 6ull * 205520896;
   float *rp, *wp;
   CK(hipMalloc(&rp, kPool));

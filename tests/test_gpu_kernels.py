@@ -443,7 +443,8 @@ def test_fused_tail(gpu, outer, num, inner):
 
 @pytest.mark.parametrize("form", ["scale", "bias", "both"])
 @pytest.mark.parametrize("residual_first", [False, True])
-@pytest.mark.parametrize("outer,num,inner", [(2, 8, 196), (3, 5, 7), (2, 3, 1030)])
+# (101, 4, 12): 101 workgroups, three whole runs of 32 (which the kernel renumbers) and a rest of five
+@pytest.mark.parametrize("outer,num,inner", [(2, 8, 196), (3, 5, 7), (2, 3, 1030), (101, 4, 12)])
 def test_fused_tail_forms(gpu, form, residual_first, outer, num, inner):
     """The forms a network holds the sequence in: Scale with one parameter blob only, the
     residual as the first Eltwise input, no Reduce behind it."""

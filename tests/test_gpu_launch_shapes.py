@@ -27,6 +27,7 @@ def test_every_table_of_the_probe_is_there(table):
     assert len(re.findall(r"^stream (\w+)\s+(\d+) MB:", table, re.M)) == 6
     assert len(re.findall(r"^add chain waves (\d+) chains (\d+):", table, re.M)) == 7
     assert "DIFFERENT" not in table
+    assert "numberings same" in table  # xcd_contiguous and xcd_runs visit every work item once, grids of 1 to 3000
 
 
 def test_both_numberings_of_the_strided_reduce_give_the_same_maxima(table):

@@ -450,7 +450,8 @@ def test_pooling_by_two_without_staging(ws, gpu, pool, full, shape, kernel, pad)
 
 @pytest.mark.parametrize("pool", [0, 1])
 @pytest.mark.parametrize("shape", [(2, 3, 40, 64), (1, 2, 33, 128), (1, 1, 5, 4), (2, 2, 1, 8), (1, 1, 70, 260),
-                                   (3, 1, 2, 1028), (1, 4, 112, 112)])
+                                   (3, 1, 2, 1028), (1, 4, 112, 112),
+                                   (2, 8, 112, 112)])  # 196 workgroups: three whole runs of 64 and a rest of four
 def test_pooling_3x3_stride_1_without_staging(ws, gpu, pool, shape):
     """3x3 at stride 1 with one cell of padding on rows of a multiple of four columns: the output is as large
     as the input, and planes too large for the whole-plane kernel take the kernel without staging (asked of
