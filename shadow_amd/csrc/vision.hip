@@ -480,8 +480,8 @@ static bool plan_pool_band(const PoolArgs& p, int target_outputs, BandArgs* a) {
 // at 59 us on [64,64,112,112] where the band kernel takes 49 and this one 43;
 // workgroups of 64 or 1024 lanes 47 to 48 us, XCD-contiguous numbering no change.)
 struct HalveArgs {
-  int in_h, in_w, out_h, out_w, pad;
-  FastDiv f_pairs;  // out_w / 2 = in_w / 4
+  int in_h, in_w, out_h, out_w;
+  FastDiv f_pairs;  // lanes per output row: in_w / 4
   FastDiv f_out_h;
 };
 
@@ -570,7 +570,7 @@ __global__ __launch_bounds__(kHalveLanes) void pool_same_kernel(const float* x, 
   const uint32_t t = xcd_runs(blockIdx.x, gridDim.x, 3) * kHalveLanes + threadIdx.x;
   if (t >= tasks) return;
   uint32_t rest, v, plane, r;
-  fd_divmod(t, p.f_pairs, rest, v);  // f_pairs: vectors per row here
+  fd_divmod(t, p.f_pairs, rest, v);
   fd_divmod(rest, p.f_out_h, plane, r);
   const float neutral = MAX ? -FLT_MAX : 0.f;
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -1333,7 +1333,7 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
     const uint32_t grid = (tasks + kHalveLanes - 1) / kHalveLanes;
     if (pl->chosen(SHDW_PATH_POOL_HALVE, p.kh, grid)) return SHDW_OK;
     HalveArgs h;
-    h.in_h = p.in_h, h.in_w = p.in_w, h.out_h = p.out_h, h.out_w = p.out_w, h.pad = p.pw;
+    h.in_h = p.in_h, h.in_w = p.in_w, h.out_h = p.out_h, h.out_w = p.out_w;
     h.f_pairs = make_fastdiv(static_cast<uint32_t>(p.out_w / 2));
     h.f_out_h = make_fastdiv(static_cast<uint32_t>(p.out_h));
 #define SHDW_HALVE(KV, PV)                                                                     \
@@ -1352,7 +1352,7 @@ static int run_pooling(bool three_d, const int* in_shape, int pool_type, const i
     const uint32_t grid = (tasks + kHalveLanes - 1) / kHalveLanes;
     if (pl->chosen(SHDW_PATH_POOL_SAME, 3, grid)) return SHDW_OK;
     HalveArgs h;
-    h.in_h = p.in_h, h.in_w = p.in_w, h.out_h = p.out_h, h.out_w = p.out_w, h.pad = 1;
+    h.in_h = p.in_h, h.in_w = p.in_w, h.out_h = p.out_h, h.out_w = p.out_w;
     h.f_pairs = make_fastdiv(static_cast<uint32_t>(p.in_w / 4));
     h.f_out_h = make_fastdiv(static_cast<uint32_t>(p.out_h));
     if (pool_type == 0) pool_same_kernel<true><<<grid, kHalveLanes, 0, st>>>(x, y, tasks, h);
