@@ -12,10 +12,11 @@ comma-separated list of names) sweeps all 2^32 for them too.
 
     SHADOW_GPU_FULL_SWEEP=1 python -m pytest tests/test_gpu_exhaustive.py -m gpu -s
 
-tanh and sigmoid choose between a short and a long form per wave (all 64 lanes,
-four consecutive elements each, inside |x| < 10 resp. |x| < 87: short).  The
-sweep above hands every wave 256 consecutive bit patterns starting at a multiple
-of 256, and both limits are multiples of 256 as bit patterns, so there every
+tanh and sigmoid choose between a short and a long form per wave and vector (all
+64 lanes, four consecutive elements each, inside |x| < 9.75 resp. |x| < 87:
+short).  The sweep above hands every such choice 256 consecutive bit patterns
+starting at a multiple of 256 (a tanh wave makes two, one per vector of its lanes),
+and both limits are multiples of 256 as bit patterns, so there every
 in-range input is computed by the short form and every other input by the long
 one.  test_in_range_inputs_through_the_long_form covers what is left: all
 in-range inputs again, 255 to a wave with a NaN as the 256th, which sends the
