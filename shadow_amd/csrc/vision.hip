@@ -488,7 +488,11 @@ struct HalveArgs {
 constexpr int kHalveLanes = kBlock;
 
 // Lane i receives `from` of lane i - 1 (SHIFT = -1) or i + 1 (SHIFT = +1) of its
-// wave; the lane at the wave's end keeps `own`.
+// wave; the lane at the wave's end keeps `own`.  Whole-wave shifts are DPP
+// controls of the GFX9 family only (gfx950 has them; GFX10 and later do not).
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "vision.hip: wave_shr / wave_shl DPP controls are used as gfx950 provides them"
+#endif
 template <int SHIFT>
 SHDW_DEVICE float neighbour(float own, float from) {
   constexpr int kWaveShr1 = 0x138, kWaveShl1 = 0x130;
