@@ -965,6 +965,10 @@ def config_table(dev, sets_scale=1, cpu=None):
     ms = time_median(dev, lambda k: lib.shdw_hip_batch_norm(NH, CH, INH, AH[k].ptr, meanh.ptr, varh.ptr,
                                                             1.0, 1e-5, YH[k].ptr, st), SH, reps=20)
     add("next", "batch_norm [64,256,56,56]", 4 * NH + 8 * CH, 4 * NH, ms, NH)
+    # BatchNorm -> Scale -> ReLU as the backend's fusion pass runs it: one launch, one pass over the tensor
+    ms = time_median(dev, lambda k: lib.shdw_hip_batch_norm_scale(NH, CH, INH, AH[k].ptr, meanh.ptr, varh.ptr, 1.0, 1e-5,
+                                                                  varh.ptr, meanh.ptr, 1, YH[k].ptr, st), SH, reps=20)
+    add("next", "batch_norm_scale_relu [64,256,56,56]", 4 * NH + 16 * CH, 4 * NH, ms, NH)
     alh = dev.buf(uniform(613, 64 * CH, 0.0, 1.0))
     ms = time_median(dev, lambda k: lib.shdw_hip_axpy_rows(64 * CH, INH, alh.ptr, AH[k].ptr,
                                                            AH[(k + 1) % SH].ptr, YH[k].ptr, st), SH, reps=20)

@@ -293,6 +293,23 @@ int shdw_hip_batch_norm(int n, int channel, int inner_num, const float* x, const
                         const float* variance, float scale_factor, float eps, float* y,
                         void* stream);
 
+/* BatchNorm with global statistics followed by Scale over the same channel axis
+ * (scale and bias hold `channel` values each; either may be null, not both) and,
+ * with relu != 0, by Activate(relu), in one pass: per element
+ *   t = (x - mean[c]*scale_factor) / sqrt(|variance[c]*scale_factor| + eps);
+ *   t = t * scale[c];  t = t + bias[c];  y = relu ? (t > 0 ? t : 0) : t
+ * -- the operators' own arithmetic, so the result is theirs bit for bit.  The pair
+ * a Caffe-style model holds every normalisation in; Shadow has no such fused
+ * operator (its converter folds the pair into the convolution where there is one,
+ * python/converter/shadow/optimizer.py:181-252), the parity target is the sequence.
+ * y may alias x.
+ * ref: shadow/operators/kernels/batch_norm.cpp:11-24, scale.cpp:7-39,
+ *      activate.cpp:12 */
+int shdw_hip_batch_norm_scale(int n, int channel, int inner_num, const float* x, const float* mean,
+                              const float* variance, float scale_factor, float eps,
+                              const float* scale, const float* bias, int relu, float* y,
+                              void* stream);
+
 /* Softmax over the middle extent of x viewed as [outer_num][dim][inner_num]:
  * running maximum, exp(x - max), fp32 running sum in index order, divide.  The
  * per-column scratch blob of the reference is not needed.  y may alias x.

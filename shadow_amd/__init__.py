@@ -84,6 +84,7 @@ SIGNATURES = {
     "shdw_hip_scale_residual_relu": (_I, [_I, _I, _I, _V, _V, _V, _V, _I, _V, _V, _V]),
     "shdw_hip_axpy_rows": (_I, [_I, _I, _V, _V, _V, _V, _V]),
     "shdw_hip_batch_norm": (_I, [_I, _I, _I, _V, _V, _V, _F, _F, _V, _V]),
+    "shdw_hip_batch_norm_scale": (_I, [_I, _I, _I, _V, _V, _V, _F, _F, _V, _V, _I, _V, _V]),
     "shdw_hip_group_norm": (_I, [_I, _I, _F, _V, _V, _V, _I, _I, _V, _V]),
     "shdw_hip_group_norm_workspace_bytes": (_Z, [_I, _I]),
     "shdw_hip_group_norm_ws": (_I, [_I, _I, _F, _V, _V, _V, _I, _I, _V, _V, _Z, _V]),

@@ -59,6 +59,37 @@ struct BatchNormRows {
   static constexpr bool kTwoInputs = false;
 };
 
+// BatchNorm followed by Scale over the same channel axis and, optionally, ReLU:
+// the three operators' arithmetic, element by element, in one pass.
+template <bool HAS_SCALE, bool HAS_BIAS, bool RELU>
+struct BatchNormScaleRows {
+  const float* mean;
+  const float* variance;
+  const float* scale;
+  const float* bias;
+  float scale_factor, eps;
+  FastDiv channel;
+  SHDW_DEVICE v4f load_other(uint64_t) const { return v4f{0, 0, 0, 0}; }
+  SHDW_DEVICE float other(uint64_t) const { return 0.f; }
+  struct Row {
+    float m, d, s, b;
+  };
+  SHDW_DEVICE Row row(uint32_t r) const {
+    const uint32_t c = r - fd_div(r, channel) * channel.d;
+    const float m = mean[c] * scale_factor;
+    const float v = __builtin_fabsf(variance[c] * scale_factor) + eps;
+    return {m, __builtin_sqrtf(v), HAS_SCALE ? scale[c] : 1.f, HAS_BIAS ? bias[c] : 0.f};
+  }
+  SHDW_DEVICE float apply(float x, float, const Row& p) const {
+    float t = (x - p.m) / p.d;    // BatchNorm
+    if (HAS_SCALE) t = t * p.s;   // Scale: multiply, then add
+    if (HAS_BIAS) t = t + p.b;
+    if (RELU) t = t > 0 ? t : 0;  // Activate(relu)
+    return t;
+  }
+  static constexpr bool kTwoInputs = false;
+};
+
 // ROWVEC: inner % 4 == 0, the four elements of a vector share a row.
 template <class P, bool ROWVEC>
 __global__ __launch_bounds__(kStream) void rows_vec_kernel(P p, const float* x, float* out,
@@ -1456,6 +1487,30 @@ int shdw_hip_batch_norm(int n, int channel, int inner_num, const float* x, const
   BatchNormRows p{mean, variance, scale_factor, eps, make_fastdiv(static_cast<uint32_t>(channel))};
   return launch_rows(p, static_cast<uint32_t>(n), static_cast<uint32_t>(inner_num), x, nullptr, y,
                      static_cast<hipStream_t>(stream));
+}
+
+int shdw_hip_batch_norm_scale(int n, int channel, int inner_num, const float* x, const float* mean,
+                              const float* variance, float scale_factor, float eps, const float* scale,
+                              const float* bias, int relu, float* y, void* stream) {
+  if (n < 0 || channel < 1 || inner_num < 1 || (!scale && !bias)) return SHDW_E_INVALID_ARGUMENT;
+  if (n == 0) return SHDW_OK;
+  if (!x || !mean || !variance || !y) return SHDW_E_INVALID_ARGUMENT;
+  const FastDiv fc = make_fastdiv(static_cast<uint32_t>(channel));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint32_t count = static_cast<uint32_t>(n), inner = static_cast<uint32_t>(inner_num);
+#define SHDW_BNS(S, B, R)                                                                       \
+  do {                                                                                          \
+    BatchNormScaleRows<S, B, R> p{mean, variance, scale, bias, scale_factor, eps, fc};          \
+    return launch_rows(p, count, inner, x, nullptr, y, st);                                     \
+  } while (0)
+  if (scale && bias) {
+    if (relu) SHDW_BNS(true, true, true); else SHDW_BNS(true, true, false);
+  } else if (scale) {
+    if (relu) SHDW_BNS(true, false, true); else SHDW_BNS(true, false, false);
+  } else {
+    if (relu) SHDW_BNS(false, true, true); else SHDW_BNS(false, true, false);
+  }
+#undef SHDW_BNS
 }
 
 int shdw_hip_pooling2d(const int* in_shape, int pool_type, int kernel_h, int kernel_w,

@@ -10,6 +10,7 @@
 //   Scale(blob parameters) -> Eltwise(SUM of 2, unit coefficients)
 //                          -> Activate(relu) [-> Reduce(AVG over the trailing axes)]
 //   Eltwise(any operation, any number of inputs) -> Activate(relu)
+//   BatchNorm(global statistics) -> Scale(blob parameters, one per channel) [-> Activate(relu)]
 //
 // A blob that a group no longer writes (the Scale output, the Eltwise output when
 // the Activate is not in place) must have the next member as its only reader and

@@ -114,11 +114,13 @@ struct ScaleView {
   int num = 0, inner = 0;
 };
 
-bool view_scale(const Operator& op, Workspace* ws, ScaleView* v) {
+// `input`: the blob the Scale member works on when that is not its own first
+// input (a group whose earlier member stands in front of it).
+bool view_scale(const Operator& op, Workspace* ws, ScaleView* v, const std::shared_ptr<Blob>& input = nullptr) {
   const auto& p = op.op_param();
   const bool has_scale = op.get_single_argument<bool>("has_scale", false);
   const bool has_bias = op.get_single_argument<bool>("has_bias", false);
-  v->x = float_blob(ws, p.bottom(0));
+  v->x = input != nullptr ? input : float_blob(ws, p.bottom(0));
   if (has_scale) v->scale = float_blob(ws, p.bottom(1));
   if (has_bias) v->bias = float_blob(ws, p.bottom(has_scale ? 2 : 1));
   if (v->x == nullptr || (has_scale && v->scale == nullptr) || (has_bias && v->bias == nullptr)) return false;
@@ -232,6 +234,68 @@ class ResidualTail : public FusedGroup {
   bool residual_first_ = false;
 };
 
+// ---- BatchNorm -> Scale [-> Activate(relu)]: shdw_hip_batch_norm_scale ----
+// How a Caffe-style model holds a normalisation: statistics in one operator, the
+// learned affine pair in the next (shadow/operators/batch_norm_op.cpp:7-47,
+// scale_op.cpp:7-52).
+bool is_stats_batch_norm(const Operator& op) {
+  return op.type() == "BatchNorm" && op.op_param().top_size() == 1 &&
+         (op.op_param().bottom_size() == 3 || op.op_param().bottom_size() == 4);
+}
+
+class BatchNormScale : public FusedGroup {
+ public:
+  BatchNormScale(const OpList& ops, int bn, int scale, int relu) : bn_(ops[bn]), scale_(ops[scale]) {
+    members_ = {bn, scale};
+    if (relu >= 0) {
+      relu_ = ops[relu];
+      members_.push_back(relu);
+    }
+  }
+
+  bool Run(Workspace* ws) override {
+    const auto& p = bn_->op_param();
+    auto x = float_blob(ws, p.bottom(0));
+    auto mean = float_blob(ws, p.bottom(1)), variance = float_blob(ws, p.bottom(2));
+    if (x == nullptr || mean == nullptr || variance == nullptr || x->num_axes() < 2 || x->count() == 0) return false;
+    const int channel = x->shape(1);
+    if (mean->count() != channel || variance->count() != channel) return false;
+    // the affine pair must be one value per channel: Scale over axis 1 with parameters of that one extent
+    ScaleView v;
+    if (!view_scale(*scale_, ws, &v, x)) return false;
+    int axis = scale_->get_single_argument<int>("axis", 1);
+    if (axis < 0) axis += x->num_axes();
+    if (axis != 1 || v.num != channel || v.inner != x->count(2)) return false;
+    float scale_factor = 1;
+    if (p.bottom_size() == 4) {
+      auto factor = float_blob(ws, p.bottom(3));
+      if (factor == nullptr || factor->count() != 1) return false;
+      float value = 1;
+      factor->get_data<float>(&value, 1);  // synchronous device -> host read, as the operator does
+      scale_factor = value == 0 ? 0 : 1 / value;
+    }
+    const auto& last = relu_ != nullptr ? relu_ : scale_;
+    auto y = float_blob(ws, last->op_param().top(0));
+    if (y == nullptr || y == mean || y == variance || y == v.scale || y == v.bias) return false;
+    y->reshape(x->shape());
+    SHADOW_HIP_CHECK(shdw_hip_batch_norm_scale(
+        x->count(), channel, v.inner, x->data<float>(), mean->data<float>(), variance->data<float>(), scale_factor,
+        bn_->get_single_argument<float>("eps", 1e-5), v.scale ? v.scale->data<float>() : nullptr,
+        v.bias ? v.bias->data<float>() : nullptr, relu_ != nullptr ? 1 : 0, y->mutable_data<float>(),
+        ws->Ctx()->stream()));
+    return true;
+  }
+
+  std::string describe() const override {
+    std::string text = label(*bn_) + " + " + label(*scale_);
+    if (relu_ != nullptr) text += " + " + label(*relu_);
+    return text + " -> " + (relu_ != nullptr ? relu_ : scale_)->op_param().top(0);
+  }
+
+ private:
+  std::shared_ptr<Operator> bn_, scale_, relu_;
+};
+
 // ---- Eltwise -> Activate(relu): shdw_hip_eltwise_relu ----
 // What closes a residual block once the converter has folded the normalisation into
 // the convolution (optimizer.py:181-252): the add and the ReLU.
@@ -293,23 +357,13 @@ std::vector<std::unique_ptr<FusedGroup>> FindFusedGroups(const OpList& ops,
   std::vector<std::unique_ptr<FusedGroup>> groups;
   std::vector<bool> taken(ops.size(), false);
   const int count = static_cast<int>(ops.size());
+  // Residual tails first: a Scale whose output goes into a sum saves as much there as behind
+  // its BatchNorm, and the tail can take the mean along.
   for (int i = 0; i < count; ++i) {
     if (taken[i] || !is_blob_scale(*ops[i])) continue;
     const std::string& s = ops[i]->op_param().top(0);
     const int next = next_reader(ops, s, i);
     if (next < 0 || taken[next]) continue;
-
-    if (is_relu(*ops[next])) {
-      // in place the Scale output is the group's output and every later reader sees the
-      // activated values either way; elsewhere it is no longer written
-      if (ops[next]->op_param().top(0) != s && !sole_reader(ops, out_blob, s, i, next)) continue;
-      std::vector<int> members = {i, next};
-      if (!movable(ops, members)) continue;
-      groups.emplace_back(new ScaleRelu(ops, i, next));
-      taken[i] = taken[next] = true;
-      continue;
-    }
-
     if (!is_residual_sum(*ops[next]) || !sole_reader(ops, out_blob, s, i, next)) continue;
     const std::string& e = ops[next]->op_param().top(0);
     const int relu = next_reader(ops, e, next);
@@ -333,6 +387,46 @@ std::vector<std::unique_ptr<FusedGroup>> FindFusedGroups(const OpList& ops,
     groups.emplace_back(new ResidualTail(ops, i, next, relu, mean));
     taken[i] = taken[next] = taken[relu] = true;
     if (mean >= 0) taken[mean] = true;
+  }
+  // BatchNorm -> Scale [-> ReLU] next: it takes the Scale -> ReLU pair with it.
+  for (int i = 0; i < count; ++i) {
+    if (taken[i] || !is_stats_batch_norm(*ops[i])) continue;
+    const std::string& n = ops[i]->op_param().top(0);
+    const int scale = next_reader(ops, n, i);
+    if (scale < 0 || taken[scale] || !is_blob_scale(*ops[scale])) continue;
+    const auto& sp = ops[scale]->op_param();
+    if (sp.bottom(0) != n) continue;
+    bool as_parameter = false;  // the normalised blob must be the Scale's data, not one of its parameters
+    for (int k = 1; k < sp.bottom_size(); ++k) as_parameter = as_parameter || sp.bottom(k) == n;
+    if (as_parameter) continue;
+    const std::string& s = sp.top(0);
+    // in place the Scale output is the group's output; elsewhere the normalised blob is no longer written
+    if (s != n && !sole_reader(ops, out_blob, n, i, scale)) continue;
+    std::vector<int> members = {i, scale};
+    if (!movable(ops, members)) continue;
+    int relu = next_reader(ops, s, scale);
+    if (relu >= 0 && (taken[relu] || !is_relu(*ops[relu]))) relu = -1;
+    if (relu >= 0 && ops[relu]->op_param().top(0) != s && !sole_reader(ops, out_blob, s, scale, relu)) relu = -1;
+    if (relu >= 0) {
+      members.push_back(relu);
+      if (!movable(ops, members)) relu = -1;
+    }
+    groups.emplace_back(new BatchNormScale(ops, i, scale, relu));
+    taken[i] = taken[scale] = true;
+    if (relu >= 0) taken[relu] = true;
+  }
+  for (int i = 0; i < count; ++i) {
+    if (taken[i] || !is_blob_scale(*ops[i])) continue;
+    const std::string& s = ops[i]->op_param().top(0);
+    const int next = next_reader(ops, s, i);
+    if (next < 0 || taken[next] || !is_relu(*ops[next])) continue;
+    // in place the Scale output is the group's output and every later reader sees the
+    // activated values either way; elsewhere it is no longer written
+    if (ops[next]->op_param().top(0) != s && !sole_reader(ops, out_blob, s, i, next)) continue;
+    std::vector<int> members = {i, next};
+    if (!movable(ops, members)) continue;
+    groups.emplace_back(new ScaleRelu(ops, i, next));
+    taken[i] = taken[next] = true;
   }
   for (int i = 0; i < count; ++i) {
     if (taken[i] || !is_plain_eltwise(*ops[i])) continue;

@@ -228,6 +228,20 @@ def batch_norm(x, mean, variance, channel, inner_num, scale_factor, eps, inplace
     return y.download(count=x.size)
 
 
+def batch_norm_scale(x, mean, variance, channel, inner_num, scale_factor, eps, scale, bias, relu, inplace=False):
+    """BatchNorm -> Scale [-> ReLU] in one launch; scale or bias may be None."""
+    x = _f(x).ravel()
+    dx, dm, dv = Buffer.from_numpy(x), Buffer.from_numpy(_f(mean)), Buffer.from_numpy(_f(variance))
+    ds = Buffer.from_numpy(_f(scale)) if scale is not None else None
+    db = Buffer.from_numpy(_f(bias)) if bias is not None else None
+    y = dx if inplace else Buffer(max(4, x.nbytes))
+    check(_lib().shdw_hip_batch_norm_scale(x.size, channel, inner_num, dx.ptr, dm.ptr, dv.ptr, scale_factor, eps,
+                                           ds.ptr if ds else None, db.ptr if db else None, 1 if relu else 0,
+                                           y.ptr, None))
+    _sync()
+    return y.download(count=x.size)
+
+
 def _shifted(x, offset, inplace, n_out=None):
     """x on the device `offset` floats into its buffer, and the output buffer likewise."""
     dx = Buffer(max(4, x.nbytes) + 4 * offset)

@@ -1,5 +1,6 @@
-"""The Native backend's fusion pass: Scale -> Activate(relu) and
-Scale -> Eltwise(SUM) -> Activate(relu) [-> Reduce(AVG)] run as one launch.
+"""The Native backend's fusion pass: Scale -> Activate(relu),
+Scale -> Eltwise(SUM) -> Activate(relu) [-> Reduce(AVG)], Eltwise -> Activate(relu) and
+BatchNorm -> Scale [-> Activate(relu)] run as one launch each.
 Every network here runs three ways: fused (the default), with fuse=False, and
 through oracle.net.run (the operators one by one on the CPU).  The blobs a fused
 run still writes must carry the same bits as the unfused run's, and the oracle's
@@ -261,3 +262,96 @@ def test_full_size_bottleneck_tail_through_the_network(gpu):
         nw.forward(feed)
         assert_bit_exact(nw.blob("e"), e, "e")
         assert_bit_exact(nw.blob("pool"), pool, "pool")
+
+
+# ---- BatchNorm -> Scale [-> ReLU] -------------------------------------------------------------------------------
+def bn_net(ops, out, shape=SHAPE, factor=False, scale_param_shape=None, params=("gamma", "beta")):
+    """mean, var [, factor], then the Scale parameters as declared blobs, in that order."""
+    c = shape[1]
+    blobs = [("mean", "float", [c]), ("var", "float", [c])] + ([("factor", "float", [1])] if factor else [])
+    blobs += [(p, "float", list(scale_param_shape or [c])) for p in params]
+    return {"name": "fusion", "arg": [("out_blob", "v_s", list(out))], "blob": blobs,
+            "op": [op("Input", "in", [], ["x"], ("x", "v_i", list(shape)))] + list(ops)}
+
+
+def bn_data(shape=SHAPE, factor=None, scale_param_shape=None, seed=40):
+    c = shape[1]
+    pshape = tuple(scale_param_shape or [c])
+    weights = [normal(seed, c), uniform(seed + 1, c, 0.0, 30.0)] + ([np.array([factor], F)] if factor is not None else [])
+    weights += [uniform(seed + 2, pshape, 0.5, 1.5), normal(seed + 3, pshape, 0.3)]
+    return weights, {"x": with_specials(normal(seed + 4, shape, 2.0), seed).reshape(shape)}
+
+
+def bn_op(bottom, top, factor=False):
+    return op("BatchNorm", "bn", [bottom, "mean", "var"] + (["factor"] if factor else []), [top],
+              ("eps", "s_f", 1e-3))
+
+
+@pytest.mark.parametrize("in_place", [False, True])
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("factor", [None, 999.982, 0.0])
+def test_batch_norm_scale_relu(gpu, in_place, relu, factor):
+    """How a Caffe-style model holds a normalisation, in place (one blob name throughout) and not."""
+    n, s, y = ("x", "x", "x") if in_place else ("n", "s", "y")
+    ops = [bn_op("x", n, factor is not None), scale_op(n, s, name="sc")]
+    if relu:
+        ops.append(op("Activate", "relu", [s], [y], arg_i("type", 1)))
+    last = y if relu else s
+    ops.append(op("Unary", "neg", [last], ["out"], arg_i("operation", 13)))
+    net = bn_net(ops, ["out"], factor=factor is not None)
+    weights, feed = bn_data(factor=factor)
+    want = "bn(BatchNorm) + sc(Scale)" + (" + relu(Activate)" if relu else "") + " -> " + last
+    run_all(net, weights, feed, [last, "out"], expect_fused=[want])
+
+
+@pytest.mark.parametrize("has_scale,has_bias", [(True, False), (False, True)])
+def test_batch_norm_scale_with_one_parameter_blob(gpu, has_scale, has_bias):
+    net = bn_net([bn_op("x", "n"), scale_op("n", "s", has_scale, has_bias, name="sc"),
+                  op("Activate", "relu", ["s"], ["s"], arg_i("type", 1))], ["s"],
+                 params=["gamma"] if has_scale else ["beta"])
+    weights, feed = bn_data()
+    weights = weights[:2] + [w for w, keep in zip(weights[2:], (has_scale, has_bias)) if keep]
+    run_all(net, weights, feed, ["s"], expect_fused=["bn(BatchNorm) + sc(Scale) + relu(Activate) -> s"])
+
+
+def test_batch_norm_scale_on_long_rows_and_on_single_positions(gpu):
+    for shape in ((2, 4, 6, 64), (5, 9, 1, 1), (3, 7, 1, 3)):
+        net = bn_net([bn_op("x", "x"), scale_op("x", "x", name="sc"), op("Activate", "relu", ["x"], ["x"], arg_i("type", 1))],
+                     ["x"], shape=shape)
+        weights, feed = bn_data(shape)
+        run_all(net, weights, feed, ["x"], expect_fused=["bn(BatchNorm) + sc(Scale) + relu(Activate) -> x"])
+
+
+def test_batch_norm_scale_falls_back_where_the_parameters_are_not_one_per_channel(gpu):
+    """Scale parameters over two axes: the group exists (shapes are not known when the network is
+    built), declines at run time, and the operators run one by one."""
+    shape = (2, 4, 6, 8)
+    net = bn_net([bn_op("x", "n"), scale_op("n", "s", name="sc")], ["s"], shape=shape, scale_param_shape=[4, 6])
+    weights, feed = bn_data(shape, scale_param_shape=[4, 6])
+    run_all(net, weights, feed, ["s"], expect_fused=["bn(BatchNorm) + sc(Scale) -> s"])
+
+
+def test_batch_norm_output_with_another_reader_is_not_fused(gpu):
+    net = bn_net([bn_op("x", "n"), scale_op("n", "s", name="sc"), op("Activate", "relu", ["s"], ["y"], arg_i("type", 1)),
+                  op("Unary", "neg", ["n"], ["out"], arg_i("operation", 13))], ["y", "out"])
+    weights, feed = bn_data()
+    # the normalised blob is read again: BatchNorm stays; Scale -> ReLU still goes together
+    run_all(net, weights, feed, ["n", "y", "out"], expect_fused=["sc(Scale) + relu(Activate) -> y"])
+
+
+def test_batch_norm_in_front_of_a_residual_tail_leaves_the_scale_to_the_tail(gpu):
+    ops = [bn_op("x", "n"), scale_op("n", "s", name="sc"),
+           op("Eltwise", "add", ["s", "x"], ["e"], arg_i("operation", 1)),
+           op("Activate", "relu", ["e"], ["e"], arg_i("type", 1))]
+    net = bn_net(ops, ["e"])
+    weights, feed = bn_data()
+    run_all(net, weights, feed, ["n", "e"], expect_fused=["sc(Scale) + add(Eltwise) + relu(Activate) -> e"])
+
+
+def test_batch_norm_scale_in_front_of_a_sum_without_relu(gpu):
+    """No tail to leave the Scale to: it goes with its BatchNorm."""
+    ops = [bn_op("x", "n"), scale_op("n", "s", name="sc"),
+           op("Eltwise", "add", ["s", "x"], ["e"], arg_i("operation", 1))]
+    net = bn_net(ops, ["e"])
+    weights, feed = bn_data()
+    run_all(net, weights, feed, ["s", "e"], expect_fused=["bn(BatchNorm) + sc(Scale) -> s"])

@@ -74,6 +74,28 @@ def test_batch_norm(gpu, shape, sf):
     assert_bit_exact(gpuops.batch_norm(x, mean, var, c, inner, sf, 1e-5, inplace=True), want, "in place")
 
 
+@pytest.mark.parametrize("shape", [(2, 3, 4, 4), (4, 64, 7, 7), (3, 5, 9, 11), (2, 7, 1, 1), (1, 130, 28, 28),
+                                   (5, 9, 1, 2), (3, 7, 1, 3), (2, 5, 1, 7), (3, 1001, 1, 1)])
+@pytest.mark.parametrize("form", ["scale", "bias", "both"])
+@pytest.mark.parametrize("relu", [False, True])
+def test_batch_norm_scale_in_one_launch(gpu, shape, form, relu):
+    """BatchNorm -> Scale [-> ReLU] fused equals the oracle's operators one after the other, bit for bit."""
+    x = with_specials(normal(13, shape, 3.0), 13)
+    c, inner = shape[1], int(np.prod(shape[2:]))
+    mean, var = normal(14, c), uniform(15, c, -0.5, 900.0)
+    scale = uniform(16, c, 0.5, 1.5) if form != "bias" else None
+    bias = uniform(17, c, -0.3, 0.3) if form != "scale" else None
+    for sf in (1.0, 0.0010000181):
+        want = oracle.batch_norm(x, mean, var, c, inner, sf, 1e-5)
+        want = oracle.scale_bias(want, scale, bias, c, inner)
+        if relu:
+            want = oracle.activate(want, 1)
+        got = gpuops.batch_norm_scale(x, mean, var, c, inner, sf, 1e-5, scale, bias, relu)
+        assert_bit_exact(got, want, "batch_norm + scale")
+        got = gpuops.batch_norm_scale(x, mean, var, c, inner, sf, 1e-5, scale, bias, relu, inplace=True)
+        assert_bit_exact(got, want, "in place")
+
+
 def test_batch_norm_op(ws):
     x = normal(10, (3, 12, 6, 5), 2.0)
     mean, var = normal(11, 12), uniform(12, 12, 0.1, 5.0)
