@@ -897,6 +897,11 @@ def config_table(dev, sets_scale=1, cpu=None):
                  cpu.reduce(4, hy, sh5, ax5, hm)]
         tail_cpu = lambda: [f() for f in chain]
     add(5, "fused_tail (CPU: the four operators)", 8 * n5 + 8 * C5, 4 * n5 + 4 * 65536, ms, n5, cpu and tail_cpu)
+    # the same tail with its BatchNorm in front, as a Caffe-style model holds it (g5 > 0 serves as the variances)
+    ms = time_median(dev, lambda k: lib.shdw_hip_batch_norm_scale_residual_relu(
+        n5, C5, in5, A[k].ptr, b5.ptr, g5.ptr, 1.0, 1e-5, g5.ptr, b5.ptr, A[(k + 1) % SETS].ptr, 0, Y[k].ptr,
+        M[k].ptr, st), SETS)
+    add("next", "batch_norm + fused_tail [64,1024,14,14]", 8 * n5 + 16 * C5, 4 * n5 + 4 * 65536, ms, n5)
 
     sh7 = [128, 2048, 7, 7]  # the same reduction over 7 x 7 planes: rows of 49 floats start on odd dwords
     M7 = [dev.buf(nbytes=4 * 128 * 2048) for _ in range(SETS)]

@@ -276,6 +276,22 @@ int shdw_hip_scale_residual_relu(int n, int scale_num, int inner_num, const floa
                                  const float* scale, const float* bias, const float* residual,
                                  int residual_first, float* y, float* mean, void* stream);
 
+/* The same sequence with a BatchNorm (global statistics) in front of the Scale,
+ * how a Caffe-style model holds a bottleneck's last normalisation:
+ *   c = row % channel;
+ *   t = (x - stat_mean[c]*scale_factor) / sqrt(|stat_variance[c]*scale_factor| + eps);
+ *   s = t*scale[c] + bias[c];  y and mean as above.
+ * stat_mean, stat_variance, scale and bias hold `channel` values each (scale or
+ * bias may be NULL, not both); every step is rounded as in the five operators.
+ * ref: shadow/operators/kernels/batch_norm.cpp:11-24, batch_norm.cu:9-34 and
+ *      the references of shdw_hip_scale_residual_relu */
+int shdw_hip_batch_norm_scale_residual_relu(int n, int channel, int inner_num, const float* x,
+                                            const float* stat_mean, const float* stat_variance,
+                                            float scale_factor, float eps, const float* scale,
+                                            const float* bias, const float* residual,
+                                            int residual_first, float* y, float* mean,
+                                            void* stream);
+
 /* ==================== neighbouring operators of the path ==================== */
 
 /* Axpy: out[r*inner_num + i] = y[..] + alpha[r] * x[..] for r < outer_num

@@ -7,10 +7,10 @@
 // (shadow/backends/native/native.cpp:139-190), so a converted model runs as it is.
 //
 //   Scale(blob parameters) -> Activate(relu)                          one launch
-//   Scale(blob parameters) -> Eltwise(SUM of 2, unit coefficients)
+//   [BatchNorm(global statistics) ->] Scale(blob parameters) -> Eltwise(SUM of 2, unit coefficients)
 //                          -> Activate(relu) [-> Reduce(AVG over the trailing axes)]
-//   Eltwise(any operation, any number of inputs) -> Activate(relu)
 //   BatchNorm(global statistics) -> Scale(blob parameters, one per channel) [-> Activate(relu)]
+//   Eltwise(any operation, any number of inputs) -> Activate(relu)
 //
 // A blob that a group no longer writes (the Scale output, the Eltwise output when
 // the Activate is not in place) must have the next member as its only reader and

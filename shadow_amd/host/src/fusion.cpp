@@ -51,6 +51,13 @@ int next_reader(const OpList& ops, const std::string& blob, int producer) {
   return -1;
 }
 
+// The operator in front of `reader` that wrote `blob` last, or -1.
+int last_writer(const OpList& ops, const std::string& blob, int reader) {
+  for (int j = reader - 1; j >= 0; --j)
+    if (writes(*ops[j], blob)) return j;
+  return -1;
+}
+
 // The members run together where the last one stood.  That is the order of the
 // file as long as no operator between them writes a blob the members read or
 // write, or reads a blob they write.
@@ -137,6 +144,51 @@ bool view_scale(const Operator& op, Workspace* ws, ScaleView* v, const std::shar
   return v->num > 0 && v->inner > 0;
 }
 
+// BatchNorm on stored statistics (shadow/operators/batch_norm_op.cpp:7-47): how a
+// Caffe-style model holds a normalisation, the learned affine pair in the Scale
+// behind it.
+bool is_stats_batch_norm(const Operator& op) {
+  return op.type() == "BatchNorm" && op.op_param().top_size() == 1 &&
+         (op.op_param().bottom_size() == 3 || op.op_param().bottom_size() == 4);
+}
+
+// The BatchNorm member's view of its input: one mean and one variance per channel
+// (axis 1), the factor the optional fourth input carries, eps.
+struct NormView {
+  std::shared_ptr<Blob> x, mean, variance;
+  int channel = 0;
+  float scale_factor = 1, eps = 1e-5f;
+};
+
+bool view_batch_norm(const Operator& op, Workspace* ws, NormView* v) {
+  const auto& p = op.op_param();
+  v->x = float_blob(ws, p.bottom(0));
+  v->mean = float_blob(ws, p.bottom(1));
+  v->variance = float_blob(ws, p.bottom(2));
+  if (v->x == nullptr || v->mean == nullptr || v->variance == nullptr) return false;
+  if (v->x->num_axes() < 2 || v->x->count() == 0) return false;
+  v->channel = v->x->shape(1);
+  if (v->mean->count() != v->channel || v->variance->count() != v->channel) return false;
+  if (p.bottom_size() == 4) {
+    auto factor = float_blob(ws, p.bottom(3));
+    if (factor == nullptr || factor->count() != 1) return false;
+    float value = 1;
+    factor->get_data<float>(&value, 1);  // synchronous device -> host read, as the operator does
+    v->scale_factor = value == 0 ? 0 : 1 / value;
+  }
+  v->eps = op.get_single_argument<float>("eps", 1e-5);
+  return true;
+}
+
+// The Scale behind a BatchNorm must work on the same channels: axis 1, one
+// parameter per channel.
+bool view_scale_per_channel(const Operator& scale, Workspace* ws, const NormView& n, ScaleView* v) {
+  if (!view_scale(scale, ws, v, n.x)) return false;
+  int axis = scale.get_single_argument<int>("axis", 1);
+  if (axis < 0) axis += n.x->num_axes();
+  return axis == 1 && v->num == n.channel && v->inner == n.x->count(2);
+}
+
 std::string label(const Operator& op) { return op.name() + "(" + op.type() + ")"; }
 
 // ---- Scale -> Activate(relu): shdw_hip_scale_bias with its relu epilogue ----
@@ -167,12 +219,17 @@ class ScaleRelu : public FusedGroup {
   std::shared_ptr<Operator> scale_, relu_;
 };
 
-// ---- Scale -> Eltwise(SUM) -> Activate(relu) [-> Reduce(AVG)]: shdw_hip_scale_residual_relu ----
+// ---- [BatchNorm ->] Scale -> Eltwise(SUM) -> Activate(relu) [-> Reduce(AVG)]:
+//      shdw_hip_scale_residual_relu, shdw_hip_batch_norm_scale_residual_relu ----
 class ResidualTail : public FusedGroup {
  public:
-  ResidualTail(const OpList& ops, int scale, int sum, int relu, int mean)
+  ResidualTail(const OpList& ops, int bn, int scale, int sum, int relu, int mean)
       : scale_(ops[scale]), sum_(ops[sum]), relu_(ops[relu]) {
-    members_ = {scale, sum, relu};
+    if (bn >= 0) {
+      bn_ = ops[bn];
+      members_.push_back(bn);
+    }
+    members_.insert(members_.end(), {scale, sum, relu});
     if (mean >= 0) {
       mean_ = ops[mean];
       members_.push_back(mean);
@@ -182,15 +239,22 @@ class ResidualTail : public FusedGroup {
 
   bool Run(Workspace* ws) override {
     ScaleView v;
-    if (!view_scale(*scale_, ws, &v)) return false;
+    NormView n;
+    if (bn_ != nullptr) {
+      if (!view_batch_norm(*bn_, ws, &n) || !view_scale_per_channel(*scale_, ws, n, &v)) return false;
+    } else if (!view_scale(*scale_, ws, &v)) {
+      return false;
+    }
     auto r = float_blob(ws, sum_->op_param().bottom(residual_first_ ? 0 : 1));
     auto y = float_blob(ws, relu_->op_param().top(0));
     if (r == nullptr || y == nullptr || r->shape() != v.x->shape()) return false;
+    if (y == v.scale || y == v.bias || y == n.mean || y == n.variance) return false;
     std::shared_ptr<Blob> mean;
     VecInt mean_shape, squeezed;
     if (mean_ != nullptr) {
       mean = float_blob(ws, mean_->op_param().top(0));
       if (mean == nullptr || mean == y || mean == v.x || mean == r) return false;
+      if (mean == v.scale || mean == v.bias || mean == n.mean || mean == n.variance) return false;
       // the reduced axes must be exactly the run one parameter applies to
       const int rank = v.x->num_axes();
       VecInt axes = mean_->get_repeated_argument<int>("axes");
@@ -212,17 +276,26 @@ class ResidualTail : public FusedGroup {
     }
     y->reshape(v.x->shape());
     if (mean != nullptr) mean->reshape(mean_shape);
-    SHADOW_HIP_CHECK(shdw_hip_scale_residual_relu(
-        v.x->count(), v.num, v.inner, v.x->data<float>(), v.scale ? v.scale->data<float>() : nullptr,
-        v.bias ? v.bias->data<float>() : nullptr, r->data<float>(), residual_first_ ? 1 : 0,
-        y->mutable_data<float>(), mean != nullptr ? mean->mutable_data<float>() : nullptr,
-        ws->Ctx()->stream()));
+    const float* scale = v.scale ? v.scale->data<float>() : nullptr;
+    const float* bias = v.bias ? v.bias->data<float>() : nullptr;
+    float* mean_data = mean != nullptr ? mean->mutable_data<float>() : nullptr;
+    if (bn_ != nullptr) {
+      SHADOW_HIP_CHECK(shdw_hip_batch_norm_scale_residual_relu(
+          v.x->count(), n.channel, v.inner, v.x->data<float>(), n.mean->data<float>(), n.variance->data<float>(),
+          n.scale_factor, n.eps, scale, bias, r->data<float>(), residual_first_ ? 1 : 0, y->mutable_data<float>(),
+          mean_data, ws->Ctx()->stream()));
+    } else {
+      SHADOW_HIP_CHECK(shdw_hip_scale_residual_relu(v.x->count(), v.num, v.inner, v.x->data<float>(), scale, bias,
+                                                    r->data<float>(), residual_first_ ? 1 : 0,
+                                                    y->mutable_data<float>(), mean_data, ws->Ctx()->stream()));
+    }
     if (mean != nullptr && !mean_->get_single_argument<bool>("keep_dims", true)) mean->set_shape(squeezed);
     return true;
   }
 
   std::string describe() const override {
     std::string text = label(*scale_) + " + " + label(*sum_) + " + " + label(*relu_);
+    if (bn_ != nullptr) text = label(*bn_) + " + " + text;
     if (mean_ != nullptr) text += " + " + label(*mean_);
     text += " -> " + relu_->op_param().top(0);
     if (mean_ != nullptr) text += ", " + mean_->op_param().top(0);
@@ -230,19 +303,11 @@ class ResidualTail : public FusedGroup {
   }
 
  private:
-  std::shared_ptr<Operator> scale_, sum_, relu_, mean_;
+  std::shared_ptr<Operator> bn_, scale_, sum_, relu_, mean_;
   bool residual_first_ = false;
 };
 
 // ---- BatchNorm -> Scale [-> Activate(relu)]: shdw_hip_batch_norm_scale ----
-// How a Caffe-style model holds a normalisation: statistics in one operator, the
-// learned affine pair in the next (shadow/operators/batch_norm_op.cpp:7-47,
-// scale_op.cpp:7-52).
-bool is_stats_batch_norm(const Operator& op) {
-  return op.type() == "BatchNorm" && op.op_param().top_size() == 1 &&
-         (op.op_param().bottom_size() == 3 || op.op_param().bottom_size() == 4);
-}
-
 class BatchNormScale : public FusedGroup {
  public:
   BatchNormScale(const OpList& ops, int bn, int scale, int relu) : bn_(ops[bn]), scale_(ops[scale]) {
@@ -254,33 +319,16 @@ class BatchNormScale : public FusedGroup {
   }
 
   bool Run(Workspace* ws) override {
-    const auto& p = bn_->op_param();
-    auto x = float_blob(ws, p.bottom(0));
-    auto mean = float_blob(ws, p.bottom(1)), variance = float_blob(ws, p.bottom(2));
-    if (x == nullptr || mean == nullptr || variance == nullptr || x->num_axes() < 2 || x->count() == 0) return false;
-    const int channel = x->shape(1);
-    if (mean->count() != channel || variance->count() != channel) return false;
-    // the affine pair must be one value per channel: Scale over axis 1 with parameters of that one extent
+    NormView n;
     ScaleView v;
-    if (!view_scale(*scale_, ws, &v, x)) return false;
-    int axis = scale_->get_single_argument<int>("axis", 1);
-    if (axis < 0) axis += x->num_axes();
-    if (axis != 1 || v.num != channel || v.inner != x->count(2)) return false;
-    float scale_factor = 1;
-    if (p.bottom_size() == 4) {
-      auto factor = float_blob(ws, p.bottom(3));
-      if (factor == nullptr || factor->count() != 1) return false;
-      float value = 1;
-      factor->get_data<float>(&value, 1);  // synchronous device -> host read, as the operator does
-      scale_factor = value == 0 ? 0 : 1 / value;
-    }
+    if (!view_batch_norm(*bn_, ws, &n) || !view_scale_per_channel(*scale_, ws, n, &v)) return false;
     const auto& last = relu_ != nullptr ? relu_ : scale_;
     auto y = float_blob(ws, last->op_param().top(0));
-    if (y == nullptr || y == mean || y == variance || y == v.scale || y == v.bias) return false;
-    y->reshape(x->shape());
+    if (y == nullptr || y == n.mean || y == n.variance || y == v.scale || y == v.bias) return false;
+    y->reshape(n.x->shape());
     SHADOW_HIP_CHECK(shdw_hip_batch_norm_scale(
-        x->count(), channel, v.inner, x->data<float>(), mean->data<float>(), variance->data<float>(), scale_factor,
-        bn_->get_single_argument<float>("eps", 1e-5), v.scale ? v.scale->data<float>() : nullptr,
+        n.x->count(), n.channel, v.inner, n.x->data<float>(), n.mean->data<float>(), n.variance->data<float>(),
+        n.scale_factor, n.eps, v.scale ? v.scale->data<float>() : nullptr,
         v.bias ? v.bias->data<float>() : nullptr, relu_ != nullptr ? 1 : 0, y->mutable_data<float>(),
         ws->Ctx()->stream()));
     return true;
@@ -357,8 +405,8 @@ std::vector<std::unique_ptr<FusedGroup>> FindFusedGroups(const OpList& ops,
   std::vector<std::unique_ptr<FusedGroup>> groups;
   std::vector<bool> taken(ops.size(), false);
   const int count = static_cast<int>(ops.size());
-  // Residual tails first: a Scale whose output goes into a sum saves as much there as behind
-  // its BatchNorm, and the tail can take the mean along.
+  // Residual tails first: a Scale whose output goes into a sum belongs there, with the BatchNorm
+  // in front of it where there is one, and the tail can take the mean along.
   for (int i = 0; i < count; ++i) {
     if (taken[i] || !is_blob_scale(*ops[i])) continue;
     const std::string& s = ops[i]->op_param().top(0);
@@ -384,8 +432,20 @@ std::vector<std::unique_ptr<FusedGroup>> FindFusedGroups(const OpList& ops,
       }
       if (writes(*ops[j], y)) break;
     }
-    groups.emplace_back(new ResidualTail(ops, i, next, relu, mean));
+    // a BatchNorm whose output only this Scale reads comes along
+    int bn = last_writer(ops, ops[i]->op_param().bottom(0), i);
+    if (bn >= 0) {
+      const auto& sp = ops[i]->op_param();
+      const std::string& n = sp.bottom(0);
+      bool ok = !taken[bn] && is_stats_batch_norm(*ops[bn]) && sole_reader(ops, out_blob, n, bn, i);
+      for (int k = 1; k < sp.bottom_size(); ++k) ok = ok && sp.bottom(k) != n;
+      std::vector<int> with_bn = {bn, i, next, relu};
+      if (mean >= 0) with_bn.push_back(mean);
+      if (!ok || !movable(ops, with_bn)) bn = -1;
+    }
+    groups.emplace_back(new ResidualTail(ops, bn, i, next, relu, mean));
     taken[i] = taken[next] = taken[relu] = true;
+    if (bn >= 0) taken[bn] = true;
     if (mean >= 0) taken[mean] = true;
   }
   // BatchNorm -> Scale [-> ReLU] next: it takes the Scale -> ReLU pair with it.

@@ -209,6 +209,25 @@ def scale_residual_relu(x, scale, bias, res, scale_num, inner_num, residual_firs
     return (y.download(count=n) if y else None), (mean.download(count=rows) if mean else None)
 
 
+def batch_norm_scale_residual_relu(x, stat_mean, stat_variance, scale_factor, eps, scale, bias, res, channel, inner_num,
+                                   residual_first=False, want_y=True, want_mean=True):
+    """shdw_hip_batch_norm_scale_residual_relu: scale or bias may be None, either output may be left out."""
+    x, res = _f(x).ravel(), _f(res).ravel()
+    n = x.size
+    dx, dr = Buffer.from_numpy(x), Buffer.from_numpy(res)
+    dm, dv = Buffer.from_numpy(_f(stat_mean)), Buffer.from_numpy(_f(stat_variance))
+    ds = Buffer.from_numpy(_f(scale)) if scale is not None else None
+    db = Buffer.from_numpy(_f(bias)) if bias is not None else None
+    y = Buffer(4 * n) if want_y else None
+    rows = n // inner_num
+    mean = Buffer(4 * rows) if want_mean else None
+    check(_lib().shdw_hip_batch_norm_scale_residual_relu(
+        n, channel, inner_num, dx.ptr, dm.ptr, dv.ptr, float(scale_factor), float(eps), ds.ptr if ds else None,
+        db.ptr if db else None, dr.ptr, int(residual_first), y.ptr if y else None, mean.ptr if mean else None, None))
+    _sync()
+    return (y.download(count=n) if y else None), (mean.download(count=rows) if mean else None)
+
+
 def axpy_rows(alpha, x, y, inner_num, inplace=False):
     alpha, x, y = _f(alpha).ravel(), _f(x).ravel(), _f(y).ravel()
     da, dx, dy = Buffer.from_numpy(alpha), Buffer.from_numpy(x), Buffer.from_numpy(y)

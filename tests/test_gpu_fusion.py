@@ -339,13 +339,52 @@ def test_batch_norm_output_with_another_reader_is_not_fused(gpu):
     run_all(net, weights, feed, ["n", "y", "out"], expect_fused=["sc(Scale) + relu(Activate) -> y"])
 
 
-def test_batch_norm_in_front_of_a_residual_tail_leaves_the_scale_to_the_tail(gpu):
-    ops = [bn_op("x", "n"), scale_op("n", "s", name="sc"),
-           op("Eltwise", "add", ["s", "x"], ["e"], arg_i("operation", 1)),
+@pytest.mark.parametrize("shape", [SHAPE, (2, 8, 4, 8), (5, 3, 1, 1)])
+@pytest.mark.parametrize("residual_first", [False, True])
+@pytest.mark.parametrize("factor", [None, 999.982])
+def test_batch_norm_in_front_of_a_residual_tail_goes_with_it(gpu, shape, residual_first, factor):
+    """The last normalisation of a Caffe-style bottleneck: BatchNorm -> Scale -> Eltwise -> ReLU -> mean."""
+    ops = [bn_op("x", "n", factor is not None), scale_op("n", "s", name="sc"),
+           op("Eltwise", "add", ["r", "s"] if residual_first else ["s", "r"], ["e"], arg_i("operation", 1)),
+           op("Activate", "relu", ["e"], ["e"], arg_i("type", 1)),
+           op("Reduce", "gap", ["e"], ["pool"], arg_i("operation", 4), ("axes", "v_i", [2, 3]))]
+    net = bn_net(ops, ["e", "pool"], shape=shape, factor=factor is not None)
+    net["op"][0] = op("Input", "in", [], ["x", "r"], ("x", "v_i", list(shape)), ("r", "v_i", list(shape)))
+    weights, feed = bn_data(shape, factor=factor)
+    feed = {"x": normal(51, shape, 2.0), "r": normal(52, shape)}
+    run_all(net, weights, feed, ["e", "pool"], fp64=("pool",),
+            expect_fused=["bn(BatchNorm) + sc(Scale) + add(Eltwise) + relu(Activate) + gap(Reduce) -> e, pool"])
+
+
+def test_batch_norm_in_front_of_a_residual_tail_in_place_and_with_special_values(gpu):
+    """One blob name from the BatchNorm to the Scale, as Caffe writes it; the residual is the block's input."""
+    ops = [op("Unary", "branch", ["x"], ["t"], arg_i("operation", 13)),
+           bn_op("t", "t"), scale_op("t", "t", name="sc"),
+           op("Eltwise", "add", ["x", "t"], ["e"], arg_i("operation", 1)),
            op("Activate", "relu", ["e"], ["e"], arg_i("type", 1))]
     net = bn_net(ops, ["e"])
     weights, feed = bn_data()
-    run_all(net, weights, feed, ["n", "e"], expect_fused=["sc(Scale) + add(Eltwise) + relu(Activate) -> e"])
+    run_all(net, weights, feed, ["e"], expect_fused=["bn(BatchNorm) + sc(Scale) + add(Eltwise) + relu(Activate) -> e"])
+
+
+def test_batch_norm_whose_output_is_read_again_stays_out_of_the_tail(gpu):
+    ops = [bn_op("x", "n"), scale_op("n", "s", name="sc"),
+           op("Eltwise", "add", ["s", "x"], ["e"], arg_i("operation", 1)),
+           op("Activate", "relu", ["e"], ["e"], arg_i("type", 1)),
+           op("Unary", "neg", ["n"], ["out"], arg_i("operation", 13))]
+    net = bn_net(ops, ["e", "out"])
+    weights, feed = bn_data()
+    run_all(net, weights, feed, ["n", "e", "out"], expect_fused=["sc(Scale) + add(Eltwise) + relu(Activate) -> e"])
+
+
+def test_tail_behind_a_batch_norm_falls_back_where_the_scale_is_not_per_channel(gpu):
+    shape = (2, 4, 6, 8)
+    ops = [bn_op("x", "n"), scale_op("n", "s", name="sc"),
+           op("Eltwise", "add", ["s", "x"], ["e"], arg_i("operation", 1)),
+           op("Activate", "relu", ["e"], ["e"], arg_i("type", 1))]
+    net = bn_net(ops, ["e"], shape=shape, scale_param_shape=[4, 6])
+    weights, feed = bn_data(shape, scale_param_shape=[4, 6])
+    run_all(net, weights, feed, ["e"], expect_fused=["bn(BatchNorm) + sc(Scale) + add(Eltwise) + relu(Activate) -> e"])
 
 
 def test_batch_norm_scale_in_front_of_a_sum_without_relu(gpu):

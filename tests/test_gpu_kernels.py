@@ -467,6 +467,39 @@ def test_fused_tail_forms(gpu, form, residual_first, outer, num, inner):
     assert assert_rel_close(m, want_m, 1e-5, "mean") == 0
 
 
+@pytest.mark.parametrize("form", ["scale", "bias", "both"])
+@pytest.mark.parametrize("residual_first", [False, True])
+@pytest.mark.parametrize("outer,num,inner", [(2, 8, 196), (3, 5, 7), (2, 3, 1030), (101, 4, 12)])
+def test_fused_tail_behind_a_batch_norm(gpu, form, residual_first, outer, num, inner):
+    """BatchNorm -> Scale -> Eltwise SUM -> ReLU [-> Reduce AVG] against the five operators of the oracle."""
+    n = outer * num * inner
+    stat_mean, stat_var = normal(181, num), uniform(182, num, 0.0, 30.0)
+    s = uniform(176, num, 0.5, 1.5) if form != "bias" else None
+    b = uniform(177, num, -0.1, 0.1) if form != "scale" else None
+    factor, eps = np.float32(1 / 999.982), np.float32(1e-3)
+
+    def five(x, r):
+        t = oracle.batch_norm(x, stat_mean, stat_var, num, inner, factor, eps)
+        t = oracle.scale_bias(t, s, b, num, inner)
+        return oracle.activate(oracle.eltwise(1, [r, t] if residual_first else [t, r], [1.0, 1.0]), 1)
+
+    x, r = with_specials(normal(174, n), 3), with_specials(normal(175, n), 4)
+    y, none = gpuops.batch_norm_scale_residual_relu(x, stat_mean, stat_var, factor, eps, s, b, r, num, inner,
+                                                    residual_first, want_mean=False)
+    assert none is None
+    assert_bit_exact(y, five(x, r), "y")
+    x, r = normal(174, n), normal(175, n)  # finite values for the mean
+    y2, m = gpuops.batch_norm_scale_residual_relu(x, stat_mean, stat_var, factor, eps, s, b, r, num, inner, residual_first)
+    clean = five(x, r)
+    assert_bit_exact(y2, clean, "y with the mean")
+    want_m, _ = oracle.reduce(4, clean, [outer * num, inner], [1])
+    assert assert_rel_close(m, want_m, 1e-5, "mean") == 0
+    none, m2 = gpuops.batch_norm_scale_residual_relu(x, stat_mean, stat_var, factor, eps, s, b, r, num, inner,
+                                                     residual_first, want_y=False)
+    assert none is None
+    assert_bit_exact(m2, m, "mean without y")
+
+
 def test_argument_errors(gpu):
     import shadow_amd
     lib = gpu
@@ -488,3 +521,7 @@ def test_argument_errors(gpu):
     assert lib.shdw_hip_scale_residual_relu(16, 2, 8, p, p, p, None, 0, p, p, None) == -1     # no residual
     assert lib.shdw_hip_scale_residual_relu(15, 2, 8, p, p, p, p, 0, p, p, None) == -1        # not whole rows
     assert lib.shdw_hip_scale_residual_relu_rowmean(16, 2, 8, p, p, None, p, p, p, None) == -1
+    assert lib.shdw_hip_batch_norm_scale_residual_relu(16, 2, 8, p, None, p, 1.0, 1e-5, p, p, p, 0, p, p, None) == -1
+    assert lib.shdw_hip_batch_norm_scale_residual_relu(16, 2, 8, p, p, None, 1.0, 1e-5, p, p, p, 0, p, p, None) == -1
+    assert lib.shdw_hip_batch_norm_scale_residual_relu(16, 2, 8, p, p, p, 1.0, 1e-5, None, None, p, 0, p, p, None) == -1
+    assert lib.shdw_hip_batch_norm_scale_residual_relu(15, 2, 8, p, p, p, 1.0, 1e-5, p, p, p, 0, p, p, None) == -1
