@@ -1139,9 +1139,11 @@ def network_forward(dev, reps=50):
     return out
 
 
-def tail_text(copies):
+def tail_text(copies, batch_norm=False):
     """BASELINE configs[4] as a converted model holds it, `copies` times side by side on
-    blobs of their own, so that one run walks over more than the 256 MB Infinity Cache."""
+    blobs of their own, so that one run walks over more than the 256 MB Infinity Cache.
+    batch_norm: a BatchNorm on stored statistics in front of every Scale, as a Caffe-style
+    model holds the normalisation."""
     shape = "64 # 1024 # 14 # 14"
     names = ["x%d" % k for k in range(copies)] + ["r%d" % k for k in range(copies)]
     lines = ["[bottleneck_tails]", "[{out_blob, v_s, [%s]}]" % " # ".join("pool%d" % k for k in range(copies)),
@@ -1149,8 +1151,10 @@ def tail_text(copies):
              "[Input] | [in] | [0 %d %d] | [] | [%s] | [%s]" % (
                  len(names), len(names), "; ".join(names), "; ".join("{%s, v_i, [%s]}" % (nm, shape) for nm in names))]
     for k in range(copies):
-        lines += ["[Scale] | [bn%d] | [3 1 3] | [x%d; gamma; beta] | [s%d] | [{axis, s_i, [1]}; {has_scale, s_i, [1]}; "
-                  "{has_bias, s_i, [1]}]" % (k, k, k),
+        if batch_norm:  # beta as the means, gamma (0.5 ... 1.5) as the variances
+            lines += ["[BatchNorm] | [norm%d] | [3 1 1] | [x%d; beta; gamma] | [n%d] | [{eps, s_f, [0.001]}]" % (k, k, k)]
+        lines += ["[Scale] | [bn%d] | [3 1 3] | [%s%d; gamma; beta] | [s%d] | [{axis, s_i, [1]}; {has_scale, s_i, [1]}; "
+                  "{has_bias, s_i, [1]}]" % (k, "n" if batch_norm else "x", k, k),
                   "[Eltwise] | [add%d] | [2 1 1] | [s%d; r%d] | [e%d] | [{operation, s_i, [1]}]" % (k, k, k, k),
                   "[Activate] | [relu%d] | [1 1 1] | [e%d] | [e%d] | [{type, s_i, [1]}]" % (k, k, k),
                   "[Reduce] | [gap%d] | [1 1 2] | [e%d] | [pool%d] | [{operation, s_i, [4]}; {axes, v_i, [2 # 3]}]" % (
@@ -1158,11 +1162,12 @@ def tail_text(copies):
     return "\n".join(lines) + "\n"
 
 
-def network_tail(dev, copies=6, reps=20):
+def network_tail(dev, copies=6, reps=20, batch_norm=False):
     """Device time of the bottleneck tail (Scale -> Eltwise SUM -> ReLU -> Reduce AVG on
     [64,1024,14,14]) run by the Native backend from a model text, per tail: events on the
     backend's stream around `reps` runs of a network that holds `copies` such tails on
-    separate blobs, nothing waited for in between.  Fused: one launch per tail."""
+    separate blobs, nothing waited for in between.  Fused: one launch per tail.
+    batch_norm: the tail with a BatchNorm in front of its Scale (five operators)."""
     sa, lib = dev.sa, dev.lib
     n = 64 * 1024 * 14 * 14
     src = [dev.buf(normal(811 + k, n)) for k in range(2)]
@@ -1170,9 +1175,10 @@ def network_tail(dev, copies=6, reps=20):
     feed = {}
     for k in range(copies):
         feed["x%d" % k], feed["r%d" % k] = src[k & 1], src[(k + 1) & 1]
-    out = {"model": "%d x (Scale -> Eltwise SUM -> ReLU -> Reduce AVG{2,3}) on [64,1024,14,14]" % copies}
+    out = {"model": "%d x (%sScale -> Eltwise SUM -> ReLU -> Reduce AVG{2,3}) on [64,1024,14,14]" % (
+        copies, "BatchNorm -> " if batch_norm else "")}
     for fuse, key in ((True, "us_per_tail"), (False, "us_per_tail_unfused")):
-        with sa.Network(tail_text(copies), weights, device_input=True, fuse=fuse) as net:
+        with sa.Network(tail_text(copies, batch_norm), weights, device_input=True, fuse=fuse) as net:
             net.forward(feed)
             st = net.stream
             e0, e1 = dev.event(), dev.event()
@@ -1187,7 +1193,7 @@ def network_tail(dev, copies=6, reps=20):
                 ms = dev.elapsed_ms(e0, e1) / (reps * copies)
                 best = ms if best is None else min(best, ms)
             out[key] = round(best * 1e3, 2)
-            out["launches_per_tail" if fuse else "launches_per_tail_unfused"] = 1 if net.fused else 4
+            out["launches_per_tail" if fuse else "launches_per_tail_unfused"] = 1 if net.fused else 4 + batch_norm
     for b in src:
         b.free()
     return out
@@ -1224,8 +1230,9 @@ def final_record(full, table_path=None):
         rec["worst_of_ceiling"] = [worst["cfg"], SHORT_OP.get(worst["op"], worst["op"]), worst["frac_of_ceiling"]]
     if "network" in full:
         rec["network"] = {k: v for k, v in full["network"].items() if k not in ("model", "fused")}
-    if "network_tail" in full:
-        rec["network_tail"] = {k: v for k, v in full["network_tail"].items() if k != "model"}
+    for key in ("network_tail", "network_bn_tail"):
+        if key in full:
+            rec[key] = {k: v for k, v in full[key].items() if k != "model"}
     if table_path:
         rec["table"] = table_path
     return rec
@@ -1235,7 +1242,8 @@ def final_line(full, table_path=None):
     """final_record as one line of JSON below FINAL_LINE_LIMIT.  Should a host with a long
     device or CPU name push it over, the optional tables go first (they are in the file)."""
     rec = final_record(full, table_path)
-    for optional in (None, "step_ops", "baseline_rows", "baseline_rows_columns", "network", "network_tail"):
+    for optional in (None, "step_ops", "baseline_rows", "baseline_rows_columns", "network", "network_bn_tail",
+                     "network_tail"):
         rec.pop(optional, None)
         line = json.dumps(rec, separators=(",", ":"))
         if len(line) < FINAL_LINE_LIMIT:
@@ -1313,6 +1321,7 @@ def main():
                                "host, one thread, outputs allocated beforehand, best of %d" % args.cpu_passes)
         out["network"] = network_forward(dev)
         out["network_tail"] = network_tail(dev)
+        out["network_bn_tail"] = network_tail(dev, batch_norm=True)
     table = write_table(out, args.table)
     for r in out.get("configs", []):
         print("%-8s %-62s %9.2f us  %.3f of 8 TB/s%s" % (r["cfg"], r["op"], r["us"], r["frac"],
