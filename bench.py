@@ -974,6 +974,9 @@ def config_table(dev, sets_scale=1, cpu=None):
     ms = time_median(dev, lambda k: lib.shdw_hip_batch_norm_scale(NH, CH, INH, AH[k].ptr, meanh.ptr, varh.ptr, 1.0, 1e-5,
                                                                   varh.ptr, meanh.ptr, 1, YH[k].ptr, st), SH, reps=20)
     add("next", "batch_norm_scale_relu [64,256,56,56]", 4 * NH + 16 * CH, 4 * NH, ms, NH)
+    ms = time_median(dev, lambda k: lib.shdw_hip_lrn(I([64, CH, 56, 56]), 5, 1e-4, 0.75, 1.0, AH[k].ptr, YH[k].ptr, st),
+                     SH, reps=20)
+    add("next", "lrn across 5 channels [64,256,56,56]", 4 * NH, 4 * NH, ms, NH)
     alh = dev.buf(uniform(613, 64 * CH, 0.0, 1.0))
     ms = time_median(dev, lambda k: lib.shdw_hip_axpy_rows(64 * CH, INH, alh.ptr, AH[k].ptr,
                                                            AH[(k + 1) % SH].ptr, YH[k].ptr, st), SH, reps=20)

@@ -326,6 +326,17 @@ int shdw_hip_batch_norm_scale(int n, int channel, int inner_num, const float* x,
                               const float* scale, const float* bias, int relu, float* y,
                               void* stream);
 
+/* LRN across channels on a 4-D tensor [batch][channels][h][w]: per position a running
+ * fp32 sum of the squares of `size` neighbouring channels (the entering square is
+ * added, then the leaving one subtracted, channel after channel),
+ *   scale = k + sum * (alpha / size);   y = x * powf(scale, -beta).
+ * The reference's scale blob (a temp blob of the input's size) is not needed.
+ * size must be odd; channels >= (size - 1) / 2 (with fewer the reference writes in
+ * front of that blob); size > 63 returns SHDW_E_UNSUPPORTED.  y may alias x.
+ * ref: shadow/operators/kernels/lrn.cpp:9-60, lrn.hpp:36-46, lrn.cu */
+int shdw_hip_lrn(const int* in_shape, int size, float alpha, float beta, float k, const float* x,
+                 float* y, void* stream);
+
 /* Softmax over the middle extent of x viewed as [outer_num][dim][inner_num]:
  * running maximum, exp(x - max), fp32 running sum in index order, divide.  The
  * per-column scratch blob of the reference is not needed.  y may alias x.

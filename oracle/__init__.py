@@ -188,6 +188,15 @@ def batch_norm(x, mean, variance, channel, inner_num, scale_factor, eps):
     return out
 
 
+def lrn(x, in_shape, size, alpha, beta, k):
+    """(out, scale): Vision::LRN and the scale blob it leaves (k + alpha / size * windowed sum of squares)."""
+    x = _f(x).ravel()
+    out, scale = np.empty_like(x), np.empty_like(x)
+    lib().orc_lrn(_p(x), _ints(in_shape), int(size), ctypes.c_float(alpha), ctypes.c_float(beta), ctypes.c_float(k),
+                  _p(scale), _p(out))
+    return out, scale
+
+
 def softmax(x, outer, dim, inner):
     x = _f(x).ravel()
     out = np.empty_like(x)
@@ -381,6 +390,19 @@ def batch_norm_op(x, mean, variance, scale=None, eps=1e-5, use_global_stats=True
     _check(channel == np.size(variance), "channel == variance->count()")
     inner = int(np.prod(x.shape[2:], dtype=np.int64))
     return batch_norm(x, mean, variance, channel, inner, scale_factor, np.float32(eps)).reshape(x.shape)
+
+
+def lrn_op(x, local_size=5, alpha=1.0, beta=0.75, norm_region=0, k=1.0):
+    """shadow/operators/lrn_op.cpp:9-33 and kernels/lrn.hpp:36-46; the input must be 4-D (the kernel
+    reads in_shape[0..3]) with at least (local_size - 1) / 2 channels (fewer make the kernel's last
+    loop write in front of its scale blob)."""
+    _check(local_size % 2 == 1, "LRN only supports odd values for local_size")
+    _check(norm_region == 0, "Currently only support norm region method: Across Channels!")
+    x = _f(x)
+    _check(x.ndim == 4, "4-D input")
+    _check(x.shape[1] >= (local_size - 1) // 2, "in_c >= post_pad")
+    out, _ = lrn(x, x.shape, local_size, alpha, beta, k)
+    return out.reshape(x.shape)
 
 
 def _canonical(axis, ndim):

@@ -753,3 +753,42 @@ API void orc_resize_bilinear(const float* in, const int* in_shape, int align_cor
     }
   }
 }
+
+/* ---- shadow/operators/kernels/lrn.cpp:9-60  Vision::LRN across channels: per position
+ *      a running fp32 sum of squares over the channels (add the entering one, then
+ *      subtract the leaving one), scale = k + sum * (alpha / size), and a second pass
+ *      out = in * powf(scale, -beta).  in_c >= (size - 1) / 2 is assumed, as by the
+ *      reference (fewer channels make its third loop write in front of the buffer). ---- */
+API void orc_lrn(const float* in, const int* in_shape, int size, float alpha, float beta, float k,
+                 float* scale, float* out) {
+  int batch = in_shape[0], in_c = in_shape[1], in_h = in_shape[2], in_w = in_shape[3];
+  int step = in_h * in_w, count = batch * in_c * step;
+  int pre_pad = (size - 1) / 2, post_pad = size - pre_pad - 1;
+  float alpha_over_size = alpha / size;
+  for (int b = 0; b < batch; ++b) {
+    for (int h = 0; h < in_h; ++h) {
+      for (int w = 0; w < in_w; ++w) {
+        int offset = (b * in_c * in_h + h) * in_w + w, head = 0;
+        const float* in_off = in + offset;
+        float* scale_off = scale + offset;
+        float accum_scale = 0.f;
+        while (head < post_pad && head < in_c) {
+          accum_scale += in_off[head * step] * in_off[head * step];
+          head++;
+        }
+        while (head < in_c) {
+          accum_scale += in_off[head * step] * in_off[head * step];
+          if (head - size >= 0) accum_scale -= in_off[(head - size) * step] * in_off[(head - size) * step];
+          scale_off[(head - post_pad) * step] = k + accum_scale * alpha_over_size;
+          head++;
+        }
+        while (head < in_c + post_pad) {
+          if (head - size >= 0) accum_scale -= in_off[(head - size) * step] * in_off[(head - size) * step];
+          scale_off[(head - post_pad) * step] = k + accum_scale * alpha_over_size;
+          head++;
+        }
+      }
+    }
+  }
+  for (int i = 0; i < count; ++i) out[i] = in[i] * powf(scale[i], -beta);
+}

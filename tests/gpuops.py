@@ -228,6 +228,15 @@ def batch_norm_scale_residual_relu(x, stat_mean, stat_variance, scale_factor, ep
     return (y.download(count=n) if y else None), (mean.download(count=rows) if mean else None)
 
 
+def lrn(x, in_shape, size, alpha, beta, k, inplace=False):
+    x = _f(x).ravel()
+    dx = Buffer.from_numpy(x)
+    y = dx if inplace else Buffer(max(4, x.nbytes))
+    check(_lib().shdw_hip_lrn(ints(in_shape), int(size), float(alpha), float(beta), float(k), dx.ptr, y.ptr, None))
+    _sync()
+    return y.download(count=x.size)
+
+
 def axpy_rows(alpha, x, y, inner_num, inplace=False):
     alpha, x, y = _f(alpha).ravel(), _f(x).ravel(), _f(y).ravel()
     da, dx, dy = Buffer.from_numpy(alpha), Buffer.from_numpy(x), Buffer.from_numpy(y)

@@ -113,6 +113,59 @@ def test_batch_norm_op(ws):
         ws.create_op("BatchNorm", ["x", "mean"], ["o4"], {}).run()
 
 
+# -------------------------------------------------------------------- lrn ---
+@pytest.mark.parametrize("shape,size", [((2, 96, 55, 55), 5), ((1, 256, 27, 27), 5), ((2, 7, 3, 5), 5), ((1, 2, 4, 4), 5),
+                                        ((3, 16, 1, 1), 3), ((2, 6, 2, 3), 1), ((2, 5, 2, 2), 9), ((1, 40, 3, 3), 11),
+                                        ((3, 1, 17, 19), 3), ((1, 70, 5, 52), 63), ((300, 4, 1, 1), 3)])
+@pytest.mark.parametrize("alpha,beta,k", [(1e-4, 0.75, 1.0), (0.5, 2.0, 2.0)])
+def test_lrn(gpu, shape, size, alpha, beta, k):
+    """The running sum over the channels, its scale and the power, against the oracle's two passes."""
+    x = with_specials(normal(31, shape, 3.0), 31)
+    want, _ = oracle.lrn(x, shape, size, alpha, beta, k)
+    assert_bit_exact(gpuops.lrn(x, shape, size, alpha, beta, k), want, "lrn")
+    assert_bit_exact(gpuops.lrn(x, shape, size, alpha, beta, k, inplace=True), want, "in place")
+
+
+def test_lrn_scales_below_one_and_negative(gpu):
+    """k = 0 and a negative alpha: powf meets zeros, tiny and negative bases."""
+    shape = (2, 12, 5, 7)
+    x = normal(32, shape, 1e-3)
+    x[0, :, 0, 0] = 0
+    for alpha, k in ((1.0, 0.0), (-2.0, 1e-6), (1e30, 1.0)):
+        want, _ = oracle.lrn(x, shape, 5, alpha, 0.75, k)
+        assert_bit_exact(gpuops.lrn(x, shape, 5, alpha, 0.75, k), want, "lrn alpha %g k %g" % (alpha, k))
+
+
+def test_lrn_argument_errors(gpu):
+    lib = gpu
+    buf = shadow_amd.Buffer(4 * 2 * 3 * 4 * 4)
+    ints = shadow_amd.ints
+    sh = ints([2, 3, 4, 4])
+    assert lib.shdw_hip_lrn(sh, 4, 1.0, 0.75, 1.0, buf.ptr, buf.ptr, None) == -1   # even window
+    assert lib.shdw_hip_lrn(sh, 0, 1.0, 0.75, 1.0, buf.ptr, buf.ptr, None) == -1
+    assert lib.shdw_hip_lrn(sh, 9, 1.0, 0.75, 1.0, buf.ptr, buf.ptr, None) == -1   # four channels behind the centre, three there
+    assert lib.shdw_hip_lrn(sh, 5, 1.0, 0.75, 1.0, None, buf.ptr, None) == -1
+    assert lib.shdw_hip_lrn(ints([2, 80, 1, 1]), 65, 1.0, 0.75, 1.0, buf.ptr, buf.ptr, None) == -2  # window over 63
+    assert lib.shdw_hip_lrn(ints([2, 0, 4, 4]), 1, 1.0, 0.75, 1.0, None, None, None) == 0    # empty
+
+
+def test_lrn_op(ws):
+    x = normal(33, (2, 10, 6, 5), 2.0)
+    got = run(ws, "LRN", [("x", x)], {"local_size": 3, "alpha": 0.001, "beta": 0.75, "k": 2.0})
+    assert_bit_exact(got, oracle.lrn_op(x, 3, 0.001, 0.75, 0, 2.0), "lrn op")
+    got = run(ws, "LRN", [("x", x)], {})
+    assert_bit_exact(got, oracle.lrn_op(x), "lrn op, default arguments")
+    with pytest.raises(ShadowError, match="odd values"):
+        ws.create_op("LRN", ["x"], ["o2"], {"local_size": 4})
+    with pytest.raises(ShadowError, match="Across Channels"):
+        ws.create_op("LRN", ["x"], ["o3"], {"norm_region": 1})
+    ws.set_blob("flat", np.zeros((4, 6), F))
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("LRN", ["flat"], ["o4"], {}).run()
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("LRN", ["x"], ["o5"], {"local_size": 23}).run()
+
+
 # ---------------------------------------------------------------- softmax ---
 SOFTMAX_SHAPES = [  # outer, dim, inner: both layouts, LDS limits, odd sizes
     (1, 1, 1), (64, 1000, 1), (3, 10, 1), (5, 7, 3), (2, 21, 63), (2, 21, 64), (2, 21, 65),

@@ -359,3 +359,85 @@ def test_norm_known_values_and_checks():
         oracle.layer_norm_op(np.zeros((2, 3, 4), F), [])
     with pytest.raises(oracle.OracleCheckError):
         oracle.layer_norm_op(np.zeros((2, 3, 4), F), [4], scale=np.ones(4, F))
+
+
+# -------------------------------------------------------------------- lrn ---
+def lrn_by_planes(x, size, alpha, beta, k):
+    """The channel walk on whole [batch, h, w] planes at once: every step is one rounded fp32 numpy
+    operation, entering square added before the leaving one is subtracted."""
+    x = x.astype(F)
+    c_in, post = x.shape[1], (size - 1) // 2
+    sq = x * x
+    aos = F(alpha) / F(size)
+    accum = np.zeros(x[:, 0].shape, F)
+    scale = np.empty_like(x)
+    for head in range(c_in + post):
+        if head < c_in:
+            accum = accum + sq[:, head]
+        if head >= size:
+            accum = accum - sq[:, head - size]
+        if head >= post:
+            scale[:, head - post] = F(k) + accum * aos
+    power = oracle.binary(4, scale, np.full(scale.shape, -F(beta), F)).reshape(x.shape)  # the pinned powf
+    return x * power, scale
+
+
+@pytest.mark.parametrize("shape,size", [((2, 7, 3, 5), 5), ((1, 2, 4, 4), 5), ((3, 16, 1, 1), 3), ((2, 6, 2, 3), 1),
+                                        ((2, 5, 2, 2), 9), ((1, 40, 3, 3), 11)])
+@pytest.mark.parametrize("alpha,beta,k", [(1e-4, 0.75, 1.0), (1.0, 0.75, 1.0), (0.5, 2.0, 2.0)])
+def test_lrn_against_plane_formulation(shape, size, alpha, beta, k):
+    x = normal(61, shape, 3.0)
+    want, want_scale = lrn_by_planes(x, size, alpha, beta, k)
+    got, scale = oracle.lrn(x, shape, size, alpha, beta, k)
+    assert_bit_exact(scale.reshape(shape), want_scale, "lrn scale")
+    assert_bit_exact(got.reshape(shape), want, "lrn")
+    assert_bit_exact(oracle.lrn_op(x, size, alpha, beta, 0, k), want, "lrn op")
+
+
+def test_lrn_sum_is_a_running_one():
+    """The window sum formed afresh for every channel rounds differently from add-then-subtract."""
+    shape, size = (4, 64, 5, 5), 5
+    x = normal(62, shape, 3.0)
+    _, scale = oracle.lrn(x, shape, size, 1.0, 0.75, 1.0)
+    sq = (x * x).astype(F)
+    fresh = np.empty_like(x)
+    for c in range(shape[1]):
+        lo, hi = max(0, c - 2), min(shape[1], c + 3)
+        fresh[:, c] = F(1) + running_sum(sq[:, lo:hi], 1, F) * (F(1) / F(size))
+    assert (bits(fresh) != bits(scale.reshape(shape))).any()
+    assert np.allclose(fresh, scale.reshape(shape), rtol=1e-5)
+
+
+def test_lrn_exact_data_and_known_values():
+    # small integers and alpha / size a power of two: every operation is exact, one right answer
+    shape, size = (2, 9, 3, 3), 5
+    x = (np.arange(np.prod(shape)) % 7 - 3).astype(F).reshape(shape)
+    _, scale = oracle.lrn(x, shape, size, 5 * 2.0 ** -3, 0.75, 1.0)
+    sq = x.astype(np.float64) ** 2
+    want = np.empty(shape)
+    for c in range(shape[1]):
+        want[:, c] = 1.0 + sq[:, max(0, c - 2):c + 3].sum(1) * 2.0 ** -3
+    assert_bit_exact(scale.reshape(shape), want.astype(F), "exact scale")
+    # two channels of ones, window 3, alpha / size = 1, k = 2: both scales are 4
+    ones = np.ones((1, 2, 1, 1), F)
+    assert_bit_exact(oracle.lrn_op(ones, 3, 3.0, 1.0, 0, 2.0), np.full((1, 2, 1, 1), 0.25, F), "4^-1")
+    assert_bit_exact(oracle.lrn_op(ones, 3, 3.0, 0.5, 0, 2.0), np.full((1, 2, 1, 1), 0.5, F), "4^-1/2")
+    x = normal(63, (2, 4, 3, 3))
+    assert_bit_exact(oracle.lrn_op(x, 3, 1.0, 0.0, 0, 1.0), x, "beta 0")
+    # a window of one channel: scale = k + x^2 * alpha in the first channel; further on the sum is
+    # (previous + entering) - previous, which need not be the entering square again
+    got, scale = oracle.lrn(x, x.shape, 1, 0.5, 0.75, 1.0)
+    assert_bit_exact(scale.reshape(x.shape)[:, 0], F(1) + (x * x)[:, 0] * F(0.5), "window of one")
+
+
+def test_lrn_op_checks():
+    x = np.zeros((2, 3, 4, 4), F)
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.lrn_op(x, 4)
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.lrn_op(x, 5, norm_region=1)
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.lrn_op(np.zeros((2, 3, 4), F), 5)
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.lrn_op(x, 9)  # three channels, four behind the centre
+    oracle.lrn_op(x, 7)
