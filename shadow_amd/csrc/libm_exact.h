@@ -847,12 +847,78 @@ SHDW_LIBM_FN int powf_checkint(uint32_t iy) {
 SHDW_LIBM_FN bool powf_zeroinfnan(uint32_t ix) { return 2 * ix - 1 >= 2u * 0x7f800000u - 1; }
 SHDW_LIBM_FN bool powf_issignaling(uint32_t ix) { return 2 * (ix ^ 0x00400000u) > 2u * 0x7fc00000u; }
 
+// Whether powf(x, y) takes the straight path below: x a positive normal number,
+// y finite and not zero.
+SHDW_LIBM_FN bool powf_is_ordinary(uint32_t ix, uint32_t iy) {
+  return !(ix - 0x00800000u >= 0x7f800000u - 0x00800000u || powf_zeroinfnan(iy));
+}
+
+// x^y for the bits ix of a positive normal x and a finite y != 0 (the caller has
+// scaled a subnormal x up and moved the sign of a negative base to an odd power
+// into sign_bias).  No branches: results that overflow or underflow are put in
+// place at the end, so several of these can run side by side in one lane; any
+// other ix and y give some number and no fault.
+// log_tab is kPowfLog2Tab or a copy of it in faster memory, as tab is of kExp2fTab.
+SHDW_LIBM_FN float powf_ordinary(uint32_t ix, float y, uint32_t sign_bias, const uint64_t* tab,
+                                 const PowfLog2Entry* log_tab) {
+  // log2(x)
+  const double A0 = 0x1.27616c9496e0bp-2, A1 = -0x1.71969a075c67ap-2, A2 = 0x1.ec70a6ca7baddp-2,
+               A3 = -0x1.7154748bef6c8p-1, A4 = 0x1.71547652ab82bp0;
+  const uint32_t tmp = ix - 0x3f330000u;
+  const int i = (tmp >> 19) & 15;
+  const uint32_t top = tmp & 0xff800000u;
+  const uint32_t iz = ix - top;
+  const int k = static_cast<int32_t>(top) >> 23;
+  const double invc = log_tab[i].invc, logc = log_tab[i].logc;
+  const double z = static_cast<double>(u2f(iz));
+  const double r = __builtin_fma(z, invc, -1.0);
+  const double y0 = logc + static_cast<double>(k);
+  const double r2 = r * r;
+  double yy = __builtin_fma(A0, r, A1);
+  const double p = __builtin_fma(A2, r, A3);
+  const double r4 = r2 * r2;
+  double q = __builtin_fma(A4, r, y0);
+  q = __builtin_fma(p, r2, q);
+  const double logx = __builtin_fma(yy, r4, q);
+  const double ylogx = static_cast<double>(y) * logx;
+  // 2^(y log2 x)
+  const double C0 = 0x1.c6af84b912394p-5, C1 = 0x1.ebfce50fac4f3p-3, C2 = 0x1.62e42ff0c52d6p-1;
+  const double Shift = 0x1.8p+52 / 32;
+  double kd = ylogx + Shift;
+  const uint64_t ki = d2u(kd);
+  kd -= Shift;
+  const double rr = ylogx - kd;
+  uint64_t t = tab[ki & 31];
+  const uint64_t ski = ki + sign_bias;
+  t += ski << 47;
+  const double sc = u2d(t);
+  const double zz = __builtin_fma(C0, rr, C1);
+  const double rr2 = rr * rr;
+  double res = __builtin_fma(C2, rr, 1.0);
+  res = __builtin_fma(zz, rr2, res);
+  res = res * sc;
+  float out = static_cast<float>(res);
+  // |y log2 x| >= 126: past the largest float, below half the smallest, or the smallest itself
+  const bool far = (d2u(ylogx) >> 47 & 0xffff) >= (d2u(126.0) >> 47);
+  const bool over = far && ylogx > 0x1.fffffffd1d571p+6;
+  const bool under = far && !over && ylogx <= -150.0;
+  const bool least = far && !over && !under && ylogx < -149.0;
+  out = over ? (sign_bias ? -__builtin_inff() : __builtin_inff()) : out;
+  out = under ? (sign_bias ? -0.0f : 0.0f) : out;
+  out = least ? (sign_bias ? -0x1p-149f : 0x1p-149f) : out;
+  return out;
+}
+
+SHDW_LIBM_FN float powf_ordinary(uint32_t ix, float y, uint32_t sign_bias, const uint64_t* tab) {
+  return powf_ordinary(ix, y, sign_bias, tab, kPowfLog2Tab);
+}
+
 SHDW_LIBM_FN float exact_powf(float x, float y, const uint64_t* tab) {
   const uint32_t kSignBias = 1u << (5 + 11);
   uint32_t sign_bias = 0;
   uint32_t ix = f2u(x);
   const uint32_t iy = f2u(y);
-  if (ix - 0x00800000u >= 0x7f800000u - 0x00800000u || powf_zeroinfnan(iy)) {
+  if (!powf_is_ordinary(ix, iy)) {
     if (powf_zeroinfnan(iy)) {
       if (2 * iy == 0) return powf_issignaling(ix) ? x + y : 1.0f;
       if (ix == 0x3f800000u) return powf_issignaling(iy) ? x + y : 1.0f;
@@ -882,48 +948,7 @@ SHDW_LIBM_FN float exact_powf(float x, float y, const uint64_t* tab) {
       ix -= 23u << 23;
     }
   }
-  // log2(x)
-  const double A0 = 0x1.27616c9496e0bp-2, A1 = -0x1.71969a075c67ap-2, A2 = 0x1.ec70a6ca7baddp-2,
-               A3 = -0x1.7154748bef6c8p-1, A4 = 0x1.71547652ab82bp0;
-  const uint32_t tmp = ix - 0x3f330000u;
-  const int i = (tmp >> 19) & 15;
-  const uint32_t top = tmp & 0xff800000u;
-  const uint32_t iz = ix - top;
-  const int k = static_cast<int32_t>(top) >> 23;
-  const double invc = kPowfLog2Tab[i].invc, logc = kPowfLog2Tab[i].logc;
-  const double z = static_cast<double>(u2f(iz));
-  const double r = __builtin_fma(z, invc, -1.0);
-  const double y0 = logc + static_cast<double>(k);
-  const double r2 = r * r;
-  double yy = __builtin_fma(A0, r, A1);
-  const double p = __builtin_fma(A2, r, A3);
-  const double r4 = r2 * r2;
-  double q = __builtin_fma(A4, r, y0);
-  q = __builtin_fma(p, r2, q);
-  const double logx = __builtin_fma(yy, r4, q);
-  const double ylogx = static_cast<double>(y) * logx;
-  if ((d2u(ylogx) >> 47 & 0xffff) >= (d2u(126.0) >> 47)) {  // |y log2 x| >= 126
-    if (ylogx > 0x1.fffffffd1d571p+6) return sign_bias ? -__builtin_inff() : __builtin_inff();
-    if (ylogx <= -150.0) return sign_bias ? -0.0f : 0.0f;
-    if (ylogx < -149.0) return sign_bias ? -0x1p-149f : 0x1p-149f;
-  }
-  // 2^(y log2 x)
-  const double C0 = 0x1.c6af84b912394p-5, C1 = 0x1.ebfce50fac4f3p-3, C2 = 0x1.62e42ff0c52d6p-1;
-  const double Shift = 0x1.8p+52 / 32;
-  double kd = ylogx + Shift;
-  const uint64_t ki = d2u(kd);
-  kd -= Shift;
-  const double rr = ylogx - kd;
-  uint64_t t = tab[ki & 31];
-  const uint64_t ski = ki + sign_bias;
-  t += ski << 47;
-  const double sc = u2d(t);
-  const double zz = __builtin_fma(C0, rr, C1);
-  const double rr2 = rr * rr;
-  double res = __builtin_fma(C2, rr, 1.0);
-  res = __builtin_fma(zz, rr2, res);
-  res = res * sc;
-  return static_cast<float>(res);
+  return powf_ordinary(ix, y, sign_bias, tab);
 }
 #if !defined(__HIPCC__)
 SHDW_LIBM_FN float exact_softplusf(float x) { return exact_softplusf(x, kExp2fTab); }

@@ -6,12 +6,13 @@
 // scratch blob, and multiplies x by powf(scale, -beta) in a second pass.  The
 // order of the additions and subtractions fixes the bits, so the walk stays: one
 // lane per position, channel after channel.  What goes is the scratch blob and
-// the second pass: the window's values wait in LDS (a column of `size` floats per
-// lane, no two lanes share a bank row), the centre of the window is multiplied as
-// soon as its scale is known, x is read once and y written once.  Neighbouring
+// the second pass: the window's values wait in registers (windows of up to seven
+// channels) or in LDS (a column of `size` floats per lane, no two lanes share a
+// bank row), the centre of the window is multiplied as soon as its scale is
+// known, x is read once and y written once.  Neighbouring
 // lanes hold neighbouring positions, so every load and store of a wave is one run
-// of 256 bytes.  y may be x: a lane has read every channel it still needs before
-// it writes the one behind them.
+// of 256 bytes.  y may be x: a lane has read every channel of a round, and all
+// before it, when it writes the channels the round finishes, which lie behind them.
 #include <hip/hip_runtime.h>
 
 #include <climits>
@@ -25,13 +26,139 @@
 
 namespace shdw {
 
-// Windows of up to 63 channels: 63 KB of LDS for the 256 lanes of a workgroup.
+// Windows of up to 63 channels: 63 KB of LDS for the 256 lanes of a workgroup, beside the tables.
 constexpr int kLrnMaxSize = 63;
 
+// Channels a lane takes per round: their loads go out together, the sum walks
+// through them one by one, and only then come the powers, which do not depend on
+// one another -- eight of them side by side, in their branch-free form, hide the
+// latency of their table look-ups and fp64 chains, which the walk itself cannot
+// (one power per step of the walk: 378 us on [64,256,56,56]; in rounds: 236 us).
+constexpr uint32_t kLrnRound = 8;
+
+// powf(scale, y) for the scales of a round.  The straight path for all of them (any
+// bits may go in, see powf_ordinary); then, if some lane holds a scale that is not a
+// positive normal number, the whole function for those, one instance of its code.
+// The two tables of powf in LDS: read from there, the powers leave the vector
+// memory counter alone, so that waiting for a table entry is not waiting for the
+// next round's channels, which were asked for before it.
+struct LrnTables {
+  uint64_t exp2[32];
+  libm::PowfLog2Entry log2[16];
+};
+
+// All lanes of the workgroup, before any of them leaves.
+SHDW_DEVICE void lrn_stage_tables(LrnTables* t) {
+  if (threadIdx.x < 32) t->exp2[threadIdx.x] = libm::kExp2fTab[threadIdx.x];
+  if (threadIdx.x < 16) t->log2[threadIdx.x] = libm::kPowfLog2Tab[threadIdx.x];
+  __syncthreads();
+}
+
+SHDW_DEVICE void lrn_powers(const float (&scale)[kLrnRound], float y, const LrnTables* t,
+                            float (&power)[kLrnRound]) {
+  bool plain = true;
+#pragma unroll
+  for (uint32_t j = 0; j < kLrnRound; ++j) {
+    power[j] = libm::powf_ordinary(__float_as_uint(scale[j]), y, 0u, t->exp2, t->log2);
+    plain = plain && libm::powf_is_ordinary(__float_as_uint(scale[j]), __float_as_uint(y));
+  }
+  if (__builtin_amdgcn_ballot_w64(!plain) == 0) return;
+#pragma unroll 1
+  for (uint32_t pick = 0; pick < kLrnRound; ++pick) {
+    float s = scale[0];
+#pragma unroll
+    for (uint32_t j = 1; j < kLrnRound; ++j) s = pick == j ? scale[j] : s;
+    if (libm::powf_is_ordinary(__float_as_uint(s), __float_as_uint(y))) continue;
+    const float r = libm::exact_powf(s, y, libm::kExp2fTab);
+#pragma unroll
+    for (uint32_t j = 0; j < kLrnRound; ++j) power[j] = pick == j ? r : power[j];
+  }
+}
+
+// ---- windows of 1, 3, 5 and 7 channels: the window lives in registers ----
+// prev[t] is channel head0 - SIZE + t, the last SIZE channels of the round before.
+// EDGE: the first round and those that reach past the last channel, with the tests
+// of the reference's three loops; the rounds between them need none.
+// The channels of the round that starts at head0 (zeros past the last one).
+SHDW_DEVICE void lrn_fetch(const float* in, uint32_t head0, uint32_t channels, uint32_t step,
+                           float (&values)[kLrnRound]) {
+#pragma unroll
+  for (uint32_t j = 0; j < kLrnRound; ++j)
+    values[j] = head0 + j < channels ? in[static_cast<size_t>(head0 + j) * step] : 0.f;
+}
+
+// `round` holds the channels of this round on entry and those of the next on
+// return: they are asked for before the powers and arrive while those are worked
+// out.  (The channels this round writes lie behind all of them, y may be x.)
+template <int SIZE, bool EDGE>
+SHDW_DEVICE void lrn_round(const float* in, float* out, uint32_t head0, uint32_t channels, uint32_t step,
+                           float (&round)[kLrnRound], float (&prev)[SIZE], float& accum, float alpha_over_size,
+                           float neg_beta, float k, const LrnTables* tables) {
+  static_assert(SIZE % 2 == 1 && SIZE <= static_cast<int>(kLrnRound), "the window must fit into a round");
+  constexpr uint32_t post = (SIZE - 1) / 2;
+  const uint32_t steps = channels + post;  // step `head` takes channel head in and finishes channel head - post
+  float entering[kLrnRound], scale[kLrnRound], centre[kLrnRound], power[kLrnRound];
+#pragma unroll
+  for (uint32_t j = 0; j < kLrnRound; ++j) entering[j] = round[j];
+  lrn_fetch(in, head0 + kLrnRound, channels, step, round);
+#pragma unroll
+  for (uint32_t j = 0; j < kLrnRound; ++j) {
+    const uint32_t head = head0 + j;  // the same for every lane, and so is every test on it
+    scale[j] = 1.f;
+    centre[j] = 0.f;
+    if (!EDGE || head < channels) accum += entering[j] * entering[j];
+    if (!EDGE || (head >= SIZE && head < steps)) {
+      const float leaving = j >= SIZE ? entering[j >= SIZE ? j - SIZE : 0] : prev[j < SIZE ? j : 0];
+      accum -= leaving * leaving;
+    }
+    if (!EDGE || (head >= post && head < steps)) {
+      scale[j] = k + accum * alpha_over_size;
+      centre[j] = j >= post ? entering[j >= post ? j - post : 0] : prev[j < post ? SIZE - post + j : 0];
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < SIZE; ++t) prev[t] = entering[kLrnRound - SIZE + t];
+  lrn_powers(scale, neg_beta, tables, power);
+#pragma unroll
+  for (uint32_t j = 0; j < kLrnRound; ++j) {
+    const uint32_t head = head0 + j;
+    if (!EDGE || (head >= post && head < steps)) out[static_cast<size_t>(head - post) * step] = centre[j] * power[j];
+  }
+}
+
+template <int SIZE>
+__global__ __launch_bounds__(kBlock) void lrn_window_kernel(const float* x, float* y, uint32_t positions,
+                                                            uint32_t step, uint32_t channels, FastDiv f_step,
+                                                            float alpha_over_size, float neg_beta, float k) {
+  __shared__ LrnTables tables;
+  lrn_stage_tables(&tables);
+  const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+  if (p >= positions) return;
+  const uint32_t b = fd_div(p, f_step);
+  const size_t base = static_cast<size_t>(b) * channels * step + (p - b * step);
+  const float* in = x + base;
+  float* out = y + base;
+  float prev[SIZE], round[kLrnRound];
+#pragma unroll
+  for (int t = 0; t < SIZE; ++t) prev[t] = 0.f;
+  float accum = 0.f;
+  const uint32_t steps = channels + (SIZE - 1) / 2;
+  lrn_fetch(in, 0, channels, step, round);
+  for (uint32_t head0 = 0; head0 < steps; head0 += kLrnRound) {
+    if (head0 >= SIZE && head0 + kLrnRound <= channels)
+      lrn_round<SIZE, false>(in, out, head0, channels, step, round, prev, accum, alpha_over_size, neg_beta, k, &tables);
+    else
+      lrn_round<SIZE, true>(in, out, head0, channels, step, round, prev, accum, alpha_over_size, neg_beta, k, &tables);
+  }
+}
+
+// ---- any window up to kLrnMaxSize channels: the window lives in LDS ----
 __global__ __launch_bounds__(kBlock) void lrn_across_channels_kernel(
     const float* x, float* y, uint32_t positions, uint32_t step, uint32_t channels, FastDiv f_step,
     uint32_t size, float alpha_over_size, float neg_beta, float k) {
   extern __shared__ float window[];  // [size][kBlock]
+  __shared__ LrnTables tables;
+  lrn_stage_tables(&tables);
   const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
   if (p >= positions) return;  // no barrier below: a lane only meets its own column
   const uint32_t b = fd_div(p, f_step);
@@ -40,24 +167,41 @@ __global__ __launch_bounds__(kBlock) void lrn_across_channels_kernel(
   float* out = y + base;
   float* mine = window + threadIdx.x;
   const uint32_t post = (size - 1) / 2;
+  const uint32_t steps = channels + post;  // step `head` takes channel head in and finishes channel head - post
   float accum = 0.f;
   uint32_t slot_head = 0, slot_mid = 0;  // head % size and (head - post) % size
-  float entering = in[0];
-  for (uint32_t head = 0; head < channels + post; ++head) {
-    const float v = entering;
-    if (head + 1 < channels) entering = in[static_cast<size_t>(head + 1) * step];  // on its way during the powf
-    if (head < channels) accum += v * v;
-    if (head >= size) {  // channel head - size lives where channel head goes
-      const float leaving = mine[slot_head * kBlock];
-      accum -= leaving * leaving;
+  float round[kLrnRound];
+  lrn_fetch(in, 0, channels, step, round);
+  for (uint32_t head0 = 0; head0 < steps; head0 += kLrnRound) {
+    float entering[kLrnRound], scale[kLrnRound], centre[kLrnRound], power[kLrnRound];
+#pragma unroll
+    for (uint32_t j = 0; j < kLrnRound; ++j) entering[j] = round[j];
+    lrn_fetch(in, head0 + kLrnRound, channels, step, round);  // the next round's, on their way during the powers
+#pragma unroll
+    for (uint32_t j = 0; j < kLrnRound; ++j) {
+      const uint32_t head = head0 + j;
+      scale[j] = 1.f;
+      centre[j] = 0.f;
+      if (head < steps) {  // the same for every lane
+        if (head < channels) accum += entering[j] * entering[j];
+        if (head >= size) {  // channel head - size lives where channel head goes
+          const float leaving = mine[slot_head * kBlock];
+          accum -= leaving * leaving;
+        }
+        if (head < channels) mine[slot_head * kBlock] = entering[j];
+        slot_head = slot_head + 1 == size ? 0 : slot_head + 1;
+        if (head >= post) {
+          scale[j] = k + accum * alpha_over_size;
+          centre[j] = mine[slot_mid * kBlock];
+          slot_mid = slot_mid + 1 == size ? 0 : slot_mid + 1;
+        }
+      }
     }
-    if (head < channels) mine[slot_head * kBlock] = v;
-    slot_head = slot_head + 1 == size ? 0 : slot_head + 1;
-    if (head >= post) {
-      const float scale = k + accum * alpha_over_size;
-      const float centre = mine[slot_mid * kBlock];
-      out[static_cast<size_t>(head - post) * step] = centre * libm::exact_powf(scale, neg_beta, libm::kExp2fTab);
-      slot_mid = slot_mid + 1 == size ? 0 : slot_mid + 1;
+    lrn_powers(scale, neg_beta, &tables, power);
+#pragma unroll
+    for (uint32_t j = 0; j < kLrnRound; ++j) {
+      const uint32_t head = head0 + j;
+      if (head >= post && head < steps) out[static_cast<size_t>(head - post) * step] = centre[j] * power[j];
     }
   }
 }
@@ -85,9 +229,23 @@ extern "C" int shdw_hip_lrn(const int* in_shape, int size, float alpha, float be
   const uint32_t step = static_cast<uint32_t>(in_shape[2]) * static_cast<uint32_t>(in_shape[3]);
   const uint32_t positions = static_cast<uint32_t>(in_shape[0]) * step;
   const float alpha_over_size = alpha / size;  // float / int, as the reference forms it
-  const size_t lds = static_cast<size_t>(size) * kBlock * sizeof(float);
-  lrn_across_channels_kernel<<<grid_for(positions), kBlock, lds, static_cast<hipStream_t>(stream)>>>(
-      x, y, positions, step, static_cast<uint32_t>(channels), make_fastdiv(step), static_cast<uint32_t>(size),
-      alpha_over_size, -beta, k);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint32_t grid = grid_for(positions), chan = static_cast<uint32_t>(channels);
+  const FastDiv f_step = make_fastdiv(step);
+#define SHDW_LRN(S) lrn_window_kernel<S><<<grid, kBlock, 0, st>>>(x, y, positions, step, chan, f_step, alpha_over_size, -beta, k)
+  if (size == 1) {
+    SHDW_LRN(1);
+  } else if (size == 3) {
+    SHDW_LRN(3);
+  } else if (size == 5) {
+    SHDW_LRN(5);
+  } else if (size == 7) {
+    SHDW_LRN(7);
+  } else {
+    const size_t lds = static_cast<size_t>(size) * kBlock * sizeof(float);
+    lrn_across_channels_kernel<<<grid, kBlock, lds, st>>>(x, y, positions, step, chan, f_step,
+                                                          static_cast<uint32_t>(size), alpha_over_size, -beta, k);
+  }
+#undef SHDW_LRN
   return launch_status();
 }
