@@ -1,4 +1,4 @@
-"""Pins for the oracle's Axpy / BatchNorm / Softmax / Normalize / Pooling
+"""Pins for the oracle's Axpy / BatchNorm / Softmax / Normalize / Pooling / LRN
 restatements.  The reference holds no vectors for these either, so each is
 checked against an independent numpy formulation (axis operations and slicing,
 never the oracle's flat pointer walks), against exactly representable data with
