@@ -53,6 +53,7 @@ def mixed_graph():
                op("BatchNorm", "bn", ["x", "mean", "var", "factor"], ["bn"], ("eps", "s_f", F(1e-3))),
                op("Pooling", "pool", ["bn"], ["p"], arg_i("pool", 0), ("kernel_size", "v_i", [3]), ("stride", "v_i", [2]),
                   ("pad", "v_i", [1]), arg_i("full_pooling", 0)),
+               op("LRN", "lrn", ["p"], ["lr"], arg_i("local_size", 3), ("alpha", "s_f", F(1e-2)), ("beta", "s_f", F(0.75))),
                op("Unary", "abs", ["p"], ["pa"], arg_i("operation", 0)),
                op("Unary", "sqrt", ["pa"], ["ps"], arg_i("operation", 2)),
                op("Reshape", "rs", ["ps"], ["r"], ("shape", "v_i", [0, -1, 6])),
@@ -115,7 +116,7 @@ def test_mixed_graph(gpu):
     want = onet.run(net, weights, inputs)
     with shadow_amd.Network(onet.write_text(net), weights, debug=True) as nw:
         nw.forward(inputs)
-        compare(nw, want, ["bn", "p", "ps", "r", "u", "s", "nz", "rmax", "ln", "ax", "inn", "ravg", "favg", "fmax",
+        compare(nw, want, ["bn", "p", "lr", "ps", "r", "u", "s", "nz", "rmax", "ln", "ax", "inn", "ravg", "favg", "fmax",
                            "fms", "out"])
         assert nw.blob_shape("r") == [3, 40, 6] and nw.blob_shape("u") == [3, 1, 40, 6]
 
