@@ -297,6 +297,8 @@ def probe_next(dev):
     for _ in range(3):
         dev.ck(lib.shdw_hip_copy(n, x.ptr, y.ptr, st))
         dev.ck(lib.shdw_hip_batch_norm(n, C, inner, x.ptr, b.ptr, g.ptr, 1.0, 1e-5, y.ptr, st))
+        dev.ck(lib.shdw_hip_batch_norm_scale(n, C, inner, x.ptr, b.ptr, g.ptr, 1.0, 1e-5, g.ptr, b.ptr, 1, y.ptr, st))
+        dev.ck(lib.shdw_hip_lrn(I([64, C, 56, 56]), 5, 1e-4, 0.75, 1.0, x.ptr, y.ptr, st))
         dev.ck(lib.shdw_hip_axpy_rows(64 * C, inner, alpha.ptr, x.ptr, x2.ptr, y.ptr, st))
         dev.ck(lib.shdw_hip_pooling2d(I(stem_in), 0, 3, 3, 2, 2, 0, 0, I(stem_out), x.ptr, y.ptr, st))
         dev.ck(lib.shdw_hip_pooling2d(I([512, 2048, 7, 7]), 1, 7, 7, 1, 1, 0, 0, I([512, 2048, 1, 1]), x.ptr,
