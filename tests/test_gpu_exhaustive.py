@@ -4,7 +4,8 @@ By default: ALL 2^32 float bit patterns for the functions whose device code
 differs from what the host sweep (tests/test_libm_exact_cpu.py) compiles -- tanh
 (its two divisions are a reciprocal plus one correction on the device), sigmoid
 (a wave-wide choice between that short division and the full one) -- and for
-exp, softplus and gelu, which the benchmark workloads and those two build on
+exp, softplus and gelu, which the benchmark workloads and those two build on,
+and for powf(x, -0.75), LRN's default power
 (about 12 s each: the oracle side runs on a thread pool).  The other ten run
 every 61st bit pattern plus 8k-wide windows around the branch points of the
 algorithms, the same set the host sweep uses; SHADOW_GPU_FULL_SWEEP=1 (or a
@@ -38,13 +39,18 @@ WANT = os.environ.get("SHADOW_GPU_FULL_SWEEP", "")
 CASES = {"log": ("unary", 3), "exp": ("unary", 4), "sin": ("unary", 5), "cos": ("unary", 6),
          "tan": ("unary", 7), "asin": ("unary", 8), "acos": ("unary", 9), "atan": ("unary", 10),
          "sqrt": ("unary", 2), "reciprocal": ("unary", 14), "sigmoid": ("act", 3), "softplus": ("act", 4),
-         "tanh": ("act", 5), "hardswish": ("act", 7), "gelu": ("act", 8)}
-ALWAYS_FULL = ("tanh", "sigmoid", "exp", "softplus", "gelu")
+         "tanh": ("act", 5), "hardswish": ("act", 7), "gelu": ("act", 8),
+         # powf(x, -0.75) through Binary's scalar form: the power LRN takes by default
+         "pow_minus_three_quarters": ("pow", -0.75)}
+ALWAYS_FULL = ("tanh", "sigmoid", "exp", "softplus", "gelu", "pow_minus_three_quarters")
+POW = 4  # shadow/operators/kernels/binary.hpp: kAdd, kSub, kMul, kDiv, kPow, kMax, kMin
 CHUNK = 1 << 26
 SLICE = 1 << 21
 
 
 def _oracle_slice(kind, code, x):
+    if kind == "pow":
+        return oracle.binary_scalar(POW, x, code)
     return oracle.unary(code, x) if kind == "unary" else oracle.activate(x, code)
 
 
@@ -52,7 +58,10 @@ def _compare(name, bits, pool):
     """Mismatches between the GPU and the oracle on the float32 values with these bit patterns."""
     kind, code = CASES[name]
     x = bits.view(np.float32)
-    got = gpuops.unary(code, x) if kind == "unary" else gpuops.activate(x, code)
+    if kind == "pow":
+        got = gpuops.binary_scalar(POW, x, code)
+    else:
+        got = gpuops.unary(code, x) if kind == "unary" else gpuops.activate(x, code)
     parts = [x[i:i + SLICE] for i in range(0, x.size, SLICE)]
     want = np.concatenate(list(pool.map(lambda p: _oracle_slice(kind, code, p), parts)))
     same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
