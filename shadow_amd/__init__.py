@@ -218,6 +218,7 @@ HOST_SIGNATURES = {
     "shdw_host_network_create": (_V, [ctypes.c_char_p, _I, _I, _I, _I, ctypes.c_char_p, _V]),
     "shdw_host_network_create_from_binary": (_V, [ctypes.c_char_p, _I, _I, _I, _I, _V, _I, _I]),
     "shdw_host_parse_net_binary": (_I, [_V, _I, _I, ctypes.c_char_p, _Z]),
+    "shdw_host_plan_fusion": (_I, [ctypes.c_char_p, ctypes.c_char_p, _Z]),
     "shdw_host_proto_reencode": (_I, [_V, _I, _I, _V, _Z]),
     "shdw_host_serialize_net": (_I, [ctypes.c_char_p, _V, _Z]),
     "shdw_host_proto_file_reencode": (_I, [ctypes.c_char_p, ctypes.c_char_p, _I]),
@@ -375,6 +376,17 @@ def parse_net(proto_text):
     n = lib.shdw_host_parse_net(proto_text.encode(), buf, len(buf))
     host_check(n >= 0)
     return buf.value.decode()
+
+
+def plan_fusion(proto_text):
+    """The groups the Native backend's fusion pass forms for a text model, as Network.fused
+    lists them once the model is loaded (host only)."""
+    lib = host()
+    buf = ctypes.create_string_buffer(max(4096, 4 * len(proto_text) + 1024))
+    n = lib.shdw_host_plan_fusion(proto_text.encode(), buf, len(buf))
+    host_check(n >= 0)
+    text = buf.value.decode()
+    return text.split("\n") if text else []
 
 
 def parse_net_binary(data, network_index=-1):

@@ -41,13 +41,33 @@ class FusedGroup {
   virtual bool Run(Workspace* ws) = 0;
 
   // "bn(Scale) + add(Eltwise) + relu(Activate) + gap(Reduce) -> e, pool"
-  virtual std::string describe() const = 0;
+  const std::string& describe() const { return description_; }
+  void set_description(const std::string& text) { description_ = text; }
 
  protected:
   std::vector<int> members_;
+
+ private:
+  std::string description_;
 };
 
-// The groups of `ops`, ordered by their last member; no operator is in two groups.
+// A group as the matcher finds it: positions in the operator list, -1 for a member
+// the group does not have.  Found from the operators' parameters alone, so that the
+// matching can be checked without a device.
+struct FusedPlan {
+  enum Kind { kScaleRelu, kResidualTail, kBatchNormScale, kEltwiseRelu };
+  Kind kind;
+  int bn, scale, eltwise, relu, mean;
+  std::vector<int> members() const;  // ascending
+};
+
+// The groups of a network given as its operators' parameters, ordered by their last
+// member; no operator is in two groups.
+std::vector<FusedPlan> PlanFusedGroups(const std::vector<shadow::OpParam>& op_params,
+                                       const std::vector<std::string>& out_blob);
+std::string DescribeFusedPlan(const FusedPlan& plan, const std::vector<shadow::OpParam>& op_params);
+
+// PlanFusedGroups over the parameters of `ops`, each plan as the group that runs it.
 std::vector<std::unique_ptr<FusedGroup>> FindFusedGroups(
     const std::vector<std::shared_ptr<Operator>>& ops, const std::vector<std::string>& out_blob);
 

@@ -10,6 +10,7 @@
 #include <string>
 #include <vector>
 
+#include "shadow/fusion.hpp"
 #include "shadow/io.hpp"
 #include "shadow/kernel.hpp"
 #include "shadow/native.hpp"
@@ -197,6 +198,25 @@ int shdw_host_parse_net(const char* proto_text, char* buf, size_t n) {
     shadow::NetParam net;
     Parser::ParseNet(proto_text, &net);
     len = join({Parser::DumpNet(net)}, buf, n);
+  });
+  return len;
+}
+
+// Host-only.  The groups the Native backend's fusion pass would form for this text
+// model, one description per line in the order they would run; returns the length,
+// or -1 when the text is malformed or names no out_blob.
+int shdw_host_plan_fusion(const char* proto_text, char* buf, size_t n) {
+  int len = -1;
+  guarded([&] {
+    shadow::NetParam net;
+    Parser::ParseNet(proto_text, &net);
+    const ArgumentHelper arguments(net);
+    CHECK(arguments.HasArgument("out_blob")) << "Network must have out_blob argument";
+    const std::vector<shadow::OpParam> ops(net.op().begin(), net.op().end());
+    std::vector<std::string> lines;
+    for (const FusedPlan& plan : PlanFusedGroups(ops, arguments.GetRepeatedArgument<std::string>("out_blob")))
+      lines.push_back(DescribeFusedPlan(plan, ops));
+    len = join(lines, buf, n);
   });
   return len;
 }

@@ -15,11 +15,34 @@ constexpr int kReduceAvg = 4;     // shadow/operators/kernels/reduce.hpp:18
 
 using OpList = std::vector<std::shared_ptr<Operator>>;
 
-bool reads(const Operator& op, const std::string& blob) {
+// What the matcher sees of an operator: its parameters and arguments, nothing that
+// needs a device.  The accessors carry Operator's names.
+class Node {
+ public:
+  explicit Node(const shadow::OpParam& op_param) : op_param_(op_param), arg_helper_(op_param) {}
+  const shadow::OpParam& op_param() const { return op_param_; }
+  const std::string& name() const { return op_param_.name(); }
+  const std::string& type() const { return op_param_.type(); }
+  template <typename T>
+  T get_single_argument(const std::string& name, const T& default_value) const {
+    return arg_helper_.GetSingleArgument<T>(name, default_value);
+  }
+  template <typename T>
+  std::vector<T> get_repeated_argument(const std::string& name) const {
+    return arg_helper_.GetRepeatedArgument<T>(name);
+  }
+
+ private:
+  shadow::OpParam op_param_;
+  ArgumentHelper arg_helper_;
+};
+using NodeList = std::vector<Node>;
+
+bool reads(const Node& op, const std::string& blob) {
   const auto& b = op.op_param().bottom();
   return std::find(b.begin(), b.end(), blob) != b.end();
 }
-bool writes(const Operator& op, const std::string& blob) {
+bool writes(const Node& op, const std::string& blob) {
   const auto& t = op.op_param().top();
   return std::find(t.begin(), t.end(), blob) != t.end();
 }
@@ -28,70 +51,70 @@ bool writes(const Operator& op, const std::string& blob) {
 // optimizer.py:87-94), on blob names that may be written again further down:
 // between `producer` and the next operator that overwrites `blob`, `reader` is the
 // only operator that reads it, and the network does not hand it out.
-bool sole_reader(const OpList& ops, const std::vector<std::string>& out_blob, const std::string& blob,
+bool sole_reader(const NodeList& ops, const std::vector<std::string>& out_blob, const std::string& blob,
                  int producer, int reader) {
   if (std::find(out_blob.begin(), out_blob.end(), blob) != out_blob.end()) return false;
   bool seen = false;
   for (int j = producer + 1; j < static_cast<int>(ops.size()); ++j) {
-    if (reads(*ops[j], blob)) {
+    if (reads(ops[j], blob)) {
       if (j != reader) return false;
       seen = true;
     }
-    if (writes(*ops[j], blob)) break;
+    if (writes(ops[j], blob)) break;
   }
   return seen;
 }
 
 // The first operator after `producer` that reads `blob` before it is overwritten.
-int next_reader(const OpList& ops, const std::string& blob, int producer) {
+int next_reader(const NodeList& ops, const std::string& blob, int producer) {
   for (int j = producer + 1; j < static_cast<int>(ops.size()); ++j) {
-    if (reads(*ops[j], blob)) return j;
-    if (writes(*ops[j], blob)) break;
+    if (reads(ops[j], blob)) return j;
+    if (writes(ops[j], blob)) break;
   }
   return -1;
 }
 
 // The operator in front of `reader` that wrote `blob` last, or -1.
-int last_writer(const OpList& ops, const std::string& blob, int reader) {
+int last_writer(const NodeList& ops, const std::string& blob, int reader) {
   for (int j = reader - 1; j >= 0; --j)
-    if (writes(*ops[j], blob)) return j;
+    if (writes(ops[j], blob)) return j;
   return -1;
 }
 
 // The members run together where the last one stood.  That is the order of the
 // file as long as no operator between them writes a blob the members read or
 // write, or reads a blob they write.
-bool movable(const OpList& ops, const std::vector<int>& members) {
+bool movable(const NodeList& ops, const std::vector<int>& members) {
   std::set<std::string> in, out;
   for (int m : members) {
-    in.insert(ops[m]->op_param().bottom().begin(), ops[m]->op_param().bottom().end());
-    out.insert(ops[m]->op_param().top().begin(), ops[m]->op_param().top().end());
+    in.insert(ops[m].op_param().bottom().begin(), ops[m].op_param().bottom().end());
+    out.insert(ops[m].op_param().top().begin(), ops[m].op_param().top().end());
   }
   for (int j = members.front() + 1; j < members.back(); ++j) {
     if (std::find(members.begin(), members.end(), j) != members.end()) continue;
-    for (const auto& t : ops[j]->op_param().top())
+    for (const auto& t : ops[j].op_param().top())
       if (in.count(t) || out.count(t)) return false;
-    for (const auto& b : ops[j]->op_param().bottom())
+    for (const auto& b : ops[j].op_param().bottom())
       if (out.count(b)) return false;
   }
   return true;
 }
 
-bool is_relu(const Operator& op) {
+bool is_relu(const Node& op) {
   return op.type() == "Activate" && op.get_single_argument<int>("type", 1) == kActivateRelu &&
          op.op_param().bottom_size() == 1 && op.op_param().top_size() == 1;
 }
 
 // Scale with its parameters as input blobs (not scale_value / bias_value, which
 // are staged through the temp buffer on every run).
-bool is_blob_scale(const Operator& op) {
+bool is_blob_scale(const Node& op) {
   if (op.type() != "Scale" || op.op_param().top_size() != 1) return false;
   const bool has_scale = op.get_single_argument<bool>("has_scale", false);
   const bool has_bias = op.get_single_argument<bool>("has_bias", false);
   return (has_scale || has_bias) && op.op_param().bottom_size() == (has_scale && has_bias ? 3 : 2);
 }
 
-bool is_residual_sum(const Operator& op) {
+bool is_residual_sum(const Node& op) {
   if (op.type() != "Eltwise" || op.op_param().bottom_size() != 2 || op.op_param().top_size() != 1) return false;
   if (op.get_single_argument<int>("operation", -1) != kEltwiseSum) return false;
   for (float c : op.get_repeated_argument<float>("coeff"))
@@ -102,7 +125,7 @@ bool is_residual_sum(const Operator& op) {
   return p.bottom(0) != p.bottom(1) && p.top(0) != p.bottom(0) && p.top(0) != p.bottom(1);
 }
 
-bool is_mean(const Operator& op) {
+bool is_mean(const Node& op) {
   return op.type() == "Reduce" && op.get_single_argument<int>("operation", 0) == kReduceAvg &&
          op.op_param().bottom_size() == 1 && op.op_param().top_size() == 1 &&
          op.op_param().top(0) != op.op_param().bottom(0);
@@ -147,7 +170,7 @@ bool view_scale(const Operator& op, Workspace* ws, ScaleView* v, const std::shar
 // BatchNorm on stored statistics (shadow/operators/batch_norm_op.cpp:7-47): how a
 // Caffe-style model holds a normalisation, the learned affine pair in the Scale
 // behind it.
-bool is_stats_batch_norm(const Operator& op) {
+bool is_stats_batch_norm(const Node& op) {
   return op.type() == "BatchNorm" && op.op_param().top_size() == 1 &&
          (op.op_param().bottom_size() == 3 || op.op_param().bottom_size() == 4);
 }
@@ -189,7 +212,7 @@ bool view_scale_per_channel(const Operator& scale, Workspace* ws, const NormView
   return axis == 1 && v->num == n.channel && v->inner == n.x->count(2);
 }
 
-std::string label(const Operator& op) { return op.name() + "(" + op.type() + ")"; }
+std::string label(const Node& op) { return op.name() + "(" + op.type() + ")"; }
 
 // ---- Scale -> Activate(relu): shdw_hip_scale_bias with its relu epilogue ----
 class ScaleRelu : public FusedGroup {
@@ -211,9 +234,6 @@ class ScaleRelu : public FusedGroup {
     return true;
   }
 
-  std::string describe() const override {
-    return label(*scale_) + " + " + label(*relu_) + " -> " + relu_->op_param().top(0);
-  }
 
  private:
   std::shared_ptr<Operator> scale_, relu_;
@@ -293,14 +313,6 @@ class ResidualTail : public FusedGroup {
     return true;
   }
 
-  std::string describe() const override {
-    std::string text = label(*scale_) + " + " + label(*sum_) + " + " + label(*relu_);
-    if (bn_ != nullptr) text = label(*bn_) + " + " + text;
-    if (mean_ != nullptr) text += " + " + label(*mean_);
-    text += " -> " + relu_->op_param().top(0);
-    if (mean_ != nullptr) text += ", " + mean_->op_param().top(0);
-    return text;
-  }
 
  private:
   std::shared_ptr<Operator> bn_, scale_, sum_, relu_, mean_;
@@ -334,11 +346,6 @@ class BatchNormScale : public FusedGroup {
     return true;
   }
 
-  std::string describe() const override {
-    std::string text = label(*bn_) + " + " + label(*scale_);
-    if (relu_ != nullptr) text += " + " + label(*relu_);
-    return text + " -> " + (relu_ != nullptr ? relu_ : scale_)->op_param().top(0);
-  }
 
  private:
   std::shared_ptr<Operator> bn_, scale_, relu_;
@@ -347,7 +354,7 @@ class BatchNormScale : public FusedGroup {
 // ---- Eltwise -> Activate(relu): shdw_hip_eltwise_relu ----
 // What closes a residual block once the converter has folded the normalisation into
 // the convolution (optimizer.py:181-252): the add and the ReLU.
-bool is_plain_eltwise(const Operator& op) {
+bool is_plain_eltwise(const Node& op) {
   if (op.type() != "Eltwise" || op.op_param().bottom_size() < 2 || op.op_param().top_size() != 1) return false;
   const int operation = op.get_single_argument<int>("operation", -1);
   if (operation < 0 || operation > 3) return false;
@@ -390,9 +397,6 @@ class EltwiseRelu : public FusedGroup {
     return true;
   }
 
-  std::string describe() const override {
-    return label(*eltwise_) + " + " + label(*relu_) + " -> " + relu_->op_param().top(0);
-  }
 
  private:
   std::shared_ptr<Operator> eltwise_, relu_;
@@ -400,23 +404,32 @@ class EltwiseRelu : public FusedGroup {
 
 }  // namespace
 
-std::vector<std::unique_ptr<FusedGroup>> FindFusedGroups(const OpList& ops,
-                                                         const std::vector<std::string>& out_blob) {
-  std::vector<std::unique_ptr<FusedGroup>> groups;
+std::vector<int> FusedPlan::members() const {
+  std::vector<int> all;
+  for (int m : {bn, scale, eltwise, relu, mean})
+    if (m >= 0) all.push_back(m);
+  std::sort(all.begin(), all.end());
+  return all;
+}
+
+std::vector<FusedPlan> PlanFusedGroups(const std::vector<shadow::OpParam>& op_params,
+                                       const std::vector<std::string>& out_blob) {
+  const NodeList ops(op_params.begin(), op_params.end());
+  std::vector<FusedPlan> groups;
   std::vector<bool> taken(ops.size(), false);
   const int count = static_cast<int>(ops.size());
   // Residual tails first: a Scale whose output goes into a sum belongs there, with the BatchNorm
   // in front of it where there is one, and the tail can take the mean along.
   for (int i = 0; i < count; ++i) {
-    if (taken[i] || !is_blob_scale(*ops[i])) continue;
-    const std::string& s = ops[i]->op_param().top(0);
+    if (taken[i] || !is_blob_scale(ops[i])) continue;
+    const std::string& s = ops[i].op_param().top(0);
     const int next = next_reader(ops, s, i);
     if (next < 0 || taken[next]) continue;
-    if (!is_residual_sum(*ops[next]) || !sole_reader(ops, out_blob, s, i, next)) continue;
-    const std::string& e = ops[next]->op_param().top(0);
+    if (!is_residual_sum(ops[next]) || !sole_reader(ops, out_blob, s, i, next)) continue;
+    const std::string& e = ops[next].op_param().top(0);
     const int relu = next_reader(ops, e, next);
-    if (relu < 0 || taken[relu] || !is_relu(*ops[relu])) continue;
-    const std::string& y = ops[relu]->op_param().top(0);
+    if (relu < 0 || taken[relu] || !is_relu(ops[relu])) continue;
+    const std::string& y = ops[relu].op_param().top(0);
     // not in place: the sum itself is no longer written, so nobody else may want it;
     // in place: every reader further down sees the activated values either way
     if (y != e && !sole_reader(ops, out_blob, e, next, relu)) continue;
@@ -425,36 +438,36 @@ std::vector<std::unique_ptr<FusedGroup>> FindFusedGroups(const OpList& ops,
     if (!movable(ops, members)) continue;
     int mean = -1;
     for (int j = relu + 1; j < count; ++j) {
-      if (!taken[j] && is_mean(*ops[j]) && ops[j]->op_param().bottom(0) == y) {
+      if (!taken[j] && is_mean(ops[j]) && ops[j].op_param().bottom(0) == y) {
         std::vector<int> with_mean = {i, next, relu, j};
         if (movable(ops, with_mean)) mean = j;
         break;
       }
-      if (writes(*ops[j], y)) break;
+      if (writes(ops[j], y)) break;
     }
     // a BatchNorm whose output only this Scale reads comes along
-    int bn = last_writer(ops, ops[i]->op_param().bottom(0), i);
+    int bn = last_writer(ops, ops[i].op_param().bottom(0), i);
     if (bn >= 0) {
-      const auto& sp = ops[i]->op_param();
+      const auto& sp = ops[i].op_param();
       const std::string& n = sp.bottom(0);
-      bool ok = !taken[bn] && is_stats_batch_norm(*ops[bn]) && sole_reader(ops, out_blob, n, bn, i);
+      bool ok = !taken[bn] && is_stats_batch_norm(ops[bn]) && sole_reader(ops, out_blob, n, bn, i);
       for (int k = 1; k < sp.bottom_size(); ++k) ok = ok && sp.bottom(k) != n;
       std::vector<int> with_bn = {bn, i, next, relu};
       if (mean >= 0) with_bn.push_back(mean);
       if (!ok || !movable(ops, with_bn)) bn = -1;
     }
-    groups.emplace_back(new ResidualTail(ops, bn, i, next, relu, mean));
+    groups.push_back(FusedPlan{FusedPlan::kResidualTail, bn, i, next, relu, mean});
     taken[i] = taken[next] = taken[relu] = true;
     if (bn >= 0) taken[bn] = true;
     if (mean >= 0) taken[mean] = true;
   }
   // BatchNorm -> Scale [-> ReLU] next: it takes the Scale -> ReLU pair with it.
   for (int i = 0; i < count; ++i) {
-    if (taken[i] || !is_stats_batch_norm(*ops[i])) continue;
-    const std::string& n = ops[i]->op_param().top(0);
+    if (taken[i] || !is_stats_batch_norm(ops[i])) continue;
+    const std::string& n = ops[i].op_param().top(0);
     const int scale = next_reader(ops, n, i);
-    if (scale < 0 || taken[scale] || !is_blob_scale(*ops[scale])) continue;
-    const auto& sp = ops[scale]->op_param();
+    if (scale < 0 || taken[scale] || !is_blob_scale(ops[scale])) continue;
+    const auto& sp = ops[scale].op_param();
     if (sp.bottom(0) != n) continue;
     bool as_parameter = false;  // the normalised blob must be the Scale's data, not one of its parameters
     for (int k = 1; k < sp.bottom_size(); ++k) as_parameter = as_parameter || sp.bottom(k) == n;
@@ -465,44 +478,95 @@ std::vector<std::unique_ptr<FusedGroup>> FindFusedGroups(const OpList& ops,
     std::vector<int> members = {i, scale};
     if (!movable(ops, members)) continue;
     int relu = next_reader(ops, s, scale);
-    if (relu >= 0 && (taken[relu] || !is_relu(*ops[relu]))) relu = -1;
-    if (relu >= 0 && ops[relu]->op_param().top(0) != s && !sole_reader(ops, out_blob, s, scale, relu)) relu = -1;
+    if (relu >= 0 && (taken[relu] || !is_relu(ops[relu]))) relu = -1;
+    if (relu >= 0 && ops[relu].op_param().top(0) != s && !sole_reader(ops, out_blob, s, scale, relu)) relu = -1;
     if (relu >= 0) {
       members.push_back(relu);
       if (!movable(ops, members)) relu = -1;
     }
-    groups.emplace_back(new BatchNormScale(ops, i, scale, relu));
+    groups.push_back(FusedPlan{FusedPlan::kBatchNormScale, i, scale, -1, relu, -1});
     taken[i] = taken[scale] = true;
     if (relu >= 0) taken[relu] = true;
   }
   for (int i = 0; i < count; ++i) {
-    if (taken[i] || !is_blob_scale(*ops[i])) continue;
-    const std::string& s = ops[i]->op_param().top(0);
+    if (taken[i] || !is_blob_scale(ops[i])) continue;
+    const std::string& s = ops[i].op_param().top(0);
     const int next = next_reader(ops, s, i);
-    if (next < 0 || taken[next] || !is_relu(*ops[next])) continue;
+    if (next < 0 || taken[next] || !is_relu(ops[next])) continue;
     // in place the Scale output is the group's output and every later reader sees the
     // activated values either way; elsewhere it is no longer written
-    if (ops[next]->op_param().top(0) != s && !sole_reader(ops, out_blob, s, i, next)) continue;
+    if (ops[next].op_param().top(0) != s && !sole_reader(ops, out_blob, s, i, next)) continue;
     std::vector<int> members = {i, next};
     if (!movable(ops, members)) continue;
-    groups.emplace_back(new ScaleRelu(ops, i, next));
+    groups.push_back(FusedPlan{FusedPlan::kScaleRelu, -1, i, -1, next, -1});
     taken[i] = taken[next] = true;
   }
   for (int i = 0; i < count; ++i) {
-    if (taken[i] || !is_plain_eltwise(*ops[i])) continue;
-    const std::string& e = ops[i]->op_param().top(0);
+    if (taken[i] || !is_plain_eltwise(ops[i])) continue;
+    const std::string& e = ops[i].op_param().top(0);
     const int relu = next_reader(ops, e, i);
-    if (relu < 0 || taken[relu] || !is_relu(*ops[relu])) continue;
-    if (ops[relu]->op_param().top(0) != e && !sole_reader(ops, out_blob, e, i, relu)) continue;
+    if (relu < 0 || taken[relu] || !is_relu(ops[relu])) continue;
+    if (ops[relu].op_param().top(0) != e && !sole_reader(ops, out_blob, e, i, relu)) continue;
     std::vector<int> members = {i, relu};
     if (!movable(ops, members)) continue;
-    groups.emplace_back(new EltwiseRelu(ops, i, relu));
+    groups.push_back(FusedPlan{FusedPlan::kEltwiseRelu, -1, -1, i, relu, -1});
     taken[i] = taken[relu] = true;
   }
-  std::sort(groups.begin(), groups.end(),
-            [](const std::unique_ptr<FusedGroup>& a, const std::unique_ptr<FusedGroup>& b) {
-              return a->members().back() < b->members().back();
-            });
+  std::sort(groups.begin(), groups.end(), [](const FusedPlan& a, const FusedPlan& b) {
+    return a.members().back() < b.members().back();
+  });
+  return groups;
+}
+
+std::string DescribeFusedPlan(const FusedPlan& plan, const std::vector<shadow::OpParam>& op_params) {
+  const auto name = [&](int position) { return label(Node(op_params[position])); };
+  const auto top = [&](int position) { return op_params[position].top(0); };
+  switch (plan.kind) {
+    case FusedPlan::kScaleRelu:
+      return name(plan.scale) + " + " + name(plan.relu) + " -> " + top(plan.relu);
+    case FusedPlan::kEltwiseRelu:
+      return name(plan.eltwise) + " + " + name(plan.relu) + " -> " + top(plan.relu);
+    case FusedPlan::kBatchNormScale: {
+      std::string text = name(plan.bn) + " + " + name(plan.scale);
+      if (plan.relu >= 0) text += " + " + name(plan.relu);
+      return text + " -> " + top(plan.relu >= 0 ? plan.relu : plan.scale);
+    }
+    case FusedPlan::kResidualTail: {
+      std::string text = name(plan.scale) + " + " + name(plan.eltwise) + " + " + name(plan.relu);
+      if (plan.bn >= 0) text = name(plan.bn) + " + " + text;
+      if (plan.mean >= 0) text += " + " + name(plan.mean);
+      text += " -> " + top(plan.relu);
+      if (plan.mean >= 0) text += ", " + top(plan.mean);
+      return text;
+    }
+  }
+  return "";
+}
+
+std::vector<std::unique_ptr<FusedGroup>> FindFusedGroups(const OpList& ops,
+                                                         const std::vector<std::string>& out_blob) {
+  std::vector<shadow::OpParam> op_params;
+  for (const auto& op : ops) op_params.push_back(op->op_param());
+  std::vector<std::unique_ptr<FusedGroup>> groups;
+  for (const FusedPlan& plan : PlanFusedGroups(op_params, out_blob)) {
+    std::unique_ptr<FusedGroup> group;
+    switch (plan.kind) {
+      case FusedPlan::kScaleRelu:
+        group.reset(new ScaleRelu(ops, plan.scale, plan.relu));
+        break;
+      case FusedPlan::kEltwiseRelu:
+        group.reset(new EltwiseRelu(ops, plan.eltwise, plan.relu));
+        break;
+      case FusedPlan::kBatchNormScale:
+        group.reset(new BatchNormScale(ops, plan.bn, plan.scale, plan.relu));
+        break;
+      case FusedPlan::kResidualTail:
+        group.reset(new ResidualTail(ops, plan.bn, plan.scale, plan.eltwise, plan.relu, plan.mean));
+        break;
+    }
+    group->set_description(DescribeFusedPlan(plan, op_params));
+    groups.push_back(std::move(group));
+  }
   return groups;
 }
 
