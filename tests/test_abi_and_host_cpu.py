@@ -167,6 +167,22 @@ def test_entry_points_validate_before_touching_the_device():
     assert 8 * 8 < lib.shdw_hip_ssd_normalize_workspace_bytes(8, 512, 1444, 1) <= 8 * 64 * 8  # several parts per item
     assert lib.shdw_hip_ssd_normalize_workspace_bytes(4096, 2, 8, 1) == 4096 * 8
     assert lib.shdw_hip_batch_norm(0, 4, 1, None, None, None, 1.0, 0.0, None, None) == 0
+    assert lib.shdw_hip_batch_norm_scale(8, 2, 4, p, p, p, 1.0, 0.0, None, None, 1, p, None) == E  # neither scale nor bias
+    assert lib.shdw_hip_batch_norm_scale(8, 0, 4, p, p, p, 1.0, 0.0, p, p, 1, p, None) == E
+    assert lib.shdw_hip_batch_norm_scale(8, 2, 4, p, None, p, 1.0, 0.0, p, p, 0, p, None) == E
+    assert lib.shdw_hip_batch_norm_scale(0, 2, 4, None, None, None, 1.0, 0.0, p, None, 0, None, None) == 0
+    assert lib.shdw_hip_batch_norm_scale_residual_relu(16, 2, 8, p, p, None, 1.0, 0.0, p, p, p, 0, p, p, None) == E
+    assert lib.shdw_hip_batch_norm_scale_residual_relu(16, 2, 8, p, p, p, 1.0, 0.0, p, p, None, 0, p, p, None) == E
+    assert lib.shdw_hip_batch_norm_scale_residual_relu(15, 2, 8, p, p, p, 1.0, 0.0, p, p, p, 0, p, p, None) == E
+    assert lib.shdw_hip_batch_norm_scale_residual_relu(0, 2, 8, p, p, p, 1.0, 0.0, p, p, p, 0, p, p, None) == 0
+    lrn = ints([2, 3, 4, 4])
+    assert lib.shdw_hip_lrn(lrn, 4, 1.0, 0.75, 1.0, p, p, None) == E            # even window
+    assert lib.shdw_hip_lrn(lrn, 9, 1.0, 0.75, 1.0, p, p, None) == E            # four channels behind the centre, three there
+    assert lib.shdw_hip_lrn(lrn, 5, 1.0, 0.75, 1.0, None, p, None) == E
+    assert lib.shdw_hip_lrn(None, 5, 1.0, 0.75, 1.0, p, p, None) == E
+    assert lib.shdw_hip_lrn(ints([2, 80, 1, 1]), 65, 1.0, 0.75, 1.0, p, p, None) == U   # windows over 63 channels
+    assert lib.shdw_hip_lrn(ints([65536, 65536, 1, 1]), 5, 1.0, 0.75, 1.0, p, p, None) == U
+    assert lib.shdw_hip_lrn(ints([2, 0, 4, 4]), 1, 1.0, 0.75, 1.0, None, None, None) == 0
     assert lib.shdw_hip_axpy_rows(65536, 65536, p, p, p, p, None) == E
     assert lib.shdw_hip_axpy_rows(4, 4, None, p, p, p, None) == E
     assert lib.shdw_hip_group_norm(2, 8, 1e-5, p, p, None, 1, 1, p, None) == E
