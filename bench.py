@@ -979,6 +979,13 @@ def config_table(dev, sets_scale=1, cpu=None):
     ms = time_median(dev, lambda k: lib.shdw_hip_lrn(I([64, CH, 56, 56]), 5, 1e-4, 0.75, 1.0, AH[k].ptr, YH[k].ptr, st),
                      SH, reps=20)
     add("next", "lrn across 5 channels [64,256,56,56]", 4 * NH, 4 * NH, ms, NH)
+    # GridSample with a mildly warped identity grid (what a spatial transformer produces): bilinear, zeros outside
+    gy, gx = np.meshgrid(np.linspace(-1, 1, 56), np.linspace(-1, 1, 56), indexing="ij")
+    warp = np.stack([gx, gy], -1).astype(np.float32)[None] + uniform(614, (64, 56, 56, 2), -0.05, 0.05)
+    gridh = dev.buf(np.ascontiguousarray(warp, np.float32).ravel())
+    hw = I([64, CH, 56, 56])
+    ms = time_median(dev, lambda k: lib.shdw_hip_grid_sample(hw, hw, 1, 0, AH[k].ptr, gridh.ptr, YH[k].ptr, st), SH, reps=20)
+    add("next", "grid_sample bilinear, warped identity [64,256,56,56]", 4 * NH + 8 * 64 * 3136, 4 * NH, ms, NH)
     alh = dev.buf(uniform(613, 64 * CH, 0.0, 1.0))
     ms = time_median(dev, lambda k: lib.shdw_hip_axpy_rows(64 * CH, INH, alh.ptr, AH[k].ptr,
                                                            AH[(k + 1) % SH].ptr, YH[k].ptr, st), SH, reps=20)

@@ -337,6 +337,19 @@ int shdw_hip_batch_norm_scale(int n, int channel, int inner_num, const float* x,
 int shdw_hip_lrn(const int* in_shape, int size, float alpha, float beta, float k, const float* x,
                  float* y, void* stream);
 
+/* GridSample: x [batch][channel][in_h][in_w], grid [batch][out_h][out_w][2] holding
+ * (x, y) in [-1, 1], y [batch][channel][out_h][out_w]; the source coordinate is
+ * (v + 1) / 2 * (extent - 1).  mode 0: the nearest cell (roundf), 1: the four cells
+ * around it, weighted in the reference's order of operations.  padding_mode 0:
+ * zeros outside the input, 1: coordinates clamped to the border.  Every index is
+ * clamped before use, so no grid value reads outside x.  A float that fits no int
+ * converts as in the reference's x86-64 build (INT_MIN); a NaN coordinate in mode 1,
+ * with which the reference indexes outside its input, gives NaN.  y must not be x.
+ * ref: shadow/operators/kernels/grid_sample.cpp:9-100, grid_sample.cu,
+ *      shadow/operators/grid_sample_op.cpp:9-47 */
+int shdw_hip_grid_sample(const int* in_shape, const int* out_shape, int mode, int padding_mode,
+                         const float* x, const float* grid, float* y, void* stream);
+
 /* Softmax over the middle extent of x viewed as [outer_num][dim][inner_num]:
  * running maximum, exp(x - max), fp32 running sum in index order, divide.  The
  * per-column scratch blob of the reference is not needed.  y may alias x.

@@ -197,6 +197,13 @@ def lrn(x, in_shape, size, alpha, beta, k):
     return out, scale
 
 
+def grid_sample(x, in_shape, grid, mode, padding_mode, out_shape):
+    x, grid = _f(x).ravel(), _f(grid).ravel()
+    out = np.empty(int(np.prod(out_shape, dtype=np.int64)), np.float32)
+    lib().orc_grid_sample(_p(x), _ints(in_shape), _p(grid), int(mode), int(padding_mode), _ints(out_shape), _p(out))
+    return out
+
+
 def softmax(x, outer, dim, inner):
     x = _f(x).ravel()
     out = np.empty_like(x)
@@ -403,6 +410,18 @@ def lrn_op(x, local_size=5, alpha=1.0, beta=0.75, norm_region=0, k=1.0):
     _check(x.shape[1] >= (local_size - 1) // 2, "in_c >= post_pad")
     out, _ = lrn(x, x.shape, local_size, alpha, beta, k)
     return out.reshape(x.shape)
+
+
+def grid_sample_op(x, grid, mode=1, padding_mode=0):
+    """shadow/operators/grid_sample_op.cpp:9-47: x [b, c, h, w], grid [b, out_h, out_w, 2] -> [b, c, out_h, out_w]"""
+    _check(mode in (0, 1), "mode_ == 0 || mode_ == 1")
+    _check(padding_mode in (0, 1), "padding_mode_ == 0 || padding_mode_ == 1")
+    x, grid = _f(x), _f(grid)
+    _check(x.ndim == 4 and grid.ndim == 4, "4-D input and grid")
+    _check(x.shape[0] == grid.shape[0], "input->shape(0) == grid->shape(0)")
+    _check(grid.shape[3] == 2, "grid->shape(3) == 2")
+    out_shape = [x.shape[0], x.shape[1], grid.shape[1], grid.shape[2]]
+    return grid_sample(x, x.shape, grid, mode, padding_mode, out_shape).reshape(out_shape)
 
 
 def _canonical(axis, ndim):

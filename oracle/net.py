@@ -229,6 +229,9 @@ def _run_op(op, blobs):
         oracle._check(len(x) >= 3, "inputs.size() >= 3")
         return oracle.batch_norm_op(x[0], x[1], x[2], x[3] if len(x) == 4 else None,
                                     _single(a, "eps", F(1e-5)), bool(_single(a, "use_global_stats", True)))
+    if t == "GridSample":
+        oracle._check(len(x) == 2, "inputs.size() == 2")
+        return oracle.grid_sample_op(x[0], x[1], _single(a, "mode", 1), _single(a, "padding_mode", 0))
     if t == "LRN":
         return oracle.lrn_op(x[0], _single(a, "local_size", 5), _single(a, "alpha", F(1)), _single(a, "beta", F(0.75)),
                              _single(a, "norm_region", 0), _single(a, "k", F(1)))

@@ -792,3 +792,70 @@ API void orc_lrn(const float* in, const int* in_shape, int size, float alpha, fl
   }
   for (int i = 0; i < count; ++i) out[i] = in[i] * powf(scale[i], -beta);
 }
+
+/* ---- shadow/operators/kernels/grid_sample.cpp:9-100  Vision::GridSample ----
+ * grid holds (x, y) in [-1, 1] per output position; (v + 1) / 2 * (extent - 1) is the
+ * source coordinate.  mode 0: the nearest source cell (roundf, then the conversion to
+ * int), mode 1: the four cells around the coordinate, weights in the reference's order
+ * of operations.  padding_mode 0: outside the input reads as 0; 1: coordinates are
+ * clamped to the border.
+ * Where the reference leaves the value to the machine this follows what its x86-64
+ * build does: a float that does not fit an int converts to INT_MIN.  A NaN coordinate
+ * in mode 1 makes the reference index far outside its input; here it gives NaN. */
+static int to_int_x86(float v) {
+  return (v >= -2147483648.f && v < 2147483648.f) ? (int)v : (-2147483647 - 1);
+}
+
+API void orc_grid_sample(const float* in, const int* in_shape, const float* grid, int mode,
+                         int padding_mode, const int* out_shape, float* out) {
+  int batch = in_shape[0], channel = in_shape[1], in_h = in_shape[2], in_w = in_shape[3];
+  int out_h = out_shape[2], out_w = out_shape[3];
+  for (int b = 0; b < batch; ++b) {
+    for (int c = 0; c < channel; ++c) {
+      for (int h = 0; h < out_h; ++h) {
+        for (int w = 0; w < out_w; ++w) {
+          int grid_offset = ((b * out_h + h) * out_w + w) * 2;
+          float x = grid[grid_offset], y = grid[grid_offset + 1];
+          if (mode == 0) {
+            int src_h = to_int_x86(roundf((y + 1) / 2.f * (in_h - 1)));
+            int src_w = to_int_x86(roundf((x + 1) / 2.f * (in_w - 1)));
+            if (padding_mode == 1) {
+              src_h = src_h < 0 ? 0 : (src_h > in_h - 1 ? in_h - 1 : src_h);
+              src_w = src_w < 0 ? 0 : (src_w > in_w - 1 ? in_w - 1 : src_w);
+            } else if (src_h < 0 || src_w < 0 || src_h > in_h - 1 || src_w > in_w - 1) {
+              *out++ = 0.f;
+              continue;
+            }
+            *out++ = in[((b * channel + c) * in_h + src_h) * in_w + src_w];
+            continue;
+          }
+          float src_h_f = (y + 1) / 2.f * (in_h - 1);
+          float src_w_f = (x + 1) / 2.f * (in_w - 1);
+          if (padding_mode == 1) {
+            src_h_f = std_min(std_max(src_h_f, 0.f), in_h - 1.f);
+            src_w_f = std_min(std_max(src_w_f, 0.f), in_w - 1.f);
+          } else if (src_h_f < 0 || src_w_f < 0 || src_h_f > in_h - 1 || src_w_f > in_w - 1) {
+            *out++ = 0.f;
+            continue;
+          }
+          if (src_h_f != src_h_f || src_w_f != src_w_f) {
+            *out++ = NAN;
+            continue;
+          }
+          int src_h_0 = (int)floorf(src_h_f), src_h_1 = (int)ceilf(src_h_f);
+          int src_w_0 = (int)floorf(src_w_f), src_w_1 = (int)ceilf(src_w_f);
+          src_h_0 = src_h_0 < 0 ? 0 : src_h_0;
+          src_h_1 = src_h_1 > in_h - 1 ? in_h - 1 : src_h_1;
+          src_w_0 = src_w_0 < 0 ? 0 : src_w_0;
+          src_w_1 = src_w_1 > in_w - 1 ? in_w - 1 : src_w_1;
+          float sh = src_h_f - src_h_0, sw = src_w_f - src_w_0;
+          int h_offset = (b * channel + c) * in_h;
+          int i0 = (h_offset + src_h_0) * in_w + src_w_0, i1 = (h_offset + src_h_1) * in_w + src_w_0;
+          int i2 = (h_offset + src_h_0) * in_w + src_w_1, i3 = (h_offset + src_h_1) * in_w + src_w_1;
+          *out++ = (1 - sh) * (1 - sw) * in[i0] + sh * (1 - sw) * in[i1] + (1 - sh) * sw * in[i2] +
+                   sh * sw * in[i3];
+        }
+      }
+    }
+  }
+}

@@ -83,6 +83,7 @@ SIGNATURES = {
                                      ctypes.POINTER(ctypes.c_uint)]),
     "shdw_hip_scale_residual_relu": (_I, [_I, _I, _I, _V, _V, _V, _V, _I, _V, _V, _V]),
     "shdw_hip_batch_norm_scale_residual_relu": (_I, [_I, _I, _I, _V, _V, _V, _F, _F, _V, _V, _V, _I, _V, _V, _V]),
+    "shdw_hip_grid_sample": (_I, [c_int_p, c_int_p, _I, _I, _V, _V, _V, _V]),
     "shdw_hip_lrn": (_I, [c_int_p, _I, _F, _F, _F, _V, _V, _V]),
     "shdw_hip_axpy_rows": (_I, [_I, _I, _V, _V, _V, _V, _V]),
     "shdw_hip_batch_norm": (_I, [_I, _I, _I, _V, _V, _V, _F, _F, _V, _V]),

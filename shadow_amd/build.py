@@ -34,7 +34,7 @@ HIP_FLAGS = [
     "-Wno-unused-command-line-argument",
 ]
 HIP_SOURCES = ["elementwise.hip", "broadcast.hip", "reduce.hip", "fused.hip", "vision.hip", "softmax.hip", "norm.hip", "movers.hip",
-               "lrn.hip", "runtime.hip"]
+               "lrn.hip", "grid_sample.hip", "runtime.hip"]
 
 def _run(cmd):
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

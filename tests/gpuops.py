@@ -228,6 +228,18 @@ def batch_norm_scale_residual_relu(x, stat_mean, stat_variance, scale_factor, ep
     return (y.download(count=n) if y else None), (mean.download(count=rows) if mean else None)
 
 
+def grid_sample(x, in_shape, grid, mode, padding_mode, out_shape):
+    x, grid = _f(x).ravel(), _f(grid).ravel()
+    n_out = int(np.prod(out_shape, dtype=np.int64))
+    assert x.size == int(np.prod(in_shape, dtype=np.int64)) and grid.size == 2 * out_shape[0] * out_shape[2] * out_shape[3]
+    dx, dg = Buffer.from_numpy(x), Buffer.from_numpy(grid)
+    y = Buffer(max(4, 4 * n_out))
+    check(_lib().shdw_hip_grid_sample(ints(in_shape), ints(out_shape), int(mode), int(padding_mode), dx.ptr, dg.ptr,
+                                      y.ptr, None))
+    _sync()
+    return y.download(count=n_out)
+
+
 def lrn(x, in_shape, size, alpha, beta, k, inplace=False):
     x = _f(x).ravel()
     dx = Buffer.from_numpy(x)

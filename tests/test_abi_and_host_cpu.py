@@ -118,7 +118,8 @@ def keys(fn):
 
 def test_registries_hold_exactly_the_gpu_default_kernels():
     h = shadow_amd.host()
-    kernels = ["Activate", "Axpy", "BatchNorm", "Binary", "Concat", "Eltwise", "Gather", "GroupNorm", "LRN", "LayerNorm",
+    kernels = ["Activate", "Axpy", "BatchNorm", "Binary", "Concat", "Eltwise", "Gather", "GridSample", "GroupNorm", "LRN",
+               "LayerNorm",
                "Normalize", "Pad", "Permute", "Pooling", "Reduce", "Reorg", "Resize", "SSDNormalize", "Scale",
                "ShuffleChannel", "Slice", "Softmax", "Stack", "Unary"]
     # InstanceNorm runs on the GroupNorm kernel (shadow/operators/instance_norm_op.cpp:14)

@@ -166,6 +166,88 @@ def test_lrn_op(ws):
         ws.create_op("LRN", ["x"], ["o5"], {"local_size": 23}).run()
 
 
+# ------------------------------------------------------------ grid sample ---
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("padding_mode", [0, 1])
+@pytest.mark.parametrize("shape,out_hw", [((2, 3, 5, 7), (4, 6)), ((1, 13, 1, 9), (3, 3)), ((3, 1, 8, 1), (2, 5)),
+                                          ((2, 20, 6, 6), (11, 13)), ((2, 64, 56, 56), (56, 56)), ((1, 8, 31, 17), (64, 70)),
+                                          ((300, 2, 3, 3), (1, 1))])
+def test_grid_sample(gpu, mode, padding_mode, shape, out_hw):
+    x = with_specials(normal(41, shape, 2.0), 41)
+    grid = uniform(42, (shape[0],) + out_hw + (2,), -1.3, 1.3)  # a fifth of the coordinates outside the input
+    out_shape = list(shape[:2]) + list(out_hw)
+    want = oracle.grid_sample(x, shape, grid, mode, padding_mode, out_shape)
+    assert_bit_exact(gpuops.grid_sample(x, shape, grid, mode, padding_mode, out_shape), want, "grid sample")
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("padding_mode", [0, 1])
+def test_grid_sample_on_cell_centres_ties_and_coordinates_that_fit_no_int(gpu, mode, padding_mode):
+    shape, out_hw = (2, 5, 9, 5), (9, 8)
+    x = normal(43, shape)
+    gy, gx = np.meshgrid(np.linspace(-1, 1, 9), np.linspace(-1, 1, 8), indexing="ij")  # rows: exact centres; columns: ties and thirds
+    grid = np.broadcast_to(np.stack([gx, gy], -1).astype(F), (2,) + out_hw + (2,)).copy()
+    grid[1, 0, :, 0] = [1e30, -1e30, np.inf, -np.inf, 3e9, -3e9, 2.0 ** 31, -1.0000001]
+    grid[1, 1, :, 1] = [1e30, -1e30, np.inf, -np.inf, 3e9, -3e9, 2.0 ** 31, 1.0000001]
+    if mode == 0:  # a NaN coordinate has a defined answer in the nearest mode only (the conversion's)
+        grid[1, 2, :4, 0] = np.nan
+        grid[1, 3, 4:, 1] = np.nan
+    out_shape = list(shape[:2]) + list(out_hw)
+    want = oracle.grid_sample(x, shape, grid, mode, padding_mode, out_shape)
+    assert_bit_exact(gpuops.grid_sample(x, shape, grid, mode, padding_mode, out_shape), want, "grid sample")
+
+
+def test_grid_sample_bilinear_gives_nan_for_a_nan_coordinate(gpu):
+    shape, out_hw = (1, 3, 4, 4), (2, 2)
+    x = normal(44, shape)
+    grid = np.zeros((1, 2, 2, 2), F)
+    grid[0, 0, 0, 0] = np.nan
+    grid[0, 1, 1, 1] = np.nan
+    for padding_mode in (0, 1):
+        got = gpuops.grid_sample(x, shape, grid, 1, padding_mode, [1, 3, 2, 2]).reshape(1, 3, 2, 2)
+        assert np.isnan(got[:, :, 0, 0]).all() and np.isnan(got[:, :, 1, 1]).all()
+        assert_bit_exact(got, oracle.grid_sample(x, shape, grid, 1, padding_mode, [1, 3, 2, 2]), "the oracle's rule")
+
+
+def test_grid_sample_argument_errors(gpu):
+    lib, ints = gpu, shadow_amd.ints
+    buf = shadow_amd.Buffer(4 * 64)
+    a, o = ints([1, 2, 2, 2]), ints([1, 2, 2, 2])
+    assert lib.shdw_hip_grid_sample(a, o, 2, 0, buf.ptr, buf.ptr, buf.ptr, None) == -1
+    assert lib.shdw_hip_grid_sample(a, o, 1, 2, buf.ptr, buf.ptr, buf.ptr, None) == -1
+    assert lib.shdw_hip_grid_sample(a, ints([1, 3, 2, 2]), 1, 0, buf.ptr, buf.ptr, buf.ptr, None) == -1   # channels differ
+    assert lib.shdw_hip_grid_sample(a, ints([2, 2, 2, 2]), 1, 0, buf.ptr, buf.ptr, buf.ptr, None) == -1   # batches differ
+    assert lib.shdw_hip_grid_sample(a, o, 1, 0, buf.ptr, buf.ptr, buf.ptr, None) == -1                    # output is the input
+    assert lib.shdw_hip_grid_sample(a, o, 1, 0, None, buf.ptr, buf.ptr, None) == -1
+    assert lib.shdw_hip_grid_sample(ints([1, 2, 0, 2]), o, 1, 0, buf.ptr, buf.ptr, buf.ptr, None) == -1   # nothing to sample
+    assert lib.shdw_hip_grid_sample(a, ints([1, 2, 0, 2]), 1, 0, None, None, None, None) == 0             # nothing to fill
+
+
+def test_grid_sample_op(ws):
+    x, grid = normal(45, (2, 6, 7, 5), 2.0), uniform(46, (2, 4, 9, 2), -1.2, 1.2)
+    for mode in (0, 1):
+        for padding_mode in (0, 1):
+            got = run(ws, "GridSample", [("x", x), ("grid", grid)], {"mode": mode, "padding_mode": padding_mode})
+            assert got.shape == (2, 6, 4, 9)
+            assert_bit_exact(got, oracle.grid_sample_op(x, grid, mode, padding_mode), "grid sample op")
+    got = run(ws, "GridSample", [("x", x), ("grid", grid)], {})
+    assert_bit_exact(got, oracle.grid_sample_op(x, grid), "bilinear with zeros outside by default")
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("GridSample", ["x", "grid"], ["o2"], {"mode": 2})
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("GridSample", ["x", "grid"], ["o3"], {"padding_mode": 2})
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("GridSample", ["x"], ["o4"], {}).run()
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("GridSample", ["x", "grid"], ["x"], {}).run()
+    ws.set_blob("three", np.zeros((2, 4, 9, 3), F))
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("GridSample", ["x", "three"], ["o5"], {}).run()
+    ws.set_blob("other", np.zeros((3, 4, 9, 2), F))
+    with pytest.raises(ShadowError, match="Check Failed"):
+        ws.create_op("GridSample", ["x", "other"], ["o6"], {}).run()
+
+
 # ---------------------------------------------------------------- softmax ---
 SOFTMAX_SHAPES = [  # outer, dim, inner: both layouts, LDS limits, odd sizes
     (1, 1, 1), (64, 1000, 1), (3, 10, 1), (5, 7, 3), (2, 21, 63), (2, 21, 64), (2, 21, 65),

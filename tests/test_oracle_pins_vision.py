@@ -1,4 +1,4 @@
-"""Pins for the oracle's Axpy / BatchNorm / Softmax / Normalize / Pooling / LRN
+"""Pins for the oracle's Axpy / BatchNorm / Softmax / Normalize / Pooling / LRN / GridSample
 restatements.  The reference holds no vectors for these either, so each is
 checked against an independent numpy formulation (axis operations and slicing,
 never the oracle's flat pointer walks), against exactly representable data with
@@ -441,3 +441,91 @@ def test_lrn_op_checks():
     with pytest.raises(oracle.OracleCheckError):
         oracle.lrn_op(x, 9)  # three channels, four behind the centre
     oracle.lrn_op(x, 7)
+
+
+# ------------------------------------------------------------ grid sample ---
+def grid_sample_by_arrays(x, grid, mode, padding_mode):
+    """Whole-array numpy: coordinates, masks, gathers with take_along_axis-free fancy indexing and the
+    reference's order of float32 operations; finite coordinates that fit an int."""
+    x, grid = x.astype(F), grid.astype(F)
+    b, c, in_h, in_w = x.shape
+    gx, gy = grid[..., 0], grid[..., 1]                      # [b, out_h, out_w]
+    fh = (gy + F(1)) / F(2) * F(in_h - 1)
+    fw = (gx + F(1)) / F(2) * F(in_w - 1)
+    bi = np.arange(b)[:, None, None, None]
+    ci = np.arange(c)[None, :, None, None]
+    if mode == 0:
+        away = lambda v: np.where(v >= 0, np.floor(v + F(0.5)), np.ceil(v - F(0.5)))  # half away from zero
+        h, w = away(fh.astype(np.float64)).astype(np.int64), away(fw.astype(np.float64)).astype(np.int64)
+        outside = (h < 0) | (w < 0) | (h > in_h - 1) | (w > in_w - 1)
+        h, w = np.clip(h, 0, in_h - 1), np.clip(w, 0, in_w - 1)
+        out = x[bi, ci, h[:, None], w[:, None]]
+        return np.where(outside[:, None] & (padding_mode == 0), F(0), out).astype(F)
+    outside = (fh < 0) | (fw < 0) | (fh > in_h - 1) | (fw > in_w - 1)
+    if padding_mode == 1:
+        fh, fw = np.clip(fh, F(0), F(in_h - 1)), np.clip(fw, F(0), F(in_w - 1))
+    safe_h, safe_w = np.clip(fh, 0, in_h - 1), np.clip(fw, 0, in_w - 1)  # masked out below where it matters
+    h0, h1 = np.floor(safe_h).astype(np.int64), np.ceil(safe_h).astype(np.int64)
+    w0, w1 = np.floor(safe_w).astype(np.int64), np.ceil(safe_w).astype(np.int64)
+    sh, sw = (safe_h - h0.astype(F))[:, None], (safe_w - w0.astype(F))[:, None]
+    pick = lambda hh, ww: x[bi, ci, hh[:, None], ww[:, None]]
+    one = F(1)
+    out = ((one - sh) * (one - sw) * pick(h0, w0) + sh * (one - sw) * pick(h1, w0) + (one - sh) * sw * pick(h0, w1)
+           + sh * sw * pick(h1, w1))
+    if padding_mode == 0:
+        out = np.where(outside[:, None], F(0), out)
+    return out.astype(F)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("padding_mode", [0, 1])
+@pytest.mark.parametrize("shape,out_hw", [((2, 3, 5, 7), (4, 6)), ((1, 2, 1, 9), (3, 3)), ((3, 1, 8, 1), (2, 5)),
+                                          ((2, 4, 6, 6), (11, 13))])
+def test_grid_sample_against_array_formulation(mode, padding_mode, shape, out_hw):
+    x = normal(71, shape, 2.0)
+    grid = uniform(72, (shape[0],) + out_hw + (2,), -1.3, 1.3)  # a fifth of the coordinates outside the input
+    want = grid_sample_by_arrays(x, grid, mode, padding_mode)
+    assert_bit_exact(oracle.grid_sample_op(x, grid, mode, padding_mode), want, "grid sample")
+
+
+def test_grid_sample_known_values():
+    x = np.arange(15, dtype=F).reshape(1, 1, 5, 3)  # extents whose cell centres are exact coordinates
+    gy, gx = np.meshgrid(np.linspace(-1, 1, 5), np.linspace(-1, 1, 3), indexing="ij")
+    centres = np.stack([gx, gy], -1).astype(F)[None]
+    for mode in (0, 1):
+        assert_bit_exact(oracle.grid_sample_op(x, centres, mode, 0), x, "the grid of the cell centres gives the input back")
+    # half way between cells 0 and 1 of the first row, and between rows 0 and 1 of the first column
+    mid = np.array([[[[-0.5, -1.0], [-1.0, -0.75]]]], F)
+    assert_bit_exact(oracle.grid_sample_op(x, mid, 1, 0), F([[[[0.5, 1.5]]]]), "averages")
+    # outside: zeros, or the border cell
+    far = np.array([[[[-2.0, -1.0], [3.0, 1.0], [0.0, 40.0]]]], F)
+    assert_bit_exact(oracle.grid_sample_op(x, far, 1, 0), np.zeros((1, 1, 1, 3), F), "zeros outside")
+    assert_bit_exact(oracle.grid_sample_op(x, far, 0, 0), np.zeros((1, 1, 1, 3), F), "zeros outside, nearest")
+    assert_bit_exact(oracle.grid_sample_op(x, far, 0, 1), F([[[[0, 14, 13]]]]), "border, nearest")
+    assert_bit_exact(oracle.grid_sample_op(x, far, 1, 1), F([[[[0, 14, 13]]]]), "border, bilinear")
+    # a tie goes away from zero: coordinate 0.5 of a row of two is cell 1
+    two = F([[[[5, 7]]]])
+    assert_bit_exact(oracle.grid_sample_op(two, F([[[[0.0, 0.0]]]]), 0, 0), F([[[[7]]]]), "round half away from zero")
+
+
+def test_grid_sample_coordinates_that_fit_no_int_and_checks():
+    x = np.arange(6, dtype=F).reshape(1, 1, 2, 3)
+    huge = np.array([[[[1e30, 0.0], [-1e30, 0.0], [np.inf, -1.0], [np.nan, 1.0]]]], F)
+    # nearest: the conversion of the reference's x86-64 build gives INT_MIN: zero, or clamped to cell 0
+    assert_bit_exact(oracle.grid_sample_op(x, huge, 0, 0), np.zeros((1, 1, 1, 4), F), "nearest, zeros")
+    assert_bit_exact(oracle.grid_sample_op(x, huge, 0, 1), F([[[[3, 3, 0, 3]]]]), "nearest, border")
+    # bilinear: clamped or rejected before any conversion; a NaN coordinate gives NaN
+    got = oracle.grid_sample_op(x, huge, 1, 1).ravel()
+    assert_bit_exact(got[:3], F([3.5, 1.5, 2]), "bilinear, border")  # rows 0 and 1 half and half in the border column
+    assert np.isnan(got[3])
+    got = oracle.grid_sample_op(x, huge, 1, 0).ravel()
+    assert_bit_exact(got[:3], F([0, 0, 0]), "bilinear, zeros")
+    assert np.isnan(got[3])
+    grid = np.zeros((1, 2, 2, 2), F)
+    for bad in (dict(mode=2), dict(padding_mode=2)):
+        with pytest.raises(oracle.OracleCheckError):
+            oracle.grid_sample_op(x, grid, **bad)
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.grid_sample_op(x, np.zeros((2, 2, 2, 2), F))
+    with pytest.raises(oracle.OracleCheckError):
+        oracle.grid_sample_op(x, np.zeros((1, 2, 2, 3), F))
