@@ -294,8 +294,13 @@ def probe_next(dev):
     ssd_ws = dev.buf(nbytes=max(8, lib.shdw_hip_ssd_normalize_workspace_bytes(64, 512, 1444, 1)))
     ssd_sc = dev.buf(uniform(208, 512, 10.0, 30.0))
     stem_in, stem_out = [64, 64, 112, 112], [64, 64, 56, 56]
+    gy, gx = np.meshgrid(np.linspace(-1, 1, 56), np.linspace(-1, 1, 56), indexing="ij")
+    warp = np.stack([gx, gy], -1).astype(np.float32)[None] + uniform(614, (64, 56, 56, 2), -0.05, 0.05)
+    grid = dev.buf(np.ascontiguousarray(warp, np.float32).ravel())
+    whole = I([64, C, 56, 56])
     for _ in range(3):
         dev.ck(lib.shdw_hip_copy(n, x.ptr, y.ptr, st))
+        dev.ck(lib.shdw_hip_grid_sample(whole, whole, 1, 0, x.ptr, grid.ptr, y.ptr, st))
         dev.ck(lib.shdw_hip_batch_norm(n, C, inner, x.ptr, b.ptr, g.ptr, 1.0, 1e-5, y.ptr, st))
         dev.ck(lib.shdw_hip_batch_norm_scale(n, C, inner, x.ptr, b.ptr, g.ptr, 1.0, 1e-5, g.ptr, b.ptr, 1, y.ptr, st))
         dev.ck(lib.shdw_hip_lrn(I([64, C, 56, 56]), 5, 1e-4, 0.75, 1.0, x.ptr, y.ptr, st))
