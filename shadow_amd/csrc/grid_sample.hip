@@ -48,7 +48,7 @@ __global__ __launch_bounds__(kBlock) void grid_sample_kernel(const float* x, con
   // cell, and whatever the grid's warp adds): numbered so that each XCD owns a contiguous
   // range of (channel share, position group) pairs they find them in their own L2.
   // [64,256,56,56] with a grid warped by +-1.4 cells: 427 MB fetched for 207 with the
-  // workgroups dealt out round-robin.
+  // workgroups dealt out round-robin, 257 MB so.
   uint32_t share, group;
   fd_divmod(xcd_contiguous(blockIdx.x, gridDim.x), f_groups, share, group);
   const uint32_t p = group * kBlock + threadIdx.x;
