@@ -2,7 +2,9 @@
  * TEST INFRASTRUCTURE -- NOT PART OF THE PRODUCT.
  *
  * CPU restatement, in plain C, of the loops that junluan/shadow runs on the host
- * for its Unary / Binary / Eltwise / Reduce / Activate / Scale operators when
+ * for its Unary / Binary / Eltwise / Reduce / Activate / Scale operators, and for
+ * the operators next to them (Axpy, BatchNorm, LRN, GridSample, Pooling, Softmax,
+ * Normalize, SSDNormalize, Group/Instance/LayerNorm, and the data movers), when
  * built without Eigen/BLAS/DNNL (the "plain loop + libm" branch).  It is the
  * checker for the HIP kernels and the CPU leg of the benchmark; nothing under
  * shadow_amd/ may call it.
