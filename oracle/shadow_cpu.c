@@ -19,6 +19,13 @@
  * fp64 evaluations within 1 ulp.  The reference holds no test vectors for this
  * path and its own build needs a cmake-generated header, so no compiled
  * reference backs these checks.
+ *
+ * Parity unpinned: the last bit of everything that comes from libm (orc_unary's
+ * log / exp / sin / cos / tan / asin / acos / atan, pow, sigmoid, softplus, tanh,
+ * gelu, the expf inside softmax, the powf inside normalize and lrn) is whatever the
+ * host's libm gives, as in the reference; tests/golden/libm_glibc235.npz records
+ * the glibc 2.35 values the device code is built to.  orc_grid_sample: a coordinate
+ * that fits no int, and a NaN coordinate in the bilinear mode (see there).
  */
 #include <float.h>
 #include <math.h>
