@@ -9,9 +9,8 @@
 // the second pass: the window's values wait in registers (windows of up to seven
 // channels) or in LDS (a column of `size` floats per lane, no two lanes share a
 // bank row), the centre of the window is multiplied as soon as its scale is
-// known, x is read once and y written once.  Neighbouring
-// lanes hold neighbouring positions, so every load and store of a wave is one run
-// of 256 bytes.  y may be x: a lane has read every channel of a round, and all
+// known, x is read once and y written once.  Neighbouring lanes hold neighbouring
+// positions, so every load and store of a wave is one run of 256 bytes.  y may be x: a lane has read every channel of a round, and all
 // before it, when it writes the channels the round finishes, which lie behind them.
 #include <hip/hip_runtime.h>
 
@@ -33,12 +32,10 @@ constexpr int kLrnMaxSize = 63;
 // through them one by one, and only then come the powers, which do not depend on
 // one another -- eight of them side by side, in their branch-free form, hide the
 // latency of their table look-ups and fp64 chains, which the walk itself cannot
-// (one power per step of the walk: 378 us on [64,256,56,56]; in rounds: 236 us).
+// (one power per step of the walk: 378 us on [64,256,56,56]; in rounds: 236 us; with the
+// window in registers, the next round's loads under way and the tables in LDS: 140 us).
 constexpr uint32_t kLrnRound = 8;
 
-// powf(scale, y) for the scales of a round.  The straight path for all of them (any
-// bits may go in, see powf_ordinary); then, if some lane holds a scale that is not a
-// positive normal number, the whole function for those, one instance of its code.
 // The two tables of powf in LDS: read from there, the powers leave the vector
 // memory counter alone, so that waiting for a table entry is not waiting for the
 // next round's channels, which were asked for before it.
@@ -54,6 +51,9 @@ SHDW_DEVICE void lrn_stage_tables(LrnTables* t) {
   __syncthreads();
 }
 
+// powf(scale, y) for the scales of a round.  The straight path for all of them (any
+// bits may go in, see powf_ordinary); then, if some lane holds a scale that is not a
+// positive normal number, the whole function for those, one instance of its code.
 SHDW_DEVICE void lrn_powers(const float (&scale)[kLrnRound], float y, const LrnTables* t,
                             float (&power)[kLrnRound]) {
   bool plain = true;
@@ -75,10 +75,6 @@ SHDW_DEVICE void lrn_powers(const float (&scale)[kLrnRound], float y, const LrnT
   }
 }
 
-// ---- windows of 1, 3, 5 and 7 channels: the window lives in registers ----
-// prev[t] is channel head0 - SIZE + t, the last SIZE channels of the round before.
-// EDGE: the first round and those that reach past the last channel, with the tests
-// of the reference's three loops; the rounds between them need none.
 // The channels of the round that starts at head0 (zeros past the last one).
 SHDW_DEVICE void lrn_fetch(const float* in, uint32_t head0, uint32_t channels, uint32_t step,
                            float (&values)[kLrnRound]) {
@@ -87,6 +83,10 @@ SHDW_DEVICE void lrn_fetch(const float* in, uint32_t head0, uint32_t channels, u
     values[j] = head0 + j < channels ? in[static_cast<size_t>(head0 + j) * step] : 0.f;
 }
 
+// ---- windows of 1, 3, 5 and 7 channels: the window lives in registers ----
+// prev[t] is channel head0 - SIZE + t, the last SIZE channels of the round before.
+// EDGE: the first round and those that reach past the last channel, with the tests
+// of the reference's three loops; the rounds between them need none.
 // `round` holds the channels of this round on entry and those of the next on
 // return: they are asked for before the powers and arrive while those are worked
 // out.  (The channels this round writes lie behind all of them, y may be x.)
