@@ -103,3 +103,13 @@ def test_movers(ws, big):
     assert_bit_exact(got, oracle.reorg_op(big.reshape(64, 64, 112, 112), 1, 2), "reorg")
     got = run(ws, "Pad", [("x", big)], {"paddings": [1, 1, 1, 1], "value": 0.5}, tops=["pd"])
     assert_bit_exact(got, np.pad(big, ((0, 0), (0, 0), (1, 1), (1, 1)), constant_values=F(0.5)), "pad")
+
+
+def test_lrn_and_grid_sample(ws, big):
+    got = run(ws, "LRN", [("x", big)], {"local_size": 5, "alpha": 1e-4, "beta": 0.75, "k": 1.0}, tops=["lrn"])
+    assert_bit_exact(got, oracle.lrn_op(big, 5, 1e-4, 0.75, 0, 1.0), "lrn")
+    gy, gx = np.meshgrid(np.linspace(-1, 1, 56), np.linspace(-1, 1, 56), indexing="ij")
+    grid = np.stack([gx, gy], -1).astype(F)[None] + uniform(906, (64, 56, 56, 2), -0.08, 0.08)  # leaves the input at the rim
+    for mode in (0, 1):
+        got = run(ws, "GridSample", [("x", big), ("grid", grid)], {"mode": mode, "padding_mode": mode}, tops=["gs%d" % mode])
+        assert_bit_exact(got, oracle.grid_sample_op(big, grid, mode, mode), "grid sample %d" % mode)
