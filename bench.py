@@ -477,6 +477,26 @@ def sweep(dev):
         for typ, nm in ((0, "nearest"), (1, "bilinear")):
             us = tm(lambda k: lib.shdw_hip_resize(I(shape), I(out), typ, 0, X[k].ptr, Y[k].ptr, st))
             show("resize", "%s %s -> %dx%d" % (nm, shape, out_hw[0], out_hw[1]), us, 4 * (min(n_in, 4 * n_out) + n_out))
+    # GridSample: the grid of the cell centres warped by up to 1.4 cells, and positions drawn at random inside the input
+    for shape in ([16, 256, 56, 56], [64, 64, 56, 56], [1024, 256, 7, 7], [4, 3, 1024, 1024]):
+        b, c, h, w = shape
+        gy, gx = np.meshgrid(np.linspace(-1, 1, h), np.linspace(-1, 1, w), indexing="ij")
+        centres = np.stack([gx, gy], -1).astype(np.float32)[None]
+        grids = (("warped identity", dev.buf(np.ascontiguousarray(centres + uniform(31, (b, h, w, 2), -2.8 / h, 2.8 / h)).ravel())),
+                 ("random positions", dev.buf(uniform(32, b * h * w * 2, -1.0, 1.0))))
+        for what, g in grids:
+            for mode, nm in ((0, "nearest"), (1, "bilinear")):
+                us = tm(lambda k: lib.shdw_hip_grid_sample(I(shape), I(shape), mode, 0, X[k].ptr, g.ptr, Y[k].ptr, st))
+                show("grid sample", "%s %s, %s" % (nm, shape, what), us, 8 * b * c * h * w + 8 * b * h * w)
+        for _, g in grids:
+            g.free()
+    # LRN: the window in registers (3, 5, 7) and in LDS (9, 15), few and many channels
+    for shape, size in (([16, 256, 56, 56], 5), ([16, 256, 56, 56], 3), ([16, 256, 56, 56], 9), ([44, 96, 55, 55], 5),
+                        ([68, 256, 27, 27], 5), ([1024, 256, 7, 7], 5), ([256, 256, 14, 14], 15), ([64, 8, 158, 158], 7)):
+        n = int(np.prod(shape))
+        assert n <= N
+        us = tm(lambda k: lib.shdw_hip_lrn(I(shape), size, 1e-4, 0.75, 1.0, X[k].ptr, Y[k].ptr, st))
+        show("lrn", "window %d on %s" % (size, shape), us, 8 * n)
     for shape, stride in (([64, 64, 56, 56], 2), ([138, 64, 38, 38], 2), ([64, 16, 112, 112], 4), ([36, 512, 26, 26], 2)):
         n = int(np.prod(shape))
         for typ, nm in ((0, "darknet"), (1, "natural")):

@@ -93,7 +93,7 @@ SHDW_DEVICE void lrn_fetch(const float* in, uint32_t head0, uint32_t channels, u
 template <int SIZE, bool EDGE>
 SHDW_DEVICE void lrn_round(const float* in, float* out, uint32_t head0, uint32_t channels, uint32_t step,
                            float (&round)[kLrnRound], float (&prev)[SIZE], float& accum, float alpha_over_size,
-                           float neg_beta, float k, const LrnTables* tables) {
+                           float neg_beta, float k, const LrnTables* tables, bool finish) {
   static_assert(SIZE % 2 == 1 && SIZE <= static_cast<int>(kLrnRound), "the window must fit into a round");
   constexpr uint32_t post = (SIZE - 1) / 2;
   const uint32_t steps = channels + post;  // step `head` takes channel head in and finishes channel head - post
@@ -118,6 +118,7 @@ SHDW_DEVICE void lrn_round(const float* in, float* out, uint32_t head0, uint32_t
   }
 #pragma unroll
   for (int t = 0; t < SIZE; ++t) prev[t] = entering[kLrnRound - SIZE + t];
+  if (!finish) return;  // a round in front of this workgroup's share: only the sum had to pass through it
   lrn_powers(scale, neg_beta, tables, power);
 #pragma unroll
   for (uint32_t j = 0; j < kLrnRound; ++j) {
@@ -143,12 +144,20 @@ __global__ __launch_bounds__(kBlock) void lrn_window_kernel(const float* x, floa
   for (int t = 0; t < SIZE; ++t) prev[t] = 0.f;
   float accum = 0.f;
   const uint32_t steps = channels + (SIZE - 1) / 2;
+  // gridDim.y workgroups share the rounds of a position: each walks the sum from the
+  // first channel on, which is cheap, and works out the powers of its own rounds only
+  const uint32_t rounds = (steps + kLrnRound - 1) / kLrnRound;
+  const uint32_t first = blockIdx.y * rounds / gridDim.y * kLrnRound;
+  const uint32_t end = (blockIdx.y + 1) * rounds / gridDim.y * kLrnRound;
   lrn_fetch(in, 0, channels, step, round);
-  for (uint32_t head0 = 0; head0 < steps; head0 += kLrnRound) {
+  for (uint32_t head0 = 0; head0 < end; head0 += kLrnRound) {
+    const bool finish = head0 >= first;
     if (head0 >= SIZE && head0 + kLrnRound <= channels)
-      lrn_round<SIZE, false>(in, out, head0, channels, step, round, prev, accum, alpha_over_size, neg_beta, k, &tables);
+      lrn_round<SIZE, false>(in, out, head0, channels, step, round, prev, accum, alpha_over_size, neg_beta, k, &tables,
+                             finish);
     else
-      lrn_round<SIZE, true>(in, out, head0, channels, step, round, prev, accum, alpha_over_size, neg_beta, k, &tables);
+      lrn_round<SIZE, true>(in, out, head0, channels, step, round, prev, accum, alpha_over_size, neg_beta, k, &tables,
+                            finish);
   }
 }
 
@@ -171,8 +180,11 @@ __global__ __launch_bounds__(kBlock) void lrn_across_channels_kernel(
   float accum = 0.f;
   uint32_t slot_head = 0, slot_mid = 0;  // head % size and (head - post) % size
   float round[kLrnRound];
+  const uint32_t rounds = (steps + kLrnRound - 1) / kLrnRound;  // shared out over gridDim.y as above
+  const uint32_t first = blockIdx.y * rounds / gridDim.y * kLrnRound;
+  const uint32_t end = (blockIdx.y + 1) * rounds / gridDim.y * kLrnRound;
   lrn_fetch(in, 0, channels, step, round);
-  for (uint32_t head0 = 0; head0 < steps; head0 += kLrnRound) {
+  for (uint32_t head0 = 0; head0 < end; head0 += kLrnRound) {
     float entering[kLrnRound], scale[kLrnRound], centre[kLrnRound], power[kLrnRound];
 #pragma unroll
     for (uint32_t j = 0; j < kLrnRound; ++j) entering[j] = round[j];
@@ -197,6 +209,7 @@ __global__ __launch_bounds__(kBlock) void lrn_across_channels_kernel(
         }
       }
     }
+    if (head0 < first) continue;  // in front of this workgroup's share: only the sum had to pass through
     lrn_powers(scale, neg_beta, &tables, power);
 #pragma unroll
     for (uint32_t j = 0; j < kLrnRound; ++j) {
@@ -232,7 +245,21 @@ extern "C" int shdw_hip_lrn(const int* in_shape, int size, float alpha, float be
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint32_t grid = grid_for(positions), chan = static_cast<uint32_t>(channels);
   const FastDiv f_step = make_fastdiv(step);
-#define SHDW_LRN(S) lrn_window_kernel<S><<<grid, kBlock, 0, st>>>(x, y, positions, step, chan, f_step, alpha_over_size, -beta, k)
+  // A tensor with few positions has few waves, and each walks all the channels one round after
+  // the other (82 us for 256 channels, however few the waves).  Up to eight workgroups then share
+  // the rounds of a position, about 4096 waves in all and four rounds each at the least; measured
+  // on 12.8 M elements: [16,256,56,56] (784 waves) 82 -> 65, 56, 60, 77 us with 2, 4, 8, 16 shares,
+  // [44,96,55,55] (2080 waves) 49 -> 42, 47, 55; [64,256,56,56] (3136 waves) 141 -> 139, 149.
+  // In place a workgroup would overwrite what another still has to read: one share.
+  const uint32_t waves = (positions + kWave - 1) / kWave;
+  const uint32_t rounds = (chan + static_cast<uint32_t>(post) + kLrnRound - 1) / kLrnRound;
+  uint32_t shares = (4096 + waves / 2) / waves;
+  const uint32_t most = waves <= 512 ? 8u : 4u;
+  shares = shares > most ? most : shares;
+  shares = shares > rounds / 4 ? rounds / 4 : shares;
+  if (x == y || shares < 1) shares = 1;
+#define SHDW_LRN(S) \
+  lrn_window_kernel<S><<<dim3(grid, shares), kBlock, 0, st>>>(x, y, positions, step, chan, f_step, alpha_over_size, -beta, k)
   if (size == 1) {
     SHDW_LRN(1);
   } else if (size == 3) {
@@ -243,7 +270,7 @@ extern "C" int shdw_hip_lrn(const int* in_shape, int size, float alpha, float be
     SHDW_LRN(7);
   } else {
     const size_t lds = static_cast<size_t>(size) * kBlock * sizeof(float);
-    lrn_across_channels_kernel<<<grid, kBlock, lds, st>>>(x, y, positions, step, chan, f_step,
+    lrn_across_channels_kernel<<<dim3(grid, shares), kBlock, lds, st>>>(x, y, positions, step, chan, f_step,
                                                           static_cast<uint32_t>(size), alpha_over_size, -beta, k);
   }
 #undef SHDW_LRN
